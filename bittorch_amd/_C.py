@@ -1,0 +1,291 @@
+"""``bittorch._C`` look-alike over the C-ABI HIP library.
+
+Same four entry points, argument order and keyword names as the reference's
+pybind11 module (``csrc/bindings/bittorch_bindings.cpp:34-88``) with the host
+checks of ``csrc/core/dispatch.cpp:52-142``; additional entry points expose
+the fused quantize+pack kernel and the int8 pipeline stages.  Tensors are
+passed to the library as raw device pointers; outputs and scratch are
+allocated here with torch so the library itself never allocates.
+
+Importing this module raises ``ImportError`` when the library is not built.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from . import _lib
+
+_L = _lib.load()  # ImportError here == "extension not available"
+
+_DT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+_INT8_OUT = 3
+
+
+def _check(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _status(rc: int) -> None:
+    if rc != 0:
+        raise RuntimeError(_lib.last_error() or f"libbittorch_hip call failed ({rc})")
+
+
+def _stream(t: Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: Optional[Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _dt(t: Tensor, what: str) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise RuntimeError(f"{what} must be float32, float16 or bfloat16, got {t.dtype}") from None
+
+
+def _workspace(nbytes: int, device) -> Optional[Tensor]:
+    return torch.empty(nbytes, dtype=torch.uint8, device=device) if nbytes > 0 else None
+
+
+def _all_cuda(*ts: Optional[Tensor]) -> bool:
+    return all(t is None or t.is_cuda for t in ts)
+
+
+def _prep_vec(v: Tensor, x: Tensor) -> Tensor:
+    """scale / bias operand: contiguous, in a dtype the kernels read (fp32 or 16-bit)."""
+    if v.dtype not in _DT:
+        v = v.to(x.dtype if x.dtype in _DT else torch.float32)
+    return v.contiguous()
+
+
+def dummy(input: Tensor) -> Tensor:
+    """Copy of the input (reference ``dispatch.cpp:7-9``)."""
+    return input.clone()
+
+
+def _float64_packed(X, W_T, scale, bias, in_features):
+    from .quant.ternary_packed import unpack_ternary_transposed
+    w = unpack_ternary_transposed(W_T, in_features).to(X.dtype) * scale.to(X.dtype).unsqueeze(1)
+    return torch.nn.functional.linear(X, w, None if bias is None else bias.to(X.dtype))
+
+
+def ternary_linear_forward(X: Tensor, W_tern: Tensor, scale: Tensor,
+                           bias: Optional[Tensor] = None) -> Tensor:
+    """``Y = X @ (W_tern * scale).T + bias`` with dense int8 ternary weights ``[N, K]``.
+
+    Reference: ``bittorch_bindings.cpp:41-46``, ``dispatch.cpp:52-87``.
+    """
+    _check(X.dim() >= 1, "X must have at least 1 dimension")
+    _check(X.numel() > 0, "X is empty")
+    _check(W_tern.dim() == 2, "W_tern must be 2D [N, K]")
+    _check(W_tern.dtype == torch.int8, "W_tern must be int8")
+    _check(scale.dim() == 1, "scale must be 1D [N]")
+    K = X.shape[-1]
+    N, WK = W_tern.shape
+    _check(K == WK, "input K doesn't match weight K")
+    _check(scale.shape[0] in (N, 1), "scale size doesn't match N")
+    if bias is not None:
+        _check(bias.dim() == 1 and bias.shape[0] == N, "bias shape mismatch")
+    _check(_all_cuda(X, W_tern, scale, bias), "All tensors must be CUDA")
+    if X.dtype == torch.float64:
+        w = W_tern.to(X.dtype) * scale.to(X.dtype).unsqueeze(1)
+        return torch.nn.functional.linear(X, w, None if bias is None else bias.to(X.dtype))
+    x2 = X.contiguous().reshape(-1, K)
+    W_tern = W_tern.contiguous()
+    scale = _prep_vec(scale, x2)
+    bias = None if bias is None else _prep_vec(bias, x2)
+    B = x2.shape[0]
+    y = torch.empty((B, N), dtype=X.dtype, device=X.device)
+    with torch.cuda.device(X.device):
+        _status(_L.bt_ternary_linear_forward(
+            x2.data_ptr(), _dt(x2, "X"), W_tern.data_ptr(), scale.data_ptr(), _dt(scale, "scale"),
+            scale.numel(), _ptr(bias), 0 if bias is None else _dt(bias, "bias"), y.data_ptr(),
+            B, N, K, _stream(X)))
+    return y.reshape(*X.shape[:-1], N)
+
+
+def _packed_checks(X, W_T, scale, bias, in_features, flatten: bool = True):
+    _check(X.dim() >= 1, "X must have at least 1 dimension")
+    _check(X.numel() > 0, "X is empty")
+    _check(W_T.dim() == 2, "W_T must be 2D [K_bytes, N]")
+    _check(W_T.dtype == torch.uint8, "W_T must be uint8")
+    _check(scale.dim() == 1, "scale must be 1D [N]")
+    K = X.shape[-1]
+    K_bytes, N = W_T.shape
+    _check(K == in_features, "input K doesn't match in_features")
+    _check(K_bytes == (in_features + 3) // 4, "K_bytes doesn't match ceil(K/4)")
+    _check(scale.shape[0] in (N, 1), "scale size doesn't match N")
+    if bias is not None:
+        _check(bias.dim() == 1 and bias.shape[0] == N, "bias shape mismatch")
+    _check(_all_cuda(X, W_T, scale, bias), "All tensors must be CUDA")
+    return K, N
+
+
+def ternary_linear_packed_forward(X: Tensor, W_T: Tensor, scale: Tensor,
+                                  bias: Optional[Tensor] = None, in_features: int = -1) -> Tensor:
+    """Packed-weight forward, fp32 accumulation; ``W_T`` is ``[ceil(K/4), N]`` uint8.
+
+    Reference: ``bittorch_bindings.cpp:48-63``, ``dispatch.cpp:105-142``.  ``scale``
+    may be fp32 or the activation dtype and may have one entry (per-tensor scale).
+    """
+    if in_features < 0:
+        in_features = X.shape[-1]
+    K, N = _packed_checks(X, W_T, scale, bias, in_features)
+    if X.dtype == torch.float64:
+        return _float64_packed(X, W_T, scale, bias, in_features)
+    x2 = X.contiguous().reshape(-1, K)
+    W_T = W_T.contiguous()
+    scale = _prep_vec(scale, x2)
+    bias = None if bias is None else _prep_vec(bias, x2)
+    B = x2.shape[0]
+    xdt = _dt(x2, "X")
+    y = torch.empty((B, N), dtype=X.dtype, device=X.device)
+    with torch.cuda.device(X.device):
+        ws_bytes = _L.bt_packed_forward_workspace_bytes(B, N, K, xdt)
+        ws = _workspace(ws_bytes, X.device)
+        _status(_L.bt_ternary_linear_packed_forward(
+            x2.data_ptr(), xdt, W_T.data_ptr(), scale.data_ptr(), _dt(scale, "scale"), scale.numel(),
+            _ptr(bias), 0 if bias is None else _dt(bias, "bias"), y.data_ptr(), B, N, K,
+            _ptr(ws), ws_bytes, _stream(X)))
+    return y.reshape(*X.shape[:-1], N)
+
+
+def ternary_linear_tensor_core_forward(X: Tensor, W_T: Tensor, scale: Tensor,
+                                       bias: Optional[Tensor] = None, in_features: int = -1,
+                                       version: int = 1) -> Tensor:
+    """Matrix-core forward; ``X`` must be 2-D as in the reference.
+
+    version 1: float compute (the reference's validation kernel,
+    ``ternary_gemm_tensor_core.cu:120-271``) -- served by the fp32-accumulate
+    packed kernel.  version 2: per-row int8 activations, int8 MFMA, int32
+    accumulators (``:349-657`` with the whole-row activation scale).
+    """
+    _check(X.dim() == 2, "X must be 2D")
+    _check(version in (1, 2), "version must be 1 (V1 float) or 2 (V2 mma.sync)")
+    if in_features < 0:
+        in_features = X.shape[-1]
+    K, N = _packed_checks(X, W_T, scale, bias, in_features)
+    if version == 1:
+        return ternary_linear_packed_forward(X, W_T, scale, bias, in_features)
+    _check(X.dtype in _DT, "X must be float32, float16 or bfloat16 for version 2")
+    x2 = X.contiguous()
+    W_T = W_T.contiguous()
+    scale = _prep_vec(scale, x2)
+    bias = None if bias is None else _prep_vec(bias, x2)
+    B = x2.shape[0]
+    y = torch.empty((B, N), dtype=X.dtype, device=X.device)
+    with torch.cuda.device(X.device):
+        ws_bytes = _L.bt_tensor_core_workspace_bytes(B, N, K)
+        ws = _workspace(ws_bytes, X.device)
+        _status(_L.bt_ternary_linear_tensor_core_forward(
+            x2.data_ptr(), _dt(x2, "X"), W_T.data_ptr(), scale.data_ptr(), _dt(scale, "scale"),
+            scale.numel(), _ptr(bias), 0 if bias is None else _dt(bias, "bias"), y.data_ptr(),
+            B, N, K, _ptr(ws), ws_bytes, _stream(X)))
+    return y
+
+
+# ---- additive entry points (no counterpart in the reference module) ----------------------
+
+
+def ternary_quantize_pack(weight: Tensor, threshold_factor: float = 0.05, per_channel: bool = True,
+                          want_packed: bool = True, want_tern: bool = False
+                          ) -> Tuple[Optional[Tensor], Tensor, Optional[Tensor]]:
+    """Fused quantize + pack of master weights ``[N, K]`` on the GPU.
+
+    Returns ``(packed_T uint8 [ceil(K/4), N] | None, scale, w_tern int8 [N, K] | None)``;
+    ``scale`` has the weight dtype and shape ``(N,)`` (per channel) or ``()`` (per tensor),
+    exactly what ``quant.ternary_quantize`` returns.
+    """
+    _check(weight.dim() == 2, "weight must be 2D [N, K]")
+    _check(weight.is_cuda, "All tensors must be CUDA")
+    w = weight.detach().contiguous()
+    N, K = w.shape
+    _check(N > 0 and K > 0, "weight is empty")
+    wdt = _dt(w, "weight")
+    dev = w.device
+    packed = torch.empty(((K + 3) // 4, N), dtype=torch.uint8, device=dev) if want_packed else None
+    tern = torch.empty((N, K), dtype=torch.int8, device=dev) if want_tern else None
+    scale = torch.empty((N if per_channel else 1,), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _status(_L.bt_quantize_pack(w.data_ptr(), wdt, N, K, float(threshold_factor),
+                                    int(bool(per_channel)), _ptr(packed), scale.data_ptr(),
+                                    _ptr(tern), _stream(w)))
+    scale = scale.to(weight.dtype)
+    if not per_channel:
+        scale = scale.squeeze(0)
+    return packed, scale, tern
+
+
+def act_quant_int8(X: Tensor) -> Tuple[Tensor, Tensor]:
+    """Per-row int8 activation quantization: ``(Q int8 [B,K], s_x fp32 [B])``."""
+    _check(X.dim() == 2 and X.numel() > 0, "X must be 2D and non-empty")
+    _check(X.is_cuda, "All tensors must be CUDA")
+    x = X.contiguous()
+    B, K = x.shape
+    q = torch.empty((B, K), dtype=torch.int8, device=x.device)
+    s = torch.empty((B,), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        _status(_L.bt_act_quant_i8(x.data_ptr(), _dt(x, "X"), B, K, q.data_ptr(), s.data_ptr(),
+                                   _stream(x)))
+    return q, s
+
+
+def ternary_gemm_int8(Q: Tensor, s_x: Tensor, W_T: Tensor, scale: Tensor,
+                      bias: Optional[Tensor] = None, in_features: int = -1,
+                      out_dtype: torch.dtype = torch.float32, return_acc: bool = False):
+    """int8 activations x packed ternary weights; optionally also the int32 accumulators."""
+    _check(Q.dim() == 2 and Q.dtype == torch.int8, "Q must be 2D int8")
+    if in_features < 0:
+        in_features = Q.shape[-1]
+    K, N = _packed_checks(Q, W_T, scale, bias, in_features)
+    _check(s_x.dtype == torch.float32 and s_x.numel() == Q.shape[0], "s_x must be fp32 [B]")
+    _check(_all_cuda(s_x), "All tensors must be CUDA")
+    _check(out_dtype in _DT, "out_dtype must be float32, float16 or bfloat16")
+    q = Q.contiguous()
+    W_T = W_T.contiguous()
+    s_x = s_x.contiguous()
+    scale = _prep_vec(scale, s_x)
+    bias = None if bias is None else _prep_vec(bias, s_x)
+    B = q.shape[0]
+    y = torch.empty((B, N), dtype=out_dtype, device=q.device)
+    acc = torch.empty((B, N), dtype=torch.int32, device=q.device) if return_acc else None
+    with torch.cuda.device(q.device):
+        ws_bytes = _L.bt_gemm_i8_workspace_bytes(B, N, K)
+        ws = _workspace(ws_bytes, q.device)
+        _status(_L.bt_ternary_gemm_i8(
+            q.data_ptr(), s_x.data_ptr(), W_T.data_ptr(), scale.data_ptr(), _dt(scale, "scale"),
+            scale.numel(), _ptr(bias), 0 if bias is None else _dt(bias, "bias"), y.data_ptr(),
+            _DT[out_dtype], _ptr(acc), B, N, K, _ptr(ws), ws_bytes, _stream(q)))
+    return (y, acc) if return_acc else y
+
+
+def unpack_dequant(W_T: Tensor, in_features: int, scale: Optional[Tensor] = None,
+                   out_dtype: torch.dtype = torch.float32) -> Tensor:
+    """Dense ``[N, K]`` weights from packed ``W_T``: ``decode * scale[:, None]``
+    (``out_dtype`` float) or the plain ternary values (``out_dtype=torch.int8``)."""
+    _check(W_T.dim() == 2 and W_T.dtype == torch.uint8, "W_T must be 2D uint8")
+    _check(W_T.shape[0] == (in_features + 3) // 4, "K_bytes doesn't match ceil(K/4)")
+    _check(_all_cuda(W_T, scale), "All tensors must be CUDA")
+    W_T = W_T.contiguous()
+    N = W_T.shape[1]
+    if out_dtype == torch.int8:
+        odt, scale_f = _INT8_OUT, None
+    else:
+        _check(out_dtype in _DT, "out_dtype must be float32, float16, bfloat16 or int8")
+        odt = _DT[out_dtype]
+        scale_f = None if scale is None else scale.reshape(-1).to(torch.float32).contiguous()
+        if scale_f is not None:
+            _check(scale_f.numel() in (N, 1), "scale size doesn't match N")
+    out = torch.empty((N, in_features), dtype=out_dtype, device=W_T.device)
+    with torch.cuda.device(W_T.device):
+        _status(_L.bt_unpack_dequant(W_T.data_ptr(), _ptr(scale_f),
+                                     0 if scale_f is None else scale_f.numel(), out.data_ptr(), odt,
+                                     N, in_features, _stream(W_T)))
+    return out

@@ -1,0 +1,165 @@
+// Internal helpers shared by the gfx950 kernels of libbittorch_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <algorithm>
+#include <type_traits>
+
+#include "../../include/bittorch_hip.h"
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+namespace bt {
+
+// operand modes of the streaming kernel
+enum { MODE_I8 = 0, MODE_F16 = 1, MODE_BF16 = 2 };
+
+// ---- host side: error text + launch check --------------------------------
+void set_error(const char* fmt, ...);
+int check_launch(const char* what);
+
+static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// ---- element access by dtype tag (BT_F32 / BT_F16 / BT_BF16) --------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) {
+    return __builtin_bit_cast(float, (uint32_t)h << 16);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);  // quiet NaN
+    u += 0x7fffu + ((u >> 16) & 1u);                                             // RNE
+    return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
+    return (float)__builtin_bit_cast(_Float16, h);
+}
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+    return __builtin_bit_cast(uint16_t, (_Float16)f);  // v_cvt_f16_f32, RNE
+}
+
+template <int DT>
+__device__ __forceinline__ float load_elem(const void* p, int64_t i) {
+    if constexpr (DT == BT_F32) return ((const float*)p)[i];
+    else if constexpr (DT == BT_F16) return f16_bits_to_f32(((const uint16_t*)p)[i]);
+    else return bf16_bits_to_f32(((const uint16_t*)p)[i]);
+}
+template <int DT>
+__device__ __forceinline__ void store_elem(void* p, int64_t i, float v) {
+    if constexpr (DT == BT_F32) ((float*)p)[i] = v;
+    else if constexpr (DT == BT_F16) ((uint16_t*)p)[i] = f32_to_f16_bits(v);
+    else ((uint16_t*)p)[i] = f32_to_bf16_bits(v);
+}
+// run-time dtype (scale / bias vectors: a handful of loads per thread)
+__device__ __forceinline__ float load_elem_rt(const void* p, int dt, int64_t i) {
+    if (dt == BT_F32) return ((const float*)p)[i];
+    if (dt == BT_F16) return f16_bits_to_f32(((const uint16_t*)p)[i]);
+    return bf16_bits_to_f32(((const uint16_t*)p)[i]);
+}
+// round a float to the grid of dtype dt and widen it again
+__device__ __forceinline__ float round_to_dtype(float v, int dt) {
+    if (dt == BT_F16) return f16_bits_to_f32(f32_to_f16_bits(v));
+    if (dt == BT_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(v));
+    return v;
+}
+static inline int dtype_size(int dt) { return dt == BT_F32 ? 4 : 2; }
+
+// Epilogue operand bundle (scale / bias vectors and their element types).
+struct Epilogue {
+    const void* scale;
+    const void* bias;  // may be null
+    int scale_dtype;
+    int bias_dtype;
+    int scale_bcast;  // 1: scale has one entry that applies to every column
+};
+__device__ __forceinline__ float epi_scale(const Epilogue& e, int64_t n) {
+    return load_elem_rt(e.scale, e.scale_dtype, e.scale_bcast ? 0 : n);
+}
+__device__ __forceinline__ float epi_bias(const Epilogue& e, int64_t n) {
+    return e.bias ? load_elem_rt(e.bias, e.bias_dtype, n) : 0.0f;
+}
+// fp32 accumulate path: one multiply, one add, each rounded (no fma contraction)
+__device__ __forceinline__ float epi_float(float acc, float s, float b) {
+    return __fadd_rn(__fmul_rn(acc, s), b);
+}
+// int8 path: ((float(acc) * s_x) / 127) * w_scale + bias, left to right
+__device__ __forceinline__ float epi_int8(int32_t acc127, float sx, float ws, float b) {
+    float r = __fmul_rn((float)acc127, sx);
+    r = __fdiv_rn(r, 127.0f);
+    r = __fmul_rn(r, ws);
+    return __fadd_rn(r, b);
+}
+
+// ---- 2-bit decode in registers -------------------------------------------
+// v_perm_b32: result byte i = byte sel[i] of the 8-byte value {hi,lo}
+// (0..3 -> lo, 4..7 -> hi); sel 8 -> 0xFF if bit 15 of lo is set else 0x00;
+// sel 12 -> 0x00.
+__device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) {
+    return __builtin_amdgcn_perm(hi, lo, sel);
+}
+
+// g[i] = { r0.byte[i], r1.byte[i], r2.byte[i], r3.byte[i] }  (byte 0 first)
+__device__ __forceinline__ void transpose4x4_bytes(uint32_t r0, uint32_t r1, uint32_t r2,
+                                                   uint32_t r3, uint32_t (&g)[4]) {
+    const uint32_t a_lo = perm(r1, r0, 0x05010400u);  // r0.b0 r1.b0 r0.b1 r1.b1
+    const uint32_t a_hi = perm(r1, r0, 0x07030602u);  // r0.b2 r1.b2 r0.b3 r1.b3
+    const uint32_t b_lo = perm(r3, r2, 0x05010400u);
+    const uint32_t b_hi = perm(r3, r2, 0x07030602u);
+    g[0] = perm(b_lo, a_lo, 0x05040100u);
+    g[1] = perm(b_lo, a_lo, 0x07060302u);
+    g[2] = perm(b_hi, a_hi, 0x05040100u);
+    g[3] = perm(b_hi, a_hi, 0x07060302u);
+}
+
+// G holds four packed bytes (four consecutive kb rows of one output column).
+// Returns 16 int8 weights in {-1,0,+1}: dword c, byte r = weight (row r, slot c),
+// i.e. k = 4*(kb0 + r) + c.  Codes: 1 -> +1, 2 -> -1, 0 and 3 -> 0.
+// Slots 0 and 2 index a 4-entry byte table with the code itself; slots 1 and 3
+// use the code still shifted left by two (0,4,8,12) as the selector, which the
+// table {lo.byte0 = 0, hi.byte0 = +1, "8" = 0xFF via lo bit 15, "12" = 0} decodes
+// without a shift.
+__device__ __forceinline__ v4i decode16_i8(uint32_t G) {
+    const uint32_t lutA_lo = 0x00FF0100u;  // sel 0..3 -> 0, +1, -1, 0
+    const uint32_t lutB_lo = 0x0000FF00u;  // byte0 = 0 (sel 0); bit 15 set (sel 8 -> 0xFF)
+    const uint32_t lutB_hi = 0x00000001u;  // sel 4 -> +1
+    const uint32_t H = G >> 4;
+    v4i out;
+    out[0] = (int)perm(0u, lutA_lo, G & 0x03030303u);
+    out[1] = (int)perm(lutB_hi, lutB_lo, G & 0x0C0C0C0Cu);
+    out[2] = (int)perm(0u, lutA_lo, H & 0x03030303u);
+    out[3] = (int)perm(lutB_hi, lutB_lo, H & 0x0C0C0C0Cu);
+    return out;
+}
+
+// M.byte1 / M.byte3 hold the packed bytes of two consecutive kb rows of one
+// output column.  Returns eight 16-bit floats: dword c = { w(row0, slot c),
+// w(row1, slot c) }, where the non-zero weights have high byte HI_POS / HI_NEG
+// and low byte 0 (fp16: +-1.0 = 0x3C00 / 0xBC00; bf16: +-2.0 = 0x4000 / 0xC000).
+template <uint32_t LUT>
+__device__ __forceinline__ u32x4 decode8_16bit(uint32_t M) {
+    u32x4 out;
+    out[0] = perm(0u, LUT, M & 0x03000300u);
+    out[1] = perm(0u, LUT, (M >> 2) & 0x03000300u);
+    out[2] = perm(0u, LUT, (M >> 4) & 0x03000300u);
+    out[3] = perm(0u, LUT, (M >> 6) & 0x03000300u);
+    return out;
+}
+constexpr uint32_t LUT_F16_ONE = 0x00BC3C00u;   // sel 0..3 -> 0x00, 0x3C, 0xBC, 0x00
+constexpr uint32_t LUT_BF16_TWO = 0x00C04000u;  // sel 0..3 -> 0x00, 0x40, 0xC0, 0x00
+
+__device__ __forceinline__ int decode2(uint32_t code) { return (int)(code == 1u) - (int)(code == 2u); }
+
+// ---- wave64 reductions ------------------------------------------------------
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+}  // namespace bt

@@ -1,0 +1,223 @@
+// extern "C" entry points of libbittorch_hip.so: validation and kernel choice.
+// Replaces the host dispatch of the reference (csrc/core/dispatch.cpp:52-142).
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+#include "bt_common.h"
+
+namespace bt {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+int check_launch(const char* what) {
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("%s: HIP launch failed: %s", what, hipGetErrorString(e));
+        return BT_ERR_LAUNCH;
+    }
+    return BT_OK;
+}
+
+// kernels in the other translation units
+bool stream_supported(int64_t N, const void* W_T);
+size_t stream_workspace_bytes(int mode, int64_t M, int64_t N, int64_t Kb);
+int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, const uint8_t* W_T,
+                  const Epilogue& epi, void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N,
+                  int64_t K, void* workspace, size_t ws_bytes, hipStream_t st);
+int launch_packed_generic(const void* X, int x_dtype, const uint8_t* W_T, const Epilogue& epi, void* Y,
+                          int64_t B, int64_t N, int64_t K, hipStream_t st);
+int launch_unpacked(const void* X, int x_dtype, const int8_t* W, const Epilogue& epi, void* Y, int64_t B,
+                    int64_t N, int64_t K, hipStream_t st);
+int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x, hipStream_t st);
+bool gemm_i8_supported(int64_t N, const void* W_T);
+int launch_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const Epilogue& epi, void* Y,
+                   int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st);
+
+static bool valid_dtype(int dt) { return dt == BT_F32 || dt == BT_F16 || dt == BT_BF16; }
+
+static int make_epilogue(const char* who, const void* scale, int scale_dtype, int64_t scale_len,
+                         const void* bias, int bias_dtype, int64_t N, Epilogue* e) {
+    if (!scale) {
+        set_error("%s: scale is null", who);
+        return BT_ERR_INVALID;
+    }
+    if (scale_len != N && scale_len != 1) {
+        set_error("%s: scale size doesn't match N (%lld entries, N=%lld)", who, (long long)scale_len,
+                  (long long)N);
+        return BT_ERR_INVALID;
+    }
+    if (!valid_dtype(scale_dtype) || (bias && !valid_dtype(bias_dtype))) {
+        set_error("%s: unsupported scale/bias dtype", who);
+        return BT_ERR_INVALID;
+    }
+    e->scale = scale;
+    e->bias = bias;
+    e->scale_dtype = scale_dtype;
+    e->bias_dtype = bias_dtype;
+    e->scale_bcast = (scale_len == 1 && N != 1) ? 1 : 0;
+    return BT_OK;
+}
+
+static int check_shape(const char* who, const void* X, const void* W, const void* Y, int x_dtype,
+                       int64_t B, int64_t N, int64_t K) {
+    if (!X || !W || !Y) {
+        set_error("%s: null tensor pointer", who);
+        return BT_ERR_INVALID;
+    }
+    if (B <= 0 || N <= 0 || K <= 0) {
+        set_error("%s: empty shape (B=%lld N=%lld K=%lld)", who, (long long)B, (long long)N, (long long)K);
+        return BT_ERR_INVALID;
+    }
+    if (!valid_dtype(x_dtype)) {
+        set_error("%s: unsupported activation dtype %d", who, x_dtype);
+        return BT_ERR_INVALID;
+    }
+    return BT_OK;
+}
+
+// The matrix-core paths write Y with vector stores and use 32-bit indices
+// inside a 16-row block.
+static bool fast_path_ok(const void* Y, int64_t N, int64_t K) {
+    return ((uintptr_t)Y) % 16 == 0 && N < (1ll << 30) && K < (1ll << 30);
+}
+
+// int32 accumulators hold sum_k q*127w with |q| <= 127
+static const int64_t kMaxKInt8 = 133000;
+
+// batches up to this many rows go through the streaming (decode-shape) kernel
+static const int64_t kStreamMaxRows = 32;
+
+static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+}  // namespace bt
+
+using namespace bt;
+
+extern "C" int bt_abi_version(void) { return BT_ABI_VERSION; }
+
+extern "C" const char* bt_last_error(void) { return g_err; }
+
+extern "C" int bt_ternary_linear_forward(const void* X, int x_dtype, const int8_t* W_tern, const void* scale,
+                                         int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
+                                         void* Y, int64_t B, int64_t N, int64_t K, void* stream) {
+    const char* who = "bt_ternary_linear_forward";
+    int rc = check_shape(who, X, W_tern, Y, x_dtype, B, N, K);
+    if (rc) return rc;
+    Epilogue epi;
+    rc = make_epilogue(who, scale, scale_dtype, scale_len, bias, bias_dtype, N, &epi);
+    if (rc) return rc;
+    return launch_unpacked(X, x_dtype, W_tern, epi, Y, B, N, K, (hipStream_t)stream);
+}
+
+static bool packed_uses_stream(int x_dtype, const void* W_T, const void* Y, int64_t N, int64_t K) {
+    if (getenv("BITTORCH_KERNEL") && !strcmp(getenv("BITTORCH_KERNEL"), "generic")) return false;
+    return x_dtype != BT_F32 && stream_supported(N, W_T) && fast_path_ok(Y, N, K);
+}
+
+extern "C" size_t bt_packed_forward_workspace_bytes(int64_t B, int64_t N, int64_t K, int x_dtype) {
+    if (B <= 0 || N <= 0 || K <= 0 || x_dtype == BT_F32 || N % 4 != 0) return 0;
+    return stream_workspace_bytes(x_dtype == BT_F16 ? MODE_F16 : MODE_BF16, B, N, ceil_div(K, 4));
+}
+
+extern "C" int bt_ternary_linear_packed_forward(const void* X, int x_dtype, const uint8_t* W_T,
+                                                const void* scale, int scale_dtype, int64_t scale_len,
+                                                const void* bias, int bias_dtype, void* Y, int64_t B,
+                                                int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
+                                                void* stream) {
+    const char* who = "bt_ternary_linear_packed_forward";
+    int rc = check_shape(who, X, W_T, Y, x_dtype, B, N, K);
+    if (rc) return rc;
+    Epilogue epi;
+    rc = make_epilogue(who, scale, scale_dtype, scale_len, bias, bias_dtype, N, &epi);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    if (packed_uses_stream(x_dtype, W_T, Y, N, K)) {
+        const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
+        return launch_stream(mode, X, 2, nullptr, W_T, epi, Y, x_dtype, nullptr, B, N, K, workspace,
+                             workspace_bytes, st);
+    }
+    return launch_packed_generic(X, x_dtype, W_T, epi, Y, B, N, K, st);
+}
+
+extern "C" int bt_act_quant_i8(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x,
+                               void* stream) {
+    if (!X || !Q || !s_x || B <= 0 || K <= 0 || !valid_dtype(x_dtype)) {
+        set_error("bt_act_quant_i8: null pointer, empty shape or bad dtype");
+        return BT_ERR_INVALID;
+    }
+    return launch_act_quant(X, x_dtype, B, K, Q, s_x, (hipStream_t)stream);
+}
+
+extern "C" size_t bt_gemm_i8_workspace_bytes(int64_t B, int64_t N, int64_t K) {
+    if (B <= 0 || N <= 0 || K <= 0 || N % 4 != 0) return 0;
+    if (B > kStreamMaxRows) return 0;
+    return stream_workspace_bytes(MODE_I8, B, N, ceil_div(K, 4));
+}
+
+extern "C" int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const void* scale,
+                                  int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
+                                  void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N, int64_t K,
+                                  void* workspace, size_t workspace_bytes, void* stream) {
+    const char* who = "bt_ternary_gemm_i8";
+    int rc = check_shape(who, Q, W_T, Y, y_dtype, B, N, K);
+    if (rc) return rc;
+    if (!s_x) {
+        set_error("%s: s_x is null", who);
+        return BT_ERR_INVALID;
+    }
+    if (K > kMaxKInt8) {
+        set_error("%s: K=%lld could overflow the int32 accumulators (limit %lld)", who, (long long)K,
+                  (long long)kMaxKInt8);
+        return BT_ERR_INVALID;
+    }
+    if (N % 4 != 0 || ((uintptr_t)W_T) % 16 != 0 || !fast_path_ok(Y, N, K) ||
+        (acc_out && ((uintptr_t)acc_out) % 16 != 0)) {
+        set_error("%s: needs N %% 4 == 0 and 16-byte aligned W_T / Y / acc_out (N=%lld)", who, (long long)N);
+        return BT_ERR_INVALID;
+    }
+    Epilogue epi;
+    rc = make_epilogue(who, scale, scale_dtype, scale_len, bias, bias_dtype, N, &epi);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    if (B <= kStreamMaxRows)
+        return launch_stream(MODE_I8, Q, 1, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, workspace,
+                             workspace_bytes, st);
+    return launch_gemm_i8(Q, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, st);
+}
+
+extern "C" size_t bt_tensor_core_workspace_bytes(int64_t B, int64_t N, int64_t K) {
+    if (B <= 0 || N <= 0 || K <= 0) return 0;
+    return align256((size_t)B * K) + align256((size_t)B * 4) + bt_gemm_i8_workspace_bytes(B, N, K);
+}
+
+extern "C" int bt_ternary_linear_tensor_core_forward(const void* X, int x_dtype, const uint8_t* W_T,
+                                                     const void* scale, int scale_dtype, int64_t scale_len,
+                                                     const void* bias, int bias_dtype, void* Y, int64_t B,
+                                                     int64_t N, int64_t K, void* workspace,
+                                                     size_t workspace_bytes, void* stream) {
+    const char* who = "bt_ternary_linear_tensor_core_forward";
+    int rc = check_shape(who, X, W_T, Y, x_dtype, B, N, K);
+    if (rc) return rc;
+    const size_t need = bt_tensor_core_workspace_bytes(B, N, K);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace) % 256 != 0) {
+        set_error("%s: workspace of %zu bytes (256-byte aligned) needed, %zu given", who, need, workspace_bytes);
+        return BT_ERR_WORKSPACE;
+    }
+    int8_t* Q = (int8_t*)workspace;
+    float* s_x = (float*)((uint8_t*)workspace + align256((size_t)B * K));
+    uint8_t* rest = (uint8_t*)s_x + align256((size_t)B * 4);
+    const size_t rest_bytes = workspace_bytes - (size_t)(rest - (uint8_t*)workspace);
+    rc = bt_act_quant_i8(X, x_dtype, B, K, Q, s_x, stream);
+    if (rc) return rc;
+    return bt_ternary_gemm_i8(Q, s_x, W_T, scale, scale_dtype, scale_len, bias, bias_dtype, Y, x_dtype, nullptr,
+                              B, N, K, rest, rest_bytes, stream);
+}

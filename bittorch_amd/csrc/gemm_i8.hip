@@ -1,0 +1,303 @@
+// Prefill-shape int8 x packed-ternary GEMM for gfx950 on the int8 matrix cores.
+//
+// Arithmetic restated from the reference's experimental tensor-core kernel with
+// the whole-row activation scale (csrc/kernels/ternary_gemm_tensor_core.cu:73-75,
+// :343-347, :439, :583-589, :652):
+//   acc_i32[m,n] = sum_k q[m,k] * 127*w[k,n]
+//   y[m,n]       = (float(acc) * s_x[m] / 127) * scale[n] + bias[n]
+// (the MFMA runs on +-1 weights; the accumulators are multiplied by 127 exactly
+// in the epilogue, which is the same integer).
+//
+// Tiling: a 256-thread workgroup owns a 128 x 256 output tile.  Its four waves
+// split the 256 columns (64 each) and all walk the same 128 rows, so every
+// weight is decoded exactly once per workgroup and the decode cost (about 0.7
+// VALU operations per weight) is shared by 128 rows of MFMA work.
+//   * Activations (int8, row-major [M,K]) go through LDS, double buffered, 128 k
+//     per stage, stored in MFMA operand order: slot (sub, mb, lane) is the 16
+//     bytes lane (i = lane%16, g = lane/16) feeds to v_mfma_i32_16x16x64_i8 for
+//     row block mb and k64 sub-step sub.
+//   * Weights never touch LDS: lane (j, g) of wave w loads one dword (four
+//     output columns nb + 64w + 4j .. +3) from each of the four rows
+//     kb + 4g .. 4g+3, transposes the 4x4 bytes and decodes them in registers
+//     into the B operands of four MFMAs (one per column).
+#include "bt_common.h"
+
+namespace bt {
+
+constexpr int G_BM = 128;
+constexpr int G_BN = 256;
+constexpr int G_BK = 128;           // k per LDS stage (two k64 MFMA sub-steps)
+constexpr int G_MB = G_BM / 16;     // 16-row blocks per tile
+constexpr int G_STAGE_BYTES = G_BM * G_BK;  // 16 KiB
+
+struct GemmParams {
+    const int8_t* Q;      // [M, K]
+    const float* s_x;     // [M]
+    const uint8_t* W_T;   // [Kb, N]
+    void* Y;              // [M, N]
+    int32_t* acc_out;     // optional [M, N]
+    Epilogue epi;
+    int64_t M, N, K, Kb;
+    int y_dtype;
+    int tiles_m, tiles_n;
+    int per_xcd;          // workgroups per XCD (grid = 8 * per_xcd)
+    int q_vec_ok;         // rows of Q are 16-byte aligned
+};
+
+__device__ __forceinline__ void store4(void* Y, int dt, int64_t idx, const float (&v)[4]) {
+    if (dt == BT_F32) {
+        *(float4*)((float*)Y + idx) = make_float4(v[0], v[1], v[2], v[3]);
+    } else {
+        uint16_t h[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) h[i] = (dt == BT_F16) ? f32_to_f16_bits(v[i]) : f32_to_bf16_bits(v[i]);
+        uint2 o;
+        o.x = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
+        o.y = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
+        *(uint2*)((uint16_t*)Y + idx) = o;
+    }
+}
+
+__global__ __launch_bounds__(256) void gemm_i8_kernel(GemmParams p) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * G_STAGE_BYTES];
+
+    // XCD-aware tile order: the 8 XCDs each take a contiguous run of tiles, and
+    // runs are walked in groups of four row tiles so that one XCD's L2 holds a
+    // compact block of activation rows and weight columns.
+    const int64_t lin = (int64_t)(blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
+    if (lin >= (int64_t)p.tiles_m * p.tiles_n) return;
+    constexpr int GM = 4;
+    const int64_t group = lin / (GM * p.tiles_n);
+    const int64_t first_m = group * GM;
+    const int gm = (p.tiles_m - first_m < GM) ? (int)(p.tiles_m - first_m) : GM;
+    const int64_t in_group = lin - group * GM * p.tiles_n;
+    const int tile_m = (int)(first_m + in_group % gm);
+    const int tile_n = (int)(in_group / gm);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int j = lane & 15;
+    const int g = lane >> 4;
+    const int64_t m0 = (int64_t)tile_m * G_BM;
+    const int64_t ncol = (int64_t)tile_n * G_BN + 64 * wave + 4 * j;
+    const bool col_ok = ncol < p.N;
+
+    // A staging role of this thread: one row, one k64 sub-step (64 bytes)
+    const int a_row = tid & (G_BM - 1);
+    const int a_sub = tid >> 7;
+    const int64_t a_m = m0 + a_row;
+    const bool a_ok = a_m < p.M;
+    const int8_t* a_src = p.Q + a_m * p.K;
+
+    uint4 a_reg[4];
+    uint32_t b_reg[2][4];
+
+    auto load_a = [&](int64_t k0) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const int64_t k = k0 + 64 * a_sub + 16 * c;
+            uint4 v = make_uint4(0u, 0u, 0u, 0u);
+            if (a_ok && k < p.K) {
+                if (p.q_vec_ok && k + 16 <= p.K) {
+                    v = *(const uint4*)(a_src + k);
+                } else {
+                    uint32_t d[4] = {0u, 0u, 0u, 0u};
+                    for (int e = 0; e < 16; e++)
+                        if (k + e < p.K) d[e >> 2] |= (uint32_t)(uint8_t)a_src[k + e] << (8 * (e & 3));
+                    v = make_uint4(d[0], d[1], d[2], d[3]);
+                }
+            }
+            a_reg[c] = v;
+        }
+    };
+    auto store_a = [&](int buf) {
+        uint8_t* base = lds + buf * G_STAGE_BYTES;
+        const int mb = a_row >> 4, i = a_row & 15;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            uint32_t t[4];
+            transpose4x4_bytes(a_reg[c].x, a_reg[c].y, a_reg[c].z, a_reg[c].w, t);
+            // slot (sub, mb, lane = c*16 + i)
+            *(uint4*)(base + ((size_t)((a_sub * G_MB + mb) * 64 + c * 16 + i) << 4)) = make_uint4(t[0], t[1], t[2], t[3]);
+        }
+    };
+    auto load_b = [&](int64_t k0) {
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int64_t kb = (k0 >> 2) + 16 * sub + 4 * g + r;
+                b_reg[sub][r] = (col_ok && kb < p.Kb) ? *(const uint32_t*)(p.W_T + kb * p.N + ncol) : 0u;
+            }
+        }
+    };
+
+    v4i acc[G_MB][4];
+#pragma unroll
+    for (int mb = 0; mb < G_MB; mb++)
+#pragma unroll
+        for (int t = 0; t < 4; t++) acc[mb][t] = v4i{0, 0, 0, 0};
+
+    const int nstages = (int)((p.K + G_BK - 1) / G_BK);
+    load_a(0);
+    load_b(0);
+    store_a(0);
+    __syncthreads();
+
+    for (int s = 0; s < nstages; s++) {
+        const int cur = s & 1;
+        uint32_t b_cur[2][4];
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) b_cur[sub][r] = b_reg[sub][r];
+        const bool more = (s + 1 < nstages);
+        if (more) {
+            load_a((int64_t)(s + 1) * G_BK);
+            load_b((int64_t)(s + 1) * G_BK);
+        }
+        const uint8_t* a_base = lds + cur * G_STAGE_BYTES;
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++) {
+            uint32_t G[4];
+            transpose4x4_bytes(b_cur[sub][0], b_cur[sub][1], b_cur[sub][2], b_cur[sub][3], G);
+            v4i b[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) b[t] = decode16_i8(G[t]);
+#pragma unroll
+            for (int mb = 0; mb < G_MB; mb++) {
+                const uint4 av = *(const uint4*)(a_base + ((size_t)((sub * G_MB + mb) * 64 + lane) << 4));
+                const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+#pragma unroll
+                for (int t = 0; t < 4; t++)
+                    acc[mb][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[t], acc[mb][t], 0, 0, 0);
+            }
+        }
+        if (more) store_a(cur ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: lane (j, g) holds rows 16mb + 4g + r, columns ncol .. ncol+3 --------
+    if (!col_ok) return;
+    float ws[4], bs[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        ws[t] = epi_scale(p.epi, ncol + t);
+        bs[t] = epi_bias(p.epi, ncol + t);
+    }
+#pragma unroll
+    for (int mb = 0; mb < G_MB; mb++) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int64_t m = m0 + 16 * mb + 4 * g + r;
+            if (m >= p.M) continue;
+            const float sx = p.s_x[m];
+            float y[4];
+            int32_t a127[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                a127[t] = acc[mb][t][r] * 127;
+                y[t] = epi_int8(a127[t], sx, ws[t], bs[t]);
+            }
+            store4(p.Y, p.y_dtype, m * p.N + ncol, y);
+            if (p.acc_out) *(int4*)(p.acc_out + m * p.N + ncol) = make_int4(a127[0], a127[1], a127[2], a127[3]);
+        }
+    }
+}
+
+// Per-row int8 activation quantizer: one wave per row, two passes over the row
+// (the second pass hits in cache; a row is at most a few tens of KiB).
+template <int DT>
+__global__ __launch_bounds__(256) void act_quant_kernel(const void* __restrict__ X, int64_t B, int64_t K,
+                                                        int8_t* __restrict__ Q, float* __restrict__ s_x) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= B) return;
+    const int64_t base = row * K;
+    constexpr int ES = (DT == BT_F32) ? 4 : 2;
+    const bool vec_ok = (K % 8 == 0) && (((uintptr_t)X) % 16 == 0) && (((uintptr_t)Q) % 8 == 0);
+
+    auto load8 = [&](int64_t k, float (&v)[8]) {
+        if (vec_ok) {
+            if constexpr (DT == BT_F32) {
+                const float4 a = *(const float4*)((const float*)X + base + k);
+                const float4 b = *(const float4*)((const float*)X + base + k + 4);
+                v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+                v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+            } else {
+                const uint4 u = *(const uint4*)((const uint16_t*)X + base + k);
+                const uint32_t d[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const uint16_t h = (uint16_t)(d[e >> 1] >> (16 * (e & 1)));
+                    v[e] = (DT == BT_F16) ? f16_bits_to_f32(h) : bf16_bits_to_f32(h);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[e] = (k + e < K) ? load_elem<DT>(X, base + k + e) : 0.0f;
+        }
+    };
+    (void)ES;
+
+    float amax = 0.0f;
+    for (int64_t k = (int64_t)lane * 8; k < K; k += 512) {
+        float v[8];
+        load8(k, v);
+#pragma unroll
+        for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(v[e]));
+    }
+    amax = wave_max(amax);
+    const float s = (amax > 1e-6f) ? __fdiv_rn(amax, 127.0f) : 1.0f;
+    const float inv = __fdiv_rn(1.0f, s);
+    if (lane == 0) s_x[row] = s;
+
+    for (int64_t k = (int64_t)lane * 8; k < K; k += 512) {
+        float v[8];
+        load8(k, v);
+        uint32_t lo = 0, hi = 0;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            float r = roundf(__fmul_rn(v[e], inv));
+            r = fmaxf(-127.0f, fminf(127.0f, r));
+            const uint32_t byte = (uint32_t)(uint8_t)(int8_t)(int)r;
+            if (e < 4) lo |= byte << (8 * e);
+            else hi |= byte << (8 * (e - 4));
+        }
+        if (vec_ok) {
+            *(uint2*)(Q + base + k) = make_uint2(lo, hi);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+                if (k + e < K) Q[base + k + e] = (int8_t)(((e < 4 ? lo : hi) >> (8 * (e & 3))) & 0xff);
+        }
+    }
+}
+
+int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x, hipStream_t st) {
+    const dim3 grid((unsigned)ceil_div(B, 4)), block(256);
+    if (x_dtype == BT_F32) hipLaunchKernelGGL(act_quant_kernel<BT_F32>, grid, block, 0, st, X, B, K, Q, s_x);
+    else if (x_dtype == BT_F16) hipLaunchKernelGGL(act_quant_kernel<BT_F16>, grid, block, 0, st, X, B, K, Q, s_x);
+    else hipLaunchKernelGGL(act_quant_kernel<BT_BF16>, grid, block, 0, st, X, B, K, Q, s_x);
+    return check_launch("bt_act_quant_i8");
+}
+
+bool gemm_i8_supported(int64_t N, const void* W_T) { return N % 4 == 0 && ((uintptr_t)W_T) % 4 == 0; }
+
+int launch_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const Epilogue& epi, void* Y,
+                   int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st) {
+    GemmParams p;
+    p.Q = Q; p.s_x = s_x; p.W_T = W_T; p.Y = Y; p.acc_out = acc_out; p.epi = epi;
+    p.M = M; p.N = N; p.K = K; p.Kb = ceil_div(K, 4);
+    p.y_dtype = y_dtype;
+    p.tiles_m = (int)ceil_div(M, G_BM);
+    p.tiles_n = (int)ceil_div(N, G_BN);
+    const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
+    p.per_xcd = (int)ceil_div(total, 8);
+    p.q_vec_ok = (((uintptr_t)Q) % 16 == 0) && (K % 16 == 0);
+    hipLaunchKernelGGL(gemm_i8_kernel, dim3((unsigned)(p.per_xcd * 8)), dim3(256), 0, st, p);
+    return check_launch("bt_ternary_gemm_i8");
+}
+
+}  // namespace bt

@@ -1,0 +1,178 @@
+// Shape-generic kernels: any N, K, B and fp32/fp16/bf16 activations.  They back
+// the matrix-core kernels for shapes or alignments those do not take, the
+// dense-int8-weight entry point, and the packed -> dense conversion.
+// fp32 accumulation runs over k in ascending order, exactly the order of the
+// reference kernels (csrc/kernels/ternary_gemm.cu:59-63,
+// csrc/kernels/ternary_gemm_production.cu:126-133).
+#include "bt_common.h"
+
+namespace bt {
+
+// Y[b,n] = (sum_k x[b,k] * decode(W_T[k/4,n], k%4)) * scale[n] + bias[n]
+// One thread per output column, 256 columns per workgroup, grid.y = batch row.
+template <int XDT>
+__global__ __launch_bounds__(256) void packed_generic_kernel(const void* __restrict__ X,
+                                                             const uint8_t* __restrict__ W_T, Epilogue epi,
+                                                             void* __restrict__ Y, int64_t N, int64_t K,
+                                                             int64_t Kb) {
+    const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t b = blockIdx.y;
+    if (n >= N) return;
+    const int64_t xrow = b * K;
+    float acc = 0.0f;
+    for (int64_t kb = 0; kb < Kb; kb++) {
+        const uint32_t byte = W_T[kb * N + n];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int64_t k = 4 * kb + i;
+            if (k < K) {
+                const float w = (float)decode2((byte >> (2 * i)) & 3u);
+                acc = __fadd_rn(acc, __fmul_rn(load_elem<XDT>(X, xrow + k), w));
+            }
+        }
+    }
+    store_elem<XDT>(Y, b * N + n, epi_float(acc, epi_scale(epi, n), epi_bias(epi, n)));
+}
+
+int launch_packed_generic(const void* X, int x_dtype, const uint8_t* W_T, const Epilogue& epi, void* Y,
+                          int64_t B, int64_t N, int64_t K, hipStream_t st) {
+    const int64_t Kb = ceil_div(K, 4);
+    const dim3 grid((unsigned)ceil_div(N, 256), (unsigned)B), block(256);
+    if (B > 65535) {
+        set_error("packed forward (generic kernel): batch %lld exceeds 65535 rows", (long long)B);
+        return BT_ERR_INVALID;
+    }
+    if (x_dtype == BT_F32)
+        hipLaunchKernelGGL(packed_generic_kernel<BT_F32>, grid, block, 0, st, X, W_T, epi, Y, N, K, Kb);
+    else if (x_dtype == BT_F16)
+        hipLaunchKernelGGL(packed_generic_kernel<BT_F16>, grid, block, 0, st, X, W_T, epi, Y, N, K, Kb);
+    else
+        hipLaunchKernelGGL(packed_generic_kernel<BT_BF16>, grid, block, 0, st, X, W_T, epi, Y, N, K, Kb);
+    return check_launch("packed_generic");
+}
+
+// Dense int8 weights W [N,K]: 64 columns x 16 batch rows per workgroup, K in
+// tiles of 64 staged through LDS (weights transposed there so that the k loop
+// reads conflict-free).
+template <int XDT>
+__global__ __launch_bounds__(256) void unpacked_kernel(const void* __restrict__ X, const int8_t* __restrict__ W,
+                                                       Epilogue epi, void* __restrict__ Y, int64_t B, int64_t N,
+                                                       int64_t K) {
+    __shared__ float xs[16][64];
+    __shared__ int8_t ws[64][68];  // [k][n], padded
+    const int nl = threadIdx.x & 63;
+    const int bs = threadIdx.x >> 6;  // rows bs*4 .. bs*4+3
+    const int64_t n0 = (int64_t)blockIdx.x * 64;
+    const int64_t b0 = (int64_t)blockIdx.y * 16;
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int64_t k0 = 0; k0 < K; k0 += 64) {
+        for (int idx = threadIdx.x; idx < 16 * 64; idx += 256) {
+            const int r = idx >> 6, kk = idx & 63;
+            const int64_t b = b0 + r, k = k0 + kk;
+            xs[r][kk] = (b < B && k < K) ? load_elem<XDT>(X, b * K + k) : 0.0f;
+        }
+        for (int idx = threadIdx.x; idx < 64 * 64; idx += 256) {
+            const int r = idx >> 6, kk = idx & 63;  // r: column n, kk: k (contiguous in memory)
+            const int64_t n = n0 + r, k = k0 + kk;
+            ws[kk][r] = (n < N && k < K) ? W[n * K + k] : (int8_t)0;
+        }
+        __syncthreads();
+        const int klim = (K - k0 < 64) ? (int)(K - k0) : 64;
+        for (int kk = 0; kk < klim; kk++) {
+            const float w = (float)ws[kk][nl];
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[r] = __fadd_rn(acc[r], __fmul_rn(xs[bs * 4 + r][kk], w));
+        }
+        __syncthreads();
+    }
+    const int64_t n = n0 + nl;
+    if (n >= N) return;
+    const float s = epi_scale(epi, n);
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int64_t b = b0 + bs * 4 + r;
+        if (b >= B) continue;
+        // acc *= scale; acc += bias (only when a bias is given)
+        float v = __fmul_rn(acc[r], s);
+        if (epi.bias) v = __fadd_rn(v, epi_bias(epi, n));
+        store_elem<XDT>(Y, b * N + n, v);
+    }
+}
+
+int launch_unpacked(const void* X, int x_dtype, const int8_t* W, const Epilogue& epi, void* Y, int64_t B,
+                    int64_t N, int64_t K, hipStream_t st) {
+    const dim3 grid((unsigned)ceil_div(N, 64), (unsigned)ceil_div(B, 16)), block(256);
+    if (ceil_div(B, 16) > 65535) {
+        set_error("bt_ternary_linear_forward: batch %lld too large", (long long)B);
+        return BT_ERR_INVALID;
+    }
+    if (x_dtype == BT_F32) hipLaunchKernelGGL(unpacked_kernel<BT_F32>, grid, block, 0, st, X, W, epi, Y, B, N, K);
+    else if (x_dtype == BT_F16) hipLaunchKernelGGL(unpacked_kernel<BT_F16>, grid, block, 0, st, X, W, epi, Y, B, N, K);
+    else hipLaunchKernelGGL(unpacked_kernel<BT_BF16>, grid, block, 0, st, X, W, epi, Y, B, N, K);
+    return check_launch("bt_ternary_linear_forward");
+}
+
+// out[n, k] = decode(W_T[k/4, n]) * scale[n]   (scale == nullptr: plain decode)
+// Tile: 64 columns x 16 kb rows (64 k) through LDS for the transpose.
+template <int ODT>
+__global__ __launch_bounds__(256) void unpack_dequant_kernel(const uint8_t* __restrict__ W_T,
+                                                             const float* __restrict__ scale, int scale_bcast,
+                                                             void* __restrict__ out, int64_t N, int64_t K,
+                                                             int64_t Kb) {
+    __shared__ uint8_t tile[16][65];
+    const int64_t n0 = (int64_t)blockIdx.x * 64;
+    const int64_t kb0 = (int64_t)blockIdx.y * 16;
+    for (int idx = threadIdx.x; idx < 16 * 64; idx += 256) {
+        const int r = idx >> 6, c = idx & 63;
+        const int64_t kb = kb0 + r, n = n0 + c;
+        tile[r][c] = (kb < Kb && n < N) ? W_T[kb * N + n] : (uint8_t)0;
+    }
+    __syncthreads();
+    const int c = threadIdx.x >> 2;     // column within the tile
+    const int part = threadIdx.x & 3;   // kb rows part*4 .. part*4+3
+    const int64_t n = n0 + c;
+    if (n >= N) return;
+    const float s = scale ? scale[scale_bcast ? 0 : n] : 1.0f;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const uint32_t byte = tile[part * 4 + r][c];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int64_t k = 4 * (kb0 + part * 4 + r) + i;
+            if (k < K) {
+                const float w = (float)decode2((byte >> (2 * i)) & 3u);
+                if constexpr (ODT == 3) ((int8_t*)out)[n * K + k] = (int8_t)w;
+                else store_elem<ODT>(out, n * K + k, __fmul_rn(w, s));
+            }
+        }
+    }
+}
+
+}  // namespace bt
+
+extern "C" int bt_unpack_dequant(const uint8_t* W_T, const float* scale, int64_t scale_len, void* out,
+                                 int out_dtype, int64_t N, int64_t K, void* stream) {
+    using namespace bt;
+    if (!W_T || !out || N <= 0 || K <= 0) {
+        set_error("bt_unpack_dequant: null pointer or empty shape");
+        return BT_ERR_INVALID;
+    }
+    if (scale && scale_len != N && scale_len != 1) {
+        set_error("bt_unpack_dequant: scale has %lld entries, expected %lld or 1", (long long)scale_len, (long long)N);
+        return BT_ERR_INVALID;
+    }
+    const int64_t Kb = ceil_div(K, 4);
+    const dim3 grid((unsigned)ceil_div(N, 64), (unsigned)ceil_div(Kb, 16)), block(256);
+    hipStream_t st = (hipStream_t)stream;
+    const int bc = (scale_len == 1) ? 1 : 0;
+    switch (out_dtype) {
+        case BT_F32: hipLaunchKernelGGL(unpack_dequant_kernel<BT_F32>, grid, block, 0, st, W_T, scale, bc, out, N, K, Kb); break;
+        case BT_F16: hipLaunchKernelGGL(unpack_dequant_kernel<BT_F16>, grid, block, 0, st, W_T, scale, bc, out, N, K, Kb); break;
+        case BT_BF16: hipLaunchKernelGGL(unpack_dequant_kernel<BT_BF16>, grid, block, 0, st, W_T, scale, bc, out, N, K, Kb); break;
+        case 3: hipLaunchKernelGGL(unpack_dequant_kernel<3>, grid, block, 0, st, W_T, scale, bc, out, N, K, Kb); break;
+        default:
+            set_error("bt_unpack_dequant: unsupported output dtype %d", out_dtype);
+            return BT_ERR_INVALID;
+    }
+    return check_launch("bt_unpack_dequant");
+}

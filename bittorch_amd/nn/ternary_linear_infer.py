@@ -1,0 +1,82 @@
+"""``TernaryLinearInference``: deployment layer that holds only packed weights.
+
+API mirror of ``bittorch/nn/ternary_linear_infer.py:22-193``.  Buffers:
+``weight_packed`` uint8 ``[ceil(K/4), N]`` (transposed layout), ``scale`` ``[N]``,
+optional ``bias``; nothing is trainable.  GPU inputs go to the packed HIP
+kernels; CPU inputs unpack and use ``F.linear`` as the reference does.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch import Tensor
+
+from ..quant.ternary import ternary_quantize
+from ..quant.ternary_packed import pack_ternary_transposed, unpack_ternary_transposed
+
+
+class TernaryLinearInference(nn.Module):
+    def __init__(self, in_features: int, out_features: int, weight_packed: Tensor, scale: Tensor,
+                 bias: Optional[Tensor] = None):
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.register_buffer("weight_packed", weight_packed)
+        self.register_buffer("scale", scale)
+        self.register_buffer("bias", bias)
+        self.requires_grad_(False)
+
+    def forward(self, x: Tensor) -> Tensor:
+        if x.is_cuda:
+            from ..ops.ternary_linear_packed import ternary_linear_packed_forward
+            return ternary_linear_packed_forward(x, self.weight_packed, self.scale,
+                                                 self.in_features, self.bias)
+        # CPU (reference :98-104): unpack, fold the scale in, dense product
+        w = unpack_ternary_transposed(self.weight_packed, self.in_features).to(x.dtype)
+        w = w * self.scale.unsqueeze(1).to(x.dtype)
+        return F.linear(x, w, self.bias)
+
+    def extra_repr(self) -> str:
+        dense = 4 * self.out_features * self.in_features
+        ratio = dense / (self.weight_packed.numel() + 2 * self.scale.numel())
+        return (f"in_features={self.in_features}, out_features={self.out_features}, "
+                f"bias={self.bias is not None}, packed_bytes={self.weight_packed.numel()}, "
+                f"reduction={ratio:.1f}x")
+
+    @classmethod
+    def from_unpacked(cls, w_tern: Tensor, scale: Tensor,
+                      bias: Optional[Tensor] = None) -> "TernaryLinearInference":
+        """Pack already-quantized ``w_tern`` ``(N, K)`` (reference ``:119-148``)."""
+        packed_t, in_features = pack_ternary_transposed(w_tern)
+        return cls(in_features, w_tern.shape[0], packed_t, scale, bias)
+
+    @property
+    def packed_size_bytes(self) -> int:
+        return self.weight_packed.numel()
+
+    @property
+    def effective_bits_per_weight(self) -> float:
+        bits = 8 * self.weight_packed.numel() + 16 * self.scale.numel()
+        return bits / (self.out_features * self.in_features)
+
+
+def create_ternary_linear_inference(in_features: int, out_features: int, weight: Tensor,
+                                    bias: Optional[Tensor] = None,
+                                    threshold_factor: float = 0.05) -> TernaryLinearInference:
+    """Quantize + pack full-precision ``weight`` into an inference layer (reference ``:163-193``).
+
+    GPU weights go through the fused quantize+pack kernel, whose bytes and scales
+    equal those of the torch path bit for bit.
+    """
+    if weight.is_cuda and weight.dtype in (torch.float32, torch.float16, torch.bfloat16):
+        from .ternary_linear import _cuda_kernel_available
+        if _cuda_kernel_available():
+            from .. import _C
+            packed, scale, _ = _C.ternary_quantize_pack(weight, threshold_factor, True)
+            return TernaryLinearInference(in_features, out_features, packed, scale, bias)
+    w_tern, scale = ternary_quantize(weight, threshold_factor=threshold_factor)
+    return TernaryLinearInference.from_unpacked(w_tern, scale, bias)

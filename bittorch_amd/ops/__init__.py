@@ -1,0 +1,13 @@
+"""Functional operations (same names as ``bittorch.ops``)."""
+
+from .ternary_linear import ternary_linear, ternary_linear_forward_cuda
+from .ternary_linear_packed import has_packed_cuda_support, ternary_linear_packed_forward
+from .ternary_linear_tensor_core import ternary_linear_tensor_core_forward
+
+__all__ = [
+    "ternary_linear",
+    "ternary_linear_forward_cuda",
+    "ternary_linear_packed_forward",
+    "has_packed_cuda_support",
+    "ternary_linear_tensor_core_forward",
+]

@@ -1,0 +1,145 @@
+/*
+ * C ABI of libbittorch_hip.so: the MI355X (gfx950) ternary-linear backend.
+ *
+ * Plain pointers and sizes only; no C++ or torch types cross this boundary.
+ * All pointers except the optional ones are DEVICE pointers owned by the
+ * caller; the library never allocates or frees device memory and keeps no
+ * mutable global state, so calls on different streams are independent.
+ * Kernels are enqueued on `stream` (a hipStream_t passed as void*; NULL is
+ * the default stream) and the call returns without synchronising.
+ *
+ * Every function returns 0 on success or a negative bt_status; the text of
+ * the last failure on the calling thread is available from bt_last_error().
+ *
+ * Entry points replace the reference's pybind11 module `bittorch._C`
+ * (csrc/bindings/bittorch_bindings.cpp:34-88) and the host dispatch behind it
+ * (csrc/core/dispatch.cpp:52-142); each declaration cites what it replaces.
+ */
+#ifndef BITTORCH_HIP_H
+#define BITTORCH_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BT_ABI_VERSION 1
+
+/* element types of activations / scales / biases / outputs */
+typedef enum { BT_F32 = 0, BT_F16 = 1, BT_BF16 = 2 } bt_dtype;
+
+typedef enum {
+    BT_OK = 0,
+    BT_ERR_INVALID = -1,   /* bad shape / dtype / null pointer */
+    BT_ERR_WORKSPACE = -2, /* workspace too small */
+    BT_ERR_LAUNCH = -3     /* HIP reported a launch error */
+} bt_status;
+
+/* ABI version of the loaded library (BT_ABI_VERSION at build time). */
+int bt_abi_version(void);
+
+/* Message of the last failure on this thread ("" if none). */
+const char* bt_last_error(void);
+
+/*
+ * Fused ternary quantize + 2-bit pack.
+ * Replaces the torch op chains of bittorch/quant/ternary.py:122-142
+ * (absmax scale, threshold, sign) and bittorch/quant/ternary_packed.py:50-73,
+ * :202-206 (encode, pack, transpose) with one pass over the master weights.
+ *
+ *   W          [N,K] row-major master weights of type w_dtype
+ *   packed_T   [ceil(K/4), N] uint8 out, byte [kb,n] = W[n,4kb..4kb+3] codes
+ *              (+1 -> 1, -1 -> 2, 0 -> 0; element i in bits 2i..2i+1)
+ *   scale      fp32 out: [N] row absmax (per_channel != 0) or [1] tensor absmax,
+ *              floored at 1e-8 rounded to w_dtype
+ *   w_tern     optional [N,K] int8 out with the ternary values (may be NULL)
+ *   packed_T may be NULL if only scale / w_tern are wanted.
+ */
+int bt_quantize_pack(const void* W, int w_dtype, int64_t N, int64_t K, double threshold_factor,
+                     int per_channel, uint8_t* packed_T, float* scale, int8_t* w_tern,
+                     void* stream);
+
+/*
+ * Unpacked-weight forward: Y = X @ (W_tern * scale).T + bias, fp32 accumulate.
+ * Replaces bittorch._C.ternary_linear_forward (bittorch_bindings.cpp:41-46,
+ * dispatch.cpp:52-87, csrc/kernels/ternary_gemm.cu:206-279).
+ *   X [B,K] x_dtype, W_tern [N,K] int8, Y [B,N] x_dtype.
+ *   scale: scale_len entries (N, or 1 = broadcast) of scale_dtype.
+ *   bias: NULL or N entries of bias_dtype.
+ */
+int bt_ternary_linear_forward(const void* X, int x_dtype, const int8_t* W_tern, const void* scale,
+                              int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
+                              void* Y, int64_t B, int64_t N, int64_t K, void* stream);
+
+/*
+ * Packed-weight forward with fp32 accumulation (decode GEMV / small batch / any B).
+ * Replaces bittorch._C.ternary_linear_packed_forward (bittorch_bindings.cpp:48-63,
+ * dispatch.cpp:105-142, csrc/kernels/ternary_gemm_production.cu:286-362).
+ *   X [B,K] x_dtype; W_T [ceil(K/4),N] uint8; Y [B,N] x_dtype.
+ *   workspace: scratch for split-K partial sums, at least
+ *   bt_packed_forward_workspace_bytes(B,N,K,x_dtype) bytes (may be NULL if that is 0).
+ */
+size_t bt_packed_forward_workspace_bytes(int64_t B, int64_t N, int64_t K, int x_dtype);
+int bt_ternary_linear_packed_forward(const void* X, int x_dtype, const uint8_t* W_T,
+                                     const void* scale, int scale_dtype, int64_t scale_len,
+                                     const void* bias, int bias_dtype, void* Y, int64_t B,
+                                     int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
+                                     void* stream);
+
+/*
+ * Per-row int8 activation quantizer (whole-row absmax scale).
+ * Restates the activation stage of kernel_v2_tensor_core
+ * (csrc/kernels/ternary_gemm_tensor_core.cu:431-459, :343-347):
+ *   s_x[b] = amax > 1e-6 ? amax/127 : 1;  Q = clamp(roundf(X * (1/s_x)), -127, 127)
+ *   X [B,K] x_dtype -> Q [B,K] int8, s_x [B] fp32.
+ */
+int bt_act_quant_i8(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x,
+                    void* stream);
+
+/*
+ * int8 x packed-ternary GEMM on the matrix cores, int32 accumulators.
+ * Restates the MMA stage and epilogue of kernel_v2_tensor_core
+ * (ternary_gemm_tensor_core.cu:583-589, :652): weights decode to +-127,
+ *   y = (float(acc) * s_x[b] / 127.0f) * scale[n] + bias[n].
+ *   Q [B,K] int8, s_x [B] fp32, W_T [ceil(K/4),N] uint8, Y [B,N] y_dtype.
+ *   acc_out: optional [B,N] int32 copy of the raw accumulators (may be NULL).
+ *   workspace: at least bt_gemm_i8_workspace_bytes(B,N,K) bytes.
+ */
+size_t bt_gemm_i8_workspace_bytes(int64_t B, int64_t N, int64_t K);
+int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const void* scale,
+                       int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
+                       void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N, int64_t K,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Matrix-core forward from float activations: bt_act_quant_i8 followed by
+ * bt_ternary_gemm_i8.  Replaces bittorch._C.ternary_linear_tensor_core_forward
+ * (bittorch_bindings.cpp:65-87, ternary_gemm_tensor_core.cu:663-727) for
+ * version == 2; version == 1 (the reference's float-compute validation kernel,
+ * :120-271) is served by bt_ternary_linear_packed_forward.
+ *   workspace: at least bt_tensor_core_workspace_bytes(B,N,K) bytes; holds Q, s_x and
+ *   the GEMM's own scratch.
+ */
+size_t bt_tensor_core_workspace_bytes(int64_t B, int64_t N, int64_t K);
+int bt_ternary_linear_tensor_core_forward(const void* X, int x_dtype, const uint8_t* W_T,
+                                          const void* scale, int scale_dtype, int64_t scale_len,
+                                          const void* bias, int bias_dtype, void* Y, int64_t B,
+                                          int64_t N, int64_t K, void* workspace,
+                                          size_t workspace_bytes, void* stream);
+
+/*
+ * Packed weights -> dense ternary or effective weights, for the training
+ * backward (grad_x = grad_y @ (w_tern * scale)) without keeping a dense copy
+ * alive between forward and backward (the reference saves one,
+ * bittorch/nn/ternary_linear_cuda.py:62-66).
+ *   out [N,K] of out_dtype = decode(W_T) * scale[n]   (scale NULL -> plain decode)
+ */
+int bt_unpack_dequant(const uint8_t* W_T, const float* scale, int64_t scale_len, void* out,
+                      int out_dtype, int64_t N, int64_t K, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BITTORCH_HIP_H */

@@ -1,0 +1,332 @@
+/*
+ * CPU oracle for the ternary-linear hot path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This file restates, in plain scalar C, the arithmetic of the reference
+ * implementation so that the HIP kernels can be diffed against it.  It is
+ * never linked into, imported by or called from the shipped package; only the
+ * tests, the smoke check and the benchmark's cpu_baseline leg may use it.
+ *
+ * Every function names the reference lines it follows (paths relative to the
+ * reference checkout).  Parity status of each function:
+ *
+ *   bto_quantize        pinned   (reference-held known answers, torch CPU ops
+ *                                 executing the same formula, brute force)
+ *   bto_pack / unpack   pinned   (reference-held byte known answers 0x49, 85,
+ *                                 170, 0; round trip; K%4 != 0 padding)
+ *   bto_linear_packed   pinned   (textbook x @ (w*s).T + b in float64, all-zero
+ *                                 and all-ones weights, the reference's JS
+ *                                 known-answer vectors)
+ *   bto_linear_unpacked pinned   (same checks as bto_linear_packed)
+ *   bto_act_quant_i8    parity unpinned by the reference (no reference test
+ *   bto_gemm_i8         touches the int8 path); pinned here only by brute
+ *                       force on tiny inputs, exact integer identities and
+ *                       agreement with the float path inside the int8
+ *                       quantisation error bound.
+ *
+ * Build: gcc -O2 -fPIC -shared -ffp-contract=off -fopenmp (see Makefile).
+ * -ffp-contract=off keeps every multiply and add separately rounded, which is
+ * what the comments below mean by "one fp32 multiply, then one fp32 add".
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stddef.h>
+#include <string.h>
+
+/* dtype tags shared with include/bittorch_hip.h */
+enum { BTO_F32 = 0, BTO_F16 = 1, BTO_BF16 = 2 };
+
+/* ---- rounding helpers: float -> (fp16|bf16) -> float, round-nearest-even -- */
+
+static float round_to_bf16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return f; /* NaN */
+    uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7fffu + lsb;
+    u &= 0xffff0000u;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+static float round_to_f16(float f) {
+    /* IEEE binary16 round-to-nearest-even, done by hand (no _Float16 in gcc 11/x86):
+     * scale into the half grid with exact power-of-two multiplies so that the
+     * fp32 adder performs the rounding, including the subnormal range. */
+    if (!(fabsf(f) <= 3.4e38f)) return f;          /* NaN / Inf pass through */
+    if (fabsf(f) >= 65520.0f) return copysignf(INFINITY, f);
+    float a = fabsf(f);
+    float r;
+    if (a < 6.103515625e-05f) {
+        /* subnormal half: multiples of 2^-24 */
+        const float magic = 12582912.0f; /* 1.5 * 2^23: adds round to integer, RNE */
+        float t = a * 16777216.0f;       /* / 2^-24, exact */
+        t = (t + magic) - magic;
+        r = t * 5.9604644775390625e-08f; /* * 2^-24, exact */
+    } else {
+        /* normal half: keep 11 significant bits */
+        uint32_t u;
+        memcpy(&u, &a, 4);
+        uint32_t lsb = (u >> 13) & 1u;
+        u += 0xfffu + lsb;
+        u &= 0xffffe000u;
+        memcpy(&r, &u, 4);
+    }
+    return copysignf(r, f);
+}
+
+static float round_to_dtype(float f, int dtype) {
+    if (dtype == BTO_F16) return round_to_f16(f);
+    if (dtype == BTO_BF16) return round_to_bf16(f);
+    return f;
+}
+
+/* exported so tests can check the helpers against torch's casts */
+float bto_round_to_dtype(float f, int dtype) { return round_to_dtype(f, dtype); }
+
+/*
+ * Ternary quantizer.  Follows bittorch/quant/ternary.py:100-150.
+ *
+ *   per_channel: scale[n] = max_k |W[n,k]|, clamped below at 1e-8   (:122-127)
+ *   per tensor : scale    = max_{n,k} |W[n,k]|, clamped             (:130-131)
+ *   threshold  = threshold_factor * scale                            (:134)
+ *   w_tern     = sign(W) where |W| > threshold (strict), else 0     (:137-142)
+ *
+ * W holds the master weights already widened to float; `dtype` says which
+ * type the reference tensor had, because torch evaluates `0.05 * scale` and
+ * the clamp in float and then rounds the result back to that type.  The
+ * Python scalar threshold_factor reaches the multiply as a float
+ * (`(float)0.05`), so the threshold is fl(tf_f32 * scale) rounded to dtype.
+ *
+ * scale has N entries (per_channel) or 1 entry.  w_tern may be NULL.
+ */
+void bto_quantize(const float* W, int64_t N, int64_t K, double threshold_factor,
+                  int per_channel, int dtype, int8_t* w_tern, float* scale) {
+    const float tf = (float)threshold_factor;
+    const float clamp_min = round_to_dtype(1e-8f, dtype);
+    float gmax = 0.0f;
+    if (!per_channel) {
+        for (int64_t i = 0; i < N * K; i++) {
+            float a = fabsf(W[i]);
+            if (a > gmax) gmax = a;
+        }
+        if (gmax < clamp_min) gmax = clamp_min;
+        scale[0] = gmax;
+    }
+    for (int64_t n = 0; n < N; n++) {
+        const float* row = W + n * K;
+        float s;
+        if (per_channel) {
+            s = 0.0f;
+            for (int64_t k = 0; k < K; k++) {
+                float a = fabsf(row[k]);
+                if (a > s) s = a;
+            }
+            if (s < clamp_min) s = clamp_min;
+            scale[n] = s;
+        } else {
+            s = gmax;
+        }
+        const float thr = round_to_dtype(tf * s, dtype);
+        if (w_tern) {
+            for (int64_t k = 0; k < K; k++) {
+                float w = row[k];
+                int8_t t = 0;
+                if (fabsf(w) > thr) t = (w > 0.0f) ? 1 : -1;
+                w_tern[n * K + k] = t;
+            }
+        }
+    }
+}
+
+/*
+ * 2-bit codec.  Follows bittorch/quant/ternary_packed.py:22-75.
+ *   code: +1 -> 1, -1 -> 2, 0 -> 0                                   (:59-61)
+ *   byte = c0 | c1<<2 | c2<<4 | c3<<6, c_i = element k = 4*kb + i    (:68-73)
+ *   K is zero-padded up to a multiple of four                        (:51-55)
+ * packed is [N, Kb] row-major, Kb = ceil(K/4).
+ */
+void bto_pack(const int8_t* w_tern, int64_t N, int64_t K, uint8_t* packed) {
+    const int64_t Kb = (K + 3) / 4;
+    for (int64_t n = 0; n < N; n++) {
+        for (int64_t kb = 0; kb < Kb; kb++) {
+            unsigned byte = 0;
+            for (int i = 0; i < 4; i++) {
+                int64_t k = 4 * kb + i;
+                int8_t w = (k < K) ? w_tern[n * K + k] : 0;
+                unsigned c = (w == 1) ? 1u : (w == -1) ? 2u : 0u;
+                byte |= c << (2 * i);
+            }
+            packed[n * Kb + kb] = (uint8_t)byte;
+        }
+    }
+}
+
+/*
+ * Transposed layout.  Follows bittorch/quant/ternary_packed.py:174-206:
+ * packed_T = pack_ternary(w).T.contiguous(), shape [Kb, N]; byte [kb, n]
+ * holds W[n, 4kb .. 4kb+3].
+ */
+void bto_pack_transposed(const int8_t* w_tern, int64_t N, int64_t K, uint8_t* packed_T) {
+    const int64_t Kb = (K + 3) / 4;
+    for (int64_t n = 0; n < N; n++) {
+        for (int64_t kb = 0; kb < Kb; kb++) {
+            unsigned byte = 0;
+            for (int i = 0; i < 4; i++) {
+                int64_t k = 4 * kb + i;
+                int8_t w = (k < K) ? w_tern[n * K + k] : 0;
+                unsigned c = (w == 1) ? 1u : (w == -1) ? 2u : 0u;
+                byte |= c << (2 * i);
+            }
+            packed_T[kb * N + n] = (uint8_t)byte;
+        }
+    }
+}
+
+/* code -> value; 3 ("reserved") decodes to 0.
+ * bittorch/quant/ternary_packed.py:112-115,
+ * csrc/kernels/ternary_gemm_production.cu:37-39 */
+static inline int decode2(unsigned code) { return (int)(code == 1u) - (int)(code == 2u); }
+
+/* Follows bittorch/quant/ternary_packed.py:78-120 (slices the K padding off). */
+void bto_unpack(const uint8_t* packed, int64_t N, int64_t K, int8_t* w_tern) {
+    const int64_t Kb = (K + 3) / 4;
+    for (int64_t n = 0; n < N; n++)
+        for (int64_t k = 0; k < K; k++)
+            w_tern[n * K + k] = (int8_t)decode2((packed[n * Kb + k / 4] >> (2 * (k % 4))) & 3u);
+}
+
+/* Follows bittorch/quant/ternary_packed.py:209-223. */
+void bto_unpack_transposed(const uint8_t* packed_T, int64_t N, int64_t K, int8_t* w_tern) {
+    for (int64_t n = 0; n < N; n++)
+        for (int64_t k = 0; k < K; k++)
+            w_tern[n * K + k] = (int8_t)decode2((packed_T[(k / 4) * N + n] >> (2 * (k % 4))) & 3u);
+}
+
+/*
+ * Packed float-accumulate linear.  Follows
+ * csrc/kernels/ternary_gemm_production.cu:53-142 (and :158-250):
+ *   acc (fp32) += X[b,k] * decode(W_T[k/4, n], k%4), k ascending      (:126-133)
+ *   Y[b,n] = cast(acc * scale[n] + bias[n])                           (:139-141)
+ * x*w is exact for w in {-1,0,+1}, so fused or unfused multiply-add give the
+ * same accumulator.  The epilogue here is one fp32 multiply then one fp32 add.
+ * X is [B,K] widened to float; scale has scale_len entries (N, or 1 = broadcast);
+ * bias may be NULL.  Y is the fp32 value before the cast to the output dtype.
+ */
+void bto_linear_packed(const float* X, const uint8_t* W_T, const float* scale,
+                       int64_t scale_len, const float* bias, float* Y, int64_t B,
+                       int64_t N, int64_t K) {
+#pragma omp parallel for schedule(static)
+    for (int64_t n = 0; n < N; n++) {
+        const float s = scale[scale_len == 1 ? 0 : n];
+        const float bv = bias ? bias[n] : 0.0f;
+        for (int64_t b = 0; b < B; b++) {
+            float acc = 0.0f;
+            for (int64_t k = 0; k < K; k++) {
+                int w = decode2((W_T[(k / 4) * N + n] >> (2 * (k % 4))) & 3u);
+                acc += X[b * K + k] * (float)w;
+            }
+            float r = acc * s;
+            r = r + bv;
+            Y[b * N + n] = r;
+        }
+    }
+}
+
+/* Same contraction in float64 throughout: the high-precision truth that the
+ * tolerance tests measure both the oracle and the kernels against. */
+void bto_linear_packed_f64(const float* X, const uint8_t* W_T, const float* scale,
+                           int64_t scale_len, const float* bias, double* Y, int64_t B,
+                           int64_t N, int64_t K) {
+#pragma omp parallel for schedule(static)
+    for (int64_t n = 0; n < N; n++) {
+        const double s = scale[scale_len == 1 ? 0 : n];
+        const double bv = bias ? bias[n] : 0.0;
+        for (int64_t b = 0; b < B; b++) {
+            double acc = 0.0;
+            for (int64_t k = 0; k < K; k++) {
+                int w = decode2((W_T[(k / 4) * N + n] >> (2 * (k % 4))) & 3u);
+                acc += (double)X[b * K + k] * (double)w;
+            }
+            Y[b * N + n] = acc * s + bv;
+        }
+    }
+}
+
+/*
+ * Unpacked (dense int8 weights) float-accumulate linear.  Follows
+ * csrc/kernels/ternary_gemm.cu:41-73: acc += float(X)*float(W), k ascending
+ * (:59-63), acc *= scale[n] (:65-66), acc += bias[n] (:68-70).
+ */
+void bto_linear_unpacked(const float* X, const int8_t* W, const float* scale,
+                         int64_t scale_len, const float* bias, float* Y, int64_t B,
+                         int64_t N, int64_t K) {
+#pragma omp parallel for schedule(static)
+    for (int64_t n = 0; n < N; n++) {
+        const float s = scale[scale_len == 1 ? 0 : n];
+        for (int64_t b = 0; b < B; b++) {
+            float acc = 0.0f;
+            for (int64_t k = 0; k < K; k++) acc += X[b * K + k] * (float)W[n * K + k];
+            acc = acc * s;
+            if (bias) acc = acc + bias[n];
+            Y[b * N + n] = acc;
+        }
+    }
+}
+
+/*
+ * Per-row int8 activation quantizer.  Follows
+ * csrc/kernels/ternary_gemm_tensor_core.cu:431-441 and :343-347,:456-457 with
+ * the scale taken over the WHOLE row (the reference recomputes it per 32-wide
+ * K tile and keeps only the last one for the epilogue, which is only
+ * self-consistent for K <= 32; the whole-row form is the intended one):
+ *   amax = max_k |x|;  s_x = amax > 1e-6 ? amax / 127 : 1            (:439)
+ *   inv  = 1.0f / s_x                                                 (:456)
+ *   q    = (int8) clamp(roundf(x * inv), -127, 127)                   (:343-347)
+ * roundf rounds halfway cases away from zero.
+ */
+void bto_act_quant_i8(const float* X, int64_t B, int64_t K, int8_t* Q, float* s_x) {
+    for (int64_t b = 0; b < B; b++) {
+        const float* row = X + b * K;
+        float amax = 0.0f;
+        for (int64_t k = 0; k < K; k++) amax = fmaxf(amax, fabsf(row[k]));
+        const float s = (amax > 1e-6f) ? (amax / 127.0f) : 1.0f;
+        const float inv = 1.0f / s;
+        s_x[b] = s;
+        for (int64_t k = 0; k < K; k++) {
+            float v = row[k] * inv;
+            v = fmaxf(-127.0f, fminf(127.0f, roundf(v)));
+            Q[b * K + k] = (int8_t)v;
+        }
+    }
+}
+
+/*
+ * int8 x ternary GEMM with int32 accumulators.  Follows
+ * csrc/kernels/ternary_gemm_tensor_core.cu:73-75 (weights decode to +-127),
+ * :583-589 (int8*int8 -> int32 accumulate) and :652
+ *   y = (float(acc) * s_x / 127.0f) * w_scale + bias
+ * evaluated left to right, each operation rounded to fp32.
+ * acc (nullable) receives the raw int32 accumulators [B,N]; Y the fp32 result.
+ */
+void bto_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const float* scale,
+                 int64_t scale_len, const float* bias, int32_t* acc_out, float* Y, int64_t B,
+                 int64_t N, int64_t K) {
+#pragma omp parallel for schedule(static)
+    for (int64_t n = 0; n < N; n++) {
+        const float ws = scale[scale_len == 1 ? 0 : n];
+        const float bv = bias ? bias[n] : 0.0f;
+        for (int64_t b = 0; b < B; b++) {
+            int32_t acc = 0;
+            for (int64_t k = 0; k < K; k++) {
+                int w = 127 * decode2((W_T[(k / 4) * N + n] >> (2 * (k % 4))) & 3u);
+                acc += (int32_t)Q[b * K + k] * w;
+            }
+            if (acc_out) acc_out[b * N + n] = acc;
+            float r = (float)acc * s_x[b];
+            r = r / 127.0f;
+            r = r * ws;
+            r = r + bv;
+            Y[b * N + n] = r;
+        }
+    }
+}

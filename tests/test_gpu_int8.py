@@ -1,0 +1,106 @@
+"""GPU parity: int8 activation quantizer and int8 x ternary matrix-core GEMM vs the
+CPU oracle.  int8 activations, activation scales and int32 accumulators are
+bit-exact; float outputs are bit-exact in fp32 and equal after the same final
+rounding in bf16/fp16 (the epilogue performs the oracle's operations one by one)."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import announce
+from _util import f32np, random_ternary, rel_err, seeded_acts
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("b,k", [(1, 1), (3, 7), (16, 4096), (5, 11008), (64, 520), (2, 100000)])
+def test_act_quant_bit_exact(oracle, dtype, b, k):
+    from bittorch_amd import _C
+    announce("act_quant", dtype, b, k)
+    x = seeded_acts(b, k, seed=b + k, dtype=dtype, outliers=True)
+    if b > 2:
+        x[1] = 0  # all-zero row: scale 1
+    q, s = _C.act_quant_int8(x.cuda())
+    torch.cuda.synchronize()
+    oq, os_ = oracle.act_quant_i8(f32np(x))
+    np.testing.assert_array_equal(s.cpu().numpy(), os_)
+    np.testing.assert_array_equal(q.cpu().numpy(), oq)
+
+
+def _gemm_case(oracle, b, n, k, out_dtype, seed=0, bias=True, outliers=False):
+    from bittorch_amd import _C
+    from bittorch_amd.quant import pack_ternary_transposed
+    w = random_ternary(n, k, seed=seed)
+    packed = pack_ternary_transposed(w)[0]
+    g = torch.Generator().manual_seed(seed + 1)
+    scale = torch.rand(n, generator=g) * 0.05 + 0.01
+    bias_t = torch.randn(n, generator=g) * 0.01 if bias else None
+    x = seeded_acts(b, k, seed=seed + 2, dtype=out_dtype, outliers=outliers)
+    oq, os_, oacc, oy = oracle.linear_i8(f32np(x), packed.numpy(), f32np(scale), k,
+                                         None if bias_t is None else f32np(bias_t))
+    q, s = _C.act_quant_int8(x.cuda())
+    y, acc = _C.ternary_gemm_int8(q, s, packed.cuda(), scale.cuda(),
+                                  None if bias_t is None else bias_t.cuda(), k, out_dtype=out_dtype,
+                                  return_acc=True)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(q.cpu().numpy(), oq)
+    np.testing.assert_array_equal(acc.cpu().numpy(), oacc)
+    expect = torch.from_numpy(oy).to(out_dtype)
+    assert torch.equal(y.cpu(), expect), (b, n, k, out_dtype)
+    # fused entry point (quantize + GEMM in one call) gives the same output
+    y2 = _C.ternary_linear_tensor_core_forward(x.cuda(), packed.cuda(), scale.cuda(),
+                                               None if bias_t is None else bias_t.cuda(), k, 2)
+    assert torch.equal(y2.cpu(), expect)
+    return x, packed, scale, bias_t, oy
+
+
+# streaming (decode-shape) kernel: B <= 32
+@pytest.mark.parametrize("b,n,k", [(1, 64, 64), (16, 256, 4096), (16, 1024, 11008), (5, 48, 100),
+                                   (32, 128, 512), (17, 512, 1000), (2, 16, 20)])
+def test_gemm_i8_small_batch_bit_exact(oracle, b, n, k):
+    announce("gemm_i8 small", b, n, k)
+    _gemm_case(oracle, b, n, k, torch.bfloat16, seed=b + n)
+    _gemm_case(oracle, b, n, k, torch.float32, seed=b + n + 1, bias=False)
+
+
+# prefill kernel: B > 32, including ragged M / N / K tiles
+@pytest.mark.parametrize("b,n,k", [(128, 256, 128), (256, 512, 1024), (33, 64, 64), (130, 260, 132),
+                                   (64, 4, 16), (200, 1024, 4096), (129, 300, 1000), (2048, 256, 512)])
+def test_gemm_i8_prefill_bit_exact(oracle, b, n, k):
+    announce("gemm_i8 prefill", b, n, k)
+    _gemm_case(oracle, b, n, k, torch.bfloat16, seed=n + k, outliers=True)
+    _gemm_case(oracle, b, n, k, torch.float16, seed=n + k + 1)
+    _gemm_case(oracle, b, n, k, torch.float32, seed=n + k + 2, bias=False)
+
+
+def test_gemm_i8_close_to_float_path(oracle):
+    """int8 path vs the unquantized float product: inside the int8 quantisation error."""
+    announce("gemm_i8 vs float")
+    x, packed, scale, bias, oy = _gemm_case(oracle, 64, 256, 1024, torch.float32, seed=5)
+    truth = oracle.linear_packed(f32np(x), packed.numpy(), f32np(scale), 1024, f32np(bias), f64=True)
+    assert rel_err(oy, truth) < 2e-2
+
+
+def test_gemm_i8_full_size_properties():
+    """Config-4 shape [2048,4096] x [4096,4096]: linearity in the weights' sign and
+    agreement of two independent kernels (streaming rows vs prefill tiles)."""
+    from bittorch_amd import _C
+    from bittorch_amd.quant import pack_ternary_transposed
+    announce("gemm_i8 full size")
+    w = random_ternary(4096, 4096, seed=1)
+    packed = pack_ternary_transposed(w)[0].cuda()
+    packed_neg = pack_ternary_transposed(-w)[0].cuda()
+    x = seeded_acts(2048, 4096, seed=2, dtype=torch.bfloat16, outliers=True).cuda()
+    scale = torch.ones(4096, device="cuda")
+    q, s = _C.act_quant_int8(x)
+    _, acc = _C.ternary_gemm_int8(q, s, packed, scale, None, 4096, return_acc=True)
+    _, acc_neg = _C.ternary_gemm_int8(q, s, packed_neg, scale, None, 4096, return_acc=True)
+    assert torch.equal(acc, -acc_neg)
+    # rows 100..115 through the streaming kernel
+    _, acc_rows = _C.ternary_gemm_int8(q[100:116].contiguous(), s[100:116].contiguous(), packed, scale,
+                                       None, 4096, return_acc=True)
+    assert torch.equal(acc_rows, acc[100:116])
+    # against torch integer matmul on a slice (CPU, exact)
+    w127 = (w[:64].to(torch.int32) * 127)
+    ref = q[:32].cpu().to(torch.int32) @ w127.t()
+    assert torch.equal(acc[:32, :64].cpu(), ref)

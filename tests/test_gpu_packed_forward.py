@@ -1,0 +1,171 @@
+"""GPU parity: packed fp32-accumulate forward (decode GEMV / small batch / generic)
+vs the CPU oracle.  Tolerances: <= 1e-3 (fp32 out), <= 1e-2 (fp16/bf16 out),
+relative to the largest output magnitude; the float64 oracle is the truth the
+fp32-accumulate oracle itself is also measured against."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import announce
+from _util import f32np, random_ternary, rel_err, seeded_acts, seeded_weights
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-3, torch.float16: 1e-2, torch.bfloat16: 1e-2}
+
+
+def _case(oracle, b, n, k, dtype, bias=True, seed=0, scale_dtype=None, per_tensor=False):
+    from bittorch_amd import _C
+    from bittorch_amd.quant import pack_ternary_transposed
+    w = random_ternary(n, k, seed=seed)
+    g = torch.Generator().manual_seed(seed + 7)
+    scale = (torch.rand(1 if per_tensor else n, generator=g) * 0.05 + 0.01)
+    bias_t = (torch.randn(n, generator=g) * 0.01) if bias else None
+    x = seeded_acts(b, k, seed=seed + 3, dtype=dtype)
+    packed, _ = pack_ternary_transposed(w)
+    sdt = scale_dtype or dtype
+    scale_d = scale.to(sdt)
+    bias_d = None if bias_t is None else bias_t.to(dtype)
+    y = _C.ternary_linear_packed_forward(x.cuda(), packed.cuda(), scale_d.cuda(),
+                                         None if bias_d is None else bias_d.cuda(), k)
+    torch.cuda.synchronize()
+    assert y.dtype == dtype and tuple(y.shape) == (b, n)
+    args = (f32np(x), packed.numpy(), f32np(scale_d), k, None if bias_d is None else f32np(bias_d))
+    truth = oracle.linear_packed(*args, f64=True)
+    ref = oracle.linear_packed(*args)
+    got = f32np(y)
+    # the oracle's own distance from the truth bounds what fp32 accumulation may cost
+    assert rel_err(ref, truth) < 1e-5
+    assert rel_err(got, truth) < TOL[dtype], (b, n, k, dtype)
+    return got, ref.astype(np.float32)
+
+
+def test_config2_decode_gemv_fp16(oracle):
+    """x fp16 [1,4096] x W [4096,4096], per-tensor fp32 scale, fp16 bias."""
+    announce("config2 gemv fp16")
+    from bittorch_amd import _C
+    w = seeded_weights(4096, 4096, seed=0).cuda()
+    packed, scale, _ = _C.ternary_quantize_pack(w, 0.05, per_channel=False)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(1, 4096, generator=g).half()
+    bias = (torch.randn(4096, generator=g) * 0.01).half()
+    y = _C.ternary_linear_packed_forward(x.cuda(), packed, scale.reshape(1), bias.cuda(), 4096)
+    torch.cuda.synchronize()
+    truth = oracle.linear_packed(f32np(x), packed.cpu().numpy(), f32np(scale.reshape(1)), 4096,
+                                 f32np(bias), f64=True)
+    assert rel_err(f32np(y), truth) < 1e-2
+    # fp16 output of the exactly rounded result differs from ours by at most 1 ulp-ish
+    exact16 = torch.from_numpy(truth).to(torch.float16).float().numpy()
+    assert np.mean(exact16 != f32np(y)) < 0.02
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("b,n,k", [(1, 64, 64), (4, 16, 8), (8, 32, 64), (1, 4096, 4096), (16, 1024, 4096),
+                                   (3, 256, 11008), (16, 512, 512), (33, 128, 256), (64, 256, 768),
+                                   (2, 48, 100), (5, 40, 36)])
+def test_packed_forward_shapes(oracle, dtype, b, n, k):
+    announce("packed_forward", dtype, b, n, k)
+    _case(oracle, b, n, k, dtype, seed=b + n + k)
+
+
+@pytest.mark.parametrize("k", [1, 2, 3, 5, 6, 7, 9, 13, 17, 31, 65])
+@pytest.mark.parametrize("n", [4, 32, 67])
+def test_packed_forward_ragged_k_and_n(oracle, k, n):
+    announce("packed_forward ragged", n, k)
+    for dtype in (torch.float32, torch.float16):
+        _case(oracle, 3, n, k, dtype, seed=k)
+
+
+@pytest.mark.parametrize("b", [1, 2, 4, 8, 15, 16, 17, 32, 64])
+def test_packed_forward_batch_sizes(oracle, b):
+    announce("packed_forward batch", b)
+    _case(oracle, b, 128, 256, torch.float16, seed=b)
+    _case(oracle, b, 128, 256, torch.bfloat16, seed=b)
+
+
+def test_packed_forward_fp32_generic_is_bit_exact(oracle):
+    """The generic kernel accumulates in the reference's k order: equal to the oracle bit for bit."""
+    announce("packed_forward fp32 bit exact")
+    for (b, n, k) in [(32, 256, 512), (7, 33, 17), (1, 1, 1), (2, 100, 1000)]:
+        got, ref = _case(oracle, b, n, k, torch.float32, seed=11)
+        np.testing.assert_array_equal(got, ref)
+
+
+def test_packed_forward_mixed_scale_dtypes(oracle):
+    announce("packed_forward scale dtypes")
+    _case(oracle, 1, 256, 512, torch.float16, scale_dtype=torch.float32, per_tensor=True)
+    _case(oracle, 4, 256, 512, torch.bfloat16, scale_dtype=torch.float32)
+    _case(oracle, 4, 256, 512, torch.float16, bias=False)
+
+
+def test_packed_forward_known_answers(oracle):
+    """All-zero weights give the bias; all-ones weights give row sums; reserved code 3 is zero."""
+    from bittorch_amd import _C
+    from bittorch_amd.quant import pack_ternary_transposed
+    announce("packed_forward known answers")
+    for dtype in (torch.float32, torch.float16, torch.bfloat16):
+        x = seeded_acts(4, 64, seed=2, dtype=dtype).cuda()
+        bias = torch.linspace(-1, 1, 32).to(dtype).cuda()
+        ones_scale = torch.ones(32, dtype=dtype).cuda()
+        zeros = pack_ternary_transposed(torch.zeros(32, 64))[0].cuda()
+        y = _C.ternary_linear_packed_forward(x, zeros, ones_scale, bias, 64)
+        assert torch.equal(y, bias.expand(4, 32))
+        threes = torch.full_like(zeros, 0xFF)
+        y = _C.ternary_linear_packed_forward(x, threes, ones_scale, bias, 64)
+        assert torch.equal(y, bias.expand(4, 32))
+        ones = pack_ternary_transposed(torch.ones(32, 64))[0].cuda()
+        y = _C.ternary_linear_packed_forward(x, ones, ones_scale, None, 64)
+        ref = x.float().sum(dim=1, keepdim=True).expand(4, 32)
+        assert torch.allclose(y.float(), ref, rtol=1e-2, atol=1e-2)
+    # the reference's JS known-answer vectors
+    wts = torch.tensor([[1, -1, 0, 0], [-1, 1, 0, 0]], dtype=torch.float32)
+    p = pack_ternary_transposed(wts)[0].cuda()
+    x = torch.tensor([[10.0, 3.0, 0.0, 0.0]]).cuda()
+    y = _C.ternary_linear_packed_forward(x, p, torch.ones(2).cuda(), None, 4)
+    assert y.tolist() == [[7.0, -7.0]]
+    wts = torch.tensor([[1, 0, 0, 0], [0, 1, 0, 0]], dtype=torch.float32)
+    p = pack_ternary_transposed(wts)[0].cuda()
+    x = torch.tensor([[4.0, 8.0, 0.0, 0.0]]).cuda()
+    y = _C.ternary_linear_packed_forward(x, p, torch.tensor([2.0, 0.5]).cuda(), None, 4)
+    assert y.tolist() == [[8.0, 4.0]]
+
+
+def test_packed_forward_stream_configs_agree(oracle):
+    """Every tile width / wave count / split-K of the streaming kernel gives the same sums
+    (int-exact decode; fp32 sums differ only by association)."""
+    from bittorch_amd import _C
+    from bittorch_amd.quant import pack_ternary_transposed
+    announce("packed_forward stream configs")
+    w = random_ternary(512, 1024, seed=4)
+    packed = pack_ternary_transposed(w)[0].cuda()
+    x = seeded_acts(5, 1024, seed=5, dtype=torch.float16).cuda()
+    scale = torch.ones(512, dtype=torch.float16).cuda()
+    truth = oracle.linear_packed(f32np(x), packed.cpu().numpy(), f32np(scale), 1024, f64=True)
+    try:
+        for cfg in ("16,4,1", "16,2,4", "8,8,2", "4,4,8", "4,16,1", "8,4,16", "16,16,3"):
+            os.environ["BITTORCH_STREAM_CFG"] = cfg
+            y = _C.ternary_linear_packed_forward(x, packed, scale, None, 1024)
+            torch.cuda.synchronize()
+            assert rel_err(f32np(y), truth) < 2e-3, cfg
+    finally:
+        os.environ.pop("BITTORCH_STREAM_CFG", None)
+
+
+def test_unpacked_forward_matches_oracle(oracle):
+    from bittorch_amd import _C
+    announce("unpacked forward")
+    for (b, n, k) in [(4, 8, 16), (1, 1, 1), (17, 67, 123), (32, 256, 512)]:
+        w = random_ternary(n, k, seed=k)
+        g = torch.Generator().manual_seed(1)
+        scale = torch.rand(n, generator=g)
+        bias = torch.randn(n, generator=g)
+        x = seeded_acts(b, k, seed=2)
+        y = _C.ternary_linear_forward(x.cuda(), w.cuda(), scale.cuda(), bias.cuda())
+        ref = oracle.linear_unpacked(f32np(x), w.numpy(), f32np(scale), f32np(bias))
+        np.testing.assert_array_equal(f32np(y), ref)
+        y16 = _C.ternary_linear_forward(x.half().cuda(), w.cuda(), scale.half().cuda(), None)
+        assert y16.dtype == torch.float16
+        ref16 = oracle.linear_unpacked(f32np(x.half()), w.numpy(), f32np(scale.half()), None)
+        assert rel_err(f32np(y16), ref16) < 1e-2

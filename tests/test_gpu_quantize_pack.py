@@ -1,0 +1,93 @@
+"""GPU parity: fused quantize + 2-bit pack kernel vs the CPU oracle (bit-exact)."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import announce
+from _util import BT_DT, f32np, seeded_weights
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(oracle, w_cpu, tf, per_channel, want_tern=True):
+    from bittorch_amd import _C
+    w = w_cpu.cuda()
+    packed, scale, tern = _C.ternary_quantize_pack(w, tf, per_channel, want_packed=True, want_tern=want_tern)
+    torch.cuda.synchronize()
+    o_tern, o_scale = oracle.ternary_quantize(f32np(w_cpu), tf, per_channel, dtype=BT_DT[w_cpu.dtype])
+    o_packed, _ = oracle.pack_ternary_transposed(o_tern)
+    np.testing.assert_array_equal(f32np(scale).reshape(-1), o_scale.reshape(-1))
+    np.testing.assert_array_equal(packed.cpu().numpy(), o_packed)
+    if want_tern:
+        np.testing.assert_array_equal(tern.cpu().numpy(), o_tern)
+    return packed, scale
+
+
+# (N, K): config shapes, ragged N (not a multiple of 16), K % 4 != 0, tiny, each ITERS variant
+SHAPES = [(256, 512), (16, 64), (1, 1), (3, 4), (7, 33), (17, 123), (33, 5), (64, 1024), (40, 1028),
+          (48, 2048), (32, 4096), (24, 5000), (16, 8192), (16, 11008), (16, 12288), (8, 12292), (4, 20000)]
+
+
+@pytest.mark.parametrize("n,k", SHAPES)
+@pytest.mark.parametrize("per_channel", [True, False])
+def test_quantize_pack_matches_oracle_fp32(oracle, n, k, per_channel):
+    announce("quantize_pack fp32", n, k, per_channel)
+    _run(oracle, seeded_weights(n, k, seed=n * 131 + k), 0.05, per_channel)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n,k", [(256, 512), (7, 33), (32, 4096), (16, 11008)])
+def test_quantize_pack_matches_oracle_16bit(oracle, n, k, dtype):
+    announce("quantize_pack", dtype, n, k)
+    _run(oracle, seeded_weights(n, k, seed=5, dtype=dtype), 0.05, True)
+    _run(oracle, seeded_weights(n, k, seed=6, dtype=dtype), 0.05, False)
+
+
+@pytest.mark.parametrize("tf", [0.0, 0.01, 0.1, 0.5, 1.0])
+def test_quantize_pack_threshold_factors(oracle, tf):
+    announce("quantize_pack tf", tf)
+    w = seeded_weights(64, 256, seed=9, std=1.0)
+    w[3, 7] = 0.0
+    w[5] = 0.0  # all-zero row: scale floors at 1e-8, all codes zero
+    _run(oracle, w, tf, True)
+    _run(oracle, w, tf, False)
+
+
+def test_quantize_pack_extreme_magnitudes(oracle):
+    announce("quantize_pack magnitudes")
+    for mag in (1e-10, 1e10):
+        _run(oracle, seeded_weights(32, 64, seed=3, std=1.0) * mag, 0.05, True)
+
+
+def test_quantize_pack_matches_torch_ops_full_size(oracle):
+    """Config-2 shape: kernel vs the torch op chain on the same GPU tensor (bit-exact)."""
+    from bittorch_amd import _C
+    from bittorch_amd.quant import pack_ternary_transposed, ternary_quantize
+    announce("quantize_pack 4096x4096 vs torch ops")
+    w = seeded_weights(4096, 4096, seed=0).cuda()
+    for per_channel in (True, False):
+        packed, scale, _ = _C.ternary_quantize_pack(w, 0.05, per_channel)
+        w_tern, s_ref = ternary_quantize(w, 0.05, per_channel)
+        p_ref, _ = pack_ternary_transposed(w_tern)
+        assert torch.equal(scale, s_ref)
+        assert torch.equal(packed, p_ref)
+    # the 11008-wide rows of config 3
+    w = seeded_weights(256, 11008, seed=1).cuda()
+    packed, scale, _ = _C.ternary_quantize_pack(w, 0.05, True)
+    w_tern, s_ref = ternary_quantize(w, 0.05, True)
+    assert torch.equal(scale, s_ref)
+    assert torch.equal(packed, pack_ternary_transposed(w_tern)[0])
+
+
+def test_unpack_dequant_roundtrip(oracle):
+    from bittorch_amd import _C
+    announce("unpack_dequant")
+    for n, k in [(64, 128), (17, 123), (256, 512), (100, 4096)]:
+        w = seeded_weights(n, k, seed=n + k).cuda()
+        packed, scale, tern = _C.ternary_quantize_pack(w, 0.05, True, want_tern=True)
+        back = _C.unpack_dequant(packed, k, out_dtype=torch.int8)
+        assert torch.equal(back, tern)
+        np.testing.assert_array_equal(back.cpu().numpy(),
+                                      oracle.unpack_ternary_transposed(packed.cpu().numpy(), k))
+        deq = _C.unpack_dequant(packed, k, scale, out_dtype=torch.float32)
+        assert torch.equal(deq, tern.float() * scale.unsqueeze(1))
