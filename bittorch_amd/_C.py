@@ -50,8 +50,28 @@ def _dt(t: Tensor, what: str) -> int:
         raise RuntimeError(f"{what} must be float32, float16 or bfloat16, got {t.dtype}") from None
 
 
+_COUNTER_BYTES = 16384  # BT_WORKSPACE_COUNTER_BYTES: must be zero on entry, is zero on exit
+_ws_cache = {}
+
+
 def _workspace(nbytes: int, device) -> Optional[Tensor]:
-    return torch.empty(nbytes, dtype=torch.uint8, device=device) if nbytes > 0 else None
+    """Scratch buffer for the current stream of ``device``, kept between calls.
+
+    The library needs the head of the buffer zeroed once and restores the zeros
+    itself, so the buffer is cleared when it is (re)allocated and then reused.
+    One buffer per (device, stream): calls on one stream run in order.
+    """
+    if nbytes <= 0:
+        return None
+    key = (device.index if device.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(device).cuda_stream)
+    buf = _ws_cache.get(key)
+    if buf is None or buf.numel() < nbytes:
+        size = max(nbytes, 1 << 20)
+        buf = torch.empty(size, dtype=torch.uint8, device=device)
+        buf[:_COUNTER_BYTES].zero_()
+        _ws_cache[key] = buf
+    return buf
 
 
 def _all_cuda(*ts: Optional[Tensor]) -> bool:
@@ -153,7 +173,7 @@ def ternary_linear_packed_forward(X: Tensor, W_T: Tensor, scale: Tensor,
         _status(_L.bt_ternary_linear_packed_forward(
             x2.data_ptr(), xdt, W_T.data_ptr(), scale.data_ptr(), _dt(scale, "scale"), scale.numel(),
             _ptr(bias), 0 if bias is None else _dt(bias, "bias"), y.data_ptr(), B, N, K,
-            _ptr(ws), ws_bytes, _stream(X)))
+            _ptr(ws), 0 if ws is None else ws.numel(), _stream(X)))
     return y.reshape(*X.shape[:-1], N)
 
 
@@ -187,7 +207,7 @@ def ternary_linear_tensor_core_forward(X: Tensor, W_T: Tensor, scale: Tensor,
         _status(_L.bt_ternary_linear_tensor_core_forward(
             x2.data_ptr(), _dt(x2, "X"), W_T.data_ptr(), scale.data_ptr(), _dt(scale, "scale"),
             scale.numel(), _ptr(bias), 0 if bias is None else _dt(bias, "bias"), y.data_ptr(),
-            B, N, K, _ptr(ws), ws_bytes, _stream(X)))
+            B, N, K, _ptr(ws), 0 if ws is None else ws.numel(), _stream(X)))
     return y
 
 
@@ -262,7 +282,7 @@ def ternary_gemm_int8(Q: Tensor, s_x: Tensor, W_T: Tensor, scale: Tensor,
         _status(_L.bt_ternary_gemm_i8(
             q.data_ptr(), s_x.data_ptr(), W_T.data_ptr(), scale.data_ptr(), _dt(scale, "scale"),
             scale.numel(), _ptr(bias), 0 if bias is None else _dt(bias, "bias"), y.data_ptr(),
-            _DT[out_dtype], _ptr(acc), B, N, K, _ptr(ws), ws_bytes, _stream(q)))
+            _DT[out_dtype], _ptr(acc), B, N, K, _ptr(ws), 0 if ws is None else ws.numel(), _stream(q)))
     return (y, acc) if return_acc else y
 
 

@@ -124,7 +124,7 @@ static bool packed_uses_stream(int x_dtype, const void* W_T, const void* Y, int6
 }
 
 extern "C" size_t bt_packed_forward_workspace_bytes(int64_t B, int64_t N, int64_t K, int x_dtype) {
-    if (B <= 0 || N <= 0 || K <= 0 || x_dtype == BT_F32 || N % 4 != 0) return 0;
+    if (B <= 0 || N <= 0 || K <= 0 || x_dtype == BT_F32) return 0;
     return stream_workspace_bytes(x_dtype == BT_F16 ? MODE_F16 : MODE_BF16, B, N, ceil_div(K, 4));
 }
 
@@ -158,8 +158,7 @@ extern "C" int bt_act_quant_i8(const void* X, int x_dtype, int64_t B, int64_t K,
 }
 
 extern "C" size_t bt_gemm_i8_workspace_bytes(int64_t B, int64_t N, int64_t K) {
-    if (B <= 0 || N <= 0 || K <= 0 || N % 4 != 0) return 0;
-    if (B > kStreamMaxRows) return 0;
+    if (B <= 0 || N <= 0 || K <= 0) return 0;
     return stream_workspace_bytes(MODE_I8, B, N, ceil_div(K, 4));
 }
 
@@ -179,16 +178,17 @@ extern "C" int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8
                   (long long)kMaxKInt8);
         return BT_ERR_INVALID;
     }
-    if (N % 4 != 0 || ((uintptr_t)W_T) % 16 != 0 || !fast_path_ok(Y, N, K) ||
-        (acc_out && ((uintptr_t)acc_out) % 16 != 0)) {
-        set_error("%s: needs N %% 4 == 0 and 16-byte aligned W_T / Y / acc_out (N=%lld)", who, (long long)N);
+    if (((uintptr_t)W_T) % 16 != 0 || !fast_path_ok(Y, N, K) || (acc_out && ((uintptr_t)acc_out) % 16 != 0)) {
+        set_error("%s: W_T, Y and acc_out must be 16-byte aligned", who);
         return BT_ERR_INVALID;
     }
     Epilogue epi;
     rc = make_epilogue(who, scale, scale_dtype, scale_len, bias, bias_dtype, N, &epi);
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
-    if (B <= kStreamMaxRows)
+    // decode-shape batches, and any batch whose N the tiled kernel's 4-column
+    // vector accesses cannot take, stream the weights once per 16 rows
+    if (B <= kStreamMaxRows || !gemm_i8_supported(N, W_T))
         return launch_stream(MODE_I8, Q, 1, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, workspace,
                              workspace_bytes, st);
     return launch_gemm_i8(Q, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, st);
@@ -196,7 +196,8 @@ extern "C" int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8
 
 extern "C" size_t bt_tensor_core_workspace_bytes(int64_t B, int64_t N, int64_t K) {
     if (B <= 0 || N <= 0 || K <= 0) return 0;
-    return align256((size_t)B * K) + align256((size_t)B * 4) + bt_gemm_i8_workspace_bytes(B, N, K);
+    // [GEMM scratch (ticket counters first)] [Q int8 B*K] [s_x fp32 B]
+    return align256(bt_gemm_i8_workspace_bytes(B, N, K)) + align256((size_t)B * K) + align256((size_t)B * 4);
 }
 
 extern "C" int bt_ternary_linear_tensor_core_forward(const void* X, int x_dtype, const uint8_t* W_T,
@@ -212,12 +213,11 @@ extern "C" int bt_ternary_linear_tensor_core_forward(const void* X, int x_dtype,
         set_error("%s: workspace of %zu bytes (256-byte aligned) needed, %zu given", who, need, workspace_bytes);
         return BT_ERR_WORKSPACE;
     }
-    int8_t* Q = (int8_t*)workspace;
-    float* s_x = (float*)((uint8_t*)workspace + align256((size_t)B * K));
-    uint8_t* rest = (uint8_t*)s_x + align256((size_t)B * 4);
-    const size_t rest_bytes = workspace_bytes - (size_t)(rest - (uint8_t*)workspace);
+    const size_t gemm_bytes = align256(bt_gemm_i8_workspace_bytes(B, N, K));
+    int8_t* Q = (int8_t*)((uint8_t*)workspace + gemm_bytes);
+    float* s_x = (float*)((uint8_t*)Q + align256((size_t)B * K));
     rc = bt_act_quant_i8(X, x_dtype, B, K, Q, s_x, stream);
     if (rc) return rc;
     return bt_ternary_gemm_i8(Q, s_x, W_T, scale, scale_dtype, scale_len, bias, bias_dtype, Y, x_dtype, nullptr,
-                              B, N, K, rest, rest_bytes, stream);
+                              B, N, K, workspace, gemm_bytes, stream);
 }

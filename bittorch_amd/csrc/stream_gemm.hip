@@ -10,16 +10,22 @@
 //
 // Work decomposition.  A wave "step" covers RS consecutive kb rows (16 for int8,
 // 8 for 16-bit floats) and 16*NW output columns: lane (j = lane%16, g = lane/16)
-// loads NW consecutive bytes (one dword, two, or four: a 128-bit load) from each
-// of the KBG = RS/4 rows kb0 + g*KBG + r.  Those bytes are the B operands of NW
-// MFMA instructions: MFMA t multiplies the 16 activation rows with output columns
-// n = nb + NW*j + t.  The k order inside an MFMA is free as long as both operands
-// agree, so the activation fragments are laid out once per workgroup (in LDS) in
-// the order the cheapest weight decode produces.
-// A workgroup covers one column tile and one slice of K (grid.y = split-K); its
-// waves take steps round-robin and their accumulators are summed through LDS in
-// a fixed order.  With split-K > 1 the per-slice sums go to a workspace and a
-// second kernel adds them, again in a fixed order, and applies the epilogue.
+// loads NW consecutive bytes (a byte, a short, a dword, two or four dwords) from
+// each of the KBG = RS/4 rows kb0 + g*KBG + r.  Those bytes are the B operands of
+// NW MFMA instructions: MFMA t multiplies the 16 activation rows with output
+// columns n = nb + NW*j + t.  The k order inside an MFMA is free as long as both
+// operands agree, so each lane loads its 16 bytes of activations (row i = lane%16,
+// the same k range as its weights) straight from global memory and permutes them
+// into the order the cheapest weight decode produces.
+// A wave issues the loads of PF steps before it computes any of them, which is
+// what keeps enough bytes in flight to cover the HBM latency.
+// A workgroup owns one column tile over the WHOLE of K: there is no split-K
+// across workgroups, hence no partial sums in memory, no second pass and no
+// inter-workgroup synchronisation.  The tile width is chosen so that there are
+// enough tiles for every CU (down to 16 columns, one byte per lane and row);
+// tiles that share 128-byte lines of W_T are placed on the same XCD so the
+// line is fetched from HBM once.  The waves of a workgroup take steps
+// round-robin and their accumulators are summed through LDS in wave order.
 #include "bt_common.h"
 
 namespace bt {
@@ -30,28 +36,32 @@ struct StreamParams {
     const float* s_x;     // MODE_I8: per-row activation scales [M]
     void* Y;              // [M, N] of y_dtype
     int32_t* acc_out;     // MODE_I8, optional raw accumulators [M, N]
-    void* partial;        // [S][M][N] 32-bit words when S > 1
     Epilogue epi;
     int64_t N, K, Kb;
-    int64_t kb_per_split; // multiple of RS
+    int tiles;            // column tiles
+    int per_xcd;          // tiles per XCD (grid = 8 * per_xcd)
     int M;                // 1..16
     int y_dtype;
-    int x_vec_ok;         // activations may be read with 16-byte loads
+    int x_vec_ok;         // activation rows may be read with 16-byte loads
 };
 
 template <int NW> struct RawVec;
 template <> struct RawVec<16> { typedef uint4 type; };
 template <> struct RawVec<8> { typedef uint2 type; };
 template <> struct RawVec<4> { typedef uint32_t type; };
+template <> struct RawVec<2> { typedef uint16_t type; };
+template <> struct RawVec<1> { typedef uint8_t type; };
 
+// NW bytes of one kb row into ceil(NW/4) dwords (zero extended / zero when !ok)
 template <int NW>
-__device__ __forceinline__ void load_raw(const uint8_t* p, bool ok, uint32_t (&d)[NW / 4]) {
+__device__ __forceinline__ void load_raw(const uint8_t* p, bool ok, uint32_t (&d)[(NW + 3) / 4]) {
     if (ok) {
-        typename RawVec<NW>::type v = *(const typename RawVec<NW>::type*)p;
-        __builtin_memcpy(d, &v, NW);
+        const typename RawVec<NW>::type v = *(const typename RawVec<NW>::type*)p;
+        if constexpr (NW >= 4) __builtin_memcpy(d, &v, NW);
+        else d[0] = (uint32_t)v;
     } else {
 #pragma unroll
-        for (int i = 0; i < NW / 4; i++) d[i] = 0u;
+        for (int i = 0; i < (NW + 3) / 4; i++) d[i] = 0u;
     }
 }
 
@@ -79,310 +89,248 @@ __device__ __forceinline__ void finish_output(const StreamParams& p, int row, in
     store_out(p.Y, p.y_dtype, (int64_t)row * p.N + n, y);
 }
 
-template <int MODE, int NW, int WAVES>
+template <int MODE>
+__device__ __forceinline__ uint32_t add_bits(uint32_t a, uint32_t b) {
+    if constexpr (MODE == MODE_I8) return (uint32_t)((int32_t)a + (int32_t)b);
+    else return __builtin_bit_cast(uint32_t, __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b));
+}
+
+// 16 bytes of activations for lane (row i, group g) of one step, in natural k order
+template <int MODE>
+__device__ __forceinline__ uint4 load_x_frag(const StreamParams& p, int i, int64_t k) {
+    constexpr int GE = (MODE == MODE_I8) ? 16 : 8;
+    uint4 v = make_uint4(0u, 0u, 0u, 0u);
+    if (i < p.M && k < p.K) {
+        if constexpr (MODE == MODE_I8) {
+            const uint8_t* src = (const uint8_t*)p.X + (int64_t)i * p.K + k;
+            if (p.x_vec_ok && k + GE <= p.K) {
+                v = *(const uint4*)src;
+            } else {
+                uint32_t d[4] = {0u, 0u, 0u, 0u};
+                for (int e = 0; e < GE; e++)
+                    if (k + e < p.K) d[e >> 2] |= (uint32_t)src[e] << (8 * (e & 3));
+                v = make_uint4(d[0], d[1], d[2], d[3]);
+            }
+        } else {
+            const uint16_t* src = (const uint16_t*)p.X + (int64_t)i * p.K + k;
+            if (p.x_vec_ok && k + GE <= p.K) {
+                v = *(const uint4*)src;
+            } else {
+                uint32_t d[4] = {0u, 0u, 0u, 0u};
+                for (int e = 0; e < GE; e++)
+                    if (k + e < p.K) d[e >> 1] |= (uint32_t)src[e] << (16 * (e & 1));
+                v = make_uint4(d[0], d[1], d[2], d[3]);
+            }
+        }
+    }
+    return v;
+}
+
+template <int MODE, int NW, int WAVES, int PF>
 __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
     constexpr int KBG = (MODE == MODE_I8) ? 4 : 2;  // kb rows per lane group
     constexpr int RS = 4 * KBG;                     // kb rows per wave step
-    constexpr int GE = (MODE == MODE_I8) ? 16 : 8;  // activation elements per group
     constexpr int TILE_N = 16 * NW;
-    constexpr int ND = NW / 4;
+    constexpr int ND = (NW + 3) / 4;                // dwords per lane and row
     typedef typename std::conditional<MODE == MODE_I8, v4i, v4f>::type acc_t;
 
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    extern __shared__ __attribute__((aligned(16))) uint32_t red[];  // [WAVES][M][TILE_N]
+
+    // consecutive tiles on one XCD (workgroups are dealt round-robin over 8 XCDs)
+    const int tile = (int)(blockIdx.x & 7) * p.per_xcd + (int)(blockIdx.x >> 3);
+    if (tile >= p.tiles) return;
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int j = lane & 15;
     const int g = lane >> 4;
-    const int64_t nb = (int64_t)blockIdx.x * TILE_N;
-    const int64_t kb0 = (int64_t)blockIdx.y * p.kb_per_split;
-    const int64_t kb1 = (kb0 + p.kb_per_split < p.Kb) ? kb0 + p.kb_per_split : p.Kb;
-    const int nsteps = (int)((kb1 - kb0 + RS - 1) / RS);
+    const int64_t nb = (int64_t)tile * TILE_N;
+    const int nsteps = (int)((p.Kb + RS - 1) / RS);
     const int64_t ncol = nb + (int64_t)NW * j;
     const bool col_ok = ncol < p.N;
-
-    uint32_t raw[KBG][ND];
-    auto load_step = [&](int step) {
-#pragma unroll
-        for (int r = 0; r < KBG; r++) {
-            const int64_t kb = kb0 + (int64_t)step * RS + g * KBG + r;
-            load_raw<NW>(p.W_T + kb * p.N + ncol, col_ok && kb < kb1, raw[r]);
-        }
-    };
-
-    // weights first: their HBM latency overlaps the activation staging below
-    int step = wave;
-    if (step < nsteps) load_step(step);
-
-    // ---- stage the activation fragments of this K slice into LDS --------------
-    // slot (step s, lane l = gl*16 + i) holds the 16 bytes lane l feeds to the MFMA
-    // in step s: row i, group gl, elements in decode order.
-    {
-        const int ngroups = nsteps * 4;
-        const int64_t k_base = 4 * kb0;
-        for (int idx = threadIdx.x; idx < ngroups * 16; idx += WAVES * 64) {
-            const int i = idx & 15;
-            const int gidx = idx >> 4;
-            const int64_t k = k_base + (int64_t)gidx * GE;
-            uint32_t d[4] = {0u, 0u, 0u, 0u};
-            if (i < p.M && k < p.K) {
-                if constexpr (MODE == MODE_I8) {
-                    const int8_t* src = (const int8_t*)p.X + (int64_t)i * p.K + k;
-                    if (p.x_vec_ok && k + 16 <= p.K) {
-                        const uint4 v = *(const uint4*)src;
-                        d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
-                    } else {
-                        for (int e = 0; e < 16; e++)
-                            if (k + e < p.K) d[e >> 2] |= (uint32_t)(uint8_t)src[e] << (8 * (e & 3));
-                    }
-                    uint32_t t[4];
-                    transpose4x4_bytes(d[0], d[1], d[2], d[3], t);
-                    d[0] = t[0]; d[1] = t[1]; d[2] = t[2]; d[3] = t[3];
-                } else {
-                    const uint16_t* src = (const uint16_t*)p.X + (int64_t)i * p.K + k;
-                    if (p.x_vec_ok && k + 8 <= p.K) {
-                        const uint4 v = *(const uint4*)src;
-                        d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
-                    } else {
-                        for (int e = 0; e < 8; e++)
-                            if (k + e < p.K) d[e >> 1] |= (uint32_t)src[e] << (16 * (e & 1));
-                    }
-                    // natural halves h0..h7 -> dword c = { h[c], h[4+c] }
-                    const uint32_t o0 = perm(d[2], d[0], 0x05040100u);
-                    const uint32_t o1 = perm(d[2], d[0], 0x07060302u);
-                    const uint32_t o2 = perm(d[3], d[1], 0x05040100u);
-                    const uint32_t o3 = perm(d[3], d[1], 0x07060302u);
-                    d[0] = o0; d[1] = o1; d[2] = o2; d[3] = o3;
-                }
-            }
-            const int s = gidx >> 2, gl = gidx & 3;
-            *(uint4*)(smem + ((size_t)(s * 64 + gl * 16 + i) << 4)) = make_uint4(d[0], d[1], d[2], d[3]);
-        }
-    }
-    __syncthreads();
+    const uint8_t* wcol = p.W_T + ncol;
 
     acc_t acc[NW];
 #pragma unroll
     for (int t = 0; t < NW; t++) acc[t] = acc_t{0, 0, 0, 0};
 
-    while (step < nsteps) {
-        uint32_t cur[KBG][ND];
+    for (int base = wave; base < nsteps; base += WAVES * PF) {
+        uint32_t raw[PF][KBG][ND];
+        uint4 xa[PF];
 #pragma unroll
-        for (int r = 0; r < KBG; r++)
+        for (int f = 0; f < PF; f++) {
+            const int step = base + f * WAVES;
+            const int64_t kbs = (int64_t)step * RS + g * KBG;
 #pragma unroll
-            for (int d = 0; d < ND; d++) cur[r][d] = raw[r][d];
-        const int next = step + WAVES;
-        if (next < nsteps) load_step(next);
-
-        const uint4 av = *(const uint4*)(smem + ((size_t)(step * 64 + lane) << 4));
+            for (int r = 0; r < KBG; r++)
+                load_raw<NW>(wcol + (kbs + r) * p.N, col_ok && kbs + r < p.Kb, raw[f][r]);
+            xa[f] = load_x_frag<MODE>(p, j, 4 * kbs);
+        }
 #pragma unroll
-        for (int d = 0; d < ND; d++) {
+        for (int f = 0; f < PF; f++) {
+            if (base + f * WAVES >= nsteps) break;  // uniform per wave
             if constexpr (MODE == MODE_I8) {
-                const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
-                uint32_t G[4];
-                transpose4x4_bytes(cur[0][d], cur[1][d], cur[2][d], cur[3][d], G);
+                uint32_t ta[4];
+                transpose4x4_bytes(xa[f].x, xa[f].y, xa[f].z, xa[f].w, ta);
+                const v4i a = {(int)ta[0], (int)ta[1], (int)ta[2], (int)ta[3]};
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const v4i b = decode16_i8(G[i]);
-                    acc[4 * d + i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[4 * d + i], 0, 0, 0);
-                }
-            } else {
-                const u32x4 au = {av.x, av.y, av.z, av.w};
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    // bytes: [zero, row0.byte i, zero, row1.byte i]
-                    const uint32_t sel = ((uint32_t)(4 + i) << 24) | (0x0Cu << 16) | ((uint32_t)i << 8) | 0x0Cu;
-                    const uint32_t M2 = perm(cur[1][d], cur[0][d], sel);
-                    if constexpr (MODE == MODE_F16) {
-                        const u32x4 bu = decode8_16bit<LUT_F16_ONE>(M2);
-                        acc[4 * d + i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                            __builtin_bit_cast(v8h, au), __builtin_bit_cast(v8h, bu), acc[4 * d + i], 0, 0, 0);
+                for (int d = 0; d < ND; d++) {
+                    uint32_t G[4];
+                    if constexpr (NW == 1) {
+                        // one byte per row: G = {row0, row1, row2, row3}
+                        G[0] = raw[f][0][0] | (raw[f][1][0] << 8) | (raw[f][2][0] << 16) | (raw[f][3][0] << 24);
                     } else {
-                        const u32x4 bu = decode8_16bit<LUT_BF16_TWO>(M2);
-                        acc[4 * d + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                            __builtin_bit_cast(v8bf, au), __builtin_bit_cast(v8bf, bu), acc[4 * d + i], 0, 0, 0);
+                        transpose4x4_bytes(raw[f][0][d], raw[f][1][d], raw[f][2][d], raw[f][3][d], G);
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        if (4 * d + i < NW) {
+                            const v4i b = decode16_i8(G[i]);
+                            acc[4 * d + i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[4 * d + i], 0, 0, 0);
+                        }
                     }
                 }
-            }
-        }
-        step = next;
-    }
-
-    // ---- sum the waves' accumulators through LDS (fixed order) -------------------
-    // red[row][t*16 + j] (32-bit words); lane (j, g) holds rows 4g..4g+3 of column t*16+j
-    __syncthreads();  // every wave is done reading the activation stage
-    uint32_t* red = (uint32_t*)smem;
-    for (int w = 0; w < WAVES; w++) {
-        if (wave == w) {
+            } else {
+                // natural halves h0..h7 -> dword c = { h[c], h[4+c] } (the decode's k order)
+                const u32x4 au = {perm(xa[f].z, xa[f].x, 0x05040100u), perm(xa[f].z, xa[f].x, 0x07060302u),
+                                  perm(xa[f].w, xa[f].y, 0x05040100u), perm(xa[f].w, xa[f].y, 0x07060302u)};
 #pragma unroll
-            for (int t = 0; t < NW; t++) {
+                for (int d = 0; d < ND; d++) {
 #pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    const int row = 4 * g + r;
-                    if (row < p.M) {
-                        uint32_t* slot = red + row * TILE_N + t * 16 + j;
-                        if constexpr (MODE == MODE_I8) {
-                            const int32_t v = acc[t][r] + (w == 0 ? 0 : (int32_t)*slot);
-                            *slot = (uint32_t)v;
-                        } else {
-                            const float v = (w == 0) ? acc[t][r] : __fadd_rn(__builtin_bit_cast(float, *slot), acc[t][r]);
-                            *slot = __builtin_bit_cast(uint32_t, v);
+                    for (int i = 0; i < 4; i++) {
+                        if (4 * d + i < NW) {
+                            // bytes: [zero, row0.byte i, zero, row1.byte i]
+                            const uint32_t sel = ((uint32_t)(4 + i) << 24) | (0x0Cu << 16) | ((uint32_t)i << 8) | 0x0Cu;
+                            const uint32_t M2 = perm(raw[f][1][d], raw[f][0][d], sel);
+                            if constexpr (MODE == MODE_F16) {
+                                const u32x4 bu = decode8_16bit<LUT_F16_ONE>(M2);
+                                acc[4 * d + i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                    __builtin_bit_cast(v8h, au), __builtin_bit_cast(v8h, bu), acc[4 * d + i], 0, 0, 0);
+                            } else {
+                                const u32x4 bu = decode8_16bit<LUT_BF16_TWO>(M2);
+                                acc[4 * d + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                                    __builtin_bit_cast(v8bf, au), __builtin_bit_cast(v8bf, bu), acc[4 * d + i], 0, 0, 0);
+                            }
                         }
                     }
                 }
             }
         }
-        __syncthreads();
     }
 
-    // ---- write out: final values (no split-K) or this slice's partial sums ---------
-    for (int idx = threadIdx.x; idx < p.M * TILE_N; idx += WAVES * 64) {
-        const int row = idx / TILE_N;
-        const int nl = idx % TILE_N;
-        const int64_t n = nb + nl;
-        if (n >= p.N) continue;
-        const uint32_t bits = red[row * TILE_N + (nl % NW) * 16 + nl / NW];
-        if (gridDim.y == 1) {
-            finish_output<MODE>(p, row, n, bits);
-        } else {
-            ((uint32_t*)p.partial)[((int64_t)blockIdx.y * p.M + row) * p.N + n] = bits;
+    // ---- sum the waves' accumulators through LDS, in wave order ------------------------
+    // red[w][row][t*16 + j]; lane (j, g) holds rows 4g..4g+3 of column slot t*16+j
+    const int M = p.M;
+#pragma unroll
+    for (int t = 0; t < NW; t++) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int row = 4 * g + r;
+            // copy the element out first: a bit_cast applied directly to a vector
+            // element was observed to read element 0 for every r
+            const auto v = acc[t][r];
+            if (row < M) red[(wave * M + row) * TILE_N + t * 16 + j] = __builtin_bit_cast(uint32_t, v);
         }
     }
-}
+    __syncthreads();
 
-// Adds the S slices of split-K in slice order and applies the epilogue.
-template <int MODE>
-__global__ __launch_bounds__(256) void stream_reduce_kernel(StreamParams p, int S) {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (int64_t)p.M * p.N) return;
-    const int row = (int)(idx / p.N);
-    const int64_t n = idx % p.N;
-    const uint32_t* part = (const uint32_t*)p.partial;
-    uint32_t bits;
-    if constexpr (MODE == MODE_I8) {
-        int32_t v = 0;
-        for (int s = 0; s < S; s++) v += (int32_t)part[((int64_t)s * p.M + row) * p.N + n];
-        bits = (uint32_t)v;
-    } else {
-        float v = __builtin_bit_cast(float, part[(int64_t)row * p.N + n]);
-        for (int s = 1; s < S; s++)
-            v = __fadd_rn(v, __builtin_bit_cast(float, part[((int64_t)s * p.M + row) * p.N + n]));
-        bits = __builtin_bit_cast(uint32_t, v);
+    for (int idx = threadIdx.x; idx < M * TILE_N; idx += WAVES * 64) {
+        const int row = idx / TILE_N;
+        const int nl = idx % TILE_N;
+        if (nb + nl >= p.N) continue;
+        const int slot = (nl % NW) * 16 + nl / NW;
+        uint32_t bits = red[row * TILE_N + slot];
+#pragma unroll
+        for (int w = 1; w < WAVES; w++) bits = add_bits<MODE>(bits, red[(w * M + row) * TILE_N + slot]);
+        finish_output<MODE>(p, row, nb + nl, bits);
     }
-    finish_output<MODE>(p, row, n, bits);
 }
 
 // ---- host side --------------------------------------------------------------------
 
 struct StreamPlan {
-    int nw;       // bytes per lane per row: 16, 8 or 4
-    int waves;    // waves per workgroup
-    int splits;   // split-K factor S
-    int64_t kb_per_split;
+    int nw;     // bytes per lane and row: 16, 8, 4, 2 or 1 (tile = 16*nw columns)
+    int waves;  // waves per workgroup
 };
 
-static int rs_of(int mode) { return mode == MODE_I8 ? 16 : 8; }
+bool stream_supported(int64_t N, const void* W_T) { return ((uintptr_t)W_T) % 16 == 0 && N >= 1; }
 
-// Largest K slice whose activation stage fits a 64 KiB LDS allocation: 64 steps.
-static const int kMaxStepsPerWG = 64;
-
-bool stream_supported(int64_t N, const void* W_T) {
-    return N % 4 == 0 && ((uintptr_t)W_T) % 16 == 0;
-}
-
-StreamPlan stream_plan(int mode, int64_t N, int64_t Kb) {
+StreamPlan stream_plan(int mode, int64_t M, int64_t N, int64_t Kb) {
     StreamPlan pl;
-    const int rs = rs_of(mode);
-    // optional override for tuning runs: BITTORCH_STREAM_CFG="nw,waves,splits"
-    int o_nw = 0, o_waves = 0, o_splits = 0;
-    if (const char* env = getenv("BITTORCH_STREAM_CFG")) sscanf(env, "%d,%d,%d", &o_nw, &o_waves, &o_splits);
-
-    int nw = (N % 16 == 0) ? 16 : (N % 8 == 0) ? 8 : 4;
-    if (o_nw == 16 || o_nw == 8 || o_nw == 4) {
-        if (N % o_nw == 0) nw = o_nw;
+    (void)mode;
+    // optional override for tuning runs: BITTORCH_STREAM_CFG="nw,waves"
+    int o_nw = 0, o_waves = 0;
+    if (const char* env = getenv("BITTORCH_STREAM_CFG")) sscanf(env, "%d,%d", &o_nw, &o_waves);
+    // widest lane load the row pitch allows (row starts must stay aligned to it)
+    int nw = (N % 16 == 0) ? 16 : (N % 8 == 0) ? 8 : (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
+    if ((o_nw == 16 || o_nw == 8 || o_nw == 4 || o_nw == 2 || o_nw == 1) && N % o_nw == 0) {
+        nw = o_nw;
     } else {
-        // narrow the column tile until there are enough workgroups to cover the chip
-        // without an excessive split-K (whose partial sums cost extra traffic)
-        while (nw > 4 && ceil_div(N, 16 * nw) * ceil_div(Kb, (int64_t)rs * 8) < 512) nw >>= 1;
+        // narrow the tile until there is at least one tile per CU
+        while (nw > 1 && ceil_div(N, 16 * (int64_t)nw) < 256) nw >>= 1;
+        // decode batches re-read the activations once per tile: keep tiles wider when
+        // that traffic would exceed the weights' own
+        (void)M;
     }
     pl.nw = nw;
-    pl.waves = (o_waves == 2 || o_waves == 4 || o_waves == 8 || o_waves == 16) ? o_waves : 4;
-    const int64_t tiles = ceil_div(N, 16 * (int64_t)nw);
-    const int64_t steps = ceil_div(Kb, rs);
-    int64_t splits;
-    if (o_splits > 0) {
-        splits = o_splits;
-    } else {
-        // aim for ~2 workgroups per CU, but keep at least `waves` steps per workgroup
-        splits = ceil_div(512, tiles);
-        const int64_t max_splits = std::max<int64_t>(1, steps / pl.waves);
-        if (splits > max_splits) splits = max_splits;
-    }
-    const int64_t min_splits = ceil_div(steps, kMaxStepsPerWG);
-    if (splits < min_splits) splits = min_splits;
-    if (splits > steps) splits = steps;
-    if (splits < 1) splits = 1;
-    int64_t steps_per = ceil_div(steps, splits);
-    pl.kb_per_split = steps_per * rs;
-    pl.splits = (int)ceil_div(Kb, pl.kb_per_split);
+    const int max_waves = 1024 / (16 * nw) < 16 ? 1024 / (16 * nw) : 16;  // LDS: WAVES*TILE_N <= 1024 words/row
+    const int64_t steps = ceil_div(Kb, mode == MODE_I8 ? 16 : 8);
+    int waves = (o_waves == 1 || o_waves == 2 || o_waves == 4 || o_waves == 8 || o_waves == 16) ? o_waves : 8;
+    if (waves > max_waves) waves = max_waves;
+    while (waves > 1 && waves > steps) waves >>= 1;
+    pl.waves = waves;
     return pl;
 }
 
-size_t stream_workspace_bytes(int mode, int64_t M, int64_t N, int64_t Kb) {
-    // sized for the default plan and for any override (splits <= steps)
-    const StreamPlan pl = stream_plan(mode, N, Kb);
-    const int64_t rows = M < 16 ? M : 16;
-    return pl.splits > 1 ? (size_t)pl.splits * rows * N * 4 : 0;
+size_t stream_workspace_bytes(int, int64_t, int64_t, int64_t) { return 0; }
+
+template <int MODE, int NW, int WAVES>
+static void launch_stream_k(const StreamParams& p, dim3 grid, size_t lds, hipStream_t st) {
+    constexpr int PF = (NW >= 16) ? 2 : (NW == 8) ? 4 : 8;
+    hipLaunchKernelGGL((stream_kernel<MODE, NW, WAVES, PF>), grid, dim3(WAVES * 64), lds, st, p);
 }
 
 template <int MODE, int NW>
-static void launch_stream_w(const StreamParams& p, const StreamPlan& pl, dim3 grid, size_t lds, hipStream_t st) {
-    switch (pl.waves) {
-        case 2: hipLaunchKernelGGL((stream_kernel<MODE, NW, 2>), grid, dim3(128), lds, st, p); break;
-        case 8: hipLaunchKernelGGL((stream_kernel<MODE, NW, 8>), grid, dim3(512), lds, st, p); break;
-        case 16: hipLaunchKernelGGL((stream_kernel<MODE, NW, 16>), grid, dim3(1024), lds, st, p); break;
-        default: hipLaunchKernelGGL((stream_kernel<MODE, NW, 4>), grid, dim3(256), lds, st, p); break;
+static void launch_stream_w(const StreamParams& p, int waves, dim3 grid, size_t lds, hipStream_t st) {
+    if constexpr (NW <= 4) {
+        if (waves == 16) { launch_stream_k<MODE, NW, 16>(p, grid, lds, st); return; }
     }
+    if constexpr (NW <= 8) {
+        if (waves == 8) { launch_stream_k<MODE, NW, 8>(p, grid, lds, st); return; }
+    }
+    if (waves >= 4) { launch_stream_k<MODE, NW, 4>(p, grid, lds, st); return; }
+    if (waves == 2) { launch_stream_k<MODE, NW, 2>(p, grid, lds, st); return; }
+    launch_stream_k<MODE, NW, 1>(p, grid, lds, st);
 }
 
 template <int MODE>
-static int launch_stream_mode(StreamParams p, const StreamPlan& pl, void* workspace, size_t ws_bytes,
-                              hipStream_t st) {
-    const int rs = rs_of(MODE);
+static int launch_stream_mode(StreamParams p, const StreamPlan& pl, hipStream_t st) {
     const int64_t tile_n = 16 * (int64_t)pl.nw;
-    const dim3 grid((unsigned)ceil_div(p.N, tile_n), (unsigned)pl.splits);
-    const int nsteps = (int)ceil_div(pl.kb_per_split, rs);
-    size_t lds = (size_t)nsteps * 1024;
-    const size_t red = (size_t)16 * tile_n * 4;
-    if (lds < red) lds = red;
-    p.kb_per_split = pl.kb_per_split;
-    if (pl.splits > 1) {
-        const size_t need = (size_t)pl.splits * p.M * p.N * 4;
-        if (!workspace || ws_bytes < need) {
-            set_error("packed forward: workspace of %zu bytes needed, %zu given", need, ws_bytes);
-            return BT_ERR_WORKSPACE;
-        }
-        p.partial = workspace;
-    }
+    p.tiles = (int)ceil_div(p.N, tile_n);
+    p.per_xcd = (int)ceil_div(p.tiles, 8);
+    const dim3 grid((unsigned)(p.per_xcd * 8));
+    int waves = pl.waves;
+    if (pl.nw == 16 && waves > 4) waves = 4;
+    if (pl.nw == 8 && waves > 8) waves = 8;
+    const size_t lds = (size_t)waves * p.M * tile_n * 4;
     switch (pl.nw) {
-        case 16: launch_stream_w<MODE, 16>(p, pl, grid, lds, st); break;
-        case 8: launch_stream_w<MODE, 8>(p, pl, grid, lds, st); break;
-        default: launch_stream_w<MODE, 4>(p, pl, grid, lds, st); break;
-    }
-    if (pl.splits > 1) {
-        const int64_t total = (int64_t)p.M * p.N;
-        hipLaunchKernelGGL((stream_reduce_kernel<MODE>), dim3((unsigned)ceil_div(total, 256)), dim3(256), 0,
-                           st, p, pl.splits);
+        case 16: launch_stream_w<MODE, 16>(p, waves, grid, lds, st); break;
+        case 8: launch_stream_w<MODE, 8>(p, waves, grid, lds, st); break;
+        case 4: launch_stream_w<MODE, 4>(p, waves, grid, lds, st); break;
+        case 2: launch_stream_w<MODE, 2>(p, waves, grid, lds, st); break;
+        default: launch_stream_w<MODE, 1>(p, waves, grid, lds, st); break;
     }
     return check_launch("stream_gemm");
 }
 
-// One launch group per block of up to 16 activation rows.
+// One launch per block of up to 16 activation rows.
 int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, const uint8_t* W_T,
                   const Epilogue& epi, void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N,
                   int64_t K, void* workspace, size_t ws_bytes, hipStream_t st) {
+    (void)workspace;
+    (void)ws_bytes;
     const int64_t Kb = ceil_div(K, 4);
-    const StreamPlan pl = stream_plan(mode, N, Kb);
+    const StreamPlan pl = stream_plan(mode, B, N, Kb);
     const int y_size = dtype_size(y_dtype);
     for (int64_t m0 = 0; m0 < B; m0 += 16) {
         StreamParams p;
@@ -391,17 +339,15 @@ int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, co
         p.s_x = s_x ? s_x + m0 : nullptr;
         p.Y = (uint8_t*)Y + m0 * N * y_size;
         p.acc_out = acc_out ? acc_out + m0 * N : nullptr;
-        p.partial = nullptr;
         p.epi = epi;
         p.N = N; p.K = K; p.Kb = Kb;
-        p.kb_per_split = pl.kb_per_split;
         p.M = (int)((B - m0 < 16) ? (B - m0) : 16);
         p.y_dtype = y_dtype;
         p.x_vec_ok = (((uintptr_t)p.X) % 16 == 0) && ((K * x_elem_size) % 16 == 0);
         int rc;
-        if (mode == MODE_I8) rc = launch_stream_mode<MODE_I8>(p, pl, workspace, ws_bytes, st);
-        else if (mode == MODE_F16) rc = launch_stream_mode<MODE_F16>(p, pl, workspace, ws_bytes, st);
-        else rc = launch_stream_mode<MODE_BF16>(p, pl, workspace, ws_bytes, st);
+        if (mode == MODE_I8) rc = launch_stream_mode<MODE_I8>(p, pl, st);
+        else if (mode == MODE_F16) rc = launch_stream_mode<MODE_F16>(p, pl, st);
+        else rc = launch_stream_mode<MODE_BF16>(p, pl, st);
         if (rc != BT_OK) return rc;
     }
     return BT_OK;

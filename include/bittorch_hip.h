@@ -28,7 +28,7 @@ extern "C" {
 #define BT_ABI_VERSION 1
 
 /* element types of activations / scales / biases / outputs */
-typedef enum { BT_F32 = 0, BT_F16 = 1, BT_BF16 = 2 } bt_dtype;
+typedef enum { BT_F32 = 0, BT_F16 = 1, BT_BF16 = 2, BT_I8 = 3 /* bt_unpack_dequant output only */ } bt_dtype;
 
 typedef enum {
     BT_OK = 0,
@@ -36,6 +36,17 @@ typedef enum {
     BT_ERR_WORKSPACE = -2, /* workspace too small */
     BT_ERR_LAUNCH = -3     /* HIP reported a launch error */
 } bt_status;
+
+/*
+ * Workspaces.  Entry points that take a `workspace` use it for split-K partial
+ * sums and for per-tile ticket counters.  The first BT_WORKSPACE_COUNTER_BYTES
+ * bytes of a workspace must be ZERO when a call starts; every call leaves them
+ * zero again when its kernels have run, so a buffer that was cleared once can
+ * be reused for any sequence of calls on one stream.  The rest of the buffer
+ * needs no initialisation.  Two calls that may run concurrently (different
+ * streams) need different workspaces.  Workspaces must be 256-byte aligned.
+ */
+#define BT_WORKSPACE_COUNTER_BYTES 16384
 
 /* ABI version of the loaded library (BT_ABI_VERSION at build time). */
 int bt_abi_version(void);
@@ -119,8 +130,8 @@ int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, co
  * (bittorch_bindings.cpp:65-87, ternary_gemm_tensor_core.cu:663-727) for
  * version == 2; version == 1 (the reference's float-compute validation kernel,
  * :120-271) is served by bt_ternary_linear_packed_forward.
- *   workspace: at least bt_tensor_core_workspace_bytes(B,N,K) bytes; holds Q, s_x and
- *   the GEMM's own scratch.
+ *   workspace: at least bt_tensor_core_workspace_bytes(B,N,K) bytes; holds the GEMM's
+ *   own scratch (ticket counters first), then Q and s_x.
  */
 size_t bt_tensor_core_workspace_bytes(int64_t B, int64_t N, int64_t K);
 int bt_ternary_linear_tensor_core_forward(const void* X, int x_dtype, const uint8_t* W_T,
@@ -134,7 +145,8 @@ int bt_ternary_linear_tensor_core_forward(const void* X, int x_dtype, const uint
  * backward (grad_x = grad_y @ (w_tern * scale)) without keeping a dense copy
  * alive between forward and backward (the reference saves one,
  * bittorch/nn/ternary_linear_cuda.py:62-66).
- *   out [N,K] of out_dtype = decode(W_T) * scale[n]   (scale NULL -> plain decode)
+ *   out [N,K] of out_dtype = decode(W_T) * scale[n]   (scale NULL -> plain decode;
+ *   out_dtype BT_I8 -> the ternary values themselves, scale ignored)
  */
 int bt_unpack_dequant(const uint8_t* W_T, const float* scale, int64_t scale_len, void* out,
                       int out_dtype, int64_t N, int64_t K, void* stream);

@@ -133,8 +133,8 @@ def test_packed_forward_known_answers(oracle):
 
 
 def test_packed_forward_stream_configs_agree(oracle):
-    """Every tile width / wave count / split-K of the streaming kernel gives the same sums
-    (int-exact decode; fp32 sums differ only by association)."""
+    """Every tile width / wave count of the streaming kernel gives the same sums
+    (exact decode; fp32 sums differ only by association)."""
     from bittorch_amd import _C
     from bittorch_amd.quant import pack_ternary_transposed
     announce("packed_forward stream configs")
@@ -144,7 +144,7 @@ def test_packed_forward_stream_configs_agree(oracle):
     scale = torch.ones(512, dtype=torch.float16).cuda()
     truth = oracle.linear_packed(f32np(x), packed.cpu().numpy(), f32np(scale), 1024, f64=True)
     try:
-        for cfg in ("16,4,1", "16,2,4", "8,8,2", "4,4,8", "4,16,1", "8,4,16", "16,16,3"):
+        for cfg in ("16,4", "16,1", "8,8", "8,2", "4,4", "4,16", "2,8", "2,16", "1,1", "1,4", "1,16"):
             os.environ["BITTORCH_STREAM_CFG"] = cfg
             y = _C.ternary_linear_packed_forward(x, packed, scale, None, 1024)
             torch.cuda.synchronize()
