@@ -1,0 +1,268 @@
+#!/usr/bin/env python3
+"""Benchmark of the ternary-linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" is one pass of the decode GEMV of BASELINE.json's config 2 through the
+C-ABI library: x fp16 [1,4096] times packed ternary W [4096,4096] (per-tensor fp32
+scale, fp16 bias).  The steps walk round-robin over distinct weight buffers whose
+total size exceeds the 256 MB Infinity Cache, so every step streams its 4 MiB of
+packed weights from HBM.  W warm-up steps, then exactly K steps (captured in one
+HIP graph so that host launch overhead is not what is measured) are timed between
+two device synchronisations.  Prints ONE JSON line.
+
+The same line carries the roofline of the dominant kernel (HIP-event timed over the
+timed region), the CPU oracle timed on the host cores beside it, and the secondary
+figures of the metric (int8 TOPS at M=2048, small-batch decode, quantize+pack).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
+INT8_PEAK_TOPS = 5000.0     # MI355X dense int8 MFMA
+METRIC = "packed ternary GEMM GB/s (M=1) & int8 TOPS (M=2048), % of roofline, 1 GPU"
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU baseline sample length")
+    return ap.parse_args()
+
+
+def graph_time(fn, steps, warmup, torch):
+    """(wall ms, event ms) for `steps` calls of fn(i) replayed as one HIP graph."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for i in range(warmup):
+            fn(i)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for i in range(steps):
+            fn(i)
+    graph.replay()  # untimed: first replay uploads the graph
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return wall_ms, e0.elapsed_time(e1)
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU's throughput; --gpus {args.gpus} is not supported "
+              "(this path has no multi-GPU part: it shards by output columns without collectives)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from bittorch_amd import _C  # ImportError if the HIP library is not built
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    torch.manual_seed(0)
+
+    # ---- config 2: decode GEMV -------------------------------------------------------
+    N = K = 4096
+    weight_bytes = N * (K // 4)
+    nsets = 128  # 512 MiB of packed weights > 256 MB Infinity Cache
+    g = torch.Generator().manual_seed(0)
+    w0 = (torch.randn(N, K, generator=g) * 0.02).to(dev)
+    x = torch.randn(1, K, generator=g).half().to(dev)
+    bias = (torch.randn(N, generator=g) * 0.01).half().to(dev)
+    packed0, scale0, _ = _C.ternary_quantize_pack(w0, 0.05, per_channel=False)
+    scale = scale0.reshape(1).float()
+    zero_frac = float((_C.unpack_dequant(packed0, K, out_dtype=torch.int8) == 0).float().mean())
+    packs = [packed0]
+    for _ in range(nsets - 1):
+        wi = torch.randn(N, K, device=dev) * 0.02
+        packs.append(_C.ternary_quantize_pack(wi, 0.05, per_channel=False)[0])
+    del wi
+    torch.cuda.synchronize()
+
+    def step(i):
+        return _C.ternary_linear_packed_forward(x, packs[i % nsets], scale, bias, K)
+
+    wall_ms, ev_ms = graph_time(step, args.steps, args.warmup, torch)
+    ms_per_step = wall_ms / args.steps
+    kernel_us = ev_ms / args.steps * 1e3
+    value = weight_bytes / (ms_per_step * 1e-3) / 1e9
+    achieved = weight_bytes / (kernel_us * 1e-6) / 1e9
+
+    out = {
+        "metric": METRIC,
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16 x 2-bit ternary -> f32 accumulate",
+        "data": "synthetic (seed 0; N(0,0.02) master weights quantized with threshold 0.05, "
+                f"{zero_frac * 100:.1f}% zeros; N(0,1) activations)",
+        "config": {
+            "workload": "config 2 decode GEMV: x fp16 [1,4096] x packed ternary W [4096,4096], "
+                        "per-tensor fp32 scale, fp16 bias",
+            "M": 1, "N": N, "K": K,
+            "weight_sets": nsets,
+            "weight_bytes_per_step": weight_bytes,
+            "timing": "one HIP graph of all steps, replayed once between synchronisations",
+        },
+        "roofline": {
+            "kernel": "bt::stream_kernel (fp16 activations)",
+            "bound": "hbm",
+            "achieved": round(achieved, 2),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "launch_us": round(kernel_us, 3),
+            "algorithmic_bytes_per_launch": weight_bytes,
+        },
+    }
+
+    # ---- secondary figures of the metric ------------------------------------------------
+    if not args.no_extra:
+        extra = {}
+
+        def rand_packed(n, k, count):
+            outp = []
+            for _ in range(count):
+                c = torch.randint(0, 3, (4, (k + 3) // 4, n), device=dev, dtype=torch.uint8)
+                outp.append((c[0] | (c[1] << 2) | (c[2] << 4) | (c[3] << 6)).contiguous())
+            return outp
+
+        def acts(m, k, outliers):
+            a = torch.randn(m, k, device=dev)
+            if outliers:
+                a = torch.where(torch.rand(m, k, device=dev) < 0.001, a * 20, a)
+            return a.bfloat16()
+
+        # config 4: prefill, int8 activations on the matrix cores
+        for (m, n, k) in ((2048, 4096, 4096), (2048, 11008, 4096)):
+            ws = rand_packed(n, k, 2)
+            xa = acts(m, k, True)
+            sc = torch.rand(n, device=dev) * 0.05 + 0.01
+            q, s = _C.act_quant_int8(xa)
+            steps = 50
+            _, ev = graph_time(lambda i: _C.ternary_gemm_int8(q, s, ws[i % 2], sc, None, k,
+                                                              out_dtype=torch.bfloat16), steps, 5, torch)
+            _, ev_full = graph_time(lambda i: _C.ternary_linear_tensor_core_forward(xa, ws[i % 2], sc, None, k, 2),
+                                    steps, 5, torch)
+            ops = 2.0 * m * n * k
+            tops = ops / (ev / steps * 1e-3) / 1e12
+            extra[f"prefill_int8_M{m}_N{n}_K{k}"] = {
+                "gemm_us": round(ev / steps * 1e3, 2),
+                "tops": round(tops, 1),
+                "frac_of_int8_peak": round(tops / INT8_PEAK_TOPS, 4),
+                "with_act_quant_us": round(ev_full / steps * 1e3, 2),
+                "tops_with_act_quant": round(ops / (ev_full / steps * 1e-3) / 1e12, 1),
+            }
+            del ws, xa, q, s
+        # config 3: small-batch decode, int8 activations
+        for (m, n, k) in ((16, 11008, 4096), (16, 4096, 11008)):
+            cnt = max(2, int(400e6 // (n * k // 4)))
+            ws = rand_packed(n, k, cnt)
+            xa = acts(m, k, False)
+            sc = torch.rand(n, device=dev) * 0.05 + 0.01
+            steps = 200
+            _, ev = graph_time(lambda i: _C.ternary_linear_tensor_core_forward(xa, ws[i % cnt], sc, None, k, 2),
+                               steps, 10, torch)
+            us = ev / steps * 1e3
+            gbps = n * ((k + 3) // 4) / (us * 1e-6) / 1e9
+            extra[f"decode_int8_M{m}_N{n}_K{k}"] = {
+                "us": round(us, 2), "weight_GBps": round(gbps, 1),
+                "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
+                "note": "activation quantization + GEMM per step",
+            }
+            del ws
+        # quantize + pack of fp32 master weights
+        for (n, k) in ((4096, 4096), (11008, 4096)):
+            cnt = max(2, int(600e6 // (n * k * 4)))
+            masters = [torch.randn(n, k, device=dev) * 0.02 for _ in range(cnt)]
+            steps = 40
+            _, ev = graph_time(lambda i: _C.ternary_quantize_pack(masters[i % cnt], 0.05, True), steps, 4, torch)
+            us = ev / steps * 1e3
+            nbytes = 4 * n * k + n * ((k + 3) // 4) + 4 * n
+            extra[f"quantize_pack_N{n}_K{k}"] = {
+                "us": round(us, 2), "GBps": round(nbytes / (us * 1e-6) / 1e9, 1),
+                "frac_of_hbm_peak": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+            }
+            del masters
+        out["secondary"] = extra
+
+    # ---- CPU baseline: the oracle (a scalar C port of the reference arithmetic) -------------
+    if not args.no_cpu:
+        from oracle import oracle as o
+        o.build()
+        x_np = x.float().cpu().numpy()
+        p_np = packed0.cpu().numpy()
+        s_np = scale.cpu().numpy()
+        b_np = bias.float().cpu().numpy()
+        threads = o.num_threads()
+        o.linear_packed(x_np, p_np, s_np, K, b_np)  # warm
+        t0 = time.perf_counter()
+        iters = 0
+        while time.perf_counter() - t0 < args.cpu_seconds:
+            o.linear_packed(x_np, p_np, s_np, K, b_np)
+            iters += 1
+        dt = (time.perf_counter() - t0) / iters
+        out["cpu_baseline"] = {
+            "value": round(weight_bytes / dt / 1e9, 4),
+            "unit": "GB/s",
+            "cores": threads,
+            "kind": "port",
+            "sample": f"{iters} passes of the same M=1 4096x4096 GEMV through oracle/bt_oracle.c "
+                      f"(OpenMP over output columns, {threads} threads), {args.cpu_seconds:.0f} s",
+            "ms_per_step": round(dt * 1e3, 3),
+        }
+        # the reference's own CPU route (unpack + dense product) in plain torch, for scale
+        torch.set_num_threads(max(1, min(threads, os.cpu_count() or 1)))
+        from bittorch_amd.nn import TernaryLinearInference
+        layer = TernaryLinearInference(K, N, packed0.cpu(), scale.cpu().expand(N).contiguous(), bias.float().cpu())
+        xc = x.float().cpu()
+        layer(xc)
+        t0 = time.perf_counter()
+        it2 = 0
+        while time.perf_counter() - t0 < 3.0:
+            layer(xc)
+            it2 += 1
+        dt2 = (time.perf_counter() - t0) / it2
+        out["cpu_baseline"]["torch_unpack_linear_ms_per_step"] = round(dt2 * 1e3, 3)
+        out["cpu_baseline"]["torch_unpack_linear_GBps"] = round(weight_bytes / dt2 / 1e9, 4)
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

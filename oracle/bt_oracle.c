@@ -80,6 +80,14 @@ static float round_to_dtype(float f, int dtype) {
     return f;
 }
 
+/* threads the OpenMP loops below will use (reported with the CPU baseline) */
+#ifdef _OPENMP
+#include <omp.h>
+int bto_num_threads(void) { return omp_get_max_threads(); }
+#else
+int bto_num_threads(void) { return 1; }
+#endif
+
 /* exported so tests can check the helpers against torch's casts */
 float bto_round_to_dtype(float f, int dtype) { return round_to_dtype(f, dtype); }
 

@@ -56,6 +56,13 @@ def lib() -> ctypes.CDLL:
     return _lib
 
 
+def num_threads() -> int:
+    """OpenMP threads the oracle's loops run on."""
+    fn = lib().bto_num_threads
+    fn.restype = ctypes.c_int
+    return int(fn())
+
+
 def _p(a: Optional[np.ndarray]):
     return None if a is None else a.ctypes.data_as(_vp)
 
