@@ -1,0 +1,181 @@
+"""GPU parity at the module boundary: TernaryLinear / TernaryLinearCUDA /
+TernaryLinearInference on the HIP kernels vs the plain torch backend and the oracle
+(what the reference pins in tests/test_ternary_cuda.py, tests/test_gradient_consistency.py,
+tests/test_amp.py, tests/test_packed_kernel.py:285-347, tests/test_robustness.py)."""
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+from conftest import announce
+from _util import f32np, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _pair(in_f, out_f, **kw):
+    from bittorch_amd.nn import TernaryLinear
+    torch.manual_seed(0)
+    hip = TernaryLinear(in_f, out_f, backend="cuda", **kw).cuda()
+    ref = TernaryLinear(in_f, out_f, backend="python", **kw).cuda()
+    ref.load_state_dict(hip.state_dict())
+    return hip, ref
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1), (4, 16, 8), (7, 33, 17), (32, 512, 256), (17, 123, 67),
+                                   (2, 5, 64, 32), (8, 1024, 1024)])
+def test_module_forward_matches_python_backend(shape):
+    *lead, in_f, out_f = shape
+    announce("module forward", shape)
+    hip, ref = _pair(in_f, out_f)
+    x = torch.randn(*lead, in_f, device="cuda")
+    y, y_ref = hip(x), ref(x)
+    assert y.shape == y_ref.shape == (*lead, out_f)
+    assert torch.allclose(y, y_ref, rtol=1e-4, atol=1e-4)
+
+
+def test_config1_plumbing_gpu(oracle):
+    """Config 1 on the GPU: TernaryLinear(512->256, bias), batch 32, fp32, seed 0."""
+    from bittorch_amd.nn import TernaryLinear, create_ternary_linear_inference
+    announce("config1 gpu")
+    g = torch.Generator().manual_seed(0)
+    layer = TernaryLinear(512, 256, bias=True, threshold_factor=0.05)
+    with torch.no_grad():
+        layer.weight.copy_(torch.randn(256, 512, generator=g) * 0.02)
+        layer.bias.copy_(torch.randn(256, generator=g) * 0.01)
+    x = torch.randn(32, 512, generator=g)
+    o_t, o_s = oracle.ternary_quantize(layer.weight.detach().numpy(), 0.05, True)
+    o_p, _ = oracle.pack_ternary_transposed(o_t)
+    ref = oracle.linear_packed(x.numpy(), o_p, o_s, 512, layer.bias.detach().numpy())
+    layer = layer.cuda()
+    y = layer(x.cuda())
+    np.testing.assert_array_equal(f32np(y), ref)  # fp32 generic kernel: oracle's k order
+    inf = create_ternary_linear_inference(512, 256, layer.weight.detach(), layer.bias.detach())
+    np.testing.assert_array_equal(inf.weight_packed.cpu().numpy(), o_p)
+    np.testing.assert_array_equal(inf.scale.cpu().numpy(), o_s)
+    np.testing.assert_array_equal(f32np(inf(x.cuda())), ref)
+
+
+def test_gradients_match_python_backend():
+    announce("gradients")
+    for (b, in_f, out_f, bias) in [(8, 64, 32, True), (5, 33, 17, False), (16, 256, 128, True)]:
+        hip, ref = _pair(in_f, out_f, bias=bias)
+        x1 = torch.randn(b, in_f, device="cuda", requires_grad=True)
+        x2 = x1.detach().clone().requires_grad_(True)
+        g = torch.randn(b, out_f, device="cuda")
+        (hip(x1) * g).sum().backward()
+        (ref(x2) * g).sum().backward()
+        assert torch.allclose(hip.weight.grad, ref.weight.grad, rtol=1e-4, atol=1e-4)
+        assert torch.allclose(x1.grad, x2.grad, rtol=1e-4, atol=1e-4)
+        if bias:
+            assert torch.allclose(hip.bias.grad, ref.bias.grad, rtol=1e-4, atol=1e-4)
+        cos = nn.functional.cosine_similarity(hip.weight.grad.flatten(), ref.weight.grad.flatten(), dim=0)
+        assert cos > 0.99
+
+
+def test_amp_autocast_forward_backward():
+    from bittorch_amd.nn import TernaryLinearCUDA
+    announce("amp")
+    torch.manual_seed(0)
+    layer = TernaryLinearCUDA(256, 128).cuda()
+    x = torch.randn(16, 256, device="cuda", requires_grad=True)
+    y32 = layer(x)
+    with torch.autocast("cuda", dtype=torch.float16):
+        y16 = layer(x)
+    assert y16.dtype == torch.float16 and torch.isfinite(y16).all()
+    assert torch.allclose(y16.float(), y32, rtol=1e-2, atol=1e-2)
+    scaler_loss = y16.float().pow(2).mean()
+    scaler_loss.backward()
+    assert torch.isfinite(layer.weight.grad).all() and torch.isfinite(x.grad).all()
+    assert layer.weight.grad.dtype == torch.float32
+
+
+def test_half_and_bf16_modules():
+    from bittorch_amd.nn import TernaryLinear
+    announce("16-bit modules")
+    for dtype in (torch.float16, torch.bfloat16):
+        torch.manual_seed(1)
+        hip = TernaryLinear(512, 256).cuda().to(dtype)
+        x = torch.randn(4, 512, device="cuda", dtype=dtype)
+        y = hip(x)
+        assert y.dtype == dtype
+        w_t, s = hip.get_quantized_weight()
+        ref = x.float() @ (w_t.float() * s.float().unsqueeze(1)).t() + hip.bias.float()
+        assert rel_err(f32np(y), f32np(ref)) < 1e-2
+
+
+def test_inference_module_gpu_matches_cpu_route():
+    from bittorch_amd.nn import TernaryLinearInference, create_ternary_linear_inference
+    from bittorch_amd.quant import ternary_quantize
+    announce("inference module")
+    for (b, in_f, out_f) in [(1, 768, 768), (32, 1024, 4096), (3, 13, 5), (16, 4096, 4096), (8, 4096, 11008)]:
+        torch.manual_seed(in_f)
+        w = torch.randn(out_f, in_f) * 0.02
+        bias = torch.randn(out_f) * 0.01
+        w_t, s = ternary_quantize(w)
+        cpu_mod = TernaryLinearInference.from_unpacked(w_t, s, bias)
+        gpu_mod = create_ternary_linear_inference(in_f, out_f, w.cuda(), bias.cuda())
+        assert torch.equal(gpu_mod.weight_packed.cpu(), cpu_mod.weight_packed)
+        assert torch.equal(gpu_mod.scale.cpu(), cpu_mod.scale)
+        x = torch.randn(b, in_f)
+        for dtype, tol in ((torch.float32, 1e-3), (torch.float16, 1e-2), (torch.bfloat16, 1e-2)):
+            y = gpu_mod.to(dtype)(x.cuda().to(dtype)) if dtype != torch.float32 else gpu_mod(x.cuda())
+            truth = x.to(dtype).double() @ (w_t.double() * s.to(dtype).double().unsqueeze(1)).t() + bias.to(dtype).double()
+            assert rel_err(f32np(y), truth.numpy()) < tol, (b, in_f, out_f, dtype)
+        gpu_mod.float()
+    # moving a CPU-built module to the GPU keeps the buffers and works
+    moved = cpu_mod.cuda()
+    assert moved.weight_packed.is_cuda and moved(x.cuda()).shape == (b, out_f)
+
+
+def test_functional_ops():
+    import bittorch_amd as bt
+    from bittorch_amd.quant import pack_ternary_transposed, ternary_quantize
+    announce("functional ops")
+    torch.manual_seed(3)
+    w = torch.randn(64, 128, device="cuda")
+    bias = torch.randn(64, device="cuda")
+    x = torch.randn(4, 7, 128, device="cuda")
+    w_t, s = ternary_quantize(w)
+    ref = x @ (w_t * s.unsqueeze(1)).t() + bias
+    y1 = bt.ops.ternary_linear(x, w, bias)
+    y2 = bt.ops.ternary_linear_forward_cuda(x, w_t.to(torch.int8), s, bias)
+    y3 = bt.ops.ternary_linear_packed_forward(x, pack_ternary_transposed(w_t)[0], s, 128, bias)
+    for y in (y1, y2, y3):
+        assert y.shape == (4, 7, 64) and torch.allclose(y, ref, rtol=1e-4, atol=1e-4)
+    x2 = x.reshape(-1, 128)
+    y4 = bt.ops.ternary_linear_tensor_core_forward(x2, pack_ternary_transposed(w_t)[0], s, 128, bias, version=1)
+    assert torch.allclose(y4, ref.reshape(-1, 64), rtol=1e-4, atol=1e-4)
+    y5 = bt.ops.ternary_linear_tensor_core_forward(x2, pack_ternary_transposed(w_t)[0], s, 128, bias, version=2)
+    assert rel_err(f32np(y5), f32np(ref.reshape(-1, 64))) < 2e-2
+    # float64 inputs are served too (reference dispatches double)
+    y6 = bt.ops.ternary_linear_packed_forward(x.double(), pack_ternary_transposed(w_t)[0], s.double(), 128, bias.double())
+    assert y6.dtype == torch.float64 and torch.allclose(y6, ref.double(), rtol=1e-4, atol=1e-4)
+    assert bt.ops.has_packed_cuda_support()
+
+
+def test_determinism_and_batched_equals_looped():
+    hip, _ = _pair(256, 128)
+    announce("determinism")
+    x = torch.randn(16, 256, device="cuda")
+    y1, y2 = hip(x), hip(x)
+    assert torch.equal(y1, y2)
+    rows = torch.cat([hip(x[i:i + 1]) for i in range(16)])
+    assert torch.allclose(rows, y1, atol=1e-6)
+    assert torch.equal(hip(torch.zeros(3, 256, device="cuda")), hip.bias.detach().expand(3, 128))
+
+
+def test_xor_training_on_gpu():
+    from bittorch_amd.nn import TernaryLinearCUDA
+    announce("xor gpu")
+    torch.manual_seed(42)
+    model = nn.Sequential(TernaryLinearCUDA(2, 16), nn.ReLU(), TernaryLinearCUDA(16, 1)).cuda()
+    xs = torch.tensor([[0.0, 0.0], [0.0, 1.0], [1.0, 0.0], [1.0, 1.0]], device="cuda")
+    ys = torch.tensor([[0.0], [1.0], [1.0], [0.0]], device="cuda")
+    opt = torch.optim.Adam(model.parameters(), lr=0.01)
+    for _ in range(1500):
+        opt.zero_grad()
+        loss = nn.functional.binary_cross_entropy_with_logits(model(xs), ys)
+        loss.backward()
+        opt.step()
+    assert ((model(xs) > 0).float() == ys).all()

@@ -1,0 +1,261 @@
+"""Pins the CPU oracle (oracle/bt_oracle.c) without the GPU:
+reference-held known answers (tests/golden/known_answers.json), brute force in
+pure Python on tiny inputs, closed forms / invariants, and torch's CPU ops
+executing the reference's formula as an independent library routine."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from _util import random_ternary, seeded_acts, seeded_weights
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "known_answers.json")) as fh:
+    GOLD = json.load(fh)
+
+
+def _filled(spec):
+    return np.full(spec["shape"], spec["value"], dtype=np.float32)
+
+
+# ---------------------------------------------------------------- quantizer (a1)
+@pytest.mark.parametrize("case", GOLD["quantize"], ids=lambda c: c["cite"])
+def test_quantize_known_answers(oracle, case):
+    w = np.array(case["weight"], dtype=np.float32) if "weight" in case else _filled(case["weight_fill"])
+    w_tern, scale = oracle.ternary_quantize(w, case["tf"], case["per_channel"])
+    if "scale" in case:
+        np.testing.assert_allclose(scale, np.array(case["scale"], dtype=np.float32), rtol=1e-6)
+        np.testing.assert_array_equal(w_tern, np.array(case["w_tern"]))
+    else:
+        assert (scale == case["scale_fill"]).all() and (w_tern == case["w_tern_fill"]).all()
+
+
+def test_quantize_brute_force(oracle):
+    """Element-by-element Python evaluation of the definition on small tensors."""
+    rng = np.random.default_rng(0)
+    for per_channel in (True, False):
+        w = rng.standard_normal((5, 7)).astype(np.float32)
+        w[2, 3] = 0.0
+        w[4] = 0.0
+        got_t, got_s = oracle.ternary_quantize(w, 0.3, per_channel)
+        tf = np.float32(0.3)
+        for n in range(5):
+            s = np.abs(w[n]).max() if per_channel else np.abs(w).max()
+            s = max(np.float32(s), np.float32(1e-8))
+            assert got_s[n if per_channel else 0] == s
+            thr = np.float32(tf * s)
+            for k in range(7):
+                expect = 0 if not (abs(w[n, k]) > thr) else (1 if w[n, k] > 0 else -1)
+                assert got_t[n, k] == expect
+
+
+def test_quantize_edge_semantics(oracle):
+    # tf = 0: only true zeros map to 0 (reference tests/test_ternary_quant.py:180-189)
+    w = seeded_weights(32, 64, seed=1, std=1.0).numpy()
+    w[0, 0] = 0.0
+    t, _ = oracle.ternary_quantize(w, 0.0)
+    assert (t == 0).sum() == (w == 0).sum()
+    # tf = 1: nothing exceeds its own row maximum (tests/test_ternary_quant.py:191-197)
+    t, _ = oracle.ternary_quantize(w, 1.0)
+    assert (t == 0).all()
+    # signs are preserved, values are ternary (:17-27, :80-87)
+    t, _ = oracle.ternary_quantize(w, 0.05)
+    assert set(np.unique(t)) <= {-1, 0, 1}
+    assert ((t == 0) | (np.sign(w) == t)).all()
+    # all-zero row: scale is the floor, codes are zero
+    z = np.zeros((2, 8), dtype=np.float32)
+    t, s = oracle.ternary_quantize(z, 0.05)
+    assert (t == 0).all() and (s == np.float32(1e-8)).all()
+    # threshold compare is strict: an element equal to the threshold is dropped
+    w2 = np.array([[1.0, 0.5, -0.5, 0.25]], dtype=np.float32)
+    t, _ = oracle.ternary_quantize(w2, 0.5)
+    np.testing.assert_array_equal(t, [[1, 0, 0, 0]])
+
+
+@pytest.mark.parametrize("dtype,tag", [(torch.float32, 0), (torch.float16, 1), (torch.bfloat16, 2)])
+@pytest.mark.parametrize("per_channel", [True, False])
+def test_quantize_matches_torch_ops(oracle, dtype, tag, per_channel):
+    """torch's CPU kernels evaluating abs/max/clamp/mul/gt/sign/where fix the rounding of
+    the threshold (fl(0.05f * scale) in the weight dtype); the oracle must agree bit for bit."""
+    from bittorch_amd.quant import ternary_quantize
+    for seed, (n, k), std in ((0, (64, 128), 0.02), (1, (7, 33), 1.0), (2, (16, 1000), 1e-4)):
+        w = seeded_weights(n, k, seed=seed, std=std, dtype=dtype)
+        ref_t, ref_s = ternary_quantize(w, 0.05, per_channel)
+        got_t, got_s = oracle.ternary_quantize(w.float().numpy(), 0.05, per_channel, dtype=tag)
+        np.testing.assert_array_equal(got_t, ref_t.float().numpy().astype(np.int8))
+        np.testing.assert_array_equal(got_s.reshape(-1), ref_s.float().reshape(-1).numpy())
+
+
+# ---------------------------------------------------------------- codec (a3-a5)
+@pytest.mark.parametrize("case", GOLD["pack"], ids=lambda c: c["cite"])
+def test_pack_known_answers(oracle, case):
+    w = np.array(case["w_tern"], dtype=np.int8) if "w_tern" in case else _filled(case["w_tern_fill"]).astype(np.int8)
+    packed, k = oracle.pack_ternary(w)
+    assert packed.dtype == np.uint8 and k == w.shape[1]
+    if "packed" in case:
+        np.testing.assert_array_equal(packed, np.array(case["packed"], dtype=np.uint8))
+    if "packed_fill" in case:
+        assert (packed == case["packed_fill"]).all()
+    if "packed_shape" in case:
+        assert list(packed.shape) == case["packed_shape"]
+    np.testing.assert_array_equal(oracle.unpack_ternary(packed, k), w)
+    packed_t, _ = oracle.pack_ternary_transposed(w)
+    np.testing.assert_array_equal(packed_t, packed.T)
+    np.testing.assert_array_equal(oracle.unpack_ternary_transposed(packed_t, k), w)
+
+
+def test_pack_brute_force_and_roundtrip(oracle):
+    for (n, k) in [(1, 1), (3, 5), (7, 13), (4, 8), (32, 64), (9, 31)]:
+        w = random_ternary(n, k, seed=n * 17 + k).numpy()
+        packed, _ = oracle.pack_ternary(w)
+        assert packed.shape == (n, (k + 3) // 4)
+        for r in range(n):
+            for kb in range((k + 3) // 4):
+                byte = 0
+                for i in range(4):
+                    kk = 4 * kb + i
+                    v = int(w[r, kk]) if kk < k else 0
+                    byte |= {0: 0, 1: 1, -1: 2}[v] << (2 * i)
+                assert packed[r, kb] == byte
+        np.testing.assert_array_equal(oracle.unpack_ternary(packed, k), w)
+
+
+def test_unpack_reserved_code_is_zero(oracle):
+    packed = np.array([[0xFF, 0b11100100]], dtype=np.uint8)  # codes 3,3,3,3 | 0,1,2,3
+    np.testing.assert_array_equal(oracle.unpack_ternary(packed, 8), [[0, 0, 0, 0, 0, 1, -1, 0]])
+
+
+def test_codec_matches_torch_host_functions(oracle):
+    from bittorch_amd.quant import pack_ternary, pack_ternary_transposed, unpack_ternary_transposed
+    for (n, k) in [(256, 512), (17, 123), (5, 6)]:
+        w = random_ternary(n, k, seed=3)
+        np.testing.assert_array_equal(oracle.pack_ternary(w.numpy())[0], pack_ternary(w)[0].numpy())
+        pt = pack_ternary_transposed(w)[0]
+        np.testing.assert_array_equal(oracle.pack_ternary_transposed(w.numpy())[0], pt.numpy())
+        np.testing.assert_array_equal(oracle.unpack_ternary_transposed(pt.numpy(), k),
+                                      unpack_ternary_transposed(pt, k).numpy())
+
+
+@pytest.mark.parametrize("case", GOLD["sizes"], ids=lambda c: c["cite"])
+def test_packed_size_known_answers(case):
+    from bittorch_amd.quant import get_packed_size
+    assert get_packed_size(case["out_features"], case["in_features"]) == case["packed_size"]
+
+
+# ---------------------------------------------------------------- float linear (a6)
+@pytest.mark.parametrize("case", GOLD["matmul"], ids=lambda c: c["cite"])
+def test_linear_known_answers(oracle, case):
+    w = np.array(case["weights"], dtype=np.int8)
+    packed_t, k = oracle.pack_ternary_transposed(w)
+    x = np.array(case["input"], dtype=np.float32)
+    scale = np.array(case["scales"], dtype=np.float32)
+    expect = np.array(case["output"], dtype=np.float32)
+    np.testing.assert_array_equal(oracle.linear_packed(x, packed_t, scale, k), expect)
+    np.testing.assert_array_equal(oracle.linear_unpacked(x, w, scale), expect)
+    np.testing.assert_array_equal(oracle.linear_packed(x, packed_t, scale, k, f64=True), expect)
+
+
+def test_linear_textbook_and_special_cases(oracle):
+    for (b, n, k) in [(4, 8, 16), (3, 33, 17), (1, 1, 1), (8, 64, 130)]:
+        w = random_ternary(n, k, seed=k).numpy()
+        x = seeded_acts(b, k, seed=1).numpy()
+        rng = np.random.default_rng(k)
+        scale = rng.random(n).astype(np.float32)
+        bias = rng.standard_normal(n).astype(np.float32)
+        packed_t, _ = oracle.pack_ternary_transposed(w)
+        truth = x.astype(np.float64) @ (w.astype(np.float64) * scale[:, None].astype(np.float64)).T + bias
+        y64 = oracle.linear_packed(x, packed_t, scale, k, bias, f64=True)
+        np.testing.assert_allclose(y64, truth, rtol=1e-12, atol=1e-12)
+        y32 = oracle.linear_packed(x, packed_t, scale, k, bias)
+        np.testing.assert_allclose(y32, truth, rtol=1e-4, atol=1e-4)
+        np.testing.assert_array_equal(oracle.linear_unpacked(x, w, scale, bias), y32)
+        # per-tensor scale broadcasts
+        y1 = oracle.linear_packed(x, packed_t, scale[:1], k, bias)
+        np.testing.assert_array_equal(y1, oracle.linear_packed(x, packed_t, np.full(n, scale[0], np.float32), k, bias))
+    # all-zero weights give the bias, all-ones weights give the row sums
+    # (reference tests/test_ternary_cuda.py:216-247)
+    x = seeded_acts(4, 16, seed=2).numpy()
+    bias = np.arange(8, dtype=np.float32)
+    z, _ = oracle.pack_ternary_transposed(np.zeros((8, 16), np.int8))
+    np.testing.assert_array_equal(oracle.linear_packed(x, z, np.ones(8, np.float32), 16, bias), np.tile(bias, (4, 1)))
+    o1, _ = oracle.pack_ternary_transposed(np.ones((8, 16), np.int8))
+    got = oracle.linear_packed(x, o1, np.ones(8, np.float32), 16)
+    np.testing.assert_allclose(got, np.tile(x.sum(1, keepdims=True), (1, 8)), rtol=1e-5, atol=1e-5)
+
+
+def test_linear_sequential_fp32_order(oracle):
+    """The fp32 path adds in ascending k: a case where the order is visible."""
+    x = np.array([[1e8, 1.0, -1e8, 1.0]], dtype=np.float32)
+    w = np.ones((1, 4), dtype=np.int8)
+    p, _ = oracle.pack_ternary_transposed(w)
+    # ((1e8 + 1) - 1e8) + 1 = 1 in fp32 (the first +1 is absorbed), 2 in exact arithmetic
+    assert oracle.linear_packed(x, p, np.ones(1, np.float32), 4)[0, 0] == 1.0
+    assert oracle.linear_packed(x, p, np.ones(1, np.float32), 4, f64=True)[0, 0] == 2.0
+
+
+# ---------------------------------------------------------------- int8 path (a7)
+def test_act_quant_brute_force(oracle):
+    import math
+    x = np.array([[0.5, -1.0, 2.0, 0.0], [0.0, 0.0, 0.0, 0.0], [1e-7, -1e-7, 0.0, 5e-8],
+                  [127.0, 63.5, -63.5, 0.4999]], dtype=np.float32)
+    q, s = oracle.act_quant_i8(x)
+    for r in range(x.shape[0]):
+        amax = np.float32(np.abs(x[r]).max())
+        se = np.float32(amax / np.float32(127.0)) if amax > np.float32(1e-6) else np.float32(1.0)
+        assert s[r] == se
+        inv = np.float32(1.0) / se
+        for c in range(x.shape[1]):
+            v = float(np.float32(x[r, c] * inv))
+            rounded = math.floor(abs(v) + 0.5) * (1 if v >= 0 else -1)  # half away from zero
+            assert q[r, c] == max(-127, min(127, rounded))
+    # the row maximum always maps to +-127; halves round away from zero
+    np.testing.assert_array_equal(q[0], [32, -64, 127, 0])
+    np.testing.assert_array_equal(q[3], [127, 64, -64, 0])
+    np.testing.assert_array_equal(q[1], [0, 0, 0, 0])
+    assert s[1] == 1.0 and s[2] == 1.0  # amax <= 1e-6 -> scale 1
+
+
+def test_gemm_i8_brute_force_and_identities(oracle):
+    rng = np.random.default_rng(5)
+    b, n, k = 3, 6, 10
+    q = rng.integers(-127, 128, size=(b, k)).astype(np.int8)
+    s_x = rng.random(b).astype(np.float32) + 0.1
+    w = random_ternary(n, k, seed=8).numpy()
+    scale = rng.random(n).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    p, _ = oracle.pack_ternary_transposed(w)
+    acc, y = oracle.gemm_i8(q, s_x, p, scale, k, bias)
+    for i in range(b):
+        for j in range(n):
+            a = sum(int(q[i, kk]) * 127 * int(w[j, kk]) for kk in range(k))
+            assert acc[i, j] == a
+            r = np.float32(np.float32(a) * s_x[i])
+            r = np.float32(r / np.float32(127.0))
+            r = np.float32(r * scale[j])
+            r = np.float32(r + bias[j])
+            assert y[i, j] == r
+    # integer GEMM equals numpy's exact integer product; sign flip of W negates it
+    np.testing.assert_array_equal(acc, q.astype(np.int64) @ (127 * w.astype(np.int64)).T)
+    pn, _ = oracle.pack_ternary_transposed(-w)
+    np.testing.assert_array_equal(oracle.gemm_i8(q, s_x, pn, scale, k)[0], -acc)
+
+
+def test_int8_path_tracks_float_path(oracle):
+    """The whole int8 route stays inside the quantisation error of 8-bit activations."""
+    b, n, k = 8, 64, 512
+    x = seeded_acts(b, k, seed=4).numpy()
+    w = random_ternary(n, k, seed=2).numpy()
+    p, _ = oracle.pack_ternary_transposed(w)
+    scale = np.full(n, 0.03, np.float32)
+    _, _, _, y8 = oracle.linear_i8(x, p, scale, k)
+    y = oracle.linear_packed(x, p, scale, k, f64=True)
+    assert np.abs(y8 - y).max() / np.abs(y).max() < 2e-2
+
+
+def test_round_helpers_match_torch(oracle):
+    vals = [1e-8, 6e-8, 3e-8, 65519.0, 65520.0, 0.05, 0.1, 1.0009765625, 3.14159, 1e-40, -2.5e-5]
+    for v in vals:
+        assert oracle.round_to_dtype(v, 1) == float(torch.tensor(v, dtype=torch.float32).half().float())
+        assert oracle.round_to_dtype(v, 2) == float(torch.tensor(v, dtype=torch.float32).bfloat16().float())
