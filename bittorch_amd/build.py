@@ -32,6 +32,14 @@ HIPCC_FLAGS = [
 ]
 
 
+# per-source extra flags
+EXTRA_FLAGS = {
+    # the iterative ILP scheduler keeps the MFMA accumulators in place across the
+    # software-pipelined main loop (the default strategy permutes them every iteration)
+    "gemm_i8.hip": ["-mllvm", "-amdgpu-sched-strategy=iterative-ilp"],
+}
+
+
 def _hipcc() -> str:
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(exe):
@@ -47,7 +55,8 @@ def build(verbose: bool = False, extra_flags=()) -> str:
 
     def compile_one(src: str) -> str:
         obj = os.path.join(OUT_DIR, os.path.splitext(src)[0] + ".o")
-        cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc, *HIPCC_FLAGS, *EXTRA_FLAGS.get(src, []), *extra_flags, "-c",
+               os.path.join(CSRC, src), "-o", obj]
         res = subprocess.run(cmd, capture_output=True, text=True)
         if res.returncode != 0:
             raise RuntimeError(f"hipcc failed on {src}:\n{res.stdout}\n{res.stderr}")

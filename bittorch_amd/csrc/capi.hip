@@ -38,7 +38,7 @@ int launch_packed_generic(const void* X, int x_dtype, const uint8_t* W_T, const 
 int launch_unpacked(const void* X, int x_dtype, const int8_t* W, const Epilogue& epi, void* Y, int64_t B,
                     int64_t N, int64_t K, hipStream_t st);
 int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x, hipStream_t st);
-bool gemm_i8_supported(int64_t N, const void* W_T);
+bool gemm_i8_supported(int64_t N, int64_t K, const void* Q, const void* W_T);
 int launch_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const Epilogue& epi, void* Y,
                    int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st);
 
@@ -188,7 +188,7 @@ extern "C" int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8
     hipStream_t st = (hipStream_t)stream;
     // decode-shape batches, and any batch whose N the tiled kernel's 4-column
     // vector accesses cannot take, stream the weights once per 16 rows
-    if (B <= kStreamMaxRows || !gemm_i8_supported(N, W_T))
+    if (B <= kStreamMaxRows || !gemm_i8_supported(N, K, Q, W_T))
         return launch_stream(MODE_I8, Q, 1, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, workspace,
                              workspace_bytes, st);
     return launch_gemm_i8(Q, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, st);

@@ -41,7 +41,6 @@ struct GemmParams {
     int y_dtype;
     int tiles_m, tiles_n;
     int per_xcd;          // workgroups per XCD (grid = 8 * per_xcd)
-    int q_vec_ok;         // rows of Q are 16-byte aligned
 };
 
 __device__ __forceinline__ void store4(void* Y, int dt, int64_t idx, const float (&v)[4]) {
@@ -58,6 +57,43 @@ __device__ __forceinline__ void store4(void* Y, int dt, int64_t idx, const float
     }
 }
 
+template <int YDT>
+__device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&acc)[G_MB][4], int64_t m0, int g,
+                                              int64_t ncol) {
+    float ws[4], bs[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        ws[t] = epi_scale(p.epi, ncol + t);
+        bs[t] = epi_bias(p.epi, ncol + t);
+    }
+#pragma unroll
+    for (int mb = 0; mb < G_MB; mb++) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int64_t m = m0 + 16 * mb + 4 * g + r;
+            if (m >= p.M) continue;
+            const float sx = p.s_x[m];
+            float y[4];
+            int32_t a127[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const int32_t a = acc[mb][t][r];
+                a127[t] = a * 127;
+                y[t] = epi_int8(a127[t], sx, ws[t], bs[t]);
+            }
+            store4(p.Y, YDT, m * p.N + ncol, y);
+            if (p.acc_out) *(int4*)(p.acc_out + m * p.N + ncol) = make_int4(a127[0], a127[1], a127[2], a127[3]);
+        }
+    }
+}
+
+// Scheduling hints: one group = `n` instructions of the class `mask`
+// (0x008 MFMA, 0x002 VALU, 0x100 LDS read, 0x200 LDS write, 0x020 VMEM read).
+#define BT_SCHED(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+
+// TAIL = false: K is a multiple of the 128-wide stage and the main loop is branch free.
+// TAIL = true: any K % 16 == 0; the last, partial stage is masked (slower bookkeeping).
+template <bool TAIL>
 __global__ __launch_bounds__(256) void gemm_i8_kernel(GemmParams p) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * G_STAGE_BYTES];
 
@@ -83,32 +119,63 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(GemmParams p) {
     const int64_t ncol = (int64_t)tile_n * G_BN + 64 * wave + 4 * j;
     const bool col_ok = ncol < p.N;
 
-    // A staging role of this thread: one row, one k64 sub-step (64 bytes)
-    const int a_row = tid & (G_BM - 1);
+    // Addresses are a wave-uniform base (advanced once per stage) plus a 32-bit
+    // per-lane offset fixed for the whole kernel.  Loads are unconditional with
+    // clamped rows / columns: rows past M and columns past N only feed outputs that
+    // are never stored; the K tail is zeroed in the A operand of the last stage.
+    // (The host guarantees K % 16 == 0, N % 4 == 0, aligned bases, 32-bit offsets.)
+    const int a_row = tid & (G_BM - 1);  // A staging role: one row, one k64 sub-step
     const int a_sub = tid >> 7;
-    const int64_t a_m = m0 + a_row;
-    const bool a_ok = a_m < p.M;
-    const int8_t* a_src = p.Q + a_m * p.K;
+    const int64_t rows_left = p.M - m0;
+    const uint32_t a_row_c = (uint32_t)((a_row < rows_left) ? a_row : rows_left - 1);
+    const uint32_t a_off = a_row_c * (uint32_t)p.K + 64u * a_sub;
+    const uint32_t b_off = (uint32_t)(col_ok ? ncol : 0) + (uint32_t)(4 * g) * (uint32_t)p.N;
+    const int8_t* a_base = p.Q + m0 * p.K;  // uniform
+    const uint8_t* b_base = p.W_T;          // uniform
+    const int64_t N = p.N;
+    const int nfull = (int)(p.K / G_BK);
+    const int nstages = (int)((p.K + G_BK - 1) / G_BK);
 
-    uint4 a_reg[4];
-    uint32_t b_reg[2][4];
+    uint4 a_reg[4];        // global -> LDS staging registers (one stage in flight)
+    uint32_t b_reg[2][4];  // packed weights in flight (same stage as a_reg)
 
-    auto load_a = [&](int64_t k0) {
+    auto load_full = [&](int64_t k0) {
+        const int8_t* ab = a_base + k0;
+#pragma unroll
+        for (int c = 0; c < 4; c++) a_reg[c] = *(const uint4*)(ab + 16 * c + a_off);
+        const uint8_t* bb = b_base + (k0 >> 2) * N;
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) b_reg[sub][r] = *(const uint32_t*)(bb + (16 * sub + r) * N + b_off);
+    };
+    auto load_tail = [&](int64_t k0) {
+        // last, partial stage: k beyond K reads a clamped address and is zeroed in A
+        const int8_t* ab = a_base + k0;
 #pragma unroll
         for (int c = 0; c < 4; c++) {
-            const int64_t k = k0 + 64 * a_sub + 16 * c;
-            uint4 v = make_uint4(0u, 0u, 0u, 0u);
-            if (a_ok && k < p.K) {
-                if (p.q_vec_ok && k + 16 <= p.K) {
-                    v = *(const uint4*)(a_src + k);
-                } else {
-                    uint32_t d[4] = {0u, 0u, 0u, 0u};
-                    for (int e = 0; e < 16; e++)
-                        if (k + e < p.K) d[e >> 2] |= (uint32_t)(uint8_t)a_src[k + e] << (8 * (e & 3));
-                    v = make_uint4(d[0], d[1], d[2], d[3]);
-                }
+            const bool in = (k0 + 64 * a_sub + 16 * c) < p.K;
+            const uint4 v = *(const uint4*)(ab + (in ? 16 * c : 0) + (in ? a_off : a_row_c * (uint32_t)p.K));
+            const uint32_t m = in ? 0xFFFFFFFFu : 0u;
+            a_reg[c] = make_uint4(v.x & m, v.y & m, v.z & m, v.w & m);
+        }
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                int64_t kb = (k0 >> 2) + 16 * sub + r + 4 * g;
+                kb = kb < p.Kb ? kb : p.Kb - 1;
+                b_reg[sub][r] = *(const uint32_t*)(b_base + kb * N + (col_ok ? ncol : 0));
             }
-            a_reg[c] = v;
+    };
+    auto load_stage = [&](int st) {  // st uniform
+        if constexpr (TAIL) {
+            if (st >= nstages) st = nstages - 1;
+            if (st < nfull) load_full((int64_t)st * G_BK);
+            else load_tail((int64_t)st * G_BK);
+        } else {
+            // past the end: reload the last stage (never consumed) instead of branching
+            load_full((int64_t)(st < nstages ? st : nstages - 1) * G_BK);
         }
     };
     auto store_a = [&](int buf) {
@@ -122,15 +189,16 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(GemmParams p) {
             *(uint4*)(base + ((size_t)((a_sub * G_MB + mb) * 64 + c * 16 + i) << 4)) = make_uint4(t[0], t[1], t[2], t[3]);
         }
     };
-    auto load_b = [&](int64_t k0) {
+    auto decode_b = [&](const uint32_t (&raw)[4], v4i (&b)[4]) {
+        uint32_t G[4];
+        transpose4x4_bytes(raw[0], raw[1], raw[2], raw[3], G);
 #pragma unroll
-        for (int sub = 0; sub < 2; sub++) {
+        for (int t = 0; t < 4; t++) b[t] = decode16_i8(G[t]);
+    };
+    auto read_a = [&](int buf, int sub, uint4 (&frag)[G_MB]) {
+        const uint8_t* a_lds = lds + buf * G_STAGE_BYTES + sub * (G_MB * 1024) + ((size_t)lane << 4);
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int64_t kb = (k0 >> 2) + 16 * sub + 4 * g + r;
-                b_reg[sub][r] = (col_ok && kb < p.Kb) ? *(const uint32_t*)(p.W_T + kb * p.N + ncol) : 0u;
-            }
-        }
+        for (int mb = 0; mb < G_MB; mb++) frag[mb] = *(const uint4*)(a_lds + mb * 1024);
     };
 
     v4i acc[G_MB][4];
@@ -139,71 +207,83 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(GemmParams p) {
 #pragma unroll
         for (int t = 0; t < 4; t++) acc[mb][t] = v4i{0, 0, 0, 0};
 
-    const int nstages = (int)((p.K + G_BK - 1) / G_BK);
-    load_a(0);
-    load_b(0);
-    store_a(0);
-    __syncthreads();
+    auto mma = [&](const uint4 (&frag)[G_MB], const v4i (&b)[4]) {
+#pragma unroll
+        for (int mb = 0; mb < G_MB; mb++) {
+            const v4i a = {(int)frag[mb].x, (int)frag[mb].y, (int)frag[mb].z, (int)frag[mb].w};
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+                acc[mb][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[t], acc[mb][t], 0, 0, 0);
+        }
+    };
 
+    // ---- software pipeline ------------------------------------------------------------
+    // Stage s computes from LDS buffer s%2.  At its top a workgroup writes stage s+1
+    // (loaded from global during stage s-1) into the other buffer and issues the global
+    // loads of stage s+2; one barrier in the middle of the stage publishes that buffer.
+    // Operand fragments run one sub-step ahead: while sub-step 0 multiplies, the
+    // fragments of sub-step 1 are read from LDS and its weights decoded, and so on.
+    uint32_t b_cur[2][4], b_nxt[2][4];
+    uint4 fragA[G_MB], fragB[G_MB];
+    v4i bdA[4], bdB[4];
+
+    load_stage(0);
+    store_a(0);
+#pragma unroll
+    for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) b_cur[sub][r] = b_reg[sub][r];
+    load_stage(1);
+    __syncthreads();
+    read_a(0, 0, fragA);
+    decode_b(b_cur[0], bdA);
+
+    // interleave hints for one sub-step: 32 MFMAs with the LDS reads, the decode VALU work
+    // and (sub-step 0) the staging writes and global loads spread between them
+#define BT_SUBSTEP_HINTS(with_staging)                                   \
+    _Pragma("unroll") for (int i = 0; i < 32; i++) {                     \
+        BT_SCHED(0x008, 1);                                              \
+        if ((i & 3) == 0) BT_SCHED(0x100, 1);                            \
+        BT_SCHED(0x002, (with_staging) ? 3 : 2);                         \
+        if ((with_staging) && (i & 7) == 1) BT_SCHED(0x200, 1);          \
+        if ((with_staging) && (i % 3) == 2) BT_SCHED(0x020, 1);          \
+    }
+
+    // Every stage runs the same straight-line body; the last one prefetches a clamped
+    // (already consumed) stage whose data is never used, which costs one redundant stage
+    // of loads but keeps the loop free of branches and peeled copies.
     for (int s = 0; s < nstages; s++) {
         const int cur = s & 1;
-        uint32_t b_cur[2][4];
+        // top: publish stage s+1 to the other buffer, start loading stage s+2
+        store_a(cur ^ 1);
 #pragma unroll
         for (int sub = 0; sub < 2; sub++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) b_cur[sub][r] = b_reg[sub][r];
-        const bool more = (s + 1 < nstages);
-        if (more) {
-            load_a((int64_t)(s + 1) * G_BK);
-            load_b((int64_t)(s + 1) * G_BK);
-        }
-        const uint8_t* a_base = lds + cur * G_STAGE_BYTES;
-#pragma unroll
-        for (int sub = 0; sub < 2; sub++) {
-            uint32_t G[4];
-            transpose4x4_bytes(b_cur[sub][0], b_cur[sub][1], b_cur[sub][2], b_cur[sub][3], G);
-            v4i b[4];
-#pragma unroll
-            for (int t = 0; t < 4; t++) b[t] = decode16_i8(G[t]);
-#pragma unroll
-            for (int mb = 0; mb < G_MB; mb++) {
-                const uint4 av = *(const uint4*)(a_base + ((size_t)((sub * G_MB + mb) * 64 + lane) << 4));
-                const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
-#pragma unroll
-                for (int t = 0; t < 4; t++)
-                    acc[mb][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[t], acc[mb][t], 0, 0, 0);
-            }
-        }
-        if (more) store_a(cur ^ 1);
+            for (int r = 0; r < 4; r++) b_nxt[sub][r] = b_reg[sub][r];
+        load_stage(s + 2);
+        // sub-step 0 multiplies; sub-step 1's operands are fetched / decoded meanwhile
+        read_a(cur, 1, fragB);
+        decode_b(b_cur[1], bdB);
+        mma(fragA, bdA);
+        BT_SUBSTEP_HINTS(true)
         __syncthreads();
+        // sub-step 1 multiplies; the next stage's sub-step 0 operands are prepared
+        read_a(cur ^ 1, 0, fragA);
+        decode_b(b_nxt[0], bdA);
+        mma(fragB, bdB);
+        BT_SUBSTEP_HINTS(false)
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) b_cur[sub][r] = b_nxt[sub][r];
     }
+#undef BT_SUBSTEP_HINTS
 
     // ---- epilogue: lane (j, g) holds rows 16mb + 4g + r, columns ncol .. ncol+3 --------
     if (!col_ok) return;
-    float ws[4], bs[4];
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-        ws[t] = epi_scale(p.epi, ncol + t);
-        bs[t] = epi_bias(p.epi, ncol + t);
-    }
-#pragma unroll
-    for (int mb = 0; mb < G_MB; mb++) {
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const int64_t m = m0 + 16 * mb + 4 * g + r;
-            if (m >= p.M) continue;
-            const float sx = p.s_x[m];
-            float y[4];
-            int32_t a127[4];
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-                a127[t] = acc[mb][t][r] * 127;
-                y[t] = epi_int8(a127[t], sx, ws[t], bs[t]);
-            }
-            store4(p.Y, p.y_dtype, m * p.N + ncol, y);
-            if (p.acc_out) *(int4*)(p.acc_out + m * p.N + ncol) = make_int4(a127[0], a127[1], a127[2], a127[3]);
-        }
-    }
+    if (p.y_dtype == BT_BF16) gemm_epilogue<BT_BF16>(p, acc, m0, g, ncol);
+    else if (p.y_dtype == BT_F16) gemm_epilogue<BT_F16>(p, acc, m0, g, ncol);
+    else gemm_epilogue<BT_F32>(p, acc, m0, g, ncol);
 }
 
 // Per-row int8 activation quantizer: one wave per row, two passes over the row
@@ -283,7 +363,12 @@ int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q
     return check_launch("bt_act_quant_i8");
 }
 
-bool gemm_i8_supported(int64_t N, const void* W_T) { return N % 4 == 0 && ((uintptr_t)W_T) % 4 == 0; }
+// the tiled kernel reads Q with 16-byte loads and W_T / Y with 4-column vectors
+bool gemm_i8_supported(int64_t N, int64_t K, const void* Q, const void* W_T) {
+    // 32-bit per-lane offsets: a row tile of Q and the whole of W_T stay below 4 GiB
+    return N % 4 == 0 && K % 16 == 0 && ((uintptr_t)W_T) % 4 == 0 && ((uintptr_t)Q) % 16 == 0 &&
+           (G_BM + 1) * K < (1ll << 32) && ceil_div(K, 4) * N < (1ll << 32);
+}
 
 int launch_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const Epilogue& epi, void* Y,
                    int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st) {
@@ -295,8 +380,10 @@ int launch_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const 
     p.tiles_n = (int)ceil_div(N, G_BN);
     const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
     p.per_xcd = (int)ceil_div(total, 8);
-    p.q_vec_ok = (((uintptr_t)Q) % 16 == 0) && (K % 16 == 0);
-    hipLaunchKernelGGL(gemm_i8_kernel, dim3((unsigned)(p.per_xcd * 8)), dim3(256), 0, st, p);
+    if (K % G_BK == 0)
+        hipLaunchKernelGGL(gemm_i8_kernel<false>, dim3((unsigned)(p.per_xcd * 8)), dim3(256), 0, st, p);
+    else
+        hipLaunchKernelGGL(gemm_i8_kernel<true>, dim3((unsigned)(p.per_xcd * 8)), dim3(256), 0, st, p);
     return check_launch("bt_ternary_gemm_i8");
 }
 
