@@ -59,7 +59,7 @@ __device__ __forceinline__ void store4(void* Y, int dt, int64_t idx, const float
 
 template <int YDT>
 __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&acc)[G_MB][4], int64_t m0, int g,
-                                              int64_t ncol) {
+                                              int64_t ncol, int mb0) {
     float ws[4], bs[4];
 #pragma unroll
     for (int t = 0; t < 4; t++) {
@@ -67,17 +67,18 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&a
         bs[t] = epi_bias(p.epi, ncol + t);
     }
 #pragma unroll
-    for (int mb = 0; mb < G_MB; mb++) {
+    for (int mbi = 0; mbi < 4; mbi++) {
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            const int64_t m = m0 + 16 * mb + 4 * g + r;
+            const int64_t m = m0 + 16 * (mb0 + mbi) + 4 * g + r;
             if (m >= p.M) continue;
             const float sx = p.s_x[m];
             float y[4];
             int32_t a127[4];
 #pragma unroll
             for (int t = 0; t < 4; t++) {
-                const int32_t a = acc[mb][t][r];
+                // registers are indexed statically: pick the row block of this K half
+                const int32_t a = (mb0 == 0) ? acc[mbi][t][r] : acc[4 + mbi][t][r];
                 a127[t] = a * 127;
                 y[t] = epi_int8(a127[t], sx, ws[t], bs[t]);
             }
@@ -87,15 +88,18 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&a
     }
 }
 
-// Scheduling hints: one group = `n` instructions of the class `mask`
-// (0x008 MFMA, 0x002 VALU, 0x100 LDS read, 0x200 LDS write, 0x020 VMEM read).
-#define BT_SCHED(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
-
 // TAIL = false: K is a multiple of the 128-wide stage and the main loop is branch free.
 // TAIL = true: any K % 16 == 0; the last, partial stage is masked (slower bookkeeping).
+//
+// 512 threads = 8 waves: wave w works on columns 64*(w&3) .. +63 of the tile and on
+// k64 sub-step (w>>2) of every 128-wide stage, so the two waves that share a SIMD
+// split K between them (each weight is still decoded once per workgroup) and one
+// wave's LDS / barrier / decode latency hides behind the other's MFMAs.  The two
+// K halves are added through LDS once, after the main loop, and each half of the
+// workgroup finishes 64 of the 128 rows.
 template <bool TAIL>
-__global__ __launch_bounds__(256) void gemm_i8_kernel(GemmParams p) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * G_STAGE_BYTES];
+__global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[65536];  // 2 A stages; reused for the K-half exchange
 
     // XCD-aware tile order: the 8 XCDs each take a contiguous run of tiles, and
     // runs are walked in groups of four row tiles so that one XCD's L2 holds a
@@ -113,10 +117,12 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(GemmParams p) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
+    const int wn = wave & 3;     // column quarter
+    const int kgrp = wave >> 2;  // k64 sub-step of each stage
     const int j = lane & 15;
     const int g = lane >> 4;
     const int64_t m0 = (int64_t)tile_m * G_BM;
-    const int64_t ncol = (int64_t)tile_n * G_BN + 64 * wave + 4 * j;
+    const int64_t ncol = (int64_t)tile_n * G_BN + 64 * wn + 4 * j;
     const bool col_ok = ncol < p.N;
 
     // Addresses are a wave-uniform base (advanced once per stage) plus a 32-bit
@@ -124,49 +130,45 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(GemmParams p) {
     // clamped rows / columns: rows past M and columns past N only feed outputs that
     // are never stored; the K tail is zeroed in the A operand of the last stage.
     // (The host guarantees K % 16 == 0, N % 4 == 0, aligned bases, 32-bit offsets.)
-    const int a_row = tid & (G_BM - 1);  // A staging role: one row, one k64 sub-step
-    const int a_sub = tid >> 7;
+    const int a_row = tid & (G_BM - 1);  // A staging role: one row, 32 of its 128 stage bytes
+    const int a_part = tid >> 7;         // bytes 32*a_part .. +31 -> sub-step a_part>>1, chunks 2*(a_part&1), +1
     const int64_t rows_left = p.M - m0;
     const uint32_t a_row_c = (uint32_t)((a_row < rows_left) ? a_row : rows_left - 1);
-    const uint32_t a_off = a_row_c * (uint32_t)p.K + 64u * a_sub;
-    const uint32_t b_off = (uint32_t)(col_ok ? ncol : 0) + (uint32_t)(4 * g) * (uint32_t)p.N;
+    const uint32_t a_off = a_row_c * (uint32_t)p.K + 32u * a_part;
+    const uint32_t b_off = (uint32_t)(col_ok ? ncol : 0) + (uint32_t)(16 * kgrp + 4 * g) * (uint32_t)p.N;
     const int8_t* a_base = p.Q + m0 * p.K;  // uniform
     const uint8_t* b_base = p.W_T;          // uniform
     const int64_t N = p.N;
     const int nfull = (int)(p.K / G_BK);
     const int nstages = (int)((p.K + G_BK - 1) / G_BK);
 
-    uint4 a_reg[4];        // global -> LDS staging registers (one stage in flight)
-    uint32_t b_reg[2][4];  // packed weights in flight (same stage as a_reg)
+    uint4 a_reg[2];     // global -> LDS staging registers (one stage in flight)
+    uint32_t b_reg[4];  // packed weights in flight (same stage as a_reg)
 
     auto load_full = [&](int64_t k0) {
         const int8_t* ab = a_base + k0;
-#pragma unroll
-        for (int c = 0; c < 4; c++) a_reg[c] = *(const uint4*)(ab + 16 * c + a_off);
+        a_reg[0] = *(const uint4*)(ab + a_off);
+        a_reg[1] = *(const uint4*)(ab + 16 + a_off);
         const uint8_t* bb = b_base + (k0 >> 2) * N;
 #pragma unroll
-        for (int sub = 0; sub < 2; sub++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) b_reg[sub][r] = *(const uint32_t*)(bb + (16 * sub + r) * N + b_off);
+        for (int r = 0; r < 4; r++) b_reg[r] = *(const uint32_t*)(bb + r * N + b_off);
     };
     auto load_tail = [&](int64_t k0) {
         // last, partial stage: k beyond K reads a clamped address and is zeroed in A
         const int8_t* ab = a_base + k0;
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            const bool in = (k0 + 64 * a_sub + 16 * c) < p.K;
+        for (int c = 0; c < 2; c++) {
+            const bool in = (k0 + 32 * a_part + 16 * c) < p.K;
             const uint4 v = *(const uint4*)(ab + (in ? 16 * c : 0) + (in ? a_off : a_row_c * (uint32_t)p.K));
             const uint32_t m = in ? 0xFFFFFFFFu : 0u;
             a_reg[c] = make_uint4(v.x & m, v.y & m, v.z & m, v.w & m);
         }
 #pragma unroll
-        for (int sub = 0; sub < 2; sub++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                int64_t kb = (k0 >> 2) + 16 * sub + r + 4 * g;
-                kb = kb < p.Kb ? kb : p.Kb - 1;
-                b_reg[sub][r] = *(const uint32_t*)(b_base + kb * N + (col_ok ? ncol : 0));
-            }
+        for (int r = 0; r < 4; r++) {
+            int64_t kb = (k0 >> 2) + 16 * kgrp + r + 4 * g;
+            kb = kb < p.Kb ? kb : p.Kb - 1;
+            b_reg[r] = *(const uint32_t*)(b_base + kb * N + (col_ok ? ncol : 0));
+        }
     };
     auto load_stage = [&](int st) {  // st uniform
         if constexpr (TAIL) {
@@ -179,26 +181,16 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(GemmParams p) {
         }
     };
     auto store_a = [&](int buf) {
+        // slot (sub, mb, lane = c*16 + i) holds the 16 bytes MFMA lane (i, g = c) reads
         uint8_t* base = lds + buf * G_STAGE_BYTES;
-        const int mb = a_row >> 4, i = a_row & 15;
+        const int mb = a_row >> 4, i = a_row & 15, sub = a_part >> 1;
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
+        for (int e = 0; e < 2; e++) {
+            const int c = 2 * (a_part & 1) + e;
             uint32_t t[4];
-            transpose4x4_bytes(a_reg[c].x, a_reg[c].y, a_reg[c].z, a_reg[c].w, t);
-            // slot (sub, mb, lane = c*16 + i)
-            *(uint4*)(base + ((size_t)((a_sub * G_MB + mb) * 64 + c * 16 + i) << 4)) = make_uint4(t[0], t[1], t[2], t[3]);
+            transpose4x4_bytes(a_reg[e].x, a_reg[e].y, a_reg[e].z, a_reg[e].w, t);
+            *(uint4*)(base + ((size_t)((sub * G_MB + mb) * 64 + c * 16 + i) << 4)) = make_uint4(t[0], t[1], t[2], t[3]);
         }
-    };
-    auto decode_b = [&](const uint32_t (&raw)[4], v4i (&b)[4]) {
-        uint32_t G[4];
-        transpose4x4_bytes(raw[0], raw[1], raw[2], raw[3], G);
-#pragma unroll
-        for (int t = 0; t < 4; t++) b[t] = decode16_i8(G[t]);
-    };
-    auto read_a = [&](int buf, int sub, uint4 (&frag)[G_MB]) {
-        const uint8_t* a_lds = lds + buf * G_STAGE_BYTES + sub * (G_MB * 1024) + ((size_t)lane << 4);
-#pragma unroll
-        for (int mb = 0; mb < G_MB; mb++) frag[mb] = *(const uint4*)(a_lds + mb * 1024);
     };
 
     v4i acc[G_MB][4];
@@ -207,83 +199,85 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(GemmParams p) {
 #pragma unroll
         for (int t = 0; t < 4; t++) acc[mb][t] = v4i{0, 0, 0, 0};
 
-    auto mma = [&](const uint4 (&frag)[G_MB], const v4i (&b)[4]) {
+    // ---- main loop --------------------------------------------------------------------
+    // Stage s is computed from LDS buffer s%2.  At the top of stage s every thread writes
+    // its piece of stage s+1 (loaded from global during stage s-1) into the other buffer
+    // and issues the global loads of stage s+2; the barrier at the end of the stage both
+    // publishes that buffer and retires the reads of the current one.  The last stage
+    // prefetches a clamped, never consumed stage instead of branching.
+    load_stage(0);
+    store_a(0);
+    uint32_t b_cur[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) b_cur[r] = b_reg[r];
+    load_stage(1);
+    __syncthreads();
+
+    for (int s = 0; s < nstages; s++) {
+        const int cur = s & 1;
+        store_a(cur ^ 1);
+        uint32_t b_nxt[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) b_nxt[r] = b_reg[r];
+        load_stage(s + 2);
+
+        uint32_t G[4];
+        transpose4x4_bytes(b_cur[0], b_cur[1], b_cur[2], b_cur[3], G);
+        v4i b[4];
+#pragma unroll
+        for (int t = 0; t < 4; t++) b[t] = decode16_i8(G[t]);
+        const uint8_t* a_lds = lds + cur * G_STAGE_BYTES + kgrp * (G_MB * 1024) + ((size_t)lane << 4);
 #pragma unroll
         for (int mb = 0; mb < G_MB; mb++) {
-            const v4i a = {(int)frag[mb].x, (int)frag[mb].y, (int)frag[mb].z, (int)frag[mb].w};
+            const uint4 av = *(const uint4*)(a_lds + mb * 1024);
+            const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
 #pragma unroll
             for (int t = 0; t < 4; t++)
                 acc[mb][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[t], acc[mb][t], 0, 0, 0);
         }
-    };
-
-    // ---- software pipeline ------------------------------------------------------------
-    // Stage s computes from LDS buffer s%2.  At its top a workgroup writes stage s+1
-    // (loaded from global during stage s-1) into the other buffer and issues the global
-    // loads of stage s+2; one barrier in the middle of the stage publishes that buffer.
-    // Operand fragments run one sub-step ahead: while sub-step 0 multiplies, the
-    // fragments of sub-step 1 are read from LDS and its weights decoded, and so on.
-    uint32_t b_cur[2][4], b_nxt[2][4];
-    uint4 fragA[G_MB], fragB[G_MB];
-    v4i bdA[4], bdB[4];
-
-    load_stage(0);
-    store_a(0);
 #pragma unroll
-    for (int sub = 0; sub < 2; sub++)
-#pragma unroll
-        for (int r = 0; r < 4; r++) b_cur[sub][r] = b_reg[sub][r];
-    load_stage(1);
-    __syncthreads();
-    read_a(0, 0, fragA);
-    decode_b(b_cur[0], bdA);
-
-    // interleave hints for one sub-step: 32 MFMAs with the LDS reads, the decode VALU work
-    // and (sub-step 0) the staging writes and global loads spread between them
-#define BT_SUBSTEP_HINTS(with_staging)                                   \
-    _Pragma("unroll") for (int i = 0; i < 32; i++) {                     \
-        BT_SCHED(0x008, 1);                                              \
-        if ((i & 3) == 0) BT_SCHED(0x100, 1);                            \
-        BT_SCHED(0x002, (with_staging) ? 3 : 2);                         \
-        if ((with_staging) && (i & 7) == 1) BT_SCHED(0x200, 1);          \
-        if ((with_staging) && (i % 3) == 2) BT_SCHED(0x020, 1);          \
-    }
-
-    // Every stage runs the same straight-line body; the last one prefetches a clamped
-    // (already consumed) stage whose data is never used, which costs one redundant stage
-    // of loads but keeps the loop free of branches and peeled copies.
-    for (int s = 0; s < nstages; s++) {
-        const int cur = s & 1;
-        // top: publish stage s+1 to the other buffer, start loading stage s+2
-        store_a(cur ^ 1);
-#pragma unroll
-        for (int sub = 0; sub < 2; sub++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) b_nxt[sub][r] = b_reg[sub][r];
-        load_stage(s + 2);
-        // sub-step 0 multiplies; sub-step 1's operands are fetched / decoded meanwhile
-        read_a(cur, 1, fragB);
-        decode_b(b_cur[1], bdB);
-        mma(fragA, bdA);
-        BT_SUBSTEP_HINTS(true)
+        for (int r = 0; r < 4; r++) b_cur[r] = b_nxt[r];
         __syncthreads();
-        // sub-step 1 multiplies; the next stage's sub-step 0 operands are prepared
-        read_a(cur ^ 1, 0, fragA);
-        decode_b(b_nxt[0], bdA);
-        mma(fragB, bdB);
-        BT_SUBSTEP_HINTS(false)
-#pragma unroll
-        for (int sub = 0; sub < 2; sub++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) b_cur[sub][r] = b_nxt[sub][r];
     }
-#undef BT_SUBSTEP_HINTS
 
-    // ---- epilogue: lane (j, g) holds rows 16mb + 4g + r, columns ncol .. ncol+3 --------
+    // ---- add the two K halves: waves (wn, 0) and (wn, 1) hold partial sums of the same
+    // outputs.  K half 1 hands over row blocks 0..3, K half 0 hands over row blocks 4..7;
+    // word (q, wn, lane) of the exchange buffer is register q of that lane.
+    {
+        int32_t* xch = (int32_t*)lds;
+        const int slot = wn * 64 + lane;
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const int giver = 1 - half;  // K half that hands over row blocks 4*half .. 4*half+3
+            if (kgrp == giver) {
+#pragma unroll
+                for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        const v4i v = acc[4 * half + mb][t];
+                        *(int4*)(xch + ((mb * 4 + t) * 256 + slot) * 4) = make_int4(v[0], v[1], v[2], v[3]);
+                    }
+            }
+            __syncthreads();
+            if (kgrp != giver) {
+#pragma unroll
+                for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        const int4 v = *(const int4*)(xch + ((mb * 4 + t) * 256 + slot) * 4);
+                        acc[4 * half + mb][t] += v4i{v.x, v.y, v.z, v.w};
+                    }
+            }
+            __syncthreads();
+        }
+    }
+
+    // ---- epilogue: K half h finishes row blocks 4h .. 4h+3; lane (j, g) holds rows
+    // 16mb + 4g + r, columns ncol .. ncol+3 -------------------------------------------
     if (!col_ok) return;
-    if (p.y_dtype == BT_BF16) gemm_epilogue<BT_BF16>(p, acc, m0, g, ncol);
-    else if (p.y_dtype == BT_F16) gemm_epilogue<BT_F16>(p, acc, m0, g, ncol);
-    else gemm_epilogue<BT_F32>(p, acc, m0, g, ncol);
+    if (p.y_dtype == BT_BF16) gemm_epilogue<BT_BF16>(p, acc, m0, g, ncol, 4 * kgrp);
+    else if (p.y_dtype == BT_F16) gemm_epilogue<BT_F16>(p, acc, m0, g, ncol, 4 * kgrp);
+    else gemm_epilogue<BT_F32>(p, acc, m0, g, ncol, 4 * kgrp);
 }
 
 // Per-row int8 activation quantizer: one wave per row, two passes over the row
@@ -381,9 +375,9 @@ int launch_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const 
     const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
     p.per_xcd = (int)ceil_div(total, 8);
     if (K % G_BK == 0)
-        hipLaunchKernelGGL(gemm_i8_kernel<false>, dim3((unsigned)(p.per_xcd * 8)), dim3(256), 0, st, p);
+        hipLaunchKernelGGL(gemm_i8_kernel<false>, dim3((unsigned)(p.per_xcd * 8)), dim3(512), 0, st, p);
     else
-        hipLaunchKernelGGL(gemm_i8_kernel<true>, dim3((unsigned)(p.per_xcd * 8)), dim3(256), 0, st, p);
+        hipLaunchKernelGGL(gemm_i8_kernel<true>, dim3((unsigned)(p.per_xcd * 8)), dim3(512), 0, st, p);
     return check_launch("bt_ternary_gemm_i8");
 }
 
