@@ -32,10 +32,7 @@ __device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) {
     return __builtin_bit_cast(float, (uint32_t)h << 16);
 }
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-    uint32_t u = __builtin_bit_cast(uint32_t, f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);  // quiet NaN
-    u += 0x7fffu + ((u >> 16) & 1u);                                             // RNE
-    return (uint16_t)(u >> 16);
+    return __builtin_bit_cast(uint16_t, (__bf16)f);  // v_cvt_pk_bf16_f32, RNE
 }
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
     return (float)__builtin_bit_cast(_Float16, h);
@@ -88,13 +85,25 @@ __device__ __forceinline__ float epi_bias(const Epilogue& e, int64_t n) {
 __device__ __forceinline__ float epi_float(float acc, float s, float b) {
     return __fadd_rn(__fmul_rn(acc, s), b);
 }
+// x / 127.0f, correctly rounded, in three operations: q0 = x * RN(1/127), one fused
+// residual and one fused correction.  Checked exhaustively against IEEE division for
+// every finite fp32 x; the only difference is the sign of the result for x = -0.0,
+// which the int8 epilogue cannot produce (float(int) * positive scale is never -0).
+__device__ __forceinline__ float div127(float x) {
+    const float y = 1.0f / 127.0f;
+    const float q0 = x * y;
+    const float r = __builtin_fmaf(-127.0f, q0, x);
+    return __builtin_fmaf(r, y, q0);
+}
 // int8 path: ((float(acc) * s_x) / 127) * w_scale + bias, left to right
 __device__ __forceinline__ float epi_int8(int32_t acc127, float sx, float ws, float b) {
     float r = __fmul_rn((float)acc127, sx);
-    r = __fdiv_rn(r, 127.0f);
+    r = div127(r);
     r = __fmul_rn(r, ws);
     return __fadd_rn(r, b);
 }
+// 127 * a without the quarter-rate 32-bit multiply
+__device__ __forceinline__ int32_t times127(int32_t a) { return (int32_t)(((uint32_t)a << 7) - (uint32_t)a); }
 
 // ---- 2-bit decode in registers -------------------------------------------
 // v_perm_b32: result byte i = byte sel[i] of the 8-byte value {hi,lo}

@@ -57,9 +57,10 @@ __device__ __forceinline__ void store4(void* Y, int dt, int64_t idx, const float
     }
 }
 
-template <int YDT>
+// Finishes four 16-row blocks (acc[MB0 .. MB0+3]) of the tile.
+template <int YDT, int MB0>
 __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&acc)[G_MB][4], int64_t m0, int g,
-                                              int64_t ncol, int mb0) {
+                                              int64_t ncol) {
     float ws[4], bs[4];
 #pragma unroll
     for (int t = 0; t < 4; t++) {
@@ -70,22 +71,28 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&a
     for (int mbi = 0; mbi < 4; mbi++) {
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            const int64_t m = m0 + 16 * (mb0 + mbi) + 4 * g + r;
+            const int64_t m = m0 + 16 * (MB0 + mbi) + 4 * g + r;
             if (m >= p.M) continue;
             const float sx = p.s_x[m];
             float y[4];
             int32_t a127[4];
 #pragma unroll
             for (int t = 0; t < 4; t++) {
-                // registers are indexed statically: pick the row block of this K half
-                const int32_t a = (mb0 == 0) ? acc[mbi][t][r] : acc[4 + mbi][t][r];
-                a127[t] = a * 127;
+                const int32_t a = acc[MB0 + mbi][t][r];
+                a127[t] = times127(a);
                 y[t] = epi_int8(a127[t], sx, ws[t], bs[t]);
             }
             store4(p.Y, YDT, m * p.N + ncol, y);
             if (p.acc_out) *(int4*)(p.acc_out + m * p.N + ncol) = make_int4(a127[0], a127[1], a127[2], a127[3]);
         }
     }
+}
+template <int MB0>
+__device__ __forceinline__ void gemm_epilogue_dt(const GemmParams& p, const v4i (&acc)[G_MB][4], int64_t m0, int g,
+                                                 int64_t ncol) {
+    if (p.y_dtype == BT_BF16) gemm_epilogue<BT_BF16, MB0>(p, acc, m0, g, ncol);
+    else if (p.y_dtype == BT_F16) gemm_epilogue<BT_F16, MB0>(p, acc, m0, g, ncol);
+    else gemm_epilogue<BT_F32, MB0>(p, acc, m0, g, ncol);
 }
 
 // TAIL = false: K is a multiple of the 128-wide stage and the main loop is branch free.
@@ -142,10 +149,11 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     const int nfull = (int)(p.K / G_BK);
     const int nstages = (int)((p.K + G_BK - 1) / G_BK);
 
-    uint4 a_reg[2];     // global -> LDS staging registers (one stage in flight)
-    uint32_t b_reg[4];  // packed weights in flight (same stage as a_reg)
+    // two stages of operands in flight: set s%2 holds stage s until it is written to LDS
+    uint4 a_set[2][2];
+    uint32_t b_set[2][4];
 
-    auto load_full = [&](int64_t k0) {
+    auto load_full = [&](int64_t k0, uint4 (&a_reg)[2], uint32_t (&b_reg)[4]) {
         const int8_t* ab = a_base + k0;
         a_reg[0] = *(const uint4*)(ab + a_off);
         a_reg[1] = *(const uint4*)(ab + 16 + a_off);
@@ -153,7 +161,7 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
 #pragma unroll
         for (int r = 0; r < 4; r++) b_reg[r] = *(const uint32_t*)(bb + r * N + b_off);
     };
-    auto load_tail = [&](int64_t k0) {
+    auto load_tail = [&](int64_t k0, uint4 (&a_reg)[2], uint32_t (&b_reg)[4]) {
         // last, partial stage: k beyond K reads a clamped address and is zeroed in A
         const int8_t* ab = a_base + k0;
 #pragma unroll
@@ -170,17 +178,17 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
             b_reg[r] = *(const uint32_t*)(b_base + kb * N + (col_ok ? ncol : 0));
         }
     };
-    auto load_stage = [&](int st) {  // st uniform
+    auto load_stage = [&](int st, uint4 (&a_reg)[2], uint32_t (&b_reg)[4]) {  // st uniform
         if constexpr (TAIL) {
             if (st >= nstages) st = nstages - 1;
-            if (st < nfull) load_full((int64_t)st * G_BK);
-            else load_tail((int64_t)st * G_BK);
+            if (st < nfull) load_full((int64_t)st * G_BK, a_reg, b_reg);
+            else load_tail((int64_t)st * G_BK, a_reg, b_reg);
         } else {
             // past the end: reload the last stage (never consumed) instead of branching
-            load_full((int64_t)(st < nstages ? st : nstages - 1) * G_BK);
+            load_full((int64_t)(st < nstages ? st : nstages - 1) * G_BK, a_reg, b_reg);
         }
     };
-    auto store_a = [&](int buf) {
+    auto store_a = [&](int buf, const uint4 (&a_reg)[2]) {
         // slot (sub, mb, lane = c*16 + i) holds the 16 bytes MFMA lane (i, g = c) reads
         uint8_t* base = lds + buf * G_STAGE_BYTES;
         const int mb = a_row >> 4, i = a_row & 15, sub = a_part >> 1;
@@ -201,25 +209,28 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
 
     // ---- main loop --------------------------------------------------------------------
     // Stage s is computed from LDS buffer s%2.  At the top of stage s every thread writes
-    // its piece of stage s+1 (loaded from global during stage s-1) into the other buffer
-    // and issues the global loads of stage s+2; the barrier at the end of the stage both
-    // publishes that buffer and retires the reads of the current one.  The last stage
-    // prefetches a clamped, never consumed stage instead of branching.
-    load_stage(0);
-    store_a(0);
-    uint32_t b_cur[4];
+    // its piece of stage s+1 into the other buffer and re-uses those registers for the
+    // global loads of stage s+3, so a load has two full stages to arrive.  The barrier at
+    // the end of a stage both publishes the buffer just written and retires the reads of
+    // the current one.  Stages past the end are clamped (loaded, never consumed) instead
+    // of branched around; the loop handles two stages per trip so that the register sets
+    // are indexed statically.
+    uint32_t b_cur[4], b_nxt[4];
+    load_stage(0, a_set[0], b_set[0]);
+    load_stage(1, a_set[1], b_set[1]);
+    store_a(0, a_set[0]);
 #pragma unroll
-    for (int r = 0; r < 4; r++) b_cur[r] = b_reg[r];
-    load_stage(1);
+    for (int r = 0; r < 4; r++) b_cur[r] = b_set[0][r];
+    load_stage(2, a_set[0], b_set[0]);
     __syncthreads();
 
-    for (int s = 0; s < nstages; s++) {
+    auto stage = [&](int s, uint4 (&a_reg)[2], uint32_t (&b_reg)[4]) {
+        // a_reg / b_reg hold stage s+1 on entry and are reloaded with stage s+3
         const int cur = s & 1;
-        store_a(cur ^ 1);
-        uint32_t b_nxt[4];
+        store_a(cur ^ 1, a_reg);
 #pragma unroll
         for (int r = 0; r < 4; r++) b_nxt[r] = b_reg[r];
-        load_stage(s + 2);
+        load_stage(s + 3, a_reg, b_reg);
 
         uint32_t G[4];
         transpose4x4_bytes(b_cur[0], b_cur[1], b_cur[2], b_cur[3], G);
@@ -238,6 +249,10 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
 #pragma unroll
         for (int r = 0; r < 4; r++) b_cur[r] = b_nxt[r];
         __syncthreads();
+    };
+    for (int s = 0; s < nstages; s += 2) {
+        stage(s, a_set[1], b_set[1]);
+        if (s + 1 < nstages) stage(s + 1, a_set[0], b_set[0]);
     }
 
     // ---- add the two K halves: waves (wn, 0) and (wn, 1) hold partial sums of the same
@@ -275,9 +290,8 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     // ---- epilogue: K half h finishes row blocks 4h .. 4h+3; lane (j, g) holds rows
     // 16mb + 4g + r, columns ncol .. ncol+3 -------------------------------------------
     if (!col_ok) return;
-    if (p.y_dtype == BT_BF16) gemm_epilogue<BT_BF16>(p, acc, m0, g, ncol, 4 * kgrp);
-    else if (p.y_dtype == BT_F16) gemm_epilogue<BT_F16>(p, acc, m0, g, ncol, 4 * kgrp);
-    else gemm_epilogue<BT_F32>(p, acc, m0, g, ncol, 4 * kgrp);
+    if (kgrp == 0) gemm_epilogue_dt<0>(p, acc, m0, g, ncol);  // wave-uniform branch
+    else gemm_epilogue_dt<4>(p, acc, m0, g, ncol);
 }
 
 // Per-row int8 activation quantizer: one wave per row, two passes over the row

@@ -77,7 +77,7 @@ __device__ __forceinline__ void finish_output(const StreamParams& p, int row, in
     const float b = epi_bias(p.epi, n);
     float y;
     if constexpr (MODE == MODE_I8) {
-        const int32_t acc127 = (int32_t)bits * 127;  // MFMA ran on +-1 weights
+        const int32_t acc127 = times127((int32_t)bits);  // MFMA ran on +-1 weights
         if (p.acc_out) p.acc_out[(int64_t)row * p.N + n] = acc127;
         y = epi_int8(acc127, p.s_x[row], s, b);
     } else if constexpr (MODE == MODE_F16) {
