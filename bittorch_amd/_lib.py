@@ -12,7 +12,8 @@ import os
 from typing import Optional
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "_hip", "libbittorch_hip.so")
+# BITTORCH_HIP_LIBRARY points at another build of the library (A/B comparisons)
+LIB_PATH = os.environ.get("BITTORCH_HIP_LIBRARY") or os.path.join(_HERE, "_hip", "libbittorch_hip.so")
 
 ABI_VERSION = 1
 
