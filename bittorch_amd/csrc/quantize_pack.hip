@@ -6,44 +6,27 @@
 // fl(tf * scale) in the weight dtype, code = |w| > thr ? (w > 0 ? 1 : 2) : 0,
 // byte[kb, n] = c0 | c1<<2 | c2<<4 | c3<<6 for k = 4kb..4kb+3.
 //
-// Layout of the work: a 256-thread workgroup owns 16 consecutive output rows
-// n0..n0+15, wave w the four rows n0+4w..n0+4w+3.  A wave keeps one whole row in
-// registers (ITERS float4 groups per lane), reduces its absmax across the 64
-// lanes, encodes, and ORs the row's bytes into a dword per kb that ends up
-// holding the four rows of the wave.  The dwords go through LDS so that the
-// transposed store writes 16 contiguous bytes per kb row.
+// Two kernels share that arithmetic:
+//   * quantize_pack_fast_kernel: K a multiple of 256, N a multiple of the row tile,
+//     aligned pointers.  A wave keeps one whole row in registers (K/64 values per
+//     lane), reduces its absmax across the 64 lanes, encodes, and hands the row's
+//     bytes to LDS; a workgroup owns R = WAVES*RPW consecutive rows, so the
+//     transposed store writes R contiguous bytes per packed_T row.  One read of W.
+//   * quantize_pack_generic_kernel: any shape, alignment and dtype, optional dense
+//     ternary output; reads every row twice (absmax pass, encode pass) and walks K
+//     in segments so that the LDS tile is bounded.
+#include <cstdlib>
+
 #include "bt_common.h"
 
 namespace bt {
 
 // Workgroup b of a grid of 8*per_xcd workgroups -> tile index such that
 // consecutive tiles run on the same XCD (workgroups are dealt round-robin over
-// the 8 XCDs), so the 16-byte pieces of one packed_T cache line that
-// neighbouring tiles write meet in one L2.
+// the 8 XCDs), so the pieces of one packed_T cache line that neighbouring tiles
+// write meet in one L2.
 __device__ __forceinline__ int64_t xcd_tile(int64_t b, int64_t per_xcd) {
     return (b & 7) * per_xcd + (b >> 3);
-}
-
-template <int DT>
-__device__ __forceinline__ void load4(const void* W, int64_t elem, int64_t row_end, bool vec_ok,
-                                      float (&v)[4]) {
-    // four consecutive elements starting at `elem`; zero past row_end
-    if (vec_ok && elem + 4 <= row_end) {
-        if constexpr (DT == BT_F32) {
-            const float4 t = *(const float4*)((const float*)W + elem);
-            v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-        } else {
-            const uint2 t = *(const uint2*)((const uint16_t*)W + elem);
-            const uint16_t h[4] = {(uint16_t)(t.x & 0xffff), (uint16_t)(t.x >> 16),
-                                   (uint16_t)(t.y & 0xffff), (uint16_t)(t.y >> 16)};
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                v[i] = (DT == BT_F16) ? f16_bits_to_f32(h[i]) : bf16_bits_to_f32(h[i]);
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < 4; i++) v[i] = (elem + i < row_end) ? load_elem<DT>(W, elem + i) : 0.0f;
-    }
 }
 
 __device__ __forceinline__ uint32_t encode4(const float (&v)[4], float thr, uint32_t& tern4) {
@@ -60,198 +43,336 @@ __device__ __forceinline__ uint32_t encode4(const float (&v)[4], float thr, uint
     return byte;
 }
 
-// ITERS > 0: rows of up to ITERS*256 elements held in registers (single pass).
-// ITERS == 0: any K; the row is read twice (absmax pass, encode pass).
-template <int DT, int ITERS>
-__global__ __launch_bounds__(256) void quantize_pack_kernel(
-    const void* __restrict__ W, int64_t N, int64_t K, int64_t Kb, float tf, float clamp_min,
-    int per_channel, uint8_t* __restrict__ packed_T, float* __restrict__ scale,
-    int8_t* __restrict__ w_tern, int64_t tiles, int64_t per_xcd) {
-    extern __shared__ uint32_t lds[];  // [Kb][4]: dword (kb, wave) = 4 row bytes
+// ---- fast kernel ---------------------------------------------------------------------
+// ITERS float4 groups per lane (>= K/256), WAVES waves, RPW rows per wave one after another.
+// LDS tile: byte (kb, row) at kb*PITCHB + row, PITCHB = R + 4: the odd dword pitch keeps the
+// column writes (lanes = consecutive kb) and the row reads free of bank conflicts.
+template <int DT, int ITERS, int WAVES, int RPW>
+__global__ __launch_bounds__(WAVES * 64) void quantize_pack_fast_kernel(
+    const void* __restrict__ W, int N, int K, float tf, float clamp_min, int per_channel,
+    uint8_t* __restrict__ packed_T, float* __restrict__ scale, int tiles, int per_xcd) {
+    constexpr int R = WAVES * RPW;
+    constexpr int PITCHB = R + 4;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_b[];
+    const int tile = (int)xcd_tile(blockIdx.x, per_xcd);
+    if (tile >= tiles) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n0 = tile * R;
+    const int nfull = K >> 8;  // complete 256-element chunks (uniform)
+    const int Kb = K >> 2;
+    const float tensor_scale = per_channel ? 0.0f : fmaxf(scale[0], clamp_min);
+    uint32_t pk[ITERS];
+#pragma unroll
+    for (int j = 0; j < ITERS; j++) pk[j] = 0;
+#pragma unroll 1  // one row in registers at a time
+    for (int r = 0; r < RPW; r++) {
+        const int n = n0 + RPW * wave + r;
+        float4 v[ITERS];
+        if constexpr (DT == BT_F32) {
+            const float4* rowp = (const float4*)((const float*)W + (int64_t)n * K) + lane;
+#pragma unroll
+            for (int j = 0; j < ITERS; j++) v[j] = (j < nfull) ? rowp[j * 64] : make_float4(0.f, 0.f, 0.f, 0.f);
+        } else {
+            const uint2* rowp = (const uint2*)((const uint16_t*)W + (int64_t)n * K) + lane;
+#pragma unroll
+            for (int j = 0; j < ITERS; j++) {
+                const uint2 t = (j < nfull) ? rowp[j * 64] : make_uint2(0u, 0u);
+                if constexpr (DT == BT_F16)
+                    v[j] = make_float4(f16_bits_to_f32((uint16_t)t.x), f16_bits_to_f32((uint16_t)(t.x >> 16)),
+                                       f16_bits_to_f32((uint16_t)t.y), f16_bits_to_f32((uint16_t)(t.y >> 16)));
+                else
+                    v[j] = make_float4(bf16_bits_to_f32((uint16_t)t.x), bf16_bits_to_f32((uint16_t)(t.x >> 16)),
+                                       bf16_bits_to_f32((uint16_t)t.y), bf16_bits_to_f32((uint16_t)(t.y >> 16)));
+            }
+        }
+        float amax = 0.0f;
+#pragma unroll
+        for (int j = 0; j < ITERS; j++)
+            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[j].x), fabsf(v[j].y)), fmaxf(fabsf(v[j].z), fabsf(v[j].w))));
+        float s;
+        if (per_channel) {
+            s = fmaxf(wave_max(amax), clamp_min);
+            if (lane == 0) scale[n] = s;
+        } else {
+            s = tensor_scale;
+        }
+        const float thr = round_to_dtype(__fmul_rn(tf, s), DT);
+#pragma unroll
+        for (int j = 0; j < ITERS; j++) {
+            const float a[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+            uint32_t t4;
+            pk[j] |= encode4(a, thr, t4) << (8 * r);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < ITERS; j++) {
+        if (j < nfull) {
+            uint8_t* dst = lds_b + (j * 64 + lane) * PITCHB + wave * RPW;
+            if constexpr (RPW == 4) *(uint32_t*)dst = pk[j];
+            else if constexpr (RPW == 2) *(uint16_t*)dst = (uint16_t)pk[j];
+            else *dst = (uint8_t)pk[j];
+        }
+    }
+    __syncthreads();
+    constexpr int Q = R / 16;  // 16-byte pieces per packed_T row segment
+    for (int idx = threadIdx.x; idx < Kb * Q; idx += WAVES * 64) {
+        const int kb = idx / Q, q = idx % Q;
+        const uint32_t* src = (const uint32_t*)(lds_b + kb * PITCHB + 16 * q);
+        *(uint4*)(packed_T + (int64_t)kb * N + n0 + 16 * q) = make_uint4(src[0], src[1], src[2], src[3]);
+    }
+}
 
+template <int DT, int ITERS, int WAVES, int RPW>
+static int launch_fast_cfg(const void* W, int64_t N, int64_t K, float tf, float clamp_min, int per_channel,
+                           uint8_t* packed_T, float* scale, hipStream_t st) {
+    constexpr int R = WAVES * RPW;
+    const int tiles = (int)(N / R);
+    const int per_xcd = (int)ceil_div(tiles, 8);
+    const size_t lds = (size_t)(K / 4) * (R + 4);
+    auto kern = quantize_pack_fast_kernel<DT, ITERS, WAVES, RPW>;
+    if (lds > 64 * 1024 &&
+        hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+        set_error("bt_quantize_pack: cannot reserve %zu bytes of LDS", lds);
+        return BT_ERR_LAUNCH;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(WAVES * 64), lds, st, W, (int)N, (int)K, tf,
+                       clamp_min, per_channel, packed_T, scale, tiles, per_xcd);
+    return check_launch("bt_quantize_pack");
+}
+
+// Row tile for the fast kernel: as many rows per wave (bytes per packed_T segment) as still
+// leave more than one tile per CU; at least 16 rows per workgroup (one 16-byte piece).
+template <int DT, int ITERS, int WAVES>
+static int launch_fast_rows(const void* W, int64_t N, int64_t K, float tf, float clamp_min, int per_channel,
+                            uint8_t* packed_T, float* scale, hipStream_t st, int* rc) {
+    constexpr int MIN_RPW = (WAVES >= 16) ? 1 : (WAVES >= 8) ? 2 : 4;
+    int rpw = 0;
+    if (const char* env = getenv("BITTORCH_QP_RPW")) rpw = atoi(env);
+    if (rpw != 1 && rpw != 2 && rpw != 4) {
+        rpw = 4;
+        while (rpw > MIN_RPW && (N % (WAVES * rpw) != 0 || N / (WAVES * rpw) < 320)) rpw >>= 1;
+    }
+    if (rpw < MIN_RPW) rpw = MIN_RPW;
+    if (N % (WAVES * rpw) != 0 || (size_t)(K / 4) * (WAVES * rpw + 4) > 150 * 1024) return 0;
+    if (rpw == 4) {
+        *rc = launch_fast_cfg<DT, ITERS, WAVES, 4>(W, N, K, tf, clamp_min, per_channel, packed_T, scale, st);
+    } else if (rpw == 2) {
+        if constexpr (MIN_RPW <= 2)
+            *rc = launch_fast_cfg<DT, ITERS, WAVES, 2>(W, N, K, tf, clamp_min, per_channel, packed_T, scale, st);
+    } else {
+        if constexpr (MIN_RPW <= 1)
+            *rc = launch_fast_cfg<DT, ITERS, WAVES, 1>(W, N, K, tf, clamp_min, per_channel, packed_T, scale, st);
+    }
+    return 1;
+}
+
+// returns 1 if the fast kernel took the call (rc holds its status), 0 if the shape does not
+// qualify.  Register budget: a row of K elements costs K/64 data registers per lane, so 16 waves
+// per workgroup fit K <= 4096, 8 waves K <= 8192, 4 waves K <= 11008.
+template <int DT>
+static int try_launch_fast(const void* W, int64_t N, int64_t K, float tf, float clamp_min, int per_channel,
+                           uint8_t* packed_T, float* scale, int8_t* w_tern, hipStream_t st, int* rc) {
+    if (!packed_T || w_tern || K % 256 != 0 || ((uintptr_t)W) % 16 != 0 || ((uintptr_t)packed_T) % 16 != 0 ||
+        N * K >= (1ll << 31) || getenv("BITTORCH_QP_GENERIC"))
+        return 0;
+    const int chunks = (int)(K / 256);
+#define BT_QF(IT, WV) \
+    if (chunks <= IT) return launch_fast_rows<DT, IT, WV>(W, N, K, tf, clamp_min, per_channel, packed_T, scale, st, rc)
+    BT_QF(4, 16);
+    BT_QF(8, 16);
+    BT_QF(16, 16);
+    BT_QF(24, 8);
+    BT_QF(32, 8);
+    BT_QF(43, 4);
+#undef BT_QF
+    return 0;
+}
+
+// ---- generic kernel --------------------------------------------------------------------
+template <int DT>
+__device__ __forceinline__ void load4(const void* W, int64_t elem, int64_t row_end, bool vec_ok, float (&v)[4]) {
+    // four consecutive elements starting at `elem`; zero past row_end
+    if (vec_ok && elem + 4 <= row_end) {
+        if constexpr (DT == BT_F32) {
+            const float4 t = *(const float4*)((const float*)W + elem);
+            v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+        } else {
+            const uint2 t = *(const uint2*)((const uint16_t*)W + elem);
+            const uint16_t h[4] = {(uint16_t)(t.x & 0xffff), (uint16_t)(t.x >> 16),
+                                   (uint16_t)(t.y & 0xffff), (uint16_t)(t.y >> 16)};
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[i] = (DT == BT_F16) ? f16_bits_to_f32(h[i]) : bf16_bits_to_f32(h[i]);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) v[i] = (elem + i < row_end) ? load_elem<DT>(W, elem + i) : 0.0f;
+    }
+}
+
+// 256 threads own 16 rows (wave w rows n0+4w .. +3).  Pass 1: the four row scales.
+// Pass 2, per segment of up to G_SEG packed rows: encode, put the four rows' bytes into one
+// dword per kb in LDS (pitch 5 dwords), then 16-byte transposed stores.
+constexpr int G_SEG = 2048;
+template <int DT>
+__global__ __launch_bounds__(256) void quantize_pack_generic_kernel(
+    const void* __restrict__ W, int64_t N, int64_t K, int64_t Kb, float tf, float clamp_min, int per_channel,
+    uint8_t* __restrict__ packed_T, float* __restrict__ scale, int8_t* __restrict__ w_tern, int64_t tiles,
+    int64_t per_xcd) {
+    constexpr int PITCH = 5;
+    __shared__ uint32_t lds[G_SEG * PITCH];
     const int64_t tile = xcd_tile(blockIdx.x, per_xcd);
     if (tile >= tiles) return;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int64_t n0 = tile * 16;
-    // 16-byte (fp32) / 8-byte (16-bit) vector loads need aligned rows
     const bool vec_ok = (K % 4 == 0) && (((uintptr_t)W) % 16 == 0);
+    const bool tern_vec = vec_ok && (((uintptr_t)w_tern) % 4 == 0);
     const float tensor_scale = per_channel ? 0.0f : fmaxf(scale[0], clamp_min);
 
-    if constexpr (ITERS > 0) {
-        uint32_t pk[ITERS];
+    float thr[4];
 #pragma unroll
-        for (int j = 0; j < ITERS; j++) pk[j] = 0;
-
-        for (int r = 0; r < 4; r++) {
-            const int64_t n = n0 + 4 * wave + r;
-            if (n >= N) break;  // uniform per wave
-            const int64_t row0 = n * K, row_end = row0 + K;
-            float v[ITERS][4];
+    for (int r = 0; r < 4; r++) {
+        const int64_t n = n0 + 4 * wave + r;
+        float s = tensor_scale;
+        if (per_channel && n < N) {  // uniform per wave
+            const int64_t row0 = n * K;
             float amax = 0.0f;
+            for (int64_t kb = lane; kb < Kb; kb += 64) {
+                float v[4];
+                load4<DT>(W, row0 + 4 * kb, row0 + K, vec_ok, v);
+                amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))));
+            }
+            s = fmaxf(wave_max(amax), clamp_min);
+            if (lane == 0) scale[n] = s;
+        }
+        thr[r] = round_to_dtype(__fmul_rn(tf, s), DT);
+    }
+
+    const bool full = (n0 + 16 <= N) && (N % 16 == 0) && (((uintptr_t)packed_T) % 16 == 0);
+    for (int64_t seg0 = 0; seg0 < Kb; seg0 += G_SEG) {
+        const int seg_len = (int)((Kb - seg0 < G_SEG) ? (Kb - seg0) : G_SEG);
+        for (int kl = lane; kl < seg_len; kl += 64) {
+            const int64_t kb = seg0 + kl;
+            uint32_t word = 0;
 #pragma unroll
-            for (int j = 0; j < ITERS; j++) {
-                const int64_t kb = (int64_t)j * 64 + lane;
-                if (kb < Kb) {
-                    load4<DT>(W, row0 + 4 * kb, row_end, vec_ok, v[j]);
-                } else {
-                    v[j][0] = v[j][1] = v[j][2] = v[j][3] = 0.0f;
+            for (int r = 0; r < 4; r++) {
+                const int64_t n = n0 + 4 * wave + r;
+                if (n < N) {
+                    const int64_t row0 = n * K, row_end = row0 + K;
+                    float v[4];
+                    load4<DT>(W, row0 + 4 * kb, row_end, vec_ok, v);
+                    uint32_t tern4;
+                    word |= encode4(v, thr[r], tern4) << (8 * r);
+                    if (w_tern) {
+                        const int64_t e = row0 + 4 * kb;
+                        if (tern_vec && e + 4 <= row_end) {
+                            *(uint32_t*)(w_tern + e) = tern4;
+                        } else {
+                            for (int i = 0; i < 4; i++)
+                                if (e + i < row_end) w_tern[e + i] = (int8_t)((tern4 >> (8 * i)) & 0xff);
+                        }
+                    }
                 }
-                amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[j][0]), fabsf(v[j][1])),
-                                         fmaxf(fabsf(v[j][2]), fabsf(v[j][3]))));
             }
-            float s;
-            if (per_channel) {
-                s = fmaxf(wave_max(amax), clamp_min);
-                if (lane == 0) scale[n] = s;
+            if (packed_T) lds[kl * PITCH + wave] = word;
+        }
+        if (!packed_T) continue;  // uniform
+        __syncthreads();
+        for (int kl = threadIdx.x; kl < seg_len; kl += 256) {
+            const uint32_t d[4] = {lds[kl * PITCH], lds[kl * PITCH + 1], lds[kl * PITCH + 2], lds[kl * PITCH + 3]};
+            uint8_t* dst = packed_T + (seg0 + kl) * N + n0;
+            if (full) {
+                *(uint4*)dst = make_uint4(d[0], d[1], d[2], d[3]);
             } else {
-                s = tensor_scale;
+                for (int i = 0; i < 16; i++)
+                    if (n0 + i < N) dst[i] = (uint8_t)((d[i >> 2] >> (8 * (i & 3))) & 0xff);
             }
-            const float thr = round_to_dtype(__fmul_rn(tf, s), DT);
+        }
+        __syncthreads();
+    }
+}
+
+// tensor absmax into scale[0] (the bit pattern of a non-negative float orders like a uint)
+template <int DT>
+__global__ __launch_bounds__(256) void absmax_kernel(const void* __restrict__ W, int64_t total, int vec_ok,
+                                                     float* __restrict__ scale) {
+    float amax = 0.0f;
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    const int64_t tid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    int64_t done = 0;
+    if (vec_ok) {
+        // 16-byte loads, four per thread in flight
+        constexpr int EPV = (DT == BT_F32) ? 4 : 8;  // elements per 16 bytes
+        const int64_t nvec = total / EPV;
+        const uint4* p = (const uint4*)W;
+        for (int64_t i = tid; i < nvec; i += 4 * stride) {
+            uint4 q[4];
 #pragma unroll
-            for (int j = 0; j < ITERS; j++) {
-                const int64_t kb = (int64_t)j * 64 + lane;
-                uint32_t tern4;
-                const uint32_t byte = encode4(v[j], thr, tern4);
-                pk[j] |= byte << (8 * r);
-                if (w_tern && kb < Kb) {
-                    const int64_t e = row0 + 4 * kb;
-                    if (vec_ok && e + 4 <= row_end) {
-                        *(uint32_t*)(w_tern + e) = tern4;
+            for (int u = 0; u < 4; u++)
+                q[u] = (i + u * stride < nvec) ? p[i + u * stride] : make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const uint32_t d[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    if constexpr (DT == BT_F32) {
+                        amax = fmaxf(amax, fabsf(__builtin_bit_cast(float, d[e])));
+                    } else if constexpr (DT == BT_F16) {
+                        amax = fmaxf(amax, fabsf(f16_bits_to_f32((uint16_t)d[e])));
+                        amax = fmaxf(amax, fabsf(f16_bits_to_f32((uint16_t)(d[e] >> 16))));
                     } else {
-                        for (int i = 0; i < 4; i++)
-                            if (e + i < row_end) w_tern[e + i] = (int8_t)((tern4 >> (8 * i)) & 0xff);
+                        amax = fmaxf(amax, fabsf(bf16_bits_to_f32((uint16_t)d[e])));
+                        amax = fmaxf(amax, fabsf(bf16_bits_to_f32((uint16_t)(d[e] >> 16))));
                     }
                 }
             }
         }
-        if (packed_T) {
-#pragma unroll
-            for (int j = 0; j < ITERS; j++) {
-                const int64_t kb = (int64_t)j * 64 + lane;
-                if (kb < Kb) lds[kb * 4 + wave] = pk[j];
-            }
-        }
-    } else {
-        for (int r = 0; r < 4; r++) {
-            const int64_t n = n0 + 4 * wave + r;
-            if (n >= N) break;
-            const int64_t row0 = n * K, row_end = row0 + K;
-            float s;
-            if (per_channel) {
-                float amax = 0.0f;
-                for (int64_t kb = lane; kb < Kb; kb += 64) {
-                    float v[4];
-                    load4<DT>(W, row0 + 4 * kb, row_end, vec_ok, v);
-                    amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])),
-                                             fmaxf(fabsf(v[2]), fabsf(v[3]))));
-                }
-                s = fmaxf(wave_max(amax), clamp_min);
-                if (lane == 0) scale[n] = s;
-            } else {
-                s = tensor_scale;
-            }
-            const float thr = round_to_dtype(__fmul_rn(tf, s), DT);
-            for (int64_t kb = lane; kb < Kb; kb += 64) {
-                float v[4];
-                load4<DT>(W, row0 + 4 * kb, row_end, vec_ok, v);
-                uint32_t tern4;
-                const uint32_t byte = encode4(v, thr, tern4);
-                if (packed_T) {
-                    // bytes of the wave's four rows share a dword; rows run one after
-                    // another in this wave, so a plain read-modify-write is race free
-                    uint32_t cur = (r == 0) ? 0u : lds[kb * 4 + wave];
-                    lds[kb * 4 + wave] = cur | (byte << (8 * r));
-                }
-                if (w_tern) {
-                    const int64_t e = row0 + 4 * kb;
-                    for (int i = 0; i < 4; i++)
-                        if (e + i < row_end) w_tern[e + i] = (int8_t)((tern4 >> (8 * i)) & 0xff);
-                }
-            }
-        }
+        done = nvec * EPV;
     }
-    if (!packed_T) return;
-    // rows past N in a ragged last tile leave their byte lanes untouched: zero them
-    // by construction (pk starts at 0; for ITERS == 0 a wave with no valid row
-    // never wrote its dword), so make such dwords explicit zeros
-    if (n0 + 4 * wave >= N) {
-        for (int64_t kb = lane; kb < Kb; kb += 64) lds[kb * 4 + wave] = 0u;
-    }
-    __syncthreads();
-
-    const bool full = (n0 + 16 <= N) && (N % 16 == 0) && (((uintptr_t)packed_T) % 16 == 0);
-    for (int64_t kb = threadIdx.x; kb < Kb; kb += 256) {
-        const uint4 q = *(const uint4*)(lds + kb * 4);
-        uint8_t* dst = packed_T + kb * N + n0;
-        if (full) {
-            *(uint4*)dst = q;
-        } else {
-            const uint32_t d[4] = {q.x, q.y, q.z, q.w};
-            for (int i = 0; i < 16; i++)
-                if (n0 + i < N) dst[i] = (uint8_t)((d[i >> 2] >> (8 * (i & 3))) & 0xff);
-        }
-    }
-}
-
-// tensor absmax into scale[0] (bit pattern of a non-negative float orders like a uint)
-template <int DT>
-__global__ __launch_bounds__(256) void absmax_kernel(const void* __restrict__ W, int64_t total,
-                                                     float* __restrict__ scale) {
-    float amax = 0.0f;
-    const int64_t stride = (int64_t)gridDim.x * 256;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride)
-        amax = fmaxf(amax, fabsf(load_elem<DT>(W, i)));
+    for (int64_t i = done + tid; i < total; i += stride) amax = fmaxf(amax, fabsf(load_elem<DT>(W, i)));
+    // one atomic per workgroup, and only if it can still raise the maximum: atomics of all
+    // XCDs on one address serialise at roughly ten nanoseconds each
+    __shared__ float part[4];
     amax = wave_max(amax);
-    if ((threadIdx.x & 63) == 0) atomicMax((unsigned int*)scale, __builtin_bit_cast(unsigned int, amax));
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        amax = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
+        if (amax > __hip_atomic_load(scale, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+            atomicMax((unsigned int*)scale, __builtin_bit_cast(unsigned int, amax));
+    }
 }
 
 __global__ void set_scalar_kernel(float* p, float v) { *p = v; }
 __global__ void floor_scalar_kernel(float* p, float floor_v) { *p = fmaxf(*p, floor_v); }
 
 template <int DT>
-static int launch_quantize(const void* W, int64_t N, int64_t K, float tf, float clamp_min,
-                           int per_channel, uint8_t* packed_T, float* scale, int8_t* w_tern,
-                           hipStream_t st) {
+static int launch_quantize(const void* W, int64_t N, int64_t K, float tf, float clamp_min, int per_channel,
+                           uint8_t* packed_T, float* scale, int8_t* w_tern, hipStream_t st) {
+    int rc = BT_OK;
+    if (try_launch_fast<DT>(W, N, K, tf, clamp_min, per_channel, packed_T, scale, w_tern, st, &rc)) return rc;
     const int64_t Kb = ceil_div(K, 4);
     const int64_t tiles = ceil_div(N, 16);
     const int64_t per_xcd = ceil_div(tiles, 8);
-    const dim3 grid((unsigned)(per_xcd * 8)), block(256);
-    const size_t lds = packed_T ? (size_t)Kb * 16 : 0;
-    if (lds > 160 * 1024 - 1024) {
-        set_error("bt_quantize_pack: K=%lld too large for the LDS transpose tile", (long long)K);
-        return BT_ERR_INVALID;
-    }
-#define BT_QP(IT)                                                                              \
-    hipLaunchKernelGGL((quantize_pack_kernel<DT, IT>), grid, block, lds, st, W, N, K, Kb, tf,  \
-                       clamp_min, per_channel, packed_T, scale, w_tern, tiles, per_xcd)
-    if (lds > 64 * 1024) {
-        // beyond the default dynamic LDS limit: raise it for the generic variant
-        if (hipFuncSetAttribute((const void*)quantize_pack_kernel<DT, 0>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
-            set_error("bt_quantize_pack: cannot reserve %zu bytes of LDS", lds);
-            return BT_ERR_LAUNCH;
-        }
-    }
-    if (K <= 1024) BT_QP(4);
-    else if (K <= 2048) BT_QP(8);
-    else if (K <= 4096) BT_QP(16);
-    else if (K <= 8192) BT_QP(32);
-    else if (K <= 12288) BT_QP(48);
-    else BT_QP(0);
-#undef BT_QP
+    hipLaunchKernelGGL(quantize_pack_generic_kernel<DT>, dim3((unsigned)(per_xcd * 8)), dim3(256), 0, st, W, N, K,
+                       Kb, tf, clamp_min, per_channel, packed_T, scale, w_tern, tiles, per_xcd);
     return check_launch("bt_quantize_pack");
+}
+
+template <int DT>
+static void launch_absmax(const void* W, int64_t total, float* scale, hipStream_t st) {
+    const int vec_ok = (((uintptr_t)W) % 16 == 0) ? 1 : 0;
+    const unsigned blocks = (unsigned)std::min<int64_t>(std::max<int64_t>(ceil_div(total, 256 * 16), 1), 1024);
+    hipLaunchKernelGGL(absmax_kernel<DT>, dim3(blocks), dim3(256), 0, st, W, total, vec_ok, scale);
 }
 
 }  // namespace bt
 
-extern "C" int bt_quantize_pack(const void* W, int w_dtype, int64_t N, int64_t K,
-                                double threshold_factor, int per_channel, uint8_t* packed_T,
-                                float* scale, int8_t* w_tern, void* stream) {
+extern "C" int bt_quantize_pack(const void* W, int w_dtype, int64_t N, int64_t K, double threshold_factor,
+                                int per_channel, uint8_t* packed_T, float* scale, int8_t* w_tern, void* stream) {
     using namespace bt;
     if (!W || !scale || N <= 0 || K <= 0) {
-        set_error("bt_quantize_pack: null pointer or empty shape (N=%lld K=%lld)", (long long)N,
-                  (long long)K);
+        set_error("bt_quantize_pack: null pointer or empty shape (N=%lld K=%lld)", (long long)N, (long long)K);
         return BT_ERR_INVALID;
     }
     if (w_dtype != BT_F32 && w_dtype != BT_F16 && w_dtype != BT_BF16) {
@@ -270,15 +391,12 @@ extern "C" int bt_quantize_pack(const void* W, int w_dtype, int64_t N, int64_t K
         clamp_min = __builtin_bit_cast(float, u);
     }
     if (!per_channel) {
+        // tensor scale: zero, absmax over everything, quantize against it, then floor it
         hipLaunchKernelGGL(set_scalar_kernel, dim3(1), dim3(1), 0, st, scale, 0.0f);
         const int64_t total = N * K;
-        const unsigned blocks = (unsigned)std::min<int64_t>(ceil_div(total, 256 * 16), 2048);
-        if (w_dtype == BT_F32)
-            hipLaunchKernelGGL(absmax_kernel<BT_F32>, dim3(blocks), dim3(256), 0, st, W, total, scale);
-        else if (w_dtype == BT_F16)
-            hipLaunchKernelGGL(absmax_kernel<BT_F16>, dim3(blocks), dim3(256), 0, st, W, total, scale);
-        else
-            hipLaunchKernelGGL(absmax_kernel<BT_BF16>, dim3(blocks), dim3(256), 0, st, W, total, scale);
+        if (w_dtype == BT_F32) launch_absmax<BT_F32>(W, total, scale, st);
+        else if (w_dtype == BT_F16) launch_absmax<BT_F16>(W, total, scale, st);
+        else launch_absmax<BT_BF16>(W, total, scale, st);
     }
     int rc;
     if (w_dtype == BT_F32)
