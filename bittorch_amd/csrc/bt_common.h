@@ -59,6 +59,17 @@ __device__ __forceinline__ float load_elem_rt(const void* p, int dt, int64_t i) 
     if (dt == BT_F16) return f16_bits_to_f32(((const uint16_t*)p)[i]);
     return bf16_bits_to_f32(((const uint16_t*)p)[i]);
 }
+// The same in two halves, so that a caller can issue the load early and convert late:
+// the load leaves raw bits in a register (no use, hence no wait, inside the dtype branch).
+__device__ __forceinline__ uint32_t load_bits_rt(const void* p, int dt, int64_t i) {
+    if (dt == BT_F32) return ((const uint32_t*)p)[i];
+    return (uint32_t)((const uint16_t*)p)[i];
+}
+__device__ __forceinline__ float bits_to_f32_rt(uint32_t bits, int dt) {
+    if (dt == BT_F32) return __builtin_bit_cast(float, bits);
+    if (dt == BT_F16) return f16_bits_to_f32((uint16_t)bits);
+    return bf16_bits_to_f32((uint16_t)bits);
+}
 // round a float to the grid of dtype dt and widen it again
 __device__ __forceinline__ float round_to_dtype(float v, int dt) {
     if (dt == BT_F16) return f16_bits_to_f32(f32_to_f16_bits(v));

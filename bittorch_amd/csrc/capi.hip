@@ -28,7 +28,7 @@ int check_launch(const char* what) {
 }
 
 // kernels in the other translation units
-bool stream_supported(int64_t N, const void* W_T);
+bool stream_supported(int64_t N, int64_t K, const void* W_T);
 size_t stream_workspace_bytes(int mode, int64_t M, int64_t N, int64_t Kb);
 int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, const uint8_t* W_T,
                   const Epilogue& epi, void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N,
@@ -120,7 +120,7 @@ extern "C" int bt_ternary_linear_forward(const void* X, int x_dtype, const int8_
 
 static bool packed_uses_stream(int x_dtype, const void* W_T, const void* Y, int64_t N, int64_t K) {
     if (getenv("BITTORCH_KERNEL") && !strcmp(getenv("BITTORCH_KERNEL"), "generic")) return false;
-    return x_dtype != BT_F32 && stream_supported(N, W_T) && fast_path_ok(Y, N, K);
+    return x_dtype != BT_F32 && stream_supported(N, K, W_T) && fast_path_ok(Y, N, K);
 }
 
 extern "C" size_t bt_packed_forward_workspace_bytes(int64_t B, int64_t N, int64_t K, int x_dtype) {
@@ -188,9 +188,15 @@ extern "C" int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8
     hipStream_t st = (hipStream_t)stream;
     // decode-shape batches, and any batch whose N the tiled kernel's 4-column
     // vector accesses cannot take, stream the weights once per 16 rows
-    if (B <= kStreamMaxRows || !gemm_i8_supported(N, K, Q, W_T))
+    if (B <= kStreamMaxRows || !gemm_i8_supported(N, K, Q, W_T)) {
+        if (!stream_supported(N, K, W_T)) {
+            set_error("%s: packed weight matrix of %lld x %lld bytes exceeds the 4 GiB the kernels address", who,
+                      (long long)ceil_div(K, 4), (long long)N);
+            return BT_ERR_INVALID;
+        }
         return launch_stream(MODE_I8, Q, 1, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, workspace,
                              workspace_bytes, st);
+    }
     return launch_gemm_i8(Q, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, st);
 }
 

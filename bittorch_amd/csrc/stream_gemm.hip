@@ -52,17 +52,14 @@ template <> struct RawVec<4> { typedef uint32_t type; };
 template <> struct RawVec<2> { typedef uint16_t type; };
 template <> struct RawVec<1> { typedef uint8_t type; };
 
-// NW bytes of one kb row into ceil(NW/4) dwords (zero extended / zero when !ok)
+// NW bytes at W_T + off into ceil(NW/4) dwords (zero extended).  The load is unconditional
+// (the caller clamps `off` to a valid location): a load under a per-lane predicate becomes a
+// branch with a wait behind it, which serialises the stream.
 template <int NW>
-__device__ __forceinline__ void load_raw(const uint8_t* p, bool ok, uint32_t (&d)[(NW + 3) / 4]) {
-    if (ok) {
-        const typename RawVec<NW>::type v = *(const typename RawVec<NW>::type*)p;
-        if constexpr (NW >= 4) __builtin_memcpy(d, &v, NW);
-        else d[0] = (uint32_t)v;
-    } else {
-#pragma unroll
-        for (int i = 0; i < (NW + 3) / 4; i++) d[i] = 0u;
-    }
+__device__ __forceinline__ void load_raw(const uint8_t* base, uint32_t off, uint32_t (&d)[(NW + 3) / 4]) {
+    const typename RawVec<NW>::type v = *(const typename RawVec<NW>::type*)(base + off);
+    if constexpr (NW >= 4) __builtin_memcpy(d, &v, NW);
+    else d[0] = (uint32_t)v;
 }
 
 __device__ __forceinline__ void store_out(void* Y, int dt, int64_t idx, float v) {
@@ -72,9 +69,8 @@ __device__ __forceinline__ void store_out(void* Y, int dt, int64_t idx, float v)
 }
 
 template <int MODE>
-__device__ __forceinline__ void finish_output(const StreamParams& p, int row, int64_t n, uint32_t bits) {
-    const float s = epi_scale(p.epi, n);
-    const float b = epi_bias(p.epi, n);
+__device__ __forceinline__ void finish_output(const StreamParams& p, int row, int64_t n, uint32_t bits, float s,
+                                              float b) {
     float y;
     if constexpr (MODE == MODE_I8) {
         const int32_t acc127 = times127((int32_t)bits);  // MFMA ran on +-1 weights
@@ -95,35 +91,33 @@ __device__ __forceinline__ uint32_t add_bits(uint32_t a, uint32_t b) {
     else return __builtin_bit_cast(uint32_t, __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b));
 }
 
-// 16 bytes of activations for lane (row i, group g) of one step, in natural k order
-template <int MODE>
-__device__ __forceinline__ uint4 load_x_frag(const StreamParams& p, int i, int64_t k) {
+// 16 bytes of activations for lane (row i, group g) of one step, in natural k order.
+// XV: rows are 16-byte aligned and K is a multiple of the 16-byte group, so a group that
+// starts below K lies wholly inside its row; the load is unconditional on a clamped address
+// (xrow = element offset of row min(i, M-1)) and the caller zeroes groups at k >= K when it
+// consumes them.  !XV: element-wise gather (unaligned or ragged rows), zero filled.
+template <int MODE, bool XV>
+__device__ __forceinline__ uint4 load_x_frag(const StreamParams& p, uint32_t xrow, int i, int k) {
     constexpr int GE = (MODE == MODE_I8) ? 16 : 8;
-    uint4 v = make_uint4(0u, 0u, 0u, 0u);
-    if (i < p.M && k < p.K) {
-        if constexpr (MODE == MODE_I8) {
-            const uint8_t* src = (const uint8_t*)p.X + (int64_t)i * p.K + k;
-            if (p.x_vec_ok && k + GE <= p.K) {
-                v = *(const uint4*)src;
-            } else {
-                uint32_t d[4] = {0u, 0u, 0u, 0u};
+    constexpr int ES = (MODE == MODE_I8) ? 1 : 2;
+    if constexpr (XV) {
+        const uint32_t kc = (uint32_t)min(k, (int)p.K - GE);
+        return *(const uint4*)((const uint8_t*)p.X + (xrow + kc) * ES);
+    } else {
+        uint32_t d[4] = {0u, 0u, 0u, 0u};
+        if (i < p.M && k < p.K) {
+            if constexpr (MODE == MODE_I8) {
+                const uint8_t* src = (const uint8_t*)p.X + (int64_t)i * p.K + k;
                 for (int e = 0; e < GE; e++)
                     if (k + e < p.K) d[e >> 2] |= (uint32_t)src[e] << (8 * (e & 3));
-                v = make_uint4(d[0], d[1], d[2], d[3]);
-            }
-        } else {
-            const uint16_t* src = (const uint16_t*)p.X + (int64_t)i * p.K + k;
-            if (p.x_vec_ok && k + GE <= p.K) {
-                v = *(const uint4*)src;
             } else {
-                uint32_t d[4] = {0u, 0u, 0u, 0u};
+                const uint16_t* src = (const uint16_t*)p.X + (int64_t)i * p.K + k;
                 for (int e = 0; e < GE; e++)
                     if (k + e < p.K) d[e >> 1] |= (uint32_t)src[e] << (16 * (e & 1));
-                v = make_uint4(d[0], d[1], d[2], d[3]);
             }
         }
+        return make_uint4(d[0], d[1], d[2], d[3]);
     }
-    return v;
 }
 
 template <int MODE, int NW, int WAVES, int PF>
@@ -148,27 +142,58 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
     const int nsteps = (int)((p.Kb + RS - 1) / RS);
     const int64_t ncol = nb + (int64_t)NW * j;
     const bool col_ok = ncol < p.N;
-    const uint8_t* wcol = p.W_T + ncol;
+    // 32-bit offsets from the uniform base pointers (the host checks that they fit), advanced
+    // by uniform strides: row kb of step s, group g, r is kb = s*RS + g*KBG + r.  Rows past the
+    // end are clamped to the last row; their products vanish because the activations at
+    // k >= K are zero, and columns past N are computed on column 0's bytes and never stored.
+    const uint32_t col_off = col_ok ? (uint32_t)ncol : 0u;
+    const uint32_t N32 = (uint32_t)p.N;
+    const uint32_t last_off = (uint32_t)(p.Kb - 1) * N32 + col_off;
+    const uint32_t step_stride = (uint32_t)(WAVES * RS) * N32;
+    uint32_t woff = (uint32_t)(wave * RS + g * KBG) * N32 + col_off;
+    int k0 = 4 * (wave * RS + g * KBG);
+    const uint32_t xrow = (uint32_t)min(j, p.M - 1) * (uint32_t)p.K;
+
+    // epilogue operands of this thread's output column, requested before the weight stream
+    // so that their latency hides behind it (raw bits now, conversion after the reduction)
+    constexpr bool PRE = (WAVES * 64) % TILE_N == 0;  // a thread finishes one column only
+    uint32_t pre_s = 0u, pre_b = 0u;
+    if constexpr (PRE) {
+        const int64_t n = nb + (int)(threadIdx.x % TILE_N);
+        if ((int)threadIdx.x < p.M * TILE_N && n < p.N) {
+            pre_s = load_bits_rt(p.epi.scale, p.epi.scale_dtype, p.epi.scale_bcast ? 0 : n);
+            if (p.epi.bias) pre_b = load_bits_rt(p.epi.bias, p.epi.bias_dtype, n);
+        }
+    }
 
     acc_t acc[NW];
 #pragma unroll
     for (int t = 0; t < NW; t++) acc[t] = acc_t{0, 0, 0, 0};
 
-    for (int base = wave; base < nsteps; base += WAVES * PF) {
+    for (int base = wave; base < nsteps; base += WAVES * PF, woff += PF * step_stride, k0 += 4 * WAVES * RS * PF) {
         uint32_t raw[PF][KBG][ND];
         uint4 xa[PF];
 #pragma unroll
         for (int f = 0; f < PF; f++) {
-            const int step = base + f * WAVES;
-            const int64_t kbs = (int64_t)step * RS + g * KBG;
 #pragma unroll
             for (int r = 0; r < KBG; r++)
-                load_raw<NW>(wcol + (kbs + r) * p.N, col_ok && kbs + r < p.Kb, raw[f][r]);
-            xa[f] = load_x_frag<MODE>(p, j, 4 * kbs);
+                load_raw<NW>(p.W_T, min(woff + (uint32_t)f * step_stride + (uint32_t)r * N32, last_off), raw[f][r]);
+        }
+        if (p.x_vec_ok) {
+#pragma unroll
+            for (int f = 0; f < PF; f++) xa[f] = load_x_frag<MODE, true>(p, xrow, j, k0 + f * 4 * WAVES * RS);
+        } else {
+#pragma unroll
+            for (int f = 0; f < PF; f++) xa[f] = load_x_frag<MODE, false>(p, xrow, j, k0 + f * 4 * WAVES * RS);
         }
 #pragma unroll
         for (int f = 0; f < PF; f++) {
             if (base + f * WAVES >= nsteps) break;  // uniform per wave
+            {
+                const bool k_ok = k0 + f * 4 * WAVES * RS < (int)p.K;  // no-op for the gathered path
+                xa[f].x = k_ok ? xa[f].x : 0u; xa[f].y = k_ok ? xa[f].y : 0u;
+                xa[f].z = k_ok ? xa[f].z : 0u; xa[f].w = k_ok ? xa[f].w : 0u;
+            }
             if constexpr (MODE == MODE_I8) {
                 uint32_t ta[4];
                 transpose4x4_bytes(xa[f].x, xa[f].y, xa[f].z, xa[f].w, ta);
@@ -242,7 +267,15 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
         uint32_t bits = red[row * TILE_N + slot];
 #pragma unroll
         for (int w = 1; w < WAVES; w++) bits = add_bits<MODE>(bits, red[(w * M + row) * TILE_N + slot]);
-        finish_output<MODE>(p, row, nb + nl, bits);
+        float s, b;
+        if constexpr (PRE) {
+            s = bits_to_f32_rt(pre_s, p.epi.scale_dtype);
+            b = p.epi.bias ? bits_to_f32_rt(pre_b, p.epi.bias_dtype) : 0.0f;
+        } else {
+            s = epi_scale(p.epi, nb + nl);
+            b = epi_bias(p.epi, nb + nl);
+        }
+        finish_output<MODE>(p, row, nb + nl, bits, s, b);
     }
 }
 
@@ -253,7 +286,11 @@ struct StreamPlan {
     int waves;  // waves per workgroup
 };
 
-bool stream_supported(int64_t N, const void* W_T) { return ((uintptr_t)W_T) % 16 == 0 && N >= 1; }
+// the kernel addresses W_T and X with 32-bit offsets from their base pointers
+bool stream_supported(int64_t N, int64_t K, const void* W_T) {
+    // (rows up to 16*16*16 past the end enter the offset arithmetic before they are clamped)
+    return ((uintptr_t)W_T) % 16 == 0 && N >= 1 && (ceil_div(K, 4) + 8192) * N < (1ll << 32) && K < (1ll << 26);
+}
 
 StreamPlan stream_plan(int mode, int64_t M, int64_t N, int64_t Kb) {
     StreamPlan pl;
