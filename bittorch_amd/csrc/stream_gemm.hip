@@ -8,24 +8,32 @@
 //   int8 path (csrc/kernels/ternary_gemm_tensor_core.cu:583-589, :652):
 //       acc_i32 = sum_k q[b,k] * (127 w[k,n]);  y = (acc * s_x[b] / 127) * scale[n] + bias[n]
 //
-// Work decomposition.  A wave "step" covers RS consecutive kb rows (16 for int8,
-// 8 for 16-bit floats) and 16*NW output columns: lane (j = lane%16, g = lane/16)
-// loads NW consecutive bytes (a byte, a short, a dword, two or four dwords) from
-// each of the KBG = RS/4 rows kb0 + g*KBG + r.  Those bytes are the B operands of
-// NW MFMA instructions: MFMA t multiplies the 16 activation rows with output
-// columns n = nb + NW*j + t.  The k order inside an MFMA is free as long as both
-// operands agree, so each lane loads its 16 bytes of activations (row i = lane%16,
-// the same k range as its weights) straight from global memory and permutes them
-// into the order the cheapest weight decode produces.
+// Work decomposition.  A wave "step" covers 16 consecutive kb rows (64 values of k)
+// and TILE_N output columns.  Lane (j = lane%16, g = lane/16) ends up holding, per
+// column it serves, one dword G = the packed bytes of rows kb0+4g .. kb0+4g+3: the B
+// operand of one 16x16x64 int8 MFMA, or of two 16x16x32 fp16/bf16 MFMAs.  The k order
+// inside an MFMA is free as long as both operands agree, so the activations are
+// permuted into the order the cheapest weight decode produces.
+//
+// How G gets into the lane depends on the tile width (template LD).  What limits a
+// narrow tile is the number of vector memory instructions a CU can issue, not bytes:
+//   LD_V4/8/16  lane loads 4/8/16 consecutive bytes (that many columns) from each of
+//               its four rows and transposes 4x4 byte blocks in registers;
+//   LD_Q1/Q2    16/32-column tiles: the four lanes of a quad load one dword each
+//               (rows 4g+q, the same four columns) and exchange bytes with DPP
+//               quad permutes - one load instruction per 16x16 block instead of four;
+//   LD_BYTE     N not a multiple of 4: one byte per lane and row.
 // A wave issues the loads of PF steps before it computes any of them, which is
 // what keeps enough bytes in flight to cover the HBM latency.
 // A workgroup owns one column tile over the WHOLE of K: there is no split-K
 // across workgroups, hence no partial sums in memory, no second pass and no
-// inter-workgroup synchronisation.  The tile width is chosen so that there are
-// enough tiles for every CU (down to 16 columns, one byte per lane and row);
-// tiles that share 128-byte lines of W_T are placed on the same XCD so the
-// line is fetched from HBM once.  The waves of a workgroup take steps
-// round-robin and their accumulators are summed through LDS in wave order.
+// inter-workgroup synchronisation.  Tiles that share 128-byte lines of W_T are
+// placed on the same XCD so the line is fetched from HBM once.  The waves of a
+// workgroup take contiguous ranges of steps and their accumulators are summed
+// through LDS in wave order.
+// Activations: for M = 1 (XLDS) a wave fetches its whole K-slice of x with one or a
+// few fully coalesced loads into LDS and reads operand fragments from there; for
+// M > 1 every lane loads its own 16-element fragment per step.
 #include "bt_common.h"
 
 namespace bt {
@@ -45,22 +53,13 @@ struct StreamParams {
     int x_vec_ok;         // activation rows may be read with 16-byte loads
 };
 
-template <int NW> struct RawVec;
+enum { LD_BYTE = 0, LD_Q1 = 1, LD_Q2 = 2, LD_V4 = 4, LD_V8 = 8, LD_V16 = 16 };
+constexpr int XC_MAX = 4;  // XLDS: 16-byte chunks of the x slice per lane
+
+template <int NB> struct RawVec;
 template <> struct RawVec<16> { typedef uint4 type; };
 template <> struct RawVec<8> { typedef uint2 type; };
 template <> struct RawVec<4> { typedef uint32_t type; };
-template <> struct RawVec<2> { typedef uint16_t type; };
-template <> struct RawVec<1> { typedef uint8_t type; };
-
-// NW bytes at W_T + off into ceil(NW/4) dwords (zero extended).  The load is unconditional
-// (the caller clamps `off` to a valid location): a load under a per-lane predicate becomes a
-// branch with a wait behind it, which serialises the stream.
-template <int NW>
-__device__ __forceinline__ void load_raw(const uint8_t* base, uint32_t off, uint32_t (&d)[(NW + 3) / 4]) {
-    const typename RawVec<NW>::type v = *(const typename RawVec<NW>::type*)(base + off);
-    if constexpr (NW >= 4) __builtin_memcpy(d, &v, NW);
-    else d[0] = (uint32_t)v;
-}
 
 __device__ __forceinline__ void store_out(void* Y, int dt, int64_t idx, float v) {
     if (dt == BT_F32) ((float*)Y)[idx] = v;
@@ -91,13 +90,14 @@ __device__ __forceinline__ uint32_t add_bits(uint32_t a, uint32_t b) {
     else return __builtin_bit_cast(uint32_t, __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b));
 }
 
-// 16 bytes of activations for lane (row i, group g) of one step, in natural k order.
+// 16 bytes of activations of row i starting at element k, in natural k order.
 // XV: rows are 16-byte aligned and K is a multiple of the 16-byte group, so a group that
 // starts below K lies wholly inside its row; the load is unconditional on a clamped address
 // (xrow = element offset of row min(i, M-1)) and the caller zeroes groups at k >= K when it
-// consumes them.  !XV: element-wise gather (unaligned or ragged rows), zero filled.
+// consumes them: a load under a per-lane predicate becomes a branch with a wait behind it,
+// which serialises the stream.  !XV: element-wise gather (unaligned or ragged rows), zero filled.
 template <int MODE, bool XV>
-__device__ __forceinline__ uint4 load_x_frag(const StreamParams& p, uint32_t xrow, int i, int k) {
+__device__ __forceinline__ uint4 load_x16(const StreamParams& p, uint32_t xrow, int i, int k) {
     constexpr int GE = (MODE == MODE_I8) ? 16 : 8;
     constexpr int ES = (MODE == MODE_I8) ? 1 : 2;
     if constexpr (XV) {
@@ -120,15 +120,39 @@ __device__ __forceinline__ uint4 load_x_frag(const StreamParams& p, uint32_t xro
     }
 }
 
-template <int MODE, int NW, int WAVES, int PF>
+__device__ __forceinline__ uint4 zero_unless(uint4 v, bool ok) {
+    v.x = ok ? v.x : 0u; v.y = ok ? v.y : 0u; v.z = ok ? v.z : 0u; v.w = ok ? v.w : 0u;
+    return v;
+}
+
+// d = the dword this lane loaded (row 4g+q, four columns); returns the bytes of column q of
+// the dwords of quad lanes 0..3, i.e. rows 4g..4g+3 of this lane's own column.
+__device__ __forceinline__ uint32_t quad_transpose(uint32_t d, uint32_t sel_q) {
+    const uint32_t v0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d, 0x00, 0xf, 0xf, false);
+    const uint32_t v1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d, 0x55, 0xf, 0xf, false);
+    const uint32_t v2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d, 0xAA, 0xf, 0xf, false);
+    const uint32_t v3 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d, 0xFF, 0xf, 0xf, false);
+    const uint32_t t01 = perm(v1, v0, sel_q);  // [v0.b[q], v1.b[q], -, -]
+    const uint32_t t23 = perm(v3, v2, sel_q);
+    return perm(t23, t01, 0x05040100u);
+}
+
+template <int MODE, int LD, int WAVES, int PF, bool XLDS>
 __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
-    constexpr int KBG = (MODE == MODE_I8) ? 4 : 2;  // kb rows per lane group
-    constexpr int RS = 4 * KBG;                     // kb rows per wave step
-    constexpr int TILE_N = 16 * NW;
-    constexpr int ND = (NW + 3) / 4;                // dwords per lane and row
+    constexpr bool QUAD = (LD == LD_Q1 || LD == LD_Q2);
+    constexpr bool BYTE = (LD == LD_BYTE);
+    constexpr int NACC = BYTE ? 1 : LD;             // output columns per lane
+    constexpr int TILE_N = 16 * NACC;
+    constexpr int RAWN = BYTE ? 4 : LD;             // raw dwords per lane and step
+    constexpr int ND = (LD >= 4) ? LD / 4 : 1;      // LD_V*: dwords per lane and row
+    constexpr int NCO = QUAD ? LD : 1;              // column offsets per lane
+    constexpr int ES = (MODE == MODE_I8) ? 1 : 2;   // bytes per activation
+    constexpr int XN = (MODE == MODE_I8) ? 1 : 2;   // 16-byte pieces of x per lane and step
+    constexpr bool TWO = (NACC <= 2);               // second accumulator chain
+    constexpr int NACC2 = TWO ? NACC : 1;
     typedef typename std::conditional<MODE == MODE_I8, v4i, v4f>::type acc_t;
 
-    extern __shared__ __attribute__((aligned(16))) uint32_t red[];  // [WAVES][M][TILE_N]
+    extern __shared__ __attribute__((aligned(16))) uint32_t red[];  // [WAVES][M][TILE_N], then x slices
 
     // consecutive tiles on one XCD (workgroups are dealt round-robin over 8 XCDs)
     const int tile = (int)(blockIdx.x & 7) * p.per_xcd + (int)(blockIdx.x >> 3);
@@ -138,21 +162,34 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
     const int wave = threadIdx.x >> 6;
     const int j = lane & 15;
     const int g = lane >> 4;
+    const int q = lane & 3;
     const int64_t nb = (int64_t)tile * TILE_N;
-    const int nsteps = (int)((p.Kb + RS - 1) / RS);
-    const int64_t ncol = nb + (int64_t)NW * j;
-    const bool col_ok = ncol < p.N;
+    const int nsteps = (int)((p.Kb + 15) >> 4);
+    const int spw = (nsteps + WAVES - 1) / WAVES;  // steps per wave, contiguous
+    const int s_begin = wave * spw;
+    const int s_end = min(nsteps, s_begin + spw);
+
     // 32-bit offsets from the uniform base pointers (the host checks that they fit), advanced
-    // by uniform strides: row kb of step s, group g, r is kb = s*RS + g*KBG + r.  Rows past the
-    // end are clamped to the last row; their products vanish because the activations at
-    // k >= K are zero, and columns past N are computed on column 0's bytes and never stored.
-    const uint32_t col_off = col_ok ? (uint32_t)ncol : 0u;
+    // by uniform strides.  Rows past the end are clamped to the last row; their products
+    // vanish because the activations at k >= K are zero.  Columns past N are computed on
+    // column 0's bytes and never stored.
     const uint32_t N32 = (uint32_t)p.N;
-    const uint32_t last_off = (uint32_t)(p.Kb - 1) * N32 + col_off;
-    const uint32_t step_stride = (uint32_t)(WAVES * RS) * N32;
-    uint32_t woff = (uint32_t)(wave * RS + g * KBG) * N32 + col_off;
-    int k0 = 4 * (wave * RS + g * KBG);
+    const uint32_t last_rowoff = (uint32_t)(p.Kb - 1) * N32;
+    uint32_t coloff[NCO];
+    if constexpr (QUAD) {
+#pragma unroll
+        for (int cb = 0; cb < NCO; cb++) {
+            const int64_t c = nb + 16 * cb + (j & ~3);
+            coloff[cb] = (c < p.N) ? (uint32_t)c : 0u;
+        }
+    } else {
+        const int64_t c = nb + (int64_t)NACC * j;
+        coloff[0] = (c < p.N) ? (uint32_t)c : 0u;
+    }
+    uint32_t rowoff = (uint32_t)(s_begin * 16 + 4 * g + (QUAD ? q : 0)) * N32;
+    int k0 = s_begin * 64 + 16 * g;  // first k of this lane's fragment in step s_begin
     const uint32_t xrow = (uint32_t)min(j, p.M - 1) * (uint32_t)p.K;
+    const uint32_t sel_q = 0x0C0C0000u | ((uint32_t)(4 + q) << 8) | (uint32_t)q;
 
     // epilogue operands of this thread's output column, requested before the weight stream
     // so that their latency hides behind it (raw bits now, conversion after the reduction)
@@ -166,88 +203,154 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
         }
     }
 
-    acc_t acc[NW];
+    // XLDS (M == 1): the wave's K-slice of x, [s_begin*64, (s_begin+spw)*64), as 16-byte
+    // chunks, chunk c = lane + 64u; zero beyond K
+    uint8_t* xs = (uint8_t*)(red + WAVES * p.M * TILE_N) + (size_t)wave * (XC_MAX * 64 * 16);
+    uint4 xr[XLDS ? XC_MAX : 1];
+    const int nchunks = spw * 64 * ES / 16;
+    if constexpr (XLDS) {
+        constexpr int EPC = 16 / ES;
 #pragma unroll
-    for (int t = 0; t < NW; t++) acc[t] = acc_t{0, 0, 0, 0};
+        for (int u = 0; u < XC_MAX; u++) {
+            if (u * 64 < nchunks) {  // uniform
+                const int k = s_begin * 64 + (lane + 64 * u) * EPC;
+                xr[u] = *(const uint4*)((const uint8_t*)p.X + (uint32_t)min(k, (int)p.K - EPC) * ES);
+            }
+        }
+    }
 
-    for (int base = wave; base < nsteps; base += WAVES * PF, woff += PF * step_stride, k0 += 4 * WAVES * RS * PF) {
-        uint32_t raw[PF][KBG][ND];
-        uint4 xa[PF];
+    acc_t acc[NACC], acc2[NACC2];
+#pragma unroll
+    for (int t = 0; t < NACC; t++) acc[t] = acc_t{0, 0, 0, 0};
+#pragma unroll
+    for (int t = 0; t < NACC2; t++) acc2[t] = acc_t{0, 0, 0, 0};
+
+    for (int base = s_begin; base < s_end; base += PF, rowoff += PF * 16 * N32, k0 += PF * 64) {
+        uint32_t raw[PF][RAWN];
+        uint4 xa[PF][XN];
 #pragma unroll
         for (int f = 0; f < PF; f++) {
+            const uint32_t ro = rowoff + (uint32_t)(f * 16) * N32;
+            if constexpr (BYTE) {
 #pragma unroll
-            for (int r = 0; r < KBG; r++)
-                load_raw<NW>(p.W_T, min(woff + (uint32_t)f * step_stride + (uint32_t)r * N32, last_off), raw[f][r]);
+                for (int r = 0; r < 4; r++)
+                    raw[f][r] = (uint32_t)p.W_T[min(ro + (uint32_t)r * N32, last_rowoff) + coloff[0]];
+            } else if constexpr (QUAD) {
+                const uint32_t rc = min(ro, last_rowoff);
+#pragma unroll
+                for (int cb = 0; cb < NCO; cb++) raw[f][cb] = *(const uint32_t*)(p.W_T + (rc + coloff[cb]));
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const typename RawVec<LD>::type v = *(const typename RawVec<LD>::type*)(
+                        p.W_T + (min(ro + (uint32_t)r * N32, last_rowoff) + coloff[0]));
+                    __builtin_memcpy(&raw[f][r * ND], &v, LD);
+                }
+            }
         }
-        if (p.x_vec_ok) {
+        if constexpr (!XLDS) {
+            if (p.x_vec_ok) {
 #pragma unroll
-            for (int f = 0; f < PF; f++) xa[f] = load_x_frag<MODE, true>(p, xrow, j, k0 + f * 4 * WAVES * RS);
+                for (int f = 0; f < PF; f++)
+#pragma unroll
+                    for (int h = 0; h < XN; h++) xa[f][h] = load_x16<MODE, true>(p, xrow, j, k0 + f * 64 + 8 * h);
+            } else {
+#pragma unroll
+                for (int f = 0; f < PF; f++)
+#pragma unroll
+                    for (int h = 0; h < XN; h++) xa[f][h] = load_x16<MODE, false>(p, xrow, j, k0 + f * 64 + 8 * h);
+            }
         } else {
+            if (base == s_begin) {  // uniform: park the x slice in LDS once its loads have landed
+                constexpr int EPC = 16 / ES;
 #pragma unroll
-            for (int f = 0; f < PF; f++) xa[f] = load_x_frag<MODE, false>(p, xrow, j, k0 + f * 4 * WAVES * RS);
+                for (int u = 0; u < XC_MAX; u++) {
+                    if (u * 64 < nchunks) {
+                        const int k = s_begin * 64 + (lane + 64 * u) * EPC;
+                        *(uint4*)(xs + (lane + 64 * u) * 16) = zero_unless(xr[u], k < (int)p.K);
+                    }
+                }
+            }
         }
 #pragma unroll
         for (int f = 0; f < PF; f++) {
-            if (base + f * WAVES >= nsteps) break;  // uniform per wave
-            {
-                const bool k_ok = k0 + f * 4 * WAVES * RS < (int)p.K;  // no-op for the gathered path
-                xa[f].x = k_ok ? xa[f].x : 0u; xa[f].y = k_ok ? xa[f].y : 0u;
-                xa[f].z = k_ok ? xa[f].z : 0u; xa[f].w = k_ok ? xa[f].w : 0u;
+            if (base + f >= s_end) break;  // uniform per wave
+            if constexpr (XLDS) {
+                // LDS accesses of one wave execute in order: the slice written above is visible
+                const uint8_t* src = xs + ((base + f - s_begin) * 64 + 16 * g) * ES;
+#pragma unroll
+                for (int h = 0; h < XN; h++) xa[f][h] = *(const uint4*)(src + 16 * h);
+            } else {
+#pragma unroll
+                for (int h = 0; h < XN; h++)  // no-op for the gathered path
+                    xa[f][h] = zero_unless(xa[f][h], k0 + f * 64 + 8 * h < (int)p.K);
+            }
+            // G[t]: packed bytes of rows 4g..4g+3 of the column accumulator t serves
+            uint32_t G[NACC];
+            if constexpr (BYTE) {
+                G[0] = raw[f][0] | (raw[f][1] << 8) | (raw[f][2] << 16) | (raw[f][3] << 24);
+            } else if constexpr (QUAD) {
+#pragma unroll
+                for (int cb = 0; cb < NCO; cb++) G[cb] = quad_transpose(raw[f][cb], sel_q);
+            } else {
+#pragma unroll
+                for (int d = 0; d < ND; d++) {
+                    uint32_t Gd[4];
+                    transpose4x4_bytes(raw[f][0 * ND + d], raw[f][1 * ND + d], raw[f][2 * ND + d], raw[f][3 * ND + d], Gd);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) G[4 * d + i] = Gd[i];
+                }
             }
             if constexpr (MODE == MODE_I8) {
                 uint32_t ta[4];
-                transpose4x4_bytes(xa[f].x, xa[f].y, xa[f].z, xa[f].w, ta);
+                transpose4x4_bytes(xa[f][0].x, xa[f][0].y, xa[f][0].z, xa[f][0].w, ta);
                 const v4i a = {(int)ta[0], (int)ta[1], (int)ta[2], (int)ta[3]};
 #pragma unroll
-                for (int d = 0; d < ND; d++) {
-                    uint32_t G[4];
-                    if constexpr (NW == 1) {
-                        // one byte per row: G = {row0, row1, row2, row3}
-                        G[0] = raw[f][0][0] | (raw[f][1][0] << 8) | (raw[f][2][0] << 16) | (raw[f][3][0] << 24);
-                    } else {
-                        transpose4x4_bytes(raw[f][0][d], raw[f][1][d], raw[f][2][d], raw[f][3][d], G);
-                    }
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        if (4 * d + i < NW) {
-                            const v4i b = decode16_i8(G[i]);
-                            acc[4 * d + i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[4 * d + i], 0, 0, 0);
-                        }
-                    }
+                for (int t = 0; t < NACC; t++) {
+                    const v4i b = decode16_i8(G[t]);
+                    if (TWO && (f & 1))
+                        acc2[TWO ? t : 0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc2[TWO ? t : 0], 0, 0, 0);
+                    else
+                        acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[t], 0, 0, 0);
                 }
             } else {
                 // natural halves h0..h7 -> dword c = { h[c], h[4+c] } (the decode's k order)
-                const u32x4 au = {perm(xa[f].z, xa[f].x, 0x05040100u), perm(xa[f].z, xa[f].x, 0x07060302u),
-                                  perm(xa[f].w, xa[f].y, 0x05040100u), perm(xa[f].w, xa[f].y, 0x07060302u)};
+                u32x4 au[2];
 #pragma unroll
-                for (int d = 0; d < ND; d++) {
+                for (int h = 0; h < 2; h++)
+                    au[h] = u32x4{perm(xa[f][h].z, xa[f][h].x, 0x05040100u), perm(xa[f][h].z, xa[f][h].x, 0x07060302u),
+                                  perm(xa[f][h].w, xa[f][h].y, 0x05040100u), perm(xa[f][h].w, xa[f][h].y, 0x07060302u)};
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        if (4 * d + i < NW) {
-                            // bytes: [zero, row0.byte i, zero, row1.byte i]
-                            const uint32_t sel = ((uint32_t)(4 + i) << 24) | (0x0Cu << 16) | ((uint32_t)i << 8) | 0x0Cu;
-                            const uint32_t M2 = perm(raw[f][1][d], raw[f][0][d], sel);
-                            if constexpr (MODE == MODE_F16) {
-                                const u32x4 bu = decode8_16bit<LUT_F16_ONE>(M2);
-                                acc[4 * d + i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                    __builtin_bit_cast(v8h, au), __builtin_bit_cast(v8h, bu), acc[4 * d + i], 0, 0, 0);
-                            } else {
-                                const u32x4 bu = decode8_16bit<LUT_BF16_TWO>(M2);
-                                acc[4 * d + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                                    __builtin_bit_cast(v8bf, au), __builtin_bit_cast(v8bf, bu), acc[4 * d + i], 0, 0, 0);
-                            }
+                for (int t = 0; t < NACC; t++) {
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        // bytes [zero, row 2h, zero, row 2h+1] of G
+                        const uint32_t M2 = perm(0u, G[t], h == 0 ? 0x010C000Cu : 0x030C020Cu);
+                        acc_t& dst = (TWO && h == 1) ? acc2[TWO ? t : 0] : acc[t];
+                        if constexpr (MODE == MODE_F16) {
+                            const u32x4 bu = decode8_16bit<LUT_F16_ONE>(M2);
+                            dst = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, au[h]),
+                                                                         __builtin_bit_cast(v8h, bu), dst, 0, 0, 0);
+                        } else {
+                            const u32x4 bu = decode8_16bit<LUT_BF16_TWO>(M2);
+                            dst = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, au[h]),
+                                                                          __builtin_bit_cast(v8bf, bu), dst, 0, 0, 0);
                         }
                     }
                 }
             }
         }
     }
+    if constexpr (TWO) {
+#pragma unroll
+        for (int t = 0; t < NACC; t++) acc[t] += acc2[t];
+    }
 
     // ---- sum the waves' accumulators through LDS, in wave order ------------------------
-    // red[w][row][t*16 + j]; lane (j, g) holds rows 4g..4g+3 of column slot t*16+j
+    // red[w][row][slot]; lane (j, g) holds rows 4g..4g+3 of slot t*16 + j
     const int M = p.M;
 #pragma unroll
-    for (int t = 0; t < NW; t++) {
+    for (int t = 0; t < NACC; t++) {
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const int row = 4 * g + r;
@@ -263,7 +366,8 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
         const int row = idx / TILE_N;
         const int nl = idx % TILE_N;
         if (nb + nl >= p.N) continue;
-        const int slot = (nl % NW) * 16 + nl / NW;
+        // column nl of the tile sits in slot t*16 + j: LD_V*: nl = NACC*j + t; else nl = 16*t + j
+        const int slot = (LD >= 4) ? (nl % NACC) * 16 + nl / NACC : nl;
         uint32_t bits = red[row * TILE_N + slot];
 #pragma unroll
         for (int w = 1; w < WAVES; w++) bits = add_bits<MODE>(bits, red[(w * M + row) * TILE_N + slot]);
@@ -282,8 +386,8 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
 // ---- host side --------------------------------------------------------------------
 
 struct StreamPlan {
-    int nw;     // bytes per lane and row: 16, 8, 4, 2 or 1 (tile = 16*nw columns)
-    int waves;  // waves per workgroup
+    int ld;     // LD_* tile shape (tile = 16 columns for LD_BYTE, else 16*ld)
+    int waves;  // waves per workgroup: 4, 8 or 16
 };
 
 // the kernel addresses W_T and X with 32-bit offsets from their base pointers
@@ -292,70 +396,84 @@ bool stream_supported(int64_t N, int64_t K, const void* W_T) {
     return ((uintptr_t)W_T) % 16 == 0 && N >= 1 && (ceil_div(K, 4) + 8192) * N < (1ll << 32) && K < (1ll << 26);
 }
 
+static int ld_columns(int ld) { return ld == LD_BYTE ? 16 : 16 * ld; }
+
 StreamPlan stream_plan(int mode, int64_t M, int64_t N, int64_t Kb) {
     StreamPlan pl;
     (void)mode;
-    // optional override for tuning runs: BITTORCH_STREAM_CFG="nw,waves"
-    int o_nw = 0, o_waves = 0;
-    if (const char* env = getenv("BITTORCH_STREAM_CFG")) sscanf(env, "%d,%d", &o_nw, &o_waves);
-    // widest lane load the row pitch allows (row starts must stay aligned to it)
-    int nw = (N % 16 == 0) ? 16 : (N % 8 == 0) ? 8 : (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
-    if ((o_nw == 16 || o_nw == 8 || o_nw == 4 || o_nw == 2 || o_nw == 1) && N % o_nw == 0) {
-        nw = o_nw;
+    (void)Kb;
+    // optional override for tuning runs: BITTORCH_STREAM_CFG="ld,waves"
+    int o_ld = -1, o_waves = 0;
+    if (const char* env = getenv("BITTORCH_STREAM_CFG")) sscanf(env, "%d,%d", &o_ld, &o_waves);
+    int ld;
+    if (N % 4 != 0) {
+        ld = LD_BYTE;  // row starts are not dword aligned
+    } else if ((o_ld == 16 || o_ld == 8 || o_ld == 4 || o_ld == 2 || o_ld == 1) && (o_ld < 4 || N % o_ld == 0)) {
+        ld = o_ld;
     } else {
-        // narrow the tile until there is at least one tile per CU
-        while (nw > 1 && ceil_div(N, 16 * (int64_t)nw) < 256) nw >>= 1;
-        // decode batches re-read the activations once per tile: keep tiles wider when
-        // that traffic would exceed the weights' own
-        (void)M;
+        // widest lane load the row pitch allows, narrowed until there are enough tiles to
+        // occupy the chip (measured: 172 tiles of 64 columns beat 344 of 32 for a 16-row
+        // batch, which re-reads its activations once per tile; a single row prefers >= 256)
+        ld = (N % 16 == 0) ? 16 : (N % 8 == 0) ? 8 : 4;
+        const int min_tiles = (M > 4) ? 160 : 256;
+        while (ld > 1 && ceil_div(N, ld_columns(ld)) < min_tiles) ld >>= 1;
     }
-    pl.nw = nw;
-    const int max_waves = 1024 / (16 * nw) < 16 ? 1024 / (16 * nw) : 16;  // LDS: WAVES*TILE_N <= 1024 words/row
-    const int64_t steps = ceil_div(Kb, mode == MODE_I8 ? 16 : 8);
-    int waves = (o_waves == 1 || o_waves == 2 || o_waves == 4 || o_waves == 8 || o_waves == 16) ? o_waves : 8;
+    pl.ld = ld;
+    const int max_waves = (ld == 16) ? 4 : (ld == 8 || ld == LD_BYTE) ? 8 : 16;  // LDS: WAVES*TILE_N <= 1024 words per row
+    int waves = (o_waves == 4 || o_waves == 8 || o_waves == 16) ? o_waves : 8;
     if (waves > max_waves) waves = max_waves;
-    while (waves > 1 && waves > steps) waves >>= 1;
     pl.waves = waves;
     return pl;
 }
 
 size_t stream_workspace_bytes(int, int64_t, int64_t, int64_t) { return 0; }
 
-template <int MODE, int NW, int WAVES>
-static void launch_stream_k(const StreamParams& p, dim3 grid, size_t lds, hipStream_t st) {
-    constexpr int PF = (NW >= 16) ? 2 : (NW == 8) ? 4 : 8;
-    hipLaunchKernelGGL((stream_kernel<MODE, NW, WAVES, PF>), grid, dim3(WAVES * 64), lds, st, p);
+template <int MODE, int LD, int WAVES>
+static void launch_stream_k(const StreamParams& p, bool xlds, dim3 grid, size_t lds, hipStream_t st) {
+    constexpr int PF = (LD == 16) ? 2 : (LD == 8) ? 4 : (LD == 4 && MODE != MODE_I8) ? 4 : 8;
+    if constexpr (LD <= 4) {  // decode-shape tiles: the M = 1 variant with x staged in LDS
+        if (xlds) {
+            hipLaunchKernelGGL((stream_kernel<MODE, LD, WAVES, PF, true>), grid, dim3(WAVES * 64), lds, st, p);
+            return;
+        }
+    }
+    hipLaunchKernelGGL((stream_kernel<MODE, LD, WAVES, PF, false>), grid, dim3(WAVES * 64), lds, st, p);
 }
 
-template <int MODE, int NW>
-static void launch_stream_w(const StreamParams& p, int waves, dim3 grid, size_t lds, hipStream_t st) {
-    if constexpr (NW <= 4) {
-        if (waves == 16) { launch_stream_k<MODE, NW, 16>(p, grid, lds, st); return; }
+template <int MODE, int LD>
+static void launch_stream_w(const StreamParams& p, int waves, bool xlds, dim3 grid, size_t lds, hipStream_t st) {
+    if constexpr (LD <= 4) {
+        if (waves == 16) { launch_stream_k<MODE, LD, 16>(p, xlds, grid, lds, st); return; }
     }
-    if constexpr (NW <= 8) {
-        if (waves == 8) { launch_stream_k<MODE, NW, 8>(p, grid, lds, st); return; }
+    if constexpr (LD <= 8) {
+        if (waves == 8) { launch_stream_k<MODE, LD, 8>(p, xlds, grid, lds, st); return; }
     }
-    if (waves >= 4) { launch_stream_k<MODE, NW, 4>(p, grid, lds, st); return; }
-    if (waves == 2) { launch_stream_k<MODE, NW, 2>(p, grid, lds, st); return; }
-    launch_stream_k<MODE, NW, 1>(p, grid, lds, st);
+    launch_stream_k<MODE, LD, 4>(p, xlds, grid, lds, st);
 }
 
 template <int MODE>
 static int launch_stream_mode(StreamParams p, const StreamPlan& pl, hipStream_t st) {
-    const int64_t tile_n = 16 * (int64_t)pl.nw;
+    const int64_t tile_n = ld_columns(pl.ld);
     p.tiles = (int)ceil_div(p.N, tile_n);
     p.per_xcd = (int)ceil_div(p.tiles, 8);
     const dim3 grid((unsigned)(p.per_xcd * 8));
-    int waves = pl.waves;
-    if (pl.nw == 16 && waves > 4) waves = 4;
-    if (pl.nw == 8 && waves > 8) waves = 8;
-    const size_t lds = (size_t)waves * p.M * tile_n * 4;
-    switch (pl.nw) {
-        case 16: launch_stream_w<MODE, 16>(p, waves, grid, lds, st); break;
-        case 8: launch_stream_w<MODE, 8>(p, waves, grid, lds, st); break;
-        case 4: launch_stream_w<MODE, 4>(p, waves, grid, lds, st); break;
-        case 2: launch_stream_w<MODE, 2>(p, waves, grid, lds, st); break;
-        default: launch_stream_w<MODE, 1>(p, waves, grid, lds, st); break;
+    const int waves = pl.waves;
+    // x slice in LDS: one row, aligned, at most XC_MAX 16-byte chunks per lane and wave, and
+    // within the default 64 KiB of dynamic LDS
+    const int es = (MODE == MODE_I8) ? 1 : 2;
+    const int64_t spw = ceil_div(ceil_div(p.Kb, 16), waves);
+    const size_t red_bytes = (size_t)waves * p.M * tile_n * 4;
+    const size_t xs_bytes = (size_t)waves * XC_MAX * 64 * 16;
+    const bool xlds = p.M == 1 && p.x_vec_ok && pl.ld <= 4 && spw * 64 * es <= XC_MAX * 64 * 16 &&
+                      p.K >= 16 / es && red_bytes + xs_bytes <= 64 * 1024 && !getenv("BITTORCH_STREAM_NOXLDS");
+    const size_t lds = red_bytes + (xlds ? xs_bytes : 0);
+    switch (pl.ld) {
+        case 16: launch_stream_w<MODE, 16>(p, waves, xlds, grid, lds, st); break;
+        case 8: launch_stream_w<MODE, 8>(p, waves, xlds, grid, lds, st); break;
+        case 4: launch_stream_w<MODE, 4>(p, waves, xlds, grid, lds, st); break;
+        case 2: launch_stream_w<MODE, 2>(p, waves, xlds, grid, lds, st); break;
+        case 1: launch_stream_w<MODE, 1>(p, waves, xlds, grid, lds, st); break;
+        default: launch_stream_w<MODE, 0>(p, waves, xlds, grid, lds, st); break;
     }
     return check_launch("stream_gemm");
 }
