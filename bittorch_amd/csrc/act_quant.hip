@@ -1,0 +1,168 @@
+// Per-row int8 activation quantization for gfx950 (HBM-bound).
+//
+// Arithmetic restated from the reference (csrc/kernels/ternary_gemm_tensor_core.cu:343-347,
+// :439, :456-457) with the row scale taken over the whole row:
+//   amax = max_k |x[b,k]|;  s_x[b] = amax > 1e-6 ? amax / 127 : 1
+//   q[b,k] = (int8) clamp(roundf(x[b,k] * (1 / s_x[b])), -127, 127)
+#include <cstdlib>
+
+#include "bt_common.h"
+
+namespace bt {
+
+// Per-row int8 activation quantizer: one wave per row, two passes over the row
+// (the second pass hits in cache; a row is at most a few tens of KiB).
+template <int DT>
+__global__ __launch_bounds__(256) void act_quant_kernel(const void* __restrict__ X, int64_t B, int64_t K,
+                                                        int8_t* __restrict__ Q, float* __restrict__ s_x) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= B) return;
+    const int64_t base = row * K;
+    constexpr int ES = (DT == BT_F32) ? 4 : 2;
+    const bool vec_ok = (K % 8 == 0) && (((uintptr_t)X) % 16 == 0) && (((uintptr_t)Q) % 8 == 0);
+
+    auto load8 = [&](int64_t k, float (&v)[8]) {
+        if (vec_ok) {
+            if constexpr (DT == BT_F32) {
+                const float4 a = *(const float4*)((const float*)X + base + k);
+                const float4 b = *(const float4*)((const float*)X + base + k + 4);
+                v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+                v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+            } else {
+                const uint4 u = *(const uint4*)((const uint16_t*)X + base + k);
+                const uint32_t d[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const uint16_t h = (uint16_t)(d[e >> 1] >> (16 * (e & 1)));
+                    v[e] = (DT == BT_F16) ? f16_bits_to_f32(h) : bf16_bits_to_f32(h);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[e] = (k + e < K) ? load_elem<DT>(X, base + k + e) : 0.0f;
+        }
+    };
+    (void)ES;
+
+    float amax = 0.0f;
+    for (int64_t k = (int64_t)lane * 8; k < K; k += 512) {
+        float v[8];
+        load8(k, v);
+#pragma unroll
+        for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(v[e]));
+    }
+    amax = wave_max(amax);
+    const float s = (amax > 1e-6f) ? __fdiv_rn(amax, 127.0f) : 1.0f;
+    const float inv = __fdiv_rn(1.0f, s);
+    if (lane == 0) s_x[row] = s;
+
+    for (int64_t k = (int64_t)lane * 8; k < K; k += 512) {
+        float v[8];
+        load8(k, v);
+        uint32_t lo = 0, hi = 0;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            float r = roundf(__fmul_rn(v[e], inv));
+            r = fmaxf(-127.0f, fminf(127.0f, r));
+            const uint32_t byte = (uint32_t)(uint8_t)(int8_t)(int)r;
+            if (e < 4) lo |= byte << (8 * e);
+            else hi |= byte << (8 * (e - 4));
+        }
+        if (vec_ok) {
+            *(uint2*)(Q + base + k) = make_uint2(lo, hi);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+                if (k + e < K) Q[base + k + e] = (int8_t)(((e < 4 ? lo : hi) >> (8 * (e & 3))) & 0xff);
+        }
+    }
+}
+
+// One workgroup per row, the row held in registers between the absmax pass and the
+// quantization: X is read once and the row's latency chain is load -> reduce -> store.
+// Needs K % 8 == 0, K <= 2048*ITERS and aligned pointers (16 bytes X, 8 bytes Q).
+template <int DT, int ITERS>
+__global__ __launch_bounds__(256) void act_quant_row_kernel(const void* __restrict__ X, int K,
+                                                            int8_t* __restrict__ Q, float* __restrict__ s_x) {
+    __shared__ float part[4];
+    const int tid = threadIdx.x;
+    const int64_t base = (int64_t)blockIdx.x * K;
+    float v[ITERS][8];
+#pragma unroll
+    for (int i = 0; i < ITERS; i++) {
+        const int k = (i * 256 + tid) * 8;
+        const int kc = min(k, K - 8);  // clamped, unconditional loads; zeroed below
+        if constexpr (DT == BT_F32) {
+            const float4 a = *(const float4*)((const float*)X + base + kc);
+            const float4 b = *(const float4*)((const float*)X + base + kc + 4);
+            v[i][0] = a.x; v[i][1] = a.y; v[i][2] = a.z; v[i][3] = a.w;
+            v[i][4] = b.x; v[i][5] = b.y; v[i][6] = b.z; v[i][7] = b.w;
+        } else {
+            const uint4 u = *(const uint4*)((const uint16_t*)X + base + kc);
+            const uint32_t d[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const uint16_t h = (uint16_t)(d[e >> 1] >> (16 * (e & 1)));
+                v[i][e] = (DT == BT_F16) ? f16_bits_to_f32(h) : bf16_bits_to_f32(h);
+            }
+        }
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < ITERS; i++) {
+        const bool ok = (i * 256 + tid) * 8 < K;
+#pragma unroll
+        for (int e = 0; e < 8; e++) amax = fmaxf(amax, ok ? fabsf(v[i][e]) : 0.0f);
+    }
+    amax = wave_max(amax);
+    if ((tid & 63) == 0) part[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
+    const float s = (amax > 1e-6f) ? __fdiv_rn(amax, 127.0f) : 1.0f;
+    const float inv = __fdiv_rn(1.0f, s);
+    if (tid == 0) s_x[blockIdx.x] = s;
+#pragma unroll
+    for (int i = 0; i < ITERS; i++) {
+        const int k = (i * 256 + tid) * 8;
+        uint32_t lo = 0, hi = 0;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            float r = roundf(__fmul_rn(v[i][e], inv));
+            r = fmaxf(-127.0f, fminf(127.0f, r));
+            const uint32_t byte = (uint32_t)(uint8_t)(int8_t)(int)r;
+            if (e < 4) lo |= byte << (8 * e);
+            else hi |= byte << (8 * (e - 4));
+        }
+        if (k < K) *(uint2*)(Q + base + k) = make_uint2(lo, hi);
+    }
+}
+
+template <int DT>
+static bool launch_act_quant_rows(const void* X, int64_t B, int64_t K, int8_t* Q, float* s_x, hipStream_t st) {
+    if (K % 8 != 0 || K > 16384 || ((uintptr_t)X) % 16 != 0 || ((uintptr_t)Q) % 8 != 0 || B > 0x7fffffff ||
+        getenv("BITTORCH_ACTQ_GENERIC"))
+        return false;
+    const dim3 grid((unsigned)B), block(256);
+    const int k = (int)K;
+    if (K <= 2048) hipLaunchKernelGGL((act_quant_row_kernel<DT, 1>), grid, block, 0, st, X, k, Q, s_x);
+    else if (K <= 4096) hipLaunchKernelGGL((act_quant_row_kernel<DT, 2>), grid, block, 0, st, X, k, Q, s_x);
+    else if (K <= 8192) hipLaunchKernelGGL((act_quant_row_kernel<DT, 4>), grid, block, 0, st, X, k, Q, s_x);
+    else if (K <= 12288) hipLaunchKernelGGL((act_quant_row_kernel<DT, 6>), grid, block, 0, st, X, k, Q, s_x);
+    else hipLaunchKernelGGL((act_quant_row_kernel<DT, 8>), grid, block, 0, st, X, k, Q, s_x);
+    return true;
+}
+
+int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x, hipStream_t st) {
+    const bool done = (x_dtype == BT_F32)   ? launch_act_quant_rows<BT_F32>(X, B, K, Q, s_x, st)
+                      : (x_dtype == BT_F16) ? launch_act_quant_rows<BT_F16>(X, B, K, Q, s_x, st)
+                                            : launch_act_quant_rows<BT_BF16>(X, B, K, Q, s_x, st);
+    if (done) return check_launch("bt_act_quant_i8");
+    const dim3 grid((unsigned)ceil_div(B, 4)), block(256);
+    if (x_dtype == BT_F32) hipLaunchKernelGGL(act_quant_kernel<BT_F32>, grid, block, 0, st, X, B, K, Q, s_x);
+    else if (x_dtype == BT_F16) hipLaunchKernelGGL(act_quant_kernel<BT_F16>, grid, block, 0, st, X, B, K, Q, s_x);
+    else hipLaunchKernelGGL(act_quant_kernel<BT_BF16>, grid, block, 0, st, X, B, K, Q, s_x);
+    return check_launch("bt_act_quant_i8");
+}
+
+}  // namespace bt

@@ -20,6 +20,8 @@
 //     output columns nb + 64w + 4j .. +3) from each of the four rows
 //     kb + 4g .. 4g+3, transposes the 4x4 bytes and decodes them in registers
 //     into the B operands of four MFMAs (one per column).
+#include <cstdlib>
+
 #include "bt_common.h"
 
 namespace bt {
@@ -292,83 +294,6 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     if (!col_ok) return;
     if (kgrp == 0) gemm_epilogue_dt<0>(p, acc, m0, g, ncol);  // wave-uniform branch
     else gemm_epilogue_dt<4>(p, acc, m0, g, ncol);
-}
-
-// Per-row int8 activation quantizer: one wave per row, two passes over the row
-// (the second pass hits in cache; a row is at most a few tens of KiB).
-template <int DT>
-__global__ __launch_bounds__(256) void act_quant_kernel(const void* __restrict__ X, int64_t B, int64_t K,
-                                                        int8_t* __restrict__ Q, float* __restrict__ s_x) {
-    const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= B) return;
-    const int64_t base = row * K;
-    constexpr int ES = (DT == BT_F32) ? 4 : 2;
-    const bool vec_ok = (K % 8 == 0) && (((uintptr_t)X) % 16 == 0) && (((uintptr_t)Q) % 8 == 0);
-
-    auto load8 = [&](int64_t k, float (&v)[8]) {
-        if (vec_ok) {
-            if constexpr (DT == BT_F32) {
-                const float4 a = *(const float4*)((const float*)X + base + k);
-                const float4 b = *(const float4*)((const float*)X + base + k + 4);
-                v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
-                v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-            } else {
-                const uint4 u = *(const uint4*)((const uint16_t*)X + base + k);
-                const uint32_t d[4] = {u.x, u.y, u.z, u.w};
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const uint16_t h = (uint16_t)(d[e >> 1] >> (16 * (e & 1)));
-                    v[e] = (DT == BT_F16) ? f16_bits_to_f32(h) : bf16_bits_to_f32(h);
-                }
-            }
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; e++) v[e] = (k + e < K) ? load_elem<DT>(X, base + k + e) : 0.0f;
-        }
-    };
-    (void)ES;
-
-    float amax = 0.0f;
-    for (int64_t k = (int64_t)lane * 8; k < K; k += 512) {
-        float v[8];
-        load8(k, v);
-#pragma unroll
-        for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(v[e]));
-    }
-    amax = wave_max(amax);
-    const float s = (amax > 1e-6f) ? __fdiv_rn(amax, 127.0f) : 1.0f;
-    const float inv = __fdiv_rn(1.0f, s);
-    if (lane == 0) s_x[row] = s;
-
-    for (int64_t k = (int64_t)lane * 8; k < K; k += 512) {
-        float v[8];
-        load8(k, v);
-        uint32_t lo = 0, hi = 0;
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            float r = roundf(__fmul_rn(v[e], inv));
-            r = fmaxf(-127.0f, fminf(127.0f, r));
-            const uint32_t byte = (uint32_t)(uint8_t)(int8_t)(int)r;
-            if (e < 4) lo |= byte << (8 * e);
-            else hi |= byte << (8 * (e - 4));
-        }
-        if (vec_ok) {
-            *(uint2*)(Q + base + k) = make_uint2(lo, hi);
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; e++)
-                if (k + e < K) Q[base + k + e] = (int8_t)(((e < 4 ? lo : hi) >> (8 * (e & 3))) & 0xff);
-        }
-    }
-}
-
-int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x, hipStream_t st) {
-    const dim3 grid((unsigned)ceil_div(B, 4)), block(256);
-    if (x_dtype == BT_F32) hipLaunchKernelGGL(act_quant_kernel<BT_F32>, grid, block, 0, st, X, B, K, Q, s_x);
-    else if (x_dtype == BT_F16) hipLaunchKernelGGL(act_quant_kernel<BT_F16>, grid, block, 0, st, X, B, K, Q, s_x);
-    else hipLaunchKernelGGL(act_quant_kernel<BT_BF16>, grid, block, 0, st, X, B, K, Q, s_x);
-    return check_launch("bt_act_quant_i8");
 }
 
 // the tiled kernel reads Q with 16-byte loads and W_T / Y with 4-column vectors
