@@ -237,6 +237,24 @@ def main():
                 "tops_with_act_quant": round(ops / (ev_full / steps * 1e-3) / 1e12, 1),
             }
             del ws, xa, q, s
+        # what the matrix cores sustain on register operands only (no memory in the loop)
+        probe_ops = _C.probe_mfma_int8(dev)  # warm
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(5):
+            probe_ops = _C.probe_mfma_int8(dev)
+        e1.record()
+        torch.cuda.synchronize()
+        probe_tops = probe_ops * 5 / (e0.elapsed_time(e1) * 1e-3) / 1e12
+        extra["mfma_i8_register_only_probe"] = {
+            "tops": round(probe_tops, 1), "frac_of_int8_peak": round(probe_tops / INT8_PEAK_TOPS, 4),
+            "note": "2048 workgroups x 8 waves of back-to-back v_mfma_i32_16x16x64_i8, 8 accumulators per wave",
+        }
+        for key in list(extra):
+            if key.startswith("prefill_int8"):
+                extra[key]["frac_of_probe"] = round(extra[key]["tops"] / probe_tops, 4)
         # config 3: small-batch decode, int8 activations
         for (m, n, k) in ((16, 11008, 4096), (16, 4096, 11008)):
             cnt = max(2, int(400e6 // (n * k // 4)))

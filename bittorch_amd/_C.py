@@ -309,3 +309,15 @@ def unpack_dequant(W_T: Tensor, in_features: int, scale: Optional[Tensor] = None
                                      0 if scale_f is None else scale_f.numel(), out.data_ptr(), odt,
                                      N, in_features, _stream(W_T)))
     return out
+
+
+def probe_mfma_int8(device, blocks: int = 2048, iters: int = 4096, random_operands: bool = False):
+    """Launches the int8 matrix-core rate probe on the current stream; returns the number
+    of integer operations the launch performs (time it from outside)."""
+    import ctypes
+
+    out = torch.zeros(1, dtype=torch.int32, device=device)
+    ops = ctypes.c_double(0.0)
+    with torch.cuda.device(device):
+        _status(_L.bt_probe_mfma_i8(blocks, iters, int(random_operands), out.data_ptr(), ctypes.addressof(ops), _stream(out)))
+    return ops.value

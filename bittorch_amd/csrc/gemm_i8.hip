@@ -8,18 +8,20 @@
 // (the MFMA runs on +-1 weights; the accumulators are multiplied by 127 exactly
 // in the epilogue, which is the same integer).
 //
-// Tiling: a 256-thread workgroup owns a 128 x 256 output tile.  Its four waves
-// split the 256 columns (64 each) and all walk the same 128 rows, so every
-// weight is decoded exactly once per workgroup and the decode cost (about 0.7
-// VALU operations per weight) is shared by 128 rows of MFMA work.
+// Tiling: a 512-thread workgroup (8 waves) owns a 128 x 256 output tile.  Wave w works on
+// columns 64*(w&3) .. +63 of the tile and on k64 sub-step (w>>2) of every 128-wide K stage,
+// walking all 128 rows, so every weight is decoded exactly once per workgroup and the decode
+// cost (about 0.7 VALU operations per weight) is shared by 128 rows of MFMA work; the two K
+// halves are added through LDS once after the main loop.
 //   * Activations (int8, row-major [M,K]) go through LDS, double buffered, 128 k
 //     per stage, stored in MFMA operand order: slot (sub, mb, lane) is the 16
 //     bytes lane (i = lane%16, g = lane/16) feeds to v_mfma_i32_16x16x64_i8 for
 //     row block mb and k64 sub-step sub.
-//   * Weights never touch LDS: lane (j, g) of wave w loads one dword (four
-//     output columns nb + 64w + 4j .. +3) from each of the four rows
-//     kb + 4g .. 4g+3, transposes the 4x4 bytes and decodes them in registers
-//     into the B operands of four MFMAs (one per column).
+//   * Weights never touch LDS: lane (j, g) loads one dword (four output columns
+//     nb + 64*(w&3) + 4j .. +3) from each of the four rows kb + 4g .. 4g+3, transposes
+//     the 4x4 bytes and decodes them in registers into the B operands of four MFMAs
+//     (one per column).
+//   * The stage is software-pipelined inside the wave (see the main loop).
 #include <cstdlib>
 
 #include "bt_common.h"
@@ -139,8 +141,11 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     // clamped rows / columns: rows past M and columns past N only feed outputs that
     // are never stored; the K tail is zeroed in the A operand of the last stage.
     // (The host guarantees K % 16 == 0, N % 4 == 0, aligned bases, 32-bit offsets.)
-    const int a_row = tid & (G_BM - 1);  // A staging role: one row, 32 of its 128 stage bytes
-    const int a_part = tid >> 7;         // bytes 32*a_part .. +31 -> sub-step a_part>>1, chunks 2*(a_part&1), +1
+    // A staging role: one row, 32 of its 128 stage bytes.  A wave stages one 16-row block:
+    // its 64 lanes touch 16 cache lines per load (four 32-byte parts of each row's line), and
+    // eight consecutive lanes write 128 contiguous bytes of LDS.
+    const int a_row = 16 * wave + (lane & 15);
+    const int a_part = lane >> 4;  // bytes 32*a_part .. +31 -> sub-step a_part>>1, chunks 2*(a_part&1), +1
     const int64_t rows_left = p.M - m0;
     const uint32_t a_row_c = (uint32_t)((a_row < rows_left) ? a_row : rows_left - 1);
     const uint32_t a_off = a_row_c * (uint32_t)p.K + 32u * a_part;
@@ -155,39 +160,48 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     uint4 a_set[2][2];
     uint32_t b_set[2][4];
 
-    auto load_full = [&](int64_t k0, uint4 (&a_reg)[2], uint32_t (&b_reg)[4]) {
-        const int8_t* ab = a_base + k0;
-        a_reg[0] = *(const uint4*)(ab + a_off);
-        a_reg[1] = *(const uint4*)(ab + 16 + a_off);
-        const uint8_t* bb = b_base + (k0 >> 2) * N;
+    // part: 1 = activations, 2 = weights, 3 = both
+    auto load_full = [&](int64_t k0, int part, uint4 (&a_reg)[2], uint32_t (&b_reg)[4]) {
+        if (part & 1) {
+            const int8_t* ab = a_base + k0;
+            a_reg[0] = *(const uint4*)(ab + a_off);
+            a_reg[1] = *(const uint4*)(ab + 16 + a_off);
+        }
+        if (part & 2) {
+            const uint8_t* bb = b_base + (k0 >> 2) * N;
 #pragma unroll
-        for (int r = 0; r < 4; r++) b_reg[r] = *(const uint32_t*)(bb + r * N + b_off);
+            for (int r = 0; r < 4; r++) b_reg[r] = *(const uint32_t*)(bb + r * N + b_off);
+        }
     };
-    auto load_tail = [&](int64_t k0, uint4 (&a_reg)[2], uint32_t (&b_reg)[4]) {
+    auto load_tail = [&](int64_t k0, int part, uint4 (&a_reg)[2], uint32_t (&b_reg)[4]) {
         // last, partial stage: k beyond K reads a clamped address and is zeroed in A
-        const int8_t* ab = a_base + k0;
+        if (part & 1) {
+            const int8_t* ab = a_base + k0;
 #pragma unroll
-        for (int c = 0; c < 2; c++) {
-            const bool in = (k0 + 32 * a_part + 16 * c) < p.K;
-            const uint4 v = *(const uint4*)(ab + (in ? 16 * c : 0) + (in ? a_off : a_row_c * (uint32_t)p.K));
-            const uint32_t m = in ? 0xFFFFFFFFu : 0u;
-            a_reg[c] = make_uint4(v.x & m, v.y & m, v.z & m, v.w & m);
+            for (int c = 0; c < 2; c++) {
+                const bool in = (k0 + 32 * a_part + 16 * c) < p.K;
+                const uint4 v = *(const uint4*)(ab + (in ? 16 * c : 0) + (in ? a_off : a_row_c * (uint32_t)p.K));
+                const uint32_t m = in ? 0xFFFFFFFFu : 0u;
+                a_reg[c] = make_uint4(v.x & m, v.y & m, v.z & m, v.w & m);
+            }
         }
+        if (part & 2) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            int64_t kb = (k0 >> 2) + 16 * kgrp + r + 4 * g;
-            kb = kb < p.Kb ? kb : p.Kb - 1;
-            b_reg[r] = *(const uint32_t*)(b_base + kb * N + (col_ok ? ncol : 0));
+            for (int r = 0; r < 4; r++) {
+                int64_t kb = (k0 >> 2) + 16 * kgrp + r + 4 * g;
+                kb = kb < p.Kb ? kb : p.Kb - 1;
+                b_reg[r] = *(const uint32_t*)(b_base + kb * N + (col_ok ? ncol : 0));
+            }
         }
     };
-    auto load_stage = [&](int st, uint4 (&a_reg)[2], uint32_t (&b_reg)[4]) {  // st uniform
+    auto load_stage = [&](int st, int part, uint4 (&a_reg)[2], uint32_t (&b_reg)[4]) {  // st, part uniform
         if constexpr (TAIL) {
             if (st >= nstages) st = nstages - 1;
-            if (st < nfull) load_full((int64_t)st * G_BK, a_reg, b_reg);
-            else load_tail((int64_t)st * G_BK, a_reg, b_reg);
+            if (st < nfull) load_full((int64_t)st * G_BK, part, a_reg, b_reg);
+            else load_tail((int64_t)st * G_BK, part, a_reg, b_reg);
         } else {
             // past the end: reload the last stage (never consumed) instead of branching
-            load_full((int64_t)(st < nstages ? st : nstages - 1) * G_BK, a_reg, b_reg);
+            load_full((int64_t)(st < nstages ? st : nstages - 1) * G_BK, part, a_reg, b_reg);
         }
     };
     auto store_a = [&](int buf, const uint4 (&a_reg)[2]) {
@@ -210,52 +224,126 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
         for (int t = 0; t < 4; t++) acc[mb][t] = v4i{0, 0, 0, 0};
 
     // ---- main loop --------------------------------------------------------------------
-    // Stage s is computed from LDS buffer s%2.  At the top of stage s every thread writes
-    // its piece of stage s+1 into the other buffer and re-uses those registers for the
-    // global loads of stage s+3, so a load has two full stages to arrive.  The barrier at
-    // the end of a stage both publishes the buffer just written and retires the reads of
-    // the current one.  Stages past the end are clamped (loaded, never consumed) instead
-    // of branched around; the loop handles two stages per trip so that the register sets
-    // are indexed statically.
-    uint32_t b_cur[4], b_nxt[4];
-    load_stage(0, a_set[0], b_set[0]);
-    load_stage(1, a_set[1], b_set[1]);
-    store_a(0, a_set[0]);
+    // Stage s is computed from LDS buffer s%2 and is software-pipelined inside the wave so
+    // that the matrix cores never wait for the stage's own operand preparation:
+    //   * on entry the wave already holds the decoded weights of stage s (b_dec) and the
+    //     activation fragments of row blocks 0..3 (a_lo);
+    //   * it writes its piece of stage s+1 into the other LDS buffer, re-uses those registers
+    //     for the global loads of stage s+3 (two full stages to arrive), requests row blocks
+    //     4..7 (a_hi), and issues the 16 MFMAs of row blocks 0..3 while the weights of stage
+    //     s+1 are being decoded in the shadow of those MFMAs;
+    //   * the one barrier of the stage publishes buffer (s+1)%2; row blocks 0..3 of stage
+    //     s+1 are requested right behind it and arrive under the 16 MFMAs of row blocks 4..7.
+    // Stages past the end are clamped (loaded, never consumed) instead of branched around;
+    // the loop handles two stages per trip so that the register sets are indexed statically.
+    v4i b_dec[2][4];
+    uint4 a_lo[4], a_hi[4];
+    const uint32_t a_lds_off = (uint32_t)(kgrp * (G_MB * 1024)) + ((uint32_t)lane << 4);
+    auto decode_b = [&](const uint32_t (&raw)[4], v4i (&out)[4]) {
+        uint32_t G[4];
+        transpose4x4_bytes(raw[0], raw[1], raw[2], raw[3], G);
 #pragma unroll
-    for (int r = 0; r < 4; r++) b_cur[r] = b_set[0][r];
-    load_stage(2, a_set[0], b_set[0]);
-    __syncthreads();
+        for (int t = 0; t < 4; t++) out[t] = decode16_i8(G[t]);
+    };
+    auto read_a = [&](int buf, int mb0, uint4 (&dst)[4]) {
+        const uint8_t* a_lds = lds + buf * G_STAGE_BYTES + a_lds_off;
+#pragma unroll
+        for (int i = 0; i < 4; i++) dst[i] = *(const uint4*)(a_lds + (mb0 + i) * 1024);
+    };
+    auto mfma_half = [&](int mb0, const uint4 (&av)[4], const v4i (&b)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const v4i a = {(int)av[i].x, (int)av[i].y, (int)av[i].z, (int)av[i].w};
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+                acc[mb0 + i][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[t], acc[mb0 + i][t], 0, 0, 0);
+        }
+    };
 
-    auto stage = [&](int s, uint4 (&a_reg)[2], uint32_t (&b_reg)[4]) {
+    load_stage(0, 3, a_set[0], b_set[0]);
+    load_stage(1, 3, a_set[1], b_set[1]);
+    store_a(0, a_set[0]);
+    decode_b(b_set[0], b_dec[0]);
+    load_stage(2, 3, a_set[0], b_set[0]);
+    __syncthreads();
+    read_a(0, 0, a_lo);
+
+    // decode of the next stage's weights cut into slices of at most five VALU operations,
+    // one slice issued behind each of the later MFMAs of row blocks 0..3 (an MFMA occupies the matrix pipe
+    // for 16 cycles; the VALU operations of the same wave behind it run in its shadow)
+    uint32_t d_t[4], d_G[4], d_H[4];
+    auto decode_slice = [&](int c, const uint32_t (&raw)[4], v4i (&out)[4]) {
+        const uint32_t lutA_lo = 0x00FF0100u, lutB_lo = 0x0000FF00u, lutB_hi = 0x00000001u;
+        auto partA = [&](int t) {
+            d_H[t] = d_G[t] >> 4;
+            out[t][0] = (int)perm(0u, lutA_lo, d_G[t] & 0x03030303u);
+        };
+        auto partB = [&](int t) {
+            out[t][1] = (int)perm(lutB_hi, lutB_lo, d_G[t] & 0x0C0C0C0Cu);
+            out[t][2] = (int)perm(0u, lutA_lo, d_H[t] & 0x03030303u);
+        };
+        auto partC = [&](int t) { out[t][3] = (int)perm(lutB_hi, lutB_lo, d_H[t] & 0x0C0C0C0Cu); };
+        switch (c) {
+            case 4:
+                d_t[0] = perm(raw[1], raw[0], 0x05010400u);
+                d_t[1] = perm(raw[1], raw[0], 0x07030602u);
+                d_t[2] = perm(raw[3], raw[2], 0x05010400u);
+                d_t[3] = perm(raw[3], raw[2], 0x07030602u);
+                break;
+            case 5:
+                d_G[0] = perm(d_t[2], d_t[0], 0x05040100u);
+                d_G[1] = perm(d_t[2], d_t[0], 0x07060302u);
+                d_G[2] = perm(d_t[3], d_t[1], 0x05040100u);
+                d_G[3] = perm(d_t[3], d_t[1], 0x07060302u);
+                break;
+            case 6: partA(0); break;
+            case 7: partB(0); break;
+            case 8: partC(0); partA(1); break;
+            case 9: partB(1); break;
+            case 10: partC(1); partA(2); break;
+            case 11: partB(2); break;
+            case 12: partC(2); partA(3); break;
+            case 13: partB(3); break;
+            case 14: partC(3); break;
+            default: break;
+        }
+    };
+
+    auto stage = [&](int s, uint4 (&a_reg)[2], uint32_t (&b_reg)[4], const v4i (&b_cur)[4], v4i (&b_nxt)[4]) {
         // a_reg / b_reg hold stage s+1 on entry and are reloaded with stage s+3
         const int cur = s & 1;
         store_a(cur ^ 1, a_reg);
+        load_stage(s + 3, 1, a_reg, b_reg);
+        read_a(cur, 4, a_hi);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int r = 0; r < 4; r++) b_nxt[r] = b_reg[r];
-        load_stage(s + 3, a_reg, b_reg);
-
-        uint32_t G[4];
-        transpose4x4_bytes(b_cur[0], b_cur[1], b_cur[2], b_cur[3], G);
-        v4i b[4];
-#pragma unroll
-        for (int t = 0; t < 4; t++) b[t] = decode16_i8(G[t]);
-        const uint8_t* a_lds = lds + cur * G_STAGE_BYTES + kgrp * (G_MB * 1024) + ((size_t)lane << 4);
-#pragma unroll
-        for (int mb = 0; mb < G_MB; mb++) {
-            const uint4 av = *(const uint4*)(a_lds + mb * 1024);
-            const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
-#pragma unroll
-            for (int t = 0; t < 4; t++)
-                acc[mb][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[t], acc[mb][t], 0, 0, 0);
+        for (int c = 0; c < 16; c++) {
+            const int i = c >> 2, t = c & 3;
+            const v4i a = {(int)a_lo[i].x, (int)a_lo[i].y, (int)a_lo[i].z, (int)a_lo[i].w};
+            acc[i][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b_cur[t], acc[i][t], 0, 0, 0);
+            decode_slice(c, b_reg, b_nxt);
+            __builtin_amdgcn_sched_barrier(0);  // keep the slice behind its MFMA
         }
-#pragma unroll
-        for (int r = 0; r < 4; r++) b_cur[r] = b_nxt[r];
+        // the raw weights are dead now: their registers take the loads of stage s+3 directly
+        // (a copy of a register with a load in flight would have to wait for that load)
+        load_stage(s + 3, 2, a_reg, b_reg);
+        __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        read_a(cur ^ 1, 0, a_lo);
+        mfma_half(4, a_hi, b_cur);
+        __builtin_amdgcn_sched_barrier(0);
     };
-    for (int s = 0; s < nstages; s += 2) {
-        stage(s, a_set[1], b_set[1]);
-        if (s + 1 < nstages) stage(s + 1, a_set[0], b_set[0]);
+    // (an odd last stage is peeled: with a conditional second half inside the loop the two
+    // paths to the loop header leave different loads outstanding, and the wait the compiler
+    // puts at the top of the loop then drains the whole queue, freshly issued loads included)
+    int s = 0;
+    for (; s + 1 < nstages; s += 2) {
+        stage(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
+        stage(s + 1, a_set[0], b_set[0], b_dec[1], b_dec[0]);
     }
+    if (s < nstages) stage(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
+    __syncthreads();  // every wave is done with the stage buffers before they are reused
 
     // ---- add the two K halves: waves (wn, 0) and (wn, 1) hold partial sums of the same
     // outputs.  K half 1 hands over row blocks 0..3, K half 0 hands over row blocks 4..7;
@@ -313,10 +401,9 @@ int launch_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const 
     p.tiles_n = (int)ceil_div(N, G_BN);
     const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
     p.per_xcd = (int)ceil_div(total, 8);
-    if (K % G_BK == 0)
-        hipLaunchKernelGGL(gemm_i8_kernel<false>, dim3((unsigned)(p.per_xcd * 8)), dim3(512), 0, st, p);
-    else
-        hipLaunchKernelGGL(gemm_i8_kernel<true>, dim3((unsigned)(p.per_xcd * 8)), dim3(512), 0, st, p);
+    const dim3 grid((unsigned)(p.per_xcd * 8)), block(512);
+    if (K % G_BK == 0) hipLaunchKernelGGL(gemm_i8_kernel<false>, grid, block, 0, st, p);
+    else hipLaunchKernelGGL(gemm_i8_kernel<true>, grid, block, 0, st, p);
     return check_launch("bt_ternary_gemm_i8");
 }
 

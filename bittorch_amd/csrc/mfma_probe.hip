@@ -1,0 +1,95 @@
+// Measurement aid: the int8 MFMA rate the chip sustains when nothing else is in the way.
+// Every wave issues back-to-back v_mfma_i32_16x16x64_i8 on eight independent accumulators
+// held in registers; no memory traffic inside the loop.  The prefill GEMM's TOPS are
+// reported against this figure as well as against the nominal peak.
+#include "bt_common.h"
+
+namespace bt {
+
+__global__ __launch_bounds__(512) void mfma_i8_probe_kernel(int iters, int random_operands, int* __restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    v4i a = {lane, lane + 1, lane + 2, lane + 3};
+    v4i b = {lane ^ 5, lane ^ 9, lane ^ 17, lane ^ 33};
+    if (random_operands) {
+        // full-range pseudo-random bytes (switching activity of real operands): A like
+        // quantized activations, B ternary {-1, 0, +1}
+        uint32_t h = (uint32_t)(blockIdx.x * 512 + threadIdx.x) * 2654435761u + 12345u;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            h = h * 1664525u + 1013904223u;
+            a[i] = (int)h;
+            h = h * 1664525u + 1013904223u;
+            uint32_t w = 0;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const uint32_t c = (h >> (8 * e + 3)) % 3u;  // 0, 1, 2 -> 0, +1, -1
+                w |= (c == 0 ? 0x00u : c == 1 ? 0x01u : 0xFFu) << (8 * e);
+            }
+            b[i] = (int)w;
+        }
+    }
+    v4i acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) acc[t] = v4i{t, 0, 0, 0};
+    for (int i = 0; i < iters; i++) {
+#pragma unroll
+        for (int t = 0; t < 8; t++) acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[t], 0, 0, 0);
+    }
+    int s = 0;
+#pragma unroll
+    for (int t = 0; t < 8; t++) s += acc[t][0] + acc[t][1] + acc[t][2] + acc[t][3];
+    if (s == 0x7fffffff) out[0] = s;  // keeps the loop alive; practically never true
+}
+
+// Same measurement with the register footprint of the prefill GEMM's inner product: a
+// 128 x 64 accumulator tile per wave (32 accumulators = 128 VGPRs), four A and four B operand
+// fragments per 32 MFMAs.
+__global__ __launch_bounds__(512) void mfma_i8_probe_tile_kernel(int iters, int* __restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    v4i a[8], b[4], acc[8][4];
+    uint32_t h = (uint32_t)(blockIdx.x * 512 + threadIdx.x) * 2654435761u + 12345u;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) { h = h * 1664525u + 1013904223u; a[i][e] = (int)h; }
+#pragma unroll
+    for (int t = 0; t < 4; t++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) { h = h * 1664525u + 1013904223u; b[t][e] = (int)(h & 0x01010101u); }
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int t = 0; t < 4; t++) acc[i][t] = v4i{lane, i, t, 0};
+    for (int it = 0; it < iters; it += 4) {
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+            for (int t = 0; t < 4; t++) acc[i][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i], b[t], acc[i][t], 0, 0, 0);
+    }
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int t = 0; t < 4; t++) s += acc[i][t][0] + acc[i][t][1] + acc[i][t][2] + acc[i][t][3];
+    if (s == 0x7fffffff) out[0] = s;
+}
+
+}  // namespace bt
+
+extern "C" int bt_probe_mfma_i8(int blocks, int iters, int random_operands, int* out, double* ops_per_launch,
+                                void* stream) {
+    using namespace bt;
+    if (blocks <= 0 || iters <= 0 || !out) {
+        set_error("bt_probe_mfma_i8: bad arguments");
+        return BT_ERR_INVALID;
+    }
+    if (random_operands == 2)  // 32 accumulators per wave; iters is rounded up to a multiple of 4
+        hipLaunchKernelGGL(mfma_i8_probe_tile_kernel, dim3((unsigned)blocks), dim3(512), 0, (hipStream_t)stream,
+                           iters, out);
+    else
+        hipLaunchKernelGGL(mfma_i8_probe_kernel, dim3((unsigned)blocks), dim3(512), 0, (hipStream_t)stream, iters,
+                           random_operands, out);
+    // 8 waves per block, 8 MFMAs per iteration, 2*16*16*64 operations each
+    if (ops_per_launch) *ops_per_launch = (double)blocks * 8.0 * (double)iters * 8.0 * 32768.0;
+    return check_launch("bt_probe_mfma_i8");
+}

@@ -128,10 +128,10 @@ __device__ __forceinline__ uint4 zero_unless(uint4 v, bool ok) {
 // d = the dword this lane loaded (row 4g+q, four columns); returns the bytes of column q of
 // the dwords of quad lanes 0..3, i.e. rows 4g..4g+3 of this lane's own column.
 __device__ __forceinline__ uint32_t quad_transpose(uint32_t d, uint32_t sel_q) {
-    const uint32_t v0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d, 0x00, 0xf, 0xf, false);
-    const uint32_t v1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d, 0x55, 0xf, 0xf, false);
-    const uint32_t v2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d, 0xAA, 0xf, 0xf, false);
-    const uint32_t v3 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d, 0xFF, 0xf, 0xf, false);
+    const uint32_t v0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d, 0x00, 0xf, 0xf, true);
+    const uint32_t v1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d, 0x55, 0xf, 0xf, true);
+    const uint32_t v2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d, 0xAA, 0xf, 0xf, true);
+    const uint32_t v3 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d, 0xFF, 0xf, 0xf, true);
     const uint32_t t01 = perm(v1, v0, sel_q);  // [v0.b[q], v1.b[q], -, -]
     const uint32_t t23 = perm(v3, v2, sel_q);
     return perm(t23, t01, 0x05040100u);

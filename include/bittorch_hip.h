@@ -151,6 +151,19 @@ int bt_ternary_linear_tensor_core_forward(const void* X, int x_dtype, const uint
 int bt_unpack_dequant(const uint8_t* W_T, const float* scale, int64_t scale_len, void* out,
                       int out_dtype, int64_t N, int64_t K, void* stream);
 
+/*
+ * Measurement aid with no counterpart in the reference: launches `blocks`
+ * workgroups of 8 waves that each issue `iters` x 8 back-to-back
+ * v_mfma_i32_16x16x64_i8 on register operands (no memory traffic) and writes the
+ * operation count of the launch (2*16*16*64 per instruction) to *ops_per_launch.
+ * random_operands = 0: small constant operands; 1: pseudo-random int8 activations
+ * and ternary weights, i.e. the switching activity of real data.  Timing it gives
+ * the int8 matrix-core rate the chip sustains, next to which the prefill GEMM is
+ * reported.  `out` is a device int the kernel may write.
+ */
+int bt_probe_mfma_i8(int blocks, int iters, int random_operands, int* out, double* ops_per_launch,
+                     void* stream);
+
 #ifdef __cplusplus
 }
 #endif
