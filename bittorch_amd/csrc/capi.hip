@@ -39,6 +39,9 @@ int launch_unpacked(const void* X, int x_dtype, const int8_t* W, const Epilogue&
                     int64_t N, int64_t K, hipStream_t st);
 int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x, hipStream_t st);
 bool gemm_i8_supported(int64_t N, int64_t K, const void* Q, const void* W_T);
+bool gemm_f16_supported(int64_t N, int64_t K, const void* X, const void* W_T, const void* Y);
+int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, const Epilogue& epi, void* Y, int y_dtype, int64_t M,
+                    int64_t N, int64_t K, hipStream_t st);
 int launch_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const Epilogue& epi, void* Y,
                    int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st);
 
@@ -142,6 +145,9 @@ extern "C" int bt_ternary_linear_packed_forward(const void* X, int x_dtype, cons
     hipStream_t st = (hipStream_t)stream;
     if (packed_uses_stream(x_dtype, W_T, Y, N, K)) {
         const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
+        // tall batches go to the tiled matrix-core kernel, decode shapes stream the weights
+        if (B > kStreamMaxRows && gemm_f16_supported(N, K, X, W_T, Y))
+            return launch_gemm_f16(mode, X, W_T, epi, Y, x_dtype, B, N, K, st);
         return launch_stream(mode, X, 2, nullptr, W_T, epi, Y, x_dtype, nullptr, B, N, K, workspace,
                              workspace_bytes, st);
     }

@@ -1,0 +1,345 @@
+// Large-batch fp16 / bf16 x packed-ternary GEMM for gfx950 on the 16-bit matrix cores:
+// the float path of the packed forward for batches too tall for the streaming kernel.
+//
+// Arithmetic restated from the reference's large-batch packed kernel
+// (csrc/kernels/ternary_gemm_production.cu:158-250, accumulate :226-235, epilogue :244-247):
+//   acc_f32[m,n] = sum_k x[m,k] * w[k,n];   y[m,n] = acc * scale[n] + bias[n]
+// (fp32 accumulation of exact products; the summation order differs from the reference's
+// sequential loop, which the 16-bit output tolerance covers).
+//
+// Same structure as the int8 prefill kernel: a 512-thread workgroup (8 waves) owns a
+// 128 x 256 output tile; wave w works on columns 64*(w&3) .. +63 and on k32 sub-step (w>>2)
+// of every 64-wide K stage over all 128 rows; the two K halves are added through LDS once.
+//   * Activations (16-bit, row-major [M,K]) go through LDS, double buffered, 64 k per stage,
+//     stored in MFMA operand order: slot (sub, mb, lane) is the 16 bytes (8 values) lane
+//     (i = lane%16, g = lane/16) feeds to v_mfma_f32_16x16x32_{f16,bf16} for row block mb and
+//     k32 sub-step sub, with the values already in the k order the weight decode produces.
+//   * Weights never touch LDS: lane (j, g) loads one dword (four output columns) from each of
+//     the two rows kb + 2g, 2g+1 and decodes each column's two bytes into eight 16-bit weights
+//     with v_perm table lookups (fp16 +-1.0; bf16 +-2.0 with the sum halved exactly).
+//   * The stage is software-pipelined inside the wave like the int8 kernel's.
+#include <cstdlib>
+
+#include "bt_common.h"
+
+namespace bt {
+
+constexpr int F_BM = 128;
+constexpr int F_BN = 256;
+constexpr int F_BK = 64;            // k per LDS stage (two k32 MFMA sub-steps)
+constexpr int F_MB = F_BM / 16;     // 16-row blocks per tile
+constexpr int F_STAGE_BYTES = F_BM * F_BK * 2;  // 16 KiB
+
+struct GemmFParams {
+    const uint16_t* X;    // [M, K] fp16 or bf16 bits
+    const uint8_t* W_T;   // [Kb, N]
+    void* Y;              // [M, N]
+    Epilogue epi;
+    int64_t M, N, K, Kb;
+    int y_dtype;
+    int tiles_m, tiles_n;
+    int per_xcd;          // workgroups per XCD (grid = 8 * per_xcd)
+};
+
+__device__ __forceinline__ void store4f(void* Y, int dt, int64_t idx, const float (&v)[4]) {
+    if (dt == BT_F32) {
+        *(float4*)((float*)Y + idx) = make_float4(v[0], v[1], v[2], v[3]);
+    } else {
+        uint16_t h[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) h[i] = (dt == BT_F16) ? f32_to_f16_bits(v[i]) : f32_to_bf16_bits(v[i]);
+        uint2 o;
+        o.x = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
+        o.y = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
+        *(uint2*)((uint16_t*)Y + idx) = o;
+    }
+}
+
+// Finishes four 16-row blocks (acc[MB0 .. MB0+3]) of the tile.
+template <int MODE, int YDT, int MB0>
+__device__ __forceinline__ void gemm_f_epilogue(const GemmFParams& p, const v4f (&acc)[F_MB][4], int64_t m0, int g,
+                                                int64_t ncol) {
+    float ws[4], bs[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        ws[t] = epi_scale(p.epi, ncol + t);
+        bs[t] = epi_bias(p.epi, ncol + t);
+    }
+#pragma unroll
+    for (int mbi = 0; mbi < 4; mbi++) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int64_t m = m0 + 16 * (MB0 + mbi) + 4 * g + r;
+            if (m >= p.M) continue;
+            float y[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                float a = acc[MB0 + mbi][t][r];
+                if constexpr (MODE == MODE_BF16) a *= 0.5f;  // weights were decoded as +-2.0
+                y[t] = epi_float(a, ws[t], bs[t]);
+            }
+            store4f(p.Y, YDT, m * p.N + ncol, y);
+        }
+    }
+}
+template <int MODE, int MB0>
+__device__ __forceinline__ void gemm_f_epilogue_dt(const GemmFParams& p, const v4f (&acc)[F_MB][4], int64_t m0,
+                                                   int g, int64_t ncol) {
+    if (p.y_dtype == BT_BF16) gemm_f_epilogue<MODE, BT_BF16, MB0>(p, acc, m0, g, ncol);
+    else if (p.y_dtype == BT_F16) gemm_f_epilogue<MODE, BT_F16, MB0>(p, acc, m0, g, ncol);
+    else gemm_f_epilogue<MODE, BT_F32, MB0>(p, acc, m0, g, ncol);
+}
+
+// TAIL = false: K is a multiple of the 64-wide stage and the main loop is branch free.
+// TAIL = true: any K % 8 == 0; the last, partial stage is masked.
+template <int MODE, bool TAIL>
+__global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[65536];  // 2 A stages; reused for the K-half exchange
+
+    // XCD-aware tile order: the 8 XCDs each take a contiguous run of tiles, walked in groups
+    // of four row tiles so that one XCD's L2 holds a compact block of rows and columns
+    const int64_t lin = (int64_t)(blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
+    if (lin >= (int64_t)p.tiles_m * p.tiles_n) return;
+    constexpr int GM = 4;
+    const int64_t group = lin / (GM * p.tiles_n);
+    const int64_t first_m = group * GM;
+    const int gm = (p.tiles_m - first_m < GM) ? (int)(p.tiles_m - first_m) : GM;
+    const int64_t in_group = lin - group * GM * p.tiles_n;
+    const int tile_m = (int)(first_m + in_group % gm);
+    const int tile_n = (int)(in_group / gm);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wn = wave & 3;     // column quarter
+    const int kgrp = wave >> 2;  // k32 sub-step of each stage
+    const int j = lane & 15;
+    const int g = lane >> 4;
+    const int64_t m0 = (int64_t)tile_m * F_BM;
+    const int64_t ncol = (int64_t)tile_n * F_BN + 64 * wn + 4 * j;
+    const bool col_ok = ncol < p.N;
+
+    // Addresses are a wave-uniform base (advanced once per stage) plus a 32-bit per-lane
+    // offset fixed for the whole kernel.  Loads are unconditional with clamped rows / columns:
+    // rows past M and columns past N only feed outputs that are never stored; the K tail is
+    // zeroed in the A operand of the last stage.
+    // A staging role: one row, 32 of its 128 stage bytes (16 values).  A wave stages one 16-row
+    // block: its 64 lanes touch 16 cache lines per load, eight consecutive lanes write 128
+    // contiguous bytes of LDS.
+    const int a_row = 16 * wave + (lane & 15);
+    const int a_part = lane >> 4;  // values 16*a_part .. +15 -> sub-step a_part>>1, groups 2*(a_part&1), +1
+    const int64_t rows_left = p.M - m0;
+    const uint32_t a_row_c = (uint32_t)((a_row < rows_left) ? a_row : rows_left - 1);
+    const uint32_t a_off = (a_row_c * (uint32_t)p.K + 16u * a_part) * 2u;  // bytes
+    const uint32_t b_off = (uint32_t)(col_ok ? ncol : 0) + (uint32_t)(8 * kgrp + 2 * g) * (uint32_t)p.N;
+    const uint8_t* a_base = (const uint8_t*)(p.X + m0 * p.K);  // uniform
+    const uint8_t* b_base = p.W_T;                              // uniform
+    const int64_t N = p.N;
+    const int nfull = (int)(p.K / F_BK);
+    const int nstages = (int)((p.K + F_BK - 1) / F_BK);
+
+    // two stages of operands in flight: set s%2 holds stage s until it is written to LDS
+    uint4 a_set[2][2];
+    uint32_t b_set[2][2];
+
+    // part: 1 = activations, 2 = weights, 3 = both
+    auto load_full = [&](int64_t k0, int part, uint4 (&a_reg)[2], uint32_t (&b_reg)[2]) {
+        if (part & 1) {
+            const uint8_t* ab = a_base + 2 * k0;
+            a_reg[0] = *(const uint4*)(ab + a_off);
+            a_reg[1] = *(const uint4*)(ab + 16 + a_off);
+        }
+        if (part & 2) {
+            const uint8_t* bb = b_base + (k0 >> 2) * N;
+            b_reg[0] = *(const uint32_t*)(bb + b_off);
+            b_reg[1] = *(const uint32_t*)(bb + N + b_off);
+        }
+    };
+    auto load_tail = [&](int64_t k0, int part, uint4 (&a_reg)[2], uint32_t (&b_reg)[2]) {
+        // last, partial stage: k beyond K reads a clamped address and is zeroed in A
+        if (part & 1) {
+            const uint8_t* ab = a_base + 2 * k0;
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                const bool in = (k0 + 16 * a_part + 8 * c) < p.K;
+                const uint4 v = *(const uint4*)(ab + (in ? 16 * c : 0) + (in ? a_off : a_row_c * (uint32_t)p.K * 2u));
+                const uint32_t m = in ? 0xFFFFFFFFu : 0u;
+                a_reg[c] = make_uint4(v.x & m, v.y & m, v.z & m, v.w & m);
+            }
+        }
+        if (part & 2) {
+#pragma unroll
+            for (int r = 0; r < 2; r++) {
+                int64_t kb = (k0 >> 2) + 8 * kgrp + 2 * g + r;
+                kb = kb < p.Kb ? kb : p.Kb - 1;
+                b_reg[r] = *(const uint32_t*)(b_base + kb * N + (col_ok ? ncol : 0));
+            }
+        }
+    };
+    auto load_stage = [&](int st, int part, uint4 (&a_reg)[2], uint32_t (&b_reg)[2]) {  // st, part uniform
+        if constexpr (TAIL) {
+            if (st >= nstages) st = nstages - 1;
+            if (st < nfull) load_full((int64_t)st * F_BK, part, a_reg, b_reg);
+            else load_tail((int64_t)st * F_BK, part, a_reg, b_reg);
+        } else {
+            // past the end: reload the last stage (never consumed) instead of branching
+            load_full((int64_t)(st < nstages ? st : nstages - 1) * F_BK, part, a_reg, b_reg);
+        }
+    };
+    auto store_a = [&](int buf, const uint4 (&a_reg)[2]) {
+        // slot (sub, mb, lane = c*16 + i) holds the 16 bytes MFMA lane (i, g = c) reads:
+        // natural values h0..h7 -> dword d = { h[d], h[4+d] } (the decode's k order)
+        uint8_t* base = lds + buf * F_STAGE_BYTES;
+        const int mb = a_row >> 4, i = a_row & 15, sub = a_part >> 1;
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+            const int c = 2 * (a_part & 1) + e;
+            const uint4 v = a_reg[e];
+            *(uint4*)(base + ((size_t)((sub * F_MB + mb) * 64 + c * 16 + i) << 4)) =
+                make_uint4(perm(v.z, v.x, 0x05040100u), perm(v.z, v.x, 0x07060302u), perm(v.w, v.y, 0x05040100u),
+                           perm(v.w, v.y, 0x07060302u));
+        }
+    };
+
+    v4f acc[F_MB][4];
+#pragma unroll
+    for (int mb = 0; mb < F_MB; mb++)
+#pragma unroll
+        for (int t = 0; t < 4; t++) acc[mb][t] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    // ---- main loop (see the int8 kernel: same pipeline) ------------------------------------
+    // Stage s is computed from LDS buffer s%2.  On entry the wave holds the decoded weights of
+    // stage s and the activation fragments of row blocks 0..3; it writes its piece of stage s+1
+    // into the other buffer, reloads those registers with stage s+3, requests row blocks 4..7,
+    // and issues the MFMAs of row blocks 0..3 with the decode of stage s+1 sliced in behind
+    // them; the stage's one barrier publishes buffer (s+1)%2, whose row blocks 0..3 are
+    // requested right behind it and arrive under the MFMAs of row blocks 4..7.
+    u32x4 b_dec[2][4];
+    uint4 a_lo[4], a_hi[4];
+    const uint32_t a_lds_off = (uint32_t)(kgrp * (F_MB * 1024)) + ((uint32_t)lane << 4);
+    constexpr uint32_t LUT = (MODE == MODE_F16) ? LUT_F16_ONE : LUT_BF16_TWO;
+    auto decode_col = [&](const uint32_t (&raw)[2], int t, u32x4& out) {
+        // bytes [zero, row0.byte t, zero, row1.byte t]
+        const uint32_t sel = ((uint32_t)(4 + t) << 24) | (0x0Cu << 16) | ((uint32_t)t << 8) | 0x0Cu;
+        out = decode8_16bit<LUT>(perm(raw[1], raw[0], sel));
+    };
+    auto read_a = [&](int buf, int mb0, uint4 (&dst)[4]) {
+        const uint8_t* a_lds = lds + buf * F_STAGE_BYTES + a_lds_off;
+#pragma unroll
+        for (int i = 0; i < 4; i++) dst[i] = *(const uint4*)(a_lds + (mb0 + i) * 1024);
+    };
+    auto mfma = [&](const uint4& av, const u32x4& bv, v4f& c) {
+        const u32x4 a = {av.x, av.y, av.z, av.w};
+        if constexpr (MODE == MODE_F16)
+            c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, bv), c, 0, 0, 0);
+        else
+            c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, bv), c, 0, 0, 0);
+    };
+
+    load_stage(0, 3, a_set[0], b_set[0]);
+    load_stage(1, 3, a_set[1], b_set[1]);
+    store_a(0, a_set[0]);
+#pragma unroll
+    for (int t = 0; t < 4; t++) decode_col(b_set[0], t, b_dec[0][t]);
+    load_stage(2, 3, a_set[0], b_set[0]);
+    __syncthreads();
+    read_a(0, 0, a_lo);
+
+    auto stage = [&](int s, uint4 (&a_reg)[2], uint32_t (&b_reg)[2], const u32x4 (&b_cur)[4], u32x4 (&b_nxt)[4]) {
+        // a_reg / b_reg hold stage s+1 on entry and are reloaded with stage s+3
+        const int cur = s & 1;
+        store_a(cur ^ 1, a_reg);
+        load_stage(s + 3, 1, a_reg, b_reg);
+        read_a(cur, 4, a_hi);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < 16; c++) {
+            mfma(a_lo[c >> 2], b_cur[c & 3], acc[c >> 2][c & 3]);
+            if ((c & 3) == 1) decode_col(b_reg, c >> 2, b_nxt[c >> 2]);  // one column behind every fourth MFMA
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // the raw weights are dead now: their registers take the loads of stage s+3 directly
+        load_stage(s + 3, 2, a_reg, b_reg);
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        read_a(cur ^ 1, 0, a_lo);
+#pragma unroll
+        for (int c = 0; c < 16; c++) mfma(a_hi[c >> 2], b_cur[c & 3], acc[4 + (c >> 2)][c & 3]);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // (an odd last stage is peeled so that both paths into the loop header leave the same
+    // loads outstanding)
+    int s = 0;
+    for (; s + 1 < nstages; s += 2) {
+        stage(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
+        stage(s + 1, a_set[0], b_set[0], b_dec[1], b_dec[0]);
+    }
+    if (s < nstages) stage(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
+    __syncthreads();  // every wave is done with the stage buffers before they are reused
+
+    // ---- add the two K halves: K half 1 hands over row blocks 0..3, K half 0 hands over row
+    // blocks 4..7; word (q, wn, lane) of the exchange buffer is register q of that lane ----
+    {
+        float* xch = (float*)lds;
+        const int slot = wn * 64 + lane;
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const int giver = 1 - half;
+            if (kgrp == giver) {
+#pragma unroll
+                for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        const v4f v = acc[4 * half + mb][t];
+                        *(float4*)(xch + ((mb * 4 + t) * 256 + slot) * 4) = make_float4(v[0], v[1], v[2], v[3]);
+                    }
+            }
+            __syncthreads();
+            if (kgrp != giver) {
+#pragma unroll
+                for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        const float4 v = *(const float4*)(xch + ((mb * 4 + t) * 256 + slot) * 4);
+                        acc[4 * half + mb][t] += v4f{v.x, v.y, v.z, v.w};
+                    }
+            }
+            __syncthreads();
+        }
+    }
+
+    if (!col_ok) return;
+    if (kgrp == 0) gemm_f_epilogue_dt<MODE, 0>(p, acc, m0, g, ncol);  // wave-uniform branch
+    else gemm_f_epilogue_dt<MODE, 4>(p, acc, m0, g, ncol);
+}
+
+// the tiled kernel reads X with 16-byte loads and W_T / Y with 4-column vectors
+bool gemm_f16_supported(int64_t N, int64_t K, const void* X, const void* W_T, const void* Y) {
+    return N % 4 == 0 && K % 8 == 0 && K >= 8 && ((uintptr_t)W_T) % 4 == 0 && ((uintptr_t)X) % 16 == 0 &&
+           ((uintptr_t)Y) % 16 == 0 && (F_BM + 1) * K * 2 < (1ll << 32) && ceil_div(K, 4) * N < (1ll << 32);
+}
+
+int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, const Epilogue& epi, void* Y, int y_dtype, int64_t M,
+                    int64_t N, int64_t K, hipStream_t st) {
+    GemmFParams p;
+    p.X = (const uint16_t*)X; p.W_T = W_T; p.Y = Y; p.epi = epi;
+    p.M = M; p.N = N; p.K = K; p.Kb = ceil_div(K, 4);
+    p.y_dtype = y_dtype;
+    p.tiles_m = (int)ceil_div(M, F_BM);
+    p.tiles_n = (int)ceil_div(N, F_BN);
+    const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
+    p.per_xcd = (int)ceil_div(total, 8);
+    const dim3 grid((unsigned)(p.per_xcd * 8)), block(512);
+    const bool tail = K % F_BK != 0;
+    if (mode == MODE_F16) {
+        if (tail) hipLaunchKernelGGL((gemm_f16_kernel<MODE_F16, true>), grid, block, 0, st, p);
+        else hipLaunchKernelGGL((gemm_f16_kernel<MODE_F16, false>), grid, block, 0, st, p);
+    } else {
+        if (tail) hipLaunchKernelGGL((gemm_f16_kernel<MODE_BF16, true>), grid, block, 0, st, p);
+        else hipLaunchKernelGGL((gemm_f16_kernel<MODE_BF16, false>), grid, block, 0, st, p);
+    }
+    return check_launch("bt_ternary_linear_packed_forward");
+}
+
+}  // namespace bt

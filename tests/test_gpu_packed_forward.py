@@ -85,6 +85,38 @@ def test_packed_forward_batch_sizes(oracle, b):
     _case(oracle, b, 128, 256, torch.bfloat16, seed=b)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("b,n,k", [(128, 256, 64), (33, 128, 256), (200, 260, 72), (129, 512, 1000), (512, 1024, 4096),
+                                   (130, 36, 8), (257, 300, 136), (64, 256, 768)])
+def test_packed_forward_tall_batches_use_the_tiled_kernel(oracle, dtype, b, n, k):
+    """Batches above the streaming kernel's limit go to the 16-bit matrix-core GEMM: partial row
+    and column tiles, K tails that are not a multiple of the 64-wide stage, odd last stages."""
+    announce("packed_forward tall", dtype, b, n, k)
+    _case(oracle, b, n, k, dtype, seed=b + n + k)
+
+
+def test_packed_forward_tall_batch_matches_streaming_kernel(oracle):
+    """The tiled kernel and the streaming kernel (forced by splitting the batch into 16-row
+    calls) see the same exact products; they differ by fp32 summation order only."""
+    from bittorch_amd import _C
+    from bittorch_amd.quant import pack_ternary_transposed
+    announce("packed_forward tall vs stream")
+    g = torch.Generator().manual_seed(5)
+    n, k, b = 512, 2048, 256
+    w = torch.randint(-1, 2, (n, k), generator=g).float()
+    packed = pack_ternary_transposed(w)[0].cuda()
+    scale = (torch.rand(n, generator=g) + 0.5).cuda()
+    for dtype in (torch.float16, torch.bfloat16):
+        x = torch.randn(b, k, generator=g).to(dtype).cuda()
+        y_tiled = _C.ternary_linear_packed_forward(x, packed, scale, None, k)
+        y_stream = torch.cat([_C.ternary_linear_packed_forward(x[i:i + 16].contiguous(), packed, scale, None, k)
+                              for i in range(0, b, 16)])
+        ref = (x.double() @ w.double().cuda().T) * scale.double()
+        denom = ref.abs().max()
+        assert ((y_tiled.double() - ref).abs().max() / denom) < 1e-2
+        assert ((y_tiled.double() - y_stream.double()).abs().max() / denom) < 1e-2
+
+
 def test_packed_forward_fp32_generic_is_bit_exact(oracle):
     """The generic kernel accumulates in the reference's k order: equal to the oracle bit for bit."""
     announce("packed_forward fp32 bit exact")
