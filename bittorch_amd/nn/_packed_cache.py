@@ -1,0 +1,47 @@
+"""Per-module cache of the packed ternary weights.
+
+The reference re-runs ``ternary_quantize`` on the master weights in every forward
+(``bittorch/nn/ternary_linear.py:196-200``, ``bittorch/nn/ternary_linear_cuda.py:52-54``).
+The result depends on the weights only, so it is kept until they change: the key is the
+parameter's version counter (every in-place update, optimizer step or ``load_state_dict``
+bumps it), its storage address, dtype and device, and the quantizer's two settings.  With
+frozen weights (inference, evaluation, gradient accumulation) a forward then reads K*N/4
+bytes of packed weights instead of 4*K*N bytes of masters.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+from torch import Tensor
+
+
+class PackedWeightCache:
+    __slots__ = ("key", "value")
+
+    def __init__(self) -> None:
+        self.key = None
+        self.value: Optional[Tuple[Tensor, Tensor]] = None
+
+    def get(self, weight: Tensor, threshold_factor: float, per_channel: bool) -> Tuple[Tensor, Tensor]:
+        """``(packed_T uint8 [ceil(K/4), N], scale fp32 [N] or 0-dim)`` of the current weights."""
+        from .. import _C
+
+        key = (weight._version, weight.data_ptr(), weight.dtype, weight.device, float(threshold_factor),
+               bool(per_channel))
+        if key != self.key:
+            with torch.no_grad():
+                packed, scale, _ = _C.ternary_quantize_pack(weight.detach(), threshold_factor, per_channel)
+            self.key, self.value = key, (packed, scale)
+        return self.value
+
+    def clear(self) -> None:
+        self.key, self.value = None, None
+
+
+def cache_usable(x: Tensor, weight: Tensor) -> bool:
+    """The cache holds the quantization of the stored weights in their own dtype.  Under
+    autocast the autograd function quantizes an fp16 copy instead (reference semantics), and
+    float64 runs on the dense entry point, so neither uses it."""
+    return (not torch.is_autocast_enabled() and weight.dtype != torch.float64 and x.dtype != torch.float64)

@@ -18,6 +18,7 @@ import torch.nn.functional as F
 from torch import Tensor
 
 from ..quant.ternary import ternary_quantize, ternary_quantize_ste
+from ._packed_cache import PackedWeightCache, cache_usable
 
 BackendType = Literal["auto", "cuda", "python"]
 _BACKENDS = ("auto", "cuda", "python")
@@ -73,6 +74,7 @@ class TernaryLinear(nn.Module):
             self.bias = nn.Parameter(torch.empty(out_features))
         else:
             self.register_parameter("bias", None)
+        self._packed = PackedWeightCache()
         self.reset_parameters()
 
     def reset_parameters(self) -> None:
@@ -103,8 +105,11 @@ class TernaryLinear(nn.Module):
             return F.linear(x, self.weight, self.bias)
         if self._should_use_cuda_kernel(x):
             from .ternary_linear_cuda import TernaryLinearCUDAFunction
+            cached = None
+            if cache_usable(x, self.weight):  # packed weights are kept until the masters change
+                cached = self._packed.get(self.weight, self.threshold_factor, self.per_channel)
             return TernaryLinearCUDAFunction.apply(x, self.weight, self.bias, self.threshold_factor,
-                                                   self.per_channel)
+                                                   self.per_channel, cached)
         # plain torch path (reference :194-213): the scale is folded into the
         # weights, which are rounded to the activation dtype before the product
         w_q, scale = ternary_quantize_ste(self.weight, self.threshold_factor, self.per_channel)

@@ -17,6 +17,7 @@ import torch.nn as nn
 from torch import Tensor
 
 from ..quant.ternary import ternary_quantize
+from ._packed_cache import PackedWeightCache, cache_usable
 from .ternary_linear import _init_linear_params
 
 
@@ -26,7 +27,9 @@ class TernaryLinearCUDAFunction(torch.autograd.Function):
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.float16)
     def forward(ctx, x: Tensor, weight: Tensor, bias: Optional[Tensor], threshold_factor: float,
-                per_channel: bool) -> Tensor:
+                per_channel: bool, cached=None) -> Tensor:
+        """``cached``: optional ``(packed_T, scale)`` of exactly these weights (see
+        ``_packed_cache.py``); the quantize+pack kernel is skipped when it is given."""
         from .. import _C
 
         if weight.dtype == torch.float64 or x.dtype == torch.float64:
@@ -37,7 +40,10 @@ class TernaryLinearCUDAFunction(torch.autograd.Function):
             packed = None
             ctx.w_eff = w_tern * scale.reshape(-1, 1)
         else:
-            packed, scale, _ = _C.ternary_quantize_pack(weight, threshold_factor, per_channel)
+            if cached is not None:
+                packed, scale = cached
+            else:
+                packed, scale, _ = _C.ternary_quantize_pack(weight, threshold_factor, per_channel)
             out = _C.ternary_linear_packed_forward(
                 x.contiguous(), packed, scale.reshape(-1).to(x.dtype),
                 None if bias is None else bias.to(x.dtype).contiguous(), weight.shape[1])
@@ -70,7 +76,7 @@ class TernaryLinearCUDAFunction(torch.autograd.Function):
             grad_w = (g2.t() @ x2) * scale_col.to(g2.dtype)
         if ctx.has_bias and ctx.needs_input_grad[2]:
             grad_b = g2.sum(dim=0)
-        return grad_x, grad_w, grad_b, None, None
+        return grad_x, grad_w, grad_b, None, None, None
 
 
 class TernaryLinearCUDA(nn.Module):
@@ -88,6 +94,7 @@ class TernaryLinearCUDA(nn.Module):
             self.bias = nn.Parameter(torch.empty(out_features))
         else:
             self.register_parameter("bias", None)
+        self._packed = PackedWeightCache()
         self.reset_parameters()
 
     def reset_parameters(self) -> None:
@@ -96,8 +103,11 @@ class TernaryLinearCUDA(nn.Module):
     def forward(self, x: Tensor) -> Tensor:
         if not x.is_cuda:
             raise RuntimeError("TernaryLinearCUDA requires CUDA tensors. Use TernaryLinear for CPU.")
+        cached = None
+        if cache_usable(x, self.weight):
+            cached = self._packed.get(self.weight, self.threshold_factor, self.per_channel)
         return TernaryLinearCUDAFunction.apply(x, self.weight, self.bias, self.threshold_factor,
-                                               self.per_channel)
+                                               self.per_channel, cached)
 
     def extra_repr(self) -> str:
         return (f"in_features={self.in_features}, out_features={self.out_features}, "

@@ -179,3 +179,47 @@ def test_xor_training_on_gpu():
         loss.backward()
         opt.step()
     assert ((model(xs) > 0).float() == ys).all()
+
+
+def test_packed_weight_cache_follows_the_weights(monkeypatch):
+    """The packed weights are re-made exactly when the master weights change (in-place update,
+    load_state_dict, move to another dtype) and never otherwise; outputs equal an uncached run."""
+    from bittorch_amd import _C
+    from bittorch_amd.nn import TernaryLinear, TernaryLinearCUDA
+    announce("packed weight cache")
+    calls = {"n": 0}
+    real = _C.ternary_quantize_pack
+
+    def counting(*a, **k):
+        calls["n"] += 1
+        return real(*a, **k)
+
+    monkeypatch.setattr(_C, "ternary_quantize_pack", counting)
+    for cls in (TernaryLinear, TernaryLinearCUDA):
+        torch.manual_seed(1)
+        layer = cls(64, 32).cuda()
+        x = torch.randn(8, 64, device="cuda")
+        calls["n"] = 0
+        y0 = layer(x)
+        y1 = layer(x)
+        with torch.no_grad():
+            y2 = layer(x)
+        assert calls["n"] == 1 and torch.equal(y0, y1) and torch.equal(y0, y2)
+        # training step: backward works through the cached forward, the update invalidates it
+        opt = torch.optim.SGD(layer.parameters(), lr=0.5)
+        layer(x).pow(2).sum().backward()
+        assert layer.weight.grad is not None and layer.weight.grad.abs().sum() > 0
+        opt.step()
+        y3 = layer(x)
+        assert calls["n"] == 2
+        packed, scale, _ = real(layer.weight.detach(), layer.threshold_factor, layer.per_channel)
+        ref = _C.ternary_linear_packed_forward(x, packed, scale.reshape(-1), layer.bias.detach(), 64)
+        assert torch.equal(y3, ref)
+        # load_state_dict copies in place
+        other = cls(64, 32).cuda()
+        layer.load_state_dict(other.state_dict())
+        assert torch.equal(layer(x), other(x)) and calls["n"] == 4
+        # dtype change replaces the storage
+        layer.half()
+        yh = layer(x.half())
+        assert yh.dtype == torch.float16 and calls["n"] == 5
