@@ -40,6 +40,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
+    ap.add_argument("--no-block-stack", action="store_true", help="skip the 30-layer block stack (config 5)")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU baseline sample length")
     ap.add_argument("--pmc-pass", action="store_true",
                     help="no timing: a few eager launches of each kernel plus a plain copy of known size, "
@@ -72,6 +73,94 @@ def graph_time(fn, steps, warmup, torch):
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     return wall_ms, e0.elapsed_time(e1)
+
+
+def block_stack(torch, dev, layers=30, d_model=2560, heads=20, ffn=6912, batch=8, seq=512, vocab=32000):
+    """Config 5: forward of a 2B-parameter BitNet-b1.58-like stack.  q/k/v/o/gate/up/down are
+    TernaryLinear (random N(0,0.02) masters, no bias); RMSNorm, rotary-free causal SDPA, SwiGLU and
+    the embedding stay in PyTorch-ROCm; bf16 activations, a seeded token batch of batch x seq."""
+    import torch.nn as nn
+    import torch.nn.functional as F
+    import bittorch_amd as bt
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            mk = lambda i, o: bt.nn.TernaryLinear(i, o, bias=False)
+            self.q, self.k, self.v, self.o = mk(d_model, d_model), mk(d_model, d_model), mk(d_model, d_model), mk(d_model, d_model)
+            self.gate, self.up, self.down = mk(d_model, ffn), mk(d_model, ffn), mk(ffn, d_model)
+            self.n1 = nn.RMSNorm(d_model)
+            self.n2 = nn.RMSNorm(d_model)
+
+        def forward(self, x):
+            b, t, _ = x.shape
+            h = self.n1(x)
+            q = self.q(h).view(b, t, heads, -1).transpose(1, 2)
+            k = self.k(h).view(b, t, heads, -1).transpose(1, 2)
+            v = self.v(h).view(b, t, heads, -1).transpose(1, 2)
+            a = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(b, t, -1)
+            x = x + self.o(a)
+            h = self.n2(x)
+            return x + self.down(F.silu(self.gate(h)) * self.up(h))
+
+    torch.manual_seed(0)
+    with torch.device(dev):
+        emb = nn.Embedding(vocab, d_model).to(torch.bfloat16)
+        blocks = nn.ModuleList([Block() for _ in range(layers)])
+        final = nn.RMSNorm(d_model)
+    for m in blocks.modules():
+        if isinstance(m, bt.nn.TernaryLinear):
+            nn.init.normal_(m.weight, std=0.02)
+        elif isinstance(m, nn.RMSNorm):
+            m.to(torch.bfloat16)
+    final.to(torch.bfloat16)
+    tokens = torch.randint(0, vocab, (batch, seq), generator=torch.Generator().manual_seed(0)).to(dev)
+    n_tern = sum(m.weight.numel() for m in blocks.modules() if isinstance(m, bt.nn.TernaryLinear))
+
+    def forward(stack):
+        with torch.no_grad():
+            x = emb(tokens)
+            for blk in stack:
+                x = blk(x)
+            return final(x)
+
+    def timed(stack, reps, before=None):
+        forward(stack)
+        torch.cuda.synchronize()
+        best = 1e30
+        for _ in range(reps):
+            if before:
+                before()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            forward(stack)
+            torch.cuda.synchronize()
+            best = min(best, (time.perf_counter() - t0) * 1e3)
+        return best
+
+    def drop_caches():
+        for m in blocks.modules():
+            if isinstance(m, bt.nn.TernaryLinear):
+                m._packed.clear()
+
+    res = {"layers": layers, "d_model": d_model, "heads": heads, "ffn": ffn, "tokens": batch * seq,
+           "ternary_weights": n_tern,
+           "ops_per_forward_ternary_layers": 2.0 * batch * seq * n_tern}
+    res["ms_requantize_every_forward"] = round(timed(blocks, 3, drop_caches), 3)   # what the reference does
+    res["ms_packed_weights_cached"] = round(timed(blocks, 5), 3)
+    y_train = forward(blocks)
+    infer = bt.utils.convert_linear_layers(blocks, inplace=True)  # masters are freed layer by layer
+    res["ms_inference_modules"] = round(timed(infer, 5), 3)
+    y_inf = forward(infer)
+    # (the training forward rounds the scales to bf16 as the reference does; the inference
+    # modules keep them in fp32)
+    res["inference_vs_training_forward_max_rel_diff"] = round(
+        float((y_train.float() - y_inf.float()).abs().max() / y_train.float().abs().max()), 5)
+    res["ternary_TFLOPS_cached"] = round(res["ops_per_forward_ternary_layers"] / (res["ms_packed_weights_cached"] * 1e-3) / 1e12, 1)
+    res["packed_weight_bytes"] = n_tern // 4
+    del blocks, infer
+    torch.cuda.empty_cache()
+    return res
 
 
 def measured_traffic(tag):
@@ -285,6 +374,12 @@ def main():
                 "frac_of_hbm_peak": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
             }
             del masters
+        # config 5: the 30-layer block stack, end to end
+        if not args.no_block_stack:
+            try:
+                extra["block_stack_2B_forward"] = block_stack(torch, dev)
+            except RuntimeError as err:  # e.g. not enough free HBM on a shared card
+                extra["block_stack_2B_forward"] = {"skipped": str(err)[:200]}
         out["secondary"] = extra
 
     # ---- CPU baseline: the oracle (a scalar C port of the reference arithmetic) -------------

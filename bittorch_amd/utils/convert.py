@@ -1,0 +1,160 @@
+"""Model conversion, accounting and checkpoints for packed ternary layers.
+
+API mirror of ``bittorch/utils/convert.py:19-246`` (same names, arguments and result
+dictionaries).  Two things differ on purpose:
+  * layers whose weights live on the GPU are converted by the fused quantize+pack kernel
+    (one read of the master weights) instead of the quantize -> pack -> transpose chain of
+    torch ops; the bytes and scales are the same bit for bit;
+  * ``load_ternary_checkpoint`` reads with ``weights_only=True`` (a checkpoint is tensors plus
+    a plain metadata dictionary; nothing in it needs unpickling of code).
+"""
+
+from __future__ import annotations
+
+import copy
+from typing import Any, Dict, Optional
+
+import torch
+import torch.nn as nn
+
+from ..nn.ternary_linear import TernaryLinear
+from ..nn.ternary_linear_infer import TernaryLinearInference, create_ternary_linear_inference
+from ..quant.ternary import ternary_quantize
+
+
+def fp_linear_to_ternary_infer(linear: nn.Linear, threshold_factor: float = 0.05) -> TernaryLinearInference:
+    """``nn.Linear`` -> ``TernaryLinearInference`` (reference ``:19-49``): per-channel absmax
+    quantization of the weights, packed transposed storage, bias kept as it is."""
+    bias = linear.bias.data if linear.bias is not None else None
+    return create_ternary_linear_inference(linear.in_features, linear.out_features, linear.weight.data, bias,
+                                           threshold_factor)
+
+
+def ternary_linear_to_infer(ternary_linear: TernaryLinear) -> TernaryLinearInference:
+    """Trained ``TernaryLinear`` -> ``TernaryLinearInference`` with the weights the training
+    module's forward uses (reference ``:52-73``: its threshold factor and scale granularity)."""
+    bias = ternary_linear.bias.data if ternary_linear.bias is not None else None
+    weight = ternary_linear.weight.data
+    if weight.is_cuda and weight.dtype in (torch.float32, torch.float16, torch.bfloat16):
+        from ..nn.ternary_linear import _cuda_kernel_available
+        if _cuda_kernel_available():
+            from .. import _C
+            packed, scale, _ = _C.ternary_quantize_pack(weight, ternary_linear.threshold_factor,
+                                                        ternary_linear.per_channel)
+            scale = scale.reshape(-1).expand(ternary_linear.out_features).contiguous()
+            return TernaryLinearInference(ternary_linear.in_features, ternary_linear.out_features, packed, scale,
+                                          bias)
+    w_tern, scale = ternary_linear.get_quantized_weight()
+    scale = scale.reshape(-1).expand(ternary_linear.out_features).contiguous()
+    return TernaryLinearInference.from_unpacked(w_tern, scale, bias)
+
+
+def convert_linear_layers(module: nn.Module, threshold_factor: float = 0.05, skip_names: Optional[list] = None,
+                          inplace: bool = False) -> nn.Module:
+    """Replace every ``nn.Linear`` / ``TernaryLinear`` in the tree by a ``TernaryLinearInference``
+    (reference ``:76-133``).  A child is skipped when any entry of ``skip_names`` is a substring of
+    its dotted name; skipped and other modules are searched further down."""
+    skip_names = skip_names or []
+    if not inplace:
+        module = copy.deepcopy(module)
+
+    def skipped(name: str) -> bool:
+        return any(pattern in name for pattern in skip_names)
+
+    def walk(parent: nn.Module, prefix: str) -> None:
+        for name, child in list(parent.named_children()):
+            full = f"{prefix}.{name}" if prefix else name
+            if isinstance(child, nn.Linear) and not skipped(full):
+                setattr(parent, name, fp_linear_to_ternary_infer(child, threshold_factor))
+            elif isinstance(child, TernaryLinear) and not skipped(full):
+                setattr(parent, name, ternary_linear_to_infer(child))
+            else:
+                walk(child, full)
+
+    walk(module, "")
+    return module
+
+
+def count_ternary_params(module: nn.Module) -> Dict[str, int]:
+    """Weights by storage type (reference ``:136-166``): ``fp32``, ``fp16``, ``packed_ternary``, ``total``
+    (biases and scales are not counted; any non-fp16 dense weight counts as fp32, as in the reference)."""
+    counts = {"fp32": 0, "fp16": 0, "packed_ternary": 0, "total": 0}
+    for child in module.modules():
+        if isinstance(child, TernaryLinearInference):
+            n = child.out_features * child.in_features
+            counts["packed_ternary"] += n
+        elif isinstance(child, (nn.Linear, TernaryLinear)):
+            n = child.weight.numel()
+            counts["fp16" if child.weight.dtype == torch.float16 else "fp32"] += n
+        else:
+            continue
+        counts["total"] += n
+    return counts
+
+
+def get_model_memory_bytes(module: nn.Module) -> Dict[str, int]:
+    """Bytes by storage type (reference ``:169-207``): ``fp32``, ``fp16``, ``packed_ternary``,
+    ``scales``, ``total`` (the total also includes the biases)."""
+    out = {"fp32": 0, "fp16": 0, "packed_ternary": 0, "scales": 0, "total": 0}
+    for child in module.modules():
+        if isinstance(child, TernaryLinearInference):
+            packed = child.weight_packed.numel()
+            scales = child.scale.numel() * child.scale.element_size()
+            out["packed_ternary"] += packed
+            out["scales"] += scales
+            out["total"] += packed + scales
+        elif isinstance(child, (nn.Linear, TernaryLinear)):
+            nbytes = child.weight.numel() * child.weight.element_size()
+            out["fp16" if child.weight.dtype == torch.float16 else "fp32"] += nbytes
+            out["total"] += nbytes
+        else:
+            continue
+        if child.bias is not None:
+            out["total"] += child.bias.numel() * child.bias.element_size()
+    return out
+
+
+def save_ternary_checkpoint(module: nn.Module, path: str, metadata: Optional[Dict[str, Any]] = None) -> None:
+    """``{"state_dict": ..., "metadata": ...}`` written with ``torch.save`` (reference ``:210-228``).
+    State-dict keys of a packed layer: ``weight_packed`` uint8 ``[ceil(K/4), N]``, ``scale``, ``bias``."""
+    torch.save({"state_dict": module.state_dict(), "metadata": metadata or {}}, path)
+
+
+def load_ternary_checkpoint(path: str, module: nn.Module) -> Dict[str, Any]:
+    """Load such a checkpoint into a module of matching architecture and return its metadata
+    (reference ``:231-246``)."""
+    checkpoint = torch.load(path, map_location="cpu", weights_only=True)
+    module.load_state_dict(checkpoint["state_dict"])
+    return checkpoint.get("metadata", {})
+
+
+def save_ternary_safetensors(module: nn.Module, path: str, metadata: Optional[Dict[str, str]] = None) -> None:
+    """The same state dict as a safetensors file: ``<layer>.weight_packed`` U8
+    ``[ceil(K/4), N]`` and ``<layer>.scale`` F32 ``[N]`` are the tensors the reference's browser
+    runtime reads (``js/src/loaders/SafeTensorsLoader.ts:223-234``).  Metadata values must be strings."""
+    from safetensors.torch import save_file
+
+    tensors = {}
+    for k, v in module.state_dict().items():
+        t = v.detach().cpu().contiguous()
+        if k.endswith(".scale") or k == "scale":
+            t = t.float()
+        tensors[k] = t
+    save_file(tensors, path, metadata=metadata or {})
+
+
+def load_ternary_safetensors(path: str, module: nn.Module) -> Dict[str, str]:
+    """Load a safetensors state dict (scales are cast to the dtype the module holds)."""
+    from safetensors import safe_open
+
+    state = {}
+    with safe_open(path, framework="pt", device="cpu") as fh:
+        meta = fh.metadata() or {}
+        for k in fh.keys():
+            state[k] = fh.get_tensor(k)
+    own = module.state_dict()
+    for k, v in state.items():
+        if k in own and own[k].dtype != v.dtype and v.is_floating_point():
+            state[k] = v.to(own[k].dtype)
+    module.load_state_dict(state)
+    return dict(meta)

@@ -1,0 +1,136 @@
+"""Model conversion, accounting and checkpoints (mirror of bittorch/utils/convert.py; the
+reference ships no test for these, so the checks are the definitions themselves: a converted
+layer computes what the training layer's plain-torch forward computes, counts follow from the
+shapes, and a checkpoint round trip reproduces every buffer bit for bit)."""
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+import bittorch_amd as bt
+from bittorch_amd.nn import TernaryLinear, TernaryLinearInference
+from bittorch_amd.quant import pack_ternary_transposed, ternary_quantize
+from bittorch_amd.utils import (convert_linear_layers, count_ternary_params, fp_linear_to_ternary_infer,
+                                get_model_memory_bytes, load_ternary_checkpoint, load_ternary_safetensors,
+                                save_ternary_checkpoint, save_ternary_safetensors, ternary_linear_to_infer)
+
+
+def _mlp():
+    torch.manual_seed(0)
+    return nn.Sequential(nn.Linear(64, 32), nn.ReLU(), TernaryLinear(32, 16, backend="python"), nn.ReLU(),
+                         nn.Linear(16, 10))
+
+
+def test_fp_linear_to_ternary_infer_matches_definition():
+    torch.manual_seed(1)
+    lin = nn.Linear(70, 33)  # K not a multiple of 4
+    inf = fp_linear_to_ternary_infer(lin, threshold_factor=0.07)
+    assert isinstance(inf, TernaryLinearInference)
+    assert (inf.in_features, inf.out_features) == (70, 33)
+    w_tern, scale = ternary_quantize(lin.weight.data, threshold_factor=0.07)
+    packed, k = pack_ternary_transposed(w_tern)
+    assert k == 70 and torch.equal(inf.weight_packed, packed) and torch.equal(inf.scale, scale)
+    assert inf.weight_packed.shape == (18, 33) and inf.weight_packed.dtype == torch.uint8
+    x = torch.randn(5, 70)
+    ref = x @ (w_tern * scale[:, None]).T + lin.bias
+    assert torch.allclose(inf(x), ref, atol=1e-5)
+    assert not any(p.requires_grad for p in inf.parameters())
+
+
+def test_ternary_linear_to_infer_uses_the_layers_own_settings():
+    torch.manual_seed(2)
+    for per_channel in (True, False):
+        layer = TernaryLinear(48, 24, threshold_factor=0.1, per_channel=per_channel, backend="python")
+        inf = ternary_linear_to_infer(layer)
+        x = torch.randn(7, 48)
+        assert torch.allclose(inf(x), layer(x), atol=1e-5)
+        assert inf.scale.shape == (24,)
+    layer = TernaryLinear(8, 4, bias=False, backend="python")
+    assert ternary_linear_to_infer(layer).bias is None
+
+
+def test_convert_linear_layers_copy_skip_and_inplace():
+    model = _mlp()
+    x = torch.randn(3, 64)
+    conv = convert_linear_layers(model, skip_names=["4"])
+    assert isinstance(model[0], nn.Linear) and isinstance(model[2], TernaryLinear)  # original untouched
+    assert isinstance(conv[0], TernaryLinearInference) and isinstance(conv[2], TernaryLinearInference)
+    assert isinstance(conv[4], nn.Linear)
+    # the converted model equals the model whose first layer is quantized the same way
+    w_tern, scale = ternary_quantize(model[0].weight.data, threshold_factor=0.05)
+    h = torch.relu(x @ (w_tern * scale[:, None]).T + model[0].bias)
+    ref = model[4](torch.relu(model[2](h)))
+    assert torch.allclose(conv(x), ref, atol=1e-5)
+    same = convert_linear_layers(model, inplace=True)
+    assert same is model and all(isinstance(model[i], TernaryLinearInference) for i in (0, 2, 4))
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.attn = nn.ModuleDict({"q_proj": nn.Linear(8, 8), "proj": nn.Linear(8, 8)})
+            self.lm_head = nn.Linear(8, 20)
+
+    blk = convert_linear_layers(Block(), skip_names=["head"])
+    assert isinstance(blk.attn["q_proj"], TernaryLinearInference) and isinstance(blk.lm_head, nn.Linear)
+
+
+def test_counts_and_memory():
+    model = _mlp()
+    c = count_ternary_params(model)
+    assert c == {"fp32": 64 * 32 + 32 * 16 + 16 * 10, "fp16": 0, "packed_ternary": 0, "total": 64 * 32 + 32 * 16 + 160}
+    conv = convert_linear_layers(model, skip_names=["4"])
+    c = count_ternary_params(conv)
+    assert c["packed_ternary"] == 64 * 32 + 32 * 16 and c["fp32"] == 160 and c["total"] == 64 * 32 + 32 * 16 + 160
+    m = get_model_memory_bytes(conv)
+    assert m["packed_ternary"] == 16 * 32 + 8 * 16          # ceil(K/4) * N bytes
+    assert m["scales"] == 4 * (32 + 16) and m["fp32"] == 4 * 160
+    assert m["total"] == m["packed_ternary"] + m["scales"] + m["fp32"] + 4 * (32 + 16 + 10)
+    half = nn.Sequential(nn.Linear(8, 4).half())
+    assert count_ternary_params(half)["fp16"] == 32 and get_model_memory_bytes(half)["fp16"] == 64
+
+
+def test_checkpoint_round_trips(tmp_path):
+    conv = convert_linear_layers(_mlp())
+    x = torch.randn(4, 64)
+    y = conv(x)
+    path = str(tmp_path / "m.pt")
+    save_ternary_checkpoint(conv, path, metadata={"note": "unit test", "layers": 3})
+    torch.manual_seed(9)
+    fresh = convert_linear_layers(nn.Sequential(nn.Linear(64, 32), nn.ReLU(), nn.Linear(32, 16), nn.ReLU(),
+                                                nn.Linear(16, 10)))
+    assert not torch.equal(fresh(x), y)
+    meta = load_ternary_checkpoint(path, fresh)
+    assert meta == {"note": "unit test", "layers": 3}
+    assert torch.equal(fresh(x), y)
+    for k, v in conv.state_dict().items():
+        assert torch.equal(v, fresh.state_dict()[k]), k
+    assert sorted(conv.state_dict()) == ["0.bias", "0.scale", "0.weight_packed", "2.bias", "2.scale",
+                                         "2.weight_packed", "4.bias", "4.scale", "4.weight_packed"]
+
+    st = str(tmp_path / "m.safetensors")
+    save_ternary_safetensors(conv, st, metadata={"format": "bittorch"})
+    again = convert_linear_layers(nn.Sequential(nn.Linear(64, 32), nn.ReLU(), nn.Linear(32, 16), nn.ReLU(),
+                                                nn.Linear(16, 10)))
+    assert load_ternary_safetensors(st, again)["format"] == "bittorch"
+    assert torch.equal(again(x), y)
+    from safetensors import safe_open
+    with safe_open(st, framework="pt") as fh:
+        t = fh.get_tensor("0.weight_packed")
+        assert t.dtype == torch.uint8 and tuple(t.shape) == (16, 32)       # [inBytes, outFeatures]
+        assert fh.get_tensor("0.scale").dtype == torch.float32
+
+
+@pytest.mark.gpu
+def test_gpu_conversion_equals_cpu_conversion():
+    """On the GPU the fused quantize+pack kernel does the conversion: same bytes, same scales."""
+    from conftest import announce
+    announce("convert on gpu")
+    torch.manual_seed(3)
+    model = nn.Sequential(nn.Linear(256, 128), nn.ReLU(), TernaryLinear(128, 64, threshold_factor=0.08), nn.ReLU(),
+                          TernaryLinear(64, 32, per_channel=False))
+    cpu = convert_linear_layers(model)
+    gpu = convert_linear_layers(model.cuda())
+    for k, v in cpu.state_dict().items():
+        assert torch.equal(v, gpu.state_dict()[k].cpu()), k
+    x = torch.randn(9, 256)
+    assert torch.allclose(gpu(x.cuda()).cpu(), cpu(x), atol=1e-4, rtol=1e-4)
