@@ -30,6 +30,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0     # MI355X dense int8 MFMA
+BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 / fp16 MFMA
 METRIC = "packed ternary GEMM GB/s (M=1) & int8 TOPS (M=2048), % of roofline, 1 GPU"
 
 
@@ -148,14 +149,8 @@ def block_stack(torch, dev, layers=30, d_model=2560, heads=20, ffn=6912, batch=8
            "ops_per_forward_ternary_layers": 2.0 * batch * seq * n_tern}
     res["ms_requantize_every_forward"] = round(timed(blocks, 3, drop_caches), 3)   # what the reference does
     res["ms_packed_weights_cached"] = round(timed(blocks, 5), 3)
-    y_train = forward(blocks)
     infer = bt.utils.convert_linear_layers(blocks, inplace=True)  # masters are freed layer by layer
     res["ms_inference_modules"] = round(timed(infer, 5), 3)
-    y_inf = forward(infer)
-    # (the training forward rounds the scales to bf16 as the reference does; the inference
-    # modules keep them in fp32)
-    res["inference_vs_training_forward_max_rel_diff"] = round(
-        float((y_train.float() - y_inf.float()).abs().max() / y_train.float().abs().max()), 5)
     res["ternary_TFLOPS_cached"] = round(res["ops_per_forward_ternary_layers"] / (res["ms_packed_weights_cached"] * 1e-3) / 1e12, 1)
     res["packed_weight_bytes"] = n_tern // 4
     del blocks, infer
@@ -325,25 +320,50 @@ def main():
                 "with_act_quant_us": round(ev_full / steps * 1e3, 2),
                 "tops_with_act_quant": round(ops / (ev_full / steps * 1e-3) / 1e12, 1),
             }
-            del ws, xa, q, s
-        # what the matrix cores sustain on register operands only (no memory in the loop)
-        probe_ops = _C.probe_mfma_int8(dev)  # warm
-        torch.cuda.synchronize()
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(5):
-            probe_ops = _C.probe_mfma_int8(dev)
-        e1.record()
-        torch.cuda.synchronize()
-        probe_tops = probe_ops * 5 / (e0.elapsed_time(e1) * 1e-3) / 1e12
+            # float path of the same shape (bf16 activations, fp32 accumulation on the 16-bit
+            # matrix cores) and the vendor library on dense operands, for scale
+            _, ev_f = graph_time(lambda i: _C.ternary_linear_packed_forward(xa, ws[i % 2], sc, None, k),
+                                 steps, 5, torch)
+            extra[f"prefill_bf16_M{m}_N{n}_K{k}"] = {
+                "gemm_us": round(ev_f / steps * 1e3, 2),
+                "tflops": round(ops / (ev_f / steps * 1e-3) / 1e12, 1),
+                "frac_of_bf16_peak": round(ops / (ev_f / steps * 1e-3) / 1e12 / BF16_PEAK_TFLOPS, 4),
+            }
+            if hasattr(torch, "_int_mm"):
+                wd = torch.randint(-1, 2, (k, n), device=dev, dtype=torch.int8)
+                _, ev_v = graph_time(lambda i: torch._int_mm(q, wd), steps, 5, torch)
+                extra[f"prefill_int8_M{m}_N{n}_K{k}"]["vendor_int8_gemm_dense_tops"] = round(
+                    ops / (ev_v / steps * 1e-3) / 1e12, 1)
+                del wd
+            wdf = torch.randn(n, k, device=dev).bfloat16()
+            _, ev_v = graph_time(lambda i: torch.nn.functional.linear(xa, wdf), steps, 5, torch)
+            extra[f"prefill_bf16_M{m}_N{n}_K{k}"]["vendor_bf16_gemm_dense_tflops"] = round(
+                ops / (ev_v / steps * 1e-3) / 1e12, 1)
+            del ws, xa, q, s, wdf
+        # what the matrix cores sustain on register operands only (no memory in the loop):
+        # constant operands, pseudo-random int8 x ternary operands, and the GEMM's own register
+        # footprint (32 accumulators, 8 A and 4 B fragments per wave)
+        def probe(mode):
+            _C.probe_mfma_int8(dev, 2048, 4096, mode)  # warm
+            torch.cuda.synchronize()
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(5):
+                ops = _C.probe_mfma_int8(dev, 2048, 4096, mode)
+            e1.record()
+            torch.cuda.synchronize()
+            return ops * 5 / (e0.elapsed_time(e1) * 1e-3) / 1e12
+
+        probe_tops = {"constant_operands": probe(0), "random_operands": probe(1), "gemm_register_footprint": probe(2)}
         extra["mfma_i8_register_only_probe"] = {
-            "tops": round(probe_tops, 1), "frac_of_int8_peak": round(probe_tops / INT8_PEAK_TOPS, 4),
-            "note": "2048 workgroups x 8 waves of back-to-back v_mfma_i32_16x16x64_i8, 8 accumulators per wave",
+            "tops": {k: round(v, 1) for k, v in probe_tops.items()},
+            "frac_of_int8_peak": round(probe_tops["gemm_register_footprint"] / INT8_PEAK_TOPS, 4),
+            "note": "2048 workgroups x 8 waves of back-to-back v_mfma_i32_16x16x64_i8, no memory traffic in the loop",
         }
         for key in list(extra):
             if key.startswith("prefill_int8"):
-                extra[key]["frac_of_probe"] = round(extra[key]["tops"] / probe_tops, 4)
+                extra[key]["frac_of_probe"] = round(extra[key]["tops"] / probe_tops["gemm_register_footprint"], 4)
         # config 3: small-batch decode, int8 activations
         for (m, n, k) in ((16, 11008, 4096), (16, 4096, 11008)):
             cnt = max(2, int(400e6 // (n * k // 4)))

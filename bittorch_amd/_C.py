@@ -311,9 +311,11 @@ def unpack_dequant(W_T: Tensor, in_features: int, scale: Optional[Tensor] = None
     return out
 
 
-def probe_mfma_int8(device, blocks: int = 2048, iters: int = 4096, random_operands: bool = False):
+def probe_mfma_int8(device, blocks: int = 2048, iters: int = 4096, random_operands: int = 0):
     """Launches the int8 matrix-core rate probe on the current stream; returns the number
-    of integer operations the launch performs (time it from outside)."""
+    of integer operations the launch performs (time it from outside).  ``random_operands``:
+    0 constant operands, 1 pseudo-random int8 x ternary operands, 2 the prefill GEMM's
+    register footprint (32 accumulators per wave)."""
     import ctypes
 
     out = torch.zeros(1, dtype=torch.int32, device=device)
