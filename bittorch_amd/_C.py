@@ -50,17 +50,13 @@ def _dt(t: Tensor, what: str) -> int:
         raise RuntimeError(f"{what} must be float32, float16 or bfloat16, got {t.dtype}") from None
 
 
-_COUNTER_BYTES = 16384  # BT_WORKSPACE_COUNTER_BYTES: must be zero on entry, is zero on exit
 _ws_cache = {}
 
 
 def _workspace(nbytes: int, device) -> Optional[Tensor]:
-    """Scratch buffer for the current stream of ``device``, kept between calls.
-
-    The library needs the head of the buffer zeroed once and restores the zeros
-    itself, so the buffer is cleared when it is (re)allocated and then reused.
-    One buffer per (device, stream): calls on one stream run in order.
-    """
+    """Scratch buffer for the current stream of ``device``, kept between calls (the library
+    needs no initialisation of it).  One buffer per (device, stream): calls on one stream
+    run in order."""
     if nbytes <= 0:
         return None
     key = (device.index if device.index is not None else torch.cuda.current_device(),
@@ -69,7 +65,6 @@ def _workspace(nbytes: int, device) -> Optional[Tensor]:
     if buf is None or buf.numel() < nbytes:
         size = max(nbytes, 1 << 20)
         buf = torch.empty(size, dtype=torch.uint8, device=device)
-        buf[:_COUNTER_BYTES].zero_()
         _ws_cache[key] = buf
     return buf
 

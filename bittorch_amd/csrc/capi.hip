@@ -208,7 +208,7 @@ extern "C" int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8
 
 extern "C" size_t bt_tensor_core_workspace_bytes(int64_t B, int64_t N, int64_t K) {
     if (B <= 0 || N <= 0 || K <= 0) return 0;
-    // [GEMM scratch (ticket counters first)] [Q int8 B*K] [s_x fp32 B]
+    // [GEMM scratch (none at present)] [Q int8 B*K] [s_x fp32 B]
     return align256(bt_gemm_i8_workspace_bytes(B, N, K)) + align256((size_t)B * K) + align256((size_t)B * 4);
 }
 

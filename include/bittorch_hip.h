@@ -38,15 +38,17 @@ typedef enum {
 } bt_status;
 
 /*
- * Workspaces.  Entry points that take a `workspace` use it for split-K partial
- * sums and for per-tile ticket counters.  The first BT_WORKSPACE_COUNTER_BYTES
- * bytes of a workspace must be ZERO when a call starts; every call leaves them
- * zero again when its kernels have run, so a buffer that was cleared once can
- * be reused for any sequence of calls on one stream.  The rest of the buffer
- * needs no initialisation.  Two calls that may run concurrently (different
+ * Workspaces.  The library allocates nothing: an entry point that needs device
+ * scratch takes a caller-provided `workspace` of at least the number of bytes its
+ * *_workspace_bytes() query returns for the same shape (0 means none is needed and
+ * NULL may be passed).  A workspace needs no initialisation and carries nothing
+ * from one call to the next; two calls that may run concurrently (different
  * streams) need different workspaces.  Workspaces must be 256-byte aligned.
+ * At present only bt_ternary_linear_tensor_core_forward uses one (the int8
+ * activations and their row scales); the GEMM entry points keep the argument so
+ * that a kernel that needs scratch can be introduced without an ABI change.
  */
-#define BT_WORKSPACE_COUNTER_BYTES 16384
+#define BT_WORKSPACE_COUNTER_BYTES 16384 /* kept for callers that clear the head of a workspace; unused */
 
 /* ABI version of the loaded library (BT_ABI_VERSION at build time). */
 int bt_abi_version(void);
@@ -89,8 +91,11 @@ int bt_ternary_linear_forward(const void* X, int x_dtype, const int8_t* W_tern, 
  * Replaces bittorch._C.ternary_linear_packed_forward (bittorch_bindings.cpp:48-63,
  * dispatch.cpp:105-142, csrc/kernels/ternary_gemm_production.cu:286-362).
  *   X [B,K] x_dtype; W_T [ceil(K/4),N] uint8; Y [B,N] x_dtype.
- *   workspace: scratch for split-K partial sums, at least
- *   bt_packed_forward_workspace_bytes(B,N,K,x_dtype) bytes (may be NULL if that is 0).
+ *   Batches up to 32 rows stream the weights once per 16 rows (decode shape); taller
+ *   fp16 / bf16 batches run the tiled 16-bit matrix-core GEMM; fp32 activations and
+ *   unaligned operands run a generic kernel that accumulates in the reference's k order.
+ *   workspace: at least bt_packed_forward_workspace_bytes(B,N,K,x_dtype) bytes
+ *   (currently 0: may be NULL).
  */
 size_t bt_packed_forward_workspace_bytes(int64_t B, int64_t N, int64_t K, int x_dtype);
 int bt_ternary_linear_packed_forward(const void* X, int x_dtype, const uint8_t* W_T,
@@ -116,7 +121,7 @@ int bt_act_quant_i8(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q,
  *   y = (float(acc) * s_x[b] / 127.0f) * scale[n] + bias[n].
  *   Q [B,K] int8, s_x [B] fp32, W_T [ceil(K/4),N] uint8, Y [B,N] y_dtype.
  *   acc_out: optional [B,N] int32 copy of the raw accumulators (may be NULL).
- *   workspace: at least bt_gemm_i8_workspace_bytes(B,N,K) bytes.
+ *   workspace: at least bt_gemm_i8_workspace_bytes(B,N,K) bytes (currently 0: may be NULL).
  */
 size_t bt_gemm_i8_workspace_bytes(int64_t B, int64_t N, int64_t K);
 int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const void* scale,
@@ -130,8 +135,7 @@ int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, co
  * (bittorch_bindings.cpp:65-87, ternary_gemm_tensor_core.cu:663-727) for
  * version == 2; version == 1 (the reference's float-compute validation kernel,
  * :120-271) is served by bt_ternary_linear_packed_forward.
- *   workspace: at least bt_tensor_core_workspace_bytes(B,N,K) bytes; holds the GEMM's
- *   own scratch (ticket counters first), then Q and s_x.
+ *   workspace: at least bt_tensor_core_workspace_bytes(B,N,K) bytes; holds Q and s_x.
  */
 size_t bt_tensor_core_workspace_bytes(int64_t B, int64_t N, int64_t K);
 int bt_ternary_linear_tensor_core_forward(const void* X, int x_dtype, const uint8_t* W_T,
