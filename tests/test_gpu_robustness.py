@@ -1,0 +1,147 @@
+"""GPU robustness of the module path on the HIP kernels: the edge cases the reference pins in
+tests/test_robustness.py:160-260, :284-400 and tests/test_kernel_regression.py:37-190 (zero,
+tiny and huge inputs, constant weights, masked outputs in backward, batched == looped,
+big shapes, multi-step training, kernel selection by BITTORCH_KERNEL)."""
+import os
+
+import pytest
+import torch
+
+from conftest import announce
+
+pytestmark = pytest.mark.gpu
+
+
+def _layer(i, o, **kw):
+    from bittorch_amd.nn import TernaryLinear
+    torch.manual_seed(0)
+    return TernaryLinear(i, o, backend="cuda", **kw).cuda()
+
+
+def test_zero_tiny_and_huge_inputs():
+    announce("robustness inputs")
+    for dtype in (torch.float32, torch.float16, torch.bfloat16):
+        layer = _layer(32, 16).to(dtype)
+        y = layer(torch.zeros(4, 32, device="cuda", dtype=dtype))
+        assert torch.equal(y, layer.bias.detach().unsqueeze(0).expand(4, -1))
+        for mag in (1e-7, 1e3):
+            y = layer((torch.randn(4, 32, device="cuda") * mag).to(dtype))
+            assert torch.isfinite(y).all()
+    layer = _layer(32, 16)
+    y = layer(torch.randn(4, 32, device="cuda") * 1e4)
+    assert torch.isfinite(y).all()
+
+
+def test_constant_and_signed_weights():
+    announce("robustness weights")
+    layer = _layer(32, 16, threshold_factor=0.05)
+    with torch.no_grad():
+        layer.weight.fill_(0.05)            # every weight equals its row maximum -> all +1
+    x = torch.randn(4, 32, device="cuda")
+    y = layer(x)
+    ref = x.sum(dim=1, keepdim=True) * 0.05 + layer.bias
+    assert torch.allclose(y, ref, atol=1e-5)
+    with torch.no_grad():
+        layer.weight[:8] = layer.weight[:8].abs() * 2 + 0.1
+        layer.weight[8:] = -(layer.weight[8:].abs() * 2 + 0.1)
+    w_tern, _ = layer.get_quantized_weight()
+    assert (w_tern[:8] == 1).all() and (w_tern[8:] == -1).all()
+    assert torch.isfinite(layer(x)).all()
+    with torch.no_grad():
+        layer.weight.zero_()                 # all-zero rows: scale floor, codes 0, output = bias
+    assert torch.equal(layer(x), layer.bias.detach().unsqueeze(0).expand(4, -1))
+
+
+def test_backward_through_masked_outputs_and_noncontiguous_inputs():
+    announce("robustness backward")
+    layer = _layer(32, 16)
+    x = torch.randn(4, 32, device="cuda", requires_grad=True)
+    mask = torch.tensor([1, 0] * 8, device="cuda").float()
+    (layer(x) * mask).sum().backward()
+    assert torch.isfinite(x.grad).all() and torch.isfinite(layer.weight.grad).all()
+    assert layer.bias.grad.tolist() == [4.0, 0.0] * 8
+    # non-contiguous and 3-D inputs take the same path as their contiguous copies
+    big = torch.randn(6, 5, 64, device="cuda")
+    xs = big[:, :, ::2]
+    assert not xs.is_contiguous()
+    with torch.no_grad():
+        assert torch.equal(layer(xs), layer(xs.contiguous()))
+        assert layer(xs).shape == (6, 5, 16)
+
+
+def test_batched_equals_looped_all_kernels():
+    """Rows are independent in every kernel: one row at a time (streaming kernel), 48 rows
+    (tiled kernel for 16-bit inputs) and the generic fp32 kernel give the same rows."""
+    announce("robustness batched vs looped")
+    for dtype, tol in ((torch.float32, 0.0), (torch.float16, 2e-3), (torch.bfloat16, 2e-2)):
+        layer = _layer(256, 128).to(dtype)
+        x = torch.randn(48, 256, device="cuda").to(dtype)
+        with torch.no_grad():
+            yb = layer(x)
+            yl = torch.cat([layer(x[i:i + 1]) for i in range(48)])
+        if tol == 0.0:
+            assert torch.equal(yb, yl)
+        else:  # different kernels sum in a different order; outputs are rounded to 16 bits
+            assert (yb.float() - yl.float()).abs().max() <= tol * yl.float().abs().max()
+
+
+@pytest.mark.parametrize("shape", [(8, 4096, 4096), (512, 1024, 4096), (64, 11008, 4096)])
+def test_big_shape_forward_backward(shape):
+    b, i, o = shape
+    announce("robustness big", shape)
+    layer = _layer(i, o)
+    x = torch.randn(b, i, device="cuda", requires_grad=True)
+    y = layer(x)
+    assert y.shape == (b, o) and torch.isfinite(y).all()
+    y.float().pow(2).mean().backward()
+    assert torch.isfinite(x.grad).all() and torch.isfinite(layer.weight.grad).all()
+    # forward equals the plain torch backend of the same layer
+    layer.backend = "python"
+    with torch.no_grad():
+        ref = layer(x.detach())
+    assert (y.detach() - ref).abs().max() <= 1e-3 * ref.abs().max()
+
+
+def test_multi_step_training_is_stable():
+    announce("robustness training")
+    torch.manual_seed(0)
+    from bittorch_amd.nn import TernaryLinear
+    model = torch.nn.Sequential(TernaryLinear(64, 128), torch.nn.ReLU(), TernaryLinear(128, 10)).cuda()
+    opt = torch.optim.Adam(model.parameters(), lr=1e-2)
+    x = torch.randn(256, 64, device="cuda")
+    target = (x[:, :10] > 0).float()
+    first = None
+    for step in range(60):
+        loss = torch.nn.functional.binary_cross_entropy_with_logits(model(x), target)
+        opt.zero_grad()
+        loss.backward()
+        opt.step()
+        assert torch.isfinite(loss)
+        first = first if first is not None else float(loss.detach())
+    assert float(loss.detach()) < 0.7 * first
+
+
+def test_kernel_selection_env_matches_default():
+    """BITTORCH_KERNEL is read on every call (tests/test_kernel_regression.py:17-34 flips it at run
+    time): the generic kernel and the default dispatch agree."""
+    from bittorch_amd import _C
+    from bittorch_amd.quant import pack_ternary_transposed
+    announce("robustness kernel env")
+    g = torch.Generator().manual_seed(4)
+    old = os.environ.get("BITTORCH_KERNEL")
+    try:
+        for (b, n, k) in ((1, 64, 64), (7, 100, 36), (32, 512, 256), (128, 256, 1024)):
+            w = torch.randint(-1, 2, (n, k), generator=g).float()
+            packed = pack_ternary_transposed(w)[0].cuda()
+            scale = (torch.rand(n, generator=g) + 0.5).half().cuda()
+            x = torch.randn(b, k, generator=g).half().cuda()
+            os.environ["BITTORCH_KERNEL"] = "generic"
+            y_gen = _C.ternary_linear_packed_forward(x, packed, scale, None, k)
+            os.environ["BITTORCH_KERNEL"] = "auto"
+            y_def = _C.ternary_linear_packed_forward(x, packed, scale, None, k)
+            assert (y_gen.float() - y_def.float()).abs().max() <= 1e-2 * y_gen.float().abs().max()
+    finally:
+        if old is None:
+            os.environ.pop("BITTORCH_KERNEL", None)
+        else:
+            os.environ["BITTORCH_KERNEL"] = old
