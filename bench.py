@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-One "step" is one pass of the decode GEMV of BASELINE.json's config 2 through the
+One "step" is one pass of the decode GEMV (the benchmark's config 2) through the
 C-ABI library: x fp16 [1,4096] times packed ternary W [4096,4096] (per-tensor fp32
 scale, fp16 bias).  The steps walk round-robin over distinct weight buffers whose
 total size exceeds the 256 MB Infinity Cache, so every step streams its 4 MiB of

@@ -180,7 +180,7 @@ def test_inference_module_matches_dense_formula():
 
 
 def test_config1_plumbing_cpu(oracle):
-    """BASELINE config 1 on the plain torch backend: TernaryLinear(512->256), batch 32, fp32,
+    """Benchmark config 1 on the plain torch backend: TernaryLinear(512->256), batch 32, fp32,
     N(0,0.02) masters, seed 0 -- quantize / pack / forward agree with the oracle."""
     g = torch.Generator().manual_seed(0)
     layer = TernaryLinear(512, 256, bias=True, threshold_factor=0.05, backend="python")
