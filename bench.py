@@ -364,6 +364,39 @@ def main():
         for key in list(extra):
             if key.startswith("prefill_int8"):
                 extra[key]["frac_of_probe"] = round(extra[key]["tops"] / probe_tops["gemm_register_footprint"], 4)
+        # config 2 again with independent launches in flight: the same kernel on 1, 2, 4 and 8 branches
+        # of one HIP graph (each branch its own chain of launches over its own weight sets).  A single
+        # chain pays a launch gap and a full memory round trip per 4 MiB; with branches the chip's
+        # bandwidth, not the latency of one launch, sets the rate.  Not the headline figure: a decode
+        # step of one sequence is a single chain.
+        def branches_time(nb, per_branch=250):
+            streams = [torch.cuda.Stream() for _ in range(nb)]
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                main = torch.cuda.current_stream()
+                for bi, st in enumerate(streams):
+                    st.wait_stream(main)
+                    with torch.cuda.stream(st):
+                        for i in range(per_branch):
+                            _C.ternary_linear_packed_forward(x, packs[(bi * per_branch + i) % nsets], scale, bias, K)
+                for st in streams:
+                    main.wait_stream(st)
+            graph.replay()
+            torch.cuda.synchronize()
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e-3 / (nb * per_branch)
+
+        conc = {}
+        for nb in (1, 2, 4, 8):
+            t = branches_time(nb)
+            conc[f"{nb}_branches"] = {"us_per_launch": round(t * 1e6, 3), "GBps": round(weight_bytes / t / 1e9, 1),
+                                      "frac_of_hbm_peak": round(weight_bytes / t / 1e9 / HBM_PEAK_GBPS, 4)}
+        extra["decode_gemv_independent_launches_in_flight"] = conc
         # config 3: small-batch decode, int8 activations
         for (m, n, k) in ((16, 11008, 4096), (16, 4096, 11008)):
             cnt = max(2, int(400e6 // (n * k // 4)))
