@@ -32,7 +32,8 @@ bool stream_supported(int64_t N, int64_t K, const void* W_T);
 size_t stream_workspace_bytes(int mode, int64_t M, int64_t N, int64_t Kb);
 int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, const uint8_t* W_T,
                   const Epilogue& epi, void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N,
-                  int64_t K, void* workspace, size_t ws_bytes, hipStream_t st);
+                  int64_t K, int planes, hipStream_t st);
+int launch_split_f32_planes(const void* X, int64_t B, int64_t K, void* P, hipStream_t st);
 int launch_packed_generic(const void* X, int x_dtype, const uint8_t* W_T, const Epilogue& epi, void* Y,
                           int64_t B, int64_t N, int64_t K, hipStream_t st);
 int launch_unpacked(const void* X, int x_dtype, const int8_t* W, const Epilogue& epi, void* Y, int64_t B,
@@ -41,7 +42,7 @@ int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q
 bool gemm_i8_supported(int64_t N, int64_t K, const void* Q, const void* W_T);
 bool gemm_f16_supported(int64_t N, int64_t K, const void* X, const void* W_T, const void* Y);
 int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, const Epilogue& epi, void* Y, int y_dtype, int64_t M,
-                    int64_t N, int64_t K, hipStream_t st);
+                    int64_t N, int64_t K, int planes, hipStream_t st);
 int launch_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const Epilogue& epi, void* Y,
                    int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st);
 
@@ -121,13 +122,27 @@ extern "C" int bt_ternary_linear_forward(const void* X, int x_dtype, const int8_
     return launch_unpacked(X, x_dtype, W_tern, epi, Y, B, N, K, (hipStream_t)stream);
 }
 
+static bool generic_forced() {
+    const char* env = getenv("BITTORCH_KERNEL");
+    return env && !strcmp(env, "generic");
+}
+
 static bool packed_uses_stream(int x_dtype, const void* W_T, const void* Y, int64_t N, int64_t K) {
-    if (getenv("BITTORCH_KERNEL") && !strcmp(getenv("BITTORCH_KERNEL"), "generic")) return false;
+    if (generic_forced()) return false;
     return x_dtype != BT_F32 && stream_supported(N, K, W_T) && fast_path_ok(Y, N, K);
 }
 
+// fp32 activations run on the bf16 matrix-core kernels as three exact bf16 planes (hi, mid, lo)
+// when K is a multiple of the kernels' 64-wide step; the planes live in the workspace.
+static size_t f32_planes_bytes(int64_t B, int64_t K) { return align256((size_t)B * 3 * K * 2); }
+static bool packed_uses_f32_planes(const void* X, const void* W_T, const void* Y, int64_t N, int64_t K) {
+    if (generic_forced()) return false;
+    return K % 64 == 0 && ((uintptr_t)X) % 16 == 0 && stream_supported(N, 3 * K, W_T) && fast_path_ok(Y, N, 3 * K);
+}
+
 extern "C" size_t bt_packed_forward_workspace_bytes(int64_t B, int64_t N, int64_t K, int x_dtype) {
-    if (B <= 0 || N <= 0 || K <= 0 || x_dtype == BT_F32) return 0;
+    if (B <= 0 || N <= 0 || K <= 0) return 0;
+    if (x_dtype == BT_F32) return (K % 64 == 0) ? f32_planes_bytes(B, K) : 0;
     return stream_workspace_bytes(x_dtype == BT_F16 ? MODE_F16 : MODE_BF16, B, N, ceil_div(K, 4));
 }
 
@@ -147,9 +162,17 @@ extern "C" int bt_ternary_linear_packed_forward(const void* X, int x_dtype, cons
         const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
         // tall batches go to the tiled matrix-core kernel, decode shapes stream the weights
         if (B > kStreamMaxRows && gemm_f16_supported(N, K, X, W_T, Y))
-            return launch_gemm_f16(mode, X, W_T, epi, Y, x_dtype, B, N, K, st);
-        return launch_stream(mode, X, 2, nullptr, W_T, epi, Y, x_dtype, nullptr, B, N, K, workspace,
-                             workspace_bytes, st);
+            return launch_gemm_f16(mode, X, W_T, epi, Y, x_dtype, B, N, K, 1, st);
+        return launch_stream(mode, X, 2, nullptr, W_T, epi, Y, x_dtype, nullptr, B, N, K, 1, st);
+    }
+    if (x_dtype == BT_F32 && packed_uses_f32_planes(X, W_T, Y, N, K) && workspace &&
+        workspace_bytes >= f32_planes_bytes(B, K) && ((uintptr_t)workspace) % 256 == 0) {
+        // (without a workspace the call still succeeds, on the generic kernel)
+        rc = launch_split_f32_planes(X, B, K, workspace, st);
+        if (rc) return rc;
+        if (B > kStreamMaxRows && gemm_f16_supported(N, 3 * K, workspace, W_T, Y))
+            return launch_gemm_f16(MODE_BF16, workspace, W_T, epi, Y, BT_F32, B, N, K, 3, st);
+        return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, epi, Y, BT_F32, nullptr, B, N, K, 3, st);
     }
     return launch_packed_generic(X, x_dtype, W_T, epi, Y, B, N, K, st);
 }
@@ -200,8 +223,7 @@ extern "C" int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8
                       (long long)ceil_div(K, 4), (long long)N);
             return BT_ERR_INVALID;
         }
-        return launch_stream(MODE_I8, Q, 1, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, workspace,
-                             workspace_bytes, st);
+        return launch_stream(MODE_I8, Q, 1, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, 1, st);
     }
     return launch_gemm_i8(Q, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, st);
 }

@@ -35,7 +35,9 @@ struct GemmFParams {
     const uint8_t* W_T;   // [Kb, N]
     void* Y;              // [M, N]
     Epilogue epi;
-    int64_t M, N, K, Kb;
+    int64_t M, N, K, Kb;  // K: length of an activation row; Kb: packed weight rows
+    int wstages;          // 64-wide stages of W_T; a stage index beyond it wraps (see launch_gemm_f16)
+    int prehalved;        // MODE_BF16: the activations already carry the factor 1/2 of the +-2.0 weight decode
     int y_dtype;
     int tiles_m, tiles_n;
     int per_xcd;          // workgroups per XCD (grid = 8 * per_xcd)
@@ -75,7 +77,7 @@ __device__ __forceinline__ void gemm_f_epilogue(const GemmFParams& p, const v4f 
 #pragma unroll
             for (int t = 0; t < 4; t++) {
                 float a = acc[MB0 + mbi][t][r];
-                if constexpr (MODE == MODE_BF16) a *= 0.5f;  // weights were decoded as +-2.0
+                if constexpr (MODE == MODE_BF16) a *= (p.prehalved ? 1.0f : 0.5f);  // weights were decoded as +-2.0
                 y[t] = epi_float(a, ws[t], bs[t]);
             }
             store4f(p.Y, YDT, m * p.N + ncol, y);
@@ -143,14 +145,19 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     uint32_t b_set[2][2];
 
     // part: 1 = activations, 2 = weights, 3 = both
-    auto load_full = [&](int64_t k0, int part, uint4 (&a_reg)[2], uint32_t (&b_reg)[2]) {
+    auto load_full = [&](int st, int part, uint4 (&a_reg)[2], uint32_t (&b_reg)[2]) {
         if (part & 1) {
-            const uint8_t* ab = a_base + 2 * k0;
+            const uint8_t* ab = a_base + 2 * (int64_t)st * F_BK;
             a_reg[0] = *(const uint4*)(ab + a_off);
             a_reg[1] = *(const uint4*)(ab + 16 + a_off);
         }
         if (part & 2) {
-            const uint8_t* bb = b_base + (k0 >> 2) * N;
+            // the activation row may hold several planes of K values, all multiplied with the
+            // same weights: the weight stage wraps (uniform)
+            int ws = st;
+            if (ws >= p.wstages) ws -= p.wstages;
+            if (ws >= p.wstages) ws -= p.wstages;
+            const uint8_t* bb = b_base + (int64_t)ws * (F_BK / 4) * N;
             b_reg[0] = *(const uint32_t*)(bb + b_off);
             b_reg[1] = *(const uint32_t*)(bb + N + b_off);
         }
@@ -179,11 +186,11 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     auto load_stage = [&](int st, int part, uint4 (&a_reg)[2], uint32_t (&b_reg)[2]) {  // st, part uniform
         if constexpr (TAIL) {
             if (st >= nstages) st = nstages - 1;
-            if (st < nfull) load_full((int64_t)st * F_BK, part, a_reg, b_reg);
+            if (st < nfull) load_full(st, part, a_reg, b_reg);
             else load_tail((int64_t)st * F_BK, part, a_reg, b_reg);
         } else {
             // past the end: reload the last stage (never consumed) instead of branching
-            load_full((int64_t)(st < nstages ? st : nstages - 1) * F_BK, part, a_reg, b_reg);
+            load_full(st < nstages ? st : nstages - 1, part, a_reg, b_reg);
         }
     };
     auto store_a = [&](int buf, const uint4 (&a_reg)[2]) {
@@ -320,18 +327,22 @@ bool gemm_f16_supported(int64_t N, int64_t K, const void* X, const void* W_T, co
            ((uintptr_t)Y) % 16 == 0 && (F_BM + 1) * K * 2 < (1ll << 32) && ceil_div(K, 4) * N < (1ll << 32);
 }
 
+// planes = 1: X is [M, K].  planes = 3 (K % 64 == 0): X is [M, 3K], three planes of K values per
+// row whose products with the same weights are summed (fp32 activations split into three bf16 terms).
 int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, const Epilogue& epi, void* Y, int y_dtype, int64_t M,
-                    int64_t N, int64_t K, hipStream_t st) {
+                    int64_t N, int64_t K, int planes, hipStream_t st) {
     GemmFParams p;
     p.X = (const uint16_t*)X; p.W_T = W_T; p.Y = Y; p.epi = epi;
-    p.M = M; p.N = N; p.K = K; p.Kb = ceil_div(K, 4);
+    p.M = M; p.N = N; p.K = K * planes; p.Kb = ceil_div(K, 4);
+    p.wstages = (int)ceil_div(K, F_BK);
+    p.prehalved = planes == 3;
     p.y_dtype = y_dtype;
     p.tiles_m = (int)ceil_div(M, F_BM);
     p.tiles_n = (int)ceil_div(N, F_BN);
     const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
     p.per_xcd = (int)ceil_div(total, 8);
     const dim3 grid((unsigned)(p.per_xcd * 8)), block(512);
-    const bool tail = K % F_BK != 0;
+    const bool tail = p.K % F_BK != 0;
     if (mode == MODE_F16) {
         if (tail) hipLaunchKernelGGL((gemm_f16_kernel<MODE_F16, true>), grid, block, 0, st, p);
         else hipLaunchKernelGGL((gemm_f16_kernel<MODE_F16, false>), grid, block, 0, st, p);

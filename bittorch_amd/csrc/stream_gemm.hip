@@ -45,12 +45,14 @@ struct StreamParams {
     void* Y;              // [M, N] of y_dtype
     int32_t* acc_out;     // MODE_I8, optional raw accumulators [M, N]
     Epilogue epi;
-    int64_t N, K, Kb;
+    int64_t N, K, Kb;     // K: length of an activation row; Kb: packed weight rows
+    int wsteps;           // 16-row steps of W_T; a step index beyond it wraps (see launch_stream)
     int tiles;            // column tiles
     int per_xcd;          // tiles per XCD (grid = 8 * per_xcd)
     int M;                // 1..16
     int y_dtype;
     int x_vec_ok;         // activation rows may be read with 16-byte loads
+    int prehalved;        // MODE_BF16: the activations already carry the factor 1/2 of the +-2.0 weight decode
 };
 
 enum { LD_BYTE = 0, LD_Q1 = 1, LD_Q2 = 2, LD_V4 = 4, LD_V8 = 8, LD_V16 = 16 };
@@ -79,7 +81,7 @@ __device__ __forceinline__ void finish_output(const StreamParams& p, int row, in
         y = epi_float(__builtin_bit_cast(float, bits), s, b);
     } else {
         // bf16 weights were decoded as +-2.0 (low byte zero): undo exactly
-        y = epi_float(__builtin_bit_cast(float, bits) * 0.5f, s, b);
+        y = epi_float(__builtin_bit_cast(float, bits) * (p.prehalved ? 1.0f : 0.5f), s, b);
     }
     store_out(p.Y, p.y_dtype, (int64_t)row * p.N + n, y);
 }
@@ -164,7 +166,7 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
     const int g = lane >> 4;
     const int q = lane & 3;
     const int64_t nb = (int64_t)tile * TILE_N;
-    const int nsteps = (int)((p.Kb + 15) >> 4);
+    const int nsteps = (int)((p.K + 63) >> 6);
     const int spw = (nsteps + WAVES - 1) / WAVES;  // steps per wave, contiguous
     const int s_begin = wave * spw;
     const int s_end = min(nsteps, s_begin + spw);
@@ -186,7 +188,8 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
         const int64_t c = nb + (int64_t)NACC * j;
         coloff[0] = (c < p.N) ? (uint32_t)c : 0u;
     }
-    uint32_t rowoff = (uint32_t)(s_begin * 16 + 4 * g + (QUAD ? q : 0)) * N32;
+    const uint32_t lane_rowoff = (uint32_t)(4 * g + (QUAD ? q : 0)) * N32;
+    const uint32_t step_rows = 16u * N32;
     int k0 = s_begin * 64 + 16 * g;  // first k of this lane's fragment in step s_begin
     const uint32_t xrow = (uint32_t)min(j, p.M - 1) * (uint32_t)p.K;
     const uint32_t sel_q = 0x0C0C0000u | ((uint32_t)(4 + q) << 8) | (uint32_t)q;
@@ -225,12 +228,17 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
 #pragma unroll
     for (int t = 0; t < NACC2; t++) acc2[t] = acc_t{0, 0, 0, 0};
 
-    for (int base = s_begin; base < s_end; base += PF, rowoff += PF * 16 * N32, k0 += PF * 64) {
+    for (int base = s_begin; base < s_end; base += PF, k0 += PF * 64) {
         uint32_t raw[PF][RAWN];
         uint4 xa[PF][XN];
 #pragma unroll
         for (int f = 0; f < PF; f++) {
-            const uint32_t ro = rowoff + (uint32_t)(f * 16) * N32;
+            // weight step of activation step base+f (uniform): the activation row may hold several
+            // planes of K values each, all multiplied with the same weights
+            int ws = base + f;
+            if (ws >= p.wsteps) ws -= p.wsteps;
+            if (ws >= p.wsteps) ws -= p.wsteps;
+            const uint32_t ro = lane_rowoff + (uint32_t)ws * step_rows;
             if constexpr (BYTE) {
 #pragma unroll
                 for (int r = 0; r < 4; r++)
@@ -461,7 +469,7 @@ static int launch_stream_mode(StreamParams p, const StreamPlan& pl, hipStream_t 
     // x slice in LDS: one row, aligned, at most XC_MAX 16-byte chunks per lane and wave, and
     // within the default 64 KiB of dynamic LDS
     const int es = (MODE == MODE_I8) ? 1 : 2;
-    const int64_t spw = ceil_div(ceil_div(p.Kb, 16), waves);
+    const int64_t spw = ceil_div(ceil_div(p.K, 64), waves);
     const size_t red_bytes = (size_t)waves * p.M * tile_n * 4;
     const size_t xs_bytes = (size_t)waves * XC_MAX * 64 * 16;
     const bool xlds = p.M == 1 && p.x_vec_ok && pl.ld <= 4 && spw * 64 * es <= XC_MAX * 64 * 16 &&
@@ -479,26 +487,30 @@ static int launch_stream_mode(StreamParams p, const StreamPlan& pl, hipStream_t 
 }
 
 // One launch per block of up to 16 activation rows.
+// planes = 1: X is [B, K].  planes = 3 (K % 64 == 0): X is [B, 3K], three planes of K values per
+// row whose products with the same weights are summed (fp32 activations split into three bf16
+// terms); the kernel walks 3K values of k and wraps its weight row index every K.
 int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, const uint8_t* W_T,
                   const Epilogue& epi, void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N,
-                  int64_t K, void* workspace, size_t ws_bytes, hipStream_t st) {
-    (void)workspace;
-    (void)ws_bytes;
+                  int64_t K, int planes, hipStream_t st) {
     const int64_t Kb = ceil_div(K, 4);
+    const int64_t Kx = K * planes;
     const StreamPlan pl = stream_plan(mode, B, N, Kb);
     const int y_size = dtype_size(y_dtype);
     for (int64_t m0 = 0; m0 < B; m0 += 16) {
         StreamParams p;
-        p.X = (const uint8_t*)X + m0 * K * x_elem_size;
+        p.X = (const uint8_t*)X + m0 * Kx * x_elem_size;
         p.W_T = W_T;
         p.s_x = s_x ? s_x + m0 : nullptr;
         p.Y = (uint8_t*)Y + m0 * N * y_size;
         p.acc_out = acc_out ? acc_out + m0 * N : nullptr;
         p.epi = epi;
-        p.N = N; p.K = K; p.Kb = Kb;
+        p.N = N; p.K = Kx; p.Kb = Kb;
+        p.wsteps = (int)ceil_div(Kb, 16);
+        p.prehalved = planes == 3;
         p.M = (int)((B - m0 < 16) ? (B - m0) : 16);
         p.y_dtype = y_dtype;
-        p.x_vec_ok = (((uintptr_t)p.X) % 16 == 0) && ((K * x_elem_size) % 16 == 0);
+        p.x_vec_ok = (((uintptr_t)p.X) % 16 == 0) && ((Kx * x_elem_size) % 16 == 0);
         int rc;
         if (mode == MODE_I8) rc = launch_stream_mode<MODE_I8>(p, pl, st);
         else if (mode == MODE_F16) rc = launch_stream_mode<MODE_F16>(p, pl, st);

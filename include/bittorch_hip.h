@@ -44,9 +44,10 @@ typedef enum {
  * NULL may be passed).  A workspace needs no initialisation and carries nothing
  * from one call to the next; two calls that may run concurrently (different
  * streams) need different workspaces.  Workspaces must be 256-byte aligned.
- * At present only bt_ternary_linear_tensor_core_forward uses one (the int8
- * activations and their row scales); the GEMM entry points keep the argument so
- * that a kernel that needs scratch can be introduced without an ABI change.
+ * At present bt_ternary_linear_tensor_core_forward uses one (the int8 activations
+ * and their row scales) and bt_ternary_linear_packed_forward uses one for fp32
+ * activations (three bf16 planes); bt_ternary_gemm_i8 keeps the argument so that a
+ * kernel that needs scratch can be introduced without an ABI change.
  */
 #define BT_WORKSPACE_COUNTER_BYTES 16384 /* kept for callers that clear the head of a workspace; unused */
 
@@ -92,10 +93,13 @@ int bt_ternary_linear_forward(const void* X, int x_dtype, const int8_t* W_tern, 
  * dispatch.cpp:105-142, csrc/kernels/ternary_gemm_production.cu:286-362).
  *   X [B,K] x_dtype; W_T [ceil(K/4),N] uint8; Y [B,N] x_dtype.
  *   Batches up to 32 rows stream the weights once per 16 rows (decode shape); taller
- *   fp16 / bf16 batches run the tiled 16-bit matrix-core GEMM; fp32 activations and
- *   unaligned operands run a generic kernel that accumulates in the reference's k order.
+ *   batches run the tiled 16-bit matrix-core GEMM.  fp32 activations with K % 64 == 0 are
+ *   first split into three bf16 planes (x = hi + mid + lo exactly) in the workspace and run
+ *   on the same bf16 kernels with exact products and fp32 accumulation.  Other fp32 shapes,
+ *   unaligned operands, a missing workspace and BITTORCH_KERNEL=generic run a generic
+ *   kernel that accumulates in the reference's k order.
  *   workspace: at least bt_packed_forward_workspace_bytes(B,N,K,x_dtype) bytes
- *   (currently 0: may be NULL).
+ *   (6*B*K rounded up to 256 for fp32 with K % 64 == 0, otherwise 0: may be NULL).
  */
 size_t bt_packed_forward_workspace_bytes(int64_t B, int64_t N, int64_t K, int x_dtype);
 int bt_ternary_linear_packed_forward(const void* X, int x_dtype, const uint8_t* W_T,

@@ -34,7 +34,7 @@ def test_module_forward_matches_python_backend(shape):
     assert torch.allclose(y, y_ref, rtol=1e-4, atol=1e-4)
 
 
-def test_config1_plumbing_gpu(oracle):
+def test_config1_plumbing_gpu(oracle, monkeypatch):
     """Config 1 on the GPU: TernaryLinear(512->256, bias), batch 32, fp32, seed 0."""
     from bittorch_amd.nn import TernaryLinear, create_ternary_linear_inference
     announce("config1 gpu")
@@ -47,12 +47,17 @@ def test_config1_plumbing_gpu(oracle):
     o_t, o_s = oracle.ternary_quantize(layer.weight.detach().numpy(), 0.05, True)
     o_p, _ = oracle.pack_ternary_transposed(o_t)
     ref = oracle.linear_packed(x.numpy(), o_p, o_s, 512, layer.bias.detach().numpy())
+    truth = oracle.linear_packed(x.numpy(), o_p, o_s, 512, layer.bias.detach().numpy(), f64=True)
     layer = layer.cuda()
-    y = layer(x.cuda())
-    np.testing.assert_array_equal(f32np(y), ref)  # fp32 generic kernel: oracle's k order
     inf = create_ternary_linear_inference(512, 256, layer.weight.detach(), layer.bias.detach())
     np.testing.assert_array_equal(inf.weight_packed.cpu().numpy(), o_p)
     np.testing.assert_array_equal(inf.scale.cpu().numpy(), o_s)
+    # default route for fp32 with K % 64 == 0: three exact bf16 planes on the matrix cores
+    assert rel_err(f32np(layer(x.cuda())), truth) < 1e-5
+    assert rel_err(f32np(inf(x.cuda())), truth) < 1e-5
+    # the generic kernel sums in the oracle's k order: bit for bit
+    monkeypatch.setenv("BITTORCH_KERNEL", "generic")
+    np.testing.assert_array_equal(f32np(layer(x.cuda())), ref)
     np.testing.assert_array_equal(f32np(inf(x.cuda())), ref)
 
 

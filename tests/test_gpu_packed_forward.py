@@ -117,12 +117,58 @@ def test_packed_forward_tall_batch_matches_streaming_kernel(oracle):
         assert ((y_tiled.double() - y_stream.double()).abs().max() / denom) < 1e-2
 
 
-def test_packed_forward_fp32_generic_is_bit_exact(oracle):
-    """The generic kernel accumulates in the reference's k order: equal to the oracle bit for bit."""
+def test_packed_forward_fp32_generic_is_bit_exact(oracle, monkeypatch):
+    """The generic kernel accumulates in the reference's k order: equal to the oracle bit for bit
+    (shapes whose K is a multiple of 64 take the matrix-core route by default, so it is forced)."""
     announce("packed_forward fp32 bit exact")
+    monkeypatch.setenv("BITTORCH_KERNEL", "generic")
     for (b, n, k) in [(32, 256, 512), (7, 33, 17), (1, 1, 1), (2, 100, 1000)]:
         got, ref = _case(oracle, b, n, k, torch.float32, seed=11)
         np.testing.assert_array_equal(got, ref)
+
+
+@pytest.mark.parametrize("b,n,k", [(1, 4096, 4096), (1, 64, 64), (5, 100, 128), (16, 512, 1024), (33, 256, 192),
+                                   (200, 260, 448), (512, 1024, 4096)])
+def test_packed_forward_fp32_on_the_matrix_cores(oracle, b, n, k, monkeypatch):
+    """fp32 activations with K % 64 == 0 are split into three exact bf16 planes and run on the bf16
+    kernels (streaming kernel up to 32 rows, tiled kernel above): every product is exact, only the
+    fp32 summation order differs from the generic kernel - far inside the 1e-3 budget for fp32."""
+    from bittorch_amd import _C
+    from bittorch_amd.quant import pack_ternary_transposed
+    announce("packed_forward fp32 planes", b, n, k)
+    w = random_ternary(n, k, seed=k + n)
+    g = torch.Generator().manual_seed(b + 1)
+    scale = torch.rand(n, generator=g) * 0.05 + 0.01
+    bias = torch.randn(n, generator=g) * 0.01
+    # activations spanning many binades, so that all three planes carry information
+    x = torch.randn(b, k, generator=g) * torch.exp(torch.randn(b, k, generator=g) * 3)
+    packed = pack_ternary_transposed(w)[0]
+    y = _C.ternary_linear_packed_forward(x.cuda(), packed.cuda(), scale.cuda(), bias.cuda(), k)
+    assert y.dtype == torch.float32
+    truth = oracle.linear_packed(f32np(x), packed.numpy(), f32np(scale), k, f32np(bias), f64=True)
+    assert rel_err(f32np(y), truth) < 1e-5
+    monkeypatch.setenv("BITTORCH_KERNEL", "generic")
+    y_gen = _C.ternary_linear_packed_forward(x.cuda(), packed.cuda(), scale.cuda(), bias.cuda(), k)
+    assert rel_err(f32np(y), f32np(y_gen)) < 1e-5
+
+
+def test_f32_plane_split_is_exact():
+    """hi + mid + lo reproduces every fp32 activation exactly: with identity-like weights
+    (one +1 per output) the matrix-core route returns the inputs themselves."""
+    from bittorch_amd import _C
+    from bittorch_amd.quant import pack_ternary_transposed
+    announce("packed_forward fp32 planes exact")
+    k = n = 128
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(8, k, generator=g) * torch.exp(torch.randn(8, k, generator=g) * 6)
+    x[0, :4] = torch.tensor([0.0, -0.0, 1.0, -1.0])
+    x[1, :4] = torch.tensor([3.4028235e38, -3.4028235e38, 1e-30, -7e-25])
+    perm = torch.randperm(k, generator=g)
+    w = torch.zeros(n, k)
+    w[torch.arange(n), perm] = 1.0
+    packed = pack_ternary_transposed(w)[0].cuda()
+    y = _C.ternary_linear_packed_forward(x.cuda(), packed, torch.ones(n).cuda(), None, k)
+    assert torch.equal(y.cpu(), x[:, perm])
 
 
 def test_packed_forward_mixed_scale_dtypes(oracle):

@@ -70,19 +70,17 @@ def test_backward_through_masked_outputs_and_noncontiguous_inputs():
 
 
 def test_batched_equals_looped_all_kernels():
-    """Rows are independent in every kernel: one row at a time (streaming kernel), 48 rows
-    (tiled kernel for 16-bit inputs) and the generic fp32 kernel give the same rows."""
+    """Rows are independent in every kernel: one row at a time (streaming kernel) and 48 rows at
+    once (tiled kernel) give the same rows up to the fp32 summation order."""
     announce("robustness batched vs looped")
-    for dtype, tol in ((torch.float32, 0.0), (torch.float16, 2e-3), (torch.bfloat16, 2e-2)):
+    for dtype, tol in ((torch.float32, 1e-5), (torch.float16, 2e-3), (torch.bfloat16, 2e-2)):
         layer = _layer(256, 128).to(dtype)
         x = torch.randn(48, 256, device="cuda").to(dtype)
         with torch.no_grad():
             yb = layer(x)
             yl = torch.cat([layer(x[i:i + 1]) for i in range(48)])
-        if tol == 0.0:
-            assert torch.equal(yb, yl)
-        else:  # different kernels sum in a different order; outputs are rounded to 16 bits
-            assert (yb.float() - yl.float()).abs().max() <= tol * yl.float().abs().max()
+        # different kernels sum in a different order; 16-bit outputs are rounded
+        assert (yb.float() - yl.float()).abs().max() <= tol * yl.float().abs().max()
 
 
 @pytest.mark.parametrize("shape", [(8, 4096, 4096), (512, 1024, 4096), (64, 11008, 4096)])
