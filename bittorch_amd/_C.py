@@ -12,6 +12,8 @@ Importing this module raises ``ImportError`` when the library is not built.
 
 from __future__ import annotations
 
+import os
+
 from typing import Optional, Tuple
 
 import torch
@@ -91,6 +93,19 @@ def _float64_packed(X, W_T, scale, bias, in_features):
     return torch.nn.functional.linear(X, w, None if bias is None else bias.to(X.dtype))
 
 
+def pack_ternary_int8(W_tern: Tensor) -> Tensor:
+    """Dense ternary ``[N, K]`` int8 on the GPU -> packed transposed ``[ceil(K/4), N]`` uint8
+    (the bytes of ``quant.pack_ternary_transposed``)."""
+    _check(W_tern.dim() == 2 and W_tern.dtype == torch.int8, "W_tern must be 2D int8")
+    _check(W_tern.is_cuda, "All tensors must be CUDA")
+    W_tern = W_tern.contiguous()
+    N, K = W_tern.shape
+    packed = torch.empty(((K + 3) // 4, N), dtype=torch.uint8, device=W_tern.device)
+    with torch.cuda.device(W_tern.device):
+        _status(_L.bt_pack_ternary_i8(W_tern.data_ptr(), N, K, packed.data_ptr(), _stream(W_tern)))
+    return packed
+
+
 def ternary_linear_forward(X: Tensor, W_tern: Tensor, scale: Tensor,
                            bias: Optional[Tensor] = None) -> Tensor:
     """``Y = X @ (W_tern * scale).T + bias`` with dense int8 ternary weights ``[N, K]``.
@@ -112,8 +127,12 @@ def ternary_linear_forward(X: Tensor, W_tern: Tensor, scale: Tensor,
     if X.dtype == torch.float64:
         w = W_tern.to(X.dtype) * scale.to(X.dtype).unsqueeze(1)
         return torch.nn.functional.linear(X, w, None if bias is None else bias.to(X.dtype))
-    x2 = X.contiguous().reshape(-1, K)
     W_tern = W_tern.contiguous()
+    if os.environ.get("BITTORCH_KERNEL", "auto") != "generic":
+        # the weights are packed on the device (one read of N*K bytes) and the call joins the
+        # packed matrix-core path; entries are taken as ternary (sign of anything non-zero)
+        return ternary_linear_packed_forward(X, pack_ternary_int8(W_tern), scale, bias, K)
+    x2 = X.contiguous().reshape(-1, K)
     scale = _prep_vec(scale, x2)
     bias = None if bias is None else _prep_vec(bias, x2)
     B = x2.shape[0]

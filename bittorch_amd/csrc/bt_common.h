@@ -45,6 +45,7 @@ template <int DT>
 __device__ __forceinline__ float load_elem(const void* p, int64_t i) {
     if constexpr (DT == BT_F32) return ((const float*)p)[i];
     else if constexpr (DT == BT_F16) return f16_bits_to_f32(((const uint16_t*)p)[i]);
+    else if constexpr (DT == BT_I8) return (float)((const int8_t*)p)[i];
     else return bf16_bits_to_f32(((const uint16_t*)p)[i]);
 }
 template <int DT>

@@ -196,6 +196,10 @@ __device__ __forceinline__ void load4(const void* W, int64_t elem, int64_t row_e
         if constexpr (DT == BT_F32) {
             const float4 t = *(const float4*)((const float*)W + elem);
             v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+        } else if constexpr (DT == BT_I8) {
+            const uint32_t t = *(const uint32_t*)((const int8_t*)W + elem);
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[i] = (float)(int8_t)(t >> (8 * i));
         } else {
             const uint2 t = *(const uint2*)((const uint16_t*)W + elem);
             const uint16_t h[4] = {(uint16_t)(t.x & 0xffff), (uint16_t)(t.x >> 16),
@@ -217,7 +221,8 @@ template <int DT>
 __global__ __launch_bounds__(256) void quantize_pack_generic_kernel(
     const void* __restrict__ W, int64_t N, int64_t K, int64_t Kb, float tf, float clamp_min, int per_channel,
     uint8_t* __restrict__ packed_T, float* __restrict__ scale, int8_t* __restrict__ w_tern, int64_t tiles,
-    int64_t per_xcd) {
+    int64_t per_xcd, float fixed_thr) {
+    // fixed_thr >= 0: no scale at all, the threshold is given (packing of already ternary weights)
     constexpr int PITCH = 5;
     __shared__ uint32_t lds[G_SEG * PITCH];
     const int64_t tile = xcd_tile(blockIdx.x, per_xcd);
@@ -227,7 +232,7 @@ __global__ __launch_bounds__(256) void quantize_pack_generic_kernel(
     const int64_t n0 = tile * 16;
     const bool vec_ok = (K % 4 == 0) && (((uintptr_t)W) % 16 == 0);
     const bool tern_vec = vec_ok && (((uintptr_t)w_tern) % 4 == 0);
-    const float tensor_scale = per_channel ? 0.0f : fmaxf(scale[0], clamp_min);
+    const float tensor_scale = (per_channel || fixed_thr >= 0.0f) ? 0.0f : fmaxf(scale[0], clamp_min);
 
     float thr[4];
 #pragma unroll
@@ -245,7 +250,7 @@ __global__ __launch_bounds__(256) void quantize_pack_generic_kernel(
             s = fmaxf(wave_max(amax), clamp_min);
             if (lane == 0) scale[n] = s;
         }
-        thr[r] = round_to_dtype(__fmul_rn(tf, s), DT);
+        thr[r] = (fixed_thr >= 0.0f) ? fixed_thr : round_to_dtype(__fmul_rn(tf, s), DT);
     }
 
     const bool full = (n0 + 16 <= N) && (N % 16 == 0) && (((uintptr_t)packed_T) % 16 == 0);
@@ -355,7 +360,7 @@ static int launch_quantize(const void* W, int64_t N, int64_t K, float tf, float 
     const int64_t tiles = ceil_div(N, 16);
     const int64_t per_xcd = ceil_div(tiles, 8);
     hipLaunchKernelGGL(quantize_pack_generic_kernel<DT>, dim3((unsigned)(per_xcd * 8)), dim3(256), 0, st, W, N, K,
-                       Kb, tf, clamp_min, per_channel, packed_T, scale, w_tern, tiles, per_xcd);
+                       Kb, tf, clamp_min, per_channel, packed_T, scale, w_tern, tiles, per_xcd, -1.0f);
     return check_launch("bt_quantize_pack");
 }
 
@@ -411,4 +416,20 @@ extern "C" int bt_quantize_pack(const void* W, int w_dtype, int64_t N, int64_t K
         return check_launch("bt_quantize_pack(floor)");
     }
     return BT_OK;
+}
+
+extern "C" int bt_pack_ternary_i8(const int8_t* W_tern, int64_t N, int64_t K, uint8_t* packed_T, void* stream) {
+    using namespace bt;
+    if (!W_tern || !packed_T || N <= 0 || K <= 0) {
+        set_error("bt_pack_ternary_i8: null pointer or empty shape (N=%lld K=%lld)", (long long)N, (long long)K);
+        return BT_ERR_INVALID;
+    }
+    const int64_t Kb = ceil_div(K, 4);
+    const int64_t tiles = ceil_div(N, 16);
+    const int64_t per_xcd = ceil_div(tiles, 8);
+    // codes: +1 -> 1, -1 -> 2, anything of magnitude <= 0.5 (i.e. 0) -> 0
+    hipLaunchKernelGGL(quantize_pack_generic_kernel<BT_I8>, dim3((unsigned)(per_xcd * 8)), dim3(256), 0,
+                       (hipStream_t)stream, (const void*)W_tern, N, K, Kb, 0.0f, 0.0f, 0, packed_T, (float*)nullptr,
+                       (int8_t*)nullptr, tiles, per_xcd, 0.5f);
+    return check_launch("bt_pack_ternary_i8");
 }

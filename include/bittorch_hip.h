@@ -160,6 +160,15 @@ int bt_unpack_dequant(const uint8_t* W_T, const float* scale, int64_t scale_len,
                       int out_dtype, int64_t N, int64_t K, void* stream);
 
 /*
+ * Dense ternary weights -> packed transposed layout, on the device.
+ * Replaces pack_ternary_transposed (bittorch/quant/ternary_packed.py:174-206) for weights
+ * that are already ternary: W_tern [N,K] int8 in {-1,0,+1} -> packed_T [ceil(K/4),N] uint8.
+ * The host side uses it to serve bittorch._C.ternary_linear_forward (dense int8 weights)
+ * with the packed matrix-core kernels.
+ */
+int bt_pack_ternary_i8(const int8_t* W_tern, int64_t N, int64_t K, uint8_t* packed_T, void* stream);
+
+/*
  * Measurement aid with no counterpart in the reference: launches `blocks`
  * workgroups of 8 waves that each issue `iters` x 8 back-to-back
  * v_mfma_i32_16x16x64_i8 on register operands (no memory traffic) and writes the

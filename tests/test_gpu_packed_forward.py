@@ -231,19 +231,42 @@ def test_packed_forward_stream_configs_agree(oracle):
         os.environ.pop("BITTORCH_STREAM_CFG", None)
 
 
-def test_unpacked_forward_matches_oracle(oracle):
+def test_unpacked_forward_matches_oracle(oracle, monkeypatch):
+    """Dense int8 weights: by default they are packed on the device and take the packed kernels
+    (exact products, fp32 sums in a different order); the dense generic kernel sums in the
+    reference's k order, bit for bit."""
     from bittorch_amd import _C
     announce("unpacked forward")
-    for (b, n, k) in [(4, 8, 16), (1, 1, 1), (17, 67, 123), (32, 256, 512)]:
+    for (b, n, k) in [(4, 8, 16), (1, 1, 1), (17, 67, 123), (32, 256, 512), (200, 128, 192)]:
         w = random_ternary(n, k, seed=k)
         g = torch.Generator().manual_seed(1)
         scale = torch.rand(n, generator=g)
         bias = torch.randn(n, generator=g)
         x = seeded_acts(b, k, seed=2)
-        y = _C.ternary_linear_forward(x.cuda(), w.cuda(), scale.cuda(), bias.cuda())
         ref = oracle.linear_unpacked(f32np(x), w.numpy(), f32np(scale), f32np(bias))
-        np.testing.assert_array_equal(f32np(y), ref)
-        y16 = _C.ternary_linear_forward(x.half().cuda(), w.cuda(), scale.half().cuda(), None)
-        assert y16.dtype == torch.float16
         ref16 = oracle.linear_unpacked(f32np(x.half()), w.numpy(), f32np(scale.half()), None)
-        assert rel_err(f32np(y16), ref16) < 1e-2
+        for forced in (False, True):
+            if forced:
+                monkeypatch.setenv("BITTORCH_KERNEL", "generic")
+            else:
+                monkeypatch.delenv("BITTORCH_KERNEL", raising=False)
+            y = _C.ternary_linear_forward(x.cuda(), w.cuda(), scale.cuda(), bias.cuda())
+            if forced:
+                np.testing.assert_array_equal(f32np(y), ref)
+            else:
+                assert rel_err(f32np(y), ref) < 1e-5
+            y16 = _C.ternary_linear_forward(x.half().cuda(), w.cuda(), scale.half().cuda(), None)
+            assert y16.dtype == torch.float16
+            assert rel_err(f32np(y16), ref16) < 1e-2
+
+
+def test_device_pack_of_dense_ternary_weights():
+    """bt_pack_ternary_i8 writes the bytes of pack_ternary_transposed, for ragged shapes too."""
+    from bittorch_amd import _C
+    from bittorch_amd.quant import pack_ternary_transposed
+    announce("pack_ternary_int8")
+    for (n, k) in [(1, 1), (16, 4), (33, 17), (67, 123), (256, 512), (100, 1000), (4096, 1024)]:
+        w = random_ternary(n, k, seed=n + k)
+        got = _C.pack_ternary_int8(w.cuda())
+        want, _ = pack_ternary_transposed(w)
+        assert torch.equal(got.cpu(), want), (n, k)
