@@ -133,16 +133,50 @@ __global__ __launch_bounds__(256) void unpack_dequant_kernel(const uint8_t* __re
     const int64_t n = n0 + c;
     if (n >= N) return;
     const float s = scale ? scale[scale_bcast ? 0 : n] : 1.0f;
+    // 16 consecutive k of one output row per thread; the four threads of a column cover 64 k
+    float w[16];
 #pragma unroll
     for (int r = 0; r < 4; r++) {
         const uint32_t byte = tile[part * 4 + r][c];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int64_t k = 4 * (kb0 + part * 4 + r) + i;
-            if (k < K) {
-                const float w = (float)decode2((byte >> (2 * i)) & 3u);
-                if constexpr (ODT == 3) ((int8_t*)out)[n * K + k] = (int8_t)w;
-                else store_elem<ODT>(out, n * K + k, __fmul_rn(w, s));
+        for (int i = 0; i < 4; i++) w[4 * r + i] = (float)decode2((byte >> (2 * i)) & 3u);
+    }
+    const int64_t k0 = 4 * (kb0 + part * 4);
+    constexpr int OES = (ODT == 3) ? 1 : (ODT == BT_F32) ? 4 : 2;
+    uint8_t* dst = (uint8_t*)out + (n * K + k0) * OES;
+    if (k0 + 16 <= K && (((uintptr_t)dst) % 16 == 0)) {
+        if constexpr (ODT == 3) {
+            uint32_t d[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+                d[q] = (uint32_t)(uint8_t)(int8_t)w[4 * q] | ((uint32_t)(uint8_t)(int8_t)w[4 * q + 1] << 8) |
+                       ((uint32_t)(uint8_t)(int8_t)w[4 * q + 2] << 16) | ((uint32_t)(uint8_t)(int8_t)w[4 * q + 3] << 24);
+            *(uint4*)dst = make_uint4(d[0], d[1], d[2], d[3]);
+        } else if constexpr (ODT == BT_F32) {
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+                ((float4*)dst)[q] = make_float4(__fmul_rn(w[4 * q], s), __fmul_rn(w[4 * q + 1], s),
+                                                __fmul_rn(w[4 * q + 2], s), __fmul_rn(w[4 * q + 3], s));
+        } else {
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                uint32_t d[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float a = __fmul_rn(w[8 * q + 2 * e], s), b = __fmul_rn(w[8 * q + 2 * e + 1], s);
+                    const uint32_t lo = (ODT == BT_F16) ? f32_to_f16_bits(a) : f32_to_bf16_bits(a);
+                    const uint32_t hi = (ODT == BT_F16) ? f32_to_f16_bits(b) : f32_to_bf16_bits(b);
+                    d[e] = lo | (hi << 16);
+                }
+                ((uint4*)dst)[q] = make_uint4(d[0], d[1], d[2], d[3]);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            if (k0 + i < K) {
+                if constexpr (ODT == 3) ((int8_t*)out)[n * K + k0 + i] = (int8_t)w[i];
+                else store_elem<ODT>(out, n * K + k0 + i, __fmul_rn(w[i], s));
             }
         }
     }
