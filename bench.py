@@ -474,6 +474,30 @@ def main():
         dt2 = (time.perf_counter() - t0) / it2
         out["cpu_baseline"]["torch_unpack_linear_ms_per_step"] = round(dt2 * 1e3, 3)
         out["cpu_baseline"]["torch_unpack_linear_GBps"] = round(weight_bytes / dt2 / 1e9, 4)
+        # the training module's plain-torch backend on the CPU (quantize the fp32 masters every call,
+        # then a dense product), and the dense product alone on pre-quantized effective weights
+        from bittorch_amd.nn import TernaryLinear
+
+        def cpu_time(fn, seconds=3.0):
+            fn()
+            t0 = time.perf_counter()
+            n = 0
+            while time.perf_counter() - t0 < seconds:
+                fn()
+                n += 1
+            return (time.perf_counter() - t0) / n
+
+        tl = TernaryLinear(K, N, bias=True, per_channel=False, backend="python")
+        with torch.no_grad():
+            tl.weight.copy_(w0.cpu())
+            tl.bias.copy_(bias.float().cpu())
+            dt3 = cpu_time(lambda: tl(xc))
+            w_tern, s_cpu = tl.get_quantized_weight()
+            w_eff = (w_tern * s_cpu).contiguous()
+            dt4 = cpu_time(lambda: torch.nn.functional.linear(xc, w_eff, tl.bias))
+        out["cpu_baseline"]["torch_python_backend_requantize_ms_per_step"] = round(dt3 * 1e3, 3)
+        out["cpu_baseline"]["torch_prequantized_dense_fp32_ms_per_step"] = round(dt4 * 1e3, 3)
+        out["cpu_baseline"]["torch_threads"] = torch.get_num_threads()
 
     print(json.dumps(out))
 
