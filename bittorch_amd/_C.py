@@ -162,18 +162,29 @@ def _packed_checks(X, W_T, scale, bias, in_features, flatten: bool = True):
     return K, N
 
 
+def _residual_2d(residual: Tensor, like: Tensor, lead_shape, N: int) -> Tensor:
+    _check(residual.shape == (*lead_shape, N), "residual shape doesn't match the output")
+    _check(residual.dtype == like.dtype, "residual must have the output's dtype")
+    _check(residual.device == like.device, "All tensors must be CUDA")
+    return residual.contiguous().reshape(-1, N)
+
+
 def ternary_linear_packed_forward(X: Tensor, W_T: Tensor, scale: Tensor,
-                                  bias: Optional[Tensor] = None, in_features: int = -1) -> Tensor:
+                                  bias: Optional[Tensor] = None, in_features: int = -1,
+                                  residual: Optional[Tensor] = None) -> Tensor:
     """Packed-weight forward, fp32 accumulation; ``W_T`` is ``[ceil(K/4), N]`` uint8.
 
     Reference: ``bittorch_bindings.cpp:48-63``, ``dispatch.cpp:105-142``.  ``scale``
     may be fp32 or the activation dtype and may have one entry (per-tensor scale).
+    ``residual`` (additive, not in the reference): a tensor of the output's shape and dtype
+    added in the kernel's epilogue with the two roundings of ``linear(x) + residual``.
     """
     if in_features < 0:
         in_features = X.shape[-1]
     K, N = _packed_checks(X, W_T, scale, bias, in_features)
     if X.dtype == torch.float64:
-        return _float64_packed(X, W_T, scale, bias, in_features)
+        y = _float64_packed(X, W_T, scale, bias, in_features)
+        return y if residual is None else y + residual
     x2 = X.contiguous().reshape(-1, K)
     W_T = W_T.contiguous()
     scale = _prep_vec(scale, x2)
@@ -184,10 +195,17 @@ def ternary_linear_packed_forward(X: Tensor, W_T: Tensor, scale: Tensor,
     with torch.cuda.device(X.device):
         ws_bytes = _L.bt_packed_forward_workspace_bytes(B, N, K, xdt)
         ws = _workspace(ws_bytes, X.device)
-        _status(_L.bt_ternary_linear_packed_forward(
-            x2.data_ptr(), xdt, W_T.data_ptr(), scale.data_ptr(), _dt(scale, "scale"), scale.numel(),
-            _ptr(bias), 0 if bias is None else _dt(bias, "bias"), y.data_ptr(), B, N, K,
-            _ptr(ws), 0 if ws is None else ws.numel(), _stream(X)))
+        if residual is None:
+            _status(_L.bt_ternary_linear_packed_forward(
+                x2.data_ptr(), xdt, W_T.data_ptr(), scale.data_ptr(), _dt(scale, "scale"), scale.numel(),
+                _ptr(bias), 0 if bias is None else _dt(bias, "bias"), y.data_ptr(), B, N, K,
+                _ptr(ws), 0 if ws is None else ws.numel(), _stream(X)))
+        else:
+            res = _residual_2d(residual, X, X.shape[:-1], N)
+            _status(_L.bt_ternary_linear_packed_forward_res(
+                x2.data_ptr(), xdt, W_T.data_ptr(), scale.data_ptr(), _dt(scale, "scale"), scale.numel(),
+                _ptr(bias), 0 if bias is None else _dt(bias, "bias"), res.data_ptr(), y.data_ptr(), B, N, K,
+                _ptr(ws), 0 if ws is None else ws.numel(), _stream(X)))
     return y.reshape(*X.shape[:-1], N)
 
 
@@ -273,8 +291,10 @@ def act_quant_int8(X: Tensor) -> Tuple[Tensor, Tensor]:
 
 def ternary_gemm_int8(Q: Tensor, s_x: Tensor, W_T: Tensor, scale: Tensor,
                       bias: Optional[Tensor] = None, in_features: int = -1,
-                      out_dtype: torch.dtype = torch.float32, return_acc: bool = False):
-    """int8 activations x packed ternary weights; optionally also the int32 accumulators."""
+                      out_dtype: torch.dtype = torch.float32, return_acc: bool = False,
+                      residual: Optional[Tensor] = None):
+    """int8 activations x packed ternary weights; optionally also the int32 accumulators.
+    ``residual`` ``[B, N]`` in ``out_dtype`` is added in the epilogue (``linear + residual``)."""
     _check(Q.dim() == 2 and Q.dtype == torch.int8, "Q must be 2D int8")
     if in_features < 0:
         in_features = Q.shape[-1]
@@ -293,11 +313,86 @@ def ternary_gemm_int8(Q: Tensor, s_x: Tensor, W_T: Tensor, scale: Tensor,
     with torch.cuda.device(q.device):
         ws_bytes = _L.bt_gemm_i8_workspace_bytes(B, N, K)
         ws = _workspace(ws_bytes, q.device)
-        _status(_L.bt_ternary_gemm_i8(
-            q.data_ptr(), s_x.data_ptr(), W_T.data_ptr(), scale.data_ptr(), _dt(scale, "scale"),
-            scale.numel(), _ptr(bias), 0 if bias is None else _dt(bias, "bias"), y.data_ptr(),
-            _DT[out_dtype], _ptr(acc), B, N, K, _ptr(ws), 0 if ws is None else ws.numel(), _stream(q)))
+        if residual is None:
+            _status(_L.bt_ternary_gemm_i8(
+                q.data_ptr(), s_x.data_ptr(), W_T.data_ptr(), scale.data_ptr(), _dt(scale, "scale"),
+                scale.numel(), _ptr(bias), 0 if bias is None else _dt(bias, "bias"), y.data_ptr(),
+                _DT[out_dtype], _ptr(acc), B, N, K, _ptr(ws), 0 if ws is None else ws.numel(), _stream(q)))
+        else:
+            res = _residual_2d(residual, y, (B,), N)
+            _status(_L.bt_ternary_gemm_i8_res(
+                q.data_ptr(), s_x.data_ptr(), W_T.data_ptr(), scale.data_ptr(), _dt(scale, "scale"),
+                scale.numel(), _ptr(bias), 0 if bias is None else _dt(bias, "bias"), res.data_ptr(),
+                y.data_ptr(), _DT[out_dtype], _ptr(acc), B, N, K, _stream(q)))
     return (y, acc) if return_acc else y
+
+
+def _row_op_outputs(x2: Tensor, store: bool, quantize: bool):
+    _check(store or quantize, "nothing to compute: store and quantize are both False")
+    B, K = x2.shape
+    h = torch.empty((B, K), dtype=x2.dtype, device=x2.device) if store else None
+    q = torch.empty((B, K), dtype=torch.int8, device=x2.device) if quantize else None
+    s = torch.empty((B,), dtype=torch.float32, device=x2.device) if quantize else None
+    return h, q, s
+
+
+def _row_op_result(h, q, s, lead_shape, K):
+    if h is not None:
+        h = h.reshape(*lead_shape, K)
+    if q is None:
+        return h
+    return (q, s) if h is None else (h, q, s)
+
+
+def _rows_2d(t: Tensor, K: int) -> Tensor:
+    """A 2-D view with unit inner stride (row stride kept: slices of a wider matrix stay in place)."""
+    if t.dim() == 2 and t.stride(1) == 1 and t.stride(0) >= K:
+        return t
+    return t.contiguous().reshape(-1, K)
+
+
+def swiglu(gate: Tensor, up: Tensor, store: bool = True, quantize: bool = False):
+    """``silu(gate) * up`` in one pass, rounded as the two separate torch ops round it.
+
+    Returns the product (``store``), or with ``quantize`` its per-row int8 form ``(Q, s_x)`` for
+    :func:`ternary_gemm_int8` -- ``(h, Q, s_x)`` when both are asked for.  ``gate`` and ``up`` may
+    be column slices of one wider matrix (the output of a fused gate/up projection)."""
+    _check(gate.shape == up.shape and gate.dtype == up.dtype, "gate and up must match in shape and dtype")
+    _check(gate.dim() >= 1 and gate.numel() > 0, "gate is empty")
+    _check(gate.dtype in _DT, "gate must be float32, float16 or bfloat16")
+    _check(_all_cuda(gate, up), "All tensors must be CUDA")
+    K = gate.shape[-1]
+    g2, u2 = _rows_2d(gate, K), _rows_2d(up, K)
+    h, q, s = _row_op_outputs(g2, store, quantize)
+    with torch.cuda.device(gate.device):
+        _status(_L.bt_swiglu(g2.data_ptr(), g2.stride(0), u2.data_ptr(), u2.stride(0), _dt(g2, "gate"),
+                             g2.shape[0], K, _ptr(h), _ptr(q), _ptr(s), _stream(gate)))
+    if q is not None and gate.dim() != 2:
+        q = q.reshape(*gate.shape[:-1], K)
+        s = s.reshape(gate.shape[:-1])
+    return _row_op_result(h, q, s, gate.shape[:-1], K)
+
+
+def rmsnorm(x: Tensor, weight: Optional[Tensor] = None, eps: float = 1e-6, store: bool = True,
+            quantize: bool = False):
+    """RMSNorm over the last dimension, ``(x * rsqrt(mean(x^2) + eps)) * weight``; with
+    ``quantize`` also (or only, ``store=False``) the per-row int8 form of the result."""
+    _check(x.dim() >= 1 and x.numel() > 0, "x is empty")
+    _check(x.dtype in _DT, "x must be float32, float16 or bfloat16")
+    K = x.shape[-1]
+    if weight is not None:
+        _check(weight.dim() == 1 and weight.shape[0] == K, "weight must be 1D [K]")
+        weight = weight.to(x.dtype).contiguous()
+    _check(_all_cuda(x, weight), "All tensors must be CUDA")
+    x2 = _rows_2d(x, K)
+    h, q, s = _row_op_outputs(x2, store, quantize)
+    with torch.cuda.device(x.device):
+        _status(_L.bt_rmsnorm(x2.data_ptr(), x2.stride(0), _ptr(weight), float(eps), _dt(x2, "x"),
+                              x2.shape[0], K, _ptr(h), _ptr(q), _ptr(s), _stream(x)))
+    if q is not None and x.dim() != 2:
+        q = q.reshape(*x.shape[:-1], K)
+        s = s.reshape(x.shape[:-1])
+    return _row_op_result(h, q, s, x.shape[:-1], K)
 
 
 def unpack_dequant(W_T: Tensor, in_features: int, scale: Optional[Tensor] = None,

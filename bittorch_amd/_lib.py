@@ -42,6 +42,12 @@ SIGNATURES = {
     "bt_unpack_dequant": (_int, [_vp, _vp, _i64, _vp, _int, _i64, _i64, _vp]),
     "bt_pack_ternary_i8": (_int, [_vp, _i64, _i64, _vp, _vp]),
     "bt_probe_mfma_i8": (_int, [_int, _int, _int, _vp, _vp, _vp]),
+    "bt_ternary_linear_packed_forward_res": (_int, [_vp, _int, _vp, _vp, _int, _i64, _vp, _int, _vp, _vp,
+                                                    _i64, _i64, _i64, _vp, _sz, _vp]),
+    "bt_ternary_gemm_i8_res": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _vp, _int, _vp, _vp, _int, _vp,
+                                      _i64, _i64, _i64, _vp]),
+    "bt_swiglu": (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _vp, _vp, _vp, _vp]),
+    "bt_rmsnorm": (_int, [_vp, _i64, _vp, ctypes.c_float, _int, _i64, _i64, _vp, _vp, _vp, _vp]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

@@ -38,6 +38,10 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
     return (float)__builtin_bit_cast(_Float16, h);
 }
 __device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+    // The empty asm keeps the conversion a conversion of the fp32 value: without it the compiler
+    // folds "(half)(a * b + c)" into v_fma_mixlo_f16, which rounds the exact result once, where
+    // the reference (and the CPU restatement) round to fp32 first and to fp16 second.
+    asm("" : "+v"(f));
     return __builtin_bit_cast(uint16_t, (_Float16)f);  // v_cvt_f16_f32, RNE
 }
 
@@ -86,12 +90,41 @@ struct Epilogue {
     int scale_dtype;
     int bias_dtype;
     int scale_bcast;  // 1: scale has one entry that applies to every column
+    const void* residual;  // optional [B, N] in the output's dtype, added to the finished output
 };
 __device__ __forceinline__ float epi_scale(const Epilogue& e, int64_t n) {
     return load_elem_rt(e.scale, e.scale_dtype, e.scale_bcast ? 0 : n);
 }
 __device__ __forceinline__ float epi_bias(const Epilogue& e, int64_t n) {
     return e.bias ? load_elem_rt(e.bias, e.bias_dtype, n) : 0.0f;
+}
+// Residual connection folded into the epilogue: y is first rounded to the output dtype, then the
+// residual is added in fp32 and the sum rounded again by the store -- the two roundings of an
+// unfused "linear, then add" in that dtype, so fusing does not change a bit.  (The fp32 sum of two
+// 16-bit values is exact unless their exponents are more than 13 apart, and then the smaller one
+// cannot move the larger across a rounding boundary: rounding the fp32 sum equals rounding the
+// exact sum.)
+__device__ __forceinline__ float sum_in_dtype(float y_rounded, float r, int dt) {
+    (void)dt;
+    return __fadd_rn(y_rounded, r);
+}
+__device__ __forceinline__ float add_residual(float y, const void* res, int dt, int64_t idx) {
+    return sum_in_dtype(round_to_dtype(y, dt), load_elem_rt(res, dt, idx), dt);
+}
+// four consecutive outputs (idx % 4 == 0, residual 16-byte aligned for fp32, 8-byte for 16-bit)
+__device__ __forceinline__ void add_residual4(float (&y)[4], const void* res, int dt, int64_t idx) {
+    float r[4];
+    if (dt == BT_F32) {
+        const float4 v = *(const float4*)((const float*)res + idx);
+        r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w;
+    } else {
+        const uint2 v = *(const uint2*)((const uint16_t*)res + idx);
+        const uint32_t d[2] = {v.x, v.y};
+#pragma unroll
+        for (int i = 0; i < 4; i++) r[i] = bits_to_f32_rt((d[i >> 1] >> (16 * (i & 1))) & 0xffffu, dt);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) y[i] = sum_in_dtype(round_to_dtype(y[i], dt), r[i], dt);
 }
 // fp32 accumulate path: one multiply, one add, each rounded (no fma contraction)
 __device__ __forceinline__ float epi_float(float acc, float s, float b) {

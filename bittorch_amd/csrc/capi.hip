@@ -40,6 +40,8 @@ int launch_unpacked(const void* X, int x_dtype, const int8_t* W, const Epilogue&
                     int64_t N, int64_t K, hipStream_t st);
 int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x, hipStream_t st);
 bool gemm_i8_supported(int64_t N, int64_t K, const void* Q, const void* W_T);
+int launch_row_op(int op, int dtype, const void* A, int64_t lda, const void* Bv, int64_t ldb, float eps, int64_t B,
+                  int64_t K, void* H, int8_t* Q, float* s_x, hipStream_t st, const char* who);
 bool gemm_f16_supported(int64_t N, int64_t K, const void* X, const void* W_T, const void* Y);
 int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, const Epilogue& epi, void* Y, int y_dtype, int64_t M,
                     int64_t N, int64_t K, int planes, hipStream_t st);
@@ -68,6 +70,7 @@ static int make_epilogue(const char* who, const void* scale, int scale_dtype, in
     e->scale_dtype = scale_dtype;
     e->bias_dtype = bias_dtype;
     e->scale_bcast = (scale_len == 1 && N != 1) ? 1 : 0;
+    e->residual = nullptr;
     return BT_OK;
 }
 
@@ -146,16 +149,26 @@ extern "C" size_t bt_packed_forward_workspace_bytes(int64_t B, int64_t N, int64_
     return stream_workspace_bytes(x_dtype == BT_F16 ? MODE_F16 : MODE_BF16, B, N, ceil_div(K, 4));
 }
 
-extern "C" int bt_ternary_linear_packed_forward(const void* X, int x_dtype, const uint8_t* W_T,
-                                                const void* scale, int scale_dtype, int64_t scale_len,
-                                                const void* bias, int bias_dtype, void* Y, int64_t B,
-                                                int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
-                                                void* stream) {
-    const char* who = "bt_ternary_linear_packed_forward";
+// residual (optional): [B, N] in Y's dtype, 16-byte aligned; Y = round(round(linear) + residual)
+static int set_residual(const char* who, const void* residual, Epilogue* e) {
+    if (residual && ((uintptr_t)residual) % 16 != 0) {
+        set_error("%s: residual must be 16-byte aligned", who);
+        return BT_ERR_INVALID;
+    }
+    e->residual = residual;
+    return BT_OK;
+}
+
+static int packed_forward_impl(const char* who, const void* X, int x_dtype, const uint8_t* W_T, const void* scale,
+                               int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
+                               const void* residual, void* Y, int64_t B, int64_t N, int64_t K, void* workspace,
+                               size_t workspace_bytes, void* stream) {
     int rc = check_shape(who, X, W_T, Y, x_dtype, B, N, K);
     if (rc) return rc;
     Epilogue epi;
     rc = make_epilogue(who, scale, scale_dtype, scale_len, bias, bias_dtype, N, &epi);
+    if (rc) return rc;
+    rc = set_residual(who, residual, &epi);
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
     if (packed_uses_stream(x_dtype, W_T, Y, N, K)) {
@@ -177,6 +190,24 @@ extern "C" int bt_ternary_linear_packed_forward(const void* X, int x_dtype, cons
     return launch_packed_generic(X, x_dtype, W_T, epi, Y, B, N, K, st);
 }
 
+extern "C" int bt_ternary_linear_packed_forward(const void* X, int x_dtype, const uint8_t* W_T,
+                                                const void* scale, int scale_dtype, int64_t scale_len,
+                                                const void* bias, int bias_dtype, void* Y, int64_t B,
+                                                int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
+                                                void* stream) {
+    return packed_forward_impl("bt_ternary_linear_packed_forward", X, x_dtype, W_T, scale, scale_dtype, scale_len, bias,
+                               bias_dtype, nullptr, Y, B, N, K, workspace, workspace_bytes, stream);
+}
+
+extern "C" int bt_ternary_linear_packed_forward_res(const void* X, int x_dtype, const uint8_t* W_T,
+                                                    const void* scale, int scale_dtype, int64_t scale_len,
+                                                    const void* bias, int bias_dtype, const void* residual,
+                                                    void* Y, int64_t B, int64_t N, int64_t K, void* workspace,
+                                                    size_t workspace_bytes, void* stream) {
+    return packed_forward_impl("bt_ternary_linear_packed_forward_res", X, x_dtype, W_T, scale, scale_dtype, scale_len,
+                               bias, bias_dtype, residual, Y, B, N, K, workspace, workspace_bytes, stream);
+}
+
 extern "C" int bt_act_quant_i8(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x,
                                void* stream) {
     if (!X || !Q || !s_x || B <= 0 || K <= 0 || !valid_dtype(x_dtype)) {
@@ -191,11 +222,9 @@ extern "C" size_t bt_gemm_i8_workspace_bytes(int64_t B, int64_t N, int64_t K) {
     return stream_workspace_bytes(MODE_I8, B, N, ceil_div(K, 4));
 }
 
-extern "C" int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const void* scale,
-                                  int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
-                                  void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N, int64_t K,
-                                  void* workspace, size_t workspace_bytes, void* stream) {
-    const char* who = "bt_ternary_gemm_i8";
+static int gemm_i8_impl(const char* who, const int8_t* Q, const float* s_x, const uint8_t* W_T, const void* scale,
+                        int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype, const void* residual,
+                        void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N, int64_t K, void* stream) {
     int rc = check_shape(who, Q, W_T, Y, y_dtype, B, N, K);
     if (rc) return rc;
     if (!s_x) {
@@ -214,6 +243,8 @@ extern "C" int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8
     Epilogue epi;
     rc = make_epilogue(who, scale, scale_dtype, scale_len, bias, bias_dtype, N, &epi);
     if (rc) return rc;
+    rc = set_residual(who, residual, &epi);
+    if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
     // decode-shape batches, and any batch whose N the tiled kernel's 4-column
     // vector accesses cannot take, stream the weights once per 16 rows
@@ -226,6 +257,23 @@ extern "C" int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8
         return launch_stream(MODE_I8, Q, 1, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, 1, st);
     }
     return launch_gemm_i8(Q, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, st);
+}
+
+extern "C" int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const void* scale,
+                                  int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
+                                  void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N, int64_t K,
+                                  void* workspace, size_t workspace_bytes, void* stream) {
+    (void)workspace; (void)workspace_bytes;
+    return gemm_i8_impl("bt_ternary_gemm_i8", Q, s_x, W_T, scale, scale_dtype, scale_len, bias, bias_dtype, nullptr, Y,
+                        y_dtype, acc_out, B, N, K, stream);
+}
+
+extern "C" int bt_ternary_gemm_i8_res(const int8_t* Q, const float* s_x, const uint8_t* W_T, const void* scale,
+                                      int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
+                                      const void* residual, void* Y, int y_dtype, int32_t* acc_out, int64_t B,
+                                      int64_t N, int64_t K, void* stream) {
+    return gemm_i8_impl("bt_ternary_gemm_i8_res", Q, s_x, W_T, scale, scale_dtype, scale_len, bias, bias_dtype, residual,
+                        Y, y_dtype, acc_out, B, N, K, stream);
 }
 
 extern "C" size_t bt_tensor_core_workspace_bytes(int64_t B, int64_t N, int64_t K) {
@@ -254,4 +302,46 @@ extern "C" int bt_ternary_linear_tensor_core_forward(const void* X, int x_dtype,
     if (rc) return rc;
     return bt_ternary_gemm_i8(Q, s_x, W_T, scale, scale_dtype, scale_len, bias, bias_dtype, Y, x_dtype, nullptr,
                               B, N, K, workspace, gemm_bytes, stream);
+}
+
+// ---- fused producers of the GEMM activations (row_ops.hip) ----------------------------------
+static int check_row_op(const char* who, const void* A, int dtype, int64_t B, int64_t K, int64_t lda, void* H,
+                        int8_t* Q, float* s_x) {
+    if (!A || B <= 0 || K <= 0 || !valid_dtype(dtype)) {
+        set_error("%s: null pointer, empty shape or bad dtype", who);
+        return BT_ERR_INVALID;
+    }
+    if (lda < K || K > 0x7fffffff || B > 0x7fffffff) {
+        set_error("%s: row stride %lld below K=%lld, or shape beyond 2^31", who, (long long)lda, (long long)K);
+        return BT_ERR_INVALID;
+    }
+    if (!H && !Q) {
+        set_error("%s: no output requested (H and Q both null)", who);
+        return BT_ERR_INVALID;
+    }
+    if (Q && !s_x) {
+        set_error("%s: Q given without s_x", who);
+        return BT_ERR_INVALID;
+    }
+    return BT_OK;
+}
+
+extern "C" int bt_swiglu(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, int dtype, int64_t B,
+                         int64_t K, void* H, int8_t* Q, float* s_x, void* stream) {
+    const char* who = "bt_swiglu";
+    int rc = check_row_op(who, gate, dtype, B, K, ld_gate, H, Q, s_x);
+    if (rc) return rc;
+    if (!up || ld_up < K) {
+        set_error("%s: up is null or its row stride is below K", who);
+        return BT_ERR_INVALID;
+    }
+    return launch_row_op(0, dtype, gate, ld_gate, up, ld_up, 0.0f, B, K, H, Q, s_x, (hipStream_t)stream, who);
+}
+
+extern "C" int bt_rmsnorm(const void* X, int64_t ld_x, const void* weight, float eps, int dtype, int64_t B,
+                          int64_t K, void* Y, int8_t* Q, float* s_x, void* stream) {
+    const char* who = "bt_rmsnorm";
+    int rc = check_row_op(who, X, dtype, B, K, ld_x, Y, Q, s_x);
+    if (rc) return rc;
+    return launch_row_op(1, dtype, X, ld_x, weight, 0, eps, B, K, Y, Q, s_x, (hipStream_t)stream, who);
 }

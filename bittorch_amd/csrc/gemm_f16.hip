@@ -80,6 +80,7 @@ __device__ __forceinline__ void gemm_f_epilogue(const GemmFParams& p, const v4f 
                 if constexpr (MODE == MODE_BF16) a *= (p.prehalved ? 1.0f : 0.5f);  // weights were decoded as +-2.0
                 y[t] = epi_float(a, ws[t], bs[t]);
             }
+            if (p.epi.residual) add_residual4(y, p.epi.residual, YDT, m * p.N + ncol);
             store4f(p.Y, YDT, m * p.N + ncol, y);
         }
     }

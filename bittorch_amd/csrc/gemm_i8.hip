@@ -86,6 +86,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&a
                 a127[t] = times127(a);
                 y[t] = epi_int8(a127[t], sx, ws[t], bs[t]);
             }
+            if (p.epi.residual) add_residual4(y, p.epi.residual, YDT, m * p.N + ncol);
             store4(p.Y, YDT, m * p.N + ncol, y);
             if (p.acc_out) *(int4*)(p.acc_out + m * p.N + ncol) = make_int4(a127[0], a127[1], a127[2], a127[3]);
         }

@@ -31,7 +31,9 @@ __global__ __launch_bounds__(256) void packed_generic_kernel(const void* __restr
             }
         }
     }
-    store_elem<XDT>(Y, b * N + n, epi_float(acc, epi_scale(epi, n), epi_bias(epi, n)));
+    float y = epi_float(acc, epi_scale(epi, n), epi_bias(epi, n));
+    if (epi.residual) y = add_residual(y, epi.residual, XDT, b * N + n);
+    store_elem<XDT>(Y, b * N + n, y);
 }
 
 int launch_packed_generic(const void* X, int x_dtype, const uint8_t* W_T, const Epilogue& epi, void* Y,
@@ -95,6 +97,7 @@ __global__ __launch_bounds__(256) void unpacked_kernel(const void* __restrict__ 
         // acc *= scale; acc += bias (only when a bias is given)
         float v = __fmul_rn(acc[r], s);
         if (epi.bias) v = __fadd_rn(v, epi_bias(epi, n));
+        if (epi.residual) v = add_residual(v, epi.residual, XDT, b * N + n);
         store_elem<XDT>(Y, b * N + n, v);
     }
 }

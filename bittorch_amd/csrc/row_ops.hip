@@ -1,0 +1,281 @@
+// Row-wise producers of the ternary GEMMs' activations for gfx950 (HBM-bound), fusing what a
+// transformer block does between two ternary layers (block structure of the reference's JS
+// runtime, js/src/models/TernaryTransformer.ts:366-423 (SwiGLU MLP), :489-521 (pre-norm block)):
+//
+//   SwiGLU   h[b,k] = rd( rd(silu(g[b,k])) * u[b,k] ),   silu(x) = x / (1 + exp(-x))
+//   RMSNorm  y[b,k] = rd( (x[b,k] * r_b) * w[k] ),        r_b = 1 / sqrt(ss_b / K + eps),
+//                                                         ss_b = float(sum_k double(x[b,k])^2)
+// (rd = round to the tensor dtype; every fp32 operation rounded on its own, no contraction; exp is
+// the fixed polynomial below, so a host restatement reproduces every bit), each optionally
+// followed in the same kernel by the per-row int8 activation quantizer of the int8 GEMM
+// (csrc/kernels/ternary_gemm_tensor_core.cu:343-347, :439, :456-457, whole-row scale):
+//   amax = max_k |v|;  s_x = amax > 1e-6 ? amax / 127 : 1;  q = clamp(roundf(v * (1 / s_x)), -127, 127)
+// so that the activation makes one trip through HBM instead of three or four.
+#include <cstdlib>
+
+#include "bt_common.h"
+
+namespace bt {
+
+enum { ROW_SWIGLU = 0, ROW_RMSNORM = 1 };
+
+struct RowOpParams {
+    const void* A;      // SwiGLU: gate [B, K] (row stride lda);  RMSNorm: x [B, K] (row stride lda)
+    const void* Bv;     // SwiGLU: up [B, K] (row stride ldb);    RMSNorm: weight [K] or null
+    int64_t lda, ldb;   // row strides in elements
+    void* H;            // optional [B, K] output in the input dtype
+    int8_t* Q;          // optional [B, K] int8 output (with s_x)
+    float* s_x;         // [B]
+    float eps;
+    int K;
+};
+
+// exp(a) in fp32 by a fixed sequence of correctly rounded operations (range reduction by ln 2 in two
+// parts, degree-7 polynomial, exact scaling): a few units in the last place from exp on
+// [-87, 88.7228]; +inf above (as exp overflows), exp(-87) below (callers only add it to 1).  The
+// same sequence with fmaf() on a CPU gives the same bits.
+__device__ __forceinline__ float exp_fixed(float a) {
+    if (!(a == a)) return a;
+    if (a > 88.7228f) return __builtin_inff();  // exp overflows fp32
+    a = fmaxf(a, -87.0f);
+    const float n = rintf(__fmul_rn(a, 1.44269504088896341f));
+    float r = __builtin_fmaf(n, -0.693145751953125f, a);         // ln2 high part (exact product)
+    r = __builtin_fmaf(n, -1.42860682030941723212e-6f, r);       // ln2 low part
+    float p = 1.0f / 5040.0f;
+    p = __builtin_fmaf(p, r, 1.0f / 720.0f);
+    p = __builtin_fmaf(p, r, 1.0f / 120.0f);
+    p = __builtin_fmaf(p, r, 1.0f / 24.0f);
+    p = __builtin_fmaf(p, r, 1.0f / 6.0f);
+    p = __builtin_fmaf(p, r, 0.5f);
+    p = __builtin_fmaf(p, r, 1.0f);
+    p = __builtin_fmaf(p, r, 1.0f);
+    // p * 2^n in two steps, the first exact (n in [-126, 128]; 2^128 itself is not representable)
+    const int ni = (int)n;
+    const int n1 = ni / 2, n2 = ni - n1;
+    const float s1 = __builtin_bit_cast(float, (uint32_t)(n1 + 127) << 23);
+    const float s2 = __builtin_bit_cast(float, (uint32_t)(n2 + 127) << 23);
+    return __fmul_rn(__fmul_rn(p, s1), s2);
+}
+
+__device__ __forceinline__ float swiglu_value(float g, float u, int dt) {
+    const float e = exp_fixed(-g);
+    const float s = round_to_dtype(__fdiv_rn(g, __fadd_rn(1.0f, e)), dt);
+    return round_to_dtype(__fmul_rn(s, u), dt);
+}
+__device__ __forceinline__ float rmsnorm_value(float x, float r, float w, int dt) {
+    return round_to_dtype(__fmul_rn(__fmul_rn(x, r), w), dt);
+}
+__device__ __forceinline__ float rms_rstd(double ss, int K, float eps) {
+    const float ms = __fdiv_rn((float)ss, (float)K);
+    // sqrtf is the correctly rounded square root (__fsqrt_rn is the approximate instruction)
+    return __fdiv_rn(1.0f, sqrtf(__fadd_rn(ms, eps)));
+}
+__device__ __forceinline__ int8_t quant_i8(float v, float inv) {
+    float r = roundf(__fmul_rn(v, inv));
+    r = fmaxf(-127.0f, fminf(127.0f, r));
+    return (int8_t)(int)r;
+}
+
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+}
+
+template <int DT>
+__device__ __forceinline__ void load8(const void* base, int64_t idx, float (&v)[8]) {
+    if constexpr (DT == BT_F32) {
+        const float4 a = *(const float4*)((const float*)base + idx);
+        const float4 b = *(const float4*)((const float*)base + idx + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+        const uint4 u = *(const uint4*)((const uint16_t*)base + idx);
+        const uint32_t d[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const uint16_t h = (uint16_t)(d[e >> 1] >> (16 * (e & 1)));
+            v[e] = (DT == BT_F16) ? f16_bits_to_f32(h) : bf16_bits_to_f32(h);
+        }
+    }
+}
+template <int DT>
+__device__ __forceinline__ void store8(void* base, int64_t idx, const float (&v)[8]) {
+    if constexpr (DT == BT_F32) {
+        *(float4*)((float*)base + idx) = make_float4(v[0], v[1], v[2], v[3]);
+        *(float4*)((float*)base + idx + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    } else {
+        uint32_t d[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const uint32_t lo = (DT == BT_F16) ? f32_to_f16_bits(v[2 * e]) : f32_to_bf16_bits(v[2 * e]);
+            const uint32_t hi = (DT == BT_F16) ? f32_to_f16_bits(v[2 * e + 1]) : f32_to_bf16_bits(v[2 * e + 1]);
+            d[e] = lo | (hi << 16);
+        }
+        *(uint4*)((uint16_t*)base + idx) = make_uint4(d[0], d[1], d[2], d[3]);
+    }
+}
+
+// One workgroup per row, the row held in registers: the operands are read once, the outputs
+// written once.  Needs K % 8 == 0, K <= 2048*ITERS, 16-byte aligned rows.
+template <int OP, int DT, int ITERS>
+__global__ __launch_bounds__(256) void row_op_kernel(RowOpParams p) {
+    __shared__ double part_d[4];
+    __shared__ float part_f[4];
+    const int tid = threadIdx.x;
+    const int K = p.K;
+    const int64_t row = blockIdx.x;
+    float v[ITERS][8];
+    // clamped, unconditional loads; lanes past the row are masked where it matters
+#pragma unroll
+    for (int i = 0; i < ITERS; i++) {
+        const int k = (i * 256 + tid) * 8;
+        const int kc = min(k, K - 8);
+        load8<DT>(p.A, row * p.lda + kc, v[i]);
+    }
+    if constexpr (OP == ROW_SWIGLU) {
+#pragma unroll
+        for (int i = 0; i < ITERS; i++) {
+            const int k = (i * 256 + tid) * 8;
+            const int kc = min(k, K - 8);
+            float u[8];
+            load8<DT>(p.Bv, row * p.ldb + kc, u);
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[i][e] = swiglu_value(v[i][e], u[e], DT);
+        }
+    } else {
+        double ss = 0.0;
+#pragma unroll
+        for (int i = 0; i < ITERS; i++) {
+            const bool ok = (i * 256 + tid) * 8 < K;
+#pragma unroll
+            for (int e = 0; e < 8; e++) ss += ok ? (double)v[i][e] * (double)v[i][e] : 0.0;
+        }
+        ss = wave_sum_f64(ss);
+        if ((tid & 63) == 0) part_d[tid >> 6] = ss;
+        __syncthreads();
+        ss = (part_d[0] + part_d[1]) + (part_d[2] + part_d[3]);
+        const float r = rms_rstd(ss, K, p.eps);
+#pragma unroll
+        for (int i = 0; i < ITERS; i++) {
+            const int k = (i * 256 + tid) * 8;
+            const int kc = min(k, K - 8);
+            float w[8];
+            if (p.Bv) load8<DT>(p.Bv, kc, w);
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[i][e] = rmsnorm_value(v[i][e], r, p.Bv ? w[e] : 1.0f, DT);
+        }
+    }
+    if (p.H) {
+#pragma unroll
+        for (int i = 0; i < ITERS; i++) {
+            const int k = (i * 256 + tid) * 8;
+            if (k < K) store8<DT>(p.H, row * (int64_t)K + k, v[i]);
+        }
+    }
+    if (!p.Q) return;  // uniform
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < ITERS; i++) {
+        const bool ok = (i * 256 + tid) * 8 < K;
+#pragma unroll
+        for (int e = 0; e < 8; e++) amax = fmaxf(amax, ok ? fabsf(v[i][e]) : 0.0f);
+    }
+    amax = wave_max(amax);
+    if ((tid & 63) == 0) part_f[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(part_f[0], part_f[1]), fmaxf(part_f[2], part_f[3]));
+    const float s = (amax > 1e-6f) ? __fdiv_rn(amax, 127.0f) : 1.0f;
+    const float inv = __fdiv_rn(1.0f, s);
+    if (tid == 0) p.s_x[row] = s;
+#pragma unroll
+    for (int i = 0; i < ITERS; i++) {
+        const int k = (i * 256 + tid) * 8;
+        uint32_t lo = 0, hi = 0;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const uint32_t byte = (uint32_t)(uint8_t)quant_i8(v[i][e], inv);
+            if (e < 4) lo |= byte << (8 * e);
+            else hi |= byte << (8 * (e - 4));
+        }
+        if (k < K) *(uint2*)(p.Q + row * (int64_t)K + k) = make_uint2(lo, hi);
+    }
+}
+
+// Any K and alignment: one workgroup per row, element-wise passes that recompute the value
+// (reduction passes hit in cache).
+template <int OP, int DT>
+__global__ __launch_bounds__(256) void row_op_generic_kernel(RowOpParams p) {
+    __shared__ double part_d[4];
+    __shared__ float part_f[4];
+    const int tid = threadIdx.x;
+    const int K = p.K;
+    const int64_t row = blockIdx.x;
+    float r = 0.0f;
+    if constexpr (OP == ROW_RMSNORM) {
+        double ss = 0.0;
+        for (int k = tid; k < K; k += 256) {
+            const double x = (double)load_elem<DT>(p.A, row * p.lda + k);
+            ss += x * x;
+        }
+        ss = wave_sum_f64(ss);
+        if ((tid & 63) == 0) part_d[tid >> 6] = ss;
+        __syncthreads();
+        ss = (part_d[0] + part_d[1]) + (part_d[2] + part_d[3]);
+        r = rms_rstd(ss, K, p.eps);
+    }
+    auto value = [&](int k) {
+        const float a = load_elem<DT>(p.A, row * p.lda + k);
+        if constexpr (OP == ROW_SWIGLU) return swiglu_value(a, load_elem<DT>(p.Bv, row * p.ldb + k), DT);
+        else return rmsnorm_value(a, r, p.Bv ? load_elem<DT>(p.Bv, k) : 1.0f, DT);
+    };
+    if (p.H)
+        for (int k = tid; k < K; k += 256) store_elem<DT>(p.H, row * (int64_t)K + k, value(k));
+    if (!p.Q) return;
+    float amax = 0.0f;
+    for (int k = tid; k < K; k += 256) amax = fmaxf(amax, fabsf(value(k)));
+    amax = wave_max(amax);
+    if ((tid & 63) == 0) part_f[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(part_f[0], part_f[1]), fmaxf(part_f[2], part_f[3]));
+    const float s = (amax > 1e-6f) ? __fdiv_rn(amax, 127.0f) : 1.0f;
+    const float inv = __fdiv_rn(1.0f, s);
+    if (tid == 0) p.s_x[row] = s;
+    for (int k = tid; k < K; k += 256) p.Q[row * (int64_t)K + k] = quant_i8(value(k), inv);
+}
+
+template <int OP, int DT>
+static void launch_row_op_dt(const RowOpParams& p, int64_t B, bool fast, hipStream_t st) {
+    const dim3 grid((unsigned)B), block(256);
+    if (!fast) {
+        hipLaunchKernelGGL((row_op_generic_kernel<OP, DT>), grid, block, 0, st, p);
+        return;
+    }
+    if (p.K <= 2048) hipLaunchKernelGGL((row_op_kernel<OP, DT, 1>), grid, block, 0, st, p);
+    else if (p.K <= 4096) hipLaunchKernelGGL((row_op_kernel<OP, DT, 2>), grid, block, 0, st, p);
+    else if (p.K <= 8192) hipLaunchKernelGGL((row_op_kernel<OP, DT, 4>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((row_op_kernel<OP, DT, 8>), grid, block, 0, st, p);
+}
+
+// op: ROW_SWIGLU / ROW_RMSNORM.  The callers have checked pointers, shapes and dtypes.
+int launch_row_op(int op, int dtype, const void* A, int64_t lda, const void* Bv, int64_t ldb, float eps, int64_t B,
+                  int64_t K, void* H, int8_t* Q, float* s_x, hipStream_t st, const char* who) {
+    RowOpParams p;
+    p.A = A; p.Bv = Bv; p.lda = lda; p.ldb = ldb; p.H = H; p.Q = Q; p.s_x = s_x; p.eps = eps; p.K = (int)K;
+    const int es = dtype_size(dtype);
+    auto aligned = [&](const void* ptr, int64_t ld) { return !ptr || (((uintptr_t)ptr) % 16 == 0 && (ld * es) % 16 == 0); };
+    const bool fast = K % 8 == 0 && K <= 16384 && aligned(A, lda) && aligned(Bv, op == ROW_SWIGLU ? ldb : 8) &&
+                      aligned(H, K) && (!Q || ((uintptr_t)Q) % 8 == 0) && !getenv("BITTORCH_ROWOP_GENERIC");
+    if (op == ROW_SWIGLU) {
+        if (dtype == BT_F32) launch_row_op_dt<ROW_SWIGLU, BT_F32>(p, B, fast, st);
+        else if (dtype == BT_F16) launch_row_op_dt<ROW_SWIGLU, BT_F16>(p, B, fast, st);
+        else launch_row_op_dt<ROW_SWIGLU, BT_BF16>(p, B, fast, st);
+    } else {
+        if (dtype == BT_F32) launch_row_op_dt<ROW_RMSNORM, BT_F32>(p, B, fast, st);
+        else if (dtype == BT_F16) launch_row_op_dt<ROW_RMSNORM, BT_F16>(p, B, fast, st);
+        else launch_row_op_dt<ROW_RMSNORM, BT_BF16>(p, B, fast, st);
+    }
+    return check_launch(who);
+}
+
+}  // namespace bt

@@ -83,6 +83,7 @@ __device__ __forceinline__ void finish_output(const StreamParams& p, int row, in
         // bf16 weights were decoded as +-2.0 (low byte zero): undo exactly
         y = epi_float(__builtin_bit_cast(float, bits) * (p.prehalved ? 1.0f : 0.5f), s, b);
     }
+    if (p.epi.residual) y = add_residual(y, p.epi.residual, p.y_dtype, (int64_t)row * p.N + n);
     store_out(p.Y, p.y_dtype, (int64_t)row * p.N + n, y);
 }
 
@@ -505,6 +506,7 @@ int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, co
         p.Y = (uint8_t*)Y + m0 * N * y_size;
         p.acc_out = acc_out ? acc_out + m0 * N : nullptr;
         p.epi = epi;
+        if (epi.residual) p.epi.residual = (const uint8_t*)epi.residual + m0 * N * y_size;
         p.N = N; p.K = Kx; p.Kb = Kb;
         p.wsteps = (int)ceil_div(Kb, 16);
         p.prehalved = planes == 3;

@@ -30,15 +30,25 @@ class TernaryLinearInference(nn.Module):
         self.register_buffer("bias", bias)
         self.requires_grad_(False)
 
-    def forward(self, x: Tensor) -> Tensor:
+    def forward(self, x: Tensor, residual: Optional[Tensor] = None) -> Tensor:
+        """``residual`` (not in the reference): added to the output, on the GPU inside the kernel."""
         if x.is_cuda:
             from ..ops.ternary_linear_packed import ternary_linear_packed_forward
             return ternary_linear_packed_forward(x, self.weight_packed, self.scale,
-                                                 self.in_features, self.bias)
+                                                 self.in_features, self.bias, residual)
         # CPU (reference :98-104): unpack, fold the scale in, dense product
         w = unpack_ternary_transposed(self.weight_packed, self.in_features).to(x.dtype)
         w = w * self.scale.unsqueeze(1).to(x.dtype)
-        return F.linear(x, w, self.bias)
+        y = F.linear(x, w, self.bias)
+        return y if residual is None else y + residual
+
+    def forward_int8(self, q: Tensor, s_x: Tensor, out_dtype: torch.dtype = torch.bfloat16,
+                     residual: Optional[Tensor] = None) -> Tensor:
+        """Forward from activations already quantized per row to int8 (``ops.rmsnorm`` /
+        ``ops.swiglu`` with ``quantize=True``): int8 matrix cores, int32 accumulators (GPU only)."""
+        from ..ops.fused import ternary_linear_int8
+        return ternary_linear_int8(q, s_x, self.weight_packed, self.scale, self.in_features, self.bias,
+                                   out_dtype, residual)
 
     def extra_repr(self) -> str:
         dense = 4 * self.out_features * self.in_features

@@ -16,13 +16,15 @@ from torch import Tensor
 
 
 def ternary_linear_packed_forward(x: Tensor, w_packed_T: Tensor, scale: Tensor, in_features: int,
-                                  bias: Optional[Tensor] = None) -> Tensor:
-    """``Y = X @ (decode(W_packed_T) * scale).T + bias``; ``x`` is ``(*, K)``."""
+                                  bias: Optional[Tensor] = None, residual: Optional[Tensor] = None) -> Tensor:
+    """``Y = X @ (decode(W_packed_T) * scale).T + bias``; ``x`` is ``(*, K)``.
+
+    ``residual`` (not in the reference) is added to the result inside the kernel."""
     from .. import _C
 
     return _C.ternary_linear_packed_forward(
         x.contiguous(), w_packed_T.contiguous(), scale.contiguous(),
-        None if bias is None else bias.contiguous(), in_features)
+        None if bias is None else bias.contiguous(), in_features, residual)
 
 
 def has_packed_cuda_support() -> bool:

@@ -134,6 +134,43 @@ int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, co
                        void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * The two GEMM entry points above with a residual connection folded into the epilogue:
+ *   Y = rd( rd(linear) + residual ),   rd = round to Y's dtype
+ * i.e. exactly the two roundings of "y = linear(x); y = y + residual" in that dtype.  They have no
+ * counterpart in the reference's Python/CUDA code; they serve the pre-norm block of its JS
+ * runtime (js/src/models/TernaryTransformer.ts:489-521: x = x + attn(norm(x)); x = x + mlp(norm(x))).
+ *   residual: [B,N] in Y's dtype, 16-byte aligned; NULL = no residual (the plain entry point).
+ *   It may be Y itself (every output element is read once, by the thread that then writes it).
+ */
+int bt_ternary_linear_packed_forward_res(const void* X, int x_dtype, const uint8_t* W_T,
+                                         const void* scale, int scale_dtype, int64_t scale_len,
+                                         const void* bias, int bias_dtype, const void* residual,
+                                         void* Y, int64_t B, int64_t N, int64_t K, void* workspace,
+                                         size_t workspace_bytes, void* stream);
+int bt_ternary_gemm_i8_res(const int8_t* Q, const float* s_x, const uint8_t* W_T, const void* scale,
+                           int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
+                           const void* residual, void* Y, int y_dtype, int32_t* acc_out, int64_t B,
+                           int64_t N, int64_t K, void* stream);
+
+/*
+ * Fused producers of the GEMMs' activations (no counterpart in the reference's Python/CUDA code;
+ * block structure of its JS runtime, TernaryTransformer.ts:366-423 and :489-521).  One pass over
+ * the rows computes the value, optionally stores it in the input dtype (H / Y) and optionally
+ * quantizes it per row exactly as bt_act_quant_i8 would quantize the stored tensor (Q, s_x): at
+ * least one of the two outputs must be requested.  rd = round to dtype, fp32 arithmetic, every
+ * operation rounded on its own:
+ *   bt_swiglu:  h = rd( rd( g / (1 + exp(-g)) ) * u )       gate, up [B,K] with row strides
+ *               ld_gate, ld_up (elements; lets both halves of one [B,2K] GEMM output be read in
+ *               place); exp is a fixed fp32 polynomial (0.85 ulp), restated by the CPU oracle.
+ *   bt_rmsnorm: y = rd( (x * r) * w ),  r = 1/sqrt(float(sum double(x)^2)/K + eps)
+ *               weight [K] in the same dtype or NULL (ones).
+ */
+int bt_swiglu(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, int dtype, int64_t B,
+              int64_t K, void* H, int8_t* Q, float* s_x, void* stream);
+int bt_rmsnorm(const void* X, int64_t ld_x, const void* weight, float eps, int dtype, int64_t B,
+               int64_t K, void* Y, int8_t* Q, float* s_x, void* stream);
+
+/*
  * Matrix-core forward from float activations: bt_act_quant_i8 followed by
  * bt_ternary_gemm_i8.  Replaces bittorch._C.ternary_linear_tensor_core_forward
  * (bittorch_bindings.cpp:65-87, ternary_gemm_tensor_core.cu:663-727) for

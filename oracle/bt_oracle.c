@@ -22,6 +22,12 @@
  *                       force on tiny inputs, exact integer identities and
  *                       agreement with the float path inside the int8
  *                       quantisation error bound.
+ *   bto_swiglu          no counterpart in the reference's Python/CUDA code (the
+ *   bto_rmsnorm         block glue lives in its JS runtime, in float64 maths):
+ *   bto_exp_fixed       these restate THIS library's fused row operations so
+ *                       that the kernels can be diffed bit for bit; pinned by
+ *                       float64 closed forms (silu, exp, rms) to a stated
+ *                       tolerance and by torch's own ops in the tests.
  *
  * Build: gcc -O2 -fPIC -shared -ffp-contract=off -fopenmp (see Makefile).
  * -ffp-contract=off keeps every multiply and add separately rounded, which is
@@ -31,6 +37,7 @@
 #include <stdint.h>
 #include <stddef.h>
 #include <string.h>
+#include <stdlib.h>
 
 /* dtype tags shared with include/bittorch_hip.h */
 enum { BTO_F32 = 0, BTO_F16 = 1, BTO_BF16 = 2 };
@@ -336,5 +343,85 @@ void bto_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const fl
             r = r + bv;
             Y[b * N + n] = r;
         }
+    }
+}
+
+/* ---- fused row operations (restating bittorch_amd/csrc/row_ops.hip) -------------------- */
+
+/* exp(a) by a fixed sequence of correctly rounded fp32 operations: +inf above 88.7228, a clamped to -87 below,
+ * n = rint(a*log2(e)), r = a - n*ln2 (two-part ln2, fused), degree-7 Taylor polynomial in Horner
+ * form with fused multiply-adds, then two exact power-of-two scalings. */
+float bto_exp_fixed(float a) {
+    if (!(a == a)) return a;
+    if (a > 88.7228f) return INFINITY;  /* exp overflows fp32 */
+    a = fmaxf(a, -87.0f);
+    const float n = rintf(a * 1.44269504088896341f);
+    float r = fmaf(n, -0.693145751953125f, a);
+    r = fmaf(n, -1.42860682030941723212e-6f, r);
+    float p = 1.0f / 5040.0f;
+    p = fmaf(p, r, 1.0f / 720.0f);
+    p = fmaf(p, r, 1.0f / 120.0f);
+    p = fmaf(p, r, 1.0f / 24.0f);
+    p = fmaf(p, r, 1.0f / 6.0f);
+    p = fmaf(p, r, 0.5f);
+    p = fmaf(p, r, 1.0f);
+    p = fmaf(p, r, 1.0f);
+    const int ni = (int)n;
+    const int n1 = ni / 2, n2 = ni - n1;
+    uint32_t u1 = (uint32_t)(n1 + 127) << 23, u2 = (uint32_t)(n2 + 127) << 23;
+    float s1, s2;
+    memcpy(&s1, &u1, 4);
+    memcpy(&s2, &u2, 4);
+    return (p * s1) * s2;
+}
+
+static void quant_row_i8(const float* v, int64_t K, int8_t* q, float* s_out) {
+    float amax = 0.0f;
+    for (int64_t k = 0; k < K; k++) amax = fmaxf(amax, fabsf(v[k]));
+    const float s = (amax > 1e-6f) ? (amax / 127.0f) : 1.0f;
+    const float inv = 1.0f / s;
+    *s_out = s;
+    for (int64_t k = 0; k < K; k++) q[k] = (int8_t)fmaxf(-127.0f, fminf(127.0f, roundf(v[k] * inv)));
+}
+
+/* SwiGLU of the block's MLP (js/src/models/TernaryTransformer.ts:366-423: silu(gate) * up):
+ *   h = rd( rd( g / (1 + exp_fixed(-g)) ) * u ),  rd = round to dtype
+ * gate / up are fp32 arrays holding values already on the dtype's grid.  H (nullable) receives h
+ * as fp32; Q / s_x (nullable) the per-row int8 quantisation of h (same formulas as
+ * bto_act_quant_i8). */
+void bto_swiglu(const float* gate, const float* up, int dtype, int64_t B, int64_t K, float* H, int8_t* Q,
+                float* s_x) {
+#pragma omp parallel for schedule(static)
+    for (int64_t b = 0; b < B; b++) {
+        float* v = (float*)malloc((size_t)K * sizeof(float));
+        for (int64_t k = 0; k < K; k++) {
+            const float g = gate[b * K + k];
+            const float e = bto_exp_fixed(-g);
+            const float sl = round_to_dtype(g / (1.0f + e), dtype);
+            v[k] = round_to_dtype(sl * up[b * K + k], dtype);
+        }
+        if (H) memcpy(H + b * K, v, (size_t)K * sizeof(float));
+        if (Q) quant_row_i8(v, K, Q + b * K, s_x + b);
+        free(v);
+    }
+}
+
+/* RMSNorm of the pre-norm block (TernaryTransformer.ts:489-521):
+ *   ss = float( sum_k double(x_k)^2 );  r = 1 / sqrtf(ss / K + eps);  y_k = rd( (x_k * r) * w_k )
+ * weight may be null (all ones). */
+void bto_rmsnorm(const float* X, const float* weight, float eps, int dtype, int64_t B, int64_t K, float* Y,
+                 int8_t* Q, float* s_x) {
+#pragma omp parallel for schedule(static)
+    for (int64_t b = 0; b < B; b++) {
+        float* v = (float*)malloc((size_t)K * sizeof(float));
+        double ss = 0.0;
+        for (int64_t k = 0; k < K; k++) ss += (double)X[b * K + k] * (double)X[b * K + k];
+        const float ms = (float)ss / (float)K;
+        const float r = 1.0f / sqrtf(ms + eps);
+        for (int64_t k = 0; k < K; k++)
+            v[k] = round_to_dtype((X[b * K + k] * r) * (weight ? weight[k] : 1.0f), dtype);
+        if (Y) memcpy(Y + b * K, v, (size_t)K * sizeof(float));
+        if (Q) quant_row_i8(v, K, Q + b * K, s_x + b);
+        free(v);
     }
 }

@@ -53,6 +53,10 @@ def lib() -> ctypes.CDLL:
         _lib.bto_linear_unpacked.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64]
         _lib.bto_act_quant_i8.argtypes = [_vp, _i64, _i64, _vp, _vp]
         _lib.bto_gemm_i8.argtypes = [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64]
+        _lib.bto_exp_fixed.restype = ctypes.c_float
+        _lib.bto_exp_fixed.argtypes = [ctypes.c_float]
+        _lib.bto_swiglu.argtypes = [_vp, _vp, ctypes.c_int, _i64, _i64, _vp, _vp, _vp]
+        _lib.bto_rmsnorm.argtypes = [_vp, _vp, ctypes.c_float, ctypes.c_int, _i64, _i64, _vp, _vp, _vp]
     return _lib
 
 
@@ -188,3 +192,31 @@ def linear_i8(x, w_packed_t, scale, in_features: int, bias=None):
     q, s = act_quant_i8(x)
     acc, y = gemm_i8(q, s, w_packed_t, scale, in_features, bias)
     return q, s, acc, y
+
+
+def exp_fixed(a: float) -> float:
+    """The fixed-sequence fp32 exp the fused SwiGLU uses."""
+    return float(lib().bto_exp_fixed(float(a)))
+
+
+def swiglu(gate, up, dtype: int = 0):
+    """(h f32 [B,K] on the dtype's grid, q int8 [B,K], s_x f32 [B]) of silu(gate)*up."""
+    gate, up = _f32(gate), _f32(up)
+    b, k = gate.shape
+    h = np.empty((b, k), dtype=np.float32)
+    q = np.empty((b, k), dtype=np.int8)
+    s = np.empty((b,), dtype=np.float32)
+    lib().bto_swiglu(_p(gate), _p(up), dtype, b, k, _p(h), _p(q), _p(s))
+    return h, q, s
+
+
+def rmsnorm(x, weight=None, eps: float = 1e-6, dtype: int = 0):
+    """(y f32 [B,K] on the dtype's grid, q int8 [B,K], s_x f32 [B]) of RMSNorm(x) * weight."""
+    x = _f32(x)
+    weight = None if weight is None else _f32(weight).reshape(-1)
+    b, k = x.shape
+    y = np.empty((b, k), dtype=np.float32)
+    q = np.empty((b, k), dtype=np.int8)
+    s = np.empty((b,), dtype=np.float32)
+    lib().bto_rmsnorm(_p(x), _p(weight), eps, dtype, b, k, _p(y), _p(q), _p(s))
+    return y, q, s

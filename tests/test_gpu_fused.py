@@ -1,0 +1,230 @@
+"""GPU parity of the fused block glue: SwiGLU, RMSNorm (each with the optional per-row int8
+quantization) and the residual folded into the GEMM epilogues.
+
+* against the CPU oracle: bit-exact (values on the dtype's grid, int8 codes, activation scales);
+* against torch's own unfused ops on the GPU: equal up to one unit in the last place of the
+  tensor dtype (torch's silu uses the device library's exp, this library a fixed polynomial);
+* the residual: bit-exact against "linear, then add" on every kernel path.
+"""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from conftest import announce
+from _util import BT_DT, f32np, random_ternary, seeded_acts
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.float16, torch.bfloat16]
+# fast path (row in registers), K % 8 != 0 (generic), largest fast K, beyond it (generic)
+SHAPES = [(1, 8), (3, 7), (5, 520), (16, 4096), (4, 6912), (2, 16384), (2, 20000)]
+
+
+def _ulp_close(got, ref, dtype, ulps=1):
+    got, ref = got.float(), ref.float()
+    if dtype == torch.float32:
+        tol = torch.abs(ref) * (ulps * 2.0 ** -23) + 1e-37
+    elif dtype == torch.float16:
+        tol = torch.clamp(torch.abs(ref) * (ulps * 2.0 ** -10), min=ulps * 2.0 ** -24)
+    else:
+        tol = torch.abs(ref) * (ulps * 2.0 ** -7) + 1e-37
+    bad = torch.abs(got - ref) > tol
+    return int(bad.sum())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("b,k", SHAPES)
+def test_swiglu_matches_oracle_bit_for_bit(oracle, dtype, b, k):
+    from bittorch_amd import _C
+    announce("swiglu", dtype, b, k)
+    g = seeded_acts(b, k, seed=b + k, dtype=dtype, outliers=True) * 3
+    u = seeded_acts(b, k, seed=b + k + 1, dtype=dtype)
+    if b > 2:
+        u[1] = 0  # all-zero product row: scale 1, codes 0
+    h, q, s = _C.swiglu(g.cuda(), u.cuda(), store=True, quantize=True)
+    torch.cuda.synchronize()
+    oh, oq, os_ = oracle.swiglu(f32np(g), f32np(u), BT_DT[dtype])
+    np.testing.assert_array_equal(f32np(h), oh)
+    np.testing.assert_array_equal(s.cpu().numpy(), os_)
+    np.testing.assert_array_equal(q.cpu().numpy(), oq)
+    # the quantized output alone, and the stored output alone, are the same values
+    q2, s2 = _C.swiglu(g.cuda(), u.cuda(), store=False, quantize=True)
+    h2 = _C.swiglu(g.cuda(), u.cuda())
+    assert torch.equal(q2, q) and torch.equal(s2, s) and torch.equal(h2, h)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu_against_torch_ops(dtype):
+    from bittorch_amd import _C
+    announce("swiglu vs torch", dtype)
+    g = (seeded_acts(64, 6912, seed=3, dtype=dtype, outliers=True) * 3).cuda()
+    u = seeded_acts(64, 6912, seed=4, dtype=dtype).cuda()
+    ref = F.silu(g) * u
+    got = _C.swiglu(g, u)
+    # fp32: two different exp implementations (each below 1 ulp), one add, one divide, one multiply
+    assert _ulp_close(got, ref, dtype, ulps=4 if dtype == torch.float32 else 1) == 0
+    # and the fused quantization is the stand-alone quantizer applied to the stored product
+    q, s = _C.swiglu(g, u, store=False, quantize=True)
+    q_ref, s_ref = _C.act_quant_int8(got)
+    assert torch.equal(q, q_ref) and torch.equal(s, s_ref)
+
+
+def test_swiglu_special_values():
+    from bittorch_amd import _C
+    g = torch.tensor([[0.0, -0.0, 100.0, -100.0, 1e-30, float("inf"), -float("inf"), float("nan")]]).cuda()
+    u = torch.ones_like(g)
+    h = _C.swiglu(g, u).cpu()[0]
+    assert h[0] == 0 and h[1] == 0 and h[2] == 100.0
+    assert h[3] == 0                         # -100 / (1 + inf): exp(100) overflows fp32, as in torch
+    assert float(h[4]) == pytest.approx(0.5e-30, rel=1e-6)
+    assert h[5] == float("inf")
+    assert torch.isnan(h[6]) or h[6] == 0    # -inf * 0
+    assert torch.isnan(h[7])
+
+
+def test_swiglu_reads_halves_of_one_wide_matrix_in_place(oracle):
+    from bittorch_amd import _C
+    announce("swiglu strided")
+    gu = seeded_acts(33, 2 * 1024, seed=9, dtype=torch.bfloat16).cuda()
+    g, u = gu[:, :1024], gu[:, 1024:]
+    h = _C.swiglu(g, u)
+    assert torch.equal(h, _C.swiglu(g.contiguous(), u.contiguous()))
+    oh, _, _ = oracle.swiglu(f32np(g), f32np(u), BT_DT[torch.bfloat16])
+    np.testing.assert_array_equal(f32np(h), oh)
+    # 3-D inputs keep their leading shape
+    h3, q3, s3 = _C.swiglu(g.contiguous().view(3, 11, 1024), u.contiguous().view(3, 11, 1024), True, True)
+    assert h3.shape == (3, 11, 1024) and q3.shape == (3, 11, 1024) and s3.shape == (3, 11)
+    assert torch.equal(h3.view(33, 1024), h)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("b,k", SHAPES)
+@pytest.mark.parametrize("with_weight", [True, False])
+def test_rmsnorm_matches_oracle_bit_for_bit(oracle, dtype, b, k, with_weight):
+    from bittorch_amd import _C
+    announce("rmsnorm", dtype, b, k, with_weight)
+    x = seeded_acts(b, k, seed=b + k + 5, dtype=dtype, outliers=True)
+    if b > 2:
+        x[1] = 0  # all-zero row: rsqrt(eps), outputs 0
+    w = (1 + 0.1 * torch.randn(k, generator=torch.Generator().manual_seed(k))).to(dtype) if with_weight else None
+    eps = 1e-5
+    y, q, s = _C.rmsnorm(x.cuda(), None if w is None else w.cuda(), eps, store=True, quantize=True)
+    torch.cuda.synchronize()
+    oy, oq, os_ = oracle.rmsnorm(f32np(x), None if w is None else f32np(w), eps, BT_DT[dtype])
+    np.testing.assert_array_equal(f32np(y), oy)
+    np.testing.assert_array_equal(s.cpu().numpy(), os_)
+    np.testing.assert_array_equal(q.cpu().numpy(), oq)
+    q2, s2 = _C.rmsnorm(x.cuda(), None if w is None else w.cuda(), eps, store=False, quantize=True)
+    assert torch.equal(q2, q) and torch.equal(s2, s)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_against_torch(dtype):
+    from bittorch_amd import _C
+    announce("rmsnorm vs torch", dtype)
+    x = seeded_acts(64, 2560, seed=7, dtype=dtype, outliers=True).cuda()
+    w = (1 + 0.1 * torch.randn(2560, generator=torch.Generator().manual_seed(1))).to(dtype).cuda()
+    got = _C.rmsnorm(x, w, 1e-5)
+    ref64 = (x.double() * torch.rsqrt(x.double().pow(2).mean(-1, keepdim=True) + 1e-5) * w.double())
+    assert _ulp_close(got, ref64.to(dtype), dtype, ulps=2 if dtype == torch.float32 else 1) == 0
+    ref_t = F.rms_norm(x, (2560,), w, 1e-5)
+    assert _ulp_close(got, ref_t, dtype, ulps=4 if dtype == torch.float32 else 2) == 0
+
+
+def _packed_case(n, k, seed=0):
+    from bittorch_amd.quant import pack_ternary_transposed
+    w = random_ternary(n, k, seed=seed)
+    packed = pack_ternary_transposed(w)[0].cuda()
+    g = torch.Generator().manual_seed(seed + 1)
+    scale = (torch.rand(n, generator=g) * 0.05 + 0.01).cuda()
+    bias = (torch.randn(n, generator=g) * 0.01).cuda()
+    return packed, scale, bias
+
+
+# (B, N, K): streaming kernel, tiled 16-bit GEMM (whole and ragged tiles), generic shapes
+RES_SHAPES = [(1, 4096, 4096), (16, 1000, 520), (33, 256, 128), (200, 520, 192), (130, 260, 70), (5, 37, 23)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("b,n,k", RES_SHAPES)
+def test_residual_in_packed_forward_equals_linear_then_add(dtype, b, n, k):
+    from bittorch_amd import _C
+    announce("residual packed", dtype, b, n, k)
+    packed, scale, bias = _packed_case(n, k, seed=b + n)
+    x = seeded_acts(b, k, seed=3, dtype=dtype).cuda()
+    res = seeded_acts(b, n, seed=4, dtype=dtype).cuda()
+    y = _C.ternary_linear_packed_forward(x, packed, scale, bias, k)
+    fused = _C.ternary_linear_packed_forward(x, packed, scale, bias, k, res)
+    assert torch.equal(fused, y + res)
+
+
+@pytest.mark.parametrize("out_dtype", DTYPES)
+@pytest.mark.parametrize("b,n,k", [(1, 4096, 4096), (16, 1000, 520), (200, 520, 256), (130, 260, 80)])
+def test_residual_in_int8_gemm_equals_linear_then_add(out_dtype, b, n, k):
+    from bittorch_amd import _C
+    announce("residual int8", out_dtype, b, n, k)
+    packed, scale, bias = _packed_case(n, k, seed=b + n)
+    x = seeded_acts(b, k, seed=5, dtype=torch.bfloat16, outliers=True).cuda()
+    res = seeded_acts(b, n, seed=6, dtype=out_dtype).cuda()
+    q, s = _C.act_quant_int8(x)
+    y = _C.ternary_gemm_int8(q, s, packed, scale, bias, k, out_dtype)
+    fused = _C.ternary_gemm_int8(q, s, packed, scale, bias, k, out_dtype, residual=res)
+    assert torch.equal(fused, y + res)
+
+
+def test_residual_on_the_generic_kernel(monkeypatch):
+    from bittorch_amd import _C
+    monkeypatch.setenv("BITTORCH_KERNEL", "generic")
+    packed, scale, bias = _packed_case(260, 70, seed=2)
+    x = seeded_acts(9, 70, seed=3).cuda()
+    res = seeded_acts(9, 260, seed=4).cuda()
+    y = _C.ternary_linear_packed_forward(x, packed, scale, bias, 70)
+    assert torch.equal(_C.ternary_linear_packed_forward(x, packed, scale, bias, 70, res), y + res)
+
+
+def test_residual_argument_errors():
+    from bittorch_amd import _C
+    packed, scale, bias = _packed_case(64, 32)
+    x = seeded_acts(4, 32, dtype=torch.float16).cuda()
+    with pytest.raises(RuntimeError, match="residual shape"):
+        _C.ternary_linear_packed_forward(x, packed, scale, bias, 32, torch.zeros(4, 63, dtype=torch.float16).cuda())
+    with pytest.raises(RuntimeError, match="residual must have the output's dtype"):
+        _C.ternary_linear_packed_forward(x, packed, scale, bias, 32, torch.zeros(4, 64).cuda())
+    with pytest.raises(RuntimeError, match="nothing to compute"):
+        _C.swiglu(x, x, store=False, quantize=False)
+    with pytest.raises(RuntimeError, match="gate and up must match"):
+        _C.swiglu(x, x[:, :16])
+
+
+@pytest.mark.parametrize("compute", ["float", "int8"])
+def test_ternary_swiglu_module_equals_its_unfused_composition(compute):
+    import bittorch_amd as bt
+    from bittorch_amd import _C
+    announce("TernarySwiGLU", compute)
+    d, ffn, tokens = 256, 640, 48
+    mk = lambda i, o, seed: bt.nn.create_ternary_linear_inference(
+        i, o, (torch.randn(o, i, generator=torch.Generator().manual_seed(seed)) * 0.02).cuda())
+    gate, up, down = mk(d, ffn, 1), mk(d, ffn, 2), mk(ffn, d, 3)
+    mlp = bt.nn.TernarySwiGLU(gate, up, down, compute=compute)
+    x = seeded_acts(tokens, d, seed=8, dtype=torch.bfloat16).cuda()
+    nw = (1 + 0.1 * torch.randn(d, generator=torch.Generator().manual_seed(4))).bfloat16().cuda()
+    got = mlp(x, nw, 1e-5, residual=x)
+    h = _C.rmsnorm(x, nw, 1e-5)
+    if compute == "float":
+        ref = down(_C.swiglu(gate(h), up(h))) + x
+    else:
+        q, s = _C.act_quant_int8(h)
+        g = _C.ternary_gemm_int8(q, s, gate.weight_packed, gate.scale, None, d, torch.bfloat16)
+        u = _C.ternary_gemm_int8(q, s, up.weight_packed, up.scale, None, d, torch.bfloat16)
+        q2, s2 = _C.act_quant_int8(_C.swiglu(g, u))
+        ref = _C.ternary_gemm_int8(q2, s2, down.weight_packed, down.scale, None, ffn, torch.bfloat16) + x
+    assert torch.equal(got, ref)
+    # and against plain torch glue around the same layers, to bf16 accuracy
+    ht = F.rms_norm(x, (d,), nw, 1e-5)
+    ref_t = down(F.silu(gate(ht)) * up(ht)) + x
+    err = (got.float() - ref_t.float()).abs().max() / ref_t.float().abs().max()
+    assert err < (2e-2 if compute == "float" else 6e-2)
+    # without a norm the input itself is the activation
+    got2 = mlp(x)
+    assert got2.shape == (tokens, d) and torch.isfinite(got2.float()).all()

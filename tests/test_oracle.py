@@ -259,3 +259,71 @@ def test_round_helpers_match_torch(oracle):
     for v in vals:
         assert oracle.round_to_dtype(v, 1) == float(torch.tensor(v, dtype=torch.float32).half().float())
         assert oracle.round_to_dtype(v, 2) == float(torch.tensor(v, dtype=torch.float32).bfloat16().float())
+
+
+# ---- fused row operations (this library's own glue; pinned by float64 closed forms) ------------
+
+def test_exp_fixed_is_within_one_ulp_of_exp(oracle):
+    rng = np.random.default_rng(0)
+    xs = np.concatenate([np.linspace(-87, 88.72, 4001), rng.normal(0, 4, 4000), [0.0, -0.0, 1.0, -1.0]])
+    xs = xs.astype(np.float32)
+    got = np.array([oracle.exp_fixed(float(x)) for x in xs], dtype=np.float64)
+    ref = np.exp(xs.astype(np.float64))
+    ulp = np.spacing(ref.astype(np.float32)).astype(np.float64)
+    assert np.max(np.abs(got - ref) / ulp) < 1.0
+    assert oracle.exp_fixed(0.0) == 1.0
+    assert np.isnan(oracle.exp_fixed(float("nan")))
+    # overflows like exp; saturates at exp(-87) below (callers only ever add it to 1)
+    assert oracle.exp_fixed(1000.0) == float("inf") and oracle.exp_fixed(88.8) == float("inf")
+    assert oracle.exp_fixed(88.72) < np.finfo(np.float32).max
+    assert oracle.exp_fixed(-1000.0) == oracle.exp_fixed(-87.0) > 0
+
+
+@pytest.mark.parametrize("dtype,rel", [(0, 3e-7), (1, 1.0 / 1024), (2, 1.0 / 128)])
+def test_swiglu_oracle_against_float64_closed_form(oracle, dtype, rel):
+    rng = np.random.default_rng(1)
+    g = (rng.normal(0, 3, (7, 130))).astype(np.float32)
+    u = rng.normal(0, 1, (7, 130)).astype(np.float32)
+    if dtype:
+        td = torch.float16 if dtype == 1 else torch.bfloat16
+        g = torch.from_numpy(g).to(td).float().numpy()
+        u = torch.from_numpy(u).to(td).float().numpy()
+    h, q, s = oracle.swiglu(g, u, dtype)
+    ref = g.astype(np.float64) / (1 + np.exp(-g.astype(np.float64))) * u
+    assert np.all(np.abs(h - ref) <= rel * np.abs(ref) + 1e-30)
+    # a swapped operand or a missing silu would fail this: silu(g)*u != silu(u)*g in general
+    assert not np.allclose(h, u / (1 + np.exp(-u)) * g, rtol=1e-2)
+    # the quantization is the stand-alone quantizer applied to h
+    q_ref, s_ref = oracle.act_quant_i8(h)
+    np.testing.assert_array_equal(q, q_ref)
+    np.testing.assert_array_equal(s, s_ref)
+    # exact special cases: g = 0 gives 0; u = 0 gives 0
+    h0, _, s0 = oracle.swiglu(np.zeros((1, 8), np.float32), np.ones((1, 8), np.float32), dtype)
+    assert np.all(h0 == 0) and s0[0] == 1.0
+
+
+@pytest.mark.parametrize("dtype,rel", [(0, 3e-7), (1, 1.0 / 1024), (2, 1.0 / 128)])
+def test_rmsnorm_oracle_against_float64_closed_form(oracle, dtype, rel):
+    rng = np.random.default_rng(2)
+    x = rng.normal(0, 2, (5, 257)).astype(np.float32)
+    w = (1 + 0.1 * rng.normal(0, 1, 257)).astype(np.float32)
+    if dtype:
+        td = torch.float16 if dtype == 1 else torch.bfloat16
+        x = torch.from_numpy(x).to(td).float().numpy()
+        w = torch.from_numpy(w).to(td).float().numpy()
+    eps = 1e-5
+    y, q, s = oracle.rmsnorm(x, w, eps, dtype)
+    x64 = x.astype(np.float64)
+    ref = x64 / np.sqrt((x64 ** 2).mean(-1, keepdims=True) + eps) * w
+    assert np.all(np.abs(y - ref) <= rel * np.abs(ref) + 1e-30)
+    y1, _, _ = oracle.rmsnorm(x, None, eps, dtype)
+    ref1 = x64 / np.sqrt((x64 ** 2).mean(-1, keepdims=True) + eps)
+    assert np.all(np.abs(y1 - ref1) <= rel * np.abs(ref1) + 1e-30)
+    # invariant: without weight the output rows have unit RMS (up to eps and rounding)
+    assert np.allclose(np.sqrt((y1.astype(np.float64) ** 2).mean(-1)), 1.0, rtol=5 * rel + 1e-5)
+    # a constant row c maps to sign(c) * w (eps negligible)
+    yc, _, _ = oracle.rmsnorm(np.full((1, 257), -3.0, np.float32), w, 1e-12, 0)
+    assert np.allclose(yc[0], -w, rtol=1e-6)
+    q_ref, s_ref = oracle.act_quant_i8(y)
+    np.testing.assert_array_equal(q, q_ref)
+    np.testing.assert_array_equal(s, s_ref)
