@@ -118,7 +118,8 @@ __device__ __forceinline__ void store8(void* base, int64_t idx, const float (&v)
 
 // One workgroup per row, the row held in registers: the operands are read once, the outputs
 // written once.  Needs K % 8 == 0, K <= 2048*ITERS, 16-byte aligned rows.
-template <int OP, int DT, int ITERS>
+// QUANT = false: nothing outlives the store of an element, so SwiGLU streams through few registers.
+template <int OP, int DT, int ITERS, bool QUANT>
 __global__ __launch_bounds__(256) void row_op_kernel(RowOpParams p) {
     __shared__ double part_d[4];
     __shared__ float part_f[4];
@@ -173,7 +174,7 @@ __global__ __launch_bounds__(256) void row_op_kernel(RowOpParams p) {
             if (k < K) store8<DT>(p.H, row * (int64_t)K + k, v[i]);
         }
     }
-    if (!p.Q) return;  // uniform
+    if constexpr (!QUANT) return;
     float amax = 0.0f;
 #pragma unroll
     for (int i = 0; i < ITERS; i++) {
@@ -244,6 +245,16 @@ __global__ __launch_bounds__(256) void row_op_generic_kernel(RowOpParams p) {
     for (int k = tid; k < K; k += 256) p.Q[row * (int64_t)K + k] = quant_i8(value(k), inv);
 }
 
+template <int OP, int DT, bool QUANT>
+static void launch_row_op_iters(const RowOpParams& p, dim3 grid, dim3 block, hipStream_t st) {
+    if (p.K <= 2048) hipLaunchKernelGGL((row_op_kernel<OP, DT, 1, QUANT>), grid, block, 0, st, p);
+    else if (p.K <= 4096) hipLaunchKernelGGL((row_op_kernel<OP, DT, 2, QUANT>), grid, block, 0, st, p);
+    else if (p.K <= 6144) hipLaunchKernelGGL((row_op_kernel<OP, DT, 3, QUANT>), grid, block, 0, st, p);
+    else if (p.K <= 8192) hipLaunchKernelGGL((row_op_kernel<OP, DT, 4, QUANT>), grid, block, 0, st, p);
+    else if (p.K <= 12288) hipLaunchKernelGGL((row_op_kernel<OP, DT, 6, QUANT>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((row_op_kernel<OP, DT, 8, QUANT>), grid, block, 0, st, p);
+}
+
 template <int OP, int DT>
 static void launch_row_op_dt(const RowOpParams& p, int64_t B, bool fast, hipStream_t st) {
     const dim3 grid((unsigned)B), block(256);
@@ -251,10 +262,8 @@ static void launch_row_op_dt(const RowOpParams& p, int64_t B, bool fast, hipStre
         hipLaunchKernelGGL((row_op_generic_kernel<OP, DT>), grid, block, 0, st, p);
         return;
     }
-    if (p.K <= 2048) hipLaunchKernelGGL((row_op_kernel<OP, DT, 1>), grid, block, 0, st, p);
-    else if (p.K <= 4096) hipLaunchKernelGGL((row_op_kernel<OP, DT, 2>), grid, block, 0, st, p);
-    else if (p.K <= 8192) hipLaunchKernelGGL((row_op_kernel<OP, DT, 4>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((row_op_kernel<OP, DT, 8>), grid, block, 0, st, p);
+    if (p.Q) launch_row_op_iters<OP, DT, true>(p, grid, block, st);
+    else launch_row_op_iters<OP, DT, false>(p, grid, block, st);
 }
 
 // op: ROW_SWIGLU / ROW_RMSNORM.  The callers have checked pointers, shapes and dtypes.
