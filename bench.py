@@ -155,7 +155,8 @@ def block_stack(torch, dev, layers=30, d_model=2560, heads=20, ffn=6912, batch=8
     # (parity of every fused piece against its unfused sequence is a GPU test; end-to-end outputs of 30
     # random layers differ chaotically on any last-bit change and are not compared here)
     # the same converted stack with the glue between the ternary layers fused: residual adds in the
-    # GEMM epilogues, silu(gate)*up in one kernel, RMSNorm from this library ...
+    # GEMM epilogues, silu(gate)*up in one kernel, RMSNorm from this library, q|k|v and gate|up each
+    # one GEMM over concatenated columns (fewer, fuller waves of tiles) ...
     from bittorch_amd.ops import fused
 
     def heads_of(t, b, s):
@@ -166,10 +167,10 @@ def block_stack(torch, dev, layers=30, d_model=2560, heads=20, ffn=6912, batch=8
         if int8:  # ... and, BitNet-style, every projection on the int8 matrix cores from activations
             # that leave the norm / SwiGLU kernels already quantized per token
             qh, sh = fused.rmsnorm(x, blk.n1.weight, blk.n1.eps or torch.finfo(x.dtype).eps, store=False, quantize=True)
-            q, k, v = (m.forward_int8(qh, sh, x.dtype) for m in (blk.q, blk.k, blk.v))
+            qkv = blk.qkv.forward_int8(qh, sh, x.dtype)
         else:
-            h = fused.rmsnorm(x, blk.n1.weight, blk.n1.eps or torch.finfo(x.dtype).eps)
-            q, k, v = blk.q(h), blk.k(h), blk.v(h)
+            qkv = blk.qkv(fused.rmsnorm(x, blk.n1.weight, blk.n1.eps or torch.finfo(x.dtype).eps))
+        q, k, v = qkv.split(d_model, dim=-1)  # one GEMM over the concatenated q|k|v columns
         a = F.scaled_dot_product_attention(heads_of(q, b, s), heads_of(k, b, s), heads_of(v, b, s), is_causal=True)
         a = a.transpose(1, 2).reshape(b, s, -1)
         if int8:
@@ -198,7 +199,8 @@ def block_stack(torch, dev, layers=30, d_model=2560, heads=20, ffn=6912, batch=8
         return best
 
     for blk in infer:
-        blk.mlp = bt.nn.TernarySwiGLU(blk.gate, blk.up, blk.down, compute="float")
+        blk.qkv = bt.utils.fuse_ternary_linear_inference(blk.q, blk.k, blk.v)
+        blk.mlp = bt.nn.TernarySwiGLU(blk.gate, blk.up, blk.down, compute="float", fuse_gate_up=True)
     res["ms_inference_fused_glue"] = round(timed_fused(False), 3)
     for blk in infer:
         blk.mlp.compute = "int8"

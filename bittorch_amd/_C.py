@@ -346,8 +346,11 @@ def _row_op_result(h, q, s, lead_shape, K):
 
 def _rows_2d(t: Tensor, K: int) -> Tensor:
     """A 2-D view with unit inner stride (row stride kept: slices of a wider matrix stay in place)."""
-    if t.dim() == 2 and t.stride(1) == 1 and t.stride(0) >= K:
-        return t
+    if t.stride(-1) == 1 and t.dim() >= 2 and t.stride(-2) >= K:
+        lead_ok = all(t.stride(i) == t.stride(i + 1) * t.shape[i + 1] for i in range(t.dim() - 2))
+        if lead_ok:  # the leading dimensions collapse into one row index with a single stride
+            rows = t.numel() // K
+            return t if t.dim() == 2 else t.as_strided((rows, K), (t.stride(-2), 1), t.storage_offset())
     return t.contiguous().reshape(-1, K)
 
 

@@ -19,16 +19,39 @@ from .ternary_linear_infer import TernaryLinearInference
 
 
 class TernarySwiGLU(nn.Module):
+    """``fuse_gate_up=True`` stores gate and up as one layer of ``2 * ffn`` columns (one GEMM launch;
+    SwiGLU then reads the two halves of its output in place)."""
+
     def __init__(self, gate: TernaryLinearInference, up: TernaryLinearInference, down: TernaryLinearInference,
-                 compute: str = "float"):
+                 compute: str = "float", fuse_gate_up: bool = False):
         super().__init__()
         if compute not in ("float", "int8"):
             raise ValueError(f"compute must be 'float' or 'int8', got {compute!r}")
         if not (gate.in_features == up.in_features and gate.out_features == up.out_features
                 and down.in_features == gate.out_features):
             raise ValueError("gate/up/down shapes do not form an MLP")
-        self.gate, self.up, self.down = gate, up, down
+        self.ffn = gate.out_features
         self.compute = compute
+        self.down = down
+        if fuse_gate_up:
+            from ..utils.convert import fuse_ternary_linear_inference
+            self.gate_up = fuse_ternary_linear_inference(gate, up)
+            self.gate = self.up = None
+        else:
+            self.gate_up = None
+            self.gate, self.up = gate, up
+
+    def _gate_up(self, h: Tensor):
+        if self.gate_up is None:
+            return self.gate(h), self.up(h)
+        gu = self.gate_up(h)
+        return gu[..., :self.ffn], gu[..., self.ffn:]
+
+    def _gate_up_int8(self, q: Tensor, s: Tensor, dtype):
+        if self.gate_up is None:
+            return self.gate.forward_int8(q, s, dtype), self.up.forward_int8(q, s, dtype)
+        gu = self.gate_up.forward_int8(q, s, dtype)
+        return gu[..., :self.ffn], gu[..., self.ffn:]
 
     def forward(self, x: Tensor, norm_weight: Optional[Tensor] = None, eps: Optional[float] = None,
                 residual: Optional[Tensor] = None) -> Tensor:
@@ -39,17 +62,17 @@ class TernarySwiGLU(nn.Module):
         if not x.is_cuda:
             import torch.nn.functional as F
             h = x if eps is None else F.rms_norm(x, (x.shape[-1],), norm_weight, eps)
-            return self.down(F.silu(self.gate(h)) * self.up(h), residual)
+            g, u = self._gate_up(h)
+            return self.down(F.silu(g) * u, residual)
         if self.compute == "float":
             h = x if eps is None else fused.rmsnorm(x, norm_weight, eps)
-            return self.down(fused.swiglu(self.gate(h), self.up(h)), residual)
+            return self.down(fused.swiglu(*self._gate_up(h)), residual)
         if eps is None:
             from .. import _C
             q, s = _C.act_quant_int8(x.reshape(-1, x.shape[-1]))
             q, s = q.reshape(x.shape), s.reshape(x.shape[:-1])
         else:
             q, s = fused.rmsnorm(x, norm_weight, eps, store=False, quantize=True)
-        g = self.gate.forward_int8(q, s, x.dtype)
-        u = self.up.forward_int8(q, s, x.dtype)
+        g, u = self._gate_up_int8(q, s, x.dtype)
         q2, s2 = fused.swiglu(g, u, store=False, quantize=True)
         return self.down.forward_int8(q2, s2, x.dtype, residual)

@@ -4,6 +4,7 @@ from .convert import (
     convert_linear_layers,
     count_ternary_params,
     fp_linear_to_ternary_infer,
+    fuse_ternary_linear_inference,
     get_model_memory_bytes,
     load_ternary_checkpoint,
     load_ternary_safetensors,
@@ -16,6 +17,7 @@ __all__ = [
     "fp_linear_to_ternary_infer",
     "ternary_linear_to_infer",
     "convert_linear_layers",
+    "fuse_ternary_linear_inference",
     "count_ternary_params",
     "get_model_memory_bytes",
     "save_ternary_checkpoint",

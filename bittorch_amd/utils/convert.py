@@ -75,6 +75,29 @@ def convert_linear_layers(module: nn.Module, threshold_factor: float = 0.05, ski
     return module
 
 
+def fuse_ternary_linear_inference(*layers: TernaryLinearInference) -> TernaryLinearInference:
+    """One inference layer computing ``concat([l(x) for l in layers], dim=-1)``.
+
+    Packed weights are laid out ``[ceil(K/4), N]``, so layers that share their input (q/k/v, or
+    gate/up: the reference's JS runtime stores ``kv_proj`` fused the same way,
+    ``js/src/models/TernaryTransformer.ts:141-188``) concatenate along the column axis; every
+    output column keeps its own weights, scale and bias, so each slice of the result equals the
+    separate layer's output bit for bit, while one launch covers all the columns (fewer, fuller
+    waves of tiles on the 256 compute units)."""
+    if not layers:
+        raise ValueError("no layers to fuse")
+    k = layers[0].in_features
+    if any(l.in_features != k for l in layers):
+        raise ValueError("layers must share in_features")
+    if any((l.bias is None) != (layers[0].bias is None) for l in layers):
+        raise ValueError("either all layers have a bias or none")
+    packed = torch.cat([l.weight_packed for l in layers], dim=1).contiguous()
+    scale = torch.cat([l.scale.reshape(-1).expand(l.out_features) if l.scale.numel() == 1 else l.scale
+                       for l in layers]).contiguous()
+    bias = None if layers[0].bias is None else torch.cat([l.bias for l in layers]).contiguous()
+    return TernaryLinearInference(k, sum(l.out_features for l in layers), packed, scale, bias)
+
+
 def count_ternary_params(module: nn.Module) -> Dict[str, int]:
     """Weights by storage type (reference ``:136-166``): ``fp32``, ``fp16``, ``packed_ternary``, ``total``
     (biases and scales are not counted; any non-fp16 dense weight counts as fp32, as in the reference)."""

@@ -228,3 +228,40 @@ def test_ternary_swiglu_module_equals_its_unfused_composition(compute):
     # without a norm the input itself is the activation
     got2 = mlp(x)
     assert got2.shape == (tokens, d) and torch.isfinite(got2.float()).all()
+
+
+def test_fused_layers_equal_the_separate_layers_bit_for_bit():
+    import bittorch_amd as bt
+    announce("fuse_ternary_linear_inference")
+    d, tokens = 256, 70
+    mk = lambda o, seed: bt.nn.create_ternary_linear_inference(
+        d, o, (torch.randn(o, d, generator=torch.Generator().manual_seed(seed)) * 0.02).cuda(),
+        (torch.randn(o, generator=torch.Generator().manual_seed(seed + 9)) * 0.01).cuda())
+    q, k, v = mk(256, 1), mk(128, 2), mk(64, 3)
+    qkv = bt.utils.fuse_ternary_linear_inference(q, k, v)
+    assert qkv.out_features == 448 and qkv.weight_packed.shape == (64, 448)
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        x = seeded_acts(tokens, d, seed=5, dtype=dtype).cuda()
+        y = qkv(x)
+        assert torch.equal(y[:, :256], q(x)) and torch.equal(y[:, 256:384], k(x)) and torch.equal(y[:, 384:], v(x))
+    x1 = seeded_acts(1, d, seed=6, dtype=torch.float16).cuda()   # decode shape: streaming kernel
+    y1 = qkv(x1)
+    assert torch.equal(y1[:, :256], q(x1)) and torch.equal(y1[:, 384:], v(x1))
+    with pytest.raises(ValueError, match="share in_features"):
+        bt.utils.fuse_ternary_linear_inference(q, mk(32, 4).__class__(128, 32, q.weight_packed[:32, :32].contiguous(),
+                                                                      q.scale[:32].contiguous()))
+
+
+@pytest.mark.parametrize("compute", ["float", "int8"])
+def test_swiglu_module_with_fused_gate_up_equals_the_unfused_module(compute):
+    import bittorch_amd as bt
+    announce("TernarySwiGLU fused gate_up", compute)
+    d, ffn = 256, 640
+    mk = lambda i, o, seed: bt.nn.create_ternary_linear_inference(
+        i, o, (torch.randn(o, i, generator=torch.Generator().manual_seed(seed)) * 0.02).cuda())
+    gate, up, down = mk(d, ffn, 1), mk(d, ffn, 2), mk(ffn, d, 3)
+    a = bt.nn.TernarySwiGLU(gate, up, down, compute=compute)
+    b = bt.nn.TernarySwiGLU(gate, up, down, compute=compute, fuse_gate_up=True)
+    x = seeded_acts(3 * 16, d, seed=8, dtype=torch.bfloat16).cuda().view(3, 16, d)
+    nw = torch.ones(d).bfloat16().cuda()
+    assert torch.equal(a(x, nw, 1e-5, residual=x), b(x, nw, 1e-5, residual=x))
