@@ -42,6 +42,9 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
     ap.add_argument("--no-block-stack", action="store_true", help="skip the 30-layer block stack (config 5)")
+    ap.add_argument("--block-stack-only", type=int, default=0, metavar="LAYERS",
+                    help="no GEMV timing: run the config-5 block stack with this many layers and print its "
+                         "timings (the workload of profiles/block_stack_kernel_trace.txt)")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU baseline sample length")
     ap.add_argument("--pmc-pass", action="store_true",
                     help="no timing: a few eager launches of each kernel plus a plain copy of known size, "
@@ -295,6 +298,10 @@ def main():
 
     if args.pmc_pass:
         pmc_pass(torch, _C, dev, step, x)
+        return
+    if args.block_stack_only:
+        del packs
+        print(json.dumps({"block_stack": block_stack(torch, dev, layers=args.block_stack_only)}))
         return
 
     wall_ms, ev_ms = graph_time(step, args.steps, args.warmup, torch)
