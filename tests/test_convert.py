@@ -134,3 +134,39 @@ def test_gpu_conversion_equals_cpu_conversion():
         assert torch.equal(v, gpu.state_dict()[k].cpu()), k
     x = torch.randn(9, 256)
     assert torch.allclose(gpu(x.cuda()).cpu(), cpu(x), atol=1e-4, rtol=1e-4)
+
+
+def test_fused_layers_on_the_cpu_path_equal_the_separate_layers():
+    import bittorch_amd as bt
+    torch.manual_seed(0)
+    mk = lambda o: bt.nn.create_ternary_linear_inference(64, o, torch.randn(o, 64) * 0.02, torch.randn(o) * 0.01)
+    a, b = mk(48), mk(16)
+    ab = bt.utils.fuse_ternary_linear_inference(a, b)
+    assert ab.in_features == 64 and ab.out_features == 64 and ab.weight_packed.shape == (16, 64)
+    x = torch.randn(5, 64)
+    y = ab(x)
+    assert torch.equal(y[:, :48], a(x)) and torch.equal(y[:, 48:], b(x))
+    with pytest.raises(ValueError, match="share in_features"):
+        bt.utils.fuse_ternary_linear_inference(a, bt.nn.create_ternary_linear_inference(32, 8, torch.randn(8, 32)))
+    with pytest.raises(ValueError, match="bias"):
+        bt.utils.fuse_ternary_linear_inference(a, bt.nn.create_ternary_linear_inference(64, 8, torch.randn(8, 64)))
+
+
+def test_ternary_swiglu_cpu_path_and_argument_checks():
+    import torch.nn.functional as F
+    import bittorch_amd as bt
+    torch.manual_seed(1)
+    mk = lambda i, o: bt.nn.create_ternary_linear_inference(i, o, torch.randn(o, i) * 0.02)
+    gate, up, down = mk(32, 80), mk(32, 80), mk(80, 32)
+    x = torch.randn(7, 32)
+    nw = torch.ones(32)
+    for fuse in (False, True):
+        mlp = bt.nn.TernarySwiGLU(gate, up, down, fuse_gate_up=fuse)
+        h = F.rms_norm(x, (32,), nw, 1e-5)
+        ref = down(F.silu(gate(h)) * up(h)) + x
+        assert torch.allclose(mlp(x, nw, 1e-5, residual=x), ref, rtol=1e-5, atol=1e-6)
+        assert torch.allclose(mlp(x), down(F.silu(gate(x)) * up(x)), rtol=1e-5, atol=1e-6)
+    with pytest.raises(ValueError, match="compute must be"):
+        bt.nn.TernarySwiGLU(gate, up, down, compute="fp8")
+    with pytest.raises(ValueError, match="do not form an MLP"):
+        bt.nn.TernarySwiGLU(gate, up, mk(64, 32))
