@@ -31,7 +31,7 @@ struct RowOpParams {
 };
 
 // exp(a) in fp32 by a fixed sequence of correctly rounded operations (range reduction by ln 2 in two
-// parts, degree-7 polynomial, exact scaling): a few units in the last place from exp on
+// parts, degree-7 polynomial, exact scaling by 2^n): a few units in the last place from exp on
 // [-87, 88.7228]; +inf above (as exp overflows), exp(-87) below (callers only add it to 1).  The
 // same sequence with fmaf() on a CPU gives the same bits.
 __device__ __forceinline__ float exp_fixed(float a) {
@@ -49,12 +49,8 @@ __device__ __forceinline__ float exp_fixed(float a) {
     p = __builtin_fmaf(p, r, 0.5f);
     p = __builtin_fmaf(p, r, 1.0f);
     p = __builtin_fmaf(p, r, 1.0f);
-    // p * 2^n in two steps, the first exact (n in [-126, 128]; 2^128 itself is not representable)
-    const int ni = (int)n;
-    const int n1 = ni / 2, n2 = ni - n1;
-    const float s1 = __builtin_bit_cast(float, (uint32_t)(n1 + 127) << 23);
-    const float s2 = __builtin_bit_cast(float, (uint32_t)(n2 + 127) << 23);
-    return __fmul_rn(__fmul_rn(p, s1), s2);
+    // p * 2^n, exact: the result is a normal number (n >= -126) or overflows like exp itself
+    return __builtin_ldexpf(p, (int)n);
 }
 
 __device__ __forceinline__ float swiglu_value(float g, float u, int dt) {

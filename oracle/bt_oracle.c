@@ -350,7 +350,7 @@ void bto_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const fl
 
 /* exp(a) by a fixed sequence of correctly rounded fp32 operations: +inf above 88.7228, a clamped to -87 below,
  * n = rint(a*log2(e)), r = a - n*ln2 (two-part ln2, fused), degree-7 Taylor polynomial in Horner
- * form with fused multiply-adds, then two exact power-of-two scalings. */
+ * form with fused multiply-adds, then the exact scaling by 2^n. */
 float bto_exp_fixed(float a) {
     if (!(a == a)) return a;
     if (a > 88.7228f) return INFINITY;  /* exp overflows fp32 */
@@ -366,13 +366,7 @@ float bto_exp_fixed(float a) {
     p = fmaf(p, r, 0.5f);
     p = fmaf(p, r, 1.0f);
     p = fmaf(p, r, 1.0f);
-    const int ni = (int)n;
-    const int n1 = ni / 2, n2 = ni - n1;
-    uint32_t u1 = (uint32_t)(n1 + 127) << 23, u2 = (uint32_t)(n2 + 127) << 23;
-    float s1, s2;
-    memcpy(&s1, &u1, 4);
-    memcpy(&s2, &u2, 4);
-    return (p * s1) * s2;
+    return ldexpf(p, (int)n);
 }
 
 static void quant_row_i8(const float* v, int64_t K, int8_t* q, float* s_out) {
