@@ -247,9 +247,9 @@ def test_fused_layers_equal_the_separate_layers_bit_for_bit():
     x1 = seeded_acts(1, d, seed=6, dtype=torch.float16).cuda()   # decode shape: streaming kernel
     y1 = qkv(x1)
     assert torch.equal(y1[:, :256], q(x1)) and torch.equal(y1[:, 384:], v(x1))
+    other = bt.nn.create_ternary_linear_inference(128, 32, (torch.randn(32, 128) * 0.02).cuda())
     with pytest.raises(ValueError, match="share in_features"):
-        bt.utils.fuse_ternary_linear_inference(q, mk(32, 4).__class__(128, 32, q.weight_packed[:32, :32].contiguous(),
-                                                                      q.scale[:32].contiguous()))
+        bt.utils.fuse_ternary_linear_inference(q, other)
 
 
 @pytest.mark.parametrize("compute", ["float", "int8"])
