@@ -489,6 +489,30 @@ def main():
                 "frac_of_hbm_peak": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
             }
             del masters
+        # block glue (config-5 shapes, bf16): fused kernels against the torch sequences they replace
+        import torch.nn.functional as F
+        glue = {}
+        for (m, k) in ((4096, 6912), (4096, 2560)):
+            gs = [torch.randn(m, k, device=dev).bfloat16() for _ in range(4)]
+            us_ = [torch.randn(m, k, device=dev).bfloat16() for _ in range(4)]
+            nw = torch.ones(k, device=dev).bfloat16()
+            nb = m * k * 2
+            cases = {
+                "swiglu": (lambda i: _C.swiglu(gs[i % 4], us_[i % 4]), 3 * nb),
+                "swiglu_torch_2_kernels": (lambda i: F.silu(gs[i % 4]) * us_[i % 4], 3 * nb),
+                "swiglu_quantized": (lambda i: _C.swiglu(gs[i % 4], us_[i % 4], False, True), 2 * nb + nb // 2),
+                "swiglu_quantized_torch_plus_act_quant": (lambda i: _C.act_quant_int8(F.silu(gs[i % 4]) * us_[i % 4]), 2 * nb + nb // 2),
+                "rmsnorm": (lambda i: _C.rmsnorm(gs[i % 4], nw, 1e-5), 2 * nb),
+                "rmsnorm_torch": (lambda i: F.rms_norm(gs[i % 4], (k,), nw, 1e-5), 2 * nb),
+                "rmsnorm_quantized": (lambda i: _C.rmsnorm(gs[i % 4], nw, 1e-5, False, True), nb + nb // 2),
+                "rmsnorm_quantized_torch_plus_act_quant": (lambda i: _C.act_quant_int8(F.rms_norm(gs[i % 4], (k,), nw, 1e-5)), nb + nb // 2),
+            }
+            for name, (fn, nbytes) in cases.items():
+                _, ev = graph_time(fn, 40, 4, torch)
+                us = ev / 40 * 1e3
+                glue[f"{name}_{m}x{k}"] = {"us": round(us, 2), "algorithmic_GBps": round(nbytes / (us * 1e-6) / 1e9, 1)}
+            del gs, us_
+        extra["block_glue_bf16"] = glue
         # config 5: the 30-layer block stack, end to end
         if not args.no_block_stack:
             try:
