@@ -60,12 +60,12 @@ __device__ __forceinline__ void store4f(void* Y, int dt, int64_t idx, const floa
 // Finishes four 16-row blocks (acc[MB0 .. MB0+3]) of the tile.
 template <int MODE, int YDT, int MB0>
 __device__ __forceinline__ void gemm_f_epilogue(const GemmFParams& p, const v4f (&acc)[F_MB][4], int64_t m0, int g,
-                                                int64_t ncol) {
+                                                int64_t ncol, const uint32_t (&ws_bits)[4], const uint32_t (&bs_bits)[4]) {
     float ws[4], bs[4];
 #pragma unroll
     for (int t = 0; t < 4; t++) {
-        ws[t] = epi_scale(p.epi, ncol + t);
-        bs[t] = epi_bias(p.epi, ncol + t);
+        ws[t] = bits_to_f32_rt(ws_bits[t], p.epi.scale_dtype);
+        bs[t] = p.epi.bias ? bits_to_f32_rt(bs_bits[t], p.epi.bias_dtype) : 0.0f;
     }
 #pragma unroll
     for (int mbi = 0; mbi < 4; mbi++) {
@@ -87,10 +87,11 @@ __device__ __forceinline__ void gemm_f_epilogue(const GemmFParams& p, const v4f 
 }
 template <int MODE, int MB0>
 __device__ __forceinline__ void gemm_f_epilogue_dt(const GemmFParams& p, const v4f (&acc)[F_MB][4], int64_t m0,
-                                                   int g, int64_t ncol) {
-    if (p.y_dtype == BT_BF16) gemm_f_epilogue<MODE, BT_BF16, MB0>(p, acc, m0, g, ncol);
-    else if (p.y_dtype == BT_F16) gemm_f_epilogue<MODE, BT_F16, MB0>(p, acc, m0, g, ncol);
-    else gemm_f_epilogue<MODE, BT_F32, MB0>(p, acc, m0, g, ncol);
+                                                   int g, int64_t ncol, const uint32_t (&ws_bits)[4],
+                                                   const uint32_t (&bs_bits)[4]) {
+    if (p.y_dtype == BT_BF16) gemm_f_epilogue<MODE, BT_BF16, MB0>(p, acc, m0, g, ncol, ws_bits, bs_bits);
+    else if (p.y_dtype == BT_F16) gemm_f_epilogue<MODE, BT_F16, MB0>(p, acc, m0, g, ncol, ws_bits, bs_bits);
+    else gemm_f_epilogue<MODE, BT_F32, MB0>(p, acc, m0, g, ncol, ws_bits, bs_bits);
 }
 
 // TAIL = false: K is a multiple of the 64-wide stage and the main loop is branch free.
@@ -286,6 +287,15 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     if (s < nstages) stage(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
     __syncthreads();  // every wave is done with the stage buffers before they are reused
 
+    // column scales and biases (raw bits) requested ahead of the exchange, which covers their latency
+    uint32_t ws_bits[4], bs_bits[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const int64_t n = col_ok ? ncol + t : 0;
+        ws_bits[t] = load_bits_rt(p.epi.scale, p.epi.scale_dtype, p.epi.scale_bcast ? 0 : n);
+        bs_bits[t] = p.epi.bias ? load_bits_rt(p.epi.bias, p.epi.bias_dtype, n) : 0u;
+    }
+
     // ---- add the two K halves: K half 1 hands over row blocks 0..3, K half 0 hands over row
     // blocks 4..7; word (q, wn, lane) of the exchange buffer is register q of that lane ----
     {
@@ -318,8 +328,8 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     }
 
     if (!col_ok) return;
-    if (kgrp == 0) gemm_f_epilogue_dt<MODE, 0>(p, acc, m0, g, ncol);  // wave-uniform branch
-    else gemm_f_epilogue_dt<MODE, 4>(p, acc, m0, g, ncol);
+    if (kgrp == 0) gemm_f_epilogue_dt<MODE, 0>(p, acc, m0, g, ncol, ws_bits, bs_bits);  // wave-uniform branch
+    else gemm_f_epilogue_dt<MODE, 4>(p, acc, m0, g, ncol, ws_bits, bs_bits);
 }
 
 // the tiled kernel reads X with 16-byte loads and W_T / Y with 4-column vectors

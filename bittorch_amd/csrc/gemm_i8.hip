@@ -62,14 +62,37 @@ __device__ __forceinline__ void store4(void* Y, int dt, int64_t idx, const float
 }
 
 // Finishes four 16-row blocks (acc[MB0 .. MB0+3]) of the tile.
+// The epilogue's operands (row scales of the wave's 16 rows, column scales and biases as raw bits)
+// are requested before the K-half exchange, whose LDS round trips cover their latency.
+struct EpiOperands {
+    float sx[4][4];  // [row block within the half][r]
+    uint32_t ws_bits[4], bs_bits[4];
+};
+__device__ __forceinline__ void load_epi_operands(const GemmParams& p, int64_t m0, int mb0, int g, int64_t ncol,
+                                                  bool col_ok, EpiOperands& e) {
+#pragma unroll
+    for (int mbi = 0; mbi < 4; mbi++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int64_t m = m0 + 16 * (mb0 + mbi) + 4 * g + r;
+            e.sx[mbi][r] = p.s_x[m < p.M ? m : p.M - 1];
+        }
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const int64_t n = col_ok ? ncol + t : 0;
+        e.ws_bits[t] = load_bits_rt(p.epi.scale, p.epi.scale_dtype, p.epi.scale_bcast ? 0 : n);
+        e.bs_bits[t] = p.epi.bias ? load_bits_rt(p.epi.bias, p.epi.bias_dtype, n) : 0u;
+    }
+}
+
 template <int YDT, int MB0>
 __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&acc)[G_MB][4], int64_t m0, int g,
-                                              int64_t ncol) {
+                                              int64_t ncol, const EpiOperands& e) {
     float ws[4], bs[4];
 #pragma unroll
     for (int t = 0; t < 4; t++) {
-        ws[t] = epi_scale(p.epi, ncol + t);
-        bs[t] = epi_bias(p.epi, ncol + t);
+        ws[t] = bits_to_f32_rt(e.ws_bits[t], p.epi.scale_dtype);
+        bs[t] = p.epi.bias ? bits_to_f32_rt(e.bs_bits[t], p.epi.bias_dtype) : 0.0f;
     }
 #pragma unroll
     for (int mbi = 0; mbi < 4; mbi++) {
@@ -77,7 +100,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&a
         for (int r = 0; r < 4; r++) {
             const int64_t m = m0 + 16 * (MB0 + mbi) + 4 * g + r;
             if (m >= p.M) continue;
-            const float sx = p.s_x[m];
+            const float sx = e.sx[mbi][r];
             float y[4];
             int32_t a127[4];
 #pragma unroll
@@ -94,10 +117,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&a
 }
 template <int MB0>
 __device__ __forceinline__ void gemm_epilogue_dt(const GemmParams& p, const v4i (&acc)[G_MB][4], int64_t m0, int g,
-                                                 int64_t ncol) {
-    if (p.y_dtype == BT_BF16) gemm_epilogue<BT_BF16, MB0>(p, acc, m0, g, ncol);
-    else if (p.y_dtype == BT_F16) gemm_epilogue<BT_F16, MB0>(p, acc, m0, g, ncol);
-    else gemm_epilogue<BT_F32, MB0>(p, acc, m0, g, ncol);
+                                                 int64_t ncol, const EpiOperands& e) {
+    if (p.y_dtype == BT_BF16) gemm_epilogue<BT_BF16, MB0>(p, acc, m0, g, ncol, e);
+    else if (p.y_dtype == BT_F16) gemm_epilogue<BT_F16, MB0>(p, acc, m0, g, ncol, e);
+    else gemm_epilogue<BT_F32, MB0>(p, acc, m0, g, ncol, e);
 }
 
 // TAIL = false: K is a multiple of the 128-wide stage and the main loop is branch free.
@@ -346,6 +369,9 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     if (s < nstages) stage(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
     __syncthreads();  // every wave is done with the stage buffers before they are reused
 
+    EpiOperands epi_ops;
+    load_epi_operands(p, m0, 4 * kgrp, g, ncol, col_ok, epi_ops);
+
     // ---- add the two K halves: waves (wn, 0) and (wn, 1) hold partial sums of the same
     // outputs.  K half 1 hands over row blocks 0..3, K half 0 hands over row blocks 4..7;
     // word (q, wn, lane) of the exchange buffer is register q of that lane.
@@ -381,8 +407,8 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     // ---- epilogue: K half h finishes row blocks 4h .. 4h+3; lane (j, g) holds rows
     // 16mb + 4g + r, columns ncol .. ncol+3 -------------------------------------------
     if (!col_ok) return;
-    if (kgrp == 0) gemm_epilogue_dt<0>(p, acc, m0, g, ncol);  // wave-uniform branch
-    else gemm_epilogue_dt<4>(p, acc, m0, g, ncol);
+    if (kgrp == 0) gemm_epilogue_dt<0>(p, acc, m0, g, ncol, epi_ops);  // wave-uniform branch
+    else gemm_epilogue_dt<4>(p, acc, m0, g, ncol, epi_ops);
 }
 
 // the tiled kernel reads Q with 16-byte loads and W_T / Y with 4-column vectors
