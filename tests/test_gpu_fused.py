@@ -265,3 +265,33 @@ def test_swiglu_module_with_fused_gate_up_equals_the_unfused_module(compute):
     x = seeded_acts(3 * 16, d, seed=8, dtype=torch.bfloat16).cuda().view(3, 16, d)
     nw = torch.ones(d).bfloat16().cuda()
     assert torch.equal(a(x, nw, 1e-5, residual=x), b(x, nw, 1e-5, residual=x))
+
+
+def test_block_glue_at_config5_sizes():
+    """Full-size shapes of the block stack (4096 tokens, d 2560, FFN 6912, bf16) through properties that
+    need no CPU pass: the fused quantization equals the stand-alone quantizer on the stored tensor, the
+    stored tensor agrees with torch's operators to one unit in the last place, RMSNorm rows have unit
+    RMS, and the residual epilogue of a tall GEMM equals linear-then-add."""
+    from bittorch_amd import _C
+    announce("block glue, full size")
+    g = torch.Generator(device="cuda").manual_seed(0)
+    gate = torch.randn(4096, 6912, device="cuda", generator=g).bfloat16() * 2
+    up = torch.randn(4096, 6912, device="cuda", generator=g).bfloat16()
+    h, q, s = _C.swiglu(gate, up, True, True)
+    q_ref, s_ref = _C.act_quant_int8(h)
+    assert torch.equal(q, q_ref) and torch.equal(s, s_ref)
+    assert _ulp_close(h, F.silu(gate) * up, torch.bfloat16, ulps=1) == 0
+    del gate, up, h, q, q_ref
+
+    x = torch.randn(4096, 2560, device="cuda", generator=g).bfloat16() * 3
+    y, q, s = _C.rmsnorm(x, None, 1e-6, True, True)
+    q_ref, s_ref = _C.act_quant_int8(y)
+    assert torch.equal(q, q_ref) and torch.equal(s, s_ref)
+    rms = y.float().pow(2).mean(-1).sqrt()
+    assert torch.allclose(rms, torch.ones_like(rms), atol=5e-3)
+
+    packed, scale, _ = _packed_case(2560, 2560, seed=11)
+    lin = _C.ternary_linear_packed_forward(y, packed, scale, None, 2560)
+    assert torch.equal(_C.ternary_linear_packed_forward(y, packed, scale, None, 2560, x), lin + x)
+    lin8 = _C.ternary_gemm_int8(q, s, packed, scale, None, 2560, torch.bfloat16)
+    assert torch.equal(_C.ternary_gemm_int8(q, s, packed, scale, None, 2560, torch.bfloat16, residual=x), lin8 + x)
