@@ -276,7 +276,19 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
                 for (int u = 0; u < XC_MAX; u++) {
                     if (u * 64 < nchunks) {
                         const int k = s_begin * 64 + (lane + 64 * u) * EPC;
-                        *(uint4*)(xs + (lane + 64 * u) * 16) = zero_unless(xr[u], k < (int)p.K);
+                        // parked in the order the MFMA wants (each 16-byte chunk is one operand
+                        // fragment), so that the steps below read their A operand ready-made
+                        const uint4 v = zero_unless(xr[u], k < (int)p.K);
+                        uint4 o;
+                        if constexpr (MODE == MODE_I8) {
+                            uint32_t t4[4];
+                            transpose4x4_bytes(v.x, v.y, v.z, v.w, t4);
+                            o = make_uint4(t4[0], t4[1], t4[2], t4[3]);
+                        } else {
+                            o = make_uint4(perm(v.z, v.x, 0x05040100u), perm(v.z, v.x, 0x07060302u),
+                                           perm(v.w, v.y, 0x05040100u), perm(v.w, v.y, 0x07060302u));
+                        }
+                        *(uint4*)(xs + (lane + 64 * u) * 16) = o;
                     }
                 }
             }
@@ -312,7 +324,11 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
             }
             if constexpr (MODE == MODE_I8) {
                 uint32_t ta[4];
-                transpose4x4_bytes(xa[f][0].x, xa[f][0].y, xa[f][0].z, xa[f][0].w, ta);
+                if constexpr (XLDS) {  // already in operand order
+                    ta[0] = xa[f][0].x; ta[1] = xa[f][0].y; ta[2] = xa[f][0].z; ta[3] = xa[f][0].w;
+                } else {
+                    transpose4x4_bytes(xa[f][0].x, xa[f][0].y, xa[f][0].z, xa[f][0].w, ta);
+                }
                 const v4i a = {(int)ta[0], (int)ta[1], (int)ta[2], (int)ta[3]};
 #pragma unroll
                 for (int t = 0; t < NACC; t++) {
@@ -326,9 +342,13 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
                 // natural halves h0..h7 -> dword c = { h[c], h[4+c] } (the decode's k order)
                 u32x4 au[2];
 #pragma unroll
-                for (int h = 0; h < 2; h++)
-                    au[h] = u32x4{perm(xa[f][h].z, xa[f][h].x, 0x05040100u), perm(xa[f][h].z, xa[f][h].x, 0x07060302u),
-                                  perm(xa[f][h].w, xa[f][h].y, 0x05040100u), perm(xa[f][h].w, xa[f][h].y, 0x07060302u)};
+                for (int h = 0; h < 2; h++) {
+                    if constexpr (XLDS)  // already in operand order
+                        au[h] = u32x4{xa[f][h].x, xa[f][h].y, xa[f][h].z, xa[f][h].w};
+                    else
+                        au[h] = u32x4{perm(xa[f][h].z, xa[f][h].x, 0x05040100u), perm(xa[f][h].z, xa[f][h].x, 0x07060302u),
+                                      perm(xa[f][h].w, xa[f][h].y, 0x05040100u), perm(xa[f][h].w, xa[f][h].y, 0x07060302u)};
+                }
 #pragma unroll
                 for (int t = 0; t < NACC; t++) {
 #pragma unroll
