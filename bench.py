@@ -169,16 +169,17 @@ def block_stack(torch, dev, layers=30, d_model=2560, heads=20, ffn=6912, batch=8
         b, s, _ = x.shape
         if int8:  # ... and, BitNet-style, every projection on the int8 matrix cores from activations
             # that leave the norm / SwiGLU kernels already quantized per token
-            qh, sh = fused.rmsnorm(x, blk.n1.weight, blk.n1.eps or torch.finfo(x.dtype).eps, store=False, quantize=True)
-            qkv = blk.qkv.forward_int8(qh, sh, x.dtype)
+            qh, sh = fused.rmsnorm(x, blk.n1.weight, blk.n1.eps or torch.finfo(x.dtype).eps, store=False, quantize=True,
+                                   operand_order=True)
+            qkv = blk.qkv.forward_int8(qh, sh, x.dtype, None, True)
         else:
             qkv = blk.qkv(fused.rmsnorm(x, blk.n1.weight, blk.n1.eps or torch.finfo(x.dtype).eps))
         q, k, v = qkv.split(d_model, dim=-1)  # one GEMM over the concatenated q|k|v columns
         a = F.scaled_dot_product_attention(heads_of(q, b, s), heads_of(k, b, s), heads_of(v, b, s), is_causal=True)
         a = a.transpose(1, 2).reshape(b, s, -1)
         if int8:
-            qa, sa = bt._C.act_quant_int8(a.reshape(b * s, -1))
-            x = blk.o.forward_int8(qa, sa, x.dtype, x.reshape(b * s, -1)).view(b, s, -1)
+            qa, sa = bt._C.act_quant_int8(a.reshape(b * s, -1), True)
+            x = blk.o.forward_int8(qa, sa, x.dtype, x.reshape(b * s, -1), True).view(b, s, -1)
         else:
             x = blk.o(a, x)
         return blk.mlp(x, blk.n2.weight, blk.n2.eps or torch.finfo(x.dtype).eps, residual=x)

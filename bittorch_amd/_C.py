@@ -275,8 +275,12 @@ def ternary_quantize_pack(weight: Tensor, threshold_factor: float = 0.05, per_ch
     return packed, scale, tern
 
 
-def act_quant_int8(X: Tensor) -> Tuple[Tensor, Tensor]:
-    """Per-row int8 activation quantization: ``(Q int8 [B,K], s_x fp32 [B])``."""
+def act_quant_int8(X: Tensor, operand_order: bool = False) -> Tuple[Tensor, Tensor]:
+    """Per-row int8 activation quantization: ``(Q int8 [B,K], s_x fp32 [B])``.
+
+    ``operand_order=True`` (K % 16 == 0) writes every 16-byte group of ``Q`` in the order the
+    int8 GEMMs feed the matrix cores; such a ``Q`` must go to :func:`ternary_gemm_int8` with
+    ``q_operand_order=True``."""
     _check(X.dim() == 2 and X.numel() > 0, "X must be 2D and non-empty")
     _check(X.is_cuda, "All tensors must be CUDA")
     x = X.contiguous()
@@ -284,17 +288,18 @@ def act_quant_int8(X: Tensor) -> Tuple[Tensor, Tensor]:
     q = torch.empty((B, K), dtype=torch.int8, device=x.device)
     s = torch.empty((B,), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
-        _status(_L.bt_act_quant_i8(x.data_ptr(), _dt(x, "X"), B, K, q.data_ptr(), s.data_ptr(),
-                                   _stream(x)))
+        _status(_L.bt_act_quant_i8_layout(x.data_ptr(), _dt(x, "X"), B, K, q.data_ptr(), s.data_ptr(),
+                                          1 if operand_order else 0, _stream(x)))
     return q, s
 
 
 def ternary_gemm_int8(Q: Tensor, s_x: Tensor, W_T: Tensor, scale: Tensor,
                       bias: Optional[Tensor] = None, in_features: int = -1,
                       out_dtype: torch.dtype = torch.float32, return_acc: bool = False,
-                      residual: Optional[Tensor] = None):
+                      residual: Optional[Tensor] = None, q_operand_order: bool = False):
     """int8 activations x packed ternary weights; optionally also the int32 accumulators.
-    ``residual`` ``[B, N]`` in ``out_dtype`` is added in the epilogue (``linear + residual``)."""
+    ``residual`` ``[B, N]`` in ``out_dtype`` is added in the epilogue (``linear + residual``);
+    ``q_operand_order`` says that ``Q`` was written with ``operand_order=True``."""
     _check(Q.dim() == 2 and Q.dtype == torch.int8, "Q must be 2D int8")
     if in_features < 0:
         in_features = Q.shape[-1]
@@ -313,16 +318,16 @@ def ternary_gemm_int8(Q: Tensor, s_x: Tensor, W_T: Tensor, scale: Tensor,
     with torch.cuda.device(q.device):
         ws_bytes = _L.bt_gemm_i8_workspace_bytes(B, N, K)
         ws = _workspace(ws_bytes, q.device)
-        if residual is None:
+        if residual is None and not q_operand_order:
             _status(_L.bt_ternary_gemm_i8(
                 q.data_ptr(), s_x.data_ptr(), W_T.data_ptr(), scale.data_ptr(), _dt(scale, "scale"),
                 scale.numel(), _ptr(bias), 0 if bias is None else _dt(bias, "bias"), y.data_ptr(),
                 _DT[out_dtype], _ptr(acc), B, N, K, _ptr(ws), 0 if ws is None else ws.numel(), _stream(q)))
         else:
-            res = _residual_2d(residual, y, (B,), N)
+            res = None if residual is None else _residual_2d(residual, y, (B,), N)
             _status(_L.bt_ternary_gemm_i8_res(
-                q.data_ptr(), s_x.data_ptr(), W_T.data_ptr(), scale.data_ptr(), _dt(scale, "scale"),
-                scale.numel(), _ptr(bias), 0 if bias is None else _dt(bias, "bias"), res.data_ptr(),
+                q.data_ptr(), 1 if q_operand_order else 0, s_x.data_ptr(), W_T.data_ptr(), scale.data_ptr(),
+                _dt(scale, "scale"), scale.numel(), _ptr(bias), 0 if bias is None else _dt(bias, "bias"), _ptr(res),
                 y.data_ptr(), _DT[out_dtype], _ptr(acc), B, N, K, _stream(q)))
     return (y, acc) if return_acc else y
 
@@ -354,7 +359,7 @@ def _rows_2d(t: Tensor, K: int) -> Tensor:
     return t.contiguous().reshape(-1, K)
 
 
-def swiglu(gate: Tensor, up: Tensor, store: bool = True, quantize: bool = False):
+def swiglu(gate: Tensor, up: Tensor, store: bool = True, quantize: bool = False, operand_order: bool = False):
     """``silu(gate) * up`` in one pass, rounded as the two separate torch ops round it.
 
     Returns the product (``store``), or with ``quantize`` its per-row int8 form ``(Q, s_x)`` for
@@ -369,7 +374,7 @@ def swiglu(gate: Tensor, up: Tensor, store: bool = True, quantize: bool = False)
     h, q, s = _row_op_outputs(g2, store, quantize)
     with torch.cuda.device(gate.device):
         _status(_L.bt_swiglu(g2.data_ptr(), g2.stride(0), u2.data_ptr(), u2.stride(0), _dt(g2, "gate"),
-                             g2.shape[0], K, _ptr(h), _ptr(q), _ptr(s), _stream(gate)))
+                             g2.shape[0], K, _ptr(h), _ptr(q), _ptr(s), 1 if operand_order else 0, _stream(gate)))
     if q is not None and gate.dim() != 2:
         q = q.reshape(*gate.shape[:-1], K)
         s = s.reshape(gate.shape[:-1])
@@ -377,7 +382,7 @@ def swiglu(gate: Tensor, up: Tensor, store: bool = True, quantize: bool = False)
 
 
 def rmsnorm(x: Tensor, weight: Optional[Tensor] = None, eps: float = 1e-6, store: bool = True,
-            quantize: bool = False):
+            quantize: bool = False, operand_order: bool = False):
     """RMSNorm over the last dimension, ``(x * rsqrt(mean(x^2) + eps)) * weight``; with
     ``quantize`` also (or only, ``store=False``) the per-row int8 form of the result."""
     _check(x.dim() >= 1 and x.numel() > 0, "x is empty")
@@ -391,7 +396,7 @@ def rmsnorm(x: Tensor, weight: Optional[Tensor] = None, eps: float = 1e-6, store
     h, q, s = _row_op_outputs(x2, store, quantize)
     with torch.cuda.device(x.device):
         _status(_L.bt_rmsnorm(x2.data_ptr(), x2.stride(0), _ptr(weight), float(eps), _dt(x2, "x"),
-                              x2.shape[0], K, _ptr(h), _ptr(q), _ptr(s), _stream(x)))
+                              x2.shape[0], K, _ptr(h), _ptr(q), _ptr(s), 1 if operand_order else 0, _stream(x)))
     if q is not None and x.dim() != 2:
         q = q.reshape(*x.shape[:-1], K)
         s = s.reshape(x.shape[:-1])

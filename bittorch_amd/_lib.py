@@ -44,10 +44,11 @@ SIGNATURES = {
     "bt_probe_mfma_i8": (_int, [_int, _int, _int, _vp, _vp, _vp]),
     "bt_ternary_linear_packed_forward_res": (_int, [_vp, _int, _vp, _vp, _int, _i64, _vp, _int, _vp, _vp,
                                                     _i64, _i64, _i64, _vp, _sz, _vp]),
-    "bt_ternary_gemm_i8_res": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _vp, _int, _vp, _vp, _int, _vp,
+    "bt_ternary_gemm_i8_res": (_int, [_vp, _int, _vp, _vp, _vp, _int, _i64, _vp, _int, _vp, _vp, _int, _vp,
                                       _i64, _i64, _i64, _vp]),
-    "bt_swiglu": (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _vp, _vp, _vp, _vp]),
-    "bt_rmsnorm": (_int, [_vp, _i64, _vp, ctypes.c_float, _int, _i64, _i64, _vp, _vp, _vp, _vp]),
+    "bt_swiglu": (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _vp, _vp, _vp, _int, _vp]),
+    "bt_rmsnorm": (_int, [_vp, _i64, _vp, ctypes.c_float, _int, _i64, _i64, _vp, _vp, _vp, _int, _vp]),
+    "bt_act_quant_i8_layout": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _int, _vp]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

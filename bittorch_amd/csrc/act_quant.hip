@@ -14,7 +14,8 @@ namespace bt {
 // (the second pass hits in cache; a row is at most a few tens of KiB).
 template <int DT>
 __global__ __launch_bounds__(256) void act_quant_kernel(const void* __restrict__ X, int64_t B, int64_t K,
-                                                        int8_t* __restrict__ Q, float* __restrict__ s_x) {
+                                                        int8_t* __restrict__ Q, float* __restrict__ s_x,
+                                                        int q_layout) {
     const int lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= B) return;
@@ -69,8 +70,8 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const void* __restrict__
             if (e < 4) lo |= byte << (8 * e);
             else hi |= byte << (8 * (e - 4));
         }
-        if (vec_ok) {
-            *(uint2*)(Q + base + k) = make_uint2(lo, hi);
+        if (vec_ok) {  // (operand order is only requested with K % 16 == 0 and aligned rows: this path)
+            *(uint2*)(Q + base + k) = q_layout == Q_OPERAND_ORDER ? q_to_operand_order(lo, hi, lane & 1) : make_uint2(lo, hi);
         } else {
 #pragma unroll
             for (int e = 0; e < 8; e++)
@@ -84,7 +85,8 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const void* __restrict__
 // Needs K % 8 == 0, K <= 2048*ITERS and aligned pointers (16 bytes X, 8 bytes Q).
 template <int DT, int ITERS>
 __global__ __launch_bounds__(256) void act_quant_row_kernel(const void* __restrict__ X, int K,
-                                                            int8_t* __restrict__ Q, float* __restrict__ s_x) {
+                                                            int8_t* __restrict__ Q, float* __restrict__ s_x,
+                                                            int q_layout) {
     __shared__ float part[4];
     const int tid = threadIdx.x;
     const int64_t base = (int64_t)blockIdx.x * K;
@@ -134,34 +136,38 @@ __global__ __launch_bounds__(256) void act_quant_row_kernel(const void* __restri
             if (e < 4) lo |= byte << (8 * e);
             else hi |= byte << (8 * (e - 4));
         }
-        if (k < K) *(uint2*)(Q + base + k) = make_uint2(lo, hi);
+        const uint2 o = q_layout == Q_OPERAND_ORDER ? q_to_operand_order(lo, hi, tid & 1) : make_uint2(lo, hi);
+        if (k < K) *(uint2*)(Q + base + k) = o;  // K % 16 == 0 in operand order: both lanes of a pair store
     }
 }
 
 template <int DT>
-static bool launch_act_quant_rows(const void* X, int64_t B, int64_t K, int8_t* Q, float* s_x, hipStream_t st) {
+static bool launch_act_quant_rows(const void* X, int64_t B, int64_t K, int8_t* Q, float* s_x, int ql, hipStream_t st) {
     if (K % 8 != 0 || K > 16384 || ((uintptr_t)X) % 16 != 0 || ((uintptr_t)Q) % 8 != 0 || B > 0x7fffffff ||
         getenv("BITTORCH_ACTQ_GENERIC"))
         return false;
     const dim3 grid((unsigned)B), block(256);
     const int k = (int)K;
-    if (K <= 2048) hipLaunchKernelGGL((act_quant_row_kernel<DT, 1>), grid, block, 0, st, X, k, Q, s_x);
-    else if (K <= 4096) hipLaunchKernelGGL((act_quant_row_kernel<DT, 2>), grid, block, 0, st, X, k, Q, s_x);
-    else if (K <= 8192) hipLaunchKernelGGL((act_quant_row_kernel<DT, 4>), grid, block, 0, st, X, k, Q, s_x);
-    else if (K <= 12288) hipLaunchKernelGGL((act_quant_row_kernel<DT, 6>), grid, block, 0, st, X, k, Q, s_x);
-    else hipLaunchKernelGGL((act_quant_row_kernel<DT, 8>), grid, block, 0, st, X, k, Q, s_x);
+    if (K <= 2048) hipLaunchKernelGGL((act_quant_row_kernel<DT, 1>), grid, block, 0, st, X, k, Q, s_x, ql);
+    else if (K <= 4096) hipLaunchKernelGGL((act_quant_row_kernel<DT, 2>), grid, block, 0, st, X, k, Q, s_x, ql);
+    else if (K <= 8192) hipLaunchKernelGGL((act_quant_row_kernel<DT, 4>), grid, block, 0, st, X, k, Q, s_x, ql);
+    else if (K <= 12288) hipLaunchKernelGGL((act_quant_row_kernel<DT, 6>), grid, block, 0, st, X, k, Q, s_x, ql);
+    else hipLaunchKernelGGL((act_quant_row_kernel<DT, 8>), grid, block, 0, st, X, k, Q, s_x, ql);
     return true;
 }
 
-int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x, hipStream_t st) {
-    const bool done = (x_dtype == BT_F32)   ? launch_act_quant_rows<BT_F32>(X, B, K, Q, s_x, st)
-                      : (x_dtype == BT_F16) ? launch_act_quant_rows<BT_F16>(X, B, K, Q, s_x, st)
-                                            : launch_act_quant_rows<BT_BF16>(X, B, K, Q, s_x, st);
+// q_layout = Q_OPERAND_ORDER needs K % 16 == 0, X 16-byte and Q 8-byte aligned (the callers check)
+int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x, int q_layout,
+                     hipStream_t st) {
+    const int ql = q_layout;
+    const bool done = (x_dtype == BT_F32)   ? launch_act_quant_rows<BT_F32>(X, B, K, Q, s_x, ql, st)
+                      : (x_dtype == BT_F16) ? launch_act_quant_rows<BT_F16>(X, B, K, Q, s_x, ql, st)
+                                            : launch_act_quant_rows<BT_BF16>(X, B, K, Q, s_x, ql, st);
     if (done) return check_launch("bt_act_quant_i8");
     const dim3 grid((unsigned)ceil_div(B, 4)), block(256);
-    if (x_dtype == BT_F32) hipLaunchKernelGGL(act_quant_kernel<BT_F32>, grid, block, 0, st, X, B, K, Q, s_x);
-    else if (x_dtype == BT_F16) hipLaunchKernelGGL(act_quant_kernel<BT_F16>, grid, block, 0, st, X, B, K, Q, s_x);
-    else hipLaunchKernelGGL(act_quant_kernel<BT_BF16>, grid, block, 0, st, X, B, K, Q, s_x);
+    if (x_dtype == BT_F32) hipLaunchKernelGGL(act_quant_kernel<BT_F32>, grid, block, 0, st, X, B, K, Q, s_x, ql);
+    else if (x_dtype == BT_F16) hipLaunchKernelGGL(act_quant_kernel<BT_F16>, grid, block, 0, st, X, B, K, Q, s_x, ql);
+    else hipLaunchKernelGGL(act_quant_kernel<BT_BF16>, grid, block, 0, st, X, B, K, Q, s_x, ql);
     return check_launch("bt_act_quant_i8");
 }
 

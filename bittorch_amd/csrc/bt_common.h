@@ -207,6 +207,33 @@ __device__ __forceinline__ u32x4 decode8_16bit(uint32_t M) {
 constexpr uint32_t LUT_F16_ONE = 0x00BC3C00u;   // sel 0..3 -> 0x00, 0x3C, 0xBC, 0x00
 constexpr uint32_t LUT_BF16_TWO = 0x00C04000u;  // sel 0..3 -> 0x00, 0x40, 0xC0, 0x00
 
+// ---- layout of quantized activations ----------------------------------------
+// Q_ROW_MAJOR: int8 [B, K] as is.  Q_OPERAND_ORDER (K % 16 == 0): the same rows, but every aligned
+// 16-byte group stored as the 4x4 byte transpose of its natural order (byte 4c+r holds element
+// 4r+c): the k order in which the in-register weight decode lays out an MFMA operand, so that the
+// GEMMs feed activations to the matrix cores without permuting them first.
+enum { Q_ROW_MAJOR = 0, Q_OPERAND_ORDER = 1 };
+
+// Two neighbouring lanes hold the 16 quantized bytes of one group (even lane: elements 0..7 as
+// lo, hi; odd lane: elements 8..15).  Returns this lane's 8 bytes of the transposed group.
+// Both lanes of a pair must call it (it exchanges registers between them).
+__device__ __forceinline__ uint2 q_to_operand_order(uint32_t lo, uint32_t hi, int lane_parity) {
+    // the neighbour's two dwords through a DPP quad permute [1,0,3,2] (no LDS round trip)
+    const uint32_t plo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)lo, 0xB1, 0xf, 0xf, true);
+    const uint32_t phi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)hi, 0xB1, 0xf, 0xf, true);
+    // rows r0..r3 of the 4x4 byte block = elements 0-3, 4-7, 8-11, 12-15
+    const bool odd = lane_parity != 0;
+    const uint32_t r0 = odd ? plo : lo, r1 = odd ? phi : hi, r2 = odd ? lo : plo, r3 = odd ? hi : phi;
+    // the even lane keeps columns 0,1 of the block (transposed rows 0,1), the odd lane columns 2,3
+    const uint32_t sel = odd ? 0x07030602u : 0x05010400u;
+    const uint32_t ta = perm(r1, r0, sel), tb = perm(r3, r2, sel);
+    return make_uint2(perm(tb, ta, 0x05040100u), perm(tb, ta, 0x07060302u));
+}
+// position of element k of a row in the operand-order layout
+__device__ __forceinline__ int64_t q_operand_order_pos(int64_t k) {
+    return (k & ~(int64_t)15) | ((k & 3) << 2) | ((k >> 2) & 3);
+}
+
 __device__ __forceinline__ int decode2(uint32_t code) { return (int)(code == 1u) - (int)(code == 2u); }
 
 // ---- wave64 reductions ------------------------------------------------------

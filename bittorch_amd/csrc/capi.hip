@@ -32,20 +32,21 @@ bool stream_supported(int64_t N, int64_t K, const void* W_T);
 size_t stream_workspace_bytes(int mode, int64_t M, int64_t N, int64_t Kb);
 int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, const uint8_t* W_T,
                   const Epilogue& epi, void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N,
-                  int64_t K, int planes, hipStream_t st);
+                  int64_t K, int planes, int q_layout, hipStream_t st);
 int launch_split_f32_planes(const void* X, int64_t B, int64_t K, void* P, hipStream_t st);
 int launch_packed_generic(const void* X, int x_dtype, const uint8_t* W_T, const Epilogue& epi, void* Y,
                           int64_t B, int64_t N, int64_t K, hipStream_t st);
 int launch_unpacked(const void* X, int x_dtype, const int8_t* W, const Epilogue& epi, void* Y, int64_t B,
                     int64_t N, int64_t K, hipStream_t st);
-int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x, hipStream_t st);
+int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x, int q_layout,
+                     hipStream_t st);
 bool gemm_i8_supported(int64_t N, int64_t K, const void* Q, const void* W_T);
 int launch_row_op(int op, int dtype, const void* A, int64_t lda, const void* Bv, int64_t ldb, float eps, int64_t B,
-                  int64_t K, void* H, int8_t* Q, float* s_x, hipStream_t st, const char* who);
+                  int64_t K, void* H, int8_t* Q, float* s_x, int q_layout, hipStream_t st, const char* who);
 bool gemm_f16_supported(int64_t N, int64_t K, const void* X, const void* W_T, const void* Y);
 int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, const Epilogue& epi, void* Y, int y_dtype, int64_t M,
                     int64_t N, int64_t K, int planes, hipStream_t st);
-int launch_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const Epilogue& epi, void* Y,
+int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_T, const Epilogue& epi, void* Y,
                    int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st);
 
 static bool valid_dtype(int dt) { return dt == BT_F32 || dt == BT_F16 || dt == BT_BF16; }
@@ -176,7 +177,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         // tall batches go to the tiled matrix-core kernel, decode shapes stream the weights
         if (B > kStreamMaxRows && gemm_f16_supported(N, K, X, W_T, Y))
             return launch_gemm_f16(mode, X, W_T, epi, Y, x_dtype, B, N, K, 1, st);
-        return launch_stream(mode, X, 2, nullptr, W_T, epi, Y, x_dtype, nullptr, B, N, K, 1, st);
+        return launch_stream(mode, X, 2, nullptr, W_T, epi, Y, x_dtype, nullptr, B, N, K, 1, Q_ROW_MAJOR, st);
     }
     if (x_dtype == BT_F32 && packed_uses_f32_planes(X, W_T, Y, N, K) && workspace &&
         workspace_bytes >= f32_planes_bytes(B, K) && ((uintptr_t)workspace) % 256 == 0) {
@@ -185,7 +186,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         if (rc) return rc;
         if (B > kStreamMaxRows && gemm_f16_supported(N, 3 * K, workspace, W_T, Y))
             return launch_gemm_f16(MODE_BF16, workspace, W_T, epi, Y, BT_F32, B, N, K, 3, st);
-        return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, epi, Y, BT_F32, nullptr, B, N, K, 3, st);
+        return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, epi, Y, BT_F32, nullptr, B, N, K, 3, Q_ROW_MAJOR, st);
     }
     return launch_packed_generic(X, x_dtype, W_T, epi, Y, B, N, K, st);
 }
@@ -214,7 +215,34 @@ extern "C" int bt_act_quant_i8(const void* X, int x_dtype, int64_t B, int64_t K,
         set_error("bt_act_quant_i8: null pointer, empty shape or bad dtype");
         return BT_ERR_INVALID;
     }
-    return launch_act_quant(X, x_dtype, B, K, Q, s_x, (hipStream_t)stream);
+    return launch_act_quant(X, x_dtype, B, K, Q, s_x, Q_ROW_MAJOR, (hipStream_t)stream);
+}
+
+// q_layout: BT_Q_ROW_MAJOR or BT_Q_OPERAND_ORDER (K % 16 == 0, X 16-byte and Q 16-byte aligned)
+static int check_q_layout(const char* who, int q_layout, int64_t K, const void* Q, const void* X) {
+    if (q_layout == Q_ROW_MAJOR) return BT_OK;
+    if (q_layout != Q_OPERAND_ORDER) {
+        set_error("%s: unknown q_layout %d", who, q_layout);
+        return BT_ERR_INVALID;
+    }
+    if (K % 16 != 0 || ((uintptr_t)Q) % 16 != 0 || (X && ((uintptr_t)X) % 16 != 0)) {
+        set_error("%s: the operand-order layout needs K %% 16 == 0 and 16-byte aligned buffers (K=%lld)", who,
+                  (long long)K);
+        return BT_ERR_INVALID;
+    }
+    return BT_OK;
+}
+
+extern "C" int bt_act_quant_i8_layout(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x,
+                                      int q_layout, void* stream) {
+    const char* who = "bt_act_quant_i8_layout";
+    if (!X || !Q || !s_x || B <= 0 || K <= 0 || !valid_dtype(x_dtype)) {
+        set_error("%s: null pointer, empty shape or bad dtype", who);
+        return BT_ERR_INVALID;
+    }
+    const int rc = check_q_layout(who, q_layout, K, Q, X);
+    if (rc) return rc;
+    return launch_act_quant(X, x_dtype, B, K, Q, s_x, q_layout, (hipStream_t)stream);
 }
 
 extern "C" size_t bt_gemm_i8_workspace_bytes(int64_t B, int64_t N, int64_t K) {
@@ -222,7 +250,7 @@ extern "C" size_t bt_gemm_i8_workspace_bytes(int64_t B, int64_t N, int64_t K) {
     return stream_workspace_bytes(MODE_I8, B, N, ceil_div(K, 4));
 }
 
-static int gemm_i8_impl(const char* who, const int8_t* Q, const float* s_x, const uint8_t* W_T, const void* scale,
+static int gemm_i8_impl(const char* who, const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_T, const void* scale,
                         int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype, const void* residual,
                         void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N, int64_t K, void* stream) {
     int rc = check_shape(who, Q, W_T, Y, y_dtype, B, N, K);
@@ -231,6 +259,8 @@ static int gemm_i8_impl(const char* who, const int8_t* Q, const float* s_x, cons
         set_error("%s: s_x is null", who);
         return BT_ERR_INVALID;
     }
+    rc = check_q_layout(who, q_layout, K, Q, nullptr);
+    if (rc) return rc;
     if (K > kMaxKInt8) {
         set_error("%s: K=%lld could overflow the int32 accumulators (limit %lld)", who, (long long)K,
                   (long long)kMaxKInt8);
@@ -254,9 +284,9 @@ static int gemm_i8_impl(const char* who, const int8_t* Q, const float* s_x, cons
                       (long long)ceil_div(K, 4), (long long)N);
             return BT_ERR_INVALID;
         }
-        return launch_stream(MODE_I8, Q, 1, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, 1, st);
+        return launch_stream(MODE_I8, Q, 1, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, 1, q_layout, st);
     }
-    return launch_gemm_i8(Q, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, st);
+    return launch_gemm_i8(Q, q_layout, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, st);
 }
 
 extern "C" int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const void* scale,
@@ -264,15 +294,15 @@ extern "C" int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8
                                   void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N, int64_t K,
                                   void* workspace, size_t workspace_bytes, void* stream) {
     (void)workspace; (void)workspace_bytes;
-    return gemm_i8_impl("bt_ternary_gemm_i8", Q, s_x, W_T, scale, scale_dtype, scale_len, bias, bias_dtype, nullptr, Y,
+    return gemm_i8_impl("bt_ternary_gemm_i8", Q, Q_ROW_MAJOR, s_x, W_T, scale, scale_dtype, scale_len, bias, bias_dtype, nullptr, Y,
                         y_dtype, acc_out, B, N, K, stream);
 }
 
-extern "C" int bt_ternary_gemm_i8_res(const int8_t* Q, const float* s_x, const uint8_t* W_T, const void* scale,
+extern "C" int bt_ternary_gemm_i8_res(const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_T, const void* scale,
                                       int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
                                       const void* residual, void* Y, int y_dtype, int32_t* acc_out, int64_t B,
                                       int64_t N, int64_t K, void* stream) {
-    return gemm_i8_impl("bt_ternary_gemm_i8_res", Q, s_x, W_T, scale, scale_dtype, scale_len, bias, bias_dtype, residual,
+    return gemm_i8_impl("bt_ternary_gemm_i8_res", Q, q_layout, s_x, W_T, scale, scale_dtype, scale_len, bias, bias_dtype, residual,
                         Y, y_dtype, acc_out, B, N, K, stream);
 }
 
@@ -298,10 +328,17 @@ extern "C" int bt_ternary_linear_tensor_core_forward(const void* X, int x_dtype,
     const size_t gemm_bytes = align256(bt_gemm_i8_workspace_bytes(B, N, K));
     int8_t* Q = (int8_t*)((uint8_t*)workspace + gemm_bytes);
     float* s_x = (float*)((uint8_t*)Q + align256((size_t)B * K));
-    rc = bt_act_quant_i8(X, x_dtype, B, K, Q, s_x, stream);
+    // Q is private to this call: written in operand order whenever the layout applies, so that
+    // neither GEMM kernel has to permute activations
+    // (BITTORCH_Q_LAYOUT=rowmajor keeps the row-major layout, for A/B runs)
+    const char* lay = getenv("BITTORCH_Q_LAYOUT");
+    const int q_layout = (K % 16 == 0 && ((uintptr_t)X) % 16 == 0 && !(lay && !strcmp(lay, "rowmajor")))
+                             ? Q_OPERAND_ORDER : Q_ROW_MAJOR;
+    rc = launch_act_quant(X, x_dtype, B, K, Q, s_x, q_layout, (hipStream_t)stream);
     if (rc) return rc;
-    return bt_ternary_gemm_i8(Q, s_x, W_T, scale, scale_dtype, scale_len, bias, bias_dtype, Y, x_dtype, nullptr,
-                              B, N, K, workspace, gemm_bytes, stream);
+    (void)gemm_bytes;
+    return gemm_i8_impl(who, Q, q_layout, s_x, W_T, scale, scale_dtype, scale_len, bias, bias_dtype, nullptr, Y, x_dtype,
+                        nullptr, B, N, K, stream);
 }
 
 // ---- fused producers of the GEMM activations (row_ops.hip) ----------------------------------
@@ -327,7 +364,7 @@ static int check_row_op(const char* who, const void* A, int dtype, int64_t B, in
 }
 
 extern "C" int bt_swiglu(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, int dtype, int64_t B,
-                         int64_t K, void* H, int8_t* Q, float* s_x, void* stream) {
+                         int64_t K, void* H, int8_t* Q, float* s_x, int q_layout, void* stream) {
     const char* who = "bt_swiglu";
     int rc = check_row_op(who, gate, dtype, B, K, ld_gate, H, Q, s_x);
     if (rc) return rc;
@@ -335,13 +372,15 @@ extern "C" int bt_swiglu(const void* gate, int64_t ld_gate, const void* up, int6
         set_error("%s: up is null or its row stride is below K", who);
         return BT_ERR_INVALID;
     }
-    return launch_row_op(0, dtype, gate, ld_gate, up, ld_up, 0.0f, B, K, H, Q, s_x, (hipStream_t)stream, who);
+    if (Q && (rc = check_q_layout(who, q_layout, K, Q, nullptr))) return rc;
+    return launch_row_op(0, dtype, gate, ld_gate, up, ld_up, 0.0f, B, K, H, Q, s_x, q_layout, (hipStream_t)stream, who);
 }
 
 extern "C" int bt_rmsnorm(const void* X, int64_t ld_x, const void* weight, float eps, int dtype, int64_t B,
-                          int64_t K, void* Y, int8_t* Q, float* s_x, void* stream) {
+                          int64_t K, void* Y, int8_t* Q, float* s_x, int q_layout, void* stream) {
     const char* who = "bt_rmsnorm";
     int rc = check_row_op(who, X, dtype, B, K, ld_x, Y, Q, s_x);
     if (rc) return rc;
-    return launch_row_op(1, dtype, X, ld_x, weight, 0, eps, B, K, Y, Q, s_x, (hipStream_t)stream, who);
+    if (Q && (rc = check_q_layout(who, q_layout, K, Q, nullptr))) return rc;
+    return launch_row_op(1, dtype, X, ld_x, weight, 0, eps, B, K, Y, Q, s_x, q_layout, (hipStream_t)stream, who);
 }

@@ -132,7 +132,9 @@ __device__ __forceinline__ void gemm_epilogue_dt(const GemmParams& p, const v4i 
 // wave's LDS / barrier / decode latency hides behind the other's MFMAs.  The two
 // K halves are added through LDS once, after the main loop, and each half of the
 // workgroup finishes 64 of the 128 rows.
-template <bool TAIL>
+// QOO = true: Q is in operand order (16-byte groups already transposed by the quantizer), and
+// the staging copies them to LDS untouched.
+template <bool TAIL, bool QOO>
 __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[65536];  // 2 A stages; reused for the K-half exchange
 
@@ -236,7 +238,11 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
         for (int e = 0; e < 2; e++) {
             const int c = 2 * (a_part & 1) + e;
             uint32_t t[4];
-            transpose4x4_bytes(a_reg[e].x, a_reg[e].y, a_reg[e].z, a_reg[e].w, t);
+            if constexpr (QOO) {
+                t[0] = a_reg[e].x; t[1] = a_reg[e].y; t[2] = a_reg[e].z; t[3] = a_reg[e].w;
+            } else {
+                transpose4x4_bytes(a_reg[e].x, a_reg[e].y, a_reg[e].z, a_reg[e].w, t);
+            }
             *(uint4*)(base + ((size_t)((sub * G_MB + mb) * 64 + c * 16 + i) << 4)) = make_uint4(t[0], t[1], t[2], t[3]);
         }
     };
@@ -418,7 +424,7 @@ bool gemm_i8_supported(int64_t N, int64_t K, const void* Q, const void* W_T) {
            (G_BM + 1) * K < (1ll << 32) && ceil_div(K, 4) * N < (1ll << 32);
 }
 
-int launch_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const Epilogue& epi, void* Y,
+int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_T, const Epilogue& epi, void* Y,
                    int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st) {
     GemmParams p;
     p.Q = Q; p.s_x = s_x; p.W_T = W_T; p.Y = Y; p.acc_out = acc_out; p.epi = epi;
@@ -429,8 +435,14 @@ int launch_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const 
     const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
     p.per_xcd = (int)ceil_div(total, 8);
     const dim3 grid((unsigned)(p.per_xcd * 8)), block(512);
-    if (K % G_BK == 0) hipLaunchKernelGGL(gemm_i8_kernel<false>, grid, block, 0, st, p);
-    else hipLaunchKernelGGL(gemm_i8_kernel<true>, grid, block, 0, st, p);
+    const bool qoo = q_layout == Q_OPERAND_ORDER;
+    if (K % G_BK == 0) {
+        if (qoo) hipLaunchKernelGGL((gemm_i8_kernel<false, true>), grid, block, 0, st, p);
+        else hipLaunchKernelGGL((gemm_i8_kernel<false, false>), grid, block, 0, st, p);
+    } else {
+        if (qoo) hipLaunchKernelGGL((gemm_i8_kernel<true, true>), grid, block, 0, st, p);
+        else hipLaunchKernelGGL((gemm_i8_kernel<true, false>), grid, block, 0, st, p);
+    }
     return check_launch("bt_ternary_gemm_i8");
 }
 

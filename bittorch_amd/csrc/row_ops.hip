@@ -28,6 +28,7 @@ struct RowOpParams {
     float* s_x;         // [B]
     float eps;
     int K;
+    int q_layout;       // Q_ROW_MAJOR / Q_OPERAND_ORDER (K % 16 == 0)
 };
 
 // exp(a) in fp32 by a fixed sequence of correctly rounded operations (range reduction by ln 2 in two
@@ -195,7 +196,8 @@ __global__ __launch_bounds__(256) void row_op_kernel(RowOpParams p) {
             if (e < 4) lo |= byte << (8 * e);
             else hi |= byte << (8 * (e - 4));
         }
-        if (k < K) *(uint2*)(p.Q + row * (int64_t)K + k) = make_uint2(lo, hi);
+        const uint2 o = p.q_layout == Q_OPERAND_ORDER ? q_to_operand_order(lo, hi, tid & 1) : make_uint2(lo, hi);
+        if (k < K) *(uint2*)(p.Q + row * (int64_t)K + k) = o;
     }
 }
 
@@ -238,7 +240,10 @@ __global__ __launch_bounds__(256) void row_op_generic_kernel(RowOpParams p) {
     const float s = (amax > 1e-6f) ? __fdiv_rn(amax, 127.0f) : 1.0f;
     const float inv = __fdiv_rn(1.0f, s);
     if (tid == 0) p.s_x[row] = s;
-    for (int k = tid; k < K; k += 256) p.Q[row * (int64_t)K + k] = quant_i8(value(k), inv);
+    for (int k = tid; k < K; k += 256) {
+        const int64_t pos = p.q_layout == Q_OPERAND_ORDER ? q_operand_order_pos(k) : k;
+        p.Q[row * (int64_t)K + pos] = quant_i8(value(k), inv);
+    }
 }
 
 template <int OP, int DT, bool QUANT>
@@ -264,9 +269,10 @@ static void launch_row_op_dt(const RowOpParams& p, int64_t B, bool fast, hipStre
 
 // op: ROW_SWIGLU / ROW_RMSNORM.  The callers have checked pointers, shapes and dtypes.
 int launch_row_op(int op, int dtype, const void* A, int64_t lda, const void* Bv, int64_t ldb, float eps, int64_t B,
-                  int64_t K, void* H, int8_t* Q, float* s_x, hipStream_t st, const char* who) {
+                  int64_t K, void* H, int8_t* Q, float* s_x, int q_layout, hipStream_t st, const char* who) {
     RowOpParams p;
     p.A = A; p.Bv = Bv; p.lda = lda; p.ldb = ldb; p.H = H; p.Q = Q; p.s_x = s_x; p.eps = eps; p.K = (int)K;
+    p.q_layout = q_layout;
     const int es = dtype_size(dtype);
     auto aligned = [&](const void* ptr, int64_t ld) { return !ptr || (((uintptr_t)ptr) % 16 == 0 && (ld * es) % 16 == 0); };
     const bool fast = K % 8 == 0 && K <= 16384 && aligned(A, lda) && aligned(Bv, op == ROW_SWIGLU ? ldb : 8) &&

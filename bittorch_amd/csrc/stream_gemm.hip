@@ -53,6 +53,7 @@ struct StreamParams {
     int y_dtype;
     int x_vec_ok;         // activation rows may be read with 16-byte loads
     int prehalved;        // MODE_BF16: the activations already carry the factor 1/2 of the +-2.0 weight decode
+    int x_operand_order;  // MODE_I8: X is in the quantizer's operand order (16-byte groups transposed)
 };
 
 enum { LD_BYTE = 0, LD_Q1 = 1, LD_Q2 = 2, LD_V4 = 4, LD_V8 = 8, LD_V16 = 16 };
@@ -281,8 +282,8 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
                         const uint4 v = zero_unless(xr[u], k < (int)p.K);
                         uint4 o;
                         if constexpr (MODE == MODE_I8) {
-                            uint32_t t4[4];
-                            transpose4x4_bytes(v.x, v.y, v.z, v.w, t4);
+                            uint32_t t4[4] = {v.x, v.y, v.z, v.w};
+                            if (!p.x_operand_order) transpose4x4_bytes(v.x, v.y, v.z, v.w, t4);  // uniform
                             o = make_uint4(t4[0], t4[1], t4[2], t4[3]);
                         } else {
                             o = make_uint4(perm(v.z, v.x, 0x05040100u), perm(v.z, v.x, 0x07060302u),
@@ -325,6 +326,8 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
             if constexpr (MODE == MODE_I8) {
                 uint32_t ta[4];
                 if constexpr (XLDS) {  // already in operand order
+                    ta[0] = xa[f][0].x; ta[1] = xa[f][0].y; ta[2] = xa[f][0].z; ta[3] = xa[f][0].w;
+                } else if (p.x_operand_order) {  // uniform
                     ta[0] = xa[f][0].x; ta[1] = xa[f][0].y; ta[2] = xa[f][0].z; ta[3] = xa[f][0].w;
                 } else {
                     transpose4x4_bytes(xa[f][0].x, xa[f][0].y, xa[f][0].z, xa[f][0].w, ta);
@@ -511,9 +514,10 @@ static int launch_stream_mode(StreamParams p, const StreamPlan& pl, hipStream_t 
 // planes = 1: X is [B, K].  planes = 3 (K % 64 == 0): X is [B, 3K], three planes of K values per
 // row whose products with the same weights are summed (fp32 activations split into three bf16
 // terms); the kernel walks 3K values of k and wraps its weight row index every K.
+// q_layout: MODE_I8 only (Q_OPERAND_ORDER needs K % 16 == 0 and 16-byte aligned rows)
 int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, const uint8_t* W_T,
                   const Epilogue& epi, void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N,
-                  int64_t K, int planes, hipStream_t st) {
+                  int64_t K, int planes, int q_layout, hipStream_t st) {
     const int64_t Kb = ceil_div(K, 4);
     const int64_t Kx = K * planes;
     const StreamPlan pl = stream_plan(mode, B, N, Kb);
@@ -530,6 +534,7 @@ int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, co
         p.N = N; p.K = Kx; p.Kb = Kb;
         p.wsteps = (int)ceil_div(Kb, 16);
         p.prehalved = planes == 3;
+        p.x_operand_order = (mode == MODE_I8 && q_layout == Q_OPERAND_ORDER) ? 1 : 0;
         p.M = (int)((B - m0 < 16) ? (B - m0) : 16);
         p.y_dtype = y_dtype;
         p.x_vec_ok = (((uintptr_t)p.X) % 16 == 0) && ((Kx * x_elem_size) % 16 == 0);

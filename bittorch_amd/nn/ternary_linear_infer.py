@@ -43,12 +43,13 @@ class TernaryLinearInference(nn.Module):
         return y if residual is None else y + residual
 
     def forward_int8(self, q: Tensor, s_x: Tensor, out_dtype: torch.dtype = torch.bfloat16,
-                     residual: Optional[Tensor] = None) -> Tensor:
+                     residual: Optional[Tensor] = None, q_operand_order: bool = False) -> Tensor:
         """Forward from activations already quantized per row to int8 (``ops.rmsnorm`` /
-        ``ops.swiglu`` with ``quantize=True``): int8 matrix cores, int32 accumulators (GPU only)."""
+        ``ops.swiglu`` / ``ops.act_quant_int8`` with ``quantize=True``): int8 matrix cores, int32
+        accumulators (GPU only).  ``q_operand_order`` as in :func:`ops.ternary_linear_int8`."""
         from ..ops.fused import ternary_linear_int8
         return ternary_linear_int8(q, s_x, self.weight_packed, self.scale, self.in_features, self.bias,
-                                   out_dtype, residual)
+                                   out_dtype, residual, q_operand_order)
 
     def extra_repr(self) -> str:
         dense = 4 * self.out_features * self.in_features

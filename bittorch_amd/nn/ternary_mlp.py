@@ -47,10 +47,10 @@ class TernarySwiGLU(nn.Module):
         gu = self.gate_up(h)
         return gu[..., :self.ffn], gu[..., self.ffn:]
 
-    def _gate_up_int8(self, q: Tensor, s: Tensor, dtype):
+    def _gate_up_int8(self, q: Tensor, s: Tensor, dtype, oo: bool):
         if self.gate_up is None:
-            return self.gate.forward_int8(q, s, dtype), self.up.forward_int8(q, s, dtype)
-        gu = self.gate_up.forward_int8(q, s, dtype)
+            return (self.gate.forward_int8(q, s, dtype, None, oo), self.up.forward_int8(q, s, dtype, None, oo))
+        gu = self.gate_up.forward_int8(q, s, dtype, None, oo)
         return gu[..., :self.ffn], gu[..., self.ffn:]
 
     def forward(self, x: Tensor, norm_weight: Optional[Tensor] = None, eps: Optional[float] = None,
@@ -67,12 +67,12 @@ class TernarySwiGLU(nn.Module):
         if self.compute == "float":
             h = x if eps is None else fused.rmsnorm(x, norm_weight, eps)
             return self.down(fused.swiglu(*self._gate_up(h)), residual)
+        # the int8 activations stay inside this call: hand them over in the matrix cores' own order
+        oo1, oo2 = x.shape[-1] % 16 == 0, self.ffn % 16 == 0
         if eps is None:
-            from .. import _C
-            q, s = _C.act_quant_int8(x.reshape(-1, x.shape[-1]))
-            q, s = q.reshape(x.shape), s.reshape(x.shape[:-1])
+            q, s = fused.act_quant_int8(x, oo1)
         else:
-            q, s = fused.rmsnorm(x, norm_weight, eps, store=False, quantize=True)
-        g, u = self._gate_up_int8(q, s, x.dtype)
-        q2, s2 = fused.swiglu(g, u, store=False, quantize=True)
-        return self.down.forward_int8(q2, s2, x.dtype, residual)
+            q, s = fused.rmsnorm(x, norm_weight, eps, store=False, quantize=True, operand_order=oo1)
+        g, u = self._gate_up_int8(q, s, x.dtype, oo1)
+        q2, s2 = fused.swiglu(g, u, store=False, quantize=True, operand_order=oo2)
+        return self.down.forward_int8(q2, s2, x.dtype, residual, oo2)

@@ -6,7 +6,9 @@
   quantized per row to int8 for the int8 matrix-core GEMM;
 * :func:`rmsnorm` -- RMSNorm, optionally with the same quantization fused in;
 * :func:`ternary_linear_int8` -- the int8 GEMM on pre-quantized activations, so that one
-  quantization feeds several projections (q/k/v, gate/up), with an optional residual.
+  quantization feeds several projections (q/k/v, gate/up), with an optional residual;
+* ``operand_order=True`` on the quantizing side with ``q_operand_order=True`` on the GEMM side
+  hands the int8 activations over in the order the matrix cores consume them.
 
 The residual connection itself is an argument of the linear layers' forward
 (``residual=``): the add happens in the GEMM epilogue.
@@ -20,27 +22,39 @@ import torch
 from torch import Tensor
 
 
-def swiglu(gate: Tensor, up: Tensor, store: bool = True, quantize: bool = False):
+def swiglu(gate: Tensor, up: Tensor, store: bool = True, quantize: bool = False, operand_order: bool = False):
     from .. import _C
 
-    return _C.swiglu(gate, up, store, quantize)
+    return _C.swiglu(gate, up, store, quantize, operand_order)
 
 
 def rmsnorm(x: Tensor, weight: Optional[Tensor] = None, eps: float = 1e-6, store: bool = True,
-            quantize: bool = False):
+            quantize: bool = False, operand_order: bool = False):
     from .. import _C
 
-    return _C.rmsnorm(x, weight, eps, store, quantize)
+    return _C.rmsnorm(x, weight, eps, store, quantize, operand_order)
+
+
+def act_quant_int8(x: Tensor, operand_order: bool = False) -> Tuple[Tensor, Tensor]:
+    """Per-row int8 quantization of ``x`` ``(*, K)``: ``(q int8 (*, K), s_x fp32 (*))``."""
+    from .. import _C
+
+    q, s = _C.act_quant_int8(x.reshape(-1, x.shape[-1]), operand_order)
+    return q.reshape(x.shape), s.reshape(x.shape[:-1])
 
 
 def ternary_linear_int8(q: Tensor, s_x: Tensor, w_packed_T: Tensor, scale: Tensor, in_features: int,
                         bias: Optional[Tensor] = None, out_dtype: torch.dtype = torch.bfloat16,
-                        residual: Optional[Tensor] = None) -> Tensor:
-    """``q`` int8 ``(*, K)`` with per-row scales ``s_x`` ``(*)`` -> ``(*, N)`` in ``out_dtype``."""
+                        residual: Optional[Tensor] = None, q_operand_order: bool = False) -> Tensor:
+    """``q`` int8 ``(*, K)`` with per-row scales ``s_x`` ``(*)`` -> ``(*, N)`` in ``out_dtype``.
+
+    ``q_operand_order``: ``q`` was produced with ``operand_order=True`` (every 16-byte group already
+    in the order the matrix cores take it; K % 16 == 0), which spares the GEMM a permutation."""
     from .. import _C
 
     lead = q.shape[:-1]
     y = _C.ternary_gemm_int8(q.reshape(-1, q.shape[-1]), s_x.reshape(-1), w_packed_T, scale, bias, in_features,
                              out_dtype, False,
-                             None if residual is None else residual.reshape(-1, residual.shape[-1]))
+                             None if residual is None else residual.reshape(-1, residual.shape[-1]),
+                             q_operand_order)
     return y.reshape(*lead, y.shape[-1])

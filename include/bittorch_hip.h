@@ -119,6 +119,22 @@ int bt_act_quant_i8(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q,
                     void* stream);
 
 /*
+ * Layout of quantized activations between a quantizing kernel and an int8 GEMM (no counterpart in
+ * the reference, whose kernel quantizes inside its own shared memory):
+ *   BT_Q_ROW_MAJOR      int8 [B,K] as is (what bt_act_quant_i8 writes and bt_ternary_gemm_i8 reads);
+ *   BT_Q_OPERAND_ORDER  the same rows with every aligned 16-byte group stored as the 4x4 byte
+ *                       transpose of its natural order (byte 4c+r = element 4r+c): the k order the
+ *                       in-register weight decode gives the matrix-core operands, so the GEMMs copy
+ *                       activations to the matrix cores without permuting them (4 % faster at
+ *                       2048x4096x4096).  Needs K % 16 == 0 and 16-byte aligned buffers.
+ * A buffer must be read with the layout it was written in; bt_ternary_linear_tensor_core_forward
+ * picks the operand order by itself for its private Q.
+ */
+enum { BT_Q_ROW_MAJOR = 0, BT_Q_OPERAND_ORDER = 1 };
+int bt_act_quant_i8_layout(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x,
+                           int q_layout, void* stream);
+
+/*
  * int8 x packed-ternary GEMM on the matrix cores, int32 accumulators.
  * Restates the MMA stage and epilogue of kernel_v2_tensor_core
  * (ternary_gemm_tensor_core.cu:583-589, :652): weights decode to +-127,
@@ -140,6 +156,7 @@ int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, co
  * counterpart in the reference's Python/CUDA code; they serve the pre-norm block of its JS
  * runtime (js/src/models/TernaryTransformer.ts:489-521: x = x + attn(norm(x)); x = x + mlp(norm(x))).
  *   residual: [B,N] in Y's dtype, 16-byte aligned; NULL = no residual (the plain entry point).
+ *   q_layout (int8 variant): layout Q was written in.
  *   It may be Y itself (every output element is read once, by the thread that then writes it).
  */
 int bt_ternary_linear_packed_forward_res(const void* X, int x_dtype, const uint8_t* W_T,
@@ -147,7 +164,7 @@ int bt_ternary_linear_packed_forward_res(const void* X, int x_dtype, const uint8
                                          const void* bias, int bias_dtype, const void* residual,
                                          void* Y, int64_t B, int64_t N, int64_t K, void* workspace,
                                          size_t workspace_bytes, void* stream);
-int bt_ternary_gemm_i8_res(const int8_t* Q, const float* s_x, const uint8_t* W_T, const void* scale,
+int bt_ternary_gemm_i8_res(const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_T, const void* scale,
                            int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
                            const void* residual, void* Y, int y_dtype, int32_t* acc_out, int64_t B,
                            int64_t N, int64_t K, void* stream);
@@ -164,11 +181,12 @@ int bt_ternary_gemm_i8_res(const int8_t* Q, const float* s_x, const uint8_t* W_T
  *               place); exp is a fixed fp32 polynomial (0.85 ulp), restated by the CPU oracle.
  *   bt_rmsnorm: y = rd( (x * r) * w ),  r = 1/sqrt(float(sum double(x)^2)/K + eps)
  *               weight [K] in the same dtype or NULL (ones).
+ *   q_layout: layout of Q (BT_Q_ROW_MAJOR / BT_Q_OPERAND_ORDER, see bt_act_quant_i8_layout).
  */
 int bt_swiglu(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, int dtype, int64_t B,
-              int64_t K, void* H, int8_t* Q, float* s_x, void* stream);
+              int64_t K, void* H, int8_t* Q, float* s_x, int q_layout, void* stream);
 int bt_rmsnorm(const void* X, int64_t ld_x, const void* weight, float eps, int dtype, int64_t B,
-               int64_t K, void* Y, int8_t* Q, float* s_x, void* stream);
+               int64_t K, void* Y, int8_t* Q, float* s_x, int q_layout, void* stream);
 
 /*
  * Matrix-core forward from float activations: bt_act_quant_i8 followed by

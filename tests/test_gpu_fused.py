@@ -295,3 +295,50 @@ def test_block_glue_at_config5_sizes():
     assert torch.equal(_C.ternary_linear_packed_forward(y, packed, scale, None, 2560, x), lin + x)
     lin8 = _C.ternary_gemm_int8(q, s, packed, scale, None, 2560, torch.bfloat16)
     assert torch.equal(_C.ternary_gemm_int8(q, s, packed, scale, None, 2560, torch.bfloat16, residual=x), lin8 + x)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("b,n,k", [(1, 4096, 4096), (16, 1000, 528), (33, 256, 128), (200, 520, 272), (130, 260, 80)])
+def test_operand_order_activations_give_the_same_results(oracle, dtype, b, n, k):
+    """Q written in the matrix cores' operand order is the row-major Q with every 16-byte group
+    transposed 4x4, and both int8 GEMM kernels return the same bits from either layout."""
+    from bittorch_amd import _C
+    announce("operand order", dtype, b, n, k)
+    packed, scale, bias = _packed_case(n, k, seed=b + n)
+    x = seeded_acts(b, k, seed=5, dtype=dtype, outliers=True).cuda()
+    q, s = _C.act_quant_int8(x)
+    qo, so = _C.act_quant_int8(x, operand_order=True)
+    assert torch.equal(s, so)
+    assert torch.equal(qo.view(b, k // 16, 4, 4), q.view(b, k // 16, 4, 4).transpose(2, 3))
+    res = seeded_acts(b, n, seed=6, dtype=torch.bfloat16).cuda()
+    y, acc = _C.ternary_gemm_int8(q, s, packed, scale, bias, k, torch.bfloat16, return_acc=True)
+    yo, acco = _C.ternary_gemm_int8(qo, so, packed, scale, bias, k, torch.bfloat16, return_acc=True, q_operand_order=True)
+    assert torch.equal(acc, acco) and torch.equal(y, yo)
+    yr = _C.ternary_gemm_int8(qo, so, packed, scale, bias, k, torch.bfloat16, residual=res, q_operand_order=True)
+    assert torch.equal(yr, y + res)
+    # the fused producers write the same layout
+    g2 = seeded_acts(b, k, seed=7, dtype=dtype).cuda()
+    qs, ss = _C.swiglu(x, g2, False, True)
+    qso, sso = _C.swiglu(x, g2, False, True, operand_order=True)
+    assert torch.equal(ss, sso) and torch.equal(qso.view(b, k // 16, 4, 4), qs.view(b, k // 16, 4, 4).transpose(2, 3))
+    qn, sn = _C.rmsnorm(x, None, 1e-5, False, True)
+    qno, sno = _C.rmsnorm(x, None, 1e-5, False, True, operand_order=True)
+    assert torch.equal(sn, sno) and torch.equal(qno.view(b, k // 16, 4, 4), qn.view(b, k // 16, 4, 4).transpose(2, 3))
+
+
+def test_operand_order_needs_whole_groups():
+    from bittorch_amd import _C
+    x = seeded_acts(4, 40, dtype=torch.bfloat16).cuda()
+    with pytest.raises(RuntimeError, match="operand-order layout needs K % 16 == 0"):
+        _C.act_quant_int8(x, operand_order=True)
+    with pytest.raises(RuntimeError, match="operand-order layout needs K % 16 == 0"):
+        _C.swiglu(x, x, False, True, operand_order=True)
+
+
+def test_operand_order_on_the_generic_row_kernels(monkeypatch):
+    from bittorch_amd import _C
+    monkeypatch.setenv("BITTORCH_ROWOP_GENERIC", "1")
+    x = seeded_acts(5, 64, dtype=torch.float16).cuda()
+    qn, _ = _C.rmsnorm(x, None, 1e-5, False, True)
+    qo, _ = _C.rmsnorm(x, None, 1e-5, False, True, operand_order=True)
+    assert torch.equal(qo.view(5, 4, 4, 4), qn.view(5, 4, 4, 4).transpose(2, 3))
