@@ -327,3 +327,38 @@ def test_rmsnorm_oracle_against_float64_closed_form(oracle, dtype, rel):
     q_ref, s_ref = oracle.act_quant_i8(y)
     np.testing.assert_array_equal(q, q_ref)
     np.testing.assert_array_equal(s, s_ref)
+
+
+# ---- property tests over arbitrary small shapes (hypothesis) ------------------------------------
+
+def test_codec_and_quantizer_properties_over_random_shapes(oracle):
+    from hypothesis import given, settings, strategies as st
+
+    @settings(max_examples=60, deadline=None)
+    @given(n=st.integers(1, 9), k=st.integers(1, 37), seed=st.integers(0, 2 ** 16), tf=st.sampled_from([0.0, 0.05, 0.3, 1.0]),
+           per_channel=st.booleans())
+    def run(n, k, seed, tf, per_channel):
+        rng = np.random.default_rng(seed)
+        w = (rng.normal(0, 0.02, (n, k)) * rng.choice([0.0, 1.0, 50.0], (n, 1))).astype(np.float32)
+        tern, scale = oracle.ternary_quantize(w, tf, per_channel)
+        # codes are ternary; the scale is the (row or tensor) absmax floored at 1e-8; an entry is kept
+        # exactly when its magnitude exceeds fl32(tf * scale) and then carries the sign of the weight
+        assert set(np.unique(tern)).issubset({-1, 0, 1})
+        amax = np.abs(w).max(axis=1) if per_channel else np.full(n, np.abs(w).max())
+        np.testing.assert_array_equal(np.broadcast_to(scale.reshape(-1), (n,)) if per_channel else np.full(n, scale.reshape(-1)[0]),
+                                      np.maximum(amax, np.float32(1e-8)).astype(np.float32))
+        thr = (np.float32(tf) * np.maximum(amax, np.float32(1e-8)).astype(np.float32)).astype(np.float32)
+        keep = np.abs(w) > thr[:, None]
+        np.testing.assert_array_equal(tern, (np.sign(w) * keep).astype(np.int8))
+        # pack -> unpack is the identity for every K (padding codes are zero and sliced off), and the
+        # transposed layout is the transpose of the row-major one
+        packed, kk = oracle.pack_ternary(tern)
+        assert kk == k and packed.shape == (n, (k + 3) // 4)
+        np.testing.assert_array_equal(oracle.unpack_ternary(packed, k), tern)
+        packed_t, _ = oracle.pack_ternary_transposed(tern)
+        np.testing.assert_array_equal(packed_t, packed.T)
+        np.testing.assert_array_equal(oracle.unpack_ternary_transposed(packed_t, k), tern)
+        if k % 4:
+            assert not np.any(packed[:, -1] >> (2 * (k % 4)))  # padding slots hold code 0
+
+    run()
