@@ -143,3 +143,23 @@ def test_kernel_selection_env_matches_default():
             os.environ.pop("BITTORCH_KERNEL", None)
         else:
             os.environ["BITTORCH_KERNEL"] = old
+
+
+@pytest.mark.parametrize("n,k", [(128256, 4096), (50257, 768), (8192, 28672)])
+def test_vocabulary_wide_and_very_deep_layers(n, k):
+    """Output widths of a vocabulary projection (one of them odd: byte-granular loads) and a K beyond
+    any FFN: both paths against a dense fp32 product of the dequantized weights."""
+    from bittorch_amd import _C
+    announce("wide / deep layer", n, k)
+    dev = torch.device("cuda")
+    w = torch.randn(n, k, device=dev, generator=torch.Generator(device="cuda").manual_seed(n)) * 0.02
+    packed, scale, _ = _C.ternary_quantize_pack(w, 0.05, True)
+    wd = _C.unpack_dequant(packed, k, scale, torch.float32)
+    del w
+    for m in (1, 7, 64):
+        x = torch.randn(m, k, device=dev).bfloat16()
+        ref = x.float() @ wd.t()
+        y = _C.ternary_linear_packed_forward(x, packed, scale, None, k)
+        assert ((y.float() - ref).abs().max() / ref.abs().max()).item() < 1e-2
+        y8 = _C.ternary_linear_tensor_core_forward(x, packed, scale, None, k, 2)
+        assert ((y8.float() - ref).abs().max() / ref.abs().max()).item() < 5e-2
