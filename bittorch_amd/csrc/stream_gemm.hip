@@ -432,7 +432,6 @@ static int ld_columns(int ld) { return ld == LD_BYTE ? 16 : 16 * ld; }
 
 StreamPlan stream_plan(int mode, int64_t M, int64_t N, int64_t Kb) {
     StreamPlan pl;
-    (void)mode;
     (void)Kb;
     // optional override for tuning runs: BITTORCH_STREAM_CFG="ld,waves"
     int o_ld = -1, o_waves = 0;
@@ -446,7 +445,9 @@ StreamPlan stream_plan(int mode, int64_t M, int64_t N, int64_t Kb) {
         // widest lane load the row pitch allows, narrowed until there are enough tiles to
         // occupy the chip (measured: 172 tiles of 64 columns beat 344 of 32 for a 16-row
         // batch, which re-reads its activations once per tile; a single row prefers >= 256)
-        ld = (N % 16 == 0) ? 16 : (N % 8 == 0) ? 8 : 4;
+        // (the int8 mode, whose decode is light, does better with 128-column tiles and 8 waves than
+        // with 256-column tiles and 4 on very wide layers: 23.5 -> 17.4 us at N = 65536, K = 4096)
+        ld = (N % 16 == 0 && mode != MODE_I8) ? 16 : (N % 8 == 0) ? 8 : 4;
         const int min_tiles = (M > 4) ? 160 : 256;
         while (ld > 1 && ceil_div(N, ld_columns(ld)) < min_tiles) ld >>= 1;
     }
