@@ -524,6 +524,47 @@ def main():
                 glue[f"{name}_{m}x{k}"] = {"us": round(us, 2), "algorithmic_GBps": round(nbytes / (us * 1e-6) / 1e9, 1)}
             del gs, us_
         extra["block_glue_bf16"] = glue
+        # one decode token through the ternary layers of a config-5 block (M = 1, bf16, HIP graph over 16 distinct
+        # layers' weights): seven separate GEMVs + torch glue against q|k|v and gate|up as single launches with the
+        # glue fused; attention itself (KV cache) is left out of both
+        import bittorch_amd as bt
+        d_model, ffn, nl = 2560, 6912, 16  # 16 x 19.8 MB of packed weights: beyond the Infinity Cache
+        def mk(i, o):
+            pk = rand_packed(o, i, 1)[0]
+            return bt.nn.TernaryLinearInference(i, o, pk, torch.rand(o, device=dev) * 0.05 + 0.01)
+        layers_ = [{nm: mk(*sh) for nm, sh in (("q", (d_model, d_model)), ("k", (d_model, d_model)), ("v", (d_model, d_model)),
+                                              ("o", (d_model, d_model)), ("gate", (d_model, ffn)), ("up", (d_model, ffn)),
+                                              ("down", (ffn, d_model)))} for _ in range(nl)]
+        for L in layers_:
+            L["qkv"] = bt.utils.fuse_ternary_linear_inference(L["q"], L["k"], L["v"])
+            L["mlp"] = bt.nn.TernarySwiGLU(L["gate"], L["up"], L["down"], compute="float", fuse_gate_up=True)
+        xt = torch.randn(1, d_model, device=dev).bfloat16()
+        nw = torch.ones(d_model, device=dev).bfloat16()
+        eps = 1e-5
+
+        def decode_plain(i):
+            L = layers_[i % nl]
+            h = F.rms_norm(xt, (d_model,), nw, eps)
+            a = L["q"](h) + L["k"](h) + L["v"](h)          # stands in for attention over the cache
+            x1 = xt + L["o"](a)
+            h2 = F.rms_norm(x1, (d_model,), nw, eps)
+            return x1 + L["down"](F.silu(L["gate"](h2)) * L["up"](h2))
+
+        def decode_fused(i):
+            L = layers_[i % nl]
+            qkv = L["qkv"](_C.rmsnorm(xt, nw, eps))
+            a = qkv[:, :d_model] + qkv[:, d_model:2 * d_model] + qkv[:, 2 * d_model:]
+            x1 = L["o"](a, xt)
+            return L["mlp"](x1, nw, eps, residual=x1)
+
+        _, ev_p = graph_time(decode_plain, 64, 8, torch)
+        _, ev_f = graph_time(decode_fused, 64, 8, torch)
+        extra["decode_token_per_block_bf16"] = {
+            "us_seven_gemvs_torch_glue": round(ev_p / 64 * 1e3, 2),
+            "us_fused_layers_and_glue": round(ev_f / 64 * 1e3, 2),
+            "packed_weight_bytes_per_block": (4 * d_model * d_model + 3 * d_model * ffn) // 4,
+        }
+        del layers_
         # config 5: the 30-layer block stack, end to end
         if not args.no_block_stack:
             try:
