@@ -526,7 +526,8 @@ def main():
         extra["block_glue_bf16"] = glue
         # one decode token through the ternary layers of a config-5 block (M = 1, bf16, HIP graph over 16 distinct
         # layers' weights): seven separate GEMVs + torch glue against q|k|v and gate|up as single launches with the
-        # glue fused; attention itself (KV cache) is left out of both
+        # glue fused (RMSNorm and SwiGLU inside the GEMV kernels that consume them, residuals in their epilogues);
+        # attention itself (KV cache) is left out of both
         import bittorch_amd as bt
         d_model, ffn, nl = 2560, 6912, 16  # 16 x 19.8 MB of packed weights: beyond the Infinity Cache
         def mk(i, o):
@@ -552,7 +553,7 @@ def main():
 
         def decode_fused(i):
             L = layers_[i % nl]
-            qkv = L["qkv"](_C.rmsnorm(xt, nw, eps))
+            qkv = L["qkv"](xt, None, (nw, eps))            # RMSNorm inside the GEMV kernel
             a = qkv[:, :d_model] + qkv[:, d_model:2 * d_model] + qkv[:, 2 * d_model:]
             x1 = L["o"](a, xt)
             return L["mlp"](x1, nw, eps, residual=x1)

@@ -209,6 +209,46 @@ def ternary_linear_packed_forward(X: Tensor, W_T: Tensor, scale: Tensor,
     return y.reshape(*X.shape[:-1], N)
 
 
+def ternary_linear_packed_forward_fused(X: Tensor, W_T: Tensor, scale: Tensor, bias: Optional[Tensor] = None,
+                                        in_features: int = -1, residual: Optional[Tensor] = None,
+                                        norm: Optional[Tuple[Optional[Tensor], float]] = None,
+                                        swiglu_up: Optional[Tensor] = None) -> Tensor:
+    """``linear(pro(X)) [+ residual]`` with ``pro`` = RMSNorm (``norm=(weight or None, eps)``) or
+    SwiGLU (``X`` is the gate, ``swiglu_up`` the other factor): the values :func:`rmsnorm` /
+    :func:`swiglu` would store, without the extra launch when ``X`` is one 16-bit row (a decode token)."""
+    _check((norm is None) != (swiglu_up is None), "exactly one of norm and swiglu_up must be given")
+    if in_features < 0:
+        in_features = X.shape[-1]
+    K, N = _packed_checks(X, W_T, scale, bias, in_features)
+    _check(X.dtype in _DT, "X must be float32, float16 or bfloat16")
+    x2 = _rows_2d(X, K)
+    W_T = W_T.contiguous()
+    scale = _prep_vec(scale, x2)
+    bias = None if bias is None else _prep_vec(bias, x2)
+    B = x2.shape[0]
+    if norm is not None:
+        w, eps = norm
+        if w is not None:
+            _check(w.dim() == 1 and w.shape[0] == K, "norm weight must be 1D [K]")
+            w = w.to(X.dtype).contiguous()
+        op, pb, ldb = 1, w, 0
+    else:
+        _check(swiglu_up.shape == X.shape and swiglu_up.dtype == X.dtype, "gate and up must match in shape and dtype")
+        u2 = _rows_2d(swiglu_up, K)
+        op, pb, ldb, eps = 2, u2, u2.stride(0), 0.0
+    _check(_all_cuda(pb), "All tensors must be CUDA")
+    xdt = _dt(x2, "X")
+    y = torch.empty((B, N), dtype=X.dtype, device=X.device)
+    res = None if residual is None else _residual_2d(residual, X, X.shape[:-1], N)
+    with torch.cuda.device(X.device):
+        ws = _workspace(_L.bt_packed_forward_fused_workspace_bytes(B, N, K, xdt), X.device)
+        _status(_L.bt_ternary_linear_packed_forward_fused(
+            x2.data_ptr(), x2.stride(0), xdt, op, _ptr(pb), ldb, float(eps), W_T.data_ptr(), scale.data_ptr(),
+            _dt(scale, "scale"), scale.numel(), _ptr(bias), 0 if bias is None else _dt(bias, "bias"), _ptr(res),
+            y.data_ptr(), B, N, K, _ptr(ws), 0 if ws is None else ws.numel(), _stream(X)))
+    return y.reshape(*X.shape[:-1], N)
+
+
 def ternary_linear_tensor_core_forward(X: Tensor, W_T: Tensor, scale: Tensor,
                                        bias: Optional[Tensor] = None, in_features: int = -1,
                                        version: int = 1) -> Tensor:

@@ -49,6 +49,9 @@ SIGNATURES = {
     "bt_swiglu": (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _vp, _vp, _vp, _int, _vp]),
     "bt_rmsnorm": (_int, [_vp, _i64, _vp, ctypes.c_float, _int, _i64, _i64, _vp, _vp, _vp, _int, _vp]),
     "bt_act_quant_i8_layout": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _int, _vp]),
+    "bt_packed_forward_fused_workspace_bytes": (_sz, [_i64, _i64, _i64, _int]),
+    "bt_ternary_linear_packed_forward_fused": (_int, [_vp, _i64, _int, _int, _vp, _i64, ctypes.c_float, _vp, _vp, _int,
+                                                      _i64, _vp, _int, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

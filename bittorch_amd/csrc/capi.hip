@@ -32,7 +32,8 @@ bool stream_supported(int64_t N, int64_t K, const void* W_T);
 size_t stream_workspace_bytes(int mode, int64_t M, int64_t N, int64_t Kb);
 int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, const uint8_t* W_T,
                   const Epilogue& epi, void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N,
-                  int64_t K, int planes, int q_layout, hipStream_t st);
+                  int64_t K, int planes, int q_layout, int pro_op, const void* pro_b, float pro_eps, hipStream_t st);
+bool stream_prologue_fusable(int mode, int64_t B, int64_t N, int64_t K, const void* X, const void* pro_b);
 int launch_split_f32_planes(const void* X, int64_t B, int64_t K, void* P, hipStream_t st);
 int launch_packed_generic(const void* X, int x_dtype, const uint8_t* W_T, const Epilogue& epi, void* Y,
                           int64_t B, int64_t N, int64_t K, hipStream_t st);
@@ -177,7 +178,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         // tall batches go to the tiled matrix-core kernel, decode shapes stream the weights
         if (B > kStreamMaxRows && gemm_f16_supported(N, K, X, W_T, Y))
             return launch_gemm_f16(mode, X, W_T, epi, Y, x_dtype, B, N, K, 1, st);
-        return launch_stream(mode, X, 2, nullptr, W_T, epi, Y, x_dtype, nullptr, B, N, K, 1, Q_ROW_MAJOR, st);
+        return launch_stream(mode, X, 2, nullptr, W_T, epi, Y, x_dtype, nullptr, B, N, K, 1, Q_ROW_MAJOR, 0, nullptr, 0.0f, st);
     }
     if (x_dtype == BT_F32 && packed_uses_f32_planes(X, W_T, Y, N, K) && workspace &&
         workspace_bytes >= f32_planes_bytes(B, K) && ((uintptr_t)workspace) % 256 == 0) {
@@ -186,7 +187,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         if (rc) return rc;
         if (B > kStreamMaxRows && gemm_f16_supported(N, 3 * K, workspace, W_T, Y))
             return launch_gemm_f16(MODE_BF16, workspace, W_T, epi, Y, BT_F32, B, N, K, 3, st);
-        return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, epi, Y, BT_F32, nullptr, B, N, K, 3, Q_ROW_MAJOR, st);
+        return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, epi, Y, BT_F32, nullptr, B, N, K, 3, Q_ROW_MAJOR, 0, nullptr, 0.0f, st);
     }
     return launch_packed_generic(X, x_dtype, W_T, epi, Y, B, N, K, st);
 }
@@ -284,7 +285,7 @@ static int gemm_i8_impl(const char* who, const int8_t* Q, int q_layout, const fl
                       (long long)ceil_div(K, 4), (long long)N);
             return BT_ERR_INVALID;
         }
-        return launch_stream(MODE_I8, Q, 1, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, 1, q_layout, st);
+        return launch_stream(MODE_I8, Q, 1, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, 1, q_layout, 0, nullptr, 0.0f, st);
     }
     return launch_gemm_i8(Q, q_layout, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, st);
 }
@@ -383,4 +384,57 @@ extern "C" int bt_rmsnorm(const void* X, int64_t ld_x, const void* weight, float
     if (rc) return rc;
     if (Q && (rc = check_q_layout(who, q_layout, K, Q, nullptr))) return rc;
     return launch_row_op(1, dtype, X, ld_x, weight, 0, eps, B, K, Y, Q, s_x, q_layout, (hipStream_t)stream, who);
+}
+
+// ---- packed forward with an activation prologue -----------------------------------------------
+extern "C" size_t bt_packed_forward_fused_workspace_bytes(int64_t B, int64_t N, int64_t K, int x_dtype) {
+    if (B <= 0 || N <= 0 || K <= 0 || !valid_dtype(x_dtype)) return 0;
+    // [the prologue's output, B x K in x_dtype, when it runs as its own kernel][the forward's own scratch]
+    return align256((size_t)B * K * dtype_size(x_dtype)) + bt_packed_forward_workspace_bytes(B, N, K, x_dtype);
+}
+
+extern "C" int bt_ternary_linear_packed_forward_fused(const void* X, int64_t ld_x, int x_dtype, int pro_op,
+                                                      const void* pro_b, int64_t ld_b, float eps,
+                                                      const uint8_t* W_T, const void* scale, int scale_dtype,
+                                                      int64_t scale_len, const void* bias, int bias_dtype,
+                                                      const void* residual, void* Y, int64_t B, int64_t N,
+                                                      int64_t K, void* workspace, size_t workspace_bytes,
+                                                      void* stream) {
+    const char* who = "bt_ternary_linear_packed_forward_fused";
+    int rc = check_shape(who, X, W_T, Y, x_dtype, B, N, K);
+    if (rc) return rc;
+    if (pro_op != 1 && pro_op != 2) {
+        set_error("%s: prologue must be BT_PRO_RMSNORM or BT_PRO_SWIGLU (got %d)", who, pro_op);
+        return BT_ERR_INVALID;
+    }
+    if (ld_x < K || (pro_op == 2 && (!pro_b || ld_b < K))) {
+        set_error("%s: row stride below K, or SwiGLU without its second operand", who);
+        return BT_ERR_INVALID;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    // one 16-bit row on the streaming kernel: the prologue runs inside the GEMV, on the row's way into LDS
+    if (x_dtype != BT_F32 && B == 1 && packed_uses_stream(x_dtype, W_T, Y, N, K)) {
+        const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
+        if (stream_prologue_fusable(mode, B, N, K, X, pro_b)) {
+            Epilogue epi;
+            rc = make_epilogue(who, scale, scale_dtype, scale_len, bias, bias_dtype, N, &epi);
+            if (rc) return rc;
+            rc = set_residual(who, residual, &epi);
+            if (rc) return rc;
+            return launch_stream(mode, X, 2, nullptr, W_T, epi, Y, x_dtype, nullptr, B, N, K, 1, Q_ROW_MAJOR, pro_op, pro_b,
+                                 eps, st);
+        }
+    }
+    // otherwise: the prologue as its own kernel into the workspace, then the plain forward
+    const size_t h_bytes = align256((size_t)B * K * dtype_size(x_dtype));
+    if (!workspace || workspace_bytes < h_bytes || ((uintptr_t)workspace) % 256 != 0) {
+        set_error("%s: workspace of %zu bytes (256-byte aligned) needed, %zu given", who,
+                  bt_packed_forward_fused_workspace_bytes(B, N, K, x_dtype), workspace_bytes);
+        return BT_ERR_WORKSPACE;
+    }
+    rc = launch_row_op(pro_op == 2 ? 0 : 1, x_dtype, X, ld_x, pro_b, ld_b, eps, B, K, workspace, nullptr, nullptr,
+                       Q_ROW_MAJOR, st, who);
+    if (rc) return rc;
+    return packed_forward_impl(who, workspace, x_dtype, W_T, scale, scale_dtype, scale_len, bias, bias_dtype, residual, Y,
+                               B, N, K, (uint8_t*)workspace + h_bytes, workspace_bytes - h_bytes, stream);
 }

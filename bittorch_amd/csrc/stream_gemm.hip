@@ -34,7 +34,7 @@
 // Activations: for M = 1 (XLDS) a wave fetches its whole K-slice of x with one or a
 // few fully coalesced loads into LDS and reads operand fragments from there; for
 // M > 1 every lane loads its own 16-element fragment per step.
-#include "bt_common.h"
+#include "row_math.h"
 
 namespace bt {
 
@@ -54,7 +54,14 @@ struct StreamParams {
     int x_vec_ok;         // activation rows may be read with 16-byte loads
     int prehalved;        // MODE_BF16: the activations already carry the factor 1/2 of the +-2.0 weight decode
     int x_operand_order;  // MODE_I8: X is in the quantizer's operand order (16-byte groups transposed)
+    // Prologue applied to the single activation row on its way into LDS (M = 1, 16-bit modes):
+    //   PRO_RMSNORM  x <- rd((x * r) * w),  w = pro_b [K] or ones, r from the whole row and pro_eps
+    //   PRO_SWIGLU   x <- rd(rd(silu(x)) * u),  u = pro_b [K]
+    int pro_op;
+    const void* pro_b;
+    float pro_eps;
 };
+enum { PRO_NONE = 0, PRO_RMSNORM = 1, PRO_SWIGLU = 2 };
 
 enum { LD_BYTE = 0, LD_Q1 = 1, LD_Q2 = 2, LD_V4 = 4, LD_V8 = 8, LD_V16 = 16 };
 constexpr int XC_MAX = 4;  // XLDS: 16-byte chunks of the x slice per lane
@@ -141,7 +148,10 @@ __device__ __forceinline__ uint32_t quad_transpose(uint32_t d, uint32_t sel_q) {
     return perm(t23, t01, 0x05040100u);
 }
 
-template <int MODE, int LD, int WAVES, int PF, bool XLDS>
+// PRO: activation prologue compiled in (PRO_NONE for all but the M = 1 variants that are launched
+// with one: a run-time switch, even a uniform one, puts branches and waits around the loads of the
+// plain kernel).
+template <int MODE, int LD, int WAVES, int PF, bool XLDS, int PRO = 0>
 __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
     constexpr bool QUAD = (LD == LD_Q1 || LD == LD_Q2);
     constexpr bool BYTE = (LD == LD_BYTE);
@@ -211,7 +221,7 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
     // XLDS (M == 1): the wave's K-slice of x, [s_begin*64, (s_begin+spw)*64), as 16-byte
     // chunks, chunk c = lane + 64u; zero beyond K
     uint8_t* xs = (uint8_t*)(red + WAVES * p.M * TILE_N) + (size_t)wave * (XC_MAX * 64 * 16);
-    uint4 xr[XLDS ? XC_MAX : 1];
+    uint4 xr[XLDS ? XC_MAX : 1], xb[(XLDS && PRO != 0) ? XC_MAX : 1];
     const int nchunks = spw * 64 * ES / 16;
     if constexpr (XLDS) {
         constexpr int EPC = 16 / ES;
@@ -220,7 +230,37 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
             if (u * 64 < nchunks) {  // uniform
                 const int k = s_begin * 64 + (lane + 64 * u) * EPC;
                 xr[u] = *(const uint4*)((const uint8_t*)p.X + (uint32_t)min(k, (int)p.K - EPC) * ES);
+                if constexpr (PRO != 0) {  // second operand; RMSNorm without a weight reads X again (unused)
+                    const uint8_t* bsrc = p.pro_b ? (const uint8_t*)p.pro_b : (const uint8_t*)p.X;
+                    xb[u] = *(const uint4*)(bsrc + (uint32_t)min(k, (int)p.K - EPC) * ES);
+                }
             }
+        }
+    }
+    // RMSNorm prologue: the row's sum of squares, by the whole workgroup (the row is a few KiB and hot
+    // in cache), accumulated in fp64 so that its fp32 value does not depend on the summation order
+    float rstd = 1.0f;
+    if constexpr (XLDS && MODE != MODE_I8 && PRO == PRO_RMSNORM) {
+        {
+            double ss = 0.0;
+            for (int k = (int)threadIdx.x * 8; k < (int)p.K; k += WAVES * 64 * 8) {
+                const uint4 v = *(const uint4*)((const uint16_t*)p.X + k);  // K % 8 == 0, aligned (XLDS)
+                const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const uint16_t h = (uint16_t)(d[e >> 1] >> (16 * (e & 1)));
+                    const double x = (double)(MODE == MODE_F16 ? f16_bits_to_f32(h) : bf16_bits_to_f32(h));
+                    ss += x * x;
+                }
+            }
+            ss = wave_sum_f64(ss);
+            double* part = (double*)red;  // the reduction buffer is free until the main loop is over
+            if (lane == 0) part[wave] = ss;
+            __syncthreads();
+            ss = 0.0;
+            for (int w = 0; w < WAVES; w++) ss += part[w];
+            __syncthreads();
+            rstd = rms_rstd(ss, (int)p.K, p.pro_eps);
         }
     }
 
@@ -279,7 +319,32 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
                         const int k = s_begin * 64 + (lane + 64 * u) * EPC;
                         // parked in the order the MFMA wants (each 16-byte chunk is one operand
                         // fragment), so that the steps below read their A operand ready-made
-                        const uint4 v = zero_unless(xr[u], k < (int)p.K);
+                        uint4 v = zero_unless(xr[u], k < (int)p.K);
+                        if constexpr (MODE != MODE_I8 && PRO != 0) {
+                            {
+                                constexpr int DT = (MODE == MODE_F16) ? BT_F16 : BT_BF16;
+                                const uint32_t a[4] = {v.x, v.y, v.z, v.w};
+                                const uint32_t bq[4] = {xb[u].x, xb[u].y, xb[u].z, xb[u].w};
+                                uint32_t r[4];
+#pragma unroll
+                                for (int d = 0; d < 4; d++) {
+                                    uint32_t out = 0;
+#pragma unroll
+                                    for (int e = 0; e < 2; e++) {
+                                        const uint16_t ha = (uint16_t)(a[d] >> (16 * e)), hb = (uint16_t)(bq[d] >> (16 * e));
+                                        const float fa = (DT == BT_F16) ? f16_bits_to_f32(ha) : bf16_bits_to_f32(ha);
+                                        const float fb = (DT == BT_F16) ? f16_bits_to_f32(hb) : bf16_bits_to_f32(hb);
+                                        float y;
+                                        if constexpr (PRO == PRO_SWIGLU) y = swiglu_value(fa, fb, DT);
+                                        else y = rmsnorm_value(fa, rstd, p.pro_b ? fb : 1.0f, DT);
+                                        const uint32_t hy = (DT == BT_F16) ? f32_to_f16_bits(y) : f32_to_bf16_bits(y);
+                                        out |= hy << (16 * e);
+                                    }
+                                    r[d] = out;
+                                }
+                                v = zero_unless(make_uint4(r[0], r[1], r[2], r[3]), k < (int)p.K);
+                            }
+                        }
                         uint4 o;
                         if constexpr (MODE == MODE_I8) {
                             uint32_t t4[4] = {v.x, v.y, v.z, v.w};
@@ -466,6 +531,16 @@ static void launch_stream_k(const StreamParams& p, bool xlds, dim3 grid, size_t 
     constexpr int PF = (LD == 16) ? 2 : (LD == 8) ? 4 : (LD == 4 && MODE != MODE_I8) ? 4 : 8;
     if constexpr (LD <= 4) {  // decode-shape tiles: the M = 1 variant with x staged in LDS
         if (xlds) {
+            if constexpr (MODE != MODE_I8) {
+                if (p.pro_op == PRO_RMSNORM) {
+                    hipLaunchKernelGGL((stream_kernel<MODE, LD, WAVES, PF, true, PRO_RMSNORM>), grid, dim3(WAVES * 64), lds, st, p);
+                    return;
+                }
+                if (p.pro_op == PRO_SWIGLU) {
+                    hipLaunchKernelGGL((stream_kernel<MODE, LD, WAVES, PF, true, PRO_SWIGLU>), grid, dim3(WAVES * 64), lds, st, p);
+                    return;
+                }
+            }
             hipLaunchKernelGGL((stream_kernel<MODE, LD, WAVES, PF, true>), grid, dim3(WAVES * 64), lds, st, p);
             return;
         }
@@ -484,6 +559,25 @@ static void launch_stream_w(const StreamParams& p, int waves, bool xlds, dim3 gr
     launch_stream_k<MODE, LD, 4>(p, xlds, grid, lds, st);
 }
 
+// x slice in LDS (the M = 1 variant): one row, aligned, at most XC_MAX 16-byte chunks per lane and
+// wave, and within the default 64 KiB of dynamic LDS
+static bool xlds_ok(int es, int M, bool x_vec_ok, const StreamPlan& pl, int64_t K) {
+    const int64_t tile_n = ld_columns(pl.ld);
+    const int64_t spw = ceil_div(ceil_div(K, 64), pl.waves);
+    const size_t red_bytes = (size_t)pl.waves * M * tile_n * 4;
+    const size_t xs_bytes = (size_t)pl.waves * XC_MAX * 64 * 16;
+    return M == 1 && x_vec_ok && pl.ld <= 4 && spw * 64 * es <= XC_MAX * 64 * 16 && K >= 16 / es &&
+           red_bytes + xs_bytes <= 64 * 1024 && !getenv("BITTORCH_STREAM_NOXLDS");
+}
+
+// Can the streaming kernel apply an RMSNorm / SwiGLU prologue to this call's activation row itself?
+// (one 16-bit row that takes the LDS-staged variant; BITTORCH_NO_PROLOGUE=1 says no, for A/B runs)
+bool stream_prologue_fusable(int mode, int64_t B, int64_t N, int64_t K, const void* X, const void* pro_b) {
+    if (mode == MODE_I8 || B != 1 || getenv("BITTORCH_NO_PROLOGUE")) return false;
+    const bool vec = ((uintptr_t)X) % 16 == 0 && (!pro_b || ((uintptr_t)pro_b) % 16 == 0) && (K * 2) % 16 == 0;
+    return xlds_ok(2, 1, vec, stream_plan(mode, 1, N, ceil_div(K, 4)), K);
+}
+
 template <int MODE>
 static int launch_stream_mode(StreamParams p, const StreamPlan& pl, hipStream_t st) {
     const int64_t tile_n = ld_columns(pl.ld);
@@ -491,15 +585,15 @@ static int launch_stream_mode(StreamParams p, const StreamPlan& pl, hipStream_t 
     p.per_xcd = (int)ceil_div(p.tiles, 8);
     const dim3 grid((unsigned)(p.per_xcd * 8));
     const int waves = pl.waves;
-    // x slice in LDS: one row, aligned, at most XC_MAX 16-byte chunks per lane and wave, and
-    // within the default 64 KiB of dynamic LDS
     const int es = (MODE == MODE_I8) ? 1 : 2;
-    const int64_t spw = ceil_div(ceil_div(p.K, 64), waves);
     const size_t red_bytes = (size_t)waves * p.M * tile_n * 4;
     const size_t xs_bytes = (size_t)waves * XC_MAX * 64 * 16;
-    const bool xlds = p.M == 1 && p.x_vec_ok && pl.ld <= 4 && spw * 64 * es <= XC_MAX * 64 * 16 &&
-                      p.K >= 16 / es && red_bytes + xs_bytes <= 64 * 1024 && !getenv("BITTORCH_STREAM_NOXLDS");
+    const bool xlds = xlds_ok(es, p.M, p.x_vec_ok != 0, pl, p.K);
     const size_t lds = red_bytes + (xlds ? xs_bytes : 0);
+    if (p.pro_op != PRO_NONE && !xlds) {
+        set_error("stream_gemm: activation prologue on a shape the callers should have routed elsewhere");
+        return BT_ERR_INVALID;
+    }
     switch (pl.ld) {
         case 16: launch_stream_w<MODE, 16>(p, waves, xlds, grid, lds, st); break;
         case 8: launch_stream_w<MODE, 8>(p, waves, xlds, grid, lds, st); break;
@@ -516,9 +610,10 @@ static int launch_stream_mode(StreamParams p, const StreamPlan& pl, hipStream_t 
 // row whose products with the same weights are summed (fp32 activations split into three bf16
 // terms); the kernel walks 3K values of k and wraps its weight row index every K.
 // q_layout: MODE_I8 only (Q_OPERAND_ORDER needs K % 16 == 0 and 16-byte aligned rows)
+// pro_op / pro_b / pro_eps: activation prologue (PRO_*), only where stream_prologue_fusable() said yes
 int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, const uint8_t* W_T,
                   const Epilogue& epi, void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N,
-                  int64_t K, int planes, int q_layout, hipStream_t st) {
+                  int64_t K, int planes, int q_layout, int pro_op, const void* pro_b, float pro_eps, hipStream_t st) {
     const int64_t Kb = ceil_div(K, 4);
     const int64_t Kx = K * planes;
     const StreamPlan pl = stream_plan(mode, B, N, Kb);
@@ -536,6 +631,7 @@ int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, co
         p.wsteps = (int)ceil_div(Kb, 16);
         p.prehalved = planes == 3;
         p.x_operand_order = (mode == MODE_I8 && q_layout == Q_OPERAND_ORDER) ? 1 : 0;
+        p.pro_op = pro_op; p.pro_b = pro_b; p.pro_eps = pro_eps;
         p.M = (int)((B - m0 < 16) ? (B - m0) : 16);
         p.y_dtype = y_dtype;
         p.x_vec_ok = (((uintptr_t)p.X) % 16 == 0) && ((Kx * x_elem_size) % 16 == 0);

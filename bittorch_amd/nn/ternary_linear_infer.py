@@ -30,8 +30,20 @@ class TernaryLinearInference(nn.Module):
         self.register_buffer("bias", bias)
         self.requires_grad_(False)
 
-    def forward(self, x: Tensor, residual: Optional[Tensor] = None) -> Tensor:
-        """``residual`` (not in the reference): added to the output, on the GPU inside the kernel."""
+    def forward(self, x: Tensor, residual: Optional[Tensor] = None, norm=None,
+                swiglu_up: Optional[Tensor] = None) -> Tensor:
+        """Additions to the reference's ``forward(x)``, all optional and GPU-fused: ``residual`` is added to
+        the output inside the kernel; ``norm=(weight or None, eps)`` applies RMSNorm to ``x`` first;
+        ``swiglu_up=u`` makes the input ``silu(x) * u`` (for a single decode token both run inside the
+        GEMV kernel itself)."""
+        if x.is_cuda and (norm is not None or swiglu_up is not None):
+            from .. import _C
+            return _C.ternary_linear_packed_forward_fused(x, self.weight_packed, self.scale, self.bias,
+                                                          self.in_features, residual, norm, swiglu_up)
+        if norm is not None:
+            x = F.rms_norm(x, (x.shape[-1],), norm[0], norm[1])
+        if swiglu_up is not None:
+            x = F.silu(x) * swiglu_up
         if x.is_cuda:
             from ..ops.ternary_linear_packed import ternary_linear_packed_forward
             return ternary_linear_packed_forward(x, self.weight_packed, self.scale,

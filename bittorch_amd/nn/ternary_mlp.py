@@ -41,10 +41,10 @@ class TernarySwiGLU(nn.Module):
             self.gate_up = None
             self.gate, self.up = gate, up
 
-    def _gate_up(self, h: Tensor):
+    def _gate_up(self, h: Tensor, norm=None):
         if self.gate_up is None:
-            return self.gate(h), self.up(h)
-        gu = self.gate_up(h)
+            return self.gate(h, None, norm), self.up(h, None, norm)
+        gu = self.gate_up(h, None, norm)
         return gu[..., :self.ffn], gu[..., self.ffn:]
 
     def _gate_up_int8(self, q: Tensor, s: Tensor, dtype, oo: bool):
@@ -65,8 +65,10 @@ class TernarySwiGLU(nn.Module):
             g, u = self._gate_up(h)
             return self.down(F.silu(g) * u, residual)
         if self.compute == "float":
-            h = x if eps is None else fused.rmsnorm(x, norm_weight, eps)
-            return self.down(fused.swiglu(*self._gate_up(h)), residual)
+            # norm and SwiGLU ride on the projections that consume them (for one decode token they run
+            # inside the GEMV kernels; otherwise as one fused kernel each ahead of the GEMM)
+            g, u = self._gate_up(x, None if eps is None else (norm_weight, eps))
+            return self.down(g, residual, None, u)
         # the int8 activations stay inside this call: hand them over in the matrix cores' own order
         oo1, oo2 = x.shape[-1] % 16 == 0, self.ffn % 16 == 0
         if eps is None:

@@ -189,6 +189,27 @@ int bt_rmsnorm(const void* X, int64_t ld_x, const void* weight, float eps, int d
                int64_t K, void* Y, int8_t* Q, float* s_x, int q_layout, void* stream);
 
 /*
+ * Packed forward with an activation prologue (no counterpart in the reference's Python/CUDA code;
+ * pre-norm block and SwiGLU MLP of its JS runtime, TernaryTransformer.ts:489-521, :366-423):
+ *   Y = linear( pro(X) ) [+ residual],   pro = BT_PRO_RMSNORM: rmsnorm(X; weight = pro_b or ones, eps)
+ *                                        pro = BT_PRO_SWIGLU:  silu(X) * pro_b   (X = gate, pro_b = up)
+ * with exactly the values bt_rmsnorm / bt_swiglu would store in x_dtype.  For a single 16-bit row
+ * (one decode token) the prologue runs inside the GEMV kernel, on the row's way into LDS, and saves a
+ * launch; every other shape runs the prologue kernel into the workspace and then the plain forward.
+ *   X [B,K] with row stride ld_x, pro_b [K] (RMSNorm, may be NULL) or [B,K] with row stride ld_b (SwiGLU).
+ *   workspace: at least bt_packed_forward_fused_workspace_bytes(B,N,K,x_dtype) bytes.
+ */
+enum { BT_PRO_NONE = 0, BT_PRO_RMSNORM = 1, BT_PRO_SWIGLU = 2 };
+size_t bt_packed_forward_fused_workspace_bytes(int64_t B, int64_t N, int64_t K, int x_dtype);
+int bt_ternary_linear_packed_forward_fused(const void* X, int64_t ld_x, int x_dtype, int pro_op,
+                                           const void* pro_b, int64_t ld_b, float eps,
+                                           const uint8_t* W_T, const void* scale, int scale_dtype,
+                                           int64_t scale_len, const void* bias, int bias_dtype,
+                                           const void* residual, void* Y, int64_t B, int64_t N,
+                                           int64_t K, void* workspace, size_t workspace_bytes,
+                                           void* stream);
+
+/*
  * Matrix-core forward from float activations: bt_act_quant_i8 followed by
  * bt_ternary_gemm_i8.  Replaces bittorch._C.ternary_linear_tensor_core_forward
  * (bittorch_bindings.cpp:65-87, ternary_gemm_tensor_core.cu:663-727) for

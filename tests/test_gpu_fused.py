@@ -342,3 +342,57 @@ def test_operand_order_on_the_generic_row_kernels(monkeypatch):
     qn, _ = _C.rmsnorm(x, None, 1e-5, False, True)
     qo, _ = _C.rmsnorm(x, None, 1e-5, False, True, operand_order=True)
     assert torch.equal(qo.view(5, 4, 4, 4), qn.view(5, 4, 4, 4).transpose(2, 3))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("b,n,k", [(1, 4096, 4096), (1, 2560, 6912), (1, 1000, 520), (1, 260, 72), (3, 512, 256), (40, 520, 192)])
+def test_forward_with_prologue_equals_the_separate_kernels(dtype, b, n, k):
+    """RMSNorm / SwiGLU applied inside the packed forward (inside the GEMV kernel for one 16-bit row,
+    as a kernel of its own otherwise) give the bits of the unfused sequence."""
+    from bittorch_amd import _C
+    announce("prologue", dtype, b, n, k)
+    packed, scale, bias = _packed_case(n, k, seed=n + k)
+    x = (seeded_acts(b, k, seed=3, dtype=dtype, outliers=True) * 2).cuda()
+    u = seeded_acts(b, k, seed=4, dtype=dtype).cuda()
+    w = (1 + 0.1 * torch.randn(k, generator=torch.Generator().manual_seed(k))).to(dtype).cuda()
+    res = seeded_acts(b, n, seed=5, dtype=dtype).cuda()
+    for norm_w in (w, None):
+        ref = _C.ternary_linear_packed_forward(_C.rmsnorm(x, norm_w, 1e-5), packed, scale, bias, k, res)
+        got = _C.ternary_linear_packed_forward_fused(x, packed, scale, bias, k, res, norm=(norm_w, 1e-5))
+        assert torch.equal(got, ref)
+    ref = _C.ternary_linear_packed_forward(_C.swiglu(x, u), packed, scale, bias, k)
+    got = _C.ternary_linear_packed_forward_fused(x, packed, scale, bias, k, swiglu_up=u)
+    assert torch.equal(got, ref)
+
+
+def test_prologue_on_halves_of_a_wide_row_and_argument_errors():
+    from bittorch_amd import _C
+    packed, scale, bias = _packed_case(512, 1024, seed=1)
+    gu = seeded_acts(1, 2048, seed=2, dtype=torch.bfloat16).cuda()
+    g, u = gu[:, :1024], gu[:, 1024:]
+    assert torch.equal(_C.ternary_linear_packed_forward_fused(g, packed, scale, None, 1024, swiglu_up=u),
+                       _C.ternary_linear_packed_forward(_C.swiglu(g, u), packed, scale, None, 1024))
+    with pytest.raises(RuntimeError, match="exactly one of norm and swiglu_up"):
+        _C.ternary_linear_packed_forward_fused(g, packed, scale, None, 1024)
+    with pytest.raises(RuntimeError, match="gate and up must match"):
+        _C.ternary_linear_packed_forward_fused(g, packed, scale, None, 1024, swiglu_up=u[:, :512])
+
+
+def test_swiglu_module_decode_token_equals_batched_rows():
+    """One token through TernarySwiGLU (prologues inside the GEMV kernels) equals the same row taken
+    from a batch (prologues as separate kernels, tiled GEMMs have another summation order: compare to
+    bf16 accuracy) and equals its own unfused composition exactly."""
+    import bittorch_amd as bt
+    from bittorch_amd import _C
+    d, ffn = 512, 1280
+    mk = lambda i, o, seed: bt.nn.create_ternary_linear_inference(
+        i, o, (torch.randn(o, i, generator=torch.Generator().manual_seed(seed)) * 0.02).cuda())
+    gate, up, down = mk(d, ffn, 1), mk(d, ffn, 2), mk(ffn, d, 3)
+    nw = (1 + 0.1 * torch.randn(d, generator=torch.Generator().manual_seed(4))).bfloat16().cuda()
+    x = seeded_acts(1, d, seed=8, dtype=torch.bfloat16).cuda()
+    for fuse in (False, True):
+        mlp = bt.nn.TernarySwiGLU(gate, up, down, fuse_gate_up=fuse)
+        got = mlp(x, nw, 1e-5, residual=x)
+        h = _C.rmsnorm(x, nw, 1e-5)
+        ref = down(_C.swiglu(gate(h), up(h))) + x
+        assert torch.equal(got, ref)
