@@ -249,6 +249,110 @@ def ternary_linear_packed_forward_fused(X: Tensor, W_T: Tensor, scale: Tensor, b
     return y.reshape(*X.shape[:-1], N)
 
 
+def retile_weights(W_T: Tensor, in_features: int) -> Tensor:
+    """Decode-tiled copy of ``W_T [ceil(K/4), N]`` (flat uint8 tensor): per 16-column tile and 16-row step
+    the 64 dwords a wave of the decode kernel loads, contiguous.  Built once; :func:`untile_weights` inverts it."""
+    _check(W_T.dim() == 2 and W_T.dtype == torch.uint8, "W_T must be 2D uint8 [K_bytes, N]")
+    _check(W_T.shape[0] == (in_features + 3) // 4, "K_bytes doesn't match ceil(K/4)")
+    _check(_all_cuda(W_T), "All tensors must be CUDA")
+    W_T = W_T.contiguous()
+    N = W_T.shape[1]
+    with torch.cuda.device(W_T.device):
+        out = torch.empty((_L.bt_tiled_weights_bytes(N, in_features),), dtype=torch.uint8, device=W_T.device)
+        _status(_L.bt_retile_weights(W_T.data_ptr(), N, in_features, out.data_ptr(), _stream(W_T)))
+    return out
+
+
+def _tiled_checks(W_tiled: Tensor, N: int, K: int):
+    _check(W_tiled.dtype == torch.uint8 and W_tiled.dim() == 1 and W_tiled.is_contiguous(),
+           "W_tiled must be the flat uint8 tensor retile_weights returned")
+    _check(N > 0 and K > 0 and W_tiled.numel() == _L.bt_tiled_weights_bytes(N, K),
+           "W_tiled size doesn't match out_features x in_features")
+
+
+def untile_weights(W_tiled: Tensor, out_features: int, in_features: int) -> Tensor:
+    """``W_T [ceil(K/4), N]`` back from its decode-tiled copy (exact inverse of :func:`retile_weights`)."""
+    _tiled_checks(W_tiled, out_features, in_features)
+    _check(_all_cuda(W_tiled), "All tensors must be CUDA")
+    with torch.cuda.device(W_tiled.device):
+        out = torch.empty(((in_features + 3) // 4, out_features), dtype=torch.uint8, device=W_tiled.device)
+        _status(_L.bt_untile_weights(W_tiled.data_ptr(), out_features, in_features, out.data_ptr(), _stream(W_tiled)))
+    return out
+
+
+def ternary_linear_tiled_forward(X: Tensor, W_tiled: Tensor, scale: Tensor, bias: Optional[Tensor] = None,
+                                 in_features: int = -1, out_features: int = -1, residual: Optional[Tensor] = None,
+                                 norm: Optional[Tuple[Optional[Tensor], float]] = None,
+                                 swiglu_up: Optional[Tensor] = None) -> Tensor:
+    """:func:`ternary_linear_packed_forward` / ``_fused`` on the decode-tiled copy of the weights (same
+    results bit for bit); the weights are streamed once per 16 rows of ``X``, so this is for decode shapes."""
+    _check(norm is None or swiglu_up is None, "at most one of norm and swiglu_up may be given")
+    _check(X.dim() >= 1 and X.numel() > 0, "X is empty")
+    K, N = X.shape[-1], out_features
+    _check(K == in_features, "input K doesn't match in_features")
+    _tiled_checks(W_tiled, N, K)
+    _check(scale.dim() == 1 and scale.shape[0] in (N, 1), "scale size doesn't match N")
+    _check(bias is None or (bias.dim() == 1 and bias.shape[0] == N), "bias shape mismatch")
+    _check(_all_cuda(X, W_tiled, scale, bias), "All tensors must be CUDA")
+    _check(X.dtype in _DT, "X must be float32, float16 or bfloat16")
+    x2 = _rows_2d(X, K) if (norm is not None or swiglu_up is not None) else X.contiguous().reshape(-1, K)
+    scale = _prep_vec(scale, x2)
+    bias = None if bias is None else _prep_vec(bias, x2)
+    B = x2.shape[0]
+    op, pb, ldb, eps = 0, None, 0, 0.0
+    if norm is not None:
+        w, eps = norm
+        if w is not None:
+            _check(w.dim() == 1 and w.shape[0] == K, "norm weight must be 1D [K]")
+            w = w.to(X.dtype).contiguous()
+        op, pb = 1, w
+    elif swiglu_up is not None:
+        _check(swiglu_up.shape == X.shape and swiglu_up.dtype == X.dtype, "gate and up must match in shape and dtype")
+        pb = _rows_2d(swiglu_up, K)
+        op, ldb = 2, pb.stride(0)
+    _check(_all_cuda(pb), "All tensors must be CUDA")
+    xdt = _dt(x2, "X")
+    y = torch.empty((B, N), dtype=X.dtype, device=X.device)
+    res = None if residual is None else _residual_2d(residual, X, X.shape[:-1], N)
+    with torch.cuda.device(X.device):
+        ws = _workspace(_L.bt_packed_forward_fused_workspace_bytes(B, N, K, xdt), X.device)
+        _status(_L.bt_ternary_linear_tiled_forward(
+            x2.data_ptr(), x2.stride(0), xdt, op, _ptr(pb), ldb, float(eps), W_tiled.data_ptr(), scale.data_ptr(),
+            _dt(scale, "scale"), scale.numel(), _ptr(bias), 0 if bias is None else _dt(bias, "bias"), _ptr(res),
+            y.data_ptr(), B, N, K, _ptr(ws), 0 if ws is None else ws.numel(), _stream(X)))
+    return y.reshape(*X.shape[:-1], N)
+
+
+def ternary_gemm_int8_tiled(Q: Tensor, s_x: Tensor, W_tiled: Tensor, scale: Tensor, bias: Optional[Tensor] = None,
+                            in_features: int = -1, out_features: int = -1,
+                            out_dtype: torch.dtype = torch.float32, return_acc: bool = False,
+                            residual: Optional[Tensor] = None, q_operand_order: bool = False):
+    """:func:`ternary_gemm_int8` on the decode-tiled copy of the weights (same results bit for bit)."""
+    _check(Q.dim() == 2 and Q.dtype == torch.int8 and Q.numel() > 0, "Q must be 2D int8")
+    K, N = Q.shape[-1], out_features
+    _check(K == in_features, "input K doesn't match in_features")
+    _tiled_checks(W_tiled, N, K)
+    _check(scale.dim() == 1 and scale.shape[0] in (N, 1), "scale size doesn't match N")
+    _check(bias is None or (bias.dim() == 1 and bias.shape[0] == N), "bias shape mismatch")
+    _check(s_x.dtype == torch.float32 and s_x.numel() == Q.shape[0], "s_x must be fp32 [B]")
+    _check(_all_cuda(Q, s_x, W_tiled, scale, bias), "All tensors must be CUDA")
+    _check(out_dtype in _DT, "out_dtype must be float32, float16 or bfloat16")
+    q = Q.contiguous()
+    s_x = s_x.contiguous()
+    scale = _prep_vec(scale, s_x)
+    bias = None if bias is None else _prep_vec(bias, s_x)
+    B = q.shape[0]
+    y = torch.empty((B, N), dtype=out_dtype, device=q.device)
+    acc = torch.empty((B, N), dtype=torch.int32, device=q.device) if return_acc else None
+    res = None if residual is None else _residual_2d(residual, y, (B,), N)
+    with torch.cuda.device(q.device):
+        _status(_L.bt_ternary_gemm_i8_tiled(
+            q.data_ptr(), 1 if q_operand_order else 0, s_x.data_ptr(), W_tiled.data_ptr(), scale.data_ptr(),
+            _dt(scale, "scale"), scale.numel(), _ptr(bias), 0 if bias is None else _dt(bias, "bias"), _ptr(res),
+            y.data_ptr(), _DT[out_dtype], _ptr(acc), B, N, K, _stream(q)))
+    return (y, acc) if return_acc else y
+
+
 def ternary_linear_tensor_core_forward(X: Tensor, W_T: Tensor, scale: Tensor,
                                        bias: Optional[Tensor] = None, in_features: int = -1,
                                        version: int = 1) -> Tensor:

@@ -214,6 +214,13 @@ constexpr uint32_t LUT_BF16_TWO = 0x00C04000u;  // sel 0..3 -> 0x00, 0x40, 0xC0,
 // GEMMs feed activations to the matrix cores without permuting them first.
 enum { Q_ROW_MAJOR = 0, Q_OPERAND_ORDER = 1 };
 
+// Layouts of the packed weights the streaming kernel reads.
+//   W_LAYOUT_ROW_MAJOR  the reference's W_T [Kb, N] (bittorch/quant/ternary_packed.py:174-206)
+//   W_LAYOUT_TILED      decode-tiled copy: dword ((t * S + s) * 64 + 16 g + j), S = ceil(Kb / 16), holds
+//                       the bytes W_T[16 s + 4 g + r, 16 t + j], r = 0..3 (low byte first), zero where the
+//                       row or the column lies outside the matrix
+enum { W_LAYOUT_ROW_MAJOR = 0, W_LAYOUT_TILED = 1 };
+
 // Two neighbouring lanes hold the 16 quantized bytes of one group (even lane: elements 0..7 as
 // lo, hi; odd lane: elements 8..15).  Returns this lane's 8 bytes of the transposed group.
 // Both lanes of a pair must call it (it exchanges registers between them).

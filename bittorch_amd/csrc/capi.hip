@@ -30,10 +30,14 @@ int check_launch(const char* what) {
 // kernels in the other translation units
 bool stream_supported(int64_t N, int64_t K, const void* W_T);
 size_t stream_workspace_bytes(int mode, int64_t M, int64_t N, int64_t Kb);
-int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, const uint8_t* W_T,
+bool stream_supported_tiled(int64_t N, int64_t K, const void* W);
+size_t tiled_bytes(int64_t N, int64_t K);
+int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, const uint8_t* W_T, int w_layout,
                   const Epilogue& epi, void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N,
-                  int64_t K, int planes, int q_layout, int pro_op, const void* pro_b, float pro_eps, hipStream_t st);
-bool stream_prologue_fusable(int mode, int64_t B, int64_t N, int64_t K, const void* X, const void* pro_b);
+                  int64_t K, int planes, int q_layout, int pro_op, const void* pro_b, float pro_eps,
+                  hipStream_t st);
+bool stream_prologue_fusable(int mode, int64_t B, int64_t N, int64_t K, const void* X, const void* pro_b, int w_layout);
+int launch_retile(const uint8_t* W_T, int64_t N, int64_t K, void* T, bool inverse, uint8_t* W_out, hipStream_t st);
 int launch_split_f32_planes(const void* X, int64_t B, int64_t K, void* P, hipStream_t st);
 int launch_packed_generic(const void* X, int x_dtype, const uint8_t* W_T, const Epilogue& epi, void* Y,
                           int64_t B, int64_t N, int64_t K, hipStream_t st);
@@ -161,8 +165,8 @@ static int set_residual(const char* who, const void* residual, Epilogue* e) {
     return BT_OK;
 }
 
-static int packed_forward_impl(const char* who, const void* X, int x_dtype, const uint8_t* W_T, const void* scale,
-                               int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
+static int packed_forward_impl(const char* who, const void* X, int x_dtype, const uint8_t* W_T, int w_layout,
+                               const void* scale, int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
                                const void* residual, void* Y, int64_t B, int64_t N, int64_t K, void* workspace,
                                size_t workspace_bytes, void* stream) {
     int rc = check_shape(who, X, W_T, Y, x_dtype, B, N, K);
@@ -173,12 +177,34 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
     rc = set_residual(who, residual, &epi);
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
+    if (w_layout == W_LAYOUT_TILED) {
+        // the decode-tiled copy is read by the streaming kernel only, once per 16 rows
+        if (!stream_supported_tiled(N, K, W_T) || !fast_path_ok(Y, N, 3 * K) || 3 * K >= (1ll << 26)) {
+            set_error("%s: tiled weights must be 256-byte aligned and below 4 GiB, Y 16-byte aligned", who);
+            return BT_ERR_INVALID;
+        }
+        if (x_dtype != BT_F32) {
+            const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
+            return launch_stream(mode, X, 2, nullptr, W_T, W_LAYOUT_TILED, epi, Y, x_dtype, nullptr, B, N, K, 1,
+                                 Q_ROW_MAJOR, 0, nullptr, 0.0f, st);
+        }
+        if (K % 64 != 0 || ((uintptr_t)X) % 16 != 0 || !workspace || workspace_bytes < f32_planes_bytes(B, K) ||
+            ((uintptr_t)workspace) % 256 != 0) {
+            set_error("%s: fp32 activations on tiled weights need K %% 64 == 0, X 16-byte aligned and a workspace of "
+                      "%zu bytes (256-byte aligned)", who, f32_planes_bytes(B, K));
+            return BT_ERR_INVALID;
+        }
+        rc = launch_split_f32_planes(X, B, K, workspace, st);
+        if (rc) return rc;
+        return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, W_LAYOUT_TILED, epi, Y, BT_F32, nullptr, B, N, K, 3,
+                             Q_ROW_MAJOR, 0, nullptr, 0.0f, st);
+    }
     if (packed_uses_stream(x_dtype, W_T, Y, N, K)) {
         const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
         // tall batches go to the tiled matrix-core kernel, decode shapes stream the weights
         if (B > kStreamMaxRows && gemm_f16_supported(N, K, X, W_T, Y))
             return launch_gemm_f16(mode, X, W_T, epi, Y, x_dtype, B, N, K, 1, st);
-        return launch_stream(mode, X, 2, nullptr, W_T, epi, Y, x_dtype, nullptr, B, N, K, 1, Q_ROW_MAJOR, 0, nullptr, 0.0f, st);
+        return launch_stream(mode, X, 2, nullptr, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, x_dtype, nullptr, B, N, K, 1, Q_ROW_MAJOR, 0, nullptr, 0.0f, st);
     }
     if (x_dtype == BT_F32 && packed_uses_f32_planes(X, W_T, Y, N, K) && workspace &&
         workspace_bytes >= f32_planes_bytes(B, K) && ((uintptr_t)workspace) % 256 == 0) {
@@ -187,7 +213,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         if (rc) return rc;
         if (B > kStreamMaxRows && gemm_f16_supported(N, 3 * K, workspace, W_T, Y))
             return launch_gemm_f16(MODE_BF16, workspace, W_T, epi, Y, BT_F32, B, N, K, 3, st);
-        return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, epi, Y, BT_F32, nullptr, B, N, K, 3, Q_ROW_MAJOR, 0, nullptr, 0.0f, st);
+        return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, BT_F32, nullptr, B, N, K, 3, Q_ROW_MAJOR, 0, nullptr, 0.0f, st);
     }
     return launch_packed_generic(X, x_dtype, W_T, epi, Y, B, N, K, st);
 }
@@ -197,7 +223,7 @@ extern "C" int bt_ternary_linear_packed_forward(const void* X, int x_dtype, cons
                                                 const void* bias, int bias_dtype, void* Y, int64_t B,
                                                 int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
                                                 void* stream) {
-    return packed_forward_impl("bt_ternary_linear_packed_forward", X, x_dtype, W_T, scale, scale_dtype, scale_len, bias,
+    return packed_forward_impl("bt_ternary_linear_packed_forward", X, x_dtype, W_T, W_LAYOUT_ROW_MAJOR, scale, scale_dtype, scale_len, bias,
                                bias_dtype, nullptr, Y, B, N, K, workspace, workspace_bytes, stream);
 }
 
@@ -206,7 +232,7 @@ extern "C" int bt_ternary_linear_packed_forward_res(const void* X, int x_dtype, 
                                                     const void* bias, int bias_dtype, const void* residual,
                                                     void* Y, int64_t B, int64_t N, int64_t K, void* workspace,
                                                     size_t workspace_bytes, void* stream) {
-    return packed_forward_impl("bt_ternary_linear_packed_forward_res", X, x_dtype, W_T, scale, scale_dtype, scale_len,
+    return packed_forward_impl("bt_ternary_linear_packed_forward_res", X, x_dtype, W_T, W_LAYOUT_ROW_MAJOR, scale, scale_dtype, scale_len,
                                bias, bias_dtype, residual, Y, B, N, K, workspace, workspace_bytes, stream);
 }
 
@@ -251,7 +277,8 @@ extern "C" size_t bt_gemm_i8_workspace_bytes(int64_t B, int64_t N, int64_t K) {
     return stream_workspace_bytes(MODE_I8, B, N, ceil_div(K, 4));
 }
 
-static int gemm_i8_impl(const char* who, const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_T, const void* scale,
+static int gemm_i8_impl(const char* who, const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_T, int w_layout,
+                        const void* scale,
                         int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype, const void* residual,
                         void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N, int64_t K, void* stream) {
     int rc = check_shape(who, Q, W_T, Y, y_dtype, B, N, K);
@@ -277,6 +304,14 @@ static int gemm_i8_impl(const char* who, const int8_t* Q, int q_layout, const fl
     rc = set_residual(who, residual, &epi);
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
+    if (w_layout == W_LAYOUT_TILED) {
+        if (!stream_supported_tiled(N, K, W_T)) {
+            set_error("%s: tiled weights must be 256-byte aligned and below 4 GiB", who);
+            return BT_ERR_INVALID;
+        }
+        return launch_stream(MODE_I8, Q, 1, s_x, W_T, w_layout, epi, Y, y_dtype, acc_out, B, N, K, 1, q_layout, 0, nullptr,
+                             0.0f, st);
+    }
     // decode-shape batches, and any batch whose N the tiled kernel's 4-column
     // vector accesses cannot take, stream the weights once per 16 rows
     if (B <= kStreamMaxRows || !gemm_i8_supported(N, K, Q, W_T)) {
@@ -285,7 +320,7 @@ static int gemm_i8_impl(const char* who, const int8_t* Q, int q_layout, const fl
                       (long long)ceil_div(K, 4), (long long)N);
             return BT_ERR_INVALID;
         }
-        return launch_stream(MODE_I8, Q, 1, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, 1, q_layout, 0, nullptr, 0.0f, st);
+        return launch_stream(MODE_I8, Q, 1, s_x, W_T, w_layout, epi, Y, y_dtype, acc_out, B, N, K, 1, q_layout, 0, nullptr, 0.0f, st);
     }
     return launch_gemm_i8(Q, q_layout, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, st);
 }
@@ -295,7 +330,7 @@ extern "C" int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8
                                   void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N, int64_t K,
                                   void* workspace, size_t workspace_bytes, void* stream) {
     (void)workspace; (void)workspace_bytes;
-    return gemm_i8_impl("bt_ternary_gemm_i8", Q, Q_ROW_MAJOR, s_x, W_T, scale, scale_dtype, scale_len, bias, bias_dtype, nullptr, Y,
+    return gemm_i8_impl("bt_ternary_gemm_i8", Q, Q_ROW_MAJOR, s_x, W_T, W_LAYOUT_ROW_MAJOR, scale, scale_dtype, scale_len, bias, bias_dtype, nullptr, Y,
                         y_dtype, acc_out, B, N, K, stream);
 }
 
@@ -303,7 +338,7 @@ extern "C" int bt_ternary_gemm_i8_res(const int8_t* Q, int q_layout, const float
                                       int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
                                       const void* residual, void* Y, int y_dtype, int32_t* acc_out, int64_t B,
                                       int64_t N, int64_t K, void* stream) {
-    return gemm_i8_impl("bt_ternary_gemm_i8_res", Q, q_layout, s_x, W_T, scale, scale_dtype, scale_len, bias, bias_dtype, residual,
+    return gemm_i8_impl("bt_ternary_gemm_i8_res", Q, q_layout, s_x, W_T, W_LAYOUT_ROW_MAJOR, scale, scale_dtype, scale_len, bias, bias_dtype, residual,
                         Y, y_dtype, acc_out, B, N, K, stream);
 }
 
@@ -338,8 +373,8 @@ extern "C" int bt_ternary_linear_tensor_core_forward(const void* X, int x_dtype,
     rc = launch_act_quant(X, x_dtype, B, K, Q, s_x, q_layout, (hipStream_t)stream);
     if (rc) return rc;
     (void)gemm_bytes;
-    return gemm_i8_impl(who, Q, q_layout, s_x, W_T, scale, scale_dtype, scale_len, bias, bias_dtype, nullptr, Y, x_dtype,
-                        nullptr, B, N, K, stream);
+    return gemm_i8_impl(who, Q, q_layout, s_x, W_T, W_LAYOUT_ROW_MAJOR, scale, scale_dtype, scale_len, bias, bias_dtype, nullptr,
+                        Y, x_dtype, nullptr, B, N, K, stream);
 }
 
 // ---- fused producers of the GEMM activations (row_ops.hip) ----------------------------------
@@ -393,14 +428,11 @@ extern "C" size_t bt_packed_forward_fused_workspace_bytes(int64_t B, int64_t N, 
     return align256((size_t)B * K * dtype_size(x_dtype)) + bt_packed_forward_workspace_bytes(B, N, K, x_dtype);
 }
 
-extern "C" int bt_ternary_linear_packed_forward_fused(const void* X, int64_t ld_x, int x_dtype, int pro_op,
-                                                      const void* pro_b, int64_t ld_b, float eps,
-                                                      const uint8_t* W_T, const void* scale, int scale_dtype,
-                                                      int64_t scale_len, const void* bias, int bias_dtype,
-                                                      const void* residual, void* Y, int64_t B, int64_t N,
-                                                      int64_t K, void* workspace, size_t workspace_bytes,
-                                                      void* stream) {
-    const char* who = "bt_ternary_linear_packed_forward_fused";
+static int fused_forward_impl(const char* who, const void* X, int64_t ld_x, int x_dtype, int pro_op, const void* pro_b,
+                              int64_t ld_b, float eps, const uint8_t* W_T, int w_layout, const void* scale,
+                              int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
+                              const void* residual, void* Y, int64_t B, int64_t N, int64_t K, void* workspace,
+                              size_t workspace_bytes, void* stream) {
     int rc = check_shape(who, X, W_T, Y, x_dtype, B, N, K);
     if (rc) return rc;
     if (pro_op != 1 && pro_op != 2) {
@@ -413,16 +445,18 @@ extern "C" int bt_ternary_linear_packed_forward_fused(const void* X, int64_t ld_
     }
     hipStream_t st = (hipStream_t)stream;
     // one 16-bit row on the streaming kernel: the prologue runs inside the GEMV, on the row's way into LDS
-    if (x_dtype != BT_F32 && B == 1 && packed_uses_stream(x_dtype, W_T, Y, N, K)) {
+    const bool streams = (w_layout == W_LAYOUT_TILED) ? (stream_supported_tiled(N, K, W_T) && fast_path_ok(Y, N, K))
+                                                      : packed_uses_stream(x_dtype, W_T, Y, N, K);
+    if (x_dtype != BT_F32 && B == 1 && streams) {
         const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
-        if (stream_prologue_fusable(mode, B, N, K, X, pro_b)) {
+        if (stream_prologue_fusable(mode, B, N, K, X, pro_b, w_layout)) {
             Epilogue epi;
             rc = make_epilogue(who, scale, scale_dtype, scale_len, bias, bias_dtype, N, &epi);
             if (rc) return rc;
             rc = set_residual(who, residual, &epi);
             if (rc) return rc;
-            return launch_stream(mode, X, 2, nullptr, W_T, epi, Y, x_dtype, nullptr, B, N, K, 1, Q_ROW_MAJOR, pro_op, pro_b,
-                                 eps, st);
+            return launch_stream(mode, X, 2, nullptr, W_T, w_layout, epi, Y, x_dtype, nullptr, B, N, K, 1, Q_ROW_MAJOR, pro_op,
+                                 pro_b, eps, st);
         }
     }
     // otherwise: the prologue as its own kernel into the workspace, then the plain forward
@@ -435,6 +469,76 @@ extern "C" int bt_ternary_linear_packed_forward_fused(const void* X, int64_t ld_
     rc = launch_row_op(pro_op == 2 ? 0 : 1, x_dtype, X, ld_x, pro_b, ld_b, eps, B, K, workspace, nullptr, nullptr,
                        Q_ROW_MAJOR, st, who);
     if (rc) return rc;
-    return packed_forward_impl(who, workspace, x_dtype, W_T, scale, scale_dtype, scale_len, bias, bias_dtype, residual, Y,
-                               B, N, K, (uint8_t*)workspace + h_bytes, workspace_bytes - h_bytes, stream);
+    return packed_forward_impl(who, workspace, x_dtype, W_T, w_layout, scale, scale_dtype, scale_len, bias, bias_dtype,
+                               residual, Y, B, N, K, (uint8_t*)workspace + h_bytes, workspace_bytes - h_bytes, stream);
+}
+
+extern "C" int bt_ternary_linear_packed_forward_fused(const void* X, int64_t ld_x, int x_dtype, int pro_op,
+                                                      const void* pro_b, int64_t ld_b, float eps,
+                                                      const uint8_t* W_T, const void* scale, int scale_dtype,
+                                                      int64_t scale_len, const void* bias, int bias_dtype,
+                                                      const void* residual, void* Y, int64_t B, int64_t N,
+                                                      int64_t K, void* workspace, size_t workspace_bytes,
+                                                      void* stream) {
+    return fused_forward_impl("bt_ternary_linear_packed_forward_fused", X, ld_x, x_dtype, pro_op, pro_b, ld_b, eps, W_T,
+                              W_LAYOUT_ROW_MAJOR, scale, scale_dtype, scale_len, bias, bias_dtype, residual, Y, B, N, K,
+                              workspace, workspace_bytes, stream);
+}
+
+// ---- decode-tiled copy of the packed weights ---------------------------------------------------
+extern "C" size_t bt_tiled_weights_bytes(int64_t N, int64_t K) {
+    if (N <= 0 || K <= 0) return 0;
+    return tiled_bytes(N, K);
+}
+
+static int check_retile(const char* who, const void* a, const void* b, int64_t N, int64_t K, const void* tiled) {
+    if (!a || !b || N <= 0 || K <= 0) {
+        set_error("%s: null pointer or empty shape", who);
+        return BT_ERR_INVALID;
+    }
+    if (((uintptr_t)tiled) % 256 != 0 || tiled_bytes(N, K) >= (1ull << 32)) {
+        set_error("%s: the tiled copy must be 256-byte aligned and below 4 GiB", who);
+        return BT_ERR_INVALID;
+    }
+    return BT_OK;
+}
+
+extern "C" int bt_retile_weights(const uint8_t* W_T, int64_t N, int64_t K, uint8_t* W_tiled, void* stream) {
+    const int rc = check_retile("bt_retile_weights", W_T, W_tiled, N, K, W_tiled);
+    if (rc) return rc;
+    return launch_retile(W_T, N, K, W_tiled, false, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int bt_untile_weights(const uint8_t* W_tiled, int64_t N, int64_t K, uint8_t* W_T, void* stream) {
+    const int rc = check_retile("bt_untile_weights", W_tiled, W_T, N, K, W_tiled);
+    if (rc) return rc;
+    return launch_retile(nullptr, N, K, (void*)W_tiled, true, W_T, (hipStream_t)stream);
+}
+
+extern "C" int bt_ternary_linear_tiled_forward(const void* X, int64_t ld_x, int x_dtype, int pro_op,
+                                               const void* pro_b, int64_t ld_b, float eps, const uint8_t* W_tiled,
+                                               const void* scale, int scale_dtype, int64_t scale_len,
+                                               const void* bias, int bias_dtype, const void* residual, void* Y,
+                                               int64_t B, int64_t N, int64_t K, void* workspace,
+                                               size_t workspace_bytes, void* stream) {
+    const char* who = "bt_ternary_linear_tiled_forward";
+    if (pro_op != 0)
+        return fused_forward_impl(who, X, ld_x, x_dtype, pro_op, pro_b, ld_b, eps, W_tiled, W_LAYOUT_TILED, scale,
+                                  scale_dtype, scale_len, bias, bias_dtype, residual, Y, B, N, K, workspace,
+                                  workspace_bytes, stream);
+    if (ld_x != K) {
+        set_error("%s: without a prologue the activation rows must be contiguous (ld_x=%lld, K=%lld)", who,
+                  (long long)ld_x, (long long)K);
+        return BT_ERR_INVALID;
+    }
+    return packed_forward_impl(who, X, x_dtype, W_tiled, W_LAYOUT_TILED, scale, scale_dtype, scale_len, bias, bias_dtype,
+                               residual, Y, B, N, K, workspace, workspace_bytes, stream);
+}
+
+extern "C" int bt_ternary_gemm_i8_tiled(const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_tiled,
+                                        const void* scale, int scale_dtype, int64_t scale_len, const void* bias,
+                                        int bias_dtype, const void* residual, void* Y, int y_dtype, int32_t* acc_out,
+                                        int64_t B, int64_t N, int64_t K, void* stream) {
+    return gemm_i8_impl("bt_ternary_gemm_i8_tiled", Q, q_layout, s_x, W_tiled, W_LAYOUT_TILED, scale, scale_dtype,
+                        scale_len, bias, bias_dtype, residual, Y, y_dtype, acc_out, B, N, K, stream);
 }

@@ -23,6 +23,11 @@
 //               (rows 4g+q, the same four columns) and exchange bytes with DPP
 //               quad permutes - one load instruction per 16x16 block instead of four;
 //   LD_BYTE     N not a multiple of 4: one byte per lane and row.
+//   LD_T1/2/4   the decode-tiled copy of the weights (W_LAYOUT_TILED, see retile_kernel): the dword
+//               G of every lane and step is stored as such, 256 contiguous bytes per 16-column tile
+//               and step, so a wave's load covers two whole cache lines and needs no transpose
+//               (a 16-column tile of the row-major W_T touches 16 bytes of 16 different lines,
+//               and the seven other tiles sharing those lines sit on other compute units).
 // A wave issues the loads of PF steps before it computes any of them, which is
 // what keeps enough bytes in flight to cover the HBM latency.
 // A workgroup owns one column tile over the WHOLE of K: there is no split-K
@@ -54,6 +59,7 @@ struct StreamParams {
     int x_vec_ok;         // activation rows may be read with 16-byte loads
     int prehalved;        // MODE_BF16: the activations already carry the factor 1/2 of the +-2.0 weight decode
     int x_operand_order;  // MODE_I8: X is in the quantizer's operand order (16-byte groups transposed)
+    int tiles16;          // LD_T*: 16-column tiles of the decode-tiled weights
     // Prologue applied to the single activation row on its way into LDS (M = 1, 16-bit modes):
     //   PRO_RMSNORM  x <- rd((x * r) * w),  w = pro_b [K] or ones, r from the whole row and pro_eps
     //   PRO_SWIGLU   x <- rd(rd(silu(x)) * u),  u = pro_b [K]
@@ -63,7 +69,7 @@ struct StreamParams {
 };
 enum { PRO_NONE = 0, PRO_RMSNORM = 1, PRO_SWIGLU = 2 };
 
-enum { LD_BYTE = 0, LD_Q1 = 1, LD_Q2 = 2, LD_V4 = 4, LD_V8 = 8, LD_V16 = 16 };
+enum { LD_BYTE = 0, LD_Q1 = 1, LD_Q2 = 2, LD_V4 = 4, LD_V8 = 8, LD_V16 = 16, LD_T1 = 101, LD_T2 = 102, LD_T4 = 104 };
 constexpr int XC_MAX = 4;  // XLDS: 16-byte chunks of the x slice per lane
 
 template <int NB> struct RawVec;
@@ -155,11 +161,12 @@ template <int MODE, int LD, int WAVES, int PF, bool XLDS, int PRO = 0>
 __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
     constexpr bool QUAD = (LD == LD_Q1 || LD == LD_Q2);
     constexpr bool BYTE = (LD == LD_BYTE);
-    constexpr int NACC = BYTE ? 1 : LD;             // output columns per lane
+    constexpr bool TILED = (LD > 100);
+    constexpr int NACC = TILED ? LD - 100 : BYTE ? 1 : LD;  // output columns per lane
     constexpr int TILE_N = 16 * NACC;
-    constexpr int RAWN = BYTE ? 4 : LD;             // raw dwords per lane and step
-    constexpr int ND = (LD >= 4) ? LD / 4 : 1;      // LD_V*: dwords per lane and row
-    constexpr int NCO = QUAD ? LD : 1;              // column offsets per lane
+    constexpr int RAWN = TILED ? NACC : BYTE ? 4 : LD;      // raw dwords per lane and step
+    constexpr int ND = (!TILED && LD >= 4) ? LD / 4 : 1;    // LD_V*: dwords per lane and row
+    constexpr int NCO = QUAD ? LD : TILED ? NACC : 1;       // column (LD_T*: tile) offsets per lane
     constexpr int ES = (MODE == MODE_I8) ? 1 : 2;   // bytes per activation
     constexpr int XN = (MODE == MODE_I8) ? 1 : 2;   // 16-byte pieces of x per lane and step
     constexpr bool TWO = (NACC <= 2);               // second accumulator chain
@@ -190,7 +197,13 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
     const uint32_t N32 = (uint32_t)p.N;
     const uint32_t last_rowoff = (uint32_t)(p.Kb - 1) * N32;
     uint32_t coloff[NCO];
-    if constexpr (QUAD) {
+    if constexpr (TILED) {
+        // byte offset of this lane's dword in step 0 of each 16-column tile; a tile past the end is
+        // computed on the last tile's bytes and never stored
+#pragma unroll
+        for (int t = 0; t < NCO; t++)
+            coloff[t] = ((uint32_t)min(tile * NACC + t, p.tiles16 - 1) * (uint32_t)p.wsteps * 64u + (uint32_t)lane) * 4u;
+    } else if constexpr (QUAD) {
 #pragma unroll
         for (int cb = 0; cb < NCO; cb++) {
             const int64_t c = nb + 16 * cb + (j & ~3);
@@ -281,7 +294,11 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
             if (ws >= p.wsteps) ws -= p.wsteps;
             if (ws >= p.wsteps) ws -= p.wsteps;
             const uint32_t ro = lane_rowoff + (uint32_t)ws * step_rows;
-            if constexpr (BYTE) {
+            if constexpr (TILED) {
+                const uint32_t so = (uint32_t)min(ws, p.wsteps - 1) * 256u;
+#pragma unroll
+                for (int t = 0; t < NCO; t++) raw[f][t] = *(const uint32_t*)(p.W_T + (coloff[t] + so));
+            } else if constexpr (BYTE) {
 #pragma unroll
                 for (int r = 0; r < 4; r++)
                     raw[f][r] = (uint32_t)p.W_T[min(ro + (uint32_t)r * N32, last_rowoff) + coloff[0]];
@@ -374,7 +391,10 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
             }
             // G[t]: packed bytes of rows 4g..4g+3 of the column accumulator t serves
             uint32_t G[NACC];
-            if constexpr (BYTE) {
+            if constexpr (TILED) {
+#pragma unroll
+                for (int t = 0; t < NACC; t++) G[t] = raw[f][t];
+            } else if constexpr (BYTE) {
                 G[0] = raw[f][0] | (raw[f][1] << 8) | (raw[f][2] << 16) | (raw[f][3] << 24);
             } else if constexpr (QUAD) {
 #pragma unroll
@@ -463,8 +483,8 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
         const int row = idx / TILE_N;
         const int nl = idx % TILE_N;
         if (nb + nl >= p.N) continue;
-        // column nl of the tile sits in slot t*16 + j: LD_V*: nl = NACC*j + t; else nl = 16*t + j
-        const int slot = (LD >= 4) ? (nl % NACC) * 16 + nl / NACC : nl;
+        // column nl of the tile sits in slot t*16 + j: LD_V*: nl = NACC*j + t; else (LD_T* too) nl = 16*t + j
+        const int slot = (LD >= 4 && !TILED) ? (nl % NACC) * 16 + nl / NACC : nl;
         uint32_t bits = red[row * TILE_N + slot];
 #pragma unroll
         for (int w = 1; w < WAVES; w++) bits = add_bits<MODE>(bits, red[(w * M + row) * TILE_N + slot]);
@@ -488,21 +508,35 @@ struct StreamPlan {
 };
 
 // the kernel addresses W_T and X with 32-bit offsets from their base pointers
+// decode-tiled copy: whole 16-column tiles and 16-row steps, 256 bytes each
+size_t tiled_bytes(int64_t N, int64_t K) { return (size_t)ceil_div(N, 16) * (size_t)ceil_div(ceil_div(K, 4), 16) * 256; }
+
+bool stream_supported_tiled(int64_t N, int64_t K, const void* W) {
+    return ((uintptr_t)W) % 256 == 0 && N >= 1 && N < (1ll << 30) && K < (1ll << 26) && tiled_bytes(N, K) < (1ull << 32);
+}
+
 bool stream_supported(int64_t N, int64_t K, const void* W_T) {
     // (rows up to 16*16*16 past the end enter the offset arithmetic before they are clamped)
     return ((uintptr_t)W_T) % 16 == 0 && N >= 1 && (ceil_div(K, 4) + 8192) * N < (1ll << 32) && K < (1ll << 26);
 }
 
-static int ld_columns(int ld) { return ld == LD_BYTE ? 16 : 16 * ld; }
+static int ld_columns(int ld) { return ld == LD_BYTE ? 16 : ld > 100 ? 16 * (ld - 100) : 16 * ld; }
 
-StreamPlan stream_plan(int mode, int64_t M, int64_t N, int64_t Kb) {
+StreamPlan stream_plan(int mode, int64_t M, int64_t N, int64_t Kb, int w_layout) {
     StreamPlan pl;
     (void)Kb;
     // optional override for tuning runs: BITTORCH_STREAM_CFG="ld,waves"
     int o_ld = -1, o_waves = 0;
     if (const char* env = getenv("BITTORCH_STREAM_CFG")) sscanf(env, "%d,%d", &o_ld, &o_waves);
     int ld;
-    if (N % 4 != 0) {
+    if (w_layout == W_LAYOUT_TILED) {
+        // 16-column tiles, up to four per workgroup (a batch re-reads its activations once per workgroup)
+        const int min_tiles = (M > 4) ? 160 : 256;
+        int nacc = 4;
+        while (nacc > 1 && ceil_div(N, 16 * nacc) < min_tiles) nacc >>= 1;
+        if (o_ld == LD_T1 || o_ld == LD_T2 || o_ld == LD_T4) nacc = o_ld - 100;
+        ld = 100 + nacc;
+    } else if (N % 4 != 0) {
         ld = LD_BYTE;  // row starts are not dword aligned
     } else if ((o_ld == 16 || o_ld == 8 || o_ld == 4 || o_ld == 2 || o_ld == 1) && (o_ld < 4 || N % o_ld == 0)) {
         ld = o_ld;
@@ -517,7 +551,7 @@ StreamPlan stream_plan(int mode, int64_t M, int64_t N, int64_t Kb) {
         while (ld > 1 && ceil_div(N, ld_columns(ld)) < min_tiles) ld >>= 1;
     }
     pl.ld = ld;
-    const int max_waves = (ld == 16) ? 4 : (ld == 8 || ld == LD_BYTE) ? 8 : 16;  // LDS: WAVES*TILE_N <= 1024 words per row
+    const int max_waves = (ld == 16) ? 4 : (ld == 8 || ld == LD_BYTE) ? 8 : 16;   // LDS: WAVES*TILE_N <= 1024 words per row
     int waves = (o_waves == 4 || o_waves == 8 || o_waves == 16) ? o_waves : 8;
     if (waves > max_waves) waves = max_waves;
     pl.waves = waves;
@@ -528,8 +562,8 @@ size_t stream_workspace_bytes(int, int64_t, int64_t, int64_t) { return 0; }
 
 template <int MODE, int LD, int WAVES>
 static void launch_stream_k(const StreamParams& p, bool xlds, dim3 grid, size_t lds, hipStream_t st) {
-    constexpr int PF = (LD == 16) ? 2 : (LD == 8) ? 4 : (LD == 4 && MODE != MODE_I8) ? 4 : 8;
-    if constexpr (LD <= 4) {  // decode-shape tiles: the M = 1 variant with x staged in LDS
+    constexpr int PF = (LD == 16) ? 2 : (LD == 8) ? 4 : ((LD == 4 || LD == LD_T4) && MODE != MODE_I8) ? 4 : 8;
+    if constexpr (LD <= 4 || LD > 100) {  // decode-shape tiles: the M = 1 variant with x staged in LDS
         if (xlds) {
             if constexpr (MODE != MODE_I8) {
                 if (p.pro_op == PRO_RMSNORM) {
@@ -550,10 +584,10 @@ static void launch_stream_k(const StreamParams& p, bool xlds, dim3 grid, size_t 
 
 template <int MODE, int LD>
 static void launch_stream_w(const StreamParams& p, int waves, bool xlds, dim3 grid, size_t lds, hipStream_t st) {
-    if constexpr (LD <= 4) {
+    if constexpr (LD <= 4 || LD > 100) {
         if (waves == 16) { launch_stream_k<MODE, LD, 16>(p, xlds, grid, lds, st); return; }
     }
-    if constexpr (LD <= 8) {
+    if constexpr (LD <= 8 || LD > 100) {
         if (waves == 8) { launch_stream_k<MODE, LD, 8>(p, xlds, grid, lds, st); return; }
     }
     launch_stream_k<MODE, LD, 4>(p, xlds, grid, lds, st);
@@ -566,16 +600,16 @@ static bool xlds_ok(int es, int M, bool x_vec_ok, const StreamPlan& pl, int64_t 
     const int64_t spw = ceil_div(ceil_div(K, 64), pl.waves);
     const size_t red_bytes = (size_t)pl.waves * M * tile_n * 4;
     const size_t xs_bytes = (size_t)pl.waves * XC_MAX * 64 * 16;
-    return M == 1 && x_vec_ok && pl.ld <= 4 && spw * 64 * es <= XC_MAX * 64 * 16 && K >= 16 / es &&
+    return M == 1 && x_vec_ok && (pl.ld <= 4 || pl.ld > 100) && spw * 64 * es <= XC_MAX * 64 * 16 && K >= 16 / es &&
            red_bytes + xs_bytes <= 64 * 1024 && !getenv("BITTORCH_STREAM_NOXLDS");
 }
 
 // Can the streaming kernel apply an RMSNorm / SwiGLU prologue to this call's activation row itself?
 // (one 16-bit row that takes the LDS-staged variant; BITTORCH_NO_PROLOGUE=1 says no, for A/B runs)
-bool stream_prologue_fusable(int mode, int64_t B, int64_t N, int64_t K, const void* X, const void* pro_b) {
+bool stream_prologue_fusable(int mode, int64_t B, int64_t N, int64_t K, const void* X, const void* pro_b, int w_layout) {
     if (mode == MODE_I8 || B != 1 || getenv("BITTORCH_NO_PROLOGUE")) return false;
     const bool vec = ((uintptr_t)X) % 16 == 0 && (!pro_b || ((uintptr_t)pro_b) % 16 == 0) && (K * 2) % 16 == 0;
-    return xlds_ok(2, 1, vec, stream_plan(mode, 1, N, ceil_div(K, 4)), K);
+    return xlds_ok(2, 1, vec, stream_plan(mode, 1, N, ceil_div(K, 4), w_layout), K);
 }
 
 template <int MODE>
@@ -600,6 +634,9 @@ static int launch_stream_mode(StreamParams p, const StreamPlan& pl, hipStream_t 
         case 4: launch_stream_w<MODE, 4>(p, waves, xlds, grid, lds, st); break;
         case 2: launch_stream_w<MODE, 2>(p, waves, xlds, grid, lds, st); break;
         case 1: launch_stream_w<MODE, 1>(p, waves, xlds, grid, lds, st); break;
+        case LD_T1: launch_stream_w<MODE, LD_T1>(p, waves, xlds, grid, lds, st); break;
+        case LD_T2: launch_stream_w<MODE, LD_T2>(p, waves, xlds, grid, lds, st); break;
+        case LD_T4: launch_stream_w<MODE, LD_T4>(p, waves, xlds, grid, lds, st); break;
         default: launch_stream_w<MODE, 0>(p, waves, xlds, grid, lds, st); break;
     }
     return check_launch("stream_gemm");
@@ -609,14 +646,15 @@ static int launch_stream_mode(StreamParams p, const StreamPlan& pl, hipStream_t 
 // planes = 1: X is [B, K].  planes = 3 (K % 64 == 0): X is [B, 3K], three planes of K values per
 // row whose products with the same weights are summed (fp32 activations split into three bf16
 // terms); the kernel walks 3K values of k and wraps its weight row index every K.
+// w_layout: W_LAYOUT_ROW_MAJOR (the reference's W_T [Kb, N]) or W_LAYOUT_TILED (retile_kernel's copy)
 // q_layout: MODE_I8 only (Q_OPERAND_ORDER needs K % 16 == 0 and 16-byte aligned rows)
 // pro_op / pro_b / pro_eps: activation prologue (PRO_*), only where stream_prologue_fusable() said yes
-int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, const uint8_t* W_T,
+int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, const uint8_t* W_T, int w_layout,
                   const Epilogue& epi, void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N,
                   int64_t K, int planes, int q_layout, int pro_op, const void* pro_b, float pro_eps, hipStream_t st) {
     const int64_t Kb = ceil_div(K, 4);
     const int64_t Kx = K * planes;
-    const StreamPlan pl = stream_plan(mode, B, N, Kb);
+    const StreamPlan pl = stream_plan(mode, B, N, Kb, w_layout);
     const int y_size = dtype_size(y_dtype);
     for (int64_t m0 = 0; m0 < B; m0 += 16) {
         StreamParams p;
@@ -629,6 +667,7 @@ int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, co
         if (epi.residual) p.epi.residual = (const uint8_t*)epi.residual + m0 * N * y_size;
         p.N = N; p.K = Kx; p.Kb = Kb;
         p.wsteps = (int)ceil_div(Kb, 16);
+        p.tiles16 = (int)ceil_div(N, 16);
         p.prehalved = planes == 3;
         p.x_operand_order = (mode == MODE_I8 && q_layout == Q_OPERAND_ORDER) ? 1 : 0;
         p.pro_op = pro_op; p.pro_b = pro_b; p.pro_eps = pro_eps;

@@ -4,10 +4,17 @@ API mirror of ``bittorch/nn/ternary_linear_infer.py:22-193``.  Buffers:
 ``weight_packed`` uint8 ``[ceil(K/4), N]`` (transposed layout), ``scale`` ``[N]``,
 optional ``bias``; nothing is trainable.  GPU inputs go to the packed HIP
 kernels; CPU inputs unpack and use ``F.linear`` as the reference does.
+
+Decode-shape calls on the GPU (up to ``DECODE_ROWS`` rows) read a second, *decode-tiled* copy of
+the packed weights that the layer builds from ``weight_packed`` on first use (same size, not part
+of the ``state_dict``; same results bit for bit, 15-25 % less time per GEMV because every load of
+the kernel then covers whole cache lines).  ``decode_tiled=False`` or ``BITTORCH_DECODE_TILED=0``
+keeps the layer on ``weight_packed`` alone.
 """
 
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
@@ -19,9 +26,13 @@ from ..quant.ternary import ternary_quantize
 from ..quant.ternary_packed import pack_ternary_transposed, unpack_ternary_transposed
 
 
+# batches up to this many rows stream the weights (once per 16 rows) instead of running the tiled GEMM
+DECODE_ROWS = 32
+
+
 class TernaryLinearInference(nn.Module):
     def __init__(self, in_features: int, out_features: int, weight_packed: Tensor, scale: Tensor,
-                 bias: Optional[Tensor] = None):
+                 bias: Optional[Tensor] = None, decode_tiled: Optional[bool] = None):
         super().__init__()
         self.in_features = in_features
         self.out_features = out_features
@@ -29,6 +40,45 @@ class TernaryLinearInference(nn.Module):
         self.register_buffer("scale", scale)
         self.register_buffer("bias", bias)
         self.requires_grad_(False)
+        if decode_tiled is None:
+            decode_tiled = os.environ.get("BITTORCH_DECODE_TILED", "1") != "0"
+        self.decode_tiled = bool(decode_tiled)
+        self._tiled: Optional[Tensor] = None
+        self._tiled_key = None
+
+    # ---- decode-tiled copy of the weights ---------------------------------------------------
+    def tiled_weights(self) -> Tensor:
+        """The decode-tiled copy of ``weight_packed`` (GPU only), built on first use and rebuilt when
+        ``weight_packed`` has moved or been written since."""
+        wp = self.weight_packed
+        key = (wp.data_ptr(), wp._version, wp.device)
+        if self._tiled is None or self._tiled_key != key:
+            from .. import _C
+            self._tiled = _C.retile_weights(wp, self.in_features)
+            self._tiled_key = key
+        return self._tiled
+
+    def prepare_decode(self) -> "TernaryLinearInference":
+        """Build the decode-tiled copy now (e.g. before capturing decode steps into a HIP graph: a
+        capture never builds it, it falls back to ``weight_packed``)."""
+        if self.decode_tiled and self.weight_packed.is_cuda:
+            self.tiled_weights()
+        return self
+
+    def _tiled_for(self, x: Tensor, rows: int) -> Optional[Tensor]:
+        if not (self.decode_tiled and x.is_cuda and rows <= DECODE_ROWS):
+            return None
+        if os.environ.get("BITTORCH_KERNEL") == "generic":  # the shape-generic kernel reads weight_packed
+            return None
+        if x.dtype not in (torch.float16, torch.bfloat16, torch.float32, torch.int8):
+            return None
+        if x.dtype == torch.float32 and self.in_features % 64 != 0:
+            return None
+        wp = self.weight_packed
+        fresh = self._tiled is not None and self._tiled_key == (wp.data_ptr(), wp._version, wp.device)
+        if not fresh and torch.cuda.is_current_stream_capturing():
+            return None
+        return self.tiled_weights()
 
     def forward(self, x: Tensor, residual: Optional[Tensor] = None, norm=None,
                 swiglu_up: Optional[Tensor] = None) -> Tensor:
@@ -36,6 +86,12 @@ class TernaryLinearInference(nn.Module):
         the output inside the kernel; ``norm=(weight or None, eps)`` applies RMSNorm to ``x`` first;
         ``swiglu_up=u`` makes the input ``silu(x) * u`` (for a single decode token both run inside the
         GEMV kernel itself)."""
+        if x.is_cuda:
+            tiled = self._tiled_for(x, x.numel() // max(x.shape[-1], 1))
+            if tiled is not None:
+                from .. import _C
+                return _C.ternary_linear_tiled_forward(x, tiled, self.scale, self.bias, self.in_features,
+                                                       self.out_features, residual, norm, swiglu_up)
         if x.is_cuda and (norm is not None or swiglu_up is not None):
             from .. import _C
             return _C.ternary_linear_packed_forward_fused(x, self.weight_packed, self.scale, self.bias,
@@ -59,6 +115,15 @@ class TernaryLinearInference(nn.Module):
         """Forward from activations already quantized per row to int8 (``ops.rmsnorm`` /
         ``ops.swiglu`` / ``ops.act_quant_int8`` with ``quantize=True``): int8 matrix cores, int32
         accumulators (GPU only).  ``q_operand_order`` as in :func:`ops.ternary_linear_int8`."""
+        tiled = self._tiled_for(q, q.numel() // max(q.shape[-1], 1))
+        if tiled is not None:
+            from .. import _C
+            lead = q.shape[:-1]
+            y = _C.ternary_gemm_int8_tiled(q.reshape(-1, q.shape[-1]), s_x.reshape(-1), tiled, self.scale, self.bias,
+                                           self.in_features, self.out_features, out_dtype, False,
+                                           None if residual is None else residual.reshape(-1, residual.shape[-1]),
+                                           q_operand_order)
+            return y.reshape(*lead, self.out_features)
         from ..ops.fused import ternary_linear_int8
         return ternary_linear_int8(q, s_x, self.weight_packed, self.scale, self.in_features, self.bias,
                                    out_dtype, residual, q_operand_order)

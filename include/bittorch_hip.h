@@ -210,6 +210,34 @@ int bt_ternary_linear_packed_forward_fused(const void* X, int64_t ld_x, int x_dt
                                            void* stream);
 
 /*
+ * Decode-tiled copy of the packed weights (no counterpart in the reference, whose kernels read
+ * W_T [Kb, N] of bittorch/quant/ternary_packed.py:174-206 only).  A decode-shape kernel gives every
+ * compute unit a 16-column tile; in the row-major W_T such a tile touches 16 bytes of each 128-byte
+ * line.  The tiled copy stores, for tile t = n / 16 and step s = kb / 16 (S = ceil(Kb / 16) steps), 64
+ * dwords: dword ((t * S + s) * 64 + 16 g + j) holds the bytes W_T[16 s + 4 g + r, 16 t + j], r = 0..3,
+ * low byte first (= 16 consecutive k of one output column), zero outside the matrix.  It is built
+ * once from W_T (bt_retile_weights, exact inverse bt_untile_weights) and holds
+ * bt_tiled_weights_bytes(N, K) = ceil(N/16) * S * 256 bytes, 256-byte aligned, below 4 GiB.
+ *   bt_ternary_linear_tiled_forward: bt_ternary_linear_packed_forward_fused on the tiled copy, with
+ *     pro_op = BT_PRO_NONE allowed (then ld_x must equal K); the weights are streamed once per 16
+ *     rows of X, so it is meant for decode shapes; fp32 X needs K % 64 == 0 and the workspace.
+ *     Results equal those of the row-major entry points bit for bit.
+ *   bt_ternary_gemm_i8_tiled: bt_ternary_gemm_i8_res on the tiled copy (same remark).
+ */
+size_t bt_tiled_weights_bytes(int64_t N, int64_t K);
+int bt_retile_weights(const uint8_t* W_T, int64_t N, int64_t K, uint8_t* W_tiled, void* stream);
+int bt_untile_weights(const uint8_t* W_tiled, int64_t N, int64_t K, uint8_t* W_T, void* stream);
+int bt_ternary_linear_tiled_forward(const void* X, int64_t ld_x, int x_dtype, int pro_op, const void* pro_b,
+                                    int64_t ld_b, float eps, const uint8_t* W_tiled, const void* scale,
+                                    int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
+                                    const void* residual, void* Y, int64_t B, int64_t N, int64_t K,
+                                    void* workspace, size_t workspace_bytes, void* stream);
+int bt_ternary_gemm_i8_tiled(const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_tiled,
+                             const void* scale, int scale_dtype, int64_t scale_len, const void* bias,
+                             int bias_dtype, const void* residual, void* Y, int y_dtype, int32_t* acc_out,
+                             int64_t B, int64_t N, int64_t K, void* stream);
+
+/*
  * Matrix-core forward from float activations: bt_act_quant_i8 followed by
  * bt_ternary_gemm_i8.  Replaces bittorch._C.ternary_linear_tensor_core_forward
  * (bittorch_bindings.cpp:65-87, ternary_gemm_tensor_core.cu:663-727) for

@@ -129,6 +129,19 @@ def unpack_ternary_transposed(packed_t, in_features: int) -> np.ndarray:
     return out
 
 
+def retile_weights(packed_t, in_features: int) -> np.ndarray:
+    """Decode-tiled copy of ``W_T [Kb, N]`` (a layout of this library, no counterpart in the reference):
+    zero-pad to whole 16-row steps and 16-column tiles, then order the bytes as
+    ``[tile t][step s][row group g][column j][row r]`` with ``kb = 16 s + 4 g + r``, ``n = 16 t + j``."""
+    w = np.ascontiguousarray(packed_t, dtype=np.uint8)
+    kb, n = w.shape
+    assert kb == (in_features + 3) // 4
+    steps, tiles = (kb + 15) // 16, (n + 15) // 16
+    padded = np.zeros((steps * 16, tiles * 16), dtype=np.uint8)
+    padded[:kb, :n] = w
+    return np.ascontiguousarray(padded.reshape(steps, 4, 4, tiles, 16).transpose(3, 0, 1, 4, 2)).reshape(-1)
+
+
 def _lin_args(x, w, scale, bias):
     x = _f32(x)
     scale = _f32(scale).reshape(-1)

@@ -1,0 +1,213 @@
+"""GPU parity of the decode-tiled copy of the packed weights.
+
+* the layout: ``retile_weights`` against the oracle's numpy restatement, byte for byte, and
+  ``untile_weights`` as its exact inverse (ragged N and K included);
+* the kernels: every forward on the tiled copy equals the same forward on the row-major ``W_T``
+  bit for bit (which the other GPU tests hold against the oracle), on decode shapes, batches that
+  span several 16-row launches, all dtypes, with bias / residual / prologues, and the int8 path
+  with its int32 accumulators;
+* one direct comparison with the oracle, so that this file stands on its own.
+"""
+import numpy as np
+import pytest
+import torch
+
+from conftest import announce
+from _util import f32np, random_ternary, rel_err, seeded_acts
+
+pytestmark = pytest.mark.gpu
+
+# (N, K): config-2 shape, ragged columns (N % 16 != 0, N % 4 != 0), ragged K, tiny, wide
+LAYOUT_SHAPES = [(4096, 4096), (100, 64), (37, 100), (16, 4), (1, 1), (250, 1030), (11008, 512)]
+
+
+def _packed(oracle, n, k, seed=0):
+    w = random_ternary(n, k, seed=seed)
+    packed_t, _ = oracle.pack_ternary_transposed(w.numpy())
+    return w, torch.from_numpy(packed_t).cuda()
+
+
+@pytest.mark.parametrize("n,k", LAYOUT_SHAPES)
+def test_retile_layout_and_inverse(oracle, n, k):
+    from bittorch_amd import _C
+    announce("retile", n, k)
+    _, wt = _packed(oracle, n, k, seed=n + k)
+    tiled = _C.retile_weights(wt, k)
+    torch.cuda.synchronize()
+    assert tiled.numel() == ((n + 15) // 16) * (((k + 3) // 4 + 15) // 16) * 256
+    np.testing.assert_array_equal(tiled.cpu().numpy(), oracle.retile_weights(wt.cpu().numpy(), k))
+    back = _C.untile_weights(tiled, n, k)
+    assert torch.equal(back, wt)
+
+
+FWD_SHAPES = [(4096, 4096), (2560, 2560), (6912, 2560), (2560, 6912), (100, 64), (37, 100), (250, 1030), (16, 8),
+              (11008, 4096)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n,k", FWD_SHAPES)
+def test_tiled_forward_equals_row_major(oracle, dtype, n, k):
+    from bittorch_amd import _C
+    _, wt = _packed(oracle, n, k, seed=1)
+    tiled = _C.retile_weights(wt, k)
+    g = torch.Generator().manual_seed(n + k)
+    scale = (torch.rand(n, generator=g) + 0.5).cuda()
+    bias = (torch.randn(n, generator=g) * 0.01).to(dtype).cuda()
+    for b in (1, 2, 5, 16, 17, 32, 40):
+        announce("tiled forward", dtype, n, k, b)
+        x = seeded_acts(b, k, seed=b, dtype=dtype).cuda()
+        res = seeded_acts(b, n, seed=b + 1, dtype=dtype).cuda()
+        ref = _C.ternary_linear_packed_forward(x, wt, scale, bias, k, residual=res)
+        got = _C.ternary_linear_tiled_forward(x, tiled, scale, bias, k, n, residual=res)
+        if b <= 32:
+            assert torch.equal(got, ref)
+        else:  # the row-major call runs the tall-batch kernel there: another summation order
+            assert rel_err(f32np(got), f32np(ref)) <= 2e-3
+    x = seeded_acts(1, k, seed=9, dtype=dtype).cuda()
+    assert torch.equal(_C.ternary_linear_tiled_forward(x, tiled, scale[:1], None, k, n),
+                       _C.ternary_linear_packed_forward(x, wt, scale[:1], None, k))
+
+
+@pytest.mark.parametrize("n,k", [(4096, 4096), (100, 64), (2560, 6912)])
+def test_tiled_forward_fp32_planes(oracle, n, k):
+    from bittorch_amd import _C
+    _, wt = _packed(oracle, n, k, seed=2)
+    tiled = _C.retile_weights(wt, k)
+    scale = (torch.rand(n) + 0.5).cuda()
+    for b in (1, 3, 20):
+        announce("tiled forward fp32", n, k, b)
+        x = seeded_acts(b, k, seed=b, dtype=torch.float32).cuda()
+        assert torch.equal(_C.ternary_linear_tiled_forward(x, tiled, scale, None, k, n),
+                           _C.ternary_linear_packed_forward(x, wt, scale, None, k))
+
+
+def test_tiled_forward_fp32_ragged_k_is_refused(oracle):
+    from bittorch_amd import _C
+    _, wt = _packed(oracle, 37, 100)
+    tiled = _C.retile_weights(wt, 100)
+    x = seeded_acts(2, 100, dtype=torch.float32).cuda()
+    with pytest.raises(RuntimeError, match="K % 64"):
+        _C.ternary_linear_tiled_forward(x, tiled, torch.ones(37).cuda(), None, 100, 37)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n,k", [(4096, 4096), (7680, 2560), (2560, 6912), (100, 64)])
+def test_tiled_prologues_equal_row_major(oracle, dtype, n, k):
+    from bittorch_amd import _C
+    _, wt = _packed(oracle, n, k, seed=3)
+    tiled = _C.retile_weights(wt, k)
+    scale = (torch.rand(n) + 0.5).cuda()
+    nw = (torch.rand(k) + 0.5).to(dtype).cuda()
+    for b in (1, 3):
+        announce("tiled prologue", dtype, n, k, b)
+        x = seeded_acts(b, k, seed=b, dtype=dtype).cuda()
+        u = seeded_acts(b, k, seed=b + 5, dtype=dtype).cuda()
+        res = seeded_acts(b, n, seed=b + 7, dtype=dtype).cuda()
+        for kw in (dict(norm=(nw, 1e-5)), dict(norm=(None, 1e-6)), dict(swiglu_up=u)):
+            ref = _C.ternary_linear_packed_forward_fused(x, wt, scale, None, k, residual=res, **kw)
+            got = _C.ternary_linear_tiled_forward(x, tiled, scale, None, k, n, residual=res, **kw)
+            assert torch.equal(got, ref)
+
+
+@pytest.mark.parametrize("n,k", [(4096, 4096), (11008, 4096), (4096, 11008), (100, 64), (37, 100)])
+def test_tiled_int8_equals_row_major(oracle, n, k):
+    from bittorch_amd import _C
+    _, wt = _packed(oracle, n, k, seed=4)
+    tiled = _C.retile_weights(wt, k)
+    scale = (torch.rand(n) + 0.5).cuda()
+    bias = (torch.randn(n) * 0.01).cuda()
+    for b in (1, 16, 33):
+        for oo in ((False, True) if k % 16 == 0 else (False,)):
+            announce("tiled int8", n, k, b, oo)
+            x = seeded_acts(b, k, seed=b, dtype=torch.bfloat16, outliers=True).cuda()
+            q, s = _C.act_quant_int8(x, oo)
+            res = seeded_acts(b, n, seed=b + 1, dtype=torch.bfloat16).cuda()
+            y0, a0 = _C.ternary_gemm_int8(q, s, wt, scale, bias, k, torch.bfloat16, True, res, oo)
+            y1, a1 = _C.ternary_gemm_int8_tiled(q, s, tiled, scale, bias, k, n, torch.bfloat16, True, res, oo)
+            assert torch.equal(a1, a0) and torch.equal(y1, y0)
+
+
+def test_tiled_forward_against_oracle(oracle):
+    from bittorch_amd import _C
+    n, k = 300, 520
+    w, wt = _packed(oracle, n, k, seed=5)
+    tiled = _C.retile_weights(wt, k)
+    scale = torch.rand(n) + 0.5
+    bias = torch.randn(n) * 0.01
+    x = seeded_acts(4, k, seed=6, dtype=torch.float16)
+    got = _C.ternary_linear_tiled_forward(x.cuda(), tiled, scale.cuda(), bias.half().cuda(), k, n)
+    ref = oracle.linear_packed(f32np(x), wt.cpu().numpy(), scale.numpy(), k, f32np(bias.half()))
+    assert rel_err(f32np(got), ref) <= 1e-3  # fp16 output rounding on fp32 sums
+
+
+def test_tiled_size_mismatch_is_refused(oracle):
+    from bittorch_amd import _C
+    _, wt = _packed(oracle, 64, 64)
+    tiled = _C.retile_weights(wt, 64)
+    x = seeded_acts(1, 64, dtype=torch.float16).cuda()
+    with pytest.raises(RuntimeError, match="W_tiled size"):
+        _C.ternary_linear_tiled_forward(x, tiled, torch.ones(80).cuda(), None, 64, 80)
+
+
+def _layer(oracle, n, k, seed=0, **kw):
+    from bittorch_amd.nn import TernaryLinearInference
+    w = random_ternary(n, k, seed=seed)
+    packed_t, _ = oracle.pack_ternary_transposed(w.numpy())
+    g = torch.Generator().manual_seed(seed)
+    return TernaryLinearInference(k, n, torch.from_numpy(packed_t), torch.rand(n, generator=g) + 0.5,
+                                  torch.randn(n, generator=g) * 0.01, **kw).cuda()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_module_uses_tiled_copy_for_decode_shapes(oracle, dtype):
+    announce("module tiled", dtype)
+    a = _layer(oracle, 640, 512, seed=3)                      # default: tiled copy on first decode call
+    b = _layer(oracle, 640, 512, seed=3, decode_tiled=False)  # weight_packed only
+    assert a.decode_tiled and a._tiled is None
+    for shape in ((512,), (1, 512), (2, 3, 512), (32, 512), (40, 512)):
+        x = seeded_acts(1, int(np.prod(shape)), seed=len(shape), dtype=dtype).reshape(shape).cuda()
+        ya, yb = a(x), b(x)
+        assert ya.shape == yb.shape == (*shape[:-1], 640)
+        assert torch.equal(ya, yb)
+    assert a._tiled is not None and b._tiled is None
+    assert "_tiled" not in a.state_dict() and set(a.state_dict()) == set(b.state_dict())
+    # prologues, residual and the int8 path go the same way
+    x = seeded_acts(1, 512, seed=8, dtype=dtype).cuda()
+    r = seeded_acts(1, 640, seed=9, dtype=dtype).cuda()
+    assert torch.equal(a(x, r, norm=(None, 1e-6)), b(x, r, norm=(None, 1e-6)))
+    assert torch.equal(a(x, swiglu_up=x.flip(-1)), b(x, swiglu_up=x.flip(-1)))
+    from bittorch_amd import _C
+    q, s = _C.act_quant_int8(x, True)
+    assert torch.equal(a.forward_int8(q, s, torch.bfloat16, None, True), b.forward_int8(q, s, torch.bfloat16, None, True))
+
+
+def test_module_rebuilds_tiled_copy_when_weights_change(oracle):
+    a = _layer(oracle, 64, 64, seed=1)
+    x = seeded_acts(1, 64, dtype=torch.float16).cuda()
+    y0 = a(x)
+    first = a._tiled
+    a.weight_packed.zero_()                      # in-place write: the copy is stale
+    assert torch.equal(a(x).float(), a.bias.half().float().expand(1, -1))
+    assert a._tiled is not first
+    other = _layer(oracle, 64, 64, seed=1)
+    a.load_state_dict(other.state_dict())        # copy_ into the buffers: stale again
+    assert torch.equal(a(x), y0)
+
+
+def test_module_never_builds_the_copy_inside_a_capture(oracle):
+    a = _layer(oracle, 256, 256, seed=2)
+    x = seeded_acts(1, 256, dtype=torch.bfloat16).cuda()
+    ref = _layer(oracle, 256, 256, seed=2, decode_tiled=False)(x)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(s):
+        with torch.cuda.graph(g, stream=s):
+            y = a(x)
+    torch.cuda.current_stream().wait_stream(s)
+    assert a._tiled is None                      # fell back to weight_packed
+    g.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(y, ref)
+    a.prepare_decode()
+    assert a._tiled is not None and torch.equal(a(x), ref)
