@@ -8,6 +8,7 @@ from .convert import (
     get_model_memory_bytes,
     load_ternary_checkpoint,
     load_ternary_safetensors,
+    prepare_decode,
     save_ternary_checkpoint,
     save_ternary_safetensors,
     ternary_linear_to_infer,
@@ -18,6 +19,7 @@ __all__ = [
     "ternary_linear_to_infer",
     "convert_linear_layers",
     "fuse_ternary_linear_inference",
+    "prepare_decode",
     "count_ternary_params",
     "get_model_memory_bytes",
     "save_ternary_checkpoint",

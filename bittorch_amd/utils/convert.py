@@ -98,6 +98,16 @@ def fuse_ternary_linear_inference(*layers: TernaryLinearInference) -> TernaryLin
     return TernaryLinearInference(k, sum(l.out_features for l in layers), packed, scale, bias)
 
 
+def prepare_decode(module: nn.Module) -> nn.Module:
+    """Build the decode-tiled weight copy of every ``TernaryLinearInference`` inside ``module`` now
+    (they are otherwise built on each layer's first decode-shape call, and never during a HIP graph
+    capture, which falls back to ``weight_packed``).  Doubles the packed-weight memory of those layers."""
+    for m in module.modules():
+        if isinstance(m, TernaryLinearInference):
+            m.prepare_decode()
+    return module
+
+
 def count_ternary_params(module: nn.Module) -> Dict[str, int]:
     """Weights by storage type (reference ``:136-166``): ``fp32``, ``fp16``, ``packed_ternary``, ``total``
     (biases and scales are not counted; any non-fp16 dense weight counts as fp32, as in the reference)."""
