@@ -249,17 +249,21 @@ def ternary_linear_packed_forward_fused(X: Tensor, W_T: Tensor, scale: Tensor, b
     return y.reshape(*X.shape[:-1], N)
 
 
-def retile_weights(W_T: Tensor, in_features: int) -> Tensor:
+def retile_weights(W_T: Tensor, in_features: int, gate_up_pairs: bool = False) -> Tensor:
     """Decode-tiled copy of ``W_T [ceil(K/4), N]`` (flat uint8 tensor): per 16-column tile and 16-row step
-    the 64 dwords a wave of the decode kernel loads, contiguous.  Built once; :func:`untile_weights` inverts it."""
+    the 64 dwords a wave of the decode kernel loads, contiguous.  Built once; :func:`untile_weights` inverts it.
+    ``gate_up_pairs`` (N % 32 == 0): the tiles of the two column halves alternate, for the SwiGLU output stage
+    of :func:`ternary_linear_tiled_forward` (such a copy serves only that)."""
     _check(W_T.dim() == 2 and W_T.dtype == torch.uint8, "W_T must be 2D uint8 [K_bytes, N]")
+    _check(not gate_up_pairs or W_T.shape[1] % 32 == 0, "gate/up pair order needs N % 32 == 0")
     _check(W_T.shape[0] == (in_features + 3) // 4, "K_bytes doesn't match ceil(K/4)")
     _check(_all_cuda(W_T), "All tensors must be CUDA")
     W_T = W_T.contiguous()
     N = W_T.shape[1]
     with torch.cuda.device(W_T.device):
         out = torch.empty((_L.bt_tiled_weights_bytes(N, in_features),), dtype=torch.uint8, device=W_T.device)
-        _status(_L.bt_retile_weights(W_T.data_ptr(), N, in_features, out.data_ptr(), _stream(W_T)))
+        _status(_L.bt_retile_weights(W_T.data_ptr(), N, in_features, 1 if gate_up_pairs else 0, out.data_ptr(),
+                                     _stream(W_T)))
     return out
 
 
@@ -270,22 +274,27 @@ def _tiled_checks(W_tiled: Tensor, N: int, K: int):
            "W_tiled size doesn't match out_features x in_features")
 
 
-def untile_weights(W_tiled: Tensor, out_features: int, in_features: int) -> Tensor:
+def untile_weights(W_tiled: Tensor, out_features: int, in_features: int, gate_up_pairs: bool = False) -> Tensor:
     """``W_T [ceil(K/4), N]`` back from its decode-tiled copy (exact inverse of :func:`retile_weights`)."""
     _tiled_checks(W_tiled, out_features, in_features)
     _check(_all_cuda(W_tiled), "All tensors must be CUDA")
     with torch.cuda.device(W_tiled.device):
         out = torch.empty(((in_features + 3) // 4, out_features), dtype=torch.uint8, device=W_tiled.device)
-        _status(_L.bt_untile_weights(W_tiled.data_ptr(), out_features, in_features, out.data_ptr(), _stream(W_tiled)))
+        _status(_L.bt_untile_weights(W_tiled.data_ptr(), out_features, in_features, 1 if gate_up_pairs else 0,
+                                     out.data_ptr(), _stream(W_tiled)))
     return out
 
 
 def ternary_linear_tiled_forward(X: Tensor, W_tiled: Tensor, scale: Tensor, bias: Optional[Tensor] = None,
                                  in_features: int = -1, out_features: int = -1, residual: Optional[Tensor] = None,
                                  norm: Optional[Tuple[Optional[Tensor], float]] = None,
-                                 swiglu_up: Optional[Tensor] = None) -> Tensor:
+                                 swiglu_up: Optional[Tensor] = None, swiglu_pairs: bool = False) -> Tensor:
     """:func:`ternary_linear_packed_forward` / ``_fused`` on the decode-tiled copy of the weights (same
-    results bit for bit); the weights are streamed once per 16 rows of ``X``, so this is for decode shapes."""
+    results bit for bit); the weights are streamed once per 16 rows of ``X``, so this is for decode shapes.
+    ``swiglu_pairs`` (copy built with ``gate_up_pairs=True``): the layer's columns are ``[gate | up]`` and the
+    output is the MLP's hidden vector ``swiglu(gate(x), up(x))`` ``[*, N/2]``, formed in the kernel's output stage."""
+    _check(not swiglu_pairs or (residual is None and swiglu_up is None and out_features % 32 == 0),
+           "swiglu_pairs needs N % 32 == 0 and takes neither a residual nor a SwiGLU prologue")
     _check(norm is None or swiglu_up is None, "at most one of norm and swiglu_up may be given")
     _check(X.dim() >= 1 and X.numel() > 0, "X is empty")
     K, N = X.shape[-1], out_features
@@ -312,15 +321,16 @@ def ternary_linear_tiled_forward(X: Tensor, W_tiled: Tensor, scale: Tensor, bias
         op, ldb = 2, pb.stride(0)
     _check(_all_cuda(pb), "All tensors must be CUDA")
     xdt = _dt(x2, "X")
-    y = torch.empty((B, N), dtype=X.dtype, device=X.device)
+    Ny = N // 2 if swiglu_pairs else N
+    y = torch.empty((B, Ny), dtype=X.dtype, device=X.device)
     res = None if residual is None else _residual_2d(residual, X, X.shape[:-1], N)
     with torch.cuda.device(X.device):
         ws = _workspace(_L.bt_packed_forward_fused_workspace_bytes(B, N, K, xdt), X.device)
         _status(_L.bt_ternary_linear_tiled_forward(
             x2.data_ptr(), x2.stride(0), xdt, op, _ptr(pb), ldb, float(eps), W_tiled.data_ptr(), scale.data_ptr(),
             _dt(scale, "scale"), scale.numel(), _ptr(bias), 0 if bias is None else _dt(bias, "bias"), _ptr(res),
-            y.data_ptr(), B, N, K, _ptr(ws), 0 if ws is None else ws.numel(), _stream(X)))
-    return y.reshape(*X.shape[:-1], N)
+            1 if swiglu_pairs else 0, y.data_ptr(), B, N, K, _ptr(ws), 0 if ws is None else ws.numel(), _stream(X)))
+    return y.reshape(*X.shape[:-1], Ny)
 
 
 def ternary_gemm_int8_tiled(Q: Tensor, s_x: Tensor, W_tiled: Tensor, scale: Tensor, bias: Optional[Tensor] = None,

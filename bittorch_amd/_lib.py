@@ -53,10 +53,10 @@ SIGNATURES = {
     "bt_ternary_linear_packed_forward_fused": (_int, [_vp, _i64, _int, _int, _vp, _i64, ctypes.c_float, _vp, _vp, _int,
                                                       _i64, _vp, _int, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp]),
     "bt_tiled_weights_bytes": (_sz, [_i64, _i64]),
-    "bt_retile_weights": (_int, [_vp, _i64, _i64, _vp, _vp]),
-    "bt_untile_weights": (_int, [_vp, _i64, _i64, _vp, _vp]),
+    "bt_retile_weights": (_int, [_vp, _i64, _i64, _int, _vp, _vp]),
+    "bt_untile_weights": (_int, [_vp, _i64, _i64, _int, _vp, _vp]),
     "bt_ternary_linear_tiled_forward": (_int, [_vp, _i64, _int, _int, _vp, _i64, ctypes.c_float, _vp, _vp, _int,
-                                               _i64, _vp, _int, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp]),
+                                               _i64, _vp, _int, _vp, _int, _vp, _i64, _i64, _i64, _vp, _sz, _vp]),
     "bt_ternary_gemm_i8_tiled": (_int, [_vp, _int, _vp, _vp, _vp, _int, _i64, _vp, _int, _vp, _vp, _int, _vp,
                                         _i64, _i64, _i64, _vp]),
 }

@@ -221,6 +221,10 @@ enum { Q_ROW_MAJOR = 0, Q_OPERAND_ORDER = 1 };
 //                       row or the column lies outside the matrix
 enum { W_LAYOUT_ROW_MAJOR = 0, W_LAYOUT_TILED = 1 };
 
+// activation prologues and output stages of the streaming kernel (BT_PRO_*, BT_EPI_* of the C ABI)
+enum { PRO_NONE = 0, PRO_RMSNORM = 1, PRO_SWIGLU = 2 };
+enum { EPI_NONE = 0, EPI_SWIGLU_PAIRS = 1 };
+
 // Two neighbouring lanes hold the 16 quantized bytes of one group (even lane: elements 0..7 as
 // lo, hi; odd lane: elements 8..15).  Returns this lane's 8 bytes of the transposed group.
 // Both lanes of a pair must call it (it exchanges registers between them).

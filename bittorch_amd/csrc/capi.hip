@@ -34,10 +34,12 @@ bool stream_supported_tiled(int64_t N, int64_t K, const void* W);
 size_t tiled_bytes(int64_t N, int64_t K);
 int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, const uint8_t* W_T, int w_layout,
                   const Epilogue& epi, void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N,
-                  int64_t K, int planes, int q_layout, int pro_op, const void* pro_b, float pro_eps,
+                  int64_t K, int planes, int q_layout, int pro_op, const void* pro_b, float pro_eps, int epi_op,
                   hipStream_t st);
-bool stream_prologue_fusable(int mode, int64_t B, int64_t N, int64_t K, const void* X, const void* pro_b, int w_layout);
-int launch_retile(const uint8_t* W_T, int64_t N, int64_t K, void* T, bool inverse, uint8_t* W_out, hipStream_t st);
+bool stream_prologue_fusable(int mode, int64_t B, int64_t N, int64_t K, const void* X, const void* pro_b, int w_layout,
+                             int epi_op);
+int launch_retile(const uint8_t* W_T, int64_t N, int64_t K, int pairs, void* T, bool inverse, uint8_t* W_out,
+                  hipStream_t st);
 int launch_split_f32_planes(const void* X, int64_t B, int64_t K, void* P, hipStream_t st);
 int launch_packed_generic(const void* X, int x_dtype, const uint8_t* W_T, const Epilogue& epi, void* Y,
                           int64_t B, int64_t N, int64_t K, hipStream_t st);
@@ -165,7 +167,7 @@ static int set_residual(const char* who, const void* residual, Epilogue* e) {
     return BT_OK;
 }
 
-static int packed_forward_impl(const char* who, const void* X, int x_dtype, const uint8_t* W_T, int w_layout,
+static int packed_forward_impl(const char* who, const void* X, int x_dtype, const uint8_t* W_T, int w_layout, int epi_op,
                                const void* scale, int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
                                const void* residual, void* Y, int64_t B, int64_t N, int64_t K, void* workspace,
                                size_t workspace_bytes, void* stream) {
@@ -177,6 +179,10 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
     rc = set_residual(who, residual, &epi);
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
+    if (epi_op != 0 && (epi_op != EPI_SWIGLU_PAIRS || w_layout != W_LAYOUT_TILED || N % 32 != 0 || residual)) {
+        set_error("%s: the SwiGLU output stage needs pair-ordered tiled weights, N %% 32 == 0 and no residual", who);
+        return BT_ERR_INVALID;
+    }
     if (w_layout == W_LAYOUT_TILED) {
         // the decode-tiled copy is read by the streaming kernel only, once per 16 rows
         if (!stream_supported_tiled(N, K, W_T) || !fast_path_ok(Y, N, 3 * K) || 3 * K >= (1ll << 26)) {
@@ -186,7 +192,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         if (x_dtype != BT_F32) {
             const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
             return launch_stream(mode, X, 2, nullptr, W_T, W_LAYOUT_TILED, epi, Y, x_dtype, nullptr, B, N, K, 1,
-                                 Q_ROW_MAJOR, 0, nullptr, 0.0f, st);
+                                 Q_ROW_MAJOR, 0, nullptr, 0.0f, epi_op, st);
         }
         if (K % 64 != 0 || ((uintptr_t)X) % 16 != 0 || !workspace || workspace_bytes < f32_planes_bytes(B, K) ||
             ((uintptr_t)workspace) % 256 != 0) {
@@ -197,14 +203,14 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         rc = launch_split_f32_planes(X, B, K, workspace, st);
         if (rc) return rc;
         return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, W_LAYOUT_TILED, epi, Y, BT_F32, nullptr, B, N, K, 3,
-                             Q_ROW_MAJOR, 0, nullptr, 0.0f, st);
+                             Q_ROW_MAJOR, 0, nullptr, 0.0f, epi_op, st);
     }
     if (packed_uses_stream(x_dtype, W_T, Y, N, K)) {
         const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
         // tall batches go to the tiled matrix-core kernel, decode shapes stream the weights
         if (B > kStreamMaxRows && gemm_f16_supported(N, K, X, W_T, Y))
             return launch_gemm_f16(mode, X, W_T, epi, Y, x_dtype, B, N, K, 1, st);
-        return launch_stream(mode, X, 2, nullptr, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, x_dtype, nullptr, B, N, K, 1, Q_ROW_MAJOR, 0, nullptr, 0.0f, st);
+        return launch_stream(mode, X, 2, nullptr, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, x_dtype, nullptr, B, N, K, 1, Q_ROW_MAJOR, 0, nullptr, 0.0f, 0, st);
     }
     if (x_dtype == BT_F32 && packed_uses_f32_planes(X, W_T, Y, N, K) && workspace &&
         workspace_bytes >= f32_planes_bytes(B, K) && ((uintptr_t)workspace) % 256 == 0) {
@@ -213,7 +219,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         if (rc) return rc;
         if (B > kStreamMaxRows && gemm_f16_supported(N, 3 * K, workspace, W_T, Y))
             return launch_gemm_f16(MODE_BF16, workspace, W_T, epi, Y, BT_F32, B, N, K, 3, st);
-        return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, BT_F32, nullptr, B, N, K, 3, Q_ROW_MAJOR, 0, nullptr, 0.0f, st);
+        return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, BT_F32, nullptr, B, N, K, 3, Q_ROW_MAJOR, 0, nullptr, 0.0f, 0, st);
     }
     return launch_packed_generic(X, x_dtype, W_T, epi, Y, B, N, K, st);
 }
@@ -223,7 +229,7 @@ extern "C" int bt_ternary_linear_packed_forward(const void* X, int x_dtype, cons
                                                 const void* bias, int bias_dtype, void* Y, int64_t B,
                                                 int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
                                                 void* stream) {
-    return packed_forward_impl("bt_ternary_linear_packed_forward", X, x_dtype, W_T, W_LAYOUT_ROW_MAJOR, scale, scale_dtype, scale_len, bias,
+    return packed_forward_impl("bt_ternary_linear_packed_forward", X, x_dtype, W_T, W_LAYOUT_ROW_MAJOR, 0, scale, scale_dtype, scale_len, bias,
                                bias_dtype, nullptr, Y, B, N, K, workspace, workspace_bytes, stream);
 }
 
@@ -232,7 +238,7 @@ extern "C" int bt_ternary_linear_packed_forward_res(const void* X, int x_dtype, 
                                                     const void* bias, int bias_dtype, const void* residual,
                                                     void* Y, int64_t B, int64_t N, int64_t K, void* workspace,
                                                     size_t workspace_bytes, void* stream) {
-    return packed_forward_impl("bt_ternary_linear_packed_forward_res", X, x_dtype, W_T, W_LAYOUT_ROW_MAJOR, scale, scale_dtype, scale_len,
+    return packed_forward_impl("bt_ternary_linear_packed_forward_res", X, x_dtype, W_T, W_LAYOUT_ROW_MAJOR, 0, scale, scale_dtype, scale_len,
                                bias, bias_dtype, residual, Y, B, N, K, workspace, workspace_bytes, stream);
 }
 
@@ -310,7 +316,7 @@ static int gemm_i8_impl(const char* who, const int8_t* Q, int q_layout, const fl
             return BT_ERR_INVALID;
         }
         return launch_stream(MODE_I8, Q, 1, s_x, W_T, w_layout, epi, Y, y_dtype, acc_out, B, N, K, 1, q_layout, 0, nullptr,
-                             0.0f, st);
+                             0.0f, 0, st);
     }
     // decode-shape batches, and any batch whose N the tiled kernel's 4-column
     // vector accesses cannot take, stream the weights once per 16 rows
@@ -320,7 +326,7 @@ static int gemm_i8_impl(const char* who, const int8_t* Q, int q_layout, const fl
                       (long long)ceil_div(K, 4), (long long)N);
             return BT_ERR_INVALID;
         }
-        return launch_stream(MODE_I8, Q, 1, s_x, W_T, w_layout, epi, Y, y_dtype, acc_out, B, N, K, 1, q_layout, 0, nullptr, 0.0f, st);
+        return launch_stream(MODE_I8, Q, 1, s_x, W_T, w_layout, epi, Y, y_dtype, acc_out, B, N, K, 1, q_layout, 0, nullptr, 0.0f, 0, st);
     }
     return launch_gemm_i8(Q, q_layout, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, st);
 }
@@ -429,7 +435,7 @@ extern "C" size_t bt_packed_forward_fused_workspace_bytes(int64_t B, int64_t N, 
 }
 
 static int fused_forward_impl(const char* who, const void* X, int64_t ld_x, int x_dtype, int pro_op, const void* pro_b,
-                              int64_t ld_b, float eps, const uint8_t* W_T, int w_layout, const void* scale,
+                              int64_t ld_b, float eps, const uint8_t* W_T, int w_layout, int epi_op, const void* scale,
                               int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
                               const void* residual, void* Y, int64_t B, int64_t N, int64_t K, void* workspace,
                               size_t workspace_bytes, void* stream) {
@@ -437,6 +443,10 @@ static int fused_forward_impl(const char* who, const void* X, int64_t ld_x, int 
     if (rc) return rc;
     if (pro_op != 1 && pro_op != 2) {
         set_error("%s: prologue must be BT_PRO_RMSNORM or BT_PRO_SWIGLU (got %d)", who, pro_op);
+        return BT_ERR_INVALID;
+    }
+    if (pro_op == PRO_SWIGLU && epi_op != EPI_NONE) {
+        set_error("%s: a SwiGLU prologue and the SwiGLU output stage do not combine", who);
         return BT_ERR_INVALID;
     }
     if (ld_x < K || (pro_op == 2 && (!pro_b || ld_b < K))) {
@@ -449,14 +459,14 @@ static int fused_forward_impl(const char* who, const void* X, int64_t ld_x, int 
                                                       : packed_uses_stream(x_dtype, W_T, Y, N, K);
     if (x_dtype != BT_F32 && B == 1 && streams) {
         const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
-        if (stream_prologue_fusable(mode, B, N, K, X, pro_b, w_layout)) {
+        if (stream_prologue_fusable(mode, B, N, K, X, pro_b, w_layout, epi_op)) {
             Epilogue epi;
             rc = make_epilogue(who, scale, scale_dtype, scale_len, bias, bias_dtype, N, &epi);
             if (rc) return rc;
             rc = set_residual(who, residual, &epi);
             if (rc) return rc;
             return launch_stream(mode, X, 2, nullptr, W_T, w_layout, epi, Y, x_dtype, nullptr, B, N, K, 1, Q_ROW_MAJOR, pro_op,
-                                 pro_b, eps, st);
+                                 pro_b, eps, epi_op, st);
         }
     }
     // otherwise: the prologue as its own kernel into the workspace, then the plain forward
@@ -469,7 +479,7 @@ static int fused_forward_impl(const char* who, const void* X, int64_t ld_x, int 
     rc = launch_row_op(pro_op == 2 ? 0 : 1, x_dtype, X, ld_x, pro_b, ld_b, eps, B, K, workspace, nullptr, nullptr,
                        Q_ROW_MAJOR, st, who);
     if (rc) return rc;
-    return packed_forward_impl(who, workspace, x_dtype, W_T, w_layout, scale, scale_dtype, scale_len, bias, bias_dtype,
+    return packed_forward_impl(who, workspace, x_dtype, W_T, w_layout, epi_op, scale, scale_dtype, scale_len, bias, bias_dtype,
                                residual, Y, B, N, K, (uint8_t*)workspace + h_bytes, workspace_bytes - h_bytes, stream);
 }
 
@@ -481,7 +491,7 @@ extern "C" int bt_ternary_linear_packed_forward_fused(const void* X, int64_t ld_
                                                       int64_t K, void* workspace, size_t workspace_bytes,
                                                       void* stream) {
     return fused_forward_impl("bt_ternary_linear_packed_forward_fused", X, ld_x, x_dtype, pro_op, pro_b, ld_b, eps, W_T,
-                              W_LAYOUT_ROW_MAJOR, scale, scale_dtype, scale_len, bias, bias_dtype, residual, Y, B, N, K,
+                              W_LAYOUT_ROW_MAJOR, 0, scale, scale_dtype, scale_len, bias, bias_dtype, residual, Y, B, N, K,
                               workspace, workspace_bytes, stream);
 }
 
@@ -503,27 +513,36 @@ static int check_retile(const char* who, const void* a, const void* b, int64_t N
     return BT_OK;
 }
 
-extern "C" int bt_retile_weights(const uint8_t* W_T, int64_t N, int64_t K, uint8_t* W_tiled, void* stream) {
-    const int rc = check_retile("bt_retile_weights", W_T, W_tiled, N, K, W_tiled);
-    if (rc) return rc;
-    return launch_retile(W_T, N, K, W_tiled, false, nullptr, (hipStream_t)stream);
+static int check_tile_order(const char* who, int order, int64_t N) {
+    if (order == 0 || (order == 1 && N % 32 == 0)) return BT_OK;
+    set_error("%s: tile order must be BT_TILES_NATURAL, or BT_TILES_GATE_UP_PAIRS with N %% 32 == 0 (order=%d, N=%lld)",
+              who, order, (long long)N);
+    return BT_ERR_INVALID;
 }
 
-extern "C" int bt_untile_weights(const uint8_t* W_tiled, int64_t N, int64_t K, uint8_t* W_T, void* stream) {
-    const int rc = check_retile("bt_untile_weights", W_tiled, W_T, N, K, W_tiled);
+extern "C" int bt_retile_weights(const uint8_t* W_T, int64_t N, int64_t K, int order, uint8_t* W_tiled, void* stream) {
+    int rc = check_retile("bt_retile_weights", W_T, W_tiled, N, K, W_tiled);
     if (rc) return rc;
-    return launch_retile(nullptr, N, K, (void*)W_tiled, true, W_T, (hipStream_t)stream);
+    if ((rc = check_tile_order("bt_retile_weights", order, N))) return rc;
+    return launch_retile(W_T, N, K, order, W_tiled, false, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int bt_untile_weights(const uint8_t* W_tiled, int64_t N, int64_t K, int order, uint8_t* W_T, void* stream) {
+    int rc = check_retile("bt_untile_weights", W_tiled, W_T, N, K, W_tiled);
+    if (rc) return rc;
+    if ((rc = check_tile_order("bt_untile_weights", order, N))) return rc;
+    return launch_retile(nullptr, N, K, order, (void*)W_tiled, true, W_T, (hipStream_t)stream);
 }
 
 extern "C" int bt_ternary_linear_tiled_forward(const void* X, int64_t ld_x, int x_dtype, int pro_op,
                                                const void* pro_b, int64_t ld_b, float eps, const uint8_t* W_tiled,
                                                const void* scale, int scale_dtype, int64_t scale_len,
-                                               const void* bias, int bias_dtype, const void* residual, void* Y,
-                                               int64_t B, int64_t N, int64_t K, void* workspace,
+                                               const void* bias, int bias_dtype, const void* residual, int epi_op,
+                                               void* Y, int64_t B, int64_t N, int64_t K, void* workspace,
                                                size_t workspace_bytes, void* stream) {
     const char* who = "bt_ternary_linear_tiled_forward";
     if (pro_op != 0)
-        return fused_forward_impl(who, X, ld_x, x_dtype, pro_op, pro_b, ld_b, eps, W_tiled, W_LAYOUT_TILED, scale,
+        return fused_forward_impl(who, X, ld_x, x_dtype, pro_op, pro_b, ld_b, eps, W_tiled, W_LAYOUT_TILED, epi_op, scale,
                                   scale_dtype, scale_len, bias, bias_dtype, residual, Y, B, N, K, workspace,
                                   workspace_bytes, stream);
     if (ld_x != K) {
@@ -531,7 +550,7 @@ extern "C" int bt_ternary_linear_tiled_forward(const void* X, int64_t ld_x, int 
                   (long long)ld_x, (long long)K);
         return BT_ERR_INVALID;
     }
-    return packed_forward_impl(who, X, x_dtype, W_tiled, W_LAYOUT_TILED, scale, scale_dtype, scale_len, bias, bias_dtype,
+    return packed_forward_impl(who, X, x_dtype, W_tiled, W_LAYOUT_TILED, epi_op, scale, scale_dtype, scale_len, bias, bias_dtype,
                                residual, Y, B, N, K, workspace, workspace_bytes, stream);
 }
 

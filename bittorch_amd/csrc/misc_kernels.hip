@@ -188,12 +188,18 @@ __global__ __launch_bounds__(256) void unpack_dequant_kernel(const uint8_t* __re
 // ---- decode-tiled copy of the packed weights (W_LAYOUT_TILED) -----------------------------------
 // One thread per dword of the tiled copy: lane = 16 g + j of step s of tile t collects the bytes of
 // rows 16 s + 4 g .. + 3 of column 16 t + j.  The sixteen threads of a g read 16 contiguous bytes per row.
+// pairs (N % 32 == 0): tile 2P of the copy is tile P of the matrix, tile 2P + 1 is tile N/32 + P, so that
+// column h of the first half (gate) and column h of the second half (up) land in one workgroup.
+__device__ __forceinline__ int64_t source_tile(int64_t t, int64_t tiles, int pairs) {
+    return pairs ? ((t & 1) ? (tiles >> 1) + (t >> 1) : (t >> 1)) : t;
+}
+
 __global__ __launch_bounds__(256) void retile_kernel(const uint8_t* __restrict__ W_T, uint32_t* __restrict__ T,
-                                                     int64_t N, int64_t Kb, int64_t S, int64_t total) {
+                                                     int64_t N, int64_t Kb, int64_t S, int64_t total, int pairs) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
     const int lane = (int)(i & 63);
-    const int64_t s = (i >> 6) % S, t = (i >> 6) / S;
+    const int64_t s = (i >> 6) % S, t = source_tile((i >> 6) / S, total / (64 * S), pairs);
     const int64_t n = 16 * t + (lane & 15), kb0 = 16 * s + 4 * (lane >> 4);
     uint32_t d = 0;
     if (n < N) {
@@ -206,24 +212,29 @@ __global__ __launch_bounds__(256) void retile_kernel(const uint8_t* __restrict__
 
 // the inverse: one thread per byte of W_T
 __global__ __launch_bounds__(256) void untile_kernel(const uint32_t* __restrict__ T, uint8_t* __restrict__ W_T,
-                                                     int64_t N, int64_t Kb, int64_t S) {
+                                                     int64_t N, int64_t Kb, int64_t S, int pairs) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= N * Kb) return;
     const int64_t kb = i / N, n = i % N;
-    const int64_t idx = ((n >> 4) * S + (kb >> 4)) * 64 + 16 * ((kb & 15) >> 2) + (n & 15);
+    int64_t t = n >> 4;  // tile of the matrix -> tile of the copy
+    if (pairs) {
+        const int64_t half = N >> 5;
+        t = (t < half) ? 2 * t : 2 * (t - half) + 1;
+    }
+    const int64_t idx = (t * S + (kb >> 4)) * 64 + 16 * ((kb & 15) >> 2) + (n & 15);
     W_T[i] = (uint8_t)(T[idx] >> (8 * (kb & 3)));
 }
 
 // forward: W_T [Kb, N] -> T;  inverse: T -> W_out [Kb, N]
-int launch_retile(const uint8_t* W_T, int64_t N, int64_t K, void* T, bool inverse, uint8_t* W_out, hipStream_t st) {
+int launch_retile(const uint8_t* W_T, int64_t N, int64_t K, int pairs, void* T, bool inverse, uint8_t* W_out, hipStream_t st) {
     const int64_t Kb = ceil_div(K, 4), S = ceil_div(Kb, 16);
     if (!inverse) {
         const int64_t total = ceil_div(N, 16) * S * 64;
         hipLaunchKernelGGL(retile_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st, W_T, (uint32_t*)T, N, Kb, S,
-                           total);
+                           total, pairs);
     } else {
         hipLaunchKernelGGL(untile_kernel, dim3((unsigned)ceil_div(N * Kb, 256)), dim3(256), 0, st, (const uint32_t*)T, W_out,
-                           N, Kb, S);
+                           N, Kb, S, pairs);
     }
     return check_launch(inverse ? "untile" : "retile");
 }

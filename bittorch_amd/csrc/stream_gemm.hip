@@ -66,8 +66,11 @@ struct StreamParams {
     int pro_op;
     const void* pro_b;
     float pro_eps;
+    // Output stage (16-bit modes on tiled weights whose 16-column tiles alternate gate, up, gate, up ...):
+    //   EPI_SWIGLU_PAIRS  Y [M, N/2]:  Y[b, h] = rd(rd(silu(g)) * u),  g = rd(linear column h), u = rd(linear
+    //                     column N/2 + h): what the SwiGLU kernel would make of the stored projections
+    int epi_op;
 };
-enum { PRO_NONE = 0, PRO_RMSNORM = 1, PRO_SWIGLU = 2 };
 
 enum { LD_BYTE = 0, LD_Q1 = 1, LD_Q2 = 2, LD_V4 = 4, LD_V8 = 8, LD_V16 = 16, LD_T1 = 101, LD_T2 = 102, LD_T4 = 104 };
 constexpr int XC_MAX = 4;  // XLDS: 16-byte chunks of the x slice per lane
@@ -154,10 +157,18 @@ __device__ __forceinline__ uint32_t quad_transpose(uint32_t d, uint32_t sel_q) {
     return perm(t23, t01, 0x05040100u);
 }
 
+// The linear value of one output column before it is stored: the accumulator scaled, biased and
+// (16-bit modes) with the decode's factor undone.
+template <int MODE>
+__device__ __forceinline__ float linear_value(const StreamParams& p, uint32_t bits, float s, float b) {
+    if constexpr (MODE == MODE_F16) return epi_float(__builtin_bit_cast(float, bits), s, b);
+    else return epi_float(__builtin_bit_cast(float, bits) * (p.prehalved ? 1.0f : 0.5f), s, b);
+}
+
 // PRO: activation prologue compiled in (PRO_NONE for all but the M = 1 variants that are launched
 // with one: a run-time switch, even a uniform one, puts branches and waits around the loads of the
 // plain kernel).
-template <int MODE, int LD, int WAVES, int PF, bool XLDS, int PRO = 0>
+template <int MODE, int LD, int WAVES, int PF, bool XLDS, int PRO = 0, int EPI = 0>
 __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
     constexpr bool QUAD = (LD == LD_Q1 || LD == LD_Q2);
     constexpr bool BYTE = (LD == LD_BYTE);
@@ -221,7 +232,7 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
 
     // epilogue operands of this thread's output column, requested before the weight stream
     // so that their latency hides behind it (raw bits now, conversion after the reduction)
-    constexpr bool PRE = (WAVES * 64) % TILE_N == 0;  // a thread finishes one column only
+    constexpr bool PRE = (WAVES * 64) % TILE_N == 0 && EPI == EPI_NONE;  // a thread finishes one column only
     uint32_t pre_s = 0u, pre_b = 0u;
     if constexpr (PRE) {
         const int64_t n = nb + (int)(threadIdx.x % TILE_N);
@@ -479,6 +490,28 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
     }
     __syncthreads();
 
+    if constexpr (EPI == EPI_SWIGLU_PAIRS && TILED && (NACC % 2 == 0) && MODE != MODE_I8) {
+        // tiles 2P and 2P+1 of the tiled copy hold columns 16P.. of the gate half and of the up half
+        const int64_t ffn = p.N >> 1;
+        for (int idx = threadIdx.x; idx < M * (TILE_N / 2); idx += WAVES * 64) {
+            const int row = idx / (TILE_N / 2);
+            const int hl = idx % (TILE_N / 2);
+            const int64_t h = (int64_t)tile * (TILE_N / 2) + hl;
+            if (h >= ffn) continue;
+            const int slot_g = (hl >> 4) * 32 + (hl & 15), slot_u = slot_g + 16;
+            uint32_t bg = red[row * TILE_N + slot_g], bu = red[row * TILE_N + slot_u];
+#pragma unroll
+            for (int w = 1; w < WAVES; w++) {
+                bg = add_bits<MODE>(bg, red[(w * M + row) * TILE_N + slot_g]);
+                bu = add_bits<MODE>(bu, red[(w * M + row) * TILE_N + slot_u]);
+            }
+            const float g = round_to_dtype(linear_value<MODE>(p, bg, epi_scale(p.epi, h), epi_bias(p.epi, h)), p.y_dtype);
+            const float u = round_to_dtype(
+                linear_value<MODE>(p, bu, epi_scale(p.epi, ffn + h), epi_bias(p.epi, ffn + h)), p.y_dtype);
+            store_out(p.Y, p.y_dtype, (int64_t)row * ffn + h, swiglu_value(g, u, p.y_dtype));
+        }
+        return;
+    }
     for (int idx = threadIdx.x; idx < M * TILE_N; idx += WAVES * 64) {
         const int row = idx / TILE_N;
         const int nl = idx % TILE_N;
@@ -522,7 +555,7 @@ bool stream_supported(int64_t N, int64_t K, const void* W_T) {
 
 static int ld_columns(int ld) { return ld == LD_BYTE ? 16 : ld > 100 ? 16 * (ld - 100) : 16 * ld; }
 
-StreamPlan stream_plan(int mode, int64_t M, int64_t N, int64_t Kb, int w_layout) {
+StreamPlan stream_plan(int mode, int64_t M, int64_t N, int64_t Kb, int w_layout, int min_nacc = 1) {
     StreamPlan pl;
     (void)Kb;
     // optional override for tuning runs: BITTORCH_STREAM_CFG="ld,waves"
@@ -533,8 +566,9 @@ StreamPlan stream_plan(int mode, int64_t M, int64_t N, int64_t Kb, int w_layout)
         // 16-column tiles, up to four per workgroup (a batch re-reads its activations once per workgroup)
         const int min_tiles = (M > 4) ? 160 : 256;
         int nacc = 4;
-        while (nacc > 1 && ceil_div(N, 16 * nacc) < min_tiles) nacc >>= 1;
+        while (nacc > min_nacc && ceil_div(N, 16 * nacc) < min_tiles) nacc >>= 1;
         if (o_ld == LD_T1 || o_ld == LD_T2 || o_ld == LD_T4) nacc = o_ld - 100;
+        if (nacc < min_nacc) nacc = min_nacc;
         ld = 100 + nacc;
     } else if (N % 4 != 0) {
         ld = LD_BYTE;  // row starts are not dword aligned
@@ -563,6 +597,17 @@ size_t stream_workspace_bytes(int, int64_t, int64_t, int64_t) { return 0; }
 template <int MODE, int LD, int WAVES>
 static void launch_stream_k(const StreamParams& p, bool xlds, dim3 grid, size_t lds, hipStream_t st) {
     constexpr int PF = (LD == 16) ? 2 : (LD == 8) ? 4 : ((LD == 4 || LD == LD_T4) && MODE != MODE_I8) ? 4 : 8;
+    if constexpr ((LD == LD_T2 || LD == LD_T4) && MODE != MODE_I8) {
+        if (p.epi_op == EPI_SWIGLU_PAIRS) {
+            if (xlds && p.pro_op == PRO_RMSNORM)
+                hipLaunchKernelGGL((stream_kernel<MODE, LD, WAVES, PF, true, PRO_RMSNORM, EPI_SWIGLU_PAIRS>), grid, dim3(WAVES * 64), lds, st, p);
+            else if (xlds)
+                hipLaunchKernelGGL((stream_kernel<MODE, LD, WAVES, PF, true, PRO_NONE, EPI_SWIGLU_PAIRS>), grid, dim3(WAVES * 64), lds, st, p);
+            else
+                hipLaunchKernelGGL((stream_kernel<MODE, LD, WAVES, PF, false, PRO_NONE, EPI_SWIGLU_PAIRS>), grid, dim3(WAVES * 64), lds, st, p);
+            return;
+        }
+    }
     if constexpr (LD <= 4 || LD > 100) {  // decode-shape tiles: the M = 1 variant with x staged in LDS
         if (xlds) {
             if constexpr (MODE != MODE_I8) {
@@ -606,10 +651,12 @@ static bool xlds_ok(int es, int M, bool x_vec_ok, const StreamPlan& pl, int64_t 
 
 // Can the streaming kernel apply an RMSNorm / SwiGLU prologue to this call's activation row itself?
 // (one 16-bit row that takes the LDS-staged variant; BITTORCH_NO_PROLOGUE=1 says no, for A/B runs)
-bool stream_prologue_fusable(int mode, int64_t B, int64_t N, int64_t K, const void* X, const void* pro_b, int w_layout) {
+bool stream_prologue_fusable(int mode, int64_t B, int64_t N, int64_t K, const void* X, const void* pro_b, int w_layout,
+                             int epi_op) {
     if (mode == MODE_I8 || B != 1 || getenv("BITTORCH_NO_PROLOGUE")) return false;
     const bool vec = ((uintptr_t)X) % 16 == 0 && (!pro_b || ((uintptr_t)pro_b) % 16 == 0) && (K * 2) % 16 == 0;
-    return xlds_ok(2, 1, vec, stream_plan(mode, 1, N, ceil_div(K, 4), w_layout), K);
+    if (epi_op != EPI_NONE && mode == MODE_I8) return false;
+    return xlds_ok(2, 1, vec, stream_plan(mode, 1, N, ceil_div(K, 4), w_layout, epi_op == EPI_SWIGLU_PAIRS ? 2 : 1), K);
 }
 
 template <int MODE>
@@ -624,6 +671,12 @@ static int launch_stream_mode(StreamParams p, const StreamPlan& pl, hipStream_t 
     const size_t xs_bytes = (size_t)waves * XC_MAX * 64 * 16;
     const bool xlds = xlds_ok(es, p.M, p.x_vec_ok != 0, pl, p.K);
     const size_t lds = red_bytes + (xlds ? xs_bytes : 0);
+    if (p.epi_op == EPI_SWIGLU_PAIRS && (MODE == MODE_I8 || (pl.ld != LD_T2 && pl.ld != LD_T4) || p.N % 32 != 0 ||
+                                         p.pro_op == PRO_SWIGLU || p.epi.residual)) {
+        set_error("stream_gemm: the SwiGLU output stage needs 16-bit activations, pair-ordered tiled weights, N %% 32 == 0, "
+                  "no SwiGLU prologue and no residual");
+        return BT_ERR_INVALID;
+    }
     if (p.pro_op != PRO_NONE && !xlds) {
         set_error("stream_gemm: activation prologue on a shape the callers should have routed elsewhere");
         return BT_ERR_INVALID;
@@ -649,19 +702,21 @@ static int launch_stream_mode(StreamParams p, const StreamPlan& pl, hipStream_t 
 // w_layout: W_LAYOUT_ROW_MAJOR (the reference's W_T [Kb, N]) or W_LAYOUT_TILED (retile_kernel's copy)
 // q_layout: MODE_I8 only (Q_OPERAND_ORDER needs K % 16 == 0 and 16-byte aligned rows)
 // pro_op / pro_b / pro_eps: activation prologue (PRO_*), only where stream_prologue_fusable() said yes
+// epi_op: EPI_SWIGLU_PAIRS makes Y [B, N/2] (tiled weights in gate/up pair order, 16-bit modes)
 int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, const uint8_t* W_T, int w_layout,
                   const Epilogue& epi, void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N,
-                  int64_t K, int planes, int q_layout, int pro_op, const void* pro_b, float pro_eps, hipStream_t st) {
+                  int64_t K, int planes, int q_layout, int pro_op, const void* pro_b, float pro_eps, int epi_op, hipStream_t st) {
     const int64_t Kb = ceil_div(K, 4);
     const int64_t Kx = K * planes;
-    const StreamPlan pl = stream_plan(mode, B, N, Kb, w_layout);
+    const StreamPlan pl = stream_plan(mode, B, N, Kb, w_layout, epi_op == EPI_SWIGLU_PAIRS ? 2 : 1);
+    const int64_t Ny = (epi_op == EPI_SWIGLU_PAIRS) ? N / 2 : N;  // columns of Y
     const int y_size = dtype_size(y_dtype);
     for (int64_t m0 = 0; m0 < B; m0 += 16) {
         StreamParams p;
         p.X = (const uint8_t*)X + m0 * Kx * x_elem_size;
         p.W_T = W_T;
         p.s_x = s_x ? s_x + m0 : nullptr;
-        p.Y = (uint8_t*)Y + m0 * N * y_size;
+        p.Y = (uint8_t*)Y + m0 * Ny * y_size;
         p.acc_out = acc_out ? acc_out + m0 * N : nullptr;
         p.epi = epi;
         if (epi.residual) p.epi.residual = (const uint8_t*)epi.residual + m0 * N * y_size;
@@ -670,7 +725,7 @@ int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, co
         p.tiles16 = (int)ceil_div(N, 16);
         p.prehalved = planes == 3;
         p.x_operand_order = (mode == MODE_I8 && q_layout == Q_OPERAND_ORDER) ? 1 : 0;
-        p.pro_op = pro_op; p.pro_b = pro_b; p.pro_eps = pro_eps;
+        p.pro_op = pro_op; p.pro_b = pro_b; p.pro_eps = pro_eps; p.epi_op = epi_op;
         p.M = (int)((B - m0 < 16) ? (B - m0) : 16);
         p.y_dtype = y_dtype;
         p.x_vec_ok = (((uintptr_t)p.X) % 16 == 0) && ((Kx * x_elem_size) % 16 == 0);

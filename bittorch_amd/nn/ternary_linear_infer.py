@@ -43,6 +43,9 @@ class TernaryLinearInference(nn.Module):
         if decode_tiled is None:
             decode_tiled = os.environ.get("BITTORCH_DECODE_TILED", "1") != "0"
         self.decode_tiled = bool(decode_tiled)
+        # "natural", or "gate_up_pairs" for a fused [gate | up] layer whose decode calls go through
+        # forward_swiglu (set by TernarySwiGLU; such a copy serves only that output stage)
+        self.tile_order = "natural"
         self._tiled: Optional[Tensor] = None
         self._tiled_key = None
 
@@ -51,10 +54,10 @@ class TernaryLinearInference(nn.Module):
         """The decode-tiled copy of ``weight_packed`` (GPU only), built on first use and rebuilt when
         ``weight_packed`` has moved or been written since."""
         wp = self.weight_packed
-        key = (wp.data_ptr(), wp._version, wp.device)
+        key = (wp.data_ptr(), wp._version, wp.device, self.tile_order)
         if self._tiled is None or self._tiled_key != key:
             from .. import _C
-            self._tiled = _C.retile_weights(wp, self.in_features)
+            self._tiled = _C.retile_weights(wp, self.in_features, self.tile_order == "gate_up_pairs")
             self._tiled_key = key
         return self._tiled
 
@@ -65,8 +68,8 @@ class TernaryLinearInference(nn.Module):
             self.tiled_weights()
         return self
 
-    def _tiled_for(self, x: Tensor, rows: int) -> Optional[Tensor]:
-        if not (self.decode_tiled and x.is_cuda and rows <= DECODE_ROWS):
+    def _tiled_for(self, x: Tensor, rows: int, order: str = "natural") -> Optional[Tensor]:
+        if not (self.decode_tiled and x.is_cuda and rows <= DECODE_ROWS and self.tile_order == order):
             return None
         if os.environ.get("BITTORCH_KERNEL") == "generic":  # the shape-generic kernel reads weight_packed
             return None
@@ -75,7 +78,7 @@ class TernaryLinearInference(nn.Module):
         if x.dtype == torch.float32 and self.in_features % 64 != 0:
             return None
         wp = self.weight_packed
-        fresh = self._tiled is not None and self._tiled_key == (wp.data_ptr(), wp._version, wp.device)
+        fresh = self._tiled is not None and self._tiled_key == (wp.data_ptr(), wp._version, wp.device, self.tile_order)
         if not fresh and torch.cuda.is_current_stream_capturing():
             return None
         return self.tiled_weights()
@@ -109,6 +112,23 @@ class TernaryLinearInference(nn.Module):
         w = w * self.scale.unsqueeze(1).to(x.dtype)
         y = F.linear(x, w, self.bias)
         return y if residual is None else y + residual
+
+    def forward_swiglu(self, x: Tensor, norm=None) -> Tensor:
+        """For a layer whose columns are ``[gate | up]``: ``swiglu(gate(h), up(h))`` ``(*, N/2)`` with ``h = x`` or
+        ``rmsnorm(x, *norm)``.  Decode-shape calls on a layer with ``tile_order == "gate_up_pairs"`` form the product
+        in the output stage of the GEMV kernel; everything else runs the projection and the SwiGLU kernel."""
+        if x.is_cuda:
+            tiled = self._tiled_for(x, x.numel() // max(x.shape[-1], 1), "gate_up_pairs")
+            if tiled is not None and x.dtype in (torch.float16, torch.bfloat16):
+                from .. import _C
+                return _C.ternary_linear_tiled_forward(x, tiled, self.scale, self.bias, self.in_features,
+                                                       self.out_features, None, norm, None, True)
+        gu = self.forward(x, None, norm)
+        half = self.out_features // 2
+        if x.is_cuda:
+            from ..ops import fused
+            return fused.swiglu(gu[..., :half], gu[..., half:])
+        return F.silu(gu[..., :half]) * gu[..., half:]
 
     def forward_int8(self, q: Tensor, s_x: Tensor, out_dtype: torch.dtype = torch.bfloat16,
                      residual: Optional[Tensor] = None, q_operand_order: bool = False) -> Tensor:

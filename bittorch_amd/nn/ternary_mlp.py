@@ -37,6 +37,9 @@ class TernarySwiGLU(nn.Module):
             from ..utils.convert import fuse_ternary_linear_inference
             self.gate_up = fuse_ternary_linear_inference(gate, up)
             self.gate = self.up = None
+            if compute == "float" and self.ffn % 16 == 0:
+                # decode-shape calls: the SwiGLU product leaves the gate|up GEMV's own output stage
+                self.gate_up.tile_order = "gate_up_pairs"
         else:
             self.gate_up = None
             self.gate, self.up = gate, up
@@ -67,7 +70,10 @@ class TernarySwiGLU(nn.Module):
         if self.compute == "float":
             # norm and SwiGLU ride on the projections that consume them (for one decode token they run
             # inside the GEMV kernels; otherwise as one fused kernel each ahead of the GEMM)
-            g, u = self._gate_up(x, None if eps is None else (norm_weight, eps))
+            norm = None if eps is None else (norm_weight, eps)
+            if self.gate_up is not None and self.gate_up.tile_order == "gate_up_pairs":
+                return self.down(self.gate_up.forward_swiglu(x, norm), residual)
+            g, u = self._gate_up(x, norm)
             return self.down(g, residual, None, u)
         # the int8 activations stay inside this call: hand them over in the matrix cores' own order
         oo1, oo2 = x.shape[-1] % 16 == 0, self.ffn % 16 == 0

@@ -218,19 +218,28 @@ int bt_ternary_linear_packed_forward_fused(const void* X, int64_t ld_x, int x_dt
  * low byte first (= 16 consecutive k of one output column), zero outside the matrix.  It is built
  * once from W_T (bt_retile_weights, exact inverse bt_untile_weights) and holds
  * bt_tiled_weights_bytes(N, K) = ceil(N/16) * S * 256 bytes, 256-byte aligned, below 4 GiB.
+ *   order: BT_TILES_NATURAL, or BT_TILES_GATE_UP_PAIRS (N % 32 == 0) for a layer whose columns are
+ *     [gate | up] of a SwiGLU MLP: tile 2P of the copy is tile P of the matrix, tile 2P + 1 is tile
+ *     N/32 + P, so that one workgroup holds column h of both halves.
  *   bt_ternary_linear_tiled_forward: bt_ternary_linear_packed_forward_fused on the tiled copy, with
  *     pro_op = BT_PRO_NONE allowed (then ld_x must equal K); the weights are streamed once per 16
  *     rows of X, so it is meant for decode shapes; fp32 X needs K % 64 == 0 and the workspace.
  *     Results equal those of the row-major entry points bit for bit.
+ *     epi_op = BT_EPI_SWIGLU_PAIRS (pair-ordered copy, no residual, no SwiGLU prologue): Y is [B, N/2],
+ *     Y[b, h] = what bt_swiglu makes of the stored projections, rd(rd(silu(g)) * u) with g = rd(linear
+ *     column h), u = rd(linear column N/2 + h): the SwiGLU MLP's hidden vector leaves the gate|up kernel
+ *     itself (structure: TernaryTransformer.ts:366-423).  A pair-ordered copy serves only this output stage.
  *   bt_ternary_gemm_i8_tiled: bt_ternary_gemm_i8_res on the tiled copy (same remark).
  */
+enum { BT_TILES_NATURAL = 0, BT_TILES_GATE_UP_PAIRS = 1 };
+enum { BT_EPI_NONE = 0, BT_EPI_SWIGLU_PAIRS = 1 };
 size_t bt_tiled_weights_bytes(int64_t N, int64_t K);
-int bt_retile_weights(const uint8_t* W_T, int64_t N, int64_t K, uint8_t* W_tiled, void* stream);
-int bt_untile_weights(const uint8_t* W_tiled, int64_t N, int64_t K, uint8_t* W_T, void* stream);
+int bt_retile_weights(const uint8_t* W_T, int64_t N, int64_t K, int order, uint8_t* W_tiled, void* stream);
+int bt_untile_weights(const uint8_t* W_tiled, int64_t N, int64_t K, int order, uint8_t* W_T, void* stream);
 int bt_ternary_linear_tiled_forward(const void* X, int64_t ld_x, int x_dtype, int pro_op, const void* pro_b,
                                     int64_t ld_b, float eps, const uint8_t* W_tiled, const void* scale,
                                     int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
-                                    const void* residual, void* Y, int64_t B, int64_t N, int64_t K,
+                                    const void* residual, int epi_op, void* Y, int64_t B, int64_t N, int64_t K,
                                     void* workspace, size_t workspace_bytes, void* stream);
 int bt_ternary_gemm_i8_tiled(const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_tiled,
                              const void* scale, int scale_dtype, int64_t scale_len, const void* bias,

@@ -129,17 +129,22 @@ def unpack_ternary_transposed(packed_t, in_features: int) -> np.ndarray:
     return out
 
 
-def retile_weights(packed_t, in_features: int) -> np.ndarray:
+def retile_weights(packed_t, in_features: int, gate_up_pairs: bool = False) -> np.ndarray:
     """Decode-tiled copy of ``W_T [Kb, N]`` (a layout of this library, no counterpart in the reference):
     zero-pad to whole 16-row steps and 16-column tiles, then order the bytes as
-    ``[tile t][step s][row group g][column j][row r]`` with ``kb = 16 s + 4 g + r``, ``n = 16 t + j``."""
+    ``[tile t][step s][row group g][column j][row r]`` with ``kb = 16 s + 4 g + r``, ``n = 16 t + j``.
+    ``gate_up_pairs`` (N % 32 == 0): the tiles of the first and of the second column half alternate."""
     w = np.ascontiguousarray(packed_t, dtype=np.uint8)
     kb, n = w.shape
     assert kb == (in_features + 3) // 4
     steps, tiles = (kb + 15) // 16, (n + 15) // 16
     padded = np.zeros((steps * 16, tiles * 16), dtype=np.uint8)
     padded[:kb, :n] = w
-    return np.ascontiguousarray(padded.reshape(steps, 4, 4, tiles, 16).transpose(3, 0, 1, 4, 2)).reshape(-1)
+    tiled = np.ascontiguousarray(padded.reshape(steps, 4, 4, tiles, 16).transpose(3, 0, 1, 4, 2))
+    if gate_up_pairs:
+        assert n % 32 == 0
+        tiled = np.ascontiguousarray(tiled.reshape(2, tiles // 2, steps, 4, 16, 4).transpose(1, 0, 2, 3, 4, 5))
+    return tiled.reshape(-1)
 
 
 def _lin_args(x, w, scale, bias):

@@ -211,3 +211,67 @@ def test_module_never_builds_the_copy_inside_a_capture(oracle):
     assert torch.equal(y, ref)
     a.prepare_decode()
     assert a._tiled is not None and torch.equal(a(x), ref)
+
+
+@pytest.mark.parametrize("n,k", [(64, 64), (96, 100), (13824, 2560), (32, 4)])
+def test_retile_gate_up_pair_order(oracle, n, k):
+    from bittorch_amd import _C
+    announce("retile pairs", n, k)
+    _, wt = _packed(oracle, n, k, seed=n + k)
+    tiled = _C.retile_weights(wt, k, True)
+    np.testing.assert_array_equal(tiled.cpu().numpy(), oracle.retile_weights(wt.cpu().numpy(), k, True))
+    assert torch.equal(_C.untile_weights(tiled, n, k, True), wt)
+    with pytest.raises(RuntimeError, match="N % 32"):
+        _C.retile_weights(wt[:, :n - 16].contiguous(), k, True)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n,k", [(13824, 2560), (64, 64), (96, 100), (8192, 4096), (320, 1030)])
+def test_swiglu_output_stage_equals_projection_then_swiglu(oracle, dtype, n, k):
+    """Y = swiglu(gate(x), up(x)) from the GEMV's output stage against the stored projections fed to the
+    SwiGLU kernel (which the fused-glue tests hold against the oracle bit for bit)."""
+    from bittorch_amd import _C
+    _, wt = _packed(oracle, n, k, seed=7)
+    tiled = _C.retile_weights(wt, k, True)
+    g = torch.Generator().manual_seed(n)
+    scale = (torch.rand(n, generator=g) + 0.5).cuda() * 0.05
+    bias = (torch.randn(n, generator=g) * 0.1).to(dtype).cuda()
+    nw = (torch.rand(k, generator=g) + 0.5).to(dtype).cuda()
+    for b in (1, 3, 16, 20):
+        x = seeded_acts(b, k, seed=b, dtype=dtype).cuda()
+        for norm in (None, (nw, 1e-5)):
+            for bs in (None, bias):
+                announce("swiglu stage", dtype, n, k, b, norm is not None, bs is not None)
+                if norm is None:
+                    gu = _C.ternary_linear_packed_forward(x, wt, scale, bs, k)
+                else:
+                    gu = _C.ternary_linear_packed_forward_fused(x, wt, scale, bs, k, norm=norm)
+                ref = _C.swiglu(gu[:, :n // 2], gu[:, n // 2:])
+                got = _C.ternary_linear_tiled_forward(x, tiled, scale, bs, k, n, None, norm, None, True)
+                assert got.shape == (b, n // 2)
+                assert torch.equal(got, ref)
+    x = seeded_acts(1, k, dtype=dtype).cuda()
+    with pytest.raises(RuntimeError):
+        _C.ternary_linear_tiled_forward(x, tiled, scale, None, k, n, torch.zeros(1, n, dtype=dtype).cuda(), None, None, True)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_ternary_swiglu_decode_uses_the_output_stage(oracle, dtype):
+    from bittorch_amd.nn import TernarySwiGLU
+    d, ffn = 256, 704
+    gate, up, down = _layer(oracle, ffn, d, seed=1), _layer(oracle, ffn, d, seed=2), _layer(oracle, d, ffn, seed=3)
+    for L in (gate, up, down):
+        L.scale.mul_(0.05)
+    fused = TernarySwiGLU(gate, up, down, compute="float", fuse_gate_up=True)
+    assert fused.gate_up.tile_order == "gate_up_pairs"
+    plain = TernarySwiGLU(gate, up, down, compute="float", fuse_gate_up=False)
+    nw = (torch.rand(d) + 0.5).to(dtype).cuda()
+    for rows in (1, 5, 40):
+        announce("TernarySwiGLU decode", dtype, rows)
+        x = seeded_acts(rows, d, seed=rows, dtype=dtype).cuda()
+        assert torch.equal(fused(x, nw, 1e-5, residual=x), plain(x, nw, 1e-5, residual=x))
+        assert torch.equal(fused(x), plain(x))
+    assert fused.gate_up._tiled is not None
+    # the fused layer called as an ordinary linear layer still gives [gate | up] in natural order
+    x = seeded_acts(1, d, dtype=dtype).cuda()
+    assert torch.equal(fused.gate_up(x), torch.cat([gate(x), up(x)], dim=-1))
