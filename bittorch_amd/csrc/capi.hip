@@ -53,8 +53,9 @@ int launch_row_op(int op, int dtype, const void* A, int64_t lda, const void* Bv,
 bool gemm_f16_supported(int64_t N, int64_t K, const void* X, const void* W_T, const void* Y);
 int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, const Epilogue& epi, void* Y, int y_dtype, int64_t M,
                     int64_t N, int64_t K, int planes, hipStream_t st);
-int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_T, const Epilogue& epi, void* Y,
-                   int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st);
+bool gemm_i8_supported_tiled(int64_t N, int64_t K, const void* Q);
+int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_T, int w_layout, const Epilogue& epi,
+                   void* Y, int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st);
 
 static bool valid_dtype(int dt) { return dt == BT_F32 || dt == BT_F16 || dt == BT_BF16; }
 
@@ -315,6 +316,8 @@ static int gemm_i8_impl(const char* who, const int8_t* Q, int q_layout, const fl
             set_error("%s: tiled weights must be 256-byte aligned and below 4 GiB", who);
             return BT_ERR_INVALID;
         }
+        if (B > kStreamMaxRows && gemm_i8_supported_tiled(N, K, Q))
+            return launch_gemm_i8(Q, q_layout, s_x, W_T, W_LAYOUT_TILED, epi, Y, y_dtype, acc_out, B, N, K, st);
         return launch_stream(MODE_I8, Q, 1, s_x, W_T, w_layout, epi, Y, y_dtype, acc_out, B, N, K, 1, q_layout, 0, nullptr,
                              0.0f, 0, st);
     }
@@ -328,7 +331,7 @@ static int gemm_i8_impl(const char* who, const int8_t* Q, int q_layout, const fl
         }
         return launch_stream(MODE_I8, Q, 1, s_x, W_T, w_layout, epi, Y, y_dtype, acc_out, B, N, K, 1, q_layout, 0, nullptr, 0.0f, 0, st);
     }
-    return launch_gemm_i8(Q, q_layout, s_x, W_T, epi, Y, y_dtype, acc_out, B, N, K, st);
+    return launch_gemm_i8(Q, q_layout, s_x, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, y_dtype, acc_out, B, N, K, st);
 }
 
 extern "C" int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const void* scale,

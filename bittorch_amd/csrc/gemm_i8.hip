@@ -45,6 +45,7 @@ struct GemmParams {
     int y_dtype;
     int tiles_m, tiles_n;
     int per_xcd;          // workgroups per XCD (grid = 8 * per_xcd)
+    int wsteps, tiles16;  // WT: 16-row steps and 16-column tiles of the decode-tiled weight copy
 };
 
 __device__ __forceinline__ void store4(void* Y, int dt, int64_t idx, const float (&v)[4]) {
@@ -134,7 +135,9 @@ __device__ __forceinline__ void gemm_epilogue_dt(const GemmParams& p, const v4i 
 // workgroup finishes 64 of the 128 rows.
 // QOO = true: Q is in operand order (16-byte groups already transposed by the quantizer), and
 // the staging copies them to LDS untouched.
-template <bool TAIL, bool QOO>
+// WT = true: W_T is the decode-tiled copy (W_LAYOUT_TILED): the four dwords a lane decodes per stage
+// (16 consecutive k of its four columns) are 16 contiguous bytes there, one load and no transpose.
+template <bool TAIL, bool QOO, bool WT = false>
 __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[65536];  // 2 A stages; reused for the K-half exchange
 
@@ -175,7 +178,13 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     const int64_t rows_left = p.M - m0;
     const uint32_t a_row_c = (uint32_t)((a_row < rows_left) ? a_row : rows_left - 1);
     const uint32_t a_off = a_row_c * (uint32_t)p.K + 32u * a_part;
-    const uint32_t b_off = (uint32_t)(col_ok ? ncol : 0) + (uint32_t)(16 * kgrp + 4 * g) * (uint32_t)p.N;
+    uint32_t b_off;
+    if constexpr (WT) {
+        const int tt = min((int)(ncol >> 4), p.tiles16 - 1);  // a tile past the end only feeds outputs never stored
+        b_off = ((uint32_t)tt * (uint32_t)p.wsteps * 64u + (uint32_t)(16 * g + 4 * (j & 3))) * 4u;
+    } else {
+        b_off = (uint32_t)(col_ok ? ncol : 0) + (uint32_t)(16 * kgrp + 4 * g) * (uint32_t)p.N;
+    }
     const int8_t* a_base = p.Q + m0 * p.K;  // uniform
     const uint8_t* b_base = p.W_T;          // uniform
     const int64_t N = p.N;
@@ -194,9 +203,15 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
             a_reg[1] = *(const uint4*)(ab + 16 + a_off);
         }
         if (part & 2) {
-            const uint8_t* bb = b_base + (k0 >> 2) * N;
+            if constexpr (WT) {
+                const int step = min((int)(k0 >> 6) + kgrp, p.wsteps - 1);  // uniform per wave
+                const uint4 v = *(const uint4*)(b_base + (size_t)step * 256 + b_off);
+                b_reg[0] = v.x; b_reg[1] = v.y; b_reg[2] = v.z; b_reg[3] = v.w;
+            } else {
+                const uint8_t* bb = b_base + (k0 >> 2) * N;
 #pragma unroll
-            for (int r = 0; r < 4; r++) b_reg[r] = *(const uint32_t*)(bb + r * N + b_off);
+                for (int r = 0; r < 4; r++) b_reg[r] = *(const uint32_t*)(bb + r * N + b_off);
+            }
         }
     };
     auto load_tail = [&](int64_t k0, int part, uint4 (&a_reg)[2], uint32_t (&b_reg)[4]) {
@@ -211,7 +226,13 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
                 a_reg[c] = make_uint4(v.x & m, v.y & m, v.z & m, v.w & m);
             }
         }
-        if (part & 2) {
+        if constexpr (WT) {
+            if (part & 2) {  // the copy is zero-padded to whole steps; a step past the end meets zeroed activations
+                const int step = min((int)(k0 >> 6) + kgrp, p.wsteps - 1);
+                const uint4 v = *(const uint4*)(b_base + (size_t)step * 256 + b_off);
+                b_reg[0] = v.x; b_reg[1] = v.y; b_reg[2] = v.z; b_reg[3] = v.w;
+            }
+        } else if (part & 2) {
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 int64_t kb = (k0 >> 2) + 16 * kgrp + r + 4 * g;
@@ -271,7 +292,8 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     const uint32_t a_lds_off = (uint32_t)(kgrp * (G_MB * 1024)) + ((uint32_t)lane << 4);
     auto decode_b = [&](const uint32_t (&raw)[4], v4i (&out)[4]) {
         uint32_t G[4];
-        transpose4x4_bytes(raw[0], raw[1], raw[2], raw[3], G);
+        if constexpr (WT) { G[0] = raw[0]; G[1] = raw[1]; G[2] = raw[2]; G[3] = raw[3]; }
+        else transpose4x4_bytes(raw[0], raw[1], raw[2], raw[3], G);
 #pragma unroll
         for (int t = 0; t < 4; t++) out[t] = decode16_i8(G[t]);
     };
@@ -315,16 +337,22 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
         auto partC = [&](int t) { out[t][3] = (int)perm(lutB_hi, lutB_lo, d_H[t] & 0x0C0C0C0Cu); };
         switch (c) {
             case 4:
-                d_t[0] = perm(raw[1], raw[0], 0x05010400u);
-                d_t[1] = perm(raw[1], raw[0], 0x07030602u);
-                d_t[2] = perm(raw[3], raw[2], 0x05010400u);
-                d_t[3] = perm(raw[3], raw[2], 0x07030602u);
+                if constexpr (!WT) {
+                    d_t[0] = perm(raw[1], raw[0], 0x05010400u);
+                    d_t[1] = perm(raw[1], raw[0], 0x07030602u);
+                    d_t[2] = perm(raw[3], raw[2], 0x05010400u);
+                    d_t[3] = perm(raw[3], raw[2], 0x07030602u);
+                }
                 break;
             case 5:
-                d_G[0] = perm(d_t[2], d_t[0], 0x05040100u);
-                d_G[1] = perm(d_t[2], d_t[0], 0x07060302u);
-                d_G[2] = perm(d_t[3], d_t[1], 0x05040100u);
-                d_G[3] = perm(d_t[3], d_t[1], 0x07060302u);
+                if constexpr (WT) {
+                    d_G[0] = raw[0]; d_G[1] = raw[1]; d_G[2] = raw[2]; d_G[3] = raw[3];
+                } else {
+                    d_G[0] = perm(d_t[2], d_t[0], 0x05040100u);
+                    d_G[1] = perm(d_t[2], d_t[0], 0x07060302u);
+                    d_G[2] = perm(d_t[3], d_t[1], 0x05040100u);
+                    d_G[3] = perm(d_t[3], d_t[1], 0x07060302u);
+                }
                 break;
             case 6: partA(0); break;
             case 7: partB(0); break;
@@ -417,6 +445,11 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     else gemm_epilogue_dt<4>(p, acc, m0, g, ncol, epi_ops);
 }
 
+// the same kernel on the decode-tiled weight copy (256-byte aligned, below 4 GiB: checked by the caller)
+bool gemm_i8_supported_tiled(int64_t N, int64_t K, const void* Q) {
+    return N % 4 == 0 && K % 16 == 0 && ((uintptr_t)Q) % 16 == 0 && (G_BM + 1) * K < (1ll << 32);
+}
+
 // the tiled kernel reads Q with 16-byte loads and W_T / Y with 4-column vectors
 bool gemm_i8_supported(int64_t N, int64_t K, const void* Q, const void* W_T) {
     // 32-bit per-lane offsets: a row tile of Q and the whole of W_T stay below 4 GiB
@@ -424,8 +457,8 @@ bool gemm_i8_supported(int64_t N, int64_t K, const void* Q, const void* W_T) {
            (G_BM + 1) * K < (1ll << 32) && ceil_div(K, 4) * N < (1ll << 32);
 }
 
-int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_T, const Epilogue& epi, void* Y,
-                   int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st) {
+int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_T, int w_layout, const Epilogue& epi,
+                   void* Y, int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st) {
     GemmParams p;
     p.Q = Q; p.s_x = s_x; p.W_T = W_T; p.Y = Y; p.acc_out = acc_out; p.epi = epi;
     p.M = M; p.N = N; p.K = K; p.Kb = ceil_div(K, 4);
@@ -435,7 +468,19 @@ int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_
     const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
     p.per_xcd = (int)ceil_div(total, 8);
     const dim3 grid((unsigned)(p.per_xcd * 8)), block(512);
+    p.wsteps = (int)ceil_div(p.Kb, 16);
+    p.tiles16 = (int)ceil_div(N, 16);
     const bool qoo = q_layout == Q_OPERAND_ORDER;
+    if (w_layout == W_LAYOUT_TILED) {
+        if (K % G_BK == 0) {
+            if (qoo) hipLaunchKernelGGL((gemm_i8_kernel<false, true, true>), grid, block, 0, st, p);
+            else hipLaunchKernelGGL((gemm_i8_kernel<false, false, true>), grid, block, 0, st, p);
+        } else {
+            if (qoo) hipLaunchKernelGGL((gemm_i8_kernel<true, true, true>), grid, block, 0, st, p);
+            else hipLaunchKernelGGL((gemm_i8_kernel<true, false, true>), grid, block, 0, st, p);
+        }
+        return check_launch("bt_ternary_gemm_i8");
+    }
     if (K % G_BK == 0) {
         if (qoo) hipLaunchKernelGGL((gemm_i8_kernel<false, true>), grid, block, 0, st, p);
         else hipLaunchKernelGGL((gemm_i8_kernel<false, false>), grid, block, 0, st, p);

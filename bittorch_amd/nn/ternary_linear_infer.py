@@ -9,7 +9,9 @@ Decode-shape calls on the GPU (up to ``DECODE_ROWS`` rows) read a second, *decod
 the packed weights that the layer builds from ``weight_packed`` on first use (same size, not part
 of the ``state_dict``; same results bit for bit, 15-25 % less time per GEMV because every load of
 the kernel then covers whole cache lines).  ``decode_tiled=False`` or ``BITTORCH_DECODE_TILED=0``
-keeps the layer on ``weight_packed`` alone.
+keeps the layer on ``weight_packed`` alone.  ``forward_int8`` reads the copy at every batch size (the
+int8 prefill GEMM loads it with one 16-byte load per lane and stage instead of four dword loads and a
+byte transpose).
 """
 
 from __future__ import annotations
@@ -61,6 +63,13 @@ class TernaryLinearInference(nn.Module):
             self._tiled_key = key
         return self._tiled
 
+    def __getstate__(self):
+        # the tiled copy is derived data: rebuilt on demand, never pickled or deep-copied
+        state = super().__getstate__() if hasattr(super(), "__getstate__") else self.__dict__.copy()
+        state = dict(state)
+        state["_tiled"], state["_tiled_key"] = None, None
+        return state
+
     def prepare_decode(self) -> "TernaryLinearInference":
         """Build the decode-tiled copy now (e.g. before capturing decode steps into a HIP graph: a
         capture never builds it, it falls back to ``weight_packed``)."""
@@ -69,7 +78,9 @@ class TernaryLinearInference(nn.Module):
         return self
 
     def _tiled_for(self, x: Tensor, rows: int, order: str = "natural") -> Optional[Tensor]:
-        if not (self.decode_tiled and x.is_cuda and rows <= DECODE_ROWS and self.tile_order == order):
+        # (int8 activations: the tiled GEMM reads the copy too, so every batch size takes it)
+        if not (self.decode_tiled and x.is_cuda and (rows <= DECODE_ROWS or x.dtype == torch.int8)
+                and self.tile_order == order):
             return None
         if os.environ.get("BITTORCH_KERNEL") == "generic":  # the shape-generic kernel reads weight_packed
             return None

@@ -109,14 +109,14 @@ def test_tiled_prologues_equal_row_major(oracle, dtype, n, k):
             assert torch.equal(got, ref)
 
 
-@pytest.mark.parametrize("n,k", [(4096, 4096), (11008, 4096), (4096, 11008), (100, 64), (37, 100)])
+@pytest.mark.parametrize("n,k", [(4096, 4096), (11008, 4096), (4096, 11008), (100, 64), (37, 100), (260, 192), (520, 1040)])
 def test_tiled_int8_equals_row_major(oracle, n, k):
     from bittorch_amd import _C
     _, wt = _packed(oracle, n, k, seed=4)
     tiled = _C.retile_weights(wt, k)
     scale = (torch.rand(n) + 0.5).cuda()
     bias = (torch.randn(n) * 0.01).cuda()
-    for b in (1, 16, 33):
+    for b in (1, 16, 33, 200):  # up to 32 rows the streaming kernel, beyond it the tiled GEMM
         for oo in ((False, True) if k % 16 == 0 else (False,)):
             announce("tiled int8", n, k, b, oo)
             x = seeded_acts(b, k, seed=b, dtype=torch.bfloat16, outliers=True).cuda()
