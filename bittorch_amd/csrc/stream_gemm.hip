@@ -261,42 +261,8 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
             }
         }
     }
-    // RMSNorm prologue: the row's sum of squares, by the whole workgroup (the row is a few KiB and hot
-    // in cache), accumulated in fp64 so that its fp32 value does not depend on the summation order
-    float rstd = 1.0f;
-    if constexpr (XLDS && MODE != MODE_I8 && PRO == PRO_RMSNORM) {
-        {
-            double ss = 0.0;
-            for (int k = (int)threadIdx.x * 8; k < (int)p.K; k += WAVES * 64 * 8) {
-                const uint4 v = *(const uint4*)((const uint16_t*)p.X + k);  // K % 8 == 0, aligned (XLDS)
-                const uint32_t d[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const uint16_t h = (uint16_t)(d[e >> 1] >> (16 * (e & 1)));
-                    const double x = (double)(MODE == MODE_F16 ? f16_bits_to_f32(h) : bf16_bits_to_f32(h));
-                    ss += x * x;
-                }
-            }
-            ss = wave_sum_f64(ss);
-            double* part = (double*)red;  // the reduction buffer is free until the main loop is over
-            if (lane == 0) part[wave] = ss;
-            __syncthreads();
-            ss = 0.0;
-            for (int w = 0; w < WAVES; w++) ss += part[w];
-            __syncthreads();
-            rstd = rms_rstd(ss, (int)p.K, p.pro_eps);
-        }
-    }
-
-    acc_t acc[NACC], acc2[NACC2];
-#pragma unroll
-    for (int t = 0; t < NACC; t++) acc[t] = acc_t{0, 0, 0, 0};
-#pragma unroll
-    for (int t = 0; t < NACC2; t++) acc2[t] = acc_t{0, 0, 0, 0};
-
-    for (int base = s_begin; base < s_end; base += PF, k0 += PF * 64) {
-        uint32_t raw[PF][RAWN];
-        uint4 xa[PF][XN];
+    // the weight loads of the PF steps from `base` on
+    auto load_weights = [&](int base, uint32_t (&raw)[PF][RAWN]) {
 #pragma unroll
         for (int f = 0; f < PF; f++) {
             // weight step of activation step base+f (uniform): the activation row may hold several
@@ -326,6 +292,123 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
                 }
             }
         }
+    };
+    // RMSNorm prologue: the row's sum of squares, by the whole workgroup (the row is a few KiB and hot
+    // in cache), accumulated in fp64 so that its fp32 value does not depend on the summation order.
+    // Its loads are requested first, then the first batch of weights, and only then is the sum formed:
+    // the reduction and its two barriers run while the weights are on their way.
+    constexpr bool PRELOAD = XLDS && MODE != MODE_I8 && PRO == PRO_RMSNORM;
+    constexpr int PVN = 4;  // 16-byte pieces of the row per thread (the LDS-staged variant's K limit / 8 / threads)
+    uint4 pv[PRELOAD ? PVN : 1];
+    if constexpr (PRELOAD) {
+#pragma unroll
+        for (int u = 0; u < PVN; u++) {
+            if (u * WAVES * 64 * 8 < (int)p.K) {  // uniform
+                const int k = ((int)threadIdx.x + u * WAVES * 64) * 8;
+                pv[u] = *(const uint4*)((const uint16_t*)p.X + min(k, (int)p.K - 8));  // K % 8 == 0, aligned (XLDS)
+            }
+        }
+    }
+    uint32_t raw0[PRELOAD ? PF : 1][PRELOAD ? RAWN : 1];
+    if constexpr (PRELOAD) load_weights(s_begin, raw0);
+    float rstd = 1.0f;
+    if constexpr (PRELOAD) {
+        double ss = 0.0;
+#pragma unroll
+        for (int u = 0; u < PVN; u++) {
+            const int k = ((int)threadIdx.x + u * WAVES * 64) * 8;
+            if (u * WAVES * 64 * 8 < (int)p.K && k < (int)p.K) {
+                const uint32_t d[4] = {pv[u].x, pv[u].y, pv[u].z, pv[u].w};
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const uint16_t h = (uint16_t)(d[e >> 1] >> (16 * (e & 1)));
+                    const double x = (double)(MODE == MODE_F16 ? f16_bits_to_f32(h) : bf16_bits_to_f32(h));
+                    ss += x * x;
+                }
+            }
+        }
+        ss = wave_sum_f64(ss);
+        double* part = (double*)red;  // the reduction buffer is free until the main loop is over
+        if (lane == 0) part[wave] = ss;
+        __syncthreads();
+        ss = 0.0;
+        for (int w = 0; w < WAVES; w++) ss += part[w];
+        __syncthreads();
+        rstd = rms_rstd(ss, (int)p.K, p.pro_eps);
+    }
+
+    // XLDS: park the wave's x slice in LDS (transformed by the prologue) once its loads have landed
+    auto park_x = [&]() {
+        constexpr int EPC = 16 / ES;
+#pragma unroll
+        for (int u = 0; u < XC_MAX; u++) {
+            if (u * 64 < nchunks) {
+                const int k = s_begin * 64 + (lane + 64 * u) * EPC;
+                // parked in the order the MFMA wants (each 16-byte chunk is one operand
+                // fragment), so that the steps below read their A operand ready-made
+                uint4 v = zero_unless(xr[u], k < (int)p.K);
+                if constexpr (MODE != MODE_I8 && PRO != 0) {
+                    {
+                        constexpr int DT = (MODE == MODE_F16) ? BT_F16 : BT_BF16;
+                        const uint32_t a[4] = {v.x, v.y, v.z, v.w};
+                        const uint32_t bq[4] = {xb[u].x, xb[u].y, xb[u].z, xb[u].w};
+                        uint32_t r[4];
+#pragma unroll
+                        for (int d = 0; d < 4; d++) {
+                            uint32_t out = 0;
+#pragma unroll
+                            for (int e = 0; e < 2; e++) {
+                                const uint16_t ha = (uint16_t)(a[d] >> (16 * e)), hb = (uint16_t)(bq[d] >> (16 * e));
+                                const float fa = (DT == BT_F16) ? f16_bits_to_f32(ha) : bf16_bits_to_f32(ha);
+                                const float fb = (DT == BT_F16) ? f16_bits_to_f32(hb) : bf16_bits_to_f32(hb);
+                                float y;
+                                if constexpr (PRO == PRO_SWIGLU) y = swiglu_value(fa, fb, DT);
+                                else y = rmsnorm_value(fa, rstd, p.pro_b ? fb : 1.0f, DT);
+                                const uint32_t hy = (DT == BT_F16) ? f32_to_f16_bits(y) : f32_to_bf16_bits(y);
+                                out |= hy << (16 * e);
+                            }
+                            r[d] = out;
+                        }
+                        v = zero_unless(make_uint4(r[0], r[1], r[2], r[3]), k < (int)p.K);
+                    }
+                }
+                uint4 o;
+                if constexpr (MODE == MODE_I8) {
+                    uint32_t t4[4] = {v.x, v.y, v.z, v.w};
+                    if (!p.x_operand_order) transpose4x4_bytes(v.x, v.y, v.z, v.w, t4);  // uniform
+                    o = make_uint4(t4[0], t4[1], t4[2], t4[3]);
+                } else {
+                    o = make_uint4(perm(v.z, v.x, 0x05040100u), perm(v.z, v.x, 0x07060302u),
+                                   perm(v.w, v.y, 0x05040100u), perm(v.w, v.y, 0x07060302u));
+                }
+                *(uint4*)(xs + (lane + 64 * u) * 16) = o;
+            }
+        }
+    };
+    // with the prologue's reduction ahead of it, the slice is parked while the first weight batch is still on its way
+    if constexpr (PRELOAD) park_x();
+
+    acc_t acc[NACC], acc2[NACC2];
+#pragma unroll
+    for (int t = 0; t < NACC; t++) acc[t] = acc_t{0, 0, 0, 0};
+#pragma unroll
+    for (int t = 0; t < NACC2; t++) acc2[t] = acc_t{0, 0, 0, 0};
+
+    for (int base = s_begin; base < s_end; base += PF, k0 += PF * 64) {
+        uint32_t raw[PF][RAWN];
+        uint4 xa[PF][XN];
+        if constexpr (PRELOAD) {
+            if (base == s_begin) {  // uniform: this batch was requested ahead of the prologue
+#pragma unroll
+                for (int f = 0; f < PF; f++)
+#pragma unroll
+                    for (int r = 0; r < RAWN; r++) raw[f][r] = raw0[f][r];
+            } else {
+                load_weights(base, raw);
+            }
+        } else {
+            load_weights(base, raw);
+        }
         if constexpr (!XLDS) {
             if (p.x_vec_ok) {
 #pragma unroll
@@ -339,52 +422,8 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
                     for (int h = 0; h < XN; h++) xa[f][h] = load_x16<MODE, false>(p, xrow, j, k0 + f * 64 + 8 * h);
             }
         } else {
-            if (base == s_begin) {  // uniform: park the x slice in LDS once its loads have landed
-                constexpr int EPC = 16 / ES;
-#pragma unroll
-                for (int u = 0; u < XC_MAX; u++) {
-                    if (u * 64 < nchunks) {
-                        const int k = s_begin * 64 + (lane + 64 * u) * EPC;
-                        // parked in the order the MFMA wants (each 16-byte chunk is one operand
-                        // fragment), so that the steps below read their A operand ready-made
-                        uint4 v = zero_unless(xr[u], k < (int)p.K);
-                        if constexpr (MODE != MODE_I8 && PRO != 0) {
-                            {
-                                constexpr int DT = (MODE == MODE_F16) ? BT_F16 : BT_BF16;
-                                const uint32_t a[4] = {v.x, v.y, v.z, v.w};
-                                const uint32_t bq[4] = {xb[u].x, xb[u].y, xb[u].z, xb[u].w};
-                                uint32_t r[4];
-#pragma unroll
-                                for (int d = 0; d < 4; d++) {
-                                    uint32_t out = 0;
-#pragma unroll
-                                    for (int e = 0; e < 2; e++) {
-                                        const uint16_t ha = (uint16_t)(a[d] >> (16 * e)), hb = (uint16_t)(bq[d] >> (16 * e));
-                                        const float fa = (DT == BT_F16) ? f16_bits_to_f32(ha) : bf16_bits_to_f32(ha);
-                                        const float fb = (DT == BT_F16) ? f16_bits_to_f32(hb) : bf16_bits_to_f32(hb);
-                                        float y;
-                                        if constexpr (PRO == PRO_SWIGLU) y = swiglu_value(fa, fb, DT);
-                                        else y = rmsnorm_value(fa, rstd, p.pro_b ? fb : 1.0f, DT);
-                                        const uint32_t hy = (DT == BT_F16) ? f32_to_f16_bits(y) : f32_to_bf16_bits(y);
-                                        out |= hy << (16 * e);
-                                    }
-                                    r[d] = out;
-                                }
-                                v = zero_unless(make_uint4(r[0], r[1], r[2], r[3]), k < (int)p.K);
-                            }
-                        }
-                        uint4 o;
-                        if constexpr (MODE == MODE_I8) {
-                            uint32_t t4[4] = {v.x, v.y, v.z, v.w};
-                            if (!p.x_operand_order) transpose4x4_bytes(v.x, v.y, v.z, v.w, t4);  // uniform
-                            o = make_uint4(t4[0], t4[1], t4[2], t4[3]);
-                        } else {
-                            o = make_uint4(perm(v.z, v.x, 0x05040100u), perm(v.z, v.x, 0x07060302u),
-                                           perm(v.w, v.y, 0x05040100u), perm(v.w, v.y, 0x07060302u));
-                        }
-                        *(uint4*)(xs + (lane + 64 * u) * 16) = o;
-                    }
-                }
+            if constexpr (!PRELOAD) {
+                if (base == s_begin) park_x();  // uniform
             }
         }
 #pragma unroll
