@@ -602,8 +602,9 @@ StreamPlan stream_plan(int mode, int64_t M, int64_t N, int64_t Kb, int w_layout,
     if (const char* env = getenv("BITTORCH_STREAM_CFG")) sscanf(env, "%d,%d", &o_ld, &o_waves);
     int ld;
     if (w_layout == W_LAYOUT_TILED) {
-        // 16-column tiles, up to four per workgroup (a batch re-reads its activations once per workgroup)
-        const int min_tiles = (M > 4) ? 160 : 256;
+        // 16-column tiles, up to four per workgroup (a batch re-reads its activations once per workgroup, and so
+        // does a prologue; 240 workgroups of two tiles tie with 480 of one at N = 7680 and win with a prologue)
+        const int min_tiles = (M > 4) ? 160 : 224;
         int nacc = 4;
         while (nacc > min_nacc && ceil_div(N, 16 * nacc) < min_tiles) nacc >>= 1;
         if (o_ld == LD_T1 || o_ld == LD_T2 || o_ld == LD_T4) nacc = o_ld - 100;
