@@ -60,6 +60,8 @@ class TernaryLinearInference(nn.Module):
         if self._tiled is None or self._tiled_key != key:
             from .. import _C
             self._tiled = _C.retile_weights(wp, self.in_features, self.tile_order == "gate_up_pairs")
+            # built once on the current stream; later calls may come from any stream
+            torch.cuda.current_stream(wp.device).synchronize()
             self._tiled_key = key
         return self._tiled
 
