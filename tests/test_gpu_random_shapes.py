@@ -59,3 +59,17 @@ def test_random_shape_sweep(oracle, b, n, k, dtype, seed):
         assert torch.equal(y8o, y8)
     yt = _C.ternary_linear_tensor_core_forward(xq, packed, scale, bias.cuda(), k, 2)
     assert torch.equal(yt, y8)
+
+    # the decode-tiled copy of the weights: layout against the oracle, int8 path bit-exact at every
+    # batch size (streaming kernel up to 32 rows, tiled GEMM beyond), float path equal to the
+    # row-major streaming kernel where that is what the row-major call runs
+    tiled = _C.retile_weights(packed, k)
+    np.testing.assert_array_equal(tiled.cpu().numpy(), oracle.retile_weights(o_packed, k))
+    y8t, acct = _C.ternary_gemm_int8_tiled(q, s, tiled, scale, bias.cuda(), k, n, dtype, True)
+    np.testing.assert_array_equal(acct.cpu().numpy(), oacc)
+    assert torch.equal(y8t, y8)
+    if dtype != torch.float32 or k % 64 == 0:
+        yt_f = _C.ternary_linear_tiled_forward(x.cuda(), tiled, scale, bias.cuda(), k, n)
+        assert rel_err(f32np(yt_f), truth) < (1e-3 if dtype == torch.float32 else 1e-2)
+        if b <= 32 and dtype != torch.float32:
+            assert torch.equal(yt_f, y)
