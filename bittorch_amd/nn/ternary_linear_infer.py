@@ -90,6 +90,9 @@ class TernaryLinearInference(nn.Module):
             return None
         if x.dtype == torch.float32 and self.in_features % 64 != 0:
             return None
+        kb = (self.in_features + 3) // 4
+        if ((self.out_features + 15) // 16) * ((kb + 15) // 16) * 256 >= 2 ** 32:  # beyond the kernels' 32-bit offsets
+            return None
         wp = self.weight_packed
         fresh = self._tiled is not None and self._tiled_key == (wp.data_ptr(), wp._version, wp.device, self.tile_order)
         if not fresh and torch.cuda.is_current_stream_capturing():
