@@ -51,8 +51,9 @@ bool gemm_i8_supported(int64_t N, int64_t K, const void* Q, const void* W_T);
 int launch_row_op(int op, int dtype, const void* A, int64_t lda, const void* Bv, int64_t ldb, float eps, int64_t B,
                   int64_t K, void* H, int8_t* Q, float* s_x, int q_layout, hipStream_t st, const char* who);
 bool gemm_f16_supported(int64_t N, int64_t K, const void* X, const void* W_T, const void* Y);
-int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, const Epilogue& epi, void* Y, int y_dtype, int64_t M,
-                    int64_t N, int64_t K, int planes, hipStream_t st);
+bool gemm_f16_supported_tiled(int64_t N, int64_t K, const void* X, const void* Y);
+int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, int w_layout, const Epilogue& epi, void* Y, int y_dtype,
+                    int64_t M, int64_t N, int64_t K, int planes, hipStream_t st);
 bool gemm_i8_supported_tiled(int64_t N, int64_t K, const void* Q);
 int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_T, int w_layout, const Epilogue& epi,
                    void* Y, int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st);
@@ -192,6 +193,9 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         }
         if (x_dtype != BT_F32) {
             const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
+            // tall batches: the tiled matrix-core GEMM reads the copy too (not with the SwiGLU output stage)
+            if (B > kStreamMaxRows && epi_op == 0 && gemm_f16_supported_tiled(N, K, X, Y))
+                return launch_gemm_f16(mode, X, W_T, W_LAYOUT_TILED, epi, Y, x_dtype, B, N, K, 1, st);
             return launch_stream(mode, X, 2, nullptr, W_T, W_LAYOUT_TILED, epi, Y, x_dtype, nullptr, B, N, K, 1,
                                  Q_ROW_MAJOR, 0, nullptr, 0.0f, epi_op, st);
         }
@@ -203,6 +207,8 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         }
         rc = launch_split_f32_planes(X, B, K, workspace, st);
         if (rc) return rc;
+        if (B > kStreamMaxRows && epi_op == 0 && gemm_f16_supported_tiled(N, 3 * K, workspace, Y))
+            return launch_gemm_f16(MODE_BF16, workspace, W_T, W_LAYOUT_TILED, epi, Y, BT_F32, B, N, K, 3, st);
         return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, W_LAYOUT_TILED, epi, Y, BT_F32, nullptr, B, N, K, 3,
                              Q_ROW_MAJOR, 0, nullptr, 0.0f, epi_op, st);
     }
@@ -210,7 +216,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
         // tall batches go to the tiled matrix-core kernel, decode shapes stream the weights
         if (B > kStreamMaxRows && gemm_f16_supported(N, K, X, W_T, Y))
-            return launch_gemm_f16(mode, X, W_T, epi, Y, x_dtype, B, N, K, 1, st);
+            return launch_gemm_f16(mode, X, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, x_dtype, B, N, K, 1, st);
         return launch_stream(mode, X, 2, nullptr, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, x_dtype, nullptr, B, N, K, 1, Q_ROW_MAJOR, 0, nullptr, 0.0f, 0, st);
     }
     if (x_dtype == BT_F32 && packed_uses_f32_planes(X, W_T, Y, N, K) && workspace &&
@@ -219,7 +225,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         rc = launch_split_f32_planes(X, B, K, workspace, st);
         if (rc) return rc;
         if (B > kStreamMaxRows && gemm_f16_supported(N, 3 * K, workspace, W_T, Y))
-            return launch_gemm_f16(MODE_BF16, workspace, W_T, epi, Y, BT_F32, B, N, K, 3, st);
+            return launch_gemm_f16(MODE_BF16, workspace, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, BT_F32, B, N, K, 3, st);
         return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, BT_F32, nullptr, B, N, K, 3, Q_ROW_MAJOR, 0, nullptr, 0.0f, 0, st);
     }
     return launch_packed_generic(X, x_dtype, W_T, epi, Y, B, N, K, st);

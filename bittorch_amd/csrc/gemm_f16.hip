@@ -41,6 +41,7 @@ struct GemmFParams {
     int y_dtype;
     int tiles_m, tiles_n;
     int per_xcd;          // workgroups per XCD (grid = 8 * per_xcd)
+    int tiles16;          // WT: 16-column tiles of the decode-tiled weight copy (its 16-row steps are the stages)
 };
 
 __device__ __forceinline__ void store4f(void* Y, int dt, int64_t idx, const float (&v)[4]) {
@@ -96,8 +97,11 @@ __device__ __forceinline__ void gemm_f_epilogue_dt(const GemmFParams& p, const v
 
 // TAIL = false: K is a multiple of the 64-wide stage and the main loop is branch free.
 // TAIL = true: any K % 8 == 0; the last, partial stage is masked.
-template <int MODE, bool TAIL>
+// WT = true: W_T is the decode-tiled copy (W_LAYOUT_TILED): the dwords of a lane's four columns in its step are
+// 16 contiguous bytes (one load instead of two), of which the k32 sub-step uses two bytes each.
+template <int MODE, bool TAIL, bool WT = false>
 __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
+    constexpr int BR = WT ? 4 : 2;  // raw weight dwords per lane and stage
     __shared__ __attribute__((aligned(16))) uint8_t lds[65536];  // 2 A stages; reused for the K-half exchange
 
     // XCD-aware tile order: the 8 XCDs each take a contiguous run of tiles, walked in groups
@@ -135,7 +139,15 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     const int64_t rows_left = p.M - m0;
     const uint32_t a_row_c = (uint32_t)((a_row < rows_left) ? a_row : rows_left - 1);
     const uint32_t a_off = (a_row_c * (uint32_t)p.K + 16u * a_part) * 2u;  // bytes
-    const uint32_t b_off = (uint32_t)(col_ok ? ncol : 0) + (uint32_t)(8 * kgrp + 2 * g) * (uint32_t)p.N;
+    uint32_t b_off;
+    if constexpr (WT) {
+        const int tt = min((int)(ncol >> 4), p.tiles16 - 1);  // a tile past the end only feeds outputs never stored
+        b_off = ((uint32_t)tt * (uint32_t)p.wstages * 64u + (uint32_t)(16 * (2 * kgrp + (g >> 1)) + 4 * (j & 3))) * 4u;
+    } else {
+        b_off = (uint32_t)(col_ok ? ncol : 0) + (uint32_t)(8 * kgrp + 2 * g) * (uint32_t)p.N;
+    }
+    // WT: bytes [zero, row 2(g&1), zero, row 2(g&1)+1] of a column's dword
+    const uint32_t sel_wt = ((uint32_t)(2 * (g & 1) + 1) << 24) | (0x0Cu << 16) | ((uint32_t)(2 * (g & 1)) << 8) | 0x0Cu;
     const uint8_t* a_base = (const uint8_t*)(p.X + m0 * p.K);  // uniform
     const uint8_t* b_base = p.W_T;                              // uniform
     const int64_t N = p.N;
@@ -144,10 +156,10 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
 
     // two stages of operands in flight: set s%2 holds stage s until it is written to LDS
     uint4 a_set[2][2];
-    uint32_t b_set[2][2];
+    uint32_t b_set[2][BR];
 
     // part: 1 = activations, 2 = weights, 3 = both
-    auto load_full = [&](int st, int part, uint4 (&a_reg)[2], uint32_t (&b_reg)[2]) {
+    auto load_full = [&](int st, int part, uint4 (&a_reg)[2], uint32_t (&b_reg)[BR]) {
         if (part & 1) {
             const uint8_t* ab = a_base + 2 * (int64_t)st * F_BK;
             a_reg[0] = *(const uint4*)(ab + a_off);
@@ -159,12 +171,17 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
             int ws = st;
             if (ws >= p.wstages) ws -= p.wstages;
             if (ws >= p.wstages) ws -= p.wstages;
-            const uint8_t* bb = b_base + (int64_t)ws * (F_BK / 4) * N;
-            b_reg[0] = *(const uint32_t*)(bb + b_off);
-            b_reg[1] = *(const uint32_t*)(bb + N + b_off);
+            if constexpr (WT) {
+                const uint4 v = *(const uint4*)(b_base + (size_t)ws * 256 + b_off);
+                b_reg[0] = v.x; b_reg[1] = v.y; b_reg[2] = v.z; b_reg[BR - 1] = v.w;
+            } else {
+                const uint8_t* bb = b_base + (int64_t)ws * (F_BK / 4) * N;
+                b_reg[0] = *(const uint32_t*)(bb + b_off);
+                b_reg[1] = *(const uint32_t*)(bb + N + b_off);
+            }
         }
     };
-    auto load_tail = [&](int64_t k0, int part, uint4 (&a_reg)[2], uint32_t (&b_reg)[2]) {
+    auto load_tail = [&](int64_t k0, int part, uint4 (&a_reg)[2], uint32_t (&b_reg)[BR]) {
         // last, partial stage: k beyond K reads a clamped address and is zeroed in A
         if (part & 1) {
             const uint8_t* ab = a_base + 2 * k0;
@@ -176,7 +193,12 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
                 a_reg[c] = make_uint4(v.x & m, v.y & m, v.z & m, v.w & m);
             }
         }
-        if (part & 2) {
+        if constexpr (WT) {
+            if (part & 2) {  // the copy is zero-padded to whole steps; this is the last step (no planes with a tail)
+                const uint4 v = *(const uint4*)(b_base + (size_t)min((int)(k0 >> 6), p.wstages - 1) * 256 + b_off);
+                b_reg[0] = v.x; b_reg[1] = v.y; b_reg[2] = v.z; b_reg[BR - 1] = v.w;
+            }
+        } else if (part & 2) {
 #pragma unroll
             for (int r = 0; r < 2; r++) {
                 int64_t kb = (k0 >> 2) + 8 * kgrp + 2 * g + r;
@@ -185,7 +207,7 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
             }
         }
     };
-    auto load_stage = [&](int st, int part, uint4 (&a_reg)[2], uint32_t (&b_reg)[2]) {  // st, part uniform
+    auto load_stage = [&](int st, int part, uint4 (&a_reg)[2], uint32_t (&b_reg)[BR]) {  // st, part uniform
         if constexpr (TAIL) {
             if (st >= nstages) st = nstages - 1;
             if (st < nfull) load_full(st, part, a_reg, b_reg);
@@ -227,10 +249,14 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     uint4 a_lo[4], a_hi[4];
     const uint32_t a_lds_off = (uint32_t)(kgrp * (F_MB * 1024)) + ((uint32_t)lane << 4);
     constexpr uint32_t LUT = (MODE == MODE_F16) ? LUT_F16_ONE : LUT_BF16_TWO;
-    auto decode_col = [&](const uint32_t (&raw)[2], int t, u32x4& out) {
-        // bytes [zero, row0.byte t, zero, row1.byte t]
-        const uint32_t sel = ((uint32_t)(4 + t) << 24) | (0x0Cu << 16) | ((uint32_t)t << 8) | 0x0Cu;
-        out = decode8_16bit<LUT>(perm(raw[1], raw[0], sel));
+    auto decode_col = [&](const uint32_t (&raw)[BR], int t, u32x4& out) {
+        if constexpr (WT) {
+            out = decode8_16bit<LUT>(perm(0u, raw[t], sel_wt));
+        } else {
+            // bytes [zero, row0.byte t, zero, row1.byte t]
+            const uint32_t sel = ((uint32_t)(4 + t) << 24) | (0x0Cu << 16) | ((uint32_t)t << 8) | 0x0Cu;
+            out = decode8_16bit<LUT>(perm(raw[1], raw[0], sel));
+        }
     };
     auto read_a = [&](int buf, int mb0, uint4 (&dst)[4]) {
         const uint8_t* a_lds = lds + buf * F_STAGE_BYTES + a_lds_off;
@@ -254,7 +280,7 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     __syncthreads();
     read_a(0, 0, a_lo);
 
-    auto stage = [&](int s, uint4 (&a_reg)[2], uint32_t (&b_reg)[2], const u32x4 (&b_cur)[4], u32x4 (&b_nxt)[4]) {
+    auto stage = [&](int s, uint4 (&a_reg)[2], uint32_t (&b_reg)[BR], const u32x4 (&b_cur)[4], u32x4 (&b_nxt)[4]) {
         // a_reg / b_reg hold stage s+1 on entry and are reloaded with stage s+3
         const int cur = s & 1;
         store_a(cur ^ 1, a_reg);
@@ -333,6 +359,12 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
 }
 
 // the tiled kernel reads X with 16-byte loads and W_T / Y with 4-column vectors
+// the same kernel on the decode-tiled weight copy (256-byte aligned, below 4 GiB: checked by the caller)
+bool gemm_f16_supported_tiled(int64_t N, int64_t K, const void* X, const void* Y) {
+    return N % 4 == 0 && K % 8 == 0 && K >= 8 && ((uintptr_t)X) % 16 == 0 && ((uintptr_t)Y) % 16 == 0 &&
+           (F_BM + 1) * K * 2 < (1ll << 32);
+}
+
 bool gemm_f16_supported(int64_t N, int64_t K, const void* X, const void* W_T, const void* Y) {
     return N % 4 == 0 && K % 8 == 0 && K >= 8 && ((uintptr_t)W_T) % 4 == 0 && ((uintptr_t)X) % 16 == 0 &&
            ((uintptr_t)Y) % 16 == 0 && (F_BM + 1) * K * 2 < (1ll << 32) && ceil_div(K, 4) * N < (1ll << 32);
@@ -340,8 +372,8 @@ bool gemm_f16_supported(int64_t N, int64_t K, const void* X, const void* W_T, co
 
 // planes = 1: X is [M, K].  planes = 3 (K % 64 == 0): X is [M, 3K], three planes of K values per
 // row whose products with the same weights are summed (fp32 activations split into three bf16 terms).
-int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, const Epilogue& epi, void* Y, int y_dtype, int64_t M,
-                    int64_t N, int64_t K, int planes, hipStream_t st) {
+int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, int w_layout, const Epilogue& epi, void* Y, int y_dtype,
+                    int64_t M, int64_t N, int64_t K, int planes, hipStream_t st) {
     GemmFParams p;
     p.X = (const uint16_t*)X; p.W_T = W_T; p.Y = Y; p.epi = epi;
     p.M = M; p.N = N; p.K = K * planes; p.Kb = ceil_div(K, 4);
@@ -354,6 +386,17 @@ int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, const Epilogue&
     p.per_xcd = (int)ceil_div(total, 8);
     const dim3 grid((unsigned)(p.per_xcd * 8)), block(512);
     const bool tail = p.K % F_BK != 0;
+    p.tiles16 = (int)ceil_div(N, 16);
+    if (w_layout == W_LAYOUT_TILED) {
+        if (mode == MODE_F16) {
+            if (tail) hipLaunchKernelGGL((gemm_f16_kernel<MODE_F16, true, true>), grid, block, 0, st, p);
+            else hipLaunchKernelGGL((gemm_f16_kernel<MODE_F16, false, true>), grid, block, 0, st, p);
+        } else {
+            if (tail) hipLaunchKernelGGL((gemm_f16_kernel<MODE_BF16, true, true>), grid, block, 0, st, p);
+            else hipLaunchKernelGGL((gemm_f16_kernel<MODE_BF16, false, true>), grid, block, 0, st, p);
+        }
+        return check_launch("bt_ternary_linear_tiled_forward");
+    }
     if (mode == MODE_F16) {
         if (tail) hipLaunchKernelGGL((gemm_f16_kernel<MODE_F16, true>), grid, block, 0, st, p);
         else hipLaunchKernelGGL((gemm_f16_kernel<MODE_F16, false>), grid, block, 0, st, p);

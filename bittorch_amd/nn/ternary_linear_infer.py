@@ -5,10 +5,10 @@ API mirror of ``bittorch/nn/ternary_linear_infer.py:22-193``.  Buffers:
 optional ``bias``; nothing is trainable.  GPU inputs go to the packed HIP
 kernels; CPU inputs unpack and use ``F.linear`` as the reference does.
 
-Decode-shape calls on the GPU (up to ``DECODE_ROWS`` rows) read a second, *decode-tiled* copy of
-the packed weights that the layer builds from ``weight_packed`` on first use (same size, not part
-of the ``state_dict``; same results bit for bit, 15-25 % less time per GEMV because every load of
-the kernel then covers whole cache lines).  ``decode_tiled=False`` or ``BITTORCH_DECODE_TILED=0``
+GPU calls read a second, *decode-tiled* copy of the packed weights that the layer builds from
+``weight_packed`` on first use (same size, not part of the ``state_dict``; same results bit for bit,
+15-25 % less time per decode GEMV because every load of the kernel then covers whole cache lines, a
+few per cent on the prefill GEMMs).  ``decode_tiled=False`` or ``BITTORCH_DECODE_TILED=0``
 keeps the layer on ``weight_packed`` alone.  ``forward_int8`` reads the copy at every batch size (the
 int8 prefill GEMM loads it with one 16-byte load per lane and stage instead of four dword loads and a
 byte transpose).
@@ -80,8 +80,9 @@ class TernaryLinearInference(nn.Module):
         return self
 
     def _tiled_for(self, x: Tensor, rows: int, order: str = "natural") -> Optional[Tensor]:
-        # (int8 activations: the tiled GEMM reads the copy too, so every batch size takes it)
-        if not (self.decode_tiled and x.is_cuda and (rows <= DECODE_ROWS or x.dtype == torch.int8)
+        # (the tiled GEMMs read the copy too, so every batch size takes it; only the SwiGLU output stage of a
+        # pair-ordered copy is a decode-shape affair)
+        if not (self.decode_tiled and x.is_cuda and (rows <= DECODE_ROWS or order == "natural")
                 and self.tile_order == order):
             return None
         if os.environ.get("BITTORCH_KERNEL") == "generic":  # the shape-generic kernel reads weight_packed
