@@ -111,7 +111,19 @@ static bool fast_path_ok(const void* Y, int64_t N, int64_t K) {
 static const int64_t kMaxKInt8 = 133000;
 
 // batches up to this many rows go through the streaming (decode-shape) kernel
-static const int64_t kStreamMaxRows = 32;
+// On the tiled weight copy the streaming kernel stays ahead for longer (a tiled GEMM of up to 128 rows
+// occupies one row of tiles, 16 workgroups at N = 4096): measured crossovers 64..96 rows with 16-bit
+// activations, 48..64 with int8.  BITTORCH_STREAM_MAX_ROWS overrides all three, for tuning runs.
+static int64_t stream_max_rows(int64_t dflt) {
+    if (const char* env = getenv("BITTORCH_STREAM_MAX_ROWS")) {
+        const long v = atol(env);
+        if (v >= 1) return v;
+    }
+    return dflt;
+}
+#define kStreamMaxRows stream_max_rows(32)
+#define kStreamMaxRowsTiledF16 stream_max_rows(64)
+#define kStreamMaxRowsTiledI8 stream_max_rows(48)
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
@@ -194,7 +206,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         if (x_dtype != BT_F32) {
             const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
             // tall batches: the tiled matrix-core GEMM reads the copy too (not with the SwiGLU output stage)
-            if (B > kStreamMaxRows && epi_op == 0 && gemm_f16_supported_tiled(N, K, X, Y))
+            if (B > kStreamMaxRowsTiledF16 && epi_op == 0 && gemm_f16_supported_tiled(N, K, X, Y))
                 return launch_gemm_f16(mode, X, W_T, W_LAYOUT_TILED, epi, Y, x_dtype, B, N, K, 1, st);
             return launch_stream(mode, X, 2, nullptr, W_T, W_LAYOUT_TILED, epi, Y, x_dtype, nullptr, B, N, K, 1,
                                  Q_ROW_MAJOR, 0, nullptr, 0.0f, epi_op, st);
@@ -207,7 +219,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         }
         rc = launch_split_f32_planes(X, B, K, workspace, st);
         if (rc) return rc;
-        if (B > kStreamMaxRows && epi_op == 0 && gemm_f16_supported_tiled(N, 3 * K, workspace, Y))
+        if (B > kStreamMaxRowsTiledF16 && epi_op == 0 && gemm_f16_supported_tiled(N, 3 * K, workspace, Y))
             return launch_gemm_f16(MODE_BF16, workspace, W_T, W_LAYOUT_TILED, epi, Y, BT_F32, B, N, K, 3, st);
         return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, W_LAYOUT_TILED, epi, Y, BT_F32, nullptr, B, N, K, 3,
                              Q_ROW_MAJOR, 0, nullptr, 0.0f, epi_op, st);
@@ -322,7 +334,7 @@ static int gemm_i8_impl(const char* who, const int8_t* Q, int q_layout, const fl
             set_error("%s: tiled weights must be 256-byte aligned and below 4 GiB", who);
             return BT_ERR_INVALID;
         }
-        if (B > kStreamMaxRows && gemm_i8_supported_tiled(N, K, Q))
+        if (B > kStreamMaxRowsTiledI8 && gemm_i8_supported_tiled(N, K, Q))
             return launch_gemm_i8(Q, q_layout, s_x, W_T, W_LAYOUT_TILED, epi, Y, y_dtype, acc_out, B, N, K, st);
         return launch_stream(MODE_I8, Q, 1, s_x, W_T, w_layout, epi, Y, y_dtype, acc_out, B, N, K, 1, q_layout, 0, nullptr,
                              0.0f, 0, st);

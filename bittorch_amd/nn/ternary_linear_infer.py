@@ -28,8 +28,8 @@ from ..quant.ternary import ternary_quantize
 from ..quant.ternary_packed import pack_ternary_transposed, unpack_ternary_transposed
 
 
-# batches up to this many rows stream the weights (once per 16 rows) instead of running the tiled GEMM
-DECODE_ROWS = 32
+# batches up to this many rows stream the tiled weights (once per 16 rows) instead of running the tiled GEMM
+DECODE_ROWS = 64
 
 
 class TernaryLinearInference(nn.Module):

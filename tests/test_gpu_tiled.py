@@ -59,7 +59,10 @@ def test_tiled_forward_equals_row_major(oracle, dtype, n, k):
         res = seeded_acts(b, n, seed=b + 1, dtype=dtype).cuda()
         ref = _C.ternary_linear_packed_forward(x, wt, scale, bias, k, residual=res)
         got = _C.ternary_linear_tiled_forward(x, tiled, scale, bias, k, n, residual=res)
-        assert torch.equal(got, ref)  # up to 32 rows both stream the weights, beyond both run the tiled GEMM
+        if b <= 32 or b > 64:  # both stream the weights / both run the tiled GEMM
+            assert torch.equal(got, ref)
+        else:  # 33..64 rows: the tiled copy is still streamed, the row-major call runs the GEMM (another summation order)
+            assert rel_err(f32np(got), f32np(ref)) <= 2e-3
     x = seeded_acts(1, k, seed=9, dtype=dtype).cuda()
     assert torch.equal(_C.ternary_linear_tiled_forward(x, tiled, scale[:1], None, k, n),
                        _C.ternary_linear_packed_forward(x, wt, scale[:1], None, k))
@@ -161,7 +164,7 @@ def test_module_uses_tiled_copy_for_decode_shapes(oracle, dtype):
     a = _layer(oracle, 640, 512, seed=3)                      # default: tiled copy on first decode call
     b = _layer(oracle, 640, 512, seed=3, decode_tiled=False)  # weight_packed only
     assert a.decode_tiled and a._tiled is None
-    for shape in ((512,), (1, 512), (2, 3, 512), (32, 512), (40, 512)):
+    for shape in ((512,), (1, 512), (2, 3, 512), (32, 512), (70, 512)):  # (33..64 rows take different kernels)
         x = seeded_acts(1, int(np.prod(shape)), seed=len(shape), dtype=dtype).reshape(shape).cuda()
         ya, yb = a(x), b(x)
         assert ya.shape == yb.shape == (*shape[:-1], 640)
@@ -263,7 +266,7 @@ def test_ternary_swiglu_decode_uses_the_output_stage(oracle, dtype):
     assert fused.gate_up.tile_order == "gate_up_pairs"
     plain = TernarySwiGLU(gate, up, down, compute="float", fuse_gate_up=False)
     nw = (torch.rand(d) + 0.5).to(dtype).cuda()
-    for rows in (1, 5, 40):
+    for rows in (1, 5, 40, 70):
         announce("TernarySwiGLU decode", dtype, rows)
         x = seeded_acts(rows, d, seed=rows, dtype=dtype).cuda()
         assert torch.equal(fused(x, nw, 1e-5, residual=x), plain(x, nw, 1e-5, residual=x))
