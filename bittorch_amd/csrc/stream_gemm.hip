@@ -54,7 +54,8 @@ struct StreamParams {
     int wsteps;           // 16-row steps of W_T; a step index beyond it wraps (see launch_stream)
     int tiles;            // column tiles
     int per_xcd;          // tiles per XCD (grid = 8 * per_xcd)
-    int M;                // 1..16
+    int M;                // 1..16: rows of a 16-row block (of the last one when the launch covers several)
+    int64_t B;            // rows of the whole call: grid.y = ceil(B / 16) blocks of 16 rows, all in one launch
     int y_dtype;
     int x_vec_ok;         // activation rows may be read with 16-byte loads
     int prehalved;        // MODE_BF16: the activations already carry the factor 1/2 of the +-2.0 weight decode
@@ -169,7 +170,7 @@ __device__ __forceinline__ float linear_value(const StreamParams& p, uint32_t bi
 // with one: a run-time switch, even a uniform one, puts branches and waits around the loads of the
 // plain kernel).
 template <int MODE, int LD, int WAVES, int PF, bool XLDS, int PRO = 0, int EPI = 0>
-__global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
+__global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p_in) {
     constexpr bool QUAD = (LD == LD_Q1 || LD == LD_Q2);
     constexpr bool BYTE = (LD == LD_BYTE);
     constexpr bool TILED = (LD > 100);
@@ -185,6 +186,24 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p) {
     typedef typename std::conditional<MODE == MODE_I8, v4i, v4f>::type acc_t;
 
     extern __shared__ __attribute__((aligned(16))) uint32_t red[];  // [WAVES][M][TILE_N], then x slices
+
+    // One launch covers every 16-row block of the call (grid.y): the blocks are independent, run
+    // concurrently and find the weights their neighbours fetched in the XCD's L2 (the same tile of every
+    // block lands on the same XCD).  This workgroup's block: rows 16*blockIdx.y .. of X, Y, s_x, ...
+    StreamParams p = p_in;
+    if constexpr (!XLDS) {  // (the LDS-staged variant is the single-row one)
+        if (p_in.B > 16) {  // uniform
+            const int64_t r0 = (int64_t)blockIdx.y * 16;
+            const int64_t ny = (EPI == EPI_SWIGLU_PAIRS) ? (p_in.N >> 1) : p_in.N;
+            const int ysz = (p_in.y_dtype == BT_F32) ? 4 : 2;
+            p.M = (int)((p_in.B - r0 < 16) ? (p_in.B - r0) : 16);
+            p.X = (const uint8_t*)p_in.X + r0 * p_in.K * ((MODE == MODE_I8) ? 1 : 2);
+            p.Y = (uint8_t*)p_in.Y + r0 * ny * ysz;
+            if (p_in.s_x) p.s_x = p_in.s_x + r0;
+            if (p_in.acc_out) p.acc_out = p_in.acc_out + r0 * p_in.N;
+            if (p_in.epi.residual) p.epi.residual = (const uint8_t*)p_in.epi.residual + r0 * p_in.N * ysz;
+        }
+    }
 
     // consecutive tiles on one XCD (workgroups are dealt round-robin over 8 XCDs)
     const int tile = (int)(blockIdx.x & 7) * p.per_xcd + (int)(blockIdx.x >> 3);
@@ -704,7 +723,7 @@ static int launch_stream_mode(StreamParams p, const StreamPlan& pl, hipStream_t 
     const int64_t tile_n = ld_columns(pl.ld);
     p.tiles = (int)ceil_div(p.N, tile_n);
     p.per_xcd = (int)ceil_div(p.tiles, 8);
-    const dim3 grid((unsigned)(p.per_xcd * 8));
+    const dim3 grid((unsigned)(p.per_xcd * 8), (unsigned)ceil_div(p.B, 16));
     const int waves = pl.waves;
     const int es = (MODE == MODE_I8) ? 1 : 2;
     const size_t red_bytes = (size_t)waves * p.M * tile_n * 4;
@@ -735,7 +754,7 @@ static int launch_stream_mode(StreamParams p, const StreamPlan& pl, hipStream_t 
     return check_launch("stream_gemm");
 }
 
-// One launch per block of up to 16 activation rows.
+// One launch for the whole call: grid.y walks its blocks of 16 activation rows.
 // planes = 1: X is [B, K].  planes = 3 (K % 64 == 0): X is [B, 3K], three planes of K values per
 // row whose products with the same weights are summed (fp32 activations split into three bf16
 // terms); the kernel walks 3K values of k and wraps its weight row index every K.
@@ -751,31 +770,32 @@ int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, co
     const StreamPlan pl = stream_plan(mode, B, N, Kb, w_layout, epi_op == EPI_SWIGLU_PAIRS ? 2 : 1);
     const int64_t Ny = (epi_op == EPI_SWIGLU_PAIRS) ? N / 2 : N;  // columns of Y
     const int y_size = dtype_size(y_dtype);
-    for (int64_t m0 = 0; m0 < B; m0 += 16) {
-        StreamParams p;
-        p.X = (const uint8_t*)X + m0 * Kx * x_elem_size;
-        p.W_T = W_T;
-        p.s_x = s_x ? s_x + m0 : nullptr;
-        p.Y = (uint8_t*)Y + m0 * Ny * y_size;
-        p.acc_out = acc_out ? acc_out + m0 * N : nullptr;
-        p.epi = epi;
-        if (epi.residual) p.epi.residual = (const uint8_t*)epi.residual + m0 * N * y_size;
-        p.N = N; p.K = Kx; p.Kb = Kb;
-        p.wsteps = (int)ceil_div(Kb, 16);
-        p.tiles16 = (int)ceil_div(N, 16);
-        p.prehalved = planes == 3;
-        p.x_operand_order = (mode == MODE_I8 && q_layout == Q_OPERAND_ORDER) ? 1 : 0;
-        p.pro_op = pro_op; p.pro_b = pro_b; p.pro_eps = pro_eps; p.epi_op = epi_op;
-        p.M = (int)((B - m0 < 16) ? (B - m0) : 16);
-        p.y_dtype = y_dtype;
-        p.x_vec_ok = (((uintptr_t)p.X) % 16 == 0) && ((Kx * x_elem_size) % 16 == 0);
-        int rc;
-        if (mode == MODE_I8) rc = launch_stream_mode<MODE_I8>(p, pl, st);
-        else if (mode == MODE_F16) rc = launch_stream_mode<MODE_F16>(p, pl, st);
-        else rc = launch_stream_mode<MODE_BF16>(p, pl, st);
-        if (rc != BT_OK) return rc;
+    if (ceil_div(B, 16) > 65535) {
+        set_error("stream_gemm: %lld rows exceed the 65535 blocks of 16 rows one launch covers", (long long)B);
+        return BT_ERR_INVALID;
     }
-    return BT_OK;
+    StreamParams p;
+    p.X = X;
+    p.W_T = W_T;
+    p.s_x = s_x;
+    p.Y = Y;
+    p.acc_out = acc_out;
+    p.epi = epi;
+    p.N = N; p.K = Kx; p.Kb = Kb;
+    p.wsteps = (int)ceil_div(Kb, 16);
+    p.tiles16 = (int)ceil_div(N, 16);
+    p.prehalved = planes == 3;
+    p.x_operand_order = (mode == MODE_I8 && q_layout == Q_OPERAND_ORDER) ? 1 : 0;
+    p.pro_op = pro_op; p.pro_b = pro_b; p.pro_eps = pro_eps; p.epi_op = epi_op;
+    p.B = B;
+    p.M = (int)((B < 16) ? B : 16);
+    p.y_dtype = y_dtype;
+    // (a row is a multiple of 16 bytes, so every 16-row block starts as aligned as the first)
+    p.x_vec_ok = (((uintptr_t)p.X) % 16 == 0) && ((Kx * x_elem_size) % 16 == 0);
+    (void)Ny; (void)y_size;
+    if (mode == MODE_I8) return launch_stream_mode<MODE_I8>(p, pl, st);
+    if (mode == MODE_F16) return launch_stream_mode<MODE_F16>(p, pl, st);
+    return launch_stream_mode<MODE_BF16>(p, pl, st);
 }
 
 }  // namespace bt

@@ -29,7 +29,7 @@ from ..quant.ternary_packed import pack_ternary_transposed, unpack_ternary_trans
 
 
 # batches up to this many rows stream the tiled weights (once per 16 rows) instead of running the tiled GEMM
-DECODE_ROWS = 64
+DECODE_ROWS = 128
 
 
 class TernaryLinearInference(nn.Module):

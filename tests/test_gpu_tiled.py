@@ -59,9 +59,9 @@ def test_tiled_forward_equals_row_major(oracle, dtype, n, k):
         res = seeded_acts(b, n, seed=b + 1, dtype=dtype).cuda()
         ref = _C.ternary_linear_packed_forward(x, wt, scale, bias, k, residual=res)
         got = _C.ternary_linear_tiled_forward(x, tiled, scale, bias, k, n, residual=res)
-        if b <= 32 or b > 64:  # both stream the weights / both run the tiled GEMM
+        if b <= 96 or b > 128:  # both stream the weights / both run the tiled GEMM
             assert torch.equal(got, ref)
-        else:  # 33..64 rows: the tiled copy is still streamed, the row-major call runs the GEMM (another summation order)
+        else:  # 97..128 rows: the tiled copy is still streamed, the row-major call runs the GEMM (another summation order)
             assert rel_err(f32np(got), f32np(ref)) <= 2e-3
     x = seeded_acts(1, k, seed=9, dtype=dtype).cuda()
     assert torch.equal(_C.ternary_linear_tiled_forward(x, tiled, scale[:1], None, k, n),
@@ -164,7 +164,7 @@ def test_module_uses_tiled_copy_for_decode_shapes(oracle, dtype):
     a = _layer(oracle, 640, 512, seed=3)                      # default: tiled copy on first decode call
     b = _layer(oracle, 640, 512, seed=3, decode_tiled=False)  # weight_packed only
     assert a.decode_tiled and a._tiled is None
-    for shape in ((512,), (1, 512), (2, 3, 512), (32, 512), (70, 512)):  # (33..64 rows take different kernels)
+    for shape in ((512,), (1, 512), (2, 3, 512), (32, 512), (70, 512)):  # (97..128 rows take different kernels)
         x = seeded_acts(1, int(np.prod(shape)), seed=len(shape), dtype=dtype).reshape(shape).cuda()
         ya, yb = a(x), b(x)
         assert ya.shape == yb.shape == (*shape[:-1], 640)
