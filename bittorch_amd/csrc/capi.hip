@@ -111,21 +111,19 @@ static bool fast_path_ok(const void* Y, int64_t N, int64_t K) {
 static const int64_t kMaxKInt8 = 133000;
 
 // batches up to this many rows go through the streaming (decode-shape) kernel
-// On the tiled weight copy the streaming kernel stays ahead for longer (its 16-row blocks run concurrently in
-// one launch, while a tiled GEMM of up to 128 rows occupies one row of tiles, 16 workgroups at N = 4096):
-// measured crossovers 128..192 rows with 16-bit activations, 96..192 with int8.  BITTORCH_STREAM_MAX_ROWS overrides all three, for tuning runs.
-static int64_t stream_max_rows(int64_t dflt) {
+// Streaming kernel or tiled GEMM?  The streaming kernel runs the 16-row blocks of a call concurrently in one
+// launch and its time grows with B * N; a tiled GEMM takes the time of one 128 x 256 tile until its tiles
+// fill the chip.  Measured crossovers (five layer shapes, both weight layouts): B * N = 1.5 .. 2.1 M outputs
+// with 16-bit activations, 1.3 .. 2.1 M with int8, i.e. while the GEMM would occupy under a fifth of the
+// compute units.  BITTORCH_STREAM_MAX_ROWS=n replaces the rule by "B <= n" (tuning runs).
+static bool prefers_stream(int64_t B, int64_t N, bool int8) {
     if (const char* env = getenv("BITTORCH_STREAM_MAX_ROWS")) {
         const long v = atol(env);
-        if (v >= 1) return v;
+        if (v >= 1) return B <= v;
     }
-    return dflt;
+    if (B <= 32) return true;
+    return B <= 4096 && B * N <= (int8 ? 1310720 : 1572864);
 }
-// (row-major W_T: crossovers 96..128 rows with 16-bit activations, 64..128 with int8)
-#define kStreamMaxRowsF16 stream_max_rows(96)
-#define kStreamMaxRowsI8 stream_max_rows(64)
-#define kStreamMaxRowsTiledF16 stream_max_rows(128)
-#define kStreamMaxRowsTiledI8 stream_max_rows(96)
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
@@ -208,7 +206,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         if (x_dtype != BT_F32) {
             const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
             // tall batches: the tiled matrix-core GEMM reads the copy too (not with the SwiGLU output stage)
-            if (B > kStreamMaxRowsTiledF16 && epi_op == 0 && gemm_f16_supported_tiled(N, K, X, Y))
+            if (!prefers_stream(B, N, false) && epi_op == 0 && gemm_f16_supported_tiled(N, K, X, Y))
                 return launch_gemm_f16(mode, X, W_T, W_LAYOUT_TILED, epi, Y, x_dtype, B, N, K, 1, st);
             return launch_stream(mode, X, 2, nullptr, W_T, W_LAYOUT_TILED, epi, Y, x_dtype, nullptr, B, N, K, 1,
                                  Q_ROW_MAJOR, 0, nullptr, 0.0f, epi_op, st);
@@ -221,7 +219,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         }
         rc = launch_split_f32_planes(X, B, K, workspace, st);
         if (rc) return rc;
-        if (B > kStreamMaxRowsTiledF16 && epi_op == 0 && gemm_f16_supported_tiled(N, 3 * K, workspace, Y))
+        if (!prefers_stream(B, N, false) && epi_op == 0 && gemm_f16_supported_tiled(N, 3 * K, workspace, Y))
             return launch_gemm_f16(MODE_BF16, workspace, W_T, W_LAYOUT_TILED, epi, Y, BT_F32, B, N, K, 3, st);
         return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, W_LAYOUT_TILED, epi, Y, BT_F32, nullptr, B, N, K, 3,
                              Q_ROW_MAJOR, 0, nullptr, 0.0f, epi_op, st);
@@ -229,7 +227,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
     if (packed_uses_stream(x_dtype, W_T, Y, N, K)) {
         const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
         // tall batches go to the tiled matrix-core kernel, decode shapes stream the weights
-        if (B > kStreamMaxRowsF16 && gemm_f16_supported(N, K, X, W_T, Y))
+        if (!prefers_stream(B, N, false) && gemm_f16_supported(N, K, X, W_T, Y))
             return launch_gemm_f16(mode, X, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, x_dtype, B, N, K, 1, st);
         return launch_stream(mode, X, 2, nullptr, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, x_dtype, nullptr, B, N, K, 1, Q_ROW_MAJOR, 0, nullptr, 0.0f, 0, st);
     }
@@ -238,7 +236,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         // (without a workspace the call still succeeds, on the generic kernel)
         rc = launch_split_f32_planes(X, B, K, workspace, st);
         if (rc) return rc;
-        if (B > kStreamMaxRowsF16 && gemm_f16_supported(N, 3 * K, workspace, W_T, Y))
+        if (!prefers_stream(B, N, false) && gemm_f16_supported(N, 3 * K, workspace, W_T, Y))
             return launch_gemm_f16(MODE_BF16, workspace, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, BT_F32, B, N, K, 3, st);
         return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, BT_F32, nullptr, B, N, K, 3, Q_ROW_MAJOR, 0, nullptr, 0.0f, 0, st);
     }
@@ -336,14 +334,14 @@ static int gemm_i8_impl(const char* who, const int8_t* Q, int q_layout, const fl
             set_error("%s: tiled weights must be 256-byte aligned and below 4 GiB", who);
             return BT_ERR_INVALID;
         }
-        if (B > kStreamMaxRowsTiledI8 && gemm_i8_supported_tiled(N, K, Q))
+        if (!prefers_stream(B, N, true) && gemm_i8_supported_tiled(N, K, Q))
             return launch_gemm_i8(Q, q_layout, s_x, W_T, W_LAYOUT_TILED, epi, Y, y_dtype, acc_out, B, N, K, st);
         return launch_stream(MODE_I8, Q, 1, s_x, W_T, w_layout, epi, Y, y_dtype, acc_out, B, N, K, 1, q_layout, 0, nullptr,
                              0.0f, 0, st);
     }
     // decode-shape batches, and any batch whose N the tiled kernel's 4-column
     // vector accesses cannot take, stream the weights once per 16 rows
-    if (B <= kStreamMaxRowsI8 || !gemm_i8_supported(N, K, Q, W_T)) {
+    if (prefers_stream(B, N, true) || !gemm_i8_supported(N, K, Q, W_T)) {
         if (!stream_supported(N, K, W_T)) {
             set_error("%s: packed weight matrix of %lld x %lld bytes exceeds the 4 GiB the kernels address", who,
                       (long long)ceil_div(K, 4), (long long)N);

@@ -623,9 +623,11 @@ StreamPlan stream_plan(int mode, int64_t M, int64_t N, int64_t Kb, int w_layout,
     if (w_layout == W_LAYOUT_TILED) {
         // 16-column tiles, up to four per workgroup (a batch re-reads its activations once per workgroup, and so
         // does a prologue; 240 workgroups of two tiles tie with 480 of one at N = 7680 and win with a prologue)
+        // (every 16-row block of the call is a grid row of the same launch: the workgroups of all blocks count)
         const int min_tiles = (M > 4) ? 160 : 224;
+        const int64_t row_blocks = ceil_div(M, 16);
         int nacc = 4;
-        while (nacc > min_nacc && ceil_div(N, 16 * nacc) < min_tiles) nacc >>= 1;
+        while (nacc > min_nacc && ceil_div(N, 16 * nacc) * row_blocks < min_tiles) nacc >>= 1;
         if (o_ld == LD_T1 || o_ld == LD_T2 || o_ld == LD_T4) nacc = o_ld - 100;
         if (nacc < min_nacc) nacc = min_nacc;
         ld = 100 + nacc;
@@ -641,7 +643,8 @@ StreamPlan stream_plan(int mode, int64_t M, int64_t N, int64_t Kb, int w_layout,
         // with 256-column tiles and 4 on very wide layers: 23.5 -> 17.4 us at N = 65536, K = 4096)
         ld = (N % 16 == 0 && mode != MODE_I8) ? 16 : (N % 8 == 0) ? 8 : 4;
         const int min_tiles = (M > 4) ? 160 : 256;
-        while (ld > 1 && ceil_div(N, ld_columns(ld)) < min_tiles) ld >>= 1;
+        const int64_t row_blocks = ceil_div(M, 16);  // all blocks of the call share one launch
+        while (ld > 1 && ceil_div(N, ld_columns(ld)) * row_blocks < min_tiles) ld >>= 1;
     }
     pl.ld = ld;
     const int max_waves = (ld == 16) ? 4 : (ld == 8 || ld == LD_BYTE) ? 8 : 16;   // LDS: WAVES*TILE_N <= 1024 words per row

@@ -64,9 +64,12 @@ def test_gemm_i8_small_batch_bit_exact(oracle, b, n, k):
 
 
 # prefill kernel: B > 32, including ragged M / N / K tiles
+@pytest.mark.parametrize("route", ["auto", "gemm"])
 @pytest.mark.parametrize("b,n,k", [(128, 256, 128), (256, 512, 1024), (33, 64, 64), (130, 260, 132),
                                    (64, 4, 16), (200, 1024, 4096), (129, 300, 1000), (2048, 256, 512)])
-def test_gemm_i8_prefill_bit_exact(oracle, b, n, k):
+def test_gemm_i8_prefill_bit_exact(oracle, b, n, k, route, monkeypatch):
+    if route == "gemm":  # batches beyond 32 rows to the tiled GEMM whatever their size (the default rule streams small outputs)
+        monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
     announce("gemm_i8 prefill", b, n, k)
     _gemm_case(oracle, b, n, k, torch.bfloat16, seed=n + k, outliers=True)
     _gemm_case(oracle, b, n, k, torch.float16, seed=n + k + 1)

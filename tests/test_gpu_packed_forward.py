@@ -85,12 +85,15 @@ def test_packed_forward_batch_sizes(oracle, b):
     _case(oracle, b, 128, 256, torch.bfloat16, seed=b)
 
 
+@pytest.mark.parametrize("route", ["auto", "gemm"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("b,n,k", [(128, 256, 64), (33, 128, 256), (200, 260, 72), (129, 512, 1000), (512, 1024, 4096),
                                    (130, 36, 8), (257, 300, 136), (64, 256, 768)])
-def test_packed_forward_tall_batches_use_the_tiled_kernel(oracle, dtype, b, n, k):
+def test_packed_forward_tall_batches_use_the_tiled_kernel(oracle, dtype, b, n, k, route, monkeypatch):
     """Batches above the streaming kernel's limit go to the 16-bit matrix-core GEMM: partial row
     and column tiles, K tails that are not a multiple of the 64-wide stage, odd last stages."""
+    if route == "gemm":  # batches beyond 32 rows to the tiled GEMM whatever their size (the default rule streams small outputs)
+        monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
     announce("packed_forward tall", dtype, b, n, k)
     _case(oracle, b, n, k, dtype, seed=b + n + k)
 
@@ -127,12 +130,15 @@ def test_packed_forward_fp32_generic_is_bit_exact(oracle, monkeypatch):
         np.testing.assert_array_equal(got, ref)
 
 
+@pytest.mark.parametrize("route", ["auto", "gemm"])
 @pytest.mark.parametrize("b,n,k", [(1, 4096, 4096), (1, 64, 64), (5, 100, 128), (16, 512, 1024), (33, 256, 192),
                                    (200, 260, 448), (512, 1024, 4096)])
-def test_packed_forward_fp32_on_the_matrix_cores(oracle, b, n, k, monkeypatch):
+def test_packed_forward_fp32_on_the_matrix_cores(oracle, b, n, k, monkeypatch, route):
     """fp32 activations with K % 64 == 0 are split into three exact bf16 planes and run on the bf16
     kernels (streaming kernel up to 32 rows, tiled kernel above): every product is exact, only the
     fp32 summation order differs from the generic kernel - far inside the 1e-3 budget for fp32."""
+    if route == "gemm":  # batches beyond 32 rows to the tiled GEMM whatever their size (the default rule streams small outputs)
+        monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
     from bittorch_amd import _C
     from bittorch_amd.quant import pack_ternary_transposed
     announce("packed_forward fp32 planes", b, n, k)

@@ -71,5 +71,5 @@ def test_random_shape_sweep(oracle, b, n, k, dtype, seed):
     if dtype != torch.float32 or k % 64 == 0:
         yt_f = _C.ternary_linear_tiled_forward(x.cuda(), tiled, scale, bias.cuda(), k, n)
         assert rel_err(f32np(yt_f), truth) < (1e-3 if dtype == torch.float32 else 1e-2)
-        if dtype != torch.float32 and (b <= 96 or b > 128):  # the same kernel family runs on either layout
+        if dtype != torch.float32 and b <= 32:  # (beyond, the plans may split K over different numbers of waves)
             assert torch.equal(yt_f, y)

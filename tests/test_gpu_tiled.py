@@ -44,9 +44,12 @@ FWD_SHAPES = [(4096, 4096), (2560, 2560), (6912, 2560), (2560, 6912), (100, 64),
               (11008, 4096)]
 
 
+@pytest.mark.parametrize("route", ["auto", "gemm"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("n,k", FWD_SHAPES)
-def test_tiled_forward_equals_row_major(oracle, dtype, n, k):
+def test_tiled_forward_equals_row_major(oracle, dtype, n, k, route, monkeypatch):
+    if route == "gemm":  # batches beyond 32 rows to the tiled GEMM whatever their size (the default rule streams small outputs)
+        monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
     from bittorch_amd import _C
     _, wt = _packed(oracle, n, k, seed=1)
     tiled = _C.retile_weights(wt, k)
@@ -59,17 +62,20 @@ def test_tiled_forward_equals_row_major(oracle, dtype, n, k):
         res = seeded_acts(b, n, seed=b + 1, dtype=dtype).cuda()
         ref = _C.ternary_linear_packed_forward(x, wt, scale, bias, k, residual=res)
         got = _C.ternary_linear_tiled_forward(x, tiled, scale, bias, k, n, residual=res)
-        if b <= 96 or b > 128:  # both stream the weights / both run the tiled GEMM
+        if b <= 32 or route == "gemm":  # (the tiled GEMMs sum in one order on either layout)
             assert torch.equal(got, ref)
-        else:  # 97..128 rows: the tiled copy is still streamed, the row-major call runs the GEMM (another summation order)
+        else:  # same kernel family on either layout, but the plans may split K over different numbers of waves
             assert rel_err(f32np(got), f32np(ref)) <= 2e-3
     x = seeded_acts(1, k, seed=9, dtype=dtype).cuda()
     assert torch.equal(_C.ternary_linear_tiled_forward(x, tiled, scale[:1], None, k, n),
                        _C.ternary_linear_packed_forward(x, wt, scale[:1], None, k))
 
 
+@pytest.mark.parametrize("route", ["auto", "gemm"])
 @pytest.mark.parametrize("n,k", [(4096, 4096), (100, 64), (2560, 6912)])
-def test_tiled_forward_fp32_planes(oracle, n, k):
+def test_tiled_forward_fp32_planes(oracle, n, k, route, monkeypatch):
+    if route == "gemm":  # batches beyond 32 rows to the tiled GEMM whatever their size (the default rule streams small outputs)
+        monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
     from bittorch_amd import _C
     _, wt = _packed(oracle, n, k, seed=2)
     tiled = _C.retile_weights(wt, k)
@@ -109,8 +115,11 @@ def test_tiled_prologues_equal_row_major(oracle, dtype, n, k):
             assert torch.equal(got, ref)
 
 
+@pytest.mark.parametrize("route", ["auto", "gemm"])
 @pytest.mark.parametrize("n,k", [(4096, 4096), (11008, 4096), (4096, 11008), (100, 64), (37, 100), (260, 192), (520, 1040)])
-def test_tiled_int8_equals_row_major(oracle, n, k):
+def test_tiled_int8_equals_row_major(oracle, n, k, route, monkeypatch):
+    if route == "gemm":  # batches beyond 32 rows to the tiled GEMM whatever their size (the default rule streams small outputs)
+        monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
     from bittorch_amd import _C
     _, wt = _packed(oracle, n, k, seed=4)
     tiled = _C.retile_weights(wt, k)
@@ -164,11 +173,14 @@ def test_module_uses_tiled_copy_for_decode_shapes(oracle, dtype):
     a = _layer(oracle, 640, 512, seed=3)                      # default: tiled copy on first decode call
     b = _layer(oracle, 640, 512, seed=3, decode_tiled=False)  # weight_packed only
     assert a.decode_tiled and a._tiled is None
-    for shape in ((512,), (1, 512), (2, 3, 512), (32, 512), (70, 512)):  # (97..128 rows take different kernels)
+    for shape in ((512,), (1, 512), (2, 3, 512), (32, 512), (70, 512)):
         x = seeded_acts(1, int(np.prod(shape)), seed=len(shape), dtype=dtype).reshape(shape).cuda()
         ya, yb = a(x), b(x)
         assert ya.shape == yb.shape == (*shape[:-1], 640)
-        assert torch.equal(ya, yb)
+        if x.numel() // 512 <= 32:
+            assert torch.equal(ya, yb)
+        else:  # (the two layouts' plans may split K over different numbers of waves)
+            assert rel_err(f32np(ya), f32np(yb)) <= (1e-5 if dtype == torch.float32 else 2e-3)
     assert a._tiled is not None and b._tiled is None
     assert "_tiled" not in a.state_dict() and set(a.state_dict()) == set(b.state_dict())
     # prologues, residual and the int8 path go the same way
@@ -269,8 +281,12 @@ def test_ternary_swiglu_decode_uses_the_output_stage(oracle, dtype):
     for rows in (1, 5, 40, 70):
         announce("TernarySwiGLU decode", dtype, rows)
         x = seeded_acts(rows, d, seed=rows, dtype=dtype).cuda()
-        assert torch.equal(fused(x, nw, 1e-5, residual=x), plain(x, nw, 1e-5, residual=x))
-        assert torch.equal(fused(x), plain(x))
+        if rows <= 32:
+            assert torch.equal(fused(x, nw, 1e-5, residual=x), plain(x, nw, 1e-5, residual=x))
+            assert torch.equal(fused(x), plain(x))
+        else:  # (wider fused layers may split K over another number of waves: same values up to output rounding)
+            assert rel_err(f32np(fused(x, nw, 1e-5, residual=x)), f32np(plain(x, nw, 1e-5, residual=x))) <= 1e-2
+            assert rel_err(f32np(fused(x)), f32np(plain(x))) <= 1e-2
     assert fused.gate_up._tiled is not None
     # the fused layer called as an ordinary linear layer still gives [gate | up] in natural order
     x = seeded_acts(1, d, dtype=dtype).cuda()
