@@ -527,6 +527,30 @@ def main():
                         "forward on the reference-layout W_T beside it",
             }
             del ws, ts
+        # batched decode / short prefill on the config-2 layer (tiled weights): the streaming kernel runs the 16-row
+        # blocks of a call concurrently in one launch; the tiled GEMM (forced with BITTORCH_STREAM_MAX_ROWS) beside it
+        bd = {}
+        n_, k_ = 4096, 4096
+        ws = rand_packed(n_, k_, 8)
+        ts = [_C.retile_weights(w, k_) for w in ws]
+        sc = torch.rand(n_, device=dev) * 0.05 + 0.01
+        for m in (32, 64, 128, 256):
+            xa = acts(m, k_, False)
+            q, s_ = _C.act_quant_int8(xa, True)
+            row = {}
+            for route, env in (("streaming", None), ("tiled_gemm", "16")):
+                if env:
+                    os.environ["BITTORCH_STREAM_MAX_ROWS"] = env
+                _, ev_f = graph_time(lambda i: _C.ternary_linear_tiled_forward(xa, ts[i % 8], sc, None, k_, n_), 40, 5, torch)
+                _, ev_i = graph_time(lambda i: _C.ternary_gemm_int8_tiled(q, s_, ts[i % 8], sc, None, k_, n_, torch.bfloat16,
+                                                                         False, None, True), 40, 5, torch)
+                os.environ.pop("BITTORCH_STREAM_MAX_ROWS", None)
+                row[f"bf16_us_{route}"] = round(ev_f / 40 * 1e3, 2)
+                row[f"int8_us_{route}"] = round(ev_i / 40 * 1e3, 2)
+            row["int8_tops"] = round(2.0 * m * n_ * k_ / (row["int8_us_streaming"] * 1e-6) / 1e12, 1)
+            bd[f"M{m}"] = row
+        extra["batched_decode_N4096_K4096"] = bd
+        del ws, ts
         # quantize + pack of fp32 master weights
         for (n, k) in ((4096, 4096), (11008, 4096)):
             cnt = max(2, int(600e6 // (n * k * 4)))
