@@ -1,6 +1,7 @@
 // Decode-shape / small-batch packed-ternary GEMM for gfx950: streams the 2-bit
 // weights W_T [Kb, N] from HBM once, decodes them in registers and feeds the
-// matrix cores.  Rows of activations per launch: M <= 16 (one MFMA row block).
+// matrix cores.  A workgroup serves one block of M <= 16 activation rows (one MFMA row block);
+// grid.y walks the blocks of a taller call, which run concurrently and share the weights in L2.
 //
 // Arithmetic restated from the reference kernels:
 //   float path (csrc/kernels/ternary_gemm_production.cu:126-141):
