@@ -114,7 +114,7 @@ static const int64_t kMaxKInt8 = 133000;
 // Streaming kernel or tiled GEMM?  The streaming kernel runs the 16-row blocks of a call concurrently in one
 // launch and its time grows with B * N; a tiled GEMM takes the time of one 128 x 256 tile until its tiles
 // fill the chip.  Measured crossovers (five layer shapes, both weight layouts): B * N = 1.5 .. 2.1 M outputs
-// with 16-bit activations, 1.3 .. 2.1 M with int8, i.e. while the GEMM would occupy under a fifth of the
+// with 16-bit activations, 1.8 .. 2.8 M with int8, i.e. while the GEMM would occupy under a fifth of the
 // compute units.  BITTORCH_STREAM_MAX_ROWS=n replaces the rule by "B <= n" (tuning runs).
 static bool prefers_stream(int64_t B, int64_t N, bool int8) {
     if (const char* env = getenv("BITTORCH_STREAM_MAX_ROWS")) {
@@ -122,7 +122,7 @@ static bool prefers_stream(int64_t B, int64_t N, bool int8) {
         if (v >= 1) return B <= v;
     }
     if (B <= 32) return true;
-    return B <= 4096 && B * N <= (int8 ? 1310720 : 1572864);
+    return B <= 4096 && B * N <= (int8 ? 1835008 : 1572864);
 }
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }

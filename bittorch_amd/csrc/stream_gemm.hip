@@ -24,7 +24,7 @@
 //               (rows 4g+q, the same four columns) and exchange bytes with DPP
 //               quad permutes - one load instruction per 16x16 block instead of four;
 //   LD_BYTE     N not a multiple of 4: one byte per lane and row.
-//   LD_T1/2/4   the decode-tiled copy of the weights (W_LAYOUT_TILED, see retile_kernel): the dword
+//   LD_T1/2/4/8 the decode-tiled copy of the weights (W_LAYOUT_TILED, see retile_kernel): the dword
 //               G of every lane and step is stored as such, 256 contiguous bytes per 16-column tile
 //               and step, so a wave's load covers two whole cache lines and needs no transpose
 //               (a 16-column tile of the row-major W_T touches 16 bytes of 16 different lines,
@@ -74,7 +74,7 @@ struct StreamParams {
     int epi_op;
 };
 
-enum { LD_BYTE = 0, LD_Q1 = 1, LD_Q2 = 2, LD_V4 = 4, LD_V8 = 8, LD_V16 = 16, LD_T1 = 101, LD_T2 = 102, LD_T4 = 104 };
+enum { LD_BYTE = 0, LD_Q1 = 1, LD_Q2 = 2, LD_V4 = 4, LD_V8 = 8, LD_V16 = 16, LD_T1 = 101, LD_T2 = 102, LD_T4 = 104, LD_T8 = 108 };
 constexpr int XC_MAX = 4;  // XLDS: 16-byte chunks of the x slice per lane
 
 template <int NB> struct RawVec;
@@ -627,9 +627,11 @@ StreamPlan stream_plan(int mode, int64_t M, int64_t N, int64_t Kb, int w_layout,
         // (every 16-row block of the call is a grid row of the same launch: the workgroups of all blocks count)
         const int min_tiles = (M > 4) ? 160 : 224;
         const int64_t row_blocks = ceil_div(M, 16);
-        int nacc = 4;
+        // (eight tiles per workgroup only for int8 batches of several blocks, whose activation re-reads they halve:
+        // 256 rows at 4096^2 16.3 -> 13.2 us; the 16-bit modes, heavier in decode, lose 5-20 % with them)
+        int nacc = (row_blocks >= 2 && min_nacc == 1 && mode == MODE_I8) ? 8 : 4;
         while (nacc > min_nacc && ceil_div(N, 16 * nacc) * row_blocks < min_tiles) nacc >>= 1;
-        if (o_ld == LD_T1 || o_ld == LD_T2 || o_ld == LD_T4) nacc = o_ld - 100;
+        if (o_ld == LD_T1 || o_ld == LD_T2 || o_ld == LD_T4 || (o_ld == LD_T8 && M > 1 && min_nacc == 1 && mode == MODE_I8)) nacc = o_ld - 100;
         if (nacc < min_nacc) nacc = min_nacc;
         ld = 100 + nacc;
     } else if (N % 4 != 0) {
@@ -648,7 +650,7 @@ StreamPlan stream_plan(int mode, int64_t M, int64_t N, int64_t Kb, int w_layout,
         while (ld > 1 && ceil_div(N, ld_columns(ld)) * row_blocks < min_tiles) ld >>= 1;
     }
     pl.ld = ld;
-    const int max_waves = (ld == 16) ? 4 : (ld == 8 || ld == LD_BYTE) ? 8 : 16;   // LDS: WAVES*TILE_N <= 1024 words per row
+    const int max_waves = (ld == 16) ? 4 : (ld == 8 || ld == LD_BYTE || ld == LD_T8) ? 8 : 16;   // LDS: WAVES*TILE_N <= 1024 words per row
     int waves = (o_waves == 4 || o_waves == 8 || o_waves == 16) ? o_waves : 8;
     if (waves > max_waves) waves = max_waves;
     pl.waves = waves;
@@ -659,7 +661,7 @@ size_t stream_workspace_bytes(int, int64_t, int64_t, int64_t) { return 0; }
 
 template <int MODE, int LD, int WAVES>
 static void launch_stream_k(const StreamParams& p, bool xlds, dim3 grid, size_t lds, hipStream_t st) {
-    constexpr int PF = (LD == 16) ? 2 : (LD == 8) ? 4 : ((LD == 4 || LD == LD_T4) && MODE != MODE_I8) ? 4 : 8;
+    constexpr int PF = (LD == 16) ? 2 : (LD == 8 || LD == LD_T8) ? 4 : ((LD == 4 || LD == LD_T4) && MODE != MODE_I8) ? 4 : 8;
     if constexpr ((LD == LD_T2 || LD == LD_T4) && MODE != MODE_I8) {
         if (p.epi_op == EPI_SWIGLU_PAIRS) {
             if (xlds && p.pro_op == PRO_RMSNORM)
@@ -671,7 +673,7 @@ static void launch_stream_k(const StreamParams& p, bool xlds, dim3 grid, size_t 
             return;
         }
     }
-    if constexpr (LD <= 4 || LD > 100) {  // decode-shape tiles: the M = 1 variant with x staged in LDS
+    if constexpr (LD <= 4 || (LD > 100 && LD != LD_T8)) {  // decode-shape tiles: the M = 1 variant with x staged in LDS
         if (xlds) {
             if constexpr (MODE != MODE_I8) {
                 if (p.pro_op == PRO_RMSNORM) {
@@ -692,7 +694,7 @@ static void launch_stream_k(const StreamParams& p, bool xlds, dim3 grid, size_t 
 
 template <int MODE, int LD>
 static void launch_stream_w(const StreamParams& p, int waves, bool xlds, dim3 grid, size_t lds, hipStream_t st) {
-    if constexpr (LD <= 4 || LD > 100) {
+    if constexpr (LD <= 4 || (LD > 100 && LD != LD_T8)) {
         if (waves == 16) { launch_stream_k<MODE, LD, 16>(p, xlds, grid, lds, st); return; }
     }
     if constexpr (LD <= 8 || LD > 100) {
@@ -708,7 +710,7 @@ static bool xlds_ok(int es, int M, bool x_vec_ok, const StreamPlan& pl, int64_t 
     const int64_t spw = ceil_div(ceil_div(K, 64), pl.waves);
     const size_t red_bytes = (size_t)pl.waves * M * tile_n * 4;
     const size_t xs_bytes = (size_t)pl.waves * XC_MAX * 64 * 16;
-    return M == 1 && x_vec_ok && (pl.ld <= 4 || pl.ld > 100) && spw * 64 * es <= XC_MAX * 64 * 16 && K >= 16 / es &&
+    return M == 1 && x_vec_ok && (pl.ld <= 4 || (pl.ld > 100 && pl.ld != LD_T8)) && spw * 64 * es <= XC_MAX * 64 * 16 && K >= 16 / es &&
            red_bytes + xs_bytes <= 64 * 1024 && !getenv("BITTORCH_STREAM_NOXLDS");
 }
 
@@ -753,6 +755,9 @@ static int launch_stream_mode(StreamParams p, const StreamPlan& pl, hipStream_t 
         case LD_T1: launch_stream_w<MODE, LD_T1>(p, waves, xlds, grid, lds, st); break;
         case LD_T2: launch_stream_w<MODE, LD_T2>(p, waves, xlds, grid, lds, st); break;
         case LD_T4: launch_stream_w<MODE, LD_T4>(p, waves, xlds, grid, lds, st); break;
+        case LD_T8:
+            if constexpr (MODE == MODE_I8) launch_stream_w<MODE, LD_T8>(p, waves, false, grid, lds, st);
+            break;
         default: launch_stream_w<MODE, 0>(p, waves, xlds, grid, lds, st); break;
     }
     return check_launch("stream_gemm");
