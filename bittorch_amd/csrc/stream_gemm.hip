@@ -250,18 +250,6 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p_in) {
     const uint32_t xrow = (uint32_t)min(j, p.M - 1) * (uint32_t)p.K;
     const uint32_t sel_q = 0x0C0C0000u | ((uint32_t)(4 + q) << 8) | (uint32_t)q;
 
-    // epilogue operands of this thread's output column, requested before the weight stream
-    // so that their latency hides behind it (raw bits now, conversion after the reduction)
-    constexpr bool PRE = (WAVES * 64) % TILE_N == 0 && EPI == EPI_NONE;  // a thread finishes one column only
-    uint32_t pre_s = 0u, pre_b = 0u;
-    if constexpr (PRE) {
-        const int64_t n = nb + (int)(threadIdx.x % TILE_N);
-        if ((int)threadIdx.x < p.M * TILE_N && n < p.N) {
-            pre_s = load_bits_rt(p.epi.scale, p.epi.scale_dtype, p.epi.scale_bcast ? 0 : n);
-            if (p.epi.bias) pre_b = load_bits_rt(p.epi.bias, p.epi.bias_dtype, n);
-        }
-    }
-
     // XLDS (M == 1): the wave's K-slice of x, [s_begin*64, (s_begin+spw)*64), as 16-byte
     // chunks, chunk c = lane + 64u; zero beyond K
     uint8_t* xs = (uint8_t*)(red + WAVES * p.M * TILE_N) + (size_t)wave * (XC_MAX * 64 * 16);
@@ -313,14 +301,18 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p_in) {
             }
         }
     };
+    // The single-row variant requests its first batch of weights as early as it can: the activation slice
+    // first (it is needed first, and loads return in order), then the weights, then everything else; the
+    // slice is transformed and parked in LDS while the weights are on their way.
     // RMSNorm prologue: the row's sum of squares, by the whole workgroup (the row is a few KiB and hot
     // in cache), accumulated in fp64 so that its fp32 value does not depend on the summation order.
-    // Its loads are requested first, then the first batch of weights, and only then is the sum formed:
-    // the reduction and its two barriers run while the weights are on their way.
-    constexpr bool PRELOAD = XLDS && MODE != MODE_I8 && PRO == PRO_RMSNORM;
+    // Its loads are requested before the weights, and the sum is formed behind them: the reduction and
+    // its two barriers run while the weights are on their way.
+    constexpr bool PRELOAD = XLDS;
+    constexpr bool PRENORM = XLDS && MODE != MODE_I8 && PRO == PRO_RMSNORM;
     constexpr int PVN = 4;  // 16-byte pieces of the row per thread (the LDS-staged variant's K limit / 8 / threads)
-    uint4 pv[PRELOAD ? PVN : 1];
-    if constexpr (PRELOAD) {
+    uint4 pv[PRENORM ? PVN : 1];
+    if constexpr (PRENORM) {
 #pragma unroll
         for (int u = 0; u < PVN; u++) {
             if (u * WAVES * 64 * 8 < (int)p.K) {  // uniform
@@ -331,8 +323,21 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p_in) {
     }
     uint32_t raw0[PRELOAD ? PF : 1][PRELOAD ? RAWN : 1];
     if constexpr (PRELOAD) load_weights(s_begin, raw0);
+
+    // epilogue operands of this thread's output column, requested early so that their latency hides behind
+    // the weight stream (raw bits now, conversion after the reduction)
+    constexpr bool PRE = (WAVES * 64) % TILE_N == 0 && EPI == EPI_NONE;  // a thread finishes one column only
+    uint32_t pre_s = 0u, pre_b = 0u;
+    if constexpr (PRE) {
+        const int64_t n = nb + (int)(threadIdx.x % TILE_N);
+        if ((int)threadIdx.x < p.M * TILE_N && n < p.N) {
+            pre_s = load_bits_rt(p.epi.scale, p.epi.scale_dtype, p.epi.scale_bcast ? 0 : n);
+            if (p.epi.bias) pre_b = load_bits_rt(p.epi.bias, p.epi.bias_dtype, n);
+        }
+    }
+
     float rstd = 1.0f;
-    if constexpr (PRELOAD) {
+    if constexpr (PRENORM) {
         double ss = 0.0;
 #pragma unroll
         for (int u = 0; u < PVN; u++) {
