@@ -45,28 +45,30 @@
 namespace bt {
 
 struct StreamParams {
+    // what a workgroup needs before it can request its first weights comes first, so that one scalar load
+    // of the kernel arguments covers it
     const void* X;        // MODE_I8: int8 [M,K]; else 16-bit activations [M,K]
     const uint8_t* W_T;   // [Kb, N]
-    const float* s_x;     // MODE_I8: per-row activation scales [M]
-    void* Y;              // [M, N] of y_dtype
-    int32_t* acc_out;     // MODE_I8, optional raw accumulators [M, N]
-    Epilogue epi;
+    const void* pro_b;    // prologue operand (see pro_op below)
     int64_t N, K, Kb;     // K: length of an activation row; Kb: packed weight rows
     int wsteps;           // 16-row steps of W_T; a step index beyond it wraps (see launch_stream)
     int tiles;            // column tiles
     int per_xcd;          // tiles per XCD (grid = 8 * per_xcd)
+    int tiles16;          // LD_T*: 16-column tiles of the decode-tiled weights
     int M;                // 1..16: rows of a 16-row block (of the last one when the launch covers several)
-    int64_t B;            // rows of the whole call: grid.y = ceil(B / 16) blocks of 16 rows, all in one launch
-    int y_dtype;
     int x_vec_ok;         // activation rows may be read with 16-byte loads
+    int64_t B;            // rows of the whole call: grid.y = ceil(B / 16) blocks of 16 rows, all in one launch
+    const float* s_x;     // MODE_I8: per-row activation scales [M]
+    void* Y;              // [M, N] of y_dtype
+    int32_t* acc_out;     // MODE_I8, optional raw accumulators [M, N]
+    Epilogue epi;
+    int y_dtype;
     int prehalved;        // MODE_BF16: the activations already carry the factor 1/2 of the +-2.0 weight decode
     int x_operand_order;  // MODE_I8: X is in the quantizer's operand order (16-byte groups transposed)
-    int tiles16;          // LD_T*: 16-column tiles of the decode-tiled weights
     // Prologue applied to the single activation row on its way into LDS (M = 1, 16-bit modes):
     //   PRO_RMSNORM  x <- rd((x * r) * w),  w = pro_b [K] or ones, r from the whole row and pro_eps
     //   PRO_SWIGLU   x <- rd(rd(silu(x)) * u),  u = pro_b [K]
     int pro_op;
-    const void* pro_b;
     float pro_eps;
     // Output stage (16-bit modes on tiled weights whose 16-column tiles alternate gate, up, gate, up ...):
     //   EPI_SWIGLU_PAIRS  Y [M, N/2]:  Y[b, h] = rd(rd(silu(g)) * u),  g = rd(linear column h), u = rd(linear
@@ -211,7 +213,9 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p_in) {
     if (tile >= p.tiles) return;
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    // (wave-uniform by construction: telling the compiler so moves the K-range and address arithmetic that
+    // derives from it to the scalar unit)
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int j = lane & 15;
     const int g = lane >> 4;
     const int q = lane & 3;
