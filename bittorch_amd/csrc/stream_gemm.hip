@@ -209,7 +209,9 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p_in) {
     }
 
     // consecutive tiles on one XCD (workgroups are dealt round-robin over 8 XCDs)
-    const int tile = (int)(blockIdx.x & 7) * p.per_xcd + (int)(blockIdx.x >> 3);
+    // (per_xcd == 0: a batch of several row blocks over few tiles; workgroups then take tiles in launch order,
+    // which deals every row block's tiles round-robin over the XCDs instead of parking them all on the first few)
+    const int tile = p.per_xcd ? (int)(blockIdx.x & 7) * p.per_xcd + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
     if (tile >= p.tiles) return;
 
     const int lane = threadIdx.x & 63;
@@ -738,7 +740,12 @@ static int launch_stream_mode(StreamParams p, const StreamPlan& pl, hipStream_t 
     const int64_t tile_n = ld_columns(pl.ld);
     p.tiles = (int)ceil_div(p.N, tile_n);
     p.per_xcd = (int)ceil_div(p.tiles, 8);
-    const dim3 grid((unsigned)(p.per_xcd * 8), (unsigned)ceil_div(p.B, 16));
+    unsigned grid_x = (unsigned)(p.per_xcd * 8);
+    if (p.B > 16 && p.tiles % 8 != 0 && p.tiles < 64) {  // few tiles, many row blocks: balance the XCDs instead
+        p.per_xcd = 0;
+        grid_x = (unsigned)p.tiles;
+    }
+    const dim3 grid(grid_x, (unsigned)ceil_div(p.B, 16));
     const int waves = pl.waves;
     const int es = (MODE == MODE_I8) ? 1 : 2;
     const size_t red_bytes = (size_t)waves * p.M * tile_n * 4;
