@@ -112,17 +112,28 @@ static const int64_t kMaxKInt8 = 133000;
 
 // batches up to this many rows go through the streaming (decode-shape) kernel
 // Streaming kernel or tiled GEMM?  The streaming kernel runs the 16-row blocks of a call concurrently in one
-// launch and its time grows with B * N; a tiled GEMM takes the time of one 128 x 256 tile until its tiles
-// fill the chip.  Measured crossovers (five layer shapes, both weight layouts): B * N = 1.5 .. 2.1 M outputs
-// with 16-bit activations, 1.8 .. 2.8 M with int8, i.e. while the GEMM would occupy under a fifth of the
-// compute units.  BITTORCH_STREAM_MAX_ROWS=n replaces the rule by "B <= n" (tuning runs).
-static bool prefers_stream(int64_t B, int64_t N, bool int8) {
+// launch and its time grows with the work, B * N * K; a tiled GEMM takes the time of one 128 x 256 tile, which
+// grows with K only, for every round of 256 tiles.  Both are priced with times fitted to measurements on this
+// chip (five layer shapes, narrow and shallow ones besides, both weight layouts), in microseconds:
+//   streaming  4 + B N K * 2.2e-9 + 0.003 workgroups (int8),  4 + B N K * 5.0e-9 + 0.004 workgroups (16-bit),
+//              workgroups = 16-row blocks x 128- resp. 64-column tiles
+//   GEMM       rounds * (8.6 + 0.0044 K) (int8),  rounds * (6.9 + 0.010 K) (16-bit)
+// which puts the crossover at 1.5 .. 2 M outputs for K = 2560 .. 4096 (the GEMM would occupy under a fifth of
+// the compute units there) and later for shallow layers.  BITTORCH_STREAM_MAX_ROWS=n replaces the rule by
+// "B <= n" (tuning and test runs).
+static bool prefers_stream(int64_t B, int64_t N, int64_t K, bool int8) {
     if (const char* env = getenv("BITTORCH_STREAM_MAX_ROWS")) {
         const long v = atol(env);
         if (v >= 1) return B <= v;
     }
     if (B <= 32) return true;
-    return B <= 4096 && B * N <= (int8 ? 1835008 : 1572864);
+    if (B > 16 * 65535) return false;
+    const double work = (double)B * (double)N * (double)K;
+    const double rounds = (double)ceil_div(ceil_div(B, 128) * ceil_div(N, 256), 256);
+    const double wgs = (double)(ceil_div(B, 16) * ceil_div(N, int8 ? 128 : 64));
+    const double t_stream = 4.0 + work * (int8 ? 2.2e-9 : 5.0e-9) + wgs * (int8 ? 0.003 : 0.004);
+    const double t_gemm = rounds * (int8 ? 8.6 + 0.0044 * (double)K : 6.9 + 0.010 * (double)K);
+    return t_stream < t_gemm;
 }
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -206,7 +217,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         if (x_dtype != BT_F32) {
             const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
             // tall batches: the tiled matrix-core GEMM reads the copy too (not with the SwiGLU output stage)
-            if (!prefers_stream(B, N, false) && epi_op == 0 && gemm_f16_supported_tiled(N, K, X, Y))
+            if (!prefers_stream(B, N, K, false) && epi_op == 0 && gemm_f16_supported_tiled(N, K, X, Y))
                 return launch_gemm_f16(mode, X, W_T, W_LAYOUT_TILED, epi, Y, x_dtype, B, N, K, 1, st);
             return launch_stream(mode, X, 2, nullptr, W_T, W_LAYOUT_TILED, epi, Y, x_dtype, nullptr, B, N, K, 1,
                                  Q_ROW_MAJOR, 0, nullptr, 0.0f, epi_op, st);
@@ -219,7 +230,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         }
         rc = launch_split_f32_planes(X, B, K, workspace, st);
         if (rc) return rc;
-        if (!prefers_stream(B, N, false) && epi_op == 0 && gemm_f16_supported_tiled(N, 3 * K, workspace, Y))
+        if (!prefers_stream(B, N, 3 * K, false) && epi_op == 0 && gemm_f16_supported_tiled(N, 3 * K, workspace, Y))
             return launch_gemm_f16(MODE_BF16, workspace, W_T, W_LAYOUT_TILED, epi, Y, BT_F32, B, N, K, 3, st);
         return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, W_LAYOUT_TILED, epi, Y, BT_F32, nullptr, B, N, K, 3,
                              Q_ROW_MAJOR, 0, nullptr, 0.0f, epi_op, st);
@@ -227,7 +238,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
     if (packed_uses_stream(x_dtype, W_T, Y, N, K)) {
         const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
         // tall batches go to the tiled matrix-core kernel, decode shapes stream the weights
-        if (!prefers_stream(B, N, false) && gemm_f16_supported(N, K, X, W_T, Y))
+        if (!prefers_stream(B, N, K, false) && gemm_f16_supported(N, K, X, W_T, Y))
             return launch_gemm_f16(mode, X, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, x_dtype, B, N, K, 1, st);
         return launch_stream(mode, X, 2, nullptr, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, x_dtype, nullptr, B, N, K, 1, Q_ROW_MAJOR, 0, nullptr, 0.0f, 0, st);
     }
@@ -236,7 +247,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         // (without a workspace the call still succeeds, on the generic kernel)
         rc = launch_split_f32_planes(X, B, K, workspace, st);
         if (rc) return rc;
-        if (!prefers_stream(B, N, false) && gemm_f16_supported(N, 3 * K, workspace, W_T, Y))
+        if (!prefers_stream(B, N, 3 * K, false) && gemm_f16_supported(N, 3 * K, workspace, W_T, Y))
             return launch_gemm_f16(MODE_BF16, workspace, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, BT_F32, B, N, K, 3, st);
         return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, BT_F32, nullptr, B, N, K, 3, Q_ROW_MAJOR, 0, nullptr, 0.0f, 0, st);
     }
@@ -334,14 +345,14 @@ static int gemm_i8_impl(const char* who, const int8_t* Q, int q_layout, const fl
             set_error("%s: tiled weights must be 256-byte aligned and below 4 GiB", who);
             return BT_ERR_INVALID;
         }
-        if (!prefers_stream(B, N, true) && gemm_i8_supported_tiled(N, K, Q))
+        if (!prefers_stream(B, N, K, true) && gemm_i8_supported_tiled(N, K, Q))
             return launch_gemm_i8(Q, q_layout, s_x, W_T, W_LAYOUT_TILED, epi, Y, y_dtype, acc_out, B, N, K, st);
         return launch_stream(MODE_I8, Q, 1, s_x, W_T, w_layout, epi, Y, y_dtype, acc_out, B, N, K, 1, q_layout, 0, nullptr,
                              0.0f, 0, st);
     }
     // decode-shape batches, and any batch whose N the tiled kernel's 4-column
     // vector accesses cannot take, stream the weights once per 16 rows
-    if (prefers_stream(B, N, true) || !gemm_i8_supported(N, K, Q, W_T)) {
+    if (prefers_stream(B, N, K, true) || !gemm_i8_supported(N, K, Q, W_T)) {
         if (!stream_supported(N, K, W_T)) {
             set_error("%s: packed weight matrix of %lld x %lld bytes exceeds the 4 GiB the kernels address", who,
                       (long long)ceil_div(K, 4), (long long)N);
