@@ -251,6 +251,10 @@ def pmc_pass(torch, _C, dev, gemv_steps, x):
     for _ in range(5):
         q, s = _C.act_quant_int8(xa)
         _C.ternary_gemm_int8(q, s, w, sc, None, k, out_dtype=torch.bfloat16)
+    wt = _C.retile_weights(w, k)  # the benchmarked variant: tiled weights, operand-order activations
+    for _ in range(5):
+        q, s = _C.act_quant_int8(xa, True)
+        _C.ternary_gemm_int8_tiled(q, s, wt, sc, None, k, n, torch.bfloat16, False, None, True)
     master = torch.randn(n, k, device=dev) * 0.02
     for _ in range(5):
         _C.ternary_quantize_pack(master, 0.05, True)
