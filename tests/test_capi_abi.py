@@ -100,3 +100,27 @@ def test_gpu_entry_points_reject_cpu_tensors():
         _C.ternary_linear_forward(x, torch.zeros(4, 8), torch.ones(4))
     with pytest.raises(RuntimeError, match="version must be"):
         _C.ternary_linear_tensor_core_forward(x, torch.zeros(2, 4, dtype=torch.uint8), torch.ones(4), None, 8, 3)
+
+
+def test_tiled_copy_size_and_argument_checks_without_a_gpu():
+    """Host-side arithmetic and validation of the tiled-weight entry points (no kernel is launched)."""
+    from bittorch_amd import _lib
+    import numpy as np
+    from oracle import oracle as o
+    lib = _lib.load()
+    for (n, k) in [(4096, 4096), (37, 100), (1, 1), (250, 1030), (11008, 512)]:
+        kb = (k + 3) // 4
+        expect = ((n + 15) // 16) * ((kb + 15) // 16) * 256
+        assert lib.bt_tiled_weights_bytes(n, k) == expect
+        # the oracle's restatement of the layout has exactly that many bytes
+        assert o.retile_weights(np.zeros((kb, n), dtype=np.uint8), k).size == expect
+    assert lib.bt_tiled_weights_bytes(0, 4) == 0
+    buf = ctypes.create_string_buffer(1024)
+    addr = (ctypes.addressof(buf) + 255) & ~255
+    assert lib.bt_retile_weights(None, 16, 64, 0, addr, None) == -1
+    assert "bt_retile_weights" in _lib.last_error()
+    assert lib.bt_retile_weights(addr, 16, 64, 0, addr + 4, None) == -1      # tiled copy not 256-byte aligned
+    assert "aligned" in _lib.last_error()
+    assert lib.bt_retile_weights(addr, 48, 64, 1, addr, None) == -1          # pair order needs N % 32 == 0
+    assert "N % 32" in _lib.last_error()
+    assert lib.bt_retile_weights(addr, 16, 64, 7, addr, None) == -1          # unknown tile order
