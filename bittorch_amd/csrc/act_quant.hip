@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const void* __restrict__
         uint32_t lo = 0, hi = 0;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            float r = roundf(__fmul_rn(v[e], inv));
+            float r = round_half_away(__fmul_rn(v[e], inv));
             r = fmaxf(-127.0f, fminf(127.0f, r));
             const uint32_t byte = (uint32_t)(uint8_t)(int8_t)(int)r;
             if (e < 4) lo |= byte << (8 * e);
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(256) void act_quant_row_kernel(const void* __restri
         uint32_t lo = 0, hi = 0;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            float r = roundf(__fmul_rn(v[i][e], inv));
+            float r = round_half_away(__fmul_rn(v[i][e], inv));
             r = fmaxf(-127.0f, fminf(127.0f, r));
             const uint32_t byte = (uint32_t)(uint8_t)(int8_t)(int)r;
             if (e < 4) lo |= byte << (8 * e);

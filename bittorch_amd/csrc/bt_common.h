@@ -212,6 +212,14 @@ constexpr uint32_t LUT_BF16_TWO = 0x00C04000u;  // sel 0..3 -> 0x00, 0x40, 0xC0,
 // 16-byte group stored as the 4x4 byte transpose of its natural order (byte 4c+r holds element
 // 4r+c): the k order in which the in-register weight decode lays out an MFMA operand, so that the
 // GEMMs feed activations to the matrix cores without permuting them first.
+// roundf (halves away from zero) in three operations: add the largest float below one half, with the sign of
+// x, and truncate.  Exact for every float: below 2^23 the sum rounds to the next integer precisely when the
+// fraction is at least one half (x + 0.5 - 2^-25 lies at most half a grid step below that integer, and the
+// tie at 1 - 2^-25 goes to the even 1.0); from 2^23 on x is an integer and the sum is x.
+__device__ __forceinline__ float round_half_away(float x) {
+    return truncf(__fadd_rn(x, copysignf(0.49999997f, x)));
+}
+
 enum { Q_ROW_MAJOR = 0, Q_OPERAND_ORDER = 1 };
 
 // Layouts of the packed weights the streaming kernel reads.

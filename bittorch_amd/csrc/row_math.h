@@ -45,7 +45,7 @@ __device__ __forceinline__ float rms_rstd(double ss, int K, float eps) {
     return __fdiv_rn(1.0f, sqrtf(__fadd_rn(ms, eps)));
 }
 __device__ __forceinline__ int8_t quant_i8(float v, float inv) {
-    float r = roundf(__fmul_rn(v, inv));
+    float r = round_half_away(__fmul_rn(v, inv));
     r = fmaxf(-127.0f, fminf(127.0f, r));
     return (int8_t)(int)r;
 }
