@@ -39,6 +39,8 @@ SIGNATURES = {
     "bt_tensor_core_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "bt_ternary_linear_tensor_core_forward": (_int, [_vp, _int, _vp, _vp, _int, _i64, _vp, _int, _vp,
                                                      _i64, _i64, _i64, _vp, _sz, _vp]),
+    "bt_ternary_linear_tensor_core_forward_static": (_int, [_vp, _int, _vp, _vp, _int, _i64, _vp, _int, _vp,
+                                                            _i64, _i64, _i64, _vp]),
     "bt_unpack_dequant": (_int, [_vp, _vp, _i64, _vp, _int, _i64, _i64, _vp]),
     "bt_pack_ternary_i8": (_int, [_vp, _i64, _i64, _vp, _vp]),
     "bt_probe_mfma_i8": (_int, [_int, _int, _int, _vp, _vp, _vp]),

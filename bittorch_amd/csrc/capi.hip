@@ -4,6 +4,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 #include "bt_common.h"
 
@@ -413,6 +414,69 @@ extern "C" int bt_ternary_linear_tensor_core_forward(const void* X, int x_dtype,
     (void)gemm_bytes;
     return gemm_i8_impl(who, Q, q_layout, s_x, W_T, W_LAYOUT_ROW_MAJOR, scale, scale_dtype, scale_len, bias, bias_dtype, nullptr,
                         Y, x_dtype, nullptr, B, N, K, stream);
+}
+
+// ---- the matrix-core forward for callers that cannot allocate ----------------------------------
+// The int8 activations Q and their row scales, which bt_ternary_linear_tensor_core_forward keeps in the caller's
+// workspace, live in a device array of this library instead.  Host code must never hand the array's
+// name to a kernel (there it is a host-side stand-in, not a device address): the device address is
+// asked for once per device with hipGetSymbolAddress and only that pointer is used afterwards.
+namespace bt {
+constexpr size_t kStaticQBytes = BT_STATIC_SCRATCH_ACTIVATION_BYTES;  // int8 activations: B * K bytes at most
+constexpr size_t kStaticRows = BT_STATIC_SCRATCH_ROWS;               // row scales: B at most
+constexpr size_t kStaticBytes = kStaticQBytes + kStaticRows * sizeof(float);
+constexpr int kStaticMaxDevices = 64;
+}  // namespace bt
+static __device__ __align__(256) unsigned char scratch[bt::kStaticBytes];
+static void* g_scratch_ptr[bt::kStaticMaxDevices];  // per device: each GPU holds its own copy of the array
+static std::mutex g_scratch_mutex;
+
+// device address of `scratch` on the current device (looked up on the first call per device)
+static int static_scratch_ptr(const char* who, unsigned char** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kStaticMaxDevices) {
+        set_error("%s: cannot identify the current device (%s, device %d)", who, hipGetErrorString(e), dev);
+        return BT_ERR_LAUNCH;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            set_error("%s: hipGetSymbolAddress(scratch) failed on device %d: %s", who, dev, hipGetErrorString(e));
+            return BT_ERR_LAUNCH;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = (unsigned char*)g_scratch_ptr[dev];
+    return BT_OK;
+}
+
+extern "C" int bt_ternary_linear_tensor_core_forward_static(const void* X, int x_dtype, const uint8_t* W_T,
+                                                            const void* scale, int scale_dtype, int64_t scale_len,
+                                                            const void* bias, int bias_dtype, void* Y, int64_t B,
+                                                            int64_t N, int64_t K, void* stream) {
+    const char* who = "bt_ternary_linear_tensor_core_forward_static";
+    int rc = check_shape(who, X, W_T, Y, x_dtype, B, N, K);
+    if (rc) return rc;
+    if ((uint64_t)B > kStaticRows || (uint64_t)K > kStaticQBytes || (uint64_t)B * (uint64_t)K > kStaticQBytes) {
+        set_error("%s: B*K = %lld x %lld exceeds the library's static scratch (B*K <= %zu bytes, B <= %zu rows); "
+                  "use bt_ternary_linear_tensor_core_forward with a workspace", who, (long long)B, (long long)K,
+                  kStaticQBytes, kStaticRows);
+        return BT_ERR_WORKSPACE;
+    }
+    unsigned char* base = nullptr;
+    rc = static_scratch_ptr(who, &base);
+    if (rc) return rc;
+    int8_t* Q = (int8_t*)base;
+    float* s_x = (float*)(base + kStaticQBytes);
+    // both are written in full by the quantizer before the GEMM reads them: nothing has to start at zero
+    const int q_layout = (K % 16 == 0 && ((uintptr_t)X) % 16 == 0) ? Q_OPERAND_ORDER : Q_ROW_MAJOR;
+    rc = launch_act_quant(X, x_dtype, B, K, Q, s_x, q_layout, (hipStream_t)stream);
+    if (rc) return rc;
+    return gemm_i8_impl(who, Q, q_layout, s_x, W_T, W_LAYOUT_ROW_MAJOR, scale, scale_dtype, scale_len, bias, bias_dtype,
+                        nullptr, Y, x_dtype, nullptr, B, N, K, stream);
 }
 
 // ---- fused producers of the GEMM activations (row_ops.hip) ----------------------------------

@@ -262,6 +262,26 @@ int bt_ternary_linear_tensor_core_forward(const void* X, int x_dtype, const uint
                                           size_t workspace_bytes, void* stream);
 
 /*
+ * bt_ternary_linear_tensor_core_forward for callers that cannot allocate device memory or pass a
+ * workspace: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * It has no counterpart in the reference.  Same arguments and bit-identical results; the int8
+ * activations and their row scales live in a device array inside the library
+ * (BT_STATIC_SCRATCH_ACTIVATION_BYTES + 4 * BT_STATIC_SCRATCH_ROWS bytes, held by every GPU the
+ * library runs on until the process ends) instead of a workspace.  The call allocates and frees
+ * nothing.  Limits: B * K <= BT_STATIC_SCRATCH_ACTIVATION_BYTES and B <= BT_STATIC_SCRATCH_ROWS,
+ * otherwise BT_ERR_WORKSPACE.  All calls on one GPU share the array: calls that may overlap on one
+ * GPU (different streams, different host threads) race; the array needs no clearing between calls
+ * (the quantizer writes everything the GEMM reads).  The first call on a device looks the array's
+ * device address up (hipGetSymbolAddress): make that call outside a stream capture.
+ */
+#define BT_STATIC_SCRATCH_ACTIVATION_BYTES (16u << 20)
+#define BT_STATIC_SCRATCH_ROWS 65536
+int bt_ternary_linear_tensor_core_forward_static(const void* X, int x_dtype, const uint8_t* W_T,
+                                                 const void* scale, int scale_dtype, int64_t scale_len,
+                                                 const void* bias, int bias_dtype, void* Y, int64_t B,
+                                                 int64_t N, int64_t K, void* stream);
+
+/*
  * Packed weights -> dense ternary or effective weights, for the training
  * backward (grad_x = grad_y @ (w_tern * scale)) without keeping a dense copy
  * alive between forward and backward (the reference saves one,
