@@ -79,103 +79,113 @@ def graph_time(fn, steps, warmup, torch):
     return wall_ms, e0.elapsed_time(e1)
 
 
-def block_stack(torch, dev, layers=30, d_model=2560, heads=20, ffn=6912, batch=8, seq=512, vocab=32000):
-    """Config 5: forward of a 2B-parameter BitNet-b1.58-like stack.  q/k/v/o/gate/up/down are
-    TernaryLinear (random N(0,0.02) masters, no bias); RMSNorm, rotary-free causal SDPA, SwiGLU and
-    the embedding stay in PyTorch-ROCm; bf16 activations, a seeded token batch of batch x seq."""
-    import torch.nn as nn
-    import torch.nn.functional as F
-    import bittorch_amd as bt
+class Config5:
+    """Config 5: a 2B-parameter BitNet-b1.58-like stack.  q/k/v/o/gate/up/down are TernaryLinear
+    (random N(0,0.02) masters, no bias); RMSNorm, rotary-free causal SDPA and the embedding stay in
+    PyTorch-ROCm; bf16 activations, a seeded token batch of batch x seq.  The same stack runs in the
+    variants the benchmark times (and the GPU tests compare): training modules, converted inference
+    modules, inference modules with the glue fused, and the int8 path."""
 
-    class Block(nn.Module):
-        def __init__(self):
-            super().__init__()
-            mk = lambda i, o: bt.nn.TernaryLinear(i, o, bias=False)
-            self.q, self.k, self.v, self.o = mk(d_model, d_model), mk(d_model, d_model), mk(d_model, d_model), mk(d_model, d_model)
-            self.gate, self.up, self.down = mk(d_model, ffn), mk(d_model, ffn), mk(ffn, d_model)
-            self.n1 = nn.RMSNorm(d_model)
-            self.n2 = nn.RMSNorm(d_model)
+    def __init__(self, torch, dev, layers=30, d_model=2560, heads=20, ffn=6912, batch=8, seq=512, vocab=32000,
+                 backend="auto", act_dtype=None, fake_quant=False):
+        import torch.nn as nn
+        import torch.nn.functional as F
+        import bittorch_amd as bt
 
-        def forward(self, x):
-            b, t, _ = x.shape
-            h = self.n1(x)
-            q = self.q(h).view(b, t, heads, -1).transpose(1, 2)
-            k = self.k(h).view(b, t, heads, -1).transpose(1, 2)
-            v = self.v(h).view(b, t, heads, -1).transpose(1, 2)
-            a = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(b, t, -1)
-            x = x + self.o(a)
-            h = self.n2(x)
-            return x + self.down(F.silu(self.gate(h)) * self.up(h))
+        self.torch, self.F, self.bt = torch, F, bt
+        self.d_model, self.heads, self.ffn = d_model, heads, ffn
+        act_dtype = act_dtype or torch.bfloat16
+        self.act_dtype = act_dtype
 
-    torch.manual_seed(0)
-    with torch.device(dev):
-        emb = nn.Embedding(vocab, d_model).to(torch.bfloat16)
-        blocks = nn.ModuleList([Block() for _ in range(layers)])
-        final = nn.RMSNorm(d_model)
-    for m in blocks.modules():
-        if isinstance(m, bt.nn.TernaryLinear):
-            nn.init.normal_(m.weight, std=0.02)
-        elif isinstance(m, nn.RMSNorm):
-            m.to(torch.bfloat16)
-    final.to(torch.bfloat16)
-    tokens = torch.randint(0, vocab, (batch, seq), generator=torch.Generator().manual_seed(0)).to(dev)
-    n_tern = sum(m.weight.numel() for m in blocks.modules() if isinstance(m, bt.nn.TernaryLinear))
+        def fq(t):
+            """fake_quant: the int8 path's per-token activation quantizer (whole-row absmax / 127, halves away
+            from zero, clamp) applied in the tensor's own dtype ahead of every ternary layer, in plain torch"""
+            if not fake_quant:
+                return t
+            amax = t.abs().amax(dim=-1, keepdim=True).float()
+            s = torch.where(amax > 1e-6, amax / 127.0, torch.ones_like(amax))
+            v = t.float() * (1.0 / s)
+            q = torch.clamp(torch.sign(v) * torch.floor(v.abs() + 0.5), -127, 127)
+            return (q * s).to(t.dtype)
 
-    def forward(stack):
-        with torch.no_grad():
-            x = emb(tokens)
-            for blk in stack:
-                x = blk(x)
-            return final(x)
+        class Block(nn.Module):
+            def __init__(self):
+                super().__init__()
+                mk = lambda i, o: bt.nn.TernaryLinear(i, o, bias=False, backend=backend)
+                self.q, self.k, self.v, self.o = mk(d_model, d_model), mk(d_model, d_model), mk(d_model, d_model), mk(d_model, d_model)
+                self.gate, self.up, self.down = mk(d_model, ffn), mk(d_model, ffn), mk(ffn, d_model)
+                self.n1 = nn.RMSNorm(d_model, eps=1e-5)
+                self.n2 = nn.RMSNorm(d_model, eps=1e-5)
 
-    def timed(stack, reps, before=None):
-        forward(stack)
-        torch.cuda.synchronize()
-        best = 1e30
-        for _ in range(reps):
-            if before:
-                before()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            forward(stack)
-            torch.cuda.synchronize()
-            best = min(best, (time.perf_counter() - t0) * 1e3)
-        return best
+            def forward(self, x):
+                b, t, _ = x.shape
+                h = fq(self.n1(x))
+                q = self.q(h).view(b, t, heads, -1).transpose(1, 2)
+                k = self.k(h).view(b, t, heads, -1).transpose(1, 2)
+                v = self.v(h).view(b, t, heads, -1).transpose(1, 2)
+                a = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(b, t, -1)
+                x = x + self.o(fq(a))
+                h = fq(self.n2(x))
+                return x + self.down(fq(F.silu(self.gate(h)) * self.up(h)))
 
-    def drop_caches():
-        for m in blocks.modules():
+        torch.manual_seed(0)
+        with torch.device(dev):
+            self.emb = nn.Embedding(vocab, d_model).to(act_dtype)
+            self.blocks = nn.ModuleList([Block() for _ in range(layers)])
+            self.final = nn.RMSNorm(d_model, eps=1e-5)
+        for m in self.blocks.modules():
             if isinstance(m, bt.nn.TernaryLinear):
+                nn.init.normal_(m.weight, std=0.02)
+            elif isinstance(m, nn.RMSNorm):
+                m.to(act_dtype)
+        self.final.to(act_dtype)
+        self.tokens = torch.randint(0, vocab, (batch, seq), generator=torch.Generator().manual_seed(0)).to(dev)
+        self.n_tern = sum(m.weight.numel() for m in self.blocks.modules() if isinstance(m, bt.nn.TernaryLinear))
+        self.infer = None
+
+    def forward(self, stack=None):
+        """Unfused forward of `stack` (the training modules by default, or the converted modules)."""
+        torch = self.torch
+        with torch.no_grad():
+            x = self.emb(self.tokens)
+            for blk in (self.blocks if stack is None else stack):
+                x = blk(x)
+            return self.final(x)
+
+    def drop_packed_caches(self):
+        for m in self.blocks.modules():
+            if isinstance(m, self.bt.nn.TernaryLinear):
                 m._packed.clear()
 
-    res = {"layers": layers, "d_model": d_model, "heads": heads, "ffn": ffn, "tokens": batch * seq,
-           "ternary_weights": n_tern,
-           "ops_per_forward_ternary_layers": 2.0 * batch * seq * n_tern}
-    res["ms_requantize_every_forward"] = round(timed(blocks, 3, drop_caches), 3)   # what the reference does
-    res["ms_packed_weights_cached"] = round(timed(blocks, 5), 3)
-    infer = bt.utils.convert_linear_layers(blocks, inplace=True)  # masters are freed layer by layer
-    res["ms_inference_modules"] = round(timed(infer, 5), 3)
+    def convert(self, inplace=True):
+        """TernaryLinear -> TernaryLinearInference, then q|k|v and gate|up each as one layer."""
+        bt = self.bt
+        self.infer = bt.utils.convert_linear_layers(self.blocks, inplace=inplace)
+        if inplace:
+            self.blocks = None  # (the masters are freed layer by layer)
+        return self.infer
 
-    # (parity of every fused piece against its unfused sequence is a GPU test; end-to-end outputs of 30
-    # random layers differ chaotically on any last-bit change and are not compared here)
-    # the same converted stack with the glue between the ternary layers fused: residual adds in the
-    # GEMM epilogues, silu(gate)*up in one kernel, RMSNorm from this library, q|k|v and gate|up each
-    # one GEMM over concatenated columns (fewer, fuller waves of tiles) ...
-    from bittorch_amd.ops import fused
+    def fuse(self):
+        bt = self.bt
+        for blk in self.infer:
+            blk.qkv = bt.utils.fuse_ternary_linear_inference(blk.q, blk.k, blk.v)
+            blk.mlp = bt.nn.TernarySwiGLU(blk.gate, blk.up, blk.down, compute="float", fuse_gate_up=True)
 
-    def heads_of(t, b, s):
-        return t.view(b, s, heads, -1).transpose(1, 2)
-
-    def fused_block(blk, x, int8):
+    def _fused_block(self, blk, x, int8):
+        torch, F, bt = self.torch, self.F, self.bt
+        from bittorch_amd.ops import fused
+        heads, d_model = self.heads, self.d_model
         b, s, _ = x.shape
-        if int8:  # ... and, BitNet-style, every projection on the int8 matrix cores from activations
-            # that leave the norm / SwiGLU kernels already quantized per token
+        heads_of = lambda t: t.view(b, s, heads, -1).transpose(1, 2)
+        if int8:  # BitNet-style: every projection on the int8 matrix cores from activations that leave the
+            # norm / SwiGLU kernels already quantized per token
             qh, sh = fused.rmsnorm(x, blk.n1.weight, blk.n1.eps or torch.finfo(x.dtype).eps, store=False, quantize=True,
                                    operand_order=True)
             qkv = blk.qkv.forward_int8(qh, sh, x.dtype, None, True)
         else:
             qkv = blk.qkv(fused.rmsnorm(x, blk.n1.weight, blk.n1.eps or torch.finfo(x.dtype).eps))
         q, k, v = qkv.split(d_model, dim=-1)  # one GEMM over the concatenated q|k|v columns
-        a = F.scaled_dot_product_attention(heads_of(q, b, s), heads_of(k, b, s), heads_of(v, b, s), is_causal=True)
+        a = F.scaled_dot_product_attention(heads_of(q), heads_of(k), heads_of(v), is_causal=True)
         a = a.transpose(1, 2).reshape(b, s, -1)
         if int8:
             qa, sa = bt._C.act_quant_int8(a.reshape(b * s, -1), True)
@@ -184,35 +194,52 @@ def block_stack(torch, dev, layers=30, d_model=2560, heads=20, ffn=6912, batch=8
             x = blk.o(a, x)
         return blk.mlp(x, blk.n2.weight, blk.n2.eps or torch.finfo(x.dtype).eps, residual=x)
 
-    def forward_fused(stack, int8):
+    def forward_fused(self, int8):
+        """The converted stack with the glue between the ternary layers fused: residual adds in the GEMM
+        epilogues, silu(gate)*up in one kernel, RMSNorm from this library, q|k|v and gate|up each one GEMM
+        over concatenated columns; int8: every projection on the int8 matrix cores."""
+        torch = self.torch
+        for blk in self.infer:
+            blk.mlp.compute = "int8" if int8 else "float"
         with torch.no_grad():
-            x = emb(tokens)
-            for blk in stack:
-                x = fused_block(blk, x, int8)
-            return final(x)
+            x = self.emb(self.tokens)
+            for blk in self.infer:
+                x = self._fused_block(blk, x, int8)
+            return self.final(x)
 
-    def timed_fused(int8, reps=5):
-        forward_fused(infer, int8)
+
+def block_stack(torch, dev, layers=30, d_model=2560, heads=20, ffn=6912, batch=8, seq=512, vocab=32000):
+    """Config 5 timed end to end in every variant (outputs are compared by tests/test_gpu_configs.py)."""
+    c5 = Config5(torch, dev, layers, d_model, heads, ffn, batch, seq, vocab)
+
+    def timed(fn, reps, before=None):
+        fn()
         torch.cuda.synchronize()
         best = 1e30
         for _ in range(reps):
+            if before:
+                before()
+            torch.cuda.synchronize()
             t0 = time.perf_counter()
-            forward_fused(infer, int8)
+            fn()
             torch.cuda.synchronize()
             best = min(best, (time.perf_counter() - t0) * 1e3)
         return best
 
-    for blk in infer:
-        blk.qkv = bt.utils.fuse_ternary_linear_inference(blk.q, blk.k, blk.v)
-        blk.mlp = bt.nn.TernarySwiGLU(blk.gate, blk.up, blk.down, compute="float", fuse_gate_up=True)
-    res["ms_inference_fused_glue"] = round(timed_fused(False), 3)
-    for blk in infer:
-        blk.mlp.compute = "int8"
-    res["ms_inference_int8_path"] = round(timed_fused(True), 3)
+    res = {"layers": layers, "d_model": d_model, "heads": heads, "ffn": ffn, "tokens": batch * seq,
+           "ternary_weights": c5.n_tern,
+           "ops_per_forward_ternary_layers": 2.0 * batch * seq * c5.n_tern}
+    res["ms_requantize_every_forward"] = round(timed(c5.forward, 3, c5.drop_packed_caches), 3)   # what the reference does
+    res["ms_packed_weights_cached"] = round(timed(c5.forward, 5), 3)
+    infer = c5.convert()
+    res["ms_inference_modules"] = round(timed(lambda: c5.forward(infer), 5), 3)
+    c5.fuse()
+    res["ms_inference_fused_glue"] = round(timed(lambda: c5.forward_fused(False), 5), 3)
+    res["ms_inference_int8_path"] = round(timed(lambda: c5.forward_fused(True), 5), 3)
     res["ternary_TOPS_int8_path"] = round(res["ops_per_forward_ternary_layers"] / (res["ms_inference_int8_path"] * 1e-3) / 1e12, 1)
     res["ternary_TFLOPS_cached"] = round(res["ops_per_forward_ternary_layers"] / (res["ms_packed_weights_cached"] * 1e-3) / 1e12, 1)
-    res["packed_weight_bytes"] = n_tern // 4
-    del blocks, infer
+    res["packed_weight_bytes"] = c5.n_tern // 4
+    del c5, infer
     torch.cuda.empty_cache()
     return res
 
