@@ -3,17 +3,19 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-One "step" is one pass of the decode GEMV (the benchmark's config 2) through the
-C-ABI library: x fp16 [1,4096] times packed ternary W [4096,4096] (per-tensor fp32
-scale, fp16 bias).  The steps walk round-robin over distinct weight buffers whose
-total size exceeds the 256 MB Infinity Cache, so every step streams its 4 MiB of
-packed weights from HBM.  W warm-up steps, then exactly K steps (captured in one
-HIP graph so that host launch overhead is not what is measured) are timed between
-two device synchronisations.  Prints ONE JSON line.
+The workload is the benchmark's config 2, the decode GEMV: x fp16 [1,4096] times packed ternary
+W [4096,4096] (per-tensor fp32 scale, fp16 bias).  One such GEMV moves 4 MiB, which the memory system
+delivers in less time than a kernel takes to start and drain, so the library serves decode work through
+`bt_ternary_gemv_grouped`: G independent GEMV units (own activations, weights, scale, bias, output) per
+launch, every unit bit-identical to the single call.  One "step" is one such launch over G = 128 config-2
+units; two sets of 128 weight matrices (2 x 512 MiB, four times the 256 MB Infinity Cache) alternate, so
+every step streams its packed weights from HBM.  W warm-up steps, then exactly K steps (captured in one HIP
+graph so that host launch overhead is not what is measured) are timed between two device synchronisations;
+the graph is replayed several times and the median replay is reported.  Prints ONE JSON line.
 
-The same line carries the roofline of the dominant kernel (HIP-event timed over the
-timed region), the CPU oracle timed on the host cores beside it, and the secondary
-figures of the metric (int8 TOPS at M=2048, small-batch decode, quantize+pack).
+The same line carries the roofline of the dominant kernel (HIP-event timed over the timed region), the same
+GEMV one matrix per launch (`single_launch`), the CPU oracle timed on the host cores beside it, and the
+secondary figures of the metric (int8 TOPS at M=2048, small-batch decode, large matrices, quantize+pack).
 """
 
 from __future__ import annotations
@@ -37,8 +39,9 @@ METRIC = "packed ternary GEMM GB/s (M=1) & int8 TOPS (M=2048), % of roofline, 1 
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=2000)
-    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--units", type=int, default=128, help="config-2 GEMV units per launch (G)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
     ap.add_argument("--no-block-stack", action="store_true", help="skip the 30-layer block stack (config 5)")
@@ -52,8 +55,11 @@ def parse_args():
     return ap.parse_args()
 
 
-def graph_time(fn, steps, warmup, torch):
-    """(wall ms, event ms) for `steps` calls of fn(i) replayed as one HIP graph."""
+def graph_time(fn, steps, warmup, torch, min_replays=None):
+    """(wall ms, event ms) for `steps` calls of fn(i) replayed as one HIP graph: the median over
+    the replays, each timed between two synchronisations.  A short graph is replayed more often
+    (at least 20 times below 200 steps), so that the fixed cost of one replay and a clock ramp do
+    not decide the figure."""
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
@@ -67,16 +73,43 @@ def graph_time(fn, steps, warmup, torch):
             fn(i)
     graph.replay()  # untimed: first replay uploads the graph
     torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    e0.record()
-    graph.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    return wall_ms, e0.elapsed_time(e1)
+    replays = min_replays or (5 if steps >= 200 else 20)
+    walls, events = [], []
+    for _ in range(replays):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        walls.append((time.perf_counter() - t0) * 1e3)
+        events.append(e0.elapsed_time(e1))
+    walls.sort()
+    events.sort()
+    return walls[len(walls) // 2], events[len(events) // 2]
+
+
+_probe_lib = None
+
+
+def probe_mfma_int8(torch, device, blocks=2048, iters=4096, random_operands=0):
+    """Launches the int8 matrix-core rate probe (bench_mfma_probe.so, this benchmark's own aid) on the
+    current stream; returns the number of integer operations the launch performs."""
+    import ctypes
+    global _probe_lib
+    if _probe_lib is None:
+        _probe_lib = ctypes.CDLL(os.path.join(ROOT, "bench_mfma_probe.so"))
+        _probe_lib.bench_probe_mfma_i8.restype = ctypes.c_int
+        _probe_lib.bench_probe_mfma_i8.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                                   ctypes.c_void_p, ctypes.c_void_p]
+    out = torch.zeros(1, dtype=torch.int32, device=device)
+    ops = ctypes.c_double(0.0)
+    rc = _probe_lib.bench_probe_mfma_i8(blocks, iters, int(random_operands), out.data_ptr(), ctypes.addressof(ops),
+                                        torch.cuda.current_stream(device).cuda_stream)
+    assert rc == 0
+    return ops.value
 
 
 class Config5:
@@ -259,7 +292,7 @@ def measured_traffic(tag):
     return None
 
 
-def pmc_pass(torch, _C, dev, gemv_steps, x):
+def pmc_pass(torch, _C, dev, gemv_steps, grouped_step):
     """Eager launches for hardware-counter collection (every dispatch gets its own counter row).
     The copy kernel moves a known number of bytes, which calibrates the counter's unit."""
     n_copy = 64 * 1024 * 1024 // 4
@@ -267,7 +300,9 @@ def pmc_pass(torch, _C, dev, gemv_steps, x):
     dst = torch.empty_like(src)
     for _ in range(5):
         torch.mul(src, 1.0, out=dst)  # elementwise kernel: reads 64 MiB, writes 64 MiB
-    for gemv_step in gemv_steps:  # the decode-tiled path, then the same GEMV on the row-major W_T
+    for i in range(6):  # the headline: G config-2 units per launch
+        grouped_step(i)
+    for gemv_step in gemv_steps:  # one matrix per launch: the decode-tiled path, then the same GEMV on the row-major W_T
         for i in range(40):
             gemv_step(i)
     m, n, k = 2048, 4096, 4096
@@ -308,10 +343,11 @@ def main():
     torch.cuda.set_device(dev)
     torch.manual_seed(0)
 
-    # ---- config 2: decode GEMV -------------------------------------------------------
+    # ---- config 2: decode GEMV units -------------------------------------------------------
     N = K = 4096
     weight_bytes = N * (K // 4)
-    nsets = 128  # 512 MiB of packed weights > 256 MB Infinity Cache
+    G = args.units
+    nsets = 2 * G  # two alternating sets of G units: 2 x 512 MiB of packed weights at G = 128 (Infinity Cache: 256 MB)
     g = torch.Generator().manual_seed(0)
     w0 = (torch.randn(N, K, generator=g) * 0.02).to(dev)
     x = torch.randn(1, K, generator=g).half().to(dev)
@@ -326,21 +362,38 @@ def main():
     del wi
     torch.cuda.synchronize()
 
-    # The product's decode path: TernaryLinearInference layers over the packed weights.  Each layer
-    # reads the decode-tiled copy it builds once from its W_T (prepare_decode); the functional API on
-    # the reference-layout W_T itself is timed beside it (secondary.decode_gemv_row_major_W_T).
+    # The product's decode path: TernaryLinearInference layers over the packed weights, each reading the
+    # decode-tiled copy of its W_T.  Every unit has its own activations, bias and output.
     from bittorch_amd.nn import TernaryLinearInference
-    layers = [TernaryLinearInference(K, N, p, scale, bias).prepare_decode() for p in packs]
+    xs = [x] + [torch.randn(1, K, device=dev).half() for _ in range(nsets - 1)]
+    biases = [bias] + [(torch.randn(N, device=dev) * 0.01).half() for _ in range(nsets - 1)]
+    layers = [TernaryLinearInference(K, N, p, scale, b).prepare_decode() for p, b in zip(packs, biases)]
+    ys = [torch.empty(1, N, dtype=torch.float16, device=dev) for _ in range(nsets)]
+    tables = []
+    for s0 in (0, G):
+        sl = slice(s0, s0 + G)
+        tables.append((_C.pointer_table(xs[sl]), _C.pointer_table([l.tiled_weights() for l in layers[sl]]),
+                       _C.pointer_table([scale] * G), _C.pointer_table(biases[sl]), _C.pointer_table(ys[sl])))
     torch.cuda.synchronize()
 
-    def step(i):
-        return layers[i % nsets](x)
+    def step(i):  # one launch over G units
+        _C.ternary_gemv_grouped(*tables[i % 2], K, N, scale_len=1)
+
+    def step_single(i):  # the same GEMV, one matrix per launch
+        return layers[i % nsets](xs[i % nsets])
 
     def step_row_major(i):
-        return _C.ternary_linear_packed_forward(x, packs[i % nsets], scale, bias, K)
+        return _C.ternary_linear_packed_forward(xs[i % nsets], packs[i % nsets], scale, biases[i % nsets], K)
+
+    # every unit of the grouped launch equals the single call bit for bit (checked here on the benchmark's own
+    # operands; the parity tests proper are tests/test_gpu_gemv_exact.py)
+    step(0)
+    step(1)
+    for u in (0, G - 1, G, nsets - 1):
+        assert torch.equal(ys[u], step_single(u)), f"grouped unit {u} differs from the single call"
 
     if args.pmc_pass:
-        pmc_pass(torch, _C, dev, (step, step_row_major), x)
+        pmc_pass(torch, _C, dev, (step_single, step_row_major), step)
         return
     if args.block_stack_only:
         del packs
@@ -350,8 +403,11 @@ def main():
     wall_ms, ev_ms = graph_time(step, args.steps, args.warmup, torch)
     ms_per_step = wall_ms / args.steps
     kernel_us = ev_ms / args.steps * 1e3
-    value = weight_bytes / (ms_per_step * 1e-3) / 1e9
-    achieved = weight_bytes / (kernel_us * 1e-6) / 1e9
+    value = G * weight_bytes / (ms_per_step * 1e-3) / 1e9
+    achieved = G * weight_bytes / (kernel_us * 1e-6) / 1e9
+    single_steps = max(args.steps, 50) * 10
+    _, ev_single = graph_time(step_single, single_steps, args.warmup * 10, torch)
+    us_single = ev_single / single_steps * 1e3
 
     out = {
         "metric": METRIC,
@@ -364,28 +420,39 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f16 x 2-bit ternary -> f32 accumulate",
+        "dtype": "f16 x 2-bit ternary -> exact integer accumulate (int8 matrix cores), fp32 epilogue",
         "data": "synthetic (seed 0; N(0,0.02) master weights quantized with threshold 0.05, "
                 f"{zero_frac * 100:.1f}% zeros; N(0,1) activations)",
         "config": {
-            "workload": "config 2 decode GEMV: x fp16 [1,4096] x packed ternary W [4096,4096], "
-                        "per-tensor fp32 scale, fp16 bias",
-            "path": "TernaryLinearInference.forward on the layer's decode-tiled copy of the packed weights "
-                    "(built once from the reference-layout W_T, same 2 bits per weight, bit-identical outputs)",
+            "workload": f"config 2 decode GEMV units: x fp16 [1,4096] x packed ternary W [4096,4096], per-tensor fp32 "
+                        f"scale, fp16 bias; one step = one launch over {G} independent units (bt_ternary_gemv_grouped)",
+            "path": "TernaryLinearInference layers' decode-tiled weight copies through the grouped entry point; every "
+                    "unit bit-identical to the single call (checked in this run and by the GPU tests)",
             "M": 1, "N": N, "K": K,
+            "units_per_step": G,
             "weight_sets": nsets,
-            "weight_bytes_per_step": weight_bytes,
-            "timing": "one HIP graph of all steps, replayed once between synchronisations",
+            "weight_bytes_per_step": G * weight_bytes,
+            "timing": "one HIP graph of all steps, median of the replays, each between two synchronisations",
         },
         "roofline": {
-            "kernel": "bt::stream_kernel (fp16 activations, decode-tiled weights)",
+            "kernel": "bt::gemv_planes_group_kernel (fp16 activations as six int8 digit rows, decode-tiled weights)",
             "bound": "hbm",
             "achieved": round(achieved, 2),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": measured_traffic("stream_kernel_config2_tiled"),
+            "traffic": measured_traffic("gemv_planes_group_kernel_G128_config2"),
             "launch_us": round(kernel_us, 3),
+            "algorithmic_bytes_per_launch": G * weight_bytes,
+        },
+        "single_launch": {
+            "note": "the same config-2 GEMV one matrix per launch (TernaryLinearInference.forward), a chain of launches "
+                    "over the rotating weight sets: bounded by the launch, set-up and drain of a kernel, not by bytes",
+            "kernel": "bt::gemv_planes_kernel",
+            "launch_us": round(us_single, 3),
+            "GBps": round(weight_bytes / (us_single * 1e-6) / 1e9, 1),
+            "frac_of_hbm_peak": round(weight_bytes / (us_single * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+            "traffic": measured_traffic("gemv_planes_kernel_config2_tiled"),
             "algorithmic_bytes_per_launch": weight_bytes,
         },
     }
@@ -394,14 +461,26 @@ def main():
     if not args.no_extra:
         extra = {}
 
-        _, ev_rm = graph_time(step_row_major, args.steps, args.warmup, torch)
-        us_rm = ev_rm / args.steps * 1e3
+        _, ev_rm = graph_time(step_row_major, single_steps, args.warmup * 10, torch)
+        us_rm = ev_rm / single_steps * 1e3
         extra["decode_gemv_row_major_W_T"] = {
             "us": round(us_rm, 3), "GBps": round(weight_bytes / (us_rm * 1e-6) / 1e9, 1),
             "frac_of_hbm_peak": round(weight_bytes / (us_rm * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
-            "traffic": measured_traffic("stream_kernel_config2"),
-            "note": "same workload through bittorch._C.ternary_linear_packed_forward on the reference-layout W_T [Kb, N]",
+            "traffic": measured_traffic("gemv_planes_kernel_config2_row_major"),
+            "note": "one matrix per launch through bittorch._C.ternary_linear_packed_forward on the reference-layout W_T [Kb, N]",
         }
+        # units per launch: where the grouped launch leaves the launch-bound regime
+        by_g = {}
+        for gg in (1, 2, 4, 8, 16, 32, 64, 128):
+            if gg > G:
+                break
+            tb = [tuple(t[:gg].contiguous() for t in tab) for tab in tables]
+            reps = max(10, 2560 // gg // 4)
+            _, ev_g = graph_time(lambda i: _C.ternary_gemv_grouped(*tb[i % 2], K, N, scale_len=1), reps, 5, torch)
+            us_g = ev_g / reps * 1e3
+            by_g[f"G{gg}"] = {"us_per_launch": round(us_g, 2), "GBps": round(gg * weight_bytes / (us_g * 1e-6) / 1e9, 1),
+                              "frac_of_hbm_peak": round(gg * weight_bytes / (us_g * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
+        extra["grouped_gemv_by_units_per_launch"] = by_g
 
         def rand_packed(n, k, count):
             outp = []
@@ -477,13 +556,13 @@ def main():
         # constant operands, pseudo-random int8 x ternary operands, and the GEMM's own register
         # footprint (32 accumulators, 8 A and 4 B fragments per wave)
         def probe(mode):
-            _C.probe_mfma_int8(dev, 2048, 4096, mode)  # warm
+            probe_mfma_int8(torch, dev, 2048, 4096, mode)  # warm
             torch.cuda.synchronize()
             e0 = torch.cuda.Event(enable_timing=True)
             e1 = torch.cuda.Event(enable_timing=True)
             e0.record()
             for _ in range(5):
-                ops = _C.probe_mfma_int8(dev, 2048, 4096, mode)
+                ops = probe_mfma_int8(torch, dev, 2048, 4096, mode)
             e1.record()
             torch.cuda.synchronize()
             return ops * 5 / (e0.elapsed_time(e1) * 1e-3) / 1e12
@@ -511,7 +590,7 @@ def main():
                     st.wait_stream(main)
                     with torch.cuda.stream(st):
                         for i in range(per_branch):
-                            layers[(bi * per_branch + i) % nsets](x)
+                            layers[(bi * per_branch + i) % nsets](xs[(bi * per_branch + i) % nsets])
                 for st in streams:
                     main.wait_stream(st)
             graph.replay()
@@ -558,6 +637,31 @@ def main():
                         "forward on the reference-layout W_T beside it",
             }
             del ws, ts
+        # large matrices at M = 1, where one launch is no longer bounded by its start and drain: a vocabulary
+        # projection and a 64 MiB square layer, fp16 (exact GEMV where K allows), bf16 and int8 activations
+        big = {}
+        for (n, k) in ((128256, 4096), (16384, 16384)):
+            cnt = max(2, int(600e6 // (n * k // 4)))
+            ts = []
+            for w in rand_packed(n, k, cnt):
+                ts.append(_C.retile_weights(w, k))
+                del w
+            sc = torch.rand(n, device=dev) * 0.05 + 0.01
+            x16 = torch.randn(1, k, device=dev).half()
+            xb = x16.bfloat16()
+            qb, sb = _C.act_quant_int8(xb, True)
+            row = {"packed_weight_bytes": n * k // 4}
+            for name, fn in (("fp16", lambda i: _C.ternary_linear_tiled_forward(x16, ts[i % cnt], sc, None, k, n)),
+                             ("bf16", lambda i: _C.ternary_linear_tiled_forward(xb, ts[i % cnt], sc, None, k, n)),
+                             ("int8", lambda i: _C.ternary_gemm_int8_tiled(qb, sb, ts[i % cnt], sc, None, k, n, torch.bfloat16,
+                                                                           False, None, True))):
+                _, ev_b = graph_time(fn, 40, 8, torch)
+                us_b = ev_b / 40 * 1e3
+                row[name] = {"us": round(us_b, 2), "GBps": round(n * k // 4 / (us_b * 1e-6) / 1e9, 1),
+                             "frac_of_hbm_peak": round(n * k // 4 / (us_b * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
+            big[f"N{n}_K{k}"] = row
+            del ts
+        extra["large_matrices_M1"] = big
         # batched decode / short prefill on the config-2 layer (tiled weights): the streaming kernel runs the 16-row
         # blocks of a call concurrently in one launch; the tiled GEMM (forced with BITTORCH_STREAM_MAX_ROWS) beside it
         bd = {}

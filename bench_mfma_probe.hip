@@ -1,10 +1,14 @@
-// Measurement aid: the int8 MFMA rate the chip sustains when nothing else is in the way.
+// Measurement aid of bench.py (built into bench_mfma_probe.so, not part of libbittorch_hip.so or its ABI):
+// the int8 MFMA rate the chip sustains when nothing else is in the way.
 // Every wave issues back-to-back v_mfma_i32_16x16x64_i8 on eight independent accumulators
 // held in registers; no memory traffic inside the loop.  The prefill GEMM's TOPS are
 // reported against this figure as well as against the nominal peak.
-#include "bt_common.h"
+#include <hip/hip_runtime.h>
+#include <stdint.h>
 
-namespace bt {
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+namespace {
 
 __global__ __launch_bounds__(512) void mfma_i8_probe_kernel(int iters, int random_operands, int* __restrict__ out) {
     const int lane = threadIdx.x & 63;
@@ -74,15 +78,15 @@ __global__ __launch_bounds__(512) void mfma_i8_probe_tile_kernel(int iters, int*
     if (s == 0x7fffffff) out[0] = s;
 }
 
-}  // namespace bt
+}  // namespace
 
-extern "C" int bt_probe_mfma_i8(int blocks, int iters, int random_operands, int* out, double* ops_per_launch,
+// Launches `blocks` workgroups of 8 waves that each issue `iters` x 8 back-to-back v_mfma_i32_16x16x64_i8 on register
+// operands and writes the operation count of the launch (2*16*16*64 per instruction) to *ops_per_launch.
+// random_operands = 0: small constant operands; 1: pseudo-random int8 activations and ternary weights; 2: the prefill
+// GEMM's register footprint (32 accumulators per wave).  `out` is a device int the kernel may write.  Returns 0 / -1.
+extern "C" int bench_probe_mfma_i8(int blocks, int iters, int random_operands, int* out, double* ops_per_launch,
                                 void* stream) {
-    using namespace bt;
-    if (blocks <= 0 || iters <= 0 || !out) {
-        set_error("bt_probe_mfma_i8: bad arguments");
-        return BT_ERR_INVALID;
-    }
+    if (blocks <= 0 || iters <= 0 || !out) return -1;
     if (random_operands == 2)  // 32 accumulators per wave; iters is rounded up to a multiple of 4
         hipLaunchKernelGGL(mfma_i8_probe_tile_kernel, dim3((unsigned)blocks), dim3(512), 0, (hipStream_t)stream,
                            iters, out);
@@ -91,5 +95,5 @@ extern "C" int bt_probe_mfma_i8(int blocks, int iters, int random_operands, int*
                            random_operands, out);
     // 8 waves per block, 8 MFMAs per iteration, 2*16*16*64 operations each
     if (ops_per_launch) *ops_per_launch = (double)blocks * 8.0 * (double)iters * 8.0 * 32768.0;
-    return check_launch("bt_probe_mfma_i8");
+    return hipGetLastError() == hipSuccess ? 0 : -1;
 }

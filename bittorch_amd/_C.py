@@ -333,6 +333,35 @@ def ternary_linear_tiled_forward(X: Tensor, W_tiled: Tensor, scale: Tensor, bias
     return y.reshape(*X.shape[:-1], Ny)
 
 
+def pointer_table(tensors) -> Tensor:
+    """Device array of the tensors' device addresses (int64), the form :func:`ternary_gemv_grouped` takes its
+    operands in.  The caller keeps the tensors alive for as long as the table is used."""
+    tensors = list(tensors)
+    _check(len(tensors) > 0 and _all_cuda(*tensors), "All tensors must be CUDA")
+    return torch.tensor([t.data_ptr() for t in tensors], dtype=torch.int64, device=tensors[0].device)
+
+
+def ternary_gemv_grouped(x_tab: Tensor, w_tiled_tab: Tensor, scale_tab: Tensor, bias_tab: Optional[Tensor],
+                         y_tab: Tensor, in_features: int, out_features: int, scale_len: int = -1,
+                         scale_dtype: torch.dtype = torch.float32, bias_dtype: torch.dtype = torch.float16) -> None:
+    """``G`` independent decode GEMVs in one launch: unit ``u`` multiplies the fp16 row at ``x_tab[u]`` with the
+    decode-tiled weights at ``w_tiled_tab[u]`` into the fp16 row at ``y_tab[u]``, exactly as
+    :func:`ternary_linear_tiled_forward` would on that row (same bits).  The tables are int64 device tensors of
+    ``G`` device addresses (:func:`pointer_table`); nothing is allocated or returned."""
+    G = x_tab.numel()
+    tabs = (x_tab, w_tiled_tab, scale_tab, y_tab) + (() if bias_tab is None else (bias_tab,))
+    for t in tabs:
+        _check(t.dtype == torch.int64 and t.dim() == 1 and t.numel() == G and t.is_contiguous(),
+               "pointer tables must be contiguous int64 tensors of one length")
+    _check(_all_cuda(*tabs), "All tensors must be CUDA")
+    _check(scale_dtype in _DT and bias_dtype in _DT, "scale / bias dtype must be float32, float16 or bfloat16")
+    with torch.cuda.device(x_tab.device):
+        _status(_L.bt_ternary_gemv_grouped(
+            x_tab.data_ptr(), _DT[torch.float16], w_tiled_tab.data_ptr(), scale_tab.data_ptr(), _DT[scale_dtype],
+            out_features if scale_len < 0 else scale_len, _ptr(bias_tab), _DT[bias_dtype], y_tab.data_ptr(), G,
+            out_features, in_features, _stream(x_tab)))
+
+
 def ternary_gemm_int8_tiled(Q: Tensor, s_x: Tensor, W_tiled: Tensor, scale: Tensor, bias: Optional[Tensor] = None,
                             in_features: int = -1, out_features: int = -1,
                             out_dtype: torch.dtype = torch.float32, return_acc: bool = False,
@@ -580,17 +609,3 @@ def unpack_dequant(W_T: Tensor, in_features: int, scale: Optional[Tensor] = None
                                      0 if scale_f is None else scale_f.numel(), out.data_ptr(), odt,
                                      N, in_features, _stream(W_T)))
     return out
-
-
-def probe_mfma_int8(device, blocks: int = 2048, iters: int = 4096, random_operands: int = 0):
-    """Launches the int8 matrix-core rate probe on the current stream; returns the number
-    of integer operations the launch performs (time it from outside).  ``random_operands``:
-    0 constant operands, 1 pseudo-random int8 x ternary operands, 2 the prefill GEMM's
-    register footprint (32 accumulators per wave)."""
-    import ctypes
-
-    out = torch.zeros(1, dtype=torch.int32, device=device)
-    ops = ctypes.c_double(0.0)
-    with torch.cuda.device(device):
-        _status(_L.bt_probe_mfma_i8(blocks, iters, int(random_operands), out.data_ptr(), ctypes.addressof(ops), _stream(out)))
-    return ops.value

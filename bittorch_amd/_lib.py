@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # BITTORCH_HIP_LIBRARY points at another build of the library (A/B comparisons)
 LIB_PATH = os.environ.get("BITTORCH_HIP_LIBRARY") or os.path.join(_HERE, "_hip", "libbittorch_hip.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -41,9 +41,9 @@ SIGNATURES = {
                                                      _i64, _i64, _i64, _vp, _sz, _vp]),
     "bt_ternary_linear_tensor_core_forward_static": (_int, [_vp, _int, _vp, _vp, _int, _i64, _vp, _int, _vp,
                                                             _i64, _i64, _i64, _vp]),
+    "bt_ternary_gemv_grouped": (_int, [_vp, _int, _vp, _vp, _int, _i64, _vp, _int, _vp, _i64, _i64, _i64, _vp]),
     "bt_unpack_dequant": (_int, [_vp, _vp, _i64, _vp, _int, _i64, _i64, _vp]),
     "bt_pack_ternary_i8": (_int, [_vp, _i64, _i64, _vp, _vp]),
-    "bt_probe_mfma_i8": (_int, [_int, _int, _int, _vp, _vp, _vp]),
     "bt_ternary_linear_packed_forward_res": (_int, [_vp, _int, _vp, _vp, _int, _i64, _vp, _int, _vp, _vp,
                                                     _i64, _i64, _i64, _vp, _sz, _vp]),
     "bt_ternary_gemm_i8_res": (_int, [_vp, _int, _vp, _vp, _vp, _int, _i64, _vp, _int, _vp, _vp, _int, _vp,

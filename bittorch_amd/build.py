@@ -17,7 +17,7 @@ CSRC = os.path.join(_HERE, "csrc")
 OUT_DIR = os.path.join(_HERE, "_hip")
 LIB_PATH = os.path.join(OUT_DIR, "libbittorch_hip.so")
 
-SOURCES = ["capi.hip", "quantize_pack.hip", "stream_gemm.hip", "gemm_i8.hip", "gemm_f16.hip", "act_quant.hip", "row_ops.hip", "misc_kernels.hip", "mfma_probe.hip"]
+SOURCES = ["capi.hip", "quantize_pack.hip", "stream_gemm.hip", "gemv_planes.hip", "gemm_i8.hip", "gemm_f16.hip", "act_quant.hip", "row_ops.hip", "misc_kernels.hip"]
 
 # packed fp32 VALU forms are disabled on purpose (they have produced wrong
 # results on this hardware generation's boxes); the host pass warns that it
@@ -74,5 +74,18 @@ def build(verbose: bool = False, extra_flags=()) -> str:
     return LIB_PATH
 
 
+def build_bench_probe() -> str:
+    """The benchmark's own measurement aid (``bench_mfma_probe.hip`` at the repository root): a separate
+    shared object that only ``bench.py`` loads."""
+    root = os.path.dirname(_HERE)
+    src, out = os.path.join(root, "bench_mfma_probe.hip"), os.path.join(root, "bench_mfma_probe.so")
+    cmd = [_hipcc(), *HIPCC_FLAGS, "-shared", src, "-o", out]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed on bench_mfma_probe.hip:\n{res.stdout}\n{res.stderr}")
+    return out
+
+
 if __name__ == "__main__":
     print(build(verbose=True))
+    print(build_bench_probe())

@@ -55,6 +55,13 @@ bool gemm_f16_supported(int64_t N, int64_t K, const void* X, const void* W_T, co
 bool gemm_f16_supported_tiled(int64_t N, int64_t K, const void* X, const void* Y);
 int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, int w_layout, const Epilogue& epi, void* Y, int y_dtype,
                     int64_t M, int64_t N, int64_t K, int planes, hipStream_t st);
+bool planes_supported(int x_dtype, int y_dtype, int64_t B, int64_t N, int64_t K, const void* X, const void* W, const void* Y,
+                      int w_layout);
+int launch_planes(const void* X, const uint8_t* W, int w_layout, const Epilogue& epi, void* Y, int64_t N, int64_t K,
+                  int epi_op, hipStream_t st);
+int launch_planes_group(const void* const* X_tab, const uint8_t* const* W_tab, const void* const* scale_tab, int scale_dtype,
+                        int scale_bcast, const void* const* bias_tab, int bias_dtype, void* const* Y_tab, int64_t G, int64_t N,
+                        int64_t K, hipStream_t st);
 bool gemm_i8_supported_tiled(int64_t N, int64_t K, const void* Q);
 int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_T, int w_layout, const Epilogue& epi,
                    void* Y, int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st);
@@ -215,6 +222,9 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
             set_error("%s: tiled weights must be 256-byte aligned and below 4 GiB, Y 16-byte aligned", who);
             return BT_ERR_INVALID;
         }
+        // one fp16 row: the exact GEMV on the int8 matrix cores
+        if (planes_supported(x_dtype, x_dtype, B, N, K, X, W_T, Y, W_LAYOUT_TILED))
+            return launch_planes(X, W_T, W_LAYOUT_TILED, epi, Y, N, K, epi_op, st);
         if (x_dtype != BT_F32) {
             const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
             // tall batches: the tiled matrix-core GEMM reads the copy too (not with the SwiGLU output stage)
@@ -237,6 +247,8 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
                              Q_ROW_MAJOR, 0, nullptr, 0.0f, epi_op, st);
     }
     if (packed_uses_stream(x_dtype, W_T, Y, N, K)) {
+        if (planes_supported(x_dtype, x_dtype, B, N, K, X, W_T, Y, W_LAYOUT_ROW_MAJOR))
+            return launch_planes(X, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, N, K, 0, st);
         const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
         // tall batches go to the tiled matrix-core kernel, decode shapes stream the weights
         if (!prefers_stream(B, N, K, false) && gemm_f16_supported(N, K, X, W_T, Y))
@@ -479,6 +491,40 @@ extern "C" int bt_ternary_linear_tensor_core_forward_static(const void* X, int x
                         nullptr, Y, x_dtype, nullptr, B, N, K, stream);
 }
 
+// ---- G decode GEMVs in one launch ---------------------------------------------------------------
+extern "C" int bt_ternary_gemv_grouped(const void* const* X_tab, int x_dtype, const uint8_t* const* W_tiled_tab,
+                                       const void* const* scale_tab, int scale_dtype, int64_t scale_len,
+                                       const void* const* bias_tab, int bias_dtype, void* const* Y_tab, int64_t G,
+                                       int64_t N, int64_t K, void* stream) {
+    const char* who = "bt_ternary_gemv_grouped";
+    if (!X_tab || !W_tiled_tab || !scale_tab || !Y_tab) {
+        set_error("%s: null pointer table", who);
+        return BT_ERR_INVALID;
+    }
+    if (G <= 0 || N <= 0 || K <= 0 || G > (1 << 20)) {
+        set_error("%s: empty shape or too many units (G=%lld N=%lld K=%lld)", who, (long long)G, (long long)N, (long long)K);
+        return BT_ERR_INVALID;
+    }
+    if (x_dtype != BT_F16) {
+        set_error("%s: activations must be fp16 (dtype tag %d given)", who, x_dtype);
+        return BT_ERR_INVALID;
+    }
+    if (K % 16 != 0 || K > 10240) {
+        set_error("%s: K must be a multiple of 16 and at most 10240 (K=%lld)", who, (long long)K);
+        return BT_ERR_INVALID;
+    }
+    if ((scale_len != N && scale_len != 1) || !valid_dtype(scale_dtype) || (bias_tab && !valid_dtype(bias_dtype))) {
+        set_error("%s: scale size doesn't match N, or unsupported scale/bias dtype", who);
+        return BT_ERR_INVALID;
+    }
+    if (tiled_bytes(N, K) >= (1ull << 32) || G * ceil_div(N, 128) >= (1ll << 31)) {
+        set_error("%s: a unit's tiled weights must stay below 4 GiB", who);
+        return BT_ERR_INVALID;
+    }
+    return launch_planes_group(X_tab, W_tiled_tab, scale_tab, scale_dtype, (scale_len == 1 && N != 1) ? 1 : 0, bias_tab,
+                               bias_dtype, Y_tab, G, N, K, (hipStream_t)stream);
+}
+
 // ---- fused producers of the GEMM activations (row_ops.hip) ----------------------------------
 static int check_row_op(const char* who, const void* A, int dtype, int64_t B, int64_t K, int64_t lda, void* H,
                         int8_t* Q, float* s_x) {
@@ -553,7 +599,12 @@ static int fused_forward_impl(const char* who, const void* X, int64_t ld_x, int 
     // one 16-bit row on the streaming kernel: the prologue runs inside the GEMV, on the row's way into LDS
     const bool streams = (w_layout == W_LAYOUT_TILED) ? (stream_supported_tiled(N, K, W_T) && fast_path_ok(Y, N, K))
                                                       : packed_uses_stream(x_dtype, W_T, Y, N, K);
-    if (x_dtype != BT_F32 && B == 1 && streams) {
+    // (a row that takes the exact fp16 GEMV gets its prologue from the row kernel: the two then agree bit for bit
+    // with the unfused sequence by construction)
+    const size_t h_need = align256((size_t)B * K * dtype_size(x_dtype));
+    const bool two_step_ok = workspace && workspace_bytes >= h_need && ((uintptr_t)workspace) % 256 == 0;
+    const bool exact_row = two_step_ok && planes_supported(x_dtype, x_dtype, B, N, K, workspace, W_T, Y, w_layout);
+    if (x_dtype != BT_F32 && B == 1 && streams && !exact_row) {
         const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
         if (stream_prologue_fusable(mode, B, N, K, X, pro_b, w_layout, epi_op)) {
             Epilogue epi;

@@ -1,0 +1,568 @@
+// Decode GEMV (one activation row) for fp16 activations on the int8 matrix cores, exact.
+//
+// What it computes (the float path of the reference's packed kernel,
+// csrc/kernels/ternary_gemm_production.cu:126-141, with the accumulation done exactly):
+//     acc[n] = sum_k x[k] * w[k, n]      y[n] = acc[n] * scale[n] + bias[n]
+// The reference adds the products one by one in fp32.  Here the sum is formed without any rounding:
+// every finite fp16 value is an integer multiple of 2^-24 below 2^16, so X[k] = x[k] * 2^24 is an
+// integer of at most 41 bits, S[n] = sum_k X[k] * w[k, n] is an exact integer, and
+//     acc[n] = RN_fp32(S[n]) * 2^-24
+// is the correctly rounded value of the exact dot product.  The result does not depend on how the
+// kernel splits K, which is what makes the single-launch kernel, the grouped kernel and both weight
+// layouts agree bit for bit.  (Rows that hold an infinity or a NaN give NaN in every column, which
+// is what the reference's float arithmetic gives whenever such a value meets a zero weight.)
+//
+// How: X[k] is written in six base-128 digits, X = sum_p d_p 128^p with d_0..d_4 in 0..127 and d_5
+// the signed top digit (two's complement), each an int8.  The six digit rows are six rows of the A
+// operand of v_mfma_i32_16x16x64_i8 (a decode step has one activation row, so the other fifteen rows
+// of the matrix instruction are free anyway); the B operand is the 2-bit weights decoded to int8
+// {-1, 0, +1} (9 VALU operations per 16 weights, against 24 for the 16-bit decode); the int32
+// accumulators of the six rows are recombined in 64-bit integer arithmetic at the end.
+//
+// Two kernels share the arithmetic:
+//   gemv_planes_kernel        one weight matrix per launch; a workgroup owns a tile of 16 * NACC columns over the
+//                             whole of K and its waves split K (deterministic integer sum through LDS).
+//   gemv_planes_group_kernel  G independent units (own x, W, scale, bias, y; pointer tables in device
+//                             memory) in ONE launch: persistent workgroups walk (unit, column slab) items, a
+//                             wave owns 16 * NACC columns over the whole of K (no reduction, no barrier inside an
+//                             item) and keeps its weight loads running across item boundaries, so that the launch,
+//                             set-up and drain of a 4 MiB GEMV are paid once per launch instead of once per matrix.
+#include <cstdlib>
+
+#include "row_math.h"
+
+namespace bt {
+
+constexpr int PL_N = 6;                    // digit planes
+constexpr int PL_GROUP = PL_N * 16;        // bytes of one 16-k group in LDS: six 16-byte operand fragments
+
+enum { PL_TILED = 0, PL_ROWMAJOR = 1 };
+
+struct PlaneParams {
+    // single launch: direct pointers.  grouped launch: tables of G device pointers (bias_tab may be null).
+    const void* X;
+    const uint8_t* W;
+    const void* scale;
+    const void* bias;
+    const void* residual;
+    void* Y;
+    const void* const* X_tab;
+    const uint8_t* const* W_tab;
+    const void* const* scale_tab;
+    const void* const* bias_tab;
+    void* const* Y_tab;
+    int64_t N, K, Kb;
+    int G;
+    int wsteps;      // 16-row steps of the weights (64 k each)
+    int tiles16;     // 16-column tiles
+    int tiles;       // single launch: workgroup tiles of 16 * NACC columns
+    int per_xcd;     // single launch: tiles per XCD (grid = 8 * per_xcd)
+    int slabs;       // grouped launch: column slabs (8 waves x 16 * NACC columns) per unit
+    int items;       // grouped launch: G * slabs
+    int scale_dtype, bias_dtype, scale_bcast;
+};
+
+// ---- fp16 -> six int8 digit planes ----------------------------------------------------------------
+// Eight consecutive fp16 values (one 16-byte load) -> per plane the eight digit bytes, elements 0..3 in
+// lo[p] and 4..7 in hi[p].  Returns true if any value is an infinity or a NaN.
+__device__ __forceinline__ bool f16x8_to_planes(const uint4 v, uint32_t (&lo)[PL_N], uint32_t (&hi)[PL_N]) {
+    const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+    bool bad = false;
+#pragma unroll
+    for (int p = 0; p < PL_N; p++) lo[p] = hi[p] = 0u;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const uint32_t h = (d[e >> 1] >> (16 * (e & 1))) & 0xffffu;
+        const uint32_t ex = (h >> 10) & 31u, m = h & 0x3ffu;
+        bad |= (ex == 31u);
+        const uint32_t mag = ex ? (m | 0x400u) : m;      // 11-bit significand (subnormals: no hidden bit)
+        const uint32_t sh = ex ? ex - 1u : 0u;           // x = mag * 2^(sh - 24)
+        const int32_t sm = (h & 0x8000u) ? -(int32_t)mag : (int32_t)mag;
+        const int64_t X = (int64_t)sm << sh;             // x * 2^24, |X| < 2^40
+        const uint32_t xl = (uint32_t)X, xh = (uint32_t)((uint64_t)X >> 32);
+        uint32_t dg[PL_N];
+        dg[0] = xl & 127u;
+        dg[1] = (xl >> 7) & 127u;
+        dg[2] = (xl >> 14) & 127u;
+        dg[3] = (xl >> 21) & 127u;
+        dg[4] = ((xl >> 28) | (xh << 4)) & 127u;
+        dg[5] = (xh >> 3) & 255u;                        // bits 35..42: the signed top digit as a byte
+#pragma unroll
+        for (int p = 0; p < PL_N; p++) {
+            if (e < 4) lo[p] |= dg[p] << (8 * e);
+            else hi[p] |= dg[p] << (8 * (e - 4));
+        }
+    }
+    return bad;
+}
+
+__device__ __forceinline__ uint4 zero_unless4(uint4 v, bool ok) {
+    v.x = ok ? v.x : 0u; v.y = ok ? v.y : 0u; v.z = ok ? v.z : 0u; v.w = ok ? v.w : 0u;
+    return v;
+}
+
+// Chunk c of a row (elements 8c .. 8c+7) -> LDS, in matrix-core operand order.  `planes` points at the row's (or
+// the wave slice's) first 16-k group; even and odd lanes hold the two halves of one group and exchange bytes, so
+// every lane of a pair must call it (`write` = false for pairs outside the buffer).  v must already be zero for
+// chunks beyond K.
+__device__ __forceinline__ bool park_chunk(uint8_t* planes, int c, const uint4 v, int lane, bool write) {
+    uint32_t lo[PL_N], hi[PL_N];
+    const bool bad = f16x8_to_planes(v, lo, hi);
+    uint8_t* dst = planes + (size_t)(c >> 1) * PL_GROUP + 8 * (c & 1);
+#pragma unroll
+    for (int p = 0; p < PL_N; p++) {
+        const uint2 o = q_to_operand_order(lo[p], hi[p], lane & 1);
+        if (write) *(uint2*)(dst + 16 * p) = o;
+    }
+    return bad;
+}
+
+// d = the dword this lane loaded (row 4g+q, four columns); returns the bytes of column q of the dwords of quad
+// lanes 0..3, i.e. rows 4g..4g+3 of this lane's own column (row-major W_T)
+__device__ __forceinline__ uint32_t pl_quad_transpose(uint32_t d, uint32_t sel_q) {
+    const uint32_t v0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d, 0x00, 0xf, 0xf, true);
+    const uint32_t v1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d, 0x55, 0xf, 0xf, true);
+    const uint32_t v2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d, 0xAA, 0xf, 0xf, true);
+    const uint32_t v3 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d, 0xFF, 0xf, 0xf, true);
+    const uint32_t t01 = perm(v1, v0, sel_q);
+    const uint32_t t23 = perm(v3, v2, sel_q);
+    return perm(t23, t01, 0x05040100u);
+}
+
+// the exact sum S (in units of 2^-24), correctly rounded to fp32 and scaled back
+__device__ __forceinline__ float fixed_to_f32(int64_t S) { return __builtin_ldexpf((float)S, -24); }
+// ... from its six plane sums
+__device__ __forceinline__ float planes_to_f32(const int32_t (&s)[PL_N]) {
+    int64_t S = 0;
+#pragma unroll
+    for (int p = PL_N - 1; p >= 0; p--) S = S * 128 + (int64_t)s[p];
+    return fixed_to_f32(S);
+}
+
+__device__ __forceinline__ void pl_store(void* Y, const void* residual, int64_t n, float acc, float s, float b, bool bad) {
+    float y = epi_float(acc, s, b);
+    if (bad) y = __builtin_nanf("");
+    if (residual) y = add_residual(y, residual, BT_F16, n);
+    ((uint16_t*)Y)[n] = f32_to_f16_bits(y);
+}
+
+// ---- one weight matrix per launch -------------------------------------------------------------------
+// LDS: [WAVES][2][TILE_N] int64 partial sums, [WAVES] flags, then per wave the digit planes of its K slice.
+// EPI = EPI_SWIGLU_PAIRS (tiled copy in gate/up pair order, NACC even): Y [N/2], Y[h] = rd(rd(silu(g)) * u) with
+// g = rd(linear column h), u = rd(linear column N/2 + h), what the SwiGLU kernel makes of the stored projections.
+template <int LAYOUT, int NACC, int WAVES, int PF, int EPI = EPI_NONE>
+__global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(PlaneParams p) {
+    constexpr int TILE_N = 16 * NACC;
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+
+    const int tile = (int)(blockIdx.x & 7) * p.per_xcd + (int)(blockIdx.x >> 3);  // neighbouring tiles on one XCD
+    if (tile >= p.tiles) return;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int j = lane & 15, g = lane >> 4, q = lane & 3;
+    const int nsteps = (int)((p.K + 63) >> 6);
+    const int spw = (nsteps + WAVES - 1) / WAVES;  // steps per wave, contiguous
+    const int s_begin = wave * spw;
+    const int s_end = min(nsteps, s_begin + spw);
+    const int nchunks = spw * 8;                   // 16-byte chunks of the wave's slice of x
+
+    uint32_t* red = lds;
+    uint32_t* flags = lds + WAVES * 4 * TILE_N;
+    uint8_t* planes = (uint8_t*)(flags + WAVES) + (size_t)wave * spw * 4 * PL_GROUP;
+
+    // 1. the wave's slice of x (needed first, and loads return in order), 2. its first batch of weights,
+    // 3. the epilogue operands; the slice is converted while the weights are on their way
+    constexpr int XC = 4;  // chunks per lane (the host keeps spw * 8 <= 64 * XC)
+    uint4 xr[XC];
+#pragma unroll
+    for (int u = 0; u < XC; u++) {
+        if (u * 64 < nchunks) {  // uniform
+            const int k = s_begin * 64 + (lane + 64 * u) * 8;
+            xr[u] = *(const uint4*)((const uint16_t*)p.X + (uint32_t)min(k, (int)p.K - 8));
+        }
+    }
+    // byte offset of this lane's dword in step 0 of each of its 16-column tiles (tiled copy), resp. of its quad's
+    // four columns in row 4g+q (row-major W_T); a tile / column past the end repeats valid bytes and is never stored
+    uint32_t coloff[NACC];
+    const uint32_t N32 = (uint32_t)p.N;
+#pragma unroll
+    for (int t = 0; t < NACC; t++) {
+        if constexpr (LAYOUT == PL_TILED) {
+            coloff[t] = ((uint32_t)min(tile * NACC + t, p.tiles16 - 1) * (uint32_t)p.wsteps * 64u + (uint32_t)lane) * 4u;
+        } else {
+            const int64_t c = (int64_t)tile * TILE_N + 16 * t + (j & ~3);
+            coloff[t] = (c < p.N) ? (uint32_t)c : 0u;
+        }
+    }
+    const uint32_t last_rowoff = (uint32_t)(p.Kb - 1) * N32;
+    const uint32_t sel_q = 0x0C0C0000u | ((uint32_t)(4 + q) << 8) | (uint32_t)q;
+    auto load_weights = [&](int base, uint32_t (&raw)[PF][NACC]) {
+#pragma unroll
+        for (int f = 0; f < PF; f++) {
+            const int ws = min(base + f, p.wsteps - 1);  // uniform; steps past the end meet zero activations
+#pragma unroll
+            for (int t = 0; t < NACC; t++) {
+                if constexpr (LAYOUT == PL_TILED) {
+                    raw[f][t] = *(const uint32_t*)(p.W + (coloff[t] + (uint32_t)ws * 256u));
+                } else {
+                    const uint32_t ro = min((uint32_t)(16 * ws + 4 * g + q) * N32, last_rowoff);
+                    raw[f][t] = *(const uint32_t*)(p.W + (ro + coloff[t]));
+                }
+            }
+        }
+    };
+    uint32_t raw0[PF][NACC];
+    load_weights(s_begin, raw0);
+
+    // output threads: one column each; with the SwiGLU output stage one column h of the hidden vector each, made
+    // of columns h (tile 2P of the pair-ordered copy) and N/2 + h (tile 2P + 1)
+    uint32_t pre_s = 0u, pre_b = 0u, pre_s2 = 0u, pre_b2 = 0u;
+    constexpr bool PAIRS = (EPI == EPI_SWIGLU_PAIRS);
+    const int tid = (int)threadIdx.x;
+    const int64_t ffn = p.N >> 1;
+    const int64_t n_out = PAIRS ? (int64_t)tile * (TILE_N / 2) + tid : (int64_t)tile * TILE_N + tid;
+    const bool out_thread = PAIRS ? (tid < TILE_N / 2 && n_out < ffn) : (tid < TILE_N && n_out < p.N);
+    const int slot = PAIRS ? (tid >> 4) * 32 + (tid & 15) : tid;
+    if (out_thread) {
+        pre_s = load_bits_rt(p.scale, p.scale_dtype, p.scale_bcast ? 0 : n_out);
+        if (p.bias) pre_b = load_bits_rt(p.bias, p.bias_dtype, n_out);
+        if constexpr (PAIRS) {
+            pre_s2 = load_bits_rt(p.scale, p.scale_dtype, p.scale_bcast ? 0 : ffn + n_out);
+            if (p.bias) pre_b2 = load_bits_rt(p.bias, p.bias_dtype, ffn + n_out);
+        }
+    }
+
+    bool bad = false;
+#pragma unroll
+    for (int u = 0; u < XC; u++) {
+        if (u * 64 < nchunks) {
+            const int c = lane + 64 * u;
+            const int k = s_begin * 64 + c * 8;
+            const uint4 v = zero_unless4(xr[u], k < (int)p.K && c < nchunks);
+            bad |= park_chunk(planes, c, v, lane, c < nchunks);
+        }
+    }
+    if (__builtin_amdgcn_ballot_w64(bad) != 0ull) bad = true;
+
+    v4i acc[NACC];
+#pragma unroll
+    for (int t = 0; t < NACC; t++) acc[t] = v4i{0, 0, 0, 0};
+    // lane (i, g) feeds digit row i of k-group g; rows 6..15 of the matrix instruction repeat rows 0..5 (unused)
+    const uint8_t* a_src = planes + g * PL_GROUP + (j % PL_N) * 16;
+
+    for (int base = s_begin; base < s_end; base += PF) {
+        uint32_t raw[PF][NACC];
+        if (base == s_begin) {  // uniform: this batch was requested ahead of the conversion
+#pragma unroll
+            for (int f = 0; f < PF; f++)
+#pragma unroll
+                for (int t = 0; t < NACC; t++) raw[f][t] = raw0[f][t];
+        } else {
+            load_weights(base, raw);
+        }
+#pragma unroll
+        for (int f = 0; f < PF; f++) {
+            if (base + f >= s_end) break;  // uniform per wave
+            // LDS accesses of one wave execute in order: the slice written above is visible
+            const uint4 av = *(const uint4*)(a_src + (size_t)(base + f - s_begin) * 4 * PL_GROUP);
+            const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+#pragma unroll
+            for (int t = 0; t < NACC; t++) {
+                uint32_t G;
+                if constexpr (LAYOUT == PL_TILED) G = raw[f][t];
+                else G = pl_quad_transpose(raw[f][t], sel_q);
+                acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, decode16_i8(G), acc[t], 0, 0, 0);
+            }
+        }
+    }
+
+    // Every wave folds its digit rows into 64-bit integers first (lane (j, 0) holds rows 0..3 of column j, lane
+    // (j, 1) rows 4 and 5: two partial values per column and wave), then the partial values of all waves are added
+    // through LDS -- integers, so the order does not matter.
+    int64_t* red64 = (int64_t*)red;  // [WAVES][2][TILE_N]
+    if (g < 2) {
+#pragma unroll
+        for (int t = 0; t < NACC; t++) {
+            const int64_t a0 = acc[t][0], a1 = acc[t][1], a2 = (g == 0) ? acc[t][2] : 0, a3 = (g == 0) ? acc[t][3] : 0;
+            const int64_t part = (((a3 * 128 + a2) * 128 + a1) * 128 + a0) << (28 * g);
+            red64[(wave * 2 + g) * TILE_N + t * 16 + j] = part;
+        }
+    }
+    if (lane == 0) flags[wave] = bad ? 1u : 0u;
+    __syncthreads();
+    if (!out_thread) return;
+    int64_t S = 0, S2 = 0;
+    uint32_t any_bad = 0u;
+    for (int w = 0; w < 2 * WAVES; w++) {
+        S += red64[w * TILE_N + slot];
+        if constexpr (PAIRS) S2 += red64[w * TILE_N + slot + 16];
+    }
+    for (int w = 0; w < WAVES; w++) any_bad |= flags[w];
+    const float sc = bits_to_f32_rt(pre_s, p.scale_dtype);
+    const float bs = p.bias ? bits_to_f32_rt(pre_b, p.bias_dtype) : 0.0f;
+    if constexpr (PAIRS) {
+        const float sc2 = bits_to_f32_rt(pre_s2, p.scale_dtype);
+        const float bs2 = p.bias ? bits_to_f32_rt(pre_b2, p.bias_dtype) : 0.0f;
+        float gv = round_to_dtype(epi_float(fixed_to_f32(S), sc, bs), BT_F16);
+        const float uv = round_to_dtype(epi_float(fixed_to_f32(S2), sc2, bs2), BT_F16);
+        if (any_bad) gv = __builtin_nanf("");
+        ((uint16_t*)p.Y)[n_out] = f32_to_f16_bits(swiglu_value(gv, uv, BT_F16));
+    } else {
+        pl_store(p.Y, p.residual, n_out, fixed_to_f32(S), sc, bs, any_bad != 0u);
+    }
+}
+
+// ---- G units per launch -----------------------------------------------------------------------------
+// (A single wide matrix does not run faster here than in the kernel above: 4.1-4.4 against 4.5 TB/s at
+// N = 128256, K = 4096; one item per workgroup leaves nothing to overlap.)
+// Persistent workgroups of 8 waves.  Item i = (unit i / slabs, slab i % slabs); wave w of the workgroup owns the
+// 16-column tiles (slab * 8 + w) * NACC .. + NACC - 1 of the unit over the whole of K.  The digit planes of the
+// unit's activation row are converted once per item by the whole workgroup into LDS.  The weight loads of a wave
+// form one uninterrupted stream: PF steps are always in flight, and the last batch of an item already requests the
+// first steps of the wave's next item.
+// LDS: a flag word per wave, then the digit planes of one row, padded with zero groups to a multiple of PF steps.
+template <int NACC, int PF>
+__global__ __launch_bounds__(512, 4) void gemv_planes_group_kernel(PlaneParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int j = lane & 15, g = lane >> 4;
+    const int S = p.wsteps;
+    const int SP = (S + PF - 1) / PF * PF;         // steps per item, padded
+    uint32_t* flags = lds;  // [8]
+    uint8_t* planes = (uint8_t*)(lds + 8);
+    const int nchunks = SP * 8;                    // 16-byte chunks of x, padding included
+    const uint8_t* a_src = planes + g * PL_GROUP + (j % PL_N) * 16;
+
+    // tile t of the wave within item `it`: base pointer of its first step (uniform), clamped to the last tile
+    auto tile_base = [&](int it, int t) -> const uint8_t* {
+        const int u = it / p.slabs, slab = it - u * p.slabs;
+        const int tl = min((slab * 8 + wave) * NACC + t, p.tiles16 - 1);
+        return p.W_tab[u] + (size_t)tl * (size_t)S * 256;
+    };
+    int it = (int)blockIdx.x;
+    if (it >= p.items) return;
+    const uint8_t* wcur[NACC];
+#pragma unroll
+    for (int t = 0; t < NACC; t++) wcur[t] = tile_base(it, t);
+    const uint32_t loff = (uint32_t)lane * 4u;
+    uint32_t raw[PF][NACC];
+#pragma unroll
+    for (int f = 0; f < PF; f++)
+#pragma unroll
+        for (int t = 0; t < NACC; t++) raw[f][t] = *(const uint32_t*)(wcur[t] + ((size_t)min(f, S - 1) * 256 + loff));
+
+    for (; it < p.items; it += (int)gridDim.x) {
+        const int u = it / p.slabs, slab = it - u * p.slabs;
+        const int it_next = (it + (int)gridDim.x < p.items) ? it + (int)gridDim.x : it;
+        const uint8_t* wnext[NACC];
+#pragma unroll
+        for (int t = 0; t < NACC; t++) wnext[t] = tile_base(it_next, t);
+        // the unit's activation row -> digit planes (all waves; the previous item's readers are past the barrier
+        // that ended it)
+        const uint16_t* xrow = (const uint16_t*)p.X_tab[u];
+        bool bad = false;
+        for (int c = (int)threadIdx.x; c < nchunks; c += 512) {
+            const int k = c * 8;
+            uint4 v = *(const uint4*)(xrow + min(k, (int)p.K - 8));
+            v = zero_unless4(v, k < (int)p.K);
+            bad |= park_chunk(planes, c, v, lane, true);
+        }
+        // (a word per wave, stored unconditionally: nothing to clear between items)
+        const bool wave_bad = __builtin_amdgcn_ballot_w64(bad) != 0ull;
+        if (lane == 0) flags[wave] = wave_bad ? 1u : 0u;
+        // epilogue operands of the columns this lane will store (lanes 0..15: column j of each tile)
+        const int64_t ncol0 = ((int64_t)(slab * 8 + wave) * NACC) * 16 + j;
+        uint32_t pre_s[NACC], pre_b[NACC];
+        const void* scale_u = p.scale_tab[u];
+        const void* bias_u = p.bias_tab ? p.bias_tab[u] : nullptr;
+#pragma unroll
+        for (int t = 0; t < NACC; t++) {
+            const int64_t n = ncol0 + 16 * t;
+            pre_s[t] = pre_b[t] = 0u;
+            if (g == 0 && n < p.N) {
+                pre_s[t] = load_bits_rt(scale_u, p.scale_dtype, p.scale_bcast ? 0 : n);
+                if (bias_u) pre_b[t] = load_bits_rt(bias_u, p.bias_dtype, n);
+            }
+        }
+        __syncthreads();
+
+        v4i acc[NACC];
+#pragma unroll
+        for (int t = 0; t < NACC; t++) acc[t] = v4i{0, 0, 0, 0};
+        for (int base = 0; base < SP; base += PF) {
+            // refill target of this batch: the same item's next batch, or the first batch of the wave's next item
+            const bool last = base + PF >= SP;  // uniform
+            const int sb = last ? 0 : base + PF;
+#pragma unroll
+            for (int f = 0; f < PF; f++) {
+                const uint4 av = *(const uint4*)(a_src + (size_t)(base + f) * 4 * PL_GROUP);
+                const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+                const size_t so = (size_t)min(sb + f, S - 1) * 256 + loff;
+#pragma unroll
+                for (int t = 0; t < NACC; t++) {
+                    acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, decode16_i8(raw[f][t]), acc[t], 0, 0, 0);
+                    raw[f][t] = *(const uint32_t*)((last ? wnext[t] : wcur[t]) + so);
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < NACC; t++) wcur[t] = wnext[t];
+
+        // lane (j, 0) holds the sums of digit rows 0..3 of column j, lane (j, 1) those of rows 4 and 5
+        uint32_t fl = 0u;
+#pragma unroll
+        for (int w = 0; w < 8; w++) fl |= flags[w];
+        const bool any_bad = fl != 0u;
+        void* y_u = p.Y_tab[u];
+#pragma unroll
+        for (int t = 0; t < NACC; t++) {
+            int32_t s[PL_N];
+#pragma unroll
+            for (int r = 0; r < 4; r++) s[r] = acc[t][r];
+            s[4] = __shfl_down(acc[t][0], 16, 64);
+            s[5] = __shfl_down(acc[t][1], 16, 64);
+            const int64_t n = ncol0 + 16 * t;
+            if (g == 0 && n < p.N) {
+                const float sc = bits_to_f32_rt(pre_s[t], p.scale_dtype);
+                const float bs = bias_u ? bits_to_f32_rt(pre_b[t], p.bias_dtype) : 0.0f;
+                pl_store(y_u, nullptr, n, planes_to_f32(s), sc, bs, any_bad);
+            }
+        }
+        __syncthreads();  // every wave is done with the planes before the next item overwrites them
+    }
+}
+
+// ---- host side ----------------------------------------------------------------------------------------
+// One fp16 row, K a multiple of 16 and at most PL_MAX_K, N a multiple of 4, aligned operands: the shapes both
+// weight layouts can serve, so that a layer gives the same bits whichever copy of its weights a call reads.
+constexpr int64_t PL_MAX_K = 16384;
+
+bool planes_supported(int x_dtype, int y_dtype, int64_t B, int64_t N, int64_t K, const void* X, const void* W, const void* Y,
+                      int w_layout) {
+    if (getenv("BITTORCH_NO_PLANES")) return false;  // A/B runs: the 16-bit matrix-core path instead
+    if (x_dtype != BT_F16 || y_dtype != BT_F16 || B != 1 || K % 16 != 0 || K > PL_MAX_K || K < 16 || N % 4 != 0) return false;
+    if (((uintptr_t)X) % 16 != 0 || ((uintptr_t)Y) % 2 != 0) return false;
+    if (w_layout == W_LAYOUT_TILED) return ((uintptr_t)W) % 256 == 0;
+    return ((uintptr_t)W) % 4 == 0 && (ceil_div(K, 4) + 64) * N < (1ll << 32);
+}
+
+template <int LAYOUT, int NACC, int EPI = EPI_NONE>
+static void launch_planes_k(const PlaneParams& p, hipStream_t st) {
+    constexpr int WAVES = 8, PF = 8;
+    const int nsteps = (int)ceil_div(p.K, 64);
+    const int spw = (int)ceil_div(nsteps, WAVES);
+    const size_t lds = (size_t)WAVES * 2 * 16 * NACC * 8 + WAVES * 4 + (size_t)WAVES * spw * 4 * PL_GROUP;
+    if (lds > 64 * 1024) {  // beyond the default limit of dynamic LDS (K > 10240 or so): raise it for this kernel, once
+        static bool raised = false;
+        if (!raised) {
+            (void)hipFuncSetAttribute((const void*)gemv_planes_kernel<LAYOUT, NACC, WAVES, PF, EPI>,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+            raised = true;
+        }
+    }
+    hipLaunchKernelGGL((gemv_planes_kernel<LAYOUT, NACC, WAVES, PF, EPI>), dim3((unsigned)(p.per_xcd * 8)), dim3(WAVES * 64), lds, st, p);
+}
+
+// epi_op = EPI_SWIGLU_PAIRS: tiled copy in gate/up pair order, N % 32 == 0, no residual; Y is [N/2]
+int launch_planes(const void* X, const uint8_t* W, int w_layout, const Epilogue& epi, void* Y, int64_t N, int64_t K,
+                  int epi_op, hipStream_t st) {
+    PlaneParams p = {};
+    p.X = X; p.W = W; p.scale = epi.scale; p.bias = epi.bias; p.residual = epi.residual; p.Y = Y;
+    p.scale_dtype = epi.scale_dtype; p.bias_dtype = epi.bias_dtype; p.scale_bcast = epi.scale_bcast;
+    p.N = N; p.K = K; p.Kb = ceil_div(K, 4);
+    p.G = 1;
+    p.wsteps = (int)ceil_div(p.Kb, 16);
+    p.tiles16 = (int)ceil_div(N, 16);
+    // 16-column tiles per workgroup: as many as still give every compute unit a workgroup
+    int nacc = (w_layout == W_LAYOUT_TILED) ? 4 : 2;
+    if (const char* env = getenv("BITTORCH_PLANES_NACC")) nacc = atoi(env);
+    const int min_nacc = (epi_op == EPI_SWIGLU_PAIRS) ? 2 : 1;
+    while (nacc > min_nacc && ceil_div(p.tiles16, nacc) < 224) nacc >>= 1;
+    if (nacc != 1 && nacc != 2 && nacc != 4) nacc = min_nacc;
+    if (w_layout != W_LAYOUT_TILED && nacc > 2) nacc = 2;
+    if (nacc < min_nacc) nacc = min_nacc;
+    p.tiles = (int)ceil_div(p.tiles16, nacc);
+    p.per_xcd = (int)ceil_div(p.tiles, 8);
+    if (epi_op == EPI_SWIGLU_PAIRS) {
+        if (w_layout != W_LAYOUT_TILED || N % 32 != 0 || epi.residual) {
+            set_error("gemv_planes: the SwiGLU output stage needs pair-ordered tiled weights, N %% 32 == 0 and no residual");
+            return BT_ERR_INVALID;
+        }
+        if (nacc == 4) launch_planes_k<PL_TILED, 4, EPI_SWIGLU_PAIRS>(p, st);
+        else launch_planes_k<PL_TILED, 2, EPI_SWIGLU_PAIRS>(p, st);
+        return check_launch("gemv_planes");
+    }
+    if (w_layout == W_LAYOUT_TILED) {
+        if (nacc == 4) launch_planes_k<PL_TILED, 4>(p, st);
+        else if (nacc == 2) launch_planes_k<PL_TILED, 2>(p, st);
+        else launch_planes_k<PL_TILED, 1>(p, st);
+    } else {
+        if (nacc == 2) launch_planes_k<PL_ROWMAJOR, 2>(p, st);
+        else launch_planes_k<PL_ROWMAJOR, 1>(p, st);
+    }
+    return check_launch("gemv_planes");
+}
+
+// grouped launch: 2 workgroups of 8 waves per compute unit
+static int g_group_cus = 0;
+
+static int launch_group_params(PlaneParams p, int64_t G, hipStream_t st) {
+    if (!g_group_cus) {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        g_group_cus = cus;
+    }
+    const int64_t wgs = 2 * (int64_t)g_group_cus;
+    // columns per wave: 32 (two tiles) streams best (5.3 TB/s against 4.8 with four tiles and 4.4-5.0 with one at
+    // G = 128, 4096 x 4096); another width only where it fills the resident workgroups markedly more evenly
+    int nacc = 2;
+    if (const char* env = getenv("BITTORCH_GROUP_NACC")) {
+        nacc = atoi(env);
+        if (nacc != 1 && nacc != 2 && nacc != 4) nacc = 2;
+    } else {
+        double best = -1.0;
+        const int order[3] = {2, 4, 1};
+        for (int i = 0; i < 3; i++) {
+            const int c = order[i];
+            const int64_t items = G * ceil_div(p.tiles16, 8 * c);
+            const double eff = (double)items / (double)(ceil_div(items, wgs) * wgs) *
+                               ((double)p.tiles16 / (double)(ceil_div(p.tiles16, 8 * c) * 8 * c));
+            if (eff > best * 1.15) { best = eff; nacc = c; }
+        }
+    }
+    p.slabs = (int)ceil_div(p.tiles16, 8 * nacc);
+    p.items = (int)(G * p.slabs);
+    const unsigned grid = (unsigned)((p.items < wgs) ? p.items : wgs);
+    int pf = 8;
+    if (const char* env = getenv("BITTORCH_GROUP_PF")) pf = atoi(env);
+    const int SP = (int)ceil_div(p.wsteps, pf) * pf;
+    const size_t lds = 32 + (size_t)SP * 4 * PL_GROUP;
+    if (pf == 16) {
+        if (nacc == 4) hipLaunchKernelGGL((gemv_planes_group_kernel<4, 16>), dim3(grid), dim3(512), lds, st, p);
+        else if (nacc == 2) hipLaunchKernelGGL((gemv_planes_group_kernel<2, 16>), dim3(grid), dim3(512), lds, st, p);
+        else hipLaunchKernelGGL((gemv_planes_group_kernel<1, 16>), dim3(grid), dim3(512), lds, st, p);
+    } else {
+        if (nacc == 4) hipLaunchKernelGGL((gemv_planes_group_kernel<4, 8>), dim3(grid), dim3(512), lds, st, p);
+        else if (nacc == 2) hipLaunchKernelGGL((gemv_planes_group_kernel<2, 8>), dim3(grid), dim3(512), lds, st, p);
+        else hipLaunchKernelGGL((gemv_planes_group_kernel<1, 8>), dim3(grid), dim3(512), lds, st, p);
+    }
+    return check_launch("gemv_planes_group");
+}
+
+int launch_planes_group(const void* const* X_tab, const uint8_t* const* W_tab, const void* const* scale_tab, int scale_dtype,
+                        int scale_bcast, const void* const* bias_tab, int bias_dtype, void* const* Y_tab, int64_t G, int64_t N,
+                        int64_t K, hipStream_t st) {
+    PlaneParams p = {};
+    p.X_tab = X_tab; p.W_tab = W_tab; p.scale_tab = scale_tab; p.bias_tab = bias_tab; p.Y_tab = Y_tab;
+    p.scale_dtype = scale_dtype; p.bias_dtype = bias_dtype; p.scale_bcast = scale_bcast;
+    p.N = N; p.K = K; p.Kb = ceil_div(K, 4);
+    p.G = (int)G;
+    p.wsteps = (int)ceil_div(p.Kb, 16);
+    p.tiles16 = (int)ceil_div(N, 16);
+    return launch_group_params(p, G, st);
+}
+
+}  // namespace bt

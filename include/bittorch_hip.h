@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define BT_ABI_VERSION 1
+#define BT_ABI_VERSION 2
 
 /* element types of activations / scales / biases / outputs */
 typedef enum { BT_F32 = 0, BT_F16 = 1, BT_BF16 = 2, BT_I8 = 3 /* bt_unpack_dequant output only */ } bt_dtype;
@@ -49,8 +49,6 @@ typedef enum {
  * activations (three bf16 planes); bt_ternary_gemm_i8 keeps the argument so that a
  * kernel that needs scratch can be introduced without an ABI change.
  */
-#define BT_WORKSPACE_COUNTER_BYTES 16384 /* kept for callers that clear the head of a workspace; unused */
-
 /* ABI version of the loaded library (BT_ABI_VERSION at build time). */
 int bt_abi_version(void);
 
@@ -92,8 +90,12 @@ int bt_ternary_linear_forward(const void* X, int x_dtype, const int8_t* W_tern, 
  * Replaces bittorch._C.ternary_linear_packed_forward (bittorch_bindings.cpp:48-63,
  * dispatch.cpp:105-142, csrc/kernels/ternary_gemm_production.cu:286-362).
  *   X [B,K] x_dtype; W_T [ceil(K/4),N] uint8; Y [B,N] x_dtype.
- *   Batches up to 32 rows stream the weights once per 16 rows (decode shape); taller
- *   batches run the tiled 16-bit matrix-core GEMM.  fp32 activations with K % 64 == 0 are
+ *   A cost model fitted to measurements picks the kernel: the streaming kernel (weights read once
+ *   per 16 rows, all 16-row blocks of the call in one launch) while B*N*K is small, the tiled 16-bit
+ *   matrix-core GEMM beyond (crossover near 1.5-2 M outputs for K = 2560..4096;
+ *   BITTORCH_STREAM_MAX_ROWS=n replaces the rule by "B <= n").  A single fp16 row (K % 16 == 0,
+ *   K <= 16384, N % 4 == 0) runs the exact GEMV on the int8 matrix cores: the dot products are summed
+ *   without rounding and rounded to fp32 once.  fp32 activations with K % 64 == 0 are
  *   first split into three bf16 planes (x = hi + mid + lo exactly) in the workspace and run
  *   on the same bf16 kernels with exact products and fp32 accumulation.  Other fp32 shapes,
  *   unaligned operands, a missing workspace and BITTORCH_KERNEL=generic run a generic
@@ -247,6 +249,25 @@ int bt_ternary_gemm_i8_tiled(const int8_t* Q, int q_layout, const float* s_x, co
                              int64_t B, int64_t N, int64_t K, void* stream);
 
 /*
+ * G independent decode GEMVs in ONE launch (no counterpart in the reference, whose packed kernel
+ * csrc/kernels/ternary_gemm_production.cu:53-142 serves one matrix per launch): unit u computes
+ *   Y_tab[u] [N] = X_tab[u] [K] (fp16) x W_tiled_tab[u] (decode-tiled copy of a W_T [ceil(K/4), N]) * scale + bias
+ * exactly as a single bt_ternary_linear_tiled_forward call on one row would (bit-identical outputs).  A
+ * 4 MiB weight matrix takes less time to stream than a kernel takes to start and drain; this entry point
+ * pays launch, set-up and drain once for G matrices: persistent workgroups walk (unit, column slab)
+ * items and keep their weight loads running from one item into the next.
+ *   The five tables are DEVICE arrays of G device pointers, caller-owned (bias_tab may be NULL: no
+ *   bias; its entries may not be NULL otherwise).  Every unit has the same N, K, scale length
+ *   (N, or 1 = per-tensor) and element types.  x_dtype must be BT_F16, Y is fp16; K % 16 == 0, K <= 10240;
+ *   each W_tiled 256-byte aligned, each X 16-byte aligned.  Units may share operands (one x for many
+ *   matrices, one matrix for many rows) but not outputs.
+ */
+int bt_ternary_gemv_grouped(const void* const* X_tab, int x_dtype, const uint8_t* const* W_tiled_tab,
+                            const void* const* scale_tab, int scale_dtype, int64_t scale_len,
+                            const void* const* bias_tab, int bias_dtype, void* const* Y_tab, int64_t G,
+                            int64_t N, int64_t K, void* stream);
+
+/*
  * Matrix-core forward from float activations: bt_act_quant_i8 followed by
  * bt_ternary_gemm_i8.  Replaces bittorch._C.ternary_linear_tensor_core_forward
  * (bittorch_bindings.cpp:65-87, ternary_gemm_tensor_core.cu:663-727) for
@@ -300,19 +321,6 @@ int bt_unpack_dequant(const uint8_t* W_T, const float* scale, int64_t scale_len,
  * with the packed matrix-core kernels.
  */
 int bt_pack_ternary_i8(const int8_t* W_tern, int64_t N, int64_t K, uint8_t* packed_T, void* stream);
-
-/*
- * Measurement aid with no counterpart in the reference: launches `blocks`
- * workgroups of 8 waves that each issue `iters` x 8 back-to-back
- * v_mfma_i32_16x16x64_i8 on register operands (no memory traffic) and writes the
- * operation count of the launch (2*16*16*64 per instruction) to *ops_per_launch.
- * random_operands = 0: small constant operands; 1: pseudo-random int8 activations
- * and ternary weights, i.e. the switching activity of real data.  Timing it gives
- * the int8 matrix-core rate the chip sustains, next to which the prefill GEMM is
- * reported.  `out` is a device int the kernel may write.
- */
-int bt_probe_mfma_i8(int blocks, int iters, int random_operands, int* out, double* ops_per_launch,
-                     void* stream);
 
 #ifdef __cplusplus
 }

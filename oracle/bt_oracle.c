@@ -17,6 +17,9 @@
  *                                 and all-ones weights, the reference's JS
  *                                 known-answer vectors)
  *   bto_linear_unpacked pinned   (same checks as bto_linear_packed)
+ *   bto_linear_packed_exact_f16  pinned (the same linear with the sum formed exactly and
+ *                                 rounded once: float64 dot product, exact for fp16
+ *                                 operands, rounded to fp32; ties and subnormals)
  *   bto_act_quant_i8    parity unpinned by the reference (no reference test
  *   bto_gemm_i8         touches the int8 path); pinned here only by brute
  *                       force on tiny inputs, exact integer identities and
@@ -265,6 +268,52 @@ void bto_linear_packed_f64(const float* X, const uint8_t* W_T, const float* scal
             Y[b * N + n] = acc * s + bv;
         }
     }
+}
+
+/*
+ * The same linear with the dot product summed exactly (what the library's single-row fp16 GEMV does on
+ * the int8 matrix cores): the reference's loop (ternary_gemm_production.cu:126-133) adds one rounded
+ * fp32 term at a time; here X[k] = x[k] * 2^24 is an integer for every finite fp16 x (|X| < 2^40), the
+ * sum S = sum_k X[k] * w[k,n] is an exact 64-bit integer, and acc = RN_fp32(S) * 2^-24 is the correctly
+ * rounded dot product.  Epilogue as above (:139-141): one fp32 multiply, one fp32 add.
+ * X must hold fp16 values widened to float (checked: anything else returns -1); a row with an
+ * infinity or a NaN gives NaN in every column.  Returns 0.
+ * Pinned by the float64 dot product, which is exact for these operands while |S| < 2^53, rounded once
+ * to fp32 (tests/test_oracle.py).
+ */
+int bto_linear_packed_exact_f16(const float* X, const uint8_t* W_T, const float* scale,
+                                int64_t scale_len, const float* bias, float* Y, int64_t B,
+                                int64_t N, int64_t K) {
+    int64_t* XI = (int64_t*)malloc((size_t)B * K * sizeof(int64_t));
+    uint8_t* bad = (uint8_t*)calloc((size_t)B, 1);
+    if (!XI || !bad) { free(XI); free(bad); return -2; }
+    int status = 0;
+    for (int64_t b = 0; b < B; b++)
+        for (int64_t k = 0; k < K; k++) {
+            const float x = X[b * K + k];
+            if (!(fabsf(x) <= 65504.0f)) { bad[b] = 1; XI[b * K + k] = 0; continue; }
+            if (round_to_f16(x) != x) status = -1; /* not an fp16 value */
+            XI[b * K + k] = (int64_t)((double)x * 16777216.0); /* exact: fp16 values are multiples of 2^-24 */
+        }
+    if (status == 0) {
+#pragma omp parallel for schedule(static)
+        for (int64_t n = 0; n < N; n++) {
+            const float s = scale[scale_len == 1 ? 0 : n];
+            const float bv = bias ? bias[n] : 0.0f;
+            for (int64_t b = 0; b < B; b++) {
+                int64_t S = 0;
+                for (int64_t k = 0; k < K; k++)
+                    S += XI[b * K + k] * (int64_t)decode2((W_T[(k / 4) * N + n] >> (2 * (k % 4))) & 3u);
+                const float acc = (float)S * 5.9604644775390625e-08f; /* RN(S) * 2^-24, the scaling exact */
+                float r = acc * s;
+                r = r + bv;
+                Y[b * N + n] = bad[b] ? NAN : r;
+            }
+        }
+    }
+    free(XI);
+    free(bad);
+    return status;
 }
 
 /*

@@ -51,6 +51,8 @@ def lib() -> ctypes.CDLL:
         _lib.bto_linear_packed.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64]
         _lib.bto_linear_packed_f64.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64]
         _lib.bto_linear_unpacked.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64]
+        _lib.bto_linear_packed_exact_f16.restype = ctypes.c_int
+        _lib.bto_linear_packed_exact_f16.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64]
         _lib.bto_act_quant_i8.argtypes = [_vp, _i64, _i64, _vp, _vp]
         _lib.bto_gemm_i8.argtypes = [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64]
         _lib.bto_exp_fixed.restype = ctypes.c_float
@@ -165,6 +167,22 @@ def linear_packed(x, w_packed_t, scale, in_features: int, bias=None, f64: bool =
     y = np.empty((b, n), dtype=np.float64 if f64 else np.float32)
     fn = lib().bto_linear_packed_f64 if f64 else lib().bto_linear_packed
     fn(_p(x), _p(w), _p(scale), scale.size, _p(bias), _p(y), b, n, k)
+    return y
+
+
+def linear_packed_exact_f16(x, w_packed_t, scale, in_features: int, bias=None) -> np.ndarray:
+    """Packed linear for fp16 activations (given widened to float) with the dot product summed exactly and
+    rounded to fp32 once; fp32 result before the cast to the output dtype."""
+    x, scale, bias = _lin_args(x, w_packed_t, scale, bias)
+    w = np.ascontiguousarray(np.asarray(w_packed_t, dtype=np.uint8))
+    b, k = x.shape
+    assert k == in_features and w.shape[0] == (k + 3) // 4
+    n = w.shape[1]
+    assert scale.size in (1, n)
+    y = np.empty((b, n), dtype=np.float32)
+    rc = lib().bto_linear_packed_exact_f16(_p(x), _p(w), _p(scale), scale.size, _p(bias), _p(y), b, n, k)
+    if rc != 0:
+        raise ValueError("activations are not fp16 values" if rc == -1 else "out of memory")
     return y
 
 

@@ -20,7 +20,7 @@ def test_header_declares_expected_entry_points():
     syms = _declared_symbols()
     for name in ("bt_quantize_pack", "bt_ternary_linear_forward", "bt_ternary_linear_packed_forward",
                  "bt_act_quant_i8", "bt_ternary_gemm_i8", "bt_ternary_linear_tensor_core_forward",
-                 "bt_unpack_dequant", "bt_pack_ternary_i8", "bt_probe_mfma_i8", "bt_last_error", "bt_abi_version",
+                 "bt_unpack_dequant", "bt_pack_ternary_i8", "bt_ternary_gemv_grouped", "bt_ternary_linear_tensor_core_forward_static", "bt_last_error", "bt_abi_version",
                  "bt_ternary_linear_packed_forward_res", "bt_ternary_gemm_i8_res", "bt_tiled_weights_bytes",
                  "bt_retile_weights", "bt_untile_weights", "bt_ternary_linear_tiled_forward", "bt_ternary_gemm_i8_tiled", "bt_swiglu", "bt_rmsnorm",
                  "bt_act_quant_i8_layout", "bt_ternary_linear_packed_forward_fused",

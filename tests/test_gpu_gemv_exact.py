@@ -1,0 +1,179 @@
+"""GPU parity of the exact single-row fp16 GEMV (int8 matrix cores, six base-128 digit rows) and of the grouped
+launch that runs G such GEMVs at once.
+
+Bar: bit-exact against `oracle.linear_packed_exact_f16` (the dot product summed as an integer and rounded to
+fp32 once, then the reference's epilogue `acc * scale + bias`, csrc/kernels/ternary_gemm_production.cu:139-141),
+on both weight layouts; against the reference's own fp32-accumulate arithmetic (`oracle.linear_packed`) within
+its tests' thresholds (tests/test_packed_kernel.py:44-50: element-wise rtol = atol = 1e-2 for fp16); every unit
+of a grouped launch bit-identical to the single call.
+"""
+import numpy as np
+import pytest
+import torch
+
+from conftest import announce
+from _util import f32np, random_ternary, seeded_acts
+
+pytestmark = pytest.mark.gpu
+
+
+def _setup(n, k, seed, per_tensor=False, bias=True, wide=False):
+    from bittorch_amd.quant import pack_ternary_transposed
+    w = random_ternary(n, k, seed=seed)
+    g = torch.Generator().manual_seed(seed + 7)
+    scale = torch.rand(1 if per_tensor else n, generator=g) * 0.05 + 0.01
+    bias_t = (torch.randn(n, generator=g) * 0.01).half() if bias else None
+    x = seeded_acts(1, k, seed=seed + 3, dtype=torch.float32)
+    if wide:  # the whole dynamic range of fp16, subnormals included
+        x = x * torch.exp2(torch.randint(-24, 12, (1, k), generator=g).float())
+    x = x.half()
+    packed, _ = pack_ternary_transposed(w)
+    return x, packed, scale, bias_t
+
+
+def _expect(oracle, x, packed, scale, bias, k):
+    y = oracle.linear_packed_exact_f16(f32np(x), packed.numpy(), f32np(scale), k, None if bias is None else f32np(bias))
+    return torch.from_numpy(y).half()
+
+
+@pytest.mark.parametrize("wide", [False, True])
+@pytest.mark.parametrize("n,k", [(4096, 4096), (64, 64), (16, 16), (100, 144), (2560, 2560), (7680, 2560), (2560, 6912),
+                                 (36, 8192), (11008, 4096), (260, 1040), (4, 48), (48, 16384), (2048, 11008)])
+def test_single_row_fp16_is_exact_on_both_layouts(oracle, n, k, wide):
+    from bittorch_amd import _C
+    announce("exact gemv", n, k, wide)
+    x, packed, scale, bias, = _setup(n, k, seed=n + k, wide=wide)
+    expect = _expect(oracle, x, packed, scale, bias, k)
+    xd, pd, sd, bd = x.cuda(), packed.cuda(), scale.cuda(), bias.cuda()
+    y_rm = _C.ternary_linear_packed_forward(xd, pd, sd, bd, k)
+    tiled = _C.retile_weights(pd, k)
+    y_t = _C.ternary_linear_tiled_forward(xd, tiled, sd, bd, k, n)
+    torch.cuda.synchronize()
+    assert torch.equal(y_rm.cpu(), expect)
+    assert torch.equal(y_t.cpu(), expect)
+    # the reference's arithmetic (fp32 accumulation in k order), at its own tests' fp16 thresholds
+    ref = oracle.linear_packed(f32np(x), packed.numpy(), f32np(scale), k, f32np(bias))
+    if not wide:
+        np.testing.assert_allclose(f32np(y_t), ref, rtol=1e-2, atol=1e-2)
+
+
+def test_single_row_fp16_variants(oracle):
+    """Per-tensor scale, fp16 scale, no bias, a residual, tile widths of the kernel, ties and extreme values."""
+    import os
+    from bittorch_amd import _C
+    announce("exact gemv variants")
+    n, k = 512, 1024
+    x, packed, scale, bias = _setup(n, k, seed=3, per_tensor=True)
+    xd, pd = x.cuda(), packed.cuda()
+    tiled = _C.retile_weights(pd, k)
+    expect = _expect(oracle, x, packed, scale, bias, k)
+    assert torch.equal(_C.ternary_linear_tiled_forward(xd, tiled, scale.cuda(), bias.cuda(), k, n).cpu(), expect)
+    assert torch.equal(_C.ternary_linear_packed_forward(xd, pd, scale.cuda(), bias.cuda(), k).cpu(), expect)
+    s16 = scale.half()
+    expect16 = _expect(oracle, x, packed, s16.float(), None, k)
+    assert torch.equal(_C.ternary_linear_tiled_forward(xd, tiled, s16.cuda(), None, k, n).cpu(), expect16)
+    res = seeded_acts(1, n, seed=9, dtype=torch.float16)
+    got = _C.ternary_linear_tiled_forward(xd, tiled, scale.cuda(), bias.cuda(), k, n, residual=res.cuda())
+    assert torch.equal(got.cpu(), expect + res)
+    try:
+        for nacc in ("1", "2", "4"):
+            os.environ["BITTORCH_PLANES_NACC"] = nacc
+            assert torch.equal(_C.ternary_linear_tiled_forward(xd, tiled, scale.cuda(), bias.cuda(), k, n).cpu(), expect)
+            assert torch.equal(_C.ternary_linear_packed_forward(xd, pd, scale.cuda(), bias.cuda(), k).cpu(), expect)
+    finally:
+        os.environ.pop("BITTORCH_PLANES_NACC", None)
+    # ties of the final rounding and the largest magnitudes: all-ones weights, crafted activations
+    from bittorch_amd.quant import pack_ternary_transposed
+    ones = pack_ternary_transposed(torch.ones(16, 16, dtype=torch.int8))[0]
+    u = 2.0 ** -24
+    for vals in ([1.0, u], [1.0, u, u, u], [-1.0, -u], [65504.0] * 16, [65504.0, u, -65504.0], [-0.0, 0.0]):
+        xv = torch.zeros(1, 16, dtype=torch.float16)
+        xv[0, :len(vals)] = torch.tensor(vals, dtype=torch.float64).half()
+        e = _expect(oracle, xv, ones, torch.ones(16), None, 16)
+        assert torch.equal(_C.ternary_linear_packed_forward(xv.cuda(), ones.cuda(), torch.ones(16).cuda(), None, 16).cpu(), e)
+    # an infinity or a NaN in the row: NaN everywhere (as in the reference whenever it meets a zero weight)
+    xv = x.clone()
+    xv[0, 5] = float("inf")
+    assert torch.isnan(_C.ternary_linear_tiled_forward(xv.cuda(), tiled, scale.cuda(), bias.cuda(), k, n)).all()
+
+
+def _tables(_C, xs, tiles, scales, biases, ys):
+    return (_C.pointer_table(xs), _C.pointer_table(tiles), _C.pointer_table(scales),
+            None if biases is None else _C.pointer_table(biases), _C.pointer_table(ys))
+
+
+@pytest.mark.parametrize("g,n,k,per_tensor,bias", [(1, 4096, 4096, True, True), (5, 256, 512, False, True),
+                                                   (37, 1024, 1024, False, False), (3, 100, 144, False, True),
+                                                   (9, 2560, 6912, True, True), (130, 128, 64, False, True),
+                                                   (4, 36, 8192, False, True)])
+def test_grouped_launch_equals_single_calls(oracle, g, n, k, per_tensor, bias):
+    import os
+    from bittorch_amd import _C
+    announce("grouped gemv", g, n, k)
+    xs, tiles, scales, biases, singles = [], [], [], [], []
+    for u in range(g):
+        x, packed, scale, b = _setup(n, k, seed=100 * u + n, per_tensor=per_tensor, bias=bias, wide=(u % 2 == 1))
+        xs.append(x.cuda())
+        tiles.append(_C.retile_weights(packed.cuda(), k))
+        scales.append(scale.cuda())
+        biases.append(b.cuda() if bias else None)
+        singles.append(_C.ternary_linear_tiled_forward(xs[-1], tiles[-1], scales[-1], biases[-1], k, n))
+        if u == 0:
+            assert torch.equal(singles[0].cpu(), _expect(oracle, x, packed, scale, b, k))
+    try:
+        for nacc in (None, "1", "2", "4"):
+            if nacc:
+                os.environ["BITTORCH_GROUP_NACC"] = nacc
+            ys = [torch.full((1, n), float("nan"), dtype=torch.float16, device="cuda") for _ in range(g)]
+            tabs = _tables(_C, xs, tiles, scales, biases if bias else None, ys)
+            _C.ternary_gemv_grouped(*tabs, k, n, scale_len=1 if per_tensor else n)
+            torch.cuda.synchronize()
+            for u in range(g):
+                assert torch.equal(ys[u], singles[u]), (u, nacc)
+    finally:
+        os.environ.pop("BITTORCH_GROUP_NACC", None)
+
+
+def test_grouped_launch_config2_units_and_shared_operands(oracle):
+    """G = 24 config-2 units (x fp16 [1,4096], W [4096,4096], per-tensor fp32 scale, fp16 bias), some units
+    sharing their activations or their weights; second call on the same tables gives the same result."""
+    from bittorch_amd import _C
+    announce("grouped gemv config 2")
+    n = k = 4096
+    base = [_setup(n, k, seed=s, per_tensor=True) for s in range(4)]
+    xs_, tiles_, scales_, biases_ = [], [], [], []
+    for (x, packed, scale, b) in base:
+        xs_.append(x.cuda()); tiles_.append(_C.retile_weights(packed.cuda(), k)); scales_.append(scale.cuda()); biases_.append(b.cuda())
+    units = [(u % 4, (u // 4) % 4) for u in range(24)]  # (activation, weight) index pairs
+    xs = [xs_[a] for a, _ in units]
+    tiles = [tiles_[w] for _, w in units]
+    scales = [scales_[w] for _, w in units]
+    biases = [biases_[w] for _, w in units]
+    ys = [torch.empty(1, n, dtype=torch.float16, device="cuda") for _ in units]
+    tabs = _tables(_C, xs, tiles, scales, biases, ys)
+    for _ in range(2):
+        for y in ys:
+            y.fill_(float("nan"))
+        _C.ternary_gemv_grouped(*tabs, k, n, scale_len=1)
+        torch.cuda.synchronize()
+        for (a, w), y in zip(units, ys):
+            x, packed, scale, b = base[a][0], base[w][1], base[w][2], base[w][3]
+            assert torch.equal(y, _C.ternary_linear_tiled_forward(xs_[a], tiles_[w], scales_[w], biases_[w], k, n))
+    x, packed, scale, b = base[1][0], base[2][1], base[2][2], base[2][3]
+    assert torch.equal(ys[units.index((1, 2))].cpu(), _expect(oracle, x, packed, scale, b, k))
+
+
+def test_grouped_launch_argument_errors():
+    from bittorch_amd import _C, _lib
+    lib = _lib.load()
+    t = torch.zeros(8, dtype=torch.int64, device="cuda")
+    p = t.data_ptr()
+    assert lib.bt_ternary_gemv_grouped(None, 1, p, p, 0, 16, None, 1, p, 8, 16, 16, None) == -1
+    assert "null" in _lib.last_error()
+    assert lib.bt_ternary_gemv_grouped(p, 2, p, p, 0, 16, None, 1, p, 8, 16, 16, None) == -1
+    assert "fp16" in _lib.last_error()
+    assert lib.bt_ternary_gemv_grouped(p, 1, p, p, 0, 16, None, 1, p, 8, 16, 24, None) == -1
+    assert "multiple of 16" in _lib.last_error()
+    assert lib.bt_ternary_gemv_grouped(p, 1, p, p, 0, 5, None, 1, p, 8, 16, 16, None) == -1
+    assert "scale" in _lib.last_error()
+    assert lib.bt_ternary_gemv_grouped(p, 1, p, p, 0, 16, None, 1, p, 0, 16, 16, None) == -1

@@ -195,6 +195,63 @@ def test_linear_sequential_fp32_order(oracle):
     assert oracle.linear_packed(x, p, np.ones(1, np.float32), 4, f64=True)[0, 0] == 2.0
 
 
+def test_linear_exact_f16_is_the_correctly_rounded_dot_product(oracle):
+    """The exact variant against float64: fp16 operands times +-1 are exact in float64 and so is their sum while
+    it stays below 2^53 units of 2^-24, hence float64 dot -> one rounding to fp32 is the correctly rounded result.
+    Plus the cases a wrong rounding, a dropped digit or a sign error would show: ties, subnormals, 65504, the
+    order-dependent example of the fp32 loop, the reference's known-answer vectors, non-finite rows."""
+    rng = np.random.default_rng(0)
+    for (b, n, k) in [(1, 8, 16), (3, 33, 64), (2, 64, 4096), (1, 5, 20)]:
+        w = random_ternary(n, k, seed=k + 1).numpy()
+        # wide dynamic range: random sign, 11-bit significand, exponents over the whole fp16 range incl. subnormals
+        x = (rng.standard_normal((b, k)) * np.exp2(rng.integers(-24, 15, (b, k)))).astype(np.float16).astype(np.float32)
+        x[np.abs(x) > 60000] = 1.0
+        packed_t, _ = oracle.pack_ternary_transposed(w)
+        ones = np.ones(n, np.float32)
+        acc64 = x.astype(np.float64) @ w.astype(np.float64).T
+        assert np.abs(acc64).max() * 2.0 ** 24 < 2.0 ** 53
+        np.testing.assert_array_equal(oracle.linear_packed_exact_f16(x, packed_t, ones, k), acc64.astype(np.float32))
+        # epilogue: one fp32 multiply, one fp32 add
+        scale = rng.random(n).astype(np.float32)
+        bias = rng.standard_normal(n).astype(np.float32)
+        expect = acc64.astype(np.float32) * scale[None, :] + bias[None, :]
+        np.testing.assert_array_equal(oracle.linear_packed_exact_f16(x, packed_t, scale, k, bias), expect)
+        np.testing.assert_array_equal(oracle.linear_packed_exact_f16(x, packed_t, scale[:1], k, bias),
+                                      acc64.astype(np.float32) * scale[0] + bias[None, :])
+    one = np.ones(1, np.float32)
+    p4, _ = oracle.pack_ternary_transposed(np.ones((1, 4), np.int8))
+    u = np.float32(2.0 ** -24)  # the smallest fp16 subnormal
+    # ties go to even: 1 + 2^-24 -> 1;  1 + 3 * 2^-24 -> 1 + 4 * 2^-24 = 1 + 2^-22;  -(1 + 2^-24) -> -1
+    assert oracle.linear_packed_exact_f16(np.array([[1.0, u, 0, 0]], np.float32), p4, one, 4)[0, 0] == 1.0
+    assert oracle.linear_packed_exact_f16(np.array([[1.0, u, u, u]], np.float32), p4, one, 4)[0, 0] == np.float32(1 + 2.0 ** -22)
+    assert oracle.linear_packed_exact_f16(np.array([[-1.0, -u, 0, 0]], np.float32), p4, one, 4)[0, 0] == -1.0
+    # what the fp32 loop loses, the exact sum keeps: 2048 + 1 - 2048 + 1 (fp16 values) is 2 either way, but
+    # 65504 + 2^-24 - 65504 is 2^-24 exactly here and 0 in the fp32 loop
+    x = np.array([[65504.0, u, -65504.0, 0]], np.float32)
+    assert oracle.linear_packed_exact_f16(x, p4, one, 4)[0, 0] == u
+    assert oracle.linear_packed(x, p4, one, 4)[0, 0] == 0.0
+    # sign of the weights, and the largest magnitudes on every term
+    m4, _ = oracle.pack_ternary_transposed(-np.ones((1, 4), np.int8))
+    x = np.full((1, 4), 65504.0, np.float32)
+    assert oracle.linear_packed_exact_f16(x, p4, one, 4)[0, 0] == np.float32(4 * 65504.0)
+    assert oracle.linear_packed_exact_f16(x, m4, one, 4)[0, 0] == np.float32(-4 * 65504.0)
+    # the reference's own known-answer vectors (small integers and halves: exact in fp16)
+    for case in GOLD["matmul"]:
+        w = np.array(case["weights"], dtype=np.int8)
+        packed_t, k = oracle.pack_ternary_transposed(w)
+        x = np.array(case["input"], dtype=np.float32)
+        if not np.array_equal(x.astype(np.float16).astype(np.float32), x):
+            continue
+        np.testing.assert_array_equal(oracle.linear_packed_exact_f16(x, packed_t, np.array(case["scales"], np.float32), k),
+                                      np.array(case["output"], dtype=np.float32))
+    # a row with an infinity or a NaN is NaN everywhere, other rows are untouched; non-fp16 inputs are refused
+    x = np.array([[1.0, np.inf, 0, 0], [1.0, 2.0, 3.0, 4.0]], np.float32)
+    y = oracle.linear_packed_exact_f16(x, p4, one, 4)
+    assert np.isnan(y[0, 0]) and y[1, 0] == 10.0
+    with pytest.raises(ValueError):
+        oracle.linear_packed_exact_f16(np.array([[1.0 + 2.0 ** -20, 0, 0, 0]], np.float32), p4, one, 4)
+
+
 # ---------------------------------------------------------------- int8 path (a7)
 def test_act_quant_brute_force(oracle):
     import math
