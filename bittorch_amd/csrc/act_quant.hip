@@ -160,6 +160,12 @@ static bool launch_act_quant_rows(const void* X, int64_t B, int64_t K, int8_t* Q
 int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x, int q_layout,
                      hipStream_t st) {
     const int ql = q_layout;
+    // the operand order is written 16 bytes at a time: callers check this too, but a buffer that cannot take it
+    // must never be written row-major under that name
+    if (ql == Q_OPERAND_ORDER && (K % 16 != 0 || ((uintptr_t)X) % 16 != 0 || ((uintptr_t)Q) % 16 != 0)) {
+        set_error("bt_act_quant_i8: the operand-order layout needs K %% 16 == 0 and 16-byte aligned X and Q");
+        return BT_ERR_INVALID;
+    }
     const bool done = (x_dtype == BT_F32)   ? launch_act_quant_rows<BT_F32>(X, B, K, Q, s_x, ql, st)
                       : (x_dtype == BT_F16) ? launch_act_quant_rows<BT_F16>(X, B, K, Q, s_x, ql, st)
                                             : launch_act_quant_rows<BT_BF16>(X, B, K, Q, s_x, ql, st);

@@ -135,7 +135,6 @@ static bool prefers_stream(int64_t B, int64_t N, int64_t K, bool int8) {
         if (v >= 1) return B <= v;
     }
     if (B <= 32) return true;
-    if (B > 16 * 65535) return false;
     const double work = (double)B * (double)N * (double)K;
     const double rounds = (double)ceil_div(ceil_div(B, 128) * ceil_div(N, 256), 256);
     const double wgs = (double)(ceil_div(B, 16) * ceil_div(N, int8 ? 128 : 64));

@@ -9,47 +9,46 @@
 namespace bt {
 
 // Y[b,n] = (sum_k x[b,k] * decode(W_T[k/4,n], k%4)) * scale[n] + bias[n]
-// One thread per output column, 256 columns per workgroup, grid.y = batch row.
+// One thread per output column, 256 columns per workgroup; grid.y walks the batch rows (any number of them: a
+// workgroup takes rows blockIdx.y, blockIdx.y + gridDim.y, ...).
 template <int XDT>
 __global__ __launch_bounds__(256) void packed_generic_kernel(const void* __restrict__ X,
                                                              const uint8_t* __restrict__ W_T, Epilogue epi,
-                                                             void* __restrict__ Y, int64_t N, int64_t K,
+                                                             void* __restrict__ Y, int64_t B, int64_t N, int64_t K,
                                                              int64_t Kb) {
     const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int64_t b = blockIdx.y;
     if (n >= N) return;
-    const int64_t xrow = b * K;
-    float acc = 0.0f;
-    for (int64_t kb = 0; kb < Kb; kb++) {
-        const uint32_t byte = W_T[kb * N + n];
+    const float s = epi_scale(epi, n), bv = epi_bias(epi, n);
+    for (int64_t b = blockIdx.y; b < B; b += gridDim.y) {
+        const int64_t xrow = b * K;
+        float acc = 0.0f;
+        for (int64_t kb = 0; kb < Kb; kb++) {
+            const uint32_t byte = W_T[kb * N + n];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int64_t k = 4 * kb + i;
-            if (k < K) {
-                const float w = (float)decode2((byte >> (2 * i)) & 3u);
-                acc = __fadd_rn(acc, __fmul_rn(load_elem<XDT>(X, xrow + k), w));
+            for (int i = 0; i < 4; i++) {
+                const int64_t k = 4 * kb + i;
+                if (k < K) {
+                    const float w = (float)decode2((byte >> (2 * i)) & 3u);
+                    acc = __fadd_rn(acc, __fmul_rn(load_elem<XDT>(X, xrow + k), w));
+                }
             }
         }
+        float y = epi_float(acc, s, bv);
+        if (epi.residual) y = add_residual(y, epi.residual, XDT, b * N + n);
+        store_elem<XDT>(Y, b * N + n, y);
     }
-    float y = epi_float(acc, epi_scale(epi, n), epi_bias(epi, n));
-    if (epi.residual) y = add_residual(y, epi.residual, XDT, b * N + n);
-    store_elem<XDT>(Y, b * N + n, y);
 }
 
 int launch_packed_generic(const void* X, int x_dtype, const uint8_t* W_T, const Epilogue& epi, void* Y,
                           int64_t B, int64_t N, int64_t K, hipStream_t st) {
     const int64_t Kb = ceil_div(K, 4);
-    const dim3 grid((unsigned)ceil_div(N, 256), (unsigned)B), block(256);
-    if (B > 65535) {
-        set_error("packed forward (generic kernel): batch %lld exceeds 65535 rows", (long long)B);
-        return BT_ERR_INVALID;
-    }
+    const dim3 grid((unsigned)ceil_div(N, 256), (unsigned)(B < 65535 ? B : 65535)), block(256);
     if (x_dtype == BT_F32)
-        hipLaunchKernelGGL(packed_generic_kernel<BT_F32>, grid, block, 0, st, X, W_T, epi, Y, N, K, Kb);
+        hipLaunchKernelGGL(packed_generic_kernel<BT_F32>, grid, block, 0, st, X, W_T, epi, Y, B, N, K, Kb);
     else if (x_dtype == BT_F16)
-        hipLaunchKernelGGL(packed_generic_kernel<BT_F16>, grid, block, 0, st, X, W_T, epi, Y, N, K, Kb);
+        hipLaunchKernelGGL(packed_generic_kernel<BT_F16>, grid, block, 0, st, X, W_T, epi, Y, B, N, K, Kb);
     else
-        hipLaunchKernelGGL(packed_generic_kernel<BT_BF16>, grid, block, 0, st, X, W_T, epi, Y, N, K, Kb);
+        hipLaunchKernelGGL(packed_generic_kernel<BT_BF16>, grid, block, 0, st, X, W_T, epi, Y, B, N, K, Kb);
     return check_launch("packed_generic");
 }
 
@@ -104,11 +103,20 @@ __global__ __launch_bounds__(256) void unpacked_kernel(const void* __restrict__ 
 
 int launch_unpacked(const void* X, int x_dtype, const int8_t* W, const Epilogue& epi, void* Y, int64_t B,
                     int64_t N, int64_t K, hipStream_t st) {
-    const dim3 grid((unsigned)ceil_div(N, 64), (unsigned)ceil_div(B, 16)), block(256);
-    if (ceil_div(B, 16) > 65535) {
-        set_error("bt_ternary_linear_forward: batch %lld too large", (long long)B);
-        return BT_ERR_INVALID;
+    // one launch covers 65535 blocks of 16 rows; a taller batch is served in slices of that many rows
+    const int64_t max_rows = 65535ll * 16;
+    if (B > max_rows) {
+        const int64_t esz = dtype_size(x_dtype);
+        for (int64_t r0 = 0; r0 < B; r0 += max_rows) {
+            Epilogue e = epi;
+            if (e.residual) e.residual = (const uint8_t*)epi.residual + r0 * N * esz;
+            const int rc = launch_unpacked((const uint8_t*)X + r0 * K * esz, x_dtype, W, e, (uint8_t*)Y + r0 * N * esz,
+                                           (B - r0 < max_rows) ? B - r0 : max_rows, N, K, st);
+            if (rc) return rc;
+        }
+        return BT_OK;
     }
+    const dim3 grid((unsigned)ceil_div(N, 64), (unsigned)ceil_div(B, 16)), block(256);
     if (x_dtype == BT_F32) hipLaunchKernelGGL(unpacked_kernel<BT_F32>, grid, block, 0, st, X, W, epi, Y, B, N, K);
     else if (x_dtype == BT_F16) hipLaunchKernelGGL(unpacked_kernel<BT_F16>, grid, block, 0, st, X, W, epi, Y, B, N, K);
     else hipLaunchKernelGGL(unpacked_kernel<BT_BF16>, grid, block, 0, st, X, W, epi, Y, B, N, K);

@@ -795,9 +795,19 @@ int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, co
     const StreamPlan pl = stream_plan(mode, B, N, Kb, w_layout, epi_op == EPI_SWIGLU_PAIRS ? 2 : 1);
     const int64_t Ny = (epi_op == EPI_SWIGLU_PAIRS) ? N / 2 : N;  // columns of Y
     const int y_size = dtype_size(y_dtype);
-    if (ceil_div(B, 16) > 65535) {
-        set_error("stream_gemm: %lld rows exceed the 65535 blocks of 16 rows one launch covers", (long long)B);
-        return BT_ERR_INVALID;
+    // one launch covers 65535 blocks of 16 rows; a taller call is served in slices of that many rows
+    const int64_t max_rows = 65535ll * 16;
+    if (B > max_rows) {
+        for (int64_t r0 = 0; r0 < B; r0 += max_rows) {
+            Epilogue e = epi;
+            if (e.residual) e.residual = (const uint8_t*)epi.residual + r0 * N * y_size;
+            const int rc = launch_stream(mode, (const uint8_t*)X + r0 * Kx * x_elem_size, x_elem_size, s_x ? s_x + r0 : nullptr, W_T,
+                                         w_layout, e, (uint8_t*)Y + r0 * Ny * y_size, y_dtype, acc_out ? acc_out + r0 * N : nullptr,
+                                         (B - r0 < max_rows) ? B - r0 : max_rows, N, K, planes, q_layout, pro_op, pro_b, pro_eps,
+                                         epi_op, st);
+            if (rc) return rc;
+        }
+        return BT_OK;
     }
     StreamParams p;
     p.X = X;
@@ -817,7 +827,6 @@ int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, co
     p.y_dtype = y_dtype;
     // (a row is a multiple of 16 bytes, so every 16-row block starts as aligned as the first)
     p.x_vec_ok = (((uintptr_t)p.X) % 16 == 0) && ((Kx * x_elem_size) % 16 == 0);
-    (void)Ny; (void)y_size;
     if (mode == MODE_I8) return launch_stream_mode<MODE_I8>(p, pl, st);
     if (mode == MODE_F16) return launch_stream_mode<MODE_F16>(p, pl, st);
     return launch_stream_mode<MODE_BF16>(p, pl, st);

@@ -2,11 +2,18 @@
 
 The reference re-runs ``ternary_quantize`` on the master weights in every forward
 (``bittorch/nn/ternary_linear.py:196-200``, ``bittorch/nn/ternary_linear_cuda.py:52-54``).
-The result depends on the weights only, so it is kept until they change: the key is the
-parameter's version counter (every in-place update, optimizer step or ``load_state_dict``
-bumps it), its storage address, dtype and device, and the quantizer's two settings.  With
-frozen weights (inference, evaluation, gradient accumulation) a forward then reads K*N/4
-bytes of packed weights instead of 4*K*N bytes of masters.
+The result depends on the weights only, so a forward that cannot be a training step (gradient
+mode off, or frozen weights) keeps it until the weights change: the key is the parameter's
+version counter (every tracked in-place update, ``load_state_dict`` or optimizer step bumps it),
+its storage address, dtype and device, and the quantizer's two settings.  Such a forward then
+reads K*N/4 bytes of packed weights instead of 4*K*N bytes of masters.
+
+A training forward (gradient mode on and ``weight.requires_grad``) never uses the cache and
+quantizes every time, exactly as the reference does: training code is where weights get written
+through ``.data`` (``w.data.clamp_()``, ``p.data.add_(...)``, EMA copies), and writes through
+``.data`` do not bump the version counter.  The one case that remains the caller's is an
+evaluation-time write through ``.data``; ``module.invalidate_packed_cache()`` (or any tracked
+write, e.g. ``with torch.no_grad(): w.copy_(...)``) makes the next forward re-quantize.
 """
 
 from __future__ import annotations
@@ -41,7 +48,9 @@ class PackedWeightCache:
 
 
 def cache_usable(x: Tensor, weight: Tensor) -> bool:
-    """The cache holds the quantization of the stored weights in their own dtype.  Under
-    autocast the autograd function quantizes an fp16 copy instead (reference semantics), and
-    float64 runs on the dense entry point, so neither uses it."""
+    """The cache holds the quantization of the stored weights in their own dtype.  A training forward
+    re-quantizes (see above).  Under autocast the autograd function quantizes an fp16 copy instead
+    (reference semantics), and float64 runs on the dense entry point, so neither uses it."""
+    if torch.is_grad_enabled() and weight.requires_grad:
+        return False
     return (not torch.is_autocast_enabled() and weight.dtype != torch.float64 and x.dtype != torch.float64)

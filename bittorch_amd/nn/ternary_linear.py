@@ -117,6 +117,11 @@ class TernaryLinear(nn.Module):
         bias = None if self.bias is None else self.bias.to(x.dtype)
         return F.linear(x, w_eff, bias)
 
+    def invalidate_packed_cache(self) -> None:
+        """Forget the cached packed weights (needed only after an evaluation-time write through ``weight.data``,
+        which the version counter the cache is keyed on does not see)."""
+        self._packed.clear()
+
     def extra_repr(self) -> str:
         return (f"in_features={self.in_features}, out_features={self.out_features}, "
                 f"bias={self.bias is not None}, threshold_factor={self.threshold_factor}, "

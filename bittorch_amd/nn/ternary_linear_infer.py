@@ -1,17 +1,20 @@
 """``TernaryLinearInference``: deployment layer that holds only packed weights.
 
-API mirror of ``bittorch/nn/ternary_linear_infer.py:22-193``.  Buffers:
-``weight_packed`` uint8 ``[ceil(K/4), N]`` (transposed layout), ``scale`` ``[N]``,
-optional ``bias``; nothing is trainable.  GPU inputs go to the packed HIP
-kernels; CPU inputs unpack and use ``F.linear`` as the reference does.
+API mirror of ``bittorch/nn/ternary_linear_infer.py:22-193``.  State: ``weight_packed`` uint8
+``[ceil(K/4), N]`` (transposed layout), ``scale`` ``[N]``, optional ``bias``; nothing is trainable.  GPU inputs go
+to the packed HIP kernels; CPU inputs unpack and use ``F.linear`` as the reference does.
 
-GPU calls read a second, *decode-tiled* copy of the packed weights that the layer builds from
-``weight_packed`` on first use (same size, not part of the ``state_dict``; same results bit for bit,
-15-25 % less time per decode GEMV because every load of the kernel then covers whole cache lines, a
-few per cent on the prefill GEMMs).  ``decode_tiled=False`` or ``BITTORCH_DECODE_TILED=0``
-keeps the layer on ``weight_packed`` alone.  ``forward_int8`` reads the copy at every batch size (the
-int8 prefill GEMM loads it with one 16-byte load per lane and stage instead of four dword loads and a
-byte transpose).
+On the GPU the layer keeps ONE copy of its weights: on its first GPU call it re-arranges ``weight_packed``
+into the *decode-tiled* layout every matrix-core kernel of the library reads (same 2 bits per weight; 15-25 %
+less time per decode GEMV because every load then covers whole cache lines, a few per cent on the prefill GEMMs)
+and releases the row-major buffer.  ``state_dict()`` still holds ``weight_packed`` in the reference's layout
+(rebuilt from the tiled copy with ``bt_untile_weights``, bit for bit), ``load_state_dict`` and ``.to()`` /
+``.cpu()`` work as usual.  Reading the attribute ``layer.weight_packed`` brings the row-major buffer back as a
+real buffer (so that in-place edits of it keep their meaning) and the layer then holds both copies until
+``drop_row_major()``; so does a call that only the row-major kernels can serve (the shape-generic kernel,
+fp32 activations with K % 64 != 0).  ``packed_weights()`` returns the reference-layout bytes without changing
+what the layer holds.  ``decode_tiled=False`` or ``BITTORCH_DECODE_TILED=0`` keeps the layer on ``weight_packed``
+alone.
 """
 
 from __future__ import annotations
@@ -45,37 +48,123 @@ class TernaryLinearInference(nn.Module):
         if decode_tiled is None:
             decode_tiled = os.environ.get("BITTORCH_DECODE_TILED", "1") != "0"
         self.decode_tiled = bool(decode_tiled)
+        # True: hold the reference-layout buffer beside the tiled copy (set once somebody needs it, see above)
+        self.keep_row_major = False
         # "natural", or "gate_up_pairs" for a fused [gate | up] layer whose decode calls go through
         # forward_swiglu (set by TernarySwiGLU; such a copy serves only that output stage)
-        self.tile_order = "natural"
+        self._tile_order = "natural"
         self._tiled: Optional[Tensor] = None
         self._tiled_key = None
 
+    # ---- which copies of the weights the layer holds ----------------------------------------
+    def _has_row_major(self) -> bool:
+        return "weight_packed" in self.__dict__["_buffers"]
+
+    def __getattr__(self, name: str):
+        if name == "weight_packed" and "_buffers" in self.__dict__ and not self._has_row_major() \
+                and self.__dict__.get("_tiled") is not None:
+            # somebody wants the buffer itself: bring it back for good (in-place edits must keep their meaning)
+            self._restore_row_major(keep=True)
+            return self._buffers["weight_packed"]
+        return super().__getattr__(name)
+
+    def _untiled(self) -> Tensor:
+        from .. import _C
+        return _C.untile_weights(self._tiled, self.out_features, self.in_features, self._tile_order == "gate_up_pairs")
+
+    def _restore_row_major(self, keep: bool) -> Tensor:
+        if not self._has_row_major():
+            wp = self._untiled()
+            self._buffers["weight_packed"] = wp
+            self._tiled_key = (wp.data_ptr(), wp._version, wp.device, self._tile_order)
+        if keep:
+            self.keep_row_major = True
+        return self._buffers["weight_packed"]
+
+    def packed_weights(self) -> Tensor:
+        """``W_T`` uint8 ``[ceil(K/4), N]`` in the reference's layout: the buffer if the layer holds it, otherwise a
+        fresh tensor rebuilt from the tiled copy (what the layer holds does not change)."""
+        return self._buffers["weight_packed"] if self._has_row_major() else self._untiled()
+
+    def drop_row_major(self) -> "TernaryLinearInference":
+        """Back to one resident copy: build the tiled copy if need be and release the row-major buffer."""
+        self.keep_row_major = False
+        if self.decode_tiled and self._has_row_major() and self._buffers["weight_packed"].is_cuda:
+            self.tiled_weights()
+        return self
+
+    @property
+    def tile_order(self) -> str:
+        return self._tile_order
+
+    @tile_order.setter
+    def tile_order(self, order: str) -> None:
+        if order not in ("natural", "gate_up_pairs"):
+            raise ValueError(f"tile_order must be 'natural' or 'gate_up_pairs', got {order!r}")
+        if order != self._tile_order and self._tiled is not None:
+            self._restore_row_major(keep=False)  # (in the old order) and re-tile on the next call
+            self._tiled, self._tiled_key = None, None
+        self._tile_order = order
+
     # ---- decode-tiled copy of the weights ---------------------------------------------------
     def tiled_weights(self) -> Tensor:
-        """The decode-tiled copy of ``weight_packed`` (GPU only), built on first use and rebuilt when
-        ``weight_packed`` has moved or been written since."""
-        wp = self.weight_packed
-        key = (wp.data_ptr(), wp._version, wp.device, self.tile_order)
+        """The decode-tiled copy of the weights (GPU only).  Built on first use from ``weight_packed``, which is
+        then released unless ``keep_row_major``; rebuilt when a held ``weight_packed`` has moved or been written."""
+        if not self._has_row_major():
+            return self._tiled
+        wp = self._buffers["weight_packed"]
+        key = (wp.data_ptr(), wp._version, wp.device, self._tile_order)
         if self._tiled is None or self._tiled_key != key:
             from .. import _C
-            self._tiled = _C.retile_weights(wp, self.in_features, self.tile_order == "gate_up_pairs")
+            self._tiled = _C.retile_weights(wp, self.in_features, self._tile_order == "gate_up_pairs")
             # built once on the current stream; later calls may come from any stream
             torch.cuda.current_stream(wp.device).synchronize()
             self._tiled_key = key
+        if not self.keep_row_major and not torch.cuda.is_current_stream_capturing():
+            del self._buffers["weight_packed"]  # one resident copy
         return self._tiled
+
+    def resident_weight_bytes(self) -> int:
+        """Bytes of packed weights the layer holds right now (tiled copy and / or row-major buffer)."""
+        n = self._buffers["weight_packed"].numel() if self._has_row_major() else 0
+        return n + (self._tiled.numel() if self._tiled is not None else 0)
+
+    # state_dict / load_state_dict / .to() / pickling see the reference's layout whatever the layer holds
+    def _save_to_state_dict(self, destination, prefix, keep_vars):
+        super()._save_to_state_dict(destination, prefix, keep_vars)
+        if not self._has_row_major():
+            moved = {prefix + name: destination.pop(prefix + name) for name in ("scale", "bias") if prefix + name in destination}
+            destination[prefix + "weight_packed"] = self._untiled()
+            destination.update(moved)  # the reference's key order: weight_packed, scale, bias
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        if not self._has_row_major():
+            self._restore_row_major(keep=False)
+        self._tiled, self._tiled_key = None, None
+        super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
+
+    def _apply(self, fn, *args, **kwargs):
+        if not self._has_row_major():
+            self._restore_row_major(keep=False)
+        self._tiled, self._tiled_key = None, None
+        return super()._apply(fn, *args, **kwargs)
 
     def __getstate__(self):
         # the tiled copy is derived data: rebuilt on demand, never pickled or deep-copied
         state = super().__getstate__() if hasattr(super(), "__getstate__") else self.__dict__.copy()
         state = dict(state)
+        if not self._has_row_major():
+            bufs = type(state["_buffers"])()
+            bufs["weight_packed"] = self._untiled()
+            bufs.update(state["_buffers"])
+            state["_buffers"] = bufs
         state["_tiled"], state["_tiled_key"] = None, None
         return state
 
     def prepare_decode(self) -> "TernaryLinearInference":
         """Build the decode-tiled copy now (e.g. before capturing decode steps into a HIP graph: a
         capture never builds it, it falls back to ``weight_packed``)."""
-        if self.decode_tiled and self.weight_packed.is_cuda:
+        if self.decode_tiled and (not self._has_row_major() or self._buffers["weight_packed"].is_cuda):
             self.tiled_weights()
         return self
 
@@ -83,7 +172,7 @@ class TernaryLinearInference(nn.Module):
         # (the tiled GEMMs read the copy too, so every batch size takes it; only the SwiGLU output stage of a
         # pair-ordered copy is a decode-shape affair)
         if not (self.decode_tiled and x.is_cuda and (rows <= DECODE_ROWS or order == "natural")
-                and self.tile_order == order):
+                and self._tile_order == order):
             return None
         if os.environ.get("BITTORCH_KERNEL") == "generic":  # the shape-generic kernel reads weight_packed
             return None
@@ -94,11 +183,18 @@ class TernaryLinearInference(nn.Module):
         kb = (self.in_features + 3) // 4
         if ((self.out_features + 15) // 16) * ((kb + 15) // 16) * 256 >= 2 ** 32:  # beyond the kernels' 32-bit offsets
             return None
-        wp = self.weight_packed
-        fresh = self._tiled is not None and self._tiled_key == (wp.data_ptr(), wp._version, wp.device, self.tile_order)
+        if not self._has_row_major():
+            return self._tiled
+        wp = self._buffers["weight_packed"]
+        fresh = self._tiled is not None and self._tiled_key == (wp.data_ptr(), wp._version, wp.device, self._tile_order)
         if not fresh and torch.cuda.is_current_stream_capturing():
             return None
         return self.tiled_weights()
+
+    def _row_major_for_call(self) -> Tensor:
+        """``weight_packed`` for a call that only the row-major kernels serve; a layer that had released it
+        holds both copies from here on."""
+        return self._restore_row_major(keep=True)
 
     def forward(self, x: Tensor, residual: Optional[Tensor] = None, norm=None,
                 swiglu_up: Optional[Tensor] = None) -> Tensor:
@@ -114,7 +210,7 @@ class TernaryLinearInference(nn.Module):
                                                        self.out_features, residual, norm, swiglu_up)
         if x.is_cuda and (norm is not None or swiglu_up is not None):
             from .. import _C
-            return _C.ternary_linear_packed_forward_fused(x, self.weight_packed, self.scale, self.bias,
+            return _C.ternary_linear_packed_forward_fused(x, self._row_major_for_call(), self.scale, self.bias,
                                                           self.in_features, residual, norm, swiglu_up)
         if norm is not None:
             x = F.rms_norm(x, (x.shape[-1],), norm[0], norm[1])
@@ -122,10 +218,10 @@ class TernaryLinearInference(nn.Module):
             x = F.silu(x) * swiglu_up
         if x.is_cuda:
             from ..ops.ternary_linear_packed import ternary_linear_packed_forward
-            return ternary_linear_packed_forward(x, self.weight_packed, self.scale,
+            return ternary_linear_packed_forward(x, self._row_major_for_call(), self.scale,
                                                  self.in_features, self.bias, residual)
         # CPU (reference :98-104): unpack, fold the scale in, dense product
-        w = unpack_ternary_transposed(self.weight_packed, self.in_features).to(x.dtype)
+        w = unpack_ternary_transposed(self.packed_weights(), self.in_features).to(x.dtype)
         w = w * self.scale.unsqueeze(1).to(x.dtype)
         y = F.linear(x, w, self.bias)
         return y if residual is None else y + residual
@@ -162,15 +258,15 @@ class TernaryLinearInference(nn.Module):
                                            q_operand_order)
             return y.reshape(*lead, self.out_features)
         from ..ops.fused import ternary_linear_int8
-        return ternary_linear_int8(q, s_x, self.weight_packed, self.scale, self.in_features, self.bias,
+        return ternary_linear_int8(q, s_x, self._row_major_for_call(), self.scale, self.in_features, self.bias,
                                    out_dtype, residual, q_operand_order)
 
     def extra_repr(self) -> str:
         dense = 4 * self.out_features * self.in_features
-        ratio = dense / (self.weight_packed.numel() + 2 * self.scale.numel())
+        ratio = dense / (self.packed_size_bytes + 2 * self.scale.numel())
         return (f"in_features={self.in_features}, out_features={self.out_features}, "
-                f"bias={self.bias is not None}, packed_bytes={self.weight_packed.numel()}, "
-                f"reduction={ratio:.1f}x")
+                f"bias={self.bias is not None}, packed_bytes={self.packed_size_bytes}, "
+                f"resident_weight_bytes={self.resident_weight_bytes()}, reduction={ratio:.1f}x")
 
     @classmethod
     def from_unpacked(cls, w_tern: Tensor, scale: Tensor,
@@ -181,11 +277,12 @@ class TernaryLinearInference(nn.Module):
 
     @property
     def packed_size_bytes(self) -> int:
-        return self.weight_packed.numel()
+        """Bytes of ``weight_packed`` (``ceil(K/4) * N``), whichever copy the layer holds."""
+        return ((self.in_features + 3) // 4) * self.out_features
 
     @property
     def effective_bits_per_weight(self) -> float:
-        bits = 8 * self.weight_packed.numel() + 16 * self.scale.numel()
+        bits = 8 * self.packed_size_bytes + 16 * self.scale.numel()
         return bits / (self.out_features * self.in_features)
 
 

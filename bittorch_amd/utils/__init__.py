@@ -3,9 +3,11 @@
 from .convert import (
     convert_linear_layers,
     count_ternary_params,
+    export_js_safetensors,
     fp_linear_to_ternary_infer,
     fuse_ternary_linear_inference,
     get_model_memory_bytes,
+    load_js_safetensors,
     load_ternary_checkpoint,
     load_ternary_safetensors,
     prepare_decode,
@@ -26,4 +28,6 @@ __all__ = [
     "load_ternary_checkpoint",
     "save_ternary_safetensors",
     "load_ternary_safetensors",
+    "export_js_safetensors",
+    "load_js_safetensors",
 ]

@@ -91,7 +91,7 @@ def fuse_ternary_linear_inference(*layers: TernaryLinearInference) -> TernaryLin
         raise ValueError("layers must share in_features")
     if any((l.bias is None) != (layers[0].bias is None) for l in layers):
         raise ValueError("either all layers have a bias or none")
-    packed = torch.cat([l.weight_packed for l in layers], dim=1).contiguous()
+    packed = torch.cat([l.packed_weights() for l in layers], dim=1).contiguous()
     scale = torch.cat([l.scale.reshape(-1).expand(l.out_features) if l.scale.numel() == 1 else l.scale
                        for l in layers]).contiguous()
     bias = None if layers[0].bias is None else torch.cat([l.bias for l in layers]).contiguous()
@@ -101,7 +101,7 @@ def fuse_ternary_linear_inference(*layers: TernaryLinearInference) -> TernaryLin
 def prepare_decode(module: nn.Module) -> nn.Module:
     """Build the decode-tiled weight copy of every ``TernaryLinearInference`` inside ``module`` now
     (they are otherwise built on each layer's first decode-shape call, and never during a HIP graph
-    capture, which falls back to ``weight_packed``).  Doubles the packed-weight memory of those layers."""
+    capture, which falls back to ``weight_packed``); the row-major buffer of a layer is released as its copy is built."""
     for m in module.modules():
         if isinstance(m, TernaryLinearInference):
             m.prepare_decode()
@@ -131,7 +131,7 @@ def get_model_memory_bytes(module: nn.Module) -> Dict[str, int]:
     out = {"fp32": 0, "fp16": 0, "packed_ternary": 0, "scales": 0, "total": 0}
     for child in module.modules():
         if isinstance(child, TernaryLinearInference):
-            packed = child.weight_packed.numel()
+            packed = child.resident_weight_bytes()  # what the layer holds: one copy unless it keeps the row-major buffer too
             scales = child.scale.numel() * child.scale.element_size()
             out["packed_ternary"] += packed
             out["scales"] += scales
@@ -191,3 +191,103 @@ def load_ternary_safetensors(path: str, module: nn.Module) -> Dict[str, str]:
             state[k] = v.to(own[k].dtype)
     module.load_state_dict(state)
     return dict(meta)
+
+
+# ---- interchange with the reference's browser runtime ----------------------------------------
+# Tensor names and shapes of js/src/models/TernaryTransformer.ts:141-188: per block i
+#   blocks.{i}.norm1.weight, blocks.{i}.norm2.weight                        F32 [dim]
+#   blocks.{i}.attn.{q_proj, kv_proj, proj}.{weight_packed, scale}          U8 [inBytes, outFeatures], F32 [outFeatures]
+#   blocks.{i}.mlp.{w_gate, w_up, w_down}.{weight_packed, scale}
+# with k and v fused along the output columns as kv_proj (its output is [k | v], :575-590), no biases, and
+# tok.weight / head.weight / norm.weight for the embedding, the output head and the final norm (:124-135).
+# The packed bytes are this library's ``weight_packed`` as they are (same codes, same [ceil(K/4), N] layout,
+# js/src/loaders/SafeTensorsLoader.ts:223-234).
+_JS_LAYERS = ("attn.q_proj", "attn.kv_proj", "attn.proj", "mlp.w_gate", "mlp.w_up", "mlp.w_down")
+_JS_DEFAULT_NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "gate": "gate", "up": "up", "down": "down",
+                     "norm1": "n1", "norm2": "n2"}
+
+
+def _as_infer(layer: nn.Module) -> TernaryLinearInference:
+    if isinstance(layer, TernaryLinearInference):
+        return layer
+    if isinstance(layer, TernaryLinear):
+        return ternary_linear_to_infer(layer)
+    if isinstance(layer, nn.Linear):
+        return fp_linear_to_ternary_infer(layer)
+    raise TypeError(f"cannot export a {type(layer).__name__} as a ternary layer")
+
+
+def export_js_safetensors(blocks, path: str, tok_embedding: Optional[torch.Tensor] = None,
+                          head: Optional[torch.Tensor] = None, final_norm: Optional[torch.Tensor] = None,
+                          metadata: Optional[Dict[str, str]] = None, names: Optional[Dict[str, str]] = None) -> None:
+    """Write a stack of transformer blocks as the ``model.safetensors`` the reference's browser runtime loads.
+
+    ``blocks``: a sequence of modules whose attributes ``names[...]`` (default ``q k v o gate up down n1 n2``) are
+    the block's seven ternary layers (``TernaryLinearInference``, or ``TernaryLinear`` / ``nn.Linear``, which are
+    quantized and packed on the way) and its two RMSNorm modules (or weight tensors).  A block that already holds
+    ``qkv`` fused keeps its ``q``, ``k``, ``v`` attributes, which are what is read.  Layers must have no bias and an
+    input width that is a multiple of 4 (the runtime derives it from the packed rows)."""
+    from safetensors.torch import save_file
+
+    names = {**_JS_DEFAULT_NAMES, **(names or {})}
+    tensors: Dict[str, torch.Tensor] = {}
+
+    def put_layer(key: str, layer: TernaryLinearInference) -> None:
+        if layer.bias is not None:
+            raise ValueError(f"{key}: the browser runtime's ternary layers have no bias")
+        if layer.in_features % 4 != 0:
+            raise ValueError(f"{key}: in_features must be a multiple of 4 (got {layer.in_features})")
+        tensors[key + ".weight_packed"] = layer.packed_weights().detach().cpu().contiguous()
+        scale = layer.scale.detach().reshape(-1)
+        if scale.numel() == 1:
+            scale = scale.expand(layer.out_features)
+        tensors[key + ".scale"] = scale.float().cpu().contiguous()
+
+    def norm_weight(obj) -> torch.Tensor:
+        w = obj.weight if isinstance(obj, nn.Module) else obj
+        return w.detach().float().cpu().contiguous()
+
+    for i, blk in enumerate(blocks):
+        get = (lambda n: blk[names[n]]) if isinstance(blk, dict) else (lambda n: getattr(blk, names[n]))
+        prefix = f"blocks.{i}"
+        tensors[f"{prefix}.norm1.weight"] = norm_weight(get("norm1"))
+        tensors[f"{prefix}.norm2.weight"] = norm_weight(get("norm2"))
+        q, k, v, o = (_as_infer(get(n)) for n in ("q", "k", "v", "o"))
+        put_layer(f"{prefix}.attn.q_proj", q)
+        put_layer(f"{prefix}.attn.kv_proj", fuse_ternary_linear_inference(k, v))
+        put_layer(f"{prefix}.attn.proj", o)
+        for js, own in (("w_gate", "gate"), ("w_up", "up"), ("w_down", "down")):
+            put_layer(f"{prefix}.mlp.{js}", _as_infer(get(own)))
+    for key, t in (("tok.weight", tok_embedding), ("head.weight", head), ("norm.weight", final_norm)):
+        if t is not None:
+            tensors[key] = norm_weight(t)
+    save_file(tensors, path, metadata=metadata or {})
+
+
+def load_js_safetensors(path: str, device=None):
+    """Read such a file back: ``(blocks, extras, metadata)`` with ``blocks[i]`` a dict of the six
+    ``TernaryLinearInference`` layers under the runtime's names (``attn.q_proj``, ``attn.kv_proj``, ``attn.proj``,
+    ``mlp.w_gate``, ``mlp.w_up``, ``mlp.w_down``) plus ``norm1`` / ``norm2`` weight tensors, and ``extras`` the
+    ``tok.weight`` / ``head.weight`` / ``norm.weight`` tensors that are present."""
+    from safetensors import safe_open
+
+    raw: Dict[str, torch.Tensor] = {}
+    with safe_open(path, framework="pt", device="cpu") as fh:
+        meta = dict(fh.metadata() or {})
+        for key in fh.keys():
+            raw[key] = fh.get_tensor(key)
+    n_blocks = 1 + max((int(k.split(".")[1]) for k in raw if k.startswith("blocks.")), default=-1)
+    blocks = []
+    for i in range(n_blocks):
+        prefix = f"blocks.{i}"
+        blk = {"norm1": raw[f"{prefix}.norm1.weight"], "norm2": raw[f"{prefix}.norm2.weight"]}
+        for name in _JS_LAYERS:
+            packed, scale = raw[f"{prefix}.{name}.weight_packed"], raw[f"{prefix}.{name}.scale"]
+            if packed.dtype != torch.uint8 or packed.dim() != 2 or scale.dim() != 1 or packed.shape[1] != scale.shape[0]:
+                raise ValueError(f"{prefix}.{name}: expected U8 [inBytes, outFeatures] and F32 [outFeatures]")
+            blk[name] = TernaryLinearInference(packed.shape[0] * 4, packed.shape[1], packed, scale.float())
+        if device is not None:
+            blk = {k: v.to(device) for k, v in blk.items()}
+        blocks.append(blk)
+    extras = {k: (v if device is None else v.to(device)) for k, v in raw.items() if not k.startswith("blocks.")}
+    return blocks, extras, meta

@@ -170,3 +170,90 @@ def test_ternary_swiglu_cpu_path_and_argument_checks():
         bt.nn.TernarySwiGLU(gate, up, down, compute="fp8")
     with pytest.raises(ValueError, match="do not form an MLP"):
         bt.nn.TernarySwiGLU(gate, up, mk(64, 32))
+
+
+class _Blk(nn.Module):
+    """A block in the shape the exporter reads: seven ternary layers and two RMSNorms."""
+    def __init__(self, d=64, kv=32, ffn=96, layer=None):
+        super().__init__()
+        mk = layer or (lambda i, o: TernaryLinear(i, o, bias=False))
+        self.q, self.k, self.v, self.o = mk(d, d), mk(d, kv), mk(d, kv), mk(d, d)
+        self.gate, self.up, self.down = mk(d, ffn), mk(d, ffn), mk(ffn, d)
+        self.n1, self.n2 = nn.RMSNorm(d), nn.RMSNorm(d)
+
+
+def test_js_runtime_export_names_shapes_and_round_trip(tmp_path):
+    """The file the reference's browser runtime loads (js/src/models/TernaryTransformer.ts:124-188): names, dtypes,
+    [inBytes, outFeatures] shapes, k|v fused as kv_proj, bytes equal to the layers' own packing."""
+    import bittorch_amd as bt
+    from safetensors import safe_open
+    torch.manual_seed(0)
+    blocks = nn.ModuleList([_Blk(), _Blk()])
+    for b in blocks:
+        nn.init.normal_(b.n1.weight)
+    emb, head, norm = torch.randn(50, 64), torch.randn(50, 64), torch.rand(64)
+    path = str(tmp_path / "model.safetensors")
+    bt.utils.export_js_safetensors(blocks, path, emb, head, norm, metadata={"format": "pt"})
+    with safe_open(path, framework="pt") as fh:
+        keys = set(fh.keys())
+        expect = {"tok.weight", "head.weight", "norm.weight"}
+        for i in range(2):
+            expect |= {f"blocks.{i}.norm1.weight", f"blocks.{i}.norm2.weight"}
+            for name in ("attn.q_proj", "attn.kv_proj", "attn.proj", "mlp.w_gate", "mlp.w_up", "mlp.w_down"):
+                expect |= {f"blocks.{i}.{name}.weight_packed", f"blocks.{i}.{name}.scale"}
+        assert keys == expect
+        assert fh.get_tensor("blocks.0.attn.kv_proj.weight_packed").shape == (16, 64)     # [64 / 4, 32 + 32]
+        assert fh.get_tensor("blocks.1.mlp.w_down.weight_packed").shape == (24, 64)
+        assert fh.get_tensor("blocks.0.mlp.w_gate.weight_packed").dtype == torch.uint8
+        assert fh.get_tensor("blocks.0.mlp.w_gate.scale").dtype == torch.float32
+        assert fh.get_tensor("blocks.0.mlp.w_gate.scale").shape == (96,)
+        assert torch.equal(fh.get_tensor("blocks.0.norm1.weight"), blocks[0].n1.weight.detach())
+        # the bytes are the layers' own packing (reference layout), k then v along the columns
+        k_inf, v_inf = bt.utils.ternary_linear_to_infer(blocks[0].k), bt.utils.ternary_linear_to_infer(blocks[0].v)
+        kv = fh.get_tensor("blocks.0.attn.kv_proj.weight_packed")
+        assert torch.equal(kv[:, :32], k_inf.weight_packed) and torch.equal(kv[:, 32:], v_inf.weight_packed)
+        assert torch.equal(fh.get_tensor("blocks.0.attn.kv_proj.scale"), torch.cat([k_inf.scale, v_inf.scale]))
+    loaded, extras, meta = bt.utils.load_js_safetensors(path)
+    assert meta == {"format": "pt"} and len(loaded) == 2 and torch.equal(extras["tok.weight"], emb)
+    x = torch.randn(3, 64)
+    blk = loaded[1]
+    ref = bt.utils.convert_linear_layers(blocks[1])
+    assert torch.equal(blk["attn.q_proj"](x), ref.q(x))
+    assert torch.equal(blk["attn.kv_proj"](x), torch.cat([ref.k(x), ref.v(x)], dim=-1))
+    h = torch.randn(3, 96)
+    assert torch.equal(blk["mlp.w_down"](h), ref.down(h))
+    with pytest.raises(ValueError, match="no bias"):
+        bt.utils.export_js_safetensors([_Blk(layer=lambda i, o: TernaryLinear(i, o, bias=True))], path)
+    with pytest.raises(ValueError, match="multiple of 4"):
+        bt.utils.export_js_safetensors([_Blk(d=66, layer=lambda i, o: TernaryLinear(i, o, bias=False))], path)
+
+
+@pytest.mark.gpu
+def test_gpu_converted_block_round_trips_through_the_js_file(tmp_path):
+    """GPU-converted block (fused quantize+pack kernel, decode-tiled resident weights) -> file -> reload on the GPU:
+    identical bytes, identical forward of every layer."""
+    import bittorch_amd as bt
+    from conftest import announce
+    announce("js export on gpu")
+    torch.manual_seed(1)
+    d, kv, ffn = 256, 128, 704
+    blocks = nn.ModuleList([_Blk(d, kv, ffn) for _ in range(2)]).cuda()
+    infer = bt.utils.convert_linear_layers(blocks)
+    x = torch.randn(5, d, device="cuda").half()
+    h = torch.randn(5, ffn, device="cuda").half()
+    before = [{n: getattr(b, n)(h if n == "down" else x) for n in ("q", "k", "v", "o", "gate", "up", "down")} for b in infer]
+    for b in infer:   # decode-shape calls have made the tiled copy the layers' only one
+        assert not b.q._has_row_major() and b.q.resident_weight_bytes() == b.q._tiled.numel()
+    path = str(tmp_path / "model.safetensors")
+    bt.utils.export_js_safetensors(infer, path)
+    cpu_path = str(tmp_path / "cpu.safetensors")
+    bt.utils.export_js_safetensors(bt.utils.convert_linear_layers(blocks.cpu()), cpu_path)
+    assert open(path, "rb").read() == open(cpu_path, "rb").read()        # byte-identical files
+    loaded, _, _ = bt.utils.load_js_safetensors(path, device="cuda")
+    for b, blk, ref in zip(infer, loaded, before):
+        assert torch.equal(blk["attn.q_proj"].packed_weights(), b.q.packed_weights())
+        assert torch.equal(blk["attn.q_proj"](x), ref["q"])
+        assert torch.equal(blk["attn.kv_proj"](x), torch.cat([ref["k"], ref["v"]], dim=-1))
+        assert torch.equal(blk["attn.proj"](x), ref["o"])
+        assert torch.equal(blk["mlp.w_gate"](x), ref["gate"]) and torch.equal(blk["mlp.w_up"](x), ref["up"])
+        assert torch.equal(blk["mlp.w_down"](h), ref["down"])

@@ -187,8 +187,9 @@ def test_xor_training_on_gpu():
 
 
 def test_packed_weight_cache_follows_the_weights(monkeypatch):
-    """The packed weights are re-made exactly when the master weights change (in-place update,
-    load_state_dict, move to another dtype) and never otherwise; outputs equal an uncached run."""
+    """A training forward quantizes every time (as the reference does, bittorch/nn/ternary_linear.py:196-200), so
+    writes through `.data` cannot go stale there; forwards without gradients keep the packed weights until a tracked
+    change (in-place update, optimizer step, load_state_dict, dtype move) or `invalidate_packed_cache()`."""
     from bittorch_amd import _C
     from bittorch_amd.nn import TernaryLinear, TernaryLinearCUDA
     announce("packed weight cache")
@@ -199,32 +200,57 @@ def test_packed_weight_cache_follows_the_weights(monkeypatch):
         calls["n"] += 1
         return real(*a, **k)
 
+    def fresh_output(layer, x):
+        packed, scale, _ = real(layer.weight.detach(), layer.threshold_factor, layer.per_channel)
+        return _C.ternary_linear_packed_forward(x, packed, scale.reshape(-1).to(x.dtype), layer.bias.detach().to(x.dtype), 64)
+
     monkeypatch.setattr(_C, "ternary_quantize_pack", counting)
     for cls in (TernaryLinear, TernaryLinearCUDA):
         torch.manual_seed(1)
         layer = cls(64, 32).cuda()
         x = torch.randn(8, 64, device="cuda")
         calls["n"] = 0
+        # gradient mode on, trainable weights: no caching, and a write through .data is seen at once
         y0 = layer(x)
         y1 = layer(x)
-        with torch.no_grad():
-            y2 = layer(x)
-        assert calls["n"] == 1 and torch.equal(y0, y1) and torch.equal(y0, y2)
-        # training step: backward works through the cached forward, the update invalidates it
+        assert calls["n"] == 2 and torch.equal(y0, y1)
+        layer.weight.data.mul_(-1.0)
+        y2 = layer(x)
+        assert calls["n"] == 3 and torch.equal(y2, fresh_output(layer, x)) and not torch.equal(y2, y0)
+        layer.weight.data.normal_(std=0.02)
         opt = torch.optim.SGD(layer.parameters(), lr=0.5)
         layer(x).pow(2).sum().backward()
         assert layer.weight.grad is not None and layer.weight.grad.abs().sum() > 0
         opt.step()
-        y3 = layer(x)
-        assert calls["n"] == 2
-        packed, scale, _ = real(layer.weight.detach(), layer.threshold_factor, layer.per_channel)
-        ref = _C.ternary_linear_packed_forward(x, packed, scale.reshape(-1), layer.bias.detach(), 64)
-        assert torch.equal(y3, ref)
+        assert torch.equal(layer(x), fresh_output(layer, x))
+        # no gradients: quantized once, reused
+        calls["n"] = 0
+        with torch.no_grad():
+            e0 = layer(x)
+            e1 = layer(x)
+            assert calls["n"] == 1 and torch.equal(e0, e1) and torch.equal(e0, fresh_output(layer, x))
+            # tracked in-place writes are followed
+            layer.weight.mul_(0.5)
+            layer.weight[0, :8] = 1.0
+            assert torch.equal(layer(x), fresh_output(layer, x)) and calls["n"] == 2
+            # a write through .data is the one thing the version counter does not see: invalidate by hand
+            layer.weight.data.mul_(-1.0)
+            layer.invalidate_packed_cache()
+            assert torch.equal(layer(x), fresh_output(layer, x)) and calls["n"] == 3
+        # frozen weights cache with gradient mode on as well (inputs may still need gradients)
+        layer.requires_grad_(False)
+        xg = x.clone().requires_grad_(True)
+        calls["n"] = 0
+        layer(xg).sum().backward()
+        layer(xg)
+        assert calls["n"] == 0 and xg.grad is not None
         # load_state_dict copies in place
         other = cls(64, 32).cuda()
         layer.load_state_dict(other.state_dict())
-        assert torch.equal(layer(x), other(x)) and calls["n"] == 4
+        with torch.no_grad():
+            assert torch.equal(layer(x), other(x))
         # dtype change replaces the storage
         layer.half()
-        yh = layer(x.half())
-        assert yh.dtype == torch.float16 and calls["n"] == 5
+        with torch.no_grad():
+            yh = layer(x.half())
+            assert yh.dtype == torch.float16 and torch.equal(yh, fresh_output(layer, x.half()))

@@ -120,6 +120,40 @@ def test_packed_forward_tall_batch_matches_streaming_kernel(oracle):
         assert ((y_tiled.double() - y_stream.double()).abs().max() / denom) < 1e-2
 
 
+def test_packed_forward_any_number_of_rows(oracle, monkeypatch):
+    """fp32 activations with K % 64 != 0 (the reference's MNIST layer, 784 -> 256) run the shape-generic kernel,
+    which takes any batch: more rows than a grid dimension holds included.  The streaming kernel serves a call
+    beyond its 65535 row blocks in slices."""
+    from bittorch_amd import _C
+    from bittorch_amd.quant import pack_ternary_transposed
+    announce("packed_forward many rows")
+    n, k = 16, 784
+    w = random_ternary(n, k, seed=1)
+    packed = pack_ternary_transposed(w)[0]
+    scale = torch.rand(n) * 0.05 + 0.01
+    bias = torch.randn(n) * 0.01
+    for b in (3, 70000):
+        x = seeded_acts(b, k, seed=b)
+        y = _C.ternary_linear_packed_forward(x.cuda(), packed.cuda(), scale.cuda(), bias.cuda(), k)
+        ref = oracle.linear_packed(f32np(x), packed.numpy(), f32np(scale), k, f32np(bias))
+        np.testing.assert_array_equal(f32np(y), ref)
+    # dense int8 weights on the generic route, same batch
+    monkeypatch.setenv("BITTORCH_KERNEL", "generic")
+    x = seeded_acts(70000, k, seed=5)
+    y = _C.ternary_linear_forward(x.cuda(), w.cuda(), scale.cuda(), bias.cuda())
+    np.testing.assert_array_equal(f32np(y), oracle.linear_unpacked(f32np(x), w.numpy(), f32np(scale), f32np(bias)))
+    monkeypatch.delenv("BITTORCH_KERNEL")
+    # streaming kernel, 16 * 65535 + 40 rows
+    monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "2000000")
+    b, k2 = 16 * 65535 + 40, 64
+    packed2 = pack_ternary_transposed(random_ternary(n, k2, seed=2))[0].cuda()
+    xb = torch.randn(b, k2, device="cuda").bfloat16()
+    yb = _C.ternary_linear_packed_forward(xb, packed2, scale.cuda(), bias.cuda(), k2)
+    for r0 in (0, 16 * 65535 - 8, b - 24):
+        part = _C.ternary_linear_packed_forward(xb[r0:r0 + 24].contiguous(), packed2, scale.cuda(), bias.cuda(), k2)
+        assert torch.equal(yb[r0:r0 + 24], part)
+
+
 def test_packed_forward_fp32_generic_is_bit_exact(oracle, monkeypatch):
     """The generic kernel accumulates in the reference's k order: equal to the oracle bit for bit
     (shapes whose K is a multiple of 64 take the matrix-core route by default, so it is forced)."""

@@ -193,6 +193,60 @@ def test_module_uses_tiled_copy_for_decode_shapes(oracle, dtype):
     assert torch.equal(a.forward_int8(q, s, torch.bfloat16, None, True), b.forward_int8(q, s, torch.bfloat16, None, True))
 
 
+def test_module_holds_one_copy_of_its_weights(oracle):
+    """After its first GPU call the layer holds the decode-tiled copy only (2 bits per weight: the 16x of the
+    reference's tests/test_packed_ternary.py:131-141 holds on the device), while state_dict(), .cpu(), pickling and
+    load_state_dict still see `weight_packed` in the reference's layout, bit for bit."""
+    import copy
+    import pickle
+    announce("module single copy")
+    n, k = 4096, 4096
+    w = random_ternary(n, k, seed=5)
+    packed_t, _ = oracle.pack_ternary_transposed(w.numpy())
+    from bittorch_amd.nn import TernaryLinearInference
+    from bittorch_amd.utils import get_model_memory_bytes
+    a = TernaryLinearInference(k, n, torch.from_numpy(packed_t), torch.rand(n) + 0.5).cuda()
+    assert a._has_row_major() and a.resident_weight_bytes() == n * k // 4
+    x = seeded_acts(1, k, dtype=torch.float16).cuda()
+    torch.cuda.synchronize()
+    base = torch.cuda.memory_allocated()
+    y = a(x)
+    assert not a._has_row_major() and "weight_packed" not in dict(a.named_buffers())
+    assert a.resident_weight_bytes() == n * k // 4                       # 0.25 bytes per weight
+    assert get_model_memory_bytes(a)["packed_ternary"] == n * k // 4
+    assert 4 * n * k / a.resident_weight_bytes() == 16.0
+    del y
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() <= base + (1 << 20)              # the row-major buffer was released
+    sd = a.state_dict()
+    assert list(sd) == ["weight_packed", "scale"]
+    np.testing.assert_array_equal(sd["weight_packed"].cpu().numpy(), packed_t)
+    np.testing.assert_array_equal(a.packed_weights().cpu().numpy(), packed_t)
+    assert not a._has_row_major()                                         # neither call changed what the layer holds
+    for clone in (copy.deepcopy(a), pickle.loads(pickle.dumps(a))):
+        assert clone._tiled is None and torch.equal(clone.weight_packed, sd["weight_packed"])
+        assert torch.equal(clone(x), a(x))
+    c = copy.deepcopy(a).cpu()
+    np.testing.assert_array_equal(c.weight_packed.numpy(), packed_t)
+    assert rel_err(f32np(c(x.cpu().float())), f32np(a(x))) < 2e-3
+    # reading the attribute brings the buffer back for good: in-place edits keep their meaning
+    wp = a.weight_packed
+    assert a._has_row_major() and a.keep_row_major and a.resident_weight_bytes() == 2 * n * k // 4
+    np.testing.assert_array_equal(wp.cpu().numpy(), packed_t)
+    wp.zero_()
+    assert torch.equal(a(x).float(), torch.zeros(1, n, device="cuda"))
+    a.load_state_dict(sd)
+    assert torch.equal(a(x), c.cuda()(x))
+    a.drop_row_major()
+    assert not a._has_row_major() and a.resident_weight_bytes() == n * k // 4
+    # a call only the row-major kernels serve (fp32 activations with K % 64 != 0) keeps both from then on
+    b = _layer(oracle, 48, 100, seed=2)
+    b(seeded_acts(1, 100, dtype=torch.float16).cuda())
+    assert not b._has_row_major()
+    b(seeded_acts(2, 100, dtype=torch.float32).cuda())
+    assert b._has_row_major() and b.keep_row_major
+
+
 def test_module_rebuilds_tiled_copy_when_weights_change(oracle):
     a = _layer(oracle, 64, 64, seed=1)
     x = seeded_acts(1, 64, dtype=torch.float16).cuda()
