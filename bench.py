@@ -343,6 +343,10 @@ def main():
     torch.cuda.set_device(dev)
     torch.manual_seed(0)
 
+    if args.block_stack_only:
+        print(json.dumps({"block_stack": block_stack(torch, dev, layers=args.block_stack_only)}))
+        return
+
     # ---- config 2: decode GEMV units -------------------------------------------------------
     N = K = 4096
     weight_bytes = N * (K // 4)
@@ -395,11 +399,6 @@ def main():
     if args.pmc_pass:
         pmc_pass(torch, _C, dev, (step_single, step_row_major), step)
         return
-    if args.block_stack_only:
-        del packs
-        print(json.dumps({"block_stack": block_stack(torch, dev, layers=args.block_stack_only)}))
-        return
-
     wall_ms, ev_ms = graph_time(step, args.steps, args.warmup, torch)
     ms_per_step = wall_ms / args.steps
     kernel_us = ev_ms / args.steps * 1e3

@@ -303,14 +303,47 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
         for (int c = 0; c < 16; c++) mfma(a_hi[c >> 2], b_cur[c & 3], acc[4 + (c >> 2)][c & 3]);
         __builtin_amdgcn_sched_barrier(0);
     };
+    // The two waves that share a SIMD (the K halves of one column quarter) run the stage in different orders, so
+    // that one of them is inside a run of MFMAs while the other stages, loads and reads LDS: K half 1 reads all
+    // eight row blocks of stage s right behind the barrier that published them, does both MFMA halves in a row and
+    // arrives at the next barrier with stage s finished; K half 0 (above) has its second half beyond the barrier.
+    auto stage_y = [&](int s, uint4 (&a_reg)[2], uint32_t (&b_reg)[BR], const u32x4 (&b_cur)[4], u32x4 (&b_nxt)[4]) {
+        const int cur = s & 1;
+        read_a(cur, 0, a_lo);
+        read_a(cur, 4, a_hi);
+        store_a(cur ^ 1, a_reg);
+        load_stage(s + 3, 1, a_reg, b_reg);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < 16; c++) {
+            mfma(a_lo[c >> 2], b_cur[c & 3], acc[c >> 2][c & 3]);
+            if ((c & 3) == 1) decode_col(b_reg, c >> 2, b_nxt[c >> 2]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        load_stage(s + 3, 2, a_reg, b_reg);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < 16; c++) mfma(a_hi[c >> 2], b_cur[c & 3], acc[4 + (c >> 2)][c & 3]);
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+    };
     // (an odd last stage is peeled so that both paths into the loop header leave the same
     // loads outstanding)
     int s = 0;
-    for (; s + 1 < nstages; s += 2) {
-        stage(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
-        stage(s + 1, a_set[0], b_set[0], b_dec[1], b_dec[0]);
+    if (kgrp == 0) {  // wave-uniform
+        for (; s + 1 < nstages; s += 2) {
+            stage(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
+            stage(s + 1, a_set[0], b_set[0], b_dec[1], b_dec[0]);
+        }
+        if (s < nstages) stage(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
+    } else {
+        for (; s + 1 < nstages; s += 2) {
+            stage_y(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
+            stage_y(s + 1, a_set[0], b_set[0], b_dec[1], b_dec[0]);
+        }
+        if (s < nstages) stage_y(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
     }
-    if (s < nstages) stage(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
     __syncthreads();  // every wave is done with the stage buffers before they are reused
 
     // column scales and biases (raw bits) requested ahead of the exchange, which covers their latency

@@ -137,7 +137,9 @@ __device__ __forceinline__ void gemm_epilogue_dt(const GemmParams& p, const v4i 
 // the staging copies them to LDS untouched.
 // WT = true: W_T is the decode-tiled copy (W_LAYOUT_TILED): the four dwords a lane decodes per stage
 // (16 consecutive k of its four columns) are 16 contiguous bytes there, one load and no transpose.
-template <bool TAIL, bool QOO, bool WT = false>
+// ANTIPHASE = false (A/B runs, BITTORCH_GEMM_INPHASE=1, benchmarked variant only): both K halves run the stage in
+// the same order.
+template <bool TAIL, bool QOO, bool WT = false, bool ANTIPHASE = true>
 __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[65536];  // 2 A stages; reused for the K-half exchange
 
@@ -335,6 +337,18 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
             out[t][2] = (int)perm(0u, lutA_lo, d_H[t] & 0x03030303u);
         };
         auto partC = [&](int t) { out[t][3] = (int)perm(lutB_hi, lutB_lo, d_H[t] & 0x0C0C0C0Cu); };
+        if constexpr (WT) {
+            // tiled weights need no transpose: the nine operations of each column are cut into four slices of at
+            // most three, one behind every one of the 16 MFMAs, so that no MFMA has to wait for the wave's own VALU work
+            const int t = c >> 2;
+            switch (c & 3) {
+                case 0: d_G[t] = raw[t]; partA(t); break;
+                case 1: out[t][1] = (int)perm(lutB_hi, lutB_lo, d_G[t] & 0x0C0C0C0Cu); break;
+                case 2: out[t][2] = (int)perm(0u, lutA_lo, d_H[t] & 0x03030303u); break;
+                default: partC(t); break;
+            }
+            return;
+        }
         switch (c) {
             case 4:
                 if constexpr (!WT) {
@@ -396,15 +410,53 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
         mfma_half(4, a_hi, b_cur);
         __builtin_amdgcn_sched_barrier(0);
     };
+    // The two waves that share a SIMD (the K halves of one column quarter) run the stage in different orders, so
+    // that one of them is inside a run of MFMAs while the other stages, loads and reads LDS: K half 1 reads all
+    // eight row blocks of stage s right behind the barrier that published them, then does both MFMA halves in a
+    // row and arrives at the next barrier with stage s finished, while K half 0 (above) is half a stage behind it
+    // and has its second MFMA half on the far side of the barrier.  Same barriers, same buffers: stage s+1 goes to
+    // the buffer whose readers all finished before the last barrier.
+    auto stage_y = [&](int s, uint4 (&a_reg)[2], uint32_t (&b_reg)[4], const v4i (&b_cur)[4], v4i (&b_nxt)[4]) {
+        const int cur = s & 1;
+        read_a(cur, 0, a_lo);
+        read_a(cur, 4, a_hi);
+        store_a(cur ^ 1, a_reg);
+        load_stage(s + 3, 1, a_reg, b_reg);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < 16; c++) {
+            const int i = c >> 2, t = c & 3;
+            const v4i a = {(int)a_lo[i].x, (int)a_lo[i].y, (int)a_lo[i].z, (int)a_lo[i].w};
+            acc[i][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b_cur[t], acc[i][t], 0, 0, 0);
+            decode_slice(c, b_reg, b_nxt);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        load_stage(s + 3, 2, a_reg, b_reg);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_setprio(1);
+        mfma_half(4, a_hi, b_cur);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_setprio(0);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+    };
     // (an odd last stage is peeled: with a conditional second half inside the loop the two
     // paths to the loop header leave different loads outstanding, and the wait the compiler
     // puts at the top of the loop then drains the whole queue, freshly issued loads included)
     int s = 0;
-    for (; s + 1 < nstages; s += 2) {
-        stage(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
-        stage(s + 1, a_set[0], b_set[0], b_dec[1], b_dec[0]);
+    if (kgrp == 0 || !ANTIPHASE) {  // wave-uniform
+        for (; s + 1 < nstages; s += 2) {
+            stage(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
+            stage(s + 1, a_set[0], b_set[0], b_dec[1], b_dec[0]);
+        }
+        if (s < nstages) stage(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
+    } else {
+        for (; s + 1 < nstages; s += 2) {
+            stage_y(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
+            stage_y(s + 1, a_set[0], b_set[0], b_dec[1], b_dec[0]);
+        }
+        if (s < nstages) stage_y(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
     }
-    if (s < nstages) stage(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
     __syncthreads();  // every wave is done with the stage buffers before they are reused
 
     EpiOperands epi_ops;
@@ -477,7 +529,8 @@ int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_
     const bool qoo = q_layout == Q_OPERAND_ORDER;
     if (w_layout == W_LAYOUT_TILED) {
         if (K % G_BK == 0) {
-            if (qoo) hipLaunchKernelGGL((gemm_i8_kernel<false, true, true>), grid, block, 0, st, p);
+            if (qoo && getenv("BITTORCH_GEMM_INPHASE")) hipLaunchKernelGGL((gemm_i8_kernel<false, true, true, false>), grid, block, 0, st, p);
+            else if (qoo) hipLaunchKernelGGL((gemm_i8_kernel<false, true, true>), grid, block, 0, st, p);
             else hipLaunchKernelGGL((gemm_i8_kernel<false, false, true>), grid, block, 0, st, p);
         } else {
             if (qoo) hipLaunchKernelGGL((gemm_i8_kernel<true, true, true>), grid, block, 0, st, p);

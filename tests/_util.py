@@ -37,3 +37,15 @@ def rel_err(got, ref):
     got = np.asarray(got, dtype=np.float64)
     ref = np.asarray(ref, dtype=np.float64)
     return float(np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-30))
+
+
+# element-wise thresholds of the reference's own kernel tests (tests/test_packed_kernel.py:44-50: rtol = atol =
+# 1e-4 for fp32; :159-199: 1e-2 for fp16; bf16, which the reference does not take, is held to the fp16 figure)
+REF_ELEMENTWISE = {torch.float32: 1e-4, torch.float16: 1e-2, torch.bfloat16: 1e-2}
+
+
+def assert_close_like_reference(got, ref, dtype):
+    """Every output element within the reference tests' `allclose(rtol, atol)` of `ref`: unlike `rel_err`, which
+    is relative to the largest output, this also holds the small-magnitude outputs."""
+    thr = REF_ELEMENTWISE[dtype]
+    np.testing.assert_allclose(np.asarray(got, dtype=np.float64), np.asarray(ref, dtype=np.float64), rtol=thr, atol=thr)

@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from conftest import announce
-from _util import f32np, random_ternary, rel_err, seeded_acts, seeded_weights
+from _util import assert_close_like_reference, f32np, random_ternary, rel_err, seeded_acts, seeded_weights
 
 pytestmark = pytest.mark.gpu
 
@@ -39,6 +39,7 @@ def _case(oracle, b, n, k, dtype, bias=True, seed=0, scale_dtype=None, per_tenso
     # the oracle's own distance from the truth bounds what fp32 accumulation may cost
     assert rel_err(ref, truth) < 1e-5
     assert rel_err(got, truth) < TOL[dtype], (b, n, k, dtype)
+    assert_close_like_reference(got, truth, dtype)
     return got, ref.astype(np.float32)
 
 

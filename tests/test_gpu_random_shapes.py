@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from conftest import announce
-from _util import BT_DT, f32np, random_ternary, rel_err, seeded_acts, seeded_weights
+from _util import BT_DT, f32np, random_ternary, rel_err, seeded_acts, seeded_weights, assert_close_like_reference
 
 pytestmark = pytest.mark.gpu
 
@@ -41,6 +41,7 @@ def test_random_shape_sweep(oracle, b, n, k, dtype, seed):
     y = _C.ternary_linear_packed_forward(x.cuda(), packed, scale, bias.cuda(), k)
     truth = oracle.linear_packed(f32np(x), o_packed, o_scale, k, f32np(bias), f64=True)
     assert rel_err(f32np(y), truth) < (1e-3 if dtype == torch.float32 else 1e-2)
+    assert_close_like_reference(f32np(y), truth, dtype)
     res = seeded_acts(b, n, seed=seed + 3, dtype=dtype).cuda()
     assert torch.equal(_C.ternary_linear_packed_forward(x.cuda(), packed, scale, bias.cuda(), k, res), y + res)
 
@@ -71,5 +72,6 @@ def test_random_shape_sweep(oracle, b, n, k, dtype, seed):
     if dtype != torch.float32 or k % 64 == 0:
         yt_f = _C.ternary_linear_tiled_forward(x.cuda(), tiled, scale, bias.cuda(), k, n)
         assert rel_err(f32np(yt_f), truth) < (1e-3 if dtype == torch.float32 else 1e-2)
+        assert_close_like_reference(f32np(yt_f), truth, dtype)
         if dtype != torch.float32 and b <= 32:  # (beyond, the plans may split K over different numbers of waves)
             assert torch.equal(yt_f, y)
