@@ -31,18 +31,29 @@ class TernarySwiGLU(nn.Module):
                 and down.in_features == gate.out_features):
             raise ValueError("gate/up/down shapes do not form an MLP")
         self.ffn = gate.out_features
-        self.compute = compute
         self.down = down
         if fuse_gate_up:
             from ..utils.convert import fuse_ternary_linear_inference
             self.gate_up = fuse_ternary_linear_inference(gate, up)
             self.gate = self.up = None
-            if compute == "float" and self.ffn % 16 == 0:
-                # decode-shape calls: the SwiGLU product leaves the gate|up GEMV's own output stage
-                self.gate_up.tile_order = "gate_up_pairs"
         else:
             self.gate_up = None
             self.gate, self.up = gate, up
+        self.compute = compute
+
+    @property
+    def compute(self) -> str:
+        return self._compute
+
+    @compute.setter
+    def compute(self, mode: str) -> None:
+        if mode not in ("float", "int8"):
+            raise ValueError(f"compute must be 'float' or 'int8', got {mode!r}")
+        self._compute = mode
+        if self.gate_up is not None:
+            # float: decode-shape calls let the SwiGLU product leave the gate|up GEMV's own output stage, which wants
+            # the tiles of the two halves alternating; int8: the GEMMs read the copy in natural order
+            self.gate_up.tile_order = "gate_up_pairs" if (mode == "float" and self.ffn % 16 == 0) else "natural"
 
     def _gate_up(self, h: Tensor, norm=None):
         if self.gate_up is None:
