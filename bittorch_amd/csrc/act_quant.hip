@@ -181,39 +181,57 @@ int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q
 // bf16 (upper 16 bits) of what the terms before it leave (24 significand bits = 3 x 8).  Ternary
 // weights are exact in bf16, so the three products per weight are exact and the 16-bit matrix
 // cores accumulate them in fp32: fp32 inputs run on the bf16 kernels without losing a bit of
-// the activations.  X [B,K] fp32 -> P [B,3K] bf16 bits, row b = [hi(K) | mid(K) | lo(K)] / 2.
-__global__ __launch_bounds__(256) void split_f32_planes_kernel(const float* __restrict__ X, int64_t B, int64_t K,
+// the activations.  X [B,K] fp32 -> P [B,3*Kp] bf16 bits, row b = [hi(Kp) | mid(Kp) | lo(Kp)] / 2,
+// Kp = K rounded up to the kernels' 64-wide step, the padding zero (it meets padding codes or clamped
+// weight rows: 0 * w = 0 exactly).
+__device__ __forceinline__ void split3(float x, uint16_t& hi, uint16_t& mid, uint16_t& lo) {
+    const uint32_t u0 = __builtin_bit_cast(uint32_t, x) & 0xFFFF0000u;
+    const float r1 = x - __builtin_bit_cast(float, u0);
+    const uint32_t u1 = __builtin_bit_cast(uint32_t, r1) & 0xFFFF0000u;
+    const float r2 = r1 - __builtin_bit_cast(float, u1);
+    // stored halved (exact): the bf16 kernels decode the weights as +-2.0, and x * 2 would
+    // overflow for |x| above half the fp32 range
+    hi = (uint16_t)(__builtin_bit_cast(uint32_t, __builtin_bit_cast(float, u0) * 0.5f) >> 16);
+    mid = (uint16_t)(__builtin_bit_cast(uint32_t, __builtin_bit_cast(float, u1) * 0.5f) >> 16);
+    lo = (uint16_t)(__builtin_bit_cast(uint32_t, r2 * 0.5f) >> 16);
+}
+// VEC: K % 4 == 0 and X 16-byte aligned (one float4 per thread and trip); otherwise element by element
+template <bool VEC>
+__global__ __launch_bounds__(256) void split_f32_planes_kernel(const float* __restrict__ X, int64_t B, int64_t K, int64_t Kp,
                                                                uint16_t* __restrict__ P) {
-    const int64_t kq = K >> 2;  // float4 groups per row (K % 4 == 0)
+    const int64_t kq = Kp >> 2;  // groups of four per padded row
     const int64_t total = B * kq;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
         const int64_t b = i / kq, c = i - b * kq;
-        const float4 v = *(const float4*)(X + b * K + 4 * c);
-        const float x[4] = {v.x, v.y, v.z, v.w};
+        float x[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if constexpr (VEC) {
+            if (4 * c < K) {
+                const float4 v = *(const float4*)(X + b * K + 4 * c);
+                x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (4 * c + e < K) x[e] = X[b * K + 4 * c + e];
+        }
         uint16_t hi[4], mid[4], lo[4];
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const uint32_t u0 = __builtin_bit_cast(uint32_t, x[e]) & 0xFFFF0000u;
-            const float r1 = x[e] - __builtin_bit_cast(float, u0);
-            const uint32_t u1 = __builtin_bit_cast(uint32_t, r1) & 0xFFFF0000u;
-            const float r2 = r1 - __builtin_bit_cast(float, u1);
-            // stored halved (exact): the bf16 kernels decode the weights as +-2.0, and x * 2 would
-            // overflow for |x| above half the fp32 range
-            hi[e] = (uint16_t)(__builtin_bit_cast(uint32_t, __builtin_bit_cast(float, u0) * 0.5f) >> 16);
-            mid[e] = (uint16_t)(__builtin_bit_cast(uint32_t, __builtin_bit_cast(float, u1) * 0.5f) >> 16);
-            lo[e] = (uint16_t)(__builtin_bit_cast(uint32_t, r2 * 0.5f) >> 16);
-        }
-        uint16_t* row = P + b * 3 * K + 4 * c;
+        for (int e = 0; e < 4; e++) split3(x[e], hi[e], mid[e], lo[e]);
+        uint16_t* row = P + b * 3 * Kp + 4 * c;
         *(uint2*)(row) = make_uint2((uint32_t)hi[0] | ((uint32_t)hi[1] << 16), (uint32_t)hi[2] | ((uint32_t)hi[3] << 16));
-        *(uint2*)(row + K) = make_uint2((uint32_t)mid[0] | ((uint32_t)mid[1] << 16), (uint32_t)mid[2] | ((uint32_t)mid[3] << 16));
-        *(uint2*)(row + 2 * K) = make_uint2((uint32_t)lo[0] | ((uint32_t)lo[1] << 16), (uint32_t)lo[2] | ((uint32_t)lo[3] << 16));
+        *(uint2*)(row + Kp) = make_uint2((uint32_t)mid[0] | ((uint32_t)mid[1] << 16), (uint32_t)mid[2] | ((uint32_t)mid[3] << 16));
+        *(uint2*)(row + 2 * Kp) = make_uint2((uint32_t)lo[0] | ((uint32_t)lo[1] << 16), (uint32_t)lo[2] | ((uint32_t)lo[3] << 16));
     }
 }
 
-int launch_split_f32_planes(const void* X, int64_t B, int64_t K, void* P, hipStream_t st) {
-    const int64_t total = B * (K >> 2);
+// Kp: plane length, a multiple of 64 and >= K; P is 8-byte aligned
+int launch_split_f32_planes(const void* X, int64_t B, int64_t K, int64_t Kp, void* P, hipStream_t st) {
+    const int64_t total = B * (Kp >> 2);
     const unsigned blocks = (unsigned)std::min<int64_t>(std::max<int64_t>(ceil_div(total, 256), 1), 8192);
-    hipLaunchKernelGGL(split_f32_planes_kernel, dim3(blocks), dim3(256), 0, st, (const float*)X, B, K, (uint16_t*)P);
+    if (K % 4 == 0 && ((uintptr_t)X) % 16 == 0)
+        hipLaunchKernelGGL(split_f32_planes_kernel<true>, dim3(blocks), dim3(256), 0, st, (const float*)X, B, K, Kp, (uint16_t*)P);
+    else
+        hipLaunchKernelGGL(split_f32_planes_kernel<false>, dim3(blocks), dim3(256), 0, st, (const float*)X, B, K, Kp, (uint16_t*)P);
     return check_launch("bt_ternary_linear_packed_forward(split)");
 }
 

@@ -41,7 +41,7 @@ bool stream_prologue_fusable(int mode, int64_t B, int64_t N, int64_t K, const vo
                              int epi_op);
 int launch_retile(const uint8_t* W_T, int64_t N, int64_t K, int pairs, void* T, bool inverse, uint8_t* W_out,
                   hipStream_t st);
-int launch_split_f32_planes(const void* X, int64_t B, int64_t K, void* P, hipStream_t st);
+int launch_split_f32_planes(const void* X, int64_t B, int64_t K, int64_t Kp, void* P, hipStream_t st);
 int launch_packed_generic(const void* X, int x_dtype, const uint8_t* W_T, const Epilogue& epi, void* Y,
                           int64_t B, int64_t N, int64_t K, hipStream_t st);
 int launch_unpacked(const void* X, int x_dtype, const int8_t* W, const Epilogue& epi, void* Y, int64_t B,
@@ -175,17 +175,18 @@ static bool packed_uses_stream(int x_dtype, const void* W_T, const void* Y, int6
     return x_dtype != BT_F32 && stream_supported(N, K, W_T) && fast_path_ok(Y, N, K);
 }
 
-// fp32 activations run on the bf16 matrix-core kernels as three exact bf16 planes (hi, mid, lo)
-// when K is a multiple of the kernels' 64-wide step; the planes live in the workspace.
-static size_t f32_planes_bytes(int64_t B, int64_t K) { return align256((size_t)B * 3 * K * 2); }
-static bool packed_uses_f32_planes(const void* X, const void* W_T, const void* Y, int64_t N, int64_t K) {
+// fp32 activations run on the bf16 matrix-core kernels as three exact bf16 planes (hi, mid, lo), each
+// zero-padded to the kernels' 64-wide step; the planes live in the workspace.
+static int64_t plane_len(int64_t K) { return ceil_div(K, 64) * 64; }
+static size_t f32_planes_bytes(int64_t B, int64_t K) { return align256((size_t)B * 3 * plane_len(K) * 2); }
+static bool packed_uses_f32_planes(const void* W_T, const void* Y, int64_t N, int64_t K) {
     if (generic_forced()) return false;
-    return K % 64 == 0 && ((uintptr_t)X) % 16 == 0 && stream_supported(N, 3 * K, W_T) && fast_path_ok(Y, N, 3 * K);
+    return stream_supported(N, 3 * plane_len(K), W_T) && fast_path_ok(Y, N, 3 * plane_len(K));
 }
 
 extern "C" size_t bt_packed_forward_workspace_bytes(int64_t B, int64_t N, int64_t K, int x_dtype) {
     if (B <= 0 || N <= 0 || K <= 0) return 0;
-    if (x_dtype == BT_F32) return (K % 64 == 0) ? f32_planes_bytes(B, K) : 0;
+    if (x_dtype == BT_F32) return f32_planes_bytes(B, K);
     return stream_workspace_bytes(x_dtype == BT_F16 ? MODE_F16 : MODE_BF16, B, N, ceil_div(K, 4));
 }
 
@@ -232,15 +233,15 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
             return launch_stream(mode, X, 2, nullptr, W_T, W_LAYOUT_TILED, epi, Y, x_dtype, nullptr, B, N, K, 1,
                                  Q_ROW_MAJOR, 0, nullptr, 0.0f, epi_op, st);
         }
-        if (K % 64 != 0 || ((uintptr_t)X) % 16 != 0 || !workspace || workspace_bytes < f32_planes_bytes(B, K) ||
-            ((uintptr_t)workspace) % 256 != 0) {
-            set_error("%s: fp32 activations on tiled weights need K %% 64 == 0, X 16-byte aligned and a workspace of "
-                      "%zu bytes (256-byte aligned)", who, f32_planes_bytes(B, K));
+        if (!workspace || workspace_bytes < f32_planes_bytes(B, K) || ((uintptr_t)workspace) % 256 != 0) {
+            set_error("%s: fp32 activations on tiled weights need a workspace of %zu bytes (256-byte aligned)", who,
+                      f32_planes_bytes(B, K));
             return BT_ERR_INVALID;
         }
-        rc = launch_split_f32_planes(X, B, K, workspace, st);
+        const int64_t Kp = plane_len(K);
+        rc = launch_split_f32_planes(X, B, K, Kp, workspace, st);
         if (rc) return rc;
-        if (!prefers_stream(B, N, 3 * K, false) && epi_op == 0 && gemm_f16_supported_tiled(N, 3 * K, workspace, Y))
+        if (!prefers_stream(B, N, 3 * Kp, false) && epi_op == 0 && gemm_f16_supported_tiled(N, 3 * Kp, workspace, Y))
             return launch_gemm_f16(MODE_BF16, workspace, W_T, W_LAYOUT_TILED, epi, Y, BT_F32, B, N, K, 3, st);
         return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, W_LAYOUT_TILED, epi, Y, BT_F32, nullptr, B, N, K, 3,
                              Q_ROW_MAJOR, 0, nullptr, 0.0f, epi_op, st);
@@ -254,12 +255,13 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
             return launch_gemm_f16(mode, X, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, x_dtype, B, N, K, 1, st);
         return launch_stream(mode, X, 2, nullptr, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, x_dtype, nullptr, B, N, K, 1, Q_ROW_MAJOR, 0, nullptr, 0.0f, 0, st);
     }
-    if (x_dtype == BT_F32 && packed_uses_f32_planes(X, W_T, Y, N, K) && workspace &&
+    if (x_dtype == BT_F32 && packed_uses_f32_planes(W_T, Y, N, K) && workspace &&
         workspace_bytes >= f32_planes_bytes(B, K) && ((uintptr_t)workspace) % 256 == 0) {
         // (without a workspace the call still succeeds, on the generic kernel)
-        rc = launch_split_f32_planes(X, B, K, workspace, st);
+        const int64_t Kp = plane_len(K);
+        rc = launch_split_f32_planes(X, B, K, Kp, workspace, st);
         if (rc) return rc;
-        if (!prefers_stream(B, N, 3 * K, false) && gemm_f16_supported(N, 3 * K, workspace, W_T, Y))
+        if (!prefers_stream(B, N, 3 * Kp, false) && gemm_f16_supported(N, 3 * Kp, workspace, W_T, Y))
             return launch_gemm_f16(MODE_BF16, workspace, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, BT_F32, B, N, K, 3, st);
         return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, BT_F32, nullptr, B, N, K, 3, Q_ROW_MAJOR, 0, nullptr, 0.0f, 0, st);
     }

@@ -174,6 +174,14 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
             if constexpr (WT) {
                 const uint4 v = *(const uint4*)(b_base + (size_t)ws * 256 + b_off);
                 b_reg[0] = v.x; b_reg[1] = v.y; b_reg[2] = v.z; b_reg[BR - 1] = v.w;
+            } else if constexpr (TAIL) {
+                // zero-padded activation planes with K % 64 != 0: the last weight stage of a plane runs past W_T
+#pragma unroll
+                for (int r = 0; r < 2; r++) {
+                    int64_t kb = (int64_t)ws * (F_BK / 4) + 8 * kgrp + 2 * g + r;
+                    kb = kb < p.Kb ? kb : p.Kb - 1;
+                    b_reg[r] = *(const uint32_t*)(b_base + kb * N + (col_ok ? ncol : 0));
+                }
             } else {
                 const uint8_t* bb = b_base + (int64_t)ws * (F_BK / 4) * N;
                 b_reg[0] = *(const uint32_t*)(bb + b_off);
@@ -403,13 +411,14 @@ bool gemm_f16_supported(int64_t N, int64_t K, const void* X, const void* W_T, co
            ((uintptr_t)Y) % 16 == 0 && (F_BM + 1) * K * 2 < (1ll << 32) && ceil_div(K, 4) * N < (1ll << 32);
 }
 
-// planes = 1: X is [M, K].  planes = 3 (K % 64 == 0): X is [M, 3K], three planes of K values per
-// row whose products with the same weights are summed (fp32 activations split into three bf16 terms).
+// planes = 1: X is [M, K].  planes = 3: X is [M, 3*Kp], Kp = K rounded up to 64, three zero-padded planes of K
+// values per row whose products with the same weights are summed (fp32 activations split into three bf16 terms).
+// With K % 64 != 0 the last weight stage of every plane runs past W_T's rows: the TAIL instantiation clamps them.
 int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, int w_layout, const Epilogue& epi, void* Y, int y_dtype,
                     int64_t M, int64_t N, int64_t K, int planes, hipStream_t st) {
     GemmFParams p;
     p.X = (const uint16_t*)X; p.W_T = W_T; p.Y = Y; p.epi = epi;
-    p.M = M; p.N = N; p.K = K * planes; p.Kb = ceil_div(K, 4);
+    p.M = M; p.N = N; p.K = (planes == 3) ? 3 * ceil_div(K, F_BK) * F_BK : K; p.Kb = ceil_div(K, 4);
     p.wstages = (int)ceil_div(K, F_BK);
     p.prehalved = planes == 3;
     p.y_dtype = y_dtype;
@@ -418,7 +427,7 @@ int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, int w_layout, c
     const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
     p.per_xcd = (int)ceil_div(total, 8);
     const dim3 grid((unsigned)(p.per_xcd * 8)), block(512);
-    const bool tail = p.K % F_BK != 0;
+    const bool tail = K % F_BK != 0;
     p.tiles16 = (int)ceil_div(N, 16);
     if (w_layout == W_LAYOUT_TILED) {
         if (mode == MODE_F16) {

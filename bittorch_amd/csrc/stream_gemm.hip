@@ -780,9 +780,10 @@ static int launch_stream_mode(StreamParams p, const StreamPlan& pl, hipStream_t 
 }
 
 // One launch for the whole call: grid.y walks its blocks of 16 activation rows.
-// planes = 1: X is [B, K].  planes = 3 (K % 64 == 0): X is [B, 3K], three planes of K values per
-// row whose products with the same weights are summed (fp32 activations split into three bf16
-// terms); the kernel walks 3K values of k and wraps its weight row index every K.
+// planes = 1: X is [B, K].  planes = 3: X is [B, 3*Kp], Kp = K rounded up to 64, three zero-padded planes
+// of K values per row whose products with the same weights are summed (fp32 activations split into three
+// bf16 terms); the kernel walks 3*Kp values of k and wraps its weight step index every Kp (weight rows past
+// the matrix are clamped or zero padding, and meet zero activations).
 // w_layout: W_LAYOUT_ROW_MAJOR (the reference's W_T [Kb, N]) or W_LAYOUT_TILED (retile_kernel's copy)
 // q_layout: MODE_I8 only (Q_OPERAND_ORDER needs K % 16 == 0 and 16-byte aligned rows)
 // pro_op / pro_b / pro_eps: activation prologue (PRO_*), only where stream_prologue_fusable() said yes
@@ -791,7 +792,7 @@ int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, co
                   const Epilogue& epi, void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N,
                   int64_t K, int planes, int q_layout, int pro_op, const void* pro_b, float pro_eps, int epi_op, hipStream_t st) {
     const int64_t Kb = ceil_div(K, 4);
-    const int64_t Kx = K * planes;
+    const int64_t Kx = (planes == 3) ? 3 * ceil_div(K, 64) * 64 : K;
     const StreamPlan pl = stream_plan(mode, B, N, Kb, w_layout, epi_op == EPI_SWIGLU_PAIRS ? 2 : 1);
     const int64_t Ny = (epi_op == EPI_SWIGLU_PAIRS) ? N / 2 : N;  // columns of Y
     const int y_size = dtype_size(y_dtype);

@@ -11,8 +11,7 @@ and releases the row-major buffer.  ``state_dict()`` still holds ``weight_packed
 (rebuilt from the tiled copy with ``bt_untile_weights``, bit for bit), ``load_state_dict`` and ``.to()`` /
 ``.cpu()`` work as usual.  Reading the attribute ``layer.weight_packed`` brings the row-major buffer back as a
 real buffer (so that in-place edits of it keep their meaning) and the layer then holds both copies until
-``drop_row_major()``; so does a call that only the row-major kernels can serve (the shape-generic kernel,
-fp32 activations with K % 64 != 0).  ``packed_weights()`` returns the reference-layout bytes without changing
+``drop_row_major()``; so does a call that only the row-major kernels can serve (the shape-generic kernel).  ``packed_weights()`` returns the reference-layout bytes without changing
 what the layer holds.  ``decode_tiled=False`` or ``BITTORCH_DECODE_TILED=0`` keeps the layer on ``weight_packed``
 alone.
 """
@@ -177,8 +176,6 @@ class TernaryLinearInference(nn.Module):
         if os.environ.get("BITTORCH_KERNEL") == "generic":  # the shape-generic kernel reads weight_packed
             return None
         if x.dtype not in (torch.float16, torch.bfloat16, torch.float32, torch.int8):
-            return None
-        if x.dtype == torch.float32 and self.in_features % 64 != 0:
             return None
         kb = (self.in_features + 3) // 4
         if ((self.out_features + 15) // 16) * ((kb + 15) // 16) * 256 >= 2 ** 32:  # beyond the kernels' 32-bit offsets

@@ -95,13 +95,13 @@ int bt_ternary_linear_forward(const void* X, int x_dtype, const int8_t* W_tern, 
  *   matrix-core GEMM beyond (crossover near 1.5-2 M outputs for K = 2560..4096;
  *   BITTORCH_STREAM_MAX_ROWS=n replaces the rule by "B <= n").  A single fp16 row (K % 16 == 0,
  *   K <= 16384, N % 4 == 0) runs the exact GEMV on the int8 matrix cores: the dot products are summed
- *   without rounding and rounded to fp32 once.  fp32 activations with K % 64 == 0 are
- *   first split into three bf16 planes (x = hi + mid + lo exactly) in the workspace and run
- *   on the same bf16 kernels with exact products and fp32 accumulation.  Other fp32 shapes,
- *   unaligned operands, a missing workspace and BITTORCH_KERNEL=generic run a generic
+ *   without rounding and rounded to fp32 once.  fp32 activations (any K) are first split into
+ *   three bf16 planes (x = hi + mid + lo exactly), each zero-padded to a multiple of 64 values, in
+ *   the workspace and run on the same bf16 kernels with exact products and fp32 accumulation.
+ *   Unaligned operands, a missing workspace and BITTORCH_KERNEL=generic run a generic
  *   kernel that accumulates in the reference's k order.
  *   workspace: at least bt_packed_forward_workspace_bytes(B,N,K,x_dtype) bytes
- *   (6*B*K rounded up to 256 for fp32 with K % 64 == 0, otherwise 0: may be NULL).
+ *   (6*B*Kp rounded up to 256 for fp32, Kp = K rounded up to 64; 0 otherwise: may be NULL).
  */
 size_t bt_packed_forward_workspace_bytes(int64_t B, int64_t N, int64_t K, int x_dtype);
 int bt_ternary_linear_packed_forward(const void* X, int x_dtype, const uint8_t* W_T,
@@ -225,7 +225,7 @@ int bt_ternary_linear_packed_forward_fused(const void* X, int64_t ld_x, int x_dt
  *     N/32 + P, so that one workgroup holds column h of both halves.
  *   bt_ternary_linear_tiled_forward: bt_ternary_linear_packed_forward_fused on the tiled copy, with
  *     pro_op = BT_PRO_NONE allowed (then ld_x must equal K); the weights are streamed once per 16
- *     rows of X, so it is meant for decode shapes; fp32 X needs K % 64 == 0 and the workspace.
+ *     rows of X, so it is meant for decode shapes; fp32 X needs the workspace.
  *     Results equal those of the row-major entry points bit for bit.
  *     epi_op = BT_EPI_SWIGLU_PAIRS (pair-ordered copy, no residual, no SwiGLU prologue): Y is [B, N/2],
  *     Y[b, h] = what bt_swiglu makes of the stored projections, rd(rd(silu(g)) * u) with g = rd(linear

@@ -122,9 +122,9 @@ def test_packed_forward_tall_batch_matches_streaming_kernel(oracle):
 
 
 def test_packed_forward_any_number_of_rows(oracle, monkeypatch):
-    """fp32 activations with K % 64 != 0 (the reference's MNIST layer, 784 -> 256) run the shape-generic kernel,
-    which takes any batch: more rows than a grid dimension holds included.  The streaming kernel serves a call
-    beyond its 65535 row blocks in slices."""
+    """The shape-generic kernel takes any batch, more rows than a grid dimension holds included (fp32, the
+    reference's MNIST layer 784 -> 256 cut to 16 columns), and is bit-exact against the oracle.  The streaming
+    kernel serves a call beyond its 65535 row blocks in slices."""
     from bittorch_amd import _C
     from bittorch_amd.quant import pack_ternary_transposed
     announce("packed_forward many rows")
@@ -133,13 +133,13 @@ def test_packed_forward_any_number_of_rows(oracle, monkeypatch):
     packed = pack_ternary_transposed(w)[0]
     scale = torch.rand(n) * 0.05 + 0.01
     bias = torch.randn(n) * 0.01
+    monkeypatch.setenv("BITTORCH_KERNEL", "generic")
     for b in (3, 70000):
         x = seeded_acts(b, k, seed=b)
         y = _C.ternary_linear_packed_forward(x.cuda(), packed.cuda(), scale.cuda(), bias.cuda(), k)
         ref = oracle.linear_packed(f32np(x), packed.numpy(), f32np(scale), k, f32np(bias))
         np.testing.assert_array_equal(f32np(y), ref)
     # dense int8 weights on the generic route, same batch
-    monkeypatch.setenv("BITTORCH_KERNEL", "generic")
     x = seeded_acts(70000, k, seed=5)
     y = _C.ternary_linear_forward(x.cuda(), w.cuda(), scale.cuda(), bias.cuda())
     np.testing.assert_array_equal(f32np(y), oracle.linear_unpacked(f32np(x), w.numpy(), f32np(scale), f32np(bias)))
@@ -153,6 +153,43 @@ def test_packed_forward_any_number_of_rows(oracle, monkeypatch):
     for r0 in (0, 16 * 65535 - 8, b - 24):
         part = _C.ternary_linear_packed_forward(xb[r0:r0 + 24].contiguous(), packed2, scale.cuda(), bias.cuda(), k2)
         assert torch.equal(yb[r0:r0 + 24], part)
+
+
+@pytest.mark.parametrize("b,n,k", [(1, 256, 784), (64, 256, 784), (3, 16, 20), (17, 100, 1), (5, 36, 63), (40, 64, 65),
+                                   (2, 8, 130), (1200, 256, 784), (70000, 16, 784), (4096, 512, 1000)])
+def test_packed_forward_fp32_any_k_on_the_matrix_cores(oracle, b, n, k):
+    """fp32 activations whose K is not a multiple of 64 (the reference's MNIST layer, 784 -> 256) run the matrix-core
+    kernels on zero-padded bf16 planes: every element within the reference tests' fp32 thresholds
+    (tests/test_packed_kernel.py:44-50) of the oracle's k-ordered fp32 sum, both weight layouts, the streaming kernel
+    and the tiled GEMM; equal to the float64 dot product to a few fp32 roundings."""
+    from bittorch_amd import _C
+    from bittorch_amd.quant import pack_ternary_transposed
+    announce("packed_forward fp32 padded planes", b, n, k)
+    w = random_ternary(n, k, seed=n + k)
+    packed = pack_ternary_transposed(w)[0]
+    g = torch.Generator().manual_seed(b + k)
+    scale = torch.rand(n, generator=g) * 0.05 + 0.01
+    bias = torch.randn(n, generator=g) * 0.01
+    x = seeded_acts(b, k, seed=b + 1)
+    xd, pd, sd, bd = x.cuda(), packed.cuda(), scale.cuda(), bias.cuda()
+    y = _C.ternary_linear_packed_forward(xd, pd, sd, bd, k)
+    rows = slice(0, b) if b <= 4096 else slice(b - 100, b)
+    ref = oracle.linear_packed(f32np(x[rows]), packed.numpy(), f32np(scale), k, f32np(bias))
+    assert_close_like_reference(f32np(y[rows]), ref, torch.float32)
+    exact = (x.double() @ w.double().T) * scale.double() + bias.double()
+    assert float((y.cpu().double() - exact).abs().max()) <= 4e-6 * float(exact.abs().max()) + 1e-7
+    tiled = _C.retile_weights(pd, k)
+    y_t = _C.ternary_linear_tiled_forward(xd, tiled, sd, bd, k, n)
+    # (the same kernel on either layout gives the same bits; where the dispatch picks the GEMM for one layout and the
+    # streaming kernel for the other, the sums differ in their order)
+    assert float((y_t.cpu().double() - exact).abs().max()) <= 4e-6 * float(exact.abs().max()) + 1e-7
+    assert_close_like_reference(f32np(y_t[rows]), ref, torch.float32)
+    # an unaligned activation base (a view one element into a buffer): element-wise plane split
+    if b * k < 1 << 20:
+        buf = torch.zeros(b * k + 1, device="cuda")
+        buf[1:] = xd.reshape(-1)
+        y_u = _C.ternary_linear_packed_forward(buf[1:].view(b, k), pd, sd, bd, k)
+        assert torch.equal(y_u, y)
 
 
 def test_packed_forward_fp32_generic_is_bit_exact(oracle, monkeypatch):

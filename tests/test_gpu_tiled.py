@@ -8,6 +8,8 @@
   with its int32 accumulators;
 * one direct comparison with the oracle, so that this file stands on its own.
 """
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -87,13 +89,17 @@ def test_tiled_forward_fp32_planes(oracle, n, k, route, monkeypatch):
                            _C.ternary_linear_packed_forward(x, wt, scale, None, k))
 
 
-def test_tiled_forward_fp32_ragged_k_is_refused(oracle):
+def test_tiled_forward_fp32_ragged_k(oracle):
+    """fp32 rows whose K is not a multiple of 64 run on zero-padded planes: same bits as the row-major entry point
+    (N = 37 is not a multiple of 4, so both take the streaming kernel's general column path)."""
     from bittorch_amd import _C
     _, wt = _packed(oracle, 37, 100)
     tiled = _C.retile_weights(wt, 100)
     x = seeded_acts(2, 100, dtype=torch.float32).cuda()
-    with pytest.raises(RuntimeError, match="K % 64"):
-        _C.ternary_linear_tiled_forward(x, tiled, torch.ones(37).cuda(), None, 100, 37)
+    scale = torch.ones(37).cuda()
+    y = _C.ternary_linear_tiled_forward(x, tiled, scale, None, 100, 37)
+    ref = oracle.linear_packed(f32np(x.cpu()), wt.cpu().numpy(), f32np(scale.cpu()), 100, None)
+    np.testing.assert_allclose(f32np(y), ref, rtol=1e-4, atol=1e-4)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -239,12 +245,20 @@ def test_module_holds_one_copy_of_its_weights(oracle):
     assert torch.equal(a(x), c.cuda()(x))
     a.drop_row_major()
     assert not a._has_row_major() and a.resident_weight_bytes() == n * k // 4
-    # a call only the row-major kernels serve (fp32 activations with K % 64 != 0) keeps both from then on
+    # fp32 rows of any K read the tiled copy too; a call only the row-major kernels serve (the shape-generic
+    # kernel) keeps both from then on
     b = _layer(oracle, 48, 100, seed=2)
     b(seeded_acts(1, 100, dtype=torch.float16).cuda())
     assert not b._has_row_major()
-    b(seeded_acts(2, 100, dtype=torch.float32).cuda())
+    y32 = b(seeded_acts(2, 100, dtype=torch.float32).cuda())
+    assert not b._has_row_major()
+    os.environ["BITTORCH_KERNEL"] = "generic"
+    try:
+        y_gen = b(seeded_acts(2, 100, dtype=torch.float32).cuda())
+    finally:
+        os.environ.pop("BITTORCH_KERNEL")
     assert b._has_row_major() and b.keep_row_major
+    np.testing.assert_allclose(f32np(y32), f32np(y_gen), rtol=1e-4, atol=1e-4)
 
 
 def test_module_rebuilds_tiled_copy_when_weights_change(oracle):
