@@ -203,10 +203,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(PlaneParams p) 
 #pragma unroll
             for (int t = 0; t < NACC; t++) {
                 if constexpr (LAYOUT == PL_TILED) {
-                    raw[f][t] = *(const uint32_t*)(p.W + (coloff[t] + (uint32_t)ws * 256u));
+                    raw[f][t] = ldw_nt(p.W + (coloff[t] + (uint32_t)ws * 256u));
                 } else {
                     const uint32_t ro = min((uint32_t)(16 * ws + 4 * g + q) * N32, last_rowoff);
-                    raw[f][t] = *(const uint32_t*)(p.W + (ro + coloff[t]));
+                    raw[f][t] = ldw_nt(p.W + (ro + coloff[t]));
                 }
             }
         }
@@ -319,7 +319,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(PlaneParams p) 
 // 16-column tiles (slab * 8 + w) * NACC .. + NACC - 1 of the unit over the whole of K.  The digit planes of the
 // unit's activation row are converted once per item by the whole workgroup into LDS.  The weight loads of a wave
 // form one uninterrupted stream: PF steps are always in flight, and the last batch of an item already requests the
-// first steps of the wave's next item.
+// first steps of the wave's next item.  Wave w walks the steps of its tiles in rotated order, starting at step
+// (w/8 of the way through K): streams that advance in lockstep from the same step hit the same memory channels at the
+// same time (a pure read of this address stream: 5.7 TB/s in lockstep, 6.7 TB/s rotated); the sums are integers, so
+// the order does not change a bit of the result.
 // LDS: a flag word per wave, then the digit planes of one row, padded with zero groups to a multiple of PF steps.
 template <int NACC, int PF>
 __global__ __launch_bounds__(512, 4) void gemv_planes_group_kernel(PlaneParams p) {
@@ -346,11 +349,12 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_group_kernel(PlaneParams p
 #pragma unroll
     for (int t = 0; t < NACC; t++) wcur[t] = tile_base(it, t);
     const uint32_t loff = (uint32_t)lane * 4u;
+    const int rot = (wave * (SP / PF)) / 8 * PF;  // first step of this wave's walk: a whole number of batches
     uint32_t raw[PF][NACC];
 #pragma unroll
     for (int f = 0; f < PF; f++)
 #pragma unroll
-        for (int t = 0; t < NACC; t++) raw[f][t] = *(const uint32_t*)(wcur[t] + ((size_t)min(f, S - 1) * 256 + loff));
+        for (int t = 0; t < NACC; t++) raw[f][t] = ldw_nt(wcur[t] + ((size_t)min(rot + f, S - 1) * 256 + loff));
 
     for (; it < p.items; it += (int)gridDim.x) {
         const int u = it / p.slabs, slab = it - u * p.slabs;
@@ -390,10 +394,14 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_group_kernel(PlaneParams p
         v4i acc[NACC];
 #pragma unroll
         for (int t = 0; t < NACC; t++) acc[t] = v4i{0, 0, 0, 0};
-        for (int base = 0; base < SP; base += PF) {
-            // refill target of this batch: the same item's next batch, or the first batch of the wave's next item
-            const bool last = base + PF >= SP;  // uniform
-            const int sb = last ? 0 : base + PF;
+        for (int b = 0; b < SP; b += PF) {
+            // this batch covers steps base .. base + PF - 1 of the rotated walk; refill target: the same item's next
+            // batch, or the first batch of the wave's next item
+            const bool last = b + PF >= SP;  // uniform
+            int base = b + rot;
+            if (base >= SP) base -= SP;
+            int sb = base + PF;
+            if (sb >= SP) sb -= SP;  // (after the last batch this is `rot` again: where the next item starts)
 #pragma unroll
             for (int f = 0; f < PF; f++) {
                 const uint4 av = *(const uint4*)(a_src + (size_t)(base + f) * 4 * PL_GROUP);
@@ -402,7 +410,7 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_group_kernel(PlaneParams p
 #pragma unroll
                 for (int t = 0; t < NACC; t++) {
                     acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, decode16_i8(raw[f][t]), acc[t], 0, 0, 0);
-                    raw[f][t] = *(const uint32_t*)((last ? wnext[t] : wcur[t]) + so);
+                    raw[f][t] = ldw_nt((last ? wnext[t] : wcur[t]) + so);
                 }
             }
         }
@@ -430,6 +438,152 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_group_kernel(PlaneParams p
             }
         }
         __syncthreads();  // every wave is done with the planes before the next item overwrites them
+    }
+}
+
+// ---- G units per launch, K up to 8 steps per wave: contiguous walk -------------------------------------------
+// The (unit, 16-column tile) pairs of the launch form one flat sequence, and the tiled copies make a unit's tiles
+// contiguous in memory (16 * K / 4 bytes each).  Workgroup b owns a contiguous run of the sequence; its eight waves
+// split K: wave w reads steps w * SPW .. + SPW - 1 of every tile, i.e. SPW * 256 consecutive bytes, so that the
+// workgroup as a whole reads its megabyte or so front to back, 2 KiB per wave at a time -- the access pattern that
+// streams fastest on this chip (a pure read: 7.2 TB/s, against 5.7-6.7 TB/s for 16 streams per workgroup that are
+// 16 KiB apart).  A wave's slice of the activation digits does not change from tile to tile: it is converted once
+// per unit and held in SPW * 4 registers, so the loop has no LDS reads.  The partial sums of the eight waves (six
+// int32 digit-row sums per column) are added with LDS atomics into one of two accumulator arrays; every EB tiles a
+// barrier ends the chunk, one thread per column finishes it (and clears the array) while the waves are already
+// adding the next chunk into the other array.  TB tiles of loads are always in flight per wave, across chunk and
+// unit boundaries.  Integer sums: same bits as every other split of K.
+constexpr int CH_EB = 32;  // tiles per chunk (one output column per thread)
+template <int SPW, int TB>
+__global__ __launch_bounds__(512, 4) void gemv_planes_chunk_kernel(PlaneParams p) {
+    static_assert(CH_EB % TB == 0, "chunks hold whole batches");
+    __shared__ int32_t accbuf[2][CH_EB][PL_N * 16];
+    __shared__ uint32_t flags[2][8];
+    __shared__ __attribute__((aligned(16))) uint8_t planes_all[8][SPW * 4 * PL_GROUP];
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 15, g = lane >> 4;
+    const int S = p.wsteps;
+    const int T16 = p.tiles16;
+    const int64_t total = (int64_t)p.G * T16;
+    // this workgroup's run of the flat tile sequence (p.slabs = tiles per workgroup, a multiple of TB)
+    const int64_t t_begin = (int64_t)blockIdx.x * p.slabs;
+    const int64_t t_end = (t_begin + p.slabs < total) ? t_begin + p.slabs : total;
+    if (t_begin >= t_end) return;
+
+    for (int i = tid; i < 2 * CH_EB * PL_N * 16; i += 512) (&accbuf[0][0][0])[i] = 0;
+
+    // byte offset of this wave's SPW steps inside a tile (steps past the end repeat the last one and meet zero digits)
+    uint32_t soff[SPW];
+#pragma unroll
+    for (int f = 0; f < SPW; f++) soff[f] = (uint32_t)min(wave * SPW + f, S - 1) * 256u + (uint32_t)lane * 4u;
+    const size_t tile_bytes = (size_t)S * 256;
+
+    // prefetch cursor: (unit, tile) of the next tile to request, its address
+    int pf_u = (int)(t_begin / T16);
+    int pf_t = (int)(t_begin - (int64_t)pf_u * T16);
+    int64_t pf_left = t_end - t_begin;  // tiles not yet requested
+    const uint8_t* pf_ptr = p.W_tab[pf_u] + (size_t)pf_t * tile_bytes;
+    uint32_t raw[TB][SPW];
+    auto request = [&](uint32_t (&dst)[SPW]) {
+        // (past the end of the run: the last tile again, never used)
+#pragma unroll
+        for (int f = 0; f < SPW; f++) dst[f] = ldw_nt(pf_ptr + soff[f]);
+        if (pf_left > 1) {
+            pf_left--;
+            pf_t++;
+            pf_ptr += tile_bytes;
+            if (pf_t == T16) {
+                pf_t = 0;
+                pf_u++;
+                pf_ptr = p.W_tab[pf_u];
+            }
+        }
+    };
+#pragma unroll
+    for (int i = 0; i < TB; i++) request(raw[i]);
+
+    uint8_t* planes = planes_all[wave];
+    const uint8_t* a_src = planes + g * PL_GROUP + (j % PL_N) * 16;
+    uint4 areg[SPW];
+    int cur = 0;
+    __syncthreads();  // accumulators cleared
+
+    int64_t t0 = t_begin;
+    while (t0 < t_end) {
+        const int u = (int)(t0 / T16);
+        const int tile0 = (int)(t0 - (int64_t)u * T16);
+        // the wave's slice of the unit's activation row -> digit planes -> registers (once per unit and workgroup)
+        {
+            const uint16_t* xrow = (const uint16_t*)p.X_tab[u];
+            const int c = lane;                               // chunk of eight values (SPW * 8 <= 64 chunks)
+            const int k = (wave * SPW * 8 + c) * 8;
+            uint4 v = *(const uint4*)(xrow + min(k, (int)p.K - 8));
+            v = zero_unless4(v, k < (int)p.K && c < SPW * 8);
+            const bool bad = park_chunk(planes, c, v, lane, c < SPW * 8);
+            const bool wave_bad = __builtin_amdgcn_ballot_w64(bad) != 0ull;
+            if (lane == 0) flags[u & 1][wave] = wave_bad ? 1u : 0u;
+            // (LDS accesses of one wave execute in order: the slice written above is visible to its own reads)
+#pragma unroll
+            for (int f = 0; f < SPW; f++) areg[f] = *(const uint4*)(a_src + (size_t)f * 4 * PL_GROUP);
+        }
+        // chunks of this unit inside the run
+        const int64_t unit_end = (int64_t)(u + 1) * T16;
+        const int64_t u_stop = (unit_end < t_end) ? unit_end : t_end;
+        for (int64_t c0 = t0; c0 < u_stop; c0 += CH_EB) {
+            const int ntiles = (int)((u_stop - c0 < CH_EB) ? u_stop - c0 : CH_EB);  // a multiple of TB
+            for (int tb = 0; tb < ntiles; tb += TB) {
+                v4i acc[TB];
+#pragma unroll
+                for (int i = 0; i < TB; i++) acc[i] = v4i{0, 0, 0, 0};
+#pragma unroll
+                for (int f = 0; f < SPW; f++) {
+                    const v4i a = {(int)areg[f].x, (int)areg[f].y, (int)areg[f].z, (int)areg[f].w};
+#pragma unroll
+                    for (int i = 0; i < TB; i++)
+                        acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, decode16_i8(raw[i][f]), acc[i], 0, 0, 0);
+                }
+#pragma unroll
+                for (int i = 0; i < TB; i++) request(raw[i]);
+                // lane (j, 0) holds digit rows 0..3 of column j, lane (j, 1) rows 4 and 5
+#pragma unroll
+                for (int i = 0; i < TB; i++) {
+                    int32_t* dst = &accbuf[cur][tb + i][j];
+                    if (g == 0) {
+#pragma unroll
+                        for (int r = 0; r < 4; r++) atomicAdd(dst + 16 * r, acc[i][r]);
+                    } else if (g == 1) {
+                        atomicAdd(dst + 16 * 4, acc[i][0]);
+                        atomicAdd(dst + 16 * 5, acc[i][1]);
+                    }
+                }
+            }
+            __syncthreads();  // every wave has added its share of this chunk
+            {
+                const int tl = tid >> 4, jj = tid & 15;
+                const int64_t n = (int64_t)(tile0 + (int)(c0 - t0) + tl) * 16 + jj;
+                if (tl < ntiles) {
+                    int32_t sums[PL_N];
+#pragma unroll
+                    for (int r = 0; r < PL_N; r++) {
+                        sums[r] = accbuf[cur][tl][16 * r + jj];
+                        accbuf[cur][tl][16 * r + jj] = 0;
+                    }
+                    if (n < p.N) {
+                        uint32_t fl = 0u;
+#pragma unroll
+                        for (int w = 0; w < 8; w++) fl |= flags[u & 1][w];
+                        const void* bias_u = p.bias_tab ? p.bias_tab[u] : nullptr;
+                        const float sc = load_elem_rt(p.scale_tab[u], p.scale_dtype, p.scale_bcast ? 0 : n);
+                        const float bs = bias_u ? load_elem_rt(bias_u, p.bias_dtype, n) : 0.0f;
+                        pl_store(p.Y_tab[u], nullptr, n, planes_to_f32(sums), sc, bs, fl != 0u);
+                    }
+                }
+            }
+            cur ^= 1;
+        }
+        t0 = u_stop;
     }
 }
 
@@ -516,6 +670,31 @@ static int launch_group_params(PlaneParams p, int64_t G, hipStream_t st) {
         g_group_cus = cus;
     }
     const int64_t wgs = 2 * (int64_t)g_group_cus;
+    // K of at most 8 steps per wave (K <= 4096) and whole batches of tiles: the contiguous walk
+    {
+        const int spw = (int)ceil_div(p.wsteps, 8);
+        const int tb = (spw >= 5) ? 2 : 4;
+        const int64_t total = G * p.tiles16;
+        // (below 16 tiles per workgroup the per-chunk barrier and the one-off conversion weigh more than the walk gains:
+        // G = 8 units of 4096 x 4096 10.5 against 11.7 us, G = 32 equal, G = 128 92 against 85 us)
+        // BITTORCH_GROUP_WALK=1 / =0 (tests, A/B runs): always / never, where the shape allows
+        const char* force = getenv("BITTORCH_GROUP_WALK");
+        const bool want = force ? (force[0] == '1') : (total >= 16 * wgs);
+        if (spw >= 3 && spw <= 8 && p.tiles16 % tb == 0 && want) {
+            int64_t tpw = ceil_div(ceil_div(total, wgs), tb) * tb;
+            p.slabs = (int)tpw;  // tiles per workgroup
+            const unsigned grid = (unsigned)ceil_div(total, tpw);
+            switch (spw) {
+                case 3: hipLaunchKernelGGL((gemv_planes_chunk_kernel<3, 4>), dim3(grid), dim3(512), 0, st, p); break;
+                case 4: hipLaunchKernelGGL((gemv_planes_chunk_kernel<4, 4>), dim3(grid), dim3(512), 0, st, p); break;
+                case 5: hipLaunchKernelGGL((gemv_planes_chunk_kernel<5, 2>), dim3(grid), dim3(512), 0, st, p); break;
+                case 6: hipLaunchKernelGGL((gemv_planes_chunk_kernel<6, 2>), dim3(grid), dim3(512), 0, st, p); break;
+                case 7: hipLaunchKernelGGL((gemv_planes_chunk_kernel<7, 2>), dim3(grid), dim3(512), 0, st, p); break;
+                default: hipLaunchKernelGGL((gemv_planes_chunk_kernel<8, 2>), dim3(grid), dim3(512), 0, st, p); break;
+            }
+            return check_launch("gemv_planes_group");
+        }
+    }
     // columns per wave: 32 (two tiles) streams best (5.3 TB/s against 4.8 with four tiles and 4.4-5.0 with one at
     // G = 128, 4096 x 4096); another width only where it fills the resident workgroups markedly more evenly
     int nacc = 2;

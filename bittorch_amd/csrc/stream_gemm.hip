@@ -288,7 +288,7 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p_in) {
             if constexpr (TILED) {
                 const uint32_t so = (uint32_t)min(ws, p.wsteps - 1) * 256u;
 #pragma unroll
-                for (int t = 0; t < NCO; t++) raw[f][t] = *(const uint32_t*)(p.W_T + (coloff[t] + so));
+                for (int t = 0; t < NCO; t++) raw[f][t] = ldw_nt(p.W_T + (coloff[t] + so));
             } else if constexpr (BYTE) {
 #pragma unroll
                 for (int r = 0; r < 4; r++)
@@ -296,7 +296,7 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p_in) {
             } else if constexpr (QUAD) {
                 const uint32_t rc = min(ro, last_rowoff);
 #pragma unroll
-                for (int cb = 0; cb < NCO; cb++) raw[f][cb] = *(const uint32_t*)(p.W_T + (rc + coloff[cb]));
+                for (int cb = 0; cb < NCO; cb++) raw[f][cb] = ldw_nt(p.W_T + (rc + coloff[cb]));
             } else {
 #pragma unroll
                 for (int r = 0; r < 4; r++) {

@@ -105,7 +105,13 @@ def _tables(_C, xs, tiles, scales, biases, ys):
 @pytest.mark.parametrize("g,n,k,per_tensor,bias", [(1, 4096, 4096, True, True), (5, 256, 512, False, True),
                                                    (37, 1024, 1024, False, False), (3, 100, 144, False, True),
                                                    (9, 2560, 6912, True, True), (130, 128, 64, False, True),
-                                                   (4, 36, 8192, False, True)])
+                                                   (4, 36, 8192, False, True),
+                                                   # K of 3..8 steps per wave: the contiguous-walk kernel
+                                                   (7, 96, 2560, False, True), (3, 2560, 2560, True, True),
+                                                   (5, 64, 1536, False, False), (11, 4128, 3008, False, True),
+                                                   (6, 48, 3600, True, True), (4, 32, 4080, False, True),
+                                                   (70, 544, 4096, False, True), (2, 20, 1104, False, True),
+                                                   (600, 32, 2048, False, True)])
 def test_grouped_launch_equals_single_calls(oracle, g, n, k, per_tensor, bias):
     import os
     from bittorch_amd import _C
@@ -120,8 +126,14 @@ def test_grouped_launch_equals_single_calls(oracle, g, n, k, per_tensor, bias):
         singles.append(_C.ternary_linear_tiled_forward(xs[-1], tiles[-1], scales[-1], biases[-1], k, n))
         if u == 0:
             assert torch.equal(singles[0].cpu(), _expect(oracle, x, packed, scale, b, k))
+    # the library's own choice of kernel, then the contiguous-walk kernel (where the shape allows it) and the
+    # one-stream-per-wave kernel in its three widths
     try:
-        for nacc in (None, "1", "2", "4"):
+        for walk, nacc in ((None, None), ("1", None), ("0", "1"), ("0", "2"), ("0", "4")):
+            os.environ.pop("BITTORCH_GROUP_WALK", None)
+            os.environ.pop("BITTORCH_GROUP_NACC", None)
+            if walk:
+                os.environ["BITTORCH_GROUP_WALK"] = walk
             if nacc:
                 os.environ["BITTORCH_GROUP_NACC"] = nacc
             ys = [torch.full((1, n), float("nan"), dtype=torch.float16, device="cuda") for _ in range(g)]
@@ -129,9 +141,10 @@ def test_grouped_launch_equals_single_calls(oracle, g, n, k, per_tensor, bias):
             _C.ternary_gemv_grouped(*tabs, k, n, scale_len=1 if per_tensor else n)
             torch.cuda.synchronize()
             for u in range(g):
-                assert torch.equal(ys[u], singles[u]), (u, nacc)
+                assert torch.equal(ys[u], singles[u]), (u, walk, nacc)
     finally:
         os.environ.pop("BITTORCH_GROUP_NACC", None)
+        os.environ.pop("BITTORCH_GROUP_WALK", None)
 
 
 def test_grouped_launch_config2_units_and_shared_operands(oracle):
@@ -161,6 +174,29 @@ def test_grouped_launch_config2_units_and_shared_operands(oracle):
             assert torch.equal(y, _C.ternary_linear_tiled_forward(xs_[a], tiles_[w], scales_[w], biases_[w], k, n))
     x, packed, scale, b = base[1][0], base[2][1], base[2][2], base[2][3]
     assert torch.equal(ys[units.index((1, 2))].cpu(), _expect(oracle, x, packed, scale, b, k))
+
+
+def test_grouped_launch_non_finite_row_and_large_group(oracle, monkeypatch):
+    """160 units of 2048 x 2048 (the contiguous-walk kernel by the library's own rule): one unit's row holds an
+    infinity and gives NaN in every column, its neighbours are untouched."""
+    from bittorch_amd import _C
+    announce("grouped gemv non-finite")
+    n = k = 2048
+    base = [_setup(n, k, seed=s, per_tensor=False) for s in range(3)]
+    tiles_ = [_C.retile_weights(b[1].cuda(), k) for b in base]
+    g = 160
+    xs = [base[u % 3][0].clone().cuda() for u in range(g)]
+    xs[77][0, 1999] = float("inf")
+    tiles = [tiles_[u % 3] for u in range(g)]
+    scales = [base[u % 3][2].cuda() for u in range(g)]
+    biases = [base[u % 3][3].cuda() for u in range(g)]
+    ys = [torch.empty(1, n, dtype=torch.float16, device="cuda") for _ in range(g)]
+    _C.ternary_gemv_grouped(*_tables(_C, xs, tiles, scales, biases, ys), k, n, scale_len=n)
+    torch.cuda.synchronize()
+    assert torch.isnan(ys[77]).all()
+    for u in (0, 76, 78, 159):
+        b = base[u % 3]
+        assert torch.equal(ys[u].cpu(), _expect(oracle, b[0], b[1], b[2], b[3], k))
 
 
 def test_grouped_launch_argument_errors():
