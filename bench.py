@@ -434,13 +434,13 @@ def main():
             "timing": "one HIP graph of all steps, median of the replays, each between two synchronisations",
         },
         "roofline": {
-            "kernel": "bt::gemv_planes_group_kernel (fp16 activations as six int8 digit rows, decode-tiled weights)",
+            "kernel": "bt::gemv_planes_chunk_kernel (fp16 activations as six int8 digit rows, decode-tiled weights read front to back)",
             "bound": "hbm",
             "achieved": round(achieved, 2),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": measured_traffic("gemv_planes_group_kernel_G128_config2"),
+            "traffic": measured_traffic("gemv_planes_chunk_kernel_G128_config2"),
             "launch_us": round(kernel_us, 3),
             "algorithmic_bytes_per_launch": G * weight_bytes,
         },

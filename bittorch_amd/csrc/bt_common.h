@@ -160,6 +160,15 @@ __device__ __forceinline__ uint32_t ldw_nt(const void* p) {
     return __builtin_nontemporal_load((const uint32_t*)p);
 #endif
 }
+__device__ __forceinline__ uint2 ldw2_nt(const void* p) {
+#ifdef BT_NO_NT
+    return *(const uint2*)p;
+#else
+    typedef uint32_t u32x2_nt __attribute__((ext_vector_type(2)));
+    const u32x2_nt v = __builtin_nontemporal_load((const u32x2_nt*)p);
+    return make_uint2(v[0], v[1]);
+#endif
+}
 __device__ __forceinline__ uint4 ldw4_nt(const void* p) {
 #ifdef BT_NO_NT
     return *(const uint4*)p;

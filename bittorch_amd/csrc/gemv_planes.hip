@@ -484,7 +484,9 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_chunk_kernel(PlaneParams p
     int pf_u = (int)(t_begin / T16);
     int pf_t = (int)(t_begin - (int64_t)pf_u * T16);
     int64_t pf_left = t_end - t_begin;  // tiles not yet requested
-    const uint8_t* pf_ptr = p.W_tab[pf_u] + (size_t)pf_t * tile_bytes;
+    // (one matrix per launch: direct pointers instead of tables)
+    const bool tab = p.W_tab != nullptr;
+    const uint8_t* pf_ptr = (tab ? p.W_tab[pf_u] : p.W) + (size_t)pf_t * tile_bytes;
     uint32_t raw[TB][SPW];
     auto request = [&](uint32_t (&dst)[SPW]) {
         // (past the end of the run: the last tile again, never used)
@@ -497,7 +499,7 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_chunk_kernel(PlaneParams p
             if (pf_t == T16) {
                 pf_t = 0;
                 pf_u++;
-                pf_ptr = p.W_tab[pf_u];
+                pf_ptr = tab ? p.W_tab[pf_u] : p.W;
             }
         }
     };
@@ -516,7 +518,7 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_chunk_kernel(PlaneParams p
         const int tile0 = (int)(t0 - (int64_t)u * T16);
         // the wave's slice of the unit's activation row -> digit planes -> registers (once per unit and workgroup)
         {
-            const uint16_t* xrow = (const uint16_t*)p.X_tab[u];
+            const uint16_t* xrow = (const uint16_t*)(tab ? p.X_tab[u] : p.X);
             const int c = lane;                               // chunk of eight values (SPW * 8 <= 64 chunks)
             const int k = (wave * SPW * 8 + c) * 8;
             uint4 v = *(const uint4*)(xrow + min(k, (int)p.K - 8));
@@ -574,10 +576,10 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_chunk_kernel(PlaneParams p
                         uint32_t fl = 0u;
 #pragma unroll
                         for (int w = 0; w < 8; w++) fl |= flags[u & 1][w];
-                        const void* bias_u = p.bias_tab ? p.bias_tab[u] : nullptr;
-                        const float sc = load_elem_rt(p.scale_tab[u], p.scale_dtype, p.scale_bcast ? 0 : n);
+                        const void* bias_u = tab ? (p.bias_tab ? p.bias_tab[u] : nullptr) : p.bias;
+                        const float sc = load_elem_rt(tab ? p.scale_tab[u] : p.scale, p.scale_dtype, p.scale_bcast ? 0 : n);
                         const float bs = bias_u ? load_elem_rt(bias_u, p.bias_dtype, n) : 0.0f;
-                        pl_store(p.Y_tab[u], nullptr, n, planes_to_f32(sums), sc, bs, fl != 0u);
+                        pl_store(tab ? p.Y_tab[u] : p.Y, tab ? nullptr : p.residual, n, planes_to_f32(sums), sc, bs, fl != 0u);
                     }
                 }
             }
@@ -601,8 +603,49 @@ bool planes_supported(int x_dtype, int y_dtype, int64_t B, int64_t N, int64_t K,
     return ((uintptr_t)W) % 4 == 0 && (ceil_div(K, 4) + 64) * N < (1ll << 32);
 }
 
+// grouped and wide launches: 2 workgroups of 8 waves per compute unit
+static int g_group_cus = 0;
+static int64_t resident_wgs() {
+    if (!g_group_cus) {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        g_group_cus = cus;
+    }
+    return 2 * (int64_t)g_group_cus;
+}
+
+// The contiguous-walk kernel where the shape allows it: K of 3..8 steps per wave (1040 <= K <= 4096), whole batches of
+// tiles, and at least `min_tiles_per_wg` tiles per resident workgroup (below that the per-chunk barrier and the one-off
+// conversion weigh more than the walk gains: G = 8 units of 4096 x 4096 10.5 against 11.7 us, G = 32 equal, G = 128
+// 92 against 85 us).  BITTORCH_GROUP_WALK=1 / =0 (tests, A/B runs): always / never.
+static bool launch_walk(PlaneParams p, int64_t G, int64_t wgs, int min_tiles_per_wg, hipStream_t st) {
+    const int spw = (int)ceil_div(p.wsteps, 8);
+    const int tb = (spw >= 5) ? 2 : 4;
+    const int64_t total = G * p.tiles16;
+    const char* force = getenv("BITTORCH_GROUP_WALK");
+    const bool want = force ? (force[0] == '1') : (total >= min_tiles_per_wg * wgs);
+    if (spw < 3 || spw > 8 || p.tiles16 % tb != 0 || !want) return false;
+    const int64_t tpw = ceil_div(ceil_div(total, wgs), tb) * tb;
+    p.G = (int)G;
+    p.slabs = (int)tpw;  // tiles per workgroup
+    const unsigned grid = (unsigned)ceil_div(total, tpw);
+    switch (spw) {
+        case 3: hipLaunchKernelGGL((gemv_planes_chunk_kernel<3, 4>), dim3(grid), dim3(512), 0, st, p); break;
+        case 4: hipLaunchKernelGGL((gemv_planes_chunk_kernel<4, 4>), dim3(grid), dim3(512), 0, st, p); break;
+        case 5: hipLaunchKernelGGL((gemv_planes_chunk_kernel<5, 2>), dim3(grid), dim3(512), 0, st, p); break;
+        case 6: hipLaunchKernelGGL((gemv_planes_chunk_kernel<6, 2>), dim3(grid), dim3(512), 0, st, p); break;
+        case 7: hipLaunchKernelGGL((gemv_planes_chunk_kernel<7, 2>), dim3(grid), dim3(512), 0, st, p); break;
+        default: hipLaunchKernelGGL((gemv_planes_chunk_kernel<8, 2>), dim3(grid), dim3(512), 0, st, p); break;
+    }
+    return true;
+}
+
 template <int LAYOUT, int NACC, int EPI = EPI_NONE>
 static void launch_planes_k(const PlaneParams& p, hipStream_t st) {
+    // (16 or 4 waves per workgroup instead of 8: 3.72-3.74 against 3.70-3.74 us at 4096 x 4096 -- the launch is
+    // bounded by its one round trip to memory, not by how the workgroup divides the work)
     constexpr int WAVES = 8, PF = 8;
     const int nsteps = (int)ceil_div(p.K, 64);
     const int spw = (int)ceil_div(nsteps, WAVES);
@@ -647,6 +690,9 @@ int launch_planes(const void* X, const uint8_t* W, int w_layout, const Epilogue&
         else launch_planes_k<PL_TILED, 2, EPI_SWIGLU_PAIRS>(p, st);
         return check_launch("gemv_planes");
     }
+    // a matrix wide enough to give every resident workgroup a dozen tiles: the grouped launch's contiguous walk
+    // (N = 128256, K = 4096: 26.2 against 28.0 us; N = 32768: 11.7 against 10.9)
+    if (w_layout == W_LAYOUT_TILED && launch_walk(p, 1, resident_wgs(), 12, st)) return check_launch("gemv_planes");
     if (w_layout == W_LAYOUT_TILED) {
         if (nacc == 4) launch_planes_k<PL_TILED, 4>(p, st);
         else if (nacc == 2) launch_planes_k<PL_TILED, 2>(p, st);
@@ -658,43 +704,10 @@ int launch_planes(const void* X, const uint8_t* W, int w_layout, const Epilogue&
     return check_launch("gemv_planes");
 }
 
-// grouped launch: 2 workgroups of 8 waves per compute unit
-static int g_group_cus = 0;
 
 static int launch_group_params(PlaneParams p, int64_t G, hipStream_t st) {
-    if (!g_group_cus) {
-        int dev = 0, cus = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-            cus = 256;
-        g_group_cus = cus;
-    }
-    const int64_t wgs = 2 * (int64_t)g_group_cus;
-    // K of at most 8 steps per wave (K <= 4096) and whole batches of tiles: the contiguous walk
-    {
-        const int spw = (int)ceil_div(p.wsteps, 8);
-        const int tb = (spw >= 5) ? 2 : 4;
-        const int64_t total = G * p.tiles16;
-        // (below 16 tiles per workgroup the per-chunk barrier and the one-off conversion weigh more than the walk gains:
-        // G = 8 units of 4096 x 4096 10.5 against 11.7 us, G = 32 equal, G = 128 92 against 85 us)
-        // BITTORCH_GROUP_WALK=1 / =0 (tests, A/B runs): always / never, where the shape allows
-        const char* force = getenv("BITTORCH_GROUP_WALK");
-        const bool want = force ? (force[0] == '1') : (total >= 16 * wgs);
-        if (spw >= 3 && spw <= 8 && p.tiles16 % tb == 0 && want) {
-            int64_t tpw = ceil_div(ceil_div(total, wgs), tb) * tb;
-            p.slabs = (int)tpw;  // tiles per workgroup
-            const unsigned grid = (unsigned)ceil_div(total, tpw);
-            switch (spw) {
-                case 3: hipLaunchKernelGGL((gemv_planes_chunk_kernel<3, 4>), dim3(grid), dim3(512), 0, st, p); break;
-                case 4: hipLaunchKernelGGL((gemv_planes_chunk_kernel<4, 4>), dim3(grid), dim3(512), 0, st, p); break;
-                case 5: hipLaunchKernelGGL((gemv_planes_chunk_kernel<5, 2>), dim3(grid), dim3(512), 0, st, p); break;
-                case 6: hipLaunchKernelGGL((gemv_planes_chunk_kernel<6, 2>), dim3(grid), dim3(512), 0, st, p); break;
-                case 7: hipLaunchKernelGGL((gemv_planes_chunk_kernel<7, 2>), dim3(grid), dim3(512), 0, st, p); break;
-                default: hipLaunchKernelGGL((gemv_planes_chunk_kernel<8, 2>), dim3(grid), dim3(512), 0, st, p); break;
-            }
-            return check_launch("gemv_planes_group");
-        }
-    }
+    const int64_t wgs = resident_wgs();
+    if (launch_walk(p, G, wgs, 16, st)) return check_launch("gemv_planes_group");
     // columns per wave: 32 (two tiles) streams best (5.3 TB/s against 4.8 with four tiles and 4.4-5.0 with one at
     // G = 128, 4096 x 4096); another width only where it fills the resident workgroups markedly more evenly
     int nacc = 2;

@@ -71,12 +71,20 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_pack_fast_kernel(
         if constexpr (DT == BT_F32) {
             const float4* rowp = (const float4*)((const float*)W + (int64_t)n * K) + lane;
 #pragma unroll
-            for (int j = 0; j < ITERS; j++) v[j] = (j < nfull) ? rowp[j * 64] : make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int j = 0; j < ITERS; j++) {
+                if (j < nfull) {
+                    const uint4 t = ldw4_nt(rowp + j * 64);
+                    v[j] = make_float4(__builtin_bit_cast(float, t.x), __builtin_bit_cast(float, t.y),
+                                       __builtin_bit_cast(float, t.z), __builtin_bit_cast(float, t.w));
+                } else {
+                    v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+            }
         } else {
             const uint2* rowp = (const uint2*)((const uint16_t*)W + (int64_t)n * K) + lane;
 #pragma unroll
             for (int j = 0; j < ITERS; j++) {
-                const uint2 t = (j < nfull) ? rowp[j * 64] : make_uint2(0u, 0u);
+                const uint2 t = (j < nfull) ? ldw2_nt(rowp + j * 64) : make_uint2(0u, 0u);
                 if constexpr (DT == BT_F16)
                     v[j] = make_float4(f16_bits_to_f32((uint16_t)t.x), f16_bits_to_f32((uint16_t)(t.x >> 16)),
                                        f16_bits_to_f32((uint16_t)t.y), f16_bits_to_f32((uint16_t)(t.y >> 16)));
