@@ -50,15 +50,13 @@ struct GemmParams {
 
 __device__ __forceinline__ void store4(void* Y, int dt, int64_t idx, const float (&v)[4]) {
     if (dt == BT_F32) {
-        *(float4*)((float*)Y + idx) = make_float4(v[0], v[1], v[2], v[3]);
+        st4_nt((float*)Y + idx, __builtin_bit_cast(uint32_t, v[0]), __builtin_bit_cast(uint32_t, v[1]),
+               __builtin_bit_cast(uint32_t, v[2]), __builtin_bit_cast(uint32_t, v[3]));
     } else {
         uint16_t h[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) h[i] = (dt == BT_F16) ? f32_to_f16_bits(v[i]) : f32_to_bf16_bits(v[i]);
-        uint2 o;
-        o.x = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
-        o.y = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
-        *(uint2*)((uint16_t*)Y + idx) = o;
+        st2_nt((uint16_t*)Y + idx, (uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
     }
 }
 
@@ -112,7 +110,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&a
             }
             if (p.epi.residual) add_residual4(y, p.epi.residual, YDT, m * p.N + ncol);
             store4(p.Y, YDT, m * p.N + ncol, y);
-            if (p.acc_out) *(int4*)(p.acc_out + m * p.N + ncol) = make_int4(a127[0], a127[1], a127[2], a127[3]);
+            if (p.acc_out) st4_nt(p.acc_out + m * p.N + ncol, (uint32_t)a127[0], (uint32_t)a127[1], (uint32_t)a127[2], (uint32_t)a127[3]);
         }
     }
 }
