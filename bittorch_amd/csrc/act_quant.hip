@@ -96,10 +96,11 @@ __global__ __launch_bounds__(256) void act_quant_row_kernel(const void* __restri
         const int k = (i * 256 + tid) * 8;
         const int kc = min(k, K - 8);  // clamped, unconditional loads; zeroed below
         if constexpr (DT == BT_F32) {
-            const float4 a = *(const float4*)((const float*)X + base + kc);
-            const float4 b = *(const float4*)((const float*)X + base + kc + 4);
-            v[i][0] = a.x; v[i][1] = a.y; v[i][2] = a.z; v[i][3] = a.w;
-            v[i][4] = b.x; v[i][5] = b.y; v[i][6] = b.z; v[i][7] = b.w;
+            const uint4 a = *(const uint4*)((const float*)X + base + kc);
+            const uint4 b = *(const uint4*)((const float*)X + base + kc + 4);
+            const uint32_t da[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[i][e] = __builtin_bit_cast(float, da[e]);
         } else {
             const uint4 u = *(const uint4*)((const uint16_t*)X + base + kc);
             const uint32_t d[4] = {u.x, u.y, u.z, u.w};
@@ -137,7 +138,7 @@ __global__ __launch_bounds__(256) void act_quant_row_kernel(const void* __restri
             else hi |= byte << (8 * (e - 4));
         }
         const uint2 o = q_layout == Q_OPERAND_ORDER ? q_to_operand_order(lo, hi, tid & 1) : make_uint2(lo, hi);
-        if (k < K) *(uint2*)(Q + base + k) = o;  // K % 16 == 0 in operand order: both lanes of a pair store
+        if (k < K) st2_nt(Q + base + k, o.x, o.y);  // K % 16 == 0 in operand order: both lanes of a pair store
     }
 }
 
