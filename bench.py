@@ -94,7 +94,7 @@ def graph_time(fn, steps, warmup, torch, min_replays=None):
 _probe_lib = None
 
 
-def probe_mfma_int8(torch, device, blocks=2048, iters=4096, random_operands=0):
+def probe_mfma_int8(torch, device, blocks=2048, iters=4096, random_operands=0, return_clock=False):
     """Launches the int8 matrix-core rate probe (bench_mfma_probe.so, this benchmark's own aid) on the
     current stream; returns the number of integer operations the launch performs."""
     import ctypes
@@ -104,11 +104,14 @@ def probe_mfma_int8(torch, device, blocks=2048, iters=4096, random_operands=0):
         _probe_lib.bench_probe_mfma_i8.restype = ctypes.c_int
         _probe_lib.bench_probe_mfma_i8.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
                                                    ctypes.c_void_p, ctypes.c_void_p]
-    out = torch.zeros(1, dtype=torch.int32, device=device)
+    out = torch.zeros(8, dtype=torch.int32, device=device)
     ops = ctypes.c_double(0.0)
     rc = _probe_lib.bench_probe_mfma_i8(blocks, iters, int(random_operands), out.data_ptr(), ctypes.addressof(ops),
                                         torch.cuda.current_stream(device).cuda_stream)
     assert rc == 0
+    if return_clock:  # (synchronizes) shader-clock cycles per 100 MHz tick of workgroup 0's loop, in MHz
+        cyc, ticks = int(out[2]), int(out[3])
+        return ops.value, (100.0 * cyc / ticks if ticks > 0 else None)
     return ops.value
 
 
@@ -567,10 +570,14 @@ def main():
             return ops * 5 / (e0.elapsed_time(e1) * 1e-3) / 1e12
 
         probe_tops = {"constant_operands": probe(0), "random_operands": probe(1), "gemm_register_footprint": probe(2)}
+        _, probe_mhz = probe_mfma_int8(torch, dev, 2048, 4096, 2, return_clock=True)
         extra["mfma_i8_register_only_probe"] = {
             "tops": {k: round(v, 1) for k, v in probe_tops.items()},
             "frac_of_int8_peak": round(probe_tops["gemm_register_footprint"] / INT8_PEAK_TOPS, 4),
-            "note": "2048 workgroups x 8 waves of back-to-back v_mfma_i32_16x16x64_i8, no memory traffic in the loop",
+            "shader_clock_MHz_under_this_load": None if probe_mhz is None else round(probe_mhz),
+            "note": "2048 workgroups x 8 waves of back-to-back v_mfma_i32_16x16x64_i8, no memory traffic in the loop; "
+                    "the clock is what workgroup 0 measures in its loop (cycle counter against the 100 MHz real-time "
+                    "counter): the 5 POPS peak assumes 2.4 GHz",
         }
         for key in list(extra):
             if key.startswith("prefill_int8"):

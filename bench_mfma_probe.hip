@@ -48,6 +48,8 @@ __global__ __launch_bounds__(512) void mfma_i8_probe_kernel(int iters, int rando
 // Same measurement with the register footprint of the prefill GEMM's inner product: a
 // 128 x 64 accumulator tile per wave (32 accumulators = 128 VGPRs), four A and four B operand
 // fragments per 32 MFMAs.
+// out[2], out[3]: shader-clock cycles and 100 MHz real-time ticks workgroup 0 spent in the loop (the ratio is the clock
+// the chip sustains under this load).
 __global__ __launch_bounds__(512) void mfma_i8_probe_tile_kernel(int iters, int* __restrict__ out) {
     const int lane = threadIdx.x & 63;
     v4i a[8], b[4], acc[8][4];
@@ -64,11 +66,16 @@ __global__ __launch_bounds__(512) void mfma_i8_probe_tile_kernel(int iters, int*
     for (int i = 0; i < 8; i++)
 #pragma unroll
         for (int t = 0; t < 4; t++) acc[i][t] = v4i{lane, i, t, 0};
+    const unsigned long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
     for (int it = 0; it < iters; it += 4) {
 #pragma unroll
         for (int i = 0; i < 8; i++)
 #pragma unroll
             for (int t = 0; t < 4; t++) acc[i][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i], b[t], acc[i][t], 0, 0, 0);
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        out[2] = (int)(__builtin_readcyclecounter() - c0);
+        out[3] = (int)(__builtin_amdgcn_s_memrealtime() - r0);
     }
     int s = 0;
 #pragma unroll

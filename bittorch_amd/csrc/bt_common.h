@@ -141,11 +141,14 @@ __device__ __forceinline__ float div127(float x) {
     return __builtin_fmaf(r, y, q0);
 }
 // int8 path: ((float(acc) * s_x) / 127) * w_scale + bias, left to right
-__device__ __forceinline__ float epi_int8(int32_t acc127, float sx, float ws, float b) {
-    float r = __fmul_rn((float)acc127, sx);
+__device__ __forceinline__ float epi_int8_f(float acc127, float sx, float ws, float b) {
+    float r = __fmul_rn(acc127, sx);
     r = div127(r);
     r = __fmul_rn(r, ws);
     return __fadd_rn(r, b);
+}
+__device__ __forceinline__ float epi_int8(int32_t acc127, float sx, float ws, float b) {
+    return epi_int8_f((float)acc127, sx, ws, b);
 }
 // 127 * a without the quarter-rate 32-bit multiply
 __device__ __forceinline__ int32_t times127(int32_t a) { return (int32_t)(((uint32_t)a << 7) - (uint32_t)a); }

@@ -115,8 +115,9 @@ static bool fast_path_ok(const void* Y, int64_t N, int64_t K) {
     return ((uintptr_t)Y) % 16 == 0 && N < (1ll << 30) && K < (1ll << 30);
 }
 
-// int32 accumulators hold sum_k q*127w with |q| <= 127
-static const int64_t kMaxKInt8 = 133000;
+// int32 accumulators hold sum_k q*127w with |q| <= 127; the matrix cores sum q*w (|sum| <= 127 K), which the prefill
+// GEMM's epilogue converts to fp32 before it multiplies by 127: exact while 127 K < 2^24
+static const int64_t kMaxKInt8 = 132096;
 
 // batches up to this many rows go through the streaming (decode-shape) kernel
 // Streaming kernel or tiled GEMM?  The streaming kernel runs the 16-row blocks of a call concurrently in one

@@ -101,16 +101,22 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&a
             if (m >= p.M) continue;
             const float sx = e.sx[mbi][r];
             float y[4];
-            int32_t a127[4];
 #pragma unroll
             for (int t = 0; t < 4; t++) {
-                const int32_t a = acc[MB0 + mbi][t][r];
-                a127[t] = times127(a);
-                y[t] = epi_int8(a127[t], sx, ws[t], bs[t]);
+                // float(127 a) = float(a) * 127 rounded once: |a| <= 127 K < 2^24 (checked by the host), so float(a)
+                // is exact and the product rounds the same integer the reference converts (one operation less than
+                // 127 a in integers first)
+                const float a127f = __fmul_rn((float)acc[MB0 + mbi][t][r], 127.0f);
+                y[t] = epi_int8_f(a127f, sx, ws[t], bs[t]);
             }
             if (p.epi.residual) add_residual4(y, p.epi.residual, YDT, m * p.N + ncol);
             store4(p.Y, YDT, m * p.N + ncol, y);
-            if (p.acc_out) st4_nt(p.acc_out + m * p.N + ncol, (uint32_t)a127[0], (uint32_t)a127[1], (uint32_t)a127[2], (uint32_t)a127[3]);
+            if (p.acc_out) {
+                uint32_t a127[4];
+#pragma unroll
+                for (int t = 0; t < 4; t++) a127[t] = (uint32_t)times127(acc[MB0 + mbi][t][r]);
+                st4_nt(p.acc_out + m * p.N + ncol, a127[0], a127[1], a127[2], a127[3]);
+            }
         }
     }
 }
@@ -120,6 +126,38 @@ __device__ __forceinline__ void gemm_epilogue_dt(const GemmParams& p, const v4i 
     if (p.y_dtype == BT_BF16) gemm_epilogue<BT_BF16, MB0>(p, acc, m0, g, ncol, e);
     else if (p.y_dtype == BT_F16) gemm_epilogue<BT_F16, MB0>(p, acc, m0, g, ncol, e);
     else gemm_epilogue<BT_F32, MB0>(p, acc, m0, g, ncol, e);
+}
+
+// Adds the two K halves: waves (wn, 0) and (wn, 1) hold partial sums of the same outputs.  K half 1 hands over row
+// blocks 0..3, K half 0 hands over row blocks 4..7; word (q, wn, lane) of the exchange buffer (64 KiB of LDS) is
+// register q of that lane.  Every wave must be done with the buffer's previous contents.
+__device__ __forceinline__ void exchange_k_halves(v4i (&acc)[G_MB][4], uint8_t* lds, int wn, int kgrp, int lane) {
+    int32_t* xch = (int32_t*)lds;
+    const int slot = wn * 64 + lane;
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+        const int giver = 1 - half;  // K half that hands over row blocks 4*half .. 4*half+3
+        if (kgrp == giver) {
+#pragma unroll
+            for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    const v4i v = acc[4 * half + mb][t];
+                    *(int4*)(xch + ((mb * 4 + t) * 256 + slot) * 4) = make_int4(v[0], v[1], v[2], v[3]);
+                }
+        }
+        __syncthreads();
+        if (kgrp != giver) {
+#pragma unroll
+            for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    const int4 v = *(const int4*)(xch + ((mb * 4 + t) * 256 + slot) * 4);
+                    acc[4 * half + mb][t] += v4i{v.x, v.y, v.z, v.w};
+                }
+        }
+        __syncthreads();
+    }
 }
 
 // TAIL = false: K is a multiple of the 128-wide stage and the main loop is branch free.
@@ -460,37 +498,7 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     EpiOperands epi_ops;
     load_epi_operands(p, m0, 4 * kgrp, g, ncol, col_ok, epi_ops);
 
-    // ---- add the two K halves: waves (wn, 0) and (wn, 1) hold partial sums of the same
-    // outputs.  K half 1 hands over row blocks 0..3, K half 0 hands over row blocks 4..7;
-    // word (q, wn, lane) of the exchange buffer is register q of that lane.
-    {
-        int32_t* xch = (int32_t*)lds;
-        const int slot = wn * 64 + lane;
-#pragma unroll
-        for (int half = 0; half < 2; half++) {
-            const int giver = 1 - half;  // K half that hands over row blocks 4*half .. 4*half+3
-            if (kgrp == giver) {
-#pragma unroll
-                for (int mb = 0; mb < 4; mb++)
-#pragma unroll
-                    for (int t = 0; t < 4; t++) {
-                        const v4i v = acc[4 * half + mb][t];
-                        *(int4*)(xch + ((mb * 4 + t) * 256 + slot) * 4) = make_int4(v[0], v[1], v[2], v[3]);
-                    }
-            }
-            __syncthreads();
-            if (kgrp != giver) {
-#pragma unroll
-                for (int mb = 0; mb < 4; mb++)
-#pragma unroll
-                    for (int t = 0; t < 4; t++) {
-                        const int4 v = *(const int4*)(xch + ((mb * 4 + t) * 256 + slot) * 4);
-                        acc[4 * half + mb][t] += v4i{v.x, v.y, v.z, v.w};
-                    }
-            }
-            __syncthreads();
-        }
-    }
+    exchange_k_halves(acc, lds, wn, kgrp, lane);
 
     // ---- epilogue: K half h finishes row blocks 4h .. 4h+3; lane (j, g) holds rows
     // 16mb + 4g + r, columns ncol .. ncol+3 -------------------------------------------
@@ -498,6 +506,7 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     if (kgrp == 0) gemm_epilogue_dt<0>(p, acc, m0, g, ncol, epi_ops);  // wave-uniform branch
     else gemm_epilogue_dt<4>(p, acc, m0, g, ncol, epi_ops);
 }
+
 
 // the same kernel on the decode-tiled weight copy (256-byte aligned, below 4 GiB: checked by the caller)
 bool gemm_i8_supported_tiled(int64_t N, int64_t K, const void* Q) {
