@@ -82,6 +82,20 @@ def test_single_row_fp16_variants(oracle):
             assert torch.equal(_C.ternary_linear_packed_forward(xd, pd, scale.cuda(), bias.cuda(), k).cpu(), expect)
     finally:
         os.environ.pop("BITTORCH_PLANES_NACC", None)
+    # one matrix through the contiguous-walk kernel (what a very wide layer takes by itself), residual included
+    try:
+        os.environ["BITTORCH_GROUP_WALK"] = "1"
+        for (n2, k2) in ((4096, 4096), (96, 2560), (1000, 1536), (20, 3600)):
+            x2, packed2, scale2, bias2 = _setup(n2, k2, seed=n2 + k2 + 1)
+            tiled2 = _C.retile_weights(packed2.cuda(), k2)
+            expect2 = _expect(oracle, x2, packed2, scale2, bias2, k2)
+            got2 = _C.ternary_linear_tiled_forward(x2.cuda(), tiled2, scale2.cuda(), bias2.cuda(), k2, n2)
+            assert torch.equal(got2.cpu(), expect2), (n2, k2)
+            res2 = seeded_acts(1, n2, seed=5, dtype=torch.float16)
+            got2 = _C.ternary_linear_tiled_forward(x2.cuda(), tiled2, scale2.cuda(), bias2.cuda(), k2, n2, residual=res2.cuda())
+            assert torch.equal(got2.cpu(), expect2 + res2), (n2, k2)
+    finally:
+        os.environ.pop("BITTORCH_GROUP_WALK", None)
     # ties of the final rounding and the largest magnitudes: all-ones weights, crafted activations
     from bittorch_amd.quant import pack_ternary_transposed
     ones = pack_ternary_transposed(torch.ones(16, 16, dtype=torch.int8))[0]
