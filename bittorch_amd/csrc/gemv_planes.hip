@@ -503,6 +503,9 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_chunk_kernel(PlaneParams p
             }
         }
     };
+    // the first unit's slice of x is requested ahead of the weights (loads return in order, and it is needed first)
+    const int xk = (wave * SPW * 8 + lane) * 8;
+    uint4 x_first = *(const uint4*)((const uint16_t*)(tab ? p.X_tab[pf_u] : p.X) + min(xk, (int)p.K - 8));
 #pragma unroll
     for (int i = 0; i < TB; i++) request(raw[i]);
 
@@ -520,8 +523,9 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_chunk_kernel(PlaneParams p
         {
             const uint16_t* xrow = (const uint16_t*)(tab ? p.X_tab[u] : p.X);
             const int c = lane;                               // chunk of eight values (SPW * 8 <= 64 chunks)
-            const int k = (wave * SPW * 8 + c) * 8;
-            uint4 v = *(const uint4*)(xrow + min(k, (int)p.K - 8));
+            const int k = xk;
+            uint4 v = x_first;
+            if (t0 != t_begin) v = *(const uint4*)(xrow + min(k, (int)p.K - 8));  // uniform
             v = zero_unless4(v, k < (int)p.K && c < SPW * 8);
             const bool bad = park_chunk(planes, c, v, lane, c < SPW * 8);
             const bool wave_bad = __builtin_amdgcn_ballot_w64(bad) != 0ull;
@@ -535,6 +539,16 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_chunk_kernel(PlaneParams p
         const int64_t u_stop = (unit_end < t_end) ? unit_end : t_end;
         for (int64_t c0 = t0; c0 < u_stop; c0 += CH_EB) {
             const int ntiles = (int)((u_stop - c0 < CH_EB) ? u_stop - c0 : CH_EB);  // a multiple of TB
+            // this thread's output column of the chunk: its epilogue operands are requested now, a chunk ahead of their use
+            const int tl = tid >> 4, jj = tid & 15;
+            const int64_t n = (int64_t)(tile0 + (int)(c0 - t0) + tl) * 16 + jj;
+            const bool out_col = tl < ntiles && n < p.N;
+            const void* bias_u = tab ? (p.bias_tab ? p.bias_tab[u] : nullptr) : p.bias;
+            uint32_t pre_s = 0u, pre_b = 0u;
+            if (out_col) {
+                pre_s = load_bits_rt(tab ? p.scale_tab[u] : p.scale, p.scale_dtype, p.scale_bcast ? 0 : n);
+                if (bias_u) pre_b = load_bits_rt(bias_u, p.bias_dtype, n);
+            }
             for (int tb = 0; tb < ntiles; tb += TB) {
                 v4i acc[TB];
 #pragma unroll
@@ -562,25 +576,20 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_chunk_kernel(PlaneParams p
                 }
             }
             __syncthreads();  // every wave has added its share of this chunk
-            {
-                const int tl = tid >> 4, jj = tid & 15;
-                const int64_t n = (int64_t)(tile0 + (int)(c0 - t0) + tl) * 16 + jj;
-                if (tl < ntiles) {
-                    int32_t sums[PL_N];
+            if (tl < ntiles) {
+                int32_t sums[PL_N];
 #pragma unroll
-                    for (int r = 0; r < PL_N; r++) {
-                        sums[r] = accbuf[cur][tl][16 * r + jj];
-                        accbuf[cur][tl][16 * r + jj] = 0;
-                    }
-                    if (n < p.N) {
-                        uint32_t fl = 0u;
+                for (int r = 0; r < PL_N; r++) {
+                    sums[r] = accbuf[cur][tl][16 * r + jj];
+                    accbuf[cur][tl][16 * r + jj] = 0;
+                }
+                if (out_col) {
+                    uint32_t fl = 0u;
 #pragma unroll
-                        for (int w = 0; w < 8; w++) fl |= flags[u & 1][w];
-                        const void* bias_u = tab ? (p.bias_tab ? p.bias_tab[u] : nullptr) : p.bias;
-                        const float sc = load_elem_rt(tab ? p.scale_tab[u] : p.scale, p.scale_dtype, p.scale_bcast ? 0 : n);
-                        const float bs = bias_u ? load_elem_rt(bias_u, p.bias_dtype, n) : 0.0f;
-                        pl_store(tab ? p.Y_tab[u] : p.Y, tab ? nullptr : p.residual, n, planes_to_f32(sums), sc, bs, fl != 0u);
-                    }
+                    for (int w = 0; w < 8; w++) fl |= flags[u & 1][w];
+                    const float sc = bits_to_f32_rt(pre_s, p.scale_dtype);
+                    const float bs = bias_u ? bits_to_f32_rt(pre_b, p.bias_dtype) : 0.0f;
+                    pl_store(tab ? p.Y_tab[u] : p.Y, tab ? nullptr : p.residual, n, planes_to_f32(sums), sc, bs, fl != 0u);
                 }
             }
             cur ^= 1;

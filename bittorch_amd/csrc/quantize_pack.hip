@@ -157,8 +157,10 @@ static int launch_fast_rows(const void* W, int64_t N, int64_t K, float tf, float
     int rpw = 0;
     if (const char* env = getenv("BITTORCH_QP_RPW")) rpw = atoi(env);
     if (rpw != 1 && rpw != 2 && rpw != 4) {
+        // (workgroups of 8 waves run two to a compute unit: at least 640 of them, so that both places stay filled)
+        const int64_t min_tiles = (WAVES == 8 && ITERS <= 16) ? 640 : 320;
         rpw = 4;
-        while (rpw > MIN_RPW && (N % (WAVES * rpw) != 0 || N / (WAVES * rpw) < 320)) rpw >>= 1;
+        while (rpw > MIN_RPW && (N % (WAVES * rpw) != 0 || N / (WAVES * rpw) < min_tiles)) rpw >>= 1;
     }
     if (rpw < MIN_RPW) rpw = MIN_RPW;
     if (N % (WAVES * rpw) != 0 || (size_t)(K / 4) * (WAVES * rpw + 4) > 150 * 1024) return 0;
@@ -188,6 +190,11 @@ static int try_launch_fast(const void* W, int64_t N, int64_t K, float tf, float 
     if (chunks <= IT) return launch_fast_rows<DT, IT, WV>(W, N, K, tf, clamp_min, per_channel, packed_T, scale, st, rc)
     BT_QF(4, 16);
     BT_QF(8, 16);
+    // 2048 < K <= 4096 and many rows: workgroups of 8 waves (16 rows), two per compute unit, so that one loads while the
+    // other encodes and stores, and the last round is cut finer (11008 x 4096: 34.9 against 40.0 us; 4096 x 4096, one
+    // workgroup per compute unit either way, stays on 16 waves: 15.4 against 16.4 us)
+    if (chunks > 8 && chunks <= 16 && N >= 6144 && N % 16 == 0)
+        return launch_fast_rows<DT, 16, 8>(W, N, K, tf, clamp_min, per_channel, packed_T, scale, st, rc);
     BT_QF(16, 16);
     BT_QF(24, 8);
     BT_QF(32, 8);
