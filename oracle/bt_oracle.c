@@ -250,6 +250,29 @@ void bto_linear_packed(const float* X, const uint8_t* W_T, const float* scale,
     }
 }
 
+/* The same with the epilogue as one fused multiply-add, acc * s + b rounded once: what a compiler that contracts
+ * floating-point expressions (nvcc's default for ternary_gemm_production.cu:139-141) makes of the reference's source
+ * line.  The library and bto_linear_packed round the product first (the reading of the line as written); this variant
+ * exists so that the tests can bound the distance between the two readings: at most one unit in the last place of
+ * the fp32 result. */
+void bto_linear_packed_fused_epilogue(const float* X, const uint8_t* W_T, const float* scale,
+                                      int64_t scale_len, const float* bias, float* Y, int64_t B,
+                                      int64_t N, int64_t K) {
+#pragma omp parallel for schedule(static)
+    for (int64_t n = 0; n < N; n++) {
+        const float s = scale[scale_len == 1 ? 0 : n];
+        const float bv = bias ? bias[n] : 0.0f;
+        for (int64_t b = 0; b < B; b++) {
+            float acc = 0.0f;
+            for (int64_t k = 0; k < K; k++) {
+                int w = decode2((W_T[(k / 4) * N + n] >> (2 * (k % 4))) & 3u);
+                acc += X[b * K + k] * (float)w;
+            }
+            Y[b * N + n] = fmaf(acc, s, bv);
+        }
+    }
+}
+
 /* Same contraction in float64 throughout: the high-precision truth that the
  * tolerance tests measure both the oracle and the kernels against. */
 void bto_linear_packed_f64(const float* X, const uint8_t* W_T, const float* scale,

@@ -50,6 +50,7 @@ def lib() -> ctypes.CDLL:
             getattr(_lib, name).argtypes = [_vp, _i64, _i64, _vp]
         _lib.bto_linear_packed.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64]
         _lib.bto_linear_packed_f64.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64]
+        _lib.bto_linear_packed_fused_epilogue.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64]
         _lib.bto_linear_unpacked.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64]
         _lib.bto_linear_packed_exact_f16.restype = ctypes.c_int
         _lib.bto_linear_packed_exact_f16.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64]
@@ -156,8 +157,10 @@ def _lin_args(x, w, scale, bias):
     return x, scale, bias
 
 
-def linear_packed(x, w_packed_t, scale, in_features: int, bias=None, f64: bool = False) -> np.ndarray:
-    """fp32-accumulate packed linear (or the float64 truth with ``f64=True``)."""
+def linear_packed(x, w_packed_t, scale, in_features: int, bias=None, f64: bool = False,
+                  fused_epilogue: bool = False) -> np.ndarray:
+    """fp32-accumulate packed linear (or the float64 truth with ``f64=True``); ``fused_epilogue`` rounds
+    ``acc * scale + bias`` once (a contracting compiler's reading of the reference's source line)."""
     x, scale, bias = _lin_args(x, w_packed_t, scale, bias)
     w = np.ascontiguousarray(np.asarray(w_packed_t, dtype=np.uint8))
     b, k = x.shape
@@ -165,7 +168,7 @@ def linear_packed(x, w_packed_t, scale, in_features: int, bias=None, f64: bool =
     n = w.shape[1]
     assert scale.size in (1, n)
     y = np.empty((b, n), dtype=np.float64 if f64 else np.float32)
-    fn = lib().bto_linear_packed_f64 if f64 else lib().bto_linear_packed
+    fn = lib().bto_linear_packed_f64 if f64 else (lib().bto_linear_packed_fused_epilogue if fused_epilogue else lib().bto_linear_packed)
     fn(_p(x), _p(w), _p(scale), scale.size, _p(bias), _p(y), b, n, k)
     return y
 

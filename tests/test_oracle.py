@@ -419,3 +419,31 @@ def test_codec_and_quantizer_properties_over_random_shapes(oracle):
             assert not np.any(packed[:, -1] >> (2 * (k % 4)))  # padding slots hold code 0
 
     run()
+
+
+def test_epilogue_as_written_and_contracted_differ_by_one_ulp_at_most(oracle):
+    """The reference's epilogue line `acc * s + b_val` (csrc/kernels/ternary_gemm_production.cu:139-141) is compiled by
+    nvcc with floating-point contraction on by default, i.e. possibly as one fused multiply-add; the oracle and the
+    library round the product first.  Both readings are computed here: they differ in a minority of the outputs, and
+    never by more than one unit in the last place at the magnitude of the product (its rounding error, half a unit, is all
+    that separates the two before the final rounding)."""
+    rng = np.random.default_rng(7)
+    n, k, b = 257, 512, 5
+    w = rng.integers(-1, 2, size=(n, k)).astype(np.int8)
+    packed, _ = oracle.pack_ternary_transposed(w)
+    x = rng.standard_normal((b, k)).astype(np.float32)
+    scale = (rng.random(n) * 0.05 + 0.01).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    y0 = oracle.linear_packed(x, packed, scale, k, bias)
+    y1 = oracle.linear_packed(x, packed, scale, k, bias, fused_epilogue=True)
+    differing = int((y0 != y1).sum())
+    assert 0 < differing < y0.size // 2
+    # the unit: the spacing of fp32 numbers at the larger of product and sum (where the sum cancels below the product, one
+    # unit of the product is several of the sum)
+    prod = np.abs(y0.astype(np.float64) - bias)
+    ulp = np.spacing(np.maximum(prod, np.abs(y0)).astype(np.float32))
+    assert float((np.abs(y0.astype(np.float64) - y1) / ulp).max()) <= 1.0
+    # without a bias the two readings are the same operation
+    z0 = oracle.linear_packed(x, packed, scale, k, None)
+    z1 = oracle.linear_packed(x, packed, scale, k, None, fused_epilogue=True)
+    np.testing.assert_array_equal(z0, z1)
