@@ -254,8 +254,10 @@ int bt_ternary_gemm_i8_tiled(const int8_t* Q, int q_layout, const float* s_x, co
  *   Y_tab[u] [N] = X_tab[u] [K] (fp16) x W_tiled_tab[u] (decode-tiled copy of a W_T [ceil(K/4), N]) * scale + bias
  * exactly as a single bt_ternary_linear_tiled_forward call on one row would (bit-identical outputs).  A
  * 4 MiB weight matrix takes less time to stream than a kernel takes to start and drain; this entry point
- * pays launch, set-up and drain once for G matrices: persistent workgroups walk (unit, column slab)
- * items and keep their weight loads running from one item into the next.
+ * pays launch, set-up and drain once for G matrices: persistent workgroups each read a contiguous run
+ * of the (unit, 16-column tile) sequence front to back, their waves splitting K (1040 <= K <= 4096 and
+ * at least 16 tiles per workgroup; other shapes: (unit, column slab) items, a wave per tile column),
+ * and keep their weight loads running from one unit into the next.
  *   The five tables are DEVICE arrays of G device pointers, caller-owned (bias_tab may be NULL: no
  *   bias; its entries may not be NULL otherwise).  Every unit has the same N, K, scale length
  *   (N, or 1 = per-tensor) and element types.  x_dtype must be BT_F16, Y is fp16; K % 16 == 0, K <= 10240;
