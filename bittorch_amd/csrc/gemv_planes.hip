@@ -19,14 +19,18 @@
 // {-1, 0, +1} (9 VALU operations per 16 weights, against 24 for the 16-bit decode); the int32
 // accumulators of the six rows are recombined in 64-bit integer arithmetic at the end.
 //
-// Two kernels share the arithmetic:
+// Three kernels share the arithmetic:
 //   gemv_planes_kernel        one weight matrix per launch; a workgroup owns a tile of 16 * NACC columns over the
 //                             whole of K and its waves split K (deterministic integer sum through LDS).
-//   gemv_planes_group_kernel  G independent units (own x, W, scale, bias, y; pointer tables in device
-//                             memory) in ONE launch: persistent workgroups walk (unit, column slab) items, a
-//                             wave owns 16 * NACC columns over the whole of K (no reduction, no barrier inside an
-//                             item) and keeps its weight loads running across item boundaries, so that the launch,
-//                             set-up and drain of a 4 MiB GEMV are paid once per launch instead of once per matrix.
+//   gemv_planes_chunk_kernel  G independent units (own x, W, scale, bias, y; pointer tables in device memory) in ONE
+//                             launch, or one very wide matrix: persistent workgroups each read a contiguous run of
+//                             the (unit, 16-column tile) sequence front to back, their waves splitting K, so that
+//                             the launch, set-up and drain of a 4 MiB GEMV are paid once per launch instead of once
+//                             per matrix and the weights arrive in the order the memory system streams fastest.
+//   gemv_planes_group_kernel  the grouped launch for the shapes the kernel above does not take (long K, few tiles per
+//                             workgroup): (unit, column slab) items, a wave owns 16 * NACC columns over the whole of K
+//                             (no reduction, no barrier inside an item) and keeps its weight loads running across
+//                             item boundaries.
 #include <cstdlib>
 
 #include "row_math.h"
