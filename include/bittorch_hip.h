@@ -144,6 +144,8 @@ int bt_act_quant_i8_layout(const void* X, int x_dtype, int64_t B, int64_t K, int
  *   Q [B,K] int8, s_x [B] fp32, W_T [ceil(K/4),N] uint8, Y [B,N] y_dtype.
  *   acc_out: optional [B,N] int32 copy of the raw accumulators (may be NULL).
  *   workspace: at least bt_gemm_i8_workspace_bytes(B,N,K) bytes (currently 0: may be NULL).
+ *   K <= 132096 (the int8 entry points all refuse a longer K: 127*127*K must fit the int32 accumulators and
+ *   127*K the 24 significand bits of the accumulator's conversion to fp32).
  */
 size_t bt_gemm_i8_workspace_bytes(int64_t B, int64_t N, int64_t K);
 int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const void* scale,
