@@ -227,3 +227,43 @@ def test_grouped_launch_argument_errors():
     assert lib.bt_ternary_gemv_grouped(p, 1, p, p, 0, 5, None, 1, p, 8, 16, 16, None) == -1
     assert "scale" in _lib.last_error()
     assert lib.bt_ternary_gemv_grouped(p, 1, p, p, 0, 16, None, 1, p, 0, 16, 16, None) == -1
+
+
+_grp_rng = np.random.default_rng(977)
+_GROUP_CASES = [(int(_grp_rng.integers(1, 40)), int(_grp_rng.integers(1, 80)) * 4,
+                 int(_grp_rng.integers(65, 257)) * 16, bool(_grp_rng.integers(0, 2)), bool(_grp_rng.integers(0, 2)), i)
+                for i in range(24)]
+
+
+@pytest.mark.parametrize("g,n,k,per_tensor,bias,seed", _GROUP_CASES)
+def test_grouped_launch_random_shapes(oracle, g, n, k, per_tensor, bias, seed):
+    """Seeded random G, N (any multiple of 4) and K (1040 .. 4096, the range of the contiguous-walk kernel), units
+    drawn from three weight matrices and three activation rows: the walk kernel where the shape allows it and the
+    one-stream-per-wave kernel both equal the single calls, and those the oracle."""
+    import os
+    from bittorch_amd import _C
+    announce("grouped gemv random", g, n, k, per_tensor, bias, seed)
+    base = [_setup(n, k, seed=1000 + 7 * seed + s, per_tensor=per_tensor, bias=bias, wide=(s == 1)) for s in range(3)]
+    xs_ = [b[0].cuda() for b in base]
+    tiles_ = [_C.retile_weights(b[1].cuda(), k) for b in base]
+    units = [(int(_grp_rng.integers(0, 3)), int(_grp_rng.integers(0, 3))) for _ in range(g)]
+    xs = [xs_[a] for a, _ in units]
+    tiles = [tiles_[w] for _, w in units]
+    scales = [base[w][2].cuda() for _, w in units]
+    biases = [base[w][3].cuda() for _, w in units] if bias else None
+    singles = {}
+    for (a, w) in set(units):
+        singles[(a, w)] = _C.ternary_linear_tiled_forward(xs_[a], tiles_[w], base[w][2].cuda(),
+                                                          base[w][3].cuda() if bias else None, k, n)
+    a0, w0 = units[0]
+    assert torch.equal(singles[(a0, w0)].cpu(), _expect(oracle, base[a0][0], base[w0][1], base[w0][2], base[w0][3], k))
+    try:
+        for walk in ("1", "0"):
+            os.environ["BITTORCH_GROUP_WALK"] = walk
+            ys = [torch.full((1, n), float("nan"), dtype=torch.float16, device="cuda") for _ in range(g)]
+            _C.ternary_gemv_grouped(*_tables(_C, xs, tiles, scales, biases, ys), k, n, scale_len=1 if per_tensor else n)
+            torch.cuda.synchronize()
+            for u in range(g):
+                assert torch.equal(ys[u], singles[units[u]]), (u, walk)
+    finally:
+        os.environ.pop("BITTORCH_GROUP_WALK", None)
