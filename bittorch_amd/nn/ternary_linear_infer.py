@@ -85,6 +85,13 @@ class TernaryLinearInference(nn.Module):
         fresh tensor rebuilt from the tiled copy (what the layer holds does not change)."""
         return self._buffers["weight_packed"] if self._has_row_major() else self._untiled()
 
+    def invalidate_packed_cache(self) -> "TernaryLinearInference":
+        """Forget the decode-tiled copy when the layer also holds ``weight_packed``, so that the next call rebuilds it:
+        for code that wrote ``weight_packed`` through ``.data`` (a write the tensor's version counter does not see)."""
+        if self._has_row_major():
+            self._tiled, self._tiled_key = None, None
+        return self
+
     def drop_row_major(self) -> "TernaryLinearInference":
         """Back to one resident copy: build the tiled copy if need be and release the row-major buffer."""
         self.keep_row_major = False

@@ -261,6 +261,17 @@ def test_module_holds_one_copy_of_its_weights(oracle):
     np.testing.assert_allclose(f32np(y32), f32np(y_gen), rtol=1e-4, atol=1e-4)
 
 
+def test_module_invalidate_after_a_write_through_data(oracle):
+    a = _layer(oracle, 64, 64, seed=3)
+    x = seeded_acts(1, 64, dtype=torch.float16).cuda()
+    a(x)
+    wp = a.weight_packed                       # brings the buffer back; the layer holds both copies now
+    a(x)
+    wp.data.zero_()                            # not seen by the version counter
+    a.invalidate_packed_cache()
+    assert torch.equal(a(x).float(), a.bias.half().float().expand(1, -1))
+
+
 def test_module_rebuilds_tiled_copy_when_weights_change(oracle):
     a = _layer(oracle, 64, 64, seed=1)
     x = seeded_acts(1, 64, dtype=torch.float16).cuda()
