@@ -115,6 +115,39 @@ def probe_mfma_int8(torch, device, blocks=2048, iters=4096, random_operands=0, r
     return ops.value
 
 
+def probe_hbm_read(torch, device, nbytes=512 << 20):
+    """GB/s of the benchmark's read-only probe kernel (bench_mfma_probe.so) over `nbytes` of device memory, for its
+    three address patterns; each figure the median of 5 timed runs of 4 launches."""
+    import ctypes
+    global _probe_lib
+    if _probe_lib is None:
+        _probe_lib = ctypes.CDLL(os.path.join(ROOT, "bench_mfma_probe.so"))
+    fn = _probe_lib.bench_probe_hbm_read
+    fn.restype = ctypes.c_int
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    buf = torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=device)
+    out = torch.zeros(8, dtype=torch.int32, device=device)
+    st = torch.cuda.current_stream(device).cuda_stream
+    res = {}
+    for name, pattern in (("grid_stride", 0), ("contiguous_per_workgroup", 1), ("contiguous_per_workgroup_nontemporal", 2)):
+        assert fn(buf.data_ptr(), nbytes, pattern, out.data_ptr(), st) == 0  # warm
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(5):
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(4):
+                fn(buf.data_ptr(), nbytes, pattern, out.data_ptr(), st)
+            e1.record()
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1) / 4)
+        ts.sort()
+        res[name] = round(nbytes / (ts[2] * 1e-3) / 1e9, 1)
+    del buf
+    return res
+
+
 class Config5:
     """Config 5: a 2B-parameter BitNet-b1.58-like stack.  q/k/v/o/gate/up/down are TernaryLinear
     (random N(0,0.02) masters, no bias); RMSNorm, rotary-free causal SDPA and the embedding stay in
@@ -578,6 +611,14 @@ def main():
             "note": "2048 workgroups x 8 waves of back-to-back v_mfma_i32_16x16x64_i8, no memory traffic in the loop; "
                     "the clock is what workgroup 0 measures in its loop (cycle counter against the 100 MHz real-time "
                     "counter): the 5 POPS peak assumes 2.4 GHz",
+        }
+        # what a pure reader gets from the memory system on this box, next to the headline
+        read_probe = probe_hbm_read(torch, dev)
+        extra["hbm_read_only_probe"] = {
+            "GBps": read_probe,
+            "headline_frac_of_best_pattern": round(out["value"] / max(read_probe.values()), 4),
+            "note": "512 MiB read by 512 workgroups of 512 threads (grid-stride: 4096 of 256), xor-reduced; the grouped "
+                    "GEMV walks its weights in the third pattern",
         }
         for key in list(extra):
             if key.startswith("prefill_int8"):

@@ -1,5 +1,6 @@
-// Measurement aid of bench.py (built into bench_mfma_probe.so, not part of libbittorch_hip.so or its ABI):
-// the int8 MFMA rate the chip sustains when nothing else is in the way.
+// Measurement aids of bench.py (built into bench_mfma_probe.so, not part of libbittorch_hip.so or its ABI):
+// the int8 MFMA rate the chip sustains when nothing else is in the way, and (at the end of the file) the rate at which
+// the memory system feeds a pure reader.
 // Every wave issues back-to-back v_mfma_i32_16x16x64_i8 on eight independent accumulators
 // held in registers; no memory traffic inside the loop.  The prefill GEMM's TOPS are
 // reported against this figure as well as against the nominal peak.
@@ -102,5 +103,57 @@ extern "C" int bench_probe_mfma_i8(int blocks, int iters, int random_operands, i
                            random_operands, out);
     // 8 waves per block, 8 MFMAs per iteration, 2*16*16*64 operations each
     if (ops_per_launch) *ops_per_launch = (double)blocks * 8.0 * (double)iters * 8.0 * 32768.0;
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+// ---- what the memory system delivers to a pure reader ----------------------------------------------------------------
+// A read-only kernel over `bytes` of device memory, xor-reduced so that the loads stay alive; three address patterns:
+//   0  grid-stride 16-byte loads over the whole buffer (the textbook streaming loop);
+//   1  every workgroup reads its own contiguous share front to back, a wave 2 KiB (8 loads of 4 bytes per lane) at a time;
+//   2  the same with the non-temporal hint on the loads.
+// The grouped GEMV walks its weights in pattern 2; its GB/s are reported against this figure as well as against the
+// nominal 8 TB/s.
+namespace {
+__global__ __launch_bounds__(256) void read_probe_grid(const uint4* __restrict__ p, size_t n, int* out) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * 256;
+    uint32_t a = 0;
+    for (; i + 7 * stride < n; i += 8 * stride) {
+        uint4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = p[i + u * stride];
+#pragma unroll
+        for (int u = 0; u < 8; u++) a ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    if (a == 0x12345678u) out[1] = (int)a;
+}
+template <bool NT>
+__global__ __launch_bounds__(512) void read_probe_chunk(const uint32_t* __restrict__ p, size_t ndw, int* out) {
+    const size_t per_wg = ndw / gridDim.x;  // dwords
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t* base = p + (size_t)blockIdx.x * per_wg;
+    uint32_t a = 0;
+    constexpr int U = 8, BLK = U * 64;  // dwords per wave block
+    for (size_t blk = wave; (blk + 1) * BLK <= per_wg; blk += 8) {
+        uint32_t v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t* q = base + blk * BLK + (size_t)u * 64 + lane;
+            v[u] = NT ? __builtin_nontemporal_load(q) : *q;
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) a ^= v[u];
+    }
+    if (a == 0x12345678u) out[1] = (int)a;
+}
+}  // namespace
+
+// One launch of the read probe over `bytes` (a multiple of 1 MiB) at `buf`; pattern as above.  Returns 0 / -1.
+extern "C" int bench_probe_hbm_read(const void* buf, size_t bytes, int pattern, int* out, void* stream) {
+    if (!buf || !out || bytes < (1u << 20) || bytes % (1u << 20) != 0) return -1;
+    hipStream_t st = (hipStream_t)stream;
+    if (pattern == 0) hipLaunchKernelGGL(read_probe_grid, dim3(4096), dim3(256), 0, st, (const uint4*)buf, bytes / 16, out);
+    else if (pattern == 1) hipLaunchKernelGGL(read_probe_chunk<false>, dim3(512), dim3(512), 0, st, (const uint32_t*)buf, bytes / 4, out);
+    else hipLaunchKernelGGL(read_probe_chunk<true>, dim3(512), dim3(512), 0, st, (const uint32_t*)buf, bytes / 4, out);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
