@@ -517,6 +517,25 @@ def main():
                               "frac_of_hbm_peak": round(gg * weight_bytes / (us_g * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
         extra["grouped_gemv_by_units_per_launch"] = by_g
 
+        # the same launch on bf16 rows (each row scaled by its own largest exponent, summed as integers)
+        xs_bf = [t.bfloat16() for t in xs[:2 * G]]
+        bs_bf = [t.bfloat16() for t in biases[:2 * G]]
+        ys_bf = [torch.empty(1, N, dtype=torch.bfloat16, device=dev) for _ in range(2 * G)]
+        tb_bf = []
+        for s0 in (0, G):
+            sl = slice(s0, s0 + G)
+            tb_bf.append((_C.pointer_table(xs_bf[sl]), tables[s0 // G][1], tables[s0 // G][2],
+                          _C.pointer_table(bs_bf[sl]), _C.pointer_table(ys_bf[sl])))
+        _, ev_bf = graph_time(lambda i: _C.ternary_gemv_grouped(*tb_bf[i % 2], K, N, scale_len=1,
+                                                                bias_dtype=torch.bfloat16, x_dtype=torch.bfloat16),
+                              args.steps, args.warmup, torch)
+        us_bf = ev_bf / args.steps * 1e3
+        extra["grouped_gemv_bf16_rows"] = {
+            "us_per_launch": round(us_bf, 2), "GBps": round(G * weight_bytes / (us_bf * 1e-6) / 1e9, 1),
+            "frac_of_hbm_peak": round(G * weight_bytes / (us_bf * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+            "note": f"G = {G} units per launch, bf16 rows, biases and outputs",
+        }
+
         def rand_packed(n, k, count):
             outp = []
             for _ in range(count):

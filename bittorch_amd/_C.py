@@ -343,11 +343,14 @@ def pointer_table(tensors) -> Tensor:
 
 def ternary_gemv_grouped(x_tab: Tensor, w_tiled_tab: Tensor, scale_tab: Tensor, bias_tab: Optional[Tensor],
                          y_tab: Tensor, in_features: int, out_features: int, scale_len: int = -1,
-                         scale_dtype: torch.dtype = torch.float32, bias_dtype: torch.dtype = torch.float16) -> None:
+                         scale_dtype: torch.dtype = torch.float32, bias_dtype: torch.dtype = torch.float16,
+                         x_dtype: torch.dtype = torch.float16) -> None:
     """``G`` independent decode GEMVs in one launch: unit ``u`` multiplies the fp16 row at ``x_tab[u]`` with the
     decode-tiled weights at ``w_tiled_tab[u]`` into the fp16 row at ``y_tab[u]``, exactly as
     :func:`ternary_linear_tiled_forward` would on that row (same bits).  The tables are int64 device tensors of
-    ``G`` device addresses (:func:`pointer_table`); nothing is allocated or returned."""
+    ``G`` device addresses (:func:`pointer_table`); nothing is allocated or returned.
+    ``x_dtype=torch.bfloat16``: bf16 rows and outputs (1040 <= K <= 4096, N a multiple of 32, of 64 for K <= 2048);
+    each row is scaled by its own largest exponent and summed exactly on the int8 matrix cores."""
     G = x_tab.numel()
     tabs = (x_tab, w_tiled_tab, scale_tab, y_tab) + (() if bias_tab is None else (bias_tab,))
     for t in tabs:
@@ -355,9 +358,10 @@ def ternary_gemv_grouped(x_tab: Tensor, w_tiled_tab: Tensor, scale_tab: Tensor, 
                "pointer tables must be contiguous int64 tensors of one length")
     _check(_all_cuda(*tabs), "All tensors must be CUDA")
     _check(scale_dtype in _DT and bias_dtype in _DT, "scale / bias dtype must be float32, float16 or bfloat16")
+    _check(x_dtype in (torch.float16, torch.bfloat16), "x_dtype must be float16 or bfloat16")
     with torch.cuda.device(x_tab.device):
         _status(_L.bt_ternary_gemv_grouped(
-            x_tab.data_ptr(), _DT[torch.float16], w_tiled_tab.data_ptr(), scale_tab.data_ptr(), _DT[scale_dtype],
+            x_tab.data_ptr(), _DT[x_dtype], w_tiled_tab.data_ptr(), scale_tab.data_ptr(), _DT[scale_dtype],
             out_features if scale_len < 0 else scale_len, _ptr(bias_tab), _DT[bias_dtype], y_tab.data_ptr(), G,
             out_features, in_features, _stream(x_tab)))
 

@@ -59,9 +59,12 @@ bool planes_supported(int x_dtype, int y_dtype, int64_t B, int64_t N, int64_t K,
                       int w_layout);
 int launch_planes(const void* X, const uint8_t* W, int w_layout, const Epilogue& epi, void* Y, int64_t N, int64_t K,
                   int epi_op, hipStream_t st);
-int launch_planes_group(const void* const* X_tab, const uint8_t* const* W_tab, const void* const* scale_tab, int scale_dtype,
-                        int scale_bcast, const void* const* bias_tab, int bias_dtype, void* const* Y_tab, int64_t G, int64_t N,
-                        int64_t K, hipStream_t st);
+int launch_planes_group(const void* const* X_tab, int x_dtype, const uint8_t* const* W_tab, const void* const* scale_tab,
+                        int scale_dtype, int scale_bcast, const void* const* bias_tab, int bias_dtype, void* const* Y_tab,
+                        int64_t G, int64_t N, int64_t K, hipStream_t st);
+bool planes_bf16_shape_ok(int64_t N, int64_t K);
+bool planes_bf16_wide(int64_t N, int64_t K);
+int launch_planes_bf16_wide(const void* X, const uint8_t* W, const Epilogue& epi, void* Y, int64_t N, int64_t K, hipStream_t st);
 bool gemm_i8_supported_tiled(int64_t N, int64_t K, const void* Q);
 int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_T, int w_layout, const Epilogue& epi,
                    void* Y, int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st);
@@ -226,6 +229,11 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         // one fp16 row: the exact GEMV on the int8 matrix cores
         if (planes_supported(x_dtype, x_dtype, B, N, K, X, W_T, Y, W_LAYOUT_TILED))
             return launch_planes(X, W_T, W_LAYOUT_TILED, epi, Y, N, K, epi_op, st);
+        // one bf16 row times a very wide matrix (a vocabulary projection): the same kernel family, the row scaled by
+        // its largest exponent
+        if (x_dtype == BT_BF16 && B == 1 && epi_op == 0 && ((uintptr_t)X) % 16 == 0 && !getenv("BITTORCH_NO_PLANES") &&
+            planes_bf16_wide(N, K))
+            return launch_planes_bf16_wide(X, W_T, epi, Y, N, K, st);
         if (x_dtype != BT_F32) {
             const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
             // tall batches: the tiled matrix-core GEMM reads the copy too (not with the SwiGLU output stage)
@@ -507,12 +515,17 @@ extern "C" int bt_ternary_gemv_grouped(const void* const* X_tab, int x_dtype, co
         set_error("%s: empty shape or too many units (G=%lld N=%lld K=%lld)", who, (long long)G, (long long)N, (long long)K);
         return BT_ERR_INVALID;
     }
-    if (x_dtype != BT_F16) {
-        set_error("%s: activations must be fp16 (dtype tag %d given)", who, x_dtype);
+    if (x_dtype != BT_F16 && x_dtype != BT_BF16) {
+        set_error("%s: activations must be fp16 or bf16 (dtype tag %d given)", who, x_dtype);
         return BT_ERR_INVALID;
     }
     if (K % 16 != 0 || K > 10240) {
         set_error("%s: K must be a multiple of 16 and at most 10240 (K=%lld)", who, (long long)K);
+        return BT_ERR_INVALID;
+    }
+    if (x_dtype == BT_BF16 && !planes_bf16_shape_ok(N, K)) {
+        set_error("%s: bf16 units need 1040 <= K <= 4096 and N a multiple of 32 (of 64 for K <= 2048) (N=%lld K=%lld)", who,
+                  (long long)N, (long long)K);
         return BT_ERR_INVALID;
     }
     if ((scale_len != N && scale_len != 1) || !valid_dtype(scale_dtype) || (bias_tab && !valid_dtype(bias_dtype))) {
@@ -523,7 +536,7 @@ extern "C" int bt_ternary_gemv_grouped(const void* const* X_tab, int x_dtype, co
         set_error("%s: a unit's tiled weights must stay below 4 GiB", who);
         return BT_ERR_INVALID;
     }
-    return launch_planes_group(X_tab, W_tiled_tab, scale_tab, scale_dtype, (scale_len == 1 && N != 1) ? 1 : 0, bias_tab,
+    return launch_planes_group(X_tab, x_dtype, W_tiled_tab, scale_tab, scale_dtype, (scale_len == 1 && N != 1) ? 1 : 0, bias_tab,
                                bias_dtype, Y_tab, G, N, K, (hipStream_t)stream);
 }
 

@@ -64,6 +64,7 @@ struct PlaneParams {
     int slabs;       // grouped launch: column slabs (8 waves x 16 * NACC columns) per unit
     int items;       // grouped launch: G * slabs
     int scale_dtype, bias_dtype, scale_bcast;
+    int x_dtype;     // BT_F16, or BT_BF16 (contiguous-walk kernel only)
 };
 
 // ---- fp16 -> six int8 digit planes ----------------------------------------------------------------
@@ -100,6 +101,58 @@ __device__ __forceinline__ bool f16x8_to_planes(const uint4 v, uint32_t (&lo)[PL
     return bad;
 }
 
+// bf16 activations: the exponent range of bf16 (2^-133 .. 2^127) does not fit a fixed-point word, so the row is
+// scaled by its own largest exponent.  With e1 = max(biased exponent, 1) and mag the 8-bit significand, a finite value
+// is mag * 2^(e1 - 134); emax = the largest e1 of the row; X = value * 2^(166 - emax) = mag * 2^(e1 - emax + 32), an
+// integer below 2^40 in magnitude for every element.  Elements more than 32 binades below the row's largest lose low
+// bits (rounded half up in magnitude; more than 40 binades below: 0) -- an error of at most 2^-41 of the largest
+// element each, far below what an fp32 accumulator carries; all others are represented exactly.
+// The sum S of the X is exact, and acc = RN_fp32(S) * 2^(emax - 166).
+__device__ __forceinline__ int bf16_e1(uint32_t h) {  // 0 for an infinity or a NaN (not part of the maximum)
+    const int e = (int)((h >> 7) & 255u);
+    return e == 255 ? 0 : (e ? e : 1);
+}
+__device__ __forceinline__ int bf16x8_max_e1(const uint4 v) {
+    const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+    int m = 0;
+#pragma unroll
+    for (int e = 0; e < 8; e++) m = max(m, bf16_e1((d[e >> 1] >> (16 * (e & 1))) & 0xffffu));
+    return m;
+}
+__device__ __forceinline__ bool bf16x8_to_planes(const uint4 v, int emax, uint32_t (&lo)[PL_N], uint32_t (&hi)[PL_N]) {
+    const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+    bool bad = false;
+#pragma unroll
+    for (int p = 0; p < PL_N; p++) lo[p] = hi[p] = 0u;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const uint32_t h = (d[e >> 1] >> (16 * (e & 1))) & 0xffffu;
+        const uint32_t ex = (h >> 7) & 255u, m = h & 0x7fu;
+        bad |= (ex == 255u);
+        const uint32_t mag = ex ? (m | 0x80u) : m;
+        const int sh = (int)(ex ? ex : 1u) - emax + 32;  // <= 32
+        uint64_t mg;
+        if (sh >= 0) mg = (uint64_t)mag << sh;
+        else if (sh >= -8) mg = (uint64_t)((mag + (1u << (-sh - 1))) >> (-sh));
+        else mg = 0;
+        const int64_t X = (h & 0x8000u) ? -(int64_t)mg : (int64_t)mg;
+        const uint32_t xl = (uint32_t)X, xh = (uint32_t)((uint64_t)X >> 32);
+        uint32_t dg[PL_N];
+        dg[0] = xl & 127u;
+        dg[1] = (xl >> 7) & 127u;
+        dg[2] = (xl >> 14) & 127u;
+        dg[3] = (xl >> 21) & 127u;
+        dg[4] = ((xl >> 28) | (xh << 4)) & 127u;
+        dg[5] = (xh >> 3) & 255u;
+#pragma unroll
+        for (int p = 0; p < PL_N; p++) {
+            if (e < 4) lo[p] |= dg[p] << (8 * e);
+            else hi[p] |= dg[p] << (8 * (e - 4));
+        }
+    }
+    return bad;
+}
+
 __device__ __forceinline__ uint4 zero_unless4(uint4 v, bool ok) {
     v.x = ok ? v.x : 0u; v.y = ok ? v.y : 0u; v.z = ok ? v.z : 0u; v.w = ok ? v.w : 0u;
     return v;
@@ -109,9 +162,12 @@ __device__ __forceinline__ uint4 zero_unless4(uint4 v, bool ok) {
 // the wave slice's) first 16-k group; even and odd lanes hold the two halves of one group and exchange bytes, so
 // every lane of a pair must call it (`write` = false for pairs outside the buffer).  v must already be zero for
 // chunks beyond K.
-__device__ __forceinline__ bool park_chunk(uint8_t* planes, int c, const uint4 v, int lane, bool write) {
+template <int XDT = BT_F16>
+__device__ __forceinline__ bool park_chunk(uint8_t* planes, int c, const uint4 v, int lane, bool write, int emax = 0) {
     uint32_t lo[PL_N], hi[PL_N];
-    const bool bad = f16x8_to_planes(v, lo, hi);
+    bool bad;
+    if constexpr (XDT == BT_BF16) bad = bf16x8_to_planes(v, emax, lo, hi);
+    else bad = f16x8_to_planes(v, lo, hi);
     uint8_t* dst = planes + (size_t)(c >> 1) * PL_GROUP + 8 * (c & 1);
 #pragma unroll
     for (int p = 0; p < PL_N; p++) {
@@ -134,20 +190,21 @@ __device__ __forceinline__ uint32_t pl_quad_transpose(uint32_t d, uint32_t sel_q
 }
 
 // the exact sum S (in units of 2^-24), correctly rounded to fp32 and scaled back
-__device__ __forceinline__ float fixed_to_f32(int64_t S) { return __builtin_ldexpf((float)S, -24); }
+__device__ __forceinline__ float fixed_to_f32(int64_t S, int exp2 = -24) { return __builtin_ldexpf((float)S, exp2); }
 // ... from its six plane sums
-__device__ __forceinline__ float planes_to_f32(const int32_t (&s)[PL_N]) {
+__device__ __forceinline__ float planes_to_f32(const int32_t (&s)[PL_N], int exp2 = -24) {
     int64_t S = 0;
 #pragma unroll
     for (int p = PL_N - 1; p >= 0; p--) S = S * 128 + (int64_t)s[p];
-    return fixed_to_f32(S);
+    return fixed_to_f32(S, exp2);
 }
 
+template <int XDT = BT_F16>
 __device__ __forceinline__ void pl_store(void* Y, const void* residual, int64_t n, float acc, float s, float b, bool bad) {
     float y = epi_float(acc, s, b);
     if (bad) y = __builtin_nanf("");
-    if (residual) y = add_residual(y, residual, BT_F16, n);
-    ((uint16_t*)Y)[n] = f32_to_f16_bits(y);
+    if (residual) y = add_residual(y, residual, XDT, n);
+    ((uint16_t*)Y)[n] = (XDT == BT_BF16) ? f32_to_bf16_bits(y) : f32_to_f16_bits(y);
 }
 
 // ---- one weight matrix per launch -------------------------------------------------------------------
@@ -458,11 +515,14 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_group_kernel(PlaneParams p
 // adding the next chunk into the other array.  TB tiles of loads are always in flight per wave, across chunk and
 // unit boundaries.  Integer sums: same bits as every other split of K.
 constexpr int CH_EB = 32;  // tiles per chunk (one output column per thread)
-template <int SPW, int TB>
+// XDT = BT_BF16: bf16 activations and outputs, the row scaled by its largest exponent (see bf16x8_to_planes): the waves
+// exchange the maxima of their slices through LDS (one more barrier per unit) before they convert.
+template <int SPW, int TB, int XDT = BT_F16>
 __global__ __launch_bounds__(512, 4) void gemv_planes_chunk_kernel(PlaneParams p) {
     static_assert(CH_EB % TB == 0, "chunks hold whole batches");
     __shared__ int32_t accbuf[2][CH_EB][PL_N * 16];
     __shared__ uint32_t flags[2][8];
+    __shared__ int emax_slot[2][8];
     __shared__ __attribute__((aligned(16))) uint8_t planes_all[8][SPW * 4 * PL_GROUP];
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
@@ -517,6 +577,7 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_chunk_kernel(PlaneParams p
     const uint8_t* a_src = planes + g * PL_GROUP + (j % PL_N) * 16;
     uint4 areg[SPW];
     int cur = 0;
+    int emax = 0;  // bf16: the current unit's largest exponent (every wave computes it)
     __syncthreads();  // accumulators cleared
 
     int64_t t0 = t_begin;
@@ -531,7 +592,20 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_chunk_kernel(PlaneParams p
             uint4 v = x_first;
             if (t0 != t_begin) v = *(const uint4*)(xrow + min(k, (int)p.K - 8));  // uniform
             v = zero_unless4(v, k < (int)p.K && c < SPW * 8);
-            const bool bad = park_chunk(planes, c, v, lane, c < SPW * 8);
+            if constexpr (XDT == BT_BF16) {
+                // the row's largest exponent: every wave's slice maximum meets the others' in LDS (the eight slices
+                // cover the row; two sets of slots, so a wave that runs ahead into the next unit disturbs nobody)
+                int m = bf16x8_max_e1(v);
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) m = max(m, __shfl_xor(m, off, 64));
+                if (lane == 0) emax_slot[u & 1][wave] = m;
+                __syncthreads();
+                m = emax_slot[u & 1][lane & 7];
+#pragma unroll
+                for (int off = 4; off > 0; off >>= 1) m = max(m, __shfl_xor(m, off, 64));
+                emax = m;
+            }
+            const bool bad = park_chunk<XDT>(planes, c, v, lane, c < SPW * 8, emax);
             const bool wave_bad = __builtin_amdgcn_ballot_w64(bad) != 0ull;
             if (lane == 0) flags[u & 1][wave] = wave_bad ? 1u : 0u;
             // (LDS accesses of one wave execute in order: the slice written above is visible to its own reads)
@@ -593,7 +667,8 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_chunk_kernel(PlaneParams p
                     for (int w = 0; w < 8; w++) fl |= flags[u & 1][w];
                     const float sc = bits_to_f32_rt(pre_s, p.scale_dtype);
                     const float bs = bias_u ? bits_to_f32_rt(pre_b, p.bias_dtype) : 0.0f;
-                    pl_store(tab ? p.Y_tab[u] : p.Y, tab ? nullptr : p.residual, n, planes_to_f32(sums), sc, bs, fl != 0u);
+                    const int exp2 = (XDT == BT_BF16) ? emax - 166 : -24;
+                    pl_store<XDT>(tab ? p.Y_tab[u] : p.Y, tab ? nullptr : p.residual, n, planes_to_f32(sums, exp2), sc, bs, fl != 0u);
                 }
             }
             cur ^= 1;
@@ -633,25 +708,38 @@ static int64_t resident_wgs() {
 // tiles, and at least `min_tiles_per_wg` tiles per resident workgroup (below that the per-chunk barrier and the one-off
 // conversion weigh more than the walk gains: G = 8 units of 4096 x 4096 10.5 against 11.7 us, G = 32 equal, G = 128
 // 92 against 85 us).  BITTORCH_GROUP_WALK=1 / =0 (tests, A/B runs): always / never.
+// (shape only: what the kernel can serve at all)
+static bool walk_shape_ok(int wsteps, int tiles16) {
+    const int spw = (int)ceil_div(wsteps, 8);
+    const int tb = (spw >= 5) ? 2 : 4;
+    return spw >= 3 && spw <= 8 && tiles16 % tb == 0;
+}
+template <int XDT>
+static void launch_walk_k(const PlaneParams& p, int spw, unsigned grid, hipStream_t st) {
+    switch (spw) {
+        case 3: hipLaunchKernelGGL((gemv_planes_chunk_kernel<3, 4, XDT>), dim3(grid), dim3(512), 0, st, p); break;
+        case 4: hipLaunchKernelGGL((gemv_planes_chunk_kernel<4, 4, XDT>), dim3(grid), dim3(512), 0, st, p); break;
+        case 5: hipLaunchKernelGGL((gemv_planes_chunk_kernel<5, 2, XDT>), dim3(grid), dim3(512), 0, st, p); break;
+        case 6: hipLaunchKernelGGL((gemv_planes_chunk_kernel<6, 2, XDT>), dim3(grid), dim3(512), 0, st, p); break;
+        case 7: hipLaunchKernelGGL((gemv_planes_chunk_kernel<7, 2, XDT>), dim3(grid), dim3(512), 0, st, p); break;
+        default: hipLaunchKernelGGL((gemv_planes_chunk_kernel<8, 2, XDT>), dim3(grid), dim3(512), 0, st, p); break;
+    }
+}
+// min_tiles_per_wg < 0: whenever the shape allows (bf16 units have no other kernel)
 static bool launch_walk(PlaneParams p, int64_t G, int64_t wgs, int min_tiles_per_wg, hipStream_t st) {
     const int spw = (int)ceil_div(p.wsteps, 8);
     const int tb = (spw >= 5) ? 2 : 4;
     const int64_t total = G * p.tiles16;
     const char* force = getenv("BITTORCH_GROUP_WALK");
-    const bool want = force ? (force[0] == '1') : (total >= min_tiles_per_wg * wgs);
-    if (spw < 3 || spw > 8 || p.tiles16 % tb != 0 || !want) return false;
+    bool want = force ? (force[0] == '1') : (total >= min_tiles_per_wg * wgs);
+    if (min_tiles_per_wg < 0) want = true;
+    if (!walk_shape_ok(p.wsteps, p.tiles16) || !want) return false;
     const int64_t tpw = ceil_div(ceil_div(total, wgs), tb) * tb;
     p.G = (int)G;
     p.slabs = (int)tpw;  // tiles per workgroup
     const unsigned grid = (unsigned)ceil_div(total, tpw);
-    switch (spw) {
-        case 3: hipLaunchKernelGGL((gemv_planes_chunk_kernel<3, 4>), dim3(grid), dim3(512), 0, st, p); break;
-        case 4: hipLaunchKernelGGL((gemv_planes_chunk_kernel<4, 4>), dim3(grid), dim3(512), 0, st, p); break;
-        case 5: hipLaunchKernelGGL((gemv_planes_chunk_kernel<5, 2>), dim3(grid), dim3(512), 0, st, p); break;
-        case 6: hipLaunchKernelGGL((gemv_planes_chunk_kernel<6, 2>), dim3(grid), dim3(512), 0, st, p); break;
-        case 7: hipLaunchKernelGGL((gemv_planes_chunk_kernel<7, 2>), dim3(grid), dim3(512), 0, st, p); break;
-        default: hipLaunchKernelGGL((gemv_planes_chunk_kernel<8, 2>), dim3(grid), dim3(512), 0, st, p); break;
-    }
+    if (p.x_dtype == BT_BF16) launch_walk_k<BT_BF16>(p, spw, grid, st);
+    else launch_walk_k<BT_F16>(p, spw, grid, st);
     return true;
 }
 
@@ -680,6 +768,7 @@ int launch_planes(const void* X, const uint8_t* W, int w_layout, const Epilogue&
     PlaneParams p = {};
     p.X = X; p.W = W; p.scale = epi.scale; p.bias = epi.bias; p.residual = epi.residual; p.Y = Y;
     p.scale_dtype = epi.scale_dtype; p.bias_dtype = epi.bias_dtype; p.scale_bcast = epi.scale_bcast;
+    p.x_dtype = BT_F16;
     p.N = N; p.K = K; p.Kb = ceil_div(K, 4);
     p.G = 1;
     p.wsteps = (int)ceil_div(p.Kb, 16);
@@ -720,6 +809,10 @@ int launch_planes(const void* X, const uint8_t* W, int w_layout, const Epilogue&
 
 static int launch_group_params(PlaneParams p, int64_t G, hipStream_t st) {
     const int64_t wgs = resident_wgs();
+    if (p.x_dtype == BT_BF16) {  // (the caller has checked planes_bf16_shape_ok)
+        if (!launch_walk(p, G, wgs, -1, st)) return BT_ERR_INVALID;
+        return check_launch("gemv_planes_group");
+    }
     if (launch_walk(p, G, wgs, 16, st)) return check_launch("gemv_planes_group");
     // columns per wave: 32 (two tiles) streams best (5.3 TB/s against 4.8 with four tiles and 4.4-5.0 with one at
     // G = 128, 4096 x 4096); another width only where it fills the resident workgroups markedly more evenly
@@ -757,12 +850,41 @@ static int launch_group_params(PlaneParams p, int64_t G, hipStream_t st) {
     return check_launch("gemv_planes_group");
 }
 
-int launch_planes_group(const void* const* X_tab, const uint8_t* const* W_tab, const void* const* scale_tab, int scale_dtype,
-                        int scale_bcast, const void* const* bias_tab, int bias_dtype, void* const* Y_tab, int64_t G, int64_t N,
-                        int64_t K, hipStream_t st) {
+// bf16 rows run the contiguous-walk kernel only: K of 3..8 steps of 64 per wave (1040 <= K <= 4096, K % 16 == 0) and
+// whole batches of 16-column tiles (N % 32 == 0 for K > 2048, N % 64 == 0 below)
+bool planes_bf16_shape_ok(int64_t N, int64_t K) {
+    if (K % 16 != 0 || N % 4 != 0 || N <= 0 || K <= 0) return false;
+    return walk_shape_ok((int)ceil_div(ceil_div(K, 4), 16), (int)ceil_div(N, 16));
+}
+
+// One very wide bf16 matrix (a vocabulary projection) through the contiguous walk, direct pointers; the caller has
+// checked planes_bf16_shape_ok, the alignment of the operands (as planes_supported does for fp16) and that the
+// matrix gives every resident workgroup a dozen tiles (planes_bf16_wide).
+bool planes_bf16_wide(int64_t N, int64_t K) {
+    const char* force = getenv("BITTORCH_GROUP_WALK");
+    if (force && force[0] == '0') return false;
+    return planes_bf16_shape_ok(N, K) && ((force && force[0] == '1') || ceil_div(N, 16) >= 12 * resident_wgs());
+}
+int launch_planes_bf16_wide(const void* X, const uint8_t* W, const Epilogue& epi, void* Y, int64_t N, int64_t K, hipStream_t st) {
+    PlaneParams p = {};
+    p.X = X; p.W = W; p.scale = epi.scale; p.bias = epi.bias; p.residual = epi.residual; p.Y = Y;
+    p.scale_dtype = epi.scale_dtype; p.bias_dtype = epi.bias_dtype; p.scale_bcast = epi.scale_bcast;
+    p.x_dtype = BT_BF16;
+    p.N = N; p.K = K; p.Kb = ceil_div(K, 4);
+    p.G = 1;
+    p.wsteps = (int)ceil_div(p.Kb, 16);
+    p.tiles16 = (int)ceil_div(N, 16);
+    if (!launch_walk(p, 1, resident_wgs(), -1, st)) return BT_ERR_INVALID;
+    return check_launch("gemv_planes");
+}
+
+int launch_planes_group(const void* const* X_tab, int x_dtype, const uint8_t* const* W_tab, const void* const* scale_tab,
+                        int scale_dtype, int scale_bcast, const void* const* bias_tab, int bias_dtype, void* const* Y_tab,
+                        int64_t G, int64_t N, int64_t K, hipStream_t st) {
     PlaneParams p = {};
     p.X_tab = X_tab; p.W_tab = W_tab; p.scale_tab = scale_tab; p.bias_tab = bias_tab; p.Y_tab = Y_tab;
     p.scale_dtype = scale_dtype; p.bias_dtype = bias_dtype; p.scale_bcast = scale_bcast;
+    p.x_dtype = x_dtype;
     p.N = N; p.K = K; p.Kb = ceil_div(K, 4);
     p.G = (int)G;
     p.wsteps = (int)ceil_div(p.Kb, 16);

@@ -262,9 +262,21 @@ int bt_ternary_gemm_i8_tiled(const int8_t* Q, int q_layout, const float* s_x, co
  * and keep their weight loads running from one unit into the next.
  *   The five tables are DEVICE arrays of G device pointers, caller-owned (bias_tab may be NULL: no
  *   bias; its entries may not be NULL otherwise).  Every unit has the same N, K, scale length
- *   (N, or 1 = per-tensor) and element types.  x_dtype must be BT_F16, Y is fp16; K % 16 == 0, K <= 10240;
+ *   (N, or 1 = per-tensor) and element types.  x_dtype BT_F16: Y is fp16; K % 16 == 0, K <= 10240;
  *   each W_tiled 256-byte aligned, each X 16-byte aligned.  Units may share operands (one x for many
  *   matrices, one matrix for many rows) but not outputs.
+ *   x_dtype BT_BF16 (Y bf16): 1040 <= K <= 4096, K % 16 == 0, N a multiple of 32 (of 64 for K <= 2048),
+ *   else BT_ERR_INVALID.  A bf16 row spans more binades than a fixed-point sum can hold, so each row is
+ *   scaled by its own largest exponent: with E the (unbiased) exponent of the row's largest magnitude,
+ *   element x becomes the integer round_half_up(|x| * 2^(39 - E)) with its sign (exact for every element
+ *   whose exponent is within 32 of E, zero for those more than 40 below it), the integers are summed
+ *   exactly on the int8 matrix cores as six base-128 digit rows, and acc = fp32(S) * 2^(E - 39) enters
+ *   the usual epilogue y = bf16(fp32(acc * scale) + bias).  The result
+ *   does not depend on the order of summation; against the fp32 sums of the other bf16 kernels it differs
+ *   by the rounding of those sums (a few units of fp32 spacing), never by more.  A row holding Inf or NaN
+ *   gives NaN outputs.  bt_ternary_linear_tiled_forward takes the same route for ONE bf16 row (B = 1, no
+ *   prologue, epi_op = BT_EPI_NONE) times a matrix of at least 6144 column tiles of 16 (N >= 98304) within
+ *   the same K range: a vocabulary projection.
  */
 int bt_ternary_gemv_grouped(const void* const* X_tab, int x_dtype, const uint8_t* const* W_tiled_tab,
                             const void* const* scale_tab, int scale_dtype, int64_t scale_len,

@@ -20,6 +20,13 @@
  *   bto_linear_packed_exact_f16  pinned (the same linear with the sum formed exactly and
  *                                 rounded once: float64 dot product, exact for fp16
  *                                 operands, rounded to fp32; ties and subnormals)
+ *   bto_linear_packed_rowscaled_bf16  this library's own arithmetic for bf16 rows (the
+ *                                 reference's packed kernel takes fp16 / fp32): pinned by
+ *                                 the float64 dot product rounded once to fp32 wherever
+ *                                 the row spans at most 32 binades (then the scaling is
+ *                                 exact), by hand-made rows that exercise the half-up
+ *                                 rounding and the flush of far smaller elements, and by
+ *                                 the NaN / Inf rule
  *   bto_act_quant_i8    parity unpinned by the reference (no reference test
  *   bto_gemm_i8         touches the int8 path); pinned here only by brute
  *                       force on tiny inputs, exact integer identities and
@@ -336,6 +343,73 @@ int bto_linear_packed_exact_f16(const float* X, const uint8_t* W_T, const float*
     }
     free(XI);
     free(bad);
+    return status;
+}
+
+/*
+ * The same for bf16 activations (this library's own arithmetic for one bf16 row times a very wide matrix and for
+ * bf16 units of a grouped launch; no counterpart in the reference, whose packed kernel takes fp16 / fp32).  The
+ * exponent range of bf16 does not fit one fixed-point word, so each row is scaled by its own largest exponent:
+ * a finite bf16 value is mag * 2^(e1 - 134) with mag its 8-bit significand and e1 = max(biased exponent, 1);
+ * emax = the largest e1 of the row; X[k] = mag * 2^(e1 - emax + 32), an integer below 2^40 in magnitude, where an
+ * element more than 32 binades below the largest is rounded to an integer half-up in magnitude (more than 40 binades
+ * below: 0).  S = sum_k X[k] * w[k, n] exactly; acc = RN_fp32(S) * 2^(emax - 166); then the reference's epilogue.
+ * X holds bf16 values widened to float; returns -1 if one is not a bf16 value.  Rows with an infinity or a NaN: NaN.
+ */
+int bto_linear_packed_rowscaled_bf16(const float* X, const uint8_t* W_T, const float* scale,
+                                     int64_t scale_len, const float* bias, float* Y, int64_t B,
+                                     int64_t N, int64_t K) {
+    int64_t* XI = (int64_t*)malloc((size_t)B * K * sizeof(int64_t));
+    uint8_t* bad = (uint8_t*)calloc((size_t)B, 1);
+    int* emax = (int*)malloc((size_t)B * sizeof(int));
+    if (!XI || !bad || !emax) { free(XI); free(bad); free(emax); return -2; }
+    int status = 0;
+    for (int64_t b = 0; b < B; b++) {
+        int em = 1;
+        for (int64_t k = 0; k < K; k++) {
+            uint32_t u;
+            memcpy(&u, &X[b * K + k], 4);
+            if (u & 0xffffu) status = -1; /* not a bf16 value */
+            const int e = (int)((u >> 23) & 255u);
+            if (e == 255) { bad[b] = 1; continue; }
+            const int e1 = e ? e : 1;
+            if (e1 > em) em = e1;
+        }
+        emax[b] = em;
+        for (int64_t k = 0; k < K; k++) {
+            uint32_t u;
+            memcpy(&u, &X[b * K + k], 4);
+            const int e = (int)((u >> 23) & 255u);
+            if (e == 255) { XI[b * K + k] = 0; continue; }
+            const uint32_t m = (u >> 16) & 0x7fu;
+            const uint64_t mag = e ? (m | 0x80u) : m;
+            const int sh = (e ? e : 1) - em + 32;
+            uint64_t mg;
+            if (sh >= 0) mg = mag << sh;
+            else if (sh >= -8) mg = (mag + (1ull << (-sh - 1))) >> (-sh);
+            else mg = 0;
+            XI[b * K + k] = (u >> 31) ? -(int64_t)mg : (int64_t)mg;
+        }
+    }
+    if (status == 0) {
+#pragma omp parallel for schedule(static)
+        for (int64_t n = 0; n < N; n++) {
+            const float s = scale[scale_len == 1 ? 0 : n];
+            const float bv = bias ? bias[n] : 0.0f;
+            for (int64_t b = 0; b < B; b++) {
+                int64_t S = 0;
+                for (int64_t k = 0; k < K; k++)
+                    S += XI[b * K + k] * (int64_t)decode2((W_T[(k / 4) * N + n] >> (2 * (k % 4))) & 3u);
+                const float acc = ldexpf((float)S, emax[b] - 166);
+                float r = acc * s;
+                r = r + bv;
+                Y[b * N + n] = bad[b] ? NAN : r;
+            }
+        }
+    }
+    free(XI);
+    free(bad);
+    free(emax);
     return status;
 }
 

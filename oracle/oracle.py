@@ -51,6 +51,8 @@ def lib() -> ctypes.CDLL:
         _lib.bto_linear_packed.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64]
         _lib.bto_linear_packed_f64.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64]
         _lib.bto_linear_packed_fused_epilogue.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64]
+        _lib.bto_linear_packed_rowscaled_bf16.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64]
+        _lib.bto_linear_packed_rowscaled_bf16.restype = ctypes.c_int
         _lib.bto_linear_unpacked.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64]
         _lib.bto_linear_packed_exact_f16.restype = ctypes.c_int
         _lib.bto_linear_packed_exact_f16.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64]
@@ -186,6 +188,22 @@ def linear_packed_exact_f16(x, w_packed_t, scale, in_features: int, bias=None) -
     rc = lib().bto_linear_packed_exact_f16(_p(x), _p(w), _p(scale), scale.size, _p(bias), _p(y), b, n, k)
     if rc != 0:
         raise ValueError("activations are not fp16 values" if rc == -1 else "out of memory")
+    return y
+
+
+def linear_packed_rowscaled_bf16(x, w_packed_t, scale, in_features: int, bias=None) -> np.ndarray:
+    """Packed linear for bf16 activations (given widened to float): each row as integers scaled by its largest exponent,
+    the dot product summed exactly and rounded to fp32 once; fp32 result before the cast to the output dtype."""
+    x, scale, bias = _lin_args(x, w_packed_t, scale, bias)
+    w = np.ascontiguousarray(np.asarray(w_packed_t, dtype=np.uint8))
+    b, k = x.shape
+    assert k == in_features and w.shape[0] == (k + 3) // 4
+    n = w.shape[1]
+    assert scale.size in (1, n)
+    y = np.empty((b, n), dtype=np.float32)
+    rc = lib().bto_linear_packed_rowscaled_bf16(_p(x), _p(w), _p(scale), scale.size, _p(bias), _p(y), b, n, k)
+    if rc != 0:
+        raise ValueError("linear_packed_rowscaled_bf16: the activations must be bf16 values" if rc == -1 else "out of memory")
     return y
 
 

@@ -220,7 +220,7 @@ def test_grouped_launch_argument_errors():
     p = t.data_ptr()
     assert lib.bt_ternary_gemv_grouped(None, 1, p, p, 0, 16, None, 1, p, 8, 16, 16, None) == -1
     assert "null" in _lib.last_error()
-    assert lib.bt_ternary_gemv_grouped(p, 2, p, p, 0, 16, None, 1, p, 8, 16, 16, None) == -1
+    assert lib.bt_ternary_gemv_grouped(p, 0, p, p, 0, 16, None, 1, p, 8, 16, 16, None) == -1
     assert "fp16" in _lib.last_error()
     assert lib.bt_ternary_gemv_grouped(p, 1, p, p, 0, 16, None, 1, p, 8, 16, 24, None) == -1
     assert "multiple of 16" in _lib.last_error()
@@ -267,3 +267,84 @@ def test_grouped_launch_random_shapes(oracle, g, n, k, per_tensor, bias, seed):
                 assert torch.equal(ys[u], singles[units[u]]), (u, walk)
     finally:
         os.environ.pop("BITTORCH_GROUP_WALK", None)
+
+
+# ---- bf16 rows: scaled by the row's largest exponent, summed exactly ---------------------------------------------------
+def _setup_bf16(n, k, seed, per_tensor=False, bias=True, spread=0):
+    from bittorch_amd.quant import pack_ternary_transposed
+    w = random_ternary(n, k, seed=seed)
+    g = torch.Generator().manual_seed(seed + 7)
+    scale = torch.rand(1 if per_tensor else n, generator=g) * 0.05 + 0.01
+    x = seeded_acts(1, k, seed=seed + 3, dtype=torch.float32)
+    if spread:  # elements down to `spread` binades below the largest, and a row exponent far from 0
+        x = x * torch.exp2(-torch.randint(0, spread, (1, k), generator=g).float()) * (2.0 ** ((seed % 7) * 11 - 30))
+    x = x.bfloat16()
+    bias_t = (torch.randn(n, generator=g) * 0.01 * float(x.abs().max())).bfloat16() if bias else None
+    packed, _ = pack_ternary_transposed(w)
+    return x, packed, scale, bias_t
+
+
+def _expect_bf16(oracle, x, packed, scale, bias, k):
+    y = oracle.linear_packed_rowscaled_bf16(f32np(x), packed.numpy(), f32np(scale), k, None if bias is None else f32np(bias))
+    return torch.from_numpy(y).bfloat16()
+
+
+@pytest.mark.parametrize("g,n,k,per_tensor,bias,spread", [(1, 4096, 4096, True, True, 0), (7, 96, 2560, False, True, 20),
+                                                          (3, 2560, 2560, True, False, 45), (5, 64, 1536, False, True, 38),
+                                                          (11, 4128, 3008, False, True, 0), (140, 512, 2048, False, True, 30),
+                                                          (4, 32, 4080, False, True, 60)])
+def test_grouped_bf16_units_against_the_oracle(oracle, g, n, k, per_tensor, bias, spread):
+    """bf16 units of a grouped launch: bit-exact against the oracle's restatement of the row-scaled integer sum, and
+    within the reference tests' 16-bit thresholds (tests/test_packed_kernel.py:44-50) of the fp32-accumulate arithmetic."""
+    from bittorch_amd import _C
+    announce("grouped gemv bf16", g, n, k, spread)
+    sets = [_setup_bf16(n, k, seed=50 * u + n, per_tensor=per_tensor, bias=bias, spread=spread) for u in range(min(g, 5))]
+    tiles_ = [_C.retile_weights(s_[1].cuda(), k) for s_ in sets]
+    idx = [u % len(sets) for u in range(g)]
+    xs = [sets[i][0].cuda() for i in idx]
+    tiles = [tiles_[i] for i in idx]
+    scales = [sets[i][2].cuda() for i in idx]
+    biases = [sets[i][3].cuda() for i in idx] if bias else None
+    ys = [torch.full((1, n), float("nan"), dtype=torch.bfloat16, device="cuda") for _ in range(g)]
+    _C.ternary_gemv_grouped(*_tables(_C, xs, tiles, scales, biases, ys), k, n, scale_len=1 if per_tensor else n,
+                            bias_dtype=torch.bfloat16, x_dtype=torch.bfloat16)
+    torch.cuda.synchronize()
+    expects = [_expect_bf16(oracle, *s_, k) for s_ in sets]
+    for u in range(g):
+        assert torch.equal(ys[u].cpu(), expects[idx[u]]), u
+    x, packed, scale, b = sets[0]
+    ref = oracle.linear_packed(f32np(x), packed.numpy(), f32np(scale), k, None if b is None else f32np(b))
+    np.testing.assert_allclose(f32np(ys[0]), ref, rtol=1e-2, atol=1e-2 * float(np.abs(ref).max()))
+
+
+def test_bf16_row_times_a_wide_matrix_and_argument_errors(oracle):
+    """One bf16 row through the single-matrix entry point takes the same kernel where the matrix is wide enough
+    (forced here on a small one); a non-finite row gives NaN; shapes the bf16 units cannot take are refused."""
+    import os
+    from bittorch_amd import _C, _lib
+    announce("bf16 wide row")
+    n, k = 1024, 2560
+    x, packed, scale, bias = _setup_bf16(n, k, seed=5, spread=25)
+    tiled = _C.retile_weights(packed.cuda(), k)
+    y_stream = _C.ternary_linear_tiled_forward(x.cuda(), tiled, scale.cuda(), bias.cuda(), k, n)
+    try:
+        os.environ["BITTORCH_GROUP_WALK"] = "1"
+        y = _C.ternary_linear_tiled_forward(x.cuda(), tiled, scale.cuda(), bias.cuda(), k, n)
+        assert torch.equal(y.cpu(), _expect_bf16(oracle, x, packed, scale, bias, k))
+        res = seeded_acts(1, n, seed=9, dtype=torch.bfloat16)
+        y_r = _C.ternary_linear_tiled_forward(x.cuda(), tiled, scale.cuda(), bias.cuda(), k, n, residual=res.cuda())
+        assert torch.equal(y_r.cpu(), y.cpu() + res)
+        xb = x.clone()
+        xb[0, 77] = float("nan")
+        assert torch.isnan(_C.ternary_linear_tiled_forward(xb.cuda(), tiled, scale.cuda(), bias.cuda(), k, n)).all()
+    finally:
+        os.environ.pop("BITTORCH_GROUP_WALK", None)
+    # the 16-bit matrix-core kernel (what a narrow matrix takes) agrees within bf16 rounding
+    np.testing.assert_allclose(f32np(y_stream), f32np(y), rtol=2e-2, atol=2e-2 * float(f32np(y).__abs__().max()))
+    lib = _lib.load()
+    t = torch.zeros(8, dtype=torch.int64, device="cuda")
+    p = t.data_ptr()
+    assert lib.bt_ternary_gemv_grouped(p, 2, p, p, 0, 64, None, 2, p, 1, 64, 8192, None) == -1   # K beyond 4096
+    assert "bf16 units" in _lib.last_error()
+    assert lib.bt_ternary_gemv_grouped(p, 2, p, p, 0, 48, None, 2, p, 1, 48, 4096, None) == -1   # N % 32 != 0
+    assert "bf16 units" in _lib.last_error()

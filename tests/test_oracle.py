@@ -252,6 +252,78 @@ def test_linear_exact_f16_is_the_correctly_rounded_dot_product(oracle):
         oracle.linear_packed_exact_f16(np.array([[1.0 + 2.0 ** -20, 0, 0, 0]], np.float32), p4, one, 4)
 
 
+def _bf16(a):
+    """float32 array rounded to bf16 values (round to nearest even), still float32"""
+    u = np.asarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7fff + ((u >> 16) & 1)) & 0xffff0000
+    return u.astype(np.uint32).view(np.float32)
+
+
+def test_linear_rowscaled_bf16_is_the_correctly_rounded_dot_product(oracle):
+    """The bf16 variant against float64.  While every element of a row lies within 32 binades of the row's largest,
+    each is represented exactly and the result is the float64 dot product (exact for such rows) rounded once to fp32;
+    elements further down are rounded to the row's grid (half up in magnitude), which crafted rows pin, as they pin the
+    scaling by the row's exponent over the whole bf16 range, signs, ties of the final rounding and non-finite rows."""
+    rng = np.random.default_rng(1)
+    for (b, n, k) in [(1, 8, 16), (3, 33, 64), (2, 64, 4096), (1, 5, 48)]:
+        w = random_ternary(n, k, seed=k + 2).numpy()
+        # per row a base exponent anywhere in the bf16 range, elements spread over 30 binades below it
+        base = rng.integers(-100, 100, (b, 1))
+        x = _bf16(rng.standard_normal((b, k)) * np.exp2(base + rng.integers(-28, 1, (b, k))))
+        for r in range(b):  # make sure the row's largest element sits at the top of the spread
+            x[r, 0] = _bf16(np.float32(1.5) * np.exp2(np.float32(base[r, 0] + 1)))
+        packed_t, _ = oracle.pack_ternary_transposed(w)
+        ones = np.ones(n, np.float32)
+        acc64 = x.astype(np.float64) @ w.astype(np.float64).T   # exact: 8-bit significands within 31 binades, 4096 terms
+        np.testing.assert_array_equal(oracle.linear_packed_rowscaled_bf16(x, packed_t, ones, k), acc64.astype(np.float32))
+        scale = rng.random(n).astype(np.float32)
+        bias = (rng.standard_normal(n) * np.exp2(base[0, 0])).astype(np.float32)
+        expect = acc64.astype(np.float32) * scale[None, :] + bias[None, :]
+        np.testing.assert_array_equal(oracle.linear_packed_rowscaled_bf16(x, packed_t, scale, k, bias), expect)
+    one = np.ones(1, np.float32)
+    p4, _ = oracle.pack_ternary_transposed(np.ones((1, 4), np.int8))
+    m4, _ = oracle.pack_ternary_transposed(-np.ones((1, 4), np.int8))
+    f = lambda vals, p=p4: oracle.linear_packed_rowscaled_bf16(np.array([vals], np.float32), p, one, 4)[0, 0]
+    # ties of the final rounding go to even: 1 + 2^-24 -> 1; 1 + 3 * 2^-24 -> 1 + 2^-22 (all terms exact on the grid)
+    u = np.float32(2.0 ** -24)
+    assert f([1.0, u, 0, 0]) == 1.0 and f([1.0, u, u, u]) == np.float32(1 + 2.0 ** -22) and f([-1.0, -u, 0, 0]) == -1.0
+    # what an fp32 loop loses: 2^100 + 1 * 2^70 - 2^100 keeps the small term (30 binades down: exact)
+    assert f([2.0 ** 100, 2.0 ** 70, -(2.0 ** 100), 0]) == np.float32(2.0 ** 70)
+    # the grid: with the largest element 1.0 (e1 = 127) the unit is 2^-39 ... an element of 1.5 * 2^-39 rounds half up
+    # to 2 units, 1.25 * 2^-39 to 1 unit, 2^-41 (a quarter unit) to 0; signs follow the element
+    g = np.float32(2.0 ** -39)
+    assert f([1.0, 1.5 * g, -1.0, 0]) == np.float32(2 * g) and f([1.0, 1.25 * g, -1.0, 0]) == g
+    assert f([1.0, 2.0 ** -41, -1.0, 0]) == 0.0 and f([1.0, -1.5 * g, -1.0, 0]) == np.float32(-2 * g)
+    assert f([1.0, 0.5 * g, -1.0, 0]) == g               # exactly half a unit: up in magnitude
+    # the row's exponent scales the grid: the same row times 2^-100 and times 2^90 gives the same bits scaled
+    row = [1.0, 0.75, -0.375, 2.0 ** -20]
+    for e in (-100, -60, 0, 90):
+        sc = np.float32(2.0) ** e
+        assert f([v * sc for v in row]) == np.float32((1.0 + 0.75 - 0.375 + 2.0 ** -20) * 2.0 ** e)
+        assert f([v * sc for v in row], m4) == np.float32(-(1.0 + 0.75 - 0.375 + 2.0 ** -20) * 2.0 ** e)
+    # subnormal bf16 values (biased exponent 0) and an all-zero row
+    tiny = np.float32(2.0 ** -133)
+    assert f([tiny, tiny, 3 * tiny, 0]) == np.float32(5 * tiny) and f([0, 0, 0, 0]) == 0.0
+    # the largest bf16 value on every term stays finite in fp32 only up to the fp32 range
+    big = _bf16(np.float32(3.3e38))[()]
+    assert f([big, 0, 0, 0]) == big and np.isinf(f([big, big, big, big]))
+    # the reference's own known-answer vectors that are bf16 values
+    for case in GOLD["matmul"]:
+        w = np.array(case["weights"], dtype=np.int8)
+        packed_t, k = oracle.pack_ternary_transposed(w)
+        x = np.array(case["input"], dtype=np.float32)
+        if not np.array_equal(_bf16(x), x):
+            continue
+        np.testing.assert_array_equal(oracle.linear_packed_rowscaled_bf16(x, packed_t, np.array(case["scales"], np.float32), k),
+                                      np.array(case["output"], dtype=np.float32))
+    # non-finite rows: NaN everywhere, other rows untouched; inputs that are not bf16 values are refused
+    x = np.array([[1.0, np.inf, 0, 0], [1.0, 2.0, 3.0, 4.0]], np.float32)
+    y = oracle.linear_packed_rowscaled_bf16(x, p4, one, 4)
+    assert np.isnan(y[0, 0]) and y[1, 0] == 10.0
+    with pytest.raises(ValueError):
+        oracle.linear_packed_rowscaled_bf16(np.array([[1.0 + 2.0 ** -10, 0, 0, 0]], np.float32), p4, one, 4)
+
+
 # ---------------------------------------------------------------- int8 path (a7)
 def test_act_quant_brute_force(oracle):
     import math
