@@ -140,6 +140,17 @@ __device__ __forceinline__ float div127(float x) {
     const float r = __builtin_fmaf(-127.0f, q0, x);
     return __builtin_fmaf(r, y, q0);
 }
+// x / 127.0f in two operations: x * zh + RN(x * zl) with zh + zl = 1/127 to 48 bits, one fused multiply-add.
+// Checked exhaustively against IEEE division for every finite fp32 x: correctly rounded except for
+// 2^-122 <= |x| < 2^-113, where x * zl is subnormal and loses the bits that decide the rounding.  The caller
+// rules that range out (see DIV127_FAST_MIN_SX) or uses div127.
+__device__ __forceinline__ float div127_fast(float x) {
+    const float zh = 0x1.020408p-7f, zl = 0x1.020408p-35f;
+    return __builtin_fmaf(x, zh, __fmul_rn(x, zl));
+}
+// The dividend of the int8 epilogue is float(127 a) * s_x with an integer a: zero, or at least 127 |s_x| (1 - 2^-24)
+// in magnitude.  With |s_x| >= 2^-119 it is zero or above 2^-113, so div127_fast is exact for it.
+constexpr float DIV127_FAST_MIN_SX = 0x1p-119f;
 // int8 path: ((float(acc) * s_x) / 127) * w_scale + bias, left to right
 __device__ __forceinline__ float epi_int8_f(float acc127, float sx, float ws, float b) {
     float r = __fmul_rn(acc127, sx);

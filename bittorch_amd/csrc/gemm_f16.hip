@@ -350,9 +350,36 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
         }
         if (s < nstages) stage_y(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
     }
-    __syncthreads();  // every wave is done with the stage buffers before they are reused
+    // ---- add the two K halves through the stage buffers (64 KiB; word (q, wn, lane) is register q of that lane): K half 1
+    // hands over row blocks 0..3 and finishes 4..7, K half 0 the other way round.  K half 1 leaves the loop half a stage
+    // ahead and writes its share while K half 0 runs its last MFMAs (nobody reads live data from the buffers any more:
+    // K half 0 holds the fragments of those MFMAs in registers); behind the barrier K half 0 takes that share and puts
+    // its own into the slots it has just read (the LDS operations of a wave execute in order); one more barrier and
+    // K half 1 takes it.  (a + b == b + a in floating point: same bits whichever half adds.) ----
+    float* xch = (float*)lds;
+    const int slot = wn * 64 + lane;
+    auto give = [&](int mb0) {
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const v4f v = acc[mb0 + mb][t];
+                *(float4*)(xch + ((mb * 4 + t) * 256 + slot) * 4) = make_float4(v[0], v[1], v[2], v[3]);
+            }
+    };
+    auto take = [&](int mb0) {
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const float4 v = *(const float4*)(xch + ((mb * 4 + t) * 256 + slot) * 4);
+                acc[mb0 + mb][t] += v4f{v.x, v.y, v.z, v.w};
+            }
+    };
+    if (kgrp == 1) give(0);  // wave-uniform branches
+    __syncthreads();
 
-    // column scales and biases (raw bits) requested ahead of the exchange, which covers their latency
+    // column scales and biases (raw bits) requested ahead of the rest of the hand-over, which covers their latency
     uint32_t ws_bits[4], bs_bits[4];
 #pragma unroll
     for (int t = 0; t < 4; t++) {
@@ -361,36 +388,12 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
         bs_bits[t] = p.epi.bias ? load_bits_rt(p.epi.bias, p.epi.bias_dtype, n) : 0u;
     }
 
-    // ---- add the two K halves: K half 1 hands over row blocks 0..3, K half 0 hands over row
-    // blocks 4..7; word (q, wn, lane) of the exchange buffer is register q of that lane ----
-    {
-        float* xch = (float*)lds;
-        const int slot = wn * 64 + lane;
-#pragma unroll
-        for (int half = 0; half < 2; half++) {
-            const int giver = 1 - half;
-            if (kgrp == giver) {
-#pragma unroll
-                for (int mb = 0; mb < 4; mb++)
-#pragma unroll
-                    for (int t = 0; t < 4; t++) {
-                        const v4f v = acc[4 * half + mb][t];
-                        *(float4*)(xch + ((mb * 4 + t) * 256 + slot) * 4) = make_float4(v[0], v[1], v[2], v[3]);
-                    }
-            }
-            __syncthreads();
-            if (kgrp != giver) {
-#pragma unroll
-                for (int mb = 0; mb < 4; mb++)
-#pragma unroll
-                    for (int t = 0; t < 4; t++) {
-                        const float4 v = *(const float4*)(xch + ((mb * 4 + t) * 256 + slot) * 4);
-                        acc[4 * half + mb][t] += v4f{v.x, v.y, v.z, v.w};
-                    }
-            }
-            __syncthreads();
-        }
+    if (kgrp == 0) {
+        take(0);
+        give(4);
     }
+    __syncthreads();
+    if (kgrp == 1) take(4);
 
     if (!col_ok) return;
     if (kgrp == 0) gemm_f_epilogue_dt<MODE, 0>(p, acc, m0, g, ncol, ws_bits, bs_bits);  // wave-uniform branch

@@ -46,6 +46,7 @@ struct GemmParams {
     int tiles_m, tiles_n;
     int per_xcd;          // workgroups per XCD (grid = 8 * per_xcd)
     int wsteps, tiles16;  // WT: 16-row steps and 16-column tiles of the decode-tiled weight copy
+    int long_epilogue;    // A/B runs and tests (BITTORCH_GEMM_LONG_EPILOGUE=1): never the short epilogue
 };
 
 __device__ __forceinline__ void store4(void* Y, int dt, int64_t idx, const float (&v)[4]) {
@@ -120,6 +121,49 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&a
         }
     }
 }
+// The same for the common case, with the bookkeeping taken out of the per-row work: every row of the tile exists,
+// no residual, no accumulator output, and every row scale large enough for the two-operation division
+// (all wave-uniform, checked by the caller).  A row's address is a uniform base plus a 32-bit lane offset fixed
+// for the whole epilogue.  Same bits as gemm_epilogue.
+template <int YDT, int MB0>
+__device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, const v4i (&acc)[G_MB][4], int64_t m0, int g,
+                                                   int64_t ncol, const EpiOperands& e) {
+    float ws[4], bs[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        ws[t] = bits_to_f32_rt(e.ws_bits[t], p.epi.scale_dtype);
+        bs[t] = p.epi.bias ? bits_to_f32_rt(e.bs_bits[t], p.epi.bias_dtype) : 0.0f;
+    }
+    constexpr int ES = (YDT == BT_F32) ? 4 : 2;
+    const int64_t ncol0 = (int64_t)__builtin_amdgcn_readfirstlane((int)(ncol / G_BN)) * G_BN;  // the tile's first column
+    const uint32_t lane_off = ((uint32_t)(4 * g) * (uint32_t)p.N + (uint32_t)(ncol - ncol0)) * ES;
+    char* const base = (char*)p.Y + ((m0 + 16 * MB0) * p.N + ncol0) * ES;  // uniform
+    const int64_t row_bytes = p.N * ES;
+#pragma unroll
+    for (int mbi = 0; mbi < 4; mbi++) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const float sx = e.sx[mbi][r];
+            float y[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const float a127f = __fmul_rn((float)acc[MB0 + mbi][t][r], 127.0f);
+                const float q = div127_fast(__fmul_rn(a127f, sx));
+                y[t] = __fadd_rn(__fmul_rn(q, ws[t]), bs[t]);
+            }
+            char* const dst = base + (int64_t)(16 * mbi + r) * row_bytes + lane_off;
+            if constexpr (YDT == BT_F32) {
+                st4_nt((float*)dst, __builtin_bit_cast(uint32_t, y[0]), __builtin_bit_cast(uint32_t, y[1]),
+                       __builtin_bit_cast(uint32_t, y[2]), __builtin_bit_cast(uint32_t, y[3]));
+            } else {
+                uint16_t h[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) h[i] = (YDT == BT_F16) ? f32_to_f16_bits(y[i]) : f32_to_bf16_bits(y[i]);
+                st2_nt((uint16_t*)dst, (uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
+            }
+        }
+    }
+}
 template <int MB0>
 __device__ __forceinline__ void gemm_epilogue_dt(const GemmParams& p, const v4i (&acc)[G_MB][4], int64_t m0, int g,
                                                  int64_t ncol, const EpiOperands& e) {
@@ -127,37 +171,47 @@ __device__ __forceinline__ void gemm_epilogue_dt(const GemmParams& p, const v4i 
     else if (p.y_dtype == BT_F16) gemm_epilogue<BT_F16, MB0>(p, acc, m0, g, ncol, e);
     else gemm_epilogue<BT_F32, MB0>(p, acc, m0, g, ncol, e);
 }
+template <int MB0>
+__device__ __forceinline__ void gemm_epilogue_dt(const GemmParams& p, const v4i (&acc)[G_MB][4], int64_t m0, int g,
+                                                 int64_t ncol, const EpiOperands& e, bool fast) {
+    if (fast) {  // wave-uniform
+        if (p.y_dtype == BT_BF16) gemm_epilogue_fast<BT_BF16, MB0>(p, acc, m0, g, ncol, e);
+        else if (p.y_dtype == BT_F16) gemm_epilogue_fast<BT_F16, MB0>(p, acc, m0, g, ncol, e);
+        else gemm_epilogue_fast<BT_F32, MB0>(p, acc, m0, g, ncol, e);
+        return;
+    }
+    gemm_epilogue_dt<MB0>(p, acc, m0, g, ncol, e);
+}
 
-// Adds the two K halves: waves (wn, 0) and (wn, 1) hold partial sums of the same outputs.  K half 1 hands over row
-// blocks 0..3, K half 0 hands over row blocks 4..7; word (q, wn, lane) of the exchange buffer (64 KiB of LDS) is
-// register q of that lane.  Every wave must be done with the buffer's previous contents.
-__device__ __forceinline__ void exchange_k_halves(v4i (&acc)[G_MB][4], uint8_t* lds, int wn, int kgrp, int lane) {
-    int32_t* xch = (int32_t*)lds;
+// Adding the two K halves: waves (wn, 0) and (wn, 1) hold partial sums of the same outputs.  K half 1 hands over row
+// blocks 0..3 and finishes 4..7, K half 0 the other way round, through one 64 KiB area of LDS (the stage buffers, dead
+// by then): word (q, wn, lane) is register q of that lane.  Moving 64 KiB into LDS and out again is bandwidth, not
+// latency (most of a microsecond), so the order matters: K half 1, which ends the K loop half a stage ahead of K half 0,
+// writes its share while K half 0 still runs its last MFMAs; behind the barrier that ends the loop K half 0 takes that
+// share and puts its own into the same slots (a lane overwrites only words it has just read itself, and the LDS
+// operations of a wave execute in order), and one more barrier later K half 1 takes it: two barriers, and one of the
+// two writes out of the way.
+__device__ __forceinline__ void give_blocks(const v4i (&acc)[G_MB][4], int mb0, uint8_t* area, int wn, int lane) {
+    int32_t* xch = (int32_t*)area;
     const int slot = wn * 64 + lane;
 #pragma unroll
-    for (int half = 0; half < 2; half++) {
-        const int giver = 1 - half;  // K half that hands over row blocks 4*half .. 4*half+3
-        if (kgrp == giver) {
+    for (int mb = 0; mb < 4; mb++)
 #pragma unroll
-            for (int mb = 0; mb < 4; mb++)
-#pragma unroll
-                for (int t = 0; t < 4; t++) {
-                    const v4i v = acc[4 * half + mb][t];
-                    *(int4*)(xch + ((mb * 4 + t) * 256 + slot) * 4) = make_int4(v[0], v[1], v[2], v[3]);
-                }
+        for (int t = 0; t < 4; t++) {
+            const v4i v = acc[mb0 + mb][t];
+            *(int4*)(xch + ((mb * 4 + t) * 256 + slot) * 4) = make_int4(v[0], v[1], v[2], v[3]);
         }
-        __syncthreads();
-        if (kgrp != giver) {
+}
+__device__ __forceinline__ void take_blocks(v4i (&acc)[G_MB][4], int mb0, const uint8_t* area, int wn, int lane) {
+    const int32_t* xch = (const int32_t*)area;
+    const int slot = wn * 64 + lane;
 #pragma unroll
-            for (int mb = 0; mb < 4; mb++)
+    for (int mb = 0; mb < 4; mb++)
 #pragma unroll
-                for (int t = 0; t < 4; t++) {
-                    const int4 v = *(const int4*)(xch + ((mb * 4 + t) * 256 + slot) * 4);
-                    acc[4 * half + mb][t] += v4i{v.x, v.y, v.z, v.w};
-                }
+        for (int t = 0; t < 4; t++) {
+            const int4 v = *(const int4*)(xch + ((mb * 4 + t) * 256 + slot) * 4);
+            acc[mb0 + mb][t] += v4i{v.x, v.y, v.z, v.w};
         }
-        __syncthreads();
-    }
 }
 
 // TAIL = false: K is a multiple of the 128-wide stage and the main loop is branch free.
@@ -493,18 +547,32 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
         }
         if (s < nstages) stage_y(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
     }
-    __syncthreads();  // every wave is done with the stage buffers before they are reused
+    // K half 1 leaves the loop with nothing left to read from the stage buffers, and K half 0 holds the fragments of its
+    // last MFMAs in registers (what it still reads behind the last barrier of the loop belongs to a stage that does not
+    // exist and is never used): the hand-over may overwrite the buffers from here on.
+    if (kgrp == 1) give_blocks(acc, 0, lds, wn, lane);  // wave-uniform branches
+    __syncthreads();
 
     EpiOperands epi_ops;
     load_epi_operands(p, m0, 4 * kgrp, g, ncol, col_ok, epi_ops);
 
-    exchange_k_halves(acc, lds, wn, kgrp, lane);
+    if (kgrp == 0) {
+        take_blocks(acc, 0, lds, wn, lane);   // K half 1's sums of my row blocks 0..3
+        give_blocks(acc, 4, lds, wn, lane);   // my sums of its row blocks 4..7, into the slots just read
+    }
+    __syncthreads();
+    if (kgrp == 1) take_blocks(acc, 4, lds, wn, lane);
 
-    // ---- epilogue: K half h finishes row blocks 4h .. 4h+3; lane (j, g) holds rows
-    // 16mb + 4g + r, columns ncol .. ncol+3 -------------------------------------------
+    // the short epilogue where nothing needs the long one (every condition uniform over the wave)
+    bool small_sx = false;
+#pragma unroll
+    for (int mbi = 0; mbi < 4; mbi++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) small_sx |= !(__builtin_fabsf(epi_ops.sx[mbi][r]) >= DIV127_FAST_MIN_SX);
+    const bool fast = !p.long_epilogue && m0 + G_BM <= p.M && !p.epi.residual && !p.acc_out && __builtin_amdgcn_ballot_w64(small_sx) == 0ull;
     if (!col_ok) return;
-    if (kgrp == 0) gemm_epilogue_dt<0>(p, acc, m0, g, ncol, epi_ops);  // wave-uniform branch
-    else gemm_epilogue_dt<4>(p, acc, m0, g, ncol, epi_ops);
+    if (kgrp == 0) gemm_epilogue_dt<0>(p, acc, m0, g, ncol, epi_ops, fast);  // wave-uniform branch
+    else gemm_epilogue_dt<4>(p, acc, m0, g, ncol, epi_ops, fast);
 }
 
 
@@ -526,6 +594,7 @@ int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_
     p.Q = Q; p.s_x = s_x; p.W_T = W_T; p.Y = Y; p.acc_out = acc_out; p.epi = epi;
     p.M = M; p.N = N; p.K = K; p.Kb = ceil_div(K, 4);
     p.y_dtype = y_dtype;
+    p.long_epilogue = getenv("BITTORCH_GEMM_LONG_EPILOGUE") != nullptr;
     p.tiles_m = (int)ceil_div(M, G_BM);
     p.tiles_n = (int)ceil_div(N, G_BN);
     const int64_t total = (int64_t)p.tiles_m * p.tiles_n;

@@ -76,6 +76,43 @@ def test_gemm_i8_prefill_bit_exact(oracle, b, n, k, route, monkeypatch):
     _gemm_case(oracle, b, n, k, torch.float32, seed=n + k + 2, bias=False)
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_gemm_i8_epilogue_paths_agree_for_any_row_scale(oracle, out_dtype, monkeypatch):
+    """The prefill kernel has a short epilogue (full tiles, no residual, no accumulator output: division by 127 in two
+    operations) and a long one.  The short one is exact only while float(127 acc) * s_x stays out of 2^-122 .. 2^-113, so
+    a tile with a row scale below 2^-119 must take the long one: caller-made s_x with tiny, subnormal, huge, negative and
+    zero entries, every output against the oracle's true division, both epilogues forced and compared."""
+    from bittorch_amd import _C
+    from bittorch_amd.quant import pack_ternary_transposed
+    announce("gemm_i8 epilogue paths", out_dtype)
+    monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
+    b, n, k = 384, 512, 256
+    w = random_ternary(n, k, seed=3)
+    packed = pack_ternary_transposed(w)[0]
+    g = torch.Generator().manual_seed(4)
+    q = torch.randint(-127, 128, (b, k), generator=g, dtype=torch.int8)
+    scale = torch.rand(n, generator=g) * 0.05 + 0.01
+    bias = torch.randn(n, generator=g) * 0.01
+    s_x = torch.rand(b, generator=g) * 0.05 + 1e-3           # rows 0..127: ordinary scales -> short epilogue
+    s_x[128:256] = torch.tensor(2.0) ** torch.randint(-126, -100, (128,), generator=g).float()  # around the bad range
+    s_x[130] = 2.0 ** -119                                    # exactly the threshold (still the short division's range)
+    s_x[140] = 1e-42                                          # subnormal
+    s_x[150] = 0.0
+    s_x[256:] = torch.rand(128, generator=g) * 1e30           # third row tile: huge, one negative
+    s_x[300] = -0.37
+    _, oy = oracle.gemm_i8(q.numpy(), f32np(s_x), packed.numpy(), f32np(scale), k, f32np(bias))
+    expect = torch.from_numpy(oy).to(out_dtype)
+    args = (q.cuda(), s_x.cuda(), packed.cuda(), scale.cuda(), bias.cuda(), k)
+    y_short = _C.ternary_gemm_int8(*args, out_dtype=out_dtype)
+    monkeypatch.setenv("BITTORCH_GEMM_LONG_EPILOGUE", "1")
+    y_long = _C.ternary_gemm_int8(*args, out_dtype=out_dtype)
+    torch.cuda.synchronize()
+    assert torch.equal(y_long.cpu().view(torch.int16 if out_dtype != torch.float32 else torch.int32),
+                       expect.view(torch.int16 if out_dtype != torch.float32 else torch.int32))
+    assert torch.equal(y_short.cpu().view(torch.int16 if out_dtype != torch.float32 else torch.int32),
+                       expect.view(torch.int16 if out_dtype != torch.float32 else torch.int32))
+
+
 def test_gemm_i8_close_to_float_path(oracle):
     """int8 path vs the unquantized float product: inside the int8 quantisation error."""
     announce("gemm_i8 vs float")
