@@ -216,8 +216,23 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(PlaneParams p) 
     constexpr int TILE_N = 16 * NACC;
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
 
-    const int tile = (int)(blockIdx.x & 7) * p.per_xcd + (int)(blockIdx.x >> 3);  // neighbouring tiles on one XCD
+    int tile = (int)(blockIdx.x & 7) * p.per_xcd + (int)(blockIdx.x >> 3);  // neighbouring tiles on one XCD
     if (tile >= p.tiles) return;
+    // a few units in one launch (pointer tables, p.slabs workgroup tiles per unit): workgroup tile -> (unit, tile)
+    const void* Xp = p.X;
+    const uint8_t* Wp = p.W;
+    const void* scalep = p.scale;
+    const void* biasp = p.bias;
+    void* Yp = p.Y;
+    if (p.W_tab) {  // uniform
+        const int unit = tile / p.slabs;
+        tile -= unit * p.slabs;
+        Xp = p.X_tab[unit];
+        Wp = p.W_tab[unit];
+        scalep = p.scale_tab[unit];
+        biasp = p.bias_tab ? p.bias_tab[unit] : nullptr;
+        Yp = p.Y_tab[unit];
+    }
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int j = lane & 15, g = lane >> 4, q = lane & 3;
@@ -239,7 +254,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(PlaneParams p) 
     for (int u = 0; u < XC; u++) {
         if (u * 64 < nchunks) {  // uniform
             const int k = s_begin * 64 + (lane + 64 * u) * 8;
-            xr[u] = *(const uint4*)((const uint16_t*)p.X + (uint32_t)min(k, (int)p.K - 8));
+            xr[u] = *(const uint4*)((const uint16_t*)Xp + (uint32_t)min(k, (int)p.K - 8));
         }
     }
     // byte offset of this lane's dword in step 0 of each of its 16-column tiles (tiled copy), resp. of its quad's
@@ -264,10 +279,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(PlaneParams p) 
 #pragma unroll
             for (int t = 0; t < NACC; t++) {
                 if constexpr (LAYOUT == PL_TILED) {
-                    raw[f][t] = ldw_nt(p.W + (coloff[t] + (uint32_t)ws * 256u));
+                    raw[f][t] = ldw_nt(Wp + (coloff[t] + (uint32_t)ws * 256u));
                 } else {
                     const uint32_t ro = min((uint32_t)(16 * ws + 4 * g + q) * N32, last_rowoff);
-                    raw[f][t] = ldw_nt(p.W + (ro + coloff[t]));
+                    raw[f][t] = ldw_nt(Wp + (ro + coloff[t]));
                 }
             }
         }
@@ -285,11 +300,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(PlaneParams p) 
     const bool out_thread = PAIRS ? (tid < TILE_N / 2 && n_out < ffn) : (tid < TILE_N && n_out < p.N);
     const int slot = PAIRS ? (tid >> 4) * 32 + (tid & 15) : tid;
     if (out_thread) {
-        pre_s = load_bits_rt(p.scale, p.scale_dtype, p.scale_bcast ? 0 : n_out);
-        if (p.bias) pre_b = load_bits_rt(p.bias, p.bias_dtype, n_out);
+        pre_s = load_bits_rt(scalep, p.scale_dtype, p.scale_bcast ? 0 : n_out);
+        if (biasp) pre_b = load_bits_rt(biasp, p.bias_dtype, n_out);
         if constexpr (PAIRS) {
-            pre_s2 = load_bits_rt(p.scale, p.scale_dtype, p.scale_bcast ? 0 : ffn + n_out);
-            if (p.bias) pre_b2 = load_bits_rt(p.bias, p.bias_dtype, ffn + n_out);
+            pre_s2 = load_bits_rt(scalep, p.scale_dtype, p.scale_bcast ? 0 : ffn + n_out);
+            if (biasp) pre_b2 = load_bits_rt(biasp, p.bias_dtype, ffn + n_out);
         }
     }
 
@@ -360,16 +375,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(PlaneParams p) 
     }
     for (int w = 0; w < WAVES; w++) any_bad |= flags[w];
     const float sc = bits_to_f32_rt(pre_s, p.scale_dtype);
-    const float bs = p.bias ? bits_to_f32_rt(pre_b, p.bias_dtype) : 0.0f;
+    const float bs = biasp ? bits_to_f32_rt(pre_b, p.bias_dtype) : 0.0f;
     if constexpr (PAIRS) {
         const float sc2 = bits_to_f32_rt(pre_s2, p.scale_dtype);
-        const float bs2 = p.bias ? bits_to_f32_rt(pre_b2, p.bias_dtype) : 0.0f;
+        const float bs2 = biasp ? bits_to_f32_rt(pre_b2, p.bias_dtype) : 0.0f;
         float gv = round_to_dtype(epi_float(fixed_to_f32(S), sc, bs), BT_F16);
         const float uv = round_to_dtype(epi_float(fixed_to_f32(S2), sc2, bs2), BT_F16);
         if (any_bad) gv = __builtin_nanf("");
-        ((uint16_t*)p.Y)[n_out] = f32_to_f16_bits(swiglu_value(gv, uv, BT_F16));
+        ((uint16_t*)Yp)[n_out] = f32_to_f16_bits(swiglu_value(gv, uv, BT_F16));
     } else {
-        pl_store(p.Y, p.residual, n_out, fixed_to_f32(S), sc, bs, any_bad != 0u);
+        pl_store(Yp, p.residual, n_out, fixed_to_f32(S), sc, bs, any_bad != 0u);
     }
 }
 
@@ -691,6 +706,7 @@ bool planes_supported(int x_dtype, int y_dtype, int64_t B, int64_t N, int64_t K,
     return ((uintptr_t)W) % 4 == 0 && (ceil_div(K, 4) + 64) * N < (1ll << 32);
 }
 
+constexpr int64_t GROUP_UNITS_MAX_BYTES = 20ll << 20;  // (see launch_units)
 // grouped and wide launches: 2 workgroups of 8 waves per compute unit
 static int g_group_cus = 0;
 static int64_t resident_wgs() {
@@ -807,13 +823,41 @@ int launch_planes(const void* X, const uint8_t* W, int w_layout, const Epilogue&
 }
 
 
+// A few units in one launch of the one-matrix kernel (workgroup tile -> (unit, tile) through the pointer tables): every
+// workgroup converts its unit's row itself and reads 16 * NACC columns over the whole of K, as many workgroups as the
+// units have tiles.  Up to about 20 MiB of weights this beats the persistent kernels, whose workgroups each walk
+// several tiles one after another (units of 4096 x 4096: G = 1 4.8 against 9.4 us, G = 2 5.8 against 9.5, G = 4 7.7
+// against 9.9, G = 6 equal, G = 8 12.6 against 10.8).  BITTORCH_GROUP_UNITS=1 / =0 (tests, A/B runs): always / never.
+static bool launch_units(PlaneParams p, int64_t G, hipStream_t st) {
+    const char* force = getenv("BITTORCH_GROUP_UNITS");
+    if (force && force[0] == '0') return false;
+    if (p.K > PL_MAX_K) return false;
+    const int64_t bytes = G * (int64_t)p.tiles16 * p.wsteps * 256;
+    if (!(force && force[0] == '1') && bytes > (int64_t)GROUP_UNITS_MAX_BYTES) return false;
+    int nacc = 4;
+    while (nacc > 1 && G * ceil_div(p.tiles16, nacc) < 224) nacc >>= 1;
+    p.slabs = (int)ceil_div(p.tiles16, nacc);
+    if (G * p.slabs > 0x3fffffff) return false;
+    p.tiles = (int)(G * p.slabs);
+    p.per_xcd = (int)ceil_div(p.tiles, 8);
+    if (nacc == 4) launch_planes_k<PL_TILED, 4>(p, st);
+    else if (nacc == 2) launch_planes_k<PL_TILED, 2>(p, st);
+    else launch_planes_k<PL_TILED, 1>(p, st);
+    return true;
+}
+
 static int launch_group_params(PlaneParams p, int64_t G, hipStream_t st) {
     const int64_t wgs = resident_wgs();
     if (p.x_dtype == BT_BF16) {  // (the caller has checked planes_bf16_shape_ok)
         if (!launch_walk(p, G, wgs, -1, st)) return BT_ERR_INVALID;
         return check_launch("gemv_planes_group");
     }
+    {
+        const char* force = getenv("BITTORCH_GROUP_UNITS");
+        if (force && force[0] == '1' && launch_units(p, G, st)) return check_launch("gemv_planes_group");
+    }
     if (launch_walk(p, G, wgs, 16, st)) return check_launch("gemv_planes_group");
+    if (launch_units(p, G, st)) return check_launch("gemv_planes_group");
     // columns per wave: 32 (two tiles) streams best (5.3 TB/s against 4.8 with four tiles and 4.4-5.0 with one at
     // G = 128, 4096 x 4096); another width only where it fills the resident workgroups markedly more evenly
     int nacc = 2;

@@ -140,25 +140,25 @@ def test_grouped_launch_equals_single_calls(oracle, g, n, k, per_tensor, bias):
         singles.append(_C.ternary_linear_tiled_forward(xs[-1], tiles[-1], scales[-1], biases[-1], k, n))
         if u == 0:
             assert torch.equal(singles[0].cpu(), _expect(oracle, x, packed, scale, b, k))
-    # the library's own choice of kernel, then the contiguous-walk kernel (where the shape allows it) and the
-    # one-stream-per-wave kernel in its three widths
+    # the library's own choice of kernel, then the contiguous-walk kernel (where the shape allows it), the
+    # one-stream-per-wave kernel in its three widths and the one-matrix kernel over (unit, tile) workgroups
     try:
-        for walk, nacc in ((None, None), ("1", None), ("0", "1"), ("0", "2"), ("0", "4")):
-            os.environ.pop("BITTORCH_GROUP_WALK", None)
-            os.environ.pop("BITTORCH_GROUP_NACC", None)
-            if walk:
-                os.environ["BITTORCH_GROUP_WALK"] = walk
-            if nacc:
-                os.environ["BITTORCH_GROUP_NACC"] = nacc
+        for walk, nacc, units in ((None, None, None), ("1", None, "0"), ("0", "1", "0"), ("0", "2", "0"), ("0", "4", "0"),
+                                  (None, None, "1")):
+            for name, val in (("BITTORCH_GROUP_WALK", walk), ("BITTORCH_GROUP_NACC", nacc), ("BITTORCH_GROUP_UNITS", units)):
+                os.environ.pop(name, None)
+                if val:
+                    os.environ[name] = val
             ys = [torch.full((1, n), float("nan"), dtype=torch.float16, device="cuda") for _ in range(g)]
             tabs = _tables(_C, xs, tiles, scales, biases if bias else None, ys)
             _C.ternary_gemv_grouped(*tabs, k, n, scale_len=1 if per_tensor else n)
             torch.cuda.synchronize()
             for u in range(g):
-                assert torch.equal(ys[u], singles[u]), (u, walk, nacc)
+                assert torch.equal(ys[u], singles[u]), (u, walk, nacc, units)
     finally:
         os.environ.pop("BITTORCH_GROUP_NACC", None)
         os.environ.pop("BITTORCH_GROUP_WALK", None)
+        os.environ.pop("BITTORCH_GROUP_UNITS", None)
 
 
 def test_grouped_launch_config2_units_and_shared_operands(oracle):
@@ -238,8 +238,9 @@ _GROUP_CASES = [(int(_grp_rng.integers(1, 40)), int(_grp_rng.integers(1, 80)) * 
 @pytest.mark.parametrize("g,n,k,per_tensor,bias,seed", _GROUP_CASES)
 def test_grouped_launch_random_shapes(oracle, g, n, k, per_tensor, bias, seed):
     """Seeded random G, N (any multiple of 4) and K (1040 .. 4096, the range of the contiguous-walk kernel), units
-    drawn from three weight matrices and three activation rows: the walk kernel where the shape allows it and the
-    one-stream-per-wave kernel both equal the single calls, and those the oracle."""
+    drawn from three weight matrices and three activation rows: the walk kernel where the shape allows it, the
+    one-stream-per-wave kernel and the one-matrix kernel over (unit, tile) workgroups all equal the single calls, and
+    those the oracle."""
     import os
     from bittorch_amd import _C
     announce("grouped gemv random", g, n, k, per_tensor, bias, seed)
@@ -258,15 +259,17 @@ def test_grouped_launch_random_shapes(oracle, g, n, k, per_tensor, bias, seed):
     a0, w0 = units[0]
     assert torch.equal(singles[(a0, w0)].cpu(), _expect(oracle, base[a0][0], base[w0][1], base[w0][2], base[w0][3], k))
     try:
-        for walk in ("1", "0"):
+        for walk, one_matrix in (("1", "0"), ("0", "0"), ("0", "1")):
             os.environ["BITTORCH_GROUP_WALK"] = walk
+            os.environ["BITTORCH_GROUP_UNITS"] = one_matrix
             ys = [torch.full((1, n), float("nan"), dtype=torch.float16, device="cuda") for _ in range(g)]
             _C.ternary_gemv_grouped(*_tables(_C, xs, tiles, scales, biases, ys), k, n, scale_len=1 if per_tensor else n)
             torch.cuda.synchronize()
             for u in range(g):
-                assert torch.equal(ys[u], singles[units[u]]), (u, walk)
+                assert torch.equal(ys[u], singles[units[u]]), (u, walk, one_matrix)
     finally:
         os.environ.pop("BITTORCH_GROUP_WALK", None)
+        os.environ.pop("BITTORCH_GROUP_UNITS", None)
 
 
 # ---- bf16 rows: scaled by the row's largest exponent, summed exactly ---------------------------------------------------
