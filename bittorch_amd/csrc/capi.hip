@@ -519,8 +519,8 @@ extern "C" int bt_ternary_gemv_grouped(const void* const* X_tab, int x_dtype, co
         set_error("%s: activations must be fp16 or bf16 (dtype tag %d given)", who, x_dtype);
         return BT_ERR_INVALID;
     }
-    if (K % 16 != 0 || K > 10240) {
-        set_error("%s: K must be a multiple of 16 and at most 10240 (K=%lld)", who, (long long)K);
+    if (K % 16 != 0 || K > 16384) {
+        set_error("%s: K must be a multiple of 16 and at most 16384 (K=%lld)", who, (long long)K);
         return BT_ERR_INVALID;
     }
     if (x_dtype == BT_BF16 && !planes_bf16_shape_ok(N, K)) {

@@ -706,7 +706,6 @@ bool planes_supported(int x_dtype, int y_dtype, int64_t B, int64_t N, int64_t K,
     return ((uintptr_t)W) % 4 == 0 && (ceil_div(K, 4) + 64) * N < (1ll << 32);
 }
 
-constexpr int64_t GROUP_UNITS_MAX_BYTES = 20ll << 20;  // (see launch_units)
 // grouped and wide launches: 2 workgroups of 8 waves per compute unit
 static int g_group_cus = 0;
 static int64_t resident_wgs() {
@@ -823,17 +822,39 @@ int launch_planes(const void* X, const uint8_t* W, int w_layout, const Epilogue&
 }
 
 
+template <int NACC, int PF>
+static void launch_group_k(const PlaneParams& p, unsigned grid, size_t lds, hipStream_t st) {
+    if (lds > 64 * 1024) {  // the digit rows of a long activation row (K > 10240 or so): beyond the default limit of dynamic LDS
+        static bool raised = false;
+        if (!raised) {
+            (void)hipFuncSetAttribute((const void*)gemv_planes_group_kernel<NACC, PF>,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+            raised = true;
+        }
+    }
+    hipLaunchKernelGGL((gemv_planes_group_kernel<NACC, PF>), dim3(grid), dim3(512), lds, st, p);
+}
+
 // A few units in one launch of the one-matrix kernel (workgroup tile -> (unit, tile) through the pointer tables): every
 // workgroup converts its unit's row itself and reads 16 * NACC columns over the whole of K, as many workgroups as the
-// units have tiles.  Up to about 20 MiB of weights this beats the persistent kernels, whose workgroups each walk
-// several tiles one after another (units of 4096 x 4096: G = 1 4.8 against 9.4 us, G = 2 5.8 against 9.5, G = 4 7.7
-// against 9.9, G = 6 equal, G = 8 12.6 against 10.8).  BITTORCH_GROUP_UNITS=1 / =0 (tests, A/B runs): always / never.
+// units have tiles.  For a handful of units this beats the persistent kernels, whose workgroups each walk several
+// tiles one after another (units of 4096 x 4096: G = 1 4.8 against 9.4 us, G = 2 5.8 against 9.5, G = 4 7.7 against
+// 9.9, G = 6 equal, G = 8 12.6 against 10.8; units of N = 4096, K = 11008: G = 1 9.2 against 20.6, G = 4 14.9 against
+// 21.6, G = 8 21.8 against 23.6, G = 16 40.6 against 38.4).  BITTORCH_GROUP_UNITS=1 / =0 (tests, A/B runs): always / never.
 static bool launch_units(PlaneParams p, int64_t G, hipStream_t st) {
     const char* force = getenv("BITTORCH_GROUP_UNITS");
     if (force && force[0] == '0') return false;
     if (p.K > PL_MAX_K) return false;
-    const int64_t bytes = G * (int64_t)p.tiles16 * p.wsteps * 256;
-    if (!(force && force[0] == '1') && bytes > (int64_t)GROUP_UNITS_MAX_BYTES) return false;
+    if (!(force && force[0] == '1')) {
+        // microseconds, fitted to launches of G units of 4096 x 4096 and 4096 x 11008 on this chip: the persistent kernel
+        // has a floor that grows with K (a wave walks the whole of K for its columns) and streams at about 5 TB/s
+        // beyond it; the one-matrix kernel starts lower and streams at about 4 TB/s
+        const double mib = (double)G * (double)p.tiles16 * (double)p.wsteps * 256.0 / 1048576.0;
+        const double k = (double)p.K;
+        const double t_units = 1.4 + 0.0006 * k + 0.24 * mib;
+        const double t_floor = 2.6 + 0.00162 * k + 0.04 * mib, t_stream = 4.0 + 0.2 * mib;
+        if (t_units >= (t_floor > t_stream ? t_floor : t_stream)) return false;
+    }
     int nacc = 4;
     while (nacc > 1 && G * ceil_div(p.tiles16, nacc) < 224) nacc >>= 1;
     p.slabs = (int)ceil_div(p.tiles16, nacc);
@@ -883,13 +904,13 @@ static int launch_group_params(PlaneParams p, int64_t G, hipStream_t st) {
     const int SP = (int)ceil_div(p.wsteps, pf) * pf;
     const size_t lds = 32 + (size_t)SP * 4 * PL_GROUP;
     if (pf == 16) {
-        if (nacc == 4) hipLaunchKernelGGL((gemv_planes_group_kernel<4, 16>), dim3(grid), dim3(512), lds, st, p);
-        else if (nacc == 2) hipLaunchKernelGGL((gemv_planes_group_kernel<2, 16>), dim3(grid), dim3(512), lds, st, p);
-        else hipLaunchKernelGGL((gemv_planes_group_kernel<1, 16>), dim3(grid), dim3(512), lds, st, p);
+        if (nacc == 4) launch_group_k<4, 16>(p, grid, lds, st);
+        else if (nacc == 2) launch_group_k<2, 16>(p, grid, lds, st);
+        else launch_group_k<1, 16>(p, grid, lds, st);
     } else {
-        if (nacc == 4) hipLaunchKernelGGL((gemv_planes_group_kernel<4, 8>), dim3(grid), dim3(512), lds, st, p);
-        else if (nacc == 2) hipLaunchKernelGGL((gemv_planes_group_kernel<2, 8>), dim3(grid), dim3(512), lds, st, p);
-        else hipLaunchKernelGGL((gemv_planes_group_kernel<1, 8>), dim3(grid), dim3(512), lds, st, p);
+        if (nacc == 4) launch_group_k<4, 8>(p, grid, lds, st);
+        else if (nacc == 2) launch_group_k<2, 8>(p, grid, lds, st);
+        else launch_group_k<1, 8>(p, grid, lds, st);
     }
     return check_launch("gemv_planes_group");
 }

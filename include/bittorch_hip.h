@@ -259,11 +259,11 @@ int bt_ternary_gemm_i8_tiled(const int8_t* Q, int q_layout, const float* s_x, co
  * pays launch, set-up and drain once for G matrices: persistent workgroups each read a contiguous run
  * of the (unit, 16-column tile) sequence front to back, their waves splitting K (1040 <= K <= 4096 and
  * at least 16 tiles per workgroup; other shapes: (unit, column slab) items, a wave per tile column),
- * and keep their weight loads running from one unit into the next.  A launch of up to 20 MiB of weights
- * (a handful of units) runs the one-matrix kernel with one workgroup per (unit, column tile) instead.
+ * and keep their weight loads running from one unit into the next.  A handful of units (where a cost model
+ * prices it lower) run the one-matrix kernel with one workgroup per (unit, column tile) instead.
  *   The five tables are DEVICE arrays of G device pointers, caller-owned (bias_tab may be NULL: no
  *   bias; its entries may not be NULL otherwise).  Every unit has the same N, K, scale length
- *   (N, or 1 = per-tensor) and element types.  x_dtype BT_F16: Y is fp16; K % 16 == 0, K <= 10240;
+ *   (N, or 1 = per-tensor) and element types.  x_dtype BT_F16: Y is fp16; K % 16 == 0, K <= 16384;
  *   each W_tiled 256-byte aligned, each X 16-byte aligned.  Units may share operands (one x for many
  *   matrices, one matrix for many rows) but not outputs.
  *   x_dtype BT_BF16 (Y bf16): 1040 <= K <= 4096, K % 16 == 0, N a multiple of 32 (of 64 for K <= 2048),

@@ -119,7 +119,8 @@ def _tables(_C, xs, tiles, scales, biases, ys):
 @pytest.mark.parametrize("g,n,k,per_tensor,bias", [(1, 4096, 4096, True, True), (5, 256, 512, False, True),
                                                    (37, 1024, 1024, False, False), (3, 100, 144, False, True),
                                                    (9, 2560, 6912, True, True), (130, 128, 64, False, True),
-                                                   (4, 36, 8192, False, True),
+                                                   (4, 36, 8192, False, True), (3, 64, 11008, False, True),
+                                                   (2, 32, 16384, True, True),
                                                    # K of 3..8 steps per wave: the contiguous-walk kernel
                                                    (7, 96, 2560, False, True), (3, 2560, 2560, True, True),
                                                    (5, 64, 1536, False, False), (11, 4128, 3008, False, True),
