@@ -349,8 +349,8 @@ def ternary_gemv_grouped(x_tab: Tensor, w_tiled_tab: Tensor, scale_tab: Tensor, 
     decode-tiled weights at ``w_tiled_tab[u]`` into the fp16 row at ``y_tab[u]``, exactly as
     :func:`ternary_linear_tiled_forward` would on that row (same bits).  The tables are int64 device tensors of
     ``G`` device addresses (:func:`pointer_table`); nothing is allocated or returned.
-    ``x_dtype=torch.bfloat16``: bf16 rows and outputs (1040 <= K <= 4096, N a multiple of 32, of 64 for K <= 2048);
-    each row is scaled by its own largest exponent and summed exactly on the int8 matrix cores."""
+    ``x_dtype=torch.bfloat16``: bf16 rows and outputs; each row is scaled by its own largest exponent and summed
+    exactly on the int8 matrix cores."""
     G = x_tab.numel()
     tabs = (x_tab, w_tiled_tab, scale_tab, y_tab) + (() if bias_tab is None else (bias_tab,))
     for t in tabs:

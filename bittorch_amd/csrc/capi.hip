@@ -523,11 +523,6 @@ extern "C" int bt_ternary_gemv_grouped(const void* const* X_tab, int x_dtype, co
         set_error("%s: K must be a multiple of 16 and at most 16384 (K=%lld)", who, (long long)K);
         return BT_ERR_INVALID;
     }
-    if (x_dtype == BT_BF16 && !planes_bf16_shape_ok(N, K)) {
-        set_error("%s: bf16 units need 1040 <= K <= 4096 and N a multiple of 32 (of 64 for K <= 2048) (N=%lld K=%lld)", who,
-                  (long long)N, (long long)K);
-        return BT_ERR_INVALID;
-    }
     if ((scale_len != N && scale_len != 1) || !valid_dtype(scale_dtype) || (bias_tab && !valid_dtype(bias_dtype))) {
         set_error("%s: scale size doesn't match N, or unsupported scale/bias dtype", who);
         return BT_ERR_INVALID;

@@ -400,9 +400,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(PlaneParams p) 
 // same time (a pure read of this address stream: 5.7 TB/s in lockstep, 6.7 TB/s rotated); the sums are integers, so
 // the order does not change a bit of the result.
 // LDS: a flag word per wave, then the digit planes of one row, padded with zero groups to a multiple of PF steps.
-template <int NACC, int PF>
+// XDT = BT_BF16: bf16 rows and outputs; the row is read twice per item, once for its largest exponent (the waves'
+// maxima meet in LDS, one more barrier) and once for its digits (see bf16x8_to_planes).
+template <int NACC, int PF, int XDT = BT_F16>
 __global__ __launch_bounds__(512, 4) void gemv_planes_group_kernel(PlaneParams p) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+    __shared__ int emax_slot[8];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int j = lane & 15, g = lane >> 4;
@@ -441,12 +444,25 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_group_kernel(PlaneParams p
         // the unit's activation row -> digit planes (all waves; the previous item's readers are past the barrier
         // that ended it)
         const uint16_t* xrow = (const uint16_t*)p.X_tab[u];
+        int emax = 0;
+        if constexpr (XDT == BT_BF16) {
+            int m = 1;
+            for (int c = (int)threadIdx.x; c * 8 < (int)p.K; c += 512) m = max(m, bf16x8_max_e1(*(const uint4*)(xrow + min(c * 8, (int)p.K - 8))));
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) m = max(m, __shfl_xor(m, off, 64));
+            if (lane == 0) emax_slot[wave] = m;
+            __syncthreads();  // (the slots' readers of the previous item are past the barrier that ended it)
+            m = emax_slot[lane & 7];
+#pragma unroll
+            for (int off = 4; off > 0; off >>= 1) m = max(m, __shfl_xor(m, off, 64));
+            emax = m;
+        }
         bool bad = false;
         for (int c = (int)threadIdx.x; c < nchunks; c += 512) {
             const int k = c * 8;
             uint4 v = *(const uint4*)(xrow + min(k, (int)p.K - 8));
             v = zero_unless4(v, k < (int)p.K);
-            bad |= park_chunk(planes, c, v, lane, true);
+            bad |= park_chunk<XDT>(planes, c, v, lane, true, emax);
         }
         // (a word per wave, stored unconditionally: nothing to clear between items)
         const bool wave_bad = __builtin_amdgcn_ballot_w64(bad) != 0ull;
@@ -510,7 +526,7 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_group_kernel(PlaneParams p
             if (g == 0 && n < p.N) {
                 const float sc = bits_to_f32_rt(pre_s[t], p.scale_dtype);
                 const float bs = bias_u ? bits_to_f32_rt(pre_b[t], p.bias_dtype) : 0.0f;
-                pl_store(y_u, nullptr, n, planes_to_f32(s), sc, bs, any_bad);
+                pl_store<XDT>(y_u, nullptr, n, planes_to_f32(s, (XDT == BT_BF16) ? emax - 166 : -24), sc, bs, any_bad);
             }
         }
         __syncthreads();  // every wave is done with the planes before the next item overwrites them
@@ -740,7 +756,7 @@ static void launch_walk_k(const PlaneParams& p, int spw, unsigned grid, hipStrea
         default: hipLaunchKernelGGL((gemv_planes_chunk_kernel<8, 2, XDT>), dim3(grid), dim3(512), 0, st, p); break;
     }
 }
-// min_tiles_per_wg < 0: whenever the shape allows (bf16 units have no other kernel)
+// min_tiles_per_wg < 0: whenever the shape allows
 static bool launch_walk(PlaneParams p, int64_t G, int64_t wgs, int min_tiles_per_wg, hipStream_t st) {
     const int spw = (int)ceil_div(p.wsteps, 8);
     const int tb = (spw >= 5) ? 2 : 4;
@@ -822,17 +838,17 @@ int launch_planes(const void* X, const uint8_t* W, int w_layout, const Epilogue&
 }
 
 
-template <int NACC, int PF>
+template <int NACC, int PF, int XDT = BT_F16>
 static void launch_group_k(const PlaneParams& p, unsigned grid, size_t lds, hipStream_t st) {
     if (lds > 64 * 1024) {  // the digit rows of a long activation row (K > 10240 or so): beyond the default limit of dynamic LDS
         static bool raised = false;
         if (!raised) {
-            (void)hipFuncSetAttribute((const void*)gemv_planes_group_kernel<NACC, PF>,
+            (void)hipFuncSetAttribute((const void*)gemv_planes_group_kernel<NACC, PF, XDT>,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
             raised = true;
         }
     }
-    hipLaunchKernelGGL((gemv_planes_group_kernel<NACC, PF>), dim3(grid), dim3(512), lds, st, p);
+    hipLaunchKernelGGL((gemv_planes_group_kernel<NACC, PF, XDT>), dim3(grid), dim3(512), lds, st, p);
 }
 
 // A few units in one launch of the one-matrix kernel (workgroup tile -> (unit, tile) through the pointer tables): every
@@ -869,16 +885,15 @@ static bool launch_units(PlaneParams p, int64_t G, hipStream_t st) {
 
 static int launch_group_params(PlaneParams p, int64_t G, hipStream_t st) {
     const int64_t wgs = resident_wgs();
-    if (p.x_dtype == BT_BF16) {  // (the caller has checked planes_bf16_shape_ok)
-        if (!launch_walk(p, G, wgs, -1, st)) return BT_ERR_INVALID;
-        return check_launch("gemv_planes_group");
-    }
-    {
+    const bool bf16 = p.x_dtype == BT_BF16;
+    if (!bf16) {
         const char* force = getenv("BITTORCH_GROUP_UNITS");
         if (force && force[0] == '1' && launch_units(p, G, st)) return check_launch("gemv_planes_group");
     }
-    if (launch_walk(p, G, wgs, 16, st)) return check_launch("gemv_planes_group");
-    if (launch_units(p, G, st)) return check_launch("gemv_planes_group");
+    // (bf16 units have no one-matrix kernel: the walk wherever the shape allows it, which is also the faster of their
+    // two kernels for a handful of units)
+    if (launch_walk(p, G, wgs, bf16 ? -1 : 16, st)) return check_launch("gemv_planes_group");
+    if (!bf16 && launch_units(p, G, st)) return check_launch("gemv_planes_group");
     // columns per wave: 32 (two tiles) streams best (5.3 TB/s against 4.8 with four tiles and 4.4-5.0 with one at
     // G = 128, 4096 x 4096); another width only where it fills the resident workgroups markedly more evenly
     int nacc = 2;
@@ -900,10 +915,14 @@ static int launch_group_params(PlaneParams p, int64_t G, hipStream_t st) {
     p.items = (int)(G * p.slabs);
     const unsigned grid = (unsigned)((p.items < wgs) ? p.items : wgs);
     int pf = 8;
-    if (const char* env = getenv("BITTORCH_GROUP_PF")) pf = atoi(env);
+    if (const char* env = getenv("BITTORCH_GROUP_PF")) pf = bf16 ? 8 : atoi(env);
     const int SP = (int)ceil_div(p.wsteps, pf) * pf;
     const size_t lds = 32 + (size_t)SP * 4 * PL_GROUP;
-    if (pf == 16) {
+    if (bf16) {
+        if (nacc == 4) launch_group_k<4, 8, BT_BF16>(p, grid, lds, st);
+        else if (nacc == 2) launch_group_k<2, 8, BT_BF16>(p, grid, lds, st);
+        else launch_group_k<1, 8, BT_BF16>(p, grid, lds, st);
+    } else if (pf == 16) {
         if (nacc == 4) launch_group_k<4, 16>(p, grid, lds, st);
         else if (nacc == 2) launch_group_k<2, 16>(p, grid, lds, st);
         else launch_group_k<1, 16>(p, grid, lds, st);
@@ -915,7 +934,7 @@ static int launch_group_params(PlaneParams p, int64_t G, hipStream_t st) {
     return check_launch("gemv_planes_group");
 }
 
-// bf16 rows run the contiguous-walk kernel only: K of 3..8 steps of 64 per wave (1040 <= K <= 4096, K % 16 == 0) and
+// the shapes of the contiguous-walk kernel: K of 3..8 steps of 64 per wave (1040 <= K <= 4096, K % 16 == 0) and
 // whole batches of 16-column tiles (N % 32 == 0 for K > 2048, N % 64 == 0 below)
 bool planes_bf16_shape_ok(int64_t N, int64_t K) {
     if (K % 16 != 0 || N % 4 != 0 || N <= 0 || K <= 0) return false;

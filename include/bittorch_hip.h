@@ -266,8 +266,7 @@ int bt_ternary_gemm_i8_tiled(const int8_t* Q, int q_layout, const float* s_x, co
  *   (N, or 1 = per-tensor) and element types.  x_dtype BT_F16: Y is fp16; K % 16 == 0, K <= 16384;
  *   each W_tiled 256-byte aligned, each X 16-byte aligned.  Units may share operands (one x for many
  *   matrices, one matrix for many rows) but not outputs.
- *   x_dtype BT_BF16 (Y bf16): 1040 <= K <= 4096, K % 16 == 0, N a multiple of 32 (of 64 for K <= 2048),
- *   else BT_ERR_INVALID.  A bf16 row spans more binades than a fixed-point sum can hold, so each row is
+ *   x_dtype BT_BF16 (Y bf16): the same shapes.  A bf16 row spans more binades than a fixed-point sum can hold, so each row is
  *   scaled by its own largest exponent: with E the (unbiased) exponent of the row's largest magnitude,
  *   element x becomes the integer round_half_up(|x| * 2^(39 - E)) with its sign (exact for every element
  *   whose exponent is within 32 of E, zero for those more than 40 below it), the integers are summed

@@ -296,10 +296,16 @@ def _expect_bf16(oracle, x, packed, scale, bias, k):
 @pytest.mark.parametrize("g,n,k,per_tensor,bias,spread", [(1, 4096, 4096, True, True, 0), (7, 96, 2560, False, True, 20),
                                                           (3, 2560, 2560, True, False, 45), (5, 64, 1536, False, True, 38),
                                                           (11, 4128, 3008, False, True, 0), (140, 512, 2048, False, True, 30),
-                                                          (4, 32, 4080, False, True, 60)])
+                                                          (4, 32, 4080, False, True, 60),
+                                                          # shapes outside the contiguous walk: the one-stream-per-wave kernel
+                                                          (3, 100, 144, False, True, 10), (2, 36, 8192, False, True, 50),
+                                                          (5, 2560, 6912, True, True, 0), (2, 48, 16384, False, False, 33),
+                                                          (40, 16, 64, False, True, 5), (3, 520, 1024, False, True, 25)])
 def test_grouped_bf16_units_against_the_oracle(oracle, g, n, k, per_tensor, bias, spread):
     """bf16 units of a grouped launch: bit-exact against the oracle's restatement of the row-scaled integer sum, and
-    within the reference tests' 16-bit thresholds (tests/test_packed_kernel.py:44-50) of the fp32-accumulate arithmetic."""
+    within the reference tests' 16-bit thresholds (tests/test_packed_kernel.py:44-50) of the fp32-accumulate arithmetic.
+    Where the shape allows both kernels, both run."""
+    import os
     from bittorch_amd import _C
     announce("grouped gemv bf16", g, n, k, spread)
     sets = [_setup_bf16(n, k, seed=50 * u + n, per_tensor=per_tensor, bias=bias, spread=spread) for u in range(min(g, 5))]
@@ -309,13 +315,20 @@ def test_grouped_bf16_units_against_the_oracle(oracle, g, n, k, per_tensor, bias
     tiles = [tiles_[i] for i in idx]
     scales = [sets[i][2].cuda() for i in idx]
     biases = [sets[i][3].cuda() for i in idx] if bias else None
-    ys = [torch.full((1, n), float("nan"), dtype=torch.bfloat16, device="cuda") for _ in range(g)]
-    _C.ternary_gemv_grouped(*_tables(_C, xs, tiles, scales, biases, ys), k, n, scale_len=1 if per_tensor else n,
-                            bias_dtype=torch.bfloat16, x_dtype=torch.bfloat16)
-    torch.cuda.synchronize()
     expects = [_expect_bf16(oracle, *s_, k) for s_ in sets]
-    for u in range(g):
-        assert torch.equal(ys[u].cpu(), expects[idx[u]]), u
+    try:
+        for walk in (None, "0"):
+            os.environ.pop("BITTORCH_GROUP_WALK", None)
+            if walk:
+                os.environ["BITTORCH_GROUP_WALK"] = walk
+            ys = [torch.full((1, n), float("nan"), dtype=torch.bfloat16, device="cuda") for _ in range(g)]
+            _C.ternary_gemv_grouped(*_tables(_C, xs, tiles, scales, biases, ys), k, n, scale_len=1 if per_tensor else n,
+                                    bias_dtype=torch.bfloat16, x_dtype=torch.bfloat16)
+            torch.cuda.synchronize()
+            for u in range(g):
+                assert torch.equal(ys[u].cpu(), expects[idx[u]]), (u, walk)
+    finally:
+        os.environ.pop("BITTORCH_GROUP_WALK", None)
     x, packed, scale, b = sets[0]
     ref = oracle.linear_packed(f32np(x), packed.numpy(), f32np(scale), k, None if b is None else f32np(b))
     np.testing.assert_allclose(f32np(ys[0]), ref, rtol=1e-2, atol=1e-2 * float(np.abs(ref).max()))
@@ -323,7 +336,7 @@ def test_grouped_bf16_units_against_the_oracle(oracle, g, n, k, per_tensor, bias
 
 def test_bf16_row_times_a_wide_matrix_and_argument_errors(oracle):
     """One bf16 row through the single-matrix entry point takes the same kernel where the matrix is wide enough
-    (forced here on a small one); a non-finite row gives NaN; shapes the bf16 units cannot take are refused."""
+    (forced here on a small one); a non-finite row gives NaN; bad arguments of the grouped entry point are refused."""
     import os
     from bittorch_amd import _C, _lib
     announce("bf16 wide row")
@@ -348,7 +361,7 @@ def test_bf16_row_times_a_wide_matrix_and_argument_errors(oracle):
     lib = _lib.load()
     t = torch.zeros(8, dtype=torch.int64, device="cuda")
     p = t.data_ptr()
-    assert lib.bt_ternary_gemv_grouped(p, 2, p, p, 0, 64, None, 2, p, 1, 64, 8192, None) == -1   # K beyond 4096
-    assert "bf16 units" in _lib.last_error()
-    assert lib.bt_ternary_gemv_grouped(p, 2, p, p, 0, 48, None, 2, p, 1, 48, 4096, None) == -1   # N % 32 != 0
-    assert "bf16 units" in _lib.last_error()
+    assert lib.bt_ternary_gemv_grouped(p, 2, p, p, 0, 64, None, 2, p, 1, 64, 16400, None) == -1   # K beyond 16384
+    assert "at most 16384" in _lib.last_error()
+    assert lib.bt_ternary_gemv_grouped(p, 2, p, p, 0, 48, None, 2, p, 1, 48, 4104, None) == -1    # K % 16 != 0
+    assert "multiple of 16" in _lib.last_error()
