@@ -211,20 +211,20 @@ __device__ __forceinline__ void pl_store(void* Y, const void* residual, int64_t 
 // LDS: [WAVES][2][TILE_N] int64 partial sums, [WAVES] flags, then per wave the digit planes of its K slice.
 // EPI = EPI_SWIGLU_PAIRS (tiled copy in gate/up pair order, NACC even): Y [N/2], Y[h] = rd(rd(silu(g)) * u) with
 // g = rd(linear column h), u = rd(linear column N/2 + h), what the SwiGLU kernel makes of the stored projections.
-template <int LAYOUT, int NACC, int WAVES, int PF, int EPI = EPI_NONE>
+// TAB: a few units in one launch (pointer tables, p.slabs workgroup tiles per unit).
+template <int LAYOUT, int NACC, int WAVES, int PF, int EPI = EPI_NONE, bool TAB = false>
 __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(PlaneParams p) {
     constexpr int TILE_N = 16 * NACC;
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
 
     int tile = (int)(blockIdx.x & 7) * p.per_xcd + (int)(blockIdx.x >> 3);  // neighbouring tiles on one XCD
     if (tile >= p.tiles) return;
-    // a few units in one launch (pointer tables, p.slabs workgroup tiles per unit): workgroup tile -> (unit, tile)
     const void* Xp = p.X;
     const uint8_t* Wp = p.W;
     const void* scalep = p.scale;
     const void* biasp = p.bias;
     void* Yp = p.Y;
-    if (p.W_tab) {  // uniform
+    if constexpr (TAB) {  // workgroup tile -> (unit, tile)
         const int unit = tile / p.slabs;
         tile -= unit * p.slabs;
         Xp = p.X_tab[unit];
@@ -774,7 +774,7 @@ static bool launch_walk(PlaneParams p, int64_t G, int64_t wgs, int min_tiles_per
     return true;
 }
 
-template <int LAYOUT, int NACC, int EPI = EPI_NONE>
+template <int LAYOUT, int NACC, int EPI = EPI_NONE, bool TAB = false>
 static void launch_planes_k(const PlaneParams& p, hipStream_t st) {
     // (16 or 4 waves per workgroup instead of 8: 3.72-3.74 against 3.70-3.74 us at 4096 x 4096 -- the launch is
     // bounded by its one round trip to memory, not by how the workgroup divides the work)
@@ -785,12 +785,12 @@ static void launch_planes_k(const PlaneParams& p, hipStream_t st) {
     if (lds > 64 * 1024) {  // beyond the default limit of dynamic LDS (K > 10240 or so): raise it for this kernel, once
         static bool raised = false;
         if (!raised) {
-            (void)hipFuncSetAttribute((const void*)gemv_planes_kernel<LAYOUT, NACC, WAVES, PF, EPI>,
+            (void)hipFuncSetAttribute((const void*)gemv_planes_kernel<LAYOUT, NACC, WAVES, PF, EPI, TAB>,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
             raised = true;
         }
     }
-    hipLaunchKernelGGL((gemv_planes_kernel<LAYOUT, NACC, WAVES, PF, EPI>), dim3((unsigned)(p.per_xcd * 8)), dim3(WAVES * 64), lds, st, p);
+    hipLaunchKernelGGL((gemv_planes_kernel<LAYOUT, NACC, WAVES, PF, EPI, TAB>), dim3((unsigned)(p.per_xcd * 8)), dim3(WAVES * 64), lds, st, p);
 }
 
 // epi_op = EPI_SWIGLU_PAIRS: tiled copy in gate/up pair order, N % 32 == 0, no residual; Y is [N/2]
@@ -877,9 +877,9 @@ static bool launch_units(PlaneParams p, int64_t G, hipStream_t st) {
     if (G * p.slabs > 0x3fffffff) return false;
     p.tiles = (int)(G * p.slabs);
     p.per_xcd = (int)ceil_div(p.tiles, 8);
-    if (nacc == 4) launch_planes_k<PL_TILED, 4>(p, st);
-    else if (nacc == 2) launch_planes_k<PL_TILED, 2>(p, st);
-    else launch_planes_k<PL_TILED, 1>(p, st);
+    if (nacc == 4) launch_planes_k<PL_TILED, 4, EPI_NONE, true>(p, st);
+    else if (nacc == 2) launch_planes_k<PL_TILED, 2, EPI_NONE, true>(p, st);
+    else launch_planes_k<PL_TILED, 1, EPI_NONE, true>(p, st);
     return true;
 }
 
