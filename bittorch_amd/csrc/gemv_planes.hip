@@ -31,6 +31,7 @@
 //                             workgroup): (unit, column slab) items, a wave owns 16 * NACC columns over the whole of K
 //                             (no reduction, no barrier inside an item) and keeps its weight loads running across
 //                             item boundaries.
+#include <cstddef>
 #include <cstdlib>
 
 #include "row_math.h"
@@ -43,29 +44,37 @@ constexpr int PL_GROUP = PL_N * 16;        // bytes of one 16-k group in LDS: si
 enum { PL_TILED = 0, PL_ROWMAJOR = 1 };
 
 struct PlaneParams {
+    // The first 64 bytes hold what a workgroup needs before it can request its first bytes: the kernel arguments
+    // come through the scalar cache one 64-byte line at a time, and every line is a round trip that a
+    // latency-bound launch waits for.
     // single launch: direct pointers.  grouped launch: tables of G device pointers (bias_tab may be null).
     const void* X;
     const uint8_t* W;
+    int64_t K, N;
+    int wsteps;      // 16-row steps of the weights (64 k each)
+    int tiles16;     // 16-column tiles
+    int tiles;       // single launch: workgroup tiles of 16 * NACC columns
+    int per_xcd;     // single launch: tiles per XCD (grid = 8 * per_xcd)
+    int64_t Kb;
     const void* scale;
+    // ---- second line
     const void* bias;
     const void* residual;
     void* Y;
+    int scale_dtype, bias_dtype, scale_bcast;
+    int x_dtype;     // BT_F16, or BT_BF16 (grouped launches and the contiguous walk)
+    int G;
+    int slabs;       // grouped launch: column slabs (8 waves x 16 * NACC columns) per unit, or tiles per workgroup
+    int items;       // grouped launch: G * slabs
+    int pad_[3];
+    // ---- third line
     const void* const* X_tab;
     const uint8_t* const* W_tab;
     const void* const* scale_tab;
     const void* const* bias_tab;
     void* const* Y_tab;
-    int64_t N, K, Kb;
-    int G;
-    int wsteps;      // 16-row steps of the weights (64 k each)
-    int tiles16;     // 16-column tiles
-    int tiles;       // single launch: workgroup tiles of 16 * NACC columns
-    int per_xcd;     // single launch: tiles per XCD (grid = 8 * per_xcd)
-    int slabs;       // grouped launch: column slabs (8 waves x 16 * NACC columns) per unit
-    int items;       // grouped launch: G * slabs
-    int scale_dtype, bias_dtype, scale_bcast;
-    int x_dtype;     // BT_F16, or BT_BF16 (contiguous-walk kernel only)
 };
+static_assert(offsetof(PlaneParams, scale) == 56 && offsetof(PlaneParams, X_tab) == 128, "argument lines as laid out above");
 
 // ---- fp16 -> six int8 digit planes ----------------------------------------------------------------
 // Eight consecutive fp16 values (one 16-byte load) -> per plane the eight digit bytes, elements 0..3 in
