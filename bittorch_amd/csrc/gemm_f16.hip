@@ -57,9 +57,12 @@ __device__ __forceinline__ void store4f(void* Y, int dt, int64_t idx, const floa
 }
 
 // Finishes four 16-row blocks (acc[MB0 .. MB0+3]) of the tile.
-template <int MODE, int YDT, int MB0>
+// RES: the 16-bit residual of the lane's 16 rows was requested ahead of the hand-over of the K halves (full tiles
+// only); one load per row right before its use leaves a memory round trip per row exposed, 5 us per tile.
+template <int MODE, int YDT, int MB0, bool RES = false>
 __device__ __forceinline__ void gemm_f_epilogue(const GemmFParams& p, const v4f (&acc)[F_MB][4], int64_t m0, int g,
-                                                int64_t ncol, const uint32_t (&ws_bits)[4], const uint32_t (&bs_bits)[4]) {
+                                                int64_t ncol, const uint32_t (&ws_bits)[4], const uint32_t (&bs_bits)[4],
+                                                const uint2 (&res)[4][4]) {
     float ws[4], bs[4];
 #pragma unroll
     for (int t = 0; t < 4; t++) {
@@ -79,7 +82,17 @@ __device__ __forceinline__ void gemm_f_epilogue(const GemmFParams& p, const v4f 
                 if constexpr (MODE == MODE_BF16) a *= (p.prehalved ? 1.0f : 0.5f);  // weights were decoded as +-2.0
                 y[t] = epi_float(a, ws[t], bs[t]);
             }
-            if (p.epi.residual) add_residual4(y, p.epi.residual, YDT, m * p.N + ncol);
+            if constexpr (RES && YDT != BT_F32) {  // what add_residual4 does, on the bits already here
+                const uint32_t d[2] = {res[mbi][r].x, res[mbi][r].y};
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    const uint32_t h = (d[t >> 1] >> (16 * (t & 1))) & 0xffffu;
+                    const float rv = (YDT == BT_F16) ? f16_bits_to_f32((uint16_t)h) : bf16_bits_to_f32((uint16_t)h);
+                    y[t] = sum_in_dtype(round_to_dtype(y[t], YDT), rv, YDT);
+                }
+            } else if (p.epi.residual) {
+                add_residual4(y, p.epi.residual, YDT, m * p.N + ncol);
+            }
             store4f(p.Y, YDT, m * p.N + ncol, y);
         }
     }
@@ -87,10 +100,15 @@ __device__ __forceinline__ void gemm_f_epilogue(const GemmFParams& p, const v4f 
 template <int MODE, int MB0>
 __device__ __forceinline__ void gemm_f_epilogue_dt(const GemmFParams& p, const v4f (&acc)[F_MB][4], int64_t m0,
                                                    int g, int64_t ncol, const uint32_t (&ws_bits)[4],
-                                                   const uint32_t (&bs_bits)[4]) {
-    if (p.y_dtype == BT_BF16) gemm_f_epilogue<MODE, BT_BF16, MB0>(p, acc, m0, g, ncol, ws_bits, bs_bits);
-    else if (p.y_dtype == BT_F16) gemm_f_epilogue<MODE, BT_F16, MB0>(p, acc, m0, g, ncol, ws_bits, bs_bits);
-    else gemm_f_epilogue<MODE, BT_F32, MB0>(p, acc, m0, g, ncol, ws_bits, bs_bits);
+                                                   const uint32_t (&bs_bits)[4], const uint2 (&res)[4][4], bool res_here) {
+    if (res_here) {  // uniform; 16-bit outputs only
+        if (p.y_dtype == BT_BF16) gemm_f_epilogue<MODE, BT_BF16, MB0, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
+        else gemm_f_epilogue<MODE, BT_F16, MB0, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
+        return;
+    }
+    if (p.y_dtype == BT_BF16) gemm_f_epilogue<MODE, BT_BF16, MB0>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
+    else if (p.y_dtype == BT_F16) gemm_f_epilogue<MODE, BT_F16, MB0>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
+    else gemm_f_epilogue<MODE, BT_F32, MB0>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
 }
 
 // TAIL = false: K is a multiple of the 64-wide stage and the main loop is branch free.
@@ -388,6 +406,17 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
         bs_bits[t] = p.epi.bias ? load_bits_rt(p.epi.bias, p.epi.bias_dtype, n) : 0u;
     }
 
+    // the residual of a full tile's 16-bit output: all 16 rows of the lane at once, under the rest of the hand-over
+    uint2 res_pre[4][4] = {};
+    const bool res_here = p.epi.residual && p.y_dtype != BT_F32 && m0 + F_BM <= p.M;  // uniform
+    if (res_here && col_ok) {
+        const uint16_t* rb = (const uint16_t*)p.epi.residual + (m0 + 16 * (4 * kgrp) + 4 * g) * p.N + ncol;
+#pragma unroll
+        for (int mbi = 0; mbi < 4; mbi++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) res_pre[mbi][r] = *(const uint2*)(rb + (int64_t)(16 * mbi + r) * p.N);
+    }
+
     if (kgrp == 0) {
         take(0);
         give(4);
@@ -396,8 +425,8 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     if (kgrp == 1) take(4);
 
     if (!col_ok) return;
-    if (kgrp == 0) gemm_f_epilogue_dt<MODE, 0>(p, acc, m0, g, ncol, ws_bits, bs_bits);  // wave-uniform branch
-    else gemm_f_epilogue_dt<MODE, 4>(p, acc, m0, g, ncol, ws_bits, bs_bits);
+    if (kgrp == 0) gemm_f_epilogue_dt<MODE, 0>(p, acc, m0, g, ncol, ws_bits, bs_bits, res_pre, res_here);  // wave-uniform branch
+    else gemm_f_epilogue_dt<MODE, 4>(p, acc, m0, g, ncol, ws_bits, bs_bits, res_pre, res_here);
 }
 
 // the tiled kernel reads X with 16-byte loads and W_T / Y with 4-column vectors

@@ -67,7 +67,18 @@ __device__ __forceinline__ void store4(void* Y, int dt, int64_t idx, const float
 struct EpiOperands {
     float sx[4][4];  // [row block within the half][r]
     uint32_t ws_bits[4], bs_bits[4];
+    uint2 res[4][4]; // 16-bit residual of the lane's four columns in each of its 16 rows (short epilogue only)
 };
+// The residual of a 16-bit output for the short epilogue (full tile): all 16 rows requested at once, next to the
+// other epilogue operands, so that the hand-over of the K halves covers their latency.  (One load per row right
+// before its use, as the long epilogue does, leaves a memory round trip per row exposed: 5 us per tile.)
+__device__ __forceinline__ void load_epi_residual(const GemmParams& p, int64_t m0, int mb0, int g, int64_t ncol, EpiOperands& e) {
+    const uint16_t* base = (const uint16_t*)p.epi.residual + (m0 + 16 * mb0 + 4 * g) * p.N + ncol;
+#pragma unroll
+    for (int mbi = 0; mbi < 4; mbi++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) e.res[mbi][r] = *(const uint2*)(base + (int64_t)(16 * mbi + r) * p.N);
+}
 __device__ __forceinline__ void load_epi_operands(const GemmParams& p, int64_t m0, int mb0, int g, int64_t ncol,
                                                   bool col_ok, EpiOperands& e) {
 #pragma unroll
@@ -125,7 +136,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&a
 // no residual, no accumulator output, and every row scale large enough for the two-operation division
 // (all wave-uniform, checked by the caller).  A row's address is a uniform base plus a 32-bit lane offset fixed
 // for the whole epilogue.  Same bits as gemm_epilogue.
-template <int YDT, int MB0>
+template <int YDT, int MB0, bool RES = false>
 __device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, const v4i (&acc)[G_MB][4], int64_t m0, int g,
                                                    int64_t ncol, const EpiOperands& e) {
     float ws[4], bs[4];
@@ -151,6 +162,15 @@ __device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, const v4
                 const float q = div127_fast(__fmul_rn(a127f, sx));
                 y[t] = __fadd_rn(__fmul_rn(q, ws[t]), bs[t]);
             }
+            if constexpr (RES && YDT != BT_F32) {  // linear rounded to the output's dtype, then + residual (add_residual4)
+                const uint32_t d[2] = {e.res[mbi][r].x, e.res[mbi][r].y};
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    const uint32_t h = (d[t >> 1] >> (16 * (t & 1))) & 0xffffu;
+                    const float rv = (YDT == BT_F16) ? f16_bits_to_f32((uint16_t)h) : bf16_bits_to_f32((uint16_t)h);
+                    y[t] = sum_in_dtype(round_to_dtype(y[t], YDT), rv, YDT);
+                }
+            }
             char* const dst = base + (int64_t)(16 * mbi + r) * row_bytes + lane_off;
             if constexpr (YDT == BT_F32) {
                 st4_nt((float*)dst, __builtin_bit_cast(uint32_t, y[0]), __builtin_bit_cast(uint32_t, y[1]),
@@ -175,7 +195,10 @@ template <int MB0>
 __device__ __forceinline__ void gemm_epilogue_dt(const GemmParams& p, const v4i (&acc)[G_MB][4], int64_t m0, int g,
                                                  int64_t ncol, const EpiOperands& e, bool fast) {
     if (fast) {  // wave-uniform
-        if (p.y_dtype == BT_BF16) gemm_epilogue_fast<BT_BF16, MB0>(p, acc, m0, g, ncol, e);
+        if (p.epi.residual) {  // (16-bit outputs only: checked by the caller)
+            if (p.y_dtype == BT_BF16) gemm_epilogue_fast<BT_BF16, MB0, true>(p, acc, m0, g, ncol, e);
+            else gemm_epilogue_fast<BT_F16, MB0, true>(p, acc, m0, g, ncol, e);
+        } else if (p.y_dtype == BT_BF16) gemm_epilogue_fast<BT_BF16, MB0>(p, acc, m0, g, ncol, e);
         else if (p.y_dtype == BT_F16) gemm_epilogue_fast<BT_F16, MB0>(p, acc, m0, g, ncol, e);
         else gemm_epilogue_fast<BT_F32, MB0>(p, acc, m0, g, ncol, e);
         return;
@@ -555,6 +578,9 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
 
     EpiOperands epi_ops;
     load_epi_operands(p, m0, 4 * kgrp, g, ncol, col_ok, epi_ops);
+    // what can take the short epilogue as far as the launch and the tile decide (uniform); the row scales have their say below
+    const bool short_ok = !p.long_epilogue && m0 + G_BM <= p.M && !p.acc_out && (!p.epi.residual || p.y_dtype != BT_F32);
+    if (short_ok && p.epi.residual && col_ok) load_epi_residual(p, m0, 4 * kgrp, g, ncol, epi_ops);
 
     if (kgrp == 0) {
         take_blocks(acc, 0, lds, wn, lane);   // K half 1's sums of my row blocks 0..3
@@ -569,7 +595,7 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     for (int mbi = 0; mbi < 4; mbi++)
 #pragma unroll
         for (int r = 0; r < 4; r++) small_sx |= !(__builtin_fabsf(epi_ops.sx[mbi][r]) >= DIV127_FAST_MIN_SX);
-    const bool fast = !p.long_epilogue && m0 + G_BM <= p.M && !p.epi.residual && !p.acc_out && __builtin_amdgcn_ballot_w64(small_sx) == 0ull;
+    const bool fast = short_ok && __builtin_amdgcn_ballot_w64(small_sx) == 0ull;
     if (!col_ok) return;
     if (kgrp == 0) gemm_epilogue_dt<0>(p, acc, m0, g, ncol, epi_ops, fast);  // wave-uniform branch
     else gemm_epilogue_dt<4>(p, acc, m0, g, ncol, epi_ops, fast);

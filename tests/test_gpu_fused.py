@@ -173,6 +173,31 @@ def test_residual_in_int8_gemm_equals_linear_then_add(out_dtype, b, n, k):
     assert torch.equal(fused, y + res)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("b,n,k", [(256, 512, 256), (300, 520, 192), (384, 260, 128)])
+def test_residual_in_the_tiled_gemms_full_and_ragged_tiles(dtype, b, n, k, monkeypatch):
+    """Both matrix-core GEMMs forced (batches beyond 32 rows leave the streaming kernel), on both weight layouts: full
+    128-row tiles take the epilogue that requests the residual of all their rows at once (16-bit outputs), ragged ones
+    and fp32 outputs the row-by-row one; every output equals linear-then-add bit for bit, and the int8 GEMM's two
+    epilogues agree."""
+    from bittorch_amd import _C
+    announce("residual tiled gemms", dtype, b, n, k)
+    monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
+    packed, scale, bias = _packed_case(n, k, seed=b + n + 1)
+    tiled = _C.retile_weights(packed, k)
+    x = seeded_acts(b, k, seed=7, dtype=dtype).cuda()
+    res = seeded_acts(b, n, seed=8, dtype=dtype).cuda()
+    y = _C.ternary_linear_packed_forward(x, packed, scale, bias, k)
+    assert torch.equal(_C.ternary_linear_packed_forward(x, packed, scale, bias, k, res), y + res)
+    assert torch.equal(_C.ternary_linear_tiled_forward(x, tiled, scale, bias, k, n, residual=res), y + res)
+    q, s_x = _C.act_quant_int8(x)
+    y8 = _C.ternary_gemm_int8(q, s_x, packed, scale, bias, k, dtype)
+    assert torch.equal(_C.ternary_gemm_int8(q, s_x, packed, scale, bias, k, dtype, residual=res), y8 + res)
+    assert torch.equal(_C.ternary_gemm_int8_tiled(q, s_x, tiled, scale, bias, k, n, dtype, residual=res), y8 + res)
+    monkeypatch.setenv("BITTORCH_GEMM_LONG_EPILOGUE", "1")
+    assert torch.equal(_C.ternary_gemm_int8_tiled(q, s_x, tiled, scale, bias, k, n, dtype, residual=res), y8 + res)
+
+
 def test_residual_on_the_generic_kernel(monkeypatch):
     from bittorch_amd import _C
     monkeypatch.setenv("BITTORCH_KERNEL", "generic")
