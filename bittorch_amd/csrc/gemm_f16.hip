@@ -59,7 +59,9 @@ __device__ __forceinline__ void store4f(void* Y, int dt, int64_t idx, const floa
 // Finishes four 16-row blocks (acc[MB0 .. MB0+3]) of the tile.
 // RES: the 16-bit residual of the lane's 16 rows was requested ahead of the hand-over of the K halves (full tiles
 // only); one load per row right before its use leaves a memory round trip per row exposed, 5 us per tile.
-template <int MODE, int YDT, int MB0, bool RES = false>
+// FULL: every row of the tile exists: no per-row bounds checks, and a row's address is a lane offset fixed for the whole
+// epilogue plus a uniform row term (the general form pays two quarter-rate 64-bit multiplies per row).
+template <int MODE, int YDT, int MB0, bool RES = false, bool FULL = false>
 __device__ __forceinline__ void gemm_f_epilogue(const GemmFParams& p, const v4f (&acc)[F_MB][4], int64_t m0, int g,
                                                 int64_t ncol, const uint32_t (&ws_bits)[4], const uint32_t (&bs_bits)[4],
                                                 const uint2 (&res)[4][4]) {
@@ -74,7 +76,9 @@ __device__ __forceinline__ void gemm_f_epilogue(const GemmFParams& p, const v4f 
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const int64_t m = m0 + 16 * (MB0 + mbi) + 4 * g + r;
-            if (m >= p.M) continue;
+            if constexpr (!FULL) {
+                if (m >= p.M) continue;
+            }
             float y[4];
 #pragma unroll
             for (int t = 0; t < 4; t++) {
@@ -93,7 +97,23 @@ __device__ __forceinline__ void gemm_f_epilogue(const GemmFParams& p, const v4f 
             } else if (p.epi.residual) {
                 add_residual4(y, p.epi.residual, YDT, m * p.N + ncol);
             }
-            store4f(p.Y, YDT, m * p.N + ncol, y);
+            if constexpr (FULL) {
+                constexpr int ES = (YDT == BT_F32) ? 4 : 2;
+                const int64_t ncol0 = (int64_t)__builtin_amdgcn_readfirstlane((int)(ncol / F_BN)) * F_BN;  // the tile's first column
+                const uint32_t lane_off = ((uint32_t)(4 * g) * (uint32_t)p.N + (uint32_t)(ncol - ncol0)) * ES;
+                char* const dst = (char*)p.Y + ((m0 + 16 * (MB0 + mbi) + r) * p.N + ncol0) * ES + lane_off;  // uniform + lane
+                if constexpr (YDT == BT_F32) {
+                    st4_nt((float*)dst, __builtin_bit_cast(uint32_t, y[0]), __builtin_bit_cast(uint32_t, y[1]),
+                           __builtin_bit_cast(uint32_t, y[2]), __builtin_bit_cast(uint32_t, y[3]));
+                } else {
+                    uint16_t h[4];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) h[i] = (YDT == BT_F16) ? f32_to_f16_bits(y[i]) : f32_to_bf16_bits(y[i]);
+                    st2_nt((uint16_t*)dst, (uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
+                }
+            } else {
+                store4f(p.Y, YDT, m * p.N + ncol, y);
+            }
         }
     }
 }
@@ -101,9 +121,15 @@ template <int MODE, int MB0>
 __device__ __forceinline__ void gemm_f_epilogue_dt(const GemmFParams& p, const v4f (&acc)[F_MB][4], int64_t m0,
                                                    int g, int64_t ncol, const uint32_t (&ws_bits)[4],
                                                    const uint32_t (&bs_bits)[4], const uint2 (&res)[4][4], bool res_here) {
-    if (res_here) {  // uniform; 16-bit outputs only
-        if (p.y_dtype == BT_BF16) gemm_f_epilogue<MODE, BT_BF16, MB0, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
-        else gemm_f_epilogue<MODE, BT_F16, MB0, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
+    if (res_here) {  // uniform; 16-bit outputs of a full tile
+        if (p.y_dtype == BT_BF16) gemm_f_epilogue<MODE, BT_BF16, MB0, true, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
+        else gemm_f_epilogue<MODE, BT_F16, MB0, true, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
+        return;
+    }
+    if (!p.epi.residual && m0 + F_BM <= p.M) {  // uniform: a full tile without residual
+        if (p.y_dtype == BT_BF16) gemm_f_epilogue<MODE, BT_BF16, MB0, false, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
+        else if (p.y_dtype == BT_F16) gemm_f_epilogue<MODE, BT_F16, MB0, false, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
+        else gemm_f_epilogue<MODE, BT_F32, MB0, false, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
         return;
     }
     if (p.y_dtype == BT_BF16) gemm_f_epilogue<MODE, BT_BF16, MB0>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
