@@ -61,6 +61,9 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_pack_fast_kernel(
     const int nfull = K >> 8;  // complete 256-element chunks (uniform)
     const int Kb = K >> 2;
     const float tensor_scale = per_channel ? 0.0f : fmaxf(scale[0], clamp_min);
+    // The tensor scale arrives unfloored; one thread stores the floored value.  Workgroups that read it afterwards
+    // floor it again, which changes nothing.
+    if (!per_channel && tile == 0 && threadIdx.x == 0) scale[0] = tensor_scale;
     uint32_t pk[ITERS];
 #pragma unroll
     for (int j = 0; j < ITERS; j++) pk[j] = 0;
@@ -248,6 +251,8 @@ __global__ __launch_bounds__(256) void quantize_pack_generic_kernel(
     const bool vec_ok = (K % 4 == 0) && (((uintptr_t)W) % 16 == 0);
     const bool tern_vec = vec_ok && (((uintptr_t)w_tern) % 4 == 0);
     const float tensor_scale = (per_channel || fixed_thr >= 0.0f) ? 0.0f : fmaxf(scale[0], clamp_min);
+    // (the floored value goes back; readers that come later floor it again, which changes nothing)
+    if (!per_channel && fixed_thr < 0.0f && tile == 0 && threadIdx.x == 0) scale[0] = tensor_scale;
 
     float thr[4];
 #pragma unroll
@@ -321,15 +326,20 @@ __global__ __launch_bounds__(256) void absmax_kernel(const void* __restrict__ W,
     const int64_t tid = (int64_t)blockIdx.x * 256 + threadIdx.x;
     int64_t done = 0;
     if (vec_ok) {
-        // 16-byte loads, four per thread in flight
+        // 16-byte loads, four per thread in flight; every workgroup reads its own contiguous run front to back,
+        // 4 KiB at a time.  Plain loads: the quantizing kernel reads the same bytes next and finds part of them
+        // in the memory-side cache (with the non-temporal hint here the pair of kernels takes 3 us longer).
         constexpr int EPV = (DT == BT_F32) ? 4 : 8;  // elements per 16 bytes
         const int64_t nvec = total / EPV;
         const uint4* p = (const uint4*)W;
-        for (int64_t i = tid; i < nvec; i += 4 * stride) {
+        const int64_t run = (nvec + gridDim.x - 1) / gridDim.x;
+        const int64_t first = (int64_t)blockIdx.x * run;
+        const int64_t last = (first + run < nvec) ? first + run : nvec;
+        for (int64_t i = first + threadIdx.x; i < last; i += 4 * 256) {
             uint4 q[4];
 #pragma unroll
             for (int u = 0; u < 4; u++)
-                q[u] = (i + u * stride < nvec) ? p[i + u * stride] : make_uint4(0u, 0u, 0u, 0u);
+                q[u] = (i + u * 256 < last) ? p[i + u * 256] : make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
             for (int u = 0; u < 4; u++) {
                 const uint32_t d[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
@@ -364,7 +374,6 @@ __global__ __launch_bounds__(256) void absmax_kernel(const void* __restrict__ W,
 }
 
 __global__ void set_scalar_kernel(float* p, float v) { *p = v; }
-__global__ void floor_scalar_kernel(float* p, float floor_v) { *p = fmaxf(*p, floor_v); }
 
 template <int DT>
 static int launch_quantize(const void* W, int64_t N, int64_t K, float tf, float clamp_min, int per_channel,
@@ -411,7 +420,7 @@ extern "C" int bt_quantize_pack(const void* W, int w_dtype, int64_t N, int64_t K
         clamp_min = __builtin_bit_cast(float, u);
     }
     if (!per_channel) {
-        // tensor scale: zero, absmax over everything, quantize against it, then floor it
+        // tensor scale: zero, absmax over everything; the quantizing kernel floors it, for itself and in place
         hipLaunchKernelGGL(set_scalar_kernel, dim3(1), dim3(1), 0, st, scale, 0.0f);
         const int64_t total = N * K;
         if (w_dtype == BT_F32) launch_absmax<BT_F32>(W, total, scale, st);
@@ -425,12 +434,7 @@ extern "C" int bt_quantize_pack(const void* W, int w_dtype, int64_t N, int64_t K
         rc = launch_quantize<BT_F16>(W, N, K, tf, clamp_min, per_channel, packed_T, scale, w_tern, st);
     else
         rc = launch_quantize<BT_BF16>(W, N, K, tf, clamp_min, per_channel, packed_T, scale, w_tern, st);
-    if (rc != BT_OK) return rc;
-    if (!per_channel) {
-        hipLaunchKernelGGL(floor_scalar_kernel, dim3(1), dim3(1), 0, st, scale, clamp_min);
-        return check_launch("bt_quantize_pack(floor)");
-    }
-    return BT_OK;
+    return rc;
 }
 
 extern "C" int bt_pack_ternary_i8(const int8_t* W_tern, int64_t N, int64_t K, uint8_t* packed_T, void* stream) {
