@@ -515,6 +515,15 @@ def main():
             us_g = ev_g / reps * 1e3
             by_g[f"G{gg}"] = {"us_per_launch": round(us_g, 2), "GBps": round(gg * weight_bytes / (us_g * 1e-6) / 1e9, 1),
                               "frac_of_hbm_peak": round(gg * weight_bytes / (us_g * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
+        if nsets >= 2 * G and G >= 64:
+            # twice the headline's units in one launch (every weight set: 2 G x 4 MiB, four times the Infinity Cache at G = 128)
+            g2 = 2 * G
+            tb2 = (_C.pointer_table(xs[:g2]), _C.pointer_table([l.tiled_weights() for l in layers[:g2]]),
+                   _C.pointer_table([scale] * g2), _C.pointer_table(biases[:g2]), _C.pointer_table(ys[:g2]))
+            _, ev_g = graph_time(lambda i: _C.ternary_gemv_grouped(*tb2, K, N, scale_len=1), 20, 3, torch)
+            us_g = ev_g / 20 * 1e3
+            by_g[f"G{g2}"] = {"us_per_launch": round(us_g, 2), "GBps": round(g2 * weight_bytes / (us_g * 1e-6) / 1e9, 1),
+                              "frac_of_hbm_peak": round(g2 * weight_bytes / (us_g * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
         extra["grouped_gemv_by_units_per_launch"] = by_g
 
         # the same launch on bf16 rows (each row scaled by its own largest exponent, summed as integers)
