@@ -855,6 +855,12 @@ def main():
             "us_fused_layers_and_glue": round(ev_ft / 64 * 1e3, 2),
             "packed_weight_bytes_per_block": (4 * d_model * d_model + 3 * d_model * ffn) // 4,
         }
+        # the same fused sequence on fp16 rows (config 2's dtype): every GEMV is the exact kernel, RMSNorm and SwiGLU
+        # prologues inside it
+        xt = xt.half()
+        nw = nw.half()
+        _, ev_h = graph_time(decode_fused, 64, 8, torch)
+        extra["decode_token_per_block_bf16"]["us_fused_layers_and_glue_fp16_rows"] = round(ev_h / 64 * 1e3, 2)
         del layers_
         # config 5: the 30-layer block stack, end to end
         if not args.no_block_stack:

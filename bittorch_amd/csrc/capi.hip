@@ -58,7 +58,7 @@ int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, int w_layout, c
 bool planes_supported(int x_dtype, int y_dtype, int64_t B, int64_t N, int64_t K, const void* X, const void* W, const void* Y,
                       int w_layout);
 int launch_planes(const void* X, const uint8_t* W, int w_layout, const Epilogue& epi, void* Y, int64_t N, int64_t K,
-                  int epi_op, hipStream_t st);
+                  int epi_op, hipStream_t st, int pro_op = 0, const void* pro_b = nullptr, float pro_eps = 0.0f);
 int launch_planes_group(const void* const* X_tab, int x_dtype, const uint8_t* const* W_tab, const void* const* scale_tab,
                         int scale_dtype, int scale_bcast, const void* const* bias_tab, int bias_dtype, void* const* Y_tab,
                         int64_t G, int64_t N, int64_t K, hipStream_t st);
@@ -609,8 +609,21 @@ static int fused_forward_impl(const char* who, const void* X, int64_t ld_x, int 
     // one 16-bit row on the streaming kernel: the prologue runs inside the GEMV, on the row's way into LDS
     const bool streams = (w_layout == W_LAYOUT_TILED) ? (stream_supported_tiled(N, K, W_T) && fast_path_ok(Y, N, K))
                                                       : packed_uses_stream(x_dtype, W_T, Y, N, K);
-    // (a row that takes the exact fp16 GEMV gets its prologue from the row kernel: the two then agree bit for bit
-    // with the unfused sequence by construction)
+    // a row that takes the exact fp16 GEMV gets its prologue inside that kernel (same element arithmetic as the row
+    // kernel, so the result equals the unfused sequence bit for bit), or from the row kernel where that is switched off
+    if (B == 1 && !getenv("BITTORCH_NO_PROLOGUE") && ((uintptr_t)pro_b) % 16 == 0 && pro_b &&
+        streams && planes_supported(x_dtype, x_dtype, B, N, K, X, W_T, Y, w_layout)) {
+        if (epi_op != 0 && (epi_op != EPI_SWIGLU_PAIRS || w_layout != W_LAYOUT_TILED || N % 32 != 0 || residual)) {
+            set_error("%s: the SwiGLU output stage needs pair-ordered tiled weights, N %% 32 == 0 and no residual", who);
+            return BT_ERR_INVALID;
+        }
+        Epilogue epi;
+        rc = make_epilogue(who, scale, scale_dtype, scale_len, bias, bias_dtype, N, &epi);
+        if (rc) return rc;
+        rc = set_residual(who, residual, &epi);
+        if (rc) return rc;
+        return launch_planes(X, W_T, w_layout, epi, Y, N, K, epi_op, st, pro_op, pro_b, eps);
+    }
     const size_t h_need = align256((size_t)B * K * dtype_size(x_dtype));
     const bool two_step_ok = workspace && workspace_bytes >= h_need && ((uintptr_t)workspace) % 256 == 0;
     const bool exact_row = two_step_ok && planes_supported(x_dtype, x_dtype, B, N, K, workspace, W_T, Y, w_layout);

@@ -66,13 +66,15 @@ struct PlaneParams {
     int G;
     int slabs;       // grouped launch: column slabs (8 waves x 16 * NACC columns) per unit, or tiles per workgroup
     int items;       // grouped launch: G * slabs
-    int pad_[3];
+    float pro_eps;   // one-matrix kernel with an RMSNorm prologue
+    int pad_[2];
     // ---- third line
     const void* const* X_tab;
     const uint8_t* const* W_tab;
     const void* const* scale_tab;
     const void* const* bias_tab;
     void* const* Y_tab;
+    const void* pro_b;   // one-matrix kernel with a prologue: the norm weight (RMSNorm) or the second operand (SwiGLU), K values
 };
 static_assert(offsetof(PlaneParams, scale) == 56 && offsetof(PlaneParams, X_tab) == 128, "argument lines as laid out above");
 
@@ -221,7 +223,11 @@ __device__ __forceinline__ void pl_store(void* Y, const void* residual, int64_t 
 // EPI = EPI_SWIGLU_PAIRS (tiled copy in gate/up pair order, NACC even): Y [N/2], Y[h] = rd(rd(silu(g)) * u) with
 // g = rd(linear column h), u = rd(linear column N/2 + h), what the SwiGLU kernel makes of the stored projections.
 // TAB: a few units in one launch (pointer tables, p.slabs workgroup tiles per unit).
-template <int LAYOUT, int NACC, int WAVES, int PF, int EPI = EPI_NONE, bool TAB = false>
+// PRO: the activation row is produced on its way into LDS, with the row kernels' own element arithmetic (row_math.h),
+// so that the result equals "row kernel, then GEMV" bit for bit: PRO_RMSNORM x <- rd((x * r) * w) with the row's
+// sum of squares formed in double (exact for 16-bit values of ordinary spread, hence the same whichever way the
+// waves split it; their partial sums meet in LDS, one more barrier); PRO_SWIGLU x <- rd(rd(silu(x)) * u).
+template <int LAYOUT, int NACC, int WAVES, int PF, int EPI = EPI_NONE, bool TAB = false, int PRO = PRO_NONE>
 __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(PlaneParams p) {
     constexpr int TILE_N = 16 * NACC;
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
@@ -317,6 +323,64 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(PlaneParams p) 
         }
     }
 
+    if constexpr (PRO != PRO_NONE) {
+        __shared__ double ss_slot[WAVES];
+        uint4 br[XC];  // the second operand at the same positions
+#pragma unroll
+        for (int u = 0; u < XC; u++) {
+            if (u * 64 < nchunks) {
+                const int k = s_begin * 64 + (lane + 64 * u) * 8;
+                br[u] = *(const uint4*)((const uint16_t*)p.pro_b + (uint32_t)min(k, (int)p.K - 8));
+            }
+        }
+        float r = 0.0f;
+        if constexpr (PRO == PRO_RMSNORM) {
+            double ss = 0.0;
+#pragma unroll
+            for (int u = 0; u < XC; u++) {
+                if (u * 64 < nchunks) {
+                    const int c = lane + 64 * u;
+                    const int k = s_begin * 64 + c * 8;
+                    if (k < (int)p.K && c < nchunks) {  // (a clamped chunk repeats values that another lane counts)
+                        const uint32_t d[4] = {xr[u].x, xr[u].y, xr[u].z, xr[u].w};
+#pragma unroll
+                        for (int e = 0; e < 8; e++) {
+                            const double xv = (double)f16_bits_to_f32((uint16_t)(d[e >> 1] >> (16 * (e & 1))));
+                            ss += xv * xv;
+                        }
+                    }
+                }
+            }
+            ss = wave_sum_f64(ss);
+            if (lane == 0) ss_slot[wave] = ss;
+            __syncthreads();
+            ss = 0.0;
+#pragma unroll
+            for (int w = 0; w < WAVES; w++) ss += ss_slot[w];
+            r = rms_rstd(ss, (int)p.K, p.pro_eps);
+        }
+#pragma unroll
+        for (int u = 0; u < XC; u++) {
+            if (u * 64 < nchunks) {
+                const uint32_t d[4] = {xr[u].x, xr[u].y, xr[u].z, xr[u].w};
+                const uint32_t b[4] = {br[u].x, br[u].y, br[u].z, br[u].w};
+                uint32_t o[4];
+#pragma unroll
+                for (int e2 = 0; e2 < 4; e2++) {
+                    uint32_t h2 = 0u;
+#pragma unroll
+                    for (int hf = 0; hf < 2; hf++) {
+                        const float xv = f16_bits_to_f32((uint16_t)(d[e2] >> (16 * hf)));
+                        const float bv = f16_bits_to_f32((uint16_t)(b[e2] >> (16 * hf)));
+                        const float hv = (PRO == PRO_RMSNORM) ? rmsnorm_value(xv, r, bv, BT_F16) : swiglu_value(xv, bv, BT_F16);
+                        h2 |= (uint32_t)f32_to_f16_bits(hv) << (16 * hf);
+                    }
+                    o[e2] = h2;
+                }
+                xr[u] = make_uint4(o[0], o[1], o[2], o[3]);
+            }
+        }
+    }
     bool bad = false;
 #pragma unroll
     for (int u = 0; u < XC; u++) {
@@ -783,7 +847,7 @@ static bool launch_walk(PlaneParams p, int64_t G, int64_t wgs, int min_tiles_per
     return true;
 }
 
-template <int LAYOUT, int NACC, int EPI = EPI_NONE, bool TAB = false>
+template <int LAYOUT, int NACC, int EPI = EPI_NONE, bool TAB = false, int PRO = PRO_NONE>
 static void launch_planes_k(const PlaneParams& p, hipStream_t st) {
     // (16 or 4 waves per workgroup instead of 8: 3.72-3.74 against 3.70-3.74 us at 4096 x 4096 -- the launch is
     // bounded by its one round trip to memory, not by how the workgroup divides the work)
@@ -794,18 +858,20 @@ static void launch_planes_k(const PlaneParams& p, hipStream_t st) {
     if (lds > 64 * 1024) {  // beyond the default limit of dynamic LDS (K > 10240 or so): raise it for this kernel, once
         static bool raised = false;
         if (!raised) {
-            (void)hipFuncSetAttribute((const void*)gemv_planes_kernel<LAYOUT, NACC, WAVES, PF, EPI, TAB>,
+            (void)hipFuncSetAttribute((const void*)gemv_planes_kernel<LAYOUT, NACC, WAVES, PF, EPI, TAB, PRO>,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
             raised = true;
         }
     }
-    hipLaunchKernelGGL((gemv_planes_kernel<LAYOUT, NACC, WAVES, PF, EPI, TAB>), dim3((unsigned)(p.per_xcd * 8)), dim3(WAVES * 64), lds, st, p);
+    hipLaunchKernelGGL((gemv_planes_kernel<LAYOUT, NACC, WAVES, PF, EPI, TAB, PRO>), dim3((unsigned)(p.per_xcd * 8)), dim3(WAVES * 64), lds, st, p);
 }
 
 // epi_op = EPI_SWIGLU_PAIRS: tiled copy in gate/up pair order, N % 32 == 0, no residual; Y is [N/2]
+// pro_op / pro_b / pro_eps: activation prologue (PRO_*; pro_b 16-byte aligned, K values in the row's dtype)
 int launch_planes(const void* X, const uint8_t* W, int w_layout, const Epilogue& epi, void* Y, int64_t N, int64_t K,
-                  int epi_op, hipStream_t st) {
+                  int epi_op, hipStream_t st, int pro_op, const void* pro_b, float pro_eps) {
     PlaneParams p = {};
+    p.pro_b = pro_b; p.pro_eps = pro_eps;
     p.X = X; p.W = W; p.scale = epi.scale; p.bias = epi.bias; p.residual = epi.residual; p.Y = Y;
     p.scale_dtype = epi.scale_dtype; p.bias_dtype = epi.bias_dtype; p.scale_bcast = epi.scale_bcast;
     p.x_dtype = BT_F16;
@@ -828,21 +894,35 @@ int launch_planes(const void* X, const uint8_t* W, int w_layout, const Epilogue&
             set_error("gemv_planes: the SwiGLU output stage needs pair-ordered tiled weights, N %% 32 == 0 and no residual");
             return BT_ERR_INVALID;
         }
-        if (nacc == 4) launch_planes_k<PL_TILED, 4, EPI_SWIGLU_PAIRS>(p, st);
+        if (pro_op == PRO_SWIGLU) {
+            set_error("gemv_planes: a SwiGLU prologue and the SwiGLU output stage do not combine");
+            return BT_ERR_INVALID;
+        }
+        if (pro_op == PRO_RMSNORM) {
+            if (nacc == 4) launch_planes_k<PL_TILED, 4, EPI_SWIGLU_PAIRS, false, PRO_RMSNORM>(p, st);
+            else launch_planes_k<PL_TILED, 2, EPI_SWIGLU_PAIRS, false, PRO_RMSNORM>(p, st);
+        } else if (nacc == 4) launch_planes_k<PL_TILED, 4, EPI_SWIGLU_PAIRS>(p, st);
         else launch_planes_k<PL_TILED, 2, EPI_SWIGLU_PAIRS>(p, st);
         return check_launch("gemv_planes");
     }
     // a matrix wide enough to give every resident workgroup a dozen tiles: the grouped launch's contiguous walk
     // (N = 128256, K = 4096: 26.2 against 28.0 us; N = 32768: 11.7 against 10.9)
-    if (w_layout == W_LAYOUT_TILED && launch_walk(p, 1, resident_wgs(), 12, st)) return check_launch("gemv_planes");
+    if (pro_op == PRO_NONE && w_layout == W_LAYOUT_TILED && launch_walk(p, 1, resident_wgs(), 12, st)) return check_launch("gemv_planes");
+#define BT_PL_LAUNCH(LAYOUT, NACC)                                                                       \
+    do {                                                                                                 \
+        if (pro_op == PRO_RMSNORM) launch_planes_k<LAYOUT, NACC, EPI_NONE, false, PRO_RMSNORM>(p, st);   \
+        else if (pro_op == PRO_SWIGLU) launch_planes_k<LAYOUT, NACC, EPI_NONE, false, PRO_SWIGLU>(p, st); \
+        else launch_planes_k<LAYOUT, NACC>(p, st);                                                       \
+    } while (0)
     if (w_layout == W_LAYOUT_TILED) {
-        if (nacc == 4) launch_planes_k<PL_TILED, 4>(p, st);
-        else if (nacc == 2) launch_planes_k<PL_TILED, 2>(p, st);
-        else launch_planes_k<PL_TILED, 1>(p, st);
+        if (nacc == 4) BT_PL_LAUNCH(PL_TILED, 4);
+        else if (nacc == 2) BT_PL_LAUNCH(PL_TILED, 2);
+        else BT_PL_LAUNCH(PL_TILED, 1);
     } else {
-        if (nacc == 2) launch_planes_k<PL_ROWMAJOR, 2>(p, st);
-        else launch_planes_k<PL_ROWMAJOR, 1>(p, st);
+        if (nacc == 2) BT_PL_LAUNCH(PL_ROWMAJOR, 2);
+        else BT_PL_LAUNCH(PL_ROWMAJOR, 1);
     }
+#undef BT_PL_LAUNCH
     return check_launch("gemv_planes");
 }
 

@@ -198,8 +198,9 @@ int bt_rmsnorm(const void* X, int64_t ld_x, const void* weight, float eps, int d
  *   Y = linear( pro(X) ) [+ residual],   pro = BT_PRO_RMSNORM: rmsnorm(X; weight = pro_b or ones, eps)
  *                                        pro = BT_PRO_SWIGLU:  silu(X) * pro_b   (X = gate, pro_b = up)
  * with exactly the values bt_rmsnorm / bt_swiglu would store in x_dtype.  For a single 16-bit row
- * (one decode token) the prologue runs inside the GEMV kernel, on the row's way into LDS, and saves a
- * launch; every other shape runs the prologue kernel into the workspace and then the plain forward.
+ * (one decode token) the prologue runs inside the GEMV kernel (the exact fp16 GEMV or the streaming kernel,
+ * whichever the plain forward would take), on the row's way into LDS, and saves a launch; every other
+ * shape runs the prologue kernel into the workspace and then the plain forward.
  *   X [B,K] with row stride ld_x, pro_b [K] (RMSNorm, may be NULL) or [B,K] with row stride ld_b (SwiGLU).
  *   workspace: at least bt_packed_forward_fused_workspace_bytes(B,N,K,x_dtype) bytes.
  */
