@@ -847,13 +847,22 @@ static bool launch_walk(PlaneParams p, int64_t G, int64_t wgs, int min_tiles_per
     return true;
 }
 
-template <int LAYOUT, int NACC, int EPI = EPI_NONE, bool TAB = false, int PRO = PRO_NONE>
+template <int LAYOUT, int NACC, int EPI = EPI_NONE, bool TAB = false, int PRO = PRO_NONE, int PF = 8>
 static void launch_planes_k(const PlaneParams& p, hipStream_t st) {
     // (16 or 4 waves per workgroup instead of 8: 3.72-3.74 against 3.70-3.74 us at 4096 x 4096 -- the launch is
     // bounded by its one round trip to memory, not by how the workgroup divides the work)
-    constexpr int WAVES = 8, PF = 8;
+    constexpr int WAVES = 8;
     const int nsteps = (int)ceil_div(p.K, 64);
     const int spw = (int)ceil_div(nsteps, WAVES);
+    // A wave requests PF steps of weights per batch and a batch is a round trip to memory: with more than 8 steps per wave
+    // (K > 4096) the plain tiled kernel takes its whole slice in one batch of 16 or 32 (N = 2560, K = 6912: 5.6 -> 5.1 us;
+    // N = 4096, K = 11008: 8.1 -> 7.9 us, where converting the 11008 activations in every workgroup is what is left).
+    if constexpr (PF == 8 && LAYOUT == PL_TILED && EPI == EPI_NONE && !TAB) {
+        if constexpr (NACC < 4) {  // (32 steps of four tiles would not fit the registers)
+            if (spw > 16) return launch_planes_k<LAYOUT, NACC, EPI, TAB, PRO, 32>(p, st);
+        }
+        if (spw > 8) return launch_planes_k<LAYOUT, NACC, EPI, TAB, PRO, 16>(p, st);
+    }
     const size_t lds = (size_t)WAVES * 2 * 16 * NACC * 8 + WAVES * 4 + (size_t)WAVES * spw * 4 * PL_GROUP;
     if (lds > 64 * 1024) {  // beyond the default limit of dynamic LDS (K > 10240 or so): raise it for this kernel, once
         static bool raised = false;
