@@ -18,6 +18,7 @@
 //     the two rows kb + 2g, 2g+1 and decodes each column's two bytes into eight 16-bit weights
 //     with v_perm table lookups (fp16 +-1.0; bf16 +-2.0 with the sum halved exactly).
 //   * The stage is software-pipelined inside the wave like the int8 kernel's.
+#include <cstddef>
 #include <cstdlib>
 
 #include "bt_common.h"
@@ -31,18 +32,23 @@ constexpr int F_MB = F_BM / 16;     // 16-row blocks per tile
 constexpr int F_STAGE_BYTES = F_BM * F_BK * 2;  // 16 KiB
 
 struct GemmFParams {
+    // The first 64 bytes hold what a workgroup needs to find its tile and request its first operands: the kernel
+    // arguments come through the scalar cache a 64-byte line at a time.
     const uint16_t* X;    // [M, K] fp16 or bf16 bits
     const uint8_t* W_T;   // [Kb, N]
-    void* Y;              // [M, N]
-    Epilogue epi;
-    int64_t M, N, K, Kb;  // K: length of an activation row; Kb: packed weight rows
-    int wstages;          // 64-wide stages of W_T; a stage index beyond it wraps (see launch_gemm_f16)
-    int prehalved;        // MODE_BF16: the activations already carry the factor 1/2 of the +-2.0 weight decode
-    int y_dtype;
+    int64_t K, M, N;      // K: length of an activation row
     int tiles_m, tiles_n;
     int per_xcd;          // workgroups per XCD (grid = 8 * per_xcd)
+    int wstages;          // 64-wide stages of W_T; a stage index beyond it wraps (see launch_gemm_f16)
     int tiles16;          // WT: 16-column tiles of the decode-tiled weight copy (its 16-row steps are the stages)
+    int prehalved;        // MODE_BF16: the activations already carry the factor 1/2 of the +-2.0 weight decode
+    // ---- needed later
+    void* Y;              // [M, N]
+    int64_t Kb;           // packed weight rows
+    int y_dtype;
+    Epilogue epi;
 };
+static_assert(offsetof(GemmFParams, Y) == 64, "first argument line as laid out above");
 
 __device__ __forceinline__ void store4f(void* Y, int dt, int64_t idx, const float (&v)[4]) {
     if (dt == BT_F32) {
@@ -148,15 +154,19 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
 
     // XCD-aware tile order: the 8 XCDs each take a contiguous run of tiles, walked in groups
     // of four row tiles so that one XCD's L2 holds a compact block of rows and columns
-    const int64_t lin = (int64_t)(blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
-    if (lin >= (int64_t)p.tiles_m * p.tiles_n) return;
-    constexpr int GM = 4;
-    const int64_t group = lin / (GM * p.tiles_n);
-    const int64_t first_m = group * GM;
-    const int gm = (p.tiles_m - first_m < GM) ? (int)(p.tiles_m - first_m) : GM;
-    const int64_t in_group = lin - group * GM * p.tiles_n;
-    const int tile_m = (int)(first_m + in_group % gm);
-    const int tile_n = (int)(in_group / gm);
+    // (32-bit arithmetic: the host keeps the number of tiles below 2^31, and 64-bit divisions are long
+    // instruction sequences ahead of a workgroup's first load)
+    const uint32_t lin = (blockIdx.x & 7u) * (uint32_t)p.per_xcd + (blockIdx.x >> 3);
+    const uint32_t tiles_m = (uint32_t)p.tiles_m, tiles_n = (uint32_t)p.tiles_n;
+    if (lin >= tiles_m * tiles_n) return;
+    constexpr uint32_t GM = 4;
+    const uint32_t group = lin / (GM * tiles_n);
+    const uint32_t first_m = group * GM;
+    const uint32_t gm = (tiles_m - first_m < GM) ? tiles_m - first_m : GM;
+    const uint32_t in_group = lin - group * GM * tiles_n;
+    const uint32_t tn = (gm == GM) ? in_group / GM : in_group / gm;  // (the common divisor is a shift)
+    const int tile_m = (int)(first_m + (in_group - tn * gm));
+    const int tile_n = (int)tn;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -472,7 +482,7 @@ bool gemm_f16_supported(int64_t N, int64_t K, const void* X, const void* W_T, co
 // With K % 64 != 0 the last weight stage of every plane runs past W_T's rows: the TAIL instantiation clamps them.
 int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, int w_layout, const Epilogue& epi, void* Y, int y_dtype,
                     int64_t M, int64_t N, int64_t K, int planes, hipStream_t st) {
-    GemmFParams p;
+    GemmFParams p = {};
     p.X = (const uint16_t*)X; p.W_T = W_T; p.Y = Y; p.epi = epi;
     p.M = M; p.N = N; p.K = (planes == 3) ? 3 * ceil_div(K, F_BK) * F_BK : K; p.Kb = ceil_div(K, 4);
     p.wstages = (int)ceil_div(K, F_BK);
@@ -481,6 +491,10 @@ int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, int w_layout, c
     p.tiles_m = (int)ceil_div(M, F_BM);
     p.tiles_n = (int)ceil_div(N, F_BN);
     const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
+    if (total >= (1ll << 31) - 8) {
+        set_error("gemm_f16: %lld tiles of 128 x 256 outputs are more than one launch takes", (long long)total);
+        return BT_ERR_INVALID;
+    }
     p.per_xcd = (int)ceil_div(total, 8);
     const dim3 grid((unsigned)(p.per_xcd * 8)), block(512);
     const bool tail = K % F_BK != 0;

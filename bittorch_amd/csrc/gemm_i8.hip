@@ -22,6 +22,7 @@
 //     the 4x4 bytes and decodes them in registers into the B operands of four MFMAs
 //     (one per column).
 //   * The stage is software-pipelined inside the wave (see the main loop).
+#include <cstddef>
 #include <cstdlib>
 
 #include "bt_common.h"
@@ -35,19 +36,24 @@ constexpr int G_MB = G_BM / 16;     // 16-row blocks per tile
 constexpr int G_STAGE_BYTES = G_BM * G_BK;  // 16 KiB
 
 struct GemmParams {
+    // The first 64 bytes hold what a workgroup needs to find its tile and request its first operands: the kernel
+    // arguments come through the scalar cache a 64-byte line at a time.
     const int8_t* Q;      // [M, K]
-    const float* s_x;     // [M]
     const uint8_t* W_T;   // [Kb, N]
-    void* Y;              // [M, N]
-    int32_t* acc_out;     // optional [M, N]
-    Epilogue epi;
-    int64_t M, N, K, Kb;
-    int y_dtype;
+    int64_t K, M, N;
     int tiles_m, tiles_n;
     int per_xcd;          // workgroups per XCD (grid = 8 * per_xcd)
     int wsteps, tiles16;  // WT: 16-row steps and 16-column tiles of the decode-tiled weight copy
     int long_epilogue;    // A/B runs and tests (BITTORCH_GEMM_LONG_EPILOGUE=1): never the short epilogue
+    // ---- needed later
+    const float* s_x;     // [M]
+    void* Y;              // [M, N]
+    int32_t* acc_out;     // optional [M, N]
+    int64_t Kb;
+    int y_dtype;
+    Epilogue epi;
 };
+static_assert(offsetof(GemmParams, s_x) == 64, "first argument line as laid out above");
 
 __device__ __forceinline__ void store4(void* Y, int dt, int64_t idx, const float (&v)[4]) {
     if (dt == BT_F32) {
@@ -259,15 +265,19 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     // XCD-aware tile order: the 8 XCDs each take a contiguous run of tiles, and
     // runs are walked in groups of four row tiles so that one XCD's L2 holds a
     // compact block of activation rows and weight columns.
-    const int64_t lin = (int64_t)(blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
-    if (lin >= (int64_t)p.tiles_m * p.tiles_n) return;
-    constexpr int GM = 4;
-    const int64_t group = lin / (GM * p.tiles_n);
-    const int64_t first_m = group * GM;
-    const int gm = (p.tiles_m - first_m < GM) ? (int)(p.tiles_m - first_m) : GM;
-    const int64_t in_group = lin - group * GM * p.tiles_n;
-    const int tile_m = (int)(first_m + in_group % gm);
-    const int tile_n = (int)(in_group / gm);
+    // (32-bit arithmetic: the host keeps the number of tiles below 2^31, and 64-bit divisions are long
+    // instruction sequences ahead of a workgroup's first load)
+    const uint32_t lin = (blockIdx.x & 7u) * (uint32_t)p.per_xcd + (blockIdx.x >> 3);
+    const uint32_t tiles_m = (uint32_t)p.tiles_m, tiles_n = (uint32_t)p.tiles_n;
+    if (lin >= tiles_m * tiles_n) return;
+    constexpr uint32_t GM = 4;
+    const uint32_t group = lin / (GM * tiles_n);
+    const uint32_t first_m = group * GM;
+    const uint32_t gm = (tiles_m - first_m < GM) ? tiles_m - first_m : GM;
+    const uint32_t in_group = lin - group * GM * tiles_n;
+    const uint32_t tn = (gm == GM) ? in_group / GM : in_group / gm;  // (the common divisor is a shift)
+    const int tile_m = (int)(first_m + (in_group - tn * gm));
+    const int tile_n = (int)tn;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -624,6 +634,10 @@ int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_
     p.tiles_m = (int)ceil_div(M, G_BM);
     p.tiles_n = (int)ceil_div(N, G_BN);
     const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
+    if (total >= (1ll << 31) - 8) {
+        set_error("bt_ternary_gemm_i8: %lld tiles of 128 x 256 outputs are more than one launch takes", (long long)total);
+        return BT_ERR_INVALID;
+    }
     p.per_xcd = (int)ceil_div(total, 8);
     const dim3 grid((unsigned)(p.per_xcd * 8)), block(512);
     p.wsteps = (int)ceil_div(p.Kb, 16);
