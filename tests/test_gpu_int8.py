@@ -111,6 +111,24 @@ def test_gemm_i8_epilogue_paths_agree_for_any_row_scale(oracle, out_dtype, monke
                        expect.view(torch.int16 if out_dtype != torch.float32 else torch.int32))
     assert torch.equal(y_short.cpu().view(torch.int16 if out_dtype != torch.float32 else torch.int32),
                        expect.view(torch.int16 if out_dtype != torch.float32 else torch.int32))
+    # without a bias the reference still adds 0.0f, which turns a -0 product into +0: zero, negative and tiny column
+    # scales and the negative row scale above must come out the same, sign of zero included
+    monkeypatch.delenv("BITTORCH_GEMM_LONG_EPILOGUE")
+    scale2 = scale.clone()
+    scale2[0:64] = 0.0
+    scale2[64:128] = -0.03
+    scale2[256:320] = 1e-30
+    q2 = q.clone()
+    q2[:, :] = torch.where(torch.rand(b, k, generator=g) < 0.5, q2, torch.zeros_like(q2))
+    q2[5] = 0                                                  # a zero accumulator row
+    s_ok = torch.rand(b, generator=g) * 0.05 + 1e-3
+    for sx_case in (s_ok, s_x):
+        _, oy2 = oracle.gemm_i8(q2.numpy(), f32np(sx_case), packed.numpy(), f32np(scale2), k, None)
+        e2 = torch.from_numpy(oy2).to(out_dtype)
+        y2 = _C.ternary_gemm_int8(q2.cuda(), sx_case.cuda(), packed.cuda(), scale2.cuda(), None, k, out_dtype=out_dtype)
+        torch.cuda.synchronize()
+        iv = torch.int16 if out_dtype != torch.float32 else torch.int32
+        assert torch.equal(y2.cpu().view(iv), e2.view(iv))
 
 
 def test_gemm_i8_close_to_float_path(oracle):
