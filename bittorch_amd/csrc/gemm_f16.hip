@@ -320,8 +320,12 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     };
     auto read_a = [&](int buf, int mb0, uint4 (&dst)[4]) {
         const uint8_t* a_lds = lds + buf * F_STAGE_BYTES + a_lds_off;
+        // in this order, one by one: LDS returns in order, and the first MFMA of a run needs the first row block only
 #pragma unroll
-        for (int i = 0; i < 4; i++) dst[i] = *(const uint4*)(a_lds + (mb0 + i) * 1024);
+        for (int i = 0; i < 4; i++) {
+            dst[i] = *(const uint4*)(a_lds + (mb0 + i) * 1024);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     };
     auto mfma = [&](const uint4& av, const u32x4& bv, v4f& c) {
         const u32x4 a = {av.x, av.y, av.z, av.w};

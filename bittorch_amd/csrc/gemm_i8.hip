@@ -424,8 +424,13 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     };
     auto read_a = [&](int buf, int mb0, uint4 (&dst)[4]) {
         const uint8_t* a_lds = lds + buf * G_STAGE_BYTES + a_lds_off;
+        // in this order, one by one: LDS returns in order, and the first MFMA of a run needs the first row block only
+        // (left alone, the scheduler issues the reads in descending order and the run waits for all of them)
 #pragma unroll
-        for (int i = 0; i < 4; i++) dst[i] = *(const uint4*)(a_lds + (mb0 + i) * 1024);
+        for (int i = 0; i < 4; i++) {
+            dst[i] = *(const uint4*)(a_lds + (mb0 + i) * 1024);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     };
     auto mfma_half = [&](int mb0, const uint4 (&av)[4], const v4i (&b)[4]) {
 #pragma unroll
