@@ -366,6 +366,10 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
 #pragma unroll
         for (int c = 0; c < 16; c++) mfma(a_hi[c >> 2], b_cur[c & 3], acc[4 + (c >> 2)][c & 3]);
         __builtin_amdgcn_sched_barrier(0);
+        // the fragments requested for the next stage arrived during these MFMAs: saying so here (lgkmcnt(0) alone) is free,
+        // and keeps the compiler's wait for everything outstanding across the loop edge away from the next stage's first MFMA
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        __builtin_amdgcn_sched_barrier(0);
     };
     // The two waves that share a SIMD (the K halves of one column quarter) run the stage in different orders, so
     // that one of them is inside a run of MFMAs while the other stages, loads and reads LDS: K half 1 reads all
@@ -396,6 +400,8 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     // loads outstanding)
     int s = 0;
     if (kgrp == 0) {  // wave-uniform
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the first fragments, so that the loop is entered as it is re-entered
+        __builtin_amdgcn_sched_barrier(0);
         for (; s + 1 < nstages; s += 2) {
             stage(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
             stage(s + 1, a_set[0], b_set[0], b_dec[1], b_dec[0]);

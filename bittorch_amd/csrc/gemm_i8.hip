@@ -537,6 +537,12 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
         read_a(cur ^ 1, 0, a_lo);
         mfma_half(4, a_hi, b_cur);
         __builtin_amdgcn_sched_barrier(0);
+        // The fragments just requested for the next stage arrived during these MFMAs: saying so here (lgkmcnt(0), vmcnt
+        // and expcnt untouched) costs nothing, and keeps the wait the compiler otherwise puts in front of the next stage's
+        // first MFMA -- for everything outstanding across the loop edge, the four reads issued right before it included --
+        // out of the way.
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        __builtin_amdgcn_sched_barrier(0);
     };
     // The two waves that share a SIMD (the K halves of one column quarter) run the stage in different orders, so
     // that one of them is inside a run of MFMAs while the other stages, loads and reads LDS: K half 1 reads all
@@ -573,6 +579,8 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     // puts at the top of the loop then drains the whole queue, freshly issued loads included)
     int s = 0;
     if (kgrp == 0 || !ANTIPHASE) {  // wave-uniform
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the first fragments, so that the loop is entered as it is re-entered
+        __builtin_amdgcn_sched_barrier(0);
         for (; s + 1 < nstages; s += 2) {
             stage(s, a_set[1], b_set[1], b_dec[0], b_dec[1]);
             stage(s + 1, a_set[0], b_set[0], b_dec[1], b_dec[0]);
