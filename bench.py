@@ -57,9 +57,11 @@ def parse_args():
 
 def graph_time(fn, steps, warmup, torch, min_replays=None):
     """(wall ms, event ms) for `steps` calls of fn(i) replayed as one HIP graph: the median over
-    the replays, each timed between two synchronisations.  A short graph is replayed more often
-    (at least 20 times below 200 steps), so that the fixed cost of one replay and a clock ramp do
-    not decide the figure."""
+    the timed replays, each between two synchronisations.  A graph of fewer than 200 steps is timed
+    in runs of back-to-back replays that hold at least 200 steps together (the time of a run divided
+    by its replays: the fixed cost of starting a replay, some 0.1 ms, then hides behind the replay
+    before it as it does inside a long graph), and in 20 such runs instead of 5, so that neither
+    that cost nor a clock ramp decides the figure."""
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
@@ -74,6 +76,7 @@ def graph_time(fn, steps, warmup, torch, min_replays=None):
     graph.replay()  # untimed: first replay uploads the graph
     torch.cuda.synchronize()
     replays = min_replays or (5 if steps >= 200 else 20)
+    in_a_row = 1 if steps >= 200 else -(-200 // steps)
     walls, events = [], []
     for _ in range(replays):
         e0 = torch.cuda.Event(enable_timing=True)
@@ -81,11 +84,12 @@ def graph_time(fn, steps, warmup, torch, min_replays=None):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         e0.record()
-        graph.replay()
+        for _ in range(in_a_row):
+            graph.replay()
         e1.record()
         torch.cuda.synchronize()
-        walls.append((time.perf_counter() - t0) * 1e3)
-        events.append(e0.elapsed_time(e1))
+        walls.append((time.perf_counter() - t0) * 1e3 / in_a_row)
+        events.append(e0.elapsed_time(e1) / in_a_row)
     walls.sort()
     events.sort()
     return walls[len(walls) // 2], events[len(events) // 2]
