@@ -22,6 +22,7 @@
 //     the 4x4 bytes and decodes them in registers into the B operands of four MFMAs
 //     (one per column).
 //   * The stage is software-pipelined inside the wave (see the main loop).
+#include <algorithm>
 #include <cstddef>
 #include <cstdlib>
 
@@ -44,13 +45,14 @@ struct GemmParams {
     int tiles_m, tiles_n;
     int per_xcd;          // workgroups per XCD (grid = 8 * per_xcd)
     int wsteps, tiles16;  // WT: 16-row steps and 16-column tiles of the decode-tiled weight copy
-    int long_epilogue;    // A/B runs and tests (BITTORCH_GEMM_LONG_EPILOGUE=1): never the short epilogue
+    int tile_n0;          // first column tile of this launch (tiles_n counts the launch's own column tiles)
     // ---- needed later
     const float* s_x;     // [M]
     void* Y;              // [M, N]
     int32_t* acc_out;     // optional [M, N]
     int64_t Kb;
     int y_dtype;
+    int long_epilogue;    // A/B runs and tests (BITTORCH_GEMM_LONG_EPILOGUE=1): never the short epilogue
     Epilogue epi;
 };
 static_assert(offsetof(GemmParams, s_x) == 64, "first argument line as laid out above");
@@ -67,28 +69,32 @@ __device__ __forceinline__ void store4(void* Y, int dt, int64_t idx, const float
     }
 }
 
-// Finishes four 16-row blocks (acc[MB0 .. MB0+3]) of the tile.
-// The epilogue's operands (row scales of the wave's 16 rows, column scales and biases as raw bits)
+// Finishes NB 16-row blocks (acc[MB0 .. MB0+NB-1]) of the tile: NB = 4 in a tile of 128 rows, 2 or 1 in the tiles of
+// 64 and 32 rows a launch's remainder is cut into.
+// The epilogue's operands (row scales of the wave's rows, column scales and biases as raw bits)
 // are requested before the K-half exchange, whose LDS round trips cover their latency.
+template <int NB>
 struct EpiOperands {
-    float sx[4][4];  // [row block within the half][r]
+    float sx[NB][4];  // [row block within the half][r]
     uint32_t ws_bits[4], bs_bits[4];
-    uint2 res[4][4]; // 16-bit residual of the lane's four columns in each of its 16 rows (short epilogue only)
+    uint2 res[NB][4]; // 16-bit residual of the lane's four columns in each of its rows (short epilogue only)
 };
 // The residual of a 16-bit output for the short epilogue (full tile): all 16 rows requested at once, next to the
 // other epilogue operands, so that the hand-over of the K halves covers their latency.  (One load per row right
 // before its use, as the long epilogue does, leaves a memory round trip per row exposed: 5 us per tile.)
-__device__ __forceinline__ void load_epi_residual(const GemmParams& p, int64_t m0, int mb0, int g, int64_t ncol, EpiOperands& e) {
+template <int NB>
+__device__ __forceinline__ void load_epi_residual(const GemmParams& p, int64_t m0, int mb0, int g, int64_t ncol, EpiOperands<NB>& e) {
     const uint16_t* base = (const uint16_t*)p.epi.residual + (m0 + 16 * mb0 + 4 * g) * p.N + ncol;
 #pragma unroll
-    for (int mbi = 0; mbi < 4; mbi++)
+    for (int mbi = 0; mbi < NB; mbi++)
 #pragma unroll
         for (int r = 0; r < 4; r++) e.res[mbi][r] = *(const uint2*)(base + (int64_t)(16 * mbi + r) * p.N);
 }
+template <int NB>
 __device__ __forceinline__ void load_epi_operands(const GemmParams& p, int64_t m0, int mb0, int g, int64_t ncol,
-                                                  bool col_ok, EpiOperands& e) {
+                                                  bool col_ok, EpiOperands<NB>& e) {
 #pragma unroll
-    for (int mbi = 0; mbi < 4; mbi++)
+    for (int mbi = 0; mbi < NB; mbi++)
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const int64_t m = m0 + 16 * (mb0 + mbi) + 4 * g + r;
@@ -102,9 +108,9 @@ __device__ __forceinline__ void load_epi_operands(const GemmParams& p, int64_t m
     }
 }
 
-template <int YDT, int MB0>
-__device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&acc)[G_MB][4], int64_t m0, int g,
-                                              int64_t ncol, const EpiOperands& e) {
+template <int YDT, int MB0, int NB>
+__device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&acc)[2 * NB][4], int64_t m0, int g,
+                                              int64_t ncol, const EpiOperands<NB>& e) {
     float ws[4], bs[4];
 #pragma unroll
     for (int t = 0; t < 4; t++) {
@@ -112,7 +118,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&a
         bs[t] = p.epi.bias ? bits_to_f32_rt(e.bs_bits[t], p.epi.bias_dtype) : 0.0f;
     }
 #pragma unroll
-    for (int mbi = 0; mbi < 4; mbi++) {
+    for (int mbi = 0; mbi < NB; mbi++) {
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const int64_t m = m0 + 16 * (MB0 + mbi) + 4 * g + r;
@@ -142,9 +148,9 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&a
 // no residual, no accumulator output, and every row scale large enough for the two-operation division
 // (all wave-uniform, checked by the caller).  A row's address is a uniform base plus a 32-bit lane offset fixed
 // for the whole epilogue.  Same bits as gemm_epilogue.
-template <int YDT, int MB0, bool RES = false>
-__device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, const v4i (&acc)[G_MB][4], int64_t m0, int g,
-                                                   int64_t ncol, const EpiOperands& e) {
+template <int YDT, int MB0, int NB, bool RES = false>
+__device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, const v4i (&acc)[2 * NB][4], int64_t m0, int g,
+                                                   int64_t ncol, const EpiOperands<NB>& e) {
     float ws[4], bs[4];
 #pragma unroll
     for (int t = 0; t < 4; t++) {
@@ -157,7 +163,7 @@ __device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, const v4
     char* const base = (char*)p.Y + ((m0 + 16 * MB0) * p.N + ncol0) * ES;  // uniform
     const int64_t row_bytes = p.N * ES;
 #pragma unroll
-    for (int mbi = 0; mbi < 4; mbi++) {
+    for (int mbi = 0; mbi < NB; mbi++) {
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const float sx = e.sx[mbi][r];
@@ -190,26 +196,26 @@ __device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, const v4
         }
     }
 }
-template <int MB0>
-__device__ __forceinline__ void gemm_epilogue_dt(const GemmParams& p, const v4i (&acc)[G_MB][4], int64_t m0, int g,
-                                                 int64_t ncol, const EpiOperands& e) {
-    if (p.y_dtype == BT_BF16) gemm_epilogue<BT_BF16, MB0>(p, acc, m0, g, ncol, e);
-    else if (p.y_dtype == BT_F16) gemm_epilogue<BT_F16, MB0>(p, acc, m0, g, ncol, e);
-    else gemm_epilogue<BT_F32, MB0>(p, acc, m0, g, ncol, e);
+template <int MB0, int NB>
+__device__ __forceinline__ void gemm_epilogue_dt(const GemmParams& p, const v4i (&acc)[2 * NB][4], int64_t m0, int g,
+                                                 int64_t ncol, const EpiOperands<NB>& e) {
+    if (p.y_dtype == BT_BF16) gemm_epilogue<BT_BF16, MB0, NB>(p, acc, m0, g, ncol, e);
+    else if (p.y_dtype == BT_F16) gemm_epilogue<BT_F16, MB0, NB>(p, acc, m0, g, ncol, e);
+    else gemm_epilogue<BT_F32, MB0, NB>(p, acc, m0, g, ncol, e);
 }
-template <int MB0>
-__device__ __forceinline__ void gemm_epilogue_dt(const GemmParams& p, const v4i (&acc)[G_MB][4], int64_t m0, int g,
-                                                 int64_t ncol, const EpiOperands& e, bool fast) {
+template <int MB0, int NB>
+__device__ __forceinline__ void gemm_epilogue_dt(const GemmParams& p, const v4i (&acc)[2 * NB][4], int64_t m0, int g,
+                                                 int64_t ncol, const EpiOperands<NB>& e, bool fast) {
     if (fast) {  // wave-uniform
         if (p.epi.residual) {  // (16-bit outputs only: checked by the caller)
-            if (p.y_dtype == BT_BF16) gemm_epilogue_fast<BT_BF16, MB0, true>(p, acc, m0, g, ncol, e);
-            else gemm_epilogue_fast<BT_F16, MB0, true>(p, acc, m0, g, ncol, e);
-        } else if (p.y_dtype == BT_BF16) gemm_epilogue_fast<BT_BF16, MB0>(p, acc, m0, g, ncol, e);
-        else if (p.y_dtype == BT_F16) gemm_epilogue_fast<BT_F16, MB0>(p, acc, m0, g, ncol, e);
-        else gemm_epilogue_fast<BT_F32, MB0>(p, acc, m0, g, ncol, e);
+            if (p.y_dtype == BT_BF16) gemm_epilogue_fast<BT_BF16, MB0, NB, true>(p, acc, m0, g, ncol, e);
+            else gemm_epilogue_fast<BT_F16, MB0, NB, true>(p, acc, m0, g, ncol, e);
+        } else if (p.y_dtype == BT_BF16) gemm_epilogue_fast<BT_BF16, MB0, NB>(p, acc, m0, g, ncol, e);
+        else if (p.y_dtype == BT_F16) gemm_epilogue_fast<BT_F16, MB0, NB>(p, acc, m0, g, ncol, e);
+        else gemm_epilogue_fast<BT_F32, MB0, NB>(p, acc, m0, g, ncol, e);
         return;
     }
-    gemm_epilogue_dt<MB0>(p, acc, m0, g, ncol, e);
+    gemm_epilogue_dt<MB0, NB>(p, acc, m0, g, ncol, e);
 }
 
 // Adding the two K halves: waves (wn, 0) and (wn, 1) hold partial sums of the same outputs.  K half 1 hands over row
@@ -220,22 +226,24 @@ __device__ __forceinline__ void gemm_epilogue_dt(const GemmParams& p, const v4i 
 // share and puts its own into the same slots (a lane overwrites only words it has just read itself, and the LDS
 // operations of a wave execute in order), and one more barrier later K half 1 takes it: two barriers, and one of the
 // two writes out of the way.
-__device__ __forceinline__ void give_blocks(const v4i (&acc)[G_MB][4], int mb0, uint8_t* area, int wn, int lane) {
+template <int NB>
+__device__ __forceinline__ void give_blocks(const v4i (&acc)[2 * NB][4], int mb0, uint8_t* area, int wn, int lane) {
     int32_t* xch = (int32_t*)area;
     const int slot = wn * 64 + lane;
 #pragma unroll
-    for (int mb = 0; mb < 4; mb++)
+    for (int mb = 0; mb < NB; mb++)
 #pragma unroll
         for (int t = 0; t < 4; t++) {
             const v4i v = acc[mb0 + mb][t];
             *(int4*)(xch + ((mb * 4 + t) * 256 + slot) * 4) = make_int4(v[0], v[1], v[2], v[3]);
         }
 }
-__device__ __forceinline__ void take_blocks(v4i (&acc)[G_MB][4], int mb0, const uint8_t* area, int wn, int lane) {
+template <int NB>
+__device__ __forceinline__ void take_blocks(v4i (&acc)[2 * NB][4], int mb0, const uint8_t* area, int wn, int lane) {
     const int32_t* xch = (const int32_t*)area;
     const int slot = wn * 64 + lane;
 #pragma unroll
-    for (int mb = 0; mb < 4; mb++)
+    for (int mb = 0; mb < NB; mb++)
 #pragma unroll
         for (int t = 0; t < 4; t++) {
             const int4 v = *(const int4*)(xch + ((mb * 4 + t) * 256 + slot) * 4);
@@ -258,9 +266,13 @@ __device__ __forceinline__ void take_blocks(v4i (&acc)[G_MB][4], int mb0, const 
 // (16 consecutive k of its four columns) are 16 contiguous bytes there, one load and no transpose.
 // ANTIPHASE = false (A/B runs, BITTORCH_GEMM_INPHASE=1, benchmarked variant only): both K halves run the stage in
 // the same order.
-template <bool TAIL, bool QOO, bool WT = false, bool ANTIPHASE = true>
+// NB: 16-row blocks per K half and wave: 4 is the 128-row tile; 2 and 1 are the tiles of 64 and 32 rows (same columns,
+// same staging and LDS layout with rows past the tile clamped, a quarter to half of the MFMAs per decoded weight) that a
+// launch's remainder is cut into when whole tiles would leave most compute units idle (launch_gemm_i8).
+template <bool TAIL, bool QOO, bool WT = false, bool ANTIPHASE = true, int NB = 4>
 __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[65536];  // 2 A stages; reused for the K-half exchange
+    constexpr int BM = 32 * NB;  // rows of the tile
 
     // XCD-aware tile order: the 8 XCDs each take a contiguous run of tiles, and
     // runs are walked in groups of four row tiles so that one XCD's L2 holds a
@@ -277,7 +289,7 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     const uint32_t in_group = lin - group * GM * tiles_n;
     const uint32_t tn = (gm == GM) ? in_group / GM : in_group / gm;  // (the common divisor is a shift)
     const int tile_m = (int)(first_m + (in_group - tn * gm));
-    const int tile_n = (int)tn;
+    const int tile_n = (int)tn + p.tile_n0;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -286,7 +298,7 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     const int kgrp = wave >> 2;  // k64 sub-step of each stage
     const int j = lane & 15;
     const int g = lane >> 4;
-    const int64_t m0 = (int64_t)tile_m * G_BM;
+    const int64_t m0 = (int64_t)tile_m * BM;
     const int64_t ncol = (int64_t)tile_n * G_BN + 64 * wn + 4 * j;
     const bool col_ok = ncol < p.N;
 
@@ -300,7 +312,7 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     // eight consecutive lanes write 128 contiguous bytes of LDS.
     const int a_row = 16 * wave + (lane & 15);
     const int a_part = lane >> 4;  // bytes 32*a_part .. +31 -> sub-step a_part>>1, chunks 2*(a_part&1), +1
-    const int64_t rows_left = p.M - m0;
+    const int64_t rows_left = (p.M - m0 < BM) ? p.M - m0 : BM;  // (a tile of fewer than 128 rows: the other waves stage its last row again)
     const uint32_t a_row_c = (uint32_t)((a_row < rows_left) ? a_row : rows_left - 1);
     const uint32_t a_off = a_row_c * (uint32_t)p.K + 32u * a_part;
     uint32_t b_off;
@@ -393,9 +405,9 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
         }
     };
 
-    v4i acc[G_MB][4];
+    v4i acc[2 * NB][4];
 #pragma unroll
-    for (int mb = 0; mb < G_MB; mb++)
+    for (int mb = 0; mb < 2 * NB; mb++)
 #pragma unroll
         for (int t = 0; t < 4; t++) acc[mb][t] = v4i{0, 0, 0, 0};
 
@@ -413,7 +425,7 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     // Stages past the end are clamped (loaded, never consumed) instead of branched around;
     // the loop handles two stages per trip so that the register sets are indexed statically.
     v4i b_dec[2][4];
-    uint4 a_lo[4], a_hi[4];
+    uint4 a_lo[NB], a_hi[NB];
     const uint32_t a_lds_off = (uint32_t)(kgrp * (G_MB * 1024)) + ((uint32_t)lane << 4);
     auto decode_b = [&](const uint32_t (&raw)[4], v4i (&out)[4]) {
         uint32_t G[4];
@@ -422,19 +434,19 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
 #pragma unroll
         for (int t = 0; t < 4; t++) out[t] = decode16_i8(G[t]);
     };
-    auto read_a = [&](int buf, int mb0, uint4 (&dst)[4]) {
+    auto read_a = [&](int buf, int mb0, uint4 (&dst)[NB]) {
         const uint8_t* a_lds = lds + buf * G_STAGE_BYTES + a_lds_off;
         // in this order, one by one: LDS returns in order, and the first MFMA of a run needs the first row block only
         // (left alone, the scheduler issues the reads in descending order and the run waits for all of them)
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < NB; i++) {
             dst[i] = *(const uint4*)(a_lds + (mb0 + i) * 1024);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    auto mfma_half = [&](int mb0, const uint4 (&av)[4], const v4i (&b)[4]) {
+    auto mfma_half = [&](int mb0, const uint4 (&av)[NB], const v4i (&b)[4]) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < NB; i++) {
             const v4i a = {(int)av[i].x, (int)av[i].y, (int)av[i].z, (int)av[i].w};
 #pragma unroll
             for (int t = 0; t < 4; t++)
@@ -514,17 +526,18 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
         const int cur = s & 1;
         store_a(cur ^ 1, a_reg);
         load_stage(s + 3, 1, a_reg, b_reg);
-        read_a(cur, 4, a_hi);
+        read_a(cur, NB, a_hi);
         __builtin_amdgcn_sched_barrier(0);
         // the wave that issues matrix instructions goes first on its SIMD; the other wave's staging, loads
         // and LDS traffic fill the gaps (same-run A/B: 1-3 % on every shape)
         __builtin_amdgcn_s_setprio(1);
 #pragma unroll
-        for (int c = 0; c < 16; c++) {
+        for (int c = 0; c < 4 * NB; c++) {
             const int i = c >> 2, t = c & 3;
             const v4i a = {(int)a_lo[i].x, (int)a_lo[i].y, (int)a_lo[i].z, (int)a_lo[i].w};
             acc[i][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b_cur[t], acc[i][t], 0, 0, 0);
-            decode_slice(c, b_reg, b_nxt);
+#pragma unroll
+            for (int q = 0; q < 4 / NB; q++) decode_slice(c * (4 / NB) + q, b_reg, b_nxt);  // (NB = 4: one slice)
             __builtin_amdgcn_sched_barrier(0);  // keep the slice behind its MFMA
         }
         // the raw weights are dead now: their registers take the loads of stage s+3 directly
@@ -535,7 +548,7 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
         read_a(cur ^ 1, 0, a_lo);
-        mfma_half(4, a_hi, b_cur);
+        mfma_half(NB, a_hi, b_cur);
         __builtin_amdgcn_sched_barrier(0);
         // The fragments just requested for the next stage arrived during these MFMAs: saying so here (lgkmcnt(0), vmcnt
         // and expcnt untouched) costs nothing, and keeps the wait the compiler otherwise puts in front of the next stage's
@@ -553,22 +566,23 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     auto stage_y = [&](int s, uint4 (&a_reg)[2], uint32_t (&b_reg)[4], const v4i (&b_cur)[4], v4i (&b_nxt)[4]) {
         const int cur = s & 1;
         read_a(cur, 0, a_lo);
-        read_a(cur, 4, a_hi);
+        read_a(cur, NB, a_hi);
         store_a(cur ^ 1, a_reg);
         load_stage(s + 3, 1, a_reg, b_reg);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int c = 0; c < 16; c++) {
+        for (int c = 0; c < 4 * NB; c++) {
             const int i = c >> 2, t = c & 3;
             const v4i a = {(int)a_lo[i].x, (int)a_lo[i].y, (int)a_lo[i].z, (int)a_lo[i].w};
             acc[i][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b_cur[t], acc[i][t], 0, 0, 0);
-            decode_slice(c, b_reg, b_nxt);
+#pragma unroll
+            for (int q = 0; q < 4 / NB; q++) decode_slice(c * (4 / NB) + q, b_reg, b_nxt);
             __builtin_amdgcn_sched_barrier(0);
         }
         load_stage(s + 3, 2, a_reg, b_reg);
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_setprio(1);
-        mfma_half(4, a_hi, b_cur);
+        mfma_half(NB, a_hi, b_cur);
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_setprio(0);
         __syncthreads();
@@ -596,32 +610,32 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     // K half 1 leaves the loop with nothing left to read from the stage buffers, and K half 0 holds the fragments of its
     // last MFMAs in registers (what it still reads behind the last barrier of the loop belongs to a stage that does not
     // exist and is never used): the hand-over may overwrite the buffers from here on.
-    if (kgrp == 1) give_blocks(acc, 0, lds, wn, lane);  // wave-uniform branches
+    if (kgrp == 1) give_blocks<NB>(acc, 0, lds, wn, lane);  // wave-uniform branches
     __syncthreads();
 
-    EpiOperands epi_ops;
-    load_epi_operands(p, m0, 4 * kgrp, g, ncol, col_ok, epi_ops);
+    EpiOperands<NB> epi_ops;
+    load_epi_operands<NB>(p, m0, NB * kgrp, g, ncol, col_ok, epi_ops);
     // what can take the short epilogue as far as the launch and the tile decide (uniform); the row scales have their say below
-    const bool short_ok = !p.long_epilogue && m0 + G_BM <= p.M && !p.acc_out && (!p.epi.residual || p.y_dtype != BT_F32);
-    if (short_ok && p.epi.residual && col_ok) load_epi_residual(p, m0, 4 * kgrp, g, ncol, epi_ops);
+    const bool short_ok = !p.long_epilogue && m0 + BM <= p.M && !p.acc_out && (!p.epi.residual || p.y_dtype != BT_F32);
+    if (short_ok && p.epi.residual && col_ok) load_epi_residual<NB>(p, m0, NB * kgrp, g, ncol, epi_ops);
 
     if (kgrp == 0) {
-        take_blocks(acc, 0, lds, wn, lane);   // K half 1's sums of my row blocks 0..3
-        give_blocks(acc, 4, lds, wn, lane);   // my sums of its row blocks 4..7, into the slots just read
+        take_blocks<NB>(acc, 0, lds, wn, lane);   // K half 1's sums of my row blocks 0..3 (0..NB-1)
+        give_blocks<NB>(acc, NB, lds, wn, lane);  // my sums of its row blocks 4..7 (NB..2NB-1), into the slots just read
     }
     __syncthreads();
-    if (kgrp == 1) take_blocks(acc, 4, lds, wn, lane);
+    if (kgrp == 1) take_blocks<NB>(acc, NB, lds, wn, lane);
 
     // the short epilogue where nothing needs the long one (every condition uniform over the wave)
     bool small_sx = false;
 #pragma unroll
-    for (int mbi = 0; mbi < 4; mbi++)
+    for (int mbi = 0; mbi < NB; mbi++)
 #pragma unroll
         for (int r = 0; r < 4; r++) small_sx |= !(__builtin_fabsf(epi_ops.sx[mbi][r]) >= DIV127_FAST_MIN_SX);
     const bool fast = short_ok && __builtin_amdgcn_ballot_w64(small_sx) == 0ull;
     if (!col_ok) return;
-    if (kgrp == 0) gemm_epilogue_dt<0>(p, acc, m0, g, ncol, epi_ops, fast);  // wave-uniform branch
-    else gemm_epilogue_dt<4>(p, acc, m0, g, ncol, epi_ops, fast);
+    if (kgrp == 0) gemm_epilogue_dt<0, NB>(p, acc, m0, g, ncol, epi_ops, fast);  // wave-uniform branch
+    else gemm_epilogue_dt<NB, NB>(p, acc, m0, g, ncol, epi_ops, fast);
 }
 
 
@@ -637,27 +651,38 @@ bool gemm_i8_supported(int64_t N, int64_t K, const void* Q, const void* W_T) {
            (G_BM + 1) * K < (1ll << 32) && ceil_div(K, 4) * N < (1ll << 32);
 }
 
-int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_T, int w_layout, const Epilogue& epi,
-                   void* Y, int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st) {
-    GemmParams p;
-    p.Q = Q; p.s_x = s_x; p.W_T = W_T; p.Y = Y; p.acc_out = acc_out; p.epi = epi;
-    p.M = M; p.N = N; p.K = K; p.Kb = ceil_div(K, 4);
-    p.y_dtype = y_dtype;
-    p.long_epilogue = getenv("BITTORCH_GEMM_LONG_EPILOGUE") != nullptr;
-    p.tiles_m = (int)ceil_div(M, G_BM);
-    p.tiles_n = (int)ceil_div(N, G_BN);
+// compute units of the current device (asked once per process)
+static int64_t gemm_cus() {
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cus = n;
+    }
+    return cus;
+}
+
+// One launch over column tiles [tile_n0, tile_n0 + tiles_n) in tiles of 32 * NB rows.
+template <int NB>
+static int launch_gemm_i8_part(GemmParams p, int tile_n0, int tiles_n, bool qoo, bool tiled, hipStream_t st) {
+    p.tile_n0 = tile_n0;
+    p.tiles_n = tiles_n;
+    p.tiles_m = (int)ceil_div(p.M, 32 * NB);
     const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
     if (total >= (1ll << 31) - 8) {
-        set_error("bt_ternary_gemm_i8: %lld tiles of 128 x 256 outputs are more than one launch takes", (long long)total);
+        set_error("bt_ternary_gemm_i8: %lld tiles of %d x 256 outputs are more than one launch takes", (long long)total, 32 * NB);
         return BT_ERR_INVALID;
     }
     p.per_xcd = (int)ceil_div(total, 8);
     const dim3 grid((unsigned)(p.per_xcd * 8)), block(512);
-    p.wsteps = (int)ceil_div(p.Kb, 16);
-    p.tiles16 = (int)ceil_div(N, 16);
-    const bool qoo = q_layout == Q_OPERAND_ORDER;
-    if (w_layout == W_LAYOUT_TILED) {
-        if (K % G_BK == 0) {
+    const bool tail = p.K % G_BK != 0;
+    if constexpr (NB != 4) {  // (only where launch_gemm_i8 cuts finer: tiled weights, whole stages)
+        if (qoo) hipLaunchKernelGGL((gemm_i8_kernel<false, true, true, true, NB>), grid, block, 0, st, p);
+        else hipLaunchKernelGGL((gemm_i8_kernel<false, false, true, true, NB>), grid, block, 0, st, p);
+    } else if (tiled) {
+        if (!tail) {
             if (qoo && getenv("BITTORCH_GEMM_INPHASE")) hipLaunchKernelGGL((gemm_i8_kernel<false, true, true, false>), grid, block, 0, st, p);
             else if (qoo) hipLaunchKernelGGL((gemm_i8_kernel<false, true, true>), grid, block, 0, st, p);
             else hipLaunchKernelGGL((gemm_i8_kernel<false, false, true>), grid, block, 0, st, p);
@@ -665,9 +690,7 @@ int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_
             if (qoo) hipLaunchKernelGGL((gemm_i8_kernel<true, true, true>), grid, block, 0, st, p);
             else hipLaunchKernelGGL((gemm_i8_kernel<true, false, true>), grid, block, 0, st, p);
         }
-        return check_launch("bt_ternary_gemm_i8");
-    }
-    if (K % G_BK == 0) {
+    } else if (!tail) {
         if (qoo) hipLaunchKernelGGL((gemm_i8_kernel<false, true>), grid, block, 0, st, p);
         else hipLaunchKernelGGL((gemm_i8_kernel<false, false>), grid, block, 0, st, p);
     } else {
@@ -675,6 +698,47 @@ int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_
         else hipLaunchKernelGGL((gemm_i8_kernel<true, false>), grid, block, 0, st, p);
     }
     return check_launch("bt_ternary_gemm_i8");
+}
+
+int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_T, int w_layout, const Epilogue& epi,
+                   void* Y, int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st) {
+    GemmParams p = {};
+    p.Q = Q; p.s_x = s_x; p.W_T = W_T; p.Y = Y; p.acc_out = acc_out; p.epi = epi;
+    p.M = M; p.N = N; p.K = K; p.Kb = ceil_div(K, 4);
+    p.y_dtype = y_dtype;
+    p.long_epilogue = getenv("BITTORCH_GEMM_LONG_EPILOGUE") != nullptr;
+    p.wsteps = (int)ceil_div(p.Kb, 16);
+    p.tiles16 = (int)ceil_div(N, 16);
+    const bool qoo = q_layout == Q_OPERAND_ORDER, tiled = w_layout == W_LAYOUT_TILED;
+    const int64_t tiles_m = ceil_div(M, G_BM), tiles_n = ceil_div(N, G_BN), total = tiles_m * tiles_n;
+
+    // The remainder of a launch.  Workgroups take tiles in rounds of one per compute unit; when the last round holds
+    // tiles for at most half of the compute units, the column tiles of that remainder are computed in tiles of 64 or 32
+    // rows instead, two or four workgroups where there was one, in a launch of their own behind the whole tiles (same
+    // sums, same bits; a finer tile does fewer MFMAs per decoded weight, so it only pays where the alternative is idle
+    // compute units).  Cost in rounds of whole tiles, as measured: a round of half tiles 0.85, of quarter tiles 0.75 (a
+    // stage of so few MFMAs is bound by its chain of LDS read, decode and barrier, not by the matrix cores), a launch 0.1.
+    // M = 4096, N = 2560: K = 2560 36.5 -> 32.8 us, K = 6912 74.9 -> 67.3 us; N = K = 4096: M = 1024 23.9 -> 19.8 us,
+    // M = 512 23.5 -> 15.6 us.  BITTORCH_GEMM_TAIL_SPLIT=0 (tests, A/B runs): never.
+    const char* split_env = getenv("BITTORCH_GEMM_TAIL_SPLIT");
+    if (tiled && K % G_BK == 0 && !(split_env && split_env[0] == '0') && !getenv("BITTORCH_GEMM_INPHASE")) {
+        const int64_t C = gemm_cus(), rem = total % C;
+        if (rem != 0 && 2 * rem <= C) {
+            const int nb = (4 * rem <= C) ? 1 : 2;
+            const int64_t cols = std::min(tiles_n, ceil_div(rem, tiles_m));  // column tiles cut finer
+            const int64_t whole = tiles_m * (tiles_n - cols), fine = ceil_div(M, 32 * nb) * cols;
+            const double split = (double)ceil_div(whole, C) + (double)ceil_div(fine, C) * (nb == 1 ? 0.75 : 0.85) + (whole ? 0.1 : 0.0);
+            if (split < (double)ceil_div(total, C) - 0.04) {
+                if (whole) {
+                    const int rc = launch_gemm_i8_part<4>(p, 0, (int)(tiles_n - cols), qoo, tiled, st);
+                    if (rc) return rc;
+                }
+                return nb == 1 ? launch_gemm_i8_part<1>(p, (int)(tiles_n - cols), (int)cols, qoo, tiled, st)
+                               : launch_gemm_i8_part<2>(p, (int)(tiles_n - cols), (int)cols, qoo, tiled, st);
+            }
+        }
+    }
+    return launch_gemm_i8_part<4>(p, 0, (int)tiles_n, qoo, tiled, st);
 }
 
 }  // namespace bt

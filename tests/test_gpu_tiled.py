@@ -142,6 +142,50 @@ def test_tiled_int8_equals_row_major(oracle, n, k, route, monkeypatch):
             assert torch.equal(a1, a0) and torch.equal(y1, y0)
 
 
+# (M, N, K) whose 128 x 256 tiles leave most of a 256-unit chip idle in their last round, so that the launch cuts
+# the remainder finer: 320 tiles (256 whole + 64 as 256 tiles of 32 rows), 128 tiles (as 256 of 64 rows), 64 tiles (as
+# 256 of 32 rows); the same with ragged last row tiles, ragged columns and several stages of K
+REMAINDER_SHAPES = [(4096, 2560, 256), (1024, 4096, 128), (512, 4096, 384), (1000, 4096, 256), (500, 4096, 128),
+                    (512, 4000, 128), (4090, 2560, 128)]
+
+
+@pytest.mark.parametrize("m,n,k", REMAINDER_SHAPES)
+def test_tiled_int8_remainder_in_finer_tiles(oracle, m, n, k, monkeypatch):
+    """The prefill GEMM computes the column tiles of a mostly empty last round in tiles of 64 or 32 rows
+    (a second launch behind the whole tiles).  Same bits as one launch of whole tiles -- outputs and int32
+    accumulators, both activation layouts, bias, residual, 16-bit and fp32 outputs -- and equal to the oracle on
+    row slices at the start, across tile borders and at the ragged end."""
+    from bittorch_amd import _C
+    monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
+    _, wt = _packed(oracle, n, k, seed=m % 7)
+    tiled = _C.retile_weights(wt, k)
+    g = torch.Generator().manual_seed(m + n)
+    scale = torch.rand(n, generator=g) * 0.05 + 0.01
+    bias = torch.randn(n, generator=g) * 0.01
+    x = seeded_acts(m, k, seed=m + k, dtype=torch.bfloat16, outliers=True)
+    res = seeded_acts(m, n, seed=m + 1, dtype=torch.bfloat16).cuda()
+    oq, os_ = oracle.act_quant_i8(f32np(x))
+    slices = [(0, min(m, 40)), (max(0, m // 2 - 20), min(m, m // 2 + 20)), (max(0, m - 40), m)]
+    for oo in (False, True):
+        announce("remainder tiles", m, n, k, oo)
+        q, s = _C.act_quant_int8(x.cuda(), oo)
+        outs = {}
+        for split in ("0", "1"):
+            monkeypatch.setenv("BITTORCH_GEMM_TAIL_SPLIT", split)
+            y32, acc = _C.ternary_gemm_int8_tiled(q, s, tiled, scale.cuda(), bias.cuda(), k, n, torch.float32, True, None, oo)
+            y16 = _C.ternary_gemm_int8_tiled(q, s, tiled, scale.cuda(), None, k, n, torch.bfloat16, False, res, oo)
+            y16b = _C.ternary_gemm_int8_tiled(q, s, tiled, scale.cuda(), bias.cuda(), k, n, torch.float16, False, None, oo)
+            outs[split] = (y32, acc, y16, y16b)
+        torch.cuda.synchronize()
+        for a, b in zip(outs["0"], outs["1"]):
+            assert torch.equal(a, b)
+        y32, acc = outs["1"][0].cpu().numpy(), outs["1"][1].cpu().numpy()
+        for r0, r1 in slices:
+            oacc, oy = oracle.gemm_i8(oq[r0:r1], os_[r0:r1], wt.cpu().numpy(), f32np(scale), k, f32np(bias))
+            np.testing.assert_array_equal(acc[r0:r1], oacc)
+            np.testing.assert_array_equal(y32[r0:r1], oy)
+
+
 def test_tiled_forward_against_oracle(oracle):
     from bittorch_amd import _C
     n, k = 300, 520
