@@ -18,6 +18,7 @@
 //     the two rows kb + 2g, 2g+1 and decodes each column's two bytes into eight 16-bit weights
 //     with v_perm table lookups (fp16 +-1.0; bf16 +-2.0 with the sum halved exactly).
 //   * The stage is software-pipelined inside the wave like the int8 kernel's.
+#include <algorithm>
 #include <cstddef>
 #include <cstdlib>
 
@@ -41,11 +42,12 @@ struct GemmFParams {
     int per_xcd;          // workgroups per XCD (grid = 8 * per_xcd)
     int wstages;          // 64-wide stages of W_T; a stage index beyond it wraps (see launch_gemm_f16)
     int tiles16;          // WT: 16-column tiles of the decode-tiled weight copy (its 16-row steps are the stages)
-    int prehalved;        // MODE_BF16: the activations already carry the factor 1/2 of the +-2.0 weight decode
+    int tile_n0;          // first column tile of this launch (tiles_n counts the launch's own column tiles)
     // ---- needed later
     void* Y;              // [M, N]
     int64_t Kb;           // packed weight rows
     int y_dtype;
+    int prehalved;        // MODE_BF16: the activations already carry the factor 1/2 of the +-2.0 weight decode
     Epilogue epi;
 };
 static_assert(offsetof(GemmFParams, Y) == 64, "first argument line as laid out above");
@@ -62,15 +64,16 @@ __device__ __forceinline__ void store4f(void* Y, int dt, int64_t idx, const floa
     }
 }
 
-// Finishes four 16-row blocks (acc[MB0 .. MB0+3]) of the tile.
+// Finishes NB 16-row blocks (acc[MB0 .. MB0+NB-1]) of the tile: NB = 4 in a tile of 128 rows, 2 or 1 in the tiles of 64
+// and 32 rows a launch's remainder is cut into.
 // RES: the 16-bit residual of the lane's 16 rows was requested ahead of the hand-over of the K halves (full tiles
 // only); one load per row right before its use leaves a memory round trip per row exposed, 5 us per tile.
 // FULL: every row of the tile exists: no per-row bounds checks, and a row's address is a lane offset fixed for the whole
 // epilogue plus a uniform row term (the general form pays two quarter-rate 64-bit multiplies per row).
-template <int MODE, int YDT, int MB0, bool RES = false, bool FULL = false>
-__device__ __forceinline__ void gemm_f_epilogue(const GemmFParams& p, const v4f (&acc)[F_MB][4], int64_t m0, int g,
+template <int MODE, int YDT, int MB0, int NB, bool RES = false, bool FULL = false>
+__device__ __forceinline__ void gemm_f_epilogue(const GemmFParams& p, const v4f (&acc)[2 * NB][4], int64_t m0, int g,
                                                 int64_t ncol, const uint32_t (&ws_bits)[4], const uint32_t (&bs_bits)[4],
-                                                const uint2 (&res)[4][4]) {
+                                                const uint2 (&res)[NB][4]) {
     float ws[4], bs[4];
 #pragma unroll
     for (int t = 0; t < 4; t++) {
@@ -78,7 +81,7 @@ __device__ __forceinline__ void gemm_f_epilogue(const GemmFParams& p, const v4f 
         bs[t] = p.epi.bias ? bits_to_f32_rt(bs_bits[t], p.epi.bias_dtype) : 0.0f;
     }
 #pragma unroll
-    for (int mbi = 0; mbi < 4; mbi++) {
+    for (int mbi = 0; mbi < NB; mbi++) {
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const int64_t m = m0 + 16 * (MB0 + mbi) + 4 * g + r;
@@ -123,33 +126,37 @@ __device__ __forceinline__ void gemm_f_epilogue(const GemmFParams& p, const v4f 
         }
     }
 }
-template <int MODE, int MB0>
-__device__ __forceinline__ void gemm_f_epilogue_dt(const GemmFParams& p, const v4f (&acc)[F_MB][4], int64_t m0,
+template <int MODE, int MB0, int NB>
+__device__ __forceinline__ void gemm_f_epilogue_dt(const GemmFParams& p, const v4f (&acc)[2 * NB][4], int64_t m0,
                                                    int g, int64_t ncol, const uint32_t (&ws_bits)[4],
-                                                   const uint32_t (&bs_bits)[4], const uint2 (&res)[4][4], bool res_here) {
+                                                   const uint32_t (&bs_bits)[4], const uint2 (&res)[NB][4], bool res_here) {
     if (res_here) {  // uniform; 16-bit outputs of a full tile
-        if (p.y_dtype == BT_BF16) gemm_f_epilogue<MODE, BT_BF16, MB0, true, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
-        else gemm_f_epilogue<MODE, BT_F16, MB0, true, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
+        if (p.y_dtype == BT_BF16) gemm_f_epilogue<MODE, BT_BF16, MB0, NB, true, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
+        else gemm_f_epilogue<MODE, BT_F16, MB0, NB, true, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
         return;
     }
-    if (!p.epi.residual && m0 + F_BM <= p.M) {  // uniform: a full tile without residual
-        if (p.y_dtype == BT_BF16) gemm_f_epilogue<MODE, BT_BF16, MB0, false, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
-        else if (p.y_dtype == BT_F16) gemm_f_epilogue<MODE, BT_F16, MB0, false, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
-        else gemm_f_epilogue<MODE, BT_F32, MB0, false, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
+    if (!p.epi.residual && m0 + 32 * NB <= p.M) {  // uniform: a full tile without residual
+        if (p.y_dtype == BT_BF16) gemm_f_epilogue<MODE, BT_BF16, MB0, NB, false, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
+        else if (p.y_dtype == BT_F16) gemm_f_epilogue<MODE, BT_F16, MB0, NB, false, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
+        else gemm_f_epilogue<MODE, BT_F32, MB0, NB, false, true>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
         return;
     }
-    if (p.y_dtype == BT_BF16) gemm_f_epilogue<MODE, BT_BF16, MB0>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
-    else if (p.y_dtype == BT_F16) gemm_f_epilogue<MODE, BT_F16, MB0>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
-    else gemm_f_epilogue<MODE, BT_F32, MB0>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
+    if (p.y_dtype == BT_BF16) gemm_f_epilogue<MODE, BT_BF16, MB0, NB>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
+    else if (p.y_dtype == BT_F16) gemm_f_epilogue<MODE, BT_F16, MB0, NB>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
+    else gemm_f_epilogue<MODE, BT_F32, MB0, NB>(p, acc, m0, g, ncol, ws_bits, bs_bits, res);
 }
 
 // TAIL = false: K is a multiple of the 64-wide stage and the main loop is branch free.
 // TAIL = true: any K % 8 == 0; the last, partial stage is masked.
 // WT = true: W_T is the decode-tiled copy (W_LAYOUT_TILED): the dwords of a lane's four columns in its step are
 // 16 contiguous bytes (one load instead of two), of which the k32 sub-step uses two bytes each.
-template <int MODE, bool TAIL, bool WT = false>
+// NB: 16-row blocks per K half and wave: 4 is the 128-row tile; 2 and 1 are the tiles of 64 and 32 rows (same columns,
+// same staging and LDS layout with rows past the tile clamped) that a launch's remainder is cut into when whole tiles
+// would leave most compute units idle (launch_gemm_f16).
+template <int MODE, bool TAIL, bool WT = false, int NB = 4>
 __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     constexpr int BR = WT ? 4 : 2;  // raw weight dwords per lane and stage
+    constexpr int BM = 32 * NB;     // rows of the tile
     __shared__ __attribute__((aligned(16))) uint8_t lds[65536];  // 2 A stages; reused for the K-half exchange
 
     // XCD-aware tile order: the 8 XCDs each take a contiguous run of tiles, walked in groups
@@ -166,7 +173,7 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     const uint32_t in_group = lin - group * GM * tiles_n;
     const uint32_t tn = (gm == GM) ? in_group / GM : in_group / gm;  // (the common divisor is a shift)
     const int tile_m = (int)(first_m + (in_group - tn * gm));
-    const int tile_n = (int)tn;
+    const int tile_n = (int)tn + p.tile_n0;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -175,7 +182,7 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     const int kgrp = wave >> 2;  // k32 sub-step of each stage
     const int j = lane & 15;
     const int g = lane >> 4;
-    const int64_t m0 = (int64_t)tile_m * F_BM;
+    const int64_t m0 = (int64_t)tile_m * BM;
     const int64_t ncol = (int64_t)tile_n * F_BN + 64 * wn + 4 * j;
     const bool col_ok = ncol < p.N;
 
@@ -188,7 +195,7 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     // contiguous bytes of LDS.
     const int a_row = 16 * wave + (lane & 15);
     const int a_part = lane >> 4;  // values 16*a_part .. +15 -> sub-step a_part>>1, groups 2*(a_part&1), +1
-    const int64_t rows_left = p.M - m0;
+    const int64_t rows_left = (p.M - m0 < BM) ? p.M - m0 : BM;  // (a tile of fewer than 128 rows: the other waves stage its last row again)
     const uint32_t a_row_c = (uint32_t)((a_row < rows_left) ? a_row : rows_left - 1);
     const uint32_t a_off = (a_row_c * (uint32_t)p.K + 16u * a_part) * 2u;  // bytes
     uint32_t b_off;
@@ -292,9 +299,9 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
         }
     };
 
-    v4f acc[F_MB][4];
+    v4f acc[2 * NB][4];
 #pragma unroll
-    for (int mb = 0; mb < F_MB; mb++)
+    for (int mb = 0; mb < 2 * NB; mb++)
 #pragma unroll
         for (int t = 0; t < 4; t++) acc[mb][t] = v4f{0.f, 0.f, 0.f, 0.f};
 
@@ -306,7 +313,7 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     // them; the stage's one barrier publishes buffer (s+1)%2, whose row blocks 0..3 are
     // requested right behind it and arrive under the MFMAs of row blocks 4..7.
     u32x4 b_dec[2][4];
-    uint4 a_lo[4], a_hi[4];
+    uint4 a_lo[NB], a_hi[NB];
     const uint32_t a_lds_off = (uint32_t)(kgrp * (F_MB * 1024)) + ((uint32_t)lane << 4);
     constexpr uint32_t LUT = (MODE == MODE_F16) ? LUT_F16_ONE : LUT_BF16_TWO;
     auto decode_col = [&](const uint32_t (&raw)[BR], int t, u32x4& out) {
@@ -318,11 +325,11 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
             out = decode8_16bit<LUT>(perm(raw[1], raw[0], sel));
         }
     };
-    auto read_a = [&](int buf, int mb0, uint4 (&dst)[4]) {
+    auto read_a = [&](int buf, int mb0, uint4 (&dst)[NB]) {
         const uint8_t* a_lds = lds + buf * F_STAGE_BYTES + a_lds_off;
         // in this order, one by one: LDS returns in order, and the first MFMA of a run needs the first row block only
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < NB; i++) {
             dst[i] = *(const uint4*)(a_lds + (mb0 + i) * 1024);
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -349,12 +356,12 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
         const int cur = s & 1;
         store_a(cur ^ 1, a_reg);
         load_stage(s + 3, 1, a_reg, b_reg);
-        read_a(cur, 4, a_hi);
+        read_a(cur, NB, a_hi);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int c = 0; c < 16; c++) {
+        for (int c = 0; c < 4 * NB; c++) {
             mfma(a_lo[c >> 2], b_cur[c & 3], acc[c >> 2][c & 3]);
-            if ((c & 3) == 1) decode_col(b_reg, c >> 2, b_nxt[c >> 2]);  // one column behind every fourth MFMA
+            if (c % NB == (NB > 1 ? 1 : 0)) decode_col(b_reg, c / NB, b_nxt[c / NB]);  // one column behind every fourth MFMA (NB = 4)
             __builtin_amdgcn_sched_barrier(0);
         }
         // the raw weights are dead now: their registers take the loads of stage s+3 directly
@@ -364,7 +371,7 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
         __builtin_amdgcn_sched_barrier(0);
         read_a(cur ^ 1, 0, a_lo);
 #pragma unroll
-        for (int c = 0; c < 16; c++) mfma(a_hi[c >> 2], b_cur[c & 3], acc[4 + (c >> 2)][c & 3]);
+        for (int c = 0; c < 4 * NB; c++) mfma(a_hi[c >> 2], b_cur[c & 3], acc[NB + (c >> 2)][c & 3]);
         __builtin_amdgcn_sched_barrier(0);
         // the fragments requested for the next stage arrived during these MFMAs: saying so here (lgkmcnt(0) alone) is free,
         // and keeps the compiler's wait for everything outstanding across the loop edge away from the next stage's first MFMA
@@ -378,20 +385,20 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     auto stage_y = [&](int s, uint4 (&a_reg)[2], uint32_t (&b_reg)[BR], const u32x4 (&b_cur)[4], u32x4 (&b_nxt)[4]) {
         const int cur = s & 1;
         read_a(cur, 0, a_lo);
-        read_a(cur, 4, a_hi);
+        read_a(cur, NB, a_hi);
         store_a(cur ^ 1, a_reg);
         load_stage(s + 3, 1, a_reg, b_reg);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int c = 0; c < 16; c++) {
+        for (int c = 0; c < 4 * NB; c++) {
             mfma(a_lo[c >> 2], b_cur[c & 3], acc[c >> 2][c & 3]);
-            if ((c & 3) == 1) decode_col(b_reg, c >> 2, b_nxt[c >> 2]);
+            if (c % NB == (NB > 1 ? 1 : 0)) decode_col(b_reg, c / NB, b_nxt[c / NB]);
             __builtin_amdgcn_sched_barrier(0);
         }
         load_stage(s + 3, 2, a_reg, b_reg);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int c = 0; c < 16; c++) mfma(a_hi[c >> 2], b_cur[c & 3], acc[4 + (c >> 2)][c & 3]);
+        for (int c = 0; c < 4 * NB; c++) mfma(a_hi[c >> 2], b_cur[c & 3], acc[NB + (c >> 2)][c & 3]);
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
@@ -424,7 +431,7 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     const int slot = wn * 64 + lane;
     auto give = [&](int mb0) {
 #pragma unroll
-        for (int mb = 0; mb < 4; mb++)
+        for (int mb = 0; mb < NB; mb++)
 #pragma unroll
             for (int t = 0; t < 4; t++) {
                 const v4f v = acc[mb0 + mb][t];
@@ -433,7 +440,7 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     };
     auto take = [&](int mb0) {
 #pragma unroll
-        for (int mb = 0; mb < 4; mb++)
+        for (int mb = 0; mb < NB; mb++)
 #pragma unroll
             for (int t = 0; t < 4; t++) {
                 const float4 v = *(const float4*)(xch + ((mb * 4 + t) * 256 + slot) * 4);
@@ -453,26 +460,26 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     }
 
     // the residual of a full tile's 16-bit output: all 16 rows of the lane at once, under the rest of the hand-over
-    uint2 res_pre[4][4] = {};
-    const bool res_here = p.epi.residual && p.y_dtype != BT_F32 && m0 + F_BM <= p.M;  // uniform
+    uint2 res_pre[NB][4] = {};
+    const bool res_here = p.epi.residual && p.y_dtype != BT_F32 && m0 + BM <= p.M;  // uniform
     if (res_here && col_ok) {
-        const uint16_t* rb = (const uint16_t*)p.epi.residual + (m0 + 16 * (4 * kgrp) + 4 * g) * p.N + ncol;
+        const uint16_t* rb = (const uint16_t*)p.epi.residual + (m0 + 16 * (NB * kgrp) + 4 * g) * p.N + ncol;
 #pragma unroll
-        for (int mbi = 0; mbi < 4; mbi++)
+        for (int mbi = 0; mbi < NB; mbi++)
 #pragma unroll
             for (int r = 0; r < 4; r++) res_pre[mbi][r] = *(const uint2*)(rb + (int64_t)(16 * mbi + r) * p.N);
     }
 
     if (kgrp == 0) {
         take(0);
-        give(4);
+        give(NB);
     }
     __syncthreads();
-    if (kgrp == 1) take(4);
+    if (kgrp == 1) take(NB);
 
     if (!col_ok) return;
-    if (kgrp == 0) gemm_f_epilogue_dt<MODE, 0>(p, acc, m0, g, ncol, ws_bits, bs_bits, res_pre, res_here);  // wave-uniform branch
-    else gemm_f_epilogue_dt<MODE, 4>(p, acc, m0, g, ncol, ws_bits, bs_bits, res_pre, res_here);
+    if (kgrp == 0) gemm_f_epilogue_dt<MODE, 0, NB>(p, acc, m0, g, ncol, ws_bits, bs_bits, res_pre, res_here);  // wave-uniform branch
+    else gemm_f_epilogue_dt<MODE, NB, NB>(p, acc, m0, g, ncol, ws_bits, bs_bits, res_pre, res_here);
 }
 
 // the tiled kernel reads X with 16-byte loads and W_T / Y with 4-column vectors
@@ -490,26 +497,36 @@ bool gemm_f16_supported(int64_t N, int64_t K, const void* X, const void* W_T, co
 // planes = 1: X is [M, K].  planes = 3: X is [M, 3*Kp], Kp = K rounded up to 64, three zero-padded planes of K
 // values per row whose products with the same weights are summed (fp32 activations split into three bf16 terms).
 // With K % 64 != 0 the last weight stage of every plane runs past W_T's rows: the TAIL instantiation clamps them.
-int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, int w_layout, const Epilogue& epi, void* Y, int y_dtype,
-                    int64_t M, int64_t N, int64_t K, int planes, hipStream_t st) {
-    GemmFParams p = {};
-    p.X = (const uint16_t*)X; p.W_T = W_T; p.Y = Y; p.epi = epi;
-    p.M = M; p.N = N; p.K = (planes == 3) ? 3 * ceil_div(K, F_BK) * F_BK : K; p.Kb = ceil_div(K, 4);
-    p.wstages = (int)ceil_div(K, F_BK);
-    p.prehalved = planes == 3;
-    p.y_dtype = y_dtype;
-    p.tiles_m = (int)ceil_div(M, F_BM);
-    p.tiles_n = (int)ceil_div(N, F_BN);
+static int64_t gemm_f_cus() {  // compute units of the current device (asked once per process)
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cus = n;
+    }
+    return cus;
+}
+
+// One launch over column tiles [tile_n0, tile_n0 + tiles_n) in tiles of 32 * NB rows.
+template <int NB>
+static int launch_gemm_f16_part(GemmFParams p, int mode, int tile_n0, int tiles_n, bool tiled, bool tail, hipStream_t st) {
+    p.tile_n0 = tile_n0;
+    p.tiles_n = tiles_n;
+    p.tiles_m = (int)ceil_div(p.M, 32 * NB);
     const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
     if (total >= (1ll << 31) - 8) {
-        set_error("gemm_f16: %lld tiles of 128 x 256 outputs are more than one launch takes", (long long)total);
+        set_error("gemm_f16: %lld tiles of %d x 256 outputs are more than one launch takes", (long long)total, 32 * NB);
         return BT_ERR_INVALID;
     }
     p.per_xcd = (int)ceil_div(total, 8);
     const dim3 grid((unsigned)(p.per_xcd * 8)), block(512);
-    const bool tail = K % F_BK != 0;
-    p.tiles16 = (int)ceil_div(N, 16);
-    if (w_layout == W_LAYOUT_TILED) {
+    if constexpr (NB != 4) {  // (only where launch_gemm_f16 cuts finer: tiled weights, whole stages)
+        if (mode == MODE_F16) hipLaunchKernelGGL((gemm_f16_kernel<MODE_F16, false, true, NB>), grid, block, 0, st, p);
+        else hipLaunchKernelGGL((gemm_f16_kernel<MODE_BF16, false, true, NB>), grid, block, 0, st, p);
+        return check_launch("bt_ternary_linear_tiled_forward");
+    } else if (tiled) {
         if (mode == MODE_F16) {
             if (tail) hipLaunchKernelGGL((gemm_f16_kernel<MODE_F16, true, true>), grid, block, 0, st, p);
             else hipLaunchKernelGGL((gemm_f16_kernel<MODE_F16, false, true>), grid, block, 0, st, p);
@@ -527,6 +544,40 @@ int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, int w_layout, c
         else hipLaunchKernelGGL((gemm_f16_kernel<MODE_BF16, false>), grid, block, 0, st, p);
     }
     return check_launch("bt_ternary_linear_packed_forward");
+}
+
+int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, int w_layout, const Epilogue& epi, void* Y, int y_dtype,
+                    int64_t M, int64_t N, int64_t K, int planes, hipStream_t st) {
+    GemmFParams p = {};
+    p.X = (const uint16_t*)X; p.W_T = W_T; p.Y = Y; p.epi = epi;
+    p.M = M; p.N = N; p.K = (planes == 3) ? 3 * ceil_div(K, F_BK) * F_BK : K; p.Kb = ceil_div(K, 4);
+    p.wstages = (int)ceil_div(K, F_BK);
+    p.prehalved = planes == 3;
+    p.y_dtype = y_dtype;
+    p.tiles16 = (int)ceil_div(N, 16);
+    const bool tail = K % F_BK != 0, tiled = w_layout == W_LAYOUT_TILED;
+    const int64_t tiles_m = ceil_div(M, F_BM), tiles_n = ceil_div(N, F_BN), total = tiles_m * tiles_n;
+    // The remainder of a launch in tiles of 64 or 32 rows, as in the int8 GEMM (launch_gemm_i8: same rule, same prices;
+    // same sums in the same order, so the same bits).  BITTORCH_GEMM_TAIL_SPLIT=0 (tests, A/B runs): never.
+    const char* split_env = getenv("BITTORCH_GEMM_TAIL_SPLIT");
+    if (tiled && !tail && !(split_env && split_env[0] == '0')) {
+        const int64_t C = gemm_f_cus(), rem = total % C;
+        if (rem != 0 && 2 * rem <= C) {
+            const int nb = (4 * rem <= C) ? 1 : 2;
+            const int64_t cols = std::min(tiles_n, ceil_div(rem, tiles_m));  // column tiles cut finer
+            const int64_t whole = tiles_m * (tiles_n - cols), fine = ceil_div(M, 32 * nb) * cols;
+            const double split = (double)ceil_div(whole, C) + (double)ceil_div(fine, C) * (nb == 1 ? 0.75 : 0.85) + (whole ? 0.1 : 0.0);
+            if (split < (double)ceil_div(total, C) - 0.04) {
+                if (whole) {
+                    const int rc = launch_gemm_f16_part<4>(p, mode, 0, (int)(tiles_n - cols), tiled, tail, st);
+                    if (rc) return rc;
+                }
+                return nb == 1 ? launch_gemm_f16_part<1>(p, mode, (int)(tiles_n - cols), (int)cols, tiled, tail, st)
+                               : launch_gemm_f16_part<2>(p, mode, (int)(tiles_n - cols), (int)cols, tiled, tail, st);
+            }
+        }
+    }
+    return launch_gemm_f16_part<4>(p, mode, 0, (int)tiles_n, tiled, tail, st);
 }
 
 }  // namespace bt

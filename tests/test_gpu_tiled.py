@@ -186,6 +186,36 @@ def test_tiled_int8_remainder_in_finer_tiles(oracle, m, n, k, monkeypatch):
             np.testing.assert_array_equal(y32[r0:r1], oy)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("m,n,k", REMAINDER_SHAPES)
+def test_tiled_forward_remainder_in_finer_tiles(oracle, dtype, m, n, k, monkeypatch):
+    """The same for the 16-bit matrix-core GEMM (fp32 rows: three bf16 planes): finer tiles for the remainder give the
+    bits of one launch of whole tiles, with bias and with a residual, and agree with the oracle's float64-free
+    restatement of the reference's loop within the rounding of 16-bit products summed in fp32."""
+    from bittorch_amd import _C
+    monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
+    _, wt = _packed(oracle, n, k, seed=m % 5)
+    tiled = _C.retile_weights(wt, k)
+    g = torch.Generator().manual_seed(m + n + 1)
+    scale = torch.rand(n, generator=g) + 0.5
+    bias = (torch.randn(n, generator=g) * 0.01).to(dtype)
+    x = seeded_acts(m, k, seed=m + k + 1, dtype=dtype)
+    res = seeded_acts(m, n, seed=m + 2, dtype=dtype).cuda()
+    announce("remainder tiles, float", dtype, m, n, k)
+    outs = {}
+    for split in ("0", "1"):
+        monkeypatch.setenv("BITTORCH_GEMM_TAIL_SPLIT", split)
+        outs[split] = (_C.ternary_linear_tiled_forward(x.cuda(), tiled, scale.cuda(), bias.cuda(), k, n),
+                       _C.ternary_linear_tiled_forward(x.cuda(), tiled, scale.cuda(), None, k, n, residual=res))
+    torch.cuda.synchronize()
+    for a, b in zip(outs["0"], outs["1"]):
+        assert torch.equal(a, b)
+    y = f32np(outs["1"][0])
+    for r0, r1 in [(0, min(m, 40)), (max(0, m // 2 - 20), min(m, m // 2 + 20)), (max(0, m - 40), m)]:
+        ref = oracle.linear_packed(f32np(x[r0:r1]), wt.cpu().numpy(), scale.numpy(), k, f32np(bias))
+        assert rel_err(y[r0:r1], ref) <= (1e-3 if dtype == torch.float32 else 1e-2)  # output rounding of the 16-bit dtypes
+
+
 def test_tiled_forward_against_oracle(oracle):
     from bittorch_amd import _C
     n, k = 300, 520
