@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include <algorithm>
 #include <type_traits>
@@ -26,6 +27,48 @@ void set_error(const char* fmt, ...);
 int check_launch(const char* what);
 
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// ---- the remainder of a tiled GEMM launch (gemm_i8.hip, gemm_f16.hip, and the rule that routes a batch to them) ------
+// Workgroups take 128 x 256 tiles in rounds of one per compute unit.  When the last round holds tiles for at most half
+// of the compute units, the column tiles of that remainder are computed in tiles of 64 or 32 rows instead (nb = 2 or 1
+// row blocks per K half and wave), two or four workgroups where there was one, in a launch of their own behind the
+// whole tiles.  A finer tile does fewer MFMAs per decoded weight and its stage is bound by the chain LDS read -> decode
+// -> barrier, so it only pays where the alternative is idle compute units.  Prices in rounds of whole tiles, as measured
+// (int8; M = 4096, N = 2560: K = 2560 36.5 -> 32.8 us, K = 6912 74.9 -> 67.3 us; N = K = 4096: M = 1024 23.9 -> 19.8 us,
+// M = 512 23.5 -> 15.6 us): a round of half tiles 0.85, of quarter tiles 0.75, the second launch 0.1.
+struct GemmSplit {
+    int nb;          // 4: no finer tiles
+    int64_t cols;    // column tiles (of 256) cut finer, the last ones of the matrix
+    double rounds;   // price of the launch(es) in rounds of whole tiles
+};
+static inline int64_t gemm_compute_units() {  // of the current device (asked once per process)
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cus = n;
+    }
+    return cus;
+}
+// allowed: the caller's kernel has finer tiles for this call (decode-tiled weights, K in whole stages);
+// BITTORCH_GEMM_TAIL_SPLIT=0 (tests, A/B runs): never.
+static inline GemmSplit gemm_split(int64_t M, int64_t N, bool allowed) {
+    const int64_t C = gemm_compute_units();
+    const int64_t tiles_m = ceil_div(M, 128), tiles_n = ceil_div(N, 256), total = tiles_m * tiles_n;
+    GemmSplit r = {4, 0, (double)ceil_div(total, C)};
+    const char* env = getenv("BITTORCH_GEMM_TAIL_SPLIT");
+    if (!allowed || (env && env[0] == '0')) return r;
+    const int64_t rem = total % C;
+    if (rem == 0 || 2 * rem > C) return r;
+    const int nb = (4 * rem <= C) ? 1 : 2;
+    const int64_t cols = std::min(tiles_n, ceil_div(rem, tiles_m));
+    const int64_t whole = tiles_m * (tiles_n - cols), fine = ceil_div(M, 32 * nb) * cols;
+    const double split = (double)ceil_div(whole, C) + (double)ceil_div(fine, C) * (nb == 1 ? 0.75 : 0.85) + (whole ? 0.1 : 0.0);
+    if (split < r.rounds - 0.04) r = {nb, cols, split};
+    return r;
+}
 
 // ---- element access by dtype tag (BT_F32 / BT_F16 / BT_BF16) --------------
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) {

@@ -133,14 +133,15 @@ static const int64_t kMaxKInt8 = 132096;
 // which puts the crossover at 1.5 .. 2 M outputs for K = 2560 .. 4096 (the GEMM would occupy under a fifth of
 // the compute units there) and later for shallow layers.  BITTORCH_STREAM_MAX_ROWS=n replaces the rule by
 // "B <= n" (tuning and test runs).
-static bool prefers_stream(int64_t B, int64_t N, int64_t K, bool int8) {
+static bool prefers_stream(int64_t B, int64_t N, int64_t K, bool int8, bool tiled = false) {
     if (const char* env = getenv("BITTORCH_STREAM_MAX_ROWS")) {
         const long v = atol(env);
         if (v >= 1) return B <= v;
     }
     if (B <= 32) return true;
     const double work = (double)B * (double)N * (double)K;
-    const double rounds = (double)ceil_div(ceil_div(B, 128) * ceil_div(N, 256), 256);
+    // (rounds of whole tiles, or what the finer tiles of a small launch's remainder cost in them)
+    const double rounds = gemm_split(B, N, tiled && K % (int8 ? 128 : 64) == 0).rounds;
     const double wgs = (double)(ceil_div(B, 16) * ceil_div(N, int8 ? 128 : 64));
     const double t_stream = 4.0 + work * (int8 ? 2.2e-9 : 5.0e-9) + wgs * (int8 ? 0.003 : 0.004);
     const double t_gemm = rounds * (int8 ? 8.6 + 0.0044 * (double)K : 6.9 + 0.010 * (double)K);
@@ -237,7 +238,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         if (x_dtype != BT_F32) {
             const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
             // tall batches: the tiled matrix-core GEMM reads the copy too (not with the SwiGLU output stage)
-            if (!prefers_stream(B, N, K, false) && epi_op == 0 && gemm_f16_supported_tiled(N, K, X, Y))
+            if (!prefers_stream(B, N, K, false, true) && epi_op == 0 && gemm_f16_supported_tiled(N, K, X, Y))
                 return launch_gemm_f16(mode, X, W_T, W_LAYOUT_TILED, epi, Y, x_dtype, B, N, K, 1, st);
             return launch_stream(mode, X, 2, nullptr, W_T, W_LAYOUT_TILED, epi, Y, x_dtype, nullptr, B, N, K, 1,
                                  Q_ROW_MAJOR, 0, nullptr, 0.0f, epi_op, st);
@@ -250,7 +251,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         const int64_t Kp = plane_len(K);
         rc = launch_split_f32_planes(X, B, K, Kp, workspace, st);
         if (rc) return rc;
-        if (!prefers_stream(B, N, 3 * Kp, false) && epi_op == 0 && gemm_f16_supported_tiled(N, 3 * Kp, workspace, Y))
+        if (!prefers_stream(B, N, 3 * Kp, false, K % 64 == 0) && epi_op == 0 && gemm_f16_supported_tiled(N, 3 * Kp, workspace, Y))
             return launch_gemm_f16(MODE_BF16, workspace, W_T, W_LAYOUT_TILED, epi, Y, BT_F32, B, N, K, 3, st);
         return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, W_LAYOUT_TILED, epi, Y, BT_F32, nullptr, B, N, K, 3,
                              Q_ROW_MAJOR, 0, nullptr, 0.0f, epi_op, st);
@@ -368,7 +369,7 @@ static int gemm_i8_impl(const char* who, const int8_t* Q, int q_layout, const fl
             set_error("%s: tiled weights must be 256-byte aligned and below 4 GiB", who);
             return BT_ERR_INVALID;
         }
-        if (!prefers_stream(B, N, K, true) && gemm_i8_supported_tiled(N, K, Q))
+        if (!prefers_stream(B, N, K, true, true) && gemm_i8_supported_tiled(N, K, Q))
             return launch_gemm_i8(Q, q_layout, s_x, W_T, W_LAYOUT_TILED, epi, Y, y_dtype, acc_out, B, N, K, st);
         return launch_stream(MODE_I8, Q, 1, s_x, W_T, w_layout, epi, Y, y_dtype, acc_out, B, N, K, 1, q_layout, 0, nullptr,
                              0.0f, 0, st);

@@ -497,18 +497,6 @@ bool gemm_f16_supported(int64_t N, int64_t K, const void* X, const void* W_T, co
 // planes = 1: X is [M, K].  planes = 3: X is [M, 3*Kp], Kp = K rounded up to 64, three zero-padded planes of K
 // values per row whose products with the same weights are summed (fp32 activations split into three bf16 terms).
 // With K % 64 != 0 the last weight stage of every plane runs past W_T's rows: the TAIL instantiation clamps them.
-static int64_t gemm_f_cus() {  // compute units of the current device (asked once per process)
-    static int cus = 0;
-    if (!cus) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-            n = 256;
-        cus = n;
-    }
-    return cus;
-}
-
 // One launch over column tiles [tile_n0, tile_n0 + tiles_n) in tiles of 32 * NB rows.
 template <int NB>
 static int launch_gemm_f16_part(GemmFParams p, int mode, int tile_n0, int tiles_n, bool tiled, bool tail, hipStream_t st) {
@@ -556,26 +544,17 @@ int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, int w_layout, c
     p.y_dtype = y_dtype;
     p.tiles16 = (int)ceil_div(N, 16);
     const bool tail = K % F_BK != 0, tiled = w_layout == W_LAYOUT_TILED;
-    const int64_t tiles_m = ceil_div(M, F_BM), tiles_n = ceil_div(N, F_BN), total = tiles_m * tiles_n;
-    // The remainder of a launch in tiles of 64 or 32 rows, as in the int8 GEMM (launch_gemm_i8: same rule, same prices;
-    // same sums in the same order, so the same bits).  BITTORCH_GEMM_TAIL_SPLIT=0 (tests, A/B runs): never.
-    const char* split_env = getenv("BITTORCH_GEMM_TAIL_SPLIT");
-    if (tiled && !tail && !(split_env && split_env[0] == '0')) {
-        const int64_t C = gemm_f_cus(), rem = total % C;
-        if (rem != 0 && 2 * rem <= C) {
-            const int nb = (4 * rem <= C) ? 1 : 2;
-            const int64_t cols = std::min(tiles_n, ceil_div(rem, tiles_m));  // column tiles cut finer
-            const int64_t whole = tiles_m * (tiles_n - cols), fine = ceil_div(M, 32 * nb) * cols;
-            const double split = (double)ceil_div(whole, C) + (double)ceil_div(fine, C) * (nb == 1 ? 0.75 : 0.85) + (whole ? 0.1 : 0.0);
-            if (split < (double)ceil_div(total, C) - 0.04) {
-                if (whole) {
-                    const int rc = launch_gemm_f16_part<4>(p, mode, 0, (int)(tiles_n - cols), tiled, tail, st);
-                    if (rc) return rc;
-                }
-                return nb == 1 ? launch_gemm_f16_part<1>(p, mode, (int)(tiles_n - cols), (int)cols, tiled, tail, st)
-                               : launch_gemm_f16_part<2>(p, mode, (int)(tiles_n - cols), (int)cols, tiled, tail, st);
-            }
+    const int64_t tiles_n = ceil_div(N, F_BN);
+    // the remainder of a launch in tiles of 64 or 32 rows, as in the int8 GEMM (gemm_split: same rule, same prices; fp32
+    // sums in the same order, so the same bits)
+    const GemmSplit sp = gemm_split(M, N, tiled && !tail);
+    if (sp.nb != 4) {
+        if (sp.cols < tiles_n) {
+            const int rc = launch_gemm_f16_part<4>(p, mode, 0, (int)(tiles_n - sp.cols), tiled, tail, st);
+            if (rc) return rc;
         }
+        return sp.nb == 1 ? launch_gemm_f16_part<1>(p, mode, (int)(tiles_n - sp.cols), (int)sp.cols, tiled, tail, st)
+                          : launch_gemm_f16_part<2>(p, mode, (int)(tiles_n - sp.cols), (int)sp.cols, tiled, tail, st);
     }
     return launch_gemm_f16_part<4>(p, mode, 0, (int)tiles_n, tiled, tail, st);
 }

@@ -651,19 +651,6 @@ bool gemm_i8_supported(int64_t N, int64_t K, const void* Q, const void* W_T) {
            (G_BM + 1) * K < (1ll << 32) && ceil_div(K, 4) * N < (1ll << 32);
 }
 
-// compute units of the current device (asked once per process)
-static int64_t gemm_cus() {
-    static int cus = 0;
-    if (!cus) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-            n = 256;
-        cus = n;
-    }
-    return cus;
-}
-
 // One launch over column tiles [tile_n0, tile_n0 + tiles_n) in tiles of 32 * NB rows.
 template <int NB>
 static int launch_gemm_i8_part(GemmParams p, int tile_n0, int tiles_n, bool qoo, bool tiled, hipStream_t st) {
@@ -710,33 +697,17 @@ int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_
     p.wsteps = (int)ceil_div(p.Kb, 16);
     p.tiles16 = (int)ceil_div(N, 16);
     const bool qoo = q_layout == Q_OPERAND_ORDER, tiled = w_layout == W_LAYOUT_TILED;
-    const int64_t tiles_m = ceil_div(M, G_BM), tiles_n = ceil_div(N, G_BN), total = tiles_m * tiles_n;
-
-    // The remainder of a launch.  Workgroups take tiles in rounds of one per compute unit; when the last round holds
-    // tiles for at most half of the compute units, the column tiles of that remainder are computed in tiles of 64 or 32
-    // rows instead, two or four workgroups where there was one, in a launch of their own behind the whole tiles (same
-    // sums, same bits; a finer tile does fewer MFMAs per decoded weight, so it only pays where the alternative is idle
-    // compute units).  Cost in rounds of whole tiles, as measured: a round of half tiles 0.85, of quarter tiles 0.75 (a
-    // stage of so few MFMAs is bound by its chain of LDS read, decode and barrier, not by the matrix cores), a launch 0.1.
-    // M = 4096, N = 2560: K = 2560 36.5 -> 32.8 us, K = 6912 74.9 -> 67.3 us; N = K = 4096: M = 1024 23.9 -> 19.8 us,
-    // M = 512 23.5 -> 15.6 us.  BITTORCH_GEMM_TAIL_SPLIT=0 (tests, A/B runs): never.
-    const char* split_env = getenv("BITTORCH_GEMM_TAIL_SPLIT");
-    if (tiled && K % G_BK == 0 && !(split_env && split_env[0] == '0') && !getenv("BITTORCH_GEMM_INPHASE")) {
-        const int64_t C = gemm_cus(), rem = total % C;
-        if (rem != 0 && 2 * rem <= C) {
-            const int nb = (4 * rem <= C) ? 1 : 2;
-            const int64_t cols = std::min(tiles_n, ceil_div(rem, tiles_m));  // column tiles cut finer
-            const int64_t whole = tiles_m * (tiles_n - cols), fine = ceil_div(M, 32 * nb) * cols;
-            const double split = (double)ceil_div(whole, C) + (double)ceil_div(fine, C) * (nb == 1 ? 0.75 : 0.85) + (whole ? 0.1 : 0.0);
-            if (split < (double)ceil_div(total, C) - 0.04) {
-                if (whole) {
-                    const int rc = launch_gemm_i8_part<4>(p, 0, (int)(tiles_n - cols), qoo, tiled, st);
-                    if (rc) return rc;
-                }
-                return nb == 1 ? launch_gemm_i8_part<1>(p, (int)(tiles_n - cols), (int)cols, qoo, tiled, st)
-                               : launch_gemm_i8_part<2>(p, (int)(tiles_n - cols), (int)cols, qoo, tiled, st);
-            }
+    const int64_t tiles_n = ceil_div(N, G_BN);
+    // the column tiles of a mostly empty last round in finer tiles, a launch of their own behind the whole tiles
+    // (gemm_split; same sums, same bits)
+    const GemmSplit sp = gemm_split(M, N, tiled && K % G_BK == 0 && !getenv("BITTORCH_GEMM_INPHASE"));
+    if (sp.nb != 4) {
+        if (sp.cols < tiles_n) {
+            const int rc = launch_gemm_i8_part<4>(p, 0, (int)(tiles_n - sp.cols), qoo, tiled, st);
+            if (rc) return rc;
         }
+        return sp.nb == 1 ? launch_gemm_i8_part<1>(p, (int)(tiles_n - sp.cols), (int)sp.cols, qoo, tiled, st)
+                          : launch_gemm_i8_part<2>(p, (int)(tiles_n - sp.cols), (int)sp.cols, qoo, tiled, st);
     }
     return launch_gemm_i8_part<4>(p, 0, (int)tiles_n, qoo, tiled, st);
 }
