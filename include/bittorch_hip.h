@@ -235,6 +235,9 @@ int bt_ternary_linear_packed_forward_fused(const void* X, int64_t ld_x, int x_dt
  *     column h), u = rd(linear column N/2 + h): the SwiGLU MLP's hidden vector leaves the gate|up kernel
  *     itself (structure: TernaryTransformer.ts:366-423).  A pair-ordered copy serves only this output stage.
  *   bt_ternary_gemm_i8_tiled: bt_ternary_gemm_i8_res on the tiled copy (same remark).
+ *   A tall batch on the tiled copy may take two kernel launches on the stream instead of one (the column tiles of
+ *   a mostly empty last round of 128 x 256 tiles run as tiles of 64 or 32 rows behind the whole tiles): same
+ *   results, nothing for the caller to do; both launches are captured by a HIP graph like any other.
  */
 enum { BT_TILES_NATURAL = 0, BT_TILES_GATE_UP_PAIRS = 1 };
 enum { BT_EPI_NONE = 0, BT_EPI_SWIGLU_PAIRS = 1 };
