@@ -216,6 +216,41 @@ def test_tiled_forward_remainder_in_finer_tiles(oracle, dtype, m, n, k, monkeypa
         assert rel_err(y[r0:r1], ref) <= (1e-3 if dtype == torch.float32 else 1e-2)  # output rounding of the 16-bit dtypes
 
 
+def test_remainder_tiles_replay_in_a_graph(oracle, monkeypatch):
+    """The two launches of a call with finer remainder tiles are captured like any other: every replay of the graph,
+    with eager work and synchronizations between the replays, gives the eager result."""
+    from bittorch_amd import _C
+    monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
+    m, n, k = 4096, 2560, 256
+    _, wt = _packed(oracle, n, k, seed=3)
+    tiled = _C.retile_weights(wt, k)
+    scale = (torch.rand(n) * 0.05 + 0.01).cuda()
+    xs = [seeded_acts(m, k, seed=s_, dtype=torch.bfloat16, outliers=True).cuda() for s_ in (1, 2, 3)]
+    x = xs[0].clone()
+    q, s = _C.act_quant_int8(x, True)
+    eager = []
+    for xi in xs:
+        qi, si = _C.act_quant_int8(xi, True)
+        eager.append(_C.ternary_gemm_int8_tiled(qi, si, tiled, scale, None, k, n, torch.bfloat16, False, None, True))
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        _C.ternary_gemm_int8_tiled(q, s, tiled, scale, None, k, n, torch.bfloat16, False, None, True)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = _C.ternary_gemm_int8_tiled(q, s, tiled, scale, None, k, n, torch.bfloat16, False, None, True)
+    for xi, want in zip(xs, eager):
+        qi, si = _C.act_quant_int8(xi, True)  # eager work between the replays
+        q.copy_(qi)
+        s.copy_(si)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want)
+
+
 def test_tiled_forward_against_oracle(oracle):
     from bittorch_amd import _C
     n, k = 300, 520
