@@ -149,7 +149,8 @@ REMAINDER_SHAPES = [(4096, 2560, 256), (1024, 4096, 128), (512, 4096, 384), (100
                     (512, 4000, 128), (4090, 2560, 128)]
 
 
-@pytest.mark.parametrize("m,n,k", REMAINDER_SHAPES)
+# ... and config 5's two projections of 1.25 rounds at their full size
+@pytest.mark.parametrize("m,n,k", REMAINDER_SHAPES + [(4096, 2560, 2560), (4096, 2560, 6912)])
 def test_tiled_int8_remainder_in_finer_tiles(oracle, m, n, k, monkeypatch):
     """The prefill GEMM computes the column tiles of a mostly empty last round in tiles of 64 or 32 rows
     (a second launch behind the whole tiles).  Same bits as one launch of whole tiles -- outputs and int32
