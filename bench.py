@@ -375,6 +375,7 @@ def main():
 
     import torch
     from bittorch_amd import _C  # ImportError if the HIP library is not built
+    from bittorch_amd._lib import set_option
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -742,7 +743,7 @@ def main():
             del ts
         extra["large_matrices_M1"] = big
         # batched decode / short prefill on the config-2 layer (tiled weights): the streaming kernel runs the 16-row
-        # blocks of a call concurrently in one launch; the tiled GEMM (forced with BITTORCH_STREAM_MAX_ROWS) beside it
+        # blocks of a call concurrently in one launch; the tiled GEMM (forced with the library option STREAM_MAX_ROWS) beside it
         bd = {}
         n_, k_ = 4096, 4096
         ws = rand_packed(n_, k_, 8)
@@ -754,11 +755,11 @@ def main():
             row = {}
             for route, env in (("streaming", None), ("tiled_gemm", "16")):
                 if env:
-                    os.environ["BITTORCH_STREAM_MAX_ROWS"] = env
+                    set_option("STREAM_MAX_ROWS", env)
                 _, ev_f = graph_time(lambda i: _C.ternary_linear_tiled_forward(xa, ts[i % 8], sc, None, k_, n_), 40, 5, torch)
                 _, ev_i = graph_time(lambda i: _C.ternary_gemm_int8_tiled(q, s_, ts[i % 8], sc, None, k_, n_, torch.bfloat16,
                                                                          False, None, True), 40, 5, torch)
-                os.environ.pop("BITTORCH_STREAM_MAX_ROWS", None)
+                set_option("STREAM_MAX_ROWS", None)
                 row[f"bf16_us_{route}"] = round(ev_f / 40 * 1e3, 2)
                 row[f"int8_us_{route}"] = round(ev_i / 40 * 1e3, 2)
             row["int8_tops"] = round(2.0 * m * n_ * k_ / (row["int8_us_streaming"] * 1e-6) / 1e12, 1)

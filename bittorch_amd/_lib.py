@@ -26,6 +26,7 @@ _sz = ctypes.c_size_t
 SIGNATURES = {
     "bt_abi_version": (_int, []),
     "bt_last_error": (ctypes.c_char_p, []),
+    "bt_set_option": (_int, [ctypes.c_char_p, ctypes.c_char_p]),
     "bt_quantize_pack": (_int, [_vp, _int, _i64, _i64, ctypes.c_double, _int, _vp, _vp, _vp, _vp]),
     "bt_ternary_linear_forward": (_int, [_vp, _int, _vp, _vp, _int, _i64, _vp, _int, _vp, _i64, _i64,
                                          _i64, _vp]),
@@ -94,3 +95,12 @@ def load() -> ctypes.CDLL:
 
 def last_error() -> str:
     return load().bt_last_error().decode("utf-8", "replace")
+
+
+def set_option(name: Optional[str], value: Optional[str] = None) -> None:
+    """Overrides one of the library's run-time options (``bt_set_option``): ``STREAM_MAX_ROWS``, ``GROUP_WALK`` ...;
+    ``value=None`` un-sets it, ``name=None`` un-sets all of them.  The environment variable ``BITTORCH_<NAME>`` gives
+    an option its initial value, read once per process."""
+    rc = load().bt_set_option(None if name is None else name.encode(), None if value is None else str(value).encode())
+    if rc != 0:
+        raise ValueError(last_error())

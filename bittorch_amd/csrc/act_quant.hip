@@ -145,7 +145,7 @@ __global__ __launch_bounds__(256) void act_quant_row_kernel(const void* __restri
 template <int DT>
 static bool launch_act_quant_rows(const void* X, int64_t B, int64_t K, int8_t* Q, float* s_x, int ql, hipStream_t st) {
     if (K % 8 != 0 || K > 16384 || ((uintptr_t)X) % 16 != 0 || ((uintptr_t)Q) % 8 != 0 || B > 0x7fffffff ||
-        getenv("BITTORCH_ACTQ_GENERIC"))
+        tuning_env("BITTORCH_ACTQ_GENERIC"))
         return false;
     const dim3 grid((unsigned)B), block(256);
     const int k = (int)K;

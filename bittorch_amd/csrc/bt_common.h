@@ -28,6 +28,33 @@ int check_launch(const char* what);
 
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// ---- run-time options -------------------------------------------------------------------------------------------------
+// The documented switches of the library.  Each is read from the environment (BITTORCH_<NAME>) once per process, on the
+// first call that asks for any of them, and can be overridden afterwards with bt_set_option (tests and benchmarks choose a
+// code path that way); asking for one on a call is an array lookup, not a getenv.  BITTORCH_KERNEL is not among them:
+// the reference re-reads it on every call (ternary_gemm_production.cu:262-273) and so does this library.
+enum Option {
+    OPT_STREAM_MAX_ROWS,     // n: batches of up to n rows take the streaming kernel, larger ones the tiled GEMM
+    OPT_GEMM_LONG_EPILOGUE,  // 1: the tiled int8 GEMM never takes its short epilogue
+    OPT_GEMM_TAIL_SPLIT,     // 0: the remainder of a tiled GEMM launch is not cut into finer tiles
+    OPT_GROUP_WALK,          // grouped GEMV: 1 / chunk / 0 force a kernel
+    OPT_GROUP_NACC,          // grouped GEMV: 16-column blocks per wave of the slab kernel
+    OPT_GROUP_UNITS,         // grouped GEMV: 1 forces the one-matrix kernel over (unit, tile) workgroups, 0 forbids it
+    OPT_PLANES_NACC,         // exact GEMV, one matrix per launch: 16-column blocks per workgroup
+    OPT_ROWOP_GENERIC,       // 1: SwiGLU / RMSNorm rows on the shape-generic kernel
+    OPT_STREAM_CFG,          // "ld,waves": tile width and wave count of the streaming kernel
+    OPT_NO_PLANES,           // 1: a single fp16 row takes the 16-bit streaming kernel instead of the exact GEMV
+    OPT_COUNT
+};
+const char* option(Option o);  // the option's text, or nullptr when it is not set (capi.hip)
+
+// A/B switches of experiment builds (-DBT_TUNING): compiled out of the product library.
+#ifdef BT_TUNING
+static inline const char* tuning_env(const char* name) { return getenv(name); }
+#else
+static inline const char* tuning_env(const char*) { return nullptr; }
+#endif
+
 // ---- the remainder of a tiled GEMM launch (gemm_i8.hip, gemm_f16.hip, and the rule that routes a batch to them) ------
 // Workgroups take 128 x 256 tiles in rounds of one per compute unit.  When the last round holds tiles for at most half
 // of the compute units, the column tiles of that remainder are computed in tiles of 64 or 32 rows instead (nb = 2 or 1
@@ -53,12 +80,12 @@ static inline int64_t gemm_compute_units() {  // of the current device (asked on
     return cus;
 }
 // allowed: the caller's kernel has finer tiles for this call (decode-tiled weights, K in whole stages);
-// BITTORCH_GEMM_TAIL_SPLIT=0 (tests, A/B runs): never.
+// option GEMM_TAIL_SPLIT = 0 (tests, A/B runs): never.
 static inline GemmSplit gemm_split(int64_t M, int64_t N, bool allowed) {
     const int64_t C = gemm_compute_units();
     const int64_t tiles_m = ceil_div(M, 128), tiles_n = ceil_div(N, 256), total = tiles_m * tiles_n;
     GemmSplit r = {4, 0, (double)ceil_div(total, C)};
-    const char* env = getenv("BITTORCH_GEMM_TAIL_SPLIT");
+    const char* env = option(OPT_GEMM_TAIL_SPLIT);
     if (!allowed || (env && env[0] == '0')) return r;
     const int64_t rem = total % C;
     if (rem == 0 || 2 * rem > C) return r;

@@ -1,5 +1,6 @@
 // extern "C" entry points of libbittorch_hip.so: validation and kernel choice.
 // Replaces the host dispatch of the reference (csrc/core/dispatch.cpp:52-142).
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -26,6 +27,35 @@ int check_launch(const char* what) {
         return BT_ERR_LAUNCH;
     }
     return BT_OK;
+}
+
+// ---- run-time options (bt_common.h) -----------------------------------------------------------------------------------
+static const char* const kOptionNames[OPT_COUNT] = {
+    "STREAM_MAX_ROWS", "GEMM_LONG_EPILOGUE", "GEMM_TAIL_SPLIT", "GROUP_WALK", "GROUP_NACC",
+    "GROUP_UNITS", "PLANES_NACC", "ROWOP_GENERIC", "STREAM_CFG", "NO_PLANES",
+};
+struct OptionSlot {
+    char text[2][48];              // two buffers, so that a reader never sees one being rewritten by the next override
+    std::atomic<const char*> cur;  // nullptr: not set
+    int next;
+};
+static OptionSlot g_options[OPT_COUNT];
+static std::once_flag g_options_once;
+static void options_from_environment() {
+    for (int o = 0; o < OPT_COUNT; o++) {
+        char name[64];
+        snprintf(name, sizeof(name), "BITTORCH_%s", kOptionNames[o]);
+        const char* env = getenv(name);
+        if (env && strlen(env) < sizeof(g_options[o].text[0])) {
+            strcpy(g_options[o].text[0], env);
+            g_options[o].cur.store(g_options[o].text[0], std::memory_order_release);
+            g_options[o].next = 1;
+        }
+    }
+}
+const char* option(Option o) {
+    std::call_once(g_options_once, options_from_environment);
+    return g_options[o].cur.load(std::memory_order_acquire);
 }
 
 // kernels in the other translation units
@@ -131,10 +161,10 @@ static const int64_t kMaxKInt8 = 132096;
 //              workgroups = 16-row blocks x 128- resp. 64-column tiles
 //   GEMM       rounds * (8.6 + 0.0044 K) (int8),  rounds * (6.9 + 0.010 K) (16-bit)
 // which puts the crossover at 1.5 .. 2 M outputs for K = 2560 .. 4096 (the GEMM would occupy under a fifth of
-// the compute units there) and later for shallow layers.  BITTORCH_STREAM_MAX_ROWS=n replaces the rule by
+// the compute units there) and later for shallow layers.  The option STREAM_MAX_ROWS = n replaces the rule by
 // "B <= n" (tuning and test runs).
 static bool prefers_stream(int64_t B, int64_t N, int64_t K, bool int8, bool tiled = false) {
-    if (const char* env = getenv("BITTORCH_STREAM_MAX_ROWS")) {
+    if (const char* env = option(OPT_STREAM_MAX_ROWS)) {
         const long v = atol(env);
         if (v >= 1) return B <= v;
     }
@@ -157,6 +187,33 @@ using namespace bt;
 extern "C" int bt_abi_version(void) { return BT_ABI_VERSION; }
 
 extern "C" const char* bt_last_error(void) { return g_err; }
+
+extern "C" int bt_set_option(const char* name, const char* value) {
+    std::call_once(g_options_once, options_from_environment);
+    if (!name) {  // back to "not set", every option
+        for (int o = 0; o < OPT_COUNT; o++) g_options[o].cur.store(nullptr, std::memory_order_release);
+        return BT_OK;
+    }
+    if (!strncmp(name, "BITTORCH_", 9)) name += 9;
+    for (int o = 0; o < OPT_COUNT; o++) {
+        if (strcmp(name, kOptionNames[o])) continue;
+        OptionSlot& s = g_options[o];
+        if (!value) {
+            s.cur.store(nullptr, std::memory_order_release);
+            return BT_OK;
+        }
+        if (strlen(value) >= sizeof(s.text[0])) {
+            set_error("bt_set_option: value of %s is longer than %zu characters", name, sizeof(s.text[0]) - 1);
+            return BT_ERR_INVALID;
+        }
+        strcpy(s.text[s.next], value);
+        s.cur.store(s.text[s.next], std::memory_order_release);
+        s.next ^= 1;
+        return BT_OK;
+    }
+    set_error("bt_set_option: unknown option '%s'", name);
+    return BT_ERR_INVALID;
+}
 
 extern "C" int bt_ternary_linear_forward(const void* X, int x_dtype, const int8_t* W_tern, const void* scale,
                                          int scale_dtype, int64_t scale_len, const void* bias, int bias_dtype,
@@ -232,7 +289,7 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
             return launch_planes(X, W_T, W_LAYOUT_TILED, epi, Y, N, K, epi_op, st);
         // one bf16 row times a very wide matrix (a vocabulary projection): the same kernel family, the row scaled by
         // its largest exponent
-        if (x_dtype == BT_BF16 && B == 1 && epi_op == 0 && ((uintptr_t)X) % 16 == 0 && !getenv("BITTORCH_NO_PLANES") &&
+        if (x_dtype == BT_BF16 && B == 1 && epi_op == 0 && ((uintptr_t)X) % 16 == 0 && !option(OPT_NO_PLANES) &&
             planes_bf16_wide(N, K))
             return launch_planes_bf16_wide(X, W_T, epi, Y, N, K, st);
         if (x_dtype != BT_F32) {
@@ -429,7 +486,7 @@ extern "C" int bt_ternary_linear_tensor_core_forward(const void* X, int x_dtype,
     // Q is private to this call: written in operand order whenever the layout applies, so that
     // neither GEMM kernel has to permute activations
     // (BITTORCH_Q_LAYOUT=rowmajor keeps the row-major layout, for A/B runs)
-    const char* lay = getenv("BITTORCH_Q_LAYOUT");
+    const char* lay = tuning_env("BITTORCH_Q_LAYOUT");
     const int q_layout = (K % 16 == 0 && ((uintptr_t)X) % 16 == 0 && !(lay && !strcmp(lay, "rowmajor")))
                              ? Q_OPERAND_ORDER : Q_ROW_MAJOR;
     rc = launch_act_quant(X, x_dtype, B, K, Q, s_x, q_layout, (hipStream_t)stream);
@@ -612,7 +669,7 @@ static int fused_forward_impl(const char* who, const void* X, int64_t ld_x, int 
                                                       : packed_uses_stream(x_dtype, W_T, Y, N, K);
     // a row that takes the exact fp16 GEMV gets its prologue inside that kernel (same element arithmetic as the row
     // kernel, so the result equals the unfused sequence bit for bit), or from the row kernel where that is switched off
-    if (B == 1 && !getenv("BITTORCH_NO_PROLOGUE") && ((uintptr_t)pro_b) % 16 == 0 && pro_b &&
+    if (B == 1 && !tuning_env("BITTORCH_NO_PROLOGUE") && ((uintptr_t)pro_b) % 16 == 0 && pro_b &&
         streams && planes_supported(x_dtype, x_dtype, B, N, K, X, W_T, Y, w_layout)) {
         if (epi_op != 0 && (epi_op != EPI_SWIGLU_PAIRS || w_layout != W_LAYOUT_TILED || N % 32 != 0 || residual)) {
             set_error("%s: the SwiGLU output stage needs pair-ordered tiled weights, N %% 32 == 0 and no residual", who);

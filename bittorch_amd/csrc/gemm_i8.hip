@@ -52,7 +52,7 @@ struct GemmParams {
     int32_t* acc_out;     // optional [M, N]
     int64_t Kb;
     int y_dtype;
-    int long_epilogue;    // A/B runs and tests (BITTORCH_GEMM_LONG_EPILOGUE=1): never the short epilogue
+    int long_epilogue;    // A/B runs and tests (option GEMM_LONG_EPILOGUE): never the short epilogue
     Epilogue epi;
 };
 static_assert(offsetof(GemmParams, s_x) == 64, "first argument line as laid out above");
@@ -264,7 +264,7 @@ __device__ __forceinline__ void take_blocks(v4i (&acc)[2 * NB][4], int mb0, cons
 // the staging copies them to LDS untouched.
 // WT = true: W_T is the decode-tiled copy (W_LAYOUT_TILED): the four dwords a lane decodes per stage
 // (16 consecutive k of its four columns) are 16 contiguous bytes there, one load and no transpose.
-// ANTIPHASE = false (A/B runs, BITTORCH_GEMM_INPHASE=1, benchmarked variant only): both K halves run the stage in
+// ANTIPHASE = false (A/B runs of experiment builds, BITTORCH_GEMM_INPHASE=1, benchmarked variant only): both K halves run the stage in
 // the same order.
 // NB: 16-row blocks per K half and wave: 4 is the 128-row tile; 2 and 1 are the tiles of 64 and 32 rows (same columns,
 // same staging and LDS layout with rows past the tile clamped, a quarter to half of the MFMAs per decoded weight) that a
@@ -670,7 +670,7 @@ static int launch_gemm_i8_part(GemmParams p, int tile_n0, int tiles_n, bool qoo,
         else hipLaunchKernelGGL((gemm_i8_kernel<false, false, true, true, NB>), grid, block, 0, st, p);
     } else if (tiled) {
         if (!tail) {
-            if (qoo && getenv("BITTORCH_GEMM_INPHASE")) hipLaunchKernelGGL((gemm_i8_kernel<false, true, true, false>), grid, block, 0, st, p);
+            if (qoo && tuning_env("BITTORCH_GEMM_INPHASE")) hipLaunchKernelGGL((gemm_i8_kernel<false, true, true, false>), grid, block, 0, st, p);
             else if (qoo) hipLaunchKernelGGL((gemm_i8_kernel<false, true, true>), grid, block, 0, st, p);
             else hipLaunchKernelGGL((gemm_i8_kernel<false, false, true>), grid, block, 0, st, p);
         } else {
@@ -693,14 +693,14 @@ int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_
     p.Q = Q; p.s_x = s_x; p.W_T = W_T; p.Y = Y; p.acc_out = acc_out; p.epi = epi;
     p.M = M; p.N = N; p.K = K; p.Kb = ceil_div(K, 4);
     p.y_dtype = y_dtype;
-    p.long_epilogue = getenv("BITTORCH_GEMM_LONG_EPILOGUE") != nullptr;
+    p.long_epilogue = option(OPT_GEMM_LONG_EPILOGUE) != nullptr;
     p.wsteps = (int)ceil_div(p.Kb, 16);
     p.tiles16 = (int)ceil_div(N, 16);
     const bool qoo = q_layout == Q_OPERAND_ORDER, tiled = w_layout == W_LAYOUT_TILED;
     const int64_t tiles_n = ceil_div(N, G_BN);
     // the column tiles of a mostly empty last round in finer tiles, a launch of their own behind the whole tiles
     // (gemm_split; same sums, same bits)
-    const GemmSplit sp = gemm_split(M, N, tiled && K % G_BK == 0 && !getenv("BITTORCH_GEMM_INPHASE"));
+    const GemmSplit sp = gemm_split(M, N, tiled && K % G_BK == 0 && !tuning_env("BITTORCH_GEMM_INPHASE"));
     if (sp.nb != 4) {
         if (sp.cols < tiles_n) {
             const int rc = launch_gemm_i8_part<4>(p, 0, (int)(tiles_n - sp.cols), qoo, tiled, st);

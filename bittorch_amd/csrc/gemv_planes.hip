@@ -788,7 +788,7 @@ constexpr int64_t PL_MAX_K = 16384;
 
 bool planes_supported(int x_dtype, int y_dtype, int64_t B, int64_t N, int64_t K, const void* X, const void* W, const void* Y,
                       int w_layout) {
-    if (getenv("BITTORCH_NO_PLANES")) return false;  // A/B runs: the 16-bit matrix-core path instead
+    if (option(OPT_NO_PLANES)) return false;  // A/B runs: the 16-bit matrix-core path instead
     if (x_dtype != BT_F16 || y_dtype != BT_F16 || B != 1 || K % 16 != 0 || K > PL_MAX_K || K < 16 || N % 4 != 0) return false;
     if (((uintptr_t)X) % 16 != 0 || ((uintptr_t)Y) % 2 != 0) return false;
     if (w_layout == W_LAYOUT_TILED) return ((uintptr_t)W) % 256 == 0;
@@ -834,7 +834,7 @@ static bool launch_walk(PlaneParams p, int64_t G, int64_t wgs, int min_tiles_per
     const int spw = (int)ceil_div(p.wsteps, 8);
     const int tb = (spw >= 5) ? 2 : 4;
     const int64_t total = G * p.tiles16;
-    const char* force = getenv("BITTORCH_GROUP_WALK");
+    const char* force = option(OPT_GROUP_WALK);
     bool want = force ? (force[0] == '1') : (total >= min_tiles_per_wg * wgs);
     if (min_tiles_per_wg < 0) want = true;
     if (!walk_shape_ok(p.wsteps, p.tiles16) || !want) return false;
@@ -890,7 +890,7 @@ int launch_planes(const void* X, const uint8_t* W, int w_layout, const Epilogue&
     p.tiles16 = (int)ceil_div(N, 16);
     // 16-column tiles per workgroup: as many as still give every compute unit a workgroup
     int nacc = (w_layout == W_LAYOUT_TILED) ? 4 : 2;
-    if (const char* env = getenv("BITTORCH_PLANES_NACC")) nacc = atoi(env);
+    if (const char* env = option(OPT_PLANES_NACC)) nacc = atoi(env);
     const int min_nacc = (epi_op == EPI_SWIGLU_PAIRS) ? 2 : 1;
     while (nacc > min_nacc && ceil_div(p.tiles16, nacc) < 224) nacc >>= 1;
     if (nacc != 1 && nacc != 2 && nacc != 4) nacc = min_nacc;
@@ -956,7 +956,7 @@ static void launch_group_k(const PlaneParams& p, unsigned grid, size_t lds, hipS
 // 9.9, G = 6 equal, G = 8 12.6 against 10.8; units of N = 4096, K = 11008: G = 1 9.2 against 20.6, G = 4 14.9 against
 // 21.6, G = 8 21.8 against 23.6, G = 16 40.6 against 38.4).  BITTORCH_GROUP_UNITS=1 / =0 (tests, A/B runs): always / never.
 static bool launch_units(PlaneParams p, int64_t G, hipStream_t st) {
-    const char* force = getenv("BITTORCH_GROUP_UNITS");
+    const char* force = option(OPT_GROUP_UNITS);
     if (force && force[0] == '0') return false;
     if (p.K > PL_MAX_K) return false;
     if (!(force && force[0] == '1')) {
@@ -985,7 +985,7 @@ static int launch_group_params(PlaneParams p, int64_t G, hipStream_t st) {
     const int64_t wgs = resident_wgs();
     const bool bf16 = p.x_dtype == BT_BF16;
     if (!bf16) {
-        const char* force = getenv("BITTORCH_GROUP_UNITS");
+        const char* force = option(OPT_GROUP_UNITS);
         if (force && force[0] == '1' && launch_units(p, G, st)) return check_launch("gemv_planes_group");
     }
     // (bf16 units have no one-matrix kernel: the walk wherever the shape allows it, which is also the faster of their
@@ -995,7 +995,7 @@ static int launch_group_params(PlaneParams p, int64_t G, hipStream_t st) {
     // columns per wave: 32 (two tiles) streams best (5.3 TB/s against 4.8 with four tiles and 4.4-5.0 with one at
     // G = 128, 4096 x 4096); another width only where it fills the resident workgroups markedly more evenly
     int nacc = 2;
-    if (const char* env = getenv("BITTORCH_GROUP_NACC")) {
+    if (const char* env = option(OPT_GROUP_NACC)) {
         nacc = atoi(env);
         if (nacc != 1 && nacc != 2 && nacc != 4) nacc = 2;
     } else {
@@ -1013,7 +1013,7 @@ static int launch_group_params(PlaneParams p, int64_t G, hipStream_t st) {
     p.items = (int)(G * p.slabs);
     const unsigned grid = (unsigned)((p.items < wgs) ? p.items : wgs);
     int pf = 8;
-    if (const char* env = getenv("BITTORCH_GROUP_PF")) pf = bf16 ? 8 : atoi(env);
+    if (const char* env = tuning_env("BITTORCH_GROUP_PF")) pf = bf16 ? 8 : atoi(env);
     const int SP = (int)ceil_div(p.wsteps, pf) * pf;
     const size_t lds = 32 + (size_t)SP * 4 * PL_GROUP;
     if (bf16) {
@@ -1043,7 +1043,7 @@ bool planes_bf16_shape_ok(int64_t N, int64_t K) {
 // checked planes_bf16_shape_ok, the alignment of the operands (as planes_supported does for fp16) and that the
 // matrix gives every resident workgroup a dozen tiles (planes_bf16_wide).
 bool planes_bf16_wide(int64_t N, int64_t K) {
-    const char* force = getenv("BITTORCH_GROUP_WALK");
+    const char* force = option(OPT_GROUP_WALK);
     if (force && force[0] == '0') return false;
     return planes_bf16_shape_ok(N, K) && ((force && force[0] == '1') || ceil_div(N, 16) >= 12 * resident_wgs());
 }

@@ -158,7 +158,7 @@ static int launch_fast_rows(const void* W, int64_t N, int64_t K, float tf, float
                             uint8_t* packed_T, float* scale, hipStream_t st, int* rc) {
     constexpr int MIN_RPW = (WAVES >= 16) ? 1 : (WAVES >= 8) ? 2 : 4;
     int rpw = 0;
-    if (const char* env = getenv("BITTORCH_QP_RPW")) rpw = atoi(env);
+    if (const char* env = tuning_env("BITTORCH_QP_RPW")) rpw = atoi(env);
     if (rpw != 1 && rpw != 2 && rpw != 4) {
         // (workgroups of 8 waves run two to a compute unit: at least 640 of them, so that both places stay filled)
         const int64_t min_tiles = (WAVES == 8 && ITERS <= 16) ? 640 : 320;
@@ -186,7 +186,7 @@ template <int DT>
 static int try_launch_fast(const void* W, int64_t N, int64_t K, float tf, float clamp_min, int per_channel,
                            uint8_t* packed_T, float* scale, int8_t* w_tern, hipStream_t st, int* rc) {
     if (!packed_T || w_tern || K % 256 != 0 || ((uintptr_t)W) % 16 != 0 || ((uintptr_t)packed_T) % 16 != 0 ||
-        N * K >= (1ll << 31) || getenv("BITTORCH_QP_GENERIC"))
+        N * K >= (1ll << 31) || tuning_env("BITTORCH_QP_GENERIC"))
         return 0;
     const int chunks = (int)(K / 256);
 #define BT_QF(IT, WV) \

@@ -234,7 +234,7 @@ int launch_row_op(int op, int dtype, const void* A, int64_t lda, const void* Bv,
     const int es = dtype_size(dtype);
     auto aligned = [&](const void* ptr, int64_t ld) { return !ptr || (((uintptr_t)ptr) % 16 == 0 && (ld * es) % 16 == 0); };
     const bool fast = K % 8 == 0 && K <= 16384 && aligned(A, lda) && aligned(Bv, op == ROW_SWIGLU ? ldb : 8) &&
-                      aligned(H, K) && (!Q || ((uintptr_t)Q) % 8 == 0) && !getenv("BITTORCH_ROWOP_GENERIC");
+                      aligned(H, K) && (!Q || ((uintptr_t)Q) % 8 == 0) && !option(OPT_ROWOP_GENERIC);
     if (op == ROW_SWIGLU) {
         if (dtype == BT_F32) launch_row_op_dt<ROW_SWIGLU, BT_F32>(p, B, fast, st);
         else if (dtype == BT_F16) launch_row_op_dt<ROW_SWIGLU, BT_F16>(p, B, fast, st);

@@ -630,7 +630,7 @@ StreamPlan stream_plan(int mode, int64_t M, int64_t N, int64_t Kb, int w_layout,
     (void)Kb;
     // optional override for tuning runs: BITTORCH_STREAM_CFG="ld,waves"
     int o_ld = -1, o_waves = 0;
-    if (const char* env = getenv("BITTORCH_STREAM_CFG")) sscanf(env, "%d,%d", &o_ld, &o_waves);
+    if (const char* env = option(OPT_STREAM_CFG)) sscanf(env, "%d,%d", &o_ld, &o_waves);
     int ld;
     if (w_layout == W_LAYOUT_TILED) {
         // 16-column tiles, up to four per workgroup (a batch re-reads its activations once per workgroup, and so
@@ -722,14 +722,14 @@ static bool xlds_ok(int es, int M, bool x_vec_ok, const StreamPlan& pl, int64_t 
     const size_t red_bytes = (size_t)pl.waves * M * tile_n * 4;
     const size_t xs_bytes = (size_t)pl.waves * XC_MAX * 64 * 16;
     return M == 1 && x_vec_ok && (pl.ld <= 4 || (pl.ld > 100 && pl.ld != LD_T8)) && spw * 64 * es <= XC_MAX * 64 * 16 && K >= 16 / es &&
-           red_bytes + xs_bytes <= 64 * 1024 && !getenv("BITTORCH_STREAM_NOXLDS");
+           red_bytes + xs_bytes <= 64 * 1024 && !tuning_env("BITTORCH_STREAM_NOXLDS");
 }
 
 // Can the streaming kernel apply an RMSNorm / SwiGLU prologue to this call's activation row itself?
 // (one 16-bit row that takes the LDS-staged variant; BITTORCH_NO_PROLOGUE=1 says no, for A/B runs)
 bool stream_prologue_fusable(int mode, int64_t B, int64_t N, int64_t K, const void* X, const void* pro_b, int w_layout,
                              int epi_op) {
-    if (mode == MODE_I8 || B != 1 || getenv("BITTORCH_NO_PROLOGUE")) return false;
+    if (mode == MODE_I8 || B != 1 || tuning_env("BITTORCH_NO_PROLOGUE")) return false;
     const bool vec = ((uintptr_t)X) % 16 == 0 && (!pro_b || ((uintptr_t)pro_b) % 16 == 0) && (K * 2) % 16 == 0;
     if (epi_op != EPI_NONE && mode == MODE_I8) return false;
     return xlds_ok(2, 1, vec, stream_plan(mode, 1, N, ceil_div(K, 4), w_layout, epi_op == EPI_SWIGLU_PAIRS ? 2 : 1), K);

@@ -4,7 +4,8 @@
  * Plain pointers and sizes only; no C++ or torch types cross this boundary.
  * All pointers except the optional ones are DEVICE pointers owned by the
  * caller; the library never allocates or frees device memory and keeps no
- * mutable global state, so calls on different streams are independent.
+ * mutable global state besides the option table of bt_set_option, so calls on
+ * different streams are independent.
  * Kernels are enqueued on `stream` (a hipStream_t passed as void*; NULL is
  * the default stream) and the call returns without synchronising.
  *
@@ -56,6 +57,18 @@ int bt_abi_version(void);
 const char* bt_last_error(void);
 
 /*
+ * Run-time options.  The library has a small set of documented switches (kernel choice for tests, benchmarks and
+ * tuning runs): STREAM_MAX_ROWS, GEMM_LONG_EPILOGUE, GEMM_TAIL_SPLIT, GROUP_WALK, GROUP_NACC, GROUP_UNITS,
+ * PLANES_NACC, ROWOP_GENERIC, STREAM_CFG, NO_PLANES.  Each takes its initial value from the environment variable
+ * BITTORCH_<NAME>, read once per process on the first call that consults an option; bt_set_option overrides it from
+ * then on (value NULL: not set; name NULL: every option not set).  `name` may carry the BITTORCH_ prefix.  Not to be
+ * called while another thread is inside the library.  BITTORCH_KERNEL (auto | generic) is not one of them: like the
+ * reference (csrc/kernels/ternary_gemm_production.cu:262-273) the library reads it from the environment on every
+ * call.  No counterpart in the reference, which has that one switch only.
+ */
+int bt_set_option(const char* name, const char* value);
+
+/*
  * Fused ternary quantize + 2-bit pack.
  * Replaces the torch op chains of bittorch/quant/ternary.py:122-142
  * (absmax scale, threshold, sign) and bittorch/quant/ternary_packed.py:50-73,
@@ -93,7 +106,7 @@ int bt_ternary_linear_forward(const void* X, int x_dtype, const int8_t* W_tern, 
  *   A cost model fitted to measurements picks the kernel: the streaming kernel (weights read once
  *   per 16 rows, all 16-row blocks of the call in one launch) while B*N*K is small, the tiled 16-bit
  *   matrix-core GEMM beyond (crossover near 1.5-2 M outputs for K = 2560..4096;
- *   BITTORCH_STREAM_MAX_ROWS=n replaces the rule by "B <= n").  A single fp16 row (K % 16 == 0,
+ *   the option STREAM_MAX_ROWS = n replaces the rule by "B <= n").  A single fp16 row (K % 16 == 0,
  *   K <= 16384, N % 4 == 0) runs the exact GEMV on the int8 matrix cores: the dot products are summed
  *   without rounding and rounded to fp32 once.  fp32 activations (any K) are first split into
  *   three bf16 planes (x = hi + mid + lo exactly), each zero-padded to a multiple of 64 values, in

@@ -5,6 +5,13 @@ import torch
 BT_DT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 
+def set_option(name, value):
+    """Overrides a run-time option of the HIP library for the rest of the test (tests/conftest.py un-sets every
+    override when the test ends); value None un-sets it."""
+    from bittorch_amd import _lib
+    _lib.set_option(name, value)
+
+
 def seeded_weights(n, k, seed=0, std=0.02, dtype=torch.float32):
     g = torch.Generator().manual_seed(seed)
     return (torch.randn(n, k, generator=g) * std).to(dtype)

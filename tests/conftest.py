@@ -21,6 +21,15 @@ def oracle():
     return o
 
 
+@pytest.fixture(autouse=True)
+def _library_options_reset():
+    """A test may override run-time options of the HIP library (tests/_util.py: set_option); none survives it."""
+    yield
+    from bittorch_amd import _lib
+    if _lib._lib is not None:
+        _lib.set_option(None)
+
+
 def announce(*parts):
     """Name the case before a GPU step so a lost box still says what ran."""
     print("[case]", *parts, flush=True)

@@ -124,3 +124,22 @@ def test_tiled_copy_size_and_argument_checks_without_a_gpu():
     assert lib.bt_retile_weights(addr, 48, 64, 1, addr, None) == -1          # pair order needs N % 32 == 0
     assert "N % 32" in _lib.last_error()
     assert lib.bt_retile_weights(addr, 16, 64, 7, addr, None) == -1          # unknown tile order
+
+
+def test_set_option_validates_names_and_lengths():
+    """bt_set_option is host-only: known names (with or without the BITTORCH_ prefix) are accepted, set and un-set;
+    an unknown name or an over-long value is an error with a message."""
+    from bittorch_amd import _lib
+    lib = _lib.load()
+    try:
+        assert lib.bt_set_option(b"STREAM_MAX_ROWS", b"32") == 0
+        assert lib.bt_set_option(b"BITTORCH_GROUP_WALK", b"chunk") == 0
+        assert lib.bt_set_option(b"GROUP_WALK", None) == 0
+        assert lib.bt_set_option(b"NO_SUCH_OPTION", b"1") == -1
+        assert "unknown option" in _lib.last_error()
+        assert lib.bt_set_option(b"STREAM_CFG", b"x" * 100) == -1
+        assert "longer" in _lib.last_error()
+        with pytest.raises(ValueError):
+            _lib.set_option("KERNEL", "generic")  # read from the environment on every call, not an option
+    finally:
+        assert lib.bt_set_option(None, None) == 0

@@ -12,7 +12,7 @@ import torch
 import torch.nn.functional as F
 
 from conftest import announce
-from _util import BT_DT, f32np, random_ternary, seeded_acts
+from _util import BT_DT, f32np, random_ternary, seeded_acts, set_option
 
 pytestmark = pytest.mark.gpu
 
@@ -182,7 +182,7 @@ def test_residual_in_the_tiled_gemms_full_and_ragged_tiles(dtype, b, n, k, monke
     epilogues agree."""
     from bittorch_amd import _C
     announce("residual tiled gemms", dtype, b, n, k)
-    monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
+    set_option("STREAM_MAX_ROWS", "32")
     packed, scale, bias = _packed_case(n, k, seed=b + n + 1)
     tiled = _C.retile_weights(packed, k)
     x = seeded_acts(b, k, seed=7, dtype=dtype).cuda()
@@ -194,7 +194,7 @@ def test_residual_in_the_tiled_gemms_full_and_ragged_tiles(dtype, b, n, k, monke
     y8 = _C.ternary_gemm_int8(q, s_x, packed, scale, bias, k, dtype)
     assert torch.equal(_C.ternary_gemm_int8(q, s_x, packed, scale, bias, k, dtype, residual=res), y8 + res)
     assert torch.equal(_C.ternary_gemm_int8_tiled(q, s_x, tiled, scale, bias, k, n, dtype, residual=res), y8 + res)
-    monkeypatch.setenv("BITTORCH_GEMM_LONG_EPILOGUE", "1")
+    set_option("GEMM_LONG_EPILOGUE", "1")
     assert torch.equal(_C.ternary_gemm_int8_tiled(q, s_x, tiled, scale, bias, k, n, dtype, residual=res), y8 + res)
 
 
@@ -362,7 +362,7 @@ def test_operand_order_needs_whole_groups():
 
 def test_operand_order_on_the_generic_row_kernels(monkeypatch):
     from bittorch_amd import _C
-    monkeypatch.setenv("BITTORCH_ROWOP_GENERIC", "1")
+    set_option("ROWOP_GENERIC", "1")
     x = seeded_acts(5, 64, dtype=torch.float16).cuda()
     qn, _ = _C.rmsnorm(x, None, 1e-5, False, True)
     qo, _ = _C.rmsnorm(x, None, 1e-5, False, True, operand_order=True)

@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from conftest import announce
-from _util import f32np, random_ternary, seeded_acts
+from _util import f32np, random_ternary, seeded_acts, set_option
 
 pytestmark = pytest.mark.gpu
 
@@ -77,14 +77,14 @@ def test_single_row_fp16_variants(oracle):
     assert torch.equal(got.cpu(), expect + res)
     try:
         for nacc in ("1", "2", "4"):
-            os.environ["BITTORCH_PLANES_NACC"] = nacc
+            set_option("PLANES_NACC", nacc)
             assert torch.equal(_C.ternary_linear_tiled_forward(xd, tiled, scale.cuda(), bias.cuda(), k, n).cpu(), expect)
             assert torch.equal(_C.ternary_linear_packed_forward(xd, pd, scale.cuda(), bias.cuda(), k).cpu(), expect)
     finally:
-        os.environ.pop("BITTORCH_PLANES_NACC", None)
+        set_option("PLANES_NACC", None)
     # one matrix through the contiguous-walk kernel (what a very wide layer takes by itself), residual included
     try:
-        os.environ["BITTORCH_GROUP_WALK"] = "1"
+        set_option("GROUP_WALK", "1")
         for (n2, k2) in ((4096, 4096), (96, 2560), (1000, 1536), (20, 3600)):
             x2, packed2, scale2, bias2 = _setup(n2, k2, seed=n2 + k2 + 1)
             tiled2 = _C.retile_weights(packed2.cuda(), k2)
@@ -95,7 +95,7 @@ def test_single_row_fp16_variants(oracle):
             got2 = _C.ternary_linear_tiled_forward(x2.cuda(), tiled2, scale2.cuda(), bias2.cuda(), k2, n2, residual=res2.cuda())
             assert torch.equal(got2.cpu(), expect2 + res2), (n2, k2)
     finally:
-        os.environ.pop("BITTORCH_GROUP_WALK", None)
+        set_option("GROUP_WALK", None)
     # ties of the final rounding and the largest magnitudes: all-ones weights, crafted activations
     from bittorch_amd.quant import pack_ternary_transposed
     ones = pack_ternary_transposed(torch.ones(16, 16, dtype=torch.int8))[0]
@@ -146,10 +146,8 @@ def test_grouped_launch_equals_single_calls(oracle, g, n, k, per_tensor, bias):
     try:
         for walk, nacc, units in ((None, None, None), ("1", None, "0"), ("0", "1", "0"), ("0", "2", "0"), ("0", "4", "0"),
                                   (None, None, "1")):
-            for name, val in (("BITTORCH_GROUP_WALK", walk), ("BITTORCH_GROUP_NACC", nacc), ("BITTORCH_GROUP_UNITS", units)):
-                os.environ.pop(name, None)
-                if val:
-                    os.environ[name] = val
+            for name, val in (("GROUP_WALK", walk), ("GROUP_NACC", nacc), ("GROUP_UNITS", units)):
+                set_option(name, val)
             ys = [torch.full((1, n), float("nan"), dtype=torch.float16, device="cuda") for _ in range(g)]
             tabs = _tables(_C, xs, tiles, scales, biases if bias else None, ys)
             _C.ternary_gemv_grouped(*tabs, k, n, scale_len=1 if per_tensor else n)
@@ -157,9 +155,9 @@ def test_grouped_launch_equals_single_calls(oracle, g, n, k, per_tensor, bias):
             for u in range(g):
                 assert torch.equal(ys[u], singles[u]), (u, walk, nacc, units)
     finally:
-        os.environ.pop("BITTORCH_GROUP_NACC", None)
-        os.environ.pop("BITTORCH_GROUP_WALK", None)
-        os.environ.pop("BITTORCH_GROUP_UNITS", None)
+        set_option("GROUP_NACC", None)
+        set_option("GROUP_WALK", None)
+        set_option("GROUP_UNITS", None)
 
 
 def test_grouped_launch_config2_units_and_shared_operands(oracle):
@@ -261,16 +259,16 @@ def test_grouped_launch_random_shapes(oracle, g, n, k, per_tensor, bias, seed):
     assert torch.equal(singles[(a0, w0)].cpu(), _expect(oracle, base[a0][0], base[w0][1], base[w0][2], base[w0][3], k))
     try:
         for walk, one_matrix in (("1", "0"), ("0", "0"), ("0", "1")):
-            os.environ["BITTORCH_GROUP_WALK"] = walk
-            os.environ["BITTORCH_GROUP_UNITS"] = one_matrix
+            set_option("GROUP_WALK", walk)
+            set_option("GROUP_UNITS", one_matrix)
             ys = [torch.full((1, n), float("nan"), dtype=torch.float16, device="cuda") for _ in range(g)]
             _C.ternary_gemv_grouped(*_tables(_C, xs, tiles, scales, biases, ys), k, n, scale_len=1 if per_tensor else n)
             torch.cuda.synchronize()
             for u in range(g):
                 assert torch.equal(ys[u], singles[units[u]]), (u, walk, one_matrix)
     finally:
-        os.environ.pop("BITTORCH_GROUP_WALK", None)
-        os.environ.pop("BITTORCH_GROUP_UNITS", None)
+        set_option("GROUP_WALK", None)
+        set_option("GROUP_UNITS", None)
 
 
 # ---- bf16 rows: scaled by the row's largest exponent, summed exactly ---------------------------------------------------
@@ -318,9 +316,9 @@ def test_grouped_bf16_units_against_the_oracle(oracle, g, n, k, per_tensor, bias
     expects = [_expect_bf16(oracle, *s_, k) for s_ in sets]
     try:
         for walk in (None, "0"):
-            os.environ.pop("BITTORCH_GROUP_WALK", None)
+            set_option("GROUP_WALK", None)
             if walk:
-                os.environ["BITTORCH_GROUP_WALK"] = walk
+                set_option("GROUP_WALK", walk)
             ys = [torch.full((1, n), float("nan"), dtype=torch.bfloat16, device="cuda") for _ in range(g)]
             _C.ternary_gemv_grouped(*_tables(_C, xs, tiles, scales, biases, ys), k, n, scale_len=1 if per_tensor else n,
                                     bias_dtype=torch.bfloat16, x_dtype=torch.bfloat16)
@@ -328,7 +326,7 @@ def test_grouped_bf16_units_against_the_oracle(oracle, g, n, k, per_tensor, bias
             for u in range(g):
                 assert torch.equal(ys[u].cpu(), expects[idx[u]]), (u, walk)
     finally:
-        os.environ.pop("BITTORCH_GROUP_WALK", None)
+        set_option("GROUP_WALK", None)
     x, packed, scale, b = sets[0]
     ref = oracle.linear_packed(f32np(x), packed.numpy(), f32np(scale), k, None if b is None else f32np(b))
     np.testing.assert_allclose(f32np(ys[0]), ref, rtol=1e-2, atol=1e-2 * float(np.abs(ref).max()))
@@ -345,7 +343,7 @@ def test_bf16_row_times_a_wide_matrix_and_argument_errors(oracle):
     tiled = _C.retile_weights(packed.cuda(), k)
     y_stream = _C.ternary_linear_tiled_forward(x.cuda(), tiled, scale.cuda(), bias.cuda(), k, n)
     try:
-        os.environ["BITTORCH_GROUP_WALK"] = "1"
+        set_option("GROUP_WALK", "1")
         y = _C.ternary_linear_tiled_forward(x.cuda(), tiled, scale.cuda(), bias.cuda(), k, n)
         assert torch.equal(y.cpu(), _expect_bf16(oracle, x, packed, scale, bias, k))
         res = seeded_acts(1, n, seed=9, dtype=torch.bfloat16)
@@ -355,7 +353,7 @@ def test_bf16_row_times_a_wide_matrix_and_argument_errors(oracle):
         xb[0, 77] = float("nan")
         assert torch.isnan(_C.ternary_linear_tiled_forward(xb.cuda(), tiled, scale.cuda(), bias.cuda(), k, n)).all()
     finally:
-        os.environ.pop("BITTORCH_GROUP_WALK", None)
+        set_option("GROUP_WALK", None)
     # the 16-bit matrix-core kernel (what a narrow matrix takes) agrees within bf16 rounding
     np.testing.assert_allclose(f32np(y_stream), f32np(y), rtol=2e-2, atol=2e-2 * float(f32np(y).__abs__().max()))
     lib = _lib.load()

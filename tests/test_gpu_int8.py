@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from conftest import announce
-from _util import f32np, random_ternary, rel_err, seeded_acts
+from _util import f32np, random_ternary, rel_err, seeded_acts, set_option
 
 pytestmark = pytest.mark.gpu
 
@@ -69,7 +69,7 @@ def test_gemm_i8_small_batch_bit_exact(oracle, b, n, k):
                                    (64, 4, 16), (200, 1024, 4096), (129, 300, 1000), (2048, 256, 512)])
 def test_gemm_i8_prefill_bit_exact(oracle, b, n, k, route, monkeypatch):
     if route == "gemm":  # batches beyond 32 rows to the tiled GEMM whatever their size (the default rule streams small outputs)
-        monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
+        set_option("STREAM_MAX_ROWS", "32")
     announce("gemm_i8 prefill", b, n, k)
     _gemm_case(oracle, b, n, k, torch.bfloat16, seed=n + k, outliers=True)
     _gemm_case(oracle, b, n, k, torch.float16, seed=n + k + 1)
@@ -85,7 +85,7 @@ def test_gemm_i8_epilogue_paths_agree_for_any_row_scale(oracle, out_dtype, monke
     from bittorch_amd import _C
     from bittorch_amd.quant import pack_ternary_transposed
     announce("gemm_i8 epilogue paths", out_dtype)
-    monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
+    set_option("STREAM_MAX_ROWS", "32")
     b, n, k = 384, 512, 256
     w = random_ternary(n, k, seed=3)
     packed = pack_ternary_transposed(w)[0]
@@ -104,7 +104,7 @@ def test_gemm_i8_epilogue_paths_agree_for_any_row_scale(oracle, out_dtype, monke
     expect = torch.from_numpy(oy).to(out_dtype)
     args = (q.cuda(), s_x.cuda(), packed.cuda(), scale.cuda(), bias.cuda(), k)
     y_short = _C.ternary_gemm_int8(*args, out_dtype=out_dtype)
-    monkeypatch.setenv("BITTORCH_GEMM_LONG_EPILOGUE", "1")
+    set_option("GEMM_LONG_EPILOGUE", "1")
     y_long = _C.ternary_gemm_int8(*args, out_dtype=out_dtype)
     torch.cuda.synchronize()
     assert torch.equal(y_long.cpu().view(torch.int16 if out_dtype != torch.float32 else torch.int32),
@@ -113,7 +113,7 @@ def test_gemm_i8_epilogue_paths_agree_for_any_row_scale(oracle, out_dtype, monke
                        expect.view(torch.int16 if out_dtype != torch.float32 else torch.int32))
     # without a bias the reference still adds 0.0f, which turns a -0 product into +0: zero, negative and tiny column
     # scales and the negative row scale above must come out the same, sign of zero included
-    monkeypatch.delenv("BITTORCH_GEMM_LONG_EPILOGUE")
+    set_option("GEMM_LONG_EPILOGUE", None)
     scale2 = scale.clone()
     scale2[0:64] = 0.0
     scale2[64:128] = -0.03

@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from conftest import announce
-from _util import assert_close_like_reference, f32np, random_ternary, rel_err, seeded_acts, seeded_weights
+from _util import assert_close_like_reference, f32np, random_ternary, rel_err, seeded_acts, seeded_weights, set_option
 
 pytestmark = pytest.mark.gpu
 
@@ -94,7 +94,7 @@ def test_packed_forward_tall_batches_use_the_tiled_kernel(oracle, dtype, b, n, k
     """Batches above the streaming kernel's limit go to the 16-bit matrix-core GEMM: partial row
     and column tiles, K tails that are not a multiple of the 64-wide stage, odd last stages."""
     if route == "gemm":  # batches beyond 32 rows to the tiled GEMM whatever their size (the default rule streams small outputs)
-        monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
+        set_option("STREAM_MAX_ROWS", "32")
     announce("packed_forward tall", dtype, b, n, k)
     _case(oracle, b, n, k, dtype, seed=b + n + k)
 
@@ -145,7 +145,7 @@ def test_packed_forward_any_number_of_rows(oracle, monkeypatch):
     np.testing.assert_array_equal(f32np(y), oracle.linear_unpacked(f32np(x), w.numpy(), f32np(scale), f32np(bias)))
     monkeypatch.delenv("BITTORCH_KERNEL")
     # streaming kernel, 16 * 65535 + 40 rows
-    monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "2000000")
+    set_option("STREAM_MAX_ROWS", "2000000")
     b, k2 = 16 * 65535 + 40, 64
     packed2 = pack_ternary_transposed(random_ternary(n, k2, seed=2))[0].cuda()
     xb = torch.randn(b, k2, device="cuda").bfloat16()
@@ -210,7 +210,7 @@ def test_packed_forward_fp32_on_the_matrix_cores(oracle, b, n, k, monkeypatch, r
     kernels (streaming kernel up to 32 rows, tiled kernel above): every product is exact, only the
     fp32 summation order differs from the generic kernel - far inside the 1e-3 budget for fp32."""
     if route == "gemm":  # batches beyond 32 rows to the tiled GEMM whatever their size (the default rule streams small outputs)
-        monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
+        set_option("STREAM_MAX_ROWS", "32")
     from bittorch_amd import _C
     from bittorch_amd.quant import pack_ternary_transposed
     announce("packed_forward fp32 planes", b, n, k)
@@ -301,12 +301,12 @@ def test_packed_forward_stream_configs_agree(oracle):
     truth = oracle.linear_packed(f32np(x), packed.cpu().numpy(), f32np(scale), 1024, f64=True)
     try:
         for cfg in ("16,4", "16,1", "8,8", "8,2", "4,4", "4,16", "2,8", "2,16", "1,1", "1,4", "1,16"):
-            os.environ["BITTORCH_STREAM_CFG"] = cfg
+            set_option("STREAM_CFG", cfg)
             y = _C.ternary_linear_packed_forward(x, packed, scale, None, 1024)
             torch.cuda.synchronize()
             assert rel_err(f32np(y), truth) < 2e-3, cfg
     finally:
-        os.environ.pop("BITTORCH_STREAM_CFG", None)
+        set_option("STREAM_CFG", None)
 
 
 def test_unpacked_forward_matches_oracle(oracle, monkeypatch):

@@ -15,7 +15,7 @@ import pytest
 import torch
 
 from conftest import announce
-from _util import f32np, random_ternary, rel_err, seeded_acts
+from _util import f32np, random_ternary, rel_err, seeded_acts, set_option
 
 pytestmark = pytest.mark.gpu
 
@@ -51,7 +51,7 @@ FWD_SHAPES = [(4096, 4096), (2560, 2560), (6912, 2560), (2560, 6912), (100, 64),
 @pytest.mark.parametrize("n,k", FWD_SHAPES)
 def test_tiled_forward_equals_row_major(oracle, dtype, n, k, route, monkeypatch):
     if route == "gemm":  # batches beyond 32 rows to the tiled GEMM whatever their size (the default rule streams small outputs)
-        monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
+        set_option("STREAM_MAX_ROWS", "32")
     from bittorch_amd import _C
     _, wt = _packed(oracle, n, k, seed=1)
     tiled = _C.retile_weights(wt, k)
@@ -77,7 +77,7 @@ def test_tiled_forward_equals_row_major(oracle, dtype, n, k, route, monkeypatch)
 @pytest.mark.parametrize("n,k", [(4096, 4096), (100, 64), (2560, 6912)])
 def test_tiled_forward_fp32_planes(oracle, n, k, route, monkeypatch):
     if route == "gemm":  # batches beyond 32 rows to the tiled GEMM whatever their size (the default rule streams small outputs)
-        monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
+        set_option("STREAM_MAX_ROWS", "32")
     from bittorch_amd import _C
     _, wt = _packed(oracle, n, k, seed=2)
     tiled = _C.retile_weights(wt, k)
@@ -125,7 +125,7 @@ def test_tiled_prologues_equal_row_major(oracle, dtype, n, k):
 @pytest.mark.parametrize("n,k", [(4096, 4096), (11008, 4096), (4096, 11008), (100, 64), (37, 100), (260, 192), (520, 1040)])
 def test_tiled_int8_equals_row_major(oracle, n, k, route, monkeypatch):
     if route == "gemm":  # batches beyond 32 rows to the tiled GEMM whatever their size (the default rule streams small outputs)
-        monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
+        set_option("STREAM_MAX_ROWS", "32")
     from bittorch_amd import _C
     _, wt = _packed(oracle, n, k, seed=4)
     tiled = _C.retile_weights(wt, k)
@@ -157,7 +157,7 @@ def test_tiled_int8_remainder_in_finer_tiles(oracle, m, n, k, monkeypatch):
     accumulators, both activation layouts, bias, residual, 16-bit and fp32 outputs -- and equal to the oracle on
     row slices at the start, across tile borders and at the ragged end."""
     from bittorch_amd import _C
-    monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
+    set_option("STREAM_MAX_ROWS", "32")
     _, wt = _packed(oracle, n, k, seed=m % 7)
     tiled = _C.retile_weights(wt, k)
     g = torch.Generator().manual_seed(m + n)
@@ -172,7 +172,7 @@ def test_tiled_int8_remainder_in_finer_tiles(oracle, m, n, k, monkeypatch):
         q, s = _C.act_quant_int8(x.cuda(), oo)
         outs = {}
         for split in ("0", "1"):
-            monkeypatch.setenv("BITTORCH_GEMM_TAIL_SPLIT", split)
+            set_option("GEMM_TAIL_SPLIT", split)
             y32, acc = _C.ternary_gemm_int8_tiled(q, s, tiled, scale.cuda(), bias.cuda(), k, n, torch.float32, True, None, oo)
             y16 = _C.ternary_gemm_int8_tiled(q, s, tiled, scale.cuda(), None, k, n, torch.bfloat16, False, res, oo)
             y16b = _C.ternary_gemm_int8_tiled(q, s, tiled, scale.cuda(), bias.cuda(), k, n, torch.float16, False, None, oo)
@@ -194,7 +194,7 @@ def test_tiled_forward_remainder_in_finer_tiles(oracle, dtype, m, n, k, monkeypa
     bits of one launch of whole tiles, with bias and with a residual, and agree with the oracle's float64-free
     restatement of the reference's loop within the rounding of 16-bit products summed in fp32."""
     from bittorch_amd import _C
-    monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
+    set_option("STREAM_MAX_ROWS", "32")
     _, wt = _packed(oracle, n, k, seed=m % 5)
     tiled = _C.retile_weights(wt, k)
     g = torch.Generator().manual_seed(m + n + 1)
@@ -205,7 +205,7 @@ def test_tiled_forward_remainder_in_finer_tiles(oracle, dtype, m, n, k, monkeypa
     announce("remainder tiles, float", dtype, m, n, k)
     outs = {}
     for split in ("0", "1"):
-        monkeypatch.setenv("BITTORCH_GEMM_TAIL_SPLIT", split)
+        set_option("GEMM_TAIL_SPLIT", split)
         outs[split] = (_C.ternary_linear_tiled_forward(x.cuda(), tiled, scale.cuda(), bias.cuda(), k, n),
                        _C.ternary_linear_tiled_forward(x.cuda(), tiled, scale.cuda(), None, k, n, residual=res))
     torch.cuda.synchronize()
@@ -221,7 +221,7 @@ def test_remainder_tiles_replay_in_a_graph(oracle, monkeypatch):
     """The two launches of a call with finer remainder tiles are captured like any other: every replay of the graph,
     with eager work and synchronizations between the replays, gives the eager result."""
     from bittorch_amd import _C
-    monkeypatch.setenv("BITTORCH_STREAM_MAX_ROWS", "32")
+    set_option("STREAM_MAX_ROWS", "32")
     m, n, k = 4096, 2560, 256
     _, wt = _packed(oracle, n, k, seed=3)
     tiled = _C.retile_weights(wt, k)
