@@ -288,11 +288,16 @@ def untile_weights(W_tiled: Tensor, out_features: int, in_features: int, gate_up
 def ternary_linear_tiled_forward(X: Tensor, W_tiled: Tensor, scale: Tensor, bias: Optional[Tensor] = None,
                                  in_features: int = -1, out_features: int = -1, residual: Optional[Tensor] = None,
                                  norm: Optional[Tuple[Optional[Tensor], float]] = None,
-                                 swiglu_up: Optional[Tensor] = None, swiglu_pairs: bool = False) -> Tensor:
+                                 swiglu_up: Optional[Tensor] = None, swiglu_pairs: bool = False,
+                                 natural_from_pairs: bool = False) -> Tensor:
     """:func:`ternary_linear_packed_forward` / ``_fused`` on the decode-tiled copy of the weights (same
     results bit for bit); the weights are streamed once per 16 rows of ``X``, so this is for decode shapes.
     ``swiglu_pairs`` (copy built with ``gate_up_pairs=True``): the layer's columns are ``[gate | up]`` and the
-    output is the MLP's hidden vector ``swiglu(gate(x), up(x))`` ``[*, N/2]``, formed in the kernel's output stage."""
+    output is the MLP's hidden vector ``swiglu(gate(x), up(x))`` ``[*, N/2]``, formed in the kernel's output stage.
+    ``natural_from_pairs``: the same pair-ordered copy read as an ordinary linear layer (output ``[*, N]`` in natural
+    column order, bit-identical to a natural-order copy's)."""
+    _check(not (swiglu_pairs and natural_from_pairs), "swiglu_pairs and natural_from_pairs exclude each other")
+    _check(not natural_from_pairs or out_features % 32 == 0, "a pair-ordered copy has N % 32 == 0")
     _check(not swiglu_pairs or (residual is None and swiglu_up is None and out_features % 32 == 0),
            "swiglu_pairs needs N % 32 == 0 and takes neither a residual nor a SwiGLU prologue")
     _check(norm is None or swiglu_up is None, "at most one of norm and swiglu_up may be given")
@@ -329,7 +334,7 @@ def ternary_linear_tiled_forward(X: Tensor, W_tiled: Tensor, scale: Tensor, bias
         _status(_L.bt_ternary_linear_tiled_forward(
             x2.data_ptr(), x2.stride(0), xdt, op, _ptr(pb), ldb, float(eps), W_tiled.data_ptr(), scale.data_ptr(),
             _dt(scale, "scale"), scale.numel(), _ptr(bias), 0 if bias is None else _dt(bias, "bias"), _ptr(res),
-            1 if swiglu_pairs else 0, y.data_ptr(), B, N, K, _ptr(ws), 0 if ws is None else ws.numel(), _stream(X)))
+            1 if swiglu_pairs else 2 if natural_from_pairs else 0, y.data_ptr(), B, N, K, _ptr(ws), 0 if ws is None else ws.numel(), _stream(X)))
     return y.reshape(*X.shape[:-1], Ny)
 
 

@@ -356,11 +356,28 @@ enum { Q_ROW_MAJOR = 0, Q_OPERAND_ORDER = 1 };
 //   W_LAYOUT_TILED      decode-tiled copy: dword ((t * S + s) * 64 + 16 g + j), S = ceil(Kb / 16), holds
 //                       the bytes W_T[16 s + 4 g + r, 16 t + j], r = 0..3 (low byte first), zero where the
 //                       row or the column lies outside the matrix
-enum { W_LAYOUT_ROW_MAJOR = 0, W_LAYOUT_TILED = 1 };
+//   W_LAYOUT_TILED_PAIRS_AS_NATURAL  a decode-tiled copy whose tiles are stored in gate/up pair order (tile t of the
+//                       left half of the columns at 2t, tile t of the right half at 2t + 1: BT_TILES_GATE_UP_PAIRS), read
+//                       by a kernel that works in the matrix's natural column order
+enum { W_LAYOUT_ROW_MAJOR = 0, W_LAYOUT_TILED = 1, W_LAYOUT_TILED_PAIRS_AS_NATURAL = 2 };
+static inline bool layout_tiled(int w_layout) { return w_layout != W_LAYOUT_ROW_MAJOR; }
+// The kernels' `tiles16` argument: the number of 16-column tiles, negative for W_LAYOUT_TILED_PAIRS_AS_NATURAL.
+static inline int tiles16_arg(int64_t N, int w_layout) {
+    const int t = (int)ceil_div(N, 16);
+    return w_layout == W_LAYOUT_TILED_PAIRS_AS_NATURAL ? -t : t;
+}
+// Where 16-column tile t of the matrix (natural column order) sits in the copy; a tile past the end repeats the last
+// one (it only feeds outputs that are never stored).
+__device__ __forceinline__ int stored_tile16(int t, int tiles16) {
+    if (tiles16 >= 0) return min(t, tiles16 - 1);
+    const int n = -tiles16, half = n >> 1;
+    t = min(t, n - 1);
+    return t < half ? 2 * t : 2 * (t - half) + 1;
+}
 
 // activation prologues and output stages of the streaming kernel (BT_PRO_*, BT_EPI_* of the C ABI)
 enum { PRO_NONE = 0, PRO_RMSNORM = 1, PRO_SWIGLU = 2 };
-enum { EPI_NONE = 0, EPI_SWIGLU_PAIRS = 1 };
+enum { EPI_NONE = 0, EPI_SWIGLU_PAIRS = 1, EPI_NATURAL_FROM_PAIRS = 2 /* at the C ABI only: becomes a weight layout */ };
 
 // Two neighbouring lanes hold the 16 quantized bytes of one group (even lane: elements 0..7 as
 // lo, hi; odd lane: elements 8..15).  Returns this lane's 8 bytes of the transposed group.

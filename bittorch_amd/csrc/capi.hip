@@ -278,26 +278,30 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         set_error("%s: the SwiGLU output stage needs pair-ordered tiled weights, N %% 32 == 0 and no residual", who);
         return BT_ERR_INVALID;
     }
-    if (w_layout == W_LAYOUT_TILED) {
+    if (w_layout == W_LAYOUT_TILED_PAIRS_AS_NATURAL && (N % 32 != 0 || epi_op != 0)) {
+        set_error("%s: a pair-ordered tiled copy has N %% 32 == 0; its natural-order output takes no output stage", who);
+        return BT_ERR_INVALID;
+    }
+    if (layout_tiled(w_layout)) {
         // the decode-tiled copy is read by the streaming kernel only, once per 16 rows
         if (!stream_supported_tiled(N, K, W_T) || !fast_path_ok(Y, N, 3 * K) || 3 * K >= (1ll << 26)) {
             set_error("%s: tiled weights must be 256-byte aligned and below 4 GiB, Y 16-byte aligned", who);
             return BT_ERR_INVALID;
         }
         // one fp16 row: the exact GEMV on the int8 matrix cores
-        if (planes_supported(x_dtype, x_dtype, B, N, K, X, W_T, Y, W_LAYOUT_TILED))
-            return launch_planes(X, W_T, W_LAYOUT_TILED, epi, Y, N, K, epi_op, st);
+        if (planes_supported(x_dtype, x_dtype, B, N, K, X, W_T, Y, w_layout))
+            return launch_planes(X, W_T, w_layout, epi, Y, N, K, epi_op, st);
         // one bf16 row times a very wide matrix (a vocabulary projection): the same kernel family, the row scaled by
         // its largest exponent
         if (x_dtype == BT_BF16 && B == 1 && epi_op == 0 && ((uintptr_t)X) % 16 == 0 && !option(OPT_NO_PLANES) &&
-            planes_bf16_wide(N, K))
+            w_layout == W_LAYOUT_TILED && planes_bf16_wide(N, K))
             return launch_planes_bf16_wide(X, W_T, epi, Y, N, K, st);
         if (x_dtype != BT_F32) {
             const int mode = (x_dtype == BT_F16) ? MODE_F16 : MODE_BF16;
             // tall batches: the tiled matrix-core GEMM reads the copy too (not with the SwiGLU output stage)
             if (!prefers_stream(B, N, K, false, true) && epi_op == 0 && gemm_f16_supported_tiled(N, K, X, Y))
-                return launch_gemm_f16(mode, X, W_T, W_LAYOUT_TILED, epi, Y, x_dtype, B, N, K, 1, st);
-            return launch_stream(mode, X, 2, nullptr, W_T, W_LAYOUT_TILED, epi, Y, x_dtype, nullptr, B, N, K, 1,
+                return launch_gemm_f16(mode, X, W_T, w_layout, epi, Y, x_dtype, B, N, K, 1, st);
+            return launch_stream(mode, X, 2, nullptr, W_T, w_layout, epi, Y, x_dtype, nullptr, B, N, K, 1,
                                  Q_ROW_MAJOR, 0, nullptr, 0.0f, epi_op, st);
         }
         if (!workspace || workspace_bytes < f32_planes_bytes(B, K) || ((uintptr_t)workspace) % 256 != 0) {
@@ -309,8 +313,8 @@ static int packed_forward_impl(const char* who, const void* X, int x_dtype, cons
         rc = launch_split_f32_planes(X, B, K, Kp, workspace, st);
         if (rc) return rc;
         if (!prefers_stream(B, N, 3 * Kp, false, K % 64 == 0) && epi_op == 0 && gemm_f16_supported_tiled(N, 3 * Kp, workspace, Y))
-            return launch_gemm_f16(MODE_BF16, workspace, W_T, W_LAYOUT_TILED, epi, Y, BT_F32, B, N, K, 3, st);
-        return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, W_LAYOUT_TILED, epi, Y, BT_F32, nullptr, B, N, K, 3,
+            return launch_gemm_f16(MODE_BF16, workspace, W_T, w_layout, epi, Y, BT_F32, B, N, K, 3, st);
+        return launch_stream(MODE_BF16, workspace, 2, nullptr, W_T, w_layout, epi, Y, BT_F32, nullptr, B, N, K, 3,
                              Q_ROW_MAJOR, 0, nullptr, 0.0f, epi_op, st);
     }
     if (packed_uses_stream(x_dtype, W_T, Y, N, K)) {
@@ -421,13 +425,13 @@ static int gemm_i8_impl(const char* who, const int8_t* Q, int q_layout, const fl
     rc = set_residual(who, residual, &epi);
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
-    if (w_layout == W_LAYOUT_TILED) {
+    if (layout_tiled(w_layout)) {
         if (!stream_supported_tiled(N, K, W_T)) {
             set_error("%s: tiled weights must be 256-byte aligned and below 4 GiB", who);
             return BT_ERR_INVALID;
         }
         if (!prefers_stream(B, N, K, true, true) && gemm_i8_supported_tiled(N, K, Q))
-            return launch_gemm_i8(Q, q_layout, s_x, W_T, W_LAYOUT_TILED, epi, Y, y_dtype, acc_out, B, N, K, st);
+            return launch_gemm_i8(Q, q_layout, s_x, W_T, w_layout, epi, Y, y_dtype, acc_out, B, N, K, st);
         return launch_stream(MODE_I8, Q, 1, s_x, W_T, w_layout, epi, Y, y_dtype, acc_out, B, N, K, 1, q_layout, 0, nullptr,
                              0.0f, 0, st);
     }
@@ -665,7 +669,7 @@ static int fused_forward_impl(const char* who, const void* X, int64_t ld_x, int 
     }
     hipStream_t st = (hipStream_t)stream;
     // one 16-bit row on the streaming kernel: the prologue runs inside the GEMV, on the row's way into LDS
-    const bool streams = (w_layout == W_LAYOUT_TILED) ? (stream_supported_tiled(N, K, W_T) && fast_path_ok(Y, N, K))
+    const bool streams = layout_tiled(w_layout) ? (stream_supported_tiled(N, K, W_T) && fast_path_ok(Y, N, K))
                                                       : packed_uses_stream(x_dtype, W_T, Y, N, K);
     // a row that takes the exact fp16 GEMV gets its prologue inside that kernel (same element arithmetic as the row
     // kernel, so the result equals the unfused sequence bit for bit), or from the row kernel where that is switched off
@@ -769,8 +773,17 @@ extern "C" int bt_ternary_linear_tiled_forward(const void* X, int64_t ld_x, int 
                                                void* Y, int64_t B, int64_t N, int64_t K, void* workspace,
                                                size_t workspace_bytes, void* stream) {
     const char* who = "bt_ternary_linear_tiled_forward";
+    int w_layout = W_LAYOUT_TILED;
+    if (epi_op == EPI_NATURAL_FROM_PAIRS) {  // a copy in gate/up pair order, the plain linear output in natural column order
+        if (N % 32 != 0) {
+            set_error("%s: a pair-ordered tiled copy has N %% 32 == 0 (N=%lld)", who, (long long)N);
+            return BT_ERR_INVALID;
+        }
+        w_layout = W_LAYOUT_TILED_PAIRS_AS_NATURAL;
+        epi_op = EPI_NONE;
+    }
     if (pro_op != 0)
-        return fused_forward_impl(who, X, ld_x, x_dtype, pro_op, pro_b, ld_b, eps, W_tiled, W_LAYOUT_TILED, epi_op, scale,
+        return fused_forward_impl(who, X, ld_x, x_dtype, pro_op, pro_b, ld_b, eps, W_tiled, w_layout, epi_op, scale,
                                   scale_dtype, scale_len, bias, bias_dtype, residual, Y, B, N, K, workspace,
                                   workspace_bytes, stream);
     if (ld_x != K) {
@@ -778,7 +791,7 @@ extern "C" int bt_ternary_linear_tiled_forward(const void* X, int64_t ld_x, int 
                   (long long)ld_x, (long long)K);
         return BT_ERR_INVALID;
     }
-    return packed_forward_impl(who, X, x_dtype, W_tiled, W_LAYOUT_TILED, epi_op, scale, scale_dtype, scale_len, bias, bias_dtype,
+    return packed_forward_impl(who, X, x_dtype, W_tiled, w_layout, epi_op, scale, scale_dtype, scale_len, bias, bias_dtype,
                                residual, Y, B, N, K, workspace, workspace_bytes, stream);
 }
 

@@ -41,7 +41,7 @@ struct GemmFParams {
     int tiles_m, tiles_n;
     int per_xcd;          // workgroups per XCD (grid = 8 * per_xcd)
     int wstages;          // 64-wide stages of W_T; a stage index beyond it wraps (see launch_gemm_f16)
-    int tiles16;          // WT: 16-column tiles of the decode-tiled weight copy (its 16-row steps are the stages)
+    int tiles16;          // WT: 16-column tiles of the decode-tiled weight copy (its 16-row steps are the stages; < 0: stored_tile16)
     int tile_n0;          // first column tile of this launch (tiles_n counts the launch's own column tiles)
     // ---- needed later
     void* Y;              // [M, N]
@@ -200,7 +200,7 @@ __global__ __launch_bounds__(512) void gemm_f16_kernel(GemmFParams p) {
     const uint32_t a_off = (a_row_c * (uint32_t)p.K + 16u * a_part) * 2u;  // bytes
     uint32_t b_off;
     if constexpr (WT) {
-        const int tt = min((int)(ncol >> 4), p.tiles16 - 1);  // a tile past the end only feeds outputs never stored
+        const int tt = stored_tile16((int)(ncol >> 4), p.tiles16);
         b_off = ((uint32_t)tt * (uint32_t)p.wstages * 64u + (uint32_t)(16 * (2 * kgrp + (g >> 1)) + 4 * (j & 3))) * 4u;
     } else {
         b_off = (uint32_t)(col_ok ? ncol : 0) + (uint32_t)(8 * kgrp + 2 * g) * (uint32_t)p.N;
@@ -542,8 +542,8 @@ int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, int w_layout, c
     p.wstages = (int)ceil_div(K, F_BK);
     p.prehalved = planes == 3;
     p.y_dtype = y_dtype;
-    p.tiles16 = (int)ceil_div(N, 16);
-    const bool tail = K % F_BK != 0, tiled = w_layout == W_LAYOUT_TILED;
+    p.tiles16 = tiles16_arg(N, w_layout);
+    const bool tail = K % F_BK != 0, tiled = layout_tiled(w_layout);
     const int64_t tiles_n = ceil_div(N, F_BN);
     // the remainder of a launch in tiles of 64 or 32 rows, as in the int8 GEMM (gemm_split: same rule, same prices; fp32
     // sums in the same order, so the same bits)

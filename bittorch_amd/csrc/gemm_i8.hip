@@ -44,7 +44,7 @@ struct GemmParams {
     int64_t K, M, N;
     int tiles_m, tiles_n;
     int per_xcd;          // workgroups per XCD (grid = 8 * per_xcd)
-    int wsteps, tiles16;  // WT: 16-row steps and 16-column tiles of the decode-tiled weight copy
+    int wsteps, tiles16;  // WT: 16-row steps and 16-column tiles of the decode-tiled weight copy (tiles16 < 0: stored_tile16)
     int tile_n0;          // first column tile of this launch (tiles_n counts the launch's own column tiles)
     // ---- needed later
     const float* s_x;     // [M]
@@ -317,7 +317,7 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     const uint32_t a_off = a_row_c * (uint32_t)p.K + 32u * a_part;
     uint32_t b_off;
     if constexpr (WT) {
-        const int tt = min((int)(ncol >> 4), p.tiles16 - 1);  // a tile past the end only feeds outputs never stored
+        const int tt = stored_tile16((int)(ncol >> 4), p.tiles16);
         b_off = ((uint32_t)tt * (uint32_t)p.wsteps * 64u + (uint32_t)(16 * g + 4 * (j & 3))) * 4u;
     } else {
         b_off = (uint32_t)(col_ok ? ncol : 0) + (uint32_t)(16 * kgrp + 4 * g) * (uint32_t)p.N;
@@ -695,8 +695,8 @@ int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_
     p.y_dtype = y_dtype;
     p.long_epilogue = option(OPT_GEMM_LONG_EPILOGUE) != nullptr;
     p.wsteps = (int)ceil_div(p.Kb, 16);
-    p.tiles16 = (int)ceil_div(N, 16);
-    const bool qoo = q_layout == Q_OPERAND_ORDER, tiled = w_layout == W_LAYOUT_TILED;
+    p.tiles16 = tiles16_arg(N, w_layout);
+    const bool qoo = q_layout == Q_OPERAND_ORDER, tiled = layout_tiled(w_layout);
     const int64_t tiles_n = ceil_div(N, G_BN);
     // the column tiles of a mostly empty last round in finer tiles, a launch of their own behind the whole tiles
     // (gemm_split; same sums, same bits)

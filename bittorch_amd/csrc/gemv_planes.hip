@@ -67,7 +67,8 @@ struct PlaneParams {
     int slabs;       // grouped launch: column slabs (8 waves x 16 * NACC columns) per unit, or tiles per workgroup
     int items;       // grouped launch: G * slabs
     float pro_eps;   // one-matrix kernel with an RMSNorm prologue
-    int pad_[2];
+    int tiles16_signed;  // one-matrix kernel on tiled weights: tiles16, negative for a pair-ordered copy read in natural order (stored_tile16)
+    int pad_;
     // ---- third line
     const void* const* X_tab;
     const uint8_t* const* W_tab;
@@ -279,7 +280,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(PlaneParams p) 
 #pragma unroll
     for (int t = 0; t < NACC; t++) {
         if constexpr (LAYOUT == PL_TILED) {
-            coloff[t] = ((uint32_t)min(tile * NACC + t, p.tiles16 - 1) * (uint32_t)p.wsteps * 64u + (uint32_t)lane) * 4u;
+            coloff[t] = ((uint32_t)stored_tile16(tile * NACC + t, p.tiles16_signed) * (uint32_t)p.wsteps * 64u + (uint32_t)lane) * 4u;
         } else {
             const int64_t c = (int64_t)tile * TILE_N + 16 * t + (j & ~3);
             coloff[t] = (c < p.N) ? (uint32_t)c : 0u;
@@ -791,7 +792,7 @@ bool planes_supported(int x_dtype, int y_dtype, int64_t B, int64_t N, int64_t K,
     if (option(OPT_NO_PLANES)) return false;  // A/B runs: the 16-bit matrix-core path instead
     if (x_dtype != BT_F16 || y_dtype != BT_F16 || B != 1 || K % 16 != 0 || K > PL_MAX_K || K < 16 || N % 4 != 0) return false;
     if (((uintptr_t)X) % 16 != 0 || ((uintptr_t)Y) % 2 != 0) return false;
-    if (w_layout == W_LAYOUT_TILED) return ((uintptr_t)W) % 256 == 0;
+    if (layout_tiled(w_layout)) return ((uintptr_t)W) % 256 == 0;
     return ((uintptr_t)W) % 4 == 0 && (ceil_div(K, 4) + 64) * N < (1ll << 32);
 }
 
@@ -889,12 +890,13 @@ int launch_planes(const void* X, const uint8_t* W, int w_layout, const Epilogue&
     p.wsteps = (int)ceil_div(p.Kb, 16);
     p.tiles16 = (int)ceil_div(N, 16);
     // 16-column tiles per workgroup: as many as still give every compute unit a workgroup
-    int nacc = (w_layout == W_LAYOUT_TILED) ? 4 : 2;
+    p.tiles16_signed = tiles16_arg(N, w_layout);
+    int nacc = layout_tiled(w_layout) ? 4 : 2;
     if (const char* env = option(OPT_PLANES_NACC)) nacc = atoi(env);
     const int min_nacc = (epi_op == EPI_SWIGLU_PAIRS) ? 2 : 1;
     while (nacc > min_nacc && ceil_div(p.tiles16, nacc) < 224) nacc >>= 1;
     if (nacc != 1 && nacc != 2 && nacc != 4) nacc = min_nacc;
-    if (w_layout != W_LAYOUT_TILED && nacc > 2) nacc = 2;
+    if (!layout_tiled(w_layout) && nacc > 2) nacc = 2;
     if (nacc < min_nacc) nacc = min_nacc;
     p.tiles = (int)ceil_div(p.tiles16, nacc);
     p.per_xcd = (int)ceil_div(p.tiles, 8);
@@ -923,7 +925,7 @@ int launch_planes(const void* X, const uint8_t* W, int w_layout, const Epilogue&
         else if (pro_op == PRO_SWIGLU) launch_planes_k<LAYOUT, NACC, EPI_NONE, false, PRO_SWIGLU>(p, st); \
         else launch_planes_k<LAYOUT, NACC>(p, st);                                                       \
     } while (0)
-    if (w_layout == W_LAYOUT_TILED) {
+    if (layout_tiled(w_layout)) {
         if (nacc == 4) BT_PL_LAUNCH(PL_TILED, 4);
         else if (nacc == 2) BT_PL_LAUNCH(PL_TILED, 2);
         else BT_PL_LAUNCH(PL_TILED, 1);
@@ -1056,6 +1058,7 @@ int launch_planes_bf16_wide(const void* X, const uint8_t* W, const Epilogue& epi
     p.G = 1;
     p.wsteps = (int)ceil_div(p.Kb, 16);
     p.tiles16 = (int)ceil_div(N, 16);
+    p.tiles16_signed = p.tiles16;
     if (!launch_walk(p, 1, resident_wgs(), -1, st)) return BT_ERR_INVALID;
     return check_launch("gemv_planes");
 }
@@ -1071,6 +1074,7 @@ int launch_planes_group(const void* const* X_tab, int x_dtype, const uint8_t* co
     p.G = (int)G;
     p.wsteps = (int)ceil_div(p.Kb, 16);
     p.tiles16 = (int)ceil_div(N, 16);
+    p.tiles16_signed = p.tiles16;
     return launch_group_params(p, G, st);
 }
 

@@ -54,7 +54,7 @@ struct StreamParams {
     int wsteps;           // 16-row steps of W_T; a step index beyond it wraps (see launch_stream)
     int tiles;            // column tiles
     int per_xcd;          // tiles per XCD (grid = 8 * per_xcd)
-    int tiles16;          // LD_T*: 16-column tiles of the decode-tiled weights
+    int tiles16;          // LD_T*: 16-column tiles of the decode-tiled weights (< 0: stored_tile16)
     int M;                // 1..16: rows of a 16-row block (of the last one when the launch covers several)
     int x_vec_ok;         // activation rows may be read with 16-byte loads
     int64_t B;            // rows of the whole call: grid.y = ceil(B / 16) blocks of 16 rows, all in one launch
@@ -239,7 +239,7 @@ __global__ __launch_bounds__(WAVES * 64) void stream_kernel(StreamParams p_in) {
         // computed on the last tile's bytes and never stored
 #pragma unroll
         for (int t = 0; t < NCO; t++)
-            coloff[t] = ((uint32_t)min(tile * NACC + t, p.tiles16 - 1) * (uint32_t)p.wsteps * 64u + (uint32_t)lane) * 4u;
+            coloff[t] = ((uint32_t)stored_tile16(tile * NACC + t, p.tiles16) * (uint32_t)p.wsteps * 64u + (uint32_t)lane) * 4u;
     } else if constexpr (QUAD) {
 #pragma unroll
         for (int cb = 0; cb < NCO; cb++) {
@@ -632,7 +632,7 @@ StreamPlan stream_plan(int mode, int64_t M, int64_t N, int64_t Kb, int w_layout,
     int o_ld = -1, o_waves = 0;
     if (const char* env = option(OPT_STREAM_CFG)) sscanf(env, "%d,%d", &o_ld, &o_waves);
     int ld;
-    if (w_layout == W_LAYOUT_TILED) {
+    if (layout_tiled(w_layout)) {
         // 16-column tiles, up to four per workgroup (a batch re-reads its activations once per workgroup, and so
         // does a prologue; 240 workgroups of two tiles tie with 480 of one at N = 7680 and win with a prologue)
         // (every 16-row block of the call is a grid row of the same launch: the workgroups of all blocks count)
@@ -819,7 +819,7 @@ int launch_stream(int mode, const void* X, int x_elem_size, const float* s_x, co
     p.epi = epi;
     p.N = N; p.K = Kx; p.Kb = Kb;
     p.wsteps = (int)ceil_div(Kb, 16);
-    p.tiles16 = (int)ceil_div(N, 16);
+    p.tiles16 = tiles16_arg(N, w_layout);
     p.prehalved = planes == 3;
     p.x_operand_order = (mode == MODE_I8 && q_layout == Q_OPERAND_ORDER) ? 1 : 0;
     p.pro_op = pro_op; p.pro_b = pro_b; p.pro_eps = pro_eps; p.epi_op = epi_op;

@@ -11,8 +11,10 @@ and releases the row-major buffer.  ``state_dict()`` still holds ``weight_packed
 (rebuilt from the tiled copy with ``bt_untile_weights``, bit for bit), ``load_state_dict`` and ``.to()`` /
 ``.cpu()`` work as usual.  Reading the attribute ``layer.weight_packed`` brings the row-major buffer back as a
 real buffer (so that in-place edits of it keep their meaning) and the layer then holds both copies until
-``drop_row_major()``; so does a call that only the row-major kernels can serve (the shape-generic kernel).  ``packed_weights()`` returns the reference-layout bytes without changing
-what the layer holds.  ``decode_tiled=False`` or ``BITTORCH_DECODE_TILED=0`` keeps the layer on ``weight_packed``
+``drop_row_major()``; so does a call that only the row-major kernels can serve once the buffer has been released
+(the shape-generic kernel; int8 activations on a fused gate|up layer stored in pair order).  A fused gate|up layer
+in pair order (``TernarySwiGLU``'s float default) serves decode and prefill, 16-bit and fp32, from its one tiled
+copy.  ``packed_weights()`` returns the reference-layout bytes without changing what the layer holds.  ``decode_tiled=False`` or ``BITTORCH_DECODE_TILED=0`` keeps the layer on ``weight_packed``
 alone.
 """
 
@@ -175,11 +177,17 @@ class TernaryLinearInference(nn.Module):
         return self
 
     def _tiled_for(self, x: Tensor, rows: int, order: str = "natural") -> Optional[Tensor]:
-        # (the tiled GEMMs read the copy too, so every batch size takes it; only the SwiGLU output stage of a
-        # pair-ordered copy is a decode-shape affair)
-        if not (self.decode_tiled and x.is_cuda and (rows <= DECODE_ROWS or order == "natural")
-                and self._tile_order == order):
+        """The tiled copy if this call can run on it, else None.  ``order`` is what the call wants: ``"natural"`` (a
+        plain linear output; a copy in gate/up pair order serves it too, the kernels looking every column tile up
+        where the pair order put it -- float activations only, see ``_natural_from_pairs``) or ``"gate_up_pairs"``
+        (the SwiGLU output stage: pair-ordered copy, decode shapes)."""
+        if not (self.decode_tiled and x.is_cuda):
             return None
+        if order == "gate_up_pairs":
+            if self._tile_order != order or rows > DECODE_ROWS:
+                return None
+        elif self._tile_order != "natural" and x.dtype == torch.int8:
+            return None  # the int8 entry point reads natural-order copies only
         if os.environ.get("BITTORCH_KERNEL") == "generic":  # the shape-generic kernel reads weight_packed
             return None
         if x.dtype not in (torch.float16, torch.bfloat16, torch.float32, torch.int8):
@@ -195,9 +203,25 @@ class TernaryLinearInference(nn.Module):
             return None
         return self.tiled_weights()
 
+    @property
+    def _natural_from_pairs(self) -> bool:
+        """True when a plain (natural column order) call reads a copy stored in gate/up pair order."""
+        return self._tile_order == "gate_up_pairs"
+
     def _row_major_for_call(self) -> Tensor:
-        """``weight_packed`` for a call that only the row-major kernels serve; a layer that had released it
-        holds both copies from here on."""
+        """``weight_packed`` for a call that only the row-major kernels serve (the shape-generic kernel, int8
+        activations on a pair-ordered copy, a first call inside a graph capture).  A layer that still holds the
+        buffer just hands it over; one that had released it rebuilds it and holds both copies from then on
+        (``drop_row_major()`` undoes that).  Inside a stream capture a released buffer cannot come back: the kernel
+        that rebuilds it would be recorded instead of run, and ``weight_packed`` would hold nothing until the first
+        replay."""
+        if self._has_row_major():
+            return self._buffers["weight_packed"]
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError(
+                "TernaryLinearInference: this call needs the row-major weight_packed, which the layer released after "
+                "building its decode-tiled copy, and a stream capture cannot rebuild it; read layer.weight_packed "
+                "(or make this call once) before capturing")
         return self._restore_row_major(keep=True)
 
     def forward(self, x: Tensor, residual: Optional[Tensor] = None, norm=None,
@@ -211,7 +235,8 @@ class TernaryLinearInference(nn.Module):
             if tiled is not None:
                 from .. import _C
                 return _C.ternary_linear_tiled_forward(x, tiled, self.scale, self.bias, self.in_features,
-                                                       self.out_features, residual, norm, swiglu_up)
+                                                       self.out_features, residual, norm, swiglu_up, False,
+                                                       self._natural_from_pairs)
         if x.is_cuda and (norm is not None or swiglu_up is not None):
             from .. import _C
             return _C.ternary_linear_packed_forward_fused(x, self._row_major_for_call(), self.scale, self.bias,

@@ -246,14 +246,18 @@ int bt_ternary_linear_packed_forward_fused(const void* X, int64_t ld_x, int x_dt
  *     epi_op = BT_EPI_SWIGLU_PAIRS (pair-ordered copy, no residual, no SwiGLU prologue): Y is [B, N/2],
  *     Y[b, h] = what bt_swiglu makes of the stored projections, rd(rd(silu(g)) * u) with g = rd(linear
  *     column h), u = rd(linear column N/2 + h): the SwiGLU MLP's hidden vector leaves the gate|up kernel
- *     itself (structure: TernaryTransformer.ts:366-423).  A pair-ordered copy serves only this output stage.
+ *     itself (structure: TernaryTransformer.ts:366-423).
+ *     epi_op = BT_EPI_NATURAL_FROM_PAIRS (pair-ordered copy): Y is the plain linear output [B, N] in the matrix's
+ *     natural column order, every kernel looking its column tiles up where the pair order put them; bit-identical
+ *     to the same call on a natural-order copy.  With the two, one pair-ordered copy serves every call of a fused
+ *     [gate | up] layer in 16-bit and fp32 activations (the int8 entry point reads natural-order copies only).
  *   bt_ternary_gemm_i8_tiled: bt_ternary_gemm_i8_res on the tiled copy (same remark).
  *   A tall batch on the tiled copy may take two kernel launches on the stream instead of one (the column tiles of
  *   a mostly empty last round of 128 x 256 tiles run as tiles of 64 or 32 rows behind the whole tiles): same
  *   results, nothing for the caller to do; both launches are captured by a HIP graph like any other.
  */
 enum { BT_TILES_NATURAL = 0, BT_TILES_GATE_UP_PAIRS = 1 };
-enum { BT_EPI_NONE = 0, BT_EPI_SWIGLU_PAIRS = 1 };
+enum { BT_EPI_NONE = 0, BT_EPI_SWIGLU_PAIRS = 1, BT_EPI_NATURAL_FROM_PAIRS = 2 };
 size_t bt_tiled_weights_bytes(int64_t N, int64_t K);
 int bt_retile_weights(const uint8_t* W_T, int64_t N, int64_t K, int order, uint8_t* W_tiled, void* stream);
 int bt_untile_weights(const uint8_t* W_tiled, int64_t N, int64_t K, int order, uint8_t* W_T, void* stream);

@@ -480,3 +480,113 @@ def test_ternary_swiglu_decode_uses_the_output_stage(oracle, dtype):
     # the fused layer called as an ordinary linear layer still gives [gate | up] in natural order
     x = seeded_acts(1, d, dtype=dtype).cuda()
     assert torch.equal(fused.gate_up(x), torch.cat([gate(x), up(x)], dim=-1))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("n,k", [(13824, 2560), (64, 64), (96, 100), (320, 1030), (8192, 4096)])
+def test_pair_ordered_copy_read_in_natural_order(oracle, dtype, n, k):
+    """A copy in gate/up pair order read as a plain linear layer (every kernel looks its column tiles up where the pair
+    order put them) gives the bits of the natural-order copy: exact GEMV, streaming kernel, tiled GEMM, fp32 planes,
+    with bias, residual and the RMSNorm prologue."""
+    from bittorch_amd import _C
+    _, wt = _packed(oracle, n, k, seed=11)
+    nat, pairs = _C.retile_weights(wt, k), _C.retile_weights(wt, k, True)
+    g = torch.Generator().manual_seed(n + k)
+    scale = (torch.rand(n, generator=g) + 0.5).cuda() * 0.05
+    bias = (torch.randn(n, generator=g) * 0.1).to(dtype).cuda()
+    nw = (torch.rand(k, generator=g) + 0.5).to(dtype).cuda()
+    for b, route in ((1, None), (3, None), (16, None), (40, None), (200, "32"), (200, "2000000")):
+        if route is not None:
+            set_option("STREAM_MAX_ROWS", route)  # 32: the tiled GEMM; 2000000: the streaming kernel
+        x = seeded_acts(b, k, seed=b, dtype=dtype).cuda()
+        res = seeded_acts(b, n, seed=b + 1, dtype=dtype).cuda()
+        for norm in (None, (nw, 1e-5)):
+            for bs, rs in ((None, None), (bias, res)):
+                announce("natural from pairs", dtype, n, k, b, route, norm is not None, bs is not None)
+                want = _C.ternary_linear_tiled_forward(x, nat, scale, bs, k, n, rs, norm)
+                got = _C.ternary_linear_tiled_forward(x, pairs, scale, bs, k, n, rs, norm, None, False, True)
+                assert torch.equal(got, want)
+        set_option("STREAM_MAX_ROWS", None)
+    x = seeded_acts(1, k, dtype=dtype).cuda()
+    if n % 32:
+        with pytest.raises(RuntimeError):
+            _C.ternary_linear_tiled_forward(x, pairs, scale, None, k, n, None, None, None, False, True)
+
+
+def test_fused_gate_up_layer_keeps_one_copy_through_prefill_and_capture(oracle):
+    """A TernarySwiGLU in its float default stores gate|up in pair order.  Decode, prefill (more rows than the decode
+    kernels take), fp32 activations and calls recorded into a HIP graph all read that one copy: the row-major buffer
+    never comes back, and the outputs equal those of the unfused MLP."""
+    from bittorch_amd.nn import TernarySwiGLU
+    d, ffn = 256, 704
+    gate, up, down = _layer(oracle, ffn, d, seed=1), _layer(oracle, ffn, d, seed=2), _layer(oracle, d, ffn, seed=3)
+    for L in (gate, up, down):
+        L.scale.mul_(0.05)
+    fused = TernarySwiGLU(gate, up, down, compute="float", fuse_gate_up=True)
+    plain = TernarySwiGLU(gate, up, down, compute="float", fuse_gate_up=False)
+    gu = fused.gate_up
+    one_copy = gu.packed_size_bytes
+    nw = (torch.rand(d) + 0.5).bfloat16().cuda()
+    fused(seeded_acts(1, d, dtype=torch.bfloat16).cuda())  # first call builds the copy and releases weight_packed
+    assert gu.resident_weight_bytes() == ((2 * ffn + 15) // 16) * (((d + 3) // 4 + 15) // 16) * 256 and not gu._has_row_major()
+    tiled_bytes = gu.resident_weight_bytes()
+    assert tiled_bytes < 2 * one_copy
+    for dtype, rows in ((torch.bfloat16, 300), (torch.float16, 150), (torch.float32, 1), (torch.float32, 200)):
+        announce("fused gate|up one copy", dtype, rows)
+        x = seeded_acts(rows, d, seed=rows, dtype=dtype).cuda()
+        y, ref = fused(x, nw.to(dtype), 1e-5, residual=x), plain(x, nw.to(dtype), 1e-5, residual=x)
+        assert rel_err(f32np(y), f32np(ref)) <= (1e-5 if dtype == torch.float32 else 1e-2)
+        assert gu.resident_weight_bytes() == tiled_bytes and not gu._has_row_major() and not gu.keep_row_major
+    # a prefill recorded into a graph: same copy, nothing rebuilt inside the capture
+    x = seeded_acts(300, d, seed=5, dtype=torch.bfloat16).cuda()
+    want = fused(x, nw, 1e-5, residual=x)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = fused(x, nw, 1e-5, residual=x)
+    for _ in range(2):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want)
+    assert gu.resident_weight_bytes() == tiled_bytes and not gu._has_row_major()
+    # the fused layer called as a plain linear layer: natural column order from the pair-ordered copy, bit for bit
+    x1 = seeded_acts(1, d, dtype=torch.float16).cuda()
+    assert torch.equal(gu(x1), torch.cat([gate(x1), up(x1)], dim=-1))
+    assert gu.resident_weight_bytes() == tiled_bytes
+
+
+def test_row_major_fallback_keeps_its_promises(oracle):
+    """(1) A layer whose first call is recorded into a graph runs that call on weight_packed without marking the buffer
+    as one to keep: prepare_decode() afterwards still leaves one copy.  (2) A call that needs a released weight_packed
+    inside a capture is refused instead of recording the kernel that would rebuild it."""
+    a = _layer(oracle, 256, 256, seed=2)
+    x = seeded_acts(1, 256, dtype=torch.bfloat16).cuda()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(s):
+        with torch.cuda.graph(g, stream=s):
+            a(x)
+    torch.cuda.current_stream().wait_stream(s)
+    assert not a.keep_row_major and a._has_row_major()
+    del g
+    a.prepare_decode()
+    assert not a._has_row_major() and a.resident_weight_bytes() == a._tiled.numel()
+    # (2) int8 activations on a pair-ordered copy are served by the row-major kernels
+    from bittorch_amd import _C
+    b = _layer(oracle, 256, 256, seed=3)
+    b.tile_order = "gate_up_pairs"
+    b.prepare_decode()
+    assert not b._has_row_major()
+    q, sx = _C.act_quant_int8(x, False)
+    s.wait_stream(torch.cuda.current_stream())
+    g2 = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="before capturing"):
+        with torch.cuda.stream(s):
+            with torch.cuda.graph(g2, stream=s):
+                b.forward_int8(q, sx)
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    want = _layer(oracle, 256, 256, seed=3, decode_tiled=False).forward_int8(q, sx)
+    assert torch.equal(b.forward_int8(q, sx), want)   # outside a capture: rebuilt, both copies held from here on
+    assert b.keep_row_major and b._has_row_major()
