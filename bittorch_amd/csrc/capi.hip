@@ -673,7 +673,7 @@ static int fused_forward_impl(const char* who, const void* X, int64_t ld_x, int 
                                                       : packed_uses_stream(x_dtype, W_T, Y, N, K);
     // a row that takes the exact fp16 GEMV gets its prologue inside that kernel (same element arithmetic as the row
     // kernel, so the result equals the unfused sequence bit for bit), or from the row kernel where that is switched off
-    if (B == 1 && !tuning_env("BITTORCH_NO_PROLOGUE") && ((uintptr_t)pro_b) % 16 == 0 && pro_b &&
+    if (B == 1 && !tuning_env("BITTORCH_NO_PROLOGUE") && ((uintptr_t)pro_b) % 16 == 0 && (pro_b || pro_op == PRO_RMSNORM) &&
         streams && planes_supported(x_dtype, x_dtype, B, N, K, X, W_T, Y, w_layout)) {
         if (epi_op != 0 && (epi_op != EPI_SWIGLU_PAIRS || w_layout != W_LAYOUT_TILED || N % 32 != 0 || residual)) {
             set_error("%s: the SwiGLU output stage needs pair-ordered tiled weights, N %% 32 == 0 and no residual", who);

@@ -331,7 +331,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(PlaneParams p) 
         for (int u = 0; u < XC; u++) {
             if (u * 64 < nchunks) {
                 const int k = s_begin * 64 + (lane + 64 * u) * 8;
-                br[u] = *(const uint4*)((const uint16_t*)p.pro_b + (uint32_t)min(k, (int)p.K - 8));
+                // (RMSNorm without a weight: ones, as the row kernel multiplies by 1)
+                if (p.pro_b) br[u] = *(const uint4*)((const uint16_t*)p.pro_b + (uint32_t)min(k, (int)p.K - 8));
+                else br[u] = make_uint4(0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u);
             }
         }
         float r = 0.0f;

@@ -421,3 +421,35 @@ def test_swiglu_module_decode_token_equals_batched_rows():
         h = _C.rmsnorm(x, nw, 1e-5)
         ref = down(_C.swiglu(gate(h), up(h))) + x
         assert torch.equal(got, ref)
+
+
+@pytest.mark.parametrize("tiled", [False, True])
+def test_rmsnorm_prologue_without_weight_gives_the_same_bits_with_and_without_workspace(tiled):
+    """One fp16 row under RMSNorm with no norm weight (ones), through the raw C ABI: the exact GEMV applies the
+    prologue itself whether or not the caller passes a workspace, so both calls return the bits of
+    "row kernel, then forward"."""
+    from bittorch_amd import _C, _lib
+    lib = _lib.load()
+    n, k = 1024, 512
+    packed, scale, bias = _packed_case(n, k, seed=9)
+    w = _C.retile_weights(packed, k) if tiled else packed
+    x = (seeded_acts(1, k, seed=3, dtype=torch.float16, outliers=True) * 2).cuda()
+    ref = _C.ternary_linear_packed_forward(_C.rmsnorm(x, None, 1e-5), packed, scale, bias, k)
+    st = torch.cuda.current_stream().cuda_stream
+    outs = []
+    for with_ws in (False, True):
+        announce("null norm weight", tiled, with_ws)
+        y = torch.full((1, n), float("nan"), dtype=torch.float16, device="cuda")
+        nbytes = lib.bt_packed_forward_fused_workspace_bytes(1, n, k, 1) if with_ws else 0
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device="cuda")
+        args = (x.data_ptr(), k, 1, 1, None, 0, 1e-5, w.data_ptr(), scale.data_ptr(), BT_DT[scale.dtype], n,
+                bias.data_ptr(), BT_DT[bias.dtype], None)
+        tail = (y.data_ptr(), 1, n, k, ws.data_ptr() if with_ws else None, nbytes, st)
+        if tiled:
+            rc = lib.bt_ternary_linear_tiled_forward(*args, 0, *tail)
+        else:
+            rc = lib.bt_ternary_linear_packed_forward_fused(*args, *tail)
+        assert rc == 0, _lib.last_error()
+        torch.cuda.synchronize()
+        outs.append(y)
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], ref)
