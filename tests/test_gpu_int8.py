@@ -139,9 +139,11 @@ def test_gemm_i8_close_to_float_path(oracle):
     assert rel_err(oy, truth) < 2e-2
 
 
-def test_gemm_i8_full_size_properties():
-    """Config-4 shape [2048,4096] x [4096,4096]: linearity in the weights' sign and
-    agreement of two independent kernels (streaming rows vs prefill tiles)."""
+def test_gemm_i8_full_size_properties(oracle):
+    """Config-4 shape [2048,4096] x [4096,4096]: linearity in the weights' sign, agreement of two independent
+    kernels (streaming rows vs prefill tiles), and the variant the benchmark times -- decode-tiled weights with
+    operand-order activations -- against the row-major entry point (accumulators and outputs) and against the oracle
+    on a 64 x 256 slice."""
     from bittorch_amd import _C
     from bittorch_amd.quant import pack_ternary_transposed
     announce("gemm_i8 full size")
@@ -162,3 +164,24 @@ def test_gemm_i8_full_size_properties():
     w127 = (w[:64].to(torch.int32) * 127)
     ref = q[:32].cpu().to(torch.int32) @ w127.t()
     assert torch.equal(acc[:32, :64].cpu(), ref)
+    # the benchmarked pair: decode-tiled weights, activations in operand order, bf16 outputs with scale and bias
+    g = torch.Generator().manual_seed(3)
+    scale_cpu = torch.rand(4096, generator=g) * 0.05 + 0.01
+    bias_cpu = torch.randn(4096, generator=g) * 0.01
+    scale2, bias2 = scale_cpu.cuda(), bias_cpu.cuda()
+    tiled = _C.retile_weights(packed, 4096)
+    q_oo, s_oo = _C.act_quant_int8(x, True)
+    assert torch.equal(s_oo, s)
+    y_rm, acc_rm = _C.ternary_gemm_int8(q, s, packed, scale2, bias2, 4096, out_dtype=torch.bfloat16, return_acc=True)
+    assert torch.equal(acc_rm, acc)
+    y_t, acc_t = _C.ternary_gemm_int8_tiled(q_oo, s, tiled, scale2, bias2, 4096, 4096, torch.bfloat16, True, None, True)
+    assert torch.equal(acc_t, acc) and torch.equal(y_t, y_rm)
+    y_t2 = _C.ternary_gemm_int8_tiled(q_oo, s, tiled, scale2, bias2, 4096, 4096, torch.bfloat16, False, None, True)
+    assert torch.equal(y_t2, y_rm)  # (without the accumulator output the epilogue takes its short path)
+    r0, c0 = 1984, 3840  # the last row tile and column tile of the 128 x 256 tiling
+    packed_cpu = packed.cpu().numpy()
+    oq, os_, oacc, oy = oracle.linear_i8(f32np(x[r0:r0 + 64].cpu()), np.ascontiguousarray(packed_cpu[:, c0:c0 + 256]),
+                                         f32np(scale_cpu[c0:c0 + 256]), 4096, f32np(bias_cpu[c0:c0 + 256]))
+    np.testing.assert_array_equal(q[r0:r0 + 64].cpu().numpy(), oq)
+    np.testing.assert_array_equal(acc_t[r0:r0 + 64, c0:c0 + 256].cpu().numpy(), oacc)
+    assert torch.equal(y_t2[r0:r0 + 64, c0:c0 + 256].cpu(), torch.from_numpy(oy).bfloat16())
