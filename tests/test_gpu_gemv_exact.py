@@ -363,3 +363,56 @@ def test_bf16_row_times_a_wide_matrix_and_argument_errors(oracle):
     assert "at most 16384" in _lib.last_error()
     assert lib.bt_ternary_gemv_grouped(p, 2, p, p, 0, 48, None, 2, p, 1, 48, 4104, None) == -1    # K % 16 != 0
     assert "multiple of 16" in _lib.last_error()
+
+
+def test_ops_ternary_linear_grouped_equals_the_single_calls(oracle):
+    """The caller the kept API offers for the grouped launch: `ops.ternary_linear_grouped(layers, xs)` returns, row
+    by row, the bits of `layer(x_row)` for fp16 rows (and the row-scaled exact sums for bf16 rows), with a shared
+    row, per-layer rows, an `out=` buffer, cached pointer tables that notice a layer whose buffers moved, and the
+    single-call fallback for what the grouped kernel does not take."""
+    import bittorch_amd as bt
+    from bittorch_amd.nn import TernaryLinearInference
+    n, k, g = 384, 512, 6
+    layers = []
+    for u in range(g):
+        w = random_ternary(n, k, seed=40 + u)
+        packed, _ = oracle.pack_ternary_transposed(w.numpy())
+        gen = torch.Generator().manual_seed(u)
+        layers.append(TernaryLinearInference(k, n, torch.from_numpy(packed), torch.rand(n, generator=gen) * 0.05 + 0.01,
+                                             (torch.randn(n, generator=gen) * 0.01).half()).cuda())
+    xs = seeded_acts(g, k, seed=3, dtype=torch.float16).cuda()
+    announce("ops.ternary_linear_grouped fp16")
+    want = torch.cat([L(xs[u:u + 1]) for u, L in enumerate(layers)])
+    got = bt.ops.ternary_linear_grouped(layers, xs)
+    assert got.shape == (g, n) and torch.equal(got, want)
+    # again (cached tables), into a caller's buffer, from a list of rows, and one row shared by every layer
+    out = torch.empty(g, n, dtype=torch.float16, device="cuda")
+    assert bt.ops.ternary_linear_grouped(layers, xs, out=out) is out and torch.equal(out, want)
+    assert torch.equal(bt.ops.ternary_linear_grouped(layers, [xs[u] for u in range(g)]), want)
+    shared = torch.cat([L(xs[:1]) for L in layers])
+    assert torch.equal(bt.ops.ternary_linear_grouped(layers, xs[0]), shared)
+    # a layer whose buffers moved: the cached tables are rebuilt
+    layers[2].scale = layers[2].scale.clone() * 2
+    want2 = torch.cat([L(xs[u:u + 1]) for u, L in enumerate(layers)])
+    assert torch.equal(bt.ops.ternary_linear_grouped(layers, xs), want2) and not torch.equal(want2, want)
+    # bf16 rows: exact row-scaled sums, within the single call's fp32 rounding
+    for L in layers:
+        L.bias = L.bias.bfloat16()
+    xb = xs.bfloat16()
+    got_b = bt.ops.ternary_linear_grouped(layers, xb)
+    want_b = torch.cat([L(xb[u:u + 1]) for u, L in enumerate(layers)])
+    np.testing.assert_allclose(f32np(got_b), f32np(want_b), rtol=1e-2, atol=1e-2)
+    # fallbacks: fp32 rows and CPU tensors run the single calls
+    xf = xs.float()
+    for L in layers:
+        L.bias = L.bias.float()
+    assert torch.equal(bt.ops.ternary_linear_grouped(layers, xf), torch.cat([L(xf[u:u + 1]) for u, L in enumerate(layers)]))
+    cpu_layers = [TernaryLinearInference(k, n, L.packed_weights().cpu(), L.scale.cpu(), L.bias.cpu()) for L in layers[:2]]
+    yc = bt.ops.ternary_linear_grouped(cpu_layers, xf[:2].cpu())
+    assert yc.shape == (2, n) and not yc.is_cuda
+    # argument errors in the reference's style
+    with pytest.raises(RuntimeError, match="doesn't match in_features"):
+        bt.ops.ternary_linear_grouped(layers, xs[:, :k - 16])
+    other = TernaryLinearInference(k, n + 16, torch.zeros(k // 4, n + 16, dtype=torch.uint8), torch.ones(n + 16)).cuda()
+    with pytest.raises(ValueError, match="same in_features and out_features"):
+        bt.ops.ternary_linear_grouped(layers + [other], xs[0])
