@@ -371,6 +371,31 @@ def ternary_gemv_grouped(x_tab: Tensor, w_tiled_tab: Tensor, scale_tab: Tensor, 
             out_features, in_features, _stream(x_tab)))
 
 
+def ternary_gemm_int8_grouped(q_tab: Tensor, sx_tab: Tensor, w_tiled_tab: Tensor, scale_tab: Tensor,
+                              bias_tab: Optional[Tensor], y_tab: Tensor, rows: int, in_features: int, out_features: int,
+                              scale_len: int = -1, scale_dtype: torch.dtype = torch.float32,
+                              bias_dtype: torch.dtype = torch.float32, out_dtype: torch.dtype = torch.bfloat16,
+                              q_operand_order: bool = False, acc_tab: Optional[Tensor] = None) -> None:
+    """``G`` independent int8 units of ``rows`` (at most 16) activation rows each in one launch: unit ``u`` multiplies
+    the int8 rows at ``q_tab[u]`` (row scales at ``sx_tab[u]``) with the decode-tiled weights at ``w_tiled_tab[u]``
+    into ``y_tab[u]`` ``[rows, N]``, exactly as :func:`ternary_gemm_int8_tiled` would (same accumulators, same bits).
+    The tables are int64 device tensors of ``G`` device addresses (:func:`pointer_table`); ``acc_tab`` optionally
+    receives the int32 accumulators; nothing is allocated or returned."""
+    G = q_tab.numel()
+    tabs = (q_tab, sx_tab, w_tiled_tab, scale_tab, y_tab) + tuple(t for t in (bias_tab, acc_tab) if t is not None)
+    for t in tabs:
+        _check(t.dtype == torch.int64 and t.dim() == 1 and t.numel() == G and t.is_contiguous(),
+               "pointer tables must be contiguous int64 tensors of one length")
+    _check(_all_cuda(*tabs), "All tensors must be CUDA")
+    _check(scale_dtype in _DT and bias_dtype in _DT and out_dtype in _DT,
+           "scale / bias / output dtype must be float32, float16 or bfloat16")
+    with torch.cuda.device(q_tab.device):
+        _status(_L.bt_ternary_gemm_i8_grouped(
+            q_tab.data_ptr(), 1 if q_operand_order else 0, sx_tab.data_ptr(), w_tiled_tab.data_ptr(), scale_tab.data_ptr(),
+            _DT[scale_dtype], out_features if scale_len < 0 else scale_len, _ptr(bias_tab), _DT[bias_dtype],
+            y_tab.data_ptr(), _DT[out_dtype], _ptr(acc_tab), G, rows, out_features, in_features, _stream(q_tab)))
+
+
 def ternary_gemm_int8_tiled(Q: Tensor, s_x: Tensor, W_tiled: Tensor, scale: Tensor, bias: Optional[Tensor] = None,
                             in_features: int = -1, out_features: int = -1,
                             out_dtype: torch.dtype = torch.float32, return_acc: bool = False,

@@ -43,6 +43,8 @@ SIGNATURES = {
     "bt_ternary_linear_tensor_core_forward_static": (_int, [_vp, _int, _vp, _vp, _int, _i64, _vp, _int, _vp,
                                                             _i64, _i64, _i64, _vp]),
     "bt_ternary_gemv_grouped": (_int, [_vp, _int, _vp, _vp, _int, _i64, _vp, _int, _vp, _i64, _i64, _i64, _vp]),
+    "bt_ternary_gemm_i8_grouped": (_int, [_vp, _int, _vp, _vp, _vp, _int, _i64, _vp, _int, _vp, _int, _vp, _i64, _i64,
+                                          _i64, _i64, _vp]),
     "bt_unpack_dequant": (_int, [_vp, _vp, _i64, _vp, _int, _i64, _i64, _vp]),
     "bt_pack_ternary_i8": (_int, [_vp, _i64, _i64, _vp, _vp]),
     "bt_ternary_linear_packed_forward_res": (_int, [_vp, _int, _vp, _vp, _int, _i64, _vp, _int, _vp, _vp,

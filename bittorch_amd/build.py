@@ -17,7 +17,7 @@ CSRC = os.path.join(_HERE, "csrc")
 OUT_DIR = os.path.join(_HERE, "_hip")
 LIB_PATH = os.path.join(OUT_DIR, "libbittorch_hip.so")
 
-SOURCES = ["capi.hip", "quantize_pack.hip", "stream_gemm.hip", "gemv_planes.hip", "gemm_i8.hip", "gemm_f16.hip", "act_quant.hip", "row_ops.hip", "misc_kernels.hip"]
+SOURCES = ["capi.hip", "quantize_pack.hip", "stream_gemm.hip", "gemv_planes.hip", "gemv_i8_group.hip", "gemm_i8.hip", "gemm_f16.hip", "act_quant.hip", "row_ops.hip", "misc_kernels.hip"]
 
 # packed fp32 VALU forms are disabled on purpose (they have produced wrong
 # results on this hardware generation's boxes); the host pass warns that it

@@ -92,6 +92,11 @@ int launch_planes(const void* X, const uint8_t* W, int w_layout, const Epilogue&
 int launch_planes_group(const void* const* X_tab, int x_dtype, const uint8_t* const* W_tab, const void* const* scale_tab,
                         int scale_dtype, int scale_bcast, const void* const* bias_tab, int bias_dtype, void* const* Y_tab,
                         int64_t G, int64_t N, int64_t K, hipStream_t st);
+bool i8_group_supported(int64_t K);
+int launch_i8_group(const int8_t* const* Q_tab, int q_layout, const float* const* sx_tab, const uint8_t* const* W_tab,
+                    const void* const* scale_tab, int scale_dtype, int scale_bcast, const void* const* bias_tab,
+                    int bias_dtype, void* const* Y_tab, int y_dtype, int32_t* const* acc_tab, int64_t G, int64_t M,
+                    int64_t N, int64_t K, hipStream_t st);
 bool planes_bf16_shape_ok(int64_t N, int64_t K);
 bool planes_bf16_wide(int64_t N, int64_t K);
 int launch_planes_bf16_wide(const void* X, const uint8_t* W, const Epilogue& epi, void* Y, int64_t N, int64_t K, hipStream_t st);
@@ -595,6 +600,47 @@ extern "C" int bt_ternary_gemv_grouped(const void* const* X_tab, int x_dtype, co
     }
     return launch_planes_group(X_tab, x_dtype, W_tiled_tab, scale_tab, scale_dtype, (scale_len == 1 && N != 1) ? 1 : 0, bias_tab,
                                bias_dtype, Y_tab, G, N, K, (hipStream_t)stream);
+}
+
+// ---- G small-batch int8 units in one launch ------------------------------------------------------
+extern "C" int bt_ternary_gemm_i8_grouped(const int8_t* const* Q_tab, int q_layout, const float* const* sx_tab,
+                                          const uint8_t* const* W_tiled_tab, const void* const* scale_tab,
+                                          int scale_dtype, int64_t scale_len, const void* const* bias_tab,
+                                          int bias_dtype, void* const* Y_tab, int y_dtype, int32_t* const* acc_tab,
+                                          int64_t G, int64_t M, int64_t N, int64_t K, void* stream) {
+    const char* who = "bt_ternary_gemm_i8_grouped";
+    if (!Q_tab || !sx_tab || !W_tiled_tab || !scale_tab || !Y_tab) {
+        set_error("%s: null pointer table", who);
+        return BT_ERR_INVALID;
+    }
+    if (G <= 0 || N <= 0 || K <= 0 || M <= 0 || G > (1 << 20)) {
+        set_error("%s: empty shape or too many units (G=%lld M=%lld N=%lld K=%lld)", who, (long long)G, (long long)M,
+                  (long long)N, (long long)K);
+        return BT_ERR_INVALID;
+    }
+    if (M > 16) {
+        set_error("%s: a unit has at most 16 activation rows (M=%lld)", who, (long long)M);
+        return BT_ERR_INVALID;
+    }
+    if (!i8_group_supported(K)) {
+        set_error("%s: K must be a multiple of 16 and at most 11264 (K=%lld)", who, (long long)K);
+        return BT_ERR_INVALID;
+    }
+    if (q_layout != Q_ROW_MAJOR && q_layout != Q_OPERAND_ORDER) {
+        set_error("%s: q_layout must be BT_Q_ROW_MAJOR or BT_Q_OPERAND_ORDER (got %d)", who, q_layout);
+        return BT_ERR_INVALID;
+    }
+    if ((scale_len != N && scale_len != 1) || !valid_dtype(scale_dtype) || (bias_tab && !valid_dtype(bias_dtype)) ||
+        !valid_dtype(y_dtype)) {
+        set_error("%s: scale size doesn't match N, or unsupported scale/bias/output dtype", who);
+        return BT_ERR_INVALID;
+    }
+    if (tiled_bytes(N, K) >= (1ull << 32) || G * ceil_div(N, 16) >= (1ll << 31) || 17 * K >= (1ll << 31)) {
+        set_error("%s: a unit's tiled weights must stay below 4 GiB", who);
+        return BT_ERR_INVALID;
+    }
+    return launch_i8_group(Q_tab, q_layout, sx_tab, W_tiled_tab, scale_tab, scale_dtype, (scale_len == 1 && N != 1) ? 1 : 0,
+                           bias_tab, bias_dtype, Y_tab, y_dtype, acc_tab, G, M, N, K, (hipStream_t)stream);
 }
 
 // ---- fused producers of the GEMM activations (row_ops.hip) ----------------------------------

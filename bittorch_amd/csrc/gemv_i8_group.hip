@@ -1,0 +1,343 @@
+// G independent small-batch int8 units in one launch (HBM-bound): unit u multiplies its int8-quantized activation
+// rows Q_u [M <= 16, K] (row scales s_x_u [M]) with the decode-tiled ternary weights W_u into Y_u [M, N].
+//
+// Arithmetic of the reference's tensor-core kernel with the whole-row activation scale
+// (csrc/kernels/ternary_gemm_tensor_core.cu:343-347, :439, :583-589, :652), exactly as bt_ternary_gemm_i8_tiled
+// computes it for the same unit: acc_i32[m,n] = sum_k q[m,k] * 127 w[k,n] (summed on +-1 weights and multiplied by
+// 127 exactly), y = ((float(acc) * s_x[m]) / 127) * scale[n] + bias[n].  Integer sums: the result does not depend
+// on how K is split, so every unit equals the single call bit for bit.
+//
+// The reference serves one matrix per launch (ternary_gemm_production.cu:286-362); a decode-shape matrix streams in
+// less time than a kernel takes to start, and at M = 16 a one-matrix kernel re-reads the activations in every
+// workgroup (176 KB per workgroup for K = 11008, four times the weight bytes it streams).  Here persistent
+// workgroups walk the flat sequence of (unit, 16-column tile) pairs: a workgroup owns a contiguous run of it, its
+// waves split K -- wave w reads steps w * SPW .. + SPW - 1 of every tile, SPW * 256 consecutive bytes -- so the
+// workgroup reads its share of the weights front to back, the pattern that streams fastest on this chip.  A wave's
+// slice of the unit's 16 activation rows is the same for every tile of the unit: it is loaded once per unit into
+// SPW * 4 registers, already in matrix-core operand order, and the loop has no activation traffic at all.  The waves'
+// partial sums (16 rows x 16 columns of int32 per tile) meet in LDS atomics in one of two accumulator arrays; every
+// 16 or 24 tiles a barrier ends the chunk and the threads finish its outputs (epilogue, stores, clearing) while the
+// waves already add the next chunk into the other array.  TB tiles of weight loads are in flight per wave at all
+// times, across chunk and unit boundaries.
+#include <cstddef>
+
+#include "bt_common.h"
+
+namespace bt {
+
+// Tiles per chunk (I8_EB tiles x 16 rows x 16 columns of int32 per accumulator array): 24 with 8 waves, 16 with 16,
+// as measured (G = 32 units of 16 x 4096 -> 11008: 16 tiles 80.3 us, 24 tiles 73.6, 30 tiles 77.0; 16 x 11008 -> 4096
+// on 16 waves: 77.7, 81.0, 83.4).
+template <int WAVES> constexpr int i8_eb() { return WAVES == 8 ? 24 : 16; }
+
+struct I8GroupParams {
+    // tables of G device pointers
+    const int8_t* const* Q_tab;
+    const uint8_t* const* W_tab;
+    const float* const* sx_tab;
+    const void* const* scale_tab;
+    const void* const* bias_tab;  // may be null
+    void* const* Y_tab;
+    int32_t* const* acc_tab;      // may be null: raw accumulators [M, N] per unit
+    int64_t K, N;
+    int wsteps;        // 16-row steps of the weights (64 k each)
+    int tiles16;       // 16-column tiles
+    int G, M;
+    int tiles_per_wg;  // a multiple of TB
+    int q_operand_order;
+    int y_dtype, scale_dtype, bias_dtype, scale_bcast;
+};
+
+__device__ __forceinline__ void i8g_store(void* Y, int dt, int64_t idx, float v) {
+    if (dt == BT_F32) ((float*)Y)[idx] = v;
+    else if (dt == BT_F16) ((uint16_t*)Y)[idx] = f32_to_f16_bits(v);
+    else ((uint16_t*)Y)[idx] = f32_to_bf16_bits(v);
+}
+
+// Raw bits of NV (8 or 4) consecutive entries n0 .. n0 + NV - 1 of a scale / bias vector (entries past N repeat the
+// last one; bcast: one entry for all).  Whole aligned pieces come as 16- or 8-byte loads.
+template <int NV>
+__device__ __forceinline__ void load_bits_n(const void* v, int dt, int bcast, int64_t n0, int64_t N, uint32_t (&out)[NV]) {
+    if (bcast) {
+        const uint32_t b = load_bits_rt(v, dt, 0);
+#pragma unroll
+        for (int c = 0; c < NV; c++) out[c] = b;
+        return;
+    }
+    const bool whole = n0 + NV <= N && (n0 % NV) == 0 && (((uintptr_t)v) & 15) == 0;
+    if (whole && dt == BT_F32) {
+#pragma unroll
+        for (int c = 0; c < NV; c += 4) {
+            const uint4 a = *(const uint4*)((const uint32_t*)v + n0 + c);
+            out[c] = a.x; out[c + 1] = a.y; out[c + 2] = a.z; out[c + 3] = a.w;
+        }
+    } else if (whole) {
+        uint32_t d[NV / 2];
+        if constexpr (NV == 8) {
+            const uint4 a = *(const uint4*)((const uint16_t*)v + n0);
+            d[0] = a.x; d[1] = a.y; d[2] = a.z; d[3] = a.w;
+        } else {
+            const uint2 a = *(const uint2*)((const uint16_t*)v + n0);
+            d[0] = a.x; d[1] = a.y;
+        }
+#pragma unroll
+        for (int c = 0; c < NV; c++) out[c] = (d[c >> 1] >> (16 * (c & 1))) & 0xffffu;
+    } else {
+#pragma unroll
+        for (int c = 0; c < NV; c++) out[c] = load_bits_rt(v, dt, (n0 + c < N) ? n0 + c : N - 1);
+    }
+}
+
+template <int SPW, int TB, int WAVES>
+__global__ __launch_bounds__(WAVES * 64, 4) void gemv_i8_walk_kernel(I8GroupParams p) {
+    constexpr int I8_EB = i8_eb<WAVES>();
+    // Row stride of an accumulator array in ints: 4 past a multiple of 8 puts the four row groups a matrix-core result
+    // spreads over the lanes (rows 4g .. 4g+3) on two sets of banks instead of one (G = 32 units as above, 16 tiles
+    // per chunk: 87.1 -> 80.3 us).
+    constexpr int I8_ROW = I8_EB * 16 + 4;
+    static_assert(I8_EB % TB == 0, "chunks hold whole batches");
+    constexpr int THREADS = WAVES * 64;
+    __shared__ __attribute__((aligned(16))) int32_t accbuf[2][16][I8_ROW];    // [array][row][16 * tile + column]
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 15, g = lane >> 4;
+    const int S = p.wsteps;
+    const int T16 = p.tiles16;
+    const int M = p.M;
+    const int64_t total = (int64_t)p.G * T16;
+    const int64_t t_begin = (int64_t)blockIdx.x * p.tiles_per_wg;
+    const int64_t t_end = (t_begin + p.tiles_per_wg < total) ? t_begin + p.tiles_per_wg : total;
+    if (t_begin >= t_end) return;
+
+    for (int i = tid; i < 2 * 16 * I8_ROW; i += THREADS) (&accbuf[0][0][0])[i] = 0;
+
+    // byte offset of this wave's SPW steps inside a tile (a step past the end repeats the last one and meets zeroed
+    // activations)
+    // (wave-uniform step offsets and one per-lane offset: the loads take a scalar base and a 32-bit lane offset)
+    uint32_t soff[SPW];
+#pragma unroll
+    for (int f = 0; f < SPW; f++) soff[f] = (uint32_t)__builtin_amdgcn_readfirstlane(min(wave * SPW + f, S - 1) * 256);
+    const uint32_t lane_off = (uint32_t)lane * 4u;
+    const size_t tile_bytes = (size_t)S * 256;
+
+    // prefetch cursor: (unit, tile) of the next tile to request
+    int pf_u = (int)(t_begin / T16);
+    int pf_t = (int)(t_begin - (int64_t)pf_u * T16);
+    int64_t pf_left = t_end - t_begin;
+    const uint8_t* pf_ptr = p.W_tab[pf_u] + (size_t)pf_t * tile_bytes;
+    uint32_t raw[TB][SPW];
+    auto request = [&](uint32_t (&dst)[SPW]) {
+        // (past the end of the run: the last tile again, never used)
+#pragma unroll
+        for (int f = 0; f < SPW; f++) dst[f] = ldw_nt((pf_ptr + soff[f]) + lane_off);
+        if (pf_left > 1) {
+            pf_left--;
+            pf_t++;
+            pf_ptr += tile_bytes;
+            if (pf_t == T16) {
+                pf_t = 0;
+                pf_u++;
+                pf_ptr = p.W_tab[pf_u];
+            }
+        }
+    };
+    // A fragment of step f: lane (i = j, g) feeds row i, k = 64 step + 16 g .. + 15 (rows past M repeat the last row
+    // and only reach outputs that are never stored; K is a multiple of 16, so a group below K lies inside its row)
+    const uint32_t a_row = (uint32_t)min(j, M - 1) * (uint32_t)p.K;
+    uint4 areg[SPW];
+    auto load_a = [&](const int8_t* q) {
+#pragma unroll
+        for (int f = 0; f < SPW; f++) {
+            const int k = (wave * SPW + f) * 64 + 16 * g;
+            areg[f] = *(const uint4*)(q + a_row + (uint32_t)min(k, (int)p.K - 16));
+        }
+    };
+    auto finish_a = [&]() {
+#pragma unroll
+        for (int f = 0; f < SPW; f++) {
+            const int k = (wave * SPW + f) * 64 + 16 * g;
+            uint4 v = areg[f];
+            if (!p.q_operand_order) {  // (uniform) row-major bytes -> the matrix cores' order
+                uint32_t t[4];
+                transpose4x4_bytes(v.x, v.y, v.z, v.w, t);
+                v = make_uint4(t[0], t[1], t[2], t[3]);
+            }
+            const bool ok = k < (int)p.K;
+            areg[f] = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+        }
+    };
+    // the first unit's activations are requested ahead of the weights (loads return in order; they are needed first)
+    load_a(p.Q_tab[pf_u]);
+#pragma unroll
+    for (int i = 0; i < TB; i++) request(raw[i]);
+
+    int cur = 0;
+    __syncthreads();  // accumulators cleared
+
+    int64_t t0 = t_begin;
+    while (t0 < t_end) {
+        const int u = (int)(t0 / T16);
+        const int tile0 = (int)(t0 - (int64_t)u * T16);
+        if (t0 != t_begin) load_a(p.Q_tab[u]);  // (uniform)
+        finish_a();
+        const float* sx_u = p.sx_tab[u];
+        const void* scale_u = p.scale_tab[u];
+        const void* bias_u = p.bias_tab ? p.bias_tab[u] : nullptr;
+        const int64_t unit_end = (int64_t)(u + 1) * T16;
+        const int64_t u_stop = (unit_end < t_end) ? unit_end : t_end;
+        for (int64_t c0 = t0; c0 < u_stop; c0 += I8_EB) {
+            const int ntiles = (int)((u_stop - c0 < I8_EB) ? u_stop - c0 : I8_EB);  // a multiple of TB
+            for (int tb = 0; tb < ntiles; tb += TB) {
+                v4i acc[TB];
+#pragma unroll
+                for (int i = 0; i < TB; i++) acc[i] = v4i{0, 0, 0, 0};
+#pragma unroll
+                for (int f = 0; f < SPW; f++) {
+                    const v4i a = {(int)areg[f].x, (int)areg[f].y, (int)areg[f].z, (int)areg[f].w};
+#pragma unroll
+                    for (int i = 0; i < TB; i++)
+                        acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, decode16_i8(raw[i][f]), acc[i], 0, 0, 0);
+                }
+#pragma unroll
+                for (int i = 0; i < TB; i++) request(raw[i]);
+                // lane (j, g) holds rows 4g .. 4g+3 of column j
+#pragma unroll
+                for (int i = 0; i < TB; i++) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) atomicAdd(&accbuf[cur][4 * g + r][16 * (tb + i) + j], acc[i][r]);
+                }
+            }
+            __syncthreads();  // every wave has added its share of this chunk
+            // The chunk's epilogue: 16 rows x 256 columns in pieces of four columns (an 8-byte piece of a 16-bit output
+            // row; consecutive threads cover a row's columns with full-line stores), in passes over the threads.
+            // The operands are requested here rather than a chunk ahead: held across the chunk's matrix instructions
+            // they cost more registers than the wave has, and the loads that wait here are covered by the other
+            // workgroup of the compute unit and by the weight loads already in flight.
+#pragma unroll 1
+            for (int item = tid; item < I8_EB * 64; item += THREADS) {
+                const int e_row = item / (4 * I8_EB), e_tl = (item % (4 * I8_EB)) >> 2, e_j0 = 4 * (item & 3);
+                if (e_tl >= ntiles) continue;
+                const int64_t n0 = (int64_t)(tile0 + (int)(c0 - t0) + e_tl) * 16 + e_j0;
+                const bool e_on = n0 < p.N && e_row < M;
+                uint32_t pre_s[4], pre_b[4];
+                float pre_sx = 0.0f;
+                if (e_on) {
+                    pre_sx = sx_u[e_row];
+                    load_bits_n<4>(scale_u, p.scale_dtype, p.scale_bcast, n0, p.N, pre_s);
+                    if (bias_u) load_bits_n<4>(bias_u, p.bias_dtype, 0, n0, p.N, pre_b);
+                }
+                int32_t* src = &accbuf[cur][e_row][16 * e_tl + e_j0];
+                const int4 v = *(const int4*)src;
+                *(int4*)src = make_int4(0, 0, 0, 0);
+                if (!e_on) continue;
+                const int32_t a[4] = {v.x, v.y, v.z, v.w};
+                int32_t a127[4];
+                float y[4];
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    a127[c] = times127(a[c]);  // the matrix cores ran on +-1 weights
+                    const float sc = bits_to_f32_rt(pre_s[c], p.scale_dtype);
+                    const float bs = bias_u ? bits_to_f32_rt(pre_b[c], p.bias_dtype) : 0.0f;
+                    y[c] = epi_int8(a127[c], pre_sx, sc, bs);
+                }
+                const int64_t idx = (int64_t)e_row * p.N + n0;
+                void* y_u = p.Y_tab[u];
+                int32_t* acc_u = p.acc_tab ? p.acc_tab[u] : nullptr;
+                // whole pieces leave as vector stores (rows of N % 8 == 0 columns from a 16-byte aligned base)
+                const bool vec = n0 + 4 <= p.N && (p.N & 7) == 0 && (((uintptr_t)y_u) & 15) == 0 &&
+                                 (!acc_u || (((uintptr_t)acc_u) & 15) == 0);
+                if (vec) {
+                    if (p.y_dtype == BT_F32) {
+                        st4_nt((float*)y_u + idx, __builtin_bit_cast(uint32_t, y[0]), __builtin_bit_cast(uint32_t, y[1]),
+                               __builtin_bit_cast(uint32_t, y[2]), __builtin_bit_cast(uint32_t, y[3]));
+                    } else {
+                        uint32_t h[2];
+#pragma unroll
+                        for (int c = 0; c < 2; c++) {
+                            const uint32_t l = (p.y_dtype == BT_F16) ? f32_to_f16_bits(y[2 * c]) : f32_to_bf16_bits(y[2 * c]);
+                            const uint32_t m = (p.y_dtype == BT_F16) ? f32_to_f16_bits(y[2 * c + 1]) : f32_to_bf16_bits(y[2 * c + 1]);
+                            h[c] = l | (m << 16);
+                        }
+                        st2_nt((uint16_t*)y_u + idx, h[0], h[1]);
+                    }
+                    if (acc_u) st4_nt(acc_u + idx, (uint32_t)a127[0], (uint32_t)a127[1], (uint32_t)a127[2], (uint32_t)a127[3]);
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 4; c++) {
+                        if (n0 + c < p.N) {
+                            i8g_store(y_u, p.y_dtype, idx + c, y[c]);
+                            if (acc_u) acc_u[idx + c] = a127[c];
+                        }
+                    }
+                }
+            }
+            cur ^= 1;
+        }
+        t0 = u_stop;
+    }
+}
+
+// ---- host side ------------------------------------------------------------------------------------------------------
+static int64_t i8g_compute_units() {
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cus = n;
+    }
+    return cus;
+}
+
+template <int SPW, int WAVES>
+static void launch_i8_walk_tb(const I8GroupParams& p, int tb, unsigned grid, hipStream_t st) {
+    if (tb == 2) hipLaunchKernelGGL((gemv_i8_walk_kernel<SPW, 2, WAVES>), dim3(grid), dim3(WAVES * 64), 0, st, p);
+    else hipLaunchKernelGGL((gemv_i8_walk_kernel<SPW, 1, WAVES>), dim3(grid), dim3(WAVES * 64), 0, st, p);
+}
+
+// K up to 4096 (64 steps): 8 waves, two workgroups per compute unit; up to 11264 (176 steps): 16 waves, one.
+bool i8_group_supported(int64_t K) { return K % 16 == 0 && K >= 16 && K <= 11264; }
+
+int launch_i8_group(const int8_t* const* Q_tab, int q_layout, const float* const* sx_tab, const uint8_t* const* W_tab,
+                    const void* const* scale_tab, int scale_dtype, int scale_bcast, const void* const* bias_tab,
+                    int bias_dtype, void* const* Y_tab, int y_dtype, int32_t* const* acc_tab, int64_t G, int64_t M,
+                    int64_t N, int64_t K, hipStream_t st) {
+    I8GroupParams p = {};
+    p.Q_tab = Q_tab; p.W_tab = W_tab; p.sx_tab = sx_tab; p.scale_tab = scale_tab; p.bias_tab = bias_tab;
+    p.Y_tab = Y_tab; p.acc_tab = acc_tab;
+    p.K = K; p.N = N;
+    p.wsteps = (int)ceil_div(ceil_div(K, 4), 16);
+    p.tiles16 = (int)ceil_div(N, 16);
+    p.G = (int)G; p.M = (int)M;
+    p.q_operand_order = q_layout == Q_OPERAND_ORDER;
+    p.y_dtype = y_dtype; p.scale_dtype = scale_dtype; p.bias_dtype = bias_dtype; p.scale_bcast = scale_bcast;
+    const bool wide = p.wsteps > 64;
+    const int waves = wide ? 16 : 8;
+    const int spw = (int)ceil_div(p.wsteps, waves);
+    const int tb = (p.tiles16 % 2 == 0) ? 2 : 1;  // chunks inside a unit hold whole batches of tiles
+    const int64_t wgs = (wide ? 1 : 2) * i8g_compute_units();
+    const int64_t total = G * p.tiles16;
+    const int64_t tpw = ceil_div(ceil_div(total, wgs), tb) * tb;
+    p.tiles_per_wg = (int)tpw;
+    const unsigned grid = (unsigned)ceil_div(total, tpw);
+#define BT_I8G_CASE(SPW, WAVES) case SPW: launch_i8_walk_tb<SPW, WAVES>(p, tb, grid, st); break;
+    if (!wide) {
+        switch (spw) {
+            BT_I8G_CASE(1, 8) BT_I8G_CASE(2, 8) BT_I8G_CASE(3, 8) BT_I8G_CASE(4, 8)
+            BT_I8G_CASE(5, 8) BT_I8G_CASE(6, 8) BT_I8G_CASE(7, 8)
+            default: launch_i8_walk_tb<8, 8>(p, tb, grid, st); break;
+        }
+    } else {
+        switch (spw) {
+            BT_I8G_CASE(5, 16) BT_I8G_CASE(6, 16) BT_I8G_CASE(7, 16) BT_I8G_CASE(8, 16)
+            BT_I8G_CASE(9, 16) BT_I8G_CASE(10, 16)
+            default: launch_i8_walk_tb<11, 16>(p, tb, grid, st); break;
+        }
+    }
+#undef BT_I8G_CASE
+    return check_launch("bt_ternary_gemm_i8_grouped");
+}
+
+}  // namespace bt

@@ -305,6 +305,27 @@ int bt_ternary_gemv_grouped(const void* const* X_tab, int x_dtype, const uint8_t
                             int64_t N, int64_t K, void* stream);
 
 /*
+ * G independent small-batch int8 units in ONE launch (no counterpart in the reference, as above): unit u computes
+ *   Y_tab[u] [M, N] = Q_tab[u] [M, K] (int8, row scales sx_tab[u] [M]) x W_tiled_tab[u] -> ((acc * s_x) / 127) * scale + bias
+ * exactly as bt_ternary_gemm_i8_tiled would for that unit: int32 accumulators and outputs bit-identical (the
+ * arithmetic of csrc/kernels/ternary_gemm_tensor_core.cu:343-347, :439, :583-589, :652 with the whole-row scale).
+ * M <= 16 rows per unit, the same M, N, K, layouts and element types for every unit: batched decode steps through
+ * several same-shaped layers (BASELINE config 3's shapes: 16 x 4096 -> 11008 and 16 x 11008 -> 4096).  Persistent
+ * workgroups read the flat (unit, 16-column tile) sequence of the tiled copies front to back, their waves splitting
+ * K; a wave keeps its K slice of the unit's 16 rows in registers for all of the unit's tiles, so the activations are
+ * read once per workgroup and unit instead of once per workgroup and tile.
+ *   The tables are DEVICE arrays of G device pointers, caller-owned; bias_tab and acc_tab may be NULL (no bias; no
+ *   accumulator output), their entries may not be NULL otherwise.  q_layout as in bt_ternary_gemm_i8_res.
+ *   K % 16 == 0, K <= 11264; each Q 16-byte aligned, each W_tiled 256-byte aligned; acc_tab[u] [M, N] int32 receives
+ *   the accumulators (sum q * 127 w).  Units may share operands but not outputs.
+ */
+int bt_ternary_gemm_i8_grouped(const int8_t* const* Q_tab, int q_layout, const float* const* sx_tab,
+                               const uint8_t* const* W_tiled_tab, const void* const* scale_tab, int scale_dtype,
+                               int64_t scale_len, const void* const* bias_tab, int bias_dtype, void* const* Y_tab,
+                               int y_dtype, int32_t* const* acc_tab, int64_t G, int64_t M, int64_t N, int64_t K,
+                               void* stream);
+
+/*
  * Matrix-core forward from float activations: bt_act_quant_i8 followed by
  * bt_ternary_gemm_i8.  Replaces bittorch._C.ternary_linear_tensor_core_forward
  * (bittorch_bindings.cpp:65-87, ternary_gemm_tensor_core.cu:663-727) for
