@@ -157,3 +157,98 @@ extern "C" int bench_probe_hbm_read(const void* buf, size_t bytes, int pattern, 
     else hipLaunchKernelGGL(read_probe_chunk<true>, dim3(512), dim3(512), 0, st, (const uint32_t*)buf, bytes / 4, out);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
+
+// ---- what a grid-wide hand-over costs ---------------------------------------------------------------------------------
+// A chain of dependent GEMVs in ONE launch would have persistent workgroups produce a stage's output vector, make it
+// visible to the whole chip and consume it in the next stage.  This probe measures that hand-over by itself: every
+// workgroup writes its slice of an n-entry vector (agent-scope stores that go through to memory), then either
+//   mode 0  arrives at a barrier -- a counter per XCD in the XCD's own L2, the last arriver of an XCD adds to one
+//           agent-scope counter, everybody polls that one -- and reads the whole vector with plain 16-byte loads from
+//           addresses nobody has read before (a fresh buffer every round), or
+//   mode 1  has no barrier: every 32-bit entry carries the round number in its upper half and the consumers poll the
+//           data itself with agent-scope 8-byte loads until every entry is of this round, or
+//   mode 2  the barrier of mode 0 alone (nothing written or read).
+// Every wait is bounded by `spin_limit` polls: a workgroup that gives up writes the round to *status and all of its
+// threads leave; the others then give up in turn.  `check` counts entries that arrived with a wrong value.
+namespace {
+template <int MODE>
+__global__ __launch_bounds__(512) void handover_probe_kernel(int rounds, uint32_t* ctr, uint32_t* xcd_ctr, uint32_t* data,
+                                                            int n_data, int* status, int spin_limit, uint32_t* check) {
+    const int nwg = gridDim.x, wg = blockIdx.x, tid = threadIdx.x;
+    uint32_t bad = 0;
+    __shared__ int ok_s;
+    const int per = (n_data + nwg - 1) / nwg;
+    for (int r = 1; r <= rounds; r++) {
+        uint32_t* buf = data + (size_t)r * n_data;  // a fresh buffer every round
+        if (MODE != 2) {
+            for (int i = tid; i < per; i += 512) {
+                const int idx = wg * per + i;
+                if (idx < n_data) {
+                    const uint32_t val = (MODE == 1) ? (((uint32_t)r << 16) | (uint32_t)((idx * 7 + r) & 0xffff)) : (uint32_t)(r * 1000003 + idx);
+                    __hip_atomic_store(&buf[idx], val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+        }
+        if (MODE == 0 || MODE == 2) {
+            __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0): this wave's stores have been acknowledged
+            __syncthreads();
+            if (tid == 0) {
+                const int xcd = wg & 7, per_xcd = nwg >> 3;
+                const uint32_t old = __hip_atomic_fetch_add(&xcd_ctr[xcd * 32], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                if (old == (uint32_t)(r * per_xcd - 1)) __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                int spins = 0;
+                while (__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (uint32_t)(r * 8) && ++spins < spin_limit) {}
+                ok_s = spins < spin_limit;
+            }
+            __syncthreads();
+            if (!ok_s) {
+                if (tid == 0) atomicExch(status, r);
+                return;
+            }
+            if (MODE == 0) {
+                const uint4* b4 = (const uint4*)buf;
+                for (int i = tid; i < n_data / 4; i += 512) {
+                    const uint4 v = b4[i];
+                    bad += v.x != (uint32_t)(r * 1000003 + 4 * i) || v.w != (uint32_t)(r * 1000003 + 4 * i + 3);
+                }
+            }
+        } else {
+            int spins = 0;
+            const unsigned long long* b8 = (const unsigned long long*)buf;
+            for (int i = tid; i < n_data / 2; i += 512) {
+                unsigned long long v;
+                do {
+                    v = __hip_atomic_load(&b8[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                } while (((uint32_t)(v >> 48) != (uint32_t)r || (((uint32_t)v) >> 16) != (uint32_t)r) && ++spins < spin_limit);
+                bad += ((uint32_t)v & 0xffff) != (uint32_t)((2 * i * 7 + r) & 0xffff);
+            }
+            if (spins >= spin_limit) atomicExch(status, r);
+            if (__syncthreads_or(spins >= spin_limit)) return;
+        }
+    }
+    if (bad) atomicAdd(check, bad);
+}
+}  // namespace
+
+// One launch of `rounds` hand-overs by `workgroups` (a multiple of 8, at most two per compute unit: all of them must be
+// resident) persistent workgroups of 512 threads.  ctr: 1 dword, xcd_ctr: 256 dwords, status / check: 1 dword each, all
+// zeroed by the caller before every launch; data: (rounds + 1) * n_data dwords, zeroed likewise (n_data a multiple of
+// 4).  Returns 0 / -1.
+extern "C" int bench_probe_grid_handover(int mode, int workgroups, int rounds, int n_data, void* ctr, void* xcd_ctr, void* data,
+                                         void* status, void* check, int spin_limit, void* stream) {
+    if (mode < 0 || mode > 2 || workgroups <= 0 || workgroups % 8 != 0 || workgroups > 512 || rounds <= 0 || n_data <= 0 ||
+        n_data % 4 != 0 || spin_limit <= 0 || !ctr || !xcd_ctr || !data || !status || !check)
+        return -1;
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 grid((unsigned)workgroups), block(512);
+    if (mode == 0)
+        hipLaunchKernelGGL(handover_probe_kernel<0>, grid, block, 0, st, rounds, (uint32_t*)ctr, (uint32_t*)xcd_ctr, (uint32_t*)data,
+                           n_data, (int*)status, spin_limit, (uint32_t*)check);
+    else if (mode == 1)
+        hipLaunchKernelGGL(handover_probe_kernel<1>, grid, block, 0, st, rounds, (uint32_t*)ctr, (uint32_t*)xcd_ctr, (uint32_t*)data,
+                           n_data, (int*)status, spin_limit, (uint32_t*)check);
+    else
+        hipLaunchKernelGGL(handover_probe_kernel<2>, grid, block, 0, st, rounds, (uint32_t*)ctr, (uint32_t*)xcd_ctr, (uint32_t*)data,
+                           n_data, (int*)status, spin_limit, (uint32_t*)check);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
