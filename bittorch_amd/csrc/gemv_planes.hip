@@ -212,11 +212,48 @@ __device__ __forceinline__ float planes_to_f32(const int32_t (&s)[PL_N], int exp
 }
 
 template <int XDT = BT_F16>
-__device__ __forceinline__ void pl_store(void* Y, const void* residual, int64_t n, float acc, float s, float b, bool bad) {
+__device__ __forceinline__ void pl_store(void* Y, const void* residual, int64_t n, float acc, float s, float b) {
     float y = epi_float(acc, s, b);
-    if (bad) y = __builtin_nanf("");
     if (residual) y = add_residual(y, residual, XDT, n);
     ((uint16_t*)Y)[n] = (XDT == BT_BF16) ? f32_to_bf16_bits(y) : f32_to_f16_bits(y);
+}
+
+// A row that holds an infinity or a NaN has no fixed-point image; its outputs are what the reference's fp32 loop
+// leaves (ternary_gemm_production.cu:126-133: acc += x * w with w decoded to 0.0f or +-1.0f): the sum of x[k] * w[k, n]
+// over the non-finite x[k] alone, since no finite term changes it -- NaN where a NaN, an infinity on a zero weight or
+// infinities of both signs meet, otherwise the infinity with its sign.  The slow way, one thread per column scanning
+// the row: such rows are not what a kernel is tuned for.  xk(k) returns the row's element k as 16-bit pattern (after
+// the activation prologue, if the kernel has one).
+__device__ __forceinline__ int packed_code(const uint8_t* W, bool tiled, int S, int tiles16_signed, int64_t N, int64_t n, int k) {
+    size_t byte;
+    if (tiled) {
+        const int t = stored_tile16((int)(n >> 4), tiles16_signed);
+        byte = (((size_t)t * S + (k >> 6)) * 64 + 16 * ((k >> 4) & 3) + (size_t)(n & 15)) * 4 + ((k >> 2) & 3);
+    } else {
+        byte = (size_t)(k >> 2) * (size_t)N + (size_t)n;
+    }
+    return (W[byte] >> (2 * (k & 3))) & 3;
+}
+template <int XDT, typename XK>
+__device__ __forceinline__ float nonfinite_acc(XK xk, int K, const uint8_t* W, bool tiled, int S, int tiles16_signed, int64_t N,
+                                            int64_t n) {
+    float acc = 0.0f;
+    for (int k = 0; k < K; k++) {
+        const uint32_t h = xk(k);
+        const bool nonfinite = (XDT == BT_BF16) ? ((h >> 7) & 255u) == 255u : ((h >> 10) & 31u) == 31u;
+        if (!nonfinite) continue;
+        const float xv = (XDT == BT_BF16) ? bf16_bits_to_f32((uint16_t)h) : f16_bits_to_f32((uint16_t)h);
+        const int c = packed_code(W, tiled, S, tiles16_signed, N, n, k);
+        acc = __fadd_rn(acc, __fmul_rn(xv, c == 1 ? 1.0f : c == 2 ? -1.0f : 0.0f));
+    }
+    return acc;
+}
+
+// The same as a call: the grouped kernels keep this path out of their loops' register allocation that way (inlined it
+// cost the contiguous walk 4 % -- 87.9 -> 91.8 us at 128 units -- although it never runs there).
+template <int XDT>
+__device__ __noinline__ float nonfinite_acc_row(const uint16_t* xrow, int K, const uint8_t* W, int S, int tiles16, int64_t N, int64_t n) {
+    return nonfinite_acc<XDT>([&](int k) -> uint32_t { return xrow[k]; }, K, W, true, S, tiles16, N, n);
 }
 
 // ---- one weight matrix per launch -------------------------------------------------------------------
@@ -324,6 +361,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(PlaneParams p) 
         }
     }
 
+    float pro_r = 0.0f;  // RMSNorm prologue: the row's reciprocal root mean square
     if constexpr (PRO != PRO_NONE) {
         __shared__ double ss_slot[WAVES];
         uint4 br[XC];  // the second operand at the same positions
@@ -361,6 +399,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(PlaneParams p) 
 #pragma unroll
             for (int w = 0; w < WAVES; w++) ss += ss_slot[w];
             r = rms_rstd(ss, (int)p.K, p.pro_eps);
+            pro_r = r;
         }
 #pragma unroll
         for (int u = 0; u < XC; u++) {
@@ -452,15 +491,30 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(PlaneParams p) 
     for (int w = 0; w < WAVES; w++) any_bad |= flags[w];
     const float sc = bits_to_f32_rt(pre_s, p.scale_dtype);
     const float bs = biasp ? bits_to_f32_rt(pre_b, p.bias_dtype) : 0.0f;
+    float acc1 = fixed_to_f32(S), acc2 = PAIRS ? fixed_to_f32(S2) : 0.0f;
+    if (any_bad) {  // (uniform over the workgroup) the row as the kernel multiplied it: after the prologue, if any
+        const uint16_t* xrow = (const uint16_t*)Xp;
+        const uint16_t* brow = (const uint16_t*)p.pro_b;
+        const float r = pro_r;
+        auto xk = [&](int k) -> uint32_t {
+            const float xv = f16_bits_to_f32(xrow[k]);
+            if constexpr (PRO == PRO_RMSNORM) return f32_to_f16_bits(rmsnorm_value(xv, r, brow ? f16_bits_to_f32(brow[k]) : 1.0f, BT_F16));
+            else if constexpr (PRO == PRO_SWIGLU) return f32_to_f16_bits(swiglu_value(xv, f16_bits_to_f32(brow[k]), BT_F16));
+            else return xrow[k];
+        };
+        const bool tiled = LAYOUT == PL_TILED;
+        const int tsig = PAIRS ? -p.tiles16 : p.tiles16_signed;  // (the output stage reads a pair-ordered copy)
+        acc1 = nonfinite_acc<BT_F16>(xk, (int)p.K, Wp, tiled, p.wsteps, tsig, p.N, n_out);
+        if constexpr (PAIRS) acc2 = nonfinite_acc<BT_F16>(xk, (int)p.K, Wp, tiled, p.wsteps, tsig, p.N, ffn + n_out);
+    }
     if constexpr (PAIRS) {
         const float sc2 = bits_to_f32_rt(pre_s2, p.scale_dtype);
         const float bs2 = biasp ? bits_to_f32_rt(pre_b2, p.bias_dtype) : 0.0f;
-        float gv = round_to_dtype(epi_float(fixed_to_f32(S), sc, bs), BT_F16);
-        const float uv = round_to_dtype(epi_float(fixed_to_f32(S2), sc2, bs2), BT_F16);
-        if (any_bad) gv = __builtin_nanf("");
+        const float gv = round_to_dtype(epi_float(acc1, sc, bs), BT_F16);
+        const float uv = round_to_dtype(epi_float(acc2, sc2, bs2), BT_F16);
         ((uint16_t*)Yp)[n_out] = f32_to_f16_bits(swiglu_value(gv, uv, BT_F16));
     } else {
-        pl_store(Yp, p.residual, n_out, fixed_to_f32(S), sc, bs, any_bad != 0u);
+        pl_store(Yp, p.residual, n_out, acc1, sc, bs);
     }
 }
 
@@ -602,7 +656,12 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_group_kernel(PlaneParams p
             if (g == 0 && n < p.N) {
                 const float sc = bits_to_f32_rt(pre_s[t], p.scale_dtype);
                 const float bs = bias_u ? bits_to_f32_rt(pre_b[t], p.bias_dtype) : 0.0f;
-                pl_store<XDT>(y_u, nullptr, n, planes_to_f32(s, (XDT == BT_BF16) ? emax - 166 : -24), sc, bs, any_bad);
+                float av = planes_to_f32(s, (XDT == BT_BF16) ? emax - 166 : -24);
+                if (any_bad) {
+                    const uint16_t* xrow = (const uint16_t*)p.X_tab[u];
+                    av = nonfinite_acc_row<XDT>(xrow, (int)p.K, p.W_tab[u], p.wsteps, p.tiles16, p.N, n);
+                }
+                pl_store<XDT>(y_u, nullptr, n, av, sc, bs);
             }
         }
         __syncthreads();  // every wave is done with the planes before the next item overwrites them
@@ -775,7 +834,12 @@ __global__ __launch_bounds__(512, 4) void gemv_planes_chunk_kernel(PlaneParams p
                     const float sc = bits_to_f32_rt(pre_s, p.scale_dtype);
                     const float bs = bias_u ? bits_to_f32_rt(pre_b, p.bias_dtype) : 0.0f;
                     const int exp2 = (XDT == BT_BF16) ? emax - 166 : -24;
-                    pl_store<XDT>(tab ? p.Y_tab[u] : p.Y, tab ? nullptr : p.residual, n, planes_to_f32(sums, exp2), sc, bs, fl != 0u);
+                    float av = planes_to_f32(sums, exp2);
+                    if (fl != 0u) {
+                        const uint16_t* xrow = (const uint16_t*)(tab ? p.X_tab[u] : p.X);
+                        av = nonfinite_acc_row<XDT>(xrow, (int)p.K, tab ? p.W_tab[u] : p.W, p.wsteps, p.tiles16, p.N, n);
+                    }
+                    pl_store<XDT>(tab ? p.Y_tab[u] : p.Y, tab ? nullptr : p.residual, n, av, sc, bs);
                 }
             }
             cur ^= 1;

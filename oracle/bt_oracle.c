@@ -307,10 +307,24 @@ void bto_linear_packed_f64(const float* X, const uint8_t* W_T, const float* scal
  * sum S = sum_k X[k] * w[k,n] is an exact 64-bit integer, and acc = RN_fp32(S) * 2^-24 is the correctly
  * rounded dot product.  Epilogue as above (:139-141): one fp32 multiply, one fp32 add.
  * X must hold fp16 values widened to float (checked: anything else returns -1); a row with an
- * infinity or a NaN gives NaN in every column.  Returns 0.
+ * infinity or a NaN gets, column by column, what the reference's loop leaves (nonfinite_acc below).  Returns 0.
  * Pinned by the float64 dot product, which is exact for these operands while |S| < 2^53, rounded once
  * to fp32 (tests/test_oracle.py).
  */
+/* A row that holds an infinity or a NaN has no fixed-point image: its accumulator is what the reference's fp32 loop
+ * leaves (ternary_gemm_production.cu:126-133, acc += x * w with w decoded to 0.0f or +-1.0f), i.e. the sum of
+ * x[k] * w[k, n] over the non-finite x[k] alone, since no finite term changes it: NaN where a NaN, an infinity on a
+ * zero weight or infinities of both signs meet, otherwise the infinity with its sign. */
+static float nonfinite_acc(const float* xrow, const uint8_t* W_T, int64_t N, int64_t K, int64_t n) {
+    float acc = 0.0f;
+    for (int64_t k = 0; k < K; k++) {
+        const float x = xrow[k];
+        if (fabsf(x) <= 3.4028234663852886e38f) continue;
+        acc = acc + x * (float)decode2((W_T[(k / 4) * N + n] >> (2 * (k % 4))) & 3u);
+    }
+    return acc;
+}
+
 int bto_linear_packed_exact_f16(const float* X, const uint8_t* W_T, const float* scale,
                                 int64_t scale_len, const float* bias, float* Y, int64_t B,
                                 int64_t N, int64_t K) {
@@ -334,10 +348,11 @@ int bto_linear_packed_exact_f16(const float* X, const uint8_t* W_T, const float*
                 int64_t S = 0;
                 for (int64_t k = 0; k < K; k++)
                     S += XI[b * K + k] * (int64_t)decode2((W_T[(k / 4) * N + n] >> (2 * (k % 4))) & 3u);
-                const float acc = (float)S * 5.9604644775390625e-08f; /* RN(S) * 2^-24, the scaling exact */
+                float acc = (float)S * 5.9604644775390625e-08f; /* RN(S) * 2^-24, the scaling exact */
+                if (bad[b]) acc = nonfinite_acc(X + b * K, W_T, N, K, n);
                 float r = acc * s;
                 r = r + bv;
-                Y[b * N + n] = bad[b] ? NAN : r;
+                Y[b * N + n] = r;
             }
         }
     }
@@ -354,7 +369,8 @@ int bto_linear_packed_exact_f16(const float* X, const uint8_t* W_T, const float*
  * emax = the largest e1 of the row; X[k] = mag * 2^(e1 - emax + 32), an integer below 2^40 in magnitude, where an
  * element more than 32 binades below the largest is rounded to an integer half-up in magnitude (more than 40 binades
  * below: 0).  S = sum_k X[k] * w[k, n] exactly; acc = RN_fp32(S) * 2^(emax - 166); then the reference's epilogue.
- * X holds bf16 values widened to float; returns -1 if one is not a bf16 value.  Rows with an infinity or a NaN: NaN.
+ * X holds bf16 values widened to float; returns -1 if one is not a bf16 value.  Rows with an infinity or a NaN:
+ * nonfinite_acc above.
  */
 int bto_linear_packed_rowscaled_bf16(const float* X, const uint8_t* W_T, const float* scale,
                                      int64_t scale_len, const float* bias, float* Y, int64_t B,
@@ -400,10 +416,11 @@ int bto_linear_packed_rowscaled_bf16(const float* X, const uint8_t* W_T, const f
                 int64_t S = 0;
                 for (int64_t k = 0; k < K; k++)
                     S += XI[b * K + k] * (int64_t)decode2((W_T[(k / 4) * N + n] >> (2 * (k % 4))) & 3u);
-                const float acc = ldexpf((float)S, emax[b] - 166);
+                float acc = ldexpf((float)S, emax[b] - 166);
+                if (bad[b]) acc = nonfinite_acc(X + b * K, W_T, N, K, n);
                 float r = acc * s;
                 r = r + bv;
-                Y[b * N + n] = bad[b] ? NAN : r;
+                Y[b * N + n] = r;
             }
         }
     }

@@ -105,10 +105,18 @@ def test_single_row_fp16_variants(oracle):
         xv[0, :len(vals)] = torch.tensor(vals, dtype=torch.float64).half()
         e = _expect(oracle, xv, ones, torch.ones(16), None, 16)
         assert torch.equal(_C.ternary_linear_packed_forward(xv.cuda(), ones.cuda(), torch.ones(16).cuda(), None, 16).cpu(), e)
-    # an infinity or a NaN in the row: NaN everywhere (as in the reference whenever it meets a zero weight)
-    xv = x.clone()
-    xv[0, 5] = float("inf")
-    assert torch.isnan(_C.ternary_linear_tiled_forward(xv.cuda(), tiled, scale.cuda(), bias.cuda(), k, n)).all()
+    # an infinity or a NaN in the row: column by column what the reference's float loop leaves (the oracle restates it)
+    for pos, val in (((5,), float("inf")), ((5, k - 1), float("-inf")), ((0,), float("nan"))):
+        xv = x.clone()
+        for q_ in pos:
+            xv[0, q_] = val
+        e = _expect(oracle, xv, packed, scale, bias, k)
+        assert torch.isnan(e).any() and (torch.isinf(e).any() or val != val)
+        got_t = _C.ternary_linear_tiled_forward(xv.cuda(), tiled, scale.cuda(), bias.cuda(), k, n).cpu()
+        got_r = _C.ternary_linear_packed_forward(xv.cuda(), packed.cuda(), scale.cuda(), bias.cuda(), k).cpu()
+        for got in (got_t, got_r):
+            assert torch.equal(torch.isnan(got), torch.isnan(e))
+            assert torch.equal(torch.nan_to_num(got, nan=0.0), torch.nan_to_num(e, nan=0.0))
 
 
 def _tables(_C, xs, tiles, scales, biases, ys):
@@ -191,7 +199,8 @@ def test_grouped_launch_config2_units_and_shared_operands(oracle):
 
 def test_grouped_launch_non_finite_row_and_large_group(oracle, monkeypatch):
     """160 units of 2048 x 2048 (the contiguous-walk kernel by the library's own rule): one unit's row holds an
-    infinity and gives NaN in every column, its neighbours are untouched."""
+    infinity and gets what the reference's float loop leaves (NaN on zero weights, the signed infinity elsewhere), its
+    neighbours are untouched."""
     from bittorch_amd import _C
     announce("grouped gemv non-finite")
     n = k = 2048
@@ -206,7 +215,12 @@ def test_grouped_launch_non_finite_row_and_large_group(oracle, monkeypatch):
     ys = [torch.empty(1, n, dtype=torch.float16, device="cuda") for _ in range(g)]
     _C.ternary_gemv_grouped(*_tables(_C, xs, tiles, scales, biases, ys), k, n, scale_len=n)
     torch.cuda.synchronize()
-    assert torch.isnan(ys[77]).all()
+    xe = base[77 % 3][0].clone()
+    xe[0, 1999] = float("inf")
+    e77 = _expect(oracle, xe, base[77 % 3][1], base[77 % 3][2], base[77 % 3][3], k)
+    assert torch.isnan(e77).any() and torch.isinf(e77).any()   # zero weights and +-1 weights at that position
+    assert torch.equal(torch.isnan(ys[77].cpu()), torch.isnan(e77))
+    assert torch.equal(torch.nan_to_num(ys[77].cpu(), nan=0.0), torch.nan_to_num(e77, nan=0.0))
     for u in (0, 76, 78, 159):
         b = base[u % 3]
         assert torch.equal(ys[u].cpu(), _expect(oracle, b[0], b[1], b[2], b[3], k))
@@ -334,7 +348,7 @@ def test_grouped_bf16_units_against_the_oracle(oracle, g, n, k, per_tensor, bias
 
 def test_bf16_row_times_a_wide_matrix_and_argument_errors(oracle):
     """One bf16 row through the single-matrix entry point takes the same kernel where the matrix is wide enough
-    (forced here on a small one); a non-finite row gives NaN; bad arguments of the grouped entry point are refused."""
+    (forced here on a small one); a non-finite row gets the float loop's answer; bad arguments of the grouped entry point are refused."""
     import os
     from bittorch_amd import _C, _lib
     announce("bf16 wide row")
@@ -352,6 +366,11 @@ def test_bf16_row_times_a_wide_matrix_and_argument_errors(oracle):
         xb = x.clone()
         xb[0, 77] = float("nan")
         assert torch.isnan(_C.ternary_linear_tiled_forward(xb.cuda(), tiled, scale.cuda(), bias.cuda(), k, n)).all()
+        xb[0, 77] = float("inf")
+        e = _expect_bf16(oracle, xb, packed, scale, bias, k)
+        got = _C.ternary_linear_tiled_forward(xb.cuda(), tiled, scale.cuda(), bias.cuda(), k, n).cpu()
+        assert torch.isinf(e).any() and torch.equal(torch.isnan(got), torch.isnan(e))
+        assert torch.equal(torch.nan_to_num(got, nan=0.0), torch.nan_to_num(e, nan=0.0))
     finally:
         set_option("GROUP_WALK", None)
     # the 16-bit matrix-core kernel (what a narrow matrix takes) agrees within bf16 rounding
@@ -416,3 +435,46 @@ def test_ops_ternary_linear_grouped_equals_the_single_calls(oracle):
     other = TernaryLinearInference(k, n + 16, torch.zeros(k // 4, n + 16, dtype=torch.uint8), torch.ones(n + 16)).cuda()
     with pytest.raises(ValueError, match="same in_features and out_features"):
         bt.ops.ternary_linear_grouped(layers + [other], xs[0])
+
+
+def _same_with_nans(a, b):
+    return torch.equal(torch.isnan(a), torch.isnan(b)) and torch.equal(torch.nan_to_num(a, nan=0.0), torch.nan_to_num(b, nan=0.0))
+
+
+def test_non_finite_rows_through_prologues_and_the_swiglu_stage(oracle):
+    """Rows that are (or become, inside an activation prologue) non-finite: the fused calls still equal the unfused
+    sequences -- row kernel, then the exact GEMV, then the SwiGLU kernel -- NaN for NaN and infinity for infinity."""
+    from bittorch_amd import _C
+    n, k = 256, 512
+    x, packed, scale, bias = _setup(n, k, seed=21)
+    pd, sd, bd = packed.cuda(), scale.cuda(), bias.cuda()
+    nat, pairs = _C.retile_weights(pd, k), _C.retile_weights(pd, k, True)
+    g = torch.Generator().manual_seed(5)
+    nw = (torch.rand(k, generator=g) + 0.5).half().cuda()
+    up = seeded_acts(1, k, seed=6, dtype=torch.float16).cuda()
+    cases = []
+    xi = x.clone(); xi[0, 7] = float("inf"); cases.append(("inf", xi, nw))
+    xn = x.clone(); xn[0, 300] = float("nan"); cases.append(("nan", xn, nw))
+    xo = x.clone(); xo[0, 11] = 60000.0; cases.append(("overflows in the norm", xo, (nw * 6000).half()))  # finite in, Inf after the norm
+    for name, xc, w in cases:
+        announce("non-finite through prologues", name)
+        xc = xc.cuda()
+        normed = _C.rmsnorm(xc, w, 1e-5)
+        assert not torch.isfinite(normed.float()).all()
+        for tiled_, kw in ((nat, {}), (pairs, dict(natural_from_pairs=True))):
+            want = _C.ternary_linear_tiled_forward(normed, tiled_, sd, bd, k, n, **kw)
+            got = _C.ternary_linear_tiled_forward(xc, tiled_, sd, bd, k, n, norm=(w, 1e-5), **kw)
+            assert _same_with_nans(got, want), name
+        assert _same_with_nans(_C.ternary_linear_packed_forward_fused(xc, pd, sd, bd, k, norm=(w, 1e-5)),
+                               _C.ternary_linear_packed_forward(normed, pd, sd, bd, k)), name
+        # SwiGLU prologue: silu(x) * up
+        h = _C.swiglu(xc, up)
+        assert _same_with_nans(_C.ternary_linear_tiled_forward(xc, nat, sd, bd, k, n, swiglu_up=up),
+                               _C.ternary_linear_tiled_forward(h, nat, sd, bd, k, n)), name
+        # SwiGLU output stage on the pair-ordered copy (with and without the norm prologue)
+        for norm in (None, (w, 1e-5)):
+            xin = xc if norm is None else normed
+            gu = _C.ternary_linear_tiled_forward(xin, nat, sd, bd, k, n)
+            want = _C.swiglu(gu[:, :n // 2], gu[:, n // 2:])
+            got = _C.ternary_linear_tiled_forward(xc, pairs, sd, bd, k, n, None, norm, None, True)
+            assert _same_with_nans(got, want), (name, norm is not None)

@@ -244,12 +244,55 @@ def test_linear_exact_f16_is_the_correctly_rounded_dot_product(oracle):
             continue
         np.testing.assert_array_equal(oracle.linear_packed_exact_f16(x, packed_t, np.array(case["scales"], np.float32), k),
                                       np.array(case["output"], dtype=np.float32))
-    # a row with an infinity or a NaN is NaN everywhere, other rows are untouched; non-fp16 inputs are refused
+    # a row with an infinity: +inf where it meets +1 weights (the float loop's answer, pinned in its own test below),
+    # other rows are untouched; non-fp16 inputs are refused
     x = np.array([[1.0, np.inf, 0, 0], [1.0, 2.0, 3.0, 4.0]], np.float32)
     y = oracle.linear_packed_exact_f16(x, p4, one, 4)
-    assert np.isnan(y[0, 0]) and y[1, 0] == 10.0
+    assert y[0, 0] == np.inf and y[1, 0] == 10.0
     with pytest.raises(ValueError):
         oracle.linear_packed_exact_f16(np.array([[1.0 + 2.0 ** -20, 0, 0, 0]], np.float32), p4, one, 4)
+
+
+def _float_loop(x, w, n):
+    """the reference's accumulation (ternary_gemm_production.cu:126-133) for one column, in plain fp32 arithmetic"""
+    acc = np.float32(0.0)
+    with np.errstate(invalid="ignore", over="ignore"):
+        for k in range(x.shape[0]):
+            acc = np.float32(acc + np.float32(x[k] * np.float32(w[n, k])))
+    return acc
+
+
+@pytest.mark.parametrize("fn", ["linear_packed_exact_f16", "linear_packed_rowscaled_bf16"])
+def test_exact_linears_on_non_finite_rows_follow_the_float_loop(oracle, fn):
+    """A row that holds an infinity or a NaN: every column gets what the reference's fp32 loop leaves -- NaN where a
+    NaN, an infinity on a zero weight, or infinities of both signs meet; otherwise the infinity with the sign of its
+    products -- and the other rows of the call are untouched.  Pinned by running that loop in numpy."""
+    f = getattr(oracle, fn)
+    w = np.array([[1, 1, 0, -1, 1, 0, 1, -1],     # column 0: inf meets +1 (k=1): +inf
+                  [1, -1, 0, 1, 1, 0, 1, 1],      # column 1: inf meets -1: -inf
+                  [1, 0, 1, 1, -1, 0, 1, 1],      # column 2: inf meets 0: NaN
+                  [0, 1, 1, -1, -1, 1, 0, 1]], dtype=np.int8)  # column 3: +inf * 1, and (row 2) +inf * -1 as well
+    packed_t, k = oracle.pack_ternary_transposed(w)
+    one = np.ones(4, np.float32)
+    rows = np.array([[1.0, np.inf, 2.0, 0.5, -3.0, 4.0, 1.0, 1.0],       # one +inf at k = 1
+                     [1.0, 2.0, 3.0, 4.0, 5.0, 6.0, 7.0, 8.0],           # finite: untouched
+                     [1.0, np.inf, 2.0, 0.5, np.inf, 0.0, 1.0, 1.0],     # +inf at k = 1 and at k = 4
+                     [np.nan, 1.0, 2.0, 3.0, 1.0, 1.0, 1.0, 1.0],        # a NaN: NaN wherever it goes
+                     [1.0, -np.inf, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0]], np.float32)
+    y = f(rows, packed_t, one, k)
+    for b in range(rows.shape[0]):
+        for n in range(4):
+            want = _float_loop(rows[b], w, n)
+            if np.isnan(want):
+                assert np.isnan(y[b, n]), (b, n, y[b, n])
+            else:
+                assert y[b, n] == want, (b, n, y[b, n], want)
+    assert y[0, 0] == np.inf and y[0, 1] == -np.inf and np.isnan(y[0, 2]) and y[0, 3] == np.inf
+    assert y[2, 0] == np.inf and np.isnan(y[2, 1]) and np.isnan(y[2, 3])  # same sign twice; opposite signs meet
+    assert np.isnan(y[3]).all() and y[4, 1] == np.inf
+    # the epilogue applies as ever: scale and bias (a negative scale flips the infinity)
+    y2 = f(rows[:1], packed_t, np.array([-2.0, 1.0, 1.0, 1.0], np.float32), k, np.full(4, 5.0, np.float32))
+    assert y2[0, 0] == -np.inf and y2[0, 1] == -np.inf and np.isnan(y2[0, 2])
 
 
 def _bf16(a):
@@ -316,10 +359,11 @@ def test_linear_rowscaled_bf16_is_the_correctly_rounded_dot_product(oracle):
             continue
         np.testing.assert_array_equal(oracle.linear_packed_rowscaled_bf16(x, packed_t, np.array(case["scales"], np.float32), k),
                                       np.array(case["output"], dtype=np.float32))
-    # non-finite rows: NaN everywhere, other rows untouched; inputs that are not bf16 values are refused
+    # non-finite rows: the float loop's answer (own test below), other rows untouched; inputs that are not bf16 values
+    # are refused
     x = np.array([[1.0, np.inf, 0, 0], [1.0, 2.0, 3.0, 4.0]], np.float32)
     y = oracle.linear_packed_rowscaled_bf16(x, p4, one, 4)
-    assert np.isnan(y[0, 0]) and y[1, 0] == 10.0
+    assert y[0, 0] == np.inf and y[1, 0] == 10.0
     with pytest.raises(ValueError):
         oracle.linear_packed_rowscaled_bf16(np.array([[1.0 + 2.0 ** -10, 0, 0, 0]], np.float32), p4, one, 4)
 
