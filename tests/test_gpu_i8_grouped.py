@@ -132,3 +132,39 @@ def test_grouped_int8_argument_errors():
         _C.ternary_gemm_int8_grouped(t, t, t, t, None, t, 16, 16384, 64)
     with pytest.raises(RuntimeError, match="scale size"):
         _C.ternary_gemm_int8_grouped(t, t, t, t, None, t, 16, 64, 64, scale_len=3)
+
+
+def test_ops_ternary_linear_int8_grouped_equals_forward_int8(oracle):
+    """The caller in the kept API: float activations [G, M, K] (quantized in one launch) or pre-quantized q / s_x
+    through `ops.ternary_linear_int8_grouped`, unit by unit the bits of `layer.forward_int8` on the same rows; more
+    than 16 rows per unit falls back to single calls with the same result."""
+    import bittorch_amd as bt
+    from bittorch_amd import _C
+    from bittorch_amd.nn import TernaryLinearInference
+    n, k, g = 320, 1024, 5
+    layers = []
+    for u in range(g):
+        w = random_ternary(n, k, seed=60 + u)
+        packed, _ = oracle.pack_ternary_transposed(w.numpy())
+        gen = torch.Generator().manual_seed(u)
+        layers.append(TernaryLinearInference(k, n, torch.from_numpy(packed), torch.rand(n, generator=gen) * 0.05 + 0.01,
+                                             torch.randn(n, generator=gen) * 0.01).cuda())
+    for m in (16, 3, 20):
+        announce("ops.ternary_linear_int8_grouped", m)
+        xs = seeded_acts(g * m, k, seed=m, dtype=torch.bfloat16, outliers=True).view(g, m, k).cuda()
+        got = bt.ops.ternary_linear_int8_grouped(layers, xs)
+        assert got.shape == (g, m, n) and got.dtype == torch.bfloat16
+        for u, L in enumerate(layers):
+            q, s = bt.ops.act_quant_int8(xs[u], True)
+            assert torch.equal(got[u], L.forward_int8(q, s, torch.bfloat16, None, True))
+        # pre-quantized, row-major bytes, fp32 outputs, into a caller's buffer, twice (cached tables)
+        q_all, s_all = bt.ops.act_quant_int8(xs, False)
+        out = torch.empty(g, m, n, device="cuda")
+        for _ in range(2):
+            assert bt.ops.ternary_linear_int8_grouped(layers, q=q_all, s_x=s_all, out_dtype=torch.float32, out=out) is out
+        for u, L in enumerate(layers):
+            assert torch.equal(out[u], L.forward_int8(q_all[u], s_all[u], torch.float32))
+    with pytest.raises(ValueError, match="give xs, or q together with s_x"):
+        bt.ops.ternary_linear_int8_grouped(layers)
+    with pytest.raises(RuntimeError, match="doesn't match in_features"):
+        bt.ops.ternary_linear_int8_grouped(layers, torch.zeros(g, 4, k - 16, device="cuda"))
