@@ -278,6 +278,19 @@ def pmc_pass(torch, _C, dev, gemv_steps, grouped_step):
     master = torch.randn(n, k, device=dev) * 0.02
     for _ in range(5):
         _C.ternary_quantize_pack(master, 0.05, True)
+    # config 3 as 32 units of 16 int8 rows per launch (bt_ternary_gemm_i8_grouped), 16 x 4096 -> 11008
+    g8, n3, k3 = 32, 11008, 4096
+    tl = []
+    for _ in range(g8):
+        c = torch.randint(0, 3, (4, k3 // 4, n3), device=dev, dtype=torch.uint8)
+        tl.append(_C.retile_weights((c[0] | (c[1] << 2) | (c[2] << 4) | (c[3] << 6)).contiguous(), k3))
+    sc3 = torch.rand(n3, device=dev) * 0.05 + 0.01
+    qs = [_C.act_quant_int8(torch.randn(16, k3, device=dev).bfloat16(), True) for _ in range(g8)]
+    ys = [torch.empty(16, n3, dtype=torch.bfloat16, device=dev) for _ in range(g8)]
+    tabs = (_C.pointer_table([q_ for q_, _ in qs]), _C.pointer_table([s_ for _, s_ in qs]), _C.pointer_table(tl),
+            _C.pointer_table([sc3] * g8), None, _C.pointer_table(ys))
+    for _ in range(5):
+        _C.ternary_gemm_int8_grouped(*tabs, 16, k3, n3, out_dtype=torch.bfloat16, q_operand_order=True)
     torch.cuda.synchronize()
     print(json.dumps({"pmc_pass": "done", "copy_bytes_read": n_copy * 4, "copy_bytes_written": n_copy * 4,
                       "copy_kernel": "at::native vectorized elementwise (mul by scalar)"}))
