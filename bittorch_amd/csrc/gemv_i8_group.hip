@@ -54,40 +54,6 @@ __device__ __forceinline__ void i8g_store(void* Y, int dt, int64_t idx, float v)
     else ((uint16_t*)Y)[idx] = f32_to_bf16_bits(v);
 }
 
-// Raw bits of NV (8 or 4) consecutive entries n0 .. n0 + NV - 1 of a scale / bias vector (entries past N repeat the
-// last one; bcast: one entry for all).  Whole aligned pieces come as 16- or 8-byte loads.
-template <int NV>
-__device__ __forceinline__ void load_bits_n(const void* v, int dt, int bcast, int64_t n0, int64_t N, uint32_t (&out)[NV]) {
-    if (bcast) {
-        const uint32_t b = load_bits_rt(v, dt, 0);
-#pragma unroll
-        for (int c = 0; c < NV; c++) out[c] = b;
-        return;
-    }
-    const bool whole = n0 + NV <= N && (n0 % NV) == 0 && (((uintptr_t)v) & 15) == 0;
-    if (whole && dt == BT_F32) {
-#pragma unroll
-        for (int c = 0; c < NV; c += 4) {
-            const uint4 a = *(const uint4*)((const uint32_t*)v + n0 + c);
-            out[c] = a.x; out[c + 1] = a.y; out[c + 2] = a.z; out[c + 3] = a.w;
-        }
-    } else if (whole) {
-        uint32_t d[NV / 2];
-        if constexpr (NV == 8) {
-            const uint4 a = *(const uint4*)((const uint16_t*)v + n0);
-            d[0] = a.x; d[1] = a.y; d[2] = a.z; d[3] = a.w;
-        } else {
-            const uint2 a = *(const uint2*)((const uint16_t*)v + n0);
-            d[0] = a.x; d[1] = a.y;
-        }
-#pragma unroll
-        for (int c = 0; c < NV; c++) out[c] = (d[c >> 1] >> (16 * (c & 1))) & 0xffffu;
-    } else {
-#pragma unroll
-        for (int c = 0; c < NV; c++) out[c] = load_bits_rt(v, dt, (n0 + c < N) ? n0 + c : N - 1);
-    }
-}
-
 template <int SPW, int TB, int WAVES>
 __global__ __launch_bounds__(WAVES * 64, 4) void gemv_i8_walk_kernel(I8GroupParams p) {
     constexpr int I8_EB = i8_eb<WAVES>();
@@ -98,6 +64,10 @@ __global__ __launch_bounds__(WAVES * 64, 4) void gemv_i8_walk_kernel(I8GroupPara
     static_assert(I8_EB % TB == 0, "chunks hold whole batches");
     constexpr int THREADS = WAVES * 64;
     __shared__ __attribute__((aligned(16))) int32_t accbuf[2][16][I8_ROW];    // [array][row][16 * tile + column]
+    // the epilogue's operands of a chunk, staged while the chunk is computed: column scales and biases as raw bits, the
+    // unit's row scales
+    __shared__ __attribute__((aligned(16))) uint32_t ops_s[2][I8_EB * 16], ops_b[2][I8_EB * 16];
+    __shared__ float ops_sx[2][16];
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -188,6 +158,20 @@ __global__ __launch_bounds__(WAVES * 64, 4) void gemv_i8_walk_kernel(I8GroupPara
         const int64_t u_stop = (unit_end < t_end) ? unit_end : t_end;
         for (int64_t c0 = t0; c0 < u_stop; c0 += I8_EB) {
             const int ntiles = (int)((u_stop - c0 < I8_EB) ? u_stop - c0 : I8_EB);  // a multiple of TB
+            // The epilogue's operands are requested now, one column per thread, and parked in LDS at the end of the chunk:
+            // the epilogue itself then waits for nothing but LDS.  (Requested by the epilogue's own threads after the
+            // barrier they left every wave waiting on memory once per chunk; held in registers per output piece across
+            // the chunk's matrix instructions they spilled.)
+            uint32_t st_s = 0u, st_b = 0u;
+            float st_sx = 0.0f;
+            {
+                const int64_t n = (int64_t)(tile0 + (int)(c0 - t0)) * 16 + tid;
+                if (tid < ntiles * 16 && n < p.N) {
+                    st_s = load_bits_rt(scale_u, p.scale_dtype, p.scale_bcast ? 0 : n);
+                    if (bias_u) st_b = load_bits_rt(bias_u, p.bias_dtype, n);
+                }
+                if (tid < 16) st_sx = sx_u[min(tid, M - 1)];
+            }
             for (int tb = 0; tb < ntiles; tb += TB) {
                 v4i acc[TB];
 #pragma unroll
@@ -208,25 +192,23 @@ __global__ __launch_bounds__(WAVES * 64, 4) void gemv_i8_walk_kernel(I8GroupPara
                     for (int r = 0; r < 4; r++) atomicAdd(&accbuf[cur][4 * g + r][16 * (tb + i) + j], acc[i][r]);
                 }
             }
+            if (tid < I8_EB * 16) {
+                ops_s[cur][tid] = st_s;
+                ops_b[cur][tid] = st_b;
+            }
+            if (tid < 16) ops_sx[cur][tid] = st_sx;
             __syncthreads();  // every wave has added its share of this chunk
-            // The chunk's epilogue: 16 rows x 256 columns in pieces of four columns (an 8-byte piece of a 16-bit output
-            // row; consecutive threads cover a row's columns with full-line stores), in passes over the threads.
-            // The operands are requested here rather than a chunk ahead: held across the chunk's matrix instructions
-            // they cost more registers than the wave has, and the loads that wait here are covered by the other
-            // workgroup of the compute unit and by the weight loads already in flight.
+            // The chunk's epilogue: 16 rows x (16 * tiles) columns in pieces of four columns (an 8-byte piece of a 16-bit
+            // output row; consecutive threads cover a row's columns with full-line stores), in passes over the threads.
 #pragma unroll 1
             for (int item = tid; item < I8_EB * 64; item += THREADS) {
                 const int e_row = item / (4 * I8_EB), e_tl = (item % (4 * I8_EB)) >> 2, e_j0 = 4 * (item & 3);
                 if (e_tl >= ntiles) continue;
                 const int64_t n0 = (int64_t)(tile0 + (int)(c0 - t0) + e_tl) * 16 + e_j0;
                 const bool e_on = n0 < p.N && e_row < M;
-                uint32_t pre_s[4], pre_b[4];
-                float pre_sx = 0.0f;
-                if (e_on) {
-                    pre_sx = sx_u[e_row];
-                    load_bits_n<4>(scale_u, p.scale_dtype, p.scale_bcast, n0, p.N, pre_s);
-                    if (bias_u) load_bits_n<4>(bias_u, p.bias_dtype, 0, n0, p.N, pre_b);
-                }
+                const uint4 s4 = *(const uint4*)&ops_s[cur][16 * e_tl + e_j0], b4 = *(const uint4*)&ops_b[cur][16 * e_tl + e_j0];
+                const uint32_t pre_s[4] = {s4.x, s4.y, s4.z, s4.w}, pre_b[4] = {b4.x, b4.y, b4.z, b4.w};
+                const float pre_sx = ops_sx[cur][e_row];
                 int32_t* src = &accbuf[cur][e_row][16 * e_tl + e_j0];
                 const int4 v = *(const int4*)src;
                 *(int4*)src = make_int4(0, 0, 0, 0);
