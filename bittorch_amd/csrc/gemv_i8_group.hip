@@ -48,11 +48,20 @@ struct I8GroupParams {
     int y_dtype, scale_dtype, bias_dtype, scale_bcast;
 };
 
-__device__ __forceinline__ void i8g_store(void* Y, int dt, int64_t idx, float v) {
-    if (dt == BT_F32) ((float*)Y)[idx] = v;
-    else if (dt == BT_F16) ((uint16_t*)Y)[idx] = f32_to_f16_bits(v);
-    else ((uint16_t*)Y)[idx] = f32_to_bf16_bits(v);
+// A pointer read from one of the tables, pinned to scalar registers (the compiler cannot always prove a table index
+// uniform, and a pointer fetched with a vector load costs a wait for all of the wave's outstanding memory operations
+// wherever it is first used).  Rebuilt as a pointer into global memory: a bare integer cast would leave the compiler
+// with generic-address loads and stores, which wait on two counters and complete out of order.
+template <typename T>
+__device__ __forceinline__ T* uniform_ptr(T* ptr) {
+    const uint64_t v = (uint64_t)(uintptr_t)ptr;
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+    typedef __attribute__((address_space(1))) T* global_ptr;
+    return (T*)(global_ptr)(uintptr_t)(((uint64_t)hi << 32) | lo);
 }
+
+template <int YDT> struct I8YTag { static constexpr int value = YDT; };
 
 template <int SPW, int TB, int WAVES>
 __global__ __launch_bounds__(WAVES * 64, 4) void gemv_i8_walk_kernel(I8GroupParams p) {
@@ -64,9 +73,9 @@ __global__ __launch_bounds__(WAVES * 64, 4) void gemv_i8_walk_kernel(I8GroupPara
     static_assert(I8_EB % TB == 0, "chunks hold whole batches");
     constexpr int THREADS = WAVES * 64;
     __shared__ __attribute__((aligned(16))) int32_t accbuf[2][16][I8_ROW];    // [array][row][16 * tile + column]
-    // the epilogue's operands of a chunk, staged while the chunk is computed: column scales and biases as raw bits, the
-    // unit's row scales
-    __shared__ __attribute__((aligned(16))) uint32_t ops_s[2][I8_EB * 16], ops_b[2][I8_EB * 16];
+    // the epilogue's operands of a chunk, staged while the chunk is computed: column scales and biases widened to
+    // fp32 (zeros where there is no bias), the unit's row scales
+    __shared__ __attribute__((aligned(16))) float ops_s[2][I8_EB * 16], ops_b[2][I8_EB * 16];
     __shared__ float ops_sx[2][16];
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
@@ -95,7 +104,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void gemv_i8_walk_kernel(I8GroupPara
     int pf_u = (int)(t_begin / T16);
     int pf_t = (int)(t_begin - (int64_t)pf_u * T16);
     int64_t pf_left = t_end - t_begin;
-    const uint8_t* pf_ptr = p.W_tab[pf_u] + (size_t)pf_t * tile_bytes;
+    const uint8_t* pf_ptr = uniform_ptr(p.W_tab[pf_u]) + (size_t)pf_t * tile_bytes;
     uint32_t raw[TB][SPW];
     auto request = [&](uint32_t (&dst)[SPW]) {
         // (past the end of the run: the last tile again, never used)
@@ -108,7 +117,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void gemv_i8_walk_kernel(I8GroupPara
             if (pf_t == T16) {
                 pf_t = 0;
                 pf_u++;
-                pf_ptr = p.W_tab[pf_u];
+                pf_ptr = uniform_ptr(p.W_tab[pf_u]);
             }
         }
     };
@@ -138,7 +147,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void gemv_i8_walk_kernel(I8GroupPara
         }
     };
     // the first unit's activations are requested ahead of the weights (loads return in order; they are needed first)
-    load_a(p.Q_tab[pf_u]);
+    load_a(uniform_ptr(p.Q_tab[pf_u]));
 #pragma unroll
     for (int i = 0; i < TB; i++) request(raw[i]);
 
@@ -147,17 +156,23 @@ __global__ __launch_bounds__(WAVES * 64, 4) void gemv_i8_walk_kernel(I8GroupPara
 
     int64_t t0 = t_begin;
     while (t0 < t_end) {
-        const int u = (int)(t0 / T16);
-        const int tile0 = (int)(t0 - (int64_t)u * T16);
-        if (t0 != t_begin) load_a(p.Q_tab[u]);  // (uniform)
+        const int u = __builtin_amdgcn_readfirstlane((int)(t0 / T16));
+        const int tile0 = __builtin_amdgcn_readfirstlane((int)(t0 - (int64_t)u * T16));
+        if (t0 != t_begin) load_a(uniform_ptr(p.Q_tab[u]));  // (uniform)
         finish_a();
-        const float* sx_u = p.sx_tab[u];
-        const void* scale_u = p.scale_tab[u];
-        const void* bias_u = p.bias_tab ? p.bias_tab[u] : nullptr;
+        // the unit's pointers, once per unit and in scalar registers
+        const float* sx_u = uniform_ptr(p.sx_tab[u]);
+        const void* scale_u = uniform_ptr(p.scale_tab[u]);
+        const void* bias_u = p.bias_tab ? uniform_ptr(p.bias_tab[u]) : nullptr;
+        void* const y_u = uniform_ptr(p.Y_tab[u]);
+        int32_t* const acc_u = p.acc_tab ? uniform_ptr(p.acc_tab[u]) : nullptr;
+        // whole four-column pieces leave as vector stores: rows of N % 8 == 0 columns from 16-byte aligned bases
+        const bool vec_u = (p.N & 7) == 0 && (((uintptr_t)y_u) & 15) == 0 && (((uintptr_t)acc_u) & 15) == 0;
         const int64_t unit_end = (int64_t)(u + 1) * T16;
         const int64_t u_stop = (unit_end < t_end) ? unit_end : t_end;
         for (int64_t c0 = t0; c0 < u_stop; c0 += I8_EB) {
             const int ntiles = (int)((u_stop - c0 < I8_EB) ? u_stop - c0 : I8_EB);  // a multiple of TB
+            const int ctile = tile0 + (int)(c0 - t0);
             // The epilogue's operands are requested now, one column per thread, and parked in LDS at the end of the chunk:
             // the epilogue itself then waits for nothing but LDS.  (Requested by the epilogue's own threads after the
             // barrier they left every wave waiting on memory once per chunk; held in registers per output piece across
@@ -165,7 +180,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void gemv_i8_walk_kernel(I8GroupPara
             uint32_t st_s = 0u, st_b = 0u;
             float st_sx = 0.0f;
             {
-                const int64_t n = (int64_t)(tile0 + (int)(c0 - t0)) * 16 + tid;
+                const int64_t n = (int64_t)ctile * 16 + tid;
                 if (tid < ntiles * 16 && n < p.N) {
                     st_s = load_bits_rt(scale_u, p.scale_dtype, p.scale_bcast ? 0 : n);
                     if (bias_u) st_b = load_bits_rt(bias_u, p.bias_dtype, n);
@@ -193,67 +208,59 @@ __global__ __launch_bounds__(WAVES * 64, 4) void gemv_i8_walk_kernel(I8GroupPara
                 }
             }
             if (tid < I8_EB * 16) {
-                ops_s[cur][tid] = st_s;
-                ops_b[cur][tid] = st_b;
+                ops_s[cur][tid] = bits_to_f32_rt(st_s, p.scale_dtype);
+                ops_b[cur][tid] = bias_u ? bits_to_f32_rt(st_b, p.bias_dtype) : 0.0f;
             }
             if (tid < 16) ops_sx[cur][tid] = st_sx;
             __syncthreads();  // every wave has added its share of this chunk
             // The chunk's epilogue: 16 rows x (16 * tiles) columns in pieces of four columns (an 8-byte piece of a 16-bit
             // output row; consecutive threads cover a row's columns with full-line stores), in passes over the threads.
+            // The operands arrive widened to fp32 and the output's type is decided once per chunk, so the loop is the
+            // arithmetic and one store (about 60 instructions per piece).
+            auto pieces = [&](auto ytag) {
+                constexpr int YDT = decltype(ytag)::value;
 #pragma unroll 1
-            for (int item = tid; item < I8_EB * 64; item += THREADS) {
-                const int e_row = item / (4 * I8_EB), e_tl = (item % (4 * I8_EB)) >> 2, e_j0 = 4 * (item & 3);
-                if (e_tl >= ntiles) continue;
-                const int64_t n0 = (int64_t)(tile0 + (int)(c0 - t0) + e_tl) * 16 + e_j0;
-                const bool e_on = n0 < p.N && e_row < M;
-                const uint4 s4 = *(const uint4*)&ops_s[cur][16 * e_tl + e_j0], b4 = *(const uint4*)&ops_b[cur][16 * e_tl + e_j0];
-                const uint32_t pre_s[4] = {s4.x, s4.y, s4.z, s4.w}, pre_b[4] = {b4.x, b4.y, b4.z, b4.w};
-                const float pre_sx = ops_sx[cur][e_row];
-                int32_t* src = &accbuf[cur][e_row][16 * e_tl + e_j0];
-                const int4 v = *(const int4*)src;
-                *(int4*)src = make_int4(0, 0, 0, 0);
-                if (!e_on) continue;
-                const int32_t a[4] = {v.x, v.y, v.z, v.w};
-                int32_t a127[4];
-                float y[4];
-#pragma unroll
-                for (int c = 0; c < 4; c++) {
-                    a127[c] = times127(a[c]);  // the matrix cores ran on +-1 weights
-                    const float sc = bits_to_f32_rt(pre_s[c], p.scale_dtype);
-                    const float bs = bias_u ? bits_to_f32_rt(pre_b[c], p.bias_dtype) : 0.0f;
-                    y[c] = epi_int8(a127[c], pre_sx, sc, bs);
-                }
-                const int64_t idx = (int64_t)e_row * p.N + n0;
-                void* y_u = p.Y_tab[u];
-                int32_t* acc_u = p.acc_tab ? p.acc_tab[u] : nullptr;
-                // whole pieces leave as vector stores (rows of N % 8 == 0 columns from a 16-byte aligned base)
-                const bool vec = n0 + 4 <= p.N && (p.N & 7) == 0 && (((uintptr_t)y_u) & 15) == 0 &&
-                                 (!acc_u || (((uintptr_t)acc_u) & 15) == 0);
-                if (vec) {
-                    if (p.y_dtype == BT_F32) {
-                        st4_nt((float*)y_u + idx, __builtin_bit_cast(uint32_t, y[0]), __builtin_bit_cast(uint32_t, y[1]),
-                               __builtin_bit_cast(uint32_t, y[2]), __builtin_bit_cast(uint32_t, y[3]));
+                for (int item = tid; item < I8_EB * 64; item += THREADS) {
+                    const int e_row = item / (4 * I8_EB);
+                    const int col0 = (item - e_row * (4 * I8_EB)) * 4;  // first column of the piece inside the chunk
+                    if (col0 >= ntiles * 16) continue;
+                    int32_t* src = &accbuf[cur][e_row][col0];
+                    const int4 v = *(const int4*)src;
+                    *(int4*)src = make_int4(0, 0, 0, 0);
+                    const int64_t n0 = (int64_t)ctile * 16 + col0;
+                    if (n0 >= p.N || e_row >= M) continue;
+                    const float4 s4 = *(const float4*)&ops_s[cur][col0], b4 = *(const float4*)&ops_b[cur][col0];
+                    const float pre_sx = ops_sx[cur][e_row];
+                    const int32_t a127[4] = {times127(v.x), times127(v.y), times127(v.z), times127(v.w)};  // +-1 weights
+                    const float y[4] = {epi_int8(a127[0], pre_sx, s4.x, b4.x), epi_int8(a127[1], pre_sx, s4.y, b4.y),
+                                        epi_int8(a127[2], pre_sx, s4.z, b4.z), epi_int8(a127[3], pre_sx, s4.w, b4.w)};
+                    const int64_t idx = (int64_t)e_row * p.N + n0;
+                    if (vec_u) {
+                        if constexpr (YDT == BT_F32) {
+                            st4_nt((float*)y_u + idx, __builtin_bit_cast(uint32_t, y[0]), __builtin_bit_cast(uint32_t, y[1]),
+                                   __builtin_bit_cast(uint32_t, y[2]), __builtin_bit_cast(uint32_t, y[3]));
+                        } else if constexpr (YDT == BT_F16) {
+                            st2_nt((uint16_t*)y_u + idx, f32_to_f16_bits(y[0]) | ((uint32_t)f32_to_f16_bits(y[1]) << 16),
+                                   f32_to_f16_bits(y[2]) | ((uint32_t)f32_to_f16_bits(y[3]) << 16));
+                        } else {
+                            st2_nt((uint16_t*)y_u + idx, f32_to_bf16_bits(y[0]) | ((uint32_t)f32_to_bf16_bits(y[1]) << 16),
+                                   f32_to_bf16_bits(y[2]) | ((uint32_t)f32_to_bf16_bits(y[3]) << 16));
+                        }
+                        if (acc_u) st4_nt(acc_u + idx, (uint32_t)a127[0], (uint32_t)a127[1], (uint32_t)a127[2], (uint32_t)a127[3]);
                     } else {
-                        uint32_t h[2];
 #pragma unroll
-                        for (int c = 0; c < 2; c++) {
-                            const uint32_t l = (p.y_dtype == BT_F16) ? f32_to_f16_bits(y[2 * c]) : f32_to_bf16_bits(y[2 * c]);
-                            const uint32_t m = (p.y_dtype == BT_F16) ? f32_to_f16_bits(y[2 * c + 1]) : f32_to_bf16_bits(y[2 * c + 1]);
-                            h[c] = l | (m << 16);
-                        }
-                        st2_nt((uint16_t*)y_u + idx, h[0], h[1]);
-                    }
-                    if (acc_u) st4_nt(acc_u + idx, (uint32_t)a127[0], (uint32_t)a127[1], (uint32_t)a127[2], (uint32_t)a127[3]);
-                } else {
-#pragma unroll
-                    for (int c = 0; c < 4; c++) {
-                        if (n0 + c < p.N) {
-                            i8g_store(y_u, p.y_dtype, idx + c, y[c]);
-                            if (acc_u) acc_u[idx + c] = a127[c];
+                        for (int c = 0; c < 4; c++) {
+                            if (n0 + c < p.N) {
+                                store_elem<YDT>(y_u, idx + c, y[c]);
+                                if (acc_u) acc_u[idx + c] = a127[c];
+                            }
                         }
                     }
                 }
-            }
+            };
+            if (p.y_dtype == BT_F32) pieces(I8YTag<BT_F32>{});
+            else if (p.y_dtype == BT_F16) pieces(I8YTag<BT_F16>{});
+            else pieces(I8YTag<BT_BF16>{});
             cur ^= 1;
         }
         t0 = u_stop;

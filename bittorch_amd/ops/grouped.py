@@ -172,6 +172,8 @@ def ternary_linear_grouped(layers: Sequence, xs: Union[Tensor, Sequence[Tensor]]
 
 
 _MAX_K_I8 = 11264  # the grouped int8 kernel holds a wave's K slice of the 16 rows in registers
+_MIN_G_I8 = 3  # below this the one-matrix kernel, one call per unit, is the faster route (persistent workgroups
+               # that walk a single matrix leave most of the chip's request queues empty)
 
 
 def ternary_linear_int8_grouped(layers: Sequence, xs: Optional[Tensor] = None, q: Optional[Tensor] = None,
@@ -216,7 +218,7 @@ def ternary_linear_int8_grouped(layers: Sequence, xs: Optional[Tensor] = None, q
             raise RuntimeError("q must be int8 [G, M, K] and s_x fp32 [G, M]")
         q, s_x = q.contiguous(), s_x.contiguous()
     kinds = (torch.float32, torch.float16, torch.bfloat16)
-    groupable = (m <= 16 and k % 16 == 0 and k <= _MAX_K_I8 and _groupable(layers, torch.empty(0, dtype=torch.float16, device=q.device))
+    groupable = (g >= _MIN_G_I8 and m <= 16 and k % 16 == 0 and k <= _MAX_K_I8 and _groupable(layers, torch.empty(0, dtype=torch.float16, device=q.device))
                  and all(L.scale.dtype in kinds for L in layers))
     if out is not None and (out.shape != (g, m, n) or out.dtype != out_dtype or not out.is_contiguous()):
         raise ValueError("ternary_linear_int8_grouped: out must be a contiguous [G, M, N] tensor of out_dtype")

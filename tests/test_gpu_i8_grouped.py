@@ -137,7 +137,7 @@ def test_grouped_int8_argument_errors():
 def test_ops_ternary_linear_int8_grouped_equals_forward_int8(oracle):
     """The caller in the kept API: float activations [G, M, K] (quantized in one launch) or pre-quantized q / s_x
     through `ops.ternary_linear_int8_grouped`, unit by unit the bits of `layer.forward_int8` on the same rows; more
-    than 16 rows per unit falls back to single calls with the same result."""
+    than 16 rows per unit, or fewer than three units, fall back to single calls with the same result."""
     import bittorch_amd as bt
     from bittorch_amd import _C
     from bittorch_amd.nn import TernaryLinearInference
@@ -164,6 +164,11 @@ def test_ops_ternary_linear_int8_grouped_equals_forward_int8(oracle):
             assert bt.ops.ternary_linear_int8_grouped(layers, q=q_all, s_x=s_all, out_dtype=torch.float32, out=out) is out
         for u, L in enumerate(layers):
             assert torch.equal(out[u], L.forward_int8(q_all[u], s_all[u], torch.float32))
+    # two units are below the grouped kernel's break-even and go through single calls: the same bits
+    got2 = bt.ops.ternary_linear_int8_grouped(layers[:2], xs[:2])
+    for u in range(2):
+        q, s = bt.ops.act_quant_int8(xs[u], True)
+        assert torch.equal(got2[u], layers[u].forward_int8(q, s, torch.bfloat16, None, True))
     with pytest.raises(ValueError, match="give xs, or q together with s_x"):
         bt.ops.ternary_linear_int8_grouped(layers)
     with pytest.raises(RuntimeError, match="doesn't match in_features"):
