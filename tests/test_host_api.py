@@ -67,8 +67,6 @@ def test_dequantize_and_quantizer_object():
     t, sc = qz.quantize(w)
     assert torch.equal(qz.dequantize(t, sc), t * sc.unsqueeze(1))
     assert qz.bits_per_weight == 1.58 and qz.quant_type is bt.quant.QuantType.TERNARY
-    with pytest.raises(NotImplementedError):
-        bt.quant.int4_quantize(w)
 
 
 def test_compute_scale_variants():
