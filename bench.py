@@ -765,7 +765,7 @@ def main():
         extra["batched_decode_N4096_K4096"] = bd
         del ws, ts
         # quantize + pack of fp32 master weights
-        for (n, k) in ((4096, 4096), (11008, 4096)):
+        for (n, k) in ((4096, 4096), (11008, 4096), (4096, 11008)):
             cnt = max(2, int(600e6 // (n * k * 4)))
             masters = [torch.randn(n, k, device=dev) * 0.02 for _ in range(cnt)]
             steps = 40

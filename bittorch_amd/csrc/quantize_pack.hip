@@ -44,21 +44,28 @@ __device__ __forceinline__ uint32_t encode4(const float (&v)[4], float thr, uint
 }
 
 // ---- fast kernel ---------------------------------------------------------------------
-// ITERS float4 groups per lane (>= K/256), WAVES waves, RPW rows per wave one after another.
+// ITERS float4 groups per lane, WAVES waves, RPW rows per wave one after another; SPLIT waves share a row (wave w
+// holds 256-element chunks ITERS * (w % SPLIT) .. + ITERS - 1 of row slot w / SPLIT, ITERS * SPLIT >= K / 256): a long
+// row in one wave's registers leaves room for four waves per compute unit, whose encode then runs one wave per SIMD
+// with nothing to overlap it (4096 x 11008 fp32: 45.4 us, of which 9.4 us encode; split over four waves: see below).
 // LDS tile: byte (kb, row) at kb*PITCHB + row, PITCHB = R + 4: the odd dword pitch keeps the
 // column writes (lanes = consecutive kb) and the row reads free of bank conflicts.
-template <int DT, int ITERS, int WAVES, int RPW>
+template <int DT, int ITERS, int WAVES, int RPW, int SPLIT = 1>
 __global__ __launch_bounds__(WAVES * 64) void quantize_pack_fast_kernel(
     const void* __restrict__ W, int N, int K, float tf, float clamp_min, int per_channel,
     uint8_t* __restrict__ packed_T, float* __restrict__ scale, int tiles, int per_xcd) {
-    constexpr int R = WAVES * RPW;
+    constexpr int SLOTS = WAVES / SPLIT;  // rows in flight
+    constexpr int R = SLOTS * RPW;
     constexpr int PITCHB = R + 4;
+    static_assert(WAVES % SPLIT == 0, "whole row slots");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_b[];
+    __shared__ float part_max[RPW][WAVES];
     const int tile = (int)xcd_tile(blockIdx.x, per_xcd);
     if (tile >= tiles) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int slot = wave / SPLIT, part = wave % SPLIT;
     const int n0 = tile * R;
-    const int nfull = K >> 8;  // complete 256-element chunks (uniform)
+    const int nfull = (K >> 8) - part * ITERS;  // complete 256-element chunks of this wave's share (uniform)
     const int Kb = K >> 2;
     const float tensor_scale = per_channel ? 0.0f : fmaxf(scale[0], clamp_min);
     // The tensor scale arrives unfloored; one thread stores the floored value.  Workgroups that read it afterwards
@@ -67,12 +74,30 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_pack_fast_kernel(
     uint32_t pk[ITERS];
 #pragma unroll
     for (int j = 0; j < ITERS; j++) pk[j] = 0;
+    // the row's scale from its absolute maximum (this lane's share of it), stored once, and the threshold that goes with it
+    auto row_threshold = [&](int r, int n, float amax) __attribute__((always_inline)) -> float {
+        float s;
+        if (per_channel) {
+            amax = wave_max(amax);
+            if constexpr (SPLIT > 1) {  // the row's other waves (per_channel is uniform: every wave meets the barrier)
+                if (lane == 0) part_max[r][wave] = amax;
+                __syncthreads();
+#pragma unroll
+                for (int q = 0; q < SPLIT; q++) amax = fmaxf(amax, part_max[r][slot * SPLIT + q]);
+            }
+            s = fmaxf(amax, clamp_min);
+            if (lane == 0 && part == 0) scale[n] = s;
+        } else {
+            s = tensor_scale;
+        }
+        return round_to_dtype(__fmul_rn(tf, s), DT);
+    };
 #pragma unroll 1  // one row in registers at a time
     for (int r = 0; r < RPW; r++) {
-        const int n = n0 + RPW * wave + r;
+        const int n = n0 + RPW * slot + r;
         float4 v[ITERS];
         if constexpr (DT == BT_F32) {
-            const float4* rowp = (const float4*)((const float*)W + (int64_t)n * K) + lane;
+            const float4* rowp = (const float4*)((const float*)W + (int64_t)n * K) + part * ITERS * 64 + lane;
 #pragma unroll
             for (int j = 0; j < ITERS; j++) {
                 if (j < nfull) {
@@ -84,7 +109,7 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_pack_fast_kernel(
                 }
             }
         } else {
-            const uint2* rowp = (const uint2*)((const uint16_t*)W + (int64_t)n * K) + lane;
+            const uint2* rowp = (const uint2*)((const uint16_t*)W + (int64_t)n * K) + part * ITERS * 64 + lane;
 #pragma unroll
             for (int j = 0; j < ITERS; j++) {
                 const uint2 t = (j < nfull) ? ldw2_nt(rowp + j * 64) : make_uint2(0u, 0u);
@@ -100,14 +125,7 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_pack_fast_kernel(
 #pragma unroll
         for (int j = 0; j < ITERS; j++)
             amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[j].x), fabsf(v[j].y)), fmaxf(fabsf(v[j].z), fabsf(v[j].w))));
-        float s;
-        if (per_channel) {
-            s = fmaxf(wave_max(amax), clamp_min);
-            if (lane == 0) scale[n] = s;
-        } else {
-            s = tensor_scale;
-        }
-        const float thr = round_to_dtype(__fmul_rn(tf, s), DT);
+        const float thr = row_threshold(r, n, amax);
 #pragma unroll
         for (int j = 0; j < ITERS; j++) {
             const float a[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
@@ -118,7 +136,7 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_pack_fast_kernel(
 #pragma unroll
     for (int j = 0; j < ITERS; j++) {
         if (j < nfull) {
-            uint8_t* dst = lds_b + (j * 64 + lane) * PITCHB + wave * RPW;
+            uint8_t* dst = lds_b + ((part * ITERS + j) * 64 + lane) * PITCHB + slot * RPW;
             if constexpr (RPW == 4) *(uint32_t*)dst = pk[j];
             else if constexpr (RPW == 2) *(uint16_t*)dst = (uint16_t)pk[j];
             else *dst = (uint8_t)pk[j];
@@ -133,14 +151,14 @@ __global__ __launch_bounds__(WAVES * 64) void quantize_pack_fast_kernel(
     }
 }
 
-template <int DT, int ITERS, int WAVES, int RPW>
+template <int DT, int ITERS, int WAVES, int RPW, int SPLIT = 1>
 static int launch_fast_cfg(const void* W, int64_t N, int64_t K, float tf, float clamp_min, int per_channel,
                            uint8_t* packed_T, float* scale, hipStream_t st) {
-    constexpr int R = WAVES * RPW;
+    constexpr int R = (WAVES / SPLIT) * RPW;
     const int tiles = (int)(N / R);
     const int per_xcd = (int)ceil_div(tiles, 8);
     const size_t lds = (size_t)(K / 4) * (R + 4);
-    auto kern = quantize_pack_fast_kernel<DT, ITERS, WAVES, RPW>;
+    auto kern = quantize_pack_fast_kernel<DT, ITERS, WAVES, RPW, SPLIT>;
     if (lds > 64 * 1024 &&
         hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
         set_error("bt_quantize_pack: cannot reserve %zu bytes of LDS", lds);
@@ -181,7 +199,7 @@ static int launch_fast_rows(const void* W, int64_t N, int64_t K, float tf, float
 
 // returns 1 if the fast kernel took the call (rc holds its status), 0 if the shape does not
 // qualify.  Register budget: a row of K elements costs K/64 data registers per lane, so 16 waves
-// per workgroup fit K <= 4096, 8 waves K <= 8192, 4 waves K <= 11008.
+// per workgroup fit K <= 4096 with a row per wave, K <= 8192 with a row over two waves and K <= 16384 over four.
 template <int DT>
 static int try_launch_fast(const void* W, int64_t N, int64_t K, float tf, float clamp_min, int per_channel,
                            uint8_t* packed_T, float* scale, int8_t* w_tern, hipStream_t st, int* rc) {
@@ -199,10 +217,22 @@ static int try_launch_fast(const void* W, int64_t N, int64_t K, float tf, float 
     if (chunks > 8 && chunks <= 16 && N >= 6144 && N % 16 == 0)
         return launch_fast_rows<DT, 16, 8>(W, N, K, tf, clamp_min, per_channel, packed_T, scale, st, rc);
     BT_QF(16, 16);
-    BT_QF(24, 8);
-    BT_QF(32, 8);
-    BT_QF(43, 4);
 #undef BT_QF
+    // Longer rows are split over two or four waves of a 16-wave workgroup (16 rows per tile either way)
+    if (N % 16 != 0 || (size_t)(K / 4) * 20 > 150 * 1024) return 0;
+    const bool two = chunks <= 32 && !tuning_env("BITTORCH_QP_SPLIT4");
+    const int per_wave = (int)ceil_div(chunks, two ? 2 : 4);
+#define BT_QS(IT, SP, RP) \
+    if (per_wave <= IT) { \
+        *rc = launch_fast_cfg<DT, IT, 16, RP, SP>(W, N, K, tf, clamp_min, per_channel, packed_T, scale, st); \
+        return 1; \
+    }
+    if (two) {
+        BT_QS(10, 2, 2) BT_QS(12, 2, 2) BT_QS(14, 2, 2) BT_QS(16, 2, 2)
+    } else {
+        BT_QS(6, 4, 4) BT_QS(8, 4, 4) BT_QS(10, 4, 4) BT_QS(11, 4, 4) BT_QS(12, 4, 4) BT_QS(14, 4, 4) BT_QS(16, 4, 4)
+    }
+#undef BT_QS
     return 0;
 }
 

@@ -43,6 +43,24 @@ def test_quantize_pack_matches_oracle_16bit(oracle, n, k, dtype):
     _run(oracle, seeded_weights(n, k, seed=6, dtype=dtype), 0.05, False)
 
 
+# The one-read kernel (packed output only, K % 256 == 0, N % 16 == 0): a row per wave up to K = 4096, a row over two
+# waves up to 8192 and over four up to 16384 -- every registers-per-lane variant of each, with rows that fill the last
+# wave's share only partly (5120 = 20 chunks over two waves of 10; 11008 = 43 over four of 11; 9216 = 36 over four of 10).
+FAST_SHAPES = [(32, 256), (64, 1024), (32, 2048), (32, 4096), (96, 4096), (32, 4352), (32, 5120), (48, 6144),
+               (32, 6912), (16, 8192), (32, 9216), (32, 11008), (16, 12288), (16, 14336), (16, 16384)]
+
+
+@pytest.mark.parametrize("n,k", FAST_SHAPES)
+def test_quantize_pack_one_read_kernel_matches_oracle(oracle, n, k):
+    announce("quantize_pack one-read kernel", n, k)
+    for dtype, seed in ((torch.float32, 1), (torch.bfloat16, 2), (torch.float16, 3)):
+        w = seeded_weights(n, k, seed=seed * 1000 + n + k, dtype=dtype)
+        w[n // 2, k - 1] = w.abs().max() * 2   # the row's maximum in the last wave's share
+        w[1, 0] = -w.abs().max() * 3           # ... and in the first's
+        _run(oracle, w, 0.05, True, want_tern=False)
+        _run(oracle, w, 0.05, False, want_tern=False)
+
+
 @pytest.mark.parametrize("tf", [0.0, 0.01, 0.1, 0.5, 1.0])
 def test_quantize_pack_threshold_factors(oracle, tf):
     announce("quantize_pack tf", tf)
