@@ -823,7 +823,7 @@ def main():
         def decode_plain(i):
             L = layers_[i % nl]
             h = F.rms_norm(xt, (d_model,), nw, eps)
-            a = L["q"](h) + L["k"](h) + L["v"](h)          # stands in for attention over the cache
+            a, _k, _v = L["q"](h), L["k"](h), L["v"](h)    # q stands in for the attention output (k, v go to the cache)
             x1 = xt + L["o"](a)
             h2 = F.rms_norm(x1, (d_model,), nw, eps)
             return x1 + L["down"](F.silu(L["gate"](h2)) * L["up"](h2))
@@ -831,7 +831,7 @@ def main():
         def decode_fused(i):
             L = layers_[i % nl]
             qkv = L["qkv"](xt, None, (nw, eps))            # RMSNorm inside the GEMV kernel
-            a = qkv[:, :d_model] + qkv[:, d_model:2 * d_model] + qkv[:, 2 * d_model:]
+            a = qkv[:, :d_model]                           # (a view: no launch between the projections)
             x1 = L["o"](a, xt)
             return L["mlp"](x1, nw, eps, residual=x1)
 
