@@ -95,6 +95,103 @@ def test_amp_autocast_forward_backward():
     assert layer.weight.grad.dtype == torch.float32
 
 
+def test_amp_training_loop_with_grad_scaler():
+    """What the reference's AMP tests pin beyond one forward (tests/test_amp.py:209-333): a GradScaler training loop on
+    XOR lowers the loss on either backend, with no NaN or Inf in loss or gradients on the way."""
+    from bittorch_amd.nn import TernaryLinear
+    announce("amp training")
+    xor_x = torch.tensor([[0., 0.], [0., 1.], [1., 0.], [1., 1.]], device="cuda")
+    xor_y = torch.tensor([[0.], [1.], [1.], [0.]], device="cuda")
+    for backend in ("cuda", "python"):
+        torch.manual_seed(42)
+        model = nn.Sequential(TernaryLinear(2, 16, backend=backend), nn.ReLU(), TernaryLinear(16, 1, backend=backend)).cuda()
+        opt = torch.optim.Adam(model.parameters(), lr=0.01)
+        scaler = torch.amp.GradScaler("cuda")
+        losses = []
+        for _ in range(100):
+            opt.zero_grad()
+            with torch.autocast("cuda", dtype=torch.float16):
+                loss = nn.functional.binary_cross_entropy_with_logits(model(xor_x), xor_y)
+            assert torch.isfinite(loss)
+            scaler.scale(loss).backward()
+            scaler.step(opt)
+            scaler.update()
+            losses.append(loss.item())
+        assert losses[-1] < losses[0], (backend, losses[0], losses[-1])
+        for prm in model.parameters():
+            assert prm.grad is not None and prm.grad.shape == prm.shape
+
+
+def test_autocast_contexts_mixed_nested_eval_and_batch_sizes():
+    """tests/test_amp.py:335-405: one sample and a large batch under autocast, regular forwards before and after an
+    autocast one agree, a disabled inner context gives fp32, eval mode under no_grad is finite."""
+    from bittorch_amd.nn import TernaryLinear
+    announce("autocast contexts")
+    torch.manual_seed(3)
+    layer = TernaryLinear(64, 32).cuda()
+    for b in (1, 256):
+        with torch.autocast("cuda", dtype=torch.float16):
+            y = layer(torch.randn(b, 64, device="cuda"))
+        assert y.shape == (b, 32) and torch.isfinite(y).all()
+    x = torch.randn(8, 64, device="cuda")
+    y1 = layer(x)
+    with torch.autocast("cuda", dtype=torch.float16):
+        ya = layer(x)
+        with torch.autocast("cuda", enabled=False):
+            yb = layer(x)
+        yc = layer(x)
+    y3 = layer(x)
+    assert y1.dtype == y3.dtype == yb.dtype == torch.float32
+    assert torch.equal(y1, y3) and torch.equal(yb, y1)
+    assert torch.isfinite(ya).all() and torch.equal(ya, yc)
+    assert torch.allclose(ya.float(), y1, rtol=1e-2, atol=1e-2)
+    layer.eval()
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+        ye = layer(x)
+    assert torch.isfinite(ye).all()
+
+
+def test_gradient_consistency_over_seeds_shapes_and_double_precision():
+    """tests/test_gradient_consistency.py:153-250: the kernels' gradients follow the torch backend's over several seeds
+    and shapes, and the autograd function takes float64 operands (the reference runs gradcheck on it in double
+    precision and accepts either verdict: the straight-through estimator is not the derivative of the forward)."""
+    from bittorch_amd.nn.ternary_linear_cuda import TernaryLinearCUDAFunction
+    announce("gradient consistency")
+    for seed in (0, 1, 7, 42, 123):
+        torch.manual_seed(seed)
+        hip, ref = _pair(32, 16)
+        x1 = torch.randn(4, 32, device="cuda", requires_grad=True)
+        x2 = x1.detach().clone().requires_grad_(True)
+        hip(x1).sum().backward()
+        ref(x2).sum().backward()
+        assert torch.allclose(hip.weight.grad, ref.weight.grad, rtol=1e-4, atol=1e-5)
+        assert torch.allclose(x1.grad, x2.grad, rtol=1e-4, atol=1e-5)
+    for (b, in_f, out_f) in [(1, 8, 4), (3, 100, 50), (64, 16, 128), (2, 7, 3)]:
+        hip, ref = _pair(in_f, out_f)
+        x1 = torch.randn(b, in_f, device="cuda", requires_grad=True)
+        x2 = x1.detach().clone().requires_grad_(True)
+        hip(x1).pow(2).sum().backward()
+        ref(x2).pow(2).sum().backward()
+        assert torch.allclose(hip.weight.grad, ref.weight.grad, rtol=1e-3, atol=1e-4)
+        assert torch.allclose(hip.bias.grad, ref.bias.grad, rtol=1e-3, atol=1e-4)
+        assert torch.allclose(x1.grad, x2.grad, rtol=1e-3, atol=1e-4)
+    torch.manual_seed(42)
+    x = torch.randn(2, 4, device="cuda", dtype=torch.float64, requires_grad=True)
+    w = torch.randn(3, 4, device="cuda", dtype=torch.float64, requires_grad=True)
+    bias = torch.randn(3, device="cuda", dtype=torch.float64, requires_grad=True)
+    y = TernaryLinearCUDAFunction.apply(x, w, bias, 0.05, True)
+    assert y.dtype == torch.float64 and y.shape == (2, 3)
+    from bittorch_amd.quant import ternary_quantize
+    w_t, s = ternary_quantize(w.detach(), 0.05, True)
+    assert torch.allclose(y, x.detach() @ (w_t * s.unsqueeze(1)).t() + bias.detach(), rtol=1e-6, atol=1e-6)
+    y.sum().backward()
+    assert x.grad.dtype == w.grad.dtype == bias.grad.dtype == torch.float64
+    assert torch.equal(bias.grad, torch.full_like(bias, 2.0))
+    verdict = torch.autograd.gradcheck(lambda a, b_, c: TernaryLinearCUDAFunction.apply(a, b_, c, 0.05, True),
+                                       (x, w, bias), eps=1e-4, atol=1e-3, rtol=1e-2, raise_exception=False)
+    assert verdict in (True, False)
+
+
 def test_half_and_bf16_modules():
     from bittorch_amd.nn import TernaryLinear
     announce("16-bit modules")
