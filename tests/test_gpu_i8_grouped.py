@@ -65,6 +65,31 @@ def test_grouped_int8_units_equal_single_calls(oracle, n, k, m, g):
             assert torch.equal(ys[u], y1), (u, "outputs")
 
 
+_rng = np.random.default_rng(20250311)
+
+
+def _random_case(i):
+    k = 16 * int(_rng.integers(1, 705))                       # 16 .. 11264, any multiple of 16
+    if i % 3 == 0:
+        k = 16 * int(_rng.integers(1, 257))                   # ... a third of them inside the 8-wave kernel's range
+    n = int(_rng.choice([16, 20, 33, 48, 100, 250, 260, 512]))
+    return n, k, int(_rng.integers(1, 17)), int(_rng.integers(1, 10)), bool(i % 2), i
+
+
+@pytest.mark.parametrize("n,k,m,g,operand_order,seed", [_random_case(i) for i in range(18)])
+def test_grouped_int8_random_shapes_against_the_oracle(oracle, n, k, m, g, operand_order, seed):
+    """Seeded random unit counts, rows, ragged column counts and any K % 16 == 0 up to the kernel's limit, held to the
+    CPU oracle directly: int32 accumulators and fp32 outputs bit for bit."""
+    announce("grouped int8 random", n, k, m, g, operand_order)
+    units = [_unit(oracle, n, k, m, seed=97 * seed + u, bias=bool(seed % 3), operand_order=operand_order) for u in range(g)]
+    ys, accs = _run_grouped(units, m, n, k, torch.float32, operand_order)
+    for u, un in enumerate(units):
+        _, _, oacc, oy = oracle.linear_i8(f32np(un["x"].cpu()), un["packed"].cpu().numpy(), f32np(un["scale"].cpu()), k,
+                                          None if un["bias"] is None else f32np(un["bias"].cpu()))
+        np.testing.assert_array_equal(accs[u].cpu().numpy(), oacc)
+        np.testing.assert_array_equal(ys[u].cpu().numpy(), oy)
+
+
 def test_grouped_int8_against_oracle_and_shared_operands(oracle):
     """One case straight against the CPU oracle (quantized activations, accumulators, outputs), and units that
     share one weight matrix or one activation block."""
