@@ -539,7 +539,12 @@ def main():
                 return _C.ternary_gemm_int8_tiled(q_, s_, ts[i % 2], sc, None, k, n, torch.bfloat16, False, None, True)
             _, ev_qg = graph_time(quant_then_gemm, steps, 5, torch)
             _, ev_q = graph_time(lambda i: _C.act_quant_int8(xa, operand_order=True), steps, 5, torch)
-            del ts
+            # the opt-in prefill copy in the field layout (TernaryLinearInference.prepare_prefill), row sums from the quantizer
+            fs = [_C.retile_fields(t, k, n) for t in ts]
+            _, _, rs = _C.act_quant_int8(xa, operand_order=True, return_rowsum=True)
+            _, ev_fl = graph_time(lambda i: _C.ternary_gemm_int8_fields(q, s, rs, fs[i % 2], sc, None, k, n, torch.bfloat16,
+                                                                        False, None, True), steps, 5, torch)
+            del ts, fs
             _, ev_full = graph_time(lambda i: _C.ternary_linear_tensor_core_forward(xa, ws[i % 2], sc, None, k, 2),
                                     steps, 5, torch)
             ops = 2.0 * m * n * k
@@ -558,6 +563,7 @@ def main():
                 "act_quant_GBps": round(3.0 * m * k / (ev_q / steps * 1e-3) / 1e9, 1),
                 "with_act_quant_us_tiled_weights": round(ev_qg / steps * 1e3, 2),
                 "frac_of_int8_peak_with_act_quant_tiled_weights": round(ops / (ev_qg / steps * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4),
+                "gemm_us_prefill_copy_field_layout": round(ev_fl / steps * 1e3, 2),
             }
             # float path of the same shape (bf16 activations, fp32 accumulation on the 16-bit
             # matrix cores) and the vendor library on dense operands, for scale
@@ -764,6 +770,20 @@ def main():
             bd[f"M{m}"] = row
         extra["batched_decode_N4096_K4096"] = bd
         del ws, ts
+        # prefill chunks shorter than config 4's (chunked prefill): the tiled copy against the opt-in field-layout copy
+        sp = {}
+        n_ = k_ = 4096
+        wt_ = rand_packed(n_, k_, 1)[0]
+        tl_ = _C.retile_weights(wt_, k_)
+        fl_ = _C.retile_fields(tl_, k_, n_)
+        sc_ = torch.rand(n_, device=dev) * 0.05 + 0.01
+        for m in (512, 1024):
+            q_, s_, rs_ = _C.act_quant_int8(acts(m, k_, True), operand_order=True, return_rowsum=True)
+            _, ev_t = graph_time(lambda i: _C.ternary_gemm_int8_tiled(q_, s_, tl_, sc_, None, k_, n_, torch.bfloat16, False, None, True), 40, 5, torch)
+            _, ev_f = graph_time(lambda i: _C.ternary_gemm_int8_fields(q_, s_, rs_, fl_, sc_, None, k_, n_, torch.bfloat16, False, None, True), 40, 5, torch)
+            sp[f"M{m}"] = {"gemm_us_tiled_copy": round(ev_t / 40 * 1e3, 2), "gemm_us_prefill_copy_field_layout": round(ev_f / 40 * 1e3, 2)}
+        extra["short_prefill_int8_N4096_K4096"] = sp
+        del wt_, tl_, fl_
         # quantize + pack of fp32 master weights
         for (n, k) in ((4096, 4096), (11008, 4096), (4096, 11008)):
             cnt = max(2, int(600e6 // (n * k * 4)))

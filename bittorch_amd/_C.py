@@ -396,6 +396,53 @@ def ternary_gemm_int8_grouped(q_tab: Tensor, sx_tab: Tensor, w_tiled_tab: Tensor
             y_tab.data_ptr(), _DT[out_dtype], _ptr(acc_tab), G, rows, out_features, in_features, _stream(q_tab)))
 
 
+def retile_fields(W_tiled: Tensor, in_features: int, out_features: int) -> Tensor:
+    """The prefill-only field layout of a decode-tiled copy (same size; natural or pair-ordered tiles are kept in
+    their order): what :func:`ternary_gemm_int8_fields` reads."""
+    _tiled_checks(W_tiled, out_features, in_features)
+    _check(W_tiled.is_cuda, "All tensors must be CUDA")
+    with torch.cuda.device(W_tiled.device):
+        out = torch.empty_like(W_tiled)
+        _status(_L.bt_retile_fields(W_tiled.data_ptr(), out_features, in_features, out.data_ptr(), _stream(W_tiled)))
+    return out
+
+
+def ternary_gemm_int8_fields(Q: Tensor, s_x: Tensor, q_rowsum: Tensor, W_fields: Tensor, scale: Tensor,
+                             bias: Optional[Tensor] = None, in_features: int = -1, out_features: int = -1,
+                             out_dtype: torch.dtype = torch.float32, return_acc: bool = False,
+                             residual: Optional[Tensor] = None, q_operand_order: bool = False,
+                             natural_from_pairs: bool = False):
+    """:func:`ternary_gemm_int8_tiled` on the field layout (:func:`retile_fields`) with the rows' sums of ``Q``
+    (``act_quant_int8(..., return_rowsum=True)``): the same results bit for bit through a cheaper weight decode.
+    Always the tiled matrix-core GEMM (prefill batches); ``in_features`` a multiple of 128."""
+    _check(Q.dim() == 2 and Q.dtype == torch.int8 and Q.numel() > 0, "Q must be 2D int8")
+    K, N = Q.shape[-1], out_features
+    _check(K == in_features, "input K doesn't match in_features")
+    _tiled_checks(W_fields, N, K)
+    _check(scale.dim() == 1 and scale.shape[0] in (N, 1), "scale size doesn't match N")
+    _check(bias is None or (bias.dim() == 1 and bias.shape[0] == N), "bias shape mismatch")
+    _check(s_x.dtype == torch.float32 and s_x.numel() == Q.shape[0], "s_x must be fp32 [B]")
+    _check(q_rowsum.dtype == torch.int32 and q_rowsum.numel() == Q.shape[0], "q_rowsum must be int32 [B]")
+    _check(_all_cuda(Q, s_x, q_rowsum, W_fields, scale, bias), "All tensors must be CUDA")
+    _check(out_dtype in _DT, "out_dtype must be float32, float16 or bfloat16")
+    q = Q.contiguous()
+    s_x = s_x.contiguous()
+    q_rowsum = q_rowsum.contiguous()
+    scale = _prep_vec(scale, s_x)
+    bias = None if bias is None else _prep_vec(bias, s_x)
+    B = q.shape[0]
+    y = torch.empty((B, N), dtype=out_dtype, device=q.device)
+    acc = torch.empty((B, N), dtype=torch.int32, device=q.device) if return_acc else None
+    res = None if residual is None else _residual_2d(residual, y, (B,), N)
+    with torch.cuda.device(q.device):
+        _status(_L.bt_ternary_gemm_i8_fields(
+            q.data_ptr(), 1 if q_operand_order else 0, s_x.data_ptr(), q_rowsum.data_ptr(), W_fields.data_ptr(),
+            1 if natural_from_pairs else 0, scale.data_ptr(), _dt(scale, "scale"), scale.numel(), _ptr(bias),
+            0 if bias is None else _dt(bias, "bias"), _ptr(res), y.data_ptr(), _DT[out_dtype], _ptr(acc), B, N, K,
+            _stream(q)))
+    return (y, acc) if return_acc else y
+
+
 def ternary_gemm_int8_tiled(Q: Tensor, s_x: Tensor, W_tiled: Tensor, scale: Tensor, bias: Optional[Tensor] = None,
                             in_features: int = -1, out_features: int = -1,
                             out_dtype: torch.dtype = torch.float32, return_acc: bool = False,
@@ -492,12 +539,13 @@ def ternary_quantize_pack(weight: Tensor, threshold_factor: float = 0.05, per_ch
     return packed, scale, tern
 
 
-def act_quant_int8(X: Tensor, operand_order: bool = False) -> Tuple[Tensor, Tensor]:
+def act_quant_int8(X: Tensor, operand_order: bool = False, return_rowsum: bool = False):
     """Per-row int8 activation quantization: ``(Q int8 [B,K], s_x fp32 [B])``.
 
     ``operand_order=True`` (K % 16 == 0) writes every 16-byte group of ``Q`` in the order the
     int8 GEMMs feed the matrix cores; such a ``Q`` must go to :func:`ternary_gemm_int8` with
-    ``q_operand_order=True``."""
+    ``q_operand_order=True``.  ``return_rowsum=True`` adds the rows' sums of ``Q`` (int32 ``[B]``), which
+    :func:`ternary_gemm_int8_fields` needs."""
     _check(X.dim() == 2 and X.numel() > 0, "X must be 2D and non-empty")
     _check(X.is_cuda, "All tensors must be CUDA")
     x = X.contiguous()
@@ -505,6 +553,11 @@ def act_quant_int8(X: Tensor, operand_order: bool = False) -> Tuple[Tensor, Tens
     q = torch.empty((B, K), dtype=torch.int8, device=x.device)
     s = torch.empty((B,), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
+        if return_rowsum:
+            rs = torch.empty((B,), dtype=torch.int32, device=x.device)
+            _status(_L.bt_act_quant_i8_rowsum(x.data_ptr(), _dt(x, "X"), B, K, q.data_ptr(), s.data_ptr(), rs.data_ptr(),
+                                              1 if operand_order else 0, _stream(x)))
+            return q, s, rs
         _status(_L.bt_act_quant_i8_layout(x.data_ptr(), _dt(x, "X"), B, K, q.data_ptr(), s.data_ptr(),
                                           1 if operand_order else 0, _stream(x)))
     return q, s

@@ -64,6 +64,10 @@ SIGNATURES = {
                                                _i64, _vp, _int, _vp, _int, _vp, _i64, _i64, _i64, _vp, _sz, _vp]),
     "bt_ternary_gemm_i8_tiled": (_int, [_vp, _int, _vp, _vp, _vp, _int, _i64, _vp, _int, _vp, _vp, _int, _vp,
                                         _i64, _i64, _i64, _vp]),
+    "bt_act_quant_i8_rowsum": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp, _int, _vp]),
+    "bt_retile_fields": (_int, [_vp, _i64, _i64, _vp, _vp]),
+    "bt_ternary_gemm_i8_fields": (_int, [_vp, _int, _vp, _vp, _vp, _int, _vp, _int, _i64, _vp, _int, _vp, _vp, _int, _vp,
+                                         _i64, _i64, _i64, _vp]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

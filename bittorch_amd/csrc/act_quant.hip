@@ -4,6 +4,7 @@
 // :439, :456-457) with the row scale taken over the whole row:
 //   amax = max_k |x[b,k]|;  s_x[b] = amax > 1e-6 ? amax / 127 : 1
 //   q[b,k] = (int8) clamp(roundf(x[b,k] * (1 / s_x[b])), -127, 127)
+// Optionally the rows' sums of q (int32), which the field-layout prefill GEMM starts its accumulators from.
 #include <cstdlib>
 
 #include "bt_common.h"
@@ -15,7 +16,7 @@ namespace bt {
 template <int DT>
 __global__ __launch_bounds__(256) void act_quant_kernel(const void* __restrict__ X, int64_t B, int64_t K,
                                                         int8_t* __restrict__ Q, float* __restrict__ s_x,
-                                                        int q_layout) {
+                                                        int q_layout, int32_t* __restrict__ rowsum) {
     const int lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= B) return;
@@ -58,6 +59,7 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const void* __restrict__
     const float inv = __fdiv_rn(1.0f, s);
     if (lane == 0) s_x[row] = s;
 
+    int qsum = 0;
     for (int64_t k = (int64_t)lane * 8; k < K; k += 512) {
         float v[8];
         load8(k, v);
@@ -66,6 +68,7 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const void* __restrict__
         for (int e = 0; e < 8; e++) {
             float r = round_half_away(__fmul_rn(v[e], inv));
             r = fmaxf(-127.0f, fminf(127.0f, r));
+            qsum += (int)r;  // (elements past K were loaded as zero)
             const uint32_t byte = (uint32_t)(uint8_t)(int8_t)(int)r;
             if (e < 4) lo |= byte << (8 * e);
             else hi |= byte << (8 * (e - 4));
@@ -78,6 +81,10 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const void* __restrict__
                 if (k + e < K) Q[base + k + e] = (int8_t)(((e < 4 ? lo : hi) >> (8 * (e & 3))) & 0xff);
         }
     }
+    if (rowsum) {  // (uniform)
+        qsum = wave_sum_i32(qsum);
+        if (lane == 0) rowsum[row] = qsum;
+    }
 }
 
 // One workgroup per row, the row held in registers between the absmax pass and the
@@ -86,8 +93,9 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const void* __restrict__
 template <int DT, int ITERS>
 __global__ __launch_bounds__(256) void act_quant_row_kernel(const void* __restrict__ X, int K,
                                                             int8_t* __restrict__ Q, float* __restrict__ s_x,
-                                                            int q_layout) {
+                                                            int q_layout, int32_t* __restrict__ rowsum) {
     __shared__ float part[4];
+    __shared__ int part_sum[4];
     const int tid = threadIdx.x;
     const int64_t base = (int64_t)blockIdx.x * K;
     float v[ITERS][8];
@@ -125,6 +133,7 @@ __global__ __launch_bounds__(256) void act_quant_row_kernel(const void* __restri
     const float s = (amax > 1e-6f) ? __fdiv_rn(amax, 127.0f) : 1.0f;
     const float inv = __fdiv_rn(1.0f, s);
     if (tid == 0) s_x[blockIdx.x] = s;
+    int qsum = 0;
 #pragma unroll
     for (int i = 0; i < ITERS; i++) {
         const int k = (i * 256 + tid) * 8;
@@ -133,6 +142,7 @@ __global__ __launch_bounds__(256) void act_quant_row_kernel(const void* __restri
         for (int e = 0; e < 8; e++) {
             float r = round_half_away(__fmul_rn(v[i][e], inv));
             r = fmaxf(-127.0f, fminf(127.0f, r));
+            if (k < K) qsum += (int)r;  // (a clamped group past the end repeats the row's last one)
             const uint32_t byte = (uint32_t)(uint8_t)(int8_t)(int)r;
             if (e < 4) lo |= byte << (8 * e);
             else hi |= byte << (8 * (e - 4));
@@ -140,26 +150,33 @@ __global__ __launch_bounds__(256) void act_quant_row_kernel(const void* __restri
         const uint2 o = q_layout == Q_OPERAND_ORDER ? q_to_operand_order(lo, hi, tid & 1) : make_uint2(lo, hi);
         if (k < K) st2_nt(Q + base + k, o.x, o.y);  // K % 16 == 0 in operand order: both lanes of a pair store
     }
+    if (rowsum) {  // (uniform)
+        qsum = wave_sum_i32(qsum);
+        if ((tid & 63) == 0) part_sum[tid >> 6] = qsum;
+        __syncthreads();
+        if (tid == 0) rowsum[blockIdx.x] = part_sum[0] + part_sum[1] + part_sum[2] + part_sum[3];
+    }
 }
 
 template <int DT>
-static bool launch_act_quant_rows(const void* X, int64_t B, int64_t K, int8_t* Q, float* s_x, int ql, hipStream_t st) {
+static bool launch_act_quant_rows(const void* X, int64_t B, int64_t K, int8_t* Q, float* s_x, int ql, int32_t* rs,
+                                  hipStream_t st) {
     if (K % 8 != 0 || K > 16384 || ((uintptr_t)X) % 16 != 0 || ((uintptr_t)Q) % 8 != 0 || B > 0x7fffffff ||
         tuning_env("BITTORCH_ACTQ_GENERIC"))
         return false;
     const dim3 grid((unsigned)B), block(256);
     const int k = (int)K;
-    if (K <= 2048) hipLaunchKernelGGL((act_quant_row_kernel<DT, 1>), grid, block, 0, st, X, k, Q, s_x, ql);
-    else if (K <= 4096) hipLaunchKernelGGL((act_quant_row_kernel<DT, 2>), grid, block, 0, st, X, k, Q, s_x, ql);
-    else if (K <= 8192) hipLaunchKernelGGL((act_quant_row_kernel<DT, 4>), grid, block, 0, st, X, k, Q, s_x, ql);
-    else if (K <= 12288) hipLaunchKernelGGL((act_quant_row_kernel<DT, 6>), grid, block, 0, st, X, k, Q, s_x, ql);
-    else hipLaunchKernelGGL((act_quant_row_kernel<DT, 8>), grid, block, 0, st, X, k, Q, s_x, ql);
+    if (K <= 2048) hipLaunchKernelGGL((act_quant_row_kernel<DT, 1>), grid, block, 0, st, X, k, Q, s_x, ql, rs);
+    else if (K <= 4096) hipLaunchKernelGGL((act_quant_row_kernel<DT, 2>), grid, block, 0, st, X, k, Q, s_x, ql, rs);
+    else if (K <= 8192) hipLaunchKernelGGL((act_quant_row_kernel<DT, 4>), grid, block, 0, st, X, k, Q, s_x, ql, rs);
+    else if (K <= 12288) hipLaunchKernelGGL((act_quant_row_kernel<DT, 6>), grid, block, 0, st, X, k, Q, s_x, ql, rs);
+    else hipLaunchKernelGGL((act_quant_row_kernel<DT, 8>), grid, block, 0, st, X, k, Q, s_x, ql, rs);
     return true;
 }
 
 // q_layout = Q_OPERAND_ORDER needs K % 16 == 0, X 16-byte and Q 8-byte aligned (the callers check)
 int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x, int q_layout,
-                     hipStream_t st) {
+                     int32_t* rowsum, hipStream_t st) {
     const int ql = q_layout;
     // the operand order is written 16 bytes at a time: callers check this too, but a buffer that cannot take it
     // must never be written row-major under that name
@@ -167,14 +184,15 @@ int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q
         set_error("bt_act_quant_i8: the operand-order layout needs K %% 16 == 0 and 16-byte aligned X and Q");
         return BT_ERR_INVALID;
     }
-    const bool done = (x_dtype == BT_F32)   ? launch_act_quant_rows<BT_F32>(X, B, K, Q, s_x, ql, st)
-                      : (x_dtype == BT_F16) ? launch_act_quant_rows<BT_F16>(X, B, K, Q, s_x, ql, st)
-                                            : launch_act_quant_rows<BT_BF16>(X, B, K, Q, s_x, ql, st);
+    int32_t* rs = rowsum;
+    const bool done = (x_dtype == BT_F32)   ? launch_act_quant_rows<BT_F32>(X, B, K, Q, s_x, ql, rs, st)
+                      : (x_dtype == BT_F16) ? launch_act_quant_rows<BT_F16>(X, B, K, Q, s_x, ql, rs, st)
+                                            : launch_act_quant_rows<BT_BF16>(X, B, K, Q, s_x, ql, rs, st);
     if (done) return check_launch("bt_act_quant_i8");
     const dim3 grid((unsigned)ceil_div(B, 4)), block(256);
-    if (x_dtype == BT_F32) hipLaunchKernelGGL(act_quant_kernel<BT_F32>, grid, block, 0, st, X, B, K, Q, s_x, ql);
-    else if (x_dtype == BT_F16) hipLaunchKernelGGL(act_quant_kernel<BT_F16>, grid, block, 0, st, X, B, K, Q, s_x, ql);
-    else hipLaunchKernelGGL(act_quant_kernel<BT_BF16>, grid, block, 0, st, X, B, K, Q, s_x, ql);
+    if (x_dtype == BT_F32) hipLaunchKernelGGL(act_quant_kernel<BT_F32>, grid, block, 0, st, X, B, K, Q, s_x, ql, rs);
+    else if (x_dtype == BT_F16) hipLaunchKernelGGL(act_quant_kernel<BT_F16>, grid, block, 0, st, X, B, K, Q, s_x, ql, rs);
+    else hipLaunchKernelGGL(act_quant_kernel<BT_BF16>, grid, block, 0, st, X, B, K, Q, s_x, ql, rs);
     return check_launch("bt_act_quant_i8");
 }
 

@@ -359,12 +359,21 @@ enum { Q_ROW_MAJOR = 0, Q_OPERAND_ORDER = 1 };
 //   W_LAYOUT_TILED_PAIRS_AS_NATURAL  a decode-tiled copy whose tiles are stored in gate/up pair order (tile t of the
 //                       left half of the columns at 2t, tile t of the right half at 2t + 1: BT_TILES_GATE_UP_PAIRS), read
 //                       by a kernel that works in the matrix's natural column order
-enum { W_LAYOUT_ROW_MAJOR = 0, W_LAYOUT_TILED = 1, W_LAYOUT_TILED_PAIRS_AS_NATURAL = 2 };
+//   W_LAYOUT_TILED_FIELDS  prefill-only variant of the decode-tiled copy (the tiled int8 GEMM alone reads it): the same
+//                       position for every aligned group of four dwords -- columns 4 q .. 4 q + 3 of a tile at one
+//                       16-row step and row group -- but inside the group field t (bits 2 t, 2 t + 1) of byte b of
+//                       dword c holds column 4 q + t at k = 4 b + c: w + 1 for t < 3, w in two's complement for t = 3
+//                       (retile_fields_kernel); _PAIRS_AS_NATURAL as above
+enum { W_LAYOUT_ROW_MAJOR = 0, W_LAYOUT_TILED = 1, W_LAYOUT_TILED_PAIRS_AS_NATURAL = 2, W_LAYOUT_TILED_FIELDS = 3,
+       W_LAYOUT_TILED_FIELDS_PAIRS_AS_NATURAL = 4 };
 static inline bool layout_tiled(int w_layout) { return w_layout != W_LAYOUT_ROW_MAJOR; }
+static inline bool layout_fields(int w_layout) {
+    return w_layout == W_LAYOUT_TILED_FIELDS || w_layout == W_LAYOUT_TILED_FIELDS_PAIRS_AS_NATURAL;
+}
 // The kernels' `tiles16` argument: the number of 16-column tiles, negative for W_LAYOUT_TILED_PAIRS_AS_NATURAL.
 static inline int tiles16_arg(int64_t N, int w_layout) {
     const int t = (int)ceil_div(N, 16);
-    return w_layout == W_LAYOUT_TILED_PAIRS_AS_NATURAL ? -t : t;
+    return (w_layout == W_LAYOUT_TILED_PAIRS_AS_NATURAL || w_layout == W_LAYOUT_TILED_FIELDS_PAIRS_AS_NATURAL) ? -t : t;
 }
 // Where 16-column tile t of the matrix (natural column order) sits in the copy; a tile past the end repeats the last
 // one (it only feeds outputs that are never stored).
@@ -405,6 +414,11 @@ __device__ __forceinline__ int decode2(uint32_t code) { return (int)(code == 1u)
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+__device__ __forceinline__ int wave_sum_i32(int v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
     return v;
 }
 

@@ -77,7 +77,8 @@ int launch_packed_generic(const void* X, int x_dtype, const uint8_t* W_T, const 
 int launch_unpacked(const void* X, int x_dtype, const int8_t* W, const Epilogue& epi, void* Y, int64_t B,
                     int64_t N, int64_t K, hipStream_t st);
 int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x, int q_layout,
-                     hipStream_t st);
+                     int32_t* rowsum, hipStream_t st);
+int launch_retile_fields(const uint8_t* W_tiled, int64_t N, int64_t K, uint8_t* W_fields, hipStream_t st);
 bool gemm_i8_supported(int64_t N, int64_t K, const void* Q, const void* W_T);
 int launch_row_op(int op, int dtype, const void* A, int64_t lda, const void* Bv, int64_t ldb, float eps, int64_t B,
                   int64_t K, void* H, int8_t* Q, float* s_x, int q_layout, hipStream_t st, const char* who);
@@ -101,8 +102,9 @@ bool planes_bf16_shape_ok(int64_t N, int64_t K);
 bool planes_bf16_wide(int64_t N, int64_t K);
 int launch_planes_bf16_wide(const void* X, const uint8_t* W, const Epilogue& epi, void* Y, int64_t N, int64_t K, hipStream_t st);
 bool gemm_i8_supported_tiled(int64_t N, int64_t K, const void* Q);
-int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_T, int w_layout, const Epilogue& epi,
-                   void* Y, int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st);
+int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const int32_t* q_rowsum, const uint8_t* W_T, int w_layout,
+                   const Epilogue& epi, void* Y, int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K,
+                   hipStream_t st);
 
 static bool valid_dtype(int dt) { return dt == BT_F32 || dt == BT_F16 || dt == BT_BF16; }
 
@@ -368,7 +370,7 @@ extern "C" int bt_act_quant_i8(const void* X, int x_dtype, int64_t B, int64_t K,
         set_error("bt_act_quant_i8: null pointer, empty shape or bad dtype");
         return BT_ERR_INVALID;
     }
-    return launch_act_quant(X, x_dtype, B, K, Q, s_x, Q_ROW_MAJOR, (hipStream_t)stream);
+    return launch_act_quant(X, x_dtype, B, K, Q, s_x, Q_ROW_MAJOR, nullptr, (hipStream_t)stream);
 }
 
 // q_layout: BT_Q_ROW_MAJOR or BT_Q_OPERAND_ORDER (K % 16 == 0, X 16-byte and Q 16-byte aligned)
@@ -395,7 +397,19 @@ extern "C" int bt_act_quant_i8_layout(const void* X, int x_dtype, int64_t B, int
     }
     const int rc = check_q_layout(who, q_layout, K, Q, X);
     if (rc) return rc;
-    return launch_act_quant(X, x_dtype, B, K, Q, s_x, q_layout, (hipStream_t)stream);
+    return launch_act_quant(X, x_dtype, B, K, Q, s_x, q_layout, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int bt_act_quant_i8_rowsum(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x,
+                                      int32_t* q_rowsum, int q_layout, void* stream) {
+    const char* who = "bt_act_quant_i8_rowsum";
+    if (!X || !Q || !s_x || !q_rowsum || B <= 0 || K <= 0 || !valid_dtype(x_dtype)) {
+        set_error("%s: null pointer, empty shape or bad dtype", who);
+        return BT_ERR_INVALID;
+    }
+    const int rc = check_q_layout(who, q_layout, K, Q, X);
+    if (rc) return rc;
+    return launch_act_quant(X, x_dtype, B, K, Q, s_x, q_layout, q_rowsum, (hipStream_t)stream);
 }
 
 extern "C" size_t bt_gemm_i8_workspace_bytes(int64_t B, int64_t N, int64_t K) {
@@ -436,7 +450,7 @@ static int gemm_i8_impl(const char* who, const int8_t* Q, int q_layout, const fl
             return BT_ERR_INVALID;
         }
         if (!prefers_stream(B, N, K, true, true) && gemm_i8_supported_tiled(N, K, Q))
-            return launch_gemm_i8(Q, q_layout, s_x, W_T, w_layout, epi, Y, y_dtype, acc_out, B, N, K, st);
+            return launch_gemm_i8(Q, q_layout, s_x, nullptr, W_T, w_layout, epi, Y, y_dtype, acc_out, B, N, K, st);
         return launch_stream(MODE_I8, Q, 1, s_x, W_T, w_layout, epi, Y, y_dtype, acc_out, B, N, K, 1, q_layout, 0, nullptr,
                              0.0f, 0, st);
     }
@@ -450,7 +464,7 @@ static int gemm_i8_impl(const char* who, const int8_t* Q, int q_layout, const fl
         }
         return launch_stream(MODE_I8, Q, 1, s_x, W_T, w_layout, epi, Y, y_dtype, acc_out, B, N, K, 1, q_layout, 0, nullptr, 0.0f, 0, st);
     }
-    return launch_gemm_i8(Q, q_layout, s_x, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, y_dtype, acc_out, B, N, K, st);
+    return launch_gemm_i8(Q, q_layout, s_x, nullptr, W_T, W_LAYOUT_ROW_MAJOR, epi, Y, y_dtype, acc_out, B, N, K, st);
 }
 
 extern "C" int bt_ternary_gemm_i8(const int8_t* Q, const float* s_x, const uint8_t* W_T, const void* scale,
@@ -498,7 +512,7 @@ extern "C" int bt_ternary_linear_tensor_core_forward(const void* X, int x_dtype,
     const char* lay = tuning_env("BITTORCH_Q_LAYOUT");
     const int q_layout = (K % 16 == 0 && ((uintptr_t)X) % 16 == 0 && !(lay && !strcmp(lay, "rowmajor")))
                              ? Q_OPERAND_ORDER : Q_ROW_MAJOR;
-    rc = launch_act_quant(X, x_dtype, B, K, Q, s_x, q_layout, (hipStream_t)stream);
+    rc = launch_act_quant(X, x_dtype, B, K, Q, s_x, q_layout, nullptr, (hipStream_t)stream);
     if (rc) return rc;
     (void)gemm_bytes;
     return gemm_i8_impl(who, Q, q_layout, s_x, W_T, W_LAYOUT_ROW_MAJOR, scale, scale_dtype, scale_len, bias, bias_dtype, nullptr,
@@ -562,7 +576,7 @@ extern "C" int bt_ternary_linear_tensor_core_forward_static(const void* X, int x
     float* s_x = (float*)(base + kStaticQBytes);
     // both are written in full by the quantizer before the GEMM reads them: nothing has to start at zero
     const int q_layout = (K % 16 == 0 && ((uintptr_t)X) % 16 == 0) ? Q_OPERAND_ORDER : Q_ROW_MAJOR;
-    rc = launch_act_quant(X, x_dtype, B, K, Q, s_x, q_layout, (hipStream_t)stream);
+    rc = launch_act_quant(X, x_dtype, B, K, Q, s_x, q_layout, nullptr, (hipStream_t)stream);
     if (rc) return rc;
     return gemm_i8_impl(who, Q, q_layout, s_x, W_T, W_LAYOUT_ROW_MAJOR, scale, scale_dtype, scale_len, bias, bias_dtype,
                         nullptr, Y, x_dtype, nullptr, B, N, K, stream);
@@ -847,4 +861,50 @@ extern "C" int bt_ternary_gemm_i8_tiled(const int8_t* Q, int q_layout, const flo
                                         int64_t B, int64_t N, int64_t K, void* stream) {
     return gemm_i8_impl("bt_ternary_gemm_i8_tiled", Q, q_layout, s_x, W_tiled, W_LAYOUT_TILED, scale, scale_dtype,
                         scale_len, bias, bias_dtype, residual, Y, y_dtype, acc_out, B, N, K, stream);
+}
+
+// ---- the prefill-only field layout of the tiled copy ----------------------------------------------------------------
+extern "C" int bt_retile_fields(const uint8_t* W_tiled, int64_t N, int64_t K, uint8_t* W_fields, void* stream) {
+    int rc = check_retile("bt_retile_fields", W_tiled, W_fields, N, K, W_tiled);
+    if (rc) return rc;
+    if (((uintptr_t)W_fields) % 256 != 0) {
+        set_error("bt_retile_fields: W_fields must be 256-byte aligned");
+        return BT_ERR_INVALID;
+    }
+    return launch_retile_fields(W_tiled, N, K, W_fields, (hipStream_t)stream);
+}
+
+extern "C" int bt_ternary_gemm_i8_fields(const int8_t* Q, int q_layout, const float* s_x, const int32_t* q_rowsum,
+                                         const uint8_t* W_fields, int tile_order, const void* scale, int scale_dtype,
+                                         int64_t scale_len, const void* bias, int bias_dtype, const void* residual,
+                                         void* Y, int y_dtype, int32_t* acc_out, int64_t B, int64_t N, int64_t K,
+                                         void* stream) {
+    const char* who = "bt_ternary_gemm_i8_fields";
+    int rc = check_shape(who, Q, W_fields, Y, y_dtype, B, N, K);
+    if (rc) return rc;
+    if (!s_x || !q_rowsum) {
+        set_error("%s: s_x or q_rowsum is null", who);
+        return BT_ERR_INVALID;
+    }
+    rc = check_q_layout(who, q_layout, K, Q, nullptr);
+    if (rc) return rc;
+    if ((rc = check_tile_order(who, tile_order, N))) return rc;
+    if (K % 128 != 0 || K > kMaxKInt8) {
+        set_error("%s: K must be a multiple of 128 and at most %lld (K=%lld); other shapes take the decode-tiled copy", who,
+                  (long long)kMaxKInt8, (long long)K);
+        return BT_ERR_INVALID;
+    }
+    if (!fast_path_ok(Y, N, K) || (acc_out && ((uintptr_t)acc_out) % 16 != 0) || !stream_supported_tiled(N, K, W_fields) ||
+        !gemm_i8_supported_tiled(N, K, Q)) {
+        set_error("%s: N %% 4 == 0, 16-byte aligned Q, Y and acc_out and a 256-byte aligned copy below 4 GiB are needed", who);
+        return BT_ERR_INVALID;
+    }
+    Epilogue epi;
+    rc = make_epilogue(who, scale, scale_dtype, scale_len, bias, bias_dtype, N, &epi);
+    if (rc) return rc;
+    rc = set_residual(who, residual, &epi);
+    if (rc) return rc;
+    return launch_gemm_i8(Q, q_layout, s_x, q_rowsum, W_fields,
+                          tile_order ? W_LAYOUT_TILED_FIELDS_PAIRS_AS_NATURAL : W_LAYOUT_TILED_FIELDS, epi, Y, y_dtype, acc_out,
+                          B, N, K, (hipStream_t)stream);
 }

@@ -53,6 +53,7 @@ struct GemmParams {
     int64_t Kb;
     int y_dtype;
     int long_epilogue;    // A/B runs and tests (option GEMM_LONG_EPILOGUE): never the short epilogue
+    const int32_t* q_rowsum;  // FL kernels: sum of each row of Q over K (what the codes w + 1 of the field layout add)
     Epilogue epi;
 };
 static_assert(offsetof(GemmParams, s_x) == 64, "first argument line as laid out above");
@@ -108,7 +109,18 @@ __device__ __forceinline__ void load_epi_operands(const GemmParams& p, int64_t m
     }
 }
 
-template <int YDT, int MB0, int NB>
+// The field layout (W_LAYOUT_TILED_FIELDS, FL = true) leaves column block t of a lane scaled by 4^t (64 for t = 3):
+// float(acc) * (127 / 4^t) is the same real number as float(acc / 4^t) * 127 -- the scaled accumulator has the
+// significant bits of the true one and the factor is a power of two apart from 127 -- so the epilogue takes the
+// scale out in the multiplication it already has.
+template <bool FL>
+__device__ __forceinline__ constexpr float k127(int t) {
+    return FL ? (t == 0 ? 127.0f : t == 1 ? 127.0f / 4.0f : t == 2 ? 127.0f / 16.0f : 127.0f / 64.0f) : 127.0f;
+}
+template <bool FL>
+__device__ __forceinline__ constexpr int field_shift(int t) { return FL ? 2 * t : 0; }
+
+template <int YDT, int MB0, int NB, bool FL = false>
 __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&acc)[2 * NB][4], int64_t m0, int g,
                                               int64_t ncol, const EpiOperands<NB>& e) {
     float ws[4], bs[4];
@@ -130,7 +142,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&a
                 // float(127 a) = float(a) * 127 rounded once: |a| <= 127 K < 2^24 (checked by the host), so float(a)
                 // is exact and the product rounds the same integer the reference converts (one operation less than
                 // 127 a in integers first)
-                const float a127f = __fmul_rn((float)acc[MB0 + mbi][t][r], 127.0f);
+                const float a127f = __fmul_rn((float)acc[MB0 + mbi][t][r], k127<FL>(t));
                 y[t] = epi_int8_f(a127f, sx, ws[t], bs[t]);
             }
             if (p.epi.residual) add_residual4(y, p.epi.residual, YDT, m * p.N + ncol);
@@ -138,7 +150,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&a
             if (p.acc_out) {
                 uint32_t a127[4];
 #pragma unroll
-                for (int t = 0; t < 4; t++) a127[t] = (uint32_t)times127(acc[MB0 + mbi][t][r]);
+                for (int t = 0; t < 4; t++) a127[t] = (uint32_t)times127(acc[MB0 + mbi][t][r] >> field_shift<FL>(t));
                 st4_nt(p.acc_out + m * p.N + ncol, a127[0], a127[1], a127[2], a127[3]);
             }
         }
@@ -148,7 +160,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, const v4i (&a
 // no residual, no accumulator output, and every row scale large enough for the two-operation division
 // (all wave-uniform, checked by the caller).  A row's address is a uniform base plus a 32-bit lane offset fixed
 // for the whole epilogue.  Same bits as gemm_epilogue.
-template <int YDT, int MB0, int NB, bool RES = false>
+template <int YDT, int MB0, int NB, bool RES = false, bool FL = false>
 __device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, const v4i (&acc)[2 * NB][4], int64_t m0, int g,
                                                    int64_t ncol, const EpiOperands<NB>& e) {
     float ws[4], bs[4];
@@ -170,7 +182,7 @@ __device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, const v4
             float y[4];
 #pragma unroll
             for (int t = 0; t < 4; t++) {
-                const float a127f = __fmul_rn((float)acc[MB0 + mbi][t][r], 127.0f);
+                const float a127f = __fmul_rn((float)acc[MB0 + mbi][t][r], k127<FL>(t));
                 const float q = div127_fast(__fmul_rn(a127f, sx));
                 y[t] = __fadd_rn(__fmul_rn(q, ws[t]), bs[t]);
             }
@@ -196,26 +208,26 @@ __device__ __forceinline__ void gemm_epilogue_fast(const GemmParams& p, const v4
         }
     }
 }
-template <int MB0, int NB>
+template <int MB0, int NB, bool FL = false>
 __device__ __forceinline__ void gemm_epilogue_dt(const GemmParams& p, const v4i (&acc)[2 * NB][4], int64_t m0, int g,
                                                  int64_t ncol, const EpiOperands<NB>& e) {
-    if (p.y_dtype == BT_BF16) gemm_epilogue<BT_BF16, MB0, NB>(p, acc, m0, g, ncol, e);
-    else if (p.y_dtype == BT_F16) gemm_epilogue<BT_F16, MB0, NB>(p, acc, m0, g, ncol, e);
-    else gemm_epilogue<BT_F32, MB0, NB>(p, acc, m0, g, ncol, e);
+    if (p.y_dtype == BT_BF16) gemm_epilogue<BT_BF16, MB0, NB, FL>(p, acc, m0, g, ncol, e);
+    else if (p.y_dtype == BT_F16) gemm_epilogue<BT_F16, MB0, NB, FL>(p, acc, m0, g, ncol, e);
+    else gemm_epilogue<BT_F32, MB0, NB, FL>(p, acc, m0, g, ncol, e);
 }
-template <int MB0, int NB>
+template <int MB0, int NB, bool FL = false>
 __device__ __forceinline__ void gemm_epilogue_dt(const GemmParams& p, const v4i (&acc)[2 * NB][4], int64_t m0, int g,
                                                  int64_t ncol, const EpiOperands<NB>& e, bool fast) {
     if (fast) {  // wave-uniform
         if (p.epi.residual) {  // (16-bit outputs only: checked by the caller)
-            if (p.y_dtype == BT_BF16) gemm_epilogue_fast<BT_BF16, MB0, NB, true>(p, acc, m0, g, ncol, e);
-            else gemm_epilogue_fast<BT_F16, MB0, NB, true>(p, acc, m0, g, ncol, e);
-        } else if (p.y_dtype == BT_BF16) gemm_epilogue_fast<BT_BF16, MB0, NB>(p, acc, m0, g, ncol, e);
-        else if (p.y_dtype == BT_F16) gemm_epilogue_fast<BT_F16, MB0, NB>(p, acc, m0, g, ncol, e);
-        else gemm_epilogue_fast<BT_F32, MB0, NB>(p, acc, m0, g, ncol, e);
+            if (p.y_dtype == BT_BF16) gemm_epilogue_fast<BT_BF16, MB0, NB, true, FL>(p, acc, m0, g, ncol, e);
+            else gemm_epilogue_fast<BT_F16, MB0, NB, true, FL>(p, acc, m0, g, ncol, e);
+        } else if (p.y_dtype == BT_BF16) gemm_epilogue_fast<BT_BF16, MB0, NB, false, FL>(p, acc, m0, g, ncol, e);
+        else if (p.y_dtype == BT_F16) gemm_epilogue_fast<BT_F16, MB0, NB, false, FL>(p, acc, m0, g, ncol, e);
+        else gemm_epilogue_fast<BT_F32, MB0, NB, false, FL>(p, acc, m0, g, ncol, e);
         return;
     }
-    gemm_epilogue_dt<MB0, NB>(p, acc, m0, g, ncol, e);
+    gemm_epilogue_dt<MB0, NB, FL>(p, acc, m0, g, ncol, e);
 }
 
 // Adding the two K halves: waves (wn, 0) and (wn, 1) hold partial sums of the same outputs.  K half 1 hands over row
@@ -269,8 +281,16 @@ __device__ __forceinline__ void take_blocks(v4i (&acc)[2 * NB][4], int mb0, cons
 // NB: 16-row blocks per K half and wave: 4 is the 128-row tile; 2 and 1 are the tiles of 64 and 32 rows (same columns,
 // same staging and LDS layout with rows past the tile clamped, a quarter to half of the MFMAs per decoded weight) that a
 // launch's remainder is cut into when whole tiles would leave most compute units idle (launch_gemm_i8).
-template <bool TAIL, bool QOO, bool WT = false, bool ANTIPHASE = true, int NB = 4>
+// FL = true (with WT): W_T is the field-layout copy (W_LAYOUT_TILED_FIELDS, retile_fields_kernel): the same 16 bytes
+// per lane and stage, but byte b of dword c holds, in its four 2-bit fields, the weights of the lane's FOUR columns at
+// k = 4 b + c -- field t (columns 4 j + t) as w + 1 for t < 3 and as a two's-complement w for t = 3.  The B operand of
+// column block t and operand dword c is then `raw[c] & (0x03030303 << 2 t)`: one AND instead of a mask and a byte
+// permute, an int8 value 4^t (w + 1) resp. 64 w.  The sum over k of q (w + 1) is the wanted sum plus the row's sum of
+// q, which the accumulators of K half 0 start from with the opposite sign (p.q_rowsum), and the factor 4^t leaves in
+// the epilogue's multiplication by 127 (k127).  Integer sums throughout: the same accumulators, the same outputs.
+template <bool TAIL, bool QOO, bool WT = false, bool ANTIPHASE = true, int NB = 4, bool FL = false>
 __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
+    static_assert(!FL || (WT && !TAIL), "the field layout is a tiled layout; K in whole stages");
     __shared__ __attribute__((aligned(16))) uint8_t lds[65536];  // 2 A stages; reused for the K-half exchange
     constexpr int BM = 32 * NB;  // rows of the tile
 
@@ -410,6 +430,21 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     for (int mb = 0; mb < 2 * NB; mb++)
 #pragma unroll
         for (int t = 0; t < 4; t++) acc[mb][t] = v4i{0, 0, 0, 0};
+    if constexpr (FL) {
+        if (kgrp == 0) {  // (wave-uniform) lane (j, g) holds rows 16 mb + 4 g + r of its columns
+#pragma unroll
+            for (int mb = 0; mb < 2 * NB; mb++) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int64_t m = m0 + 16 * mb + 4 * g + r;
+                    const int32_t rs = p.q_rowsum[m < p.M ? m : p.M - 1];
+                    acc[mb][0][r] = -rs;
+                    acc[mb][1][r] = -(rs << 2);
+                    acc[mb][2][r] = -(rs << 4);
+                }
+            }
+        }
+    }
 
     // ---- main loop --------------------------------------------------------------------
     // Stage s is computed from LDS buffer s%2 and is software-pipelined inside the wave so
@@ -428,6 +463,13 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     uint4 a_lo[NB], a_hi[NB];
     const uint32_t a_lds_off = (uint32_t)(kgrp * (G_MB * 1024)) + ((uint32_t)lane << 4);
     auto decode_b = [&](const uint32_t (&raw)[4], v4i (&out)[4]) {
+        if constexpr (FL) {
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+#pragma unroll
+                for (int c = 0; c < 4; c++) out[t][c] = (int)(raw[c] & (0x03030303u << (2 * t)));
+            return;
+        }
         uint32_t G[4];
         if constexpr (WT) { G[0] = raw[0]; G[1] = raw[1]; G[2] = raw[2]; G[3] = raw[3]; }
         else transpose4x4_bytes(raw[0], raw[1], raw[2], raw[3], G);
@@ -467,6 +509,10 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
     // for 16 cycles; the VALU operations of the same wave behind it run in its shadow)
     uint32_t d_t[4], d_G[4], d_H[4];
     auto decode_slice = [&](int c, const uint32_t (&raw)[4], v4i (&out)[4]) {
+        if constexpr (FL) {  // one operation per slice: operand dword c & 3 of column block c >> 2
+            if (c < 16) out[c >> 2][c & 3] = (int)(raw[c & 3] & (0x03030303u << (2 * (c >> 2))));
+            return;
+        }
         const uint32_t lutA_lo = 0x00FF0100u, lutB_lo = 0x0000FF00u, lutB_hi = 0x00000001u;
         auto partA = [&](int t) {
             d_H[t] = d_G[t] >> 4;
@@ -634,8 +680,8 @@ __global__ __launch_bounds__(512) void gemm_i8_kernel(GemmParams p) {
         for (int r = 0; r < 4; r++) small_sx |= !(__builtin_fabsf(epi_ops.sx[mbi][r]) >= DIV127_FAST_MIN_SX);
     const bool fast = short_ok && __builtin_amdgcn_ballot_w64(small_sx) == 0ull;
     if (!col_ok) return;
-    if (kgrp == 0) gemm_epilogue_dt<0, NB>(p, acc, m0, g, ncol, epi_ops, fast);  // wave-uniform branch
-    else gemm_epilogue_dt<NB, NB>(p, acc, m0, g, ncol, epi_ops, fast);
+    if (kgrp == 0) gemm_epilogue_dt<0, NB, FL>(p, acc, m0, g, ncol, epi_ops, fast);  // wave-uniform branch
+    else gemm_epilogue_dt<NB, NB, FL>(p, acc, m0, g, ncol, epi_ops, fast);
 }
 
 
@@ -653,7 +699,7 @@ bool gemm_i8_supported(int64_t N, int64_t K, const void* Q, const void* W_T) {
 
 // One launch over column tiles [tile_n0, tile_n0 + tiles_n) in tiles of 32 * NB rows.
 template <int NB>
-static int launch_gemm_i8_part(GemmParams p, int tile_n0, int tiles_n, bool qoo, bool tiled, hipStream_t st) {
+static int launch_gemm_i8_part(GemmParams p, int tile_n0, int tiles_n, bool qoo, bool tiled, bool fields, hipStream_t st) {
     p.tile_n0 = tile_n0;
     p.tiles_n = tiles_n;
     p.tiles_m = (int)ceil_div(p.M, 32 * NB);
@@ -665,7 +711,10 @@ static int launch_gemm_i8_part(GemmParams p, int tile_n0, int tiles_n, bool qoo,
     p.per_xcd = (int)ceil_div(total, 8);
     const dim3 grid((unsigned)(p.per_xcd * 8)), block(512);
     const bool tail = p.K % G_BK != 0;
-    if constexpr (NB != 4) {  // (only where launch_gemm_i8 cuts finer: tiled weights, whole stages)
+    if (fields) {  // (the caller has checked: K in whole stages)
+        if (qoo) hipLaunchKernelGGL((gemm_i8_kernel<false, true, true, true, NB, true>), grid, block, 0, st, p);
+        else hipLaunchKernelGGL((gemm_i8_kernel<false, false, true, true, NB, true>), grid, block, 0, st, p);
+    } else if constexpr (NB != 4) {  // (only where launch_gemm_i8 cuts finer: tiled weights, whole stages)
         if (qoo) hipLaunchKernelGGL((gemm_i8_kernel<false, true, true, true, NB>), grid, block, 0, st, p);
         else hipLaunchKernelGGL((gemm_i8_kernel<false, false, true, true, NB>), grid, block, 0, st, p);
     } else if (tiled) {
@@ -687,29 +736,31 @@ static int launch_gemm_i8_part(GemmParams p, int tile_n0, int tiles_n, bool qoo,
     return check_launch("bt_ternary_gemm_i8");
 }
 
-int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const uint8_t* W_T, int w_layout, const Epilogue& epi,
-                   void* Y, int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K, hipStream_t st) {
+// q_rowsum: the rows' sums of Q, needed (and only read) with a field-layout copy
+int launch_gemm_i8(const int8_t* Q, int q_layout, const float* s_x, const int32_t* q_rowsum, const uint8_t* W_T, int w_layout,
+                   const Epilogue& epi, void* Y, int y_dtype, int32_t* acc_out, int64_t M, int64_t N, int64_t K,
+                   hipStream_t st) {
     GemmParams p = {};
-    p.Q = Q; p.s_x = s_x; p.W_T = W_T; p.Y = Y; p.acc_out = acc_out; p.epi = epi;
+    p.Q = Q; p.s_x = s_x; p.W_T = W_T; p.Y = Y; p.acc_out = acc_out; p.epi = epi; p.q_rowsum = q_rowsum;
     p.M = M; p.N = N; p.K = K; p.Kb = ceil_div(K, 4);
     p.y_dtype = y_dtype;
     p.long_epilogue = option(OPT_GEMM_LONG_EPILOGUE) != nullptr;
     p.wsteps = (int)ceil_div(p.Kb, 16);
     p.tiles16 = tiles16_arg(N, w_layout);
-    const bool qoo = q_layout == Q_OPERAND_ORDER, tiled = layout_tiled(w_layout);
+    const bool qoo = q_layout == Q_OPERAND_ORDER, tiled = layout_tiled(w_layout), fields = layout_fields(w_layout);
     const int64_t tiles_n = ceil_div(N, G_BN);
     // the column tiles of a mostly empty last round in finer tiles, a launch of their own behind the whole tiles
     // (gemm_split; same sums, same bits)
     const GemmSplit sp = gemm_split(M, N, tiled && K % G_BK == 0 && !tuning_env("BITTORCH_GEMM_INPHASE"));
     if (sp.nb != 4) {
         if (sp.cols < tiles_n) {
-            const int rc = launch_gemm_i8_part<4>(p, 0, (int)(tiles_n - sp.cols), qoo, tiled, st);
+            const int rc = launch_gemm_i8_part<4>(p, 0, (int)(tiles_n - sp.cols), qoo, tiled, fields, st);
             if (rc) return rc;
         }
-        return sp.nb == 1 ? launch_gemm_i8_part<1>(p, (int)(tiles_n - sp.cols), (int)sp.cols, qoo, tiled, st)
-                          : launch_gemm_i8_part<2>(p, (int)(tiles_n - sp.cols), (int)sp.cols, qoo, tiled, st);
+        return sp.nb == 1 ? launch_gemm_i8_part<1>(p, (int)(tiles_n - sp.cols), (int)sp.cols, qoo, tiled, fields, st)
+                          : launch_gemm_i8_part<2>(p, (int)(tiles_n - sp.cols), (int)sp.cols, qoo, tiled, fields, st);
     }
-    return launch_gemm_i8_part<4>(p, 0, (int)tiles_n, qoo, tiled, st);
+    return launch_gemm_i8_part<4>(p, 0, (int)tiles_n, qoo, tiled, fields, st);
 }
 
 }  // namespace bt

@@ -233,6 +233,40 @@ __global__ __launch_bounds__(256) void untile_kernel(const uint32_t* __restrict_
     W_T[i] = (uint8_t)(T[idx] >> (8 * (kb & 3)));
 }
 
+// ---- the field layout of the tiled copy (W_LAYOUT_TILED_FIELDS) ----------------------------------------------------
+// One thread per aligned group of four dwords of the tiled copy (columns 4 q .. 4 q + 3 of a tile at one step and row
+// group): a transpose of the 2-bit fields inside the group.  In the tiled copy dword t holds column t with the code of
+// k = 4 b + c at bits 8 b + 2 c; in the field layout dword c holds, at bits 8 b + 2 t, column t at k = 4 b + c --
+// as w + 1 (codes 0 / +1 / -1 -> 1 / 2 / 0) for t < 3 and as w in two's complement (0 / 1 / 3) for t = 3.
+__global__ __launch_bounds__(256) void retile_fields_kernel(const uint4* __restrict__ T, uint4* __restrict__ F, int64_t groups) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= groups) return;
+    const uint4 in = T[i];
+    const uint32_t old[4] = {in.x, in.y, in.z, in.w};
+    uint32_t out[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const uint32_t code = (old[t] >> (8 * b + 2 * c)) & 3u;  // 0: 0, 1: +1, 2: -1
+                const uint32_t f = (t < 3) ? ((code == 1u) ? 2u : (code == 2u) ? 0u : 1u) : ((code == 2u) ? 3u : code);
+                out[c] |= f << (8 * b + 2 * t);
+            }
+        }
+    }
+    F[i] = make_uint4(out[0], out[1], out[2], out[3]);
+}
+
+int launch_retile_fields(const uint8_t* W_tiled, int64_t N, int64_t K, uint8_t* W_fields, hipStream_t st) {
+    const int64_t Kb = ceil_div(K, 4), S = ceil_div(Kb, 16);
+    const int64_t groups = ceil_div(N, 16) * S * 16;  // 64 dwords per step
+    hipLaunchKernelGGL(retile_fields_kernel, dim3((unsigned)ceil_div(groups, 256)), dim3(256), 0, st, (const uint4*)W_tiled,
+                       (uint4*)W_fields, groups);
+    return check_launch("bt_retile_fields");
+}
+
 // forward: W_T [Kb, N] -> T;  inverse: T -> W_out [Kb, N]
 int launch_retile(const uint8_t* W_T, int64_t N, int64_t K, int pairs, void* T, bool inverse, uint8_t* W_out, hipStream_t st) {
     const int64_t Kb = ceil_div(K, 4), S = ceil_div(Kb, 16);

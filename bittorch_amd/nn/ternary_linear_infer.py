@@ -34,6 +34,9 @@ from ..quant.ternary_packed import pack_ternary_transposed, unpack_ternary_trans
 
 # batches up to this many rows stream the tiled weights (once per 16 rows) instead of running the tiled GEMM
 DECODE_ROWS = 128
+# From this many rows an int8 call with row sums takes the prefill GEMM on the field-layout copy (prepare_prefill):
+# below it the routing between the streaming kernel and the tiled GEMM on the decode-tiled copy does as well or better.
+PREFILL_ROWS = 384
 
 
 class TernaryLinearInference(nn.Module):
@@ -56,6 +59,9 @@ class TernaryLinearInference(nn.Module):
         self._tile_order = "natural"
         self._tiled: Optional[Tensor] = None
         self._tiled_key = None
+        # prefill-only second copy (prepare_prefill) and the tiled copy it was made from
+        self._fields: Optional[Tensor] = None
+        self._fields_src: Optional[Tensor] = None
 
     # ---- which copies of the weights the layer holds ----------------------------------------
     def _has_row_major(self) -> bool:
@@ -133,8 +139,10 @@ class TernaryLinearInference(nn.Module):
         return self._tiled
 
     def resident_weight_bytes(self) -> int:
-        """Bytes of packed weights the layer holds right now (tiled copy and / or row-major buffer)."""
+        """Bytes of packed weights the layer holds right now (tiled copy and / or row-major buffer, and the prefill
+        copy if one was asked for)."""
         n = self._buffers["weight_packed"].numel() if self._has_row_major() else 0
+        n += self._fields.numel() if self._prefill_copy() is not None else 0
         return n + (self._tiled.numel() if self._tiled is not None else 0)
 
     # state_dict / load_state_dict / .to() / pickling see the reference's layout whatever the layer holds
@@ -167,6 +175,7 @@ class TernaryLinearInference(nn.Module):
             bufs.update(state["_buffers"])
             state["_buffers"] = bufs
         state["_tiled"], state["_tiled_key"] = None, None
+        state["_fields"], state["_fields_src"] = None, None
         return state
 
     def prepare_decode(self) -> "TernaryLinearInference":
@@ -175,6 +184,31 @@ class TernaryLinearInference(nn.Module):
         if self.decode_tiled and (not self._has_row_major() or self._buffers["weight_packed"].is_cuda):
             self.tiled_weights()
         return self
+
+    def prepare_prefill(self) -> "TernaryLinearInference":
+        """Opt in to a SECOND resident copy of the weights (0.25 bytes per weight more) in the field layout that only
+        the prefill int8 GEMM reads: ``forward_int8(..., q_rowsum=...)`` with at least ``PREFILL_ROWS`` rows then
+        decodes a weight operand with one AND.  The same bits as without it; 10-16 % faster GEMMs for prefill chunks
+        of 512-1024 rows, nothing at 2048 rows and more.  Needs ``in_features % 128 == 0`` and the decode-tiled copy
+        (GPU); ``drop_prefill()`` releases it."""
+        self.prepare_decode()
+        if self._tiled is not None and self.in_features % 128 == 0:
+            from .. import _C
+            self._fields = _C.retile_fields(self._tiled, self.in_features, self.out_features)
+            self._fields_src = self._tiled
+            torch.cuda.current_stream(self._tiled.device).synchronize()
+        return self
+
+    def drop_prefill(self) -> "TernaryLinearInference":
+        self._fields, self._fields_src = None, None
+        return self
+
+    def _prefill_copy(self) -> Optional[Tensor]:
+        """The field-layout copy if it still matches the tiled copy the layer holds (a layer whose weights were
+        reloaded, moved or re-tiled simply stops using it until ``prepare_prefill`` is called again)."""
+        if self._fields is not None and self._fields_src is self._tiled and self._tiled is not None:
+            return self._fields
+        return None
 
     def _tiled_for(self, x: Tensor, rows: int, order: str = "natural") -> Optional[Tensor]:
         """The tiled copy if this call can run on it, else None.  ``order`` is what the call wants: ``"natural"`` (a
@@ -273,11 +307,23 @@ class TernaryLinearInference(nn.Module):
         return F.silu(gu[..., :half]) * gu[..., half:]
 
     def forward_int8(self, q: Tensor, s_x: Tensor, out_dtype: torch.dtype = torch.bfloat16,
-                     residual: Optional[Tensor] = None, q_operand_order: bool = False) -> Tensor:
+                     residual: Optional[Tensor] = None, q_operand_order: bool = False,
+                     q_rowsum: Optional[Tensor] = None) -> Tensor:
         """Forward from activations already quantized per row to int8 (``ops.rmsnorm`` /
         ``ops.swiglu`` / ``ops.act_quant_int8`` with ``quantize=True``): int8 matrix cores, int32
-        accumulators (GPU only).  ``q_operand_order`` as in :func:`ops.ternary_linear_int8`."""
-        tiled = self._tiled_for(q, q.numel() // max(q.shape[-1], 1))
+        accumulators (GPU only).  ``q_operand_order`` as in :func:`ops.ternary_linear_int8`.  ``q_rowsum`` (the rows'
+        sums of ``q``, ``ops.act_quant_int8(..., return_rowsum=True)``) lets a prefill batch run on the layer's
+        field-layout copy where ``prepare_prefill`` built one; the result does not depend on it."""
+        rows = q.numel() // max(q.shape[-1], 1)
+        fields = self._prefill_copy() if (q_rowsum is not None and rows >= PREFILL_ROWS and q.is_cuda) else None
+        if fields is not None and os.environ.get("BITTORCH_KERNEL") != "generic":
+            from .. import _C
+            y = _C.ternary_gemm_int8_fields(q.reshape(-1, q.shape[-1]), s_x.reshape(-1), q_rowsum.reshape(-1), fields,
+                                            self.scale, self.bias, self.in_features, self.out_features, out_dtype, False,
+                                            None if residual is None else residual.reshape(-1, residual.shape[-1]),
+                                            q_operand_order, self._natural_from_pairs)
+            return y.reshape(*q.shape[:-1], self.out_features)
+        tiled = self._tiled_for(q, rows)
         if tiled is not None:
             from .. import _C
             lead = q.shape[:-1]

@@ -35,12 +35,17 @@ def rmsnorm(x: Tensor, weight: Optional[Tensor] = None, eps: float = 1e-6, store
     return _C.rmsnorm(x, weight, eps, store, quantize, operand_order)
 
 
-def act_quant_int8(x: Tensor, operand_order: bool = False) -> Tuple[Tensor, Tensor]:
-    """Per-row int8 quantization of ``x`` ``(*, K)``: ``(q int8 (*, K), s_x fp32 (*))``."""
+def act_quant_int8(x: Tensor, operand_order: bool = False, return_rowsum: bool = False):
+    """Per-row int8 quantization of ``x`` ``(*, K)``: ``(q int8 (*, K), s_x fp32 (*))``; with ``return_rowsum`` also the
+    rows' sums of ``q`` (int32 ``(*)``), which ``TernaryLinearInference.forward_int8`` hands to the prefill GEMM on a
+    layer's field-layout copy (``prepare_prefill``)."""
     from .. import _C
 
-    q, s = _C.act_quant_int8(x.reshape(-1, x.shape[-1]), operand_order)
-    return q.reshape(x.shape), s.reshape(x.shape[:-1])
+    out = _C.act_quant_int8(x.reshape(-1, x.shape[-1]), operand_order, return_rowsum)
+    lead = x.shape[:-1]
+    if return_rowsum:
+        return out[0].reshape(x.shape), out[1].reshape(lead), out[2].reshape(lead)
+    return out[0].reshape(x.shape), out[1].reshape(lead)
 
 
 def ternary_linear_int8(q: Tensor, s_x: Tensor, w_packed_T: Tensor, scale: Tensor, in_features: int,

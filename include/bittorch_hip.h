@@ -148,6 +148,11 @@ int bt_act_quant_i8(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q,
 enum { BT_Q_ROW_MAJOR = 0, BT_Q_OPERAND_ORDER = 1 };
 int bt_act_quant_i8_layout(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x,
                            int q_layout, void* stream);
+/* The same, and q_rowsum [B] int32: the sum of each quantized row over K, which bt_ternary_gemm_i8_fields needs
+ * (same arithmetic for Q and s_x: csrc/kernels/ternary_gemm_tensor_core.cu:343-347, :439; the sums have no
+ * counterpart in the reference). */
+int bt_act_quant_i8_rowsum(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q, float* s_x, int32_t* q_rowsum,
+                           int q_layout, void* stream);
 
 /*
  * int8 x packed-ternary GEMM on the matrix cores, int32 accumulators.
@@ -270,6 +275,25 @@ int bt_ternary_gemm_i8_tiled(const int8_t* Q, int q_layout, const float* s_x, co
                              const void* scale, int scale_dtype, int64_t scale_len, const void* bias,
                              int bias_dtype, const void* residual, void* Y, int y_dtype, int32_t* acc_out,
                              int64_t B, int64_t N, int64_t K, void* stream);
+
+/*
+ * A prefill-only second form of the tiled copy, for the matrix-core int8 GEMM alone (no counterpart in the
+ * reference; the arithmetic is its int8 kernel's, csrc/kernels/ternary_gemm_tensor_core.cu:343-347, :439, :583-589,
+ * :652, and the results equal bt_ternary_gemm_i8_tiled bit for bit, int32 accumulators included).  Same size and
+ * alignment as the tiled copy (bt_tiled_weights_bytes); inside every aligned 16 bytes the 2-bit fields are
+ * transposed so that a byte holds one k of FOUR columns, three of them as w + 1 and one in two's complement, and
+ * the GEMM's operand of a column block is one AND of a loaded dword instead of a mask and a byte permute.  What
+ * the codes w + 1 add to a dot product is the row's sum of q, which the caller supplies (bt_act_quant_i8_rowsum).
+ *   bt_retile_fields: W_tiled (natural or pair-ordered, the order is kept) -> W_fields.
+ *   bt_ternary_gemm_i8_fields: always the tiled GEMM kernel (meant for prefill batches: hundreds of rows and more);
+ *     K % 128 == 0; tile_order BT_TILES_GATE_UP_PAIRS reads a pair-ordered copy and writes Y in the matrix's natural
+ *     column order; otherwise the arguments of bt_ternary_gemm_i8_tiled.
+ */
+int bt_retile_fields(const uint8_t* W_tiled, int64_t N, int64_t K, uint8_t* W_fields, void* stream);
+int bt_ternary_gemm_i8_fields(const int8_t* Q, int q_layout, const float* s_x, const int32_t* q_rowsum,
+                              const uint8_t* W_fields, int tile_order, const void* scale, int scale_dtype,
+                              int64_t scale_len, const void* bias, int bias_dtype, const void* residual, void* Y,
+                              int y_dtype, int32_t* acc_out, int64_t B, int64_t N, int64_t K, void* stream);
 
 /*
  * G independent decode GEMVs in ONE launch (no counterpart in the reference, whose packed kernel

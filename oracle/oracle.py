@@ -152,6 +152,25 @@ def retile_weights(packed_t, in_features: int, gate_up_pairs: bool = False) -> n
     return tiled.reshape(-1)
 
 
+def retile_fields(tiled, out_features: int, in_features: int) -> np.ndarray:
+    """Field layout of a decode-tiled copy (a layout of this library for its prefill GEMM, no counterpart in the
+    reference).  Every aligned 16 bytes of the tiled copy are four dwords, one per column ``t`` of a column quad, with
+    the 2-bit code of ``k = 4 b + c`` at bits ``8 b + 2 c``.  The field layout keeps the group's place and stores, at
+    bits ``8 b + 2 t`` of dword ``c``, column ``t`` at ``k = 4 b + c``: as ``w + 1`` for ``t < 3`` (codes 0 / +1 / -1
+    become 1 / 2 / 0) and as ``w`` in two's complement for ``t = 3`` (0 / 1 / 3)."""
+    t8 = np.ascontiguousarray(tiled, dtype=np.uint8)
+    assert t8.size % 16 == 0 and t8.size == ((out_features + 15) // 16) * (((in_features + 3) // 4 + 15) // 16) * 256
+    grp = t8.reshape(-1, 4, 4)                                     # [group][column t][byte b]
+    codes = np.stack([(grp >> (2 * c)) & 3 for c in range(4)], axis=-1)  # [group][t][b][c]
+    remap_lo = np.array([1, 2, 0, 0], dtype=np.uint8)              # w + 1 (code 3 never occurs)
+    remap_hi = np.array([0, 1, 3, 0], dtype=np.uint8)              # two's complement
+    out = np.zeros((grp.shape[0], 4, 4), dtype=np.uint8)           # [group][dword c][byte b]
+    for t in range(4):
+        f = (remap_lo if t < 3 else remap_hi)[codes[:, t]]         # [group][b][c]
+        out |= (f.transpose(0, 2, 1) << (2 * t)).astype(np.uint8)
+    return out.reshape(-1)
+
+
 def _lin_args(x, w, scale, bias):
     x = _f32(x)
     scale = _f32(scale).reshape(-1)

@@ -24,7 +24,8 @@ def test_header_declares_expected_entry_points():
                  "bt_ternary_linear_packed_forward_res", "bt_ternary_gemm_i8_res", "bt_tiled_weights_bytes",
                  "bt_retile_weights", "bt_untile_weights", "bt_ternary_linear_tiled_forward", "bt_ternary_gemm_i8_tiled", "bt_swiglu", "bt_rmsnorm",
                  "bt_act_quant_i8_layout", "bt_ternary_linear_packed_forward_fused",
-                 "bt_packed_forward_fused_workspace_bytes"):
+                 "bt_packed_forward_fused_workspace_bytes", "bt_act_quant_i8_rowsum", "bt_retile_fields",
+                 "bt_ternary_gemm_i8_fields", "bt_ternary_gemm_i8_grouped", "bt_set_option"):
         assert name in syms
 
 
@@ -124,6 +125,17 @@ def test_tiled_copy_size_and_argument_checks_without_a_gpu():
     assert lib.bt_retile_weights(addr, 48, 64, 1, addr, None) == -1          # pair order needs N % 32 == 0
     assert "N % 32" in _lib.last_error()
     assert lib.bt_retile_weights(addr, 16, 64, 7, addr, None) == -1          # unknown tile order
+    # the prefill-only field layout: null row sums, K outside whole 128-wide stages, a misaligned copy
+    assert lib.bt_act_quant_i8_rowsum(addr, 0, 1, 16, addr, addr, None, 0, None) == -1
+    assert "bt_act_quant_i8_rowsum" in _lib.last_error()
+    assert lib.bt_retile_fields(addr, 16, 64, addr + 4, None) == -1
+    assert "aligned" in _lib.last_error()
+    assert lib.bt_ternary_gemm_i8_fields(addr, 0, addr, None, addr, 0, addr, 0, 1, None, 0, None, addr, 0, None, 4, 16, 128,
+                                         None) == -1
+    assert "q_rowsum" in _lib.last_error()
+    assert lib.bt_ternary_gemm_i8_fields(addr, 0, addr, addr, addr, 0, addr, 0, 1, None, 0, None, addr, 0, None, 4, 16, 192,
+                                         None) == -1
+    assert "multiple of 128" in _lib.last_error()
 
 
 def test_set_option_validates_names_and_lengths():

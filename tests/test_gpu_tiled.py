@@ -142,6 +142,139 @@ def test_tiled_int8_equals_row_major(oracle, n, k, route, monkeypatch):
             assert torch.equal(a1, a0) and torch.equal(y1, y0)
 
 
+# ---- the prefill-only field layout of the tiled copy ------------------------------------------------------------------
+@pytest.mark.parametrize("n,k", LAYOUT_SHAPES + [(520, 1024)])
+def test_field_layout_against_the_oracle(oracle, n, k):
+    """`retile_fields` byte for byte against the numpy restatement, on natural and pair-ordered tiled copies."""
+    from bittorch_amd import _C
+    announce("field layout", n, k)
+    _, wt = _packed(oracle, n, k, seed=n + 2 * k)
+    for pairs in ((False, True) if n % 32 == 0 else (False,)):
+        tiled = _C.retile_weights(wt, k, pairs)
+        fields = _C.retile_fields(tiled, k, n)
+        np.testing.assert_array_equal(fields.cpu().numpy(), oracle.retile_fields(tiled.cpu().numpy(), n, k))
+
+
+def test_act_quant_row_sums(oracle):
+    """The quantizer's third output: the rows' sums of q, with q and s_x unchanged, in both layouts and on both of its
+    kernels (rows in registers / the generic one for ragged K)."""
+    from bittorch_amd import _C
+    for (b, k, dtype) in [(5, 64, torch.float32), (33, 4096, torch.bfloat16), (7, 11008, torch.float16), (3, 100, torch.float32),
+                          (2, 20000, torch.bfloat16)]:
+        announce("row sums", b, k, dtype)
+        x = seeded_acts(b, k, seed=b + k, dtype=dtype, outliers=True).cuda()
+        for oo in ((False, True) if k % 16 == 0 else (False,)):
+            q0, s0 = _C.act_quant_int8(x, oo)
+            q, s, rs = _C.act_quant_int8(x, oo, return_rowsum=True)
+            assert torch.equal(q, q0) and torch.equal(s, s0)
+            assert rs.dtype == torch.int32 and torch.equal(rs, q.to(torch.int32).sum(dim=1, dtype=torch.int32))
+        oq, _ = oracle.act_quant_i8(f32np(x.cpu()))
+        np.testing.assert_array_equal(_C.act_quant_int8(x, False, return_rowsum=True)[2].cpu().numpy(), oq.astype(np.int64).sum(axis=1))
+
+
+# (M, N, K): whole tiles, ragged rows and columns, K of one to many whole stages, a launch that cuts its remainder finer
+# (320 and 128 tiles), and config 4's second shape
+FIELD_SHAPES = [(128, 256, 128), (100, 200, 256), (130, 260, 384), (257, 520, 1024), (40, 1028, 128), (4096, 2560, 256),
+                (1024, 4096, 128), (2048, 11008, 4096)]
+
+
+@pytest.mark.parametrize("m,n,k", FIELD_SHAPES)
+def test_field_layout_gemm_equals_tiled_gemm(oracle, m, n, k):
+    """The prefill GEMM on the field layout (one AND per operand dword, accumulators started at minus the rows' sums
+    of q, the factor 4^t taken out in the epilogue's multiplication): the int32 accumulators and the output bits of
+    the GEMM on the decode-tiled copy, with both activation layouts, bias, residual, every output type, natural and
+    pair-ordered copies; and the oracle's on row slices."""
+    from bittorch_amd import _C
+    set_option("STREAM_MAX_ROWS", "32")
+    _, wt = _packed(oracle, n, k, seed=(m + k) % 13)
+    g = torch.Generator().manual_seed(m + n + k)
+    scale = torch.rand(n, generator=g) * 0.05 + 0.01
+    bias = torch.randn(n, generator=g) * 0.01
+    x = seeded_acts(m, k, seed=m + k, dtype=torch.bfloat16, outliers=True)
+    res = seeded_acts(m, n, seed=m + 1, dtype=torch.bfloat16).cuda()
+    for pairs in ((False, True) if n % 32 == 0 and m <= 300 else (False,)):
+        tiled = _C.retile_weights(wt, k, pairs)
+        fields = _C.retile_fields(tiled, k, n)
+        ref_tiled = _C.retile_weights(wt, k)
+        for oo in (False, True):
+            announce("field layout gemm", m, n, k, pairs, oo)
+            q, sx, rs = _C.act_quant_int8(x.cuda(), oo, return_rowsum=True)
+            for out_dtype, r, b in ((torch.bfloat16, res, bias), (torch.float32, None, None), (torch.float16, None, bias)):
+                bb = None if b is None else b.cuda()
+                y0, a0 = _C.ternary_gemm_int8_tiled(q, sx, ref_tiled, scale.cuda(), bb, k, n, out_dtype, True, r, oo)
+                y0n = _C.ternary_gemm_int8_tiled(q, sx, ref_tiled, scale.cuda(), bb, k, n, out_dtype, False, r, oo)
+                y1, a1 = _C.ternary_gemm_int8_fields(q, sx, rs, fields, scale.cuda(), bb, k, n, out_dtype, True, r, oo, pairs)
+                y1n = _C.ternary_gemm_int8_fields(q, sx, rs, fields, scale.cuda(), bb, k, n, out_dtype, False, r, oo, pairs)
+                assert torch.equal(a1, a0) and torch.equal(y1, y0) and torch.equal(y1n, y0n)
+    q, sx, rs = _C.act_quant_int8(x.cuda(), False, return_rowsum=True)
+    fields = _C.retile_fields(_C.retile_weights(wt, k), k, n)
+    y1, a1 = _C.ternary_gemm_int8_fields(q, sx, rs, fields, scale.cuda(), bias.cuda(), k, n, torch.float32, True)
+    oq, os_ = oracle.act_quant_i8(f32np(x))
+    for lo, hi in ((0, min(m, 24)), (max(0, m - 24), m)):
+        oacc, oy = oracle.gemm_i8(oq[lo:hi], os_[lo:hi], wt.cpu().numpy(), f32np(scale), k, f32np(bias))
+        np.testing.assert_array_equal(a1[lo:hi].cpu().numpy(), oacc)
+        np.testing.assert_array_equal(y1[lo:hi].cpu().numpy(), oy)
+
+
+def test_layer_prefill_copy_is_opt_in_and_changes_no_bits(oracle):
+    """`prepare_prefill()` adds the field-layout copy; `forward_int8` with row sums and a prefill-sized batch runs on it
+    (natural and gate/up pair-ordered layers), gives the bits of the same call without it, is not used below the row
+    threshold or without row sums, stops being used when the layer is re-tiled, and `drop_prefill()` releases it."""
+    import bittorch_amd as bt
+    from bittorch_amd.nn import TernaryLinearInference
+    from bittorch_amd.nn.ternary_linear_infer import PREFILL_ROWS
+    n, k = 512, 1024
+    w = random_ternary(n, k, seed=77)
+    packed, _ = oracle.pack_ternary_transposed(w.numpy())
+    gen = torch.Generator().manual_seed(5)
+    mk = lambda: TernaryLinearInference(k, n, torch.from_numpy(packed), torch.rand(n, generator=gen) * 0.05 + 0.01,
+                                        torch.randn(n, generator=gen) * 0.01).cuda()
+    for order in ("natural", "gate_up_pairs"):
+        announce("layer prefill copy", order)
+        gen.manual_seed(5)
+        plain = mk()
+        gen.manual_seed(5)
+        layer = mk()
+        layer.tile_order = order
+        x = seeded_acts(PREFILL_ROWS + 40, k, seed=3, dtype=torch.bfloat16, outliers=True).cuda()
+        q, s, rs = bt.ops.act_quant_int8(x, True, return_rowsum=True)
+        want = plain.forward_int8(q, s, torch.bfloat16, None, True)
+        one_copy = layer.prepare_decode().resident_weight_bytes()
+        layer.prepare_prefill()
+        assert layer.resident_weight_bytes() == 2 * one_copy
+        assert torch.equal(layer.forward_int8(q, s, torch.bfloat16, None, True, q_rowsum=rs), want)
+        res = seeded_acts(x.shape[0], n, seed=4, dtype=torch.bfloat16).cuda()
+        assert torch.equal(layer.forward_int8(q, s, torch.bfloat16, res, True, q_rowsum=rs),
+                           plain.forward_int8(q, s, torch.bfloat16, res, True))
+        # too few rows, or no row sums: the usual route, the same bits
+        assert torch.equal(layer.forward_int8(q[:64], s[:64], torch.bfloat16, None, True, q_rowsum=rs[:64]), want[:64])
+        assert torch.equal(layer.forward_int8(q, s, torch.bfloat16, None, True), want)
+        # a wrong row-sum vector would show: the copy really is in use
+        assert not torch.equal(layer.forward_int8(q, s, torch.bfloat16, None, True, q_rowsum=rs + 1), want)
+        held = layer.resident_weight_bytes()  # (a pair-ordered layer holds weight_packed by now: its plain int8 calls need it)
+        layer.drop_prefill()
+        assert layer.resident_weight_bytes() == held - one_copy
+        assert torch.equal(layer.forward_int8(q, s, torch.bfloat16, None, True, q_rowsum=rs + 1), want)
+    # re-tiling (a tile order change) orphans the copy instead of reading stale bytes
+    gen.manual_seed(5)
+    layer = mk().prepare_prefill()
+    layer.tile_order = "gate_up_pairs"
+    layer.prepare_decode()
+    assert layer._prefill_copy() is None
+    assert torch.equal(layer.forward_int8(q, s, torch.bfloat16, None, True, q_rowsum=rs), want)
+
+
+def test_field_layout_gemm_argument_errors(oracle):
+    from bittorch_amd import _C
+    _, wt = _packed(oracle, 64, 192)
+    fields = _C.retile_fields(_C.retile_weights(wt, 192), 192, 64)
+    q, sx, rs = _C.act_quant_int8(torch.randn(4, 192, device="cuda"), False, return_rowsum=True)
+    with pytest.raises(RuntimeError, match="multiple of 128"):
+        _C.ternary_gemm_int8_fields(q, sx, rs, fields, torch.ones(64, device="cuda"), None, 192, 64)
+    with pytest.raises(RuntimeError, match="q_rowsum must be int32"):
+        _C.ternary_gemm_int8_fields(q, sx, rs.float(), fields, torch.ones(64, device="cuda"), None, 192, 64)
+
+
 # (M, N, K) whose 128 x 256 tiles leave most of a 256-unit chip idle in their last round, so that the launch cuts
 # the remainder finer: 320 tiles (256 whole + 64 as 256 tiles of 32 rows), 128 tiles (as 256 of 64 rows), 64 tiles (as
 # 256 of 32 rows); the same with ragged last row tiles, ragged columns and several stages of K

@@ -563,3 +563,30 @@ def test_epilogue_as_written_and_contracted_differ_by_one_ulp_at_most(oracle):
     z0 = oracle.linear_packed(x, packed, scale, k, None)
     z1 = oracle.linear_packed(x, packed, scale, k, None, fused_epilogue=True)
     np.testing.assert_array_equal(z0, z1)
+
+
+def test_field_layout_means_what_it_says(oracle):
+    """The field layout of the tiled copy, read back by its definition with plain loops: field t of byte b of dword c
+    of a group is column 4 q + t of the group's tile at k = 64 s + 16 g + 4 b + c, stored as w + 1 (t < 3) or as w in
+    two's complement (t = 3); positions outside the matrix read as weight 0."""
+    for (n, k) in ((20, 70), (16, 64), (37, 130)):
+        w = random_ternary(n, k, seed=n + k).numpy()
+        packed, _ = oracle.pack_ternary_transposed(w)
+        tiled = oracle.retile_weights(packed, k)
+        fields = oracle.retile_fields(tiled, n, k)
+        assert fields.dtype == np.uint8 and fields.size == tiled.size
+        steps, tiles = ((k + 3) // 4 + 15) // 16, (n + 15) // 16
+        f = fields.reshape(tiles, steps, 4, 4, 4, 4)   # [tile][step s][row group g][quad q][dword c][byte b]
+        for tile in range(tiles):
+            for s in range(steps):
+                for g in range(4):
+                    for q in range(4):
+                        for c in range(4):
+                            for b in range(4):
+                                byte = int(f[tile, s, g, q, c, b])
+                                for t in range(4):
+                                    field = (byte >> (2 * t)) & 3
+                                    got = field - 1 if t < 3 else (field if field < 2 else field - 4)
+                                    col, kk = 16 * tile + 4 * q + t, 64 * s + 16 * g + 4 * b + c
+                                    want = int(w[col, kk]) if col < n and kk < k else 0
+                                    assert got == want, (n, k, tile, s, g, q, c, b, t)
