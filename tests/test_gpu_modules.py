@@ -154,7 +154,7 @@ def test_autocast_contexts_mixed_nested_eval_and_batch_sizes():
 def test_gradient_consistency_over_seeds_shapes_and_double_precision():
     """tests/test_gradient_consistency.py:153-250: the kernels' gradients follow the torch backend's over several seeds
     and shapes, and the autograd function takes float64 operands (the reference runs gradcheck on it in double
-    precision and accepts either verdict: the straight-through estimator is not the derivative of the forward)."""
+    precision and accepts either outcome: the straight-through estimator is not the derivative of the forward)."""
     from bittorch_amd.nn.ternary_linear_cuda import TernaryLinearCUDAFunction
     announce("gradient consistency")
     for seed in (0, 1, 7, 42, 123):
@@ -187,9 +187,9 @@ def test_gradient_consistency_over_seeds_shapes_and_double_precision():
     y.sum().backward()
     assert x.grad.dtype == w.grad.dtype == bias.grad.dtype == torch.float64
     assert torch.equal(bias.grad, torch.full_like(bias, 2.0))
-    verdict = torch.autograd.gradcheck(lambda a, b_, c: TernaryLinearCUDAFunction.apply(a, b_, c, 0.05, True),
+    outcome = torch.autograd.gradcheck(lambda a, b_, c: TernaryLinearCUDAFunction.apply(a, b_, c, 0.05, True),
                                        (x, w, bias), eps=1e-4, atol=1e-3, rtol=1e-2, raise_exception=False)
-    assert verdict in (True, False)
+    assert outcome in (True, False)
 
 
 def test_half_and_bf16_modules():
