@@ -629,12 +629,14 @@ def _rows_2d(t: Tensor, K: int) -> Tensor:
     return t.contiguous().reshape(-1, K)
 
 
-def swiglu(gate: Tensor, up: Tensor, store: bool = True, quantize: bool = False, operand_order: bool = False):
+def swiglu(gate: Tensor, up: Tensor, store: bool = True, quantize: bool = False, operand_order: bool = False,
+           return_rowsum: bool = False):
     """``silu(gate) * up`` in one pass, rounded as the two separate torch ops round it.
 
     Returns the product (``store``), or with ``quantize`` its per-row int8 form ``(Q, s_x)`` for
     :func:`ternary_gemm_int8` -- ``(h, Q, s_x)`` when both are asked for.  ``gate`` and ``up`` may
-    be column slices of one wider matrix (the output of a fused gate/up projection)."""
+    be column slices of one wider matrix (the output of a fused gate/up projection).  ``return_rowsum`` (with
+    ``quantize``) appends the rows' sums of ``Q`` (int32), which :func:`ternary_gemm_int8_fields` needs."""
     _check(gate.shape == up.shape and gate.dtype == up.dtype, "gate and up must match in shape and dtype")
     _check(gate.dim() >= 1 and gate.numel() > 0, "gate is empty")
     _check(gate.dtype in _DT, "gate must be float32, float16 or bfloat16")
@@ -642,19 +644,29 @@ def swiglu(gate: Tensor, up: Tensor, store: bool = True, quantize: bool = False,
     K = gate.shape[-1]
     g2, u2 = _rows_2d(gate, K), _rows_2d(up, K)
     h, q, s = _row_op_outputs(g2, store, quantize)
+    rs = None
     with torch.cuda.device(gate.device):
-        _status(_L.bt_swiglu(g2.data_ptr(), g2.stride(0), u2.data_ptr(), u2.stride(0), _dt(g2, "gate"),
-                             g2.shape[0], K, _ptr(h), _ptr(q), _ptr(s), 1 if operand_order else 0, _stream(gate)))
+        if return_rowsum:
+            _check(q is not None, "return_rowsum needs quantize=True")
+            rs = torch.empty((g2.shape[0],), dtype=torch.int32, device=gate.device)
+            _status(_L.bt_swiglu_rowsum(g2.data_ptr(), g2.stride(0), u2.data_ptr(), u2.stride(0), _dt(g2, "gate"),
+                                        g2.shape[0], K, _ptr(h), _ptr(q), _ptr(s), rs.data_ptr(),
+                                        1 if operand_order else 0, _stream(gate)))
+        else:
+            _status(_L.bt_swiglu(g2.data_ptr(), g2.stride(0), u2.data_ptr(), u2.stride(0), _dt(g2, "gate"),
+                                 g2.shape[0], K, _ptr(h), _ptr(q), _ptr(s), 1 if operand_order else 0, _stream(gate)))
     if q is not None and gate.dim() != 2:
         q = q.reshape(*gate.shape[:-1], K)
         s = s.reshape(gate.shape[:-1])
-    return _row_op_result(h, q, s, gate.shape[:-1], K)
+    out = _row_op_result(h, q, s, gate.shape[:-1], K)
+    return out if rs is None else (*out, rs.reshape(gate.shape[:-1]))
 
 
 def rmsnorm(x: Tensor, weight: Optional[Tensor] = None, eps: float = 1e-6, store: bool = True,
-            quantize: bool = False, operand_order: bool = False):
+            quantize: bool = False, operand_order: bool = False, return_rowsum: bool = False):
     """RMSNorm over the last dimension, ``(x * rsqrt(mean(x^2) + eps)) * weight``; with
-    ``quantize`` also (or only, ``store=False``) the per-row int8 form of the result."""
+    ``quantize`` also (or only, ``store=False``) the per-row int8 form of the result, and with ``return_rowsum``
+    the rows' sums of that form appended (int32)."""
     _check(x.dim() >= 1 and x.numel() > 0, "x is empty")
     _check(x.dtype in _DT, "x must be float32, float16 or bfloat16")
     K = x.shape[-1]
@@ -664,13 +676,22 @@ def rmsnorm(x: Tensor, weight: Optional[Tensor] = None, eps: float = 1e-6, store
     _check(_all_cuda(x, weight), "All tensors must be CUDA")
     x2 = _rows_2d(x, K)
     h, q, s = _row_op_outputs(x2, store, quantize)
+    rs = None
     with torch.cuda.device(x.device):
-        _status(_L.bt_rmsnorm(x2.data_ptr(), x2.stride(0), _ptr(weight), float(eps), _dt(x2, "x"),
-                              x2.shape[0], K, _ptr(h), _ptr(q), _ptr(s), 1 if operand_order else 0, _stream(x)))
+        if return_rowsum:
+            _check(q is not None, "return_rowsum needs quantize=True")
+            rs = torch.empty((x2.shape[0],), dtype=torch.int32, device=x.device)
+            _status(_L.bt_rmsnorm_rowsum(x2.data_ptr(), x2.stride(0), _ptr(weight), float(eps), _dt(x2, "x"),
+                                         x2.shape[0], K, _ptr(h), _ptr(q), _ptr(s), rs.data_ptr(),
+                                         1 if operand_order else 0, _stream(x)))
+        else:
+            _status(_L.bt_rmsnorm(x2.data_ptr(), x2.stride(0), _ptr(weight), float(eps), _dt(x2, "x"),
+                                  x2.shape[0], K, _ptr(h), _ptr(q), _ptr(s), 1 if operand_order else 0, _stream(x)))
     if q is not None and x.dim() != 2:
         q = q.reshape(*x.shape[:-1], K)
         s = s.reshape(x.shape[:-1])
-    return _row_op_result(h, q, s, x.shape[:-1], K)
+    out = _row_op_result(h, q, s, x.shape[:-1], K)
+    return out if rs is None else (*out, rs.reshape(x.shape[:-1]))
 
 
 def unpack_dequant(W_T: Tensor, in_features: int, scale: Optional[Tensor] = None,

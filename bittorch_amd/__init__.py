@@ -19,5 +19,13 @@ except ImportError:
 
 
 def has_cuda_ext() -> bool:
-    """True when the HIP library is built and loadable (name kept from the reference)."""
+    """True when the HIP library is built and loadable (name kept from the reference).  A process that imported the
+    package before the library was built finds it here on the next call."""
+    global _HAS_CUDA_EXT
+    if not _HAS_CUDA_EXT:
+        try:
+            from . import _C  # noqa: F401
+            _HAS_CUDA_EXT = True
+        except ImportError:
+            pass
     return _HAS_CUDA_EXT

@@ -65,6 +65,8 @@ SIGNATURES = {
     "bt_ternary_gemm_i8_tiled": (_int, [_vp, _int, _vp, _vp, _vp, _int, _i64, _vp, _int, _vp, _vp, _int, _vp,
                                         _i64, _i64, _i64, _vp]),
     "bt_act_quant_i8_rowsum": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp, _int, _vp]),
+    "bt_swiglu_rowsum": (_int, [_vp, _i64, _vp, _i64, _int, _i64, _i64, _vp, _vp, _vp, _vp, _int, _vp]),
+    "bt_rmsnorm_rowsum": (_int, [_vp, _i64, _vp, ctypes.c_float, _int, _i64, _i64, _vp, _vp, _vp, _vp, _int, _vp]),
     "bt_retile_fields": (_int, [_vp, _i64, _i64, _vp, _vp]),
     "bt_ternary_gemm_i8_fields": (_int, [_vp, _int, _vp, _vp, _vp, _int, _vp, _int, _i64, _vp, _int, _vp, _vp, _int, _vp,
                                          _i64, _i64, _i64, _vp]),

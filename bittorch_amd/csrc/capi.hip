@@ -81,7 +81,8 @@ int launch_act_quant(const void* X, int x_dtype, int64_t B, int64_t K, int8_t* Q
 int launch_retile_fields(const uint8_t* W_tiled, int64_t N, int64_t K, uint8_t* W_fields, hipStream_t st);
 bool gemm_i8_supported(int64_t N, int64_t K, const void* Q, const void* W_T);
 int launch_row_op(int op, int dtype, const void* A, int64_t lda, const void* Bv, int64_t ldb, float eps, int64_t B,
-                  int64_t K, void* H, int8_t* Q, float* s_x, int q_layout, hipStream_t st, const char* who);
+                  int64_t K, void* H, int8_t* Q, float* s_x, int q_layout, int32_t* rowsum, hipStream_t st,
+                  const char* who);
 bool gemm_f16_supported(int64_t N, int64_t K, const void* X, const void* W_T, const void* Y);
 bool gemm_f16_supported_tiled(int64_t N, int64_t K, const void* X, const void* Y);
 int launch_gemm_f16(int mode, const void* X, const uint8_t* W_T, int w_layout, const Epilogue& epi, void* Y, int y_dtype,
@@ -689,7 +690,20 @@ extern "C" int bt_swiglu(const void* gate, int64_t ld_gate, const void* up, int6
         return BT_ERR_INVALID;
     }
     if (Q && (rc = check_q_layout(who, q_layout, K, Q, nullptr))) return rc;
-    return launch_row_op(0, dtype, gate, ld_gate, up, ld_up, 0.0f, B, K, H, Q, s_x, q_layout, (hipStream_t)stream, who);
+    return launch_row_op(0, dtype, gate, ld_gate, up, ld_up, 0.0f, B, K, H, Q, s_x, q_layout, nullptr, (hipStream_t)stream, who);
+}
+
+extern "C" int bt_swiglu_rowsum(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, int dtype, int64_t B,
+                                int64_t K, void* H, int8_t* Q, float* s_x, int32_t* q_rowsum, int q_layout, void* stream) {
+    const char* who = "bt_swiglu_rowsum";
+    int rc = check_row_op(who, gate, dtype, B, K, ld_gate, H, Q, s_x);
+    if (rc) return rc;
+    if (!up || ld_up < K || !Q || !q_rowsum) {
+        set_error("%s: up, Q or q_rowsum is null, or up's row stride is below K", who);
+        return BT_ERR_INVALID;
+    }
+    if ((rc = check_q_layout(who, q_layout, K, Q, nullptr))) return rc;
+    return launch_row_op(0, dtype, gate, ld_gate, up, ld_up, 0.0f, B, K, H, Q, s_x, q_layout, q_rowsum, (hipStream_t)stream, who);
 }
 
 extern "C" int bt_rmsnorm(const void* X, int64_t ld_x, const void* weight, float eps, int dtype, int64_t B,
@@ -698,7 +712,20 @@ extern "C" int bt_rmsnorm(const void* X, int64_t ld_x, const void* weight, float
     int rc = check_row_op(who, X, dtype, B, K, ld_x, Y, Q, s_x);
     if (rc) return rc;
     if (Q && (rc = check_q_layout(who, q_layout, K, Q, nullptr))) return rc;
-    return launch_row_op(1, dtype, X, ld_x, weight, 0, eps, B, K, Y, Q, s_x, q_layout, (hipStream_t)stream, who);
+    return launch_row_op(1, dtype, X, ld_x, weight, 0, eps, B, K, Y, Q, s_x, q_layout, nullptr, (hipStream_t)stream, who);
+}
+
+extern "C" int bt_rmsnorm_rowsum(const void* X, int64_t ld_x, const void* weight, float eps, int dtype, int64_t B,
+                                 int64_t K, void* Y, int8_t* Q, float* s_x, int32_t* q_rowsum, int q_layout, void* stream) {
+    const char* who = "bt_rmsnorm_rowsum";
+    int rc = check_row_op(who, X, dtype, B, K, ld_x, Y, Q, s_x);
+    if (rc) return rc;
+    if (!Q || !q_rowsum) {
+        set_error("%s: Q or q_rowsum is null", who);
+        return BT_ERR_INVALID;
+    }
+    if ((rc = check_q_layout(who, q_layout, K, Q, nullptr))) return rc;
+    return launch_row_op(1, dtype, X, ld_x, weight, 0, eps, B, K, Y, Q, s_x, q_layout, q_rowsum, (hipStream_t)stream, who);
 }
 
 // ---- packed forward with an activation prologue -----------------------------------------------
@@ -769,7 +796,7 @@ static int fused_forward_impl(const char* who, const void* X, int64_t ld_x, int 
         return BT_ERR_WORKSPACE;
     }
     rc = launch_row_op(pro_op == 2 ? 0 : 1, x_dtype, X, ld_x, pro_b, ld_b, eps, B, K, workspace, nullptr, nullptr,
-                       Q_ROW_MAJOR, st, who);
+                       Q_ROW_MAJOR, nullptr, st, who);
     if (rc) return rc;
     return packed_forward_impl(who, workspace, x_dtype, W_T, w_layout, epi_op, scale, scale_dtype, scale_len, bias, bias_dtype,
                                residual, Y, B, N, K, (uint8_t*)workspace + h_bytes, workspace_bytes - h_bytes, stream);

@@ -26,6 +26,7 @@ struct RowOpParams {
     void* H;            // optional [B, K] output in the input dtype
     int8_t* Q;          // optional [B, K] int8 output (with s_x)
     float* s_x;         // [B]
+    int32_t* rowsum;    // optional [B]: the rows' sums of Q (for the field-layout prefill GEMM)
     float eps;
     int K;
     int q_layout;       // Q_ROW_MAJOR / Q_OPERAND_ORDER (K % 16 == 0)
@@ -144,18 +145,28 @@ __global__ __launch_bounds__(256) void row_op_kernel(RowOpParams p) {
     const float s = (amax > 1e-6f) ? __fdiv_rn(amax, 127.0f) : 1.0f;
     const float inv = __fdiv_rn(1.0f, s);
     if (tid == 0) p.s_x[row] = s;
+    int qsum = 0;
 #pragma unroll
     for (int i = 0; i < ITERS; i++) {
         const int k = (i * 256 + tid) * 8;
         uint32_t lo = 0, hi = 0;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            const uint32_t byte = (uint32_t)(uint8_t)quant_i8(v[i][e], inv);
+            const int8_t qv = quant_i8(v[i][e], inv);
+            if (k < K) qsum += (int)qv;
+            const uint32_t byte = (uint32_t)(uint8_t)qv;
             if (e < 4) lo |= byte << (8 * e);
             else hi |= byte << (8 * (e - 4));
         }
         const uint2 o = p.q_layout == Q_OPERAND_ORDER ? q_to_operand_order(lo, hi, tid & 1) : make_uint2(lo, hi);
         if (k < K) st2_nt(p.Q + row * (int64_t)K + k, o.x, o.y);
+    }
+    if (p.rowsum) {  // (uniform)
+        __shared__ int part_i[4];
+        qsum = wave_sum_i32(qsum);
+        if ((tid & 63) == 0) part_i[tid >> 6] = qsum;
+        __syncthreads();
+        if (tid == 0) p.rowsum[row] = (part_i[0] + part_i[1]) + (part_i[2] + part_i[3]);
     }
 }
 
@@ -198,9 +209,19 @@ __global__ __launch_bounds__(256) void row_op_generic_kernel(RowOpParams p) {
     const float s = (amax > 1e-6f) ? __fdiv_rn(amax, 127.0f) : 1.0f;
     const float inv = __fdiv_rn(1.0f, s);
     if (tid == 0) p.s_x[row] = s;
+    int qsum = 0;
     for (int k = tid; k < K; k += 256) {
         const int64_t pos = p.q_layout == Q_OPERAND_ORDER ? q_operand_order_pos(k) : k;
-        p.Q[row * (int64_t)K + pos] = quant_i8(value(k), inv);
+        const int8_t qv = quant_i8(value(k), inv);
+        qsum += (int)qv;
+        p.Q[row * (int64_t)K + pos] = qv;
+    }
+    if (p.rowsum) {  // (uniform)
+        __shared__ int part_i[4];
+        qsum = wave_sum_i32(qsum);
+        if ((tid & 63) == 0) part_i[tid >> 6] = qsum;
+        __syncthreads();
+        if (tid == 0) p.rowsum[row] = (part_i[0] + part_i[1]) + (part_i[2] + part_i[3]);
     }
 }
 
@@ -227,9 +248,10 @@ static void launch_row_op_dt(const RowOpParams& p, int64_t B, bool fast, hipStre
 
 // op: ROW_SWIGLU / ROW_RMSNORM.  The callers have checked pointers, shapes and dtypes.
 int launch_row_op(int op, int dtype, const void* A, int64_t lda, const void* Bv, int64_t ldb, float eps, int64_t B,
-                  int64_t K, void* H, int8_t* Q, float* s_x, int q_layout, hipStream_t st, const char* who) {
+                  int64_t K, void* H, int8_t* Q, float* s_x, int q_layout, int32_t* rowsum, hipStream_t st,
+                  const char* who) {
     RowOpParams p;
-    p.A = A; p.Bv = Bv; p.lda = lda; p.ldb = ldb; p.H = H; p.Q = Q; p.s_x = s_x; p.eps = eps; p.K = (int)K;
+    p.A = A; p.Bv = Bv; p.lda = lda; p.ldb = ldb; p.H = H; p.Q = Q; p.s_x = s_x; p.rowsum = Q ? rowsum : nullptr; p.eps = eps; p.K = (int)K;
     p.q_layout = q_layout;
     const int es = dtype_size(dtype);
     auto aligned = [&](const void* ptr, int64_t ld) { return !ptr || (((uintptr_t)ptr) % 16 == 0 && (ld * es) % 16 == 0); };

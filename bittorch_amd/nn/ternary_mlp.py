@@ -61,11 +61,30 @@ class TernarySwiGLU(nn.Module):
         gu = self.gate_up(h, None, norm)
         return gu[..., :self.ffn], gu[..., self.ffn:]
 
-    def _gate_up_int8(self, q: Tensor, s: Tensor, dtype, oo: bool):
+    def _gate_up_int8(self, q: Tensor, s: Tensor, dtype, oo: bool, rs: Optional[Tensor] = None):
         if self.gate_up is None:
-            return (self.gate.forward_int8(q, s, dtype, None, oo), self.up.forward_int8(q, s, dtype, None, oo))
-        gu = self.gate_up.forward_int8(q, s, dtype, None, oo)
+            return (self.gate.forward_int8(q, s, dtype, None, oo, rs), self.up.forward_int8(q, s, dtype, None, oo, rs))
+        gu = self.gate_up.forward_int8(q, s, dtype, None, oo, rs)
         return gu[..., :self.ffn], gu[..., self.ffn:]
+
+    def _linears(self):
+        return [m for m in (self.gate_up, self.gate, self.up, self.down) if m is not None]
+
+    def prepare_prefill(self) -> "TernarySwiGLU":
+        """``TernaryLinearInference.prepare_prefill()`` on every projection (a second, prefill-only copy of the weights
+        each): the int8 compute mode then hands its quantizers' row sums to the GEMMs of prefill-sized batches."""
+        for m in self._linears():
+            m.prepare_prefill()
+        return self
+
+    def drop_prefill(self) -> "TernarySwiGLU":
+        for m in self._linears():
+            m.drop_prefill()
+        return self
+
+    def _wants_rowsum(self, rows: int) -> bool:
+        from .ternary_linear_infer import PREFILL_ROWS
+        return rows >= PREFILL_ROWS and any(m._prefill_copy() is not None for m in self._linears())
 
     def forward(self, x: Tensor, norm_weight: Optional[Tensor] = None, eps: Optional[float] = None,
                 residual: Optional[Tensor] = None) -> Tensor:
@@ -88,10 +107,12 @@ class TernarySwiGLU(nn.Module):
             return self.down(g, residual, None, u)
         # the int8 activations stay inside this call: hand them over in the matrix cores' own order
         oo1, oo2 = x.shape[-1] % 16 == 0, self.ffn % 16 == 0
+        # row sums of the quantized activations ride along where a projection holds a prefill copy that wants them
+        want = self._wants_rowsum(x.numel() // max(x.shape[-1], 1))
         if eps is None:
-            q, s = fused.act_quant_int8(x, oo1)
+            q, s, *rs = fused.act_quant_int8(x, oo1, return_rowsum=want)
         else:
-            q, s = fused.rmsnorm(x, norm_weight, eps, store=False, quantize=True, operand_order=oo1)
-        g, u = self._gate_up_int8(q, s, x.dtype, oo1)
-        q2, s2 = fused.swiglu(g, u, store=False, quantize=True, operand_order=oo2)
-        return self.down.forward_int8(q2, s2, x.dtype, residual, oo2)
+            q, s, *rs = fused.rmsnorm(x, norm_weight, eps, store=False, quantize=True, operand_order=oo1, return_rowsum=want)
+        g, u = self._gate_up_int8(q, s, x.dtype, oo1, rs[0] if rs else None)
+        q2, s2, *rs2 = fused.swiglu(g, u, store=False, quantize=True, operand_order=oo2, return_rowsum=want)
+        return self.down.forward_int8(q2, s2, x.dtype, residual, oo2, rs2[0] if rs2 else None)

@@ -22,17 +22,18 @@ import torch
 from torch import Tensor
 
 
-def swiglu(gate: Tensor, up: Tensor, store: bool = True, quantize: bool = False, operand_order: bool = False):
+def swiglu(gate: Tensor, up: Tensor, store: bool = True, quantize: bool = False, operand_order: bool = False,
+           return_rowsum: bool = False):
     from .. import _C
 
-    return _C.swiglu(gate, up, store, quantize, operand_order)
+    return _C.swiglu(gate, up, store, quantize, operand_order, return_rowsum)
 
 
 def rmsnorm(x: Tensor, weight: Optional[Tensor] = None, eps: float = 1e-6, store: bool = True,
-            quantize: bool = False, operand_order: bool = False):
+            quantize: bool = False, operand_order: bool = False, return_rowsum: bool = False):
     from .. import _C
 
-    return _C.rmsnorm(x, weight, eps, store, quantize, operand_order)
+    return _C.rmsnorm(x, weight, eps, store, quantize, operand_order, return_rowsum)
 
 
 def act_quant_int8(x: Tensor, operand_order: bool = False, return_rowsum: bool = False):

@@ -31,6 +31,7 @@ class BlockStack:
 
         self.torch, self.F, self.bt = torch, F, bt
         self.attn_scale = attn_scale
+        self.prefill_copy = False  # prepare_prefill(): the int8 path on the layers' field-layout copies
         std_of = (lambda name: master_std.get(name, 0.02)) if isinstance(master_std, dict) else (lambda name: master_std)
         self.d_model, self.heads, self.ffn = d_model, heads, ffn
         act_dtype = act_dtype or torch.bfloat16
@@ -118,20 +119,32 @@ class BlockStack:
         heads_of = lambda t: t.view(b, s, heads, -1).transpose(1, 2)
         if int8:  # BitNet-style: every projection on the int8 matrix cores from activations that leave the
             # norm / SwiGLU kernels already quantized per token
-            qh, sh = fused.rmsnorm(x, blk.n1.weight, blk.n1.eps or torch.finfo(x.dtype).eps, store=False, quantize=True,
-                                   operand_order=True)
-            qkv = blk.qkv.forward_int8(qh, sh, x.dtype, None, True)
+            # (row sums of the quantized rows ride along where the layers hold a prefill copy: prepare_prefill)
+            pre = self.prefill_copy
+            qh, sh, *rs = fused.rmsnorm(x, blk.n1.weight, blk.n1.eps or torch.finfo(x.dtype).eps, store=False, quantize=True,
+                                        operand_order=True, return_rowsum=pre)
+            qkv = blk.qkv.forward_int8(qh, sh, x.dtype, None, True, rs[0] if rs else None)
         else:
             qkv = blk.qkv(fused.rmsnorm(x, blk.n1.weight, blk.n1.eps or torch.finfo(x.dtype).eps))
         q, k, v = qkv.split(d_model, dim=-1)  # one GEMM over the concatenated q|k|v columns
         a = F.scaled_dot_product_attention(heads_of(q), heads_of(k), heads_of(v), is_causal=True, scale=self.attn_scale)
         a = a.transpose(1, 2).reshape(b, s, -1)
         if int8:
-            qa, sa = bt._C.act_quant_int8(a.reshape(b * s, -1), True)
-            x = blk.o.forward_int8(qa, sa, x.dtype, x.reshape(b * s, -1), True).view(b, s, -1)
+            qa, sa, *rs = bt._C.act_quant_int8(a.reshape(b * s, -1), True, self.prefill_copy)
+            x = blk.o.forward_int8(qa, sa, x.dtype, x.reshape(b * s, -1), True, rs[0] if rs else None).view(b, s, -1)
         else:
             x = blk.o(a, x)
         return blk.mlp(x, blk.n2.weight, blk.n2.eps or torch.finfo(x.dtype).eps, residual=x)
+
+    def prepare_prefill(self, on: bool = True):
+        """Give every fused inference layer its prefill-only second weight copy (or release it): the int8 path then
+        runs its GEMMs on the field layout, with the same results."""
+        self.prefill_copy = bool(on)
+        for blk in self.infer:
+            for m in (blk.qkv, blk.o):
+                m.prepare_prefill() if on else m.drop_prefill()
+            blk.mlp.prepare_prefill() if on else blk.mlp.drop_prefill()
+        return self
 
     def forward_fused(self, int8):
         """The converted stack with the glue between the ternary layers fused: residual adds in the GEMM

@@ -209,6 +209,12 @@ int bt_swiglu(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, 
               int64_t K, void* H, int8_t* Q, float* s_x, int q_layout, void* stream);
 int bt_rmsnorm(const void* X, int64_t ld_x, const void* weight, float eps, int dtype, int64_t B,
                int64_t K, void* Y, int8_t* Q, float* s_x, int q_layout, void* stream);
+/* The same with Q required and q_rowsum [B] int32, the rows' sums of Q, as a further output (for
+ * bt_ternary_gemm_i8_fields; see bt_act_quant_i8_rowsum). */
+int bt_swiglu_rowsum(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, int dtype, int64_t B,
+                     int64_t K, void* H, int8_t* Q, float* s_x, int32_t* q_rowsum, int q_layout, void* stream);
+int bt_rmsnorm_rowsum(const void* X, int64_t ld_x, const void* weight, float eps, int dtype, int64_t B,
+                      int64_t K, void* Y, int8_t* Q, float* s_x, int32_t* q_rowsum, int q_layout, void* stream);
 
 /*
  * Packed forward with an activation prologue (no counterpart in the reference's Python/CUDA code;

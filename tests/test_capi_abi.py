@@ -25,7 +25,8 @@ def test_header_declares_expected_entry_points():
                  "bt_retile_weights", "bt_untile_weights", "bt_ternary_linear_tiled_forward", "bt_ternary_gemm_i8_tiled", "bt_swiglu", "bt_rmsnorm",
                  "bt_act_quant_i8_layout", "bt_ternary_linear_packed_forward_fused",
                  "bt_packed_forward_fused_workspace_bytes", "bt_act_quant_i8_rowsum", "bt_retile_fields",
-                 "bt_ternary_gemm_i8_fields", "bt_ternary_gemm_i8_grouped", "bt_set_option"):
+                 "bt_ternary_gemm_i8_fields", "bt_ternary_gemm_i8_grouped", "bt_set_option", "bt_swiglu_rowsum",
+                 "bt_rmsnorm_rowsum"):
         assert name in syms
 
 
@@ -136,6 +137,11 @@ def test_tiled_copy_size_and_argument_checks_without_a_gpu():
     assert lib.bt_ternary_gemm_i8_fields(addr, 0, addr, addr, addr, 0, addr, 0, 1, None, 0, None, addr, 0, None, 4, 16, 192,
                                          None) == -1
     assert "multiple of 128" in _lib.last_error()
+    # the fused quantizers' row-sum variants need both the codes and the sums
+    assert lib.bt_swiglu_rowsum(addr, 16, addr, 16, 1, 1, 16, None, addr, addr, None, 0, None) == -1
+    assert "bt_swiglu_rowsum" in _lib.last_error() and "q_rowsum" in _lib.last_error()
+    assert lib.bt_rmsnorm_rowsum(addr, 16, None, 1e-5, 1, 1, 16, None, None, addr, addr, 0, None) == -1
+    assert "bt_rmsnorm_rowsum" in _lib.last_error()
 
 
 def test_set_option_validates_names_and_lengths():

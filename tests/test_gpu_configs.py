@@ -266,3 +266,28 @@ def test_config5_block_element_wise_with_every_branch_of_order_one():
     # tensors and the truth fp32 ones (a step of amax/127 each), hence four times the bound
     ref_q = with_masters(BlockStack(dev, backend="python", act_dtype=torch.float32, fake_quant=True, **kw)).forward()
     check("int8 path", y_int8, ref_q, tol=8e-2)
+
+
+def test_config5_int8_stack_on_prefill_copies_changes_no_bits():
+    """BlockStack.prepare_prefill(): every fused layer of the full-size block gets its field-layout copy, the norm /
+    SwiGLU / activation quantizers hand the rows' sums to the GEMMs, and the int8 path's output is the same tensor,
+    bit for bit, as on the decode layout alone; releasing the copies gives the weight bytes back."""
+    from bittorch_amd.utils.block_stack import BlockStack
+    dev = torch.device("cuda:0")
+    announce("config 5 int8 path, prefill copies")
+    c5 = BlockStack(dev, layers=1)
+    c5.convert()
+    c5.fuse()
+    layers = lambda: [m for blk in c5.infer for m in (blk.qkv, blk.o, *blk.mlp._linears())]
+    y0 = c5.forward_fused(True)
+    bytes0 = sum(m.resident_weight_bytes() for m in layers())
+    c5.prepare_prefill(True)
+    assert all(m._prefill_copy() is not None for m in layers())
+    assert sum(m.resident_weight_bytes() for m in layers()) > bytes0
+    y1 = c5.forward_fused(True)
+    assert torch.equal(y1, y0)
+    # the float path never looks at the copies
+    yf = c5.forward_fused(False)
+    c5.prepare_prefill(False)
+    assert sum(m.resident_weight_bytes() for m in layers()) == bytes0
+    assert torch.equal(c5.forward_fused(False), yf) and torch.equal(c5.forward_fused(True), y0)

@@ -453,3 +453,61 @@ def test_rmsnorm_prologue_without_weight_gives_the_same_bits_with_and_without_wo
         torch.cuda.synchronize()
         outs.append(y)
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], ref)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("b,k", [(1, 16), (5, 528), (16, 4096), (3, 6912), (2, 16384), (2, 20000), (3, 7)])
+def test_fused_quantizers_return_the_row_sums_of_their_codes(dtype, b, k):
+    """SwiGLU and RMSNorm with the per-row quantizer can also write, per row, the sum of the int8 codes they emit (what
+    the prefill copy's GEMM starts its accumulators from): equal to summing the stored codes, in both storage orders,
+    on the register kernel and on the generic one, and nothing else of the result changes."""
+    from bittorch_amd import _C
+    announce("row sums of the fused quantizers", dtype, b, k)
+    g = (seeded_acts(b, k, seed=b + k, dtype=dtype, outliers=True) * 3).cuda()
+    u = seeded_acts(b, k, seed=b + k + 1, dtype=dtype).cuda()
+    if b > 2:
+        u[1] = 0
+    w = (1 + 0.1 * torch.randn(k, generator=torch.Generator().manual_seed(k))).to(dtype).cuda()
+    for oo in ([False, True] if k % 16 == 0 else [False]):
+        q, s = _C.swiglu(g, u, store=False, quantize=True, operand_order=oo)
+        q1, s1, rs = _C.swiglu(g, u, store=False, quantize=True, operand_order=oo, return_rowsum=True)
+        assert rs.dtype == torch.int32 and rs.shape == (b,)
+        assert torch.equal(q1, q) and torch.equal(s1, s)
+        assert torch.equal(rs, q.view(b, -1).to(torch.int32).sum(1, dtype=torch.int32))
+        h, q2, s2, rs2 = _C.swiglu(g, u, store=True, quantize=True, operand_order=oo, return_rowsum=True)
+        assert torch.equal(q2, q) and torch.equal(rs2, rs) and torch.equal(h, _C.swiglu(g, u))
+        q, s = _C.rmsnorm(g, w, 1e-5, store=False, quantize=True, operand_order=oo)
+        q1, s1, rs = _C.rmsnorm(g, w, 1e-5, store=False, quantize=True, operand_order=oo, return_rowsum=True)
+        assert torch.equal(q1, q) and torch.equal(s1, s)
+        assert torch.equal(rs, q.view(b, -1).to(torch.int32).sum(1, dtype=torch.int32))
+    # row sums belong to the quantizer: without it there is nothing to sum
+    with pytest.raises(RuntimeError, match="return_rowsum needs quantize"):
+        _C.swiglu(g, u, store=True, quantize=False, return_rowsum=True)
+
+
+@pytest.mark.parametrize("fuse_gate_up", [False, True])
+def test_swiglu_module_with_prefill_copies_changes_no_bits(fuse_gate_up):
+    """TernarySwiGLU.prepare_prefill(): every projection gets its field-layout copy, the quantizers hand their row
+    sums on, and prefill-sized batches run on the copies: the same bits as without, with and without the norm, and
+    decode-sized batches never touch the copies."""
+    import bittorch_amd as bt
+    from bittorch_amd.nn.ternary_linear_infer import PREFILL_ROWS
+    announce("TernarySwiGLU prefill copies", fuse_gate_up)
+    d, ffn = 512, 1280
+    mk = lambda i, o, seed: bt.nn.create_ternary_linear_inference(
+        i, o, (torch.randn(o, i, generator=torch.Generator().manual_seed(seed)) * 0.02).cuda())
+    mlp = bt.nn.TernarySwiGLU(mk(d, ffn, 1), mk(d, ffn, 2), mk(ffn, d, 3), compute="int8", fuse_gate_up=fuse_gate_up)
+    nw = (1 + 0.1 * torch.randn(d, generator=torch.Generator().manual_seed(4))).bfloat16().cuda()
+    xs = {rows: seeded_acts(rows, d, seed=rows, dtype=torch.bfloat16).cuda() for rows in (PREFILL_ROWS + 37, 24)}
+    ref = {rows: (mlp(x, nw, 1e-5, residual=x), mlp(x)) for rows, x in xs.items()}
+    before = sum(m.resident_weight_bytes() for m in mlp._linears())
+    assert mlp.prepare_prefill() is mlp
+    assert all(m._prefill_copy() is not None for m in mlp._linears())
+    assert sum(m.resident_weight_bytes() for m in mlp._linears()) > before
+    assert mlp._wants_rowsum(PREFILL_ROWS) and not mlp._wants_rowsum(PREFILL_ROWS - 1)
+    for rows, x in xs.items():
+        assert torch.equal(mlp(x, nw, 1e-5, residual=x), ref[rows][0])
+        assert torch.equal(mlp(x), ref[rows][1])
+    mlp.drop_prefill()
+    assert not mlp._wants_rowsum(PREFILL_ROWS) and sum(m.resident_weight_bytes() for m in mlp._linears()) == before
+    assert torch.equal(mlp(xs[24]), ref[24][1])
