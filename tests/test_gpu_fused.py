@@ -511,3 +511,35 @@ def test_swiglu_module_with_prefill_copies_changes_no_bits(fuse_gate_up):
     mlp.drop_prefill()
     assert not mlp._wants_rowsum(PREFILL_ROWS) and sum(m.resident_weight_bytes() for m in mlp._linears()) == before
     assert torch.equal(mlp(xs[24]), ref[24][1])
+
+
+def test_swiglu_module_on_prefill_copies_replays_in_a_graph():
+    """The int8 MLP on its prefill copies (row sums from the RMSNorm and SwiGLU quantizers, GEMMs on the field layout)
+    captured once and replayed on new inputs, with eager work between the replays: every replay equals the eager call."""
+    import bittorch_amd as bt
+    from bittorch_amd.nn.ternary_linear_infer import PREFILL_ROWS
+    announce("TernarySwiGLU prefill copies under graph replay")
+    d, ffn, rows = 512, 1280, PREFILL_ROWS + 128
+    mk = lambda i, o, seed: bt.nn.create_ternary_linear_inference(
+        i, o, (torch.randn(o, i, generator=torch.Generator().manual_seed(seed)) * 0.02).cuda())
+    mlp = bt.nn.TernarySwiGLU(mk(d, ffn, 1), mk(d, ffn, 2), mk(ffn, d, 3), compute="int8", fuse_gate_up=True).prepare_prefill()
+    nw = (1 + 0.1 * torch.randn(d, generator=torch.Generator().manual_seed(4))).bfloat16().cuda()
+    xs = [seeded_acts(rows, d, seed=s_, dtype=torch.bfloat16, outliers=True).cuda() for s_ in (11, 12, 13)]
+    eager = [mlp(xi, nw, 1e-5, residual=xi) for xi in xs]
+    x = xs[0].clone()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        mlp(x, nw, 1e-5, residual=x)  # warm-up on a side stream, as torch asks before a capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = mlp(x, nw, 1e-5, residual=x)
+    for xi, want in zip(xs, eager):
+        _ = mlp(xi[:24], nw, 1e-5)  # eager work between the replays (a decode-sized call on the same layers)
+        x.copy_(xi)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want)
