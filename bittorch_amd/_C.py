@@ -290,8 +290,10 @@ def ternary_linear_tiled_forward(X: Tensor, W_tiled: Tensor, scale: Tensor, bias
                                  norm: Optional[Tuple[Optional[Tensor], float]] = None,
                                  swiglu_up: Optional[Tensor] = None, swiglu_pairs: bool = False,
                                  natural_from_pairs: bool = False) -> Tensor:
-    """:func:`ternary_linear_packed_forward` / ``_fused`` on the decode-tiled copy of the weights (same
-    results bit for bit); the weights are streamed once per 16 rows of ``X``, so this is for decode shapes.
+    """:func:`ternary_linear_packed_forward` / ``_fused`` on the decode-tiled copy of the weights: the same results
+    bit for bit wherever both layouts take the same kernel -- always up to 32 rows; the rule that hands larger
+    batches to the tiled GEMM prices a tiled launch's remainder lower, so a batch near the crossover may stream on one
+    layout and run the GEMM on the other, with fp32 sums that differ in their last bits.
     ``swiglu_pairs`` (copy built with ``gate_up_pairs=True``): the layer's columns are ``[gate | up]`` and the
     output is the MLP's hidden vector ``swiglu(gate(x), up(x))`` ``[*, N/2]``, formed in the kernel's output stage.
     ``natural_from_pairs``: the same pair-ordered copy read as an ordinary linear layer (output ``[*, N]`` in natural

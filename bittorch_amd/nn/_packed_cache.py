@@ -6,7 +6,11 @@ The result depends on the weights only, so a forward that cannot be a training s
 mode off, or frozen weights) keeps it until the weights change: the key is the parameter's
 version counter (every tracked in-place update, ``load_state_dict`` or optimizer step bumps it),
 its storage address, dtype and device, and the quantizer's two settings.  Such a forward then
-reads K*N/4 bytes of packed weights instead of 4*K*N bytes of masters.
+reads K*N/4 bytes of packed weights instead of 4*K*N bytes of masters -- and reads them from a decode-tiled copy
+built next to the packed bytes (``_C.retile_weights``; whole-cache-line loads: what ``TernaryLinearInference`` runs
+on), which such a module then holds as well, another K*N/4 bytes.  Up to 32 rows the output is the training forward's
+bit for bit; a larger batch may be routed to another kernel on the tiled copy than on the row-major bytes, and the two
+sum in fp32 in different orders (a difference in the last bits of the sums).
 
 A training forward (gradient mode on and ``weight.requires_grad``) never uses the cache and
 quantizes every time, exactly as the reference does: training code is where weights get written
@@ -29,10 +33,12 @@ class PackedWeightCache:
 
     def __init__(self) -> None:
         self.key = None
-        self.value: Optional[Tuple[Tensor, Tensor]] = None
+        self.value: Optional[Tuple[Tensor, Tensor, Optional[Tensor]]] = None
 
-    def get(self, weight: Tensor, threshold_factor: float, per_channel: bool) -> Tuple[Tensor, Tensor]:
-        """``(packed_T uint8 [ceil(K/4), N], scale fp32 [N] or 0-dim)`` of the current weights."""
+    def get(self, weight: Tensor, threshold_factor: float, per_channel: bool) -> Tuple[Tensor, Tensor, Optional[Tensor]]:
+        """``(packed_T uint8 [ceil(K/4), N], scale fp32 [N] or 0-dim, tiled)`` of the current weights; ``tiled`` is
+        the decode-tiled copy of ``packed_T`` (``_C.retile_weights``), or None where the tiled kernels' 32-bit
+        offsets do not reach."""
         from .. import _C
 
         key = (weight._version, weight.data_ptr(), weight.dtype, weight.device, float(threshold_factor),
@@ -40,7 +46,10 @@ class PackedWeightCache:
         if key != self.key:
             with torch.no_grad():
                 packed, scale, _ = _C.ternary_quantize_pack(weight.detach(), threshold_factor, per_channel)
-            self.key, self.value = key, (packed, scale)
+                n, k = weight.shape
+                tiled_bytes = ((n + 15) // 16) * ((((k + 3) // 4) + 15) // 16) * 256
+                tiled = _C.retile_weights(packed, k) if tiled_bytes < 2 ** 32 else None
+            self.key, self.value = key, (packed, scale, tiled)
         return self.value
 
     def clear(self) -> None:

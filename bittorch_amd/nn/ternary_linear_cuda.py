@@ -10,6 +10,7 @@ bytes instead of being kept alive from the forward.
 
 from __future__ import annotations
 
+import os
 from typing import Optional, Tuple
 
 import torch
@@ -28,7 +29,7 @@ class TernaryLinearCUDAFunction(torch.autograd.Function):
     @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.float16)
     def forward(ctx, x: Tensor, weight: Tensor, bias: Optional[Tensor], threshold_factor: float,
                 per_channel: bool, cached=None) -> Tensor:
-        """``cached``: optional ``(packed_T, scale)`` of exactly these weights (see
+        """``cached``: optional ``(packed_T, scale, tiled copy or None)`` of exactly these weights (see
         ``_packed_cache.py``); the quantize+pack kernel is skipped when it is given."""
         from .. import _C
 
@@ -40,13 +41,19 @@ class TernaryLinearCUDAFunction(torch.autograd.Function):
             packed = None
             ctx.w_eff = w_tern * scale.reshape(-1, 1)
         else:
+            tiled = None
             if cached is not None:
-                packed, scale = cached
+                packed, scale, tiled = cached
             else:
                 packed, scale, _ = _C.ternary_quantize_pack(weight, threshold_factor, per_channel)
-            out = _C.ternary_linear_packed_forward(
-                x.contiguous(), packed, scale.reshape(-1).to(x.dtype),
-                None if bias is None else bias.to(x.dtype).contiguous(), weight.shape[1])
+            b = None if bias is None else bias.to(x.dtype).contiguous()
+            if (tiled is not None and x.dtype in (torch.float16, torch.bfloat16, torch.float32)
+                    and os.environ.get("BITTORCH_KERNEL") != "generic"):  # (the shape-generic kernel reads packed_T)
+                out = _C.ternary_linear_tiled_forward(x.contiguous(), tiled, scale.reshape(-1).to(x.dtype), b,
+                                                      weight.shape[1], weight.shape[0])
+            else:
+                out = _C.ternary_linear_packed_forward(x.contiguous(), packed, scale.reshape(-1).to(x.dtype), b,
+                                                       weight.shape[1])
             ctx.w_eff = None
         ctx.save_for_backward(x, packed, scale)
         ctx.in_features = weight.shape[1]

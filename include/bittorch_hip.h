@@ -253,7 +253,10 @@ int bt_ternary_linear_packed_forward_fused(const void* X, int64_t ld_x, int x_dt
  *   bt_ternary_linear_tiled_forward: bt_ternary_linear_packed_forward_fused on the tiled copy, with
  *     pro_op = BT_PRO_NONE allowed (then ld_x must equal K); the weights are streamed once per 16
  *     rows of X, so it is meant for decode shapes; fp32 X needs the workspace.
- *     Results equal those of the row-major entry points bit for bit.
+ *     Results equal those of the row-major entry points bit for bit wherever both layouts take the same kernel
+ *     (always up to 32 rows); a larger batch near the crossover between the streaming kernel and the tiled GEMM
+ *     may be routed differently on the tiled copy (its remainder tiles are cheaper), and the two kernels add the
+ *     fp32 partial sums in different orders.
  *     epi_op = BT_EPI_SWIGLU_PAIRS (pair-ordered copy, no residual, no SwiGLU prologue): Y is [B, N/2],
  *     Y[b, h] = what bt_swiglu makes of the stored projections, rd(rd(silu(g)) * u) with g = rd(linear
  *     column h), u = rd(linear column N/2 + h): the SwiGLU MLP's hidden vector leaves the gate|up kernel

@@ -351,3 +351,51 @@ def test_packed_weight_cache_follows_the_weights(monkeypatch):
         with torch.no_grad():
             yh = layer(x.half())
             assert yh.dtype == torch.float16 and torch.equal(yh, fresh_output(layer, x.half()))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_cached_forwards_read_a_decode_tiled_copy_with_the_same_bits(dtype, monkeypatch):
+    """A forward that may use the packed-weight cache runs on the decode-tiled copy the cache builds next to the packed
+    bytes.  Up to 32 rows both layouts take the same kernel and the output equals the training forward's (which
+    quantizes again and reads the row-major bytes) bit for bit; a larger batch may be routed to the streaming kernel
+    on one layout and to the tiled GEMM on the other, whose fp32 sums differ in their last bits (held here to 4e-6 of the
+    largest output in fp32 and to one unit in the last place of the largest output in 16 bits).
+    BITTORCH_KERNEL=generic keeps the row-major bytes."""
+    from bittorch_amd import _C
+    from bittorch_amd.nn import TernaryLinear
+    announce("tiled copy in the packed-weight cache", dtype)
+    seen = {"tiled": 0}
+    real = _C.ternary_linear_tiled_forward
+
+    def counting(*a, **k):
+        seen["tiled"] += 1
+        return real(*a, **k)
+
+    monkeypatch.setattr(_C, "ternary_linear_tiled_forward", counting)
+    for (n, k) in [(32, 64), (250, 1032), (2560, 2560), (37, 100)]:
+        torch.manual_seed(n + k)
+        layer = TernaryLinear(k, n, backend="cuda").cuda().to(dtype)
+        for rows in (1, 8, 200, 600):
+            x = torch.randn(rows, k, device="cuda").to(dtype)
+            before = seen["tiled"]
+            y_train = layer(x)                      # gradient mode on, trainable weights: no cache
+            assert seen["tiled"] == before
+            with torch.no_grad():
+                y_eval = layer(x)
+            assert seen["tiled"] == before + 1
+            if rows <= 32:
+                assert torch.equal(y_train.detach(), y_eval)
+            else:
+                ulp = {torch.float32: 4e-6, torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
+                diff = (y_train.detach().float() - y_eval.float()).abs()
+                assert float(diff.max()) <= ulp * float(y_eval.float().abs().max())
+        packed, scale, tiled = layer._packed.value
+        assert tiled is not None and torch.equal(_C.untile_weights(tiled, n, k), packed)
+        monkeypatch.setenv("BITTORCH_KERNEL", "generic")
+        before = seen["tiled"]
+        with torch.no_grad():
+            y_gen = layer(x)
+        assert seen["tiled"] == before
+        monkeypatch.delenv("BITTORCH_KERNEL")
+        tol = {torch.float32: 1e-4, torch.float16: 2e-3, torch.bfloat16: 1.6e-2}[dtype]
+        assert torch.allclose(y_gen.float(), y_eval.float(), rtol=tol, atol=tol * float(y_eval.float().abs().max()))
