@@ -158,6 +158,71 @@ __global__ __launch_bounds__(256) void act_quant_row_kernel(const void* __restri
     }
 }
 
+// Many short rows: one wave per row (four rows per workgroup), lane l holding the 8-element chunks i * 64 + l -- all
+// 64 lanes busy where the workgroup kernel above leaves lanes idle, the absmax a shuffle tree, no LDS and no barrier.
+// The same bits.
+template <int DT, int ITERS>
+__global__ __launch_bounds__(256) void act_quant_wave_kernel(const void* __restrict__ X, int64_t B, int K,
+                                                             int8_t* __restrict__ Q, float* __restrict__ s_x,
+                                                             int q_layout, int32_t* __restrict__ rowsum) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= B) return;  // (whole waves; the kernel has no barrier)
+    const int64_t base = row * K;
+    float v[ITERS][8];
+#pragma unroll
+    for (int i = 0; i < ITERS; i++) {
+        const int kc = min((i * 64 + lane) * 8, K - 8);  // clamped, unconditional loads; masked below
+        if constexpr (DT == BT_F32) {
+            const uint4 a = *(const uint4*)((const float*)X + base + kc);
+            const uint4 b = *(const uint4*)((const float*)X + base + kc + 4);
+            const uint32_t da[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[i][e] = __builtin_bit_cast(float, da[e]);
+        } else {
+            const uint4 u = *(const uint4*)((const uint16_t*)X + base + kc);
+            const uint32_t d[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const uint16_t h = (uint16_t)(d[e >> 1] >> (16 * (e & 1)));
+                v[i][e] = (DT == BT_F16) ? f16_bits_to_f32(h) : bf16_bits_to_f32(h);
+            }
+        }
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < ITERS; i++) {
+        const bool ok = (i * 64 + lane) * 8 < K;
+#pragma unroll
+        for (int e = 0; e < 8; e++) amax = fmaxf(amax, ok ? fabsf(v[i][e]) : 0.0f);
+    }
+    amax = wave_max(amax);
+    const float s = (amax > 1e-6f) ? __fdiv_rn(amax, 127.0f) : 1.0f;
+    const float inv = __fdiv_rn(1.0f, s);
+    if (lane == 0) s_x[row] = s;
+    int qsum = 0;
+#pragma unroll
+    for (int i = 0; i < ITERS; i++) {
+        const int k = (i * 64 + lane) * 8;
+        uint32_t lo = 0, hi = 0;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            float r = round_half_away(__fmul_rn(v[i][e], inv));
+            r = fmaxf(-127.0f, fminf(127.0f, r));
+            if (k < K) qsum += (int)r;
+            const uint32_t byte = (uint32_t)(uint8_t)(int8_t)(int)r;
+            if (e < 4) lo |= byte << (8 * e);
+            else hi |= byte << (8 * (e - 4));
+        }
+        const uint2 o = q_layout == Q_OPERAND_ORDER ? q_to_operand_order(lo, hi, lane & 1) : make_uint2(lo, hi);
+        if (k < K) st2_nt(Q + base + k, o.x, o.y);
+    }
+    if (rowsum) {  // (uniform)
+        qsum = wave_sum_i32(qsum);
+        if (lane == 0) rowsum[row] = qsum;
+    }
+}
+
 template <int DT>
 static bool launch_act_quant_rows(const void* X, int64_t B, int64_t K, int8_t* Q, float* s_x, int ql, int32_t* rs,
                                   hipStream_t st) {
@@ -166,6 +231,19 @@ static bool launch_act_quant_rows(const void* X, int64_t B, int64_t K, int8_t* Q
         return false;
     const dim3 grid((unsigned)B), block(256);
     const int k = (int)K;
+    if (B >= 2048 && K <= 3072) {  // many short rows: a wave per row (4096 x 2560 bf16 9.4 -> 7.6 us, 4096 x 1024 6.9 -> 4.5,
+                                   // 4096 x 2048 7.3 -> 6.6; from K = 3584 on the workgroup kernel is as fast or faster)
+        const dim3 wgrid((unsigned)((B + 3) / 4));
+        switch ((k + 511) / 512) {
+            case 1: hipLaunchKernelGGL((act_quant_wave_kernel<DT, 1>), wgrid, block, 0, st, X, B, k, Q, s_x, ql, rs); break;
+            case 2: hipLaunchKernelGGL((act_quant_wave_kernel<DT, 2>), wgrid, block, 0, st, X, B, k, Q, s_x, ql, rs); break;
+            case 3: hipLaunchKernelGGL((act_quant_wave_kernel<DT, 3>), wgrid, block, 0, st, X, B, k, Q, s_x, ql, rs); break;
+            case 4: hipLaunchKernelGGL((act_quant_wave_kernel<DT, 4>), wgrid, block, 0, st, X, B, k, Q, s_x, ql, rs); break;
+            case 5: hipLaunchKernelGGL((act_quant_wave_kernel<DT, 5>), wgrid, block, 0, st, X, B, k, Q, s_x, ql, rs); break;
+            default: hipLaunchKernelGGL((act_quant_wave_kernel<DT, 6>), wgrid, block, 0, st, X, B, k, Q, s_x, ql, rs); break;
+        }
+        return true;
+    }
     if (K <= 2048) hipLaunchKernelGGL((act_quant_row_kernel<DT, 1>), grid, block, 0, st, X, k, Q, s_x, ql, rs);
     else if (K <= 4096) hipLaunchKernelGGL((act_quant_row_kernel<DT, 2>), grid, block, 0, st, X, k, Q, s_x, ql, rs);
     else if (K <= 8192) hipLaunchKernelGGL((act_quant_row_kernel<DT, 4>), grid, block, 0, st, X, k, Q, s_x, ql, rs);

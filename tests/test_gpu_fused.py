@@ -543,3 +543,41 @@ def test_swiglu_module_on_prefill_copies_replays_in_a_graph():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(y, want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("b,k", [(2050, 520), (2048, 2560), (4099, 1032), (2051, 3072), (4096, 24), (4100, 2056)])
+def test_many_short_rows_match_the_oracle_bit_for_bit(oracle, dtype, b, k):
+    """Launches of thousands of short rows run one wave per row (rows that would leave a quarter of a workgroup's lanes
+    idle): the same values, codes, scales and row sums as the oracle's, for every iteration count the kernel is built
+    with, in both storage orders, with the row count not a multiple of the four rows a workgroup takes."""
+    from bittorch_amd import _C
+    announce("one wave per row", dtype, b, k)
+    g = (seeded_acts(b, k, seed=b + k, dtype=dtype, outliers=True) * 3)
+    u = seeded_acts(b, k, seed=b + k + 1, dtype=dtype)
+    u[1] = 0
+    w = (1 + 0.1 * torch.randn(k, generator=torch.Generator().manual_seed(k))).to(dtype)
+    oh, oq, os_ = oracle.swiglu(f32np(g), f32np(u), BT_DT[dtype])
+    h, q, s, rs = _C.swiglu(g.cuda(), u.cuda(), store=True, quantize=True, return_rowsum=True)
+    np.testing.assert_array_equal(f32np(h), oh)
+    np.testing.assert_array_equal(s.cpu().numpy(), os_)
+    np.testing.assert_array_equal(q.cpu().numpy(), oq)
+    np.testing.assert_array_equal(rs.cpu().numpy(), oq.astype(np.int32).sum(1))
+    assert torch.equal(_C.swiglu(g.cuda(), u.cuda()), h)
+    oy, oq, os_ = oracle.rmsnorm(f32np(g), f32np(w), 1e-5, BT_DT[dtype])
+    y, q, s = _C.rmsnorm(g.cuda(), w.cuda(), 1e-5, store=True, quantize=True)
+    np.testing.assert_array_equal(f32np(y), oy)
+    np.testing.assert_array_equal(s.cpu().numpy(), os_)
+    np.testing.assert_array_equal(q.cpu().numpy(), oq)
+    assert torch.equal(_C.rmsnorm(g.cuda(), w.cuda(), 1e-5), y)
+    if k % 16 == 0:  # operand order: the same codes, every aligned 16 of them 4 x 4 transposed
+        q2, s2 = _C.rmsnorm(g.cuda(), w.cuda(), 1e-5, store=False, quantize=True, operand_order=True)
+        assert torch.equal(s2, s)
+        assert torch.equal(q2.view(b, k // 16, 4, 4).transpose(2, 3).reshape(b, k), q)
+    # the generic kernel (element-wise passes) agrees
+    set_option("ROWOP_GENERIC", "1")
+    try:
+        y3, q3, s3 = _C.rmsnorm(g.cuda(), w.cuda(), 1e-5, store=True, quantize=True)
+    finally:
+        set_option("ROWOP_GENERIC", None)
+    assert torch.equal(y3, y) and torch.equal(q3, q) and torch.equal(s3, s)

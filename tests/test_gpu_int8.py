@@ -27,6 +27,25 @@ def test_act_quant_bit_exact(oracle, dtype, b, k):
     np.testing.assert_array_equal(q.cpu().numpy(), oq)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("b,k", [(2050, 520), (2048, 2560), (4099, 1032), (2051, 3072), (4096, 24), (2049, 2000)])
+def test_act_quant_of_many_short_rows_bit_exact(oracle, dtype, b, k):
+    """Thousands of short rows take the quantizer's one-wave-per-row kernel: codes and scales equal the oracle's, the
+    row sums equal the codes' sums, and the operand order holds the same codes 4 x 4 transposed."""
+    from bittorch_amd import _C
+    announce("act_quant, a wave per row", dtype, b, k)
+    x = seeded_acts(b, k, seed=b + k, dtype=dtype, outliers=True)
+    x[1] = 0
+    q, s, rs = _C.act_quant_int8(x.cuda(), False, True)
+    oq, os_ = oracle.act_quant_i8(f32np(x))
+    np.testing.assert_array_equal(s.cpu().numpy(), os_)
+    np.testing.assert_array_equal(q.cpu().numpy(), oq)
+    np.testing.assert_array_equal(rs.cpu().numpy(), oq.astype(np.int32).sum(1))
+    if k % 16 == 0:
+        qo, so = _C.act_quant_int8(x.cuda(), True)
+        assert torch.equal(so, s) and torch.equal(qo.view(b, k // 16, 4, 4), q.view(b, k // 16, 4, 4).transpose(2, 3))
+
+
 def _gemm_case(oracle, b, n, k, out_dtype, seed=0, bias=True, outliers=False):
     from bittorch_amd import _C
     from bittorch_amd.quant import pack_ternary_transposed
