@@ -48,7 +48,16 @@ def ternary_quantize(weight: Tensor, threshold_factor: float = 0.05,
         scale = mag.max(dim=1, keepdim=True).values.clamp(min=_SCALE_FLOOR)
     else:
         scale = mag.max().reshape(1).clamp(min=_SCALE_FLOOR)
-    keep = mag > threshold_factor * scale
+    if scale.dtype in (torch.float16, torch.bfloat16):
+        # ``threshold_factor * scale`` on a 16-bit tensor is float(threshold_factor) * float(scale), rounded to fp32 and
+        # then to the tensor's dtype -- two roundings, which is what torch's CPU kernels and the quantize+pack kernel
+        # do.  torch's ROCm kernel fuses them into ONE rounding of the exact product, which lands on the other
+        # neighbour where the fp32 product is a tie (a few elements per million at threshold_factor = 0.7): the two
+        # steps are spelled out so that every device gives the same threshold.
+        threshold = (scale.float() * threshold_factor).to(scale.dtype)
+    else:
+        threshold = threshold_factor * scale
+    keep = mag > threshold
     w_tern = torch.where(keep, torch.sign(weight), torch.zeros_like(weight))
     return w_tern, (scale.squeeze(1) if per_channel else scale.squeeze(0))
 

@@ -109,3 +109,34 @@ def test_unpack_dequant_roundtrip(oracle):
                                       oracle.unpack_ternary_transposed(packed.cpu().numpy(), k))
         deq = _C.unpack_dequant(packed, k, scale, out_dtype=torch.float32)
         assert torch.equal(deq, tern.float() * scale.unsqueeze(1))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_threshold_ties_in_16_bit_weights(oracle, dtype):
+    """``threshold_factor * scale`` on 16-bit weights is a float product rounded to fp32 and then to the weights' dtype.
+    With threshold_factor = 0.7 the fp32 product is now and then exactly half way between two 16-bit values, and a
+    weight equal to the upper one survives or not depending on which way the tie goes: the kernel, the oracle and the
+    torch path of ``quant.ternary_quantize`` on either device must all take the two roundings (torch's ROCm kernel
+    for ``scalar * half_tensor`` alone would round the exact product once and keep such a weight)."""
+    from bittorch_amd import _C
+    from bittorch_amd.quant import pack_ternary_transposed, ternary_quantize
+    announce("threshold ties", dtype)
+    ties = 0
+    for seed in (1, 2, 3, 4):
+        torch.manual_seed(seed)
+        w = (torch.randn(800, 800) * 0.02).to(dtype)
+        packed, scale, tern = _C.ternary_quantize_pack(w.cuda(), 0.7, True, True, True)
+        o_tern, o_scale = oracle.ternary_quantize(f32np(w), 0.7, True, dtype=BT_DT[dtype])
+        np.testing.assert_array_equal(tern.cpu().numpy(), o_tern)
+        for dev in ("cpu", "cuda"):
+            w_t, s = ternary_quantize(w.to(dev), 0.7, True)
+            assert torch.equal(s.cpu().float(), torch.from_numpy(o_scale))
+            np.testing.assert_array_equal(w_t.cpu().float().numpy(), o_tern.astype(np.float32))
+            if dev == "cuda":
+                assert torch.equal(pack_ternary_transposed(w_t)[0], packed)
+        if dtype == torch.float16:  # how many rows of this matrix have such a tie (the test must meet the case)
+            prod = o_scale.astype(np.float32) * np.float32(0.7)
+            near = prod.astype(np.float16)
+            away = np.nextafter(near, np.where(prod > near.astype(np.float32), np.float16(np.inf), np.float16(-np.inf)))
+            ties += int(((near.astype(np.float64) + away.astype(np.float64)) / 2 == prod.astype(np.float64)).sum())
+    assert dtype != torch.float16 or ties > 0
