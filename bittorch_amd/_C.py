@@ -166,7 +166,10 @@ def _residual_2d(residual: Tensor, like: Tensor, lead_shape, N: int) -> Tensor:
     _check(residual.shape == (*lead_shape, N), "residual shape doesn't match the output")
     _check(residual.dtype == like.dtype, "residual must have the output's dtype")
     _check(residual.device == like.device, "All tensors must be CUDA")
-    return residual.contiguous().reshape(-1, N)
+    r = residual.contiguous()
+    if r.data_ptr() % 16:  # a view that starts inside a buffer: the epilogues read the residual in 16-byte pieces
+        r = r.clone()
+    return r.reshape(-1, N)
 
 
 def ternary_linear_packed_forward(X: Tensor, W_T: Tensor, scale: Tensor,

@@ -8,6 +8,7 @@ import pytest
 import torch
 
 from conftest import announce
+from _util import random_ternary, seeded_acts
 
 pytestmark = pytest.mark.gpu
 
@@ -163,3 +164,52 @@ def test_vocabulary_wide_and_very_deep_layers(n, k):
         assert ((y.float() - ref).abs().max() / ref.abs().max()).item() < 1e-2
         y8 = _C.ternary_linear_tensor_core_forward(x, packed, scale, None, k, 2)
         assert ((y8.float() - ref).abs().max() / ref.abs().max()).item() < 5e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_operands_that_start_inside_a_buffer(dtype):
+    """Activations, scale, bias and residual handed over as views that start 1, 3 or 4 elements into a buffer (not
+    16-byte aligned), rows that are a column slice of a wider matrix, a 3-D batch: the same results as the aligned
+    call -- bit for bit on the integer paths, to the output rounding where another kernel takes the call."""
+    from bittorch_amd import _C
+    from bittorch_amd.quant import pack_ternary_transposed
+
+    def off_view(t, off):
+        buf = torch.empty(t.numel() + off, dtype=t.dtype, device=t.device)
+        buf[off:] = t.reshape(-1)
+        return buf[off:].view(t.shape)
+
+    announce("offset operands", dtype)
+    tol = {torch.float32: 3e-5, torch.bfloat16: 1.6e-2, torch.float16: 2e-3}[dtype]
+    for (m, n, k) in [(1, 256, 512), (7, 100, 72), (40, 520, 1040), (130, 64, 333)]:
+        w = random_ternary(n, k, seed=m + n)
+        packed = pack_ternary_transposed(w)[0].cuda()
+        x = seeded_acts(m, k, seed=3, dtype=dtype).cuda()
+        scale = (torch.rand(n, generator=torch.Generator().manual_seed(1)) * 0.05 + 0.01).cuda()
+        bias = seeded_acts(1, n, seed=4, dtype=dtype).reshape(-1).cuda()
+        res = seeded_acts(m, n, seed=5, dtype=dtype).cuda()
+        y0 = _C.ternary_linear_packed_forward(x, packed, scale, bias, k, res)
+        for off in (1, 3, 4):
+            y1 = _C.ternary_linear_packed_forward(off_view(x, off), packed, off_view(scale, off), off_view(bias, off), k,
+                                                  off_view(res, off))
+            assert float((y1.double() - y0.double()).abs().max()) <= tol * float(y0.double().abs().max())
+            q0, s0 = _C.act_quant_int8(x)
+            q1, s1 = _C.act_quant_int8(off_view(x, off))
+            assert torch.equal(q0, q1) and torch.equal(s0, s1)
+            u = seeded_acts(m, k, seed=6, dtype=dtype).cuda()
+            a0 = _C.swiglu(x, u, store=True, quantize=True)
+            a1 = _C.swiglu(off_view(x, off), off_view(u, off), store=True, quantize=True)
+            assert all(torch.equal(p, q) for p, q in zip(a0, a1))
+            if k % 16 == 0:
+                y8 = _C.ternary_gemm_int8(q0, s0, packed, scale, bias.float(), k, dtype, True, res)
+                y9 = _C.ternary_gemm_int8(q0, off_view(s0, off), packed, off_view(scale, off), off_view(bias.float(), off), k,
+                                          dtype, True, off_view(res, off))
+                assert torch.equal(y8[0], y9[0]) and torch.equal(y8[1], y9[1])
+        wide = seeded_acts(m, k + 24, seed=7, dtype=dtype).cuda()
+        xs = wide[:, 8:8 + k]
+        y2 = _C.ternary_linear_packed_forward(xs, packed, scale, bias, k)
+        y3 = _C.ternary_linear_packed_forward(xs.contiguous(), packed, scale, bias, k)
+        assert float((y2.double() - y3.double()).abs().max()) <= tol * float(y3.double().abs().max())
+        qa, sa = _C.act_quant_int8(xs)
+        qb, sb = _C.act_quant_int8(xs.contiguous())
+        assert torch.equal(qa, qb) and torch.equal(sa, sb)
